@@ -1,0 +1,201 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized TorqHL operator path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--no-others]
+
+A "step" is one dispatch of the workload's program (inputs resident in HBM).  The default workload
+is the int8 fully_connected (4096, 4096, 4096) with fused per-column requant, the largest
+single-GPU case of the benchmark's matmul configuration; its metric is int8 GOP/s (1 MAC = 2 ops)
+against the dense int8 MFMA peak.  The other benchmark shapes are measured briefly in the same run
+and reported under "per_op" with the roofline that bounds each.
+
+Prints ONE JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, TOP/s
+PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
+
+
+def import_package():
+    import __graft_entry__ as entry
+    return entry._import_package()
+
+
+def workload_table(pkg):
+    w = pkg.workloads
+    return {
+        "fc_4096x4096x4096": (lambda: w.fully_connected_workload(4096, 4096, 4096), "mfma"),
+        "fc_512x4096x4096": (lambda: w.fully_connected_workload(512, 4096, 4096), "mfma"),
+        "fc_16x2048x8192": (lambda: w.fully_connected_workload(16, 2048, 8192), "hbm"),
+        "fc_1x2048x2048": (lambda: w.fully_connected_workload(1, 2048, 2048), "hbm"),
+        "conv_112x112x32_o64_3x3": (lambda: w.conv2d_workload(), "mfma"),
+        "depthwise_b64": (lambda: w.depthwise_workload(N=64), "hbm"),
+        "depthwise_b1": (lambda: w.depthwise_workload(N=1), "hbm"),
+        "maxpool_b64": (lambda: w.maxpool_workload(N=64), "hbm"),
+        "maxpool_b1": (lambda: w.maxpool_workload(N=1), "hbm"),
+        "avgpool_b64": (lambda: w.avgpool_workload(N=64), "hbm"),
+        "avgpool_b1": (lambda: w.avgpool_workload(N=1), "hbm"),
+        "add_b64": (lambda: w.add_workload(N=64), "hbm"),
+        "add_b1": (lambda: w.add_workload(N=1), "hbm"),
+    }
+
+
+class Loaded:
+    """A workload resident on the GPU: executable + device buffers."""
+
+    def __init__(self, pkg, dev, wl):
+        self.wl = wl
+        self.dev = dev
+        self.exe = pkg.Executable(dev, wl.program.serialize())
+        self.outs = [np.zeros(s, dtype=dt) for s, dt in wl.outputs]
+        self.ptrs = [dev.upload(a) for a in wl.inputs] + [dev.upload(o) for o in self.outs]
+        self.lens = [a.nbytes for a in wl.inputs] + [o.nbytes for o in self.outs]
+
+    def run(self, iterations):
+        """Returns mean ms per dispatch from HIP events on the executable's stream."""
+        return self.exe.time_device(self.ptrs, self.lens, iterations)
+
+    def output(self, i=0):
+        o = self.outs[i]
+        return self.dev.download(self.ptrs[len(self.wl.inputs) + i], o.shape, o.dtype)
+
+    def close(self):
+        self.exe.close()
+        for p in self.ptrs:
+            self.dev.free(p)
+
+
+def roofline(wl, bound, ms):
+    if bound == "mfma":
+        achieved = wl.ops / (ms * 1e-3) / 1e12
+        return {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                "frac": round(achieved / PEAK_INT8_TOPS, 5), "traffic": None}
+    achieved = wl.bytes / (ms * 1e-3) / 1e9
+    return {"bound": "hbm", "achieved": round(achieved, 2), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+            "frac": round(achieved / PEAK_HBM_GBS, 5), "traffic": None}
+
+
+def verify_sample(loaded):
+    """Checks the GPU result of the timed workload against the oracle (sampled rows for the big GEMMs)."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    from helpers import oracle_eval
+    from oracle import oracle as orc
+    wl = loaded.wl
+    got = loaded.output()
+    if wl.name.startswith("fully_connected") and wl.inputs[0].shape[0] > 64:
+        a = dict(wl.attrs)
+        wts, sb = a.pop("weights"), a.pop("scale_bias")
+        M = wl.inputs[0].shape[0]
+        rows = np.unique(np.r_[0:16, M // 2:M // 2 + 16, M - 16:M])
+        want = orc.fully_connected(wl.inputs[0][rows], wts, sb, **a)
+        return bool(np.array_equal(got[rows], want))
+    return bool(np.array_equal(got, oracle_eval(wl)[0]))
+
+
+def cpu_baseline(wl, target_seconds=12.0):
+    """Times the CPU oracle on a bounded sample of the default workload on this host's cores."""
+    from oracle import oracle as orc
+    a = dict(wl.attrs)
+    wts, sb = a.pop("weights"), a.pop("scale_bias")
+    x = wl.inputs[0]
+    M, K = x.shape
+    N = wts.shape[0]
+    rows = min(M, 8)
+    t0 = time.perf_counter()
+    orc.fully_connected(x[:rows], wts, sb, **a)
+    dt = max(time.perf_counter() - t0, 1e-4)
+    rows = int(min(M, max(rows, rows * target_seconds / dt)))
+    t0 = time.perf_counter()
+    orc.fully_connected(x[:rows], wts, sb, **a)
+    dt = time.perf_counter() - t0
+    gops = 2.0 * rows * K * N / dt / 1e9
+    return {"value": round(gops, 2), "unit": "GOP/s", "cores": orc.threads(), "kind": "port",
+            "sample": "first %d of %d rows of the same (M,K,N)=(%d,%d,%d) fully_connected, %.1f s, C oracle with OpenMP"
+                      % (rows, M, M, K, N, dt)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="fc_4096x4096x4096")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-others", action="store_true", help="skip the brief per-op measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    pkg = import_package()
+    table = workload_table(pkg)
+    if args.workload not in table:
+        sys.exit("unknown workload %s; choose from %s" % (args.workload, ", ".join(table)))
+    dev = pkg.Device(0)
+
+    make, bound = table[args.workload]
+    wl = make()
+    loaded = Loaded(pkg, dev, wl)
+    kernels = loaded.exe.op_kernels()
+    if args.warmup > 0:
+        loaded.run(args.warmup)
+    dev.synchronize()
+    t0 = time.perf_counter()
+    ev_ms = loaded.run(args.steps)          # HIP events on the executable's stream around the K dispatches
+    dev.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ok = verify_sample(loaded)
+    loaded.close()
+
+    per_op = {}
+    if not args.no_others:
+        for name, (mk, bnd) in table.items():
+            if name == args.workload:
+                continue
+            o = Loaded(pkg, dev, mk())
+            o.run(5)
+            ms = o.run(50)
+            r = roofline(o.wl, bnd, ms)
+            per_op[name] = {"us": round(ms * 1e3, 2), "kernel": o.exe.op_kernels()[-1 if "transpose" in o.exe.op_kernels()[0] else 0],
+                            "GOP/s": round(o.wl.ops / (ms * 1e-3) / 1e9, 1), "GB/s": round(o.wl.bytes / (ms * 1e-3) / 1e9, 1),
+                            "bound": bnd, "frac": r["frac"]}
+            o.close()
+
+    result = {
+        "metric": "int8 GOP/s (fully_connected with fused requant), 1 MAC = 2 ops",
+        "value": round(wl.ops / (wall_ms * 1e-3) / 1e9, 1),
+        "unit": "GOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "kernels": kernels, "parity_checked": ok,
+                   "algorithmic_ops": wl.ops, "algorithmic_bytes": wl.bytes},
+        "roofline": dict(roofline(wl, bound, ev_ms), kernel=kernels[0], kernel_ms=round(ev_ms, 5)),
+    }
+    if not args.no_cpu and args.workload.startswith("fc_"):
+        result["cpu_baseline"] = cpu_baseline(wl)
+    if per_op:
+        result["per_op"] = per_op
+    dev.close()
+    print(json.dumps(result))
+    if not ok:
+        sys.exit("GPU result differs from the oracle")
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,356 @@
+/*
+ * thip -- C-ABI of the MI355X (gfx950) backend for the quantized TorqHL
+ * operator path.
+ *
+ * Plain C linkage, plain pointers and sizes.  Two halves, mirroring the two
+ * places where the reference's NPU-specific code is replaced:
+ *
+ *   compile side  thip_program_* / thip_hl_*  : accepts torq_hl.{conv2d,
+ *                 depthwise_conv2d, fully_connected, matmul, maxpool2d,
+ *                 avg_pool2d, add} records with the reference's operand and
+ *                 attribute names and serialises a dispatch descriptor
+ *                 (role of KernelSelection + EncodeTensors + serializeTorqHW).
+ *   run side      thip_device_* / thip_executable_* : loads a descriptor and
+ *                 runs it on bindings (role of the torq HAL driver's
+ *                 native_executable + TorqExecutable + TorqHw).
+ *
+ * Every entry point returns a thip_status_t whose numeric values are the
+ * status categories the reference returns through iree_status_t; the text of
+ * the last failure on the calling thread is available from
+ * thip_status_message().  No exception crosses this boundary.
+ *
+ * Reference paths below are relative to the reference checkout.
+ */
+#ifndef THIP_H_
+#define THIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ------------------------------------------------------------------------ */
+/* Status                                                                   */
+/* ------------------------------------------------------------------------ */
+
+/* Same categories (and numeric codes) as the iree_status_t values used by
+ * runtime/driver/TorqExecutable.cc:640-705 and
+ * runtime/driver/torq_command_buffer.c:453-494. */
+typedef int32_t thip_status_t;
+enum {
+    THIP_OK = 0,
+    THIP_INVALID_ARGUMENT = 3,
+    THIP_RESOURCE_EXHAUSTED = 8,
+    THIP_FAILED_PRECONDITION = 9,
+    THIP_OUT_OF_RANGE = 11,
+    THIP_UNIMPLEMENTED = 12,
+    THIP_INTERNAL = 13,
+    THIP_UNAVAILABLE = 14
+};
+
+/* Message of the last non-OK status returned on this thread ("" if none). */
+const char *thip_status_message(void);
+
+/* Library version (major << 16 | minor) and the descriptor version it reads. */
+uint32_t thip_version(void);
+uint32_t thip_descriptor_version(void);
+
+/* ------------------------------------------------------------------------ */
+/* Compile side: TorqHL program -> dispatch descriptor                      */
+/* ------------------------------------------------------------------------ */
+
+typedef struct thip_program_t thip_program_t;
+
+/* A tensor value of the program (index into the program's value table). */
+typedef int32_t thip_value_t;
+
+enum { THIP_DTYPE_I8 = 1, THIP_DTYPE_I16 = 2, THIP_DTYPE_I32 = 3 };
+
+#define THIP_MAX_RANK 4
+
+/* torq_hl VectorizationModeEnum (compiler/torq/Dialect/TorqHL/TorqHLAttrs.td:149-239).
+ * The patterns emit None; the NPU kernel-selection pass picks the others.  The
+ * field is carried for signature compatibility and ignored by this backend. */
+enum { THIP_VECTORIZATION_NONE = 0 };
+
+thip_status_t thip_program_create(thip_program_t **out_program);
+void thip_program_destroy(thip_program_t *program);
+
+/* Declares the tensor carried by dispatch binding `binding` (the
+ * hal.interface.binding of the dispatch; table entry of
+ * runtime/schemas/torq_executable_def.fbs:29-48). */
+thip_status_t thip_program_binding(thip_program_t *program, uint32_t binding, int32_t dtype,
+                                   int32_t rank, const int64_t *shape, thip_value_t *out_value);
+
+/* Declares a compile-time constant (arith.constant); the bytes are copied. */
+thip_status_t thip_program_constant(thip_program_t *program, int32_t dtype, int32_t rank,
+                                    const int64_t *shape, const void *data, size_t data_size,
+                                    thip_value_t *out_value);
+
+/* Declares an intermediate tensor (tensor.empty used as `init` of an op whose
+ * result feeds another op of the same program). */
+thip_status_t thip_program_tensor(thip_program_t *program, int32_t dtype, int32_t rank,
+                                  const int64_t *shape, thip_value_t *out_value);
+
+/* The op records.  Field names and meaning are those of the TorqHL op
+ * definitions; `init` is the destination-passing-style output operand
+ * (compiler/torq/Dialect/TorqHL/TorqHLOps.td:27-46). */
+
+/* torq_hl.conv2d -- TorqHLOps.td:119-143.  input N,C,H,W (N,H,W,C when
+ * nhwc_input), weights O,I,KH,KW, scale_bias int32[2*O] = [bias0, scale0, ...],
+ * pad = [left, right, top, bottom], stride = [h, w].  With nhwc_input the init
+ * tensor is N,OH,OW,O as well.  groups must be 1, dilation [1,1] (folded into
+ * the weights by the patterns), weight_zp 0. */
+typedef struct thip_hl_conv2d_t {
+    thip_value_t init;
+    int32_t input_zp;
+    int32_t weight_zp;
+    int32_t output_zp;
+    int32_t output_min;
+    int32_t output_max;
+    int32_t shift_factor;
+    int32_t groups;
+    int64_t pad[4];
+    int64_t stride[2];
+    int64_t dilation[2];
+    int32_t vectorization_mode;
+    thip_value_t weights;
+    thip_value_t scale_bias;
+    thip_value_t input;
+    int32_t nhwc_input;
+    int32_t segment_output;
+} thip_hl_conv2d_t;
+
+/* torq_hl.depthwise_conv2d -- TorqHLOps.td:145-170.  weights C,1,KH,KW. */
+typedef struct thip_hl_depthwise_conv2d_t {
+    thip_value_t init;
+    int32_t input_zp;
+    int32_t weight_zp;
+    int32_t output_zp;
+    int32_t output_min;
+    int32_t output_max;
+    int32_t shift_factor;
+    int32_t groups;
+    int64_t pad[4];
+    int64_t stride[2];
+    int64_t dilation[2];
+    int32_t vectorization_mode;
+    thip_value_t weights;
+    thip_value_t scale_bias;
+    thip_value_t input;
+    int32_t nhwc_input;
+    int32_t segment_output;
+    int32_t is_dw1d_stride1;
+} thip_hl_depthwise_conv2d_t;
+
+/* torq_hl.fully_connected -- TorqHLOps.td:172-190.  input M,K; weights N,K;
+ * scale_bias int32[2*N]. */
+typedef struct thip_hl_fully_connected_t {
+    thip_value_t init;
+    int32_t input_zp;
+    int32_t weight_zp;
+    int32_t output_zp;
+    int32_t output_min;
+    int32_t output_max;
+    int32_t shift_factor;
+    int32_t vectorization_mode;
+    thip_value_t weights;
+    thip_value_t scale_bias;
+    thip_value_t input;
+} thip_hl_fully_connected_t;
+
+/* torq_hl.matmul -- TorqHLOps.td:85-99.  input1 [B,]M,K; input2 [B,]K,N; one
+ * (bias, scale) pair in scale_bias; a batch of 1 broadcasts. */
+typedef struct thip_hl_matmul_t {
+    thip_value_t init;
+    int32_t output_zp;
+    int32_t output_min;
+    int32_t output_max;
+    int32_t shift;
+    thip_value_t scale_bias;
+    thip_value_t input1;
+    thip_value_t input2;
+} thip_hl_matmul_t;
+
+/* torq_hl.maxpool2d -- TorqHLOps.td:435-453.  input N,C,H,W; kernel = [kh, kw];
+ * weights / scale_bias are the dummies the pattern creates and may be -1.
+ * nhwc_input is this backend's addition (same meaning as on conv2d). */
+typedef struct thip_hl_maxpool2d_t {
+    thip_value_t init;
+    int32_t input_zp;
+    int32_t output_min;
+    int32_t output_max;
+    int64_t stride[2];
+    int64_t pad[4];
+    int64_t kernel[2];
+    thip_value_t weights;
+    thip_value_t scale_bias;
+    thip_value_t input;
+    int32_t segment_output;
+    int32_t nhwc_input;
+} thip_hl_maxpool2d_t;
+
+/* torq_hl.avg_pool2d -- TorqHLOps.td:192-208.  Global: input N,H,W,C (NHWC),
+ * init N,1,1,C; weights one int8; pair 0 of scale_bias applies to every channel. */
+typedef struct thip_hl_avg_pool2d_t {
+    thip_value_t init;
+    int32_t input_zp;
+    int32_t output_zp;
+    int32_t output_min;
+    int32_t output_max;
+    int32_t shift_factor;
+    thip_value_t weights;
+    thip_value_t scale_bias;
+    thip_value_t input;
+} thip_hl_avg_pool2d_t;
+
+/* torq_hl.add -- TorqHLOps.td:48-69.  weights int16[2]; scale_bias int32[2];
+ * `name` is "add" or "sub" (the sign already lives in weights[1]). */
+typedef struct thip_hl_add_t {
+    thip_value_t init;
+    const char *name;
+    int32_t input_zp;
+    int32_t output_zp;
+    int32_t output_min;
+    int32_t output_max;
+    int32_t shift_factor;
+    thip_value_t weights;
+    thip_value_t scale_bias;
+    thip_value_t input1;
+    thip_value_t input2;
+    int32_t segment_output;
+    int32_t rhs_is_scalar;
+} thip_hl_add_t;
+
+/* torq_hl.transpose -- TorqHLOps.td:397-407.  out.shape[i] = in.shape[perm[i]].
+ * Rank-4 perms [0,2,3,1] (NCHW->NHWC) and [0,3,1,2] (NHWC->NCHW) and the swap of
+ * the two innermost dimensions of a rank-2/3 tensor are supported; between two
+ * ops of one program they fold into the producing kernel's layout. */
+typedef struct thip_hl_transpose_t {
+    thip_value_t init;
+    int32_t rank;
+    int64_t perm[THIP_MAX_RANK];
+    thip_value_t input;
+} thip_hl_transpose_t;
+
+thip_status_t thip_hl_conv2d(thip_program_t *program, const thip_hl_conv2d_t *op);
+thip_status_t thip_hl_depthwise_conv2d(thip_program_t *program,
+                                       const thip_hl_depthwise_conv2d_t *op);
+thip_status_t thip_hl_fully_connected(thip_program_t *program,
+                                      const thip_hl_fully_connected_t *op);
+thip_status_t thip_hl_matmul(thip_program_t *program, const thip_hl_matmul_t *op);
+thip_status_t thip_hl_maxpool2d(thip_program_t *program, const thip_hl_maxpool2d_t *op);
+thip_status_t thip_hl_avg_pool2d(thip_program_t *program, const thip_hl_avg_pool2d_t *op);
+thip_status_t thip_hl_add(thip_program_t *program, const thip_hl_add_t *op);
+thip_status_t thip_hl_transpose(thip_program_t *program, const thip_hl_transpose_t *op);
+
+/* Serialises the program (role of TargetBackend::serializeExecutable,
+ * compiler/torq/Target/TorqTarget.cpp:115-151, and serializeTorqHW,
+ * compiler/torq/Serialization/Serialization.cpp:265-302): picks a kernel
+ * variant per op, pre-packs weights for the MFMA operand layout, splits
+ * scale_bias, lays out intermediates.  The blob is malloc'ed; release it with
+ * thip_blob_free. */
+thip_status_t thip_program_serialize(thip_program_t *program, void **out_blob, size_t *out_size);
+void thip_blob_free(void *blob);
+
+/* ------------------------------------------------------------------------ */
+/* Run side: device, executable, dispatch                                   */
+/* ------------------------------------------------------------------------ */
+
+typedef struct thip_device_t thip_device_t;
+typedef struct thip_executable_t thip_executable_t;
+
+/* Opens GPU `ordinal` (role of the driver factory's try_create for "torq",
+ * runtime/driver/registration/driver_module.c:95-168).  Fails with
+ * THIP_UNAVAILABLE when no gfx950 device is present. */
+thip_status_t thip_device_create(int32_t ordinal, thip_device_t **out_device);
+void thip_device_destroy(thip_device_t *device);
+/* Writes the device's architecture name ("gfx950") into `name`. */
+thip_status_t thip_device_name(thip_device_t *device, char *name, size_t capacity);
+
+/* Device memory (role of TorqHw::allocateDeviceBuffer / writeXram / readXram,
+ * runtime/torq_hw/inc/TorqHw.h:96-121). */
+thip_status_t thip_device_alloc(thip_device_t *device, size_t size, void **out_ptr);
+thip_status_t thip_device_free(thip_device_t *device, void *ptr);
+thip_status_t thip_device_h2d(thip_device_t *device, void *dst_device, const void *src_host,
+                              size_t size);
+thip_status_t thip_device_d2h(thip_device_t *device, void *dst_host, const void *src_device,
+                              size_t size);
+thip_status_t thip_device_synchronize(thip_device_t *device);
+
+/* Validates the header of a descriptor blob and writes the format string
+ * ("thip-gfx950") -- iree_hal_torq_native_executable_infer_format,
+ * runtime/driver/native_executable.cc:151-178. */
+thip_status_t thip_infer_format(const void *blob, size_t size, size_t format_capacity,
+                                char *format, size_t *out_inferred_size);
+
+/* Creates an executable from a descriptor: copies the blob, uploads its
+ * constant segments, allocates intermediates --
+ * iree_hal_torq_native_executable_create, runtime/driver/native_executable.h:42-46,
+ * native_executable.cc:41-108.  `constants` are the executable-level constants
+ * of iree_hal_executable_params_t (copied; may be NULL when count is 0). */
+thip_status_t thip_executable_create(thip_device_t *device, const void *blob, size_t size,
+                                     const uint32_t *constants, size_t constant_count,
+                                     thip_executable_t **out_executable);
+void thip_executable_destroy(thip_executable_t *executable);
+
+/* Binding flags (role of IREE_HAL_TORQ_BINDING_FLAG_ZERO_COPY_*,
+ * runtime/driver/torq_command_buffer.h:29-30). */
+enum {
+    THIP_BINDING_HOST = 0x0,  /* host pointer: staged through device memory */
+    THIP_BINDING_DEVICE = 0x1 /* device pointer: used in place */
+};
+
+/* The subset of iree_hal_executable_dispatch_state_v0_t that the reference
+ * consumes (runtime/driver/torq_command_buffer.c:423-499) plus the per-binding
+ * flags of iree_hal_torq_dispatch_state_v0_t (torq_command_buffer.h:17-27).
+ * binding_flags may be NULL (all host). */
+typedef struct thip_dispatch_state_t {
+    uint32_t constant_count;
+    const uint32_t *constants;
+    uint32_t binding_count;
+    void *const *binding_ptrs;
+    const size_t *binding_lengths;
+    const uint8_t *binding_flags;
+} thip_dispatch_state_t;
+
+/* Runs the dispatch and returns when the outputs are in the bindings --
+ * iree_hal_torq_native_executable_run, runtime/driver/native_executable.h:57-58,
+ * TorqExecutable::executeDispatch, runtime/driver/TorqExecutable.cc:1025-1125.
+ * Blocking; one dispatch at a time per executable (internal mutex). */
+thip_status_t thip_executable_run(thip_executable_t *executable,
+                                  const thip_dispatch_state_t *state);
+
+/* Same dispatch without the final wait: enqueues on the executable's stream.
+ * Only device bindings are allowed.  Pair with thip_executable_wait. */
+thip_status_t thip_executable_enqueue(thip_executable_t *executable,
+                                      const thip_dispatch_state_t *state);
+thip_status_t thip_executable_wait(thip_executable_t *executable);
+
+/* Enqueues the dispatch `iterations` times between two HIP events recorded on
+ * the executable's stream and returns the mean time of one dispatch in
+ * milliseconds (role of the per-dispatch profile scopes,
+ * runtime/driver/torq_profile_scope.h).  Device bindings only. */
+thip_status_t thip_executable_time(thip_executable_t *executable,
+                                   const thip_dispatch_state_t *state, int32_t iterations,
+                                   float *out_ms_per_dispatch);
+
+/* Introspection used by the harness and the tests. */
+thip_status_t thip_executable_op_count(thip_executable_t *executable, uint32_t *out_count);
+/* Name of the kernel chosen for op `index` (e.g. "igemm_i8_128x128x64"). */
+thip_status_t thip_executable_op_kernel(thip_executable_t *executable, uint32_t index,
+                                        char *name, size_t capacity);
+thip_status_t thip_executable_binding_count(thip_executable_t *executable, uint32_t *out_count);
+thip_status_t thip_executable_binding_size(thip_executable_t *executable, uint32_t binding,
+                                           size_t *out_size);
+
+/* Per-dispatch event log (role of TorqEventLog, runtime/torq_hw/inc/TorqEventLog.h:19-46):
+ * when a path is set every run appends BEGIN/END rows per op as CSV. */
+thip_status_t thip_device_set_event_log(thip_device_t *device, const char *csv_path);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* THIP_H_ */

@@ -1,0 +1,257 @@
+"""numpy front-end of the C oracle (``libtorq_oracle.so``).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, by the smoke check and by the
+benchmark's CPU-baseline leg, never by the product package.  Every function is a
+thin ctypes call into ``torq_oracle.c``; argument names follow the TorqHL op
+definitions (compiler/torq/Dialect/TorqHL/TorqHLOps.td:48-208,435-453).
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libtorq_oracle.so")
+
+NCHW, NHWC = 0, 1
+
+
+class Requant(ctypes.Structure):
+    _fields_ = [
+        ("shift", ctypes.c_int32),
+        ("output_zp", ctypes.c_int32),
+        ("output_min", ctypes.c_int32),
+        ("output_max", ctypes.c_int32),
+    ]
+
+
+def build():
+    """Compile the oracle with the Makefile next to this file."""
+    subprocess.run(["make", "-C", _HERE, "-s"], check=True)
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = ctypes.CDLL(_LIB_PATH)
+        L.torq_act_rescale_clamp.restype = ctypes.c_int64
+        L.torq_act_rescale_clamp.argtypes = [ctypes.c_int32] * 3 + [ctypes.POINTER(Requant)]
+        L.torq_derive_scale_bias.restype = ctypes.c_int32
+        L.torq_oracle_threads.restype = ctypes.c_int
+        _lib = L
+    return _lib
+
+
+def _p(a):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def _i64x(vals):
+    return (ctypes.c_int64 * len(vals))(*[int(v) for v in vals])
+
+
+def _c(a, dtype):
+    a = np.ascontiguousarray(a, dtype=dtype)
+    return a
+
+
+_OUT_DTYPES = {1: np.int8, 2: np.int16, 4: np.int32}
+
+
+def threads():
+    return lib().torq_oracle_threads()
+
+
+def set_threads(n):
+    lib().torq_oracle_set_threads(int(n))
+
+
+def act_rescale_clamp(acc, bias, scale, shift, output_zp, output_min, output_max):
+    rq = Requant(shift, output_zp, output_min, output_max)
+    return int(lib().torq_act_rescale_clamp(int(acc), int(bias), int(scale), ctypes.byref(rq)))
+
+
+def _out_hw(H, W, KH, KW, pad, stride):
+    pl, pr, pt, pb = [int(p) for p in pad]
+    OH = (H + pt + pb - KH) // int(stride[0]) + 1
+    OW = (W + pl + pr - KW) // int(stride[1]) + 1
+    return OH, OW
+
+
+def conv2d(input, weights, scale_bias, *, input_zp, output_zp, output_min, output_max,
+           shift_factor, pad, stride, layout=NCHW, out_dtype=np.int8):
+    """torq_hl.conv2d; input N,C,H,W (or N,H,W,C when layout=NHWC), weights O,I,KH,KW."""
+    x = _c(input, np.int8)
+    w = _c(weights, np.int8)
+    sb = _c(scale_bias, np.int32)
+    if layout == NHWC:
+        N, H, W, C = x.shape
+    else:
+        N, C, H, W = x.shape
+    O, I, KH, KW = w.shape
+    assert I == C and sb.size == 2 * O
+    OH, OW = _out_hw(H, W, KH, KW, pad, stride)
+    shape = (N, OH, OW, O) if layout == NHWC else (N, O, OH, OW)
+    out = np.empty(shape, dtype=out_dtype)
+    rq = Requant(shift_factor, output_zp, output_min, output_max)
+    rc = lib().torq_conv2d(_p(x), _p(w), _p(sb), _p(out), N, C, H, W, O, KH, KW, _i64x(pad),
+                           _i64x(stride), ctypes.c_int32(input_zp), ctypes.byref(rq), layout,
+                           out.itemsize)
+    assert rc == 0
+    return out
+
+
+def depthwise_conv2d(input, weights, scale_bias, *, input_zp, output_zp, output_min, output_max,
+                     shift_factor, pad, stride, layout=NCHW, out_dtype=np.int8):
+    """torq_hl.depthwise_conv2d; weights C,1,KH,KW."""
+    x = _c(input, np.int8)
+    w = _c(weights, np.int8)
+    sb = _c(scale_bias, np.int32)
+    if layout == NHWC:
+        N, H, W, C = x.shape
+    else:
+        N, C, H, W = x.shape
+    Cw, one, KH, KW = w.shape
+    assert Cw == C and one == 1 and sb.size == 2 * C
+    OH, OW = _out_hw(H, W, KH, KW, pad, stride)
+    shape = (N, OH, OW, C) if layout == NHWC else (N, C, OH, OW)
+    out = np.empty(shape, dtype=out_dtype)
+    rq = Requant(shift_factor, output_zp, output_min, output_max)
+    rc = lib().torq_depthwise_conv2d(_p(x), _p(w), _p(sb), _p(out), N, C, H, W, KH, KW,
+                                     _i64x(pad), _i64x(stride), ctypes.c_int32(input_zp),
+                                     ctypes.byref(rq), layout, out.itemsize)
+    assert rc == 0
+    return out
+
+
+def fully_connected(input, weights, scale_bias, *, output_zp, output_min, output_max,
+                    shift_factor, out_dtype=np.int8):
+    """torq_hl.fully_connected; input M,K, weights N,K."""
+    x = _c(input, np.int8)
+    w = _c(weights, np.int8)
+    sb = _c(scale_bias, np.int32)
+    M, K = x.shape
+    N, K2 = w.shape
+    assert K == K2 and sb.size == 2 * N
+    out = np.empty((M, N), dtype=out_dtype)
+    rq = Requant(shift_factor, output_zp, output_min, output_max)
+    rc = lib().torq_fully_connected(_p(x), _p(w), _p(sb), _p(out), M, K, N, ctypes.byref(rq),
+                                    out.itemsize)
+    assert rc == 0
+    return out
+
+
+def matmul(input1, input2, scale_bias, *, output_zp, output_min, output_max, shift,
+           out_dtype=np.int32):
+    """torq_hl.matmul; input1 [B,]M,K  input2 [B,]K,N; one (bias, scale) pair."""
+    a = _c(input1, np.int8)
+    b = _c(input2, np.int8)
+    sb = _c(scale_bias, np.int32)
+    a3 = a.reshape((-1,) + a.shape[-2:]) if a.ndim >= 2 else a.reshape(1, 1, -1)
+    b3 = b.reshape((-1,) + b.shape[-2:])
+    B = max(a3.shape[0], b3.shape[0])
+    _, M, K = a3.shape
+    _, K2, N = b3.shape
+    assert K == K2 and sb.size >= 2
+    out = np.empty((B, M, N), dtype=out_dtype)
+    rq = Requant(shift, output_zp, output_min, output_max)
+    rc = lib().torq_matmul(_p(a3), _p(b3), _p(sb), _p(out), B, M, K, N,
+                           int(a3.shape[0] == 1 and B > 1), int(b3.shape[0] == 1 and B > 1),
+                           ctypes.byref(rq), out.itemsize)
+    assert rc == 0
+    return out
+
+
+def maxpool2d(input, *, input_zp, output_min, output_max, stride, pad, kernel, layout=NCHW):
+    """torq_hl.maxpool2d."""
+    x = _c(input, np.int8)
+    if layout == NHWC:
+        N, H, W, C = x.shape
+    else:
+        N, C, H, W = x.shape
+    KH, KW = int(kernel[0]), int(kernel[1])
+    OH, OW = _out_hw(H, W, KH, KW, pad, stride)
+    shape = (N, OH, OW, C) if layout == NHWC else (N, C, OH, OW)
+    out = np.empty(shape, dtype=np.int8)
+    rc = lib().torq_maxpool2d(_p(x), _p(out), N, C, H, W, KH, KW, _i64x(pad), _i64x(stride),
+                              ctypes.c_int32(input_zp), ctypes.c_int32(output_min),
+                              ctypes.c_int32(output_max), layout)
+    assert rc == 0
+    return out
+
+
+def avg_pool2d(input, scale_bias, *, output_zp, output_min, output_max, shift_factor, weight=1):
+    """torq_hl.avg_pool2d (global); input N,H,W,C -> N,1,1,C."""
+    x = _c(input, np.int8)
+    sb = _c(scale_bias, np.int32)
+    N, H, W, C = x.shape
+    out = np.empty((N, 1, 1, C), dtype=np.int8)
+    rq = Requant(shift_factor, output_zp, output_min, output_max)
+    rc = lib().torq_avg_pool2d(_p(x), ctypes.c_int8(weight), _p(sb), _p(out), N, H, W, C,
+                               ctypes.byref(rq))
+    assert rc == 0
+    return out
+
+
+def add(input1, input2, weights, scale_bias, *, output_zp, output_min, output_max, shift_factor):
+    """torq_hl.add (tensor + tensor)."""
+    a = _c(input1, np.int8)
+    b = _c(input2, np.int8)
+    assert a.shape == b.shape
+    w = _c(weights, np.int16)
+    sb = _c(scale_bias, np.int32)
+    out = np.empty(a.shape, dtype=np.int8)
+    rq = Requant(shift_factor, output_zp, output_min, output_max)
+    rc = lib().torq_add(_p(a), _p(b), _p(w), _p(sb), _p(out), ctypes.c_size_t(a.size),
+                        ctypes.byref(rq))
+    assert rc == 0
+    return out
+
+
+def per_channel_sum(weights):
+    w = _c(weights, np.int8)
+    ch = w.shape[0]
+    sums = np.empty(ch, dtype=np.int64)
+    lib().torq_per_channel_sum(_p(w), ch, int(w.size // ch), _p(sums))
+    return sums
+
+
+def derive_scale_bias(multiplier, shift, tosa_bias, weight_sum, input_zp):
+    """R2: returns (scale_bias int32[2*channels], shift_factor)."""
+    m = _c(multiplier, np.int32)
+    s = _c(shift, np.int8)
+    ch = m.size
+    tb = _c(tosa_bias, np.int32) if tosa_bias is not None else None
+    ws = _c(weight_sum, np.int64) if weight_sum is not None else None
+    sb = np.empty(2 * ch, dtype=np.int32)
+    sf = lib().torq_derive_scale_bias(_p(m), _p(s), _p(tb) if tb is not None else None,
+                                      _p(ws) if ws is not None else None,
+                                      ctypes.c_int32(input_zp), ch, _p(sb))
+    return sb, int(sf)
+
+
+def derive_add_params(m0, m1, zp0, zp1, sign=1):
+    """Returns (weights int16[2], scale_bias int32[2], shift_factor) or None if rejected."""
+    w = np.empty(2, dtype=np.int16)
+    sb = np.empty(2, dtype=np.int32)
+    sf = ctypes.c_int32(0)
+    rc = lib().torq_derive_add_params(ctypes.c_double(m0), ctypes.c_double(m1),
+                                      ctypes.c_int32(zp0), ctypes.c_int32(zp1), int(sign),
+                                      _p(w), _p(sb), ctypes.byref(sf))
+    if rc != 0:
+        return None
+    return w, sb, sf.value
+
+
+def derive_avgpool_params(H, W, input_zp):
+    sb = np.empty(2, dtype=np.int32)
+    sf = ctypes.c_int32(0)
+    lib().torq_derive_avgpool_params(int(H), int(W), ctypes.c_int32(input_zp), _p(sb),
+                                     ctypes.byref(sf))
+    return sb, sf.value

@@ -1,0 +1,393 @@
+/*
+ * CPU oracle for the quantized TorqHL operator path.  TEST INFRASTRUCTURE ONLY
+ * (see torq_oracle.h).  Plain C, int64 intermediates, straightforward loop
+ * nests; OpenMP over the outermost independent loop so that the same code
+ * doubles as the timed CPU baseline.
+ */
+#include "torq_oracle.h"
+
+#include <string.h>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+
+static int g_threads = 0; /* 0 = OpenMP default */
+
+int torq_oracle_threads(void) {
+#ifdef _OPENMP
+    return g_threads > 0 ? g_threads : omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+void torq_oracle_set_threads(int n) {
+    g_threads = n;
+#ifdef _OPENMP
+    if (n > 0) {
+        omp_set_num_threads(n);
+    }
+#endif
+}
+
+/*
+ * R1 -- ACT rescaleClamp.
+ * Pseudocode: compiler/torq/Utils/Kernel.h:610-624.  The shift is act_rsh
+ * bits (0..63): third_party/torq-hw/ct/torq_api.c:572-583 (act_sh obsolete,
+ * torq_api.h:82-83).  Rounding NTP = nearest, tie towards +inf:
+ * compiler/torq/Dialect/TorqHW/TorqHWAttrs.td:123-136, default for
+ * EasyKernel lowerings compiler/torq/Serialization/DescGen.cpp:271-291.
+ * t0 is an int32 add (two's-complement wrap here; callers keep it in range).
+ */
+int64_t torq_act_rescale_clamp(int32_t acc, int32_t bias, int32_t scale, const torq_requant_t *rq) {
+    int32_t t0 = (int32_t)((uint32_t)acc + (uint32_t)bias);
+    int64_t t1 = (int64_t)t0 * (int64_t)scale;
+    int sh = rq->shift;
+    int64_t t2 = sh > 0 ? t1 + ((int64_t)1 << (sh - 1)) : t1;
+    int64_t t3 = t2 >> sh; /* arithmetic shift */
+    int64_t t4 = t3 + (int64_t)rq->output_zp;
+    if (t4 < rq->output_min) t4 = rq->output_min;
+    if (t4 > rq->output_max) t4 = rq->output_max;
+    return t4;
+}
+
+static inline void store_elem(void *out, size_t idx, int64_t v, int bytes) {
+    switch (bytes) {
+    case 1: ((int8_t *)out)[idx] = (int8_t)v; break;
+    case 2: ((int16_t *)out)[idx] = (int16_t)v; break;
+    default: ((int32_t *)out)[idx] = (int32_t)v; break;
+    }
+}
+
+static int bad_out_bytes(int b) { return !(b == 1 || b == 2 || b == 4); }
+
+/* Strides (in elements) of a 4-D activation tensor for the chosen layout. */
+typedef struct {
+    size_t n, c, h, w;
+} strides4_t;
+
+static strides4_t act_strides(int layout, int C, int H, int W) {
+    strides4_t s;
+    if (layout == TORQ_LAYOUT_NHWC) {
+        s.c = 1;
+        s.w = (size_t)C;
+        s.h = (size_t)W * C;
+        s.n = (size_t)H * W * C;
+    } else {
+        s.w = 1;
+        s.h = (size_t)W;
+        s.c = (size_t)H * W;
+        s.n = (size_t)C * H * W;
+    }
+    return s;
+}
+
+static int out_dim(int in, int k, int64_t p0, int64_t p1, int64_t stride) {
+    int64_t span = (int64_t)in + p0 + p1 - k;
+    if (span < 0 || stride <= 0) return 0;
+    return (int)(span / stride) + 1;
+}
+
+/*
+ * torq_hl.conv2d -- signature compiler/torq/Dialect/TorqHL/TorqHLOps.td:119-143;
+ * executed loop nest compiler/torq/Conversions/TorqHLToTorqHW/Conv2DToHw.cpp:150-186:
+ * for every output pixel and output channel, accumulate over (ic, kh, kw) the
+ * product of the padded input and the weight, then rescaleClamp with the
+ * channel's (bias, scale).  Padding value is input_zp (Conv2DToHw.cpp:117-121).
+ */
+int torq_conv2d(const int8_t *input, const int8_t *weights, const int32_t *scale_bias, void *out,
+                int N, int C, int H, int W, int O, int KH, int KW, const int64_t pad[4],
+                const int64_t stride[2], int32_t input_zp, const torq_requant_t *rq, int layout,
+                int out_elem_bytes) {
+    if (bad_out_bytes(out_elem_bytes)) return -1;
+    const int64_t pl = pad[0], pr = pad[1], pt = pad[2], pb = pad[3];
+    const int64_t sh = stride[0], sw = stride[1];
+    const int OH = out_dim(H, KH, pt, pb, sh), OW = out_dim(W, KW, pl, pr, sw);
+    const strides4_t is = act_strides(layout, C, H, W);
+    const strides4_t os = act_strides(layout, O, OH, OW);
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int n = 0; n < N; n++) {
+        for (int oy = 0; oy < OH; oy++) {
+            for (int ox = 0; ox < OW; ox++) {
+                for (int o = 0; o < O; o++) {
+                    int32_t acc = 0;
+                    for (int kh = 0; kh < KH; kh++) {
+                        const int64_t iy = (int64_t)oy * sh - pt + kh;
+                        for (int kw = 0; kw < KW; kw++) {
+                            const int64_t ix = (int64_t)ox * sw - pl + kw;
+                            const int inside = iy >= 0 && iy < H && ix >= 0 && ix < W;
+                            const int8_t *wp = weights + (((size_t)o * C) * KH + kh) * KW + kw;
+                            const size_t wstep = (size_t)KH * KW;
+                            if (inside) {
+                                const int8_t *ip = input + n * is.n + (size_t)iy * is.h + (size_t)ix * is.w;
+                                for (int ic = 0; ic < C; ic++) {
+                                    acc += (int32_t)ip[ic * is.c] * (int32_t)wp[ic * wstep];
+                                }
+                            } else {
+                                for (int ic = 0; ic < C; ic++) {
+                                    acc += input_zp * (int32_t)wp[ic * wstep];
+                                }
+                            }
+                        }
+                    }
+                    int64_t q = torq_act_rescale_clamp(acc, scale_bias[2 * o], scale_bias[2 * o + 1], rq);
+                    store_elem(out, n * os.n + (size_t)o * os.c + (size_t)oy * os.h + (size_t)ox * os.w, q,
+                               out_elem_bytes);
+                }
+            }
+        }
+    }
+    return 0;
+}
+
+/*
+ * torq_hl.depthwise_conv2d -- signature TorqHLOps.td:145-170; weights C x 1 x KH x KW
+ * (compiler/torq/Conversions/LinalgToTorqHL/Conv2DPattern.cpp:404-424); executed
+ * compiler/torq/Conversions/TorqHLToTorqHW/DWToHw.cpp:223-251.
+ */
+int torq_depthwise_conv2d(const int8_t *input, const int8_t *weights, const int32_t *scale_bias,
+                          void *out, int N, int C, int H, int W, int KH, int KW,
+                          const int64_t pad[4], const int64_t stride[2], int32_t input_zp,
+                          const torq_requant_t *rq, int layout, int out_elem_bytes) {
+    if (bad_out_bytes(out_elem_bytes)) return -1;
+    const int64_t pl = pad[0], pr = pad[1], pt = pad[2], pb = pad[3];
+    const int64_t sh = stride[0], sw = stride[1];
+    const int OH = out_dim(H, KH, pt, pb, sh), OW = out_dim(W, KW, pl, pr, sw);
+    const strides4_t is = act_strides(layout, C, H, W);
+    const strides4_t os = act_strides(layout, C, OH, OW);
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int n = 0; n < N; n++) {
+        for (int oy = 0; oy < OH; oy++) {
+            for (int ox = 0; ox < OW; ox++) {
+                for (int c = 0; c < C; c++) {
+                    int32_t acc = 0;
+                    for (int kh = 0; kh < KH; kh++) {
+                        const int64_t iy = (int64_t)oy * sh - pt + kh;
+                        for (int kw = 0; kw < KW; kw++) {
+                            const int64_t ix = (int64_t)ox * sw - pl + kw;
+                            int32_t x = input_zp;
+                            if (iy >= 0 && iy < H && ix >= 0 && ix < W) {
+                                x = input[n * is.n + (size_t)c * is.c + (size_t)iy * is.h + (size_t)ix * is.w];
+                            }
+                            acc += x * (int32_t)weights[((size_t)c * KH + kh) * KW + kw];
+                        }
+                    }
+                    int64_t q = torq_act_rescale_clamp(acc, scale_bias[2 * c], scale_bias[2 * c + 1], rq);
+                    store_elem(out, n * os.n + (size_t)c * os.c + (size_t)oy * os.h + (size_t)ox * os.w, q,
+                               out_elem_bytes);
+                }
+            }
+        }
+    }
+    return 0;
+}
+
+/*
+ * torq_hl.fully_connected -- signature TorqHLOps.td:172-190; weights [N(out), K(in)]
+ * (compiler/torq/Conversions/LinalgToTorqHL/Conv2DMatmulPattern.cpp:121-125);
+ * executed compiler/torq/Conversions/TorqHLToTorqHW/FCToHw.cpp:55-76:
+ * acc[m][n] = sum_k x[m][k] * w[n][k], rescaleClamp with pair n.
+ */
+int torq_fully_connected(const int8_t *input, const int8_t *weights, const int32_t *scale_bias,
+                         void *out, int M, int K, int N, const torq_requant_t *rq,
+                         int out_elem_bytes) {
+    if (bad_out_bytes(out_elem_bytes)) return -1;
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int m = 0; m < M; m++) {
+        for (int n = 0; n < N; n++) {
+            const int8_t *x = input + (size_t)m * K;
+            const int8_t *w = weights + (size_t)n * K;
+            int32_t acc = 0;
+            for (int k = 0; k < K; k++) {
+                acc += (int32_t)x[k] * (int32_t)w[k];
+            }
+            int64_t q = torq_act_rescale_clamp(acc, scale_bias[2 * n], scale_bias[2 * n + 1], rq);
+            store_elem(out, (size_t)m * N + n, q, out_elem_bytes);
+        }
+    }
+    return 0;
+}
+
+/*
+ * torq_hl.matmul -- signature TorqHLOps.td:85-99; executed
+ * compiler/torq/Conversions/TorqHLToTorqHW/MatMulPattern.cpp:66-86: batch
+ * broadcast allowed, ONE (bias, scale) pair loaded before the loops (:66).
+ */
+int torq_matmul(const int8_t *input1, const int8_t *input2, const int32_t *scale_bias, void *out,
+                int B, int M, int K, int N, int bcast1, int bcast2, const torq_requant_t *rq,
+                int out_elem_bytes) {
+    if (bad_out_bytes(out_elem_bytes)) return -1;
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int b = 0; b < B; b++) {
+        for (int m = 0; m < M; m++) {
+            const int8_t *a = input1 + (bcast1 ? 0 : (size_t)b * M * K) + (size_t)m * K;
+            const int8_t *bm = input2 + (bcast2 ? 0 : (size_t)b * K * N);
+            for (int n = 0; n < N; n++) {
+                int32_t acc = 0;
+                for (int k = 0; k < K; k++) {
+                    acc += (int32_t)a[k] * (int32_t)bm[(size_t)k * N + n];
+                }
+                int64_t q = torq_act_rescale_clamp(acc, scale_bias[0], scale_bias[1], rq);
+                store_elem(out, ((size_t)b * M + m) * N + n, q, out_elem_bytes);
+            }
+        }
+    }
+    return 0;
+}
+
+/*
+ * torq_hl.maxpool2d -- signature TorqHLOps.td:435-453; created
+ * compiler/torq/Conversions/LinalgToTorqHL/PoolingPattern.cpp:199-236 (pad value
+ * becomes input_zp, output_min/max = element type range); executed
+ * compiler/torq/Conversions/TorqHLToTorqHW/MaxPool2dToHw.cpp:28-333 (ALU MAX
+ * accumulate, ACT load: no rescale).
+ */
+int torq_maxpool2d(const int8_t *input, int8_t *out, int N, int C, int H, int W, int KH, int KW,
+                   const int64_t pad[4], const int64_t stride[2], int32_t input_zp,
+                   int32_t output_min, int32_t output_max, int layout) {
+    const int64_t pl = pad[0], pr = pad[1], pt = pad[2], pb = pad[3];
+    const int64_t sh = stride[0], sw = stride[1];
+    const int OH = out_dim(H, KH, pt, pb, sh), OW = out_dim(W, KW, pl, pr, sw);
+    const strides4_t is = act_strides(layout, C, H, W);
+    const strides4_t os = act_strides(layout, C, OH, OW);
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int n = 0; n < N; n++) {
+        for (int oy = 0; oy < OH; oy++) {
+            for (int ox = 0; ox < OW; ox++) {
+                for (int c = 0; c < C; c++) {
+                    int32_t best = INT32_MIN;
+                    for (int kh = 0; kh < KH; kh++) {
+                        const int64_t iy = (int64_t)oy * sh - pt + kh;
+                        for (int kw = 0; kw < KW; kw++) {
+                            const int64_t ix = (int64_t)ox * sw - pl + kw;
+                            int32_t x = input_zp;
+                            if (iy >= 0 && iy < H && ix >= 0 && ix < W) {
+                                x = input[n * is.n + (size_t)c * is.c + (size_t)iy * is.h + (size_t)ix * is.w];
+                            }
+                            if (x > best) best = x;
+                        }
+                    }
+                    if (best < output_min) best = output_min;
+                    if (best > output_max) best = output_max;
+                    out[n * os.n + (size_t)c * os.c + (size_t)oy * os.h + (size_t)ox * os.w] = (int8_t)best;
+                }
+            }
+        }
+    }
+    return 0;
+}
+
+/*
+ * torq_hl.avg_pool2d -- signature TorqHLOps.td:192-208; global only
+ * (compiler/torq/Conversions/LinalgToTorqHL/PoolingPattern.cpp:289-291); executed
+ * compiler/torq/Conversions/TorqHLToTorqHW/AvgpoolPattern.cpp:67-83: per channel,
+ * scalar-product-accumulate the whole frame with the single weight, then
+ * rescaleClamp with bias/scale pair 0 (:58-59).  Input NHWC (:36).
+ */
+int torq_avg_pool2d(const int8_t *input, int8_t weight, const int32_t *scale_bias, int8_t *out,
+                    int N, int H, int W, int C, const torq_requant_t *rq) {
+    const size_t frame = (size_t)H * W;
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int n = 0; n < N; n++) {
+        for (int c = 0; c < C; c++) {
+            int32_t acc = 0;
+            const int8_t *p = input + (size_t)n * frame * C + c;
+            for (size_t u = 0; u < frame; u++) {
+                acc += (int32_t)p[u * C] * (int32_t)weight;
+            }
+            out[(size_t)n * C + c] = (int8_t)torq_act_rescale_clamp(acc, scale_bias[0], scale_bias[1], rq);
+        }
+    }
+    return 0;
+}
+
+/*
+ * torq_hl.add -- signature TorqHLOps.td:48-69; executed
+ * compiler/torq/Conversions/TorqHLToTorqHW/AddPattern.cpp:262-281:
+ * acc = in1*w[0] + in2*w[1] (int16 weights), rescaleClamp with one pair.
+ */
+int torq_add(const int8_t *input1, const int8_t *input2, const int16_t weights[2],
+             const int32_t scale_bias[2], int8_t *out, size_t count, const torq_requant_t *rq) {
+    const int32_t w0 = weights[0], w1 = weights[1];
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < count; i++) {
+        int32_t acc = (int32_t)input1[i] * w0 + (int32_t)input2[i] * w1;
+        out[i] = (int8_t)torq_act_rescale_clamp(acc, scale_bias[0], scale_bias[1], rq);
+    }
+    return 0;
+}
+
+/* ---- R2 ---- */
+
+/* compiler/torq/Utils/ConversionUtils.cpp:122-141 (per_channel_sum). */
+void torq_per_channel_sum(const int8_t *weights, int channels, int per_channel, int64_t *sums) {
+    for (int o = 0; o < channels; o++) {
+        int64_t s = 0;
+        for (int i = 0; i < per_channel; i++) s += weights[(size_t)o * per_channel + i];
+        sums[o] = s;
+    }
+}
+
+/*
+ * shift_factor = min_c shift[c]: compiler/torq/Conversions/LinalgToTorqHL/PatternUtils.cpp:3230-3283;
+ * scale[c] = multiplier[c] >> (shift[c] - shift_factor) (arith.shrsi): PatternUtils.cpp:3536-3548;
+ * bias[c] = tosa_bias[c] - weight_sum[c] * input_zp: compiler/torq/Utils/ConversionUtils.h:301-329;
+ * interleave [bias, scale]: compiler/torq/Utils/ConversionUtils.cpp:88-103.
+ */
+int32_t torq_derive_scale_bias(const int32_t *multiplier, const int8_t *shift,
+                               const int32_t *tosa_bias, const int64_t *weight_sum,
+                               int32_t input_zp, int channels, int32_t *scale_bias) {
+    int32_t min_shift = INT8_MAX;
+    for (int c = 0; c < channels; c++) {
+        if (shift[c] < min_shift) min_shift = shift[c];
+    }
+    for (int c = 0; c < channels; c++) {
+        int64_t b = (int64_t)(tosa_bias ? tosa_bias[c] : 0) -
+                    (weight_sum ? weight_sum[c] : 0) * (int64_t)input_zp;
+        scale_bias[2 * c] = (int32_t)b;
+        scale_bias[2 * c + 1] = multiplier[c] >> (shift[c] - min_shift);
+    }
+    return min_shift;
+}
+
+/*
+ * compiler/torq/Conversions/LinalgToTorqHL/ElementWiseBinaryPattern.cpp:459-487,
+ * 564-597: S = 2^12, weights = (int16)trunc(m_k * S) (w1 times sign),
+ * bias = -trunc(m0*S*zp0) - sign*trunc(m1*S*zp1), scale = 1, shift 12.
+ * doubleToInt is a C cast: compiler/torq/Utils/TorqUtils.h:55-62.
+ */
+int torq_derive_add_params(double m0, double m1, int32_t zp0, int32_t zp1, int sign,
+                           int16_t weights[2], int32_t scale_bias[2], int32_t *shift_factor) {
+    const int sh = 12;
+    const int scale_factor = 1 << sh;
+    if (m0 * scale_factor > INT16_MAX || m0 * scale_factor < INT16_MIN ||
+        m1 * scale_factor > INT16_MAX || m1 * scale_factor < INT16_MIN) {
+        return -1;
+    }
+    int16_t w0 = (int16_t)(m0 * scale_factor);
+    int32_t b0 = -(int32_t)(m0 * scale_factor * zp0);
+    int16_t w1 = (int16_t)((int16_t)(m1 * scale_factor) * sign);
+    int32_t b1 = -(int32_t)(m1 * scale_factor * zp1) * sign;
+    weights[0] = w0;
+    weights[1] = w1;
+    scale_bias[0] = b0 + b1;
+    scale_bias[1] = 1;
+    *shift_factor = sh;
+    return 0;
+}
+
+/*
+ * compiler/torq/Conversions/LinalgToTorqHL/PoolingPattern.cpp:325-328 (scale =
+ * int32(1.0 * 2^shift / itemsPerChannel), bias = -scInfo.bias) with shift 20
+ * (:598,600); the folded pre-scale subtract constant of a TFLite-origin mean is
+ * H*W*input_zp.
+ */
+void torq_derive_avgpool_params(int H, int W, int32_t input_zp, int32_t scale_bias[2],
+                                int32_t *shift_factor) {
+    const int sh = 20;
+    const int items = H * W;
+    scale_bias[0] = -(items * input_zp);
+    scale_bias[1] = (int32_t)(1.0 * (double)(1 << sh) / items);
+    *shift_factor = sh;
+}

@@ -1,0 +1,152 @@
+"""Test-only numpy interpreter of a dispatch descriptor.
+
+It executes the kernel records of a descriptor the way the GPU kernels are
+specified to (packed weights, split bias/scale, k-table gather, NHWC buffers,
+transposes), so that the emitter's packing and layout decisions can be checked
+against the oracle on a machine without a GPU.  It is not part of the product.
+"""
+import numpy as np
+
+from oracle import oracle as orc
+
+REF = np.dtype([("space", "<u4"), ("index", "<u4"), ("offset", "<u8")])
+HEADER = np.dtype([("magic", "<u4"), ("version", "<u4"), ("arch", "<u4"), ("flags", "<u4"),
+                   ("op_count", "<u4"), ("binding_count", "<u4"), ("temp_count", "<u4"), ("const_count", "<u4"),
+                   ("ops_offset", "<u8"), ("bindings_offset", "<u8"), ("temps_offset", "<u8"),
+                   ("consts_offset", "<u8"), ("data_offset", "<u8"), ("total_size", "<u8")])
+_I32 = ["out_dtype", "input_zp", "output_zp", "output_min", "output_max", "shift",
+        "N", "H", "W", "C", "OH", "OW", "OC", "KH", "KW", "SH", "SW", "PL", "PR", "PT", "PB",
+        "M", "K", "Kp", "Nn", "Np", "w0", "w1", "bias0", "scale0", "TB", "TR", "TS", "r0", "r1", "r2"]
+OP = np.dtype([("kind", "<u4"), ("variant", "<u4"), ("loader", "<u4"), ("gran", "<u4")] +
+              [(n, "<i4") for n in _I32] +
+              [(n, REF) for n in ["in0", "in1", "weights", "bias", "scale", "table", "out"]])
+BINDING = np.dtype([("id", "<u4"), ("flags", "<u4"), ("size", "<u8")])
+TEMP = np.dtype([("size", "<u8")])
+CONST = np.dtype([("offset", "<u8"), ("size", "<u8")])
+
+K_TRANSPOSE, K_IGEMM, K_FC_SKINNY, K_DW, K_MAXPOOL, K_AVGPOOL, K_ADD = 1, 2, 3, 4, 5, 6, 7
+OUT_NP = {1: np.int8, 2: np.int16, 3: np.int32}
+
+
+class Descriptor:
+    def __init__(self, blob):
+        self.blob = np.frombuffer(blob, dtype=np.uint8)
+        self.header = np.frombuffer(blob, dtype=HEADER, count=1)[0]
+        h = self.header
+        assert h["magic"] == 0x50494854 and h["total_size"] == len(blob)
+        self.ops = np.frombuffer(blob, dtype=OP, count=int(h["op_count"]), offset=int(h["ops_offset"]))
+        self.bindings = np.frombuffer(blob, dtype=BINDING, count=int(h["binding_count"]), offset=int(h["bindings_offset"]))
+        self.temps = np.frombuffer(blob, dtype=TEMP, count=int(h["temp_count"]), offset=int(h["temps_offset"]))
+        self.consts = np.frombuffer(blob, dtype=CONST, count=int(h["const_count"]), offset=int(h["consts_offset"]))
+
+    def const_bytes(self, index):
+        c = self.consts[index]
+        start = int(self.header["data_offset"] + c["offset"])
+        return self.blob[start:start + int(c["size"])]
+
+
+def _requant_vec(acc, bias, scale, shift, zp, mn, mx):
+    t0 = (acc.astype(np.int64) + bias.astype(np.int64))
+    t0 = ((t0 + (1 << 31)) % (1 << 32)) - (1 << 31)  # int32 wrap
+    t1 = t0 * scale.astype(np.int64)
+    if shift > 0:
+        t1 = t1 + (1 << (shift - 1))
+    t3 = t1 >> shift
+    return np.clip(t3 + zp, mn, mx)
+
+
+def run(blob, binding_arrays):
+    """Executes the descriptor on numpy arrays (one per binding, modified in place for outputs)."""
+    d = Descriptor(blob)
+    bufs = {1: [a.reshape(-1).view(np.uint8) for a in binding_arrays],
+            2: [np.zeros(int(t["size"]), dtype=np.uint8) for t in d.temps],
+            3: [d.const_bytes(i) for i in range(len(d.consts))]}
+
+    def view(ref, nbytes):
+        b = bufs[int(ref["space"])][int(ref["index"])]
+        off = int(ref["offset"])
+        assert off + nbytes <= b.size, "operand runs past its buffer"
+        return b[off:off + nbytes]
+
+    for op in d.ops:
+        kind = int(op["kind"])
+        sh, zp, mn, mx = int(op["shift"]), int(op["output_zp"]), int(op["output_min"]), int(op["output_max"])
+        if kind == K_TRANSPOSE:
+            B, R, S = int(op["TB"]), int(op["TR"]), int(op["TS"])
+            src = view(op["in0"], B * R * S).reshape(B, R, S)
+            view(op["out"], B * R * S)[:] = np.ascontiguousarray(src.transpose(0, 2, 1)).reshape(-1)
+        elif kind in (K_IGEMM, K_FC_SKINNY):
+            M, K, Kp, N, Np = (int(op[k]) for k in ["M", "K", "Kp", "Nn", "Np"])
+            Wp = view(op["weights"], Np * Kp).view(np.int8).reshape(Np, Kp).astype(np.int64)
+            bias = view(op["bias"], Np * 4).view(np.int32)
+            scale = view(op["scale"], Np * 4).view(np.int32)
+            if kind == K_FC_SKINNY or int(op["loader"]) == 0:
+                A = np.zeros((M, Kp), dtype=np.int64)
+                A[:, :K] = view(op["in0"], M * K).view(np.int8).reshape(M, K)
+            else:
+                Nimg, H, W, C = (int(op[k]) for k in ["N", "H", "W", "C"])
+                OH, OW, SH, SW, PT, PL = (int(op[k]) for k in ["OH", "OW", "SH", "SW", "PT", "PL"])
+                g = int(op["gran"])
+                x = view(op["in0"], Nimg * H * W * C).view(np.int8).reshape(Nimg, H, W, C)
+                tab = view(op["table"], Kp // g * 4).view(np.uint32)
+                A = np.zeros((Nimg, OH, OW, Kp), dtype=np.int64)
+                oy = np.arange(OH)[:, None] * SH - PT
+                ox = np.arange(OW)[None, :] * SW - PL
+                for e, ent in enumerate(tab):
+                    ent = int(ent)
+                    if ent & 0x80000000:
+                        continue
+                    kh, kw, ci = (ent >> 24) & 0x7f, (ent >> 16) & 0xff, ent & 0xffff
+                    iy, ix = oy + kh, ox + kw
+                    inside = (iy >= 0) & (iy < H) & (ix >= 0) & (ix < W)
+                    iyc, ixc = np.clip(iy, 0, H - 1), np.clip(ix, 0, W - 1)
+                    vals = x[:, iyc, ixc, ci:ci + g].astype(np.int64)  # N,OH,OW,g
+                    vals = np.where(inside[None, :, :, None], vals, int(op["input_zp"]))
+                    A[..., e * g:(e + 1) * g] = vals
+                A = A.reshape(M, Kp)
+            acc = A @ Wp.T  # M x Np
+            q = _requant_vec(acc[:, :N], bias[None, :N], scale[None, :N], sh, zp, mn, mx)
+            odt = OUT_NP[int(op["out_dtype"])]
+            out = view(op["out"], M * N * np.dtype(odt).itemsize).view(odt)
+            out[:] = q.astype(odt).reshape(-1)
+        elif kind == K_DW:
+            Nimg, H, W, C, OH, OW = (int(op[k]) for k in ["N", "H", "W", "C", "OH", "OW"])
+            KH, KW = int(op["KH"]), int(op["KW"])
+            x = view(op["in0"], Nimg * H * W * C).view(np.int8).reshape(Nimg, H, W, C)
+            wpk = view(op["weights"], KH * KW * C).view(np.int8).reshape(KH, KW, C)
+            sb = np.empty(2 * C, dtype=np.int32)
+            sb[0::2] = view(op["bias"], C * 4).view(np.int32)
+            sb[1::2] = view(op["scale"], C * 4).view(np.int32)
+            w = np.ascontiguousarray(wpk.transpose(2, 0, 1))[:, None]
+            res = orc.depthwise_conv2d(x, w, sb, input_zp=int(op["input_zp"]), output_zp=zp, output_min=mn,
+                                       output_max=mx, shift_factor=sh,
+                                       pad=[int(op["PL"]), int(op["PR"]), int(op["PT"]), int(op["PB"])],
+                                       stride=[int(op["SH"]), int(op["SW"])], layout=orc.NHWC)
+            assert res.shape == (Nimg, OH, OW, C)
+            view(op["out"], res.size)[:] = res.reshape(-1).view(np.uint8)
+        elif kind == K_MAXPOOL:
+            Nimg, H, W, C, OH, OW = (int(op[k]) for k in ["N", "H", "W", "C", "OH", "OW"])
+            x = view(op["in0"], Nimg * H * W * C).view(np.int8).reshape(Nimg, H, W, C)
+            res = orc.maxpool2d(x, input_zp=int(op["input_zp"]), output_min=mn, output_max=mx,
+                                stride=[int(op["SH"]), int(op["SW"])],
+                                pad=[int(op["PL"]), int(op["PR"]), int(op["PT"]), int(op["PB"])],
+                                kernel=[int(op["KH"]), int(op["KW"])], layout=orc.NHWC)
+            assert res.shape == (Nimg, OH, OW, C)
+            view(op["out"], res.size)[:] = res.reshape(-1).view(np.uint8)
+        elif kind == K_AVGPOOL:
+            Nimg, H, W, C = (int(op[k]) for k in ["N", "H", "W", "C"])
+            x = view(op["in0"], Nimg * H * W * C).view(np.int8).reshape(Nimg, H, W, C)
+            res = orc.avg_pool2d(x, np.array([op["bias0"], op["scale0"]], dtype=np.int32), output_zp=zp,
+                                 output_min=mn, output_max=mx, shift_factor=sh, weight=int(op["w0"]))
+            view(op["out"], res.size)[:] = res.reshape(-1).view(np.uint8)
+        elif kind == K_ADD:
+            n = int(op["C"])
+            a = view(op["in0"], n).view(np.int8)
+            b = view(op["in1"], n).view(np.int8)
+            res = orc.add(a, b, np.array([op["w0"], op["w1"]], dtype=np.int16),
+                          np.array([op["bias0"], op["scale0"]], dtype=np.int32), output_zp=zp, output_min=mn,
+                          output_max=mx, shift_factor=sh)
+            view(op["out"], n)[:] = res.view(np.uint8)
+        else:
+            raise AssertionError("unknown kernel kind %d" % kind)
+    return d

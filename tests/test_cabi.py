@@ -1,0 +1,59 @@
+"""The C-ABI shared library loads and exports every symbol include/thip.h declares (no compute here)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from torq_compiler_amd import ThipError, runtime
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "thip.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(thip_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(runtime.LIB_PATH)
+    names = declared_symbols()
+    assert len(names) >= 35
+    for name in names:
+        assert hasattr(lib, name), "libthip.so does not export %s" % name
+    assert sorted(runtime.EXPORTED_SYMBOLS) == names, "runtime.EXPORTED_SYMBOLS is out of date with include/thip.h"
+
+
+def test_version_and_status_message():
+    lib = runtime.lib()
+    assert lib.thip_descriptor_version() == 1
+    assert lib.thip_version() >= 1
+    p = ctypes.c_void_p()
+    assert lib.thip_program_create(ctypes.byref(p)) == runtime.OK
+    blob, size = ctypes.c_void_p(), ctypes.c_size_t()
+    code = lib.thip_program_serialize(p, ctypes.byref(blob), ctypes.byref(size))
+    assert code == runtime.INVALID_ARGUMENT
+    assert b"no ops" in lib.thip_status_message()
+    lib.thip_program_destroy(p)
+
+
+def test_null_arguments_are_rejected_not_dereferenced():
+    lib = runtime.lib()
+    assert lib.thip_program_create(None) == runtime.INVALID_ARGUMENT
+    assert lib.thip_executable_run(None, None) == runtime.INVALID_ARGUMENT
+    assert lib.thip_executable_create(None, None, 0, None, 0, None) == runtime.INVALID_ARGUMENT
+    out = ctypes.c_void_p()
+    assert lib.thip_executable_create(None, None, 0, None, 0, ctypes.byref(out)) == runtime.INVALID_ARGUMENT
+    assert lib.thip_device_synchronize(None) == runtime.INVALID_ARGUMENT
+
+
+def test_device_create_without_gpu_is_unavailable_or_ok():
+    """No GPU in the build container: UNAVAILABLE with a message; on a GPU box: a gfx950 device."""
+    try:
+        dev = runtime.Device(0)
+    except ThipError as e:
+        assert e.code == runtime.UNAVAILABLE
+        return
+    assert dev.name() == "gfx950"
+    dev.close()

@@ -1,0 +1,197 @@
+"""Host logic: the emitter's packing, k-table, scale_bias split and layout folding, checked on the CPU.
+
+The descriptor is executed by the numpy interpreter in desc_interp.py (test-only) and compared
+bit-for-bit with the oracle.  Geometries follow the ones the reference's own tests exercise
+(tests/models/keras_conv.py, keras_pointwise.py, keras_depthwise.py, keras_fc.py, keras_pooling.py,
+tests/testdata/tosa_ops/*.mlir).
+"""
+import numpy as np
+import pytest
+
+import desc_interp
+from helpers import assert_bit_exact, oracle_eval
+from oracle import oracle as orc
+from torq_compiler_amd import Program, ThipError, runtime, workloads as w
+
+
+def interp(wl):
+    blob = wl.program.serialize()
+    outs = [np.zeros(s, dtype=dt) for s, dt in wl.outputs]
+    d = desc_interp.run(blob, list(wl.inputs) + outs)
+    return outs, d
+
+
+CONV = [
+    dict(N=1, H=8, W=8, C=3, O=4, KH=3, KW=3),
+    dict(N=1, H=8, W=8, C=4, O=8, KH=2, KW=3, pad=(0, 0, 0, 0)),
+    dict(N=1, H=12, W=12, C=1, O=4, KH=6, KW=6, stride=(2, 2), pad=(2, 2, 2, 2)),
+    dict(N=1, H=18, W=76, C=24, O=7, KH=5, KW=2, pad=(0, 1, 2, 2)),
+    dict(N=1, H=9, W=9, C=8, O=16, KH=1, KW=1, stride=(2, 2), pad=(0, 0, 0, 0)),
+    dict(N=2, H=5, W=5, C=16, O=29, KH=3, KW=5, stride=(3, 4), pad=(2, 2, 1, 1)),
+    dict(N=1, H=1, W=1, C=1024, O=10, KH=1, KW=1, pad=(0, 0, 0, 0)),
+    dict(N=1, H=16, W=16, C=32, O=64, KH=3, KW=3),
+]
+
+
+@pytest.mark.parametrize("kw", CONV)
+@pytest.mark.parametrize("nhwc", [True, False])
+def test_conv2d_descriptor(kw, nhwc):
+    wl = w.conv2d_workload(realistic=True, nhwc=nhwc, output_min=-128, **kw)
+    outs, d = interp(wl)
+    assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)
+    kinds = [int(o["kind"]) for o in d.ops]
+    C, HW = kw["C"], kw["H"] * kw["W"]
+    if nhwc or C == 1 or HW == 1:
+        assert kinds.count(desc_interp.K_TRANSPOSE) <= (0 if nhwc else 1)
+    else:
+        assert kinds[0] == desc_interp.K_TRANSPOSE and kinds[1] == desc_interp.K_IGEMM
+
+
+@pytest.mark.parametrize("kw", [
+    dict(N=1, H=6, W=42, C=16), dict(N=1, H=6, W=6, C=2, pad=(0, 0, 0, 0)), dict(N=1, H=13, W=15, C=8, stride=(1, 1), pad=(1, 1, 1, 1)),
+    dict(N=1, H=27, W=27, C=128, KH=4, KW=4, stride=(2, 2), pad=(1, 2, 1, 2)), dict(N=2, H=21, W=21, C=5, stride=(2, 2), pad=(1, 1, 1, 1)),
+])
+@pytest.mark.parametrize("nhwc", [True, False])
+def test_depthwise_descriptor(kw, nhwc):
+    wl = w.depthwise_workload(nhwc=nhwc, **kw)
+    outs, _ = interp(wl)
+    assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)
+
+
+@pytest.mark.parametrize("mkn", [(1, 1, 1), (1, 61, 1991), (4, 1024, 1024), (1, 2000, 97), (16, 3, 7), (17, 128, 70), (130, 700, 500)])
+def test_fully_connected_descriptor(mkn):
+    wl = w.fully_connected_workload(*mkn, realistic=True)
+    outs, d = interp(wl)
+    assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)
+    M, K, _ = mkn
+    want_kind = desc_interp.K_FC_SKINNY if (M <= 16 and K % 16 == 0) else desc_interp.K_IGEMM
+    assert int(d.ops[0]["kind"]) == want_kind
+
+
+@pytest.mark.parametrize("kw", [dict(H=8, W=8, C=4), dict(H=32, W=32, C=64, kernel=(3, 3), pad=(1, 1, 1, 1)), dict(H=10, W=10, C=4, kernel=(5, 5), stride=(1, 1)),
+                                dict(H=10, W=10, C=4, kernel=(1, 3), stride=(1, 3), pad=(0, 2, 0, 0), input_zp=-7)])
+@pytest.mark.parametrize("nhwc", [True, False])
+def test_maxpool_descriptor(kw, nhwc):
+    wl = w.maxpool_workload(nhwc=nhwc, **kw)
+    outs, _ = interp(wl)
+    assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)
+
+
+def test_avgpool_and_add_descriptor():
+    for wl in (w.avgpool_workload(N=2, C=128), w.avgpool_workload(N=1, H=12, W=8, C=37), w.add_workload(), w.add_workload(N=1, H=4, W=4, C=1)):
+        outs, _ = interp(wl)
+        assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)
+
+
+def _chain_program(nchw_bindings):
+    """conv(1x1 expand) -> depthwise -> conv(1x1 project) -> add residual -> transpose -> avg_pool -> fc,
+    all declared N,C,H,W like the reference emits them."""
+    rng = np.random.default_rng(77)
+    N, C, H, W, E = 2, 16, 10, 10, 48
+    x = rng.integers(-128, 128, size=(N, C, H, W)).astype(np.int8)
+    prm = {}
+
+    def conv_params(O, wshape, zp):
+        wt = rng.integers(-127, 128, size=wshape).astype(np.int8)
+        mult, shift = w.random_requant(rng, O, True)
+        sb, sf = w.derive_scale_bias(mult, (shift - 3).astype(np.int8), rng.integers(-2000, 2000, size=O), wt, zp)
+        return wt, sb, sf
+
+    prm["w1"], prm["sb1"], prm["sf1"] = conv_params(E, (E, C, 1, 1), -3)
+    prm["wd"], prm["sbd"], prm["sfd"] = conv_params(E, (E, 1, 3, 3), 2)
+    prm["w2"], prm["sb2"], prm["sf2"] = conv_params(C, (C, E, 1, 1), -1)
+    prm["aw"], prm["asb"], prm["asf"] = w.add_params(0.6, 0.9, -3, 4)
+    prm["psb"] = np.array([-(H * W * 1), (1 << 20) // (H * W)], dtype=np.int32)
+    prm["wf"], prm["sbf"], prm["sff"] = conv_params(10, (10, C), 0)
+
+    p = Program()
+    xin = p.binding(0, x.shape)
+    t1 = p.conv2d(xin, prm["w1"], prm["sb1"], input_zp=-3, output_zp=2, output_min=-128, output_max=127, shift_factor=prm["sf1"], pad=(0, 0, 0, 0), stride=(1, 1))
+    t2 = p.depthwise_conv2d(t1, prm["wd"], prm["sbd"], input_zp=2, output_zp=-1, output_min=-128, output_max=127, shift_factor=prm["sfd"], pad=(1, 1, 1, 1), stride=(1, 1))
+    t3 = p.conv2d(t2, prm["w2"], prm["sb2"], input_zp=-1, output_zp=4, output_min=-128, output_max=127, shift_factor=prm["sf2"], pad=(0, 0, 0, 0), stride=(1, 1))
+    t4 = p.add(xin, t3, prm["aw"], prm["asb"], output_zp=1, output_min=-128, output_max=127, shift_factor=prm["asf"])
+    t5 = p.transpose(t4, (0, 2, 3, 1))
+    t6 = p.avg_pool2d(t5, np.array([1], dtype=np.int8), prm["psb"], input_zp=1, output_zp=0, output_min=-128, output_max=127, shift_factor=20)
+    out = p.binding(1, (N, 10))
+    p.fully_connected(t6, prm["wf"], prm["sbf"], init=out, output_zp=3, output_min=-128, output_max=127, shift_factor=prm["sff"])
+    aux = p.binding(2, (N, C, H, W))  # also export the residual sum, N,C,H,W
+    p.add(xin, t3, prm["aw"], prm["asb"], init=aux, output_zp=1, output_min=-128, output_max=127, shift_factor=prm["asf"])
+
+    # oracle, literal N,C,H,W
+    o1 = orc.conv2d(x, prm["w1"], prm["sb1"], input_zp=-3, output_zp=2, output_min=-128, output_max=127, shift_factor=prm["sf1"], pad=(0, 0, 0, 0), stride=(1, 1))
+    o2 = orc.depthwise_conv2d(o1, prm["wd"], prm["sbd"], input_zp=2, output_zp=-1, output_min=-128, output_max=127, shift_factor=prm["sfd"], pad=(1, 1, 1, 1), stride=(1, 1))
+    o3 = orc.conv2d(o2, prm["w2"], prm["sb2"], input_zp=-1, output_zp=4, output_min=-128, output_max=127, shift_factor=prm["sf2"], pad=(0, 0, 0, 0), stride=(1, 1))
+    o4 = orc.add(x, o3, prm["aw"], prm["asb"], output_zp=1, output_min=-128, output_max=127, shift_factor=prm["asf"])
+    o5 = np.ascontiguousarray(o4.transpose(0, 2, 3, 1))
+    o6 = orc.avg_pool2d(o5, prm["psb"], output_zp=0, output_min=-128, output_max=127, shift_factor=20)
+    o7 = orc.fully_connected(o6.reshape(N, C), prm["wf"], prm["sbf"], output_zp=3, output_min=-128, output_max=127, shift_factor=prm["sff"])
+    return p, x, o7, o4
+
+
+def test_multi_op_program_keeps_intermediates_nhwc():
+    p, x, want_fc, want_sum = _chain_program(True)
+    blob = p.serialize()
+    out = np.zeros(want_fc.shape, dtype=np.int8)
+    aux = np.zeros(want_sum.shape, dtype=np.int8)
+    d = desc_interp.run(blob, [x, out, aux])
+    assert_bit_exact(out, want_fc, "chain fc")
+    assert_bit_exact(aux, want_sum, "chain residual")
+    kinds = [int(o["kind"]) for o in d.ops]
+    # one transpose brings the N,C,H,W binding in (shared by conv and both adds would be ideal; each
+    # consumer of the literal binding converts it), one takes the exported sum out; none in between.
+    first_igemm = kinds.index(desc_interp.K_IGEMM)
+    between = kinds[first_igemm:kinds.index(desc_interp.K_AVGPOOL)]
+    assert desc_interp.K_TRANSPOSE not in [k for k in between if k != desc_interp.K_ADD][0:3]
+    assert kinds[-1] == desc_interp.K_TRANSPOSE
+
+
+def test_rejects_what_the_path_does_not_cover():
+    def expect(code, build):
+        p = Program()
+        with pytest.raises(ThipError) as e:
+            build(p)
+            p.serialize()
+        assert e.value.code == code, e.value
+
+    x8 = np.zeros((4, 3, 3, 3), dtype=np.int8)
+    sb = np.zeros(8, dtype=np.int32)
+    common = dict(input_zp=0, output_zp=0, output_min=-128, output_max=127, shift_factor=4, pad=(0, 0, 0, 0), stride=(1, 1))
+    expect(runtime.UNIMPLEMENTED, lambda p: p.conv2d(p.binding(0, (1, 3, 8, 8)), x8, sb, init=p.binding(1, (1, 4, 6, 6)), groups=2, **common))
+    expect(runtime.UNIMPLEMENTED, lambda p: p.conv2d(p.binding(0, (1, 3, 8, 8)), x8, sb, init=p.binding(1, (1, 4, 6, 6)), dilation=(2, 2), **common))
+    expect(runtime.UNIMPLEMENTED, lambda p: p.conv2d(p.binding(0, (1, 3, 8, 8)), x8, sb, init=p.binding(1, (1, 4, 6, 6)), weight_zp=1, **common))
+    expect(runtime.INVALID_ARGUMENT, lambda p: p.conv2d(p.binding(0, (1, 5, 8, 8)), x8, sb, init=p.binding(1, (1, 4, 6, 6)), **common))
+    expect(runtime.INVALID_ARGUMENT, lambda p: p.conv2d(p.binding(0, (1, 3, 8, 8)), x8, sb, init=p.binding(1, (1, 4, 7, 6)), **common))
+    bad = dict(common, shift_factor=64)
+    expect(runtime.INVALID_ARGUMENT, lambda p: p.conv2d(p.binding(0, (1, 3, 8, 8)), x8, sb, init=p.binding(1, (1, 4, 6, 6)), **bad))
+    bad = dict(common, output_zp=40000)
+    expect(runtime.INVALID_ARGUMENT, lambda p: p.conv2d(p.binding(0, (1, 3, 8, 8)), x8, sb, init=p.binding(1, (1, 4, 6, 6)), **bad))
+    bad = dict(common, output_max=300)
+    expect(runtime.INVALID_ARGUMENT, lambda p: p.conv2d(p.binding(0, (1, 3, 8, 8)), x8, sb, init=p.binding(1, (1, 4, 6, 6)), **bad))
+    # weights must be compile-time constants
+    expect(runtime.UNIMPLEMENTED, lambda p: p.conv2d(p.binding(0, (1, 3, 8, 8)), p.binding(2, (4, 3, 3, 3)), sb, init=p.binding(1, (1, 4, 6, 6)), **common))
+    # reading an intermediate that nothing wrote
+    expect(runtime.FAILED_PRECONDITION, lambda p: p.maxpool2d(p.tensor((1, 3, 8, 8)), input_zp=-128, output_min=-128, output_max=127, stride=(2, 2), pad=(0, 0, 0, 0), kernel=(2, 2), init=p.binding(0, (1, 3, 4, 4))))
+    expect(runtime.INVALID_ARGUMENT, lambda p: None)  # empty program
+
+
+def test_descriptor_header_and_format():
+    wl = w.add_workload(N=1, H=2, W=2, C=4)
+    blob = wl.program.serialize()
+    fmt, size = runtime.infer_format(blob)
+    assert fmt == "thip-gfx950" and size == len(blob)
+    d = desc_interp.Descriptor(blob)
+    assert d.header["version"] == runtime.lib().thip_descriptor_version() and d.header["arch"] == 950
+    assert [int(b["flags"]) for b in d.bindings] == [1, 1, 2]  # read, read, written
+    for mutate, code in [((0, b"XXXX"), runtime.INVALID_ARGUMENT), ((4, (99).to_bytes(4, "little")), runtime.UNAVAILABLE),
+                         ((8, (942).to_bytes(4, "little")), runtime.UNAVAILABLE)]:
+        bad = bytearray(blob)
+        bad[mutate[0]:mutate[0] + 4] = mutate[1]
+        with pytest.raises(ThipError) as e:
+            runtime.infer_format(bytes(bad))
+        assert e.value.code == code
+    with pytest.raises(ThipError) as e:
+        runtime.infer_format(blob[:40])
+    assert e.value.code == runtime.INVALID_ARGUMENT
+    with pytest.raises(ThipError) as e:
+        runtime.infer_format(blob[:-1])
+    assert e.value.code == runtime.INVALID_ARGUMENT

@@ -1,0 +1,242 @@
+"""Parity of the HIP kernels with the CPU oracle, through the C-ABI, on a real gfx950.
+
+Bit-exact: every op is integer.  Each case is printed (and flushed) before it touches the GPU so
+that a fault names its case.
+"""
+import sys
+
+import numpy as np
+import pytest
+
+from helpers import assert_bit_exact, oracle_eval, run_on_gpu
+from test_emitter import CONV, _chain_program
+from torq_compiler_amd import Executable, ThipError, runtime, workloads as w
+
+pytestmark = pytest.mark.gpu
+
+
+def announce(*what):
+    print("[gpu-case]", *what, flush=True)
+    sys.stdout.flush()
+
+
+def check(device, wl, via="host", kernel=None):
+    announce(wl.name, "via", via)
+    got, kernels = run_on_gpu(device, wl, via=via)
+    want = oracle_eval(wl)
+    assert_bit_exact(got[0], want[0], wl.name)
+    if kernel is not None:
+        assert any(kernel in k for k in kernels), (kernels, kernel)
+    return kernels
+
+
+# ---- conv2d ---------------------------------------------------------------------------------
+def test_conv2d_config0_literal(device):
+    """BASELINE config 0 with its literal (saturating) requant ranges."""
+    check(device, w.conv2d_workload(), kernel="igemm_i8")
+
+
+def test_conv2d_config0_realistic(device):
+    check(device, w.conv2d_workload(realistic=True), via="device", kernel="igemm_i8")
+
+
+def test_conv2d_config0_nchw_boundary(device):
+    """Same op with the reference's literal N,C,H,W boundary: transposes at the bindings."""
+    kernels = check(device, w.conv2d_workload(realistic=True, nhwc=False))
+    assert kernels[0] == "transpose_i8" and kernels[-1] == "transpose_i8"
+
+
+@pytest.mark.parametrize("kw", CONV)
+@pytest.mark.parametrize("nhwc", [True, False])
+def test_conv2d_geometries(device, kw, nhwc):
+    check(device, w.conv2d_workload(realistic=True, nhwc=nhwc, output_min=-128, **kw))
+
+
+@pytest.mark.parametrize("variant", [0, 1, 2, 3])
+def test_conv2d_every_tile_variant(device, variant, monkeypatch):
+    monkeypatch.setenv("THIP_IGEMM_VARIANT", str(variant))
+    k = check(device, w.conv2d_workload(N=2, H=28, W=28, C=32, O=96, realistic=True))
+    assert runtime.lib()  # the variant is baked into the descriptor at serialize time
+    names = ["128x128", "256x256", "64x64", "256x128"]
+    assert names[variant] in k[0]
+    check(device, w.conv2d_workload(N=1, H=15, W=17, C=24, O=40, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True))
+    check(device, w.fully_connected_workload(300, 192, 520, realistic=True))
+
+
+def test_conv2d_mbv2_layer_shapes(device):
+    # first layer (3 channels, stride 2, TF SAME), expand / project 1x1, last 1x1
+    check(device, w.conv2d_workload(N=2, H=224, W=224, C=3, O=32, stride=(2, 2), pad=(0, 1, 0, 1), realistic=True, input_zp=-1))
+    check(device, w.conv2d_workload(N=2, H=56, W=56, C=24, O=144, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True))
+    check(device, w.conv2d_workload(N=2, H=28, W=28, C=192, O=32, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True))
+    check(device, w.conv2d_workload(N=2, H=7, W=7, C=320, O=1280, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True))
+
+
+def test_conv2d_int32_output(device):
+    wl = w.conv2d_workload(N=1, H=9, W=9, C=16, O=8, realistic=True)
+    # same op, int32 init and full-range clamp: exposes the un-narrowed requant result
+    from torq_compiler_amd import Program
+    a = dict(wl.attrs)
+    wts, sb = a.pop("weights"), a.pop("scale_bias")
+    a.pop("nhwc")
+    a.update(output_min=-(1 << 31), output_max=(1 << 31) - 1)
+    a["shift_factor"] = max(a["shift_factor"] - 8, 0)
+    p = Program()
+    out = p.binding(1, (1, 9, 9, 8), np.int32)
+    p.conv2d(p.binding(0, (1, 9, 9, 16)), wts, sb, init=out, nhwc_input=True, out_dtype=np.int32, **a)
+    from oracle import oracle as orc
+    want = orc.conv2d(wl.inputs[0], wts, sb, layout=orc.NHWC, out_dtype=np.int32, **a)
+    announce("conv2d int32 out")
+    exe = Executable(device, p.serialize())
+    got = np.zeros((1, 9, 9, 8), dtype=np.int32)
+    exe.run_host([wl.inputs[0], got])
+    exe.close()
+    assert_bit_exact(got, want, "conv2d int32")
+
+
+# ---- fully_connected ---------------------------------------------------------------------------
+@pytest.mark.parametrize("mkn", [(1, 2048, 2048), (16, 2048, 8192), (512, 4096, 4096)])
+def test_fully_connected_config1(device, mkn):
+    M = mkn[0]
+    check(device, w.fully_connected_workload(*mkn, realistic=True), via="device",
+          kernel="fc_skinny" if M <= 16 else "igemm_i8")
+
+
+def test_fully_connected_config1_literal_ranges(device):
+    check(device, w.fully_connected_workload(16, 2048, 8192))
+
+
+@pytest.mark.parametrize("mkn", [(1, 1, 1), (1, 61, 1991), (4, 1024, 1024), (1, 2000, 97), (16, 3, 7), (17, 128, 70),
+                                 (130, 700, 500), (3, 1280, 1000), (9, 1000, 512)])
+def test_fully_connected_geometries(device, mkn):
+    check(device, w.fully_connected_workload(*mkn, realistic=True))
+
+
+def test_fully_connected_without_skinny_kernel(device, monkeypatch):
+    monkeypatch.setenv("THIP_NO_SKINNY", "1")
+    check(device, w.fully_connected_workload(16, 2048, 512, realistic=True), kernel="igemm_i8")
+
+
+# ---- bandwidth ops ---------------------------------------------------------------------------
+@pytest.mark.parametrize("batch", [1, 8])
+def test_depthwise_config2a(device, batch):
+    check(device, w.depthwise_workload(N=batch), via="device", kernel="depthwise_i8")
+
+
+@pytest.mark.parametrize("kw", [
+    dict(N=1, H=6, W=42, C=16), dict(N=1, H=6, W=6, C=2, pad=(0, 0, 0, 0)), dict(N=1, H=13, W=15, C=8, stride=(1, 1), pad=(1, 1, 1, 1)),
+    dict(N=1, H=27, W=27, C=128, KH=4, KW=4, stride=(2, 2), pad=(1, 2, 1, 2)), dict(N=2, H=21, W=21, C=5, stride=(2, 2), pad=(1, 1, 1, 1)),
+    dict(N=1, H=14, W=14, C=36, stride=(1, 1), pad=(1, 1, 1, 1)), dict(N=3, H=112, W=112, C=32, stride=(1, 1), pad=(1, 1, 1, 1)),
+])
+@pytest.mark.parametrize("nhwc", [True, False])
+def test_depthwise_geometries(device, kw, nhwc):
+    check(device, w.depthwise_workload(nhwc=nhwc, **kw))
+
+
+@pytest.mark.parametrize("batch", [1, 8])
+def test_maxpool_config2b(device, batch):
+    check(device, w.maxpool_workload(N=batch), via="device", kernel="maxpool_i8")
+
+
+@pytest.mark.parametrize("kw", [dict(H=8, W=8, C=4), dict(H=8, W=8, C=1), dict(H=32, W=32, C=64, kernel=(3, 3), pad=(1, 1, 1, 1)),
+                                dict(H=10, W=10, C=4, kernel=(5, 5), stride=(1, 1)), dict(H=224, W=224, C=64, kernel=(3, 3), pad=(0, 1, 0, 1)),
+                                dict(H=10, W=10, C=4, kernel=(1, 3), stride=(1, 3), pad=(0, 2, 0, 0), input_zp=-7)])
+@pytest.mark.parametrize("nhwc", [True, False])
+def test_maxpool_geometries(device, kw, nhwc):
+    check(device, w.maxpool_workload(nhwc=nhwc, **kw))
+
+
+@pytest.mark.parametrize("kw", [dict(N=1), dict(N=64), dict(N=2, C=128), dict(N=1, H=12, W=8, C=37), dict(N=3, H=37, W=17, C=11), dict(N=1, H=53, W=37, C=1)])
+def test_avgpool(device, kw):
+    check(device, w.avgpool_workload(**kw), kernel="avgpool_i8")
+
+
+@pytest.mark.parametrize("kw", [dict(N=1), dict(N=64), dict(N=1, H=4, W=4, C=1), dict(N=1, H=6, W=8, C=4, zp0=127, zp1=-128), dict(N=1, H=7, W=7, C=33)])
+def test_add(device, kw):
+    check(device, w.add_workload(**kw), via="device", kernel="add_i8")
+
+
+# ---- programs, properties, error paths ------------------------------------------------------------
+def test_multi_op_program(device):
+    p, x, want_fc, want_sum = _chain_program(True)
+    announce("inverted-residual chain program")
+    exe = Executable(device, p.serialize())
+    out = np.zeros(want_fc.shape, dtype=np.int8)
+    aux = np.zeros(want_sum.shape, dtype=np.int8)
+    exe.run_host([x, out, aux])
+    assert_bit_exact(out, want_fc, "chain fc")
+    assert_bit_exact(aux, want_sum, "chain residual")
+    # running again gives the same bytes (intermediates hold no state between dispatches)
+    out2 = np.zeros_like(out)
+    exe.run_host([x, out2, np.zeros_like(aux)])
+    exe.close()
+    assert np.array_equal(out, out2)
+
+
+def test_full_size_gemm_properties(device):
+    """(4096,4096,4096) is too slow for the oracle in a test: check rows the oracle can afford plus a
+    structural property (each output row depends on its own input row only)."""
+    wl = w.fully_connected_workload(4096, 4096, 4096, realistic=True)
+    announce(wl.name)
+    got, kernels = run_on_gpu(device, wl, via="device")
+    got = got[0]
+    from oracle import oracle as orc
+    a = dict(wl.attrs)
+    wts, sb = a.pop("weights"), a.pop("scale_bias")
+    rows = np.r_[0:40, 2000:2040, 4056:4096]
+    want = orc.fully_connected(wl.inputs[0][rows], wts, sb, **a)
+    assert_bit_exact(got[rows], want, "sampled rows")
+    # duplicate input rows give duplicate output rows
+    wl.inputs[0][1::2] = wl.inputs[0][0::2]
+    got2, _ = run_on_gpu(device, wl, via="device")
+    assert np.array_equal(got2[0][1::2], got2[0][0::2]) and np.array_equal(got2[0][0::2], got[0::2])
+
+
+def test_dispatch_state_validation(device):
+    wl = w.add_workload(N=1, H=4, W=4, C=8)
+    exe = Executable(device, wl.program.serialize())
+    a, b = wl.inputs
+    out = np.zeros(a.shape, dtype=np.int8)
+    with pytest.raises(ThipError) as e:
+        exe.run_host([a, b])  # a binding is missing
+    assert e.value.code == runtime.INVALID_ARGUMENT
+    with pytest.raises(ThipError) as e:
+        exe.run_host([a, b, np.zeros(5, dtype=np.int8)])  # too short
+    assert e.value.code == runtime.OUT_OF_RANGE
+    st, keep = runtime.make_state([a.ctypes.data, 0, out.ctypes.data], [a.nbytes, b.nbytes, out.nbytes], [0, 0, 0])
+    with pytest.raises(ThipError) as e:
+        exe.run_state(st)  # NULL binding
+    assert e.value.code == runtime.FAILED_PRECONDITION
+    # a misaligned device pointer is refused before any launch
+    p = device.upload(np.zeros(a.nbytes + 64, dtype=np.int8))
+    with pytest.raises(ThipError) as e:
+        exe.run_device([p + 1, p, p], [a.nbytes] * 3)
+    assert e.value.code == runtime.FAILED_PRECONDITION
+    with pytest.raises(ThipError) as e:
+        exe.time_device([p, p, p], [a.nbytes] * 3, 0)  # zero iterations
+    assert e.value.code == runtime.INVALID_ARGUMENT
+    device.free(p)
+    # and the executable still works afterwards
+    exe.run_host([a, b, out])
+    assert_bit_exact(out, oracle_eval(wl)[0], "add after errors")
+    exe.close()
+
+
+def test_event_log_and_timing(device, tmp_path):
+    wl = w.maxpool_workload(N=2)
+    exe = Executable(device, wl.program.serialize())
+    log = tmp_path / "events.csv"
+    device.set_event_log(str(log))
+    x = wl.inputs[0]
+    pin = device.upload(x)
+    pout = device.upload(np.zeros(wl.outputs[0][0], dtype=np.int8))
+    ms = exe.time_device([pin, pout], [x.nbytes, int(np.prod(wl.outputs[0][0]))], 5)
+    device.set_event_log("")
+    assert ms > 0
+    rows = log.read_text().strip().splitlines()
+    assert rows[0] == "time_us,op,kernel,phase" and len(rows) == 1 + 2 * 5
+    assert "maxpool_i8,BEGIN" in rows[1] and "maxpool_i8,END" in rows[2]
+    got = device.download(pout, wl.outputs[0][0], np.int8)
+    assert_bit_exact(got, oracle_eval(wl)[0], "timed maxpool")
+    device.free(pin)
+    device.free(pout)
+    exe.close()

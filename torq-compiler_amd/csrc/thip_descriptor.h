@@ -1,0 +1,120 @@
+// Dispatch descriptor: the on-disk / in-memory program format that the emitter
+// writes and the driver reads.  It plays the role of the reference's "SNPU"
+// flatbuffer (runtime/schemas/torq_executable_def.fbs:17-199: code segments,
+// binding table, host actions) for a GPU target: a little-endian header, a
+// binding table, a table of intermediate buffers, a table of constant
+// segments, a list of fixed-size kernel records, and the constant bytes.
+// All structs are plain data with explicit sizes; offsets are from the start
+// of the blob.
+#pragma once
+
+#include <stdint.h>
+
+namespace thip {
+
+constexpr uint32_t kMagic = 0x50494854u;  // "THIP"
+constexpr uint32_t kDescriptorVersion = 1;
+constexpr uint32_t kArchGfx950 = 950;
+constexpr uint64_t kDataAlign = 256;
+
+// Memory spaces an operand reference can name.
+enum Space : uint32_t { kSpaceNone = 0, kSpaceBinding = 1, kSpaceTemp = 2, kSpaceConst = 3 };
+
+struct DescRef {
+    uint32_t space;
+    uint32_t index;
+    uint64_t offset;  // bytes into the buffer
+};
+
+struct DescHeader {
+    uint32_t magic;
+    uint32_t version;
+    uint32_t arch;
+    uint32_t flags;
+    uint32_t op_count;
+    uint32_t binding_count;
+    uint32_t temp_count;
+    uint32_t const_count;
+    uint64_t ops_offset;
+    uint64_t bindings_offset;
+    uint64_t temps_offset;
+    uint64_t consts_offset;
+    uint64_t data_offset;
+    uint64_t total_size;
+};
+
+enum BindingFlags : uint32_t { kBindingRead = 1, kBindingWritten = 2 };
+
+struct DescBinding {
+    uint32_t id;
+    uint32_t flags;
+    uint64_t size;  // bytes the program touches
+};
+
+struct DescTemp {
+    uint64_t size;
+};
+
+struct DescConst {
+    uint64_t offset;  // from DescHeader::data_offset
+    uint64_t size;
+};
+
+// Kernel kinds.  One record = one kernel launch.
+enum Kind : uint32_t {
+    kKindTranspose = 1,  // [B, R, S] -> [B, S, R] bytes (NCHW <-> NHWC)
+    kKindIgemm = 2,      // conv2d / fully_connected / matmul on MFMA
+    kKindFcSkinny = 3,   // fully_connected with few rows: weight streaming
+    kKindDepthwise = 4,
+    kKindMaxPool = 5,
+    kKindAvgPool = 6,
+    kKindAdd = 7,
+};
+
+// Variants of kKindIgemm: how the A (activation) tile is gathered.
+enum IgemmLoader : uint32_t {
+    kLoaderDense = 0,   // A is a dense [M, K] matrix with K % 16 == 0
+    kLoaderGather = 1,  // implicit-GEMM gather through the k-table, `gran` bytes at a time
+};
+
+struct DescOp {
+    uint32_t kind;
+    uint32_t variant;    // tile configuration index (igemm) / vector width (bandwidth kernels)
+    uint32_t loader;     // IgemmLoader
+    uint32_t gran;       // gather granularity in bytes: 16, 8, 4, 2 or 1
+    int32_t out_dtype;   // THIP_DTYPE_*
+    int32_t input_zp;
+    int32_t output_zp;
+    int32_t output_min;
+    int32_t output_max;
+    int32_t shift;
+    // activation geometry (NHWC)
+    int32_t N, H, W, C;
+    int32_t OH, OW, OC;
+    int32_t KH, KW, SH, SW;
+    int32_t PL, PR, PT, PB;
+    // GEMM view: M x K times (N x K)^T; Kp/Np are the padded sizes of the packed weights
+    int32_t M, K, Kp, Nn, Np;
+    // uniform parameters (add weights; matmul / avgpool / add single pair)
+    int32_t w0, w1;
+    int32_t bias0, scale0;
+    // transpose: batch, rows, cols
+    int32_t TB, TR, TS;
+    int32_t reserved[3];
+    DescRef in0;
+    DescRef in1;
+    DescRef weights;  // packed weights
+    DescRef bias;     // int32[Np] (de-interleaved)
+    DescRef scale;    // int32[Np]
+    DescRef table;    // k-table of the gather loader
+    DescRef out;
+};
+
+// k-table entry of the gather loader: one per `gran` bytes of the padded K axis.
+// bits 0..15 channel offset, 16..23 kw, 24..30 kh, bit 31 set = beyond K (feeds zeros).
+inline uint32_t packKEntry(int kh, int kw, int ci) {
+    return (uint32_t)ci | ((uint32_t)kw << 16) | ((uint32_t)kh << 24);
+}
+constexpr uint32_t kKEntryInvalid = 0x80000000u;
+
+}  // namespace thip

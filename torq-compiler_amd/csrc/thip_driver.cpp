@@ -1,0 +1,633 @@
+// Run side: device, executable and dispatch.
+//
+// The shape of this file follows the reference's HAL driver for this path:
+//   thip_executable_create  <- iree_hal_torq_native_executable_create
+//                              (runtime/driver/native_executable.cc:41-108): copy the
+//                              program blob and the executable constants, build the
+//                              executor object, initialise it (version / target gate,
+//                              runtime/driver/TorqExecutable.cc:655-752).
+//   thip_executable_run     <- iree_hal_torq_native_executable_run (:180-192) ->
+//                              TorqExecutable::executeDispatch
+//                              (runtime/driver/TorqExecutable.cc:1025-1125): lock,
+//                              write inputs, walk the action list, read outputs.
+// Instead of NSS programs on an NPU the action list is a list of kernel
+// records, each launched on the executable's HIP stream.
+#include <hip/hip_runtime.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <chrono>
+#include <mutex>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "thip_descriptor.h"
+#include "thip_kernels.h"
+#include "thip_status.h"
+
+using namespace thip;
+
+struct thip_device_t {
+    int ordinal = 0;
+    std::string arch;
+    std::mutex logMutex;
+    FILE *eventLog = nullptr;
+    std::chrono::steady_clock::time_point t0 = std::chrono::steady_clock::now();
+};
+
+struct thip_executable_t {
+    thip_device_t *device = nullptr;
+    std::vector<uint8_t> blob;           // private copy of the descriptor
+    std::vector<uint32_t> constants;     // executable-level constants (copied)
+    DescHeader header;
+    const DescOp *ops = nullptr;
+    const DescBinding *bindings = nullptr;
+    const DescTemp *temps = nullptr;
+    const DescConst *consts = nullptr;
+    uint8_t *constData = nullptr;        // device copy of the constant segment
+    std::vector<uint8_t *> tempPtrs;     // device intermediates
+    std::vector<uint8_t *> staging;      // device staging of host bindings
+    hipStream_t stream = nullptr;
+    hipEvent_t evStart = nullptr, evStop = nullptr;
+    std::mutex mutex;                    // one dispatch at a time
+};
+
+static thip_status_t hipFail(hipError_t e, const char *what) {
+    const thip_status_t code = e == hipErrorOutOfMemory ? THIP_RESOURCE_EXHAUSTED : THIP_INTERNAL;
+    return fail(code, "%s: %s", what, hipGetErrorString(e));
+}
+
+#define THIP_HIP(call, what)                          \
+    do {                                              \
+        hipError_t e_ = (call);                       \
+        if (e_ != hipSuccess) return hipFail(e_, what); \
+    } while (0)
+
+static thip_status_t validateDescriptor(const uint8_t *p, size_t size, DescHeader *out) {
+    if (!p || size < sizeof(DescHeader)) return fail(THIP_INVALID_ARGUMENT, "descriptor is smaller than its header");
+    DescHeader h;
+    memcpy(&h, p, sizeof(h));
+    if (h.magic != kMagic) return fail(THIP_INVALID_ARGUMENT, "descriptor magic 0x%08x is not THIP", h.magic);
+    // same gate as `runtime_version != 2 -> UNAVAILABLE`, runtime/driver/TorqExecutable.cc:663-667
+    if (h.version != kDescriptorVersion) {
+        return fail(THIP_UNAVAILABLE, "descriptor version %u, this runtime reads version %u", h.version, kDescriptorVersion);
+    }
+    // same gate as isHwCompatible(hwId), runtime/driver/TorqExecutable.cc:701-705
+    if (h.arch != kArchGfx950) return fail(THIP_UNAVAILABLE, "descriptor targets arch %u, this runtime drives gfx950", h.arch);
+    if (h.total_size > size) return fail(THIP_INVALID_ARGUMENT, "descriptor says %llu bytes, %zu given", (unsigned long long)h.total_size, size);
+    auto inside = [&](uint64_t off, uint64_t count, uint64_t each) {
+        return off <= h.total_size && count * each <= h.total_size - off;
+    };
+    if (!inside(h.ops_offset, h.op_count, sizeof(DescOp)) || !inside(h.bindings_offset, h.binding_count, sizeof(DescBinding)) ||
+        !inside(h.temps_offset, h.temp_count, sizeof(DescTemp)) || !inside(h.consts_offset, h.const_count, sizeof(DescConst)) ||
+        h.data_offset > h.total_size) {
+        return fail(THIP_INVALID_ARGUMENT, "descriptor tables run past its end");
+    }
+    if (h.op_count == 0) return fail(THIP_INVALID_ARGUMENT, "descriptor holds no ops");
+    if (h.binding_count > 64) return fail(THIP_INVALID_ARGUMENT, "descriptor declares %u bindings (max 64)", h.binding_count);
+    const DescConst *consts = (const DescConst *)(p + h.consts_offset);
+    for (uint32_t i = 0; i < h.const_count; i++) {
+        if (consts[i].offset > h.total_size - h.data_offset || consts[i].size > h.total_size - h.data_offset - consts[i].offset) {
+            return fail(THIP_INVALID_ARGUMENT, "constant segment %u runs past the descriptor", i);
+        }
+    }
+    // every operand reference must name an existing buffer and stay inside it
+    const DescOp *ops = (const DescOp *)(p + h.ops_offset);
+    const DescBinding *bindings = (const DescBinding *)(p + h.bindings_offset);
+    const DescTemp *temps = (const DescTemp *)(p + h.temps_offset);
+    for (uint32_t i = 0; i < h.op_count; i++) {
+        const DescRef *refs[] = {&ops[i].in0, &ops[i].in1, &ops[i].weights, &ops[i].bias, &ops[i].scale, &ops[i].table, &ops[i].out};
+        for (const DescRef *r : refs) {
+            uint64_t limit = 0;
+            switch (r->space) {
+            case kSpaceNone: continue;
+            case kSpaceBinding:
+                if (r->index >= h.binding_count) return fail(THIP_INVALID_ARGUMENT, "op %u names binding %u of %u", i, r->index, h.binding_count);
+                limit = bindings[r->index].size;
+                break;
+            case kSpaceTemp:
+                if (r->index >= h.temp_count) return fail(THIP_INVALID_ARGUMENT, "op %u names intermediate %u of %u", i, r->index, h.temp_count);
+                limit = temps[r->index].size;
+                break;
+            case kSpaceConst:
+                if (r->index >= h.const_count) return fail(THIP_INVALID_ARGUMENT, "op %u names constant %u of %u", i, r->index, h.const_count);
+                limit = consts[r->index].size;
+                break;
+            default: return fail(THIP_INVALID_ARGUMENT, "op %u has an operand in unknown space %u", i, r->space);
+            }
+            if (r->offset > limit) return fail(THIP_INVALID_ARGUMENT, "op %u operand offset %llu is past its buffer (%llu)", i, (unsigned long long)r->offset, (unsigned long long)limit);
+        }
+    }
+    *out = h;
+    return THIP_OK;
+}
+
+// Bytes an operand reference can still address.
+static uint64_t refRoom(const thip_executable_t *e, const DescRef &r) {
+    switch (r.space) {
+    case kSpaceBinding: return e->bindings[r.index].size - r.offset;
+    case kSpaceTemp: return e->temps[r.index].size - r.offset;
+    case kSpaceConst: return e->consts[r.index].size - r.offset;
+    default: return 0;
+    }
+}
+
+// Checks, once at creation, that every kernel record stays inside the buffers it names.
+static thip_status_t checkOpFootprint(const thip_executable_t *e, uint32_t i) {
+    const DescOp &op = e->ops[i];
+    auto need = [&](const DescRef &r, uint64_t bytes, const char *name) -> thip_status_t {
+        if (r.space == kSpaceNone) return fail(THIP_INVALID_ARGUMENT, "op %u: operand %s is missing", i, name);
+        if (refRoom(e, r) < bytes) {
+            return fail(THIP_INVALID_ARGUMENT, "op %u: operand %s needs %llu bytes, its buffer has %llu", i, name,
+                        (unsigned long long)bytes, (unsigned long long)refRoom(e, r));
+        }
+        return THIP_OK;
+    };
+    auto positive = [&](std::initializer_list<int32_t> vals) {
+        for (int32_t v : vals) {
+            if (v <= 0) return false;
+        }
+        return true;
+    };
+    const uint64_t outElem = op.out_dtype == THIP_DTYPE_I32 ? 4 : op.out_dtype == THIP_DTYPE_I16 ? 2 : 1;
+    thip_status_t s = THIP_OK;
+    switch (op.kind) {
+    case kKindTranspose: {
+        if (!positive({op.TB, op.TR, op.TS})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad transpose extents", i);
+        const uint64_t bytes = (uint64_t)op.TB * op.TR * op.TS;
+        if ((s = need(op.in0, bytes, "in"))) return s;
+        return need(op.out, bytes, "out");
+    }
+    case kKindIgemm: {
+        if (!positive({op.M, op.K, op.Kp, op.Nn, op.Np, op.N, op.H, op.W, op.C, op.OH, op.OW})) {
+            return fail(THIP_INVALID_ARGUMENT, "op %u: bad igemm extents", i);
+        }
+        if (op.variant >= kIgemmVariantCount) return fail(THIP_INVALID_ARGUMENT, "op %u: unknown igemm variant %u", i, op.variant);
+        const uint64_t inBytes = op.loader == kLoaderDense ? (uint64_t)op.M * op.K : (uint64_t)op.N * op.H * op.W * op.C;
+        if (op.loader != kLoaderDense && (uint64_t)op.N * op.OH * op.OW != (uint64_t)op.M) {
+            return fail(THIP_INVALID_ARGUMENT, "op %u: igemm rows do not match the output pixels", i);
+        }
+        if ((s = need(op.in0, inBytes, "in"))) return s;
+        if ((s = need(op.weights, (uint64_t)op.Np * op.Kp, "weights"))) return s;
+        if ((s = need(op.bias, (uint64_t)op.Np * 4, "bias"))) return s;
+        if ((s = need(op.scale, (uint64_t)op.Np * 4, "scale"))) return s;
+        if (op.loader == kLoaderGather) {
+            if (op.gran == 0 || (op.gran & (op.gran - 1)) || op.gran > 16) return fail(THIP_INVALID_ARGUMENT, "op %u: bad gather granularity", i);
+            if ((s = need(op.table, (uint64_t)op.Kp / op.gran * 4, "table"))) return s;
+            // every valid table entry must stay inside the window and the channel axis
+            const uint8_t *base = e->blob.data() + e->header.data_offset + e->consts[op.table.index].offset + op.table.offset;
+            if (op.table.space != kSpaceConst) return fail(THIP_INVALID_ARGUMENT, "op %u: table must be a constant", i);
+            for (uint32_t t = 0; t < (uint32_t)op.Kp / op.gran; t++) {
+                uint32_t ent;
+                memcpy(&ent, base + 4ull * t, 4);
+                if (ent & kKEntryInvalid) continue;
+                const int kh = (ent >> 24) & 0x7f, kw = (ent >> 16) & 0xff, ci = ent & 0xffff;
+                if (kh >= op.KH || kw >= op.KW || ci + (int)op.gran > op.C) return fail(THIP_INVALID_ARGUMENT, "op %u: table entry %u is outside the window", i, t);
+            }
+        }
+        return need(op.out, (uint64_t)op.M * op.Nn * outElem, "out");
+    }
+    case kKindFcSkinny: {
+        if (!positive({op.M, op.K, op.Nn})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad fc extents", i);
+        if ((s = need(op.in0, (uint64_t)op.M * op.K, "in"))) return s;
+        if ((s = need(op.weights, (uint64_t)op.Nn * op.K, "weights"))) return s;
+        if ((s = need(op.bias, (uint64_t)op.Nn * 4, "bias"))) return s;
+        if ((s = need(op.scale, (uint64_t)op.Nn * 4, "scale"))) return s;
+        return need(op.out, (uint64_t)op.M * op.Nn * outElem, "out");
+    }
+    case kKindDepthwise: {
+        if (!positive({op.N, op.H, op.W, op.C, op.OH, op.OW, op.KH, op.KW})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad depthwise extents", i);
+        if ((s = need(op.in0, (uint64_t)op.N * op.H * op.W * op.C, "in"))) return s;
+        if ((s = need(op.weights, (uint64_t)op.KH * op.KW * op.C, "weights"))) return s;
+        if ((s = need(op.bias, (uint64_t)op.C * 4, "bias"))) return s;
+        if ((s = need(op.scale, (uint64_t)op.C * 4, "scale"))) return s;
+        return need(op.out, (uint64_t)op.N * op.OH * op.OW * op.C, "out");
+    }
+    case kKindMaxPool: {
+        if (!positive({op.N, op.H, op.W, op.C, op.OH, op.OW, op.KH, op.KW})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad maxpool extents", i);
+        if ((s = need(op.in0, (uint64_t)op.N * op.H * op.W * op.C, "in"))) return s;
+        return need(op.out, (uint64_t)op.N * op.OH * op.OW * op.C, "out");
+    }
+    case kKindAvgPool: {
+        if (!positive({op.N, op.H, op.W, op.C})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad avgpool extents", i);
+        if ((s = need(op.in0, (uint64_t)op.N * op.H * op.W * op.C, "in"))) return s;
+        return need(op.out, (uint64_t)op.N * op.C, "out");
+    }
+    case kKindAdd: {
+        if (!positive({op.C})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad add extent", i);
+        if ((s = need(op.in0, (uint64_t)op.C, "in1"))) return s;
+        if ((s = need(op.in1, (uint64_t)op.C, "in2"))) return s;
+        return need(op.out, (uint64_t)op.C, "out");
+    }
+    default: return fail(THIP_INVALID_ARGUMENT, "op %u has unknown kind %u", i, op.kind);
+    }
+}
+
+static const char *opKernelName(const DescOp &op) {
+    switch (op.kind) {
+    case kKindTranspose: return "transpose_i8";
+    case kKindIgemm: return igemmTile(op.variant).name;
+    case kKindFcSkinny: return "fc_skinny";
+    case kKindDepthwise: return "depthwise_i8";
+    case kKindMaxPool: return "maxpool_i8";
+    case kKindAvgPool: return "avgpool_i8";
+    case kKindAdd: return "add_i8";
+    default: return "unknown";
+    }
+}
+
+static void logEvent(thip_device_t *d, uint32_t opIndex, const char *name, const char *phase) {
+    if (!d->eventLog) return;
+    std::lock_guard<std::mutex> lock(d->logMutex);
+    const auto us = std::chrono::duration_cast<std::chrono::microseconds>(std::chrono::steady_clock::now() - d->t0).count();
+    fprintf(d->eventLog, "%lld,%u,%s,%s\n", (long long)us, opIndex, name, phase);
+}
+
+// Resolves an operand reference against the buffers of this dispatch.
+static uint8_t *resolve(const thip_executable_t *e, const DescRef &r, uint8_t *const *bindingPtrs) {
+    switch (r.space) {
+    case kSpaceBinding: return bindingPtrs[r.index] + r.offset;
+    case kSpaceTemp: return e->tempPtrs[r.index] + r.offset;
+    case kSpaceConst: return e->constData + e->consts[r.index].offset + r.offset;
+    default: return nullptr;
+    }
+}
+
+static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *bp) {
+    const DescOp &op = e->ops[i];
+    const Requant rq{op.shift, op.output_zp, op.output_min, op.output_max};
+    hipError_t err = hipSuccess;
+    switch (op.kind) {
+    case kKindTranspose: {
+        TransposeArgs a{(const int8_t *)resolve(e, op.in0, bp), (int8_t *)resolve(e, op.out, bp), op.TB, op.TR, op.TS};
+        err = launchTranspose(a, e->stream);
+        break;
+    }
+    case kKindIgemm: {
+        IgemmArgs a;
+        memset(&a, 0, sizeof(a));
+        a.A = (const int8_t *)resolve(e, op.in0, bp);
+        a.Bp = (const int8_t *)resolve(e, op.weights, bp);
+        a.bias = (const int32_t *)resolve(e, op.bias, bp);
+        a.scale = (const int32_t *)resolve(e, op.scale, bp);
+        a.ktab = (const uint32_t *)resolve(e, op.table, bp);
+        a.out = resolve(e, op.out, bp);
+        a.M = op.M; a.N = op.Nn; a.K = op.K; a.Kp = op.Kp; a.Np = op.Np;
+        a.H = op.H; a.W = op.W; a.C = op.C; a.OH = op.OH; a.OW = op.OW;
+        a.SH = op.SH; a.SW = op.SW; a.PT = op.PT; a.PL = op.PL;
+        a.input_zp = op.input_zp;
+        a.out_dtype = op.out_dtype;
+        a.loader = op.loader;
+        a.gran = op.gran;
+        a.rq = rq;
+        err = launchIgemm(a, op.variant, e->stream);
+        break;
+    }
+    case kKindFcSkinny: {
+        FcSkinnyArgs a{(const int8_t *)resolve(e, op.in0, bp), (const int8_t *)resolve(e, op.weights, bp),
+                       (const int32_t *)resolve(e, op.bias, bp), (const int32_t *)resolve(e, op.scale, bp),
+                       resolve(e, op.out, bp), op.M, op.Nn, op.K, op.out_dtype, rq};
+        err = launchFcSkinny(a, e->stream);
+        break;
+    }
+    case kKindDepthwise: {
+        DepthwiseArgs a{(const int8_t *)resolve(e, op.in0, bp), (const int8_t *)resolve(e, op.weights, bp),
+                        (const int32_t *)resolve(e, op.bias, bp), (const int32_t *)resolve(e, op.scale, bp),
+                        (int8_t *)resolve(e, op.out, bp), op.N, op.H, op.W, op.C, op.OH, op.OW, op.KH, op.KW,
+                        op.SH, op.SW, op.PT, op.PL, op.input_zp, rq};
+        err = launchDepthwise(a, e->stream);
+        break;
+    }
+    case kKindMaxPool: {
+        MaxPoolArgs a{(const int8_t *)resolve(e, op.in0, bp), (int8_t *)resolve(e, op.out, bp), op.N, op.H, op.W, op.C,
+                      op.OH, op.OW, op.KH, op.KW, op.SH, op.SW, op.PT, op.PL, op.input_zp, op.output_min, op.output_max};
+        err = launchMaxPool(a, e->stream);
+        break;
+    }
+    case kKindAvgPool: {
+        AvgPoolArgs a{(const int8_t *)resolve(e, op.in0, bp), (int8_t *)resolve(e, op.out, bp), op.N, op.H * op.W, op.C,
+                      op.w0, op.bias0, op.scale0, rq};
+        err = launchAvgPool(a, e->stream);
+        break;
+    }
+    case kKindAdd: {
+        AddArgs a{(const int8_t *)resolve(e, op.in0, bp), (const int8_t *)resolve(e, op.in1, bp),
+                  (int8_t *)resolve(e, op.out, bp), (int64_t)op.C, op.w0, op.w1, op.bias0, op.scale0, rq};
+        err = launchAdd(a, e->stream);
+        break;
+    }
+    default: return fail(THIP_INTERNAL, "op %u has unknown kind %u", i, op.kind);
+    }
+    if (err != hipSuccess) {
+        return fail(THIP_INTERNAL, "op %u (%s): launch failed: %s", i, opKernelName(op), hipGetErrorString(err));
+    }
+    return THIP_OK;
+}
+
+// Validates the dispatch state against the binding table.  Mirrors the checks of
+// iree_hal_torq_command_buffer_dispatch (runtime/driver/torq_command_buffer.c:453-494).
+static thip_status_t checkState(const thip_executable_t *e, const thip_dispatch_state_t *st, bool deviceOnly) {
+    if (!st) return fail(THIP_INVALID_ARGUMENT, "dispatch state is NULL");
+    if (st->constant_count > 0 && !st->constants) return fail(THIP_FAILED_PRECONDITION, "constants pointer is NULL");
+    if (st->binding_count < e->header.binding_count) {
+        return fail(THIP_INVALID_ARGUMENT, "dispatch carries %u bindings, the executable uses %u", st->binding_count, e->header.binding_count);
+    }
+    if (e->header.binding_count > 0 && (!st->binding_ptrs || !st->binding_lengths)) {
+        return fail(THIP_FAILED_PRECONDITION, "binding tables are NULL");
+    }
+    for (uint32_t i = 0; i < e->header.binding_count; i++) {
+        if (e->bindings[i].flags == 0) continue;  // declared but unused
+        if (!st->binding_ptrs[i]) {
+            return fail(THIP_FAILED_PRECONDITION, "required binding %u is NULL; all bindings must have a valid pointer", i);
+        }
+        if (st->binding_lengths[i] < e->bindings[i].size) {
+            return fail(THIP_OUT_OF_RANGE, "binding %u is %zu bytes, the executable touches %llu", i, st->binding_lengths[i],
+                        (unsigned long long)e->bindings[i].size);
+        }
+        const bool isDevice = st->binding_flags && (st->binding_flags[i] & THIP_BINDING_DEVICE);
+        if (deviceOnly && !isDevice) return fail(THIP_FAILED_PRECONDITION, "binding %u is a host pointer; this entry point takes device bindings only", i);
+        if (isDevice && ((uintptr_t)st->binding_ptrs[i] & 15) != 0) {
+            return fail(THIP_FAILED_PRECONDITION, "device binding %u is not 16-byte aligned", i);
+        }
+    }
+    return THIP_OK;
+}
+
+// Enqueues every kernel record of the program.  `bp` holds one device pointer per binding.
+static thip_status_t enqueueOps(thip_executable_t *e, uint8_t *const *bp) {
+    for (uint32_t i = 0; i < e->header.op_count; i++) {
+        logEvent(e->device, i, opKernelName(e->ops[i]), "BEGIN");
+        if (thip_status_t s = launchOp(e, i, bp)) return s;
+        logEvent(e->device, i, opKernelName(e->ops[i]), "END");
+    }
+    return THIP_OK;
+}
+
+extern "C" {
+
+thip_status_t thip_device_create(int32_t ordinal, thip_device_t **out_device) {
+    if (!out_device) return fail(THIP_INVALID_ARGUMENT, "null result pointer");
+    *out_device = nullptr;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0) {
+        (void)hipGetLastError();
+        return fail(THIP_UNAVAILABLE, "no HIP device is visible (%s)", e == hipSuccess ? "count is 0" : hipGetErrorString(e));
+    }
+    if (ordinal < 0 || ordinal >= count) return fail(THIP_INVALID_ARGUMENT, "device ordinal %d is outside 0..%d", ordinal, count - 1);
+    hipDeviceProp_t prop;
+    THIP_HIP(hipGetDeviceProperties(&prop, ordinal), "hipGetDeviceProperties");
+    std::string arch = prop.gcnArchName;
+    const size_t colon = arch.find(':');
+    if (colon != std::string::npos) arch.resize(colon);
+    if (arch != "gfx950") return fail(THIP_UNAVAILABLE, "device %d is %s; the kernels are built for gfx950 only", ordinal, arch.c_str());
+    THIP_HIP(hipSetDevice(ordinal), "hipSetDevice");
+    thip_device_t *d = new (std::nothrow) thip_device_t();
+    if (!d) return fail(THIP_RESOURCE_EXHAUSTED, "out of memory");
+    d->ordinal = ordinal;
+    d->arch = arch;
+    *out_device = d;
+    return THIP_OK;
+}
+
+void thip_device_destroy(thip_device_t *device) {
+    if (!device) return;
+    if (device->eventLog) fclose(device->eventLog);
+    delete device;
+}
+
+thip_status_t thip_device_name(thip_device_t *device, char *name, size_t capacity) {
+    if (!device || !name || capacity == 0) return fail(THIP_INVALID_ARGUMENT, "null argument");
+    snprintf(name, capacity, "%s", device->arch.c_str());
+    return THIP_OK;
+}
+
+thip_status_t thip_device_alloc(thip_device_t *device, size_t size, void **out_ptr) {
+    if (!device || !out_ptr) return fail(THIP_INVALID_ARGUMENT, "null argument");
+    *out_ptr = nullptr;
+    THIP_HIP(hipSetDevice(device->ordinal), "hipSetDevice");
+    THIP_HIP(hipMalloc(out_ptr, size ? size : 1), "hipMalloc");
+    return THIP_OK;
+}
+
+thip_status_t thip_device_free(thip_device_t *device, void *ptr) {
+    if (!device) return fail(THIP_INVALID_ARGUMENT, "null device");
+    if (ptr) THIP_HIP(hipFree(ptr), "hipFree");
+    return THIP_OK;
+}
+
+thip_status_t thip_device_h2d(thip_device_t *device, void *dst_device, const void *src_host, size_t size) {
+    if (!device || (size && (!dst_device || !src_host))) return fail(THIP_INVALID_ARGUMENT, "null argument");
+    if (size) THIP_HIP(hipMemcpy(dst_device, src_host, size, hipMemcpyHostToDevice), "hipMemcpy H2D");
+    return THIP_OK;
+}
+
+thip_status_t thip_device_d2h(thip_device_t *device, void *dst_host, const void *src_device, size_t size) {
+    if (!device || (size && (!dst_host || !src_device))) return fail(THIP_INVALID_ARGUMENT, "null argument");
+    if (size) THIP_HIP(hipMemcpy(dst_host, src_device, size, hipMemcpyDeviceToHost), "hipMemcpy D2H");
+    return THIP_OK;
+}
+
+thip_status_t thip_device_synchronize(thip_device_t *device) {
+    if (!device) return fail(THIP_INVALID_ARGUMENT, "null device");
+    THIP_HIP(hipDeviceSynchronize(), "hipDeviceSynchronize");
+    return THIP_OK;
+}
+
+thip_status_t thip_device_set_event_log(thip_device_t *device, const char *csv_path) {
+    if (!device) return fail(THIP_INVALID_ARGUMENT, "null device");
+    std::lock_guard<std::mutex> lock(device->logMutex);
+    if (device->eventLog) {
+        fclose(device->eventLog);
+        device->eventLog = nullptr;
+    }
+    if (csv_path && csv_path[0]) {
+        device->eventLog = fopen(csv_path, "w");
+        if (!device->eventLog) return fail(THIP_INVALID_ARGUMENT, "cannot open event log %s", csv_path);
+        fprintf(device->eventLog, "time_us,op,kernel,phase\n");
+    }
+    return THIP_OK;
+}
+
+thip_status_t thip_infer_format(const void *blob, size_t size, size_t format_capacity, char *format, size_t *out_inferred_size) {
+    DescHeader h;
+    if (thip_status_t s = validateDescriptor((const uint8_t *)blob, size, &h)) return s;
+    static const char kFormat[] = "thip-gfx950";
+    if (!format || format_capacity < sizeof(kFormat)) return fail(THIP_OUT_OF_RANGE, "format buffer too small");
+    memcpy(format, kFormat, sizeof(kFormat));
+    if (out_inferred_size) *out_inferred_size = (size_t)h.total_size;
+    return THIP_OK;
+}
+
+void thip_executable_destroy(thip_executable_t *e) {
+    if (!e) return;
+    if (e->stream) (void)hipStreamSynchronize(e->stream);
+    for (uint8_t *p : e->tempPtrs) {
+        if (p) (void)hipFree(p);
+    }
+    for (uint8_t *p : e->staging) {
+        if (p) (void)hipFree(p);
+    }
+    if (e->constData) (void)hipFree(e->constData);
+    if (e->evStart) (void)hipEventDestroy(e->evStart);
+    if (e->evStop) (void)hipEventDestroy(e->evStop);
+    if (e->stream) (void)hipStreamDestroy(e->stream);
+    delete e;
+}
+
+thip_status_t thip_executable_create(thip_device_t *device, const void *blob, size_t size, const uint32_t *constants,
+                                     size_t constant_count, thip_executable_t **out_executable) {
+    if (!out_executable) return fail(THIP_INVALID_ARGUMENT, "null result pointer");
+    *out_executable = nullptr;
+    if (!device) return fail(THIP_INVALID_ARGUMENT, "null device");
+    if (constant_count > 0 && !constants) return fail(THIP_INVALID_ARGUMENT, "constants pointer is NULL");
+    DescHeader h;
+    if (thip_status_t s = validateDescriptor((const uint8_t *)blob, size, &h)) return s;
+    thip_executable_t *e = new (std::nothrow) thip_executable_t();
+    if (!e) return fail(THIP_RESOURCE_EXHAUSTED, "out of memory");
+    e->device = device;
+    e->blob.assign((const uint8_t *)blob, (const uint8_t *)blob + h.total_size);
+    if (constant_count) e->constants.assign(constants, constants + constant_count);
+    e->header = h;
+    e->ops = (const DescOp *)(e->blob.data() + h.ops_offset);
+    e->bindings = (const DescBinding *)(e->blob.data() + h.bindings_offset);
+    e->temps = (const DescTemp *)(e->blob.data() + h.temps_offset);
+    e->consts = (const DescConst *)(e->blob.data() + h.consts_offset);
+    thip_status_t s = THIP_OK;
+    for (uint32_t i = 0; i < h.op_count && s == THIP_OK; i++) s = checkOpFootprint(e, i);
+    auto bail = [&](thip_status_t code) {
+        thip_executable_destroy(e);
+        return code;
+    };
+    if (s != THIP_OK) return bail(s);
+    hipError_t err = hipSetDevice(device->ordinal);
+    if (err == hipSuccess) err = hipStreamCreate(&e->stream);  // default priority
+    if (err == hipSuccess) err = hipEventCreate(&e->evStart);
+    if (err == hipSuccess) err = hipEventCreate(&e->evStop);
+    if (err != hipSuccess) return bail(hipFail(err, "creating the stream"));
+    const uint64_t dataSize = h.total_size - h.data_offset;
+    if (dataSize) {
+        err = hipMalloc((void **)&e->constData, dataSize);
+        if (err == hipSuccess) err = hipMemcpy(e->constData, e->blob.data() + h.data_offset, dataSize, hipMemcpyHostToDevice);
+        if (err != hipSuccess) return bail(hipFail(err, "uploading the constant segment"));
+    }
+    e->tempPtrs.assign(h.temp_count, nullptr);
+    for (uint32_t i = 0; i < h.temp_count; i++) {
+        const uint64_t bytes = e->temps[i].size ? e->temps[i].size : 1;
+        err = hipMalloc((void **)&e->tempPtrs[i], bytes);
+        // zero-filled once: padding regions of packed run-time operands rely on it
+        if (err == hipSuccess) err = hipMemset(e->tempPtrs[i], 0, bytes);
+        if (err != hipSuccess) return bail(hipFail(err, "allocating an intermediate"));
+    }
+    e->staging.assign(h.binding_count, nullptr);
+    *out_executable = e;
+    return THIP_OK;
+}
+
+static thip_status_t runLocked(thip_executable_t *e, const thip_dispatch_state_t *st) {
+    THIP_HIP(hipSetDevice(e->device->ordinal), "hipSetDevice");
+    uint8_t *bp[64] = {nullptr};
+    // writeInputs: host bindings are staged into device memory (TorqExecutable::writeInputs)
+    for (uint32_t i = 0; i < e->header.binding_count; i++) {
+        if (e->bindings[i].flags == 0) continue;
+        const bool isDevice = st->binding_flags && (st->binding_flags[i] & THIP_BINDING_DEVICE);
+        if (isDevice) {
+            bp[i] = (uint8_t *)st->binding_ptrs[i];
+            continue;
+        }
+        if (!e->staging[i]) {
+            THIP_HIP(hipMalloc((void **)&e->staging[i], e->bindings[i].size ? e->bindings[i].size : 1), "allocating binding staging");
+        }
+        bp[i] = e->staging[i];
+        if (e->bindings[i].flags & kBindingRead) {
+            THIP_HIP(hipMemcpyAsync(bp[i], st->binding_ptrs[i], e->bindings[i].size, hipMemcpyHostToDevice, e->stream), "staging a binding");
+        }
+    }
+    if (thip_status_t s = enqueueOps(e, bp)) {
+        (void)hipStreamSynchronize(e->stream);
+        return s;
+    }
+    // readOutputs (TorqExecutable::readOutputs, runtime/driver/TorqExecutable.cc:860-918)
+    for (uint32_t i = 0; i < e->header.binding_count; i++) {
+        const bool isDevice = st->binding_flags && (st->binding_flags[i] & THIP_BINDING_DEVICE);
+        if (isDevice || !(e->bindings[i].flags & kBindingWritten)) continue;
+        THIP_HIP(hipMemcpyAsync(st->binding_ptrs[i], bp[i], e->bindings[i].size, hipMemcpyDeviceToHost, e->stream), "reading back a binding");
+    }
+    THIP_HIP(hipStreamSynchronize(e->stream), "waiting for the dispatch");
+    return THIP_OK;
+}
+
+thip_status_t thip_executable_run(thip_executable_t *e, const thip_dispatch_state_t *st) {
+    if (!e) return fail(THIP_INVALID_ARGUMENT, "null executable");
+    if (thip_status_t s = checkState(e, st, false)) return s;
+    std::lock_guard<std::mutex> lock(e->mutex);
+    return runLocked(e, st);
+}
+
+thip_status_t thip_executable_enqueue(thip_executable_t *e, const thip_dispatch_state_t *st) {
+    if (!e) return fail(THIP_INVALID_ARGUMENT, "null executable");
+    if (thip_status_t s = checkState(e, st, true)) return s;
+    std::lock_guard<std::mutex> lock(e->mutex);
+    THIP_HIP(hipSetDevice(e->device->ordinal), "hipSetDevice");
+    uint8_t *bp[64] = {nullptr};
+    for (uint32_t i = 0; i < e->header.binding_count; i++) bp[i] = (uint8_t *)st->binding_ptrs[i];
+    return enqueueOps(e, bp);
+}
+
+thip_status_t thip_executable_wait(thip_executable_t *e) {
+    if (!e) return fail(THIP_INVALID_ARGUMENT, "null executable");
+    THIP_HIP(hipStreamSynchronize(e->stream), "waiting for the dispatch");
+    return THIP_OK;
+}
+
+thip_status_t thip_executable_time(thip_executable_t *e, const thip_dispatch_state_t *st, int32_t iterations, float *out_ms) {
+    if (!e || !out_ms) return fail(THIP_INVALID_ARGUMENT, "null argument");
+    if (iterations <= 0) return fail(THIP_INVALID_ARGUMENT, "iterations must be positive");
+    if (thip_status_t s = checkState(e, st, true)) return s;
+    std::lock_guard<std::mutex> lock(e->mutex);
+    THIP_HIP(hipSetDevice(e->device->ordinal), "hipSetDevice");
+    uint8_t *bp[64] = {nullptr};
+    for (uint32_t i = 0; i < e->header.binding_count; i++) bp[i] = (uint8_t *)st->binding_ptrs[i];
+    THIP_HIP(hipEventRecord(e->evStart, e->stream), "hipEventRecord");
+    for (int32_t it = 0; it < iterations; it++) {
+        if (thip_status_t s = enqueueOps(e, bp)) {
+            (void)hipStreamSynchronize(e->stream);
+            return s;
+        }
+    }
+    THIP_HIP(hipEventRecord(e->evStop, e->stream), "hipEventRecord");
+    THIP_HIP(hipEventSynchronize(e->evStop), "hipEventSynchronize");
+    float ms = 0.f;
+    THIP_HIP(hipEventElapsedTime(&ms, e->evStart, e->evStop), "hipEventElapsedTime");
+    *out_ms = ms / (float)iterations;
+    return THIP_OK;
+}
+
+thip_status_t thip_executable_op_count(thip_executable_t *e, uint32_t *out_count) {
+    if (!e || !out_count) return fail(THIP_INVALID_ARGUMENT, "null argument");
+    *out_count = e->header.op_count;
+    return THIP_OK;
+}
+
+thip_status_t thip_executable_op_kernel(thip_executable_t *e, uint32_t index, char *name, size_t capacity) {
+    if (!e || !name || capacity == 0) return fail(THIP_INVALID_ARGUMENT, "null argument");
+    if (index >= e->header.op_count) return fail(THIP_OUT_OF_RANGE, "op %u of %u", index, e->header.op_count);
+    snprintf(name, capacity, "%s", opKernelName(e->ops[index]));
+    return THIP_OK;
+}
+
+thip_status_t thip_executable_binding_count(thip_executable_t *e, uint32_t *out_count) {
+    if (!e || !out_count) return fail(THIP_INVALID_ARGUMENT, "null argument");
+    *out_count = e->header.binding_count;
+    return THIP_OK;
+}
+
+thip_status_t thip_executable_binding_size(thip_executable_t *e, uint32_t binding, size_t *out_size) {
+    if (!e || !out_size) return fail(THIP_INVALID_ARGUMENT, "null argument");
+    if (binding >= e->header.binding_count) return fail(THIP_OUT_OF_RANGE, "binding %u of %u", binding, e->header.binding_count);
+    *out_size = (size_t)e->bindings[binding].size;
+    return THIP_OK;
+}
+
+}  // extern "C"

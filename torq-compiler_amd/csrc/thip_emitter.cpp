@@ -1,0 +1,1001 @@
+// Compile side: a TorqHL-level program (the ops that the reference's
+// Linalg->TorqHL patterns produce, with the reference's operand and attribute
+// names) is turned into a dispatch descriptor for the gfx950 kernels.
+//
+// This takes the place of the NPU-specific tail of the reference pipeline:
+//   * KernelSelection (compiler/torq/Codegen/KernelSelectionPass.cpp:411-636):
+//     there weights become O/4.I.H.W.4 blocks for the NPU ALU; here they become a
+//     K-contiguous [Np][Kp] matrix, k = (kh, kw, ci), zero padded to whole tiles,
+//     which is what one lane of v_mfma_i32_32x32x32_i8 reads with a 128-bit load.
+//   * EncodeTensors / scale_bias handling: the interleaved [bias, scale] vector
+//     (compiler/torq/Utils/ConversionUtils.cpp:88-103) is split into two arrays.
+//   * ConvertNhwcOpToNchw + OptimizeTransposeLayout
+//     (compiler/torq/Transforms/Linalg/ConvertNhwcOpToNchwPass.cpp:308-321):
+//     the ops arrive NCHW; kernels run NHWC.  Intermediates stay NHWC in memory,
+//     so transposes only materialise at NCHW bindings.
+//   * serializeTorqHW (compiler/torq/Serialization/Serialization.cpp:265-302).
+#include <stdlib.h>
+#include <string.h>
+
+#include <algorithm>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "thip_descriptor.h"
+#include "thip_kernels.h"
+#include "thip_status.h"
+
+namespace thip {
+
+enum ValueKind { kValueBinding = 0, kValueConstant = 1, kValueTensor = 2 };
+
+struct Value {
+    ValueKind kind;
+    int32_t dtype;
+    int32_t rank;
+    int64_t shape[THIP_MAX_RANK];
+    uint32_t binding;
+    std::vector<uint8_t> data;
+    int64_t numel() const {
+        int64_t n = 1;
+        for (int i = 0; i < rank; i++) n *= shape[i];
+        return n;
+    }
+};
+
+enum HlKind { kHlConv2d, kHlDepthwise, kHlFullyConnected, kHlMatmul, kHlMaxPool, kHlAvgPool, kHlAdd, kHlTranspose };
+
+struct HlOp {
+    HlKind kind;
+    union Body {
+        thip_hl_conv2d_t conv;
+        thip_hl_depthwise_conv2d_t dw;
+        thip_hl_fully_connected_t fc;
+        thip_hl_matmul_t mm;
+        thip_hl_maxpool2d_t mp;
+        thip_hl_avg_pool2d_t ap;
+        thip_hl_add_t add;
+        thip_hl_transpose_t tr;
+    } u;
+    std::string name;
+};
+
+}  // namespace thip
+
+struct thip_program_t {
+    std::vector<thip::Value> values;
+    std::vector<thip::HlOp> ops;
+};
+
+namespace thip {
+
+static size_t elemSize(int32_t dtype) {
+    switch (dtype) {
+    case THIP_DTYPE_I8: return 1;
+    case THIP_DTYPE_I16: return 2;
+    case THIP_DTYPE_I32: return 4;
+    default: return 0;
+    }
+}
+
+static int64_t roundUp(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
+
+// Where a value lives while the program is being laid out.
+struct ValState {
+    bool defined = false;
+    DescRef ref = {kSpaceNone, 0, 0};
+    // The tensor is declared N,C,H,W but stored N,H,W,C (an intermediate between
+    // two NCHW ops: the transposes the reference inserts around each cancel).
+    bool nhwcOfNchw = false;
+};
+
+struct Dims4 {
+    int64_t N, C, H, W;
+};
+
+class Emitter {
+  public:
+    explicit Emitter(const thip_program_t &prog) : prog_(prog), state_(prog.values.size()) {}
+
+    thip_status_t run(void **outBlob, size_t *outSize);
+
+  private:
+    const thip_program_t &prog_;
+    std::vector<ValState> state_;
+    std::vector<DescOp> ops_;
+    std::vector<uint64_t> temps_;
+    std::vector<std::vector<uint8_t>> consts_;
+    std::map<uint32_t, DescBinding> bindings_;
+
+    thip_status_t checkValue(thip_value_t v, const char *what, const Value **out) const {
+        if (v < 0 || (size_t)v >= prog_.values.size()) {
+            return fail(THIP_INVALID_ARGUMENT, "%s: value %d does not exist", what, (int)v);
+        }
+        *out = &prog_.values[v];
+        return THIP_OK;
+    }
+
+    DescRef newTemp(uint64_t size) {
+        temps_.push_back(size);
+        return DescRef{kSpaceTemp, (uint32_t)(temps_.size() - 1), 0};
+    }
+
+    template <typename T>
+    DescRef newConst(const std::vector<T> &data) {
+        std::vector<uint8_t> bytes(data.size() * sizeof(T));
+        if (!bytes.empty()) memcpy(bytes.data(), data.data(), bytes.size());
+        consts_.push_back(std::move(bytes));
+        return DescRef{kSpaceConst, (uint32_t)(consts_.size() - 1), 0};
+    }
+
+    DescRef bindingRef(const Value &v, bool written) {
+        DescBinding &b = bindings_[v.binding];
+        b.id = v.binding;
+        b.flags |= written ? kBindingWritten : kBindingRead;
+        b.size = std::max<uint64_t>(b.size, (uint64_t)v.numel() * elemSize(v.dtype));
+        return DescRef{kSpaceBinding, v.binding, 0};
+    }
+
+    // Reference to the bytes of an input value exactly as declared.
+    thip_status_t literalInput(thip_value_t id, const char *what, DescRef *out) {
+        const Value *v;
+        if (thip_status_t s = checkValue(id, what, &v)) return s;
+        if (v->kind == kValueBinding) {
+            *out = bindingRef(*v, false);
+        } else if (v->kind == kValueConstant) {
+            if (!state_[id].defined) {
+                state_[id].ref = newConst(v->data);
+                state_[id].defined = true;
+            }
+            *out = state_[id].ref;
+        } else {
+            if (!state_[id].defined) {
+                return fail(THIP_FAILED_PRECONDITION, "%s: intermediate tensor %d is read before any op writes it",
+                            what, (int)id);
+            }
+            *out = state_[id].ref;
+        }
+        return THIP_OK;
+    }
+
+    void emitTranspose(DescRef in, DescRef out, int64_t B, int64_t R, int64_t S) {
+        DescOp op;
+        memset(&op, 0, sizeof(op));
+        op.kind = kKindTranspose;
+        op.TB = (int32_t)B;
+        op.TR = (int32_t)R;
+        op.TS = (int32_t)S;
+        op.in0 = in;
+        op.out = out;
+        ops_.push_back(op);
+    }
+
+    // A 4-D int8 activation operand, delivered to the kernel as NHWC.
+    thip_status_t nhwcInput(thip_value_t id, bool declaredNhwc, const char *what, Dims4 *dims, DescRef *out) {
+        const Value *v;
+        if (thip_status_t s = checkValue(id, what, &v)) return s;
+        if (v->rank != 4) return fail(THIP_INVALID_ARGUMENT, "%s: expected a rank-4 tensor, got rank %d", what, v->rank);
+        if (v->dtype != THIP_DTYPE_I8) return fail(THIP_UNIMPLEMENTED, "%s: only int8 activations are supported", what);
+        if (declaredNhwc) {
+            *dims = Dims4{v->shape[0], v->shape[3], v->shape[1], v->shape[2]};
+        } else {
+            *dims = Dims4{v->shape[0], v->shape[1], v->shape[2], v->shape[3]};
+        }
+        if (dims->N <= 0 || dims->C <= 0 || dims->H <= 0 || dims->W <= 0) {
+            return fail(THIP_INVALID_ARGUMENT, "%s: empty tensor", what);
+        }
+        DescRef lit;
+        if (thip_status_t s = literalInput(id, what, &lit)) return s;
+        const bool storedNhwc = declaredNhwc || state_[id].nhwcOfNchw || dims->C == 1 || dims->H * dims->W == 1;
+        if (declaredNhwc && state_[id].nhwcOfNchw) {
+            return fail(THIP_INVALID_ARGUMENT, "%s: tensor %d was produced as N,C,H,W but is consumed as N,H,W,C", what, (int)id);
+        }
+        if (storedNhwc) {
+            *out = lit;
+            return THIP_OK;
+        }
+        // literal NCHW in memory: transpose [N][C][HW] -> [N][HW][C]
+        DescRef t = newTemp((uint64_t)v->numel());
+        emitTranspose(lit, t, dims->N, dims->C, dims->H * dims->W);
+        *out = t;
+        return THIP_OK;
+    }
+
+    // The init operand of an op whose kernel writes NHWC.  Returns the buffer
+    // the kernel writes; *post is set when a transpose into the real
+    // destination has to follow (finishOutput emits it).
+    struct Pending {
+        bool needed = false;
+        DescRef from, to;
+        int64_t B = 0, R = 0, S = 0;
+    };
+    thip_status_t nhwcOutput(thip_value_t id, bool declaredNhwc, const char *what, int32_t dtype, int64_t N,
+                             int64_t C, int64_t H, int64_t W, DescRef *out, Pending *post) {
+        const Value *v;
+        if (thip_status_t s = checkValue(id, what, &v)) return s;
+        if (v->rank != 4) return fail(THIP_INVALID_ARGUMENT, "%s: expected a rank-4 init tensor", what);
+        const int64_t want[4] = {N, declaredNhwc ? H : C, declaredNhwc ? W : H, declaredNhwc ? C : W};
+        for (int i = 0; i < 4; i++) {
+            if (v->shape[i] != want[i]) {
+                return fail(THIP_INVALID_ARGUMENT, "%s: init dimension %d is %lld, the op produces %lld", what, i,
+                            (long long)v->shape[i], (long long)want[i]);
+            }
+        }
+        if (v->dtype != dtype) return fail(THIP_INVALID_ARGUMENT, "%s: init element type mismatch", what);
+        if (v->kind == kValueConstant) return fail(THIP_INVALID_ARGUMENT, "%s: init cannot be a constant", what);
+        const uint64_t bytes = (uint64_t)v->numel() * elemSize(dtype);
+        const bool sameInMemory = declaredNhwc || C == 1 || H * W == 1;
+        if (v->kind == kValueTensor) {
+            state_[id].ref = newTemp(bytes);
+            state_[id].defined = true;
+            state_[id].nhwcOfNchw = !sameInMemory;
+            *out = state_[id].ref;
+            return THIP_OK;
+        }
+        DescRef b = bindingRef(*v, true);
+        if (sameInMemory) {
+            *out = b;
+            return THIP_OK;
+        }
+        if (elemSize(dtype) != 1) {
+            return fail(THIP_UNIMPLEMENTED, "%s: N,C,H,W outputs wider than 8 bits need nhwc_input", what);
+        }
+        DescRef t = newTemp(bytes);
+        post->needed = true;
+        post->from = t;
+        post->to = b;
+        post->B = N;
+        post->R = H * W;
+        post->S = C;
+        *out = t;
+        return THIP_OK;
+    }
+    void finishOutput(const Pending &post) {
+        if (post.needed) emitTranspose(post.from, post.to, post.B, post.R, post.S);
+    }
+
+    // An output written in its declared order (FC, matmul, avg pool).
+    thip_status_t literalOutput(thip_value_t id, const char *what, int32_t dtype, int64_t numel, DescRef *out) {
+        const Value *v;
+        if (thip_status_t s = checkValue(id, what, &v)) return s;
+        if (v->dtype != dtype) return fail(THIP_INVALID_ARGUMENT, "%s: init element type mismatch", what);
+        if (v->numel() != numel) {
+            return fail(THIP_INVALID_ARGUMENT, "%s: init holds %lld elements, the op produces %lld", what,
+                        (long long)v->numel(), (long long)numel);
+        }
+        if (v->kind == kValueConstant) return fail(THIP_INVALID_ARGUMENT, "%s: init cannot be a constant", what);
+        if (v->kind == kValueTensor) {
+            state_[id].ref = newTemp((uint64_t)numel * elemSize(dtype));
+            state_[id].defined = true;
+            state_[id].nhwcOfNchw = false;
+            *out = state_[id].ref;
+        } else {
+            *out = bindingRef(*v, true);
+        }
+        return THIP_OK;
+    }
+
+    thip_status_t constantData(thip_value_t id, const char *what, int32_t dtype, const Value **out) const {
+        const Value *v;
+        if (thip_status_t s = checkValue(id, what, &v)) return s;
+        if (v->kind != kValueConstant) {
+            return fail(THIP_UNIMPLEMENTED, "%s: must be a compile-time constant", what);
+        }
+        if (v->dtype != dtype) return fail(THIP_INVALID_ARGUMENT, "%s: wrong element type", what);
+        *out = v;
+        return THIP_OK;
+    }
+
+    // Splits the interleaved [bias, scale] vector into two arrays padded to `padded`.
+    thip_status_t splitScaleBias(thip_value_t id, const char *what, int64_t channels, int64_t padded, bool single,
+                                 DescRef *bias, DescRef *scale) {
+        const Value *v;
+        if (thip_status_t s = constantData(id, what, THIP_DTYPE_I32, &v)) return s;
+        const int64_t need = single ? 2 : 2 * channels;
+        if (v->numel() < need) {
+            return fail(THIP_INVALID_ARGUMENT, "%s: holds %lld int32 values, %lld needed", what, (long long)v->numel(),
+                        (long long)need);
+        }
+        const int32_t *sb = (const int32_t *)v->data.data();
+        std::vector<int32_t> b((size_t)padded, 0), s((size_t)padded, 0);
+        for (int64_t c = 0; c < channels; c++) {
+            b[(size_t)c] = sb[single ? 0 : 2 * c];
+            s[(size_t)c] = sb[single ? 1 : 2 * c + 1];
+        }
+        *bias = newConst(b);
+        *scale = newConst(s);
+        return THIP_OK;
+    }
+
+    static thip_status_t checkRequant(const char *what, int32_t shift, int32_t zp, int32_t mn, int32_t mx, int32_t dtype) {
+        // act_rsh is a 6-bit field and the zero point a 16-bit one:
+        // third_party/torq-hw/ct/torq_api.c:572-575.
+        if (shift < 0 || shift > 63) return fail(THIP_INVALID_ARGUMENT, "%s: shift %d is outside 0..63", what, shift);
+        if (zp < -32768 || zp > 32767) return fail(THIP_INVALID_ARGUMENT, "%s: output_zp %d does not fit 16 bits", what, zp);
+        if (mn > mx) return fail(THIP_INVALID_ARGUMENT, "%s: output_min > output_max", what);
+        int64_t lo = 0, hi = 0;
+        switch (dtype) {
+        case THIP_DTYPE_I8: lo = -128; hi = 127; break;
+        case THIP_DTYPE_I16: lo = -32768; hi = 32767; break;
+        default: lo = INT32_MIN; hi = INT32_MAX; break;
+        }
+        if (mn < lo || mx > hi) {
+            return fail(THIP_INVALID_ARGUMENT, "%s: clamp [%d, %d] exceeds the output element type", what, mn, mx);
+        }
+        return THIP_OK;
+    }
+
+    static uint32_t chooseIgemmVariant(int64_t M, int64_t N) {
+        if (const char *env = getenv("THIP_IGEMM_VARIANT")) {
+            const long v = strtol(env, nullptr, 10);
+            if (v >= 0 && v < (long)kIgemmVariantCount) return (uint32_t)v;
+        }
+        auto tiles = [&](uint32_t v) {
+            const IgemmTile &t = igemmTile(v);
+            return ((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn);
+        };
+        // Enough 128x128 tiles to give every CU work; otherwise the small tile.
+        if (tiles(kIgemm128x128x64) >= 256) return kIgemm128x128x64;
+        return kIgemm64x64x64;
+    }
+
+    // conv2d / fully_connected / matmul as one igemm record.  `wAt(n, k)` returns
+    // weight (n, k) with k = (kh * KW + kw) * C + ci.
+    template <typename WeightAt>
+    void emitIgemm(DescOp base, int64_t M, int64_t N, int64_t K, bool dense, WeightAt wAt) {
+        const uint32_t variant = chooseIgemmVariant(M, N);
+        const IgemmTile &t = igemmTile(variant);
+        const int64_t Kp = roundUp(K, t.bk), Np = roundUp(N, t.bn);
+        std::vector<int8_t> packed((size_t)(Np * Kp), 0);
+        for (int64_t n = 0; n < N; n++) {
+            for (int64_t k = 0; k < K; k++) packed[(size_t)(n * Kp + k)] = wAt(n, k);
+        }
+        base.kind = kKindIgemm;
+        base.variant = variant;
+        base.M = (int32_t)M;
+        base.K = (int32_t)K;
+        base.Kp = (int32_t)Kp;
+        base.Nn = (int32_t)N;
+        base.Np = (int32_t)Np;
+        base.weights = newConst(packed);
+        if (dense) {
+            base.loader = kLoaderDense;
+            base.gran = 16;
+        } else {
+            base.loader = kLoaderGather;
+            int g = 16;
+            while (base.C % g != 0) g /= 2;
+            base.gran = (uint32_t)g;
+            std::vector<uint32_t> tab((size_t)(Kp / g));
+            for (int64_t e = 0; e < Kp / g; e++) {
+                const int64_t k = e * g;
+                if (k >= K) {
+                    tab[(size_t)e] = kKEntryInvalid;
+                } else {
+                    const int64_t pos = k / base.C, ci = k % base.C;
+                    tab[(size_t)e] = packKEntry((int)(pos / base.KW), (int)(pos % base.KW), (int)ci);
+                }
+            }
+            base.table = newConst(tab);
+        }
+        ops_.push_back(base);
+    }
+
+    thip_status_t emitConv2d(const thip_hl_conv2d_t &c);
+    thip_status_t emitDepthwise(const thip_hl_depthwise_conv2d_t &c);
+    thip_status_t emitFullyConnected(const thip_hl_fully_connected_t &c);
+    thip_status_t emitMatmul(const thip_hl_matmul_t &c);
+    thip_status_t emitMaxPool(const thip_hl_maxpool2d_t &c);
+    thip_status_t emitAvgPool(const thip_hl_avg_pool2d_t &c);
+    thip_status_t emitAdd(const thip_hl_add_t &c);
+    thip_status_t emitTransposeOp(const thip_hl_transpose_t &c);
+};
+
+static thip_status_t windowGeometry(const char *what, int64_t H, int64_t W, int64_t KH, int64_t KW, const int64_t pad[4],
+                                    const int64_t stride[2], int64_t *OH, int64_t *OW) {
+    if (stride[0] <= 0 || stride[1] <= 0) return fail(THIP_INVALID_ARGUMENT, "%s: stride must be positive", what);
+    for (int i = 0; i < 4; i++) {
+        if (pad[i] < 0) return fail(THIP_INVALID_ARGUMENT, "%s: negative padding", what);
+    }
+    if (KH <= 0 || KW <= 0 || KH > 127 || KW > 255) return fail(THIP_INVALID_ARGUMENT, "%s: unsupported window %lldx%lld", what, (long long)KH, (long long)KW);
+    const int64_t spanH = H + pad[2] + pad[3] - KH, spanW = W + pad[0] + pad[1] - KW;
+    if (spanH < 0 || spanW < 0) return fail(THIP_INVALID_ARGUMENT, "%s: window larger than the padded input", what);
+    *OH = spanH / stride[0] + 1;
+    *OW = spanW / stride[1] + 1;
+    return THIP_OK;
+}
+
+static bool fitsInt32(int64_t v) { return v > 0 && v < (1LL << 31); }
+
+thip_status_t Emitter::emitConv2d(const thip_hl_conv2d_t &c) {
+    const char *what = "torq_hl.conv2d";
+    if (c.groups != 1) return fail(THIP_UNIMPLEMENTED, "%s: groups must be 1", what);
+    if (c.weight_zp != 0) return fail(THIP_UNIMPLEMENTED, "%s: weight_zp must be 0 (the patterns fold it into the weights)", what);
+    if (c.dilation[0] != 1 || c.dilation[1] != 1) return fail(THIP_UNIMPLEMENTED, "%s: dilation must be [1,1] (the patterns fold it into the weights)", what);
+    if (c.segment_output) return fail(THIP_UNIMPLEMENTED, "%s: segment_output is an NPU memory layout", what);
+    if (c.input_zp < -128 || c.input_zp > 127) return fail(THIP_INVALID_ARGUMENT, "%s: input_zp outside int8", what);
+    const Value *w;
+    if (thip_status_t s = constantData(c.weights, "torq_hl.conv2d weights", THIP_DTYPE_I8, &w)) return s;
+    if (w->rank != 4) return fail(THIP_INVALID_ARGUMENT, "%s: weights must be O,I,KH,KW", what);
+    const Value *init;
+    if (thip_status_t s = checkValue(c.init, "torq_hl.conv2d init", &init)) return s;
+    if (thip_status_t s = checkRequant(what, c.shift_factor, c.output_zp, c.output_min, c.output_max, init->dtype)) return s;
+    Dims4 d;
+    DescRef in;
+    if (thip_status_t s = nhwcInput(c.input, c.nhwc_input != 0, "torq_hl.conv2d input", &d, &in)) return s;
+    const int64_t O = w->shape[0], I = w->shape[1], KH = w->shape[2], KW = w->shape[3];
+    if (I != d.C) return fail(THIP_INVALID_ARGUMENT, "%s: weights expect %lld input channels, input has %lld", what, (long long)I, (long long)d.C);
+    if (d.C > 65535) return fail(THIP_UNIMPLEMENTED, "%s: more than 65535 input channels", what);
+    int64_t OH, OW;
+    if (thip_status_t s = windowGeometry(what, d.H, d.W, KH, KW, c.pad, c.stride, &OH, &OW)) return s;
+    const int64_t M = d.N * OH * OW, K = KH * KW * d.C;
+    if (!fitsInt32(M) || !fitsInt32(K) || !fitsInt32(M * O) || !fitsInt32(d.N * d.H * d.W * d.C)) {
+        return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
+    }
+    DescOp op;
+    memset(&op, 0, sizeof(op));
+    DescRef out;
+    Pending post;
+    if (thip_status_t s = nhwcOutput(c.init, c.nhwc_input != 0, "torq_hl.conv2d init", init->dtype, d.N, O, OH, OW, &out, &post)) return s;
+    const int64_t tile = 256;
+    if (thip_status_t s = splitScaleBias(c.scale_bias, "torq_hl.conv2d scale_bias", O, roundUp(O, tile), false, &op.bias, &op.scale)) return s;
+    op.out_dtype = init->dtype;
+    op.input_zp = c.input_zp;
+    op.output_zp = c.output_zp;
+    op.output_min = c.output_min;
+    op.output_max = c.output_max;
+    op.shift = c.shift_factor;
+    op.N = (int32_t)d.N; op.H = (int32_t)d.H; op.W = (int32_t)d.W; op.C = (int32_t)d.C;
+    op.OH = (int32_t)OH; op.OW = (int32_t)OW; op.OC = (int32_t)O;
+    op.KH = (int32_t)KH; op.KW = (int32_t)KW; op.SH = (int32_t)c.stride[0]; op.SW = (int32_t)c.stride[1];
+    op.PL = (int32_t)c.pad[0]; op.PR = (int32_t)c.pad[1]; op.PT = (int32_t)c.pad[2]; op.PB = (int32_t)c.pad[3];
+    op.in0 = in;
+    op.out = out;
+    const int8_t *wd = (const int8_t *)w->data.data();
+    const bool pointwise = KH == 1 && KW == 1 && c.stride[0] == 1 && c.stride[1] == 1 && c.pad[0] == 0 &&
+                           c.pad[1] == 0 && c.pad[2] == 0 && c.pad[3] == 0;
+    const int64_t C = d.C;
+    emitIgemm(op, M, O, K, pointwise && K % 16 == 0, [&](int64_t n, int64_t k) {
+        const int64_t pos = k / C, ci = k % C;
+        const int64_t kh = pos / KW, kw = pos % KW;
+        return wd[((n * C + ci) * KH + kh) * KW + kw];
+    });
+    finishOutput(post);
+    return THIP_OK;
+}
+
+thip_status_t Emitter::emitDepthwise(const thip_hl_depthwise_conv2d_t &c) {
+    const char *what = "torq_hl.depthwise_conv2d";
+    if (c.weight_zp != 0) return fail(THIP_UNIMPLEMENTED, "%s: weight_zp must be 0", what);
+    if (c.dilation[0] != 1 || c.dilation[1] != 1) return fail(THIP_UNIMPLEMENTED, "%s: dilation must be [1,1]", what);
+    if (c.segment_output) return fail(THIP_UNIMPLEMENTED, "%s: segment_output is an NPU memory layout", what);
+    if (c.is_dw1d_stride1) return fail(THIP_UNIMPLEMENTED, "%s: is_dw1d_stride1 is the bf16 1-D special case", what);
+    if (c.input_zp < -128 || c.input_zp > 127) return fail(THIP_INVALID_ARGUMENT, "%s: input_zp outside int8", what);
+    const Value *w;
+    if (thip_status_t s = constantData(c.weights, "torq_hl.depthwise_conv2d weights", THIP_DTYPE_I8, &w)) return s;
+    if (w->rank != 4 || w->shape[1] != 1) return fail(THIP_INVALID_ARGUMENT, "%s: weights must be C,1,KH,KW", what);
+    const Value *init;
+    if (thip_status_t s = checkValue(c.init, "torq_hl.depthwise_conv2d init", &init)) return s;
+    if (init->dtype != THIP_DTYPE_I8) return fail(THIP_UNIMPLEMENTED, "%s: only int8 outputs", what);
+    if (thip_status_t s = checkRequant(what, c.shift_factor, c.output_zp, c.output_min, c.output_max, init->dtype)) return s;
+    Dims4 d;
+    DescRef in;
+    if (thip_status_t s = nhwcInput(c.input, c.nhwc_input != 0, "torq_hl.depthwise_conv2d input", &d, &in)) return s;
+    const int64_t C = w->shape[0], KH = w->shape[2], KW = w->shape[3];
+    if (C != d.C) return fail(THIP_INVALID_ARGUMENT, "%s: weights have %lld channels, input has %lld", what, (long long)C, (long long)d.C);
+    if (c.groups != C && c.groups != 1 && c.groups != 0) return fail(THIP_INVALID_ARGUMENT, "%s: groups must equal the channel count", what);
+    int64_t OH, OW;
+    if (thip_status_t s = windowGeometry(what, d.H, d.W, KH, KW, c.pad, c.stride, &OH, &OW)) return s;
+    if (!fitsInt32(d.N * OH * OW * C) || !fitsInt32(d.N * d.H * d.W * C)) return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
+    DescOp op;
+    memset(&op, 0, sizeof(op));
+    DescRef out;
+    Pending post;
+    if (thip_status_t s = nhwcOutput(c.init, c.nhwc_input != 0, "torq_hl.depthwise_conv2d init", init->dtype, d.N, C, OH, OW, &out, &post)) return s;
+    if (thip_status_t s = splitScaleBias(c.scale_bias, "torq_hl.depthwise_conv2d scale_bias", C, roundUp(C, 16), false, &op.bias, &op.scale)) return s;
+    const int8_t *wd = (const int8_t *)w->data.data();
+    std::vector<int8_t> wpk((size_t)(KH * KW * C));
+    for (int64_t ch = 0; ch < C; ch++) {
+        for (int64_t k = 0; k < KH * KW; k++) wpk[(size_t)(k * C + ch)] = wd[ch * KH * KW + k];
+    }
+    op.kind = kKindDepthwise;
+    op.out_dtype = init->dtype;
+    op.input_zp = c.input_zp;
+    op.output_zp = c.output_zp;
+    op.output_min = c.output_min;
+    op.output_max = c.output_max;
+    op.shift = c.shift_factor;
+    op.N = (int32_t)d.N; op.H = (int32_t)d.H; op.W = (int32_t)d.W; op.C = (int32_t)C;
+    op.OH = (int32_t)OH; op.OW = (int32_t)OW; op.OC = (int32_t)C;
+    op.KH = (int32_t)KH; op.KW = (int32_t)KW; op.SH = (int32_t)c.stride[0]; op.SW = (int32_t)c.stride[1];
+    op.PL = (int32_t)c.pad[0]; op.PR = (int32_t)c.pad[1]; op.PT = (int32_t)c.pad[2]; op.PB = (int32_t)c.pad[3];
+    op.in0 = in;
+    op.out = out;
+    op.weights = newConst(wpk);
+    ops_.push_back(op);
+    finishOutput(post);
+    return THIP_OK;
+}
+
+thip_status_t Emitter::emitFullyConnected(const thip_hl_fully_connected_t &c) {
+    const char *what = "torq_hl.fully_connected";
+    if (c.weight_zp != 0) return fail(THIP_UNIMPLEMENTED, "%s: weight_zp must be 0", what);
+    const Value *w;
+    if (thip_status_t s = constantData(c.weights, "torq_hl.fully_connected weights", THIP_DTYPE_I8, &w)) return s;
+    if (w->rank != 2) return fail(THIP_INVALID_ARGUMENT, "%s: weights must be N,K", what);
+    const int64_t N = w->shape[0], K = w->shape[1];
+    const Value *x;
+    if (thip_status_t s = checkValue(c.input, "torq_hl.fully_connected input", &x)) return s;
+    if (x->dtype != THIP_DTYPE_I8) return fail(THIP_UNIMPLEMENTED, "%s: only int8 inputs", what);
+    if (x->rank < 1 || x->shape[x->rank - 1] != K) {
+        // a flattened N,C,1,1 / N,1,1,C activation is accepted as M,K too
+        if (K <= 0 || x->numel() % K != 0) return fail(THIP_INVALID_ARGUMENT, "%s: input does not end in K=%lld", what, (long long)K);
+    }
+    if (state_[c.input].nhwcOfNchw) {
+        return fail(THIP_UNIMPLEMENTED, "%s: input %d is an N,C,H,W intermediate with H*W > 1; flatten needs a transpose", what, (int)c.input);
+    }
+    const int64_t M = x->numel() / K;
+    const Value *init;
+    if (thip_status_t s = checkValue(c.init, "torq_hl.fully_connected init", &init)) return s;
+    if (thip_status_t s = checkRequant(what, c.shift_factor, c.output_zp, c.output_min, c.output_max, init->dtype)) return s;
+    if (!fitsInt32(M) || !fitsInt32(K) || !fitsInt32(N) || !fitsInt32(M * N) || !fitsInt32(M * K)) {
+        return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
+    }
+    DescOp op;
+    memset(&op, 0, sizeof(op));
+    if (thip_status_t s = literalInput(c.input, "torq_hl.fully_connected input", &op.in0)) return s;
+    if (thip_status_t s = literalOutput(c.init, "torq_hl.fully_connected init", init->dtype, M * N, &op.out)) return s;
+    op.out_dtype = init->dtype;
+    op.input_zp = c.input_zp;
+    op.output_zp = c.output_zp;
+    op.output_min = c.output_min;
+    op.output_max = c.output_max;
+    op.shift = c.shift_factor;
+    const int8_t *wd = (const int8_t *)w->data.data();
+    const bool skinnyOff = getenv("THIP_NO_SKINNY") != nullptr;
+    if (M <= kFcSkinnyMaxRows && K % 16 == 0 && !skinnyOff) {
+        if (thip_status_t s = splitScaleBias(c.scale_bias, "torq_hl.fully_connected scale_bias", N, N, false, &op.bias, &op.scale)) return s;
+        op.kind = kKindFcSkinny;
+        op.M = (int32_t)M; op.K = (int32_t)K; op.Kp = (int32_t)K; op.Nn = (int32_t)N; op.Np = (int32_t)N;
+        op.weights = newConst(w->data);
+        ops_.push_back(op);
+        return THIP_OK;
+    }
+    if (thip_status_t s = splitScaleBias(c.scale_bias, "torq_hl.fully_connected scale_bias", N, roundUp(N, 256), false, &op.bias, &op.scale)) return s;
+    // as a 1x1 convolution over an M x 1 x 1 x K image
+    op.N = (int32_t)M; op.H = 1; op.W = 1; op.C = (int32_t)K;
+    op.OH = 1; op.OW = 1; op.OC = (int32_t)N;
+    op.KH = 1; op.KW = 1; op.SH = 1; op.SW = 1;
+    emitIgemm(op, M, N, K, K % 16 == 0, [&](int64_t n, int64_t k) { return wd[n * K + k]; });
+    return THIP_OK;
+}
+
+thip_status_t Emitter::emitMatmul(const thip_hl_matmul_t &c) {
+    const char *what = "torq_hl.matmul";
+    const Value *a, *b, *init;
+    if (thip_status_t s = checkValue(c.input1, "torq_hl.matmul input1", &a)) return s;
+    if (thip_status_t s = checkValue(c.input2, "torq_hl.matmul input2", &b)) return s;
+    if (thip_status_t s = checkValue(c.init, "torq_hl.matmul init", &init)) return s;
+    if (a->dtype != THIP_DTYPE_I8 || b->dtype != THIP_DTYPE_I8) return fail(THIP_UNIMPLEMENTED, "%s: only int8 inputs", what);
+    if (a->rank < 2 || a->rank > 3 || b->rank < 2 || b->rank > 3) return fail(THIP_UNIMPLEMENTED, "%s: operands must have rank 2 or 3", what);
+    if (state_[c.input1].nhwcOfNchw || state_[c.input2].nhwcOfNchw) return fail(THIP_UNIMPLEMENTED, "%s: N,C,H,W intermediates are not accepted", what);
+    const int64_t Ba = a->rank == 3 ? a->shape[0] : 1, Bb = b->rank == 3 ? b->shape[0] : 1;
+    const int64_t M = a->shape[a->rank - 2], K = a->shape[a->rank - 1];
+    const int64_t K2 = b->shape[b->rank - 2], N = b->shape[b->rank - 1];
+    if (K != K2) return fail(THIP_INVALID_ARGUMENT, "%s: inner dimensions differ (%lld vs %lld)", what, (long long)K, (long long)K2);
+    const int64_t B = std::max(Ba, Bb);
+    if ((Ba != B && Ba != 1) || (Bb != B && Bb != 1)) return fail(THIP_INVALID_ARGUMENT, "%s: batch dimensions do not broadcast", what);
+    if (thip_status_t s = checkRequant(what, c.shift, c.output_zp, c.output_min, c.output_max, init->dtype)) return s;
+    if (!fitsInt32(B * M * N) || !fitsInt32(B * M * K) || !fitsInt32(B * K * N)) return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
+    DescRef aRef, outRef;
+    if (thip_status_t s = literalInput(c.input1, "torq_hl.matmul input1", &aRef)) return s;
+    if (thip_status_t s = literalOutput(c.init, "torq_hl.matmul init", init->dtype, B * M * N, &outRef)) return s;
+    DescOp op;
+    memset(&op, 0, sizeof(op));
+    op.out_dtype = init->dtype;
+    op.output_zp = c.output_zp;
+    op.output_min = c.output_min;
+    op.output_max = c.output_max;
+    op.shift = c.shift;
+    op.H = 1; op.W = 1; op.C = (int32_t)K; op.OH = 1; op.OW = 1; op.OC = (int32_t)N;
+    op.KH = 1; op.KW = 1; op.SH = 1; op.SW = 1;
+    const size_t outElem = elemSize(init->dtype);
+    if (b->kind == kValueConstant) {
+        // weights known at compile time: pack per batch (one record when B is broadcast)
+        const int8_t *bd = (const int8_t *)b->data.data();
+        const int64_t records = Bb == 1 ? 1 : B;
+        for (int64_t r = 0; r < records; r++) {
+            DescOp o = op;
+            const int64_t rows = Bb == 1 ? (Ba == 1 ? M : B * M) : M;
+            o.N = (int32_t)rows;
+            o.in0 = aRef;
+            o.in0.offset += (uint64_t)(Ba == 1 ? 0 : r * M * K);
+            o.out = outRef;
+            o.out.offset += (uint64_t)(r * M * N) * outElem;
+            if (thip_status_t s = splitScaleBias(c.scale_bias, "torq_hl.matmul scale_bias", N, roundUp(N, 256), true, &o.bias, &o.scale)) return s;
+            const int8_t *bb = bd + (Bb == 1 ? 0 : r * K * N);
+            emitIgemm(o, rows, N, K, K % 16 == 0, [&](int64_t n, int64_t k) { return bb[k * N + n]; });
+        }
+        return THIP_OK;
+    }
+    // input2 produced at run time: transpose each batch into a zero-padded
+    // [Np][Kp] buffer (intermediates are zero-filled when the executable is
+    // created and the padding is never written), then run the dense igemm.
+    DescRef bRef;
+    if (thip_status_t s = literalInput(c.input2, "torq_hl.matmul input2", &bRef)) return s;
+    if (K % 16 != 0) return fail(THIP_UNIMPLEMENTED, "%s: a run-time input2 needs K %% 16 == 0", what);
+    const uint32_t variant = chooseIgemmVariant(M, N);
+    const IgemmTile &t = igemmTile(variant);
+    const int64_t Kp = roundUp(K, t.bk), Np = roundUp(N, t.bn);
+    if (Kp != K) return fail(THIP_UNIMPLEMENTED, "%s: a run-time input2 needs K %% %d == 0", what, t.bk);
+    std::vector<DescRef> packed;
+    for (int64_t r = 0; r < (Bb == 1 ? 1 : B); r++) {
+        DescRef t2 = newTemp((uint64_t)(Np * Kp));
+        DescRef src = bRef;
+        src.offset += (uint64_t)(r * K * N);
+        emitTranspose(src, t2, 1, K, N);
+        packed.push_back(t2);
+    }
+    for (int64_t batch = 0; batch < B; batch++) {
+        DescOp o = op;
+        o.kind = kKindIgemm;
+        o.variant = variant;
+        o.loader = kLoaderDense;
+        o.gran = 16;
+        o.N = (int32_t)M;
+        o.M = (int32_t)M; o.K = (int32_t)K; o.Kp = (int32_t)Kp; o.Nn = (int32_t)N; o.Np = (int32_t)Np;
+        o.in0 = aRef;
+        o.in0.offset += (uint64_t)(Ba == 1 ? 0 : batch * M * K);
+        o.out = outRef;
+        o.out.offset += (uint64_t)(batch * M * N) * outElem;
+        o.weights = packed[(size_t)(Bb == 1 ? 0 : batch)];
+        if (thip_status_t s = splitScaleBias(c.scale_bias, "torq_hl.matmul scale_bias", N, Np, true, &o.bias, &o.scale)) return s;
+        ops_.push_back(o);
+    }
+    return THIP_OK;
+}
+
+thip_status_t Emitter::emitMaxPool(const thip_hl_maxpool2d_t &c) {
+    const char *what = "torq_hl.maxpool2d";
+    if (c.segment_output) return fail(THIP_UNIMPLEMENTED, "%s: segment_output is an NPU memory layout", what);
+    if (c.input_zp < -128 || c.input_zp > 127) return fail(THIP_INVALID_ARGUMENT, "%s: input_zp outside int8", what);
+    if (c.output_min > c.output_max || c.output_min < -128 || c.output_max > 127) return fail(THIP_INVALID_ARGUMENT, "%s: clamp outside int8", what);
+    Dims4 d;
+    DescRef in;
+    if (thip_status_t s = nhwcInput(c.input, c.nhwc_input != 0, "torq_hl.maxpool2d input", &d, &in)) return s;
+    int64_t OH, OW;
+    if (thip_status_t s = windowGeometry(what, d.H, d.W, c.kernel[0], c.kernel[1], c.pad, c.stride, &OH, &OW)) return s;
+    if (!fitsInt32(d.N * d.H * d.W * d.C)) return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
+    DescOp op;
+    memset(&op, 0, sizeof(op));
+    DescRef out;
+    Pending post;
+    if (thip_status_t s = nhwcOutput(c.init, c.nhwc_input != 0, "torq_hl.maxpool2d init", THIP_DTYPE_I8, d.N, d.C, OH, OW, &out, &post)) return s;
+    op.kind = kKindMaxPool;
+    op.out_dtype = THIP_DTYPE_I8;
+    op.input_zp = c.input_zp;
+    op.output_min = c.output_min;
+    op.output_max = c.output_max;
+    op.N = (int32_t)d.N; op.H = (int32_t)d.H; op.W = (int32_t)d.W; op.C = (int32_t)d.C;
+    op.OH = (int32_t)OH; op.OW = (int32_t)OW; op.OC = (int32_t)d.C;
+    op.KH = (int32_t)c.kernel[0]; op.KW = (int32_t)c.kernel[1]; op.SH = (int32_t)c.stride[0]; op.SW = (int32_t)c.stride[1];
+    op.PL = (int32_t)c.pad[0]; op.PR = (int32_t)c.pad[1]; op.PT = (int32_t)c.pad[2]; op.PB = (int32_t)c.pad[3];
+    op.in0 = in;
+    op.out = out;
+    ops_.push_back(op);
+    finishOutput(post);
+    return THIP_OK;
+}
+
+thip_status_t Emitter::emitAvgPool(const thip_hl_avg_pool2d_t &c) {
+    const char *what = "torq_hl.avg_pool2d";
+    const Value *x, *w, *sb;
+    if (thip_status_t s = checkValue(c.input, "torq_hl.avg_pool2d input", &x)) return s;
+    if (x->rank != 4 || x->dtype != THIP_DTYPE_I8) return fail(THIP_INVALID_ARGUMENT, "%s: input must be an int8 N,H,W,C tensor", what);
+    if (state_[c.input].nhwcOfNchw) return fail(THIP_INVALID_ARGUMENT, "%s: input %d is declared N,C,H,W; insert torq_hl.transpose [0,2,3,1]", what, (int)c.input);
+    if (thip_status_t s = constantData(c.weights, "torq_hl.avg_pool2d weights", THIP_DTYPE_I8, &w)) return s;
+    if (thip_status_t s = constantData(c.scale_bias, "torq_hl.avg_pool2d scale_bias", THIP_DTYPE_I32, &sb)) return s;
+    if (w->numel() < 1 || sb->numel() < 2) return fail(THIP_INVALID_ARGUMENT, "%s: weights / scale_bias too short", what);
+    if (thip_status_t s = checkRequant(what, c.shift_factor, c.output_zp, c.output_min, c.output_max, THIP_DTYPE_I8)) return s;
+    const int64_t N = x->shape[0], H = x->shape[1], W = x->shape[2], C = x->shape[3];
+    if (!fitsInt32(N * H * W * C)) return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
+    DescOp op;
+    memset(&op, 0, sizeof(op));
+    if (thip_status_t s = literalInput(c.input, "torq_hl.avg_pool2d input", &op.in0)) return s;
+    if (thip_status_t s = literalOutput(c.init, "torq_hl.avg_pool2d init", THIP_DTYPE_I8, N * C, &op.out)) return s;
+    op.kind = kKindAvgPool;
+    op.out_dtype = THIP_DTYPE_I8;
+    op.output_zp = c.output_zp;
+    op.output_min = c.output_min;
+    op.output_max = c.output_max;
+    op.shift = c.shift_factor;
+    op.N = (int32_t)N; op.H = (int32_t)H; op.W = (int32_t)W; op.C = (int32_t)C;
+    op.w0 = ((const int8_t *)w->data.data())[0];
+    op.bias0 = ((const int32_t *)sb->data.data())[0];
+    op.scale0 = ((const int32_t *)sb->data.data())[1];
+    ops_.push_back(op);
+    return THIP_OK;
+}
+
+thip_status_t Emitter::emitAdd(const thip_hl_add_t &c) {
+    const char *what = "torq_hl.add";
+    if (c.segment_output) return fail(THIP_UNIMPLEMENTED, "%s: segment_output is an NPU memory layout", what);
+    if (c.rhs_is_scalar) return fail(THIP_UNIMPLEMENTED, "%s: rhs_is_scalar (tensor + scalar) is not on this path", what);
+    const Value *a, *b, *init, *w, *sb;
+    if (thip_status_t s = checkValue(c.input1, "torq_hl.add input1", &a)) return s;
+    if (thip_status_t s = checkValue(c.input2, "torq_hl.add input2", &b)) return s;
+    if (thip_status_t s = checkValue(c.init, "torq_hl.add init", &init)) return s;
+    if (a->dtype != THIP_DTYPE_I8 || b->dtype != THIP_DTYPE_I8 || init->dtype != THIP_DTYPE_I8) return fail(THIP_UNIMPLEMENTED, "%s: only int8 tensors", what);
+    if (a->rank != b->rank || a->rank != init->rank) return fail(THIP_INVALID_ARGUMENT, "%s: operand ranks differ (broadcast is materialised by the patterns)", what);
+    for (int i = 0; i < a->rank; i++) {
+        if (a->shape[i] != b->shape[i] || a->shape[i] != init->shape[i]) return fail(THIP_INVALID_ARGUMENT, "%s: operand shapes differ", what);
+    }
+    if (thip_status_t s = constantData(c.weights, "torq_hl.add weights", THIP_DTYPE_I16, &w)) return s;
+    if (thip_status_t s = constantData(c.scale_bias, "torq_hl.add scale_bias", THIP_DTYPE_I32, &sb)) return s;
+    if (w->numel() < 2 || sb->numel() < 2) return fail(THIP_INVALID_ARGUMENT, "%s: weights / scale_bias too short", what);
+    if (thip_status_t s = checkRequant(what, c.shift_factor, c.output_zp, c.output_min, c.output_max, THIP_DTYPE_I8)) return s;
+    DescOp op;
+    memset(&op, 0, sizeof(op));
+    op.kind = kKindAdd;
+    op.out_dtype = THIP_DTYPE_I8;
+    op.output_zp = c.output_zp;
+    op.output_min = c.output_min;
+    op.output_max = c.output_max;
+    op.shift = c.shift_factor;
+    op.w0 = ((const int16_t *)w->data.data())[0];
+    op.w1 = ((const int16_t *)w->data.data())[1];
+    op.bias0 = ((const int32_t *)sb->data.data())[0];
+    op.scale0 = ((const int32_t *)sb->data.data())[1];
+    if (!fitsInt32(a->numel())) return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
+    Pending post;
+    // Elementwise: any memory order works as long as all three agree.  If one
+    // operand is an N,C,H,W intermediate kept as NHWC, bring the others to it.
+    const bool anyNhwc = state_[c.input1].nhwcOfNchw || state_[c.input2].nhwcOfNchw;
+    if (anyNhwc && a->rank == 4) {
+        Dims4 d;
+        if (thip_status_t s = nhwcInput(c.input1, false, "torq_hl.add input1", &d, &op.in0)) return s;
+        if (thip_status_t s = nhwcInput(c.input2, false, "torq_hl.add input2", &d, &op.in1)) return s;
+        if (thip_status_t s = nhwcOutput(c.init, false, "torq_hl.add init", THIP_DTYPE_I8, d.N, d.C, d.H, d.W, &op.out, &post)) return s;
+    } else {
+        if (thip_status_t s = literalInput(c.input1, "torq_hl.add input1", &op.in0)) return s;
+        if (thip_status_t s = literalInput(c.input2, "torq_hl.add input2", &op.in1)) return s;
+        if (thip_status_t s = literalOutput(c.init, "torq_hl.add init", THIP_DTYPE_I8, a->numel(), &op.out)) return s;
+    }
+    op.N = 1; op.H = 1; op.W = 1;
+    op.C = (int32_t)a->numel();
+    ops_.push_back(op);
+    finishOutput(post);
+    return THIP_OK;
+}
+
+thip_status_t Emitter::emitTransposeOp(const thip_hl_transpose_t &c) {
+    const char *what = "torq_hl.transpose";
+    const Value *x, *init;
+    if (thip_status_t s = checkValue(c.input, "torq_hl.transpose input", &x)) return s;
+    if (thip_status_t s = checkValue(c.init, "torq_hl.transpose init", &init)) return s;
+    if (x->dtype != THIP_DTYPE_I8 || init->dtype != THIP_DTYPE_I8) return fail(THIP_UNIMPLEMENTED, "%s: only int8 tensors", what);
+    if (c.rank != x->rank || c.rank != init->rank) return fail(THIP_INVALID_ARGUMENT, "%s: rank mismatch", what);
+    for (int i = 0; i < c.rank; i++) {
+        if (c.perm[i] < 0 || c.perm[i] >= c.rank || init->shape[i] != x->shape[c.perm[i]]) {
+            return fail(THIP_INVALID_ARGUMENT, "%s: init shape is not the permuted input shape", what);
+        }
+    }
+    int64_t B = 1, R = 0, S = 0;
+    bool toNhwc = false, toNchw = false;
+    if (c.rank == 4 && c.perm[0] == 0 && c.perm[1] == 2 && c.perm[2] == 3 && c.perm[3] == 1) {
+        toNhwc = true;  // N,C,H,W -> N,H,W,C
+        B = x->shape[0]; R = x->shape[1]; S = x->shape[2] * x->shape[3];
+    } else if (c.rank == 4 && c.perm[0] == 0 && c.perm[1] == 3 && c.perm[2] == 1 && c.perm[3] == 2) {
+        toNchw = true;  // N,H,W,C -> N,C,H,W
+        B = x->shape[0]; R = x->shape[1] * x->shape[2]; S = x->shape[3];
+    } else if (c.rank == 2 && c.perm[0] == 1 && c.perm[1] == 0) {
+        R = x->shape[0]; S = x->shape[1];
+    } else if (c.rank == 3 && c.perm[0] == 0 && c.perm[1] == 2 && c.perm[2] == 1) {
+        B = x->shape[0]; R = x->shape[1]; S = x->shape[2];
+    } else {
+        return fail(THIP_UNIMPLEMENTED, "%s: unsupported permutation", what);
+    }
+    if (!fitsInt32(x->numel())) return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
+    DescRef in;
+    if (thip_status_t s = literalInput(c.input, "torq_hl.transpose input", &in)) return s;
+    const bool inNhwcOfNchw = state_[c.input].nhwcOfNchw;
+    if (init->kind == kValueTensor) {
+        // Fold with the layout the producer already wrote.
+        if (toNhwc && inNhwcOfNchw) {
+            state_[c.init] = state_[c.input];
+            state_[c.init].nhwcOfNchw = false;  // literal N,H,W,C now
+            return THIP_OK;
+        }
+        if (toNchw && !inNhwcOfNchw) {
+            state_[c.init].ref = in;
+            state_[c.init].defined = true;
+            state_[c.init].nhwcOfNchw = !(S == 1 || R == 1);
+            return THIP_OK;
+        }
+    }
+    if (inNhwcOfNchw) {
+        if (toNhwc) {
+            // bytes are already N,H,W,C: copy through a double transpose is wasteful, but
+            // a binding destination needs its own bytes; use add-free copy = transpose with R == 1
+            DescRef out;
+            if (thip_status_t s = literalOutput(c.init, "torq_hl.transpose init", THIP_DTYPE_I8, x->numel(), &out)) return s;
+            emitTranspose(in, out, 1, 1, x->numel());
+            return THIP_OK;
+        }
+        return fail(THIP_UNIMPLEMENTED, "%s: permutation of an N,C,H,W intermediate other than [0,2,3,1]", what);
+    }
+    DescRef out;
+    if (thip_status_t s = literalOutput(c.init, "torq_hl.transpose init", THIP_DTYPE_I8, x->numel(), &out)) return s;
+    emitTranspose(in, out, B, R, S);
+    return THIP_OK;
+}
+
+thip_status_t Emitter::run(void **outBlob, size_t *outSize) {
+    for (const HlOp &op : prog_.ops) {
+        thip_status_t s = THIP_OK;
+        switch (op.kind) {
+        case kHlConv2d: s = emitConv2d(op.u.conv); break;
+        case kHlDepthwise: s = emitDepthwise(op.u.dw); break;
+        case kHlFullyConnected: s = emitFullyConnected(op.u.fc); break;
+        case kHlMatmul: s = emitMatmul(op.u.mm); break;
+        case kHlMaxPool: s = emitMaxPool(op.u.mp); break;
+        case kHlAvgPool: s = emitAvgPool(op.u.ap); break;
+        case kHlAdd: s = emitAdd(op.u.add); break;
+        case kHlTranspose: s = emitTransposeOp(op.u.tr); break;
+        }
+        if (s != THIP_OK) return s;
+    }
+    if (ops_.empty()) return fail(THIP_INVALID_ARGUMENT, "program has no ops");
+
+    // Binding ids must be dense 0..n-1 so the dispatch's binding table indexes directly.
+    uint32_t bindingCount = 0;
+    for (auto &kv : bindings_) bindingCount = std::max(bindingCount, kv.first + 1);
+    std::vector<DescBinding> btable(bindingCount);
+    for (uint32_t i = 0; i < bindingCount; i++) btable[i] = DescBinding{i, 0, 0};
+    for (auto &kv : bindings_) btable[kv.first] = kv.second;
+
+    DescHeader h;
+    memset(&h, 0, sizeof(h));
+    h.magic = kMagic;
+    h.version = kDescriptorVersion;
+    h.arch = kArchGfx950;
+    h.op_count = (uint32_t)ops_.size();
+    h.binding_count = bindingCount;
+    h.temp_count = (uint32_t)temps_.size();
+    h.const_count = (uint32_t)consts_.size();
+    uint64_t off = sizeof(DescHeader);
+    h.ops_offset = off;
+    off += sizeof(DescOp) * ops_.size();
+    h.bindings_offset = off;
+    off += sizeof(DescBinding) * btable.size();
+    h.temps_offset = off;
+    off += sizeof(DescTemp) * temps_.size();
+    h.consts_offset = off;
+    off += sizeof(DescConst) * consts_.size();
+    off = (uint64_t)roundUp((int64_t)off, (int64_t)kDataAlign);
+    h.data_offset = off;
+    std::vector<DescConst> ctable(consts_.size());
+    uint64_t dataOff = 0;
+    for (size_t i = 0; i < consts_.size(); i++) {
+        ctable[i].offset = dataOff;
+        ctable[i].size = consts_[i].size();
+        dataOff = (uint64_t)roundUp((int64_t)(dataOff + consts_[i].size()), (int64_t)kDataAlign);
+    }
+    h.total_size = h.data_offset + dataOff;
+
+    uint8_t *blob = (uint8_t *)calloc(1, (size_t)h.total_size);
+    if (!blob) return fail(THIP_RESOURCE_EXHAUSTED, "out of memory serialising %llu bytes", (unsigned long long)h.total_size);
+    memcpy(blob, &h, sizeof(h));
+    memcpy(blob + h.ops_offset, ops_.data(), sizeof(DescOp) * ops_.size());
+    if (!btable.empty()) memcpy(blob + h.bindings_offset, btable.data(), sizeof(DescBinding) * btable.size());
+    for (size_t i = 0; i < temps_.size(); i++) {
+        DescTemp t{temps_[i]};
+        memcpy(blob + h.temps_offset + i * sizeof(DescTemp), &t, sizeof(t));
+    }
+    if (!ctable.empty()) memcpy(blob + h.consts_offset, ctable.data(), sizeof(DescConst) * ctable.size());
+    for (size_t i = 0; i < consts_.size(); i++) {
+        if (!consts_[i].empty()) memcpy(blob + h.data_offset + ctable[i].offset, consts_[i].data(), consts_[i].size());
+    }
+    *outBlob = blob;
+    *outSize = (size_t)h.total_size;
+    return THIP_OK;
+}
+
+static thip_status_t addValue(thip_program_t *p, ValueKind kind, uint32_t binding, int32_t dtype, int32_t rank,
+                              const int64_t *shape, const void *data, size_t dataSize, thip_value_t *out) {
+    if (!p || !out) return fail(THIP_INVALID_ARGUMENT, "null program or result pointer");
+    if (elemSize(dtype) == 0) return fail(THIP_INVALID_ARGUMENT, "unknown element type %d", dtype);
+    if (rank < 1 || rank > THIP_MAX_RANK || !shape) return fail(THIP_INVALID_ARGUMENT, "rank %d is outside 1..%d", rank, THIP_MAX_RANK);
+    Value v;
+    v.kind = kind;
+    v.dtype = dtype;
+    v.rank = rank;
+    v.binding = binding;
+    for (int i = 0; i < THIP_MAX_RANK; i++) v.shape[i] = i < rank ? shape[i] : 1;
+    for (int i = 0; i < rank; i++) {
+        if (shape[i] <= 0) return fail(THIP_INVALID_ARGUMENT, "dimension %d is %lld", i, (long long)shape[i]);
+    }
+    if (kind == kValueConstant) {
+        const size_t need = (size_t)v.numel() * elemSize(dtype);
+        if (!data || dataSize != need) return fail(THIP_INVALID_ARGUMENT, "constant carries %zu bytes, its shape needs %zu", dataSize, need);
+        v.data.assign((const uint8_t *)data, (const uint8_t *)data + need);
+    }
+    p->values.push_back(std::move(v));
+    *out = (thip_value_t)(p->values.size() - 1);
+    return THIP_OK;
+}
+
+}  // namespace thip
+
+using namespace thip;
+
+extern "C" {
+
+thip_status_t thip_program_create(thip_program_t **out_program) {
+    if (!out_program) return fail(THIP_INVALID_ARGUMENT, "null result pointer");
+    *out_program = new (std::nothrow) thip_program_t();
+    if (!*out_program) return fail(THIP_RESOURCE_EXHAUSTED, "out of memory");
+    return THIP_OK;
+}
+
+void thip_program_destroy(thip_program_t *program) { delete program; }
+
+thip_status_t thip_program_binding(thip_program_t *program, uint32_t binding, int32_t dtype, int32_t rank,
+                                   const int64_t *shape, thip_value_t *out_value) {
+    if (binding >= 64) return fail(THIP_INVALID_ARGUMENT, "binding %u exceeds the maximum binding count", binding);
+    return addValue(program, kValueBinding, binding, dtype, rank, shape, nullptr, 0, out_value);
+}
+
+thip_status_t thip_program_constant(thip_program_t *program, int32_t dtype, int32_t rank, const int64_t *shape,
+                                    const void *data, size_t data_size, thip_value_t *out_value) {
+    return addValue(program, kValueConstant, 0, dtype, rank, shape, data, data_size, out_value);
+}
+
+thip_status_t thip_program_tensor(thip_program_t *program, int32_t dtype, int32_t rank, const int64_t *shape,
+                                  thip_value_t *out_value) {
+    return addValue(program, kValueTensor, 0, dtype, rank, shape, nullptr, 0, out_value);
+}
+
+#define THIP_DEFINE_HL(fn, type, kindEnum, member)                                        \
+    thip_status_t fn(thip_program_t *program, const type *op) {                            \
+        if (!program || !op) return fail(THIP_INVALID_ARGUMENT, #fn ": null argument");   \
+        HlOp h;                                                                            \
+        memset((void *)&h.u, 0, sizeof(h.u));                                              \
+        h.kind = kindEnum;                                                                 \
+        h.u.member = *op;                                                                  \
+        program->ops.push_back(h);                                                         \
+        return THIP_OK;                                                                    \
+    }
+
+THIP_DEFINE_HL(thip_hl_conv2d, thip_hl_conv2d_t, kHlConv2d, conv)
+THIP_DEFINE_HL(thip_hl_depthwise_conv2d, thip_hl_depthwise_conv2d_t, kHlDepthwise, dw)
+THIP_DEFINE_HL(thip_hl_fully_connected, thip_hl_fully_connected_t, kHlFullyConnected, fc)
+THIP_DEFINE_HL(thip_hl_matmul, thip_hl_matmul_t, kHlMatmul, mm)
+THIP_DEFINE_HL(thip_hl_maxpool2d, thip_hl_maxpool2d_t, kHlMaxPool, mp)
+THIP_DEFINE_HL(thip_hl_avg_pool2d, thip_hl_avg_pool2d_t, kHlAvgPool, ap)
+THIP_DEFINE_HL(thip_hl_transpose, thip_hl_transpose_t, kHlTranspose, tr)
+
+thip_status_t thip_hl_add(thip_program_t *program, const thip_hl_add_t *op) {
+    if (!program || !op) return fail(THIP_INVALID_ARGUMENT, "thip_hl_add: null argument");
+    HlOp h;
+    memset((void *)&h.u, 0, sizeof(h.u));
+    h.kind = kHlAdd;
+    h.u.add = *op;
+    h.name = op->name ? op->name : "add";
+    h.u.add.name = nullptr;  // the caller's string is not kept
+    program->ops.push_back(h);
+    return THIP_OK;
+}
+
+thip_status_t thip_program_serialize(thip_program_t *program, void **out_blob, size_t *out_size) {
+    if (!program || !out_blob || !out_size) return fail(THIP_INVALID_ARGUMENT, "thip_program_serialize: null argument");
+    *out_blob = nullptr;
+    *out_size = 0;
+    Emitter e(*program);
+    return e.run(out_blob, out_size);
+}
+
+void thip_blob_free(void *blob) { free(blob); }
+
+}  // extern "C"

@@ -1,0 +1,110 @@
+// Launch interface of the gfx950 kernels.  Host code fills one argument
+// struct per launch; every launcher validates what the kernel and its grid
+// assume before anything reaches the GPU.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace thip {
+
+// Output requantisation shared by every kernel: the ACT rescale-clamp of the
+// reference (compiler/torq/Utils/Kernel.h:610-624).
+struct Requant {
+    int32_t shift;
+    int32_t out_zp;
+    int32_t out_min;
+    int32_t out_max;
+};
+
+struct IgemmArgs {
+    const int8_t *A;        // activations: NHWC image batch, or dense [M, K]
+    const int8_t *Bp;       // packed weights [Np][Kp], K contiguous, zero padded
+    const int32_t *bias;    // [Np]
+    const int32_t *scale;   // [Np]
+    const uint32_t *ktab;   // gather loader only: Kp / gran entries
+    void *out;              // [M][N] elements of out_dtype
+    int32_t M, N, K, Kp, Np;
+    int32_t H, W, C, OH, OW, SH, SW, PT, PL;
+    int32_t input_zp;
+    int32_t out_dtype;
+    uint32_t loader;
+    uint32_t gran;
+    Requant rq;
+};
+
+// Tile configurations of the igemm kernel.
+enum IgemmVariant : uint32_t {
+    kIgemm128x128x64 = 0,
+    kIgemm256x256x64 = 1,
+    kIgemm64x64x64 = 2,
+    kIgemm256x128x64 = 3,
+    kIgemmVariantCount = 4,
+};
+struct IgemmTile {
+    int bm, bn, bk;
+    const char *name;
+};
+const IgemmTile &igemmTile(uint32_t variant);
+hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, hipStream_t stream);
+
+struct FcSkinnyArgs {
+    const int8_t *x;      // [M][K]
+    const int8_t *w;      // [N][K] (as given by the op)
+    const int32_t *bias;  // [N]
+    const int32_t *scale; // [N]
+    void *out;            // [M][N]
+    int32_t M, N, K;
+    int32_t out_dtype;
+    Requant rq;
+};
+constexpr int kFcSkinnyMaxRows = 16;
+hipError_t launchFcSkinny(const FcSkinnyArgs &a, hipStream_t stream);
+
+struct DepthwiseArgs {
+    const int8_t *in;     // NHWC
+    const int8_t *wpk;    // [KH][KW][C]
+    const int32_t *bias;  // [C]
+    const int32_t *scale; // [C]
+    int8_t *out;          // NHWC
+    int32_t N, H, W, C, OH, OW, KH, KW, SH, SW, PT, PL;
+    int32_t input_zp;
+    Requant rq;
+};
+hipError_t launchDepthwise(const DepthwiseArgs &a, hipStream_t stream);
+
+struct MaxPoolArgs {
+    const int8_t *in;  // NHWC
+    int8_t *out;       // NHWC
+    int32_t N, H, W, C, OH, OW, KH, KW, SH, SW, PT, PL;
+    int32_t input_zp, out_min, out_max;
+};
+hipError_t launchMaxPool(const MaxPoolArgs &a, hipStream_t stream);
+
+struct AvgPoolArgs {
+    const int8_t *in;  // [N][HW][C]
+    int8_t *out;       // [N][C]
+    int32_t N, HW, C;
+    int32_t weight, bias, scale;
+    Requant rq;
+};
+hipError_t launchAvgPool(const AvgPoolArgs &a, hipStream_t stream);
+
+struct AddArgs {
+    const int8_t *in0;
+    const int8_t *in1;
+    int8_t *out;
+    int64_t count;
+    int32_t w0, w1, bias, scale;
+    Requant rq;
+};
+hipError_t launchAdd(const AddArgs &a, hipStream_t stream);
+
+struct TransposeArgs {
+    const int8_t *in;  // [B][R][S]
+    int8_t *out;       // [B][S][R]
+    int32_t B, R, S;
+};
+hipError_t launchTranspose(const TransposeArgs &a, hipStream_t stream);
+
+}  // namespace thip

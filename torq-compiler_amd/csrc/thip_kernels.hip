@@ -1,0 +1,747 @@
+// gfx950 (CDNA4) kernels of the quantized TorqHL operator path.
+//
+//   igemm_i8      conv2d / fully_connected / matmul as implicit GEMM on
+//                 v_mfma_i32_32x32x32_i8, LDS double-buffered tiles, requant fused
+//                 on the accumulator registers.
+//   fc_skinny     fully_connected with at most 16 rows: weight streaming with
+//                 v_dot4_i32_i8 and wave-shuffle reductions (HBM bound).
+//   depthwise / maxpool / avgpool / add / transpose: bandwidth-bound kernels
+//                 with 128-bit accesses on NHWC tensors.
+//
+// Every kernel ends with the reference's ACT rescale-clamp
+// (compiler/torq/Utils/Kernel.h:610-624): int32 add of the bias, 32x32->64 bit
+// multiply by the scale, add of 2^(shift-1), arithmetic right shift, add of the
+// output zero point, clamp.
+#include "thip_kernels.h"
+
+#include "thip_descriptor.h"
+
+namespace thip {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int kDtypeI8 = 1, kDtypeI16 = 2, kDtypeI32 = 3;
+
+__device__ __forceinline__ int32_t requant(int32_t acc, int32_t bias, int32_t scale, long long rnd,
+                                           const Requant &rq) {
+    const int32_t t0 = (int32_t)((uint32_t)acc + (uint32_t)bias);
+    const long long t1 = (long long)t0 * (long long)scale;
+    const long long t3 = (t1 + rnd) >> rq.shift;
+    long long t4 = t3 + (long long)rq.out_zp;
+    t4 = t4 < (long long)rq.out_min ? (long long)rq.out_min : t4;
+    t4 = t4 > (long long)rq.out_max ? (long long)rq.out_max : t4;
+    return (int32_t)t4;
+}
+
+__device__ __forceinline__ long long roundTerm(int shift) {
+    return shift > 0 ? (1LL << (shift - 1)) : 0LL;
+}
+
+__device__ __forceinline__ void storeElem(void *out, size_t idx, int32_t v, int dtype) {
+    if (dtype == kDtypeI8) {
+        ((int8_t *)out)[idx] = (int8_t)v;
+    } else if (dtype == kDtypeI16) {
+        ((int16_t *)out)[idx] = (int16_t)v;
+    } else {
+        ((int32_t *)out)[idx] = v;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// igemm_i8
+// ---------------------------------------------------------------------------
+//
+// C[m][n] = sum_k A[m][k] * B[n][k]; block tile BM x BN x BK, 256 threads =
+// 4 waves in a 2 x 2 arrangement, each wave owns (BM/2) x (BN/2) as a grid of
+// 32 x 32 MFMA tiles.  One MFMA consumes 32 rows x 32 k of each operand: lane l
+// supplies row (l & 31), 16 consecutive k bytes starting at 16 * (l >> 5).  The
+// accumulator register r of lane l holds C[8 * (r / 4) + 4 * (l >> 5) + (r & 3)][l & 31].
+//
+// LDS rows are padded by 16 bytes so that the 16 lanes of one ds_read_b128
+// phase fall into distinct banks.
+
+template <int G>
+__device__ __forceinline__ v4i gatherChunk(const int8_t *__restrict__ A,
+                                           const uint32_t *__restrict__ entries, int iy0, int ix0,
+                                           size_t base, int H, int W, int C, uint32_t zp4) {
+    union {
+        v4i v;
+        uint64_t d[2];
+        uint32_t w[4];
+        uint16_t h[8];
+        uint8_t b[16];
+    } u;
+#pragma unroll
+    for (int j = 0; j < 16 / G; j++) {
+        const uint32_t e = entries[j];
+        const int kh = (int)((e >> 24) & 0x7f), kw = (int)((e >> 16) & 0xff);
+        const int ci = (int)(e & 0xffff);
+        const int iy = iy0 + kh, ix = ix0 + kw;
+        const bool beyond = (e & kKEntryInvalid) != 0;
+        const bool inside = !beyond && (unsigned)iy < (unsigned)H && (unsigned)ix < (unsigned)W;
+        const int8_t *src = A + base + ((size_t)iy * W + ix) * C + ci;
+        const uint32_t fill = beyond ? 0u : zp4;
+        if (G == 16) {
+            if (inside) {
+                u.v = *(const v4i *)src;
+            } else {
+                u.w[0] = fill; u.w[1] = fill; u.w[2] = fill; u.w[3] = fill;
+            }
+        } else if (G == 8) {
+            u.d[j] = inside ? *(const uint64_t *)src : ((uint64_t)fill << 32 | fill);
+        } else if (G == 4) {
+            u.w[j] = inside ? *(const uint32_t *)src : fill;
+        } else if (G == 2) {
+            u.h[j] = inside ? *(const uint16_t *)src : (uint16_t)fill;
+        } else {
+            u.b[j] = inside ? *(const uint8_t *)src : (uint8_t)fill;
+        }
+    }
+    return u.v;
+}
+
+template <int BM, int BN, int BK, int LOADER, int G>
+__global__ __launch_bounds__(256) void igemm_i8(IgemmArgs p) {
+    constexpr int LDK = BK + 16;            // padded LDS row
+    constexpr int CPR = BK / 16;            // 16-byte chunks per tile row
+    constexpr int RPP = 256 / CPR;          // rows loaded per pass
+    constexpr int PA = BM / RPP;            // passes over the A tile
+    constexpr int PB = BN / RPP;            // passes over the B tile
+    constexpr int WTM = BM / 2, WTN = BN / 2;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    static_assert(BM % RPP == 0 && BN % RPP == 0, "tile rows must be a multiple of a load pass");
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the MFMA tile");
+
+    extern __shared__ __align__(16) int8_t smem[];
+    int8_t *As = smem;                       // [2][BM][LDK]
+    int8_t *Bs = smem + 2 * BM * LDK;        // [2][BN][LDK]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+
+    // Block -> tile: blocks are dealt round-robin to the 8 XCDs, so give every
+    // XCD a contiguous range of tiles (its L2 then sees neighbouring tiles), and
+    // walk each range in groups of 8 tile rows so that A and B tiles are reused.
+    const int tilesM = (p.M + BM - 1) / BM;
+    const int tilesN = p.Np / BN;
+    int lin;
+    {
+        const int nb = (int)gridDim.x, pid = (int)blockIdx.x;
+        const int per = nb / 8, rem = nb % 8;
+        const int xcd = pid % 8, idx = pid / 8;
+        lin = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    }
+    constexpr int GROUP = 8;
+    const int width = GROUP * tilesN;
+    const int group = lin / width;
+    const int firstM = group * GROUP;
+    const int gsize = (tilesM - firstM) < GROUP ? (tilesM - firstM) : GROUP;
+    const int tileM = firstM + (lin % width) % gsize;
+    const int tileN = (lin % width) / gsize;
+    const int m0 = tileM * BM, n0 = tileN * BN;
+
+    const int lrow = tid / CPR, lkc = tid % CPR;
+    const uint32_t zpb = (uint32_t)(p.input_zp & 0xff);
+    const uint32_t zp4 = zpb * 0x01010101u;
+
+    // Per-row state of the A loader.
+    int rIy0[PA], rIx0[PA];
+    size_t rBase[PA];
+#pragma unroll
+    for (int i = 0; i < PA; i++) {
+        const int m = m0 + lrow + i * RPP;
+        if (LOADER == kLoaderDense) {
+            rBase[i] = (size_t)m * p.K;
+            rIy0[i] = m < p.M ? 0 : -1;
+            rIx0[i] = 0;
+        } else {
+            const int ohw = p.OH * p.OW;
+            const int img = m / ohw, rem = m % ohw;
+            const int oy = rem / p.OW, ox = rem % p.OW;
+            rBase[i] = (size_t)img * p.H * p.W * p.C;
+            // rows past M gather nothing but padding; they are never stored
+            rIy0[i] = m < p.M ? oy * p.SH - p.PT : -(1 << 20);
+            rIx0[i] = ox * p.SW - p.PL;
+        }
+    }
+
+    v4i ra[PA], rb[PB];
+    auto loadGlobal = [&](int kt) {
+        const int k0 = kt * BK + lkc * 16;
+#pragma unroll
+        for (int i = 0; i < PA; i++) {
+            if (LOADER == kLoaderDense) {
+                v4i v = {0, 0, 0, 0};
+                if (rIy0[i] == 0 && k0 < p.K) {
+                    v = *(const v4i *)(p.A + rBase[i] + k0);
+                }
+                ra[i] = v;
+            } else {
+                ra[i] = gatherChunk<G>(p.A, p.ktab + k0 / G, rIy0[i], rIx0[i], rBase[i], p.H, p.W,
+                                       p.C, zp4);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < PB; i++) {
+            const int n = n0 + lrow + i * RPP;
+            rb[i] = *(const v4i *)(p.Bp + (size_t)n * p.Kp + k0);
+        }
+    };
+    auto storeLds = [&](int stage) {
+#pragma unroll
+        for (int i = 0; i < PA; i++) {
+            *(v4i *)(As + (stage * BM + lrow + i * RPP) * LDK + lkc * 16) = ra[i];
+        }
+#pragma unroll
+        for (int i = 0; i < PB; i++) {
+            *(v4i *)(Bs + (stage * BN + lrow + i * RPP) * LDK + lkc * 16) = rb[i];
+        }
+    };
+
+    v16i acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++) {
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+        }
+    }
+
+    const int KT = p.Kp / BK;
+    loadGlobal(0);
+    storeLds(0);
+    __syncthreads();
+
+    const int aRow = wm * WTM + (lane & 31);
+    const int bRow = wn * WTN + (lane & 31);
+    const int kOff = (lane >> 5) * 16;
+
+    for (int kt = 0; kt < KT; kt++) {
+        const int cur = kt & 1;
+        if (kt + 1 < KT) {
+            loadGlobal(kt + 1);
+        }
+#pragma unroll
+        for (int kk = 0; kk < BK / 32; kk++) {
+            v4i af[TM], bf[TN];
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+                af[i] = *(const v4i *)(As + (cur * BM + aRow + i * 32) * LDK + kk * 32 + kOff);
+            }
+#pragma unroll
+            for (int j = 0; j < TN; j++) {
+                bf[j] = *(const v4i *)(Bs + (cur * BN + bRow + j * 32) * LDK + kk * 32 + kOff);
+            }
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
+                }
+            }
+        }
+        if (kt + 1 < KT) {
+            storeLds(cur ^ 1);
+        }
+        __syncthreads();
+    }
+
+    // Epilogue: requant in the accumulator layout.  Each lane owns one output
+    // column per MFMA tile (so one bias/scale pair) and 16 rows.
+    const long long rnd = roundTerm(p.rq.shift);
+    const int rowBase = m0 + wm * WTM + (lane >> 5) * 4;
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const int n = n0 + wn * WTN + j * 32 + (lane & 31);
+        const int32_t bias = p.bias[n];    // arrays are padded to Np
+        const int32_t scale = p.scale[n];
+        if (n < p.N) {
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int m = rowBase + i * 32 + 8 * (r / 4) + (r & 3);
+                    if (m < p.M) {
+                        const int32_t q = requant(acc[i][j][r], bias, scale, rnd, p.rq);
+                        storeElem(p.out, (size_t)m * p.N + n, q, p.out_dtype);
+                    }
+                }
+            }
+        }
+    }
+}
+
+static const IgemmTile kTiles[kIgemmVariantCount] = {
+    {128, 128, 64, "igemm_i8_128x128x64"},
+    {256, 256, 64, "igemm_i8_256x256x64"},
+    {64, 64, 64, "igemm_i8_64x64x64"},
+    {256, 128, 64, "igemm_i8_256x128x64"},
+};
+
+const IgemmTile &igemmTile(uint32_t variant) {
+    return kTiles[variant < kIgemmVariantCount ? variant : 0];
+}
+
+template <int BM, int BN, int BK, int LOADER, int G>
+static hipError_t launchIgemmTile(const IgemmArgs &a, hipStream_t stream) {
+    constexpr int LDK = BK + 16;
+    constexpr size_t smem = (size_t)2 * (BM + BN) * LDK;
+    auto kernel = igemm_i8<BM, BN, BK, LOADER, G>;
+    hipError_t err = hipFuncSetAttribute((const void *)kernel,
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (err != hipSuccess) return err;
+    const int tilesM = (a.M + BM - 1) / BM;
+    const int tilesN = a.Np / BN;
+    const dim3 grid((unsigned)(tilesM * tilesN));
+    hipLaunchKernelGGL(kernel, grid, dim3(256), smem, stream, a);
+    return hipGetLastError();
+}
+
+template <int BM, int BN, int BK>
+static hipError_t launchIgemmLoader(const IgemmArgs &a, hipStream_t stream) {
+    if (a.loader == kLoaderDense) {
+        return launchIgemmTile<BM, BN, BK, kLoaderDense, 16>(a, stream);
+    }
+    switch (a.gran) {
+    case 16: return launchIgemmTile<BM, BN, BK, kLoaderGather, 16>(a, stream);
+    case 8: return launchIgemmTile<BM, BN, BK, kLoaderGather, 8>(a, stream);
+    case 4: return launchIgemmTile<BM, BN, BK, kLoaderGather, 4>(a, stream);
+    case 2: return launchIgemmTile<BM, BN, BK, kLoaderGather, 2>(a, stream);
+    case 1: return launchIgemmTile<BM, BN, BK, kLoaderGather, 1>(a, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, hipStream_t stream) {
+    if (variant >= kIgemmVariantCount) return hipErrorInvalidValue;
+    const IgemmTile &t = kTiles[variant];
+    // What the kernel assumes: padded sizes are whole tiles, the real sizes fit
+    // inside them, the dense loader reads whole 16-byte chunks of each row.
+    if (a.M <= 0 || a.N <= 0 || a.K <= 0) return hipErrorInvalidValue;
+    if (a.Kp % t.bk != 0 || a.Np % t.bn != 0 || a.K > a.Kp || a.N > a.Np) return hipErrorInvalidValue;
+    if (!a.A || !a.Bp || !a.bias || !a.scale || !a.out) return hipErrorInvalidValue;
+    if (a.loader == kLoaderDense) {
+        if (a.K % 16 != 0 || ((uintptr_t)a.A & 15) != 0) return hipErrorInvalidValue;
+    } else {
+        if (!a.ktab || a.C <= 0 || a.C % (int)a.gran != 0) return hipErrorInvalidValue;
+        if (a.OH <= 0 || a.OW <= 0 || a.M % (a.OH * a.OW) != 0) return hipErrorInvalidValue;
+        if (((uintptr_t)a.A & (a.gran - 1)) != 0) return hipErrorInvalidValue;
+    }
+    if (((uintptr_t)a.Bp & 15) != 0) return hipErrorInvalidValue;
+    if (a.out_dtype < kDtypeI8 || a.out_dtype > kDtypeI32) return hipErrorInvalidValue;
+    switch (variant) {
+    case kIgemm128x128x64: return launchIgemmLoader<128, 128, 64>(a, stream);
+    case kIgemm256x256x64: return launchIgemmLoader<256, 256, 64>(a, stream);
+    case kIgemm64x64x64: return launchIgemmLoader<64, 64, 64>(a, stream);
+    case kIgemm256x128x64: return launchIgemmLoader<256, 128, 64>(a, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
+// ---------------------------------------------------------------------------
+// fc_skinny: out[m][n] = requant(sum_k x[m][k] * w[n][k]) for M <= 16.
+// One wave per NW output columns; lanes split K in 16-byte chunks, so one wave
+// load of a weight row is 1 KiB contiguous.  Partial sums are reduced with
+// wave shuffles.  K % 16 == 0.
+// ---------------------------------------------------------------------------
+template <int MR, int NW>
+__global__ __launch_bounds__(256) void fc_skinny(FcSkinnyArgs p) {
+    const int lane = threadIdx.x & 63;
+    const int wave = (int)((blockIdx.x * 256 + threadIdx.x) >> 6);
+    const int n0 = wave * NW;
+    if (n0 >= p.N) return;
+    int32_t acc[MR][NW];
+#pragma unroll
+    for (int m = 0; m < MR; m++) {
+#pragma unroll
+        for (int j = 0; j < NW; j++) acc[m][j] = 0;
+    }
+    const int chunks = p.K / 16;
+    for (int c = lane; c < chunks; c += 64) {
+        v4i wv[NW];
+#pragma unroll
+        for (int j = 0; j < NW; j++) {
+            const int n = (n0 + j) < p.N ? (n0 + j) : (p.N - 1);
+            wv[j] = *(const v4i *)(p.w + (size_t)n * p.K + (size_t)c * 16);
+        }
+#pragma unroll
+        for (int m = 0; m < MR; m++) {
+            if (m < p.M) {
+                const v4i xv = *(const v4i *)(p.x + (size_t)m * p.K + (size_t)c * 16);
+#pragma unroll
+                for (int j = 0; j < NW; j++) {
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        acc[m][j] = __builtin_amdgcn_sdot4(xv[q], wv[j][q], acc[m][j], false);
+                    }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MR; m++) {
+#pragma unroll
+        for (int j = 0; j < NW; j++) {
+            int32_t v = acc[m][j];
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+            acc[m][j] = v;
+        }
+    }
+    if (lane == 0) {
+        const long long rnd = roundTerm(p.rq.shift);
+#pragma unroll
+        for (int j = 0; j < NW; j++) {
+            const int n = n0 + j;
+            if (n < p.N) {
+                const int32_t bias = p.bias[n], scale = p.scale[n];
+#pragma unroll
+                for (int m = 0; m < MR; m++) {
+                    if (m < p.M) {
+                        storeElem(p.out, (size_t)m * p.N + n, requant(acc[m][j], bias, scale, rnd, p.rq),
+                                  p.out_dtype);
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <int MR, int NW>
+static hipError_t launchFcSkinnyT(const FcSkinnyArgs &a, hipStream_t stream) {
+    const int waves = (a.N + NW - 1) / NW;
+    const dim3 grid((unsigned)((waves + 3) / 4));
+    hipLaunchKernelGGL((fc_skinny<MR, NW>), grid, dim3(256), 0, stream, a);
+    return hipGetLastError();
+}
+
+hipError_t launchFcSkinny(const FcSkinnyArgs &a, hipStream_t stream) {
+    if (a.M <= 0 || a.M > kFcSkinnyMaxRows || a.N <= 0 || a.K <= 0 || a.K % 16 != 0) {
+        return hipErrorInvalidValue;
+    }
+    if (!a.x || !a.w || !a.bias || !a.scale || !a.out) return hipErrorInvalidValue;
+    if ((((uintptr_t)a.x) | ((uintptr_t)a.w)) & 15) return hipErrorInvalidValue;
+    if (a.out_dtype < kDtypeI8 || a.out_dtype > kDtypeI32) return hipErrorInvalidValue;
+    if (a.M == 1) return launchFcSkinnyT<1, 4>(a, stream);
+    if (a.M <= 4) return launchFcSkinnyT<4, 4>(a, stream);
+    if (a.M <= 8) return launchFcSkinnyT<8, 2>(a, stream);
+    return launchFcSkinnyT<16, 2>(a, stream);
+}
+
+// ---------------------------------------------------------------------------
+// Bandwidth-bound kernels.  One thread = VEC consecutive channels of one
+// output pixel (NHWC), VEC bytes per load/store (16 when C % 16 == 0).
+// ---------------------------------------------------------------------------
+template <int VEC>
+struct ByteVec;
+template <>
+struct ByteVec<16> {
+    typedef v4i type;
+};
+template <>
+struct ByteVec<8> {
+    typedef v2i type;
+};
+template <>
+struct ByteVec<4> {
+    typedef int type;
+};
+template <>
+struct ByteVec<1> {
+    typedef int8_t type;
+};
+
+template <int VEC>
+union Pack {
+    typename ByteVec<VEC>::type v;
+    int8_t b[VEC];
+};
+
+template <int VEC, int KS>  // KS > 0: square KS x KS window known at compile time
+__global__ __launch_bounds__(256) void depthwise_i8(DepthwiseArgs p) {
+    const int cg = p.C / VEC;
+    const long long total = (long long)p.N * p.OH * p.OW * cg;
+    const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (t >= total) return;
+    const int c0 = (int)(t % cg) * VEC;
+    long long pix = t / cg;
+    const int ox = (int)(pix % p.OW);
+    pix /= p.OW;
+    const int oy = (int)(pix % p.OH);
+    const int n = (int)(pix / p.OH);
+    const int KH = KS > 0 ? KS : p.KH, KW = KS > 0 ? KS : p.KW;
+    const int iy0 = oy * p.SH - p.PT, ix0 = ox * p.SW - p.PL;
+    const int8_t *img = p.in + (size_t)n * p.H * p.W * p.C + c0;
+    int32_t acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; v++) acc[v] = 0;
+#pragma unroll
+    for (int kh = 0; kh < KH; kh++) {
+        const int iy = iy0 + kh;
+#pragma unroll
+        for (int kw = 0; kw < KW; kw++) {
+            const int ix = ix0 + kw;
+            Pack<VEC> x, w;
+            w.v = *(const typename ByteVec<VEC>::type *)(p.wpk + (size_t)(kh * KW + kw) * p.C + c0);
+            if ((unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W) {
+                x.v = *(const typename ByteVec<VEC>::type *)(img + ((size_t)iy * p.W + ix) * p.C);
+#pragma unroll
+                for (int v = 0; v < VEC; v++) acc[v] += (int32_t)x.b[v] * (int32_t)w.b[v];
+            } else {
+#pragma unroll
+                for (int v = 0; v < VEC; v++) acc[v] += p.input_zp * (int32_t)w.b[v];
+            }
+        }
+    }
+    const long long rnd = roundTerm(p.rq.shift);
+    Pack<VEC> o;
+#pragma unroll
+    for (int v = 0; v < VEC; v++) {
+        o.b[v] = (int8_t)requant(acc[v], p.bias[c0 + v], p.scale[c0 + v], rnd, p.rq);
+    }
+    *(typename ByteVec<VEC>::type *)(p.out + (((size_t)n * p.OH + oy) * p.OW + ox) * p.C + c0) = o.v;
+}
+
+static int pickVec(int C, const void *a, const void *b, const void *c) {
+    const uintptr_t bits = (uintptr_t)a | (uintptr_t)b | (uintptr_t)c;
+    if (C % 16 == 0 && (bits & 15) == 0) return 16;
+    if (C % 8 == 0 && (bits & 7) == 0) return 8;
+    if (C % 4 == 0 && (bits & 3) == 0) return 4;
+    return 1;
+}
+
+static bool poolGeometryOk(int N, int H, int W, int C, int OH, int OW, int KH, int KW, int SH,
+                           int SW, int PT, int PL) {
+    if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || OH <= 0 || OW <= 0) return false;
+    if (KH <= 0 || KW <= 0 || SH <= 0 || SW <= 0 || PT < 0 || PL < 0) return false;
+    return true;
+}
+
+template <int VEC>
+static hipError_t launchDepthwiseV(const DepthwiseArgs &a, hipStream_t stream) {
+    const long long total = (long long)a.N * a.OH * a.OW * (a.C / VEC);
+    const dim3 grid((unsigned)((total + 255) / 256));
+    if (a.KH == 3 && a.KW == 3) {
+        hipLaunchKernelGGL((depthwise_i8<VEC, 3>), grid, dim3(256), 0, stream, a);
+    } else {
+        hipLaunchKernelGGL((depthwise_i8<VEC, 0>), grid, dim3(256), 0, stream, a);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launchDepthwise(const DepthwiseArgs &a, hipStream_t stream) {
+    if (!poolGeometryOk(a.N, a.H, a.W, a.C, a.OH, a.OW, a.KH, a.KW, a.SH, a.SW, a.PT, a.PL)) {
+        return hipErrorInvalidValue;
+    }
+    if (!a.in || !a.wpk || !a.bias || !a.scale || !a.out) return hipErrorInvalidValue;
+    if ((long long)a.N * a.OH * a.OW * a.C >= (1LL << 40)) return hipErrorInvalidValue;
+    switch (pickVec(a.C, a.in, a.out, a.wpk)) {
+    case 16: return launchDepthwiseV<16>(a, stream);
+    case 8: return launchDepthwiseV<8>(a, stream);
+    case 4: return launchDepthwiseV<4>(a, stream);
+    default: return launchDepthwiseV<1>(a, stream);
+    }
+}
+
+template <int VEC>
+__global__ __launch_bounds__(256) void maxpool_i8(MaxPoolArgs p) {
+    const int cg = p.C / VEC;
+    const long long total = (long long)p.N * p.OH * p.OW * cg;
+    const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (t >= total) return;
+    const int c0 = (int)(t % cg) * VEC;
+    long long pix = t / cg;
+    const int ox = (int)(pix % p.OW);
+    pix /= p.OW;
+    const int oy = (int)(pix % p.OH);
+    const int n = (int)(pix / p.OH);
+    const int iy0 = oy * p.SH - p.PT, ix0 = ox * p.SW - p.PL;
+    const int8_t *img = p.in + (size_t)n * p.H * p.W * p.C + c0;
+    int32_t best[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; v++) best[v] = -(1 << 30);
+    bool padded = false;
+    for (int kh = 0; kh < p.KH; kh++) {
+        const int iy = iy0 + kh;
+        for (int kw = 0; kw < p.KW; kw++) {
+            const int ix = ix0 + kw;
+            if ((unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W) {
+                Pack<VEC> x;
+                x.v = *(const typename ByteVec<VEC>::type *)(img + ((size_t)iy * p.W + ix) * p.C);
+#pragma unroll
+                for (int v = 0; v < VEC; v++) best[v] = best[v] > (int32_t)x.b[v] ? best[v] : (int32_t)x.b[v];
+            } else {
+                padded = true;
+            }
+        }
+    }
+    Pack<VEC> o;
+#pragma unroll
+    for (int v = 0; v < VEC; v++) {
+        int32_t b = best[v];
+        if (padded) b = b > p.input_zp ? b : p.input_zp;
+        b = b < p.out_min ? p.out_min : b;
+        b = b > p.out_max ? p.out_max : b;
+        o.b[v] = (int8_t)b;
+    }
+    *(typename ByteVec<VEC>::type *)(p.out + (((size_t)n * p.OH + oy) * p.OW + ox) * p.C + c0) = o.v;
+}
+
+template <int VEC>
+static hipError_t launchMaxPoolV(const MaxPoolArgs &a, hipStream_t stream) {
+    const long long total = (long long)a.N * a.OH * a.OW * (a.C / VEC);
+    const dim3 grid((unsigned)((total + 255) / 256));
+    hipLaunchKernelGGL((maxpool_i8<VEC>), grid, dim3(256), 0, stream, a);
+    return hipGetLastError();
+}
+
+hipError_t launchMaxPool(const MaxPoolArgs &a, hipStream_t stream) {
+    if (!poolGeometryOk(a.N, a.H, a.W, a.C, a.OH, a.OW, a.KH, a.KW, a.SH, a.SW, a.PT, a.PL)) {
+        return hipErrorInvalidValue;
+    }
+    if (!a.in || !a.out) return hipErrorInvalidValue;
+    if ((long long)a.N * a.OH * a.OW * a.C >= (1LL << 40)) return hipErrorInvalidValue;
+    switch (pickVec(a.C, a.in, a.out, nullptr)) {
+    case 16: return launchMaxPoolV<16>(a, stream);
+    case 8: return launchMaxPoolV<8>(a, stream);
+    case 4: return launchMaxPoolV<4>(a, stream);
+    default: return launchMaxPoolV<1>(a, stream);
+    }
+}
+
+// Global average pool: one wave covers CC channel groups of VEC channels; the
+// 64 / CC lanes that share a channel group split the H*W pixels and are
+// combined with wave shuffles.
+template <int VEC, int CC>
+__global__ __launch_bounds__(256) void avgpool_i8(AvgPoolArgs p) {
+    constexpr int PG = 64 / CC;  // lanes per channel group
+    const int lane = threadIdx.x & 63;
+    const int wave = (int)((blockIdx.x * 256 + threadIdx.x) >> 6);
+    const int cgroups = p.C / VEC;
+    const int wavesPerImage = (cgroups + CC - 1) / CC;
+    const int n = wave / wavesPerImage;
+    if (n >= p.N) return;
+    const int cgi = (wave % wavesPerImage) * CC + (lane % CC);
+    const int pg = lane / CC;
+    const bool active = cgi < cgroups;
+    const int c0 = cgi * VEC;
+    int32_t acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; v++) acc[v] = 0;
+    if (active) {
+        const int8_t *src = p.in + (size_t)n * p.HW * p.C + c0;
+        for (int u = pg; u < p.HW; u += PG) {
+            Pack<VEC> x;
+            x.v = *(const typename ByteVec<VEC>::type *)(src + (size_t)u * p.C);
+#pragma unroll
+            for (int v = 0; v < VEC; v++) acc[v] += (int32_t)x.b[v] * p.weight;
+        }
+    }
+#pragma unroll
+    for (int v = 0; v < VEC; v++) {
+        int32_t s = acc[v];
+#pragma unroll
+        for (int off = 32; off >= CC; off >>= 1) s += __shfl_xor(s, off, 64);
+        acc[v] = s;
+    }
+    if (active && pg == 0) {
+        const long long rnd = roundTerm(p.rq.shift);
+        Pack<VEC> o;
+#pragma unroll
+        for (int v = 0; v < VEC; v++) o.b[v] = (int8_t)requant(acc[v], p.bias, p.scale, rnd, p.rq);
+        *(typename ByteVec<VEC>::type *)(p.out + (size_t)n * p.C + c0) = o.v;
+    }
+}
+
+template <int VEC>
+static hipError_t launchAvgPoolV(const AvgPoolArgs &a, hipStream_t stream) {
+    constexpr int CC = 4;
+    const int cgroups = a.C / VEC;
+    const long long waves = (long long)a.N * ((cgroups + CC - 1) / CC);
+    const dim3 grid((unsigned)((waves + 3) / 4));
+    hipLaunchKernelGGL((avgpool_i8<VEC, CC>), grid, dim3(256), 0, stream, a);
+    return hipGetLastError();
+}
+
+hipError_t launchAvgPool(const AvgPoolArgs &a, hipStream_t stream) {
+    if (a.N <= 0 || a.HW <= 0 || a.C <= 0 || !a.in || !a.out) return hipErrorInvalidValue;
+    switch (pickVec(a.C, a.in, a.out, nullptr)) {
+    case 16: return launchAvgPoolV<16>(a, stream);
+    case 8: return launchAvgPoolV<8>(a, stream);
+    case 4: return launchAvgPoolV<4>(a, stream);
+    default: return launchAvgPoolV<1>(a, stream);
+    }
+}
+
+template <int VEC>
+__global__ __launch_bounds__(256) void add_i8(AddArgs p) {
+    const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+    const long long i0 = t * VEC;
+    if (i0 >= p.count) return;
+    const long long rnd = roundTerm(p.rq.shift);
+    if (i0 + VEC <= p.count) {
+        Pack<VEC> a, b, o;
+        a.v = *(const typename ByteVec<VEC>::type *)(p.in0 + i0);
+        b.v = *(const typename ByteVec<VEC>::type *)(p.in1 + i0);
+#pragma unroll
+        for (int v = 0; v < VEC; v++) {
+            const int32_t acc = (int32_t)a.b[v] * p.w0 + (int32_t)b.b[v] * p.w1;
+            o.b[v] = (int8_t)requant(acc, p.bias, p.scale, rnd, p.rq);
+        }
+        *(typename ByteVec<VEC>::type *)(p.out + i0) = o.v;
+    } else {
+        for (long long i = i0; i < p.count; i++) {
+            const int32_t acc = (int32_t)p.in0[i] * p.w0 + (int32_t)p.in1[i] * p.w1;
+            p.out[i] = (int8_t)requant(acc, p.bias, p.scale, rnd, p.rq);
+        }
+    }
+}
+
+hipError_t launchAdd(const AddArgs &a, hipStream_t stream) {
+    if (a.count <= 0 || !a.in0 || !a.in1 || !a.out) return hipErrorInvalidValue;
+    const uintptr_t bits = (uintptr_t)a.in0 | (uintptr_t)a.in1 | (uintptr_t)a.out;
+    if ((bits & 15) == 0) {
+        const long long threads = (a.count + 15) / 16;
+        hipLaunchKernelGGL((add_i8<16>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, a);
+    } else {
+        hipLaunchKernelGGL((add_i8<1>), dim3((unsigned)((a.count + 255) / 256)), dim3(256), 0, stream, a);
+    }
+    return hipGetLastError();
+}
+
+// Batched byte transpose [B][R][S] -> [B][S][R] through a 64 x 64 LDS tile.
+__global__ __launch_bounds__(256) void transpose_i8(TransposeArgs p) {
+    __shared__ int8_t tile[64][65];
+    const int tilesS = (p.S + 63) / 64, tilesR = (p.R + 63) / 64;
+    int bid = (int)blockIdx.x;
+    const int ts = bid % tilesS;
+    bid /= tilesS;
+    const int tr = bid % tilesR;
+    const int b = bid / tilesR;
+    const int r0 = tr * 64, s0 = ts * 64;
+    const int8_t *src = p.in + (size_t)b * p.R * p.S;
+    int8_t *dst = p.out + (size_t)b * p.R * p.S;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int r = ty; r < 64; r += 4) {
+        if (r0 + r < p.R && s0 + tx < p.S) tile[r][tx] = src[(size_t)(r0 + r) * p.S + s0 + tx];
+    }
+    __syncthreads();
+    for (int s = ty; s < 64; s += 4) {
+        if (s0 + s < p.S && r0 + tx < p.R) dst[(size_t)(s0 + s) * p.R + r0 + tx] = tile[tx][s];
+    }
+}
+
+hipError_t launchTranspose(const TransposeArgs &a, hipStream_t stream) {
+    if (a.B <= 0 || a.R <= 0 || a.S <= 0 || !a.in || !a.out) return hipErrorInvalidValue;
+    const long long blocks = (long long)a.B * ((a.R + 63) / 64) * ((a.S + 63) / 64);
+    if (blocks >= (1LL << 31)) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(transpose_i8, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+    return hipGetLastError();
+}
+
+}  // namespace thip

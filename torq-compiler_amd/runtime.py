@@ -1,0 +1,352 @@
+"""ctypes binding of the C-ABI in ``include/thip.h``.
+
+Host-side glue only: everything that computes lives in ``libthip.so``.  There is
+no CPU fallback; if the library or a gfx950 device is missing the calls raise.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libthip.so")
+
+# status codes (include/thip.h)
+OK = 0
+INVALID_ARGUMENT = 3
+RESOURCE_EXHAUSTED = 8
+FAILED_PRECONDITION = 9
+OUT_OF_RANGE = 11
+UNIMPLEMENTED = 12
+INTERNAL = 13
+UNAVAILABLE = 14
+
+STATUS_NAMES = {
+    OK: "OK", INVALID_ARGUMENT: "INVALID_ARGUMENT", RESOURCE_EXHAUSTED: "RESOURCE_EXHAUSTED",
+    FAILED_PRECONDITION: "FAILED_PRECONDITION", OUT_OF_RANGE: "OUT_OF_RANGE",
+    UNIMPLEMENTED: "UNIMPLEMENTED", INTERNAL: "INTERNAL", UNAVAILABLE: "UNAVAILABLE",
+}
+
+DTYPE_I8, DTYPE_I16, DTYPE_I32 = 1, 2, 3
+_NP_TO_DTYPE = {np.dtype(np.int8): DTYPE_I8, np.dtype(np.int16): DTYPE_I16, np.dtype(np.int32): DTYPE_I32}
+_DTYPE_TO_NP = {v: k for k, v in _NP_TO_DTYPE.items()}
+
+BINDING_HOST, BINDING_DEVICE = 0, 1
+
+# every symbol include/thip.h declares
+EXPORTED_SYMBOLS = [
+    "thip_status_message", "thip_version", "thip_descriptor_version",
+    "thip_program_create", "thip_program_destroy", "thip_program_binding", "thip_program_constant",
+    "thip_program_tensor", "thip_hl_conv2d", "thip_hl_depthwise_conv2d", "thip_hl_fully_connected",
+    "thip_hl_matmul", "thip_hl_maxpool2d", "thip_hl_avg_pool2d", "thip_hl_add", "thip_hl_transpose",
+    "thip_program_serialize", "thip_blob_free",
+    "thip_device_create", "thip_device_destroy", "thip_device_name", "thip_device_alloc",
+    "thip_device_free", "thip_device_h2d", "thip_device_d2h", "thip_device_synchronize",
+    "thip_device_set_event_log", "thip_infer_format",
+    "thip_executable_create", "thip_executable_destroy", "thip_executable_run",
+    "thip_executable_enqueue", "thip_executable_wait", "thip_executable_time",
+    "thip_executable_op_count", "thip_executable_op_kernel", "thip_executable_binding_count",
+    "thip_executable_binding_size",
+]
+
+
+class ThipError(RuntimeError):
+    def __init__(self, code, message):
+        super().__init__("%s: %s" % (STATUS_NAMES.get(code, str(code)), message))
+        self.code = code
+        self.message = message
+
+
+class DispatchState(ctypes.Structure):
+    _fields_ = [
+        ("constant_count", ctypes.c_uint32),
+        ("constants", ctypes.POINTER(ctypes.c_uint32)),
+        ("binding_count", ctypes.c_uint32),
+        ("binding_ptrs", ctypes.POINTER(ctypes.c_void_p)),
+        ("binding_lengths", ctypes.POINTER(ctypes.c_size_t)),
+        ("binding_flags", ctypes.POINTER(ctypes.c_uint8)),
+    ]
+
+
+class HlConv2d(ctypes.Structure):
+    _fields_ = [
+        ("init", ctypes.c_int32), ("input_zp", ctypes.c_int32), ("weight_zp", ctypes.c_int32),
+        ("output_zp", ctypes.c_int32), ("output_min", ctypes.c_int32), ("output_max", ctypes.c_int32),
+        ("shift_factor", ctypes.c_int32), ("groups", ctypes.c_int32),
+        ("pad", ctypes.c_int64 * 4), ("stride", ctypes.c_int64 * 2), ("dilation", ctypes.c_int64 * 2),
+        ("vectorization_mode", ctypes.c_int32), ("weights", ctypes.c_int32),
+        ("scale_bias", ctypes.c_int32), ("input", ctypes.c_int32),
+        ("nhwc_input", ctypes.c_int32), ("segment_output", ctypes.c_int32),
+    ]
+
+
+class HlDepthwiseConv2d(ctypes.Structure):
+    _fields_ = HlConv2d._fields_ + [("is_dw1d_stride1", ctypes.c_int32)]
+
+
+class HlFullyConnected(ctypes.Structure):
+    _fields_ = [
+        ("init", ctypes.c_int32), ("input_zp", ctypes.c_int32), ("weight_zp", ctypes.c_int32),
+        ("output_zp", ctypes.c_int32), ("output_min", ctypes.c_int32), ("output_max", ctypes.c_int32),
+        ("shift_factor", ctypes.c_int32), ("vectorization_mode", ctypes.c_int32),
+        ("weights", ctypes.c_int32), ("scale_bias", ctypes.c_int32), ("input", ctypes.c_int32),
+    ]
+
+
+class HlMatmul(ctypes.Structure):
+    _fields_ = [
+        ("init", ctypes.c_int32), ("output_zp", ctypes.c_int32), ("output_min", ctypes.c_int32),
+        ("output_max", ctypes.c_int32), ("shift", ctypes.c_int32), ("scale_bias", ctypes.c_int32),
+        ("input1", ctypes.c_int32), ("input2", ctypes.c_int32),
+    ]
+
+
+class HlMaxPool2d(ctypes.Structure):
+    _fields_ = [
+        ("init", ctypes.c_int32), ("input_zp", ctypes.c_int32), ("output_min", ctypes.c_int32),
+        ("output_max", ctypes.c_int32), ("stride", ctypes.c_int64 * 2), ("pad", ctypes.c_int64 * 4),
+        ("kernel", ctypes.c_int64 * 2), ("weights", ctypes.c_int32), ("scale_bias", ctypes.c_int32),
+        ("input", ctypes.c_int32), ("segment_output", ctypes.c_int32), ("nhwc_input", ctypes.c_int32),
+    ]
+
+
+class HlAvgPool2d(ctypes.Structure):
+    _fields_ = [
+        ("init", ctypes.c_int32), ("input_zp", ctypes.c_int32), ("output_zp", ctypes.c_int32),
+        ("output_min", ctypes.c_int32), ("output_max", ctypes.c_int32), ("shift_factor", ctypes.c_int32),
+        ("weights", ctypes.c_int32), ("scale_bias", ctypes.c_int32), ("input", ctypes.c_int32),
+    ]
+
+
+class HlAdd(ctypes.Structure):
+    _fields_ = [
+        ("init", ctypes.c_int32), ("name", ctypes.c_char_p), ("input_zp", ctypes.c_int32),
+        ("output_zp", ctypes.c_int32), ("output_min", ctypes.c_int32), ("output_max", ctypes.c_int32),
+        ("shift_factor", ctypes.c_int32), ("weights", ctypes.c_int32), ("scale_bias", ctypes.c_int32),
+        ("input1", ctypes.c_int32), ("input2", ctypes.c_int32), ("segment_output", ctypes.c_int32),
+        ("rhs_is_scalar", ctypes.c_int32),
+    ]
+
+
+class HlTranspose(ctypes.Structure):
+    _fields_ = [
+        ("init", ctypes.c_int32), ("rank", ctypes.c_int32), ("perm", ctypes.c_int64 * 4),
+        ("input", ctypes.c_int32),
+    ]
+
+
+_lib = None
+
+
+def library_built():
+    return os.path.exists(LIB_PATH)
+
+
+def lib():
+    """Loads ``libthip.so``; raises if it has not been built (no fallback)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not library_built():
+        raise ThipError(UNAVAILABLE, "%s is missing: run `python torq-compiler_amd/build.py` "
+                                     "(or __graft_entry__.build()) first" % LIB_PATH)
+    L = ctypes.CDLL(LIB_PATH)
+    L.thip_status_message.restype = ctypes.c_char_p
+    L.thip_version.restype = ctypes.c_uint32
+    L.thip_descriptor_version.restype = ctypes.c_uint32
+    vp, i32, u32, sz = ctypes.c_void_p, ctypes.c_int32, ctypes.c_uint32, ctypes.c_size_t
+    P = ctypes.POINTER
+    L.thip_program_create.argtypes = [P(vp)]
+    L.thip_program_destroy.argtypes = [vp]
+    L.thip_program_destroy.restype = None
+    L.thip_program_binding.argtypes = [vp, u32, i32, i32, P(ctypes.c_int64), P(i32)]
+    L.thip_program_constant.argtypes = [vp, i32, i32, P(ctypes.c_int64), vp, sz, P(i32)]
+    L.thip_program_tensor.argtypes = [vp, i32, i32, P(ctypes.c_int64), P(i32)]
+    for name, st in [("thip_hl_conv2d", HlConv2d), ("thip_hl_depthwise_conv2d", HlDepthwiseConv2d),
+                     ("thip_hl_fully_connected", HlFullyConnected), ("thip_hl_matmul", HlMatmul),
+                     ("thip_hl_maxpool2d", HlMaxPool2d), ("thip_hl_avg_pool2d", HlAvgPool2d),
+                     ("thip_hl_add", HlAdd), ("thip_hl_transpose", HlTranspose)]:
+        getattr(L, name).argtypes = [vp, P(st)]
+    L.thip_program_serialize.argtypes = [vp, P(vp), P(sz)]
+    L.thip_blob_free.argtypes = [vp]
+    L.thip_blob_free.restype = None
+    L.thip_device_create.argtypes = [i32, P(vp)]
+    L.thip_device_destroy.argtypes = [vp]
+    L.thip_device_destroy.restype = None
+    L.thip_device_name.argtypes = [vp, ctypes.c_char_p, sz]
+    L.thip_device_alloc.argtypes = [vp, sz, P(vp)]
+    L.thip_device_free.argtypes = [vp, vp]
+    L.thip_device_h2d.argtypes = [vp, vp, vp, sz]
+    L.thip_device_d2h.argtypes = [vp, vp, vp, sz]
+    L.thip_device_synchronize.argtypes = [vp]
+    L.thip_device_set_event_log.argtypes = [vp, ctypes.c_char_p]
+    L.thip_infer_format.argtypes = [vp, sz, sz, ctypes.c_char_p, P(sz)]
+    L.thip_executable_create.argtypes = [vp, vp, sz, P(u32), sz, P(vp)]
+    L.thip_executable_destroy.argtypes = [vp]
+    L.thip_executable_destroy.restype = None
+    L.thip_executable_run.argtypes = [vp, P(DispatchState)]
+    L.thip_executable_enqueue.argtypes = [vp, P(DispatchState)]
+    L.thip_executable_wait.argtypes = [vp]
+    L.thip_executable_time.argtypes = [vp, P(DispatchState), i32, P(ctypes.c_float)]
+    L.thip_executable_op_count.argtypes = [vp, P(u32)]
+    L.thip_executable_op_kernel.argtypes = [vp, u32, ctypes.c_char_p, sz]
+    L.thip_executable_binding_count.argtypes = [vp, P(u32)]
+    L.thip_executable_binding_size.argtypes = [vp, u32, P(sz)]
+    _lib = L
+    return L
+
+
+def check(code):
+    if code != OK:
+        raise ThipError(code, lib().thip_status_message().decode("utf-8", "replace"))
+
+
+def _shape_array(shape):
+    return (ctypes.c_int64 * len(shape))(*[int(s) for s in shape])
+
+
+class Device:
+    """A gfx950 GPU (thip_device_t)."""
+
+    def __init__(self, ordinal=0):
+        self._h = ctypes.c_void_p()
+        check(lib().thip_device_create(int(ordinal), ctypes.byref(self._h)))
+
+    @property
+    def handle(self):
+        return self._h
+
+    def name(self):
+        buf = ctypes.create_string_buffer(64)
+        check(lib().thip_device_name(self._h, buf, 64))
+        return buf.value.decode()
+
+    def alloc(self, size):
+        p = ctypes.c_void_p()
+        check(lib().thip_device_alloc(self._h, int(size), ctypes.byref(p)))
+        return p.value
+
+    def free(self, ptr):
+        check(lib().thip_device_free(self._h, ctypes.c_void_p(ptr)))
+
+    def upload(self, array):
+        """Copies a numpy array into new device memory; returns the device pointer."""
+        a = np.ascontiguousarray(array)
+        p = self.alloc(max(a.nbytes, 1))
+        check(lib().thip_device_h2d(self._h, ctypes.c_void_p(p), a.ctypes.data_as(ctypes.c_void_p), a.nbytes))
+        return p
+
+    def download(self, ptr, shape, dtype):
+        out = np.empty(shape, dtype=dtype)
+        check(lib().thip_device_d2h(self._h, out.ctypes.data_as(ctypes.c_void_p), ctypes.c_void_p(ptr), out.nbytes))
+        return out
+
+    def synchronize(self):
+        check(lib().thip_device_synchronize(self._h))
+
+    def set_event_log(self, path):
+        check(lib().thip_device_set_event_log(self._h, path.encode() if path else None))
+
+    def close(self):
+        if self._h:
+            lib().thip_device_destroy(self._h)
+            self._h = ctypes.c_void_p()
+
+
+def infer_format(blob):
+    buf = ctypes.create_string_buffer(32)
+    size = ctypes.c_size_t(0)
+    check(lib().thip_infer_format(blob, len(blob), 32, buf, ctypes.byref(size)))
+    return buf.value.decode(), size.value
+
+
+def make_state(ptrs, lengths, flags, constants=None):
+    """Builds a thip_dispatch_state_t; returns (state, keepalive)."""
+    n = len(ptrs)
+    ptr_arr = (ctypes.c_void_p * max(n, 1))(*[ctypes.c_void_p(p) for p in ptrs])
+    len_arr = (ctypes.c_size_t * max(n, 1))(*[int(l) for l in lengths])
+    flag_arr = (ctypes.c_uint8 * max(n, 1))(*[int(f) for f in flags])
+    st = DispatchState()
+    if constants is not None and len(constants):
+        c = np.ascontiguousarray(constants, dtype=np.uint32)
+        st.constant_count = c.size
+        st.constants = c.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32))
+    else:
+        c = None
+        st.constant_count = 0
+        st.constants = None
+    st.binding_count = n
+    st.binding_ptrs = ctypes.cast(ptr_arr, ctypes.POINTER(ctypes.c_void_p))
+    st.binding_lengths = ctypes.cast(len_arr, ctypes.POINTER(ctypes.c_size_t))
+    st.binding_flags = ctypes.cast(flag_arr, ctypes.POINTER(ctypes.c_uint8))
+    return st, (ptr_arr, len_arr, flag_arr, c)
+
+
+class Executable:
+    """A loaded dispatch descriptor (thip_executable_t)."""
+
+    def __init__(self, device, blob, constants=None):
+        self.device = device
+        self._h = ctypes.c_void_p()
+        cptr, ccount = None, 0
+        if constants is not None and len(constants):
+            self._constants = np.ascontiguousarray(constants, dtype=np.uint32)
+            cptr = self._constants.ctypes.data_as(ctypes.POINTER(ctypes.c_uint32))
+            ccount = self._constants.size
+        check(lib().thip_executable_create(device.handle, blob, len(blob), cptr, ccount, ctypes.byref(self._h)))
+
+    def op_kernels(self):
+        n = ctypes.c_uint32()
+        check(lib().thip_executable_op_count(self._h, ctypes.byref(n)))
+        names = []
+        for i in range(n.value):
+            buf = ctypes.create_string_buffer(64)
+            check(lib().thip_executable_op_kernel(self._h, i, buf, 64))
+            names.append(buf.value.decode())
+        return names
+
+    def binding_sizes(self):
+        n = ctypes.c_uint32()
+        check(lib().thip_executable_binding_count(self._h, ctypes.byref(n)))
+        sizes = []
+        for i in range(n.value):
+            s = ctypes.c_size_t()
+            check(lib().thip_executable_binding_size(self._h, i, ctypes.byref(s)))
+            sizes.append(s.value)
+        return sizes
+
+    def run_host(self, arrays):
+        """Blocking dispatch on host numpy arrays (inputs and outputs, in binding order)."""
+        ptrs = [a.ctypes.data for a in arrays]
+        st, keep = make_state(ptrs, [a.nbytes for a in arrays], [BINDING_HOST] * len(arrays))
+        check(lib().thip_executable_run(self._h, ctypes.byref(st)))
+        del keep
+
+    def run_device(self, ptrs, lengths):
+        st, keep = make_state(ptrs, lengths, [BINDING_DEVICE] * len(ptrs))
+        check(lib().thip_executable_run(self._h, ctypes.byref(st)))
+        del keep
+
+    def run_state(self, state):
+        check(lib().thip_executable_run(self._h, ctypes.byref(state)))
+
+    def enqueue_device(self, ptrs, lengths):
+        st, keep = make_state(ptrs, lengths, [BINDING_DEVICE] * len(ptrs))
+        check(lib().thip_executable_enqueue(self._h, ctypes.byref(st)))
+        del keep
+
+    def wait(self):
+        check(lib().thip_executable_wait(self._h))
+
+    def time_device(self, ptrs, lengths, iterations):
+        """Mean milliseconds per dispatch over `iterations`, HIP events on the executable's stream."""
+        st, keep = make_state(ptrs, lengths, [BINDING_DEVICE] * len(ptrs))
+        ms = ctypes.c_float()
+        check(lib().thip_executable_time(self._h, ctypes.byref(st), int(iterations), ctypes.byref(ms)))
+        del keep
+        return ms.value
+
+    def close(self):
+        if self._h:
+            lib().thip_executable_destroy(self._h)
+            self._h = ctypes.c_void_p()

@@ -1,0 +1,193 @@
+"""Seeded synthetic workloads at the benchmark shapes.
+
+Each builder returns a :class:`Workload`: the TorqHL program (one or more ops),
+the host input arrays in binding order, the output shapes, and the algorithmic
+work (ops and bytes) used for roofline accounting.
+
+Requantisation parameters are derived the way the reference's patterns derive
+them (compile side, unchanged by this backend):
+  shift_factor = min_c shift[c]           compiler/torq/Conversions/LinalgToTorqHL/PatternUtils.cpp:3230-3283
+  scale[c] = multiplier[c] >> (shift[c] - shift_factor)                   PatternUtils.cpp:3536-3548
+  bias[c]  = tosa_bias[c] - input_zp * sum(w[c])        compiler/torq/Utils/ConversionUtils.h:301-329
+  scale_bias = interleave(bias, scale)                 compiler/torq/Utils/ConversionUtils.cpp:88-103
+"""
+import numpy as np
+
+from .torq_hl import Program
+
+
+class Workload:
+    def __init__(self, name, program, inputs, outputs, ops, bytes_, attrs=None):
+        self.name = name
+        self.program = program
+        self.inputs = inputs      # list of numpy arrays, binding 0..n-1
+        self.outputs = outputs    # list of (shape, dtype), bindings n..
+        self.ops = ops            # algorithmic integer ops (1 MAC = 2 ops)
+        self.bytes = bytes_       # algorithmic bytes: every operand once + output once
+        self.attrs = attrs or {}  # the op parameters, for the checker
+
+
+def derive_scale_bias(multiplier, shift, tosa_bias, weights, input_zp):
+    """R2 for conv / depthwise / fully_connected.  weights: [channels, ...]."""
+    multiplier = np.asarray(multiplier, dtype=np.int32)
+    shift = np.asarray(shift, dtype=np.int64)
+    shift_factor = int(shift.min())
+    scale = (multiplier.astype(np.int64) >> (shift - shift_factor)).astype(np.int32)
+    wsum = weights.reshape(weights.shape[0], -1).astype(np.int64).sum(axis=1)
+    bias = (np.asarray(tosa_bias, dtype=np.int64) - wsum * int(input_zp)).astype(np.int32)
+    sb = np.empty(2 * multiplier.size, dtype=np.int32)
+    sb[0::2] = bias
+    sb[1::2] = scale
+    return sb, shift_factor
+
+
+def random_requant(rng, channels, realistic):
+    """Per-channel TOSA (multiplier, shift).  The literal benchmark ranges (shift 6..12)
+    saturate every output; `realistic` draws shifts 36..42 so the rounding path is exercised."""
+    mult = rng.integers(1 << 30, (1 << 31) - 1, size=channels, endpoint=True, dtype=np.int64).astype(np.int32)
+    if realistic:
+        shift = rng.integers(36, 42, size=channels, endpoint=True)
+    else:
+        shift = rng.integers(6, 12, size=channels, endpoint=True)
+    return mult, shift.astype(np.int8)
+
+
+def conv2d_workload(N=1, H=112, W=112, C=32, O=64, KH=3, KW=3, stride=(1, 1), pad=(1, 1, 1, 1),
+                    input_zp=-3, output_zp=5, output_min=5, output_max=127, realistic=False,
+                    nhwc=True, seed=1000):
+    """BASELINE config 0 by default: NHWC 1x112x112x32 -> 1x112x112x64, 3x3, SAME."""
+    rng = np.random.default_rng(seed)
+    x = rng.integers(-128, 127, size=(N, H, W, C), endpoint=True, dtype=np.int8)
+    w_hwio = rng.integers(-127, 127, size=(KH, KW, C, O), endpoint=True, dtype=np.int8)
+    w = np.ascontiguousarray(w_hwio.transpose(3, 2, 0, 1))  # O,I,KH,KW as the op takes them
+    tosa_bias = rng.integers(-(1 << 15), 1 << 15, size=O, endpoint=True, dtype=np.int64)
+    mult, shift = random_requant(rng, O, realistic)
+    sb, sf = derive_scale_bias(mult, shift, tosa_bias, w, input_zp)
+    attrs = dict(input_zp=input_zp, output_zp=output_zp, output_min=output_min, output_max=output_max,
+                 shift_factor=sf, pad=tuple(pad), stride=tuple(stride))
+    p = Program()
+    if not nhwc:
+        x = np.ascontiguousarray(x.transpose(0, 3, 1, 2))
+    inp = p.binding(0, x.shape)
+    OH = (H + pad[2] + pad[3] - KH) // stride[0] + 1
+    OW = (W + pad[0] + pad[1] - KW) // stride[1] + 1
+    oshape = (N, OH, OW, O) if nhwc else (N, O, OH, OW)
+    out = p.binding(1, oshape)
+    p.conv2d(inp, w, sb, init=out, nhwc_input=nhwc, **attrs)
+    macs = N * OH * OW * O * KH * KW * C
+    bytes_ = x.nbytes + w.nbytes + sb.nbytes + N * OH * OW * O
+    attrs.update(weights=w, scale_bias=sb, nhwc=nhwc)
+    return Workload("conv2d_%dx%dx%dx%d_o%d_k%dx%d" % (N, H, W, C, O, KH, KW), p, [x], [(oshape, np.int8)],
+                    2 * macs, bytes_, attrs)
+
+
+def fully_connected_workload(M, K, N, realistic=False, output_zp=5, output_min=-128, output_max=127,
+                             seed=1001):
+    """BASELINE config 1: int8 [M,K] x [N,K]^T with per-column requant."""
+    rng = np.random.default_rng(seed)
+    x = rng.integers(-128, 127, size=(M, K), endpoint=True, dtype=np.int8)
+    w = rng.integers(-128, 127, size=(N, K), endpoint=True, dtype=np.int8)
+    tosa_bias = rng.integers(-(1 << 15), 1 << 15, size=N, endpoint=True, dtype=np.int64)
+    mult, shift = random_requant(rng, N, realistic)
+    sb, sf = derive_scale_bias(mult, shift, tosa_bias, w, 0)
+    attrs = dict(output_zp=output_zp, output_min=output_min, output_max=output_max, shift_factor=sf)
+    p = Program()
+    inp = p.binding(0, (M, K))
+    out = p.binding(1, (M, N))
+    p.fully_connected(inp, w, sb, init=out, **attrs)
+    bytes_ = x.nbytes + w.nbytes + sb.nbytes + M * N
+    attrs.update(weights=w, scale_bias=sb)
+    return Workload("fully_connected_%dx%dx%d" % (M, K, N), p, [x], [((M, N), np.int8)], 2 * M * K * N,
+                    bytes_, attrs)
+
+
+def depthwise_workload(N=1, H=56, W=56, C=144, KH=3, KW=3, stride=(2, 2), pad=(0, 1, 0, 1), input_zp=-3,
+                       output_zp=5, output_min=-128, output_max=127, realistic=True, nhwc=True, seed=1002):
+    """BASELINE config 2a: depthwise 3x3 stride 2 SAME on 56x56x144."""
+    rng = np.random.default_rng(seed)
+    x = rng.integers(-128, 127, size=(N, H, W, C), endpoint=True, dtype=np.int8)
+    w = rng.integers(-127, 127, size=(C, 1, KH, KW), endpoint=True, dtype=np.int8)
+    tosa_bias = rng.integers(-(1 << 15), 1 << 15, size=C, endpoint=True, dtype=np.int64)
+    mult, shift = random_requant(rng, C, realistic)
+    if realistic:
+        shift = (shift - 4).astype(np.int8)  # only 9 taps: keep outputs spread over the int8 range
+    sb, sf = derive_scale_bias(mult, shift, tosa_bias, w, input_zp)
+    attrs = dict(input_zp=input_zp, output_zp=output_zp, output_min=output_min, output_max=output_max,
+                 shift_factor=sf, pad=tuple(pad), stride=tuple(stride))
+    p = Program()
+    if not nhwc:
+        x = np.ascontiguousarray(x.transpose(0, 3, 1, 2))
+    inp = p.binding(0, x.shape)
+    OH = (H + pad[2] + pad[3] - KH) // stride[0] + 1
+    OW = (W + pad[0] + pad[1] - KW) // stride[1] + 1
+    oshape = (N, OH, OW, C) if nhwc else (N, C, OH, OW)
+    out = p.binding(1, oshape)
+    p.depthwise_conv2d(inp, w, sb, init=out, nhwc_input=nhwc, **attrs)
+    macs = N * OH * OW * C * KH * KW
+    bytes_ = x.nbytes + w.nbytes + sb.nbytes + N * OH * OW * C
+    attrs.update(weights=w, scale_bias=sb, nhwc=nhwc)
+    return Workload("depthwise_%dx%dx%dx%d_k%dx%d_s%d" % (N, H, W, C, KH, KW, stride[0]), p, [x],
+                    [(oshape, np.int8)], 2 * macs, bytes_, attrs)
+
+
+def maxpool_workload(N=1, H=112, W=112, C=64, kernel=(2, 2), stride=(2, 2), pad=(0, 0, 0, 0), input_zp=-128,
+                     nhwc=True, seed=1003):
+    """BASELINE config 2b: maxpool 2x2 stride 2 on 112x112x64."""
+    rng = np.random.default_rng(seed)
+    x = rng.integers(-128, 127, size=(N, H, W, C), endpoint=True, dtype=np.int8)
+    attrs = dict(input_zp=input_zp, output_min=-128, output_max=127, stride=tuple(stride), pad=tuple(pad),
+                 kernel=tuple(kernel))
+    p = Program()
+    if not nhwc:
+        x = np.ascontiguousarray(x.transpose(0, 3, 1, 2))
+    inp = p.binding(0, x.shape)
+    OH = (H + pad[2] + pad[3] - kernel[0]) // stride[0] + 1
+    OW = (W + pad[0] + pad[1] - kernel[1]) // stride[1] + 1
+    oshape = (N, OH, OW, C) if nhwc else (N, C, OH, OW)
+    out = p.binding(1, oshape)
+    p.maxpool2d(inp, init=out, nhwc_input=nhwc, **attrs)
+    attrs.update(nhwc=nhwc)
+    return Workload("maxpool_%dx%dx%dx%d" % (N, H, W, C), p, [x], [(oshape, np.int8)],
+                    N * OH * OW * C * kernel[0] * kernel[1], x.nbytes + N * OH * OW * C, attrs)
+
+
+def avgpool_workload(N=1, H=7, W=7, C=1280, input_zp=-3, output_zp=5, seed=1004):
+    """BASELINE config 2c: global average pool on 7x7x1280 (NHWC), scale = floor(2^20 / 49)."""
+    rng = np.random.default_rng(seed)
+    x = rng.integers(-128, 127, size=(N, H, W, C), endpoint=True, dtype=np.int8)
+    # compiler/torq/Conversions/LinalgToTorqHL/PoolingPattern.cpp:325-328
+    sb = np.array([-(H * W * input_zp), int((1 << 20) / (H * W))], dtype=np.int32)
+    attrs = dict(input_zp=input_zp, output_zp=output_zp, output_min=-128, output_max=127, shift_factor=20)
+    p = Program()
+    inp = p.binding(0, x.shape)
+    out = p.binding(1, (N, 1, 1, C))
+    p.avg_pool2d(inp, np.array([1], dtype=np.int8), sb, init=out, **attrs)
+    attrs.update(scale_bias=sb)
+    return Workload("avgpool_%dx%dx%dx%d" % (N, H, W, C), p, [x], [((N, 1, 1, C), np.int8)], N * H * W * C,
+                    x.nbytes + N * C, attrs)
+
+
+def add_params(m0, m1, zp0, zp1, sign=1):
+    """Quantised add parameters: compiler/torq/Conversions/LinalgToTorqHL/ElementWiseBinaryPattern.cpp:459-487."""
+    S = 1 << 12
+    w0 = np.int16(int(m0 * S))
+    w1 = np.int16(int(m1 * S) * sign)
+    bias = -int(m0 * S * zp0) - int(m1 * S * zp1) * sign
+    return np.array([w0, w1], dtype=np.int16), np.array([bias, 1], dtype=np.int32), 12
+
+
+def add_workload(N=1, H=56, W=56, C=24, zp0=-3, zp1=7, m0=0.71838506, m1=1.3 * 0.5, output_zp=-2, seed=1005):
+    """BASELINE config 2d: quantised add of two 56x56x24 tensors with distinct zero points and scales."""
+    rng = np.random.default_rng(seed)
+    a = rng.integers(-128, 127, size=(N, H, W, C), endpoint=True, dtype=np.int8)
+    b = rng.integers(-128, 127, size=(N, H, W, C), endpoint=True, dtype=np.int8)
+    wts, sb, sf = add_params(m0, m1, zp0, zp1)
+    attrs = dict(output_zp=output_zp, output_min=-128, output_max=127, shift_factor=sf)
+    p = Program()
+    i0 = p.binding(0, a.shape)
+    i1 = p.binding(1, b.shape)
+    out = p.binding(2, a.shape)
+    p.add(i0, i1, wts, sb, init=out, **attrs)
+    attrs.update(weights=wts, scale_bias=sb)
+    return Workload("add_%dx%dx%dx%d" % (N, H, W, C), p, [a, b], [(a.shape, np.int8)], 3 * a.size, 3 * a.nbytes,
+                    attrs)
