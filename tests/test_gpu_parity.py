@@ -63,6 +63,19 @@ def test_conv2d_every_tile_variant(device, variant, monkeypatch):
     check(device, w.fully_connected_workload(300, 192, 520, realistic=True))
 
 
+@pytest.mark.parametrize("variant", [4, 5, 6, 7])
+def test_dense_igemm_every_tile_variant(device, variant, monkeypatch):
+    """The LDS-DMA kernel: whole tiles, ragged M / N / K tails, K shorter than the stage ring."""
+    monkeypatch.setenv("THIP_IGEMM_DENSE_VARIANT", str(variant))
+    k = check(device, w.fully_connected_workload(300, 192, 520, realistic=True))
+    assert "igemm_dense_i8" in k[0]
+    check(device, w.fully_connected_workload(512, 1024, 512, realistic=True))
+    check(device, w.fully_connected_workload(257, 80, 48, realistic=True))
+    check(device, w.fully_connected_workload(33, 16, 1000, realistic=True))
+    check(device, w.fully_connected_workload(1000, 4096, 272, realistic=True))
+    check(device, w.conv2d_workload(N=2, H=28, W=28, C=192, O=32, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True))
+
+
 def test_conv2d_mbv2_layer_shapes(device):
     # first layer (3 channels, stride 2, TF SAME), expand / project 1x1, last 1x1
     check(device, w.conv2d_workload(N=2, H=224, W=224, C=3, O=32, stride=(2, 2), pad=(0, 1, 0, 1), realistic=True, input_zp=-1))
@@ -98,7 +111,7 @@ def test_conv2d_int32_output(device):
 def test_fully_connected_config1(device, mkn):
     M = mkn[0]
     check(device, w.fully_connected_workload(*mkn, realistic=True), via="device",
-          kernel="fc_skinny" if M <= 16 else "igemm_i8")
+          kernel="fc_skinny" if M <= 16 else "igemm_")
 
 
 def test_fully_connected_config1_literal_ranges(device):
@@ -113,7 +126,7 @@ def test_fully_connected_geometries(device, mkn):
 
 def test_fully_connected_without_skinny_kernel(device, monkeypatch):
     monkeypatch.setenv("THIP_NO_SKINNY", "1")
-    check(device, w.fully_connected_workload(16, 2048, 512, realistic=True), kernel="igemm_i8")
+    check(device, w.fully_connected_workload(16, 2048, 512, realistic=True), kernel="igemm_")
 
 
 # ---- bandwidth ops ---------------------------------------------------------------------------

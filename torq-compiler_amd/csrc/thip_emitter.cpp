@@ -326,15 +326,28 @@ class Emitter {
         return THIP_OK;
     }
 
-    static uint32_t chooseIgemmVariant(int64_t M, int64_t N) {
-        if (const char *env = getenv("THIP_IGEMM_VARIANT")) {
-            const long v = strtol(env, nullptr, 10);
-            if (v >= 0 && v < (long)kIgemmVariantCount) return (uint32_t)v;
-        }
+    // Tile choice.  THIP_IGEMM_VARIANT / THIP_IGEMM_DENSE_VARIANT force one (for tuning runs).
+    static uint32_t chooseIgemmVariant(int64_t M, int64_t N, bool dense) {
         auto tiles = [&](uint32_t v) {
             const IgemmTile &t = igemmTile(v);
             return ((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn);
         };
+        if (dense) {
+            if (const char *env = getenv("THIP_IGEMM_DENSE_VARIANT")) {
+                const long v = strtol(env, nullptr, 10);
+                if (v >= 0 && v < (long)kIgemmVariantCount) return (uint32_t)v;
+            }
+            // the largest tile that still gives (nearly) every CU a tile
+            const uint32_t order[] = {kIgemmDense256x256, kIgemmDense128x256, kIgemmDense128x128};
+            for (uint32_t v : order) {
+                if (tiles(v) >= 224) return v;
+            }
+            return kIgemmDense64x64;
+        }
+        if (const char *env = getenv("THIP_IGEMM_VARIANT")) {
+            const long v = strtol(env, nullptr, 10);
+            if (v >= 0 && v < (long)kIgemmDense256x256) return (uint32_t)v;
+        }
         // Enough 128x128 tiles to give every CU work; otherwise the small tile.
         if (tiles(kIgemm128x128x64) >= 256) return kIgemm128x128x64;
         return kIgemm64x64x64;
@@ -344,7 +357,7 @@ class Emitter {
     // weight (n, k) with k = (kh * KW + kw) * C + ci.
     template <typename WeightAt>
     void emitIgemm(DescOp base, int64_t M, int64_t N, int64_t K, bool dense, WeightAt wAt) {
-        const uint32_t variant = chooseIgemmVariant(M, N);
+        const uint32_t variant = chooseIgemmVariant(M, N, dense);
         const IgemmTile &t = igemmTile(variant);
         const int64_t Kp = roundUp(K, t.bk), Np = roundUp(N, t.bn);
         std::vector<int8_t> packed((size_t)(Np * Kp), 0);
@@ -625,7 +638,7 @@ thip_status_t Emitter::emitMatmul(const thip_hl_matmul_t &c) {
     DescRef bRef;
     if (thip_status_t s = literalInput(c.input2, "torq_hl.matmul input2", &bRef)) return s;
     if (K % 16 != 0) return fail(THIP_UNIMPLEMENTED, "%s: a run-time input2 needs K %% 16 == 0", what);
-    const uint32_t variant = chooseIgemmVariant(M, N);
+    const uint32_t variant = chooseIgemmVariant(M, N, true);
     const IgemmTile &t = igemmTile(variant);
     const int64_t Kp = roundUp(K, t.bk), Np = roundUp(N, t.bn);
     if (Kp != K) return fail(THIP_UNIMPLEMENTED, "%s: a run-time input2 needs K %% %d == 0", what, t.bk);

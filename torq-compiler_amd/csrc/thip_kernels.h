@@ -39,7 +39,12 @@ enum IgemmVariant : uint32_t {
     kIgemm256x256x64 = 1,
     kIgemm64x64x64 = 2,
     kIgemm256x128x64 = 3,
-    kIgemmVariantCount = 4,
+    // dense [M, K] operand only: tiles moved by LDS DMA through a ring of stages
+    kIgemmDense256x256 = 4,
+    kIgemmDense128x128 = 5,
+    kIgemmDense128x256 = 6,
+    kIgemmDense64x64 = 7,
+    kIgemmVariantCount = 8,
 };
 struct IgemmTile {
     int bm, bn, bk;

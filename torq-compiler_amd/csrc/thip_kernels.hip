@@ -14,6 +14,8 @@
 // output zero point, clamp.
 #include "thip_kernels.h"
 
+#include <type_traits>
+
 #include "thip_descriptor.h"
 
 namespace thip {
@@ -27,12 +29,26 @@ constexpr int kDtypeI8 = 1, kDtypeI16 = 2, kDtypeI32 = 3;
 __device__ __forceinline__ int32_t requant(int32_t acc, int32_t bias, int32_t scale, long long rnd,
                                            const Requant &rq) {
     const int32_t t0 = (int32_t)((uint32_t)acc + (uint32_t)bias);
-    const long long t1 = (long long)t0 * (long long)scale;
-    const long long t3 = (t1 + rnd) >> rq.shift;
-    long long t4 = t3 + (long long)rq.out_zp;
-    t4 = t4 < (long long)rq.out_min ? (long long)rq.out_min : t4;
-    t4 = t4 > (long long)rq.out_max ? (long long)rq.out_max : t4;
-    return (int32_t)t4;
+    const long long t3 = ((long long)t0 * (long long)scale + rnd) >> rq.shift;
+    // clamp(t3 + zp, min, max) == clamp(t3, min - zp, max - zp) + zp; the bounds cannot overflow
+    // 64 bits, and the sum of the low words is exact because the result fits 32 bits
+    const long long lo = (long long)rq.out_min - (long long)rq.out_zp;
+    const long long hi = (long long)rq.out_max - (long long)rq.out_zp;
+    uint32_t q = (uint32_t)t3;
+    q = t3 < lo ? (uint32_t)lo : q;
+    q = t3 > hi ? (uint32_t)hi : q;
+    return (int32_t)(q + (uint32_t)rq.out_zp);
+}
+
+// Same result when shift >= 32: the shifted product fits 32 bits, so the tail is 32-bit work.
+__device__ __forceinline__ int32_t requantWideShift(int32_t acc, int32_t bias, int32_t scale, long long rnd,
+                                                    int shiftMinus32, int32_t lo, int32_t hi, int32_t zp) {
+    const int32_t t0 = (int32_t)((uint32_t)acc + (uint32_t)bias);
+    const long long t2 = (long long)t0 * (long long)scale + rnd;
+    int32_t t3 = (int32_t)(t2 >> 32) >> shiftMinus32;
+    t3 = t3 < lo ? lo : t3;
+    t3 = t3 > hi ? hi : t3;
+    return (int32_t)((uint32_t)t3 + (uint32_t)zp);
 }
 
 __device__ __forceinline__ long long roundTerm(int shift) {
@@ -276,11 +292,328 @@ __global__ __launch_bounds__(256) void igemm_i8(IgemmArgs p) {
     }
 }
 
+
+// ---------------------------------------------------------------------------
+// igemm_dense_i8: the dense [M, K] x [N, K]^T case (fully_connected, matmul,
+// stride-1 1x1 conv2d) with the tiles moved global -> LDS by the DMA path
+// (global_load_lds_dwordx4: no VGPRs, no ds_write) through a ring of STAGES
+// LDS stages, so several k-tiles of loads are in flight while one is computed.
+//
+// One DMA instruction of a wave writes 64 lanes x 16 bytes = 1 KiB of
+// consecutive LDS, i.e. 16 tile rows of 64 bytes; lanes cannot scatter.  Bank
+// conflicts are therefore avoided on the global side: the 16-byte slot at
+// position p of row r holds the logical k-chunk p ^ ((r >> 2) & 3), which makes
+// the 16 rows read by one ds_read_b128 phase fall into 16 distinct bank groups.
+//
+// The loads are issued by inline asm and waited on by hand (s_waitcnt vmcnt(n)
+// with n = loads of the tiles still allowed in flight).  Every wave issues the
+// same number of loads per k-tile (out-of-range rows and k-chunks are clamped
+// to valid addresses rather than skipped) so that the count is exact.
+//
+// The MFMA takes the weights as its row operand and the activations as its
+// column operand: accumulator register r of lane l then holds
+// C[m = l & 31][n = 8 * (r / 4) + 4 * (l >> 5) + (r & 3)], four consecutive
+// output channels per register group, which requantise into one 32-bit store.
+__device__ __forceinline__ void dmaLoad16(const void *gptr, unsigned ldsAddr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(ldsAddr), "v"(gptr) : "memory", "m0");
+}
+
+template <int N>
+__device__ __forceinline__ void waitVmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+__device__ __forceinline__ void blockBarrier() { asm volatile("s_barrier" : : : "memory"); }
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_dense_i8(IgemmArgs p) {
+    constexpr int BK = 64;
+    constexpr int NW = WAVES_M * WAVES_N;
+    constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    constexpr int LA = BM / 16 / NW, LB = BN / 16 / NW;  // DMA instructions per wave per k-tile
+    constexpr int LPT = LA + LB;
+    constexpr int A_STAGE = BM * BK, B_STAGE = BN * BK, STAGE = A_STAGE + B_STAGE;
+    static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "every wave must issue the same number of loads");
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the MFMA tile");
+    static_assert(STAGES >= 2 && STAGES <= 5 && LPT * (STAGES - 1) < 64, "vmcnt is a 6-bit counter");
+
+    extern __shared__ __align__(16) int8_t smem[];
+    const unsigned ldsBase = (unsigned)(uintptr_t)(__attribute__((address_space(3))) int8_t *)smem;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+
+    const int tilesM = (p.M + BM - 1) / BM;
+    const int tilesN = p.Np / BN;
+    int lin;
+    {
+        const int nb = (int)gridDim.x, pid = (int)blockIdx.x;
+        const int per = nb / 8, rem = nb % 8;
+        const int xcd = pid % 8, idx = pid / 8;
+        lin = xcd * per + (xcd < rem ? xcd : rem) + idx;
+    }
+    constexpr int GROUP = 8;
+    const int width = GROUP * tilesN;
+    const int group = lin / width;
+    const int firstM = group * GROUP;
+    const int gsize = (tilesM - firstM) < GROUP ? (tilesM - firstM) : GROUP;
+    const int tileM = firstM + (lin % width) % gsize;
+    const int tileN = (lin % width) / gsize;
+    const int m0 = tileM * BM, n0 = tileN * BN;
+
+    // DMA source pointers: lane l of a wave-load covers row l / 4 of its 16 rows and
+    // fetches the logical chunk that belongs at slot l % 4 of that row.
+    const int lrow = lane >> 2;
+    const int lchunk = (lane & 3) ^ ((lane >> 4) & 3);
+    const int8_t *aRow[LA];
+    const int8_t *bRow[LB];
+#pragma unroll
+    for (int i = 0; i < LA; i++) {
+        int m = m0 + 16 * (wave + NW * i) + lrow;
+        m = m < p.M ? m : p.M - 1;
+        aRow[i] = p.A + (size_t)m * p.K;
+    }
+#pragma unroll
+    for (int i = 0; i < LB; i++) {
+        const int n = n0 + 16 * (wave + NW * i) + lrow;
+        bRow[i] = p.Bp + (size_t)n * p.Kp + lchunk * 16;
+    }
+    v16i acc[TN][TM];
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[j][i][r] = 0;
+        }
+    }
+
+    // Fragment addresses: row (l & 31) of a 32-row MFMA tile, logical chunk 2 * kk + (l >> 5).
+    const int fr = lane & 31;
+    const int swz = (fr >> 2) & 3;
+    const int off0 = (((lane >> 5)) ^ swz) * 16;  // kk = 0; kk = 1 is off0 ^ 32
+    const int aFrag = (wm * WTM + fr) * BK + off0;
+    const int bFrag = A_STAGE + (wn * WTN + fr) * BK + off0;
+
+    // One (bias, scale) pair per thread, fetched now and parked in LDS for the epilogue.
+    int32_t myBias = 0, myScale = 0;
+    if (tid < BN) {
+        myBias = p.bias[n0 + tid];  // arrays are padded to Np
+        myScale = p.scale[n0 + tid];
+    }
+
+    const int KT = p.Kp / BK;
+
+    // Software pipeline.  The ring holds tiles kt+1 .. kt+STAGES while tile kt is computed.
+    // Each k-tile is two MFMA phases (k halves of 32).  While phase 0 runs, the fragments
+    // of phase 1 are read from LDS; then the wave waits for tile kt+1, meets the block at the
+    // barrier, and while phase 1 runs it refills the stage it just finished with tile
+    // kt+STAGES and reads phase 0 of tile kt+1.  LDS latency and the DMA issue thus hide
+    // under MFMAs; sched_barrier pins the interleaving the source spells out.
+    auto issueTile = [&](int kt, int part, int parts) {
+        // issues this wave's DMA loads number [part * LPT / parts, (part + 1) * LPT / parts) of tile kt
+        const unsigned stage = ldsBase + (unsigned)(kt % STAGES) * STAGE;
+        int ka = kt * BK + lchunk * 16;
+        ka = ka < p.K ? ka : 0;  // beyond K the weights are zero: any valid bytes will do
+#pragma unroll
+        for (int x = 0; x < LPT; x++) {
+            if (x * parts / LPT != part) continue;
+            if (x < LA) {
+                dmaLoad16(aRow[x] + ka, stage + (unsigned)(wave + NW * x) * 1024u);
+            } else {
+                dmaLoad16(bRow[x - LA] + kt * BK, stage + A_STAGE + (unsigned)(wave + NW * (x - LA)) * 1024u);
+            }
+        }
+    };
+    // reads fragment number x (first the TM activation fragments, then the TN weight fragments)
+    auto readFrag = [&](const int8_t *st, int kk, int x, v4i(&af)[TM], v4i(&bf)[TN]) {
+        if (x < TM) {
+            af[x] = *(const v4i *)(st + ((aFrag + x * 32 * BK) ^ (kk * 32)));
+        } else {
+            bf[x - TM] = *(const v4i *)(st + ((bFrag + (x - TM) * 32 * BK) ^ (kk * 32)));
+        }
+    };
+    constexpr int NF = TM + TN;
+
+#pragma unroll
+    for (int t = 0; t < STAGES; t++) {
+        if (t < KT) issueTile(t, 0, 1);
+    }
+    // tile 0 landed?  (tiles 1 .. STAGES-1 may stay in flight)
+    if (KT >= STAGES) {
+        waitVmcnt<LPT *(STAGES - 1)>();
+    } else {
+        waitVmcnt<0>();
+    }
+    blockBarrier();
+    v4i af0[TM], bf0[TN], af1[TM], bf1[TN];
+#pragma unroll
+    for (int x = 0; x < NF; x++) readFrag(smem, 0, x, af0, bf0);
+
+    // One k-tile.  `steady` (a compile-time flag) is the branch-free body used while a full
+    // ring of later tiles exists; the last STAGES tiles go through the general body.
+    auto step = [&](int kt, auto steady) {
+        constexpr bool kSteady = decltype(steady)::value;
+        const int8_t *st = smem + (kt % STAGES) * STAGE;
+        const int8_t *stNext = smem + ((kt + 1) % STAGES) * STAGE;
+        // phase 0: MFMAs on (af0, bf0); the reads of (af1, bf1) go out behind the first weight row
+        // (so that the wait in front of that row only covers reads issued a phase ago) and
+        // complete under the remaining rows
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+#pragma unroll
+            for (int i = 0; i < TM; i++) acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf0[j], af0[i], acc[j][i], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (j == 0) {
+#pragma unroll
+                for (int x = 0; x < NF; x++) readFrag(st, 1, x, af1, bf1);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        // tile kt+1 must have landed; tiles kt+2 .. kt+STAGES-1 may stay in flight
+        const bool more = kSteady || kt + 1 < KT;
+        if (kSteady) {
+            waitVmcnt<LPT *(STAGES - 2)>();
+        } else if (more) {
+            const int inFlight = (KT - 2 - kt) < (STAGES - 2) ? (KT - 2 - kt) : (STAGES - 2);
+            if (inFlight >= 3) {
+                waitVmcnt<LPT * 3>();
+            } else if (inFlight == 2) {
+                waitVmcnt<LPT * 2>();
+            } else if (inFlight == 1) {
+                waitVmcnt<LPT>();
+            } else {
+                waitVmcnt<0>();
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");  // this wave's reads of tile kt are complete
+        blockBarrier();  // tile kt+1 is visible to everyone, and nobody reads stage kt % STAGES any more
+        const bool refill = kSteady || kt + STAGES < KT;
+        // phase 1: MFMAs on (af1, bf1), the reads of the next phase 0 behind the first weight row,
+        // the refill of the freed stage spread between the rows
+#pragma unroll
+        for (int j = 0; j < TN; j++) {
+            if (refill) issueTile(kt + STAGES, j, TN);
+#pragma unroll
+            for (int i = 0; i < TM; i++) acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf1[j], af1[i], acc[j][i], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (j == 0 && more) {
+#pragma unroll
+                for (int x = 0; x < NF; x++) readFrag(stNext, 0, x, af0, bf0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+    };
+    int kt = 0;
+    for (; kt + STAGES < KT; kt++) step(kt, std::true_type{});
+    for (; kt < KT; kt++) step(kt, std::false_type{});
+
+    // Epilogue.  Lane l owns row m = l & 31 of each MFMA tile and, per register group g,
+    // channels n = 8 g + 4 (l >> 5) + {0..3}.  The stage ring is free now and serves as staging
+    // so that results leave as 128-bit row-contiguous stores.
+    blockBarrier();
+    constexpr int PARAMS = STAGES * STAGE - 2 * BN * 4;  // bias[BN], scale[BN] at the top of the ring
+    int32_t *ldsBias = (int32_t *)(smem + PARAMS), *ldsScale = ldsBias + BN;
+    if (tid < BN) {
+        ldsBias[tid] = myBias;
+        ldsScale[tid] = myScale;
+    }
+    __syncthreads();
+    const long long rnd = roundTerm(p.rq.shift);
+    const int hi4 = (lane >> 5) * 4;
+    const bool wide = p.out_dtype == kDtypeI8 && (p.N & 15) == 0 && (((uintptr_t)p.out) & 15) == 0;
+    const bool wideShift = p.rq.shift >= 32;
+    const int shiftMinus32 = p.rq.shift - 32;
+    const long long lo64 = (long long)p.rq.out_min - p.rq.out_zp, hi64 = (long long)p.rq.out_max - p.rq.out_zp;
+    const int32_t lo32 = (int32_t)(lo64 < INT32_MIN ? INT32_MIN : lo64), hi32 = (int32_t)(hi64 > INT32_MAX ? INT32_MAX : hi64);
+    // One 32-channel column of MFMA tiles at a time goes through the wave's own LDS slice as int32;
+    // a compact loop then requantises 16 consecutive channels of one row per lane and stores them
+    // as one 128-bit word.  (Kept as a loop: unrolled over the whole tile it outgrows the
+    // instruction cache.)
+    constexpr int EROW = 32 * 4 + 16;  // bytes per staged row: 32 int32 + padding against bank conflicts
+    static_assert((size_t)NW * WTM * EROW <= (size_t)PARAMS, "epilogue staging must fit in the stage ring");
+    int8_t *stageOut = smem + wave * (WTM * EROW);
+    const int erow = lane >> 1, ecol = (lane & 1) * 16;  // read-back: 2 lanes per row, 16 channels each
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                v4i v = {acc[j][i][4 * g], acc[j][i][4 * g + 1], acc[j][i][4 * g + 2], acc[j][i][4 * g + 3]};
+                *(v4i *)(stageOut + (i * 32 + fr) * EROW + (8 * g + hi4) * 4) = v;
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");  // wave-private slice: no block barrier needed
+        const int nl = wn * WTN + j * 32 + ecol;  // first of this lane's 16 channels, relative to n0
+        const int nb = n0 + nl;
+        int32_t bias[16], scale[16];
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const v4i b4 = *(const v4i *)(ldsBias + nl + 4 * q);
+            const v4i s4 = *(const v4i *)(ldsScale + nl + 4 * q);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                bias[4 * q + e] = b4[e];
+                scale[4 * q + e] = s4[e];
+            }
+        }
+        // the shift >= 32 case (the usual one for TFLite-derived scales) has a cheaper tail; the
+        // choice is made once per column, outside the row loop
+        auto rows = [&](auto wideShiftTag) {
+            constexpr bool kWideShift = decltype(wideShiftTag)::value;
+            for (int r0 = 0; r0 < WTM; r0 += 32) {
+                const int row = r0 + erow;
+                const int m = m0 + wm * WTM + row;
+                int32_t q[16];
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    const v4i v = *(const v4i *)(stageOut + row * EROW + (ecol + 4 * c) * 4);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        q[4 * c + e] = kWideShift ? requantWideShift(v[e], bias[4 * c + e], scale[4 * c + e], rnd, shiftMinus32, lo32, hi32, p.rq.out_zp)
+                                                  : requant(v[e], bias[4 * c + e], scale[4 * c + e], rnd, p.rq);
+                    }
+                }
+                if (m < p.M) {
+                    if (wide && nb + 15 < p.N) {
+                        v4i w;
+#pragma unroll
+                        for (int c = 0; c < 4; c++) {
+                            w[c] = (int)((uint32_t)(q[4 * c] & 0xff) | ((uint32_t)(q[4 * c + 1] & 0xff) << 8) |
+                                         ((uint32_t)(q[4 * c + 2] & 0xff) << 16) | ((uint32_t)(q[4 * c + 3] & 0xff) << 24));
+                        }
+                        *(v4i *)((int8_t *)p.out + (size_t)m * p.N + nb) = w;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 16; e++) {
+                            if (nb + e < p.N) storeElem(p.out, (size_t)m * p.N + nb + e, q[e], p.out_dtype);
+                        }
+                    }
+                }
+            }
+        };
+        if (wideShift) {
+            rows(std::true_type{});
+        } else {
+            rows(std::false_type{});
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");  // reads done before the slice is overwritten
+    }
+}
+
 static const IgemmTile kTiles[kIgemmVariantCount] = {
     {128, 128, 64, "igemm_i8_128x128x64"},
     {256, 256, 64, "igemm_i8_256x256x64"},
     {64, 64, 64, "igemm_i8_64x64x64"},
     {256, 128, 64, "igemm_i8_256x128x64"},
+    {256, 256, 64, "igemm_dense_i8_256x256x64"},
+    {128, 128, 64, "igemm_dense_i8_128x128x64"},
+    {128, 256, 64, "igemm_dense_i8_128x256x64"},
+    {64, 64, 64, "igemm_dense_i8_64x64x64"},
 };
 
 const IgemmTile &igemmTile(uint32_t variant) {
@@ -317,6 +650,19 @@ static hipError_t launchIgemmLoader(const IgemmArgs &a, hipStream_t stream) {
     }
 }
 
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU>
+static hipError_t launchIgemmDense(const IgemmArgs &a, hipStream_t stream) {
+    constexpr size_t smem = (size_t)STAGES * (BM + BN) * 64;
+    static_assert(smem * BLOCKS_PER_CU <= 160 * 1024, "LDS of one CU");
+    auto kernel = igemm_dense_i8<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU>;
+    hipError_t err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (err != hipSuccess) return err;
+    const int tilesM = (a.M + BM - 1) / BM;
+    const int tilesN = a.Np / BN;
+    hipLaunchKernelGGL(kernel, dim3((unsigned)(tilesM * tilesN)), dim3(WAVES_M * WAVES_N * 64), smem, stream, a);
+    return hipGetLastError();
+}
+
 hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, hipStream_t stream) {
     if (variant >= kIgemmVariantCount) return hipErrorInvalidValue;
     const IgemmTile &t = kTiles[variant];
@@ -332,6 +678,7 @@ hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, hipStream_t stream)
         if (a.OH <= 0 || a.OW <= 0 || a.M % (a.OH * a.OW) != 0) return hipErrorInvalidValue;
         if (((uintptr_t)a.A & (a.gran - 1)) != 0) return hipErrorInvalidValue;
     }
+    if (variant >= kIgemmDense256x256 && a.loader != kLoaderDense) return hipErrorInvalidValue;
     if (((uintptr_t)a.Bp & 15) != 0) return hipErrorInvalidValue;
     if (a.out_dtype < kDtypeI8 || a.out_dtype > kDtypeI32) return hipErrorInvalidValue;
     switch (variant) {
@@ -339,6 +686,10 @@ hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, hipStream_t stream)
     case kIgemm256x256x64: return launchIgemmLoader<256, 256, 64>(a, stream);
     case kIgemm64x64x64: return launchIgemmLoader<64, 64, 64>(a, stream);
     case kIgemm256x128x64: return launchIgemmLoader<256, 128, 64>(a, stream);
+    case kIgemmDense256x256: return launchIgemmDense<256, 256, 2, 2, 4, 1>(a, stream);
+    case kIgemmDense128x128: return launchIgemmDense<128, 128, 2, 2, 4, 2>(a, stream);
+    case kIgemmDense128x256: return launchIgemmDense<128, 256, 2, 2, 3, 2>(a, stream);
+    case kIgemmDense64x64: return launchIgemmDense<64, 64, 2, 2, 4, 4>(a, stream);
     default: return hipErrorInvalidValue;
     }
 }
