@@ -76,6 +76,14 @@ def test_dense_igemm_every_tile_variant(device, variant, monkeypatch):
     check(device, w.conv2d_workload(N=2, H=28, W=28, C=192, O=32, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True))
 
 
+@pytest.mark.parametrize("shift", [0, 1, 6, 31, 32, 33, 34, 40, 62])
+def test_igemm_shift_boundaries(device, shift):
+    """Both epilogue tails of the MFMA kernels (generic 64-bit, and 32-bit for shift >= 33) around their switch."""
+    check(device, w.fully_connected_workload(200, 256, 144, shift=shift), kernel="igemm_dense")
+    check(device, w.fully_connected_workload(40, 72, 20, shift=shift, output_zp=-7), kernel="igemm_i8")
+    check(device, w.fully_connected_workload(3, 64, 40, shift=shift), kernel="fc_skinny")
+
+
 def test_conv2d_mbv2_layer_shapes(device):
     # first layer (3 channels, stride 2, TF SAME), expand / project 1x1, last 1x1
     check(device, w.conv2d_workload(N=2, H=224, W=224, C=3, O=32, stride=(2, 2), pad=(0, 1, 0, 1), realistic=True, input_zp=-1))

@@ -40,12 +40,14 @@ __device__ __forceinline__ int32_t requant(int32_t acc, int32_t bias, int32_t sc
     return (int32_t)(q + (uint32_t)rq.out_zp);
 }
 
-// Same result when shift >= 32: the shifted product fits 32 bits, so the tail is 32-bit work.
-__device__ __forceinline__ int32_t requantWideShift(int32_t acc, int32_t bias, int32_t scale, long long rnd,
+// Same result when shift >= 33, with 32-bit work only.  Write the product as H * 2^32 + L.  The
+// rounding term 2^(shift-1) is then a multiple of 2^32, so it adds r = 2^(shift-33) to H, and
+// floor((H + r + L / 2^32) / 2^(shift-32)) = (H + r) >> (shift - 32) because L / 2^32 < 1 cannot
+// carry an integer across a multiple of 2^(shift-32).  |H| <= 2^30 and r <= 2^29: no overflow.
+__device__ __forceinline__ int32_t requantWideShift(int32_t acc, int32_t bias, int32_t scale, int32_t rndHigh,
                                                     int shiftMinus32, int32_t lo, int32_t hi, int32_t zp) {
     const int32_t t0 = (int32_t)((uint32_t)acc + (uint32_t)bias);
-    const long long t2 = (long long)t0 * (long long)scale + rnd;
-    int32_t t3 = (int32_t)(t2 >> 32) >> shiftMinus32;
+    int32_t t3 = (__mulhi(t0, scale) + rndHigh) >> shiftMinus32;
     t3 = t3 < lo ? lo : t3;
     t3 = t3 > hi ? hi : t3;
     return (int32_t)((uint32_t)t3 + (uint32_t)zp);
@@ -318,6 +320,12 @@ __device__ __forceinline__ void dmaLoad16(const void *gptr, unsigned ldsAddr) {
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(ldsAddr), "v"(gptr) : "memory", "m0");
 }
 
+// Same with the address split into a wave-uniform 64-bit base (SGPR pair) and a 32-bit per-lane
+// offset: advancing along K is then scalar work only.
+__device__ __forceinline__ void dmaLoad16(const void *base, uint32_t laneOffset, unsigned ldsAddr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(ldsAddr), "v"(laneOffset), "s"(base) : "memory", "m0");
+}
+
 template <int N>
 __device__ __forceinline__ void waitVmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
@@ -368,18 +376,20 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
     // fetches the logical chunk that belongs at slot l % 4 of that row.
     const int lrow = lane >> 2;
     const int lchunk = (lane & 3) ^ ((lane >> 4) & 3);
-    const int8_t *aRow[LA];
-    const int8_t *bRow[LB];
+    // per-lane byte offsets from the tile origins (rows past M are clamped to the last row: their
+    // results are never stored, and every wave must issue the same number of loads)
+    const int8_t *aTile = p.A + (size_t)m0 * p.K;
+    const int8_t *bTile = p.Bp + (size_t)n0 * p.Kp;
+    uint32_t aOff[LA], bOff[LB];
 #pragma unroll
     for (int i = 0; i < LA; i++) {
-        int m = m0 + 16 * (wave + NW * i) + lrow;
-        m = m < p.M ? m : p.M - 1;
-        aRow[i] = p.A + (size_t)m * p.K;
+        int r = 16 * (wave + NW * i) + lrow;
+        r = m0 + r < p.M ? r : p.M - 1 - m0;
+        aOff[i] = (uint32_t)r * (uint32_t)p.K + (uint32_t)lchunk * 16u;
     }
 #pragma unroll
     for (int i = 0; i < LB; i++) {
-        const int n = n0 + 16 * (wave + NW * i) + lrow;
-        bRow[i] = p.Bp + (size_t)n * p.Kp + lchunk * 16;
+        bOff[i] = (uint32_t)(16 * (wave + NW * i) + lrow) * (uint32_t)p.Kp + (uint32_t)lchunk * 16u;
     }
     v16i acc[TN][TM];
 #pragma unroll
@@ -413,18 +423,23 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
     // barrier, and while phase 1 runs it refills the stage it just finished with tile
     // kt+STAGES and reads phase 0 of tile kt+1.  LDS latency and the DMA issue thus hide
     // under MFMAs; sched_barrier pins the interleaving the source spells out.
-    auto issueTile = [&](int kt, int part, int parts) {
-        // issues this wave's DMA loads number [part * LPT / parts, (part + 1) * LPT / parts) of tile kt
+    auto issueTile = [&](int kt, int part, int parts, auto wholeTag) {
+        // issues this wave's DMA loads number [part * LPT / parts, (part + 1) * LPT / parts) of tile kt;
+        // `whole` promises that the tile lies entirely below K
+        constexpr bool kWhole = decltype(wholeTag)::value;
         const unsigned stage = ldsBase + (unsigned)(kt % STAGES) * STAGE;
-        int ka = kt * BK + lchunk * 16;
-        ka = ka < p.K ? ka : 0;  // beyond K the weights are zero: any valid bytes will do
+        const int8_t *aBase = aTile + kt * BK;
+        const int8_t *bBase = bTile + kt * BK;
+        // beyond K the weights are zero, so any valid bytes will do: such lanes read chunk 0 of the
+        // same k-tile (always below K) by dropping their chunk offset; offsets stay non-negative
+        const uint32_t back = (!kWhole && kt * BK + lchunk * 16 >= p.K) ? (uint32_t)(lchunk * 16) : 0u;
 #pragma unroll
         for (int x = 0; x < LPT; x++) {
             if (x * parts / LPT != part) continue;
             if (x < LA) {
-                dmaLoad16(aRow[x] + ka, stage + (unsigned)(wave + NW * x) * 1024u);
+                dmaLoad16(aBase, aOff[x] - back, stage + (unsigned)(wave + NW * x) * 1024u);
             } else {
-                dmaLoad16(bRow[x - LA] + kt * BK, stage + A_STAGE + (unsigned)(wave + NW * (x - LA)) * 1024u);
+                dmaLoad16(bBase, bOff[x - LA], stage + A_STAGE + (unsigned)(wave + NW * (x - LA)) * 1024u);
             }
         }
     };
@@ -440,7 +455,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
 
 #pragma unroll
     for (int t = 0; t < STAGES; t++) {
-        if (t < KT) issueTile(t, 0, 1);
+        if (t < KT) issueTile(t, 0, 1, std::false_type{});
     }
     // tile 0 landed?  (tiles 1 .. STAGES-1 may stay in flight)
     if (KT >= STAGES) {
@@ -453,8 +468,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
 #pragma unroll
     for (int x = 0; x < NF; x++) readFrag(smem, 0, x, af0, bf0);
 
-    // One k-tile.  `steady` (a compile-time flag) is the branch-free body used while a full
-    // ring of later tiles exists; the last STAGES tiles go through the general body.
+    // One k-tile.  `steady` (a compile-time flag) is the branch-free body used while the tile it
+    // refills the ring with exists and lies wholly below K; the rest go through the general body.
     auto step = [&](int kt, auto steady) {
         constexpr bool kSteady = decltype(steady)::value;
         const int8_t *st = smem + (kt % STAGES) * STAGE;
@@ -496,7 +511,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
         // the refill of the freed stage spread between the rows
 #pragma unroll
         for (int j = 0; j < TN; j++) {
-            if (refill) issueTile(kt + STAGES, j, TN);
+            if (refill) issueTile(kt + STAGES, j, TN, steady);
 #pragma unroll
             for (int i = 0; i < TM; i++) acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf1[j], af1[i], acc[j][i], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
@@ -508,7 +523,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
         }
     };
     int kt = 0;
-    for (; kt + STAGES < KT; kt++) step(kt, std::true_type{});
+    for (; kt + STAGES < KT - 1; kt++) step(kt, std::true_type{});
     for (; kt < KT; kt++) step(kt, std::false_type{});
 
     // Epilogue.  Lane l owns row m = l & 31 of each MFMA tile and, per register group g,
@@ -525,8 +540,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
     const long long rnd = roundTerm(p.rq.shift);
     const int hi4 = (lane >> 5) * 4;
     const bool wide = p.out_dtype == kDtypeI8 && (p.N & 15) == 0 && (((uintptr_t)p.out) & 15) == 0;
-    const bool wideShift = p.rq.shift >= 32;
+    const bool wideShift = p.rq.shift >= 33;
     const int shiftMinus32 = p.rq.shift - 32;
+    const int32_t rndHigh = wideShift ? (int32_t)(1u << (p.rq.shift - 33)) : 0;
     const long long lo64 = (long long)p.rq.out_min - p.rq.out_zp, hi64 = (long long)p.rq.out_max - p.rq.out_zp;
     const int32_t lo32 = (int32_t)(lo64 < INT32_MIN ? INT32_MIN : lo64), hi32 = (int32_t)(hi64 > INT32_MAX ? INT32_MAX : hi64);
     // One 32-channel column of MFMA tiles at a time goes through the wave's own LDS slice as int32;
@@ -561,7 +577,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
                 scale[4 * q + e] = s4[e];
             }
         }
-        // the shift >= 32 case (the usual one for TFLite-derived scales) has a cheaper tail; the
+        // the shift >= 33 case (the usual one for TFLite-derived scales) has a cheaper tail; the
         // choice is made once per column, outside the row loop
         auto rows = [&](auto wideShiftTag) {
             constexpr bool kWideShift = decltype(wideShiftTag)::value;
@@ -574,7 +590,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
                     const v4i v = *(const v4i *)(stageOut + row * EROW + (ecol + 4 * c) * 4);
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        q[4 * c + e] = kWideShift ? requantWideShift(v[e], bias[4 * c + e], scale[4 * c + e], rnd, shiftMinus32, lo32, hi32, p.rq.out_zp)
+                        q[4 * c + e] = kWideShift ? requantWideShift(v[e], bias[4 * c + e], scale[4 * c + e], rndHigh, shiftMinus32, lo32, hi32, p.rq.out_zp)
                                                   : requant(v[e], bias[4 * c + e], scale[4 * c + e], rnd, p.rq);
                     }
                 }

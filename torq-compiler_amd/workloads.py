@@ -82,13 +82,20 @@ def conv2d_workload(N=1, H=112, W=112, C=32, O=64, KH=3, KW=3, stride=(1, 1), pa
 
 
 def fully_connected_workload(M, K, N, realistic=False, output_zp=5, output_min=-128, output_max=127,
-                             seed=1001):
-    """BASELINE config 1: int8 [M,K] x [N,K]^T with per-column requant."""
+                             seed=1001, shift=None):
+    """BASELINE config 1: int8 [M,K] x [N,K]^T with per-column requant.
+
+    `shift` forces one shift_factor for every column (multipliers drawn so that outputs still spread)."""
     rng = np.random.default_rng(seed)
     x = rng.integers(-128, 127, size=(M, K), endpoint=True, dtype=np.int8)
     w = rng.integers(-128, 127, size=(N, K), endpoint=True, dtype=np.int8)
     tosa_bias = rng.integers(-(1 << 15), 1 << 15, size=N, endpoint=True, dtype=np.int64)
-    mult, shift = random_requant(rng, N, realistic)
+    if shift is None:
+        mult, shift = random_requant(rng, N, realistic)
+    else:
+        top = min(max(int(shift) - 14, 1), 31)
+        mult = rng.integers(1 << (top - 1), (1 << top) - 1, size=N, endpoint=True, dtype=np.int64).astype(np.int32)
+        shift = np.full(N, int(shift), dtype=np.int8)
     sb, sf = derive_scale_bias(mult, shift, tosa_bias, w, 0)
     attrs = dict(output_zp=output_zp, output_min=output_min, output_max=output_max, shift_factor=sf)
     p = Program()
