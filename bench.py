@@ -50,6 +50,12 @@ def workload_table(pkg):
     }
 
 
+def network_table(pkg):
+    """Whole-network workloads (BASELINE config 3); selectable with --workload, reported as images/s."""
+    w = pkg.workloads
+    return {"mbv2_b%d" % b: (lambda b=b: w.mobilenet_v2_workload(batch=b), "mfma") for b in (1, 32, 256)}
+
+
 class Loaded:
     """A workload resident on the GPU: executable + device buffers."""
 
@@ -88,10 +94,14 @@ def roofline(wl, bound, ms):
 def verify_sample(loaded):
     """Checks the GPU result of the timed workload against the oracle (sampled rows for the big GEMMs)."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
-    from helpers import oracle_eval
+    from helpers import oracle_eval, oracle_network
     from oracle import oracle as orc
     wl = loaded.wl
     got = loaded.output()
+    if wl.name.startswith("mobilenet_v2"):
+        n = min(4, wl.inputs[0].shape[0])
+        import torq_compiler_amd as pkg
+        return bool(np.array_equal(got[:n], oracle_network(pkg.workloads.mobilenet_v2_workload(batch=n))))
     if wl.name.startswith("fully_connected") and wl.inputs[0].shape[0] > 64:
         a = dict(wl.attrs)
         wts, sb = a.pop("weights"), a.pop("scale_bias")
@@ -142,6 +152,10 @@ def main():
 
     pkg = import_package()
     table = workload_table(pkg)
+    nets = network_table(pkg)
+    if args.workload in nets:
+        table = dict(table)
+        table[args.workload] = nets[args.workload]
     if args.workload not in table:
         sys.exit("unknown workload %s; choose from %s" % (args.workload, ", ".join(table)))
     dev = pkg.Device(0)
@@ -174,6 +188,22 @@ def main():
                             "bound": bnd, "frac": r["frac"]}
             o.close()
 
+    mbv2 = {}
+    if not args.no_others:
+        sys.path.insert(0, os.path.join(ROOT, "tests"))
+        from helpers import oracle_network
+        for batch in (1, 32, 256):
+            o = Loaded(pkg, dev, pkg.workloads.mobilenet_v2_workload(batch=batch))
+            o.run(2)
+            ms = o.run(10 if batch > 1 else 30)
+            check = pkg.workloads.mobilenet_v2_workload(batch=min(batch, 4))  # same seed: same weights, first images
+            same = bool(np.array_equal(o.output()[:min(batch, 4)], oracle_network(check)))
+            mbv2["batch_%d" % batch] = {"ms": round(ms, 4), "images_per_s": round(batch / (ms * 1e-3), 1),
+                                       "GOP/s": round(o.wl.ops / (ms * 1e-3) / 1e9, 1), "kernels": len(o.exe.op_kernels()),
+                                       "parity_checked": same}
+            ok = ok and same
+            o.close()
+
     result = {
         "metric": "int8 GOP/s (fully_connected with fused requant), 1 MAC = 2 ops",
         "value": round(wl.ops / (wall_ms * 1e-3) / 1e9, 1),
@@ -195,6 +225,8 @@ def main():
         result["cpu_baseline"] = cpu_baseline(wl)
     if per_op:
         result["per_op"] = per_op
+    if mbv2:
+        result["mobilenet_v2_int8_224"] = mbv2
     dev.close()
     print(json.dumps(result))
     if not ok:

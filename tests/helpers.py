@@ -63,3 +63,30 @@ def assert_bit_exact(got, want, what=""):
         first = tuple(bad[0])
         raise AssertionError("%s: %d of %d elements differ; first at %s: got %d want %d"
                              % (what, len(bad), got.size, first, int(got[first]), int(want[first])))
+
+
+def oracle_network(wl, return_all=False):
+    """Replays a network workload (wl.attrs['layers']) layer by layer with the CPU oracle, N,H,W,C."""
+    layers = wl.attrs["layers"]
+    x = wl.inputs[0]
+    if not wl.attrs["nhwc"]:
+        x = np.ascontiguousarray(x.transpose(0, 2, 3, 1))
+    tensors = [x]
+    for L in layers:
+        src = [tensors[i] for i in L.inputs]
+        a = dict(L.attrs)
+        if L.op == "conv2d":
+            t = orc.conv2d(src[0], L.weights, L.scale_bias, layout=orc.NHWC, **a)
+        elif L.op == "depthwise_conv2d":
+            t = orc.depthwise_conv2d(src[0], L.weights, L.scale_bias, layout=orc.NHWC, **a)
+        elif L.op == "add":
+            t = orc.add(src[0], src[1], L.weights, L.scale_bias, **a)
+        elif L.op == "avg_pool2d":
+            a.pop("input_zp")
+            t = orc.avg_pool2d(src[0], L.scale_bias, **a)
+        elif L.op == "fully_connected":
+            t = orc.fully_connected(src[0].reshape(src[0].shape[0], -1), L.weights, L.scale_bias, **a)
+        else:
+            raise ValueError(L.op)
+        tensors.append(t)
+    return tensors if return_all else tensors[-1]

@@ -8,7 +8,7 @@ import sys
 import numpy as np
 import pytest
 
-from helpers import assert_bit_exact, oracle_eval, run_on_gpu
+from helpers import assert_bit_exact, oracle_eval, oracle_network, run_on_gpu
 from test_emitter import CONV, _chain_program
 from torq_compiler_amd import Executable, ThipError, runtime, workloads as w
 
@@ -191,6 +191,25 @@ def test_multi_op_program(device):
     exe.run_host([x, out2, np.zeros_like(aux)])
     exe.close()
     assert np.array_equal(out, out2)
+
+
+@pytest.mark.parametrize("batch", [1, 3])
+def test_mobilenet_v2_full(device, batch):
+    """BASELINE config 3: the whole 64-op network as one program, final logits bit-exact."""
+    wl = w.mobilenet_v2_workload(batch=batch)
+    announce(wl.name)
+    got, kernels = run_on_gpu(device, wl, via="device")
+    assert_bit_exact(got[0], oracle_network(wl), wl.name)
+    assert len(kernels) == 64 and "transpose_i8" not in kernels
+
+
+def test_mobilenet_v2_nchw_declared(device):
+    """Same network declared N,C,H,W as the reference emits it: only the input binding is transposed."""
+    wl = w.mobilenet_v2_workload(batch=2, resolution=96, classes=100, nhwc=False)
+    announce(wl.name, "nchw")
+    got, kernels = run_on_gpu(device, wl)
+    assert_bit_exact(got[0], oracle_network(wl), wl.name)
+    assert kernels.count("transpose_i8") == 1 and kernels[0] == "transpose_i8"
 
 
 def test_full_size_gemm_properties(device):

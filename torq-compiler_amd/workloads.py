@@ -198,3 +198,174 @@ def add_workload(N=1, H=56, W=56, C=24, zp0=-3, zp1=7, m0=0.71838506, m1=1.3 * 0
     attrs.update(weights=wts, scale_bias=sb)
     return Workload("add_%dx%dx%dx%d" % (N, H, W, C), p, [a, b], [(a.shape, np.int8)], 3 * a.size, 3 * a.nbytes,
                     attrs)
+
+
+# ---------------------------------------------------------------------------------------------
+# MobileNetV2-1.0 int8 (BASELINE config 3)
+# ---------------------------------------------------------------------------------------------
+MBV2_BLOCKS = [(1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 3, 2), (6, 64, 4, 2), (6, 96, 3, 1), (6, 160, 3, 2), (6, 320, 1, 1)]
+
+
+def quantize_multiplier(scale):
+    """TFLite-style (multiplier in [2^30, 2^31], shift) with multiplier / 2^shift == scale."""
+    m, e = np.frexp(np.asarray(scale, dtype=np.float64))
+    mult = np.round(m * (1 << 31)).astype(np.int64)
+    shift = 31 - e
+    bump = mult == (1 << 31)
+    mult = np.where(bump, mult // 2, mult)
+    shift = np.where(bump, shift - 1, shift)
+    return mult.astype(np.int32), shift.astype(np.int8)
+
+
+def _same_pad(size, k, s):
+    """TensorFlow SAME padding: (before, after)."""
+    out = -(-size // s)
+    total = max((out - 1) * s + k - size, 0)
+    return total // 2, total - total // 2
+
+
+class Layer:
+    """One TorqHL op of a network workload: enough for the builder and for a checker to replay it."""
+
+    def __init__(self, op, inputs, attrs, weights=None, scale_bias=None):
+        self.op = op              # "conv2d" | "depthwise_conv2d" | "add" | "avg_pool2d" | "fully_connected" | "transpose"
+        self.inputs = inputs      # indices into the tensor list (0 = network input)
+        self.attrs = attrs
+        self.weights = weights
+        self.scale_bias = scale_bias
+
+
+def mobilenet_v2_layers(resolution=224, classes=1000, seed=1006, width=1.0):
+    """The layer list of MobileNetV2 with random int8 weights, int32 biases and per-channel requant
+    parameters.  Scales are calibrated the way post-training quantisation does it: a float forward
+    pass of one random image gives each layer's accumulator spread, and the per-channel scale maps
+    it onto the int8 range, so no layer saturates or collapses."""
+    import torch
+
+    rng = np.random.default_rng(seed)
+    layers = []
+    shapes = [(resolution, resolution, 3)]  # H, W, C per tensor index
+    zps = [int(rng.integers(-10, 10))]
+    # calibration activations, N,C,H,W float64, already minus their zero point
+    calib = [torch.from_numpy(rng.integers(-128, 127, size=(1, 3, resolution, resolution), endpoint=True).astype(np.float64) - zps[0])]
+
+    def conv(src, O, k, s, relu6, depthwise=False):
+        H, W, C = shapes[src]
+        zp_in = zps[src]
+        if depthwise:
+            w = rng.integers(-127, 127, size=(C, 1, k, k), endpoint=True, dtype=np.int8)
+            O_ = C
+        else:
+            w = rng.integers(-127, 127, size=(O, C, k, k), endpoint=True, dtype=np.int8)
+            O_ = O
+        pt, pb = _same_pad(H, k, s)
+        pl, pr = _same_pad(W, k, s)
+        tosa_bias = rng.integers(-(1 << 12), 1 << 12, size=O_, endpoint=True, dtype=np.int64)
+        xp = torch.nn.functional.pad(calib[src], (pl, pr, pt, pb))  # x - zp is 0 in the padding
+        acc = torch.nn.functional.conv2d(xp, torch.from_numpy(w.astype(np.float64)), stride=s, groups=C if depthwise else 1)
+        acc = acc + torch.from_numpy(tosa_bias.astype(np.float64)).reshape(1, -1, 1, 1)
+        spread = acc.std(dim=(0, 2, 3)).numpy() + 1.0
+        # ReLU6 layers keep the positive half: give it most of the range; linear layers are centred
+        eff = (60.0 if relu6 else 40.0) / spread * rng.uniform(0.8, 1.25, size=O_)
+        mult, shift = quantize_multiplier(eff)
+        sb, sf = derive_scale_bias(mult, shift, tosa_bias, w, zp_in)
+        zp_out = int(rng.integers(-128, -110)) if relu6 else int(rng.integers(-20, 20))
+        lo, hi = (zp_out if relu6 else -128), 127
+        q = torch.clamp(torch.round(acc * torch.from_numpy(eff).reshape(1, -1, 1, 1)) + zp_out, lo, hi)
+        OH, OW = -(-H // s), -(-W // s)
+        attrs = dict(input_zp=zp_in, output_zp=zp_out, output_min=lo, output_max=hi,
+                     shift_factor=sf, pad=(pl, pr, pt, pb), stride=(s, s))
+        layers.append(Layer("depthwise_conv2d" if depthwise else "conv2d", [src], attrs, w, sb))
+        shapes.append((OH, OW, O_))
+        zps.append(zp_out)
+        calib.append(q - zp_out)
+        return len(shapes) - 1
+
+    def add(a, b):
+        zp_out = int(rng.integers(-20, 20))
+        m0, m1 = float(rng.uniform(0.5, 0.8)), float(rng.uniform(0.5, 0.8))
+        wts, sb, sf = add_params(m0, m1, zps[a], zps[b])
+        layers.append(Layer("add", [a, b], dict(output_zp=zp_out, output_min=-128, output_max=127, shift_factor=sf), wts, sb))
+        shapes.append(shapes[a])
+        zps.append(zp_out)
+        calib.append(torch.clamp(torch.round(calib[a] * m0 + calib[b] * m1) + zp_out, -128, 127) - zp_out)
+        return len(shapes) - 1
+
+    def ch(c):
+        return max(8, int(c * width + 4) // 8 * 8)
+
+    t = conv(0, ch(32), 3, 2, True)
+    cin = ch(32)
+    for expand, c, n, s in MBV2_BLOCKS:
+        for i in range(n):
+            stride = s if i == 0 else 1
+            src = t
+            h = conv(t, cin * expand, 1, 1, True) if expand != 1 else t
+            h = conv(h, None, 3, stride, True, depthwise=True)
+            h = conv(h, ch(c), 1, 1, False)
+            t = add(src, h) if (stride == 1 and cin == ch(c)) else h
+            cin = ch(c)
+    t = conv(t, 1280, 1, 1, True)
+    H, W, C = shapes[t]
+    zp_out = int(rng.integers(-128, -110))
+    sb = np.array([-(H * W * zps[t]), int((1 << 20) / (H * W))], dtype=np.int32)
+    layers.append(Layer("avg_pool2d", [t], dict(input_zp=zps[t], output_zp=zp_out, output_min=-128, output_max=127,
+                                                shift_factor=20), np.array([1], dtype=np.int8), sb))
+    shapes.append((1, 1, C))
+    zps.append(zp_out)
+    pooled = calib[t].mean(dim=(2, 3))  # 1, C
+    t = len(shapes) - 1
+    w = rng.integers(-127, 127, size=(classes, C), endpoint=True, dtype=np.int8)
+    tosa_bias = rng.integers(-(1 << 12), 1 << 12, size=classes, endpoint=True, dtype=np.int64)
+    logits = pooled @ torch.from_numpy(w.astype(np.float64)).T
+    eff = 40.0 / (float(logits.std()) + 1.0) * rng.uniform(0.8, 1.25, size=classes)
+    mult, shift = quantize_multiplier(eff)
+    sb, sf = derive_scale_bias(mult, shift, tosa_bias, w, zps[t])
+    layers.append(Layer("fully_connected", [t], dict(output_zp=int(rng.integers(-20, 20)), output_min=-128, output_max=127,
+                                                     shift_factor=sf), w, sb))
+    shapes.append((1, 1, classes))
+    return layers, shapes, zps[0]
+
+
+def mobilenet_v2_workload(batch=1, resolution=224, classes=1000, seed=1006, nhwc=True, width=1.0):
+    """BASELINE config 3 as ONE program: 52 convs, 17 depthwise, 10 adds, global average pool, FC.
+
+    nhwc=True declares every tensor N,H,W,C (the layout the kernels run); nhwc=False declares the ops
+    N,C,H,W as the reference's patterns emit them, with the torq_hl.transpose the reference places in
+    front of avg_pool2d."""
+    layers, shapes, _ = mobilenet_v2_layers(resolution, classes, seed, width)
+    rng = np.random.default_rng(seed + 1)
+    H, W, C = shapes[0]
+    x = rng.integers(-128, 127, size=(batch, H, W, C), endpoint=True, dtype=np.int8)
+    if not nhwc:
+        x = np.ascontiguousarray(x.transpose(0, 3, 1, 2))
+    p = Program()
+    vals = [p.binding(0, x.shape)]
+    out_binding = p.binding(1, (batch, classes))
+    macs = 0
+    for li, L in enumerate(layers):
+        src = [vals[i] for i in L.inputs]
+        last = li == len(layers) - 1
+        if L.op == "conv2d":
+            v = p.conv2d(src[0], L.weights, L.scale_bias, nhwc_input=nhwc, **L.attrs)
+            oh, ow, oc = shapes[li + 1]
+            macs += batch * oh * ow * oc * int(np.prod(L.weights.shape[1:]))
+        elif L.op == "depthwise_conv2d":
+            v = p.depthwise_conv2d(src[0], L.weights, L.scale_bias, nhwc_input=nhwc, **L.attrs)
+            oh, ow, oc = shapes[li + 1]
+            macs += batch * oh * ow * oc * int(np.prod(L.weights.shape[2:]))
+        elif L.op == "add":
+            v = p.add(src[0], src[1], L.weights, L.scale_bias, **L.attrs)
+        elif L.op == "avg_pool2d":
+            s0 = src[0] if nhwc else p.transpose(src[0], (0, 2, 3, 1))
+            v = p.avg_pool2d(s0, L.weights, L.scale_bias, **L.attrs)
+        elif L.op == "fully_connected":
+            v = p.fully_connected(src[0], L.weights, L.scale_bias, init=out_binding if last else None, **L.attrs)
+            macs += batch * int(np.prod(L.weights.shape))
+        else:
+            raise ValueError(L.op)
+        vals.append(v)
+    wbytes = sum(L.weights.nbytes + L.scale_bias.nbytes for L in layers)
+    wl = Workload("mobilenet_v2_b%d_%d" % (batch, resolution), p, [x], [((batch, classes), np.int8)], 2 * macs,
+                  wbytes + x.nbytes + batch * classes, dict(layers=layers, shapes=shapes, nhwc=nhwc))
+    return wl
