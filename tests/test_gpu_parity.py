@@ -63,7 +63,7 @@ def test_conv2d_every_tile_variant(device, variant, monkeypatch):
     check(device, w.fully_connected_workload(300, 192, 520, realistic=True))
 
 
-@pytest.mark.parametrize("variant", [4, 5, 6, 7])
+@pytest.mark.parametrize("variant", [4, 5, 6, 7, 8, 9, 10])
 def test_dense_igemm_every_tile_variant(device, variant, monkeypatch):
     """The LDS-DMA kernel: whole tiles, ragged M / N / K tails, K shorter than the stage ring."""
     monkeypatch.setenv("THIP_IGEMM_DENSE_VARIANT", str(variant))

@@ -337,7 +337,12 @@ class Emitter {
                 const long v = strtol(env, nullptr, 10);
                 if (v >= 0 && v < (long)kIgemmVariantCount) return (uint32_t)v;
             }
-            // the largest tile that still gives (nearly) every CU a tile
+            // N narrower than a tile: one tile column of the narrowest tile that covers N, so the
+            // activations are streamed once (these shapes are bandwidth-bound, padded MFMA work is free)
+            if (N <= 128 && M >= 4096) {
+                return N <= 32 ? kIgemmDense256x32 : N <= 64 ? kIgemmDense256x64 : kIgemmDense256x128;
+            }
+            // otherwise the largest tile that still gives (nearly) every CU a tile
             const uint32_t order[] = {kIgemmDense256x256, kIgemmDense128x256, kIgemmDense128x128};
             for (uint32_t v : order) {
                 if (tiles(v) >= 224) return v;

@@ -44,7 +44,10 @@ enum IgemmVariant : uint32_t {
     kIgemmDense128x128 = 5,
     kIgemmDense128x256 = 6,
     kIgemmDense64x64 = 7,
-    kIgemmVariantCount = 8,
+    kIgemmDense256x128 = 8,
+    kIgemmDense256x64 = 9,   // narrow-N tiles for the pointwise convolutions of mobile networks
+    kIgemmDense256x32 = 10,
+    kIgemmVariantCount = 11,
 };
 struct IgemmTile {
     int bm, bn, bk;

@@ -339,10 +339,13 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
     constexpr int NW = WAVES_M * WAVES_N;
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
     constexpr int TM = WTM / 32, TN = WTN / 32;
-    constexpr int LA = BM / 16 / NW, LB = BN / 16 / NW;  // DMA instructions per wave per k-tile
+    constexpr int BWL = BN / 16;                          // wave-loads (16 rows each) that make up the B tile
+    constexpr int LA = BM / 16 / NW, LB = (BWL + NW - 1) / NW;  // DMA instructions per wave per k-tile
     constexpr int LPT = LA + LB;
     constexpr int A_STAGE = BM * BK, B_STAGE = BN * BK, STAGE = A_STAGE + B_STAGE;
-    static_assert(BM % (16 * NW) == 0 && BN % (16 * NW) == 0, "every wave must issue the same number of loads");
+    // every wave must issue the same number of loads: a narrow B tile (fewer wave-loads than
+    // waves) is loaded redundantly, several waves writing the same bytes to the same place
+    static_assert(BM % (16 * NW) == 0 && BN % 16 == 0 && (BWL % NW == 0 || BWL < NW), "unbalanced DMA loads");
     static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the MFMA tile");
     static_assert(STAGES >= 2 && STAGES <= 5 && LPT * (STAGES - 1) < 64, "vmcnt is a 6-bit counter");
 
@@ -389,7 +392,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
     }
 #pragma unroll
     for (int i = 0; i < LB; i++) {
-        bOff[i] = (uint32_t)(16 * (wave + NW * i) + lrow) * (uint32_t)p.Kp + (uint32_t)lchunk * 16u;
+        bOff[i] = (uint32_t)(16 * ((wave + NW * i) % BWL) + lrow) * (uint32_t)p.Kp + (uint32_t)lchunk * 16u;
     }
     v16i acc[TN][TM];
 #pragma unroll
@@ -439,7 +442,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
             if (x < LA) {
                 dmaLoad16(aBase, aOff[x] - back, stage + (unsigned)(wave + NW * x) * 1024u);
             } else {
-                dmaLoad16(bBase, bOff[x - LA], stage + A_STAGE + (unsigned)(wave + NW * (x - LA)) * 1024u);
+                dmaLoad16(bBase, bOff[x - LA], stage + A_STAGE + (unsigned)((wave + NW * (x - LA)) % BWL) * 1024u);
             }
         }
     };
@@ -530,7 +533,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
     // channels n = 8 g + 4 (l >> 5) + {0..3}.  The stage ring is free now and serves as staging
     // so that results leave as 128-bit row-contiguous stores.
     blockBarrier();
-    constexpr int PARAMS = STAGES * STAGE - 2 * BN * 4;  // bias[BN], scale[BN] at the top of the ring
+    constexpr int EROW = 32 * 4 + 16;          // bytes per staged row: 32 int32 + padding against bank conflicts
+    constexpr int PARAMS = NW * WTM * EROW;    // bias[BN], scale[BN] behind the staging slices
     int32_t *ldsBias = (int32_t *)(smem + PARAMS), *ldsScale = ldsBias + BN;
     if (tid < BN) {
         ldsBias[tid] = myBias;
@@ -549,8 +553,6 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
     // a compact loop then requantises 16 consecutive channels of one row per lane and stores them
     // as one 128-bit word.  (Kept as a loop: unrolled over the whole tile it outgrows the
     // instruction cache.)
-    constexpr int EROW = 32 * 4 + 16;  // bytes per staged row: 32 int32 + padding against bank conflicts
-    static_assert((size_t)NW * WTM * EROW <= (size_t)PARAMS, "epilogue staging must fit in the stage ring");
     int8_t *stageOut = smem + wave * (WTM * EROW);
     const int erow = lane >> 1, ecol = (lane & 1) * 16;  // read-back: 2 lanes per row, 16 channels each
 #pragma unroll
@@ -630,6 +632,9 @@ static const IgemmTile kTiles[kIgemmVariantCount] = {
     {128, 128, 64, "igemm_dense_i8_128x128x64"},
     {128, 256, 64, "igemm_dense_i8_128x256x64"},
     {64, 64, 64, "igemm_dense_i8_64x64x64"},
+    {256, 128, 64, "igemm_dense_i8_256x128x64"},
+    {256, 64, 64, "igemm_dense_i8_256x64x64"},
+    {256, 32, 64, "igemm_dense_i8_256x32x64"},
 };
 
 const IgemmTile &igemmTile(uint32_t variant) {
@@ -668,7 +673,10 @@ static hipError_t launchIgemmLoader(const IgemmArgs &a, hipStream_t stream) {
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU>
 static hipError_t launchIgemmDense(const IgemmArgs &a, hipStream_t stream) {
-    constexpr size_t smem = (size_t)STAGES * (BM + BN) * 64;
+    // the stage ring, reused by the epilogue as staging slices (one per wave) plus bias/scale
+    constexpr size_t ring = (size_t)STAGES * (BM + BN) * 64;
+    constexpr size_t epilogue = (size_t)(BM / WAVES_M) * (WAVES_M * WAVES_N) * (32 * 4 + 16) + 2 * BN * 4;
+    constexpr size_t smem = ring > epilogue ? ring : epilogue;
     static_assert(smem * BLOCKS_PER_CU <= 160 * 1024, "LDS of one CU");
     auto kernel = igemm_dense_i8<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU>;
     hipError_t err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -706,6 +714,9 @@ hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, hipStream_t stream)
     case kIgemmDense128x128: return launchIgemmDense<128, 128, 2, 2, 4, 2>(a, stream);
     case kIgemmDense128x256: return launchIgemmDense<128, 256, 2, 2, 3, 2>(a, stream);
     case kIgemmDense64x64: return launchIgemmDense<64, 64, 2, 2, 4, 4>(a, stream);
+    case kIgemmDense256x128: return launchIgemmDense<256, 128, 2, 2, 3, 2>(a, stream);
+    case kIgemmDense256x64: return launchIgemmDense<256, 64, 4, 1, 3, 2>(a, stream);
+    case kIgemmDense256x32: return launchIgemmDense<256, 32, 4, 1, 3, 2>(a, stream);
     default: return hipErrorInvalidValue;
     }
 }
