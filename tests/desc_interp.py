@@ -113,7 +113,12 @@ def run(blob, binding_arrays):
             Nimg, H, W, C, OH, OW = (int(op[k]) for k in ["N", "H", "W", "C", "OH", "OW"])
             KH, KW = int(op["KH"]), int(op["KW"])
             x = view(op["in0"], Nimg * H * W * C).view(np.int8).reshape(Nimg, H, W, C)
-            wpk = view(op["weights"], KH * KW * C).view(np.int8).reshape(KH, KW, C)
+            if int(op["variant"]) == 1:  # [KH][C] dwords, byte kw = tap kw
+                wd = view(op["weights"], KH * C * 4).view(np.int8).reshape(KH, C, 4)
+                assert not wd[:, :, KW:].any()
+                wpk = np.ascontiguousarray(wd[:, :, :KW].transpose(0, 2, 1))
+            else:
+                wpk = view(op["weights"], KH * KW * C).view(np.int8).reshape(KH, KW, C)
             sb = np.empty(2 * C, dtype=np.int32)
             sb[0::2] = view(op["bias"], C * 4).view(np.int32)
             sb[1::2] = view(op["scale"], C * 4).view(np.int32)

@@ -140,7 +140,7 @@ def test_fully_connected_without_skinny_kernel(device, monkeypatch):
 # ---- bandwidth ops ---------------------------------------------------------------------------
 @pytest.mark.parametrize("batch", [1, 8])
 def test_depthwise_config2a(device, batch):
-    check(device, w.depthwise_workload(N=batch), via="device", kernel="depthwise_i8")
+    check(device, w.depthwise_workload(N=batch), via="device", kernel="depthwise3x3_dot4_i8")
 
 
 @pytest.mark.parametrize("kw", [

@@ -199,7 +199,8 @@ static thip_status_t checkOpFootprint(const thip_executable_t *e, uint32_t i) {
     case kKindDepthwise: {
         if (!positive({op.N, op.H, op.W, op.C, op.OH, op.OW, op.KH, op.KW})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad depthwise extents", i);
         if ((s = need(op.in0, (uint64_t)op.N * op.H * op.W * op.C, "in"))) return s;
-        if ((s = need(op.weights, (uint64_t)op.KH * op.KW * op.C, "weights"))) return s;
+        if (op.variant > kDepthwiseDot4Rows) return fail(THIP_INVALID_ARGUMENT, "op %u: unknown depthwise variant %u", i, op.variant);
+        if ((s = need(op.weights, op.variant == kDepthwiseDot4Rows ? (uint64_t)op.KH * op.C * 4 : (uint64_t)op.KH * op.KW * op.C, "weights"))) return s;
         if ((s = need(op.bias, (uint64_t)op.C * 4, "bias"))) return s;
         if ((s = need(op.scale, (uint64_t)op.C * 4, "scale"))) return s;
         return need(op.out, (uint64_t)op.N * op.OH * op.OW * op.C, "out");
@@ -229,7 +230,7 @@ static const char *opKernelName(const DescOp &op) {
     case kKindTranspose: return "transpose_i8";
     case kKindIgemm: return igemmTile(op.variant).name;
     case kKindFcSkinny: return "fc_skinny";
-    case kKindDepthwise: return "depthwise_i8";
+    case kKindDepthwise: return op.variant == kDepthwiseDot4Rows ? "depthwise3x3_dot4_i8" : "depthwise_i8";
     case kKindMaxPool: return "maxpool_i8";
     case kKindAvgPool: return "avgpool_i8";
     case kKindAdd: return "add_i8";
@@ -295,7 +296,7 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
         DepthwiseArgs a{(const int8_t *)resolve(e, op.in0, bp), (const int8_t *)resolve(e, op.weights, bp),
                         (const int32_t *)resolve(e, op.bias, bp), (const int32_t *)resolve(e, op.scale, bp),
                         (int8_t *)resolve(e, op.out, bp), op.N, op.H, op.W, op.C, op.OH, op.OW, op.KH, op.KW,
-                        op.SH, op.SW, op.PT, op.PL, op.input_zp, rq};
+                        op.SH, op.SW, op.PT, op.PL, op.input_zp, op.variant, rq};
         err = launchDepthwise(a, e->stream);
         break;
     }

@@ -530,7 +530,22 @@ thip_status_t Emitter::emitDepthwise(const thip_hl_depthwise_conv2d_t &c) {
     op.PL = (int32_t)c.pad[0]; op.PR = (int32_t)c.pad[1]; op.PT = (int32_t)c.pad[2]; op.PB = (int32_t)c.pad[3];
     op.in0 = in;
     op.out = out;
-    op.weights = newConst(wpk);
+    if (KH == 3 && KW == 3 && C % 16 == 0 && !getenv("THIP_DEPTHWISE_GENERIC")) {
+        // one dword per (window row, channel): byte kw = tap kw, byte 3 = 0, for v_dot4_i32_i8
+        std::vector<uint32_t> wdot((size_t)(KH * C));
+        for (int64_t ch = 0; ch < C; ch++) {
+            for (int64_t kh = 0; kh < KH; kh++) {
+                uint32_t v = 0;
+                for (int64_t kw = 0; kw < KW; kw++) v |= (uint32_t)(uint8_t)wd[(ch * KH + kh) * KW + kw] << (8 * kw);
+                wdot[(size_t)(kh * C + ch)] = v;
+            }
+        }
+        op.variant = kDepthwiseDot4Rows;
+        op.weights = newConst(wdot);
+    } else {
+        op.variant = kDepthwiseGeneric;
+        op.weights = newConst(wpk);
+    }
     ops_.push_back(op);
     finishOutput(post);
     return THIP_OK;

@@ -71,13 +71,18 @@ hipError_t launchFcSkinny(const FcSkinnyArgs &a, hipStream_t stream);
 
 struct DepthwiseArgs {
     const int8_t *in;     // NHWC
-    const int8_t *wpk;    // [KH][KW][C]
+    const int8_t *wpk;    // variant 0: [KH][KW][C] bytes; variant 1: [KH][C] dwords, byte kw of a dword = tap kw
     const int32_t *bias;  // [C]
     const int32_t *scale; // [C]
     int8_t *out;          // NHWC
     int32_t N, H, W, C, OH, OW, KH, KW, SH, SW, PT, PL;
     int32_t input_zp;
+    uint32_t variant;     // DepthwiseVariant
     Requant rq;
+};
+enum DepthwiseVariant : uint32_t {
+    kDepthwiseGeneric = 0,  // any window, any channel count
+    kDepthwiseDot4Rows = 1, // 3x3 window, C % 16 == 0: one v_dot4 per window row and channel
 };
 hipError_t launchDepthwise(const DepthwiseArgs &a, hipStream_t stream);
 

@@ -885,6 +885,105 @@ __global__ __launch_bounds__(256) void depthwise_i8(DepthwiseArgs p) {
     *(typename ByteVec<VEC>::type *)(p.out + (((size_t)n * p.OH + oy) * p.OW + ox) * p.C + c0) = o.v;
 }
 
+// 3x3 depthwise with the window row as the dot dimension.  A thread owns 16 channels of P
+// horizontally adjacent output pixels.  The three taps of a window row are brought together per
+// channel with two byte permutes ([x(kw0), x(kw1), x(kw2), 0] in one register) and multiplied by the
+// matching packed weights with one v_dot4_i32_i8: 3 dot4 + 6 permutes per channel instead of 9
+// multiply-adds on unpacked bytes.  P > 1 shares the input columns that neighbouring windows have
+// in common and loads weights, bias and scale once for P outputs, which is what matters here:
+// the kernel is bound by the traffic through the vector L1, not by arithmetic.
+// SWT is the horizontal stride when it is 1 or 2 (P > 1 needs it at compile time), 0 = run time.
+template <int P, int SWT>
+__global__ __launch_bounds__(256) void depthwise3x3_dot4_i8(DepthwiseArgs p) {
+    static_assert(P == 1 || SWT > 0, "several pixels per thread need a compile-time stride");
+    const int SW = SWT > 0 ? SWT : p.SW;
+    constexpr int NC = SWT > 0 ? (P - 1) * SWT + 3 : 3;  // input columns one window row of the thread spans
+    const int cg = p.C / 16;
+    const int oxGroups = (p.OW + P - 1) / P;
+    const long long total = (long long)p.N * p.OH * oxGroups * cg;
+    const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (t >= total) return;
+    const int c0 = (int)(t % cg) * 16;
+    long long pix = t / cg;
+    const int ox0 = (int)(pix % oxGroups) * P;
+    pix /= oxGroups;
+    const int oy = (int)(pix % p.OH);
+    const int n = (int)(pix / p.OH);
+    const int iy0 = oy * p.SH - p.PT, ix0 = ox0 * SW - p.PL;
+    const int8_t *img = p.in + (size_t)n * p.H * p.W * p.C + c0;
+    const uint32_t zp4 = (uint32_t)(p.input_zp & 0xff) * 0x01010101u;
+    const uint32_t *wrow = (const uint32_t *)p.wpk + c0;
+    int32_t acc[P][16];
+#pragma unroll
+    for (int q = 0; q < P; q++) {
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[q][v] = 0;
+    }
+#pragma unroll
+    for (int kh = 0; kh < 3; kh++) {
+        const int iy = iy0 + kh;
+        const bool rowIn = (unsigned)iy < (unsigned)p.H;
+        v4i d[NC];
+#pragma unroll
+        for (int j = 0; j < NC; j++) {
+            const int ix = ix0 + j;
+            if (rowIn && (unsigned)ix < (unsigned)p.W) {
+                d[j] = *(const v4i *)(img + ((size_t)iy * p.W + ix) * p.C);
+            } else {
+                d[j] = v4i{(int)zp4, (int)zp4, (int)zp4, (int)zp4};
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const v4i w4 = *(const v4i *)(wrow + (size_t)kh * p.C + 4 * g);
+#pragma unroll
+            for (int q = 0; q < P; q++) {
+                const int j0 = SWT > 0 ? q * SWT : 0;
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    // byte c of column j0, byte c of column j0+1, then byte c of column j0+2, then zero
+                    const uint32_t t01 = __builtin_amdgcn_perm((uint32_t)d[j0 + 1][g], (uint32_t)d[j0][g], 0x0c0c0000u | ((4u + c) << 8) | (uint32_t)c);
+                    const uint32_t x3 = __builtin_amdgcn_perm((uint32_t)d[j0 + 2][g], t01, 0x0c000100u | ((4u + c) << 16));
+                    acc[q][4 * g + c] = __builtin_amdgcn_sdot4((int)x3, w4[c], acc[q][4 * g + c], false);
+                }
+            }
+        }
+    }
+    const bool wideShift = p.rq.shift >= 33;
+    const long long rnd = roundTerm(p.rq.shift);
+    const int32_t rndHigh = wideShift ? (int32_t)(1u << (p.rq.shift - 33)) : 0;
+    const long long lo64 = (long long)p.rq.out_min - p.rq.out_zp, hi64 = (long long)p.rq.out_max - p.rq.out_zp;
+    const int32_t lo32 = (int32_t)(lo64 < INT32_MIN ? INT32_MIN : lo64), hi32 = (int32_t)(hi64 > INT32_MAX ? INT32_MAX : hi64);
+    v4i o[P];
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        const v4i b4 = *(const v4i *)(p.bias + c0 + 4 * g);
+        const v4i s4 = *(const v4i *)(p.scale + c0 + 4 * g);
+#pragma unroll
+        for (int q = 0; q < P; q++) {
+            uint32_t w = 0;
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const int32_t r = wideShift ? requantWideShift(acc[q][4 * g + c], b4[c], s4[c], rndHigh, p.rq.shift - 32, lo32, hi32, p.rq.out_zp)
+                                            : requant(acc[q][4 * g + c], b4[c], s4[c], rnd, p.rq);
+                w |= (uint32_t)(r & 0xff) << (8 * c);
+            }
+            o[q][g] = (int)w;
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < P; q++) {
+        if (ox0 + q < p.OW) *(v4i *)(p.out + (((size_t)n * p.OH + oy) * p.OW + ox0 + q) * p.C + c0) = o[q];
+    }
+}
+
+template <int P, int SWT>
+static hipError_t launchDepthwiseDot4(const DepthwiseArgs &a, hipStream_t stream) {
+    const long long total = (long long)a.N * a.OH * ((a.OW + P - 1) / P) * (a.C / 16);
+    hipLaunchKernelGGL((depthwise3x3_dot4_i8<P, SWT>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a);
+    return hipGetLastError();
+}
+
 static int pickVec(int C, const void *a, const void *b, const void *c) {
     const uintptr_t bits = (uintptr_t)a | (uintptr_t)b | (uintptr_t)c;
     if (C % 16 == 0 && (bits & 15) == 0) return 16;
@@ -918,6 +1017,18 @@ hipError_t launchDepthwise(const DepthwiseArgs &a, hipStream_t stream) {
     }
     if (!a.in || !a.wpk || !a.bias || !a.scale || !a.out) return hipErrorInvalidValue;
     if ((long long)a.N * a.OH * a.OW * a.C >= (1LL << 40)) return hipErrorInvalidValue;
+    if (a.variant == kDepthwiseDot4Rows) {
+        const uintptr_t bits = (uintptr_t)a.in | (uintptr_t)a.out | (uintptr_t)a.wpk | (uintptr_t)a.bias | (uintptr_t)a.scale;
+        if (a.KH != 3 || a.KW != 3 || a.C % 16 != 0 || (bits & 15) != 0) return hipErrorInvalidValue;
+        // several pixels per thread once there is enough work to still fill the chip
+        const long long outputs = (long long)a.N * a.OH * a.OW * (a.C / 16);
+        if (a.SW == 1 && outputs >= 4 * 65536) return launchDepthwiseDot4<4, 1>(a, stream);
+        if (a.SW == 2 && outputs >= 4 * 65536) return launchDepthwiseDot4<4, 2>(a, stream);
+        if (a.SW == 1 && outputs >= 2 * 65536) return launchDepthwiseDot4<2, 1>(a, stream);
+        if (a.SW == 2 && outputs >= 2 * 65536) return launchDepthwiseDot4<2, 2>(a, stream);
+        return launchDepthwiseDot4<1, 0>(a, stream);
+    }
+    if (a.variant != kDepthwiseGeneric) return hipErrorInvalidValue;
     switch (pickVec(a.C, a.in, a.out, a.wpk)) {
     case 16: return launchDepthwiseV<16>(a, stream);
     case 8: return launchDepthwiseV<8>(a, stream);
