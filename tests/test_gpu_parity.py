@@ -212,6 +212,38 @@ def test_mobilenet_v2_nchw_declared(device):
     assert kernels.count("transpose_i8") == 1 and kernels[0] == "transpose_i8"
 
 
+def test_graph_replay_matches_oracle_every_time(device):
+    """A multi-kernel program on device bindings is captured into a HIP graph on its second dispatch.
+    Every replay, with fresh inputs and synchronisations in between, must match the oracle."""
+    wl = w.mobilenet_v2_workload(batch=2, resolution=64, classes=40, width=0.5)
+    announce(wl.name, "graph replay")
+    exe = Executable(device, wl.program.serialize())
+    x = wl.inputs[0]
+    pin = device.upload(x)
+    pout = device.upload(np.zeros((2, 40), dtype=np.int8))
+    rng = np.random.default_rng(5)
+    for it in range(6):
+        if it:
+            x[...] = rng.integers(-128, 128, size=x.shape).astype(np.int8)
+            runtime.check(runtime.lib().thip_device_h2d(device.handle, pin, x.ctypes.data, x.nbytes))
+            device.synchronize()
+        if it % 2:
+            exe.enqueue_device([pin, pout], [x.nbytes, 80])
+            exe.wait()
+        else:
+            exe.run_device([pin, pout], [x.nbytes, 80])
+        got = device.download(pout, (2, 40), np.int8)
+        assert_bit_exact(got, oracle_network(wl), "dispatch %d" % it)
+    # other buffers: eager again, then a new capture
+    pin2 = device.upload(x)
+    for it in range(3):
+        exe.run_device([pin2, pout], [x.nbytes, 80])
+        assert_bit_exact(device.download(pout, (2, 40), np.int8), oracle_network(wl), "second buffer, dispatch %d" % it)
+    for ptr in (pin, pin2, pout):
+        device.free(ptr)
+    exe.close()
+
+
 def test_full_size_gemm_properties(device):
     """(4096,4096,4096) is too slow for the oracle in a test: check rows the oracle can afford plus a
     structural property (each output row depends on its own input row only)."""

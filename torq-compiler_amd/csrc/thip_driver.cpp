@@ -14,6 +14,7 @@
 // records, each launched on the executable's HIP stream.
 #include <hip/hip_runtime.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <chrono>
@@ -51,6 +52,13 @@ struct thip_executable_t {
     hipStream_t stream = nullptr;
     hipEvent_t evStart = nullptr, evStop = nullptr;
     std::mutex mutex;                    // one dispatch at a time
+    // Multi-kernel programs on device bindings are replayed as a HIP graph: the first dispatch on a
+    // set of binding pointers runs eagerly, the second is captured, later ones are one graph launch.
+    std::vector<uint8_t *> seenPtrs;     // binding pointers of the previous device dispatch
+    std::vector<uint8_t *> graphPtrs;    // binding pointers the instantiated graph was captured with
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t graphExec = nullptr;
+    bool graphsDisabled = false;
 };
 
 static thip_status_t hipFail(hipError_t e, const char *what) {
@@ -365,6 +373,54 @@ static thip_status_t enqueueOps(thip_executable_t *e, uint8_t *const *bp) {
     return THIP_OK;
 }
 
+constexpr uint32_t kGraphMinOps = 4;
+
+static void dropGraph(thip_executable_t *e) {
+    if (e->graphExec) (void)hipGraphExecDestroy(e->graphExec);
+    if (e->graph) (void)hipGraphDestroy(e->graph);
+    e->graphExec = nullptr;
+    e->graph = nullptr;
+    e->graphPtrs.clear();
+}
+
+// Enqueues one dispatch on device bindings, through the graph when there is one.
+static thip_status_t enqueueDevice(thip_executable_t *e, uint8_t *const *bp) {
+    const uint32_t nb = e->header.binding_count;
+    const bool eligible = !e->graphsDisabled && e->header.op_count >= kGraphMinOps && !e->device->eventLog;
+    if (!eligible) return enqueueOps(e, bp);
+    std::vector<uint8_t *> key(bp, bp + nb);
+    if (e->graphExec && key == e->graphPtrs) {
+        THIP_HIP(hipGraphLaunch(e->graphExec, e->stream), "hipGraphLaunch");
+        return THIP_OK;
+    }
+    if (key != e->seenPtrs) {  // first time with these pointers: run eagerly (this also configures the kernels)
+        e->seenPtrs = key;
+        return enqueueOps(e, bp);
+    }
+    dropGraph(e);
+    THIP_HIP(hipStreamBeginCapture(e->stream, hipStreamCaptureModeThreadLocal), "hipStreamBeginCapture");
+    const thip_status_t launched = enqueueOps(e, bp);
+    hipGraph_t g = nullptr;
+    const hipError_t ended = hipStreamEndCapture(e->stream, &g);
+    if (launched != THIP_OK || ended != hipSuccess || !g) {
+        if (g) (void)hipGraphDestroy(g);
+        e->graphsDisabled = true;  // fall back to eager launches for good
+        (void)hipGetLastError();
+        if (launched != THIP_OK) return launched;
+        return enqueueOps(e, bp);
+    }
+    e->graph = g;
+    if (hipGraphInstantiate(&e->graphExec, g, nullptr, nullptr, 0) != hipSuccess) {
+        dropGraph(e);
+        e->graphsDisabled = true;
+        (void)hipGetLastError();
+        return enqueueOps(e, bp);
+    }
+    e->graphPtrs = key;
+    THIP_HIP(hipGraphLaunch(e->graphExec, e->stream), "hipGraphLaunch");
+    return THIP_OK;
+}
+
 extern "C" {
 
 thip_status_t thip_device_create(int32_t ordinal, thip_device_t **out_device) {
@@ -464,6 +520,7 @@ thip_status_t thip_infer_format(const void *blob, size_t size, size_t format_cap
 void thip_executable_destroy(thip_executable_t *e) {
     if (!e) return;
     if (e->stream) (void)hipStreamSynchronize(e->stream);
+    dropGraph(e);
     for (uint8_t *p : e->tempPtrs) {
         if (p) (void)hipFree(p);
     }
@@ -522,6 +579,7 @@ thip_status_t thip_executable_create(thip_device_t *device, const void *blob, si
         if (err != hipSuccess) return bail(hipFail(err, "allocating an intermediate"));
     }
     e->staging.assign(h.binding_count, nullptr);
+    e->graphsDisabled = getenv("THIP_NO_GRAPH") != nullptr;
     *out_executable = e;
     return THIP_OK;
 }
@@ -545,7 +603,11 @@ static thip_status_t runLocked(thip_executable_t *e, const thip_dispatch_state_t
             THIP_HIP(hipMemcpyAsync(bp[i], st->binding_ptrs[i], e->bindings[i].size, hipMemcpyHostToDevice, e->stream), "staging a binding");
         }
     }
-    if (thip_status_t s = enqueueOps(e, bp)) {
+    bool allDevice = true;
+    for (uint32_t i = 0; i < e->header.binding_count; i++) {
+        if (e->bindings[i].flags != 0 && !(st->binding_flags && (st->binding_flags[i] & THIP_BINDING_DEVICE))) allDevice = false;
+    }
+    if (thip_status_t s = allDevice ? enqueueDevice(e, bp) : enqueueOps(e, bp)) {
         (void)hipStreamSynchronize(e->stream);
         return s;
     }
@@ -573,7 +635,7 @@ thip_status_t thip_executable_enqueue(thip_executable_t *e, const thip_dispatch_
     THIP_HIP(hipSetDevice(e->device->ordinal), "hipSetDevice");
     uint8_t *bp[64] = {nullptr};
     for (uint32_t i = 0; i < e->header.binding_count; i++) bp[i] = (uint8_t *)st->binding_ptrs[i];
-    return enqueueOps(e, bp);
+    return enqueueDevice(e, bp);
 }
 
 thip_status_t thip_executable_wait(thip_executable_t *e) {
@@ -592,7 +654,7 @@ thip_status_t thip_executable_time(thip_executable_t *e, const thip_dispatch_sta
     for (uint32_t i = 0; i < e->header.binding_count; i++) bp[i] = (uint8_t *)st->binding_ptrs[i];
     THIP_HIP(hipEventRecord(e->evStart, e->stream), "hipEventRecord");
     for (int32_t it = 0; it < iterations; it++) {
-        if (thip_status_t s = enqueueOps(e, bp)) {
+        if (thip_status_t s = enqueueDevice(e, bp)) {
             (void)hipStreamSynchronize(e->stream);
             return s;
         }

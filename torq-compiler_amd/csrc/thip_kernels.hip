@@ -646,9 +646,13 @@ static hipError_t launchIgemmTile(const IgemmArgs &a, hipStream_t stream) {
     constexpr int LDK = BK + 16;
     constexpr size_t smem = (size_t)2 * (BM + BN) * LDK;
     auto kernel = igemm_i8<BM, BN, BK, LOADER, G>;
-    hipError_t err = hipFuncSetAttribute((const void *)kernel,
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (err != hipSuccess) return err;
+    // once per kernel: later launches may sit inside a stream capture, where only stream work belongs
+    static bool configured = false;
+    if (!configured) {
+        hipError_t err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (err != hipSuccess) return err;
+        configured = true;
+    }
     const int tilesM = (a.M + BM - 1) / BM;
     const int tilesN = a.Np / BN;
     const dim3 grid((unsigned)(tilesM * tilesN));
@@ -679,8 +683,12 @@ static hipError_t launchIgemmDense(const IgemmArgs &a, hipStream_t stream) {
     constexpr size_t smem = ring > epilogue ? ring : epilogue;
     static_assert(smem * BLOCKS_PER_CU <= 160 * 1024, "LDS of one CU");
     auto kernel = igemm_dense_i8<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU>;
-    hipError_t err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (err != hipSuccess) return err;
+    static bool configured = false;
+    if (!configured) {
+        hipError_t err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+        if (err != hipSuccess) return err;
+        configured = true;
+    }
     const int tilesM = (a.M + BM - 1) / BM;
     const int tilesN = a.Np / BN;
     hipLaunchKernelGGL(kernel, dim3((unsigned)(tilesM * tilesN)), dim3(WAVES_M * WAVES_N * 64), smem, stream, a);
