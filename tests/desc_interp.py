@@ -83,6 +83,29 @@ def run(blob, binding_arrays):
             if kind == K_FC_SKINNY or int(op["loader"]) == 0:
                 A = np.zeros((M, Kp), dtype=np.int64)
                 A[:, :K] = view(op["in0"], M * K).view(np.int8).reshape(M, K)
+            elif int(op["loader"]) == 2:  # one 16-byte run per window row: [kw][ci] bytes, zero-weight padding
+                Nimg, H, W, C = (int(op[k]) for k in ["N", "H", "W", "C"])
+                OH, OW, SH, SW, PT, PL = (int(op[k]) for k in ["OH", "OW", "SH", "SW", "PT", "PL"])
+                x = view(op["in0"], Nimg * H * W * C).view(np.int8).reshape(Nimg, H, W, C)
+                tab = view(op["table"], Kp // 16 * 4).view(np.uint32)
+                A = np.zeros((Nimg, OH, OW, Kp), dtype=np.int64)
+                oy = np.arange(OH)[:, None] * SH - PT
+                ox = np.arange(OW)[None, :] * SW - PL
+                for e, ent in enumerate(tab):
+                    ent = int(ent)
+                    if ent & 0x80000000:
+                        continue
+                    kh, length = (ent >> 24) & 0x7f, ent & 0xffff
+                    assert length == int(op["KW"]) * C
+                    for b in range(length):
+                        kw, ci = b // C, b % C
+                        iy, ix = oy + kh, ox + kw
+                        inside = (iy >= 0) & (iy < H) & (ix >= 0) & (ix < W)
+                        vals = x[:, np.clip(iy, 0, H - 1), np.clip(ix, 0, W - 1), ci].astype(np.int64)
+                        A[..., e * 16 + b] = np.where(inside[None], vals, int(op["input_zp"]))
+                    # bytes beyond the run are whatever memory holds: they must meet zero weights
+                    A[..., e * 16 + length:(e + 1) * 16] = 77
+                A = A.reshape(M, Kp)
             else:
                 Nimg, H, W, C = (int(op[k]) for k in ["N", "H", "W", "C"])
                 OH, OW, SH, SW, PT, PL = (int(op[k]) for k in ["OH", "OW", "SH", "SW", "PT", "PL"])

@@ -75,6 +75,11 @@ enum Kind : uint32_t {
 enum IgemmLoader : uint32_t {
     kLoaderDense = 0,   // A is a dense [M, K] matrix with K % 16 == 0
     kLoaderGather = 1,  // implicit-GEMM gather through the k-table, `gran` bytes at a time
+    // few input channels (KW * C <= 16): K is laid out as one 16-byte group per window row,
+    // [kw][ci] bytes then zero-weight padding, so that a window row is ONE unaligned 16-byte load
+    // (what it reads past the KW * C bytes meets zero weights).  Table: one entry per group,
+    // kh in bits 24..30, run length KW * C in bits 0..15.
+    kLoaderRuns = 2,
 };
 
 struct DescOp {

@@ -180,6 +180,19 @@ static thip_status_t checkOpFootprint(const thip_executable_t *e, uint32_t i) {
         if ((s = need(op.weights, (uint64_t)op.Np * op.Kp, "weights"))) return s;
         if ((s = need(op.bias, (uint64_t)op.Np * 4, "bias"))) return s;
         if ((s = need(op.scale, (uint64_t)op.Np * 4, "scale"))) return s;
+        if (op.loader > kLoaderRuns) return fail(THIP_INVALID_ARGUMENT, "op %u: unknown igemm loader %u", i, op.loader);
+        if (op.loader == kLoaderRuns) {
+            if (op.KW * op.C > 16 || op.Kp % 16 != 0) return fail(THIP_INVALID_ARGUMENT, "op %u: window row of %d bytes does not fit a 16-byte run", i, op.KW * op.C);
+            if ((s = need(op.table, (uint64_t)op.Kp / 16 * 4, "table"))) return s;
+            if (op.table.space != kSpaceConst) return fail(THIP_INVALID_ARGUMENT, "op %u: table must be a constant", i);
+            const uint8_t *base = e->blob.data() + e->header.data_offset + e->consts[op.table.index].offset + op.table.offset;
+            for (uint32_t t = 0; t < (uint32_t)op.Kp / 16; t++) {
+                uint32_t ent;
+                memcpy(&ent, base + 4ull * t, 4);
+                if (ent & kKEntryInvalid) continue;
+                if ((int)((ent >> 24) & 0x7f) >= op.KH || (int)(ent & 0xffff) != op.KW * op.C) return fail(THIP_INVALID_ARGUMENT, "op %u: run table entry %u is outside the window", i, t);
+            }
+        }
         if (op.loader == kLoaderGather) {
             if (op.gran == 0 || (op.gran & (op.gran - 1)) || op.gran > 16) return fail(THIP_INVALID_ARGUMENT, "op %u: bad gather granularity", i);
             if ((s = need(op.table, (uint64_t)op.Kp / op.gran * 4, "table"))) return s;
@@ -287,6 +300,7 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
         a.SH = op.SH; a.SW = op.SW; a.PT = op.PT; a.PL = op.PL;
         a.input_zp = op.input_zp;
         a.out_dtype = op.out_dtype;
+        a.a_bytes = (int64_t)op.N * op.H * op.W * op.C;
         a.loader = op.loader;
         a.gran = op.gran;
         a.rq = rq;

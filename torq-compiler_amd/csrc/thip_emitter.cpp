@@ -361,7 +361,8 @@ class Emitter {
     // conv2d / fully_connected / matmul as one igemm record.  `wAt(n, k)` returns
     // weight (n, k) with k = (kh * KW + kw) * C + ci.
     template <typename WeightAt>
-    void emitIgemm(DescOp base, int64_t M, int64_t N, int64_t K, bool dense, WeightAt wAt) {
+    void emitIgemm(DescOp base, int64_t M, int64_t N, int64_t K, uint32_t loader, WeightAt wAt) {
+        const bool dense = loader == kLoaderDense;
         const uint32_t variant = chooseIgemmVariant(M, N, dense);
         const IgemmTile &t = igemmTile(variant);
         const int64_t Kp = roundUp(K, t.bk), Np = roundUp(N, t.bn);
@@ -371,6 +372,7 @@ class Emitter {
         }
         base.kind = kKindIgemm;
         base.variant = variant;
+        base.loader = loader;
         base.M = (int32_t)M;
         base.K = (int32_t)K;
         base.Kp = (int32_t)Kp;
@@ -378,10 +380,16 @@ class Emitter {
         base.Np = (int32_t)Np;
         base.weights = newConst(packed);
         if (dense) {
-            base.loader = kLoaderDense;
             base.gran = 16;
+        } else if (loader == kLoaderRuns) {
+            // K = KH groups of 16 bytes; entry: kh and the run length KW * C
+            base.gran = 16;
+            std::vector<uint32_t> tab((size_t)(Kp / 16));
+            for (int64_t e = 0; e < Kp / 16; e++) {
+                tab[(size_t)e] = e < base.KH ? (((uint32_t)e << 24) | (uint32_t)(base.KW * base.C)) : kKEntryInvalid;
+            }
+            base.table = newConst(tab);
         } else {
-            base.loader = kLoaderGather;
             int g = 16;
             while (base.C % g != 0) g /= 2;
             base.gran = (uint32_t)g;
@@ -474,11 +482,20 @@ thip_status_t Emitter::emitConv2d(const thip_hl_conv2d_t &c) {
     const bool pointwise = KH == 1 && KW == 1 && c.stride[0] == 1 && c.stride[1] == 1 && c.pad[0] == 0 &&
                            c.pad[1] == 0 && c.pad[2] == 0 && c.pad[3] == 0;
     const int64_t C = d.C;
-    emitIgemm(op, M, O, K, pointwise && K % 16 == 0, [&](int64_t n, int64_t k) {
-        const int64_t pos = k / C, ci = k % C;
-        const int64_t kh = pos / KW, kw = pos % KW;
-        return wd[((n * C + ci) * KH + kh) * KW + kw];
-    });
+    if (KW * C <= 16 && C % 16 != 0 && !getenv("THIP_NO_RUN_LOADER")) {
+        // few input channels (the first layer of an image network): one 16-byte run per window row
+        emitIgemm(op, M, O, KH * 16, kLoaderRuns, [&](int64_t n, int64_t k) -> int8_t {
+            const int64_t kh = k / 16, b = k % 16;
+            if (b >= KW * C) return 0;
+            return wd[((n * C + b % C) * KH + kh) * KW + b / C];
+        });
+    } else {
+        emitIgemm(op, M, O, K, (pointwise && K % 16 == 0) ? kLoaderDense : kLoaderGather, [&](int64_t n, int64_t k) {
+            const int64_t pos = k / C, ci = k % C;
+            const int64_t kh = pos / KW, kw = pos % KW;
+            return wd[((n * C + ci) * KH + kh) * KW + kw];
+        });
+    }
     finishOutput(post);
     return THIP_OK;
 }
@@ -600,7 +617,7 @@ thip_status_t Emitter::emitFullyConnected(const thip_hl_fully_connected_t &c) {
     op.N = (int32_t)M; op.H = 1; op.W = 1; op.C = (int32_t)K;
     op.OH = 1; op.OW = 1; op.OC = (int32_t)N;
     op.KH = 1; op.KW = 1; op.SH = 1; op.SW = 1;
-    emitIgemm(op, M, N, K, K % 16 == 0, [&](int64_t n, int64_t k) { return wd[n * K + k]; });
+    emitIgemm(op, M, N, K, K % 16 == 0 ? kLoaderDense : kLoaderGather, [&](int64_t n, int64_t k) { return wd[n * K + k]; });
     return THIP_OK;
 }
 
@@ -648,7 +665,7 @@ thip_status_t Emitter::emitMatmul(const thip_hl_matmul_t &c) {
             o.out.offset += (uint64_t)(r * M * N) * outElem;
             if (thip_status_t s = splitScaleBias(c.scale_bias, "torq_hl.matmul scale_bias", N, roundUp(N, 256), true, &o.bias, &o.scale)) return s;
             const int8_t *bb = bd + (Bb == 1 ? 0 : r * K * N);
-            emitIgemm(o, rows, N, K, K % 16 == 0, [&](int64_t n, int64_t k) { return bb[k * N + n]; });
+            emitIgemm(o, rows, N, K, K % 16 == 0 ? kLoaderDense : kLoaderGather, [&](int64_t n, int64_t k) { return bb[k * N + n]; });
         }
         return THIP_OK;
     }

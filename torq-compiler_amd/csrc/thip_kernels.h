@@ -28,6 +28,7 @@ struct IgemmArgs {
     int32_t H, W, C, OH, OW, SH, SW, PT, PL;
     int32_t input_zp;
     int32_t out_dtype;
+    int64_t a_bytes;        // size of A in bytes (the run loader keeps its 16-byte loads inside it)
     uint32_t loader;
     uint32_t gran;
     Requant rq;

@@ -120,6 +120,42 @@ __device__ __forceinline__ v4i gatherChunk(const int8_t *__restrict__ A,
     return u.v;
 }
 
+// One window row of a few-channel convolution: 16 bytes starting at pixel (iy, ix0), channel 0.
+struct __attribute__((packed)) UnalignedV4 {
+    v4i v;
+};
+__device__ __forceinline__ v4i gatherRun(const int8_t *__restrict__ A, uint32_t entry, int iy0, int ix0, size_t base,
+                                         int H, int W, int C, uint32_t zpb, long long aBytes) {
+    if (entry & kKEntryInvalid) return v4i{0, 0, 0, 0};
+    const int kh = (int)((entry >> 24) & 0x7f), len = (int)(entry & 0xffff);
+    const int iy = iy0 + kh;
+    const bool rowIn = (unsigned)iy < (unsigned)H;
+    const long long off = (long long)base + ((long long)iy * W + ix0) * C;
+    if (rowIn && ix0 >= 0 && ix0 * C + len <= W * C && off + 16 <= aBytes) {
+        return ((const UnalignedV4 *)(A + off))->v;
+    }
+    // window row touches the padding (or the last bytes of the tensor): byte by byte
+    union {
+        v4i v;
+        uint8_t b[16];
+    } u;
+    int kw = 0, ci = 0;
+#pragma unroll
+    for (int b = 0; b < 16; b++) {
+        uint8_t x = 0;
+        if (b < len) {
+            const int ix = ix0 + kw;
+            x = (rowIn && (unsigned)ix < (unsigned)W) ? (uint8_t)A[off + b] : (uint8_t)zpb;
+            if (++ci == C) {
+                ci = 0;
+                kw++;
+            }
+        }
+        u.b[b] = x;
+    }
+    return u.v;
+}
+
 template <int BM, int BN, int BK, int LOADER, int G>
 __global__ __launch_bounds__(256) void igemm_i8(IgemmArgs p) {
     constexpr int LDK = BK + 16;            // padded LDS row
@@ -198,6 +234,8 @@ __global__ __launch_bounds__(256) void igemm_i8(IgemmArgs p) {
                     v = *(const v4i *)(p.A + rBase[i] + k0);
                 }
                 ra[i] = v;
+            } else if (LOADER == kLoaderRuns) {
+                ra[i] = gatherRun(p.A, p.ktab[k0 / 16], rIy0[i], rIx0[i], rBase[i], p.H, p.W, p.C, zpb, p.a_bytes);
             } else {
                 ra[i] = gatherChunk<G>(p.A, p.ktab + k0 / G, rIy0[i], rIx0[i], rBase[i], p.H, p.W,
                                        p.C, zp4);
@@ -665,6 +703,9 @@ static hipError_t launchIgemmLoader(const IgemmArgs &a, hipStream_t stream) {
     if (a.loader == kLoaderDense) {
         return launchIgemmTile<BM, BN, BK, kLoaderDense, 16>(a, stream);
     }
+    if (a.loader == kLoaderRuns) {
+        return launchIgemmTile<BM, BN, BK, kLoaderRuns, 16>(a, stream);
+    }
     switch (a.gran) {
     case 16: return launchIgemmTile<BM, BN, BK, kLoaderGather, 16>(a, stream);
     case 8: return launchIgemmTile<BM, BN, BK, kLoaderGather, 8>(a, stream);
@@ -705,10 +746,16 @@ hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, hipStream_t stream)
     if (!a.A || !a.Bp || !a.bias || !a.scale || !a.out) return hipErrorInvalidValue;
     if (a.loader == kLoaderDense) {
         if (a.K % 16 != 0 || ((uintptr_t)a.A & 15) != 0) return hipErrorInvalidValue;
-    } else {
+    } else if (a.loader == kLoaderRuns) {
+        if (!a.ktab || a.C <= 0 || a.C > 16 || a.a_bytes < 16) return hipErrorInvalidValue;
+        if (a.OH <= 0 || a.OW <= 0 || a.M % (a.OH * a.OW) != 0) return hipErrorInvalidValue;
+        if (a.a_bytes != (long long)(a.M / (a.OH * a.OW)) * a.H * a.W * a.C) return hipErrorInvalidValue;
+    } else if (a.loader == kLoaderGather) {
         if (!a.ktab || a.C <= 0 || a.C % (int)a.gran != 0) return hipErrorInvalidValue;
         if (a.OH <= 0 || a.OW <= 0 || a.M % (a.OH * a.OW) != 0) return hipErrorInvalidValue;
         if (((uintptr_t)a.A & (a.gran - 1)) != 0) return hipErrorInvalidValue;
+    } else {
+        return hipErrorInvalidValue;
     }
     if (variant >= kIgemmDense256x256 && a.loader != kLoaderDense) return hipErrorInvalidValue;
     if (((uintptr_t)a.Bp & 15) != 0) return hipErrorInvalidValue;
