@@ -353,8 +353,8 @@ class Emitter {
             const long v = strtol(env, nullptr, 10);
             if (v >= 0 && v < (long)kIgemmDense256x256) return (uint32_t)v;
         }
-        // Enough 128x128 tiles to give every CU work; otherwise the small tile.
-        if (tiles(kIgemm128x128x64) >= 256) return kIgemm128x128x64;
+        // Enough 128x128 tiles to give every CU work (and N wide enough to use them); otherwise the small tile.
+        if (N > 64 && tiles(kIgemm128x128x64) >= 256) return kIgemm128x128x64;
         return kIgemm64x64x64;
     }
 

@@ -68,14 +68,127 @@ __device__ __forceinline__ void storeElem(void *out, size_t idx, int32_t v, int 
 }
 
 // ---------------------------------------------------------------------------
+// Epilogue shared by the MFMA kernels.  The accumulators come from MFMAs that took the weights as
+// the row operand: register r of lane l of tile (j, i) holds
+// C[m = 32 i + (l & 31)][n = 32 j + 8 (r / 4) + 4 (l >> 5) + (r & 3)], four consecutive output
+// channels per register group.  `smem` is the kernel's LDS, free by now, of at least
+// igemmEpilogueLds<...>() bytes; myBias / myScale are the (bias, scale) of channel n0 + threadIdx.x.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ void blockBarrier() { asm volatile("s_barrier" : : : "memory"); }
+
+template <int WTM, int NW, int BN>
+constexpr size_t igemmEpilogueLds() {
+    return (size_t)NW * WTM * (32 * 4 + 16) + 2 * (size_t)BN * 4;
+}
+
+template <int WTM, int WTN, int NW, int BN>
+__device__ __forceinline__ void igemmEpilogue(v16i (&acc)[WTN / 32][WTM / 32], int8_t *smem, const IgemmArgs &p, int m0,
+                                              int n0, int wm, int wn, int32_t myBias, int32_t myScale) {
+    // Epilogue.  Lane l owns row m = l & 31 of each MFMA tile and, per register group g,
+    // channels n = 8 g + 4 (l >> 5) + {0..3}.  The stage ring is free now and serves as staging
+    // so that results leave as 128-bit row-contiguous stores.
+    blockBarrier();
+    constexpr int EROW = 32 * 4 + 16;          // bytes per staged row: 32 int32 + padding against bank conflicts
+    constexpr int PARAMS = NW * WTM * EROW;    // bias[BN], scale[BN] behind the staging slices
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, fr = lane & 31;
+    int32_t *ldsBias = (int32_t *)(smem + PARAMS), *ldsScale = ldsBias + BN;
+    if (tid < BN) {
+        ldsBias[tid] = myBias;
+        ldsScale[tid] = myScale;
+    }
+    __syncthreads();
+    const long long rnd = roundTerm(p.rq.shift);
+    const int hi4 = (lane >> 5) * 4;
+    const bool wide = p.out_dtype == kDtypeI8 && (p.N & 15) == 0 && (((uintptr_t)p.out) & 15) == 0;
+    const bool wideShift = p.rq.shift >= 33;
+    const int shiftMinus32 = p.rq.shift - 32;
+    const int32_t rndHigh = wideShift ? (int32_t)(1u << (p.rq.shift - 33)) : 0;
+    const long long lo64 = (long long)p.rq.out_min - p.rq.out_zp, hi64 = (long long)p.rq.out_max - p.rq.out_zp;
+    const int32_t lo32 = (int32_t)(lo64 < INT32_MIN ? INT32_MIN : lo64), hi32 = (int32_t)(hi64 > INT32_MAX ? INT32_MAX : hi64);
+    // One 32-channel column of MFMA tiles at a time goes through the wave's own LDS slice as int32;
+    // a compact loop then requantises 16 consecutive channels of one row per lane and stores them
+    // as one 128-bit word.  (Kept as a loop: unrolled over the whole tile it outgrows the
+    // instruction cache.)
+    int8_t *stageOut = smem + wave * (WTM * EROW);
+    const int erow = lane >> 1, ecol = (lane & 1) * 16;  // read-back: 2 lanes per row, 16 channels each
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                v4i v = {acc[j][i][4 * g], acc[j][i][4 * g + 1], acc[j][i][4 * g + 2], acc[j][i][4 * g + 3]};
+                *(v4i *)(stageOut + (i * 32 + fr) * EROW + (8 * g + hi4) * 4) = v;
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");  // wave-private slice: no block barrier needed
+        const int nl = wn * WTN + j * 32 + ecol;  // first of this lane's 16 channels, relative to n0
+        const int nb = n0 + nl;
+        int32_t bias[16], scale[16];
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const v4i b4 = *(const v4i *)(ldsBias + nl + 4 * q);
+            const v4i s4 = *(const v4i *)(ldsScale + nl + 4 * q);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                bias[4 * q + e] = b4[e];
+                scale[4 * q + e] = s4[e];
+            }
+        }
+        // the shift >= 33 case (the usual one for TFLite-derived scales) has a cheaper tail; the
+        // choice is made once per column, outside the row loop
+        auto rows = [&](auto wideShiftTag) {
+            constexpr bool kWideShift = decltype(wideShiftTag)::value;
+            for (int r0 = 0; r0 < WTM; r0 += 32) {
+                const int row = r0 + erow;
+                const int m = m0 + wm * WTM + row;
+                int32_t q[16];
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    const v4i v = *(const v4i *)(stageOut + row * EROW + (ecol + 4 * c) * 4);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        q[4 * c + e] = kWideShift ? requantWideShift(v[e], bias[4 * c + e], scale[4 * c + e], rndHigh, shiftMinus32, lo32, hi32, p.rq.out_zp)
+                                                  : requant(v[e], bias[4 * c + e], scale[4 * c + e], rnd, p.rq);
+                    }
+                }
+                if (m < p.M) {
+                    if (wide && nb + 15 < p.N) {
+                        v4i w;
+#pragma unroll
+                        for (int c = 0; c < 4; c++) {
+                            w[c] = (int)((uint32_t)(q[4 * c] & 0xff) | ((uint32_t)(q[4 * c + 1] & 0xff) << 8) |
+                                         ((uint32_t)(q[4 * c + 2] & 0xff) << 16) | ((uint32_t)(q[4 * c + 3] & 0xff) << 24));
+                        }
+                        *(v4i *)((int8_t *)p.out + (size_t)m * p.N + nb) = w;
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 16; e++) {
+                            if (nb + e < p.N) storeElem(p.out, (size_t)m * p.N + nb + e, q[e], p.out_dtype);
+                        }
+                    }
+                }
+            }
+        };
+        if (wideShift) {
+            rows(std::true_type{});
+        } else {
+            rows(std::false_type{});
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");  // reads done before the slice is overwritten
+    }
+}
+
+// ---------------------------------------------------------------------------
 // igemm_i8
 // ---------------------------------------------------------------------------
 //
 // C[m][n] = sum_k A[m][k] * B[n][k]; block tile BM x BN x BK, 256 threads =
 // 4 waves in a 2 x 2 arrangement, each wave owns (BM/2) x (BN/2) as a grid of
 // 32 x 32 MFMA tiles.  One MFMA consumes 32 rows x 32 k of each operand: lane l
-// supplies row (l & 31), 16 consecutive k bytes starting at 16 * (l >> 5).  The
-// accumulator register r of lane l holds C[8 * (r / 4) + 4 * (l >> 5) + (r & 3)][l & 31].
+// supplies row (l & 31), 16 consecutive k bytes starting at 16 * (l >> 5).  The weights are
+// the MFMA's row operand; the accumulator layout is described at igemmEpilogue.
 //
 // LDS rows are padded by 16 bytes so that the 16 lanes of one ds_read_b128
 // phase fall into distinct banks.
@@ -258,14 +371,20 @@ __global__ __launch_bounds__(256) void igemm_i8(IgemmArgs p) {
         }
     };
 
-    v16i acc[TM][TN];
+    v16i acc[TN][TM];
 #pragma unroll
-    for (int i = 0; i < TM; i++) {
+    for (int j = 0; j < TN; j++) {
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
+        for (int i = 0; i < TM; i++) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[i][j][r] = 0;
+            for (int r = 0; r < 16; r++) acc[j][i][r] = 0;
         }
+    }
+    // One (bias, scale) pair per thread, fetched now and parked in LDS by the epilogue.
+    int32_t myBias = 0, myScale = 0;
+    if (tid < BN) {
+        myBias = p.bias[n0 + tid];  // arrays are padded to Np
+        myScale = p.scale[n0 + tid];
     }
 
     const int KT = p.Kp / BK;
@@ -294,10 +413,11 @@ __global__ __launch_bounds__(256) void igemm_i8(IgemmArgs p) {
                 bf[j] = *(const v4i *)(Bs + (cur * BN + bRow + j * 32) * LDK + kk * 32 + kOff);
             }
 #pragma unroll
-            for (int i = 0; i < TM; i++) {
+            for (int j = 0; j < TN; j++) {
 #pragma unroll
-                for (int j = 0; j < TN; j++) {
-                    acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[i], bf[j], acc[i][j], 0, 0, 0);
+                for (int i = 0; i < TM; i++) {
+                    // weights as the row operand: a lane then holds 4 consecutive output channels
+                    acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[j][i], 0, 0, 0);
                 }
             }
         }
@@ -307,31 +427,8 @@ __global__ __launch_bounds__(256) void igemm_i8(IgemmArgs p) {
         __syncthreads();
     }
 
-    // Epilogue: requant in the accumulator layout.  Each lane owns one output
-    // column per MFMA tile (so one bias/scale pair) and 16 rows.
-    const long long rnd = roundTerm(p.rq.shift);
-    const int rowBase = m0 + wm * WTM + (lane >> 5) * 4;
-#pragma unroll
-    for (int j = 0; j < TN; j++) {
-        const int n = n0 + wn * WTN + j * 32 + (lane & 31);
-        const int32_t bias = p.bias[n];    // arrays are padded to Np
-        const int32_t scale = p.scale[n];
-        if (n < p.N) {
-#pragma unroll
-            for (int i = 0; i < TM; i++) {
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int m = rowBase + i * 32 + 8 * (r / 4) + (r & 3);
-                    if (m < p.M) {
-                        const int32_t q = requant(acc[i][j][r], bias, scale, rnd, p.rq);
-                        storeElem(p.out, (size_t)m * p.N + n, q, p.out_dtype);
-                    }
-                }
-            }
-        }
-    }
+    igemmEpilogue<WTM, WTN, 4, BN>(acc, smem, p, m0, n0, wm, wn, myBias, myScale);
 }
-
 
 // ---------------------------------------------------------------------------
 // igemm_dense_i8: the dense [M, K] x [N, K]^T case (fully_connected, matmul,
@@ -368,8 +465,6 @@ template <int N>
 __device__ __forceinline__ void waitVmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
-
-__device__ __forceinline__ void blockBarrier() { asm volatile("s_barrier" : : : "memory"); }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_dense_i8(IgemmArgs p) {
@@ -567,98 +662,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
     for (; kt + STAGES < KT - 1; kt++) step(kt, std::true_type{});
     for (; kt < KT; kt++) step(kt, std::false_type{});
 
-    // Epilogue.  Lane l owns row m = l & 31 of each MFMA tile and, per register group g,
-    // channels n = 8 g + 4 (l >> 5) + {0..3}.  The stage ring is free now and serves as staging
-    // so that results leave as 128-bit row-contiguous stores.
-    blockBarrier();
-    constexpr int EROW = 32 * 4 + 16;          // bytes per staged row: 32 int32 + padding against bank conflicts
-    constexpr int PARAMS = NW * WTM * EROW;    // bias[BN], scale[BN] behind the staging slices
-    int32_t *ldsBias = (int32_t *)(smem + PARAMS), *ldsScale = ldsBias + BN;
-    if (tid < BN) {
-        ldsBias[tid] = myBias;
-        ldsScale[tid] = myScale;
-    }
-    __syncthreads();
-    const long long rnd = roundTerm(p.rq.shift);
-    const int hi4 = (lane >> 5) * 4;
-    const bool wide = p.out_dtype == kDtypeI8 && (p.N & 15) == 0 && (((uintptr_t)p.out) & 15) == 0;
-    const bool wideShift = p.rq.shift >= 33;
-    const int shiftMinus32 = p.rq.shift - 32;
-    const int32_t rndHigh = wideShift ? (int32_t)(1u << (p.rq.shift - 33)) : 0;
-    const long long lo64 = (long long)p.rq.out_min - p.rq.out_zp, hi64 = (long long)p.rq.out_max - p.rq.out_zp;
-    const int32_t lo32 = (int32_t)(lo64 < INT32_MIN ? INT32_MIN : lo64), hi32 = (int32_t)(hi64 > INT32_MAX ? INT32_MAX : hi64);
-    // One 32-channel column of MFMA tiles at a time goes through the wave's own LDS slice as int32;
-    // a compact loop then requantises 16 consecutive channels of one row per lane and stores them
-    // as one 128-bit word.  (Kept as a loop: unrolled over the whole tile it outgrows the
-    // instruction cache.)
-    int8_t *stageOut = smem + wave * (WTM * EROW);
-    const int erow = lane >> 1, ecol = (lane & 1) * 16;  // read-back: 2 lanes per row, 16 channels each
-#pragma unroll
-    for (int j = 0; j < TN; j++) {
-#pragma unroll
-        for (int i = 0; i < TM; i++) {
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                v4i v = {acc[j][i][4 * g], acc[j][i][4 * g + 1], acc[j][i][4 * g + 2], acc[j][i][4 * g + 3]};
-                *(v4i *)(stageOut + (i * 32 + fr) * EROW + (8 * g + hi4) * 4) = v;
-            }
-        }
-        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");  // wave-private slice: no block barrier needed
-        const int nl = wn * WTN + j * 32 + ecol;  // first of this lane's 16 channels, relative to n0
-        const int nb = n0 + nl;
-        int32_t bias[16], scale[16];
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const v4i b4 = *(const v4i *)(ldsBias + nl + 4 * q);
-            const v4i s4 = *(const v4i *)(ldsScale + nl + 4 * q);
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                bias[4 * q + e] = b4[e];
-                scale[4 * q + e] = s4[e];
-            }
-        }
-        // the shift >= 33 case (the usual one for TFLite-derived scales) has a cheaper tail; the
-        // choice is made once per column, outside the row loop
-        auto rows = [&](auto wideShiftTag) {
-            constexpr bool kWideShift = decltype(wideShiftTag)::value;
-            for (int r0 = 0; r0 < WTM; r0 += 32) {
-                const int row = r0 + erow;
-                const int m = m0 + wm * WTM + row;
-                int32_t q[16];
-#pragma unroll
-                for (int c = 0; c < 4; c++) {
-                    const v4i v = *(const v4i *)(stageOut + row * EROW + (ecol + 4 * c) * 4);
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        q[4 * c + e] = kWideShift ? requantWideShift(v[e], bias[4 * c + e], scale[4 * c + e], rndHigh, shiftMinus32, lo32, hi32, p.rq.out_zp)
-                                                  : requant(v[e], bias[4 * c + e], scale[4 * c + e], rnd, p.rq);
-                    }
-                }
-                if (m < p.M) {
-                    if (wide && nb + 15 < p.N) {
-                        v4i w;
-#pragma unroll
-                        for (int c = 0; c < 4; c++) {
-                            w[c] = (int)((uint32_t)(q[4 * c] & 0xff) | ((uint32_t)(q[4 * c + 1] & 0xff) << 8) |
-                                         ((uint32_t)(q[4 * c + 2] & 0xff) << 16) | ((uint32_t)(q[4 * c + 3] & 0xff) << 24));
-                        }
-                        *(v4i *)((int8_t *)p.out + (size_t)m * p.N + nb) = w;
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 16; e++) {
-                            if (nb + e < p.N) storeElem(p.out, (size_t)m * p.N + nb + e, q[e], p.out_dtype);
-                        }
-                    }
-                }
-            }
-        };
-        if (wideShift) {
-            rows(std::true_type{});
-        } else {
-            rows(std::false_type{});
-        }
-        asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");  // reads done before the slice is overwritten
-    }
+    igemmEpilogue<WTM, WTN, NW, BN>(acc, smem, p, m0, n0, wm, wn, myBias, myScale);
 }
 
 static const IgemmTile kTiles[kIgemmVariantCount] = {
@@ -682,7 +686,9 @@ const IgemmTile &igemmTile(uint32_t variant) {
 template <int BM, int BN, int BK, int LOADER, int G>
 static hipError_t launchIgemmTile(const IgemmArgs &a, hipStream_t stream) {
     constexpr int LDK = BK + 16;
-    constexpr size_t smem = (size_t)2 * (BM + BN) * LDK;
+    constexpr size_t tiles = (size_t)2 * (BM + BN) * LDK;
+    constexpr size_t epilogue = igemmEpilogueLds<BM / 2, 4, BN>();
+    constexpr size_t smem = tiles > epilogue ? tiles : epilogue;
     auto kernel = igemm_i8<BM, BN, BK, LOADER, G>;
     // once per kernel: later launches may sit inside a stream capture, where only stream work belongs
     static bool configured = false;
