@@ -195,3 +195,85 @@ def test_descriptor_header_and_format():
     with pytest.raises(ThipError) as e:
         runtime.infer_format(blob[:-1])
     assert e.value.code == runtime.INVALID_ARGUMENT
+
+
+def _padded_chain(nhwc):
+    """conv 1x1 (16->24) -> depthwise 3x3 -> maxpool 2x2 -> conv 3x3 (24->24) -> add -> conv 1x1 (24->40):
+    every intermediate has 24 channels, which the emitter stores as 32."""
+    rng = np.random.default_rng(5)
+    N, C, H, W, B = 2, 16, 12, 12, 24
+    x = rng.integers(-128, 128, size=(N, H, W, C) if nhwc else (N, C, H, W)).astype(np.int8)
+    lay = orc.NHWC if nhwc else orc.NCHW
+    rq = dict(output_min=-128, output_max=127)
+
+    def params(O, wshape, zp):
+        wt = rng.integers(-127, 128, size=wshape).astype(np.int8)
+        mult, shift = w.random_requant(rng, O, True)
+        sb, sf = w.derive_scale_bias(mult, (shift - 3).astype(np.int8), rng.integers(-2000, 2000, size=O), wt, zp)
+        return wt, sb, sf
+
+    w1, sb1, sf1 = params(B, (B, C, 1, 1), -3)
+    wd, sbd, sfd = params(B, (B, 1, 3, 3), 2)
+    w3, sb3, sf3 = params(B, (B, B, 3, 3), 5)
+    aw, asb, asf = w.add_params(0.7, 0.8, 5, -6)
+    w5, sb5, sf5 = params(40, (40, B, 1, 1), 1)
+    p = Program()
+    xin = p.binding(0, x.shape)
+    kw = dict(nhwc_input=nhwc)
+    t1 = p.conv2d(xin, w1, sb1, input_zp=-3, output_zp=2, shift_factor=sf1, pad=(0, 0, 0, 0), stride=(1, 1), **rq, **kw)
+    t2 = p.depthwise_conv2d(t1, wd, sbd, input_zp=2, output_zp=5, shift_factor=sfd, pad=(1, 1, 1, 1), stride=(1, 1), **rq, **kw)
+    t3 = p.maxpool2d(t2, input_zp=5, stride=(2, 2), pad=(0, 0, 0, 0), kernel=(2, 2), **rq, **kw)
+    t4 = p.conv2d(t3, w3, sb3, input_zp=5, output_zp=-6, shift_factor=sf3, pad=(1, 1, 1, 1), stride=(1, 1), **rq, **kw)
+    t5 = p.add(t3, t4, aw, asb, output_zp=1, shift_factor=asf, **rq)
+    oshape = (N, H // 2, W // 2, 40) if nhwc else (N, 40, H // 2, W // 2)
+    p.conv2d(t5, w5, sb5, init=p.binding(1, oshape), input_zp=1, output_zp=0, shift_factor=sf5, pad=(0, 0, 0, 0), stride=(1, 1), **rq, **kw)
+
+    o1 = orc.conv2d(x, w1, sb1, input_zp=-3, output_zp=2, shift_factor=sf1, pad=(0, 0, 0, 0), stride=(1, 1), layout=lay, **rq)
+    o2 = orc.depthwise_conv2d(o1, wd, sbd, input_zp=2, output_zp=5, shift_factor=sfd, pad=(1, 1, 1, 1), stride=(1, 1), layout=lay, **rq)
+    o3 = orc.maxpool2d(o2, input_zp=5, stride=(2, 2), pad=(0, 0, 0, 0), kernel=(2, 2), layout=lay, **rq)
+    o4 = orc.conv2d(o3, w3, sb3, input_zp=5, output_zp=-6, shift_factor=sf3, pad=(1, 1, 1, 1), stride=(1, 1), layout=lay, **rq)
+    o5 = orc.add(o3, o4, aw, asb, output_zp=1, shift_factor=asf, **rq)
+    o6 = orc.conv2d(o5, w5, sb5, input_zp=1, output_zp=0, shift_factor=sf5, pad=(0, 0, 0, 0), stride=(1, 1), layout=lay, **rq)
+    return p, x, o6
+
+
+@pytest.mark.parametrize("nhwc", [True, False])
+@pytest.mark.parametrize("pad_off", [False, True])
+def test_channel_padding_of_intermediates(nhwc, pad_off, monkeypatch):
+    if pad_off:
+        monkeypatch.setenv("THIP_NO_CHANNEL_PAD", "1")
+    p, x, want = _padded_chain(nhwc)
+    blob = p.serialize()
+    out = np.zeros(want.shape, dtype=np.int8)
+    d = desc_interp.run(blob, [x, out])
+    assert_bit_exact(out, want, "padded chain")
+    ops = [o for o in d.ops if int(o["kind"]) != desc_interp.K_TRANSPOSE]
+    c = 24 if pad_off else 32
+    assert [int(o["kind"]) for o in ops] == [desc_interp.K_IGEMM, desc_interp.K_DW, desc_interp.K_MAXPOOL,
+                                             desc_interp.K_IGEMM, desc_interp.K_ADD, desc_interp.K_IGEMM]
+    assert int(ops[0]["Nn"]) == c and int(ops[1]["C"]) == c and int(ops[2]["C"]) == c
+    assert int(ops[3]["C"]) == c and int(ops[3]["Nn"]) == c and int(ops[3]["gran"]) == (8 if pad_off else 16)
+    assert int(ops[4]["C"]) == 2 * 6 * 6 * c
+    assert int(ops[5]["K"]) == c and int(ops[5]["loader"]) == (1 if pad_off else 0) and int(ops[5]["Nn"]) == 40
+    assert int(ops[1]["variant"]) == (0 if pad_off else 1)
+
+
+def test_channel_padding_stops_at_ops_that_read_declared_order():
+    """A 24-channel tensor that feeds avg_pool2d (or leaves through a binding) is stored as declared."""
+    rng = np.random.default_rng(6)
+    N, H, W, C, B = 2, 5, 5, 16, 24
+    x = rng.integers(-128, 128, size=(N, H, W, C)).astype(np.int8)
+    wt = rng.integers(-127, 128, size=(B, C, 1, 1)).astype(np.int8)
+    mult, shift = w.random_requant(rng, B, True)
+    sb, sf = w.derive_scale_bias(mult, (shift - 3).astype(np.int8), rng.integers(-100, 100, size=B), wt, 0)
+    psb = np.array([0, (1 << 20) // (H * W)], dtype=np.int32)
+    rq = dict(output_min=-128, output_max=127)
+    p = Program()
+    t1 = p.conv2d(p.binding(0, x.shape), wt, sb, input_zp=0, output_zp=0, shift_factor=sf, pad=(0, 0, 0, 0), stride=(1, 1), nhwc_input=True, **rq)
+    p.avg_pool2d(t1, np.array([1], dtype=np.int8), psb, init=p.binding(1, (N, 1, 1, B)), input_zp=0, output_zp=0, shift_factor=20, **rq)
+    o1 = orc.conv2d(x, wt, sb, input_zp=0, output_zp=0, shift_factor=sf, pad=(0, 0, 0, 0), stride=(1, 1), layout=orc.NHWC, **rq)
+    want = orc.avg_pool2d(o1, psb, output_zp=0, shift_factor=20, **rq)
+    out = np.zeros(want.shape, dtype=np.int8)
+    d = desc_interp.run(p.serialize(), [x, out])
+    assert_bit_exact(out, want, "conv -> avg_pool2d")
+    assert int(d.ops[0]["Nn"]) == B and int(d.ops[1]["C"]) == B

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 from helpers import assert_bit_exact, oracle_eval, oracle_network, run_on_gpu
-from test_emitter import CONV, _chain_program
+from test_emitter import CONV, _chain_program, _padded_chain
 from torq_compiler_amd import Executable, ThipError, runtime, workloads as w
 
 pytestmark = pytest.mark.gpu
@@ -191,6 +191,18 @@ def test_multi_op_program(device):
     exe.run_host([x, out2, np.zeros_like(aux)])
     exe.close()
     assert np.array_equal(out, out2)
+
+
+@pytest.mark.parametrize("nhwc", [True, False])
+def test_padded_channel_chain(device, nhwc):
+    """24-channel intermediates stored as 32: depthwise, max pool, 3x3 conv, add and pointwise conv on them."""
+    p, x, want = _padded_chain(nhwc)
+    announce("padded-channel chain nhwc=%s" % nhwc)
+    exe = Executable(device, p.serialize())
+    out = np.zeros(want.shape, dtype=np.int8)
+    exe.run_host([x, out])
+    exe.close()
+    assert_bit_exact(out, want, "padded chain")
 
 
 @pytest.mark.parametrize("batch", [1, 3])

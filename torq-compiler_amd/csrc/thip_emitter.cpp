@@ -107,6 +107,20 @@ class Emitter {
     std::vector<uint64_t> temps_;
     std::vector<std::vector<uint8_t>> consts_;
     std::map<uint32_t, DescBinding> bindings_;
+    // Physical channel count of an intermediate whose channels are padded to a multiple of 16
+    // (0 = stored as declared).  See planChannelPadding.
+    std::vector<int64_t> cpad_;
+    std::vector<int64_t> cdeclared_;  // declared channel count of a padded intermediate
+
+    int64_t physC(thip_value_t id, int64_t C) const {
+        return (id >= 0 && (size_t)id < cpad_.size() && cpad_[id]) ? cpad_[id] : C;
+    }
+    // Elements the value occupies in memory (its channel axis possibly padded).
+    int64_t physNumel(thip_value_t id) const {
+        const int64_t n = prog_.values[id].numel();
+        return cpad_[id] ? n / cdeclared_[id] * cpad_[id] : n;
+    }
+    void planChannelPadding();
 
     thip_status_t checkValue(thip_value_t v, const char *what, const Value **out) const {
         if (v < 0 || (size_t)v >= prog_.values.size()) {
@@ -224,7 +238,7 @@ class Emitter {
         }
         if (v->dtype != dtype) return fail(THIP_INVALID_ARGUMENT, "%s: init element type mismatch", what);
         if (v->kind == kValueConstant) return fail(THIP_INVALID_ARGUMENT, "%s: init cannot be a constant", what);
-        const uint64_t bytes = (uint64_t)v->numel() * elemSize(dtype);
+        const uint64_t bytes = (uint64_t)(N * H * W * physC(id, C)) * elemSize(dtype);
         const bool sameInMemory = declaredNhwc || C == 1 || H * W == 1;
         if (v->kind == kValueTensor) {
             state_[id].ref = newTemp(bytes);
@@ -256,7 +270,8 @@ class Emitter {
     }
 
     // An output written in its declared order (FC, matmul, avg pool).
-    thip_status_t literalOutput(thip_value_t id, const char *what, int32_t dtype, int64_t numel, DescRef *out) {
+    thip_status_t literalOutput(thip_value_t id, const char *what, int32_t dtype, int64_t numel, DescRef *out,
+                                int64_t physElems = 0) {
         const Value *v;
         if (thip_status_t s = checkValue(id, what, &v)) return s;
         if (v->dtype != dtype) return fail(THIP_INVALID_ARGUMENT, "%s: init element type mismatch", what);
@@ -266,7 +281,7 @@ class Emitter {
         }
         if (v->kind == kValueConstant) return fail(THIP_INVALID_ARGUMENT, "%s: init cannot be a constant", what);
         if (v->kind == kValueTensor) {
-            state_[id].ref = newTemp((uint64_t)numel * elemSize(dtype));
+            state_[id].ref = newTemp((uint64_t)(physElems ? physElems : numel) * elemSize(dtype));
             state_[id].defined = true;
             state_[id].nhwcOfNchw = false;
             *out = state_[id].ref;
@@ -455,8 +470,10 @@ thip_status_t Emitter::emitConv2d(const thip_hl_conv2d_t &c) {
     if (d.C > 65535) return fail(THIP_UNIMPLEMENTED, "%s: more than 65535 input channels", what);
     int64_t OH, OW;
     if (thip_status_t s = windowGeometry(what, d.H, d.W, KH, KW, c.pad, c.stride, &OH, &OW)) return s;
-    const int64_t M = d.N * OH * OW, K = KH * KW * d.C;
-    if (!fitsInt32(M) || !fitsInt32(K) || !fitsInt32(M * O) || !fitsInt32(d.N * d.H * d.W * d.C)) {
+    // channel counts in memory: padded intermediates carry zero-weight channels (planChannelPadding)
+    const int64_t Cin = physC(c.input, d.C), Oout = physC(c.init, O);
+    const int64_t M = d.N * OH * OW, K = KH * KW * Cin;
+    if (!fitsInt32(M) || !fitsInt32(K) || !fitsInt32(M * Oout) || !fitsInt32(d.N * d.H * d.W * Cin)) {
         return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
     }
     DescOp op;
@@ -465,15 +482,15 @@ thip_status_t Emitter::emitConv2d(const thip_hl_conv2d_t &c) {
     Pending post;
     if (thip_status_t s = nhwcOutput(c.init, c.nhwc_input != 0, "torq_hl.conv2d init", init->dtype, d.N, O, OH, OW, &out, &post)) return s;
     const int64_t tile = 256;
-    if (thip_status_t s = splitScaleBias(c.scale_bias, "torq_hl.conv2d scale_bias", O, roundUp(O, tile), false, &op.bias, &op.scale)) return s;
+    if (thip_status_t s = splitScaleBias(c.scale_bias, "torq_hl.conv2d scale_bias", O, roundUp(Oout, tile), false, &op.bias, &op.scale)) return s;
     op.out_dtype = init->dtype;
     op.input_zp = c.input_zp;
     op.output_zp = c.output_zp;
     op.output_min = c.output_min;
     op.output_max = c.output_max;
     op.shift = c.shift_factor;
-    op.N = (int32_t)d.N; op.H = (int32_t)d.H; op.W = (int32_t)d.W; op.C = (int32_t)d.C;
-    op.OH = (int32_t)OH; op.OW = (int32_t)OW; op.OC = (int32_t)O;
+    op.N = (int32_t)d.N; op.H = (int32_t)d.H; op.W = (int32_t)d.W; op.C = (int32_t)Cin;
+    op.OH = (int32_t)OH; op.OW = (int32_t)OW; op.OC = (int32_t)Oout;
     op.KH = (int32_t)KH; op.KW = (int32_t)KW; op.SH = (int32_t)c.stride[0]; op.SW = (int32_t)c.stride[1];
     op.PL = (int32_t)c.pad[0]; op.PR = (int32_t)c.pad[1]; op.PT = (int32_t)c.pad[2]; op.PB = (int32_t)c.pad[3];
     op.in0 = in;
@@ -482,17 +499,18 @@ thip_status_t Emitter::emitConv2d(const thip_hl_conv2d_t &c) {
     const bool pointwise = KH == 1 && KW == 1 && c.stride[0] == 1 && c.stride[1] == 1 && c.pad[0] == 0 &&
                            c.pad[1] == 0 && c.pad[2] == 0 && c.pad[3] == 0;
     const int64_t C = d.C;
-    if (KW * C <= 16 && C % 16 != 0 && !getenv("THIP_NO_RUN_LOADER")) {
+    if (KW * Cin <= 16 && Cin % 16 != 0 && !getenv("THIP_NO_RUN_LOADER")) {
         // few input channels (the first layer of an image network): one 16-byte run per window row
-        emitIgemm(op, M, O, KH * 16, kLoaderRuns, [&](int64_t n, int64_t k) -> int8_t {
+        emitIgemm(op, M, Oout, KH * 16, kLoaderRuns, [&](int64_t n, int64_t k) -> int8_t {
             const int64_t kh = k / 16, b = k % 16;
-            if (b >= KW * C) return 0;
+            if (b >= KW * C || n >= O) return 0;
             return wd[((n * C + b % C) * KH + kh) * KW + b / C];
         });
     } else {
-        emitIgemm(op, M, O, K, (pointwise && K % 16 == 0) ? kLoaderDense : kLoaderGather, [&](int64_t n, int64_t k) {
-            const int64_t pos = k / C, ci = k % C;
+        emitIgemm(op, M, Oout, K, (pointwise && K % 16 == 0) ? kLoaderDense : kLoaderGather, [&](int64_t n, int64_t k) -> int8_t {
+            const int64_t pos = k / Cin, ci = k % Cin;
             const int64_t kh = pos / KW, kw = pos % KW;
+            if (ci >= C || n >= O) return 0;  // padded channels meet zero weights
             return wd[((n * C + ci) * KH + kh) * KW + kw];
         });
     }
@@ -522,17 +540,19 @@ thip_status_t Emitter::emitDepthwise(const thip_hl_depthwise_conv2d_t &c) {
     if (c.groups != C && c.groups != 1 && c.groups != 0) return fail(THIP_INVALID_ARGUMENT, "%s: groups must equal the channel count", what);
     int64_t OH, OW;
     if (thip_status_t s = windowGeometry(what, d.H, d.W, KH, KW, c.pad, c.stride, &OH, &OW)) return s;
-    if (!fitsInt32(d.N * OH * OW * C) || !fitsInt32(d.N * d.H * d.W * C)) return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
+    // channels in memory (input and output of a depthwise op are padded alike); padded channels get zero weights
+    const int64_t Cp = physC(c.input, C);
+    if (!fitsInt32(d.N * OH * OW * Cp) || !fitsInt32(d.N * d.H * d.W * Cp)) return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
     DescOp op;
     memset(&op, 0, sizeof(op));
     DescRef out;
     Pending post;
     if (thip_status_t s = nhwcOutput(c.init, c.nhwc_input != 0, "torq_hl.depthwise_conv2d init", init->dtype, d.N, C, OH, OW, &out, &post)) return s;
-    if (thip_status_t s = splitScaleBias(c.scale_bias, "torq_hl.depthwise_conv2d scale_bias", C, roundUp(C, 16), false, &op.bias, &op.scale)) return s;
+    if (thip_status_t s = splitScaleBias(c.scale_bias, "torq_hl.depthwise_conv2d scale_bias", C, roundUp(Cp, 16), false, &op.bias, &op.scale)) return s;
     const int8_t *wd = (const int8_t *)w->data.data();
-    std::vector<int8_t> wpk((size_t)(KH * KW * C));
+    std::vector<int8_t> wpk((size_t)(KH * KW * Cp), 0);
     for (int64_t ch = 0; ch < C; ch++) {
-        for (int64_t k = 0; k < KH * KW; k++) wpk[(size_t)(k * C + ch)] = wd[ch * KH * KW + k];
+        for (int64_t k = 0; k < KH * KW; k++) wpk[(size_t)(k * Cp + ch)] = wd[ch * KH * KW + k];
     }
     op.kind = kKindDepthwise;
     op.out_dtype = init->dtype;
@@ -541,20 +561,20 @@ thip_status_t Emitter::emitDepthwise(const thip_hl_depthwise_conv2d_t &c) {
     op.output_min = c.output_min;
     op.output_max = c.output_max;
     op.shift = c.shift_factor;
-    op.N = (int32_t)d.N; op.H = (int32_t)d.H; op.W = (int32_t)d.W; op.C = (int32_t)C;
-    op.OH = (int32_t)OH; op.OW = (int32_t)OW; op.OC = (int32_t)C;
+    op.N = (int32_t)d.N; op.H = (int32_t)d.H; op.W = (int32_t)d.W; op.C = (int32_t)Cp;
+    op.OH = (int32_t)OH; op.OW = (int32_t)OW; op.OC = (int32_t)Cp;
     op.KH = (int32_t)KH; op.KW = (int32_t)KW; op.SH = (int32_t)c.stride[0]; op.SW = (int32_t)c.stride[1];
     op.PL = (int32_t)c.pad[0]; op.PR = (int32_t)c.pad[1]; op.PT = (int32_t)c.pad[2]; op.PB = (int32_t)c.pad[3];
     op.in0 = in;
     op.out = out;
-    if (KH == 3 && KW == 3 && C % 16 == 0 && !getenv("THIP_DEPTHWISE_GENERIC")) {
+    if (KH == 3 && KW == 3 && Cp % 16 == 0 && !getenv("THIP_DEPTHWISE_GENERIC")) {
         // one dword per (window row, channel): byte kw = tap kw, byte 3 = 0, for v_dot4_i32_i8
-        std::vector<uint32_t> wdot((size_t)(KH * C));
+        std::vector<uint32_t> wdot((size_t)(KH * Cp), 0);
         for (int64_t ch = 0; ch < C; ch++) {
             for (int64_t kh = 0; kh < KH; kh++) {
                 uint32_t v = 0;
                 for (int64_t kw = 0; kw < KW; kw++) v |= (uint32_t)(uint8_t)wd[(ch * KH + kh) * KW + kw] << (8 * kw);
-                wdot[(size_t)(kh * C + ch)] = v;
+                wdot[(size_t)(kh * Cp + ch)] = v;
             }
         }
         op.variant = kDepthwiseDot4Rows;
@@ -716,7 +736,8 @@ thip_status_t Emitter::emitMaxPool(const thip_hl_maxpool2d_t &c) {
     if (thip_status_t s = nhwcInput(c.input, c.nhwc_input != 0, "torq_hl.maxpool2d input", &d, &in)) return s;
     int64_t OH, OW;
     if (thip_status_t s = windowGeometry(what, d.H, d.W, c.kernel[0], c.kernel[1], c.pad, c.stride, &OH, &OW)) return s;
-    if (!fitsInt32(d.N * d.H * d.W * d.C)) return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
+    const int64_t Cp = physC(c.input, d.C);  // input and output are padded alike
+    if (!fitsInt32(d.N * d.H * d.W * Cp)) return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
     DescOp op;
     memset(&op, 0, sizeof(op));
     DescRef out;
@@ -727,8 +748,8 @@ thip_status_t Emitter::emitMaxPool(const thip_hl_maxpool2d_t &c) {
     op.input_zp = c.input_zp;
     op.output_min = c.output_min;
     op.output_max = c.output_max;
-    op.N = (int32_t)d.N; op.H = (int32_t)d.H; op.W = (int32_t)d.W; op.C = (int32_t)d.C;
-    op.OH = (int32_t)OH; op.OW = (int32_t)OW; op.OC = (int32_t)d.C;
+    op.N = (int32_t)d.N; op.H = (int32_t)d.H; op.W = (int32_t)d.W; op.C = (int32_t)Cp;
+    op.OH = (int32_t)OH; op.OW = (int32_t)OW; op.OC = (int32_t)Cp;
     op.KH = (int32_t)c.kernel[0]; op.KW = (int32_t)c.kernel[1]; op.SH = (int32_t)c.stride[0]; op.SW = (int32_t)c.stride[1];
     op.PL = (int32_t)c.pad[0]; op.PR = (int32_t)c.pad[1]; op.PT = (int32_t)c.pad[2]; op.PB = (int32_t)c.pad[3];
     op.in0 = in;
@@ -797,7 +818,10 @@ thip_status_t Emitter::emitAdd(const thip_hl_add_t &c) {
     op.w1 = ((const int16_t *)w->data.data())[1];
     op.bias0 = ((const int32_t *)sb->data.data())[0];
     op.scale0 = ((const int32_t *)sb->data.data())[1];
-    if (!fitsInt32(a->numel())) return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
+    // elements in memory: the three operands of an add are padded alike (padded channels hold
+    // values nobody reads)
+    const int64_t count = physNumel(c.init);
+    if (!fitsInt32(count)) return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
     Pending post;
     // Elementwise: any memory order works as long as all three agree.  If one
     // operand is an N,C,H,W intermediate kept as NHWC, bring the others to it.
@@ -810,10 +834,10 @@ thip_status_t Emitter::emitAdd(const thip_hl_add_t &c) {
     } else {
         if (thip_status_t s = literalInput(c.input1, "torq_hl.add input1", &op.in0)) return s;
         if (thip_status_t s = literalInput(c.input2, "torq_hl.add input2", &op.in1)) return s;
-        if (thip_status_t s = literalOutput(c.init, "torq_hl.add init", THIP_DTYPE_I8, a->numel(), &op.out)) return s;
+        if (thip_status_t s = literalOutput(c.init, "torq_hl.add init", THIP_DTYPE_I8, a->numel(), &op.out, count)) return s;
     }
     op.N = 1; op.H = 1; op.W = 1;
-    op.C = (int32_t)a->numel();
+    op.C = (int32_t)count;
     ops_.push_back(op);
     finishOutput(post);
     return THIP_OK;
@@ -881,7 +905,95 @@ thip_status_t Emitter::emitTransposeOp(const thip_hl_transpose_t &c) {
     return THIP_OK;
 }
 
+// Decides which intermediates are stored with their channel axis padded to a multiple of 16.
+// A pointwise convolution over such a tensor streams it with 16-byte loads (the dense loader)
+// instead of gathering 8-byte pieces, which is what the 24-channel bottlenecks of mobile
+// networks otherwise cost.  Padded channels are produced with zero weights, bias and scale and
+// met with zero weights by every consumer, so their values never reach a result.  Ops that do
+// not look at single channels (depthwise, max pool, add) tie their operands together: all of
+// them are padded or none.  Anything that reads a tensor in its declared order (bindings,
+// fully_connected, matmul, avg_pool2d, transpose) keeps the whole group unpadded.
+// THIP_NO_CHANNEL_PAD switches the pass off.
+void Emitter::planChannelPadding() {
+    const size_t n = prog_.values.size();
+    cpad_.assign(n, 0);
+    cdeclared_.assign(n, 0);
+    if (getenv("THIP_NO_CHANNEL_PAD")) return;
+    std::vector<size_t> parent(n);
+    for (size_t i = 0; i < n; i++) parent[i] = i;
+    std::vector<int64_t> chan(n, 0);  // channel count seen at the uses; -1 = must stay as declared
+    std::vector<char> touched(n, 0);
+    auto valid = [&](thip_value_t v) { return v >= 0 && (size_t)v < n; };
+    auto find = [&](size_t v) {
+        while (parent[v] != v) v = parent[v] = parent[parent[v]];
+        return v;
+    };
+    auto tie = [&](thip_value_t a, thip_value_t b) {
+        if (!valid(a) || !valid(b)) return;
+        parent[find((size_t)a)] = find((size_t)b);
+        touched[a] = touched[b] = 1;
+    };
+    auto bar = [&](thip_value_t v) {
+        if (!valid(v)) return;
+        chan[v] = -1;
+        touched[v] = 1;
+    };
+    auto use = [&](thip_value_t v, bool nhwc) {
+        if (!valid(v)) return;
+        const Value &val = prog_.values[v];
+        touched[v] = 1;
+        const int64_t C = val.rank == 4 ? val.shape[nhwc ? 3 : 1] : -1;
+        if (chan[v] == 0) chan[v] = C;
+        else if (chan[v] != C) chan[v] = -1;
+    };
+    for (const HlOp &op : prog_.ops) {
+        switch (op.kind) {
+        case kHlConv2d:
+            use(op.u.conv.input, op.u.conv.nhwc_input != 0);
+            use(op.u.conv.init, op.u.conv.nhwc_input != 0);
+            break;
+        case kHlDepthwise:
+            use(op.u.dw.input, op.u.dw.nhwc_input != 0);
+            use(op.u.dw.init, op.u.dw.nhwc_input != 0);
+            tie(op.u.dw.input, op.u.dw.init);
+            break;
+        case kHlMaxPool:
+            use(op.u.mp.input, op.u.mp.nhwc_input != 0);
+            use(op.u.mp.init, op.u.mp.nhwc_input != 0);
+            tie(op.u.mp.input, op.u.mp.init);
+            break;
+        case kHlAdd:
+            tie(op.u.add.input1, op.u.add.input2);
+            tie(op.u.add.input1, op.u.add.init);
+            break;
+        case kHlFullyConnected: bar(op.u.fc.input); bar(op.u.fc.init); break;
+        case kHlMatmul: bar(op.u.mm.input1); bar(op.u.mm.input2); bar(op.u.mm.init); break;
+        case kHlAvgPool: bar(op.u.ap.input); bar(op.u.ap.init); break;
+        case kHlTranspose: bar(op.u.tr.input); bar(op.u.tr.init); break;
+        }
+    }
+    // one verdict per group: every member an int8 rank-4 intermediate, all uses agreeing on C
+    std::vector<int64_t> groupC(n, 0);
+    for (size_t v = 0; v < n; v++) {
+        const size_t g = find(v);
+        const Value &val = prog_.values[v];
+        if (!touched[v]) continue;  // weights and other values no activation op touches
+        const bool plain = val.kind == kValueTensor && val.rank == 4 && val.dtype == THIP_DTYPE_I8;
+        if (!plain || chan[v] < 0) groupC[g] = -1;
+        else if (chan[v] > 0 && groupC[g] == 0) groupC[g] = chan[v];
+        else if (chan[v] > 0 && groupC[g] != chan[v]) groupC[g] = -1;
+    }
+    for (size_t v = 0; v < n; v++) {
+        const int64_t C = groupC[find(v)];
+        if (C > 16 && C % 16 != 0 && prog_.values[v].kind == kValueTensor) {
+            cpad_[v] = roundUp(C, 16);
+            cdeclared_[v] = C;
+        }
+    }
+}
+
 thip_status_t Emitter::run(void **outBlob, size_t *outSize) {
+    planChannelPadding();
     for (const HlOp &op : prog_.ops) {
         thip_status_t s = THIP_OK;
         switch (op.kind) {
