@@ -76,6 +76,21 @@ def test_dense_igemm_every_tile_variant(device, variant, monkeypatch):
     check(device, w.conv2d_workload(N=2, H=28, W=28, C=192, O=32, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True))
 
 
+def test_stream_igemm(device, monkeypatch):
+    """The pixel-streaming kernel (weights resident in LDS): every accumulator width, ragged M, k-step
+    counts around the prefetch ring, N ending in half a 32-channel block, both requant tails."""
+    monkeypatch.setenv("THIP_IGEMM_DENSE_VARIANT", "11")
+    for M, K, N in [(33, 16, 16), (257, 80, 48), (1000, 144, 32), (4099, 96, 112), (5000, 32, 144),
+                    (300, 192, 240), (2048, 224, 256), (70000, 32, 16)]:
+        check(device, w.fully_connected_workload(M, K, N, realistic=True), kernel="igemm_stream_i8")
+    for shift in [0, 1, 31, 32, 33, 34, 62]:
+        check(device, w.fully_connected_workload(500, 48, 80, shift=shift, output_zp=-7), kernel="igemm_stream_i8")
+    # chosen without forcing for a pointwise convolution over a large image; not when the weights outgrow LDS
+    monkeypatch.delenv("THIP_IGEMM_DENSE_VARIANT")
+    check(device, w.conv2d_workload(N=4, H=56, W=56, C=32, O=144, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True), kernel="igemm_stream_i8")
+    check(device, w.fully_connected_workload(8192, 256, 256, realistic=True), kernel="igemm_dense_i8")
+
+
 @pytest.mark.parametrize("shift", [0, 1, 6, 31, 32, 33, 34, 40, 62])
 def test_igemm_shift_boundaries(device, shift):
     """Both epilogue tails of the MFMA kernels (generic 64-bit, and 32-bit for shift >= 33) around their switch."""

@@ -342,7 +342,7 @@ class Emitter {
     }
 
     // Tile choice.  THIP_IGEMM_VARIANT / THIP_IGEMM_DENSE_VARIANT force one (for tuning runs).
-    static uint32_t chooseIgemmVariant(int64_t M, int64_t N, bool dense) {
+    static uint32_t chooseIgemmVariant(int64_t M, int64_t N, bool dense, int64_t K = 0, int32_t outDtype = 0) {
         auto tiles = [&](uint32_t v) {
             const IgemmTile &t = igemmTile(v);
             return ((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn);
@@ -350,8 +350,12 @@ class Emitter {
         if (dense) {
             if (const char *env = getenv("THIP_IGEMM_DENSE_VARIANT")) {
                 const long v = strtol(env, nullptr, 10);
-                if (v >= 0 && v < (long)kIgemmVariantCount) return (uint32_t)v;
+                if (v >= 0 && v < (long)kIgemmVariantCount && (v != (long)kIgemmStream || igemmStreamFits(N, K, outDtype))) {
+                    return (uint32_t)v;
+                }
             }
+            // a small weight matrix over many pixels: keep it in LDS and stream the pixels
+            if (M >= 4096 && igemmStreamFits(N, K, outDtype) && !getenv("THIP_NO_STREAM")) return kIgemmStream;
             // N narrower than a tile: one tile column of the narrowest tile that covers N, so the
             // activations are streamed once (these shapes are bandwidth-bound, padded MFMA work is free)
             if (N <= 128 && M >= 4096) {
@@ -378,7 +382,7 @@ class Emitter {
     template <typename WeightAt>
     void emitIgemm(DescOp base, int64_t M, int64_t N, int64_t K, uint32_t loader, WeightAt wAt) {
         const bool dense = loader == kLoaderDense;
-        const uint32_t variant = chooseIgemmVariant(M, N, dense);
+        const uint32_t variant = chooseIgemmVariant(M, N, dense, K, base.out_dtype);
         const IgemmTile &t = igemmTile(variant);
         const int64_t Kp = roundUp(K, t.bk), Np = roundUp(N, t.bn);
         std::vector<int8_t> packed((size_t)(Np * Kp), 0);

@@ -48,13 +48,20 @@ enum IgemmVariant : uint32_t {
     kIgemmDense256x128 = 8,
     kIgemmDense256x64 = 9,   // narrow-N tiles for the pointwise convolutions of mobile networks
     kIgemmDense256x32 = 10,
-    kIgemmVariantCount = 11,
+    // dense operand, weights of at most 64 KiB resident in LDS, N <= 256, int8 output: streams the pixels
+    kIgemmStream = 11,
+    kIgemmVariantCount = 12,
 };
 struct IgemmTile {
     int bm, bn, bk;
     const char *name;
 };
 const IgemmTile &igemmTile(uint32_t variant);
+// Whether the streaming variant takes this shape (its launcher checks the same).
+inline bool igemmStreamFits(int64_t N, int64_t K, int32_t out_dtype) {
+    const int64_t Np = (N + 31) / 32 * 32, Kp = (K + 31) / 32 * 32;
+    return out_dtype == 1 && N % 16 == 0 && K % 16 == 0 && Np <= 256 && Np * Kp + 8 * Np <= 64 * 1024;
+}
 hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, hipStream_t stream);
 
 struct FcSkinnyArgs {

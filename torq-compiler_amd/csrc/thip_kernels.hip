@@ -14,6 +14,7 @@
 // output zero point, clamp.
 #include "thip_kernels.h"
 
+#include <algorithm>
 #include <type_traits>
 
 #include "thip_descriptor.h"
@@ -665,6 +666,167 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
     igemmEpilogue<WTM, WTN, NW, BN>(acc, smem, p, m0, n0, wm, wn, myBias, myScale);
 }
 
+
+// ---------------------------------------------------------------------------
+// igemm_stream_i8: pointwise convolution / fully_connected with a small weight matrix
+// (Np * Kp of at most 64 KiB, N <= 256), the shape of the expand and project convolutions of
+// mobile networks at high resolution.  These are bandwidth-bound: a tile kernel spends its time
+// in load -> MFMA -> epilogue phases that do not overlap.  Here the whole weight matrix sits in
+// LDS in MFMA fragment order and every wave streams 32-pixel groups: per k-step one 16-byte
+// activation load per lane and NB MFMAs (weights as the row operand), then the requant on the
+// accumulator registers.  Lane l of an accumulator holds, for pixel l & 31, the channels
+// 8 g + 4 (l >> 5) + {0..3} of register group g; two v_permlane32_swap exchange groups between
+// the wave halves so that each lane owns 16 consecutive channels and stores them as one 128-bit
+// word: no LDS round trip and no barrier after the prologue.  Activation loads run RING k-steps
+// ahead, across group boundaries.  K % 16 == 0, N % 16 == 0, int8 output.
+// ---------------------------------------------------------------------------
+constexpr int kStreamRing = 4;
+constexpr size_t kStreamMaxLds = 64 * 1024;
+
+template <int NB>
+__global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArgs p) {
+    extern __shared__ __attribute__((aligned(16))) int8_t smem[];
+    constexpr int RING = kStreamRing;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int fr = lane & 31, half = lane >> 5;
+    const int ksteps = p.Kp / 32, nblocks = p.Np / 32;
+    // weights [Np][Kp] -> fragment order: fragment (s, j) = 64 lanes x 16 bytes, lane (n & 31) + 32 (kc & 1)
+    {
+        const int chunksPerRow = p.Kp / 16, total = p.Np * chunksPerRow;
+        for (int c = tid; c < total; c += 256) {
+            const int n = c / chunksPerRow, kc = c - n * chunksPerRow;
+            const v4i v = *(const v4i *)(p.Bp + (size_t)n * p.Kp + kc * 16);
+            *(v4i *)(smem + ((((kc >> 1) * nblocks + (n >> 5)) * 64 + (kc & 1) * 32 + (n & 31)) << 4)) = v;
+        }
+    }
+    int32_t *ldsBias = (int32_t *)(smem + (size_t)p.Np * p.Kp), *ldsScale = ldsBias + p.Np;
+    for (int c = tid; c < p.Np; c += 256) {
+        ldsBias[c] = p.bias[c];
+        ldsScale[c] = p.scale[c];
+    }
+    __syncthreads();
+
+    const int groups = (p.M + 31) / 32, stride = gridDim.x * 4;
+    const int kstepsRing = (ksteps + RING - 1) / RING * RING;
+    // 16 bytes of pixel row (32 g + fr) at k-step s; zero past K or past the last group
+    auto fetch = [&](int g, int s) -> v4i {
+        const int k = s * 32 + half * 16;
+        if (g >= groups || k >= p.K) return v4i{0, 0, 0, 0};
+        int m = g * 32 + fr;
+        m = m < p.M ? m : p.M - 1;
+        return *(const v4i *)(p.A + (size_t)m * p.K + k);
+    };
+    const bool wideShift = p.rq.shift >= 33;
+    const int shiftMinus32 = p.rq.shift - 32;
+    const int32_t rndHigh = wideShift ? (int32_t)(1u << (p.rq.shift - 33)) : 0;
+    const long long rnd = roundTerm(p.rq.shift);
+    const long long lo64 = (long long)p.rq.out_min - p.rq.out_zp, hi64 = (long long)p.rq.out_max - p.rq.out_zp;
+    const int32_t lo32 = (int32_t)(lo64 < INT32_MIN ? INT32_MIN : lo64), hi32 = (int32_t)(hi64 > INT32_MAX ? INT32_MAX : hi64);
+
+    int g = blockIdx.x * 4 + wave;
+    v4i ring[RING];
+#pragma unroll
+    for (int d = 0; d < RING; d++) ring[d] = fetch(g, d);
+    for (; g < groups; g += stride) {
+        v16i acc[NB];
+#pragma unroll
+        for (int j = 0; j < NB; j++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[j][r] = 0;
+        }
+        for (int s0 = 0; s0 < kstepsRing; s0 += RING) {
+#pragma unroll
+            for (int d = 0; d < RING; d++) {
+                const int s = s0 + d;
+                const v4i a = ring[d];
+                // slot d next holds k-step s + RING of this group, or the same slot of the next group
+                const bool wrap = s + RING >= kstepsRing;
+                ring[d] = fetch(wrap ? g + stride : g, wrap ? s + RING - kstepsRing : s + RING);
+                if (s < ksteps) {
+                    const int8_t *wfrag = smem + ((size_t)(s * nblocks) * 64 + lane) * 16;
+#pragma unroll
+                    for (int j = 0; j < NB; j++) {
+                        if (j < nblocks) {
+                            const v4i w = *(const v4i *)(wfrag + j * 1024);
+                            acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w, a, acc[j], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+        }
+        const int m = g * 32 + fr;
+        auto finish = [&](auto wideShiftTag) {
+            constexpr bool kWideShift = decltype(wideShiftTag)::value;
+#pragma unroll
+            for (int j = 0; j < NB; j++) {
+                if (j < nblocks) {
+                    uint32_t d4[4];
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        const int ch = j * 32 + 8 * q + 4 * half;
+                        const v4i b4 = *(const v4i *)(ldsBias + ch);
+                        const v4i s4 = *(const v4i *)(ldsScale + ch);
+                        uint32_t packed = 0;
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            const int32_t v = kWideShift ? requantWideShift(acc[j][4 * q + e], b4[e], s4[e], rndHigh, shiftMinus32, lo32, hi32, p.rq.out_zp)
+                                                         : requant(acc[j][4 * q + e], b4[e], s4[e], rnd, p.rq);
+                            packed |= (uint32_t)(v & 0xff) << (8 * e);
+                        }
+                        d4[q] = packed;
+                    }
+                    // lower half lanes: channels 0-3, 8-11, 16-19, 24-27; upper half: 4-7, 12-15, 20-23, 28-31.
+                    // Swap (upper of d4[0], lower of d4[2]) and (upper of d4[1], lower of d4[3]):
+                    // then {d4[0], d4[2], d4[1], d4[3]} are 16 consecutive channels, 0-15 below, 16-31 above.
+                    const auto s02 = __builtin_amdgcn_permlane32_swap(d4[0], d4[2], false, false);
+                    const auto s13 = __builtin_amdgcn_permlane32_swap(d4[1], d4[3], false, false);
+                    const v4i outv = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
+                    const int n = j * 32 + 16 * half;
+                    if (m < p.M && n < p.N) *(v4i *)((int8_t *)p.out + (size_t)m * p.N + n) = outv;
+                }
+            }
+        };
+        if (wideShift) {
+            finish(std::true_type{});
+        } else {
+            finish(std::false_type{});
+        }
+    }
+}
+
+template <int NB>
+static hipError_t launchIgemmStreamT(const IgemmArgs &a, size_t smem, hipStream_t stream) {
+    auto kernel = igemm_stream_i8<NB>;
+    static bool configured = false;
+    if (!configured) {
+        hipError_t err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kStreamMaxLds);
+        if (err != hipSuccess) return err;
+        configured = true;
+    }
+    // every block copies the weights into LDS once, then strides over the pixel groups:
+    // one resident set of blocks, each with several groups where the image is large
+    // blocks one CU holds: by registers (7, 5, 4, 3, 2 waves per SIMD for NB = 1, 2, 4, 6, 8) and by LDS
+    const int byRegs = NB <= 1 ? 7 : NB <= 2 ? 5 : NB <= 4 ? 4 : NB <= 6 ? 3 : 2;
+    const int perCu = (int)std::min<size_t>(byRegs, (160 * 1024) / smem);
+    const int groups = (a.M + 31) / 32;
+    const int blocks = std::min((groups + 3) / 4, 256 * perCu);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), smem, stream, a);
+    return hipGetLastError();
+}
+
+static hipError_t launchIgemmStream(const IgemmArgs &a, hipStream_t stream) {
+    if (a.loader != kLoaderDense || a.out_dtype != kDtypeI8) return hipErrorInvalidValue;
+    if (a.N % 16 != 0 || a.Np > 256 || ((uintptr_t)a.out & 15) != 0) return hipErrorInvalidValue;
+    const size_t smem = (size_t)a.Np * a.Kp + 8 * (size_t)a.Np;
+    if (smem > kStreamMaxLds) return hipErrorInvalidValue;
+    const int nb = a.Np / 32;
+    if (nb <= 1) return launchIgemmStreamT<1>(a, smem, stream);
+    if (nb <= 2) return launchIgemmStreamT<2>(a, smem, stream);
+    if (nb <= 4) return launchIgemmStreamT<4>(a, smem, stream);
+    if (nb <= 6) return launchIgemmStreamT<6>(a, smem, stream);
+    return launchIgemmStreamT<8>(a, smem, stream);
+}
+
 static const IgemmTile kTiles[kIgemmVariantCount] = {
     {128, 128, 64, "igemm_i8_128x128x64"},
     {256, 256, 64, "igemm_i8_256x256x64"},
@@ -677,6 +839,7 @@ static const IgemmTile kTiles[kIgemmVariantCount] = {
     {256, 128, 64, "igemm_dense_i8_256x128x64"},
     {256, 64, 64, "igemm_dense_i8_256x64x64"},
     {256, 32, 64, "igemm_dense_i8_256x32x64"},
+    {32, 32, 32, "igemm_stream_i8"},
 };
 
 const IgemmTile &igemmTile(uint32_t variant) {
@@ -778,6 +941,7 @@ hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, hipStream_t stream)
     case kIgemmDense256x128: return launchIgemmDense<256, 128, 2, 2, 3, 2>(a, stream);
     case kIgemmDense256x64: return launchIgemmDense<256, 64, 4, 1, 3, 2>(a, stream);
     case kIgemmDense256x32: return launchIgemmDense<256, 32, 4, 1, 3, 2>(a, stream);
+    case kIgemmStream: return launchIgemmStream(a, stream);
     default: return hipErrorInvalidValue;
     }
 }
