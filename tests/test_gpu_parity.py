@@ -81,7 +81,8 @@ def test_stream_igemm(device, monkeypatch):
     counts around the prefetch ring, N ending in half a 32-channel block, both requant tails."""
     monkeypatch.setenv("THIP_IGEMM_DENSE_VARIANT", "11")
     for M, K, N in [(33, 16, 16), (257, 80, 48), (1000, 144, 32), (4099, 96, 112), (5000, 32, 144),
-                    (300, 192, 240), (2048, 224, 256), (70000, 32, 16)]:
+                    (300, 192, 240), (2048, 224, 256), (70000, 32, 16),
+                    (900, 64, 384), (700, 96, 592), (513, 32, 1008)]:
         check(device, w.fully_connected_workload(M, K, N, realistic=True), kernel="igemm_stream_i8")
     for shift in [0, 1, 31, 32, 33, 34, 62]:
         check(device, w.fully_connected_workload(500, 48, 80, shift=shift, output_zp=-7), kernel="igemm_stream_i8")

@@ -57,10 +57,20 @@ struct IgemmTile {
     const char *name;
 };
 const IgemmTile &igemmTile(uint32_t variant);
-// Whether the streaming variant takes this shape (its launcher checks the same).
+// The streaming variant splits the (padded) output channels into equal chunks of at most 256, a
+// multiple of 32 each; one grid row per chunk, whose weights stay in LDS.
+__host__ __device__ inline int igemmStreamChunk(int Np) {
+    const int blocks = Np / 32, chunks = (Np + 255) / 256;
+    return (blocks + chunks - 1) / chunks * 32;
+}
+// Whether the streaming variant takes this shape (its launcher checks the same): a chunk of the
+// weights fits 64 KiB of LDS, and re-reading the activations once per chunk costs no more than
+// the output itself.
 inline bool igemmStreamFits(int64_t N, int64_t K, int32_t out_dtype) {
+    if (out_dtype != 1 || N <= 0 || K <= 0 || N % 16 != 0 || K % 16 != 0 || N > 65536 || K > 65536) return false;
     const int64_t Np = (N + 31) / 32 * 32, Kp = (K + 31) / 32 * 32;
-    return out_dtype == 1 && N % 16 == 0 && K % 16 == 0 && Np <= 256 && Np * Kp + 8 * Np <= 64 * 1024;
+    const int64_t chunk = igemmStreamChunk((int)Np), chunks = (Np + chunk - 1) / chunk;
+    return chunk * Kp + 8 * chunk <= 64 * 1024 && (chunks - 1) * K <= N;
 }
 hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, hipStream_t stream);
 

@@ -689,20 +689,23 @@ __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArg
     constexpr int RING = kStreamRing;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int fr = lane & 31, half = lane >> 5;
-    const int ksteps = p.Kp / 32, nblocks = p.Np / 32;
-    // weights [Np][Kp] -> fragment order: fragment (s, j) = 64 lanes x 16 bytes, lane (n & 31) + 32 (kc & 1)
+    // this grid row's chunk of output channels
+    const int chunk = igemmStreamChunk(p.Np), n0 = blockIdx.y * chunk;
+    const int chunkN = (p.Np - n0 < chunk ? p.Np - n0 : chunk);
+    const int ksteps = p.Kp / 32, nblocks = chunkN / 32;
+    // weights [chunkN][Kp] -> fragment order: fragment (s, j) = 64 lanes x 16 bytes, lane (n & 31) + 32 (kc & 1)
     {
-        const int chunksPerRow = p.Kp / 16, total = p.Np * chunksPerRow;
+        const int chunksPerRow = p.Kp / 16, total = chunkN * chunksPerRow;
         for (int c = tid; c < total; c += 256) {
             const int n = c / chunksPerRow, kc = c - n * chunksPerRow;
-            const v4i v = *(const v4i *)(p.Bp + (size_t)n * p.Kp + kc * 16);
+            const v4i v = *(const v4i *)(p.Bp + (size_t)(n0 + n) * p.Kp + kc * 16);
             *(v4i *)(smem + ((((kc >> 1) * nblocks + (n >> 5)) * 64 + (kc & 1) * 32 + (n & 31)) << 4)) = v;
         }
     }
-    int32_t *ldsBias = (int32_t *)(smem + (size_t)p.Np * p.Kp), *ldsScale = ldsBias + p.Np;
-    for (int c = tid; c < p.Np; c += 256) {
-        ldsBias[c] = p.bias[c];
-        ldsScale[c] = p.scale[c];
+    int32_t *ldsBias = (int32_t *)(smem + (size_t)chunkN * p.Kp), *ldsScale = ldsBias + chunkN;
+    for (int c = tid; c < chunkN; c += 256) {
+        ldsBias[c] = p.bias[n0 + c];
+        ldsScale[c] = p.scale[n0 + c];
     }
     __syncthreads();
 
@@ -781,7 +784,7 @@ __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArg
                     const auto s02 = __builtin_amdgcn_permlane32_swap(d4[0], d4[2], false, false);
                     const auto s13 = __builtin_amdgcn_permlane32_swap(d4[1], d4[3], false, false);
                     const v4i outv = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
-                    const int n = j * 32 + 16 * half;
+                    const int n = n0 + j * 32 + 16 * half;
                     if (m < p.M && n < p.N) *(v4i *)((int8_t *)p.out + (size_t)m * p.N + n) = outv;
                 }
             }
@@ -809,17 +812,19 @@ static hipError_t launchIgemmStreamT(const IgemmArgs &a, size_t smem, hipStream_
     const int byRegs = NB <= 1 ? 7 : NB <= 2 ? 5 : NB <= 4 ? 4 : NB <= 6 ? 3 : 2;
     const int perCu = (int)std::min<size_t>(byRegs, (160 * 1024) / smem);
     const int groups = (a.M + 31) / 32;
-    const int blocks = std::min((groups + 3) / 4, 256 * perCu);
-    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), smem, stream, a);
+    const int chunk = igemmStreamChunk(a.Np), chunks = (a.Np + chunk - 1) / chunk;
+    const int blocks = std::min((groups + 3) / 4, std::max(1, 256 * perCu / chunks));
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)chunks), dim3(256), smem, stream, a);
     return hipGetLastError();
 }
 
 static hipError_t launchIgemmStream(const IgemmArgs &a, hipStream_t stream) {
     if (a.loader != kLoaderDense || a.out_dtype != kDtypeI8) return hipErrorInvalidValue;
-    if (a.N % 16 != 0 || a.Np > 256 || ((uintptr_t)a.out & 15) != 0) return hipErrorInvalidValue;
-    const size_t smem = (size_t)a.Np * a.Kp + 8 * (size_t)a.Np;
-    if (smem > kStreamMaxLds) return hipErrorInvalidValue;
-    const int nb = a.Np / 32;
+    if (a.N % 16 != 0 || ((uintptr_t)a.out & 15) != 0) return hipErrorInvalidValue;
+    const int chunk = igemmStreamChunk(a.Np);
+    const size_t smem = (size_t)chunk * a.Kp + 8 * (size_t)chunk;
+    if (chunk > 256 || smem > kStreamMaxLds) return hipErrorInvalidValue;
+    const int nb = chunk / 32;
     if (nb <= 1) return launchIgemmStreamT<1>(a, smem, stream);
     if (nb <= 2) return launchIgemmStreamT<2>(a, smem, stream);
     if (nb <= 4) return launchIgemmStreamT<4>(a, smem, stream);
