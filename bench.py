@@ -41,6 +41,7 @@ def workload_table(pkg):
         "conv_112x112x32_o64_3x3": (lambda: w.conv2d_workload(), "mfma"),
         "depthwise_b64": (lambda: w.depthwise_workload(N=64), "hbm"),
         "depthwise_b1": (lambda: w.depthwise_workload(N=1), "hbm"),
+        "depthwise_s1_b256": (lambda: w.depthwise_workload(N=256, stride=(1, 1), pad=(1, 1, 1, 1)), "hbm"),
         "maxpool_b64": (lambda: w.maxpool_workload(N=64), "hbm"),
         "maxpool_b1": (lambda: w.maxpool_workload(N=1), "hbm"),
         "avgpool_b64": (lambda: w.avgpool_workload(N=64), "hbm"),

@@ -277,3 +277,26 @@ def test_channel_padding_stops_at_ops_that_read_declared_order():
     d = desc_interp.run(p.serialize(), [x, out])
     assert_bit_exact(out, want, "conv -> avg_pool2d")
     assert int(d.ops[0]["Nn"]) == B and int(d.ops[1]["C"]) == B
+
+
+def test_pre_shift_identity_and_emitter_bound():
+    """A shift below 33 with (acc + bias) << (33 - shift) still inside 32 bits equals the shift-33 form the
+    kernels evaluate with a 32-bit multiply-high; the emitter sets pre_shift only under that bound."""
+    rng = np.random.default_rng(9)
+    for shift in range(3, 33):
+        pre = 33 - shift
+        lim = 1 << (31 - pre)
+        t0 = rng.integers(-lim + 1, lim, size=20000, dtype=np.int64)
+        t0[:4] = [-lim + 1, lim - 1, 0, -1]
+        scale = rng.integers(-(1 << 31), 1 << 31, size=t0.size, dtype=np.int64)
+        scale[:4] = [(1 << 31) - 1, -(1 << 31), (1 << 31) - 1, -(1 << 31)]
+        want = [(int(a) * int(b) + (1 << (shift - 1))) >> shift for a, b in zip(t0, scale)]
+        got = [((((int(a) << pre) * int(b)) >> 32) + 1) >> 1 for a, b in zip(t0, scale)]
+        assert want == got, shift
+    # emitter: small-K op with shift 24 gets pre_shift 9; a large bias or a tiny shift gets none
+    wl = w.fully_connected_workload(64, 64, 32, shift=24)
+    assert int(desc_interp.Descriptor(wl.program.serialize()).ops[0]["pre_shift"]) == 9
+    wl = w.fully_connected_workload(64, 4096, 32, shift=24)
+    assert int(desc_interp.Descriptor(wl.program.serialize()).ops[0]["pre_shift"]) == 0
+    wl = w.fully_connected_workload(64, 64, 32, shift=2)
+    assert int(desc_interp.Descriptor(wl.program.serialize()).ops[0]["pre_shift"]) == 0

@@ -90,6 +90,14 @@ def test_stream_igemm(device, monkeypatch):
     monkeypatch.delenv("THIP_IGEMM_DENSE_VARIANT")
     check(device, w.conv2d_workload(N=4, H=56, W=56, C=32, O=144, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True), kernel="igemm_stream_i8")
     check(device, w.fully_connected_workload(8192, 256, 256, realistic=True), kernel="igemm_dense_i8")
+    # few input channels: the streaming kernel gathers one run per window row (also across the image border)
+    for kw in [dict(N=2, H=224, W=224, C=3, O=32, stride=(2, 2), pad=(0, 1, 0, 1), input_zp=-1),
+               dict(N=1, H=70, W=70, C=4, O=48, KH=5, KW=3, stride=(1, 1), pad=(1, 1, 2, 2), input_zp=9),
+               dict(N=3, H=80, W=81, C=2, O=16, KH=7, KW=7, stride=(2, 2), pad=(3, 3, 3, 3), input_zp=-128),
+               dict(N=1, H=75, W=66, C=1, O=64, KH=3, KW=3, stride=(1, 1), pad=(0, 0, 0, 0))]:
+        check(device, w.conv2d_workload(realistic=True, **kw), kernel="igemm_stream_i8")
+    monkeypatch.setenv("THIP_NO_STREAM", "1")
+    check(device, w.conv2d_workload(N=2, H=224, W=224, C=3, O=32, stride=(2, 2), pad=(0, 1, 0, 1), realistic=True, input_zp=-1), kernel="igemm_i8")
 
 
 @pytest.mark.parametrize("shift", [0, 1, 6, 31, 32, 33, 34, 40, 62])
@@ -167,6 +175,21 @@ def test_depthwise_config2a(device, batch):
 @pytest.mark.parametrize("nhwc", [True, False])
 def test_depthwise_geometries(device, kw, nhwc):
     check(device, w.depthwise_workload(nhwc=nhwc, **kw))
+
+
+@pytest.mark.parametrize("tile", ["0", "1"])
+def test_depthwise_3x3_kernels(device, tile, monkeypatch):
+    """Both 3x3 kernels (a register tile of outputs per thread, or one window row of pixels) on images whose
+    sizes are no multiples of the tiles, with and without padding, stride 1 and 2."""
+    monkeypatch.setenv("THIP_DEPTHWISE_TILE", tile)
+    for kw in [dict(N=2, H=13, W=15, C=16, stride=(1, 1), pad=(1, 1, 1, 1)), dict(N=1, H=14, W=14, C=48, stride=(1, 1), pad=(0, 0, 0, 0)),
+               dict(N=1, H=9, W=31, C=32, stride=(1, 1), pad=(1, 1, 1, 1)), dict(N=2, H=21, W=22, C=16, stride=(2, 2), pad=(0, 1, 0, 1)),
+               dict(N=1, H=15, W=13, C=80, stride=(2, 2), pad=(1, 1, 1, 1)), dict(N=1, H=3, W=3, C=16, stride=(1, 1), pad=(0, 0, 0, 0)),
+               dict(N=1, H=56, W=56, C=144, stride=(1, 1), pad=(1, 1, 1, 1), realistic=False),
+               dict(N=1, H=8, W=8, C=16, stride=(2, 2), pad=(1, 1, 1, 1), input_zp=-128),
+               dict(N=3, H=30, W=17, C=96, stride=(1, 1), pad=(1, 1, 1, 1), input_zp=7),
+               dict(N=2, H=112, W=112, C=32, stride=(2, 2), pad=(0, 1, 0, 1), input_zp=-128)]:
+        check(device, w.depthwise_workload(**kw), kernel="depthwise3x3_dot4_i8")
 
 
 @pytest.mark.parametrize("batch", [1, 8])

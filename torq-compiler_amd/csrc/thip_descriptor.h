@@ -105,7 +105,10 @@ struct DescOp {
     int32_t bias0, scale0;
     // transpose: batch, rows, cols
     int32_t TB, TR, TS;
-    int32_t reserved[3];
+    // igemm / depthwise: left shift of (acc + bias) the emitter proved lossless, with shift + pre_shift == 33
+    // (0 = none); lets the kernels requantise with 32-bit arithmetic
+    int32_t pre_shift;
+    int32_t reserved[2];
     DescRef in0;
     DescRef in1;
     DescRef weights;  // packed weights

@@ -160,6 +160,10 @@ static thip_status_t checkOpFootprint(const thip_executable_t *e, uint32_t i) {
     };
     const uint64_t outElem = op.out_dtype == THIP_DTYPE_I32 ? 4 : op.out_dtype == THIP_DTYPE_I16 ? 2 : 1;
     thip_status_t s = THIP_OK;
+    if (op.pre_shift != 0 && (op.pre_shift < 0 || op.shift + op.pre_shift != 33 ||
+                              (op.kind != kKindIgemm && op.kind != kKindDepthwise))) {
+        return fail(THIP_INVALID_ARGUMENT, "op %u: pre_shift %d does not complete shift %d to 33", i, op.pre_shift, op.shift);
+    }
     switch (op.kind) {
     case kKindTranspose: {
         if (!positive({op.TB, op.TR, op.TS})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad transpose extents", i);
@@ -278,7 +282,7 @@ static uint8_t *resolve(const thip_executable_t *e, const DescRef &r, uint8_t *c
 
 static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *bp) {
     const DescOp &op = e->ops[i];
-    const Requant rq{op.shift, op.output_zp, op.output_min, op.output_max};
+    const Requant rq{op.shift, op.output_zp, op.output_min, op.output_max, op.pre_shift};
     hipError_t err = hipSuccess;
     switch (op.kind) {
     case kKindTranspose: {

@@ -341,8 +341,24 @@ class Emitter {
         return THIP_OK;
     }
 
+    // Left shift of (acc + bias) that lifts a shift below 33 to 33 without losing a bit, or 0 when
+    // there is no such shift.  Activations are int8, so |acc| <= 128 * sum |w| per output channel;
+    // with the bias that bounds |acc + bias|, which has to stay below 2^(31 - pre).  The kernels then
+    // requantise with their 32-bit tail; the result is the same number.  THIP_NO_PRE_SHIFT turns it off.
+    int32_t planPreShift(int32_t shift, const std::vector<int64_t> &absWeightSum, DescRef bias) const {
+        if (shift >= 33 || shift < 3 || getenv("THIP_NO_PRE_SHIFT")) return 0;
+        const int32_t pre = 33 - shift;
+        const int32_t *b = (const int32_t *)consts_[bias.index].data();
+        const int64_t limit = (1LL << 31) >> pre;
+        for (size_t n = 0; n < absWeightSum.size(); n++) {
+            const int64_t bound = 128 * absWeightSum[n] + std::llabs((long long)b[n]);
+            if (bound >= limit) return 0;
+        }
+        return pre;
+    }
+
     // Tile choice.  THIP_IGEMM_VARIANT / THIP_IGEMM_DENSE_VARIANT force one (for tuning runs).
-    static uint32_t chooseIgemmVariant(int64_t M, int64_t N, bool dense, int64_t K = 0, int32_t outDtype = 0) {
+    static uint32_t chooseIgemmVariant(int64_t M, int64_t N, bool dense, int64_t K = 0, int32_t outDtype = 0, bool runs = false) {
         auto tiles = [&](uint32_t v) {
             const IgemmTile &t = igemmTile(v);
             return ((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn);
@@ -372,6 +388,8 @@ class Emitter {
             const long v = strtol(env, nullptr, 10);
             if (v >= 0 && v < (long)kIgemmDense256x256) return (uint32_t)v;
         }
+        // window-row runs of a few-channel image, few output channels: the streaming kernel gathers them too
+        if (runs && M >= 4096 && N <= 128 && igemmStreamFits(N, K, outDtype) && !getenv("THIP_NO_STREAM")) return kIgemmStream;
         // Enough 128x128 tiles to give every CU work (and N wide enough to use them); otherwise the small tile.
         if (N > 64 && tiles(kIgemm128x128x64) >= 256) return kIgemm128x128x64;
         return kIgemm64x64x64;
@@ -382,13 +400,19 @@ class Emitter {
     template <typename WeightAt>
     void emitIgemm(DescOp base, int64_t M, int64_t N, int64_t K, uint32_t loader, WeightAt wAt) {
         const bool dense = loader == kLoaderDense;
-        const uint32_t variant = chooseIgemmVariant(M, N, dense, K, base.out_dtype);
+        const uint32_t variant = chooseIgemmVariant(M, N, dense, K, base.out_dtype, loader == kLoaderRuns);
         const IgemmTile &t = igemmTile(variant);
         const int64_t Kp = roundUp(K, t.bk), Np = roundUp(N, t.bn);
         std::vector<int8_t> packed((size_t)(Np * Kp), 0);
+        std::vector<int64_t> absSum((size_t)N, 0);
         for (int64_t n = 0; n < N; n++) {
-            for (int64_t k = 0; k < K; k++) packed[(size_t)(n * Kp + k)] = wAt(n, k);
+            for (int64_t k = 0; k < K; k++) {
+                const int8_t wv = wAt(n, k);
+                packed[(size_t)(n * Kp + k)] = wv;
+                absSum[(size_t)n] += wv < 0 ? -(int64_t)wv : wv;
+            }
         }
+        base.pre_shift = planPreShift(base.shift, absSum, base.bias);
         base.kind = kKindIgemm;
         base.variant = variant;
         base.loader = loader;
@@ -555,8 +579,13 @@ thip_status_t Emitter::emitDepthwise(const thip_hl_depthwise_conv2d_t &c) {
     if (thip_status_t s = splitScaleBias(c.scale_bias, "torq_hl.depthwise_conv2d scale_bias", C, roundUp(Cp, 16), false, &op.bias, &op.scale)) return s;
     const int8_t *wd = (const int8_t *)w->data.data();
     std::vector<int8_t> wpk((size_t)(KH * KW * Cp), 0);
+    std::vector<int64_t> absSum((size_t)C, 0);
     for (int64_t ch = 0; ch < C; ch++) {
-        for (int64_t k = 0; k < KH * KW; k++) wpk[(size_t)(k * Cp + ch)] = wd[ch * KH * KW + k];
+        for (int64_t k = 0; k < KH * KW; k++) {
+            const int8_t wv = wd[ch * KH * KW + k];
+            wpk[(size_t)(k * Cp + ch)] = wv;
+            absSum[(size_t)ch] += wv < 0 ? -(int64_t)wv : wv;
+        }
     }
     op.kind = kKindDepthwise;
     op.out_dtype = init->dtype;
@@ -565,6 +594,7 @@ thip_status_t Emitter::emitDepthwise(const thip_hl_depthwise_conv2d_t &c) {
     op.output_min = c.output_min;
     op.output_max = c.output_max;
     op.shift = c.shift_factor;
+    op.pre_shift = planPreShift(op.shift, absSum, op.bias);
     op.N = (int32_t)d.N; op.H = (int32_t)d.H; op.W = (int32_t)d.W; op.C = (int32_t)Cp;
     op.OH = (int32_t)OH; op.OW = (int32_t)OW; op.OC = (int32_t)Cp;
     op.KH = (int32_t)KH; op.KW = (int32_t)KW; op.SH = (int32_t)c.stride[0]; op.SW = (int32_t)c.stride[1];

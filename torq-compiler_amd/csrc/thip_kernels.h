@@ -15,6 +15,9 @@ struct Requant {
     int32_t out_zp;
     int32_t out_min;
     int32_t out_max;
+    // 0, or 33 - shift for a shift below 33 when (acc + bias) << pre_shift is known to fit 32 bits:
+    // the MFMA and 3x3 depthwise kernels then take their 32-bit tail (the result is the same).
+    int32_t pre_shift;
 };
 
 struct IgemmArgs {
@@ -70,7 +73,7 @@ inline bool igemmStreamFits(int64_t N, int64_t K, int32_t out_dtype) {
     if (out_dtype != 1 || N <= 0 || K <= 0 || N % 16 != 0 || K % 16 != 0 || N > 65536 || K > 65536) return false;
     const int64_t Np = (N + 31) / 32 * 32, Kp = (K + 31) / 32 * 32;
     const int64_t chunk = igemmStreamChunk((int)Np), chunks = (Np + chunk - 1) / chunk;
-    return chunk * Kp + 8 * chunk <= 64 * 1024 && (chunks - 1) * K <= N;
+    return chunk * Kp + 8 * chunk + Kp / 4 <= 64 * 1024 && (chunks - 1) * K <= N;
 }
 hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, hipStream_t stream);
 

@@ -15,6 +15,7 @@
 #include "thip_kernels.h"
 
 #include <algorithm>
+#include <cstdlib>
 #include <type_traits>
 
 #include "thip_descriptor.h"
@@ -45,13 +46,50 @@ __device__ __forceinline__ int32_t requant(int32_t acc, int32_t bias, int32_t sc
 // rounding term 2^(shift-1) is then a multiple of 2^32, so it adds r = 2^(shift-33) to H, and
 // floor((H + r + L / 2^32) / 2^(shift-32)) = (H + r) >> (shift - 32) because L / 2^32 < 1 cannot
 // carry an integer across a multiple of 2^(shift-32).  |H| <= 2^30 and r <= 2^29: no overflow.
-__device__ __forceinline__ int32_t requantWideShift(int32_t acc, int32_t bias, int32_t scale, int32_t rndHigh,
-                                                    int shiftMinus32, int32_t lo, int32_t hi, int32_t zp) {
-    const int32_t t0 = (int32_t)((uint32_t)acc + (uint32_t)bias);
-    int32_t t3 = (__mulhi(t0, scale) + rndHigh) >> shiftMinus32;
-    t3 = t3 < lo ? lo : t3;
-    t3 = t3 > hi ? hi : t3;
-    return (int32_t)((uint32_t)t3 + (uint32_t)zp);
+// A smaller shift gets there through rq.pre_shift = 33 - shift: t0 * 2^pre * scale >> (shift + pre)
+// is the same number, provided t0 * 2^pre still fits 32 bits; whoever fills rq.pre_shift has
+// bounded |t0| from the weights and the bias to make sure of that.
+struct WideRequant {
+    bool on;  // rq.shift + rq.pre_shift >= 33
+    int pre, shiftMinus32;
+    int32_t rnd, lo, hi, zp;
+};
+__device__ __forceinline__ WideRequant wideRequant(const Requant &rq) {
+    WideRequant w;
+    const int sh = rq.shift + rq.pre_shift;
+    w.on = sh >= 33;
+    w.pre = rq.pre_shift;
+    w.shiftMinus32 = sh - 32;
+    w.rnd = w.on ? (int32_t)(1u << (sh - 33)) : 0;
+    const long long lo64 = (long long)rq.out_min - rq.out_zp, hi64 = (long long)rq.out_max - rq.out_zp;
+    w.lo = (int32_t)(lo64 < INT32_MIN ? INT32_MIN : lo64);
+    w.hi = (int32_t)(hi64 > INT32_MAX ? INT32_MAX : hi64);
+    w.zp = rq.out_zp;
+    // ((H + r) >> s) + zp == (H + r + zp * 2^s) >> s: fold the zero point into the rounding term
+    // where that cannot overflow (|H| <= 2^30, r <= 2^29, so |zp| * 2^s up to 2^29 is safe)
+    if (w.on && w.shiftMinus32 <= 13 && rq.out_zp >= -32768 && rq.out_zp <= 32767 && rq.out_min <= rq.out_max) {
+        w.rnd += rq.out_zp * (1 << w.shiftMinus32);  // |out_zp| < 2^15 (checked when the program is built)
+        w.lo = rq.out_min;
+        w.hi = rq.out_max;
+        w.zp = 0;
+    }
+    return w;
+}
+__device__ __forceinline__ int32_t med3(int32_t v, int32_t lo, int32_t hi) {
+    int32_t r;
+    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "v"(lo), "v"(hi));
+    return r;
+}
+__device__ __forceinline__ int32_t requantWideShift(int32_t acc, int32_t bias, int32_t scale, const WideRequant &w) {
+    const int32_t t0 = (int32_t)(((uint32_t)acc + (uint32_t)bias) << w.pre);
+    const int32_t t3 = med3((__mulhi(t0, scale) + w.rnd) >> w.shiftMinus32, w.lo, w.hi);  // lo <= hi
+    return (int32_t)((uint32_t)t3 + (uint32_t)w.zp);
+}
+// Four requantised values (each within int8 after the clamp) as the bytes of one dword.
+__device__ __forceinline__ uint32_t packBytes(int32_t a, int32_t b, int32_t c, int32_t d) {
+    const uint32_t ab = __builtin_amdgcn_perm((uint32_t)b, (uint32_t)a, 0x0c0c0400u);  // [a.0, b.0, 0, 0]
+    const uint32_t cd = __builtin_amdgcn_perm((uint32_t)d, (uint32_t)c, 0x04000c0cu);  // [0, 0, c.0, d.0]
+    return ab | cd;
 }
 
 __device__ __forceinline__ long long roundTerm(int shift) {
@@ -102,11 +140,7 @@ __device__ __forceinline__ void igemmEpilogue(v16i (&acc)[WTN / 32][WTM / 32], i
     const long long rnd = roundTerm(p.rq.shift);
     const int hi4 = (lane >> 5) * 4;
     const bool wide = p.out_dtype == kDtypeI8 && (p.N & 15) == 0 && (((uintptr_t)p.out) & 15) == 0;
-    const bool wideShift = p.rq.shift >= 33;
-    const int shiftMinus32 = p.rq.shift - 32;
-    const int32_t rndHigh = wideShift ? (int32_t)(1u << (p.rq.shift - 33)) : 0;
-    const long long lo64 = (long long)p.rq.out_min - p.rq.out_zp, hi64 = (long long)p.rq.out_max - p.rq.out_zp;
-    const int32_t lo32 = (int32_t)(lo64 < INT32_MIN ? INT32_MIN : lo64), hi32 = (int32_t)(hi64 > INT32_MAX ? INT32_MAX : hi64);
+    const WideRequant wrq = wideRequant(p.rq);
     // One 32-channel column of MFMA tiles at a time goes through the wave's own LDS slice as int32;
     // a compact loop then requantises 16 consecutive channels of one row per lane and stores them
     // as one 128-bit word.  (Kept as a loop: unrolled over the whole tile it outgrows the
@@ -150,7 +184,7 @@ __device__ __forceinline__ void igemmEpilogue(v16i (&acc)[WTN / 32][WTM / 32], i
                     const v4i v = *(const v4i *)(stageOut + row * EROW + (ecol + 4 * c) * 4);
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
-                        q[4 * c + e] = kWideShift ? requantWideShift(v[e], bias[4 * c + e], scale[4 * c + e], rndHigh, shiftMinus32, lo32, hi32, p.rq.out_zp)
+                        q[4 * c + e] = kWideShift ? requantWideShift(v[e], bias[4 * c + e], scale[4 * c + e], wrq)
                                                   : requant(v[e], bias[4 * c + e], scale[4 * c + e], rnd, p.rq);
                     }
                 }
@@ -159,8 +193,7 @@ __device__ __forceinline__ void igemmEpilogue(v16i (&acc)[WTN / 32][WTM / 32], i
                         v4i w;
 #pragma unroll
                         for (int c = 0; c < 4; c++) {
-                            w[c] = (int)((uint32_t)(q[4 * c] & 0xff) | ((uint32_t)(q[4 * c + 1] & 0xff) << 8) |
-                                         ((uint32_t)(q[4 * c + 2] & 0xff) << 16) | ((uint32_t)(q[4 * c + 3] & 0xff) << 24));
+                            w[c] = (int)packBytes(q[4 * c], q[4 * c + 1], q[4 * c + 2], q[4 * c + 3]);
                         }
                         *(v4i *)((int8_t *)p.out + (size_t)m * p.N + nb) = w;
                     } else {
@@ -172,7 +205,7 @@ __device__ __forceinline__ void igemmEpilogue(v16i (&acc)[WTN / 32][WTM / 32], i
                 }
             }
         };
-        if (wideShift) {
+        if (wrq.on) {
             rows(std::true_type{});
         } else {
             rows(std::false_type{});
@@ -245,8 +278,24 @@ __device__ __forceinline__ v4i gatherRun(const int8_t *__restrict__ A, uint32_t 
     const int iy = iy0 + kh;
     const bool rowIn = (unsigned)iy < (unsigned)H;
     const long long off = (long long)base + ((long long)iy * W + ix0) * C;
-    if (rowIn && ix0 >= 0 && ix0 * C + len <= W * C && off + 16 <= aBytes) {
-        return ((const UnalignedV4 *)(A + off))->v;
+    const uint32_t zp4 = zpb * 0x01010101u;
+    if (!rowIn) return v4i{(int)zp4, (int)zp4, (int)zp4, (int)zp4};  // bytes past the run meet zero weights
+    if (off >= 0 && off + 16 <= aBytes) {
+        v4i v = ((const UnalignedV4 *)(A + off))->v;
+        // bytes [lo, hi) of the run lie inside the image row; the others are padding
+        const int lo = ix0 < 0 ? (-ix0 * C < len ? -ix0 * C : len) : 0;
+        const int room = (W - ix0) * C;
+        const int hi = room < len ? (room > 0 ? room : 0) : len;
+        if (lo == 0 && hi == len) return v;
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            const int a = lo - 4 * d, b = hi - 4 * d;
+            const uint32_t below = a <= 0 ? 0u : a >= 4 ? 0xffffffffu : (1u << (8 * a)) - 1u;
+            const uint32_t upto = b <= 0 ? 0u : b >= 4 ? 0xffffffffu : (1u << (8 * b)) - 1u;
+            const uint32_t m = upto & ~below;
+            v[d] = (int)(((uint32_t)v[d] & m) | (zp4 & ~m));
+        }
+        return v;
     }
     // window row touches the padding (or the last bytes of the tensor): byte by byte
     union {
@@ -683,7 +732,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
 constexpr int kStreamRing = 4;
 constexpr size_t kStreamMaxLds = 64 * 1024;
 
-template <int NB>
+template <int NB, int LOADER>
 __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArgs p) {
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
     constexpr int RING = kStreamRing;
@@ -707,30 +756,52 @@ __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArg
         ldsBias[c] = p.bias[n0 + c];
         ldsScale[c] = p.scale[n0 + c];
     }
+    // run loader: the k-table next to them, so that a gather does not wait for a table load from memory
+    uint32_t *ldsTab = (uint32_t *)(ldsScale + chunkN);
+    if (LOADER == kLoaderRuns) {
+        for (int c = tid; c < p.Kp / 16; c += 256) ldsTab[c] = p.ktab[c];
+    }
     __syncthreads();
 
     const int groups = (p.M + 31) / 32, stride = gridDim.x * 4;
     const int kstepsRing = (ksteps + RING - 1) / RING * RING;
-    // 16 bytes of pixel row (32 g + fr) at k-step s; zero past K or past the last group
-    auto fetch = [&](int g, int s) -> v4i {
+    // 16 bytes of pixel row (32 g + fr) at k-step s; zero past K or past the last group.  With the
+    // run loader (few input channels: one 16-byte run per window row) the row is gathered from the
+    // image, at the window position `pos` of the lane's pixel in group g.
+    struct Pos {
+        int iy0, ix0;
+        size_t base;
+    };
+    auto locate = [&](int g) -> Pos {
+        if (LOADER != kLoaderRuns) return Pos{0, 0, 0};
+        int m = g * 32 + fr;
+        m = m < p.M ? m : p.M - 1;
+        const int plane = p.OH * p.OW;
+        const int img = m / plane, rem = m - img * plane;
+        const int oy = rem / p.OW, ox = rem - oy * p.OW;
+        return Pos{oy * p.SH - p.PT, ox * p.SW - p.PL, (size_t)img * p.H * p.W * p.C};
+    };
+    const uint32_t zpb = (uint32_t)(p.input_zp & 0xff);
+    auto fetch = [&](int g, int s, const Pos &pos) -> v4i {
         const int k = s * 32 + half * 16;
         if (g >= groups || k >= p.K) return v4i{0, 0, 0, 0};
+        if (LOADER == kLoaderRuns) {
+            return gatherRun(p.A, ldsTab[k >> 4], pos.iy0, pos.ix0, pos.base, p.H, p.W, p.C, zpb, p.a_bytes);
+        }
         int m = g * 32 + fr;
         m = m < p.M ? m : p.M - 1;
         return *(const v4i *)(p.A + (size_t)m * p.K + k);
     };
-    const bool wideShift = p.rq.shift >= 33;
-    const int shiftMinus32 = p.rq.shift - 32;
-    const int32_t rndHigh = wideShift ? (int32_t)(1u << (p.rq.shift - 33)) : 0;
+    const WideRequant wrq = wideRequant(p.rq);
     const long long rnd = roundTerm(p.rq.shift);
-    const long long lo64 = (long long)p.rq.out_min - p.rq.out_zp, hi64 = (long long)p.rq.out_max - p.rq.out_zp;
-    const int32_t lo32 = (int32_t)(lo64 < INT32_MIN ? INT32_MIN : lo64), hi32 = (int32_t)(hi64 > INT32_MAX ? INT32_MAX : hi64);
 
     int g = blockIdx.x * 4 + wave;
     v4i ring[RING];
+    Pos here = locate(g);
 #pragma unroll
-    for (int d = 0; d < RING; d++) ring[d] = fetch(g, d);
+    for (int d = 0; d < RING; d++) ring[d] = fetch(g, d, here);
     for (; g < groups; g += stride) {
+        const Pos next = locate(g + stride < groups ? g + stride : g);
         v16i acc[NB];
 #pragma unroll
         for (int j = 0; j < NB; j++) {
@@ -744,7 +815,7 @@ __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArg
                 const v4i a = ring[d];
                 // slot d next holds k-step s + RING of this group, or the same slot of the next group
                 const bool wrap = s + RING >= kstepsRing;
-                ring[d] = fetch(wrap ? g + stride : g, wrap ? s + RING - kstepsRing : s + RING);
+                ring[d] = fetch(wrap ? g + stride : g, wrap ? s + RING - kstepsRing : s + RING, wrap ? next : here);
                 if (s < ksteps) {
                     const int8_t *wfrag = smem + ((size_t)(s * nblocks) * 64 + lane) * 16;
 #pragma unroll
@@ -769,14 +840,13 @@ __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArg
                         const int ch = j * 32 + 8 * q + 4 * half;
                         const v4i b4 = *(const v4i *)(ldsBias + ch);
                         const v4i s4 = *(const v4i *)(ldsScale + ch);
-                        uint32_t packed = 0;
+                        int32_t v[4];
 #pragma unroll
                         for (int e = 0; e < 4; e++) {
-                            const int32_t v = kWideShift ? requantWideShift(acc[j][4 * q + e], b4[e], s4[e], rndHigh, shiftMinus32, lo32, hi32, p.rq.out_zp)
-                                                         : requant(acc[j][4 * q + e], b4[e], s4[e], rnd, p.rq);
-                            packed |= (uint32_t)(v & 0xff) << (8 * e);
+                            v[e] = kWideShift ? requantWideShift(acc[j][4 * q + e], b4[e], s4[e], wrq)
+                                              : requant(acc[j][4 * q + e], b4[e], s4[e], rnd, p.rq);
                         }
-                        d4[q] = packed;
+                        d4[q] = packBytes(v[0], v[1], v[2], v[3]);
                     }
                     // lower half lanes: channels 0-3, 8-11, 16-19, 24-27; upper half: 4-7, 12-15, 20-23, 28-31.
                     // Swap (upper of d4[0], lower of d4[2]) and (upper of d4[1], lower of d4[3]):
@@ -789,17 +859,18 @@ __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArg
                 }
             }
         };
-        if (wideShift) {
+        if (wrq.on) {
             finish(std::true_type{});
         } else {
             finish(std::false_type{});
         }
+        here = next;
     }
 }
 
-template <int NB>
+template <int NB, int LOADER>
 static hipError_t launchIgemmStreamT(const IgemmArgs &a, size_t smem, hipStream_t stream) {
-    auto kernel = igemm_stream_i8<NB>;
+    auto kernel = igemm_stream_i8<NB, LOADER>;
     static bool configured = false;
     if (!configured) {
         hipError_t err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kStreamMaxLds);
@@ -819,17 +890,24 @@ static hipError_t launchIgemmStreamT(const IgemmArgs &a, size_t smem, hipStream_
 }
 
 static hipError_t launchIgemmStream(const IgemmArgs &a, hipStream_t stream) {
-    if (a.loader != kLoaderDense || a.out_dtype != kDtypeI8) return hipErrorInvalidValue;
+    if ((a.loader != kLoaderDense && a.loader != kLoaderRuns) || a.out_dtype != kDtypeI8) return hipErrorInvalidValue;
     if (a.N % 16 != 0 || ((uintptr_t)a.out & 15) != 0) return hipErrorInvalidValue;
     const int chunk = igemmStreamChunk(a.Np);
-    const size_t smem = (size_t)chunk * a.Kp + 8 * (size_t)chunk;
+    const size_t smem = (size_t)chunk * a.Kp + 8 * (size_t)chunk + (a.loader == kLoaderRuns ? (size_t)a.Kp / 16 * 4 : 0);
     if (chunk > 256 || smem > kStreamMaxLds) return hipErrorInvalidValue;
     const int nb = chunk / 32;
-    if (nb <= 1) return launchIgemmStreamT<1>(a, smem, stream);
-    if (nb <= 2) return launchIgemmStreamT<2>(a, smem, stream);
-    if (nb <= 4) return launchIgemmStreamT<4>(a, smem, stream);
-    if (nb <= 6) return launchIgemmStreamT<6>(a, smem, stream);
-    return launchIgemmStreamT<8>(a, smem, stream);
+    if (a.loader == kLoaderRuns) {
+        // the first layer of an image network: few output channels
+        if (nb <= 1) return launchIgemmStreamT<1, kLoaderRuns>(a, smem, stream);
+        if (nb <= 2) return launchIgemmStreamT<2, kLoaderRuns>(a, smem, stream);
+        if (nb <= 4) return launchIgemmStreamT<4, kLoaderRuns>(a, smem, stream);
+        return hipErrorInvalidValue;
+    }
+    if (nb <= 1) return launchIgemmStreamT<1, kLoaderDense>(a, smem, stream);
+    if (nb <= 2) return launchIgemmStreamT<2, kLoaderDense>(a, smem, stream);
+    if (nb <= 4) return launchIgemmStreamT<4, kLoaderDense>(a, smem, stream);
+    if (nb <= 6) return launchIgemmStreamT<6, kLoaderDense>(a, smem, stream);
+    return launchIgemmStreamT<8, kLoaderDense>(a, smem, stream);
 }
 
 static const IgemmTile kTiles[kIgemmVariantCount] = {
@@ -931,7 +1009,9 @@ hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, hipStream_t stream)
     } else {
         return hipErrorInvalidValue;
     }
-    if (variant >= kIgemmDense256x256 && a.loader != kLoaderDense) return hipErrorInvalidValue;
+    if (variant >= kIgemmDense256x256 && a.loader != kLoaderDense && !(variant == kIgemmStream && a.loader == kLoaderRuns)) {
+        return hipErrorInvalidValue;
+    }
     if (((uintptr_t)a.Bp & 15) != 0) return hipErrorInvalidValue;
     if (a.out_dtype < kDtypeI8 || a.out_dtype > kDtypeI32) return hipErrorInvalidValue;
     switch (variant) {
@@ -1179,11 +1259,8 @@ __global__ __launch_bounds__(256) void depthwise3x3_dot4_i8(DepthwiseArgs p) {
             }
         }
     }
-    const bool wideShift = p.rq.shift >= 33;
+    const WideRequant wrq = wideRequant(p.rq);
     const long long rnd = roundTerm(p.rq.shift);
-    const int32_t rndHigh = wideShift ? (int32_t)(1u << (p.rq.shift - 33)) : 0;
-    const long long lo64 = (long long)p.rq.out_min - p.rq.out_zp, hi64 = (long long)p.rq.out_max - p.rq.out_zp;
-    const int32_t lo32 = (int32_t)(lo64 < INT32_MIN ? INT32_MIN : lo64), hi32 = (int32_t)(hi64 > INT32_MAX ? INT32_MAX : hi64);
     v4i o[P];
 #pragma unroll
     for (int g = 0; g < 4; g++) {
@@ -1194,7 +1271,7 @@ __global__ __launch_bounds__(256) void depthwise3x3_dot4_i8(DepthwiseArgs p) {
             uint32_t w = 0;
 #pragma unroll
             for (int c = 0; c < 4; c++) {
-                const int32_t r = wideShift ? requantWideShift(acc[q][4 * g + c], b4[c], s4[c], rndHigh, p.rq.shift - 32, lo32, hi32, p.rq.out_zp)
+                const int32_t r = wrq.on ? requantWideShift(acc[q][4 * g + c], b4[c], s4[c], wrq)
                                             : requant(acc[q][4 * g + c], b4[c], s4[c], rnd, p.rq);
                 w |= (uint32_t)(r & 0xff) << (8 * c);
             }
@@ -1211,6 +1288,145 @@ template <int P, int SWT>
 static hipError_t launchDepthwiseDot4(const DepthwiseArgs &a, hipStream_t stream) {
     const long long total = (long long)a.N * a.OH * ((a.OW + P - 1) / P) * (a.C / 16);
     hipLaunchKernelGGL((depthwise3x3_dot4_i8<P, SWT>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a);
+    return hipGetLastError();
+}
+
+// 3x3 depthwise for large images: a thread owns 16 channels of a tile of R x P output pixels
+// (stride S in both directions).  Each input row of the tile is loaded once and serves every
+// output row that overlaps it.  Per group of 4 channels, four adjacent columns of a row (one
+// dword each, a byte per channel) are transposed with 8 byte permutes into one dword per channel
+// holding that channel at the four columns; a v_dot4_i32_i8 with the weights [w0, w1, w2, 0]
+// gives the window row at the block's first column and, for stride 1, with [0, w0, w1, w2] the
+// one at its second column.  That is about one permute and three dot products per output instead
+// of six and three.
+template <int P, int R, int S>
+__global__ __launch_bounds__(256) void depthwise3x3_tile_i8(DepthwiseArgs p) {
+    static_assert(S == 1 || S == 2, "stride 1 or 2");
+    static_assert(S == 2 || P % 2 == 0, "stride 1 pairs the pixels of a block");
+    constexpr int NC = (P - 1) * S + 3, NR = (R - 1) * S + 3;
+    constexpr int NBK = S == 1 ? P / 2 : P;  // blocks of four columns per row; block b starts at column 2 b
+    const int cg = p.C / 16;
+    const int oxGroups = (p.OW + P - 1) / P, oyGroups = (p.OH + R - 1) / R;
+    const long long total = (long long)p.N * oyGroups * oxGroups * cg;
+    const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (t >= total) return;
+    const int c0 = (int)(t % cg) * 16;
+    long long pix = t / cg;
+    const int ox0 = (int)(pix % oxGroups) * P;
+    pix /= oxGroups;
+    const int oy0 = (int)(pix % oyGroups) * R;
+    const int n = (int)(pix / oyGroups);
+    const int iy0 = oy0 * S - p.PT, ix0 = ox0 * S - p.PL;
+    const int8_t *img = p.in + (size_t)n * p.H * p.W * p.C + c0;
+    const int zp4 = (int)((uint32_t)(p.input_zp & 0xff) * 0x01010101u);
+    v4i d[NR][NC];
+    if (iy0 >= 0 && iy0 + NR <= p.H && ix0 >= 0 && ix0 + NC <= p.W) {
+        const int8_t *base = img + ((size_t)iy0 * p.W + ix0) * p.C;
+#pragma unroll
+        for (int i = 0; i < NR; i++) {
+#pragma unroll
+            for (int j = 0; j < NC; j++) d[i][j] = *(const v4i *)(base + ((size_t)i * p.W + j) * p.C);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < NR; i++) {
+            const int iy = iy0 + i;
+            const int iyc = iy < 0 ? 0 : iy >= p.H ? p.H - 1 : iy;
+#pragma unroll
+            for (int j = 0; j < NC; j++) {
+                const int ix = ix0 + j;
+                const int ixc = ix < 0 ? 0 : ix >= p.W ? p.W - 1 : ix;
+                const v4i v = *(const v4i *)(img + ((size_t)iyc * p.W + ixc) * p.C);
+                const bool inside = iy == iyc && ix == ixc;
+                d[i][j] = inside ? v : v4i{zp4, zp4, zp4, zp4};
+            }
+        }
+    }
+    const WideRequant wrq = wideRequant(p.rq);
+    const long long rnd = roundTerm(p.rq.shift);
+    const uint32_t *wrow = (const uint32_t *)p.wpk + c0;
+    v4i o[R][P];
+    auto channels = [&](auto wideShiftTag) {
+        constexpr bool kWideShift = decltype(wideShiftTag)::value;
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            v4i wk[3];
+#pragma unroll
+            for (int kh = 0; kh < 3; kh++) wk[kh] = *(const v4i *)(wrow + (size_t)kh * p.C + 4 * g);
+            int32_t acc[R][P][4];
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+#pragma unroll
+                for (int q = 0; q < P; q++) {
+#pragma unroll
+                    for (int c = 0; c < 4; c++) acc[r][q][c] = 0;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < NR; i++) {
+#pragma unroll
+                for (int b = 0; b < NBK; b++) {
+                    const uint32_t x0 = (uint32_t)d[i][2 * b][g], x1 = (uint32_t)d[i][2 * b + 1][g], x2 = (uint32_t)d[i][2 * b + 2][g];
+                    // the last block of a stride-2 row has no fourth column; its weight is zero
+                    const uint32_t x3 = (uint32_t)d[i][2 * b + 3 < NC ? 2 * b + 3 : 2 * b + 2][g];
+                    // 4 x 4 byte transpose: tr[c] = channel c at columns 2b .. 2b+3
+                    const uint32_t lo01 = __builtin_amdgcn_perm(x1, x0, 0x05010400u), hi01 = __builtin_amdgcn_perm(x1, x0, 0x07030602u);
+                    const uint32_t lo23 = __builtin_amdgcn_perm(x3, x2, 0x05010400u), hi23 = __builtin_amdgcn_perm(x3, x2, 0x07030602u);
+                    const uint32_t tr[4] = {__builtin_amdgcn_perm(lo23, lo01, 0x05040100u), __builtin_amdgcn_perm(lo23, lo01, 0x07060302u),
+                                            __builtin_amdgcn_perm(hi23, hi01, 0x05040100u), __builtin_amdgcn_perm(hi23, hi01, 0x07060302u)};
+#pragma unroll
+                    for (int r = 0; r < R; r++) {
+                        const int kh = i - r * S;
+                        if (kh < 0 || kh > 2) continue;
+#pragma unroll
+                        for (int c = 0; c < 4; c++) {
+                            if (S == 1) {
+                                acc[r][2 * b][c] = __builtin_amdgcn_sdot4((int)tr[c], wk[kh][c], acc[r][2 * b][c], false);
+                                acc[r][2 * b + 1][c] = __builtin_amdgcn_sdot4((int)tr[c], (int)((uint32_t)wk[kh][c] << 8), acc[r][2 * b + 1][c], false);
+                            } else {
+                                acc[r][b][c] = __builtin_amdgcn_sdot4((int)tr[c], wk[kh][c], acc[r][b][c], false);
+                            }
+                        }
+                    }
+                }
+            }
+            const v4i b4 = *(const v4i *)(p.bias + c0 + 4 * g);
+            const v4i s4 = *(const v4i *)(p.scale + c0 + 4 * g);
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+#pragma unroll
+                for (int q = 0; q < P; q++) {
+                    int32_t v[4];
+#pragma unroll
+                    for (int c = 0; c < 4; c++) {
+                        v[c] = kWideShift ? requantWideShift(acc[r][q][c], b4[c], s4[c], wrq)
+                                          : requant(acc[r][q][c], b4[c], s4[c], rnd, p.rq);
+                    }
+                    o[r][q][g] = (int)packBytes(v[0], v[1], v[2], v[3]);
+                }
+            }
+        }
+    };
+    if (wrq.on) {
+        channels(std::true_type{});
+    } else {
+        channels(std::false_type{});
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+#pragma unroll
+        for (int q = 0; q < P; q++) {
+            if (oy0 + r < p.OH && ox0 + q < p.OW) {
+                *(v4i *)(p.out + (((size_t)n * p.OH + oy0 + r) * p.OW + ox0 + q) * p.C + c0) = o[r][q];
+            }
+        }
+    }
+}
+
+template <int P, int R, int S>
+static hipError_t launchDepthwiseTile(const DepthwiseArgs &a, hipStream_t stream) {
+    const long long total = (long long)a.N * ((a.OH + R - 1) / R) * ((a.OW + P - 1) / P) * (a.C / 16);
+    hipLaunchKernelGGL((depthwise3x3_tile_i8<P, R, S>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a);
     return hipGetLastError();
 }
 
@@ -1252,6 +1468,13 @@ hipError_t launchDepthwise(const DepthwiseArgs &a, hipStream_t stream) {
         if (a.KH != 3 || a.KW != 3 || a.C % 16 != 0 || (bits & 15) != 0) return hipErrorInvalidValue;
         // several pixels per thread once there is enough work to still fill the chip
         const long long outputs = (long long)a.N * a.OH * a.OW * (a.C / 16);
+        // a register tile of outputs per thread where that still leaves every CU several blocks
+        // (THIP_DEPTHWISE_TILE=0 / 1 switches that kernel off / on for every size, for tests and tuning)
+        const char *tileEnv = getenv("THIP_DEPTHWISE_TILE");
+        const bool tileOff = tileEnv && tileEnv[0] == '0', tileOn = tileEnv && tileEnv[0] == '1';
+        if (!tileOff) {
+            if (a.SW == 1 && a.SH == 1 && (tileOn || outputs >= 8 * 4 * 65536)) return launchDepthwiseTile<4, 2, 1>(a, stream);
+        }
         if (a.SW == 1 && outputs >= 4 * 65536) return launchDepthwiseDot4<4, 1>(a, stream);
         if (a.SW == 2 && outputs >= 4 * 65536) return launchDepthwiseDot4<4, 2>(a, stream);
         if (a.SW == 1 && outputs >= 2 * 65536) return launchDepthwiseDot4<2, 1>(a, stream);
