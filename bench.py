@@ -82,14 +82,29 @@ class Loaded:
             self.dev.free(p)
 
 
-def roofline(wl, bound, ms):
+# HBM bytes per launch of each workload's kernel, from rocprofv3 counters: FETCH_SIZE * 1.9993 + WRITE_SIZE * 1.0
+# (KiB per dispatch; the factors are what the same counters read for a plain 256 MiB copy, --copy-calibration).
+MEASURED_TRAFFIC = {
+    "fc_4096x4096x4096": (49396.2 * 1.9993 + 16569.0) * 1024,
+    "fc_512x4096x4096": (16452.6 * 1.9993 + 2048.0) * 1024,
+    "fc_16x2048x8192": (8553.6 * 1.9993 + 512.0) * 1024,
+    "conv_112x112x32_o64_3x3": (359.4 * 1.9993 + 784.0) * 1024,
+    "depthwise_b64": (17042.9 * 1.9993 + 7105.0) * 1024,
+    "avgpool_b64": (1991.6 * 1.9993 + 80.0) * 1024,
+    "add_b64": (4727.1 * 1.9993 + 4704.0) * 1024,
+}
+
+
+def roofline(wl, bound, ms, name=None):
+    traffic = MEASURED_TRAFFIC.get(name)
+    traffic = None if traffic is None else int(round(traffic))
     if bound == "mfma":
         achieved = wl.ops / (ms * 1e-3) / 1e12
         return {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
-                "frac": round(achieved / PEAK_INT8_TOPS, 5), "traffic": None}
+                "frac": round(achieved / PEAK_INT8_TOPS, 5), "traffic": traffic}
     achieved = wl.bytes / (ms * 1e-3) / 1e9
     return {"bound": "hbm", "achieved": round(achieved, 2), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-            "frac": round(achieved / PEAK_HBM_GBS, 5), "traffic": None}
+            "frac": round(achieved / PEAK_HBM_GBS, 5), "traffic": traffic}
 
 
 def verify_sample(loaded):
@@ -147,6 +162,8 @@ def main():
     ap.add_argument("--workload", default="fc_4096x4096x4096")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-others", action="store_true", help="skip the brief per-op measurements")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy (a 1x1 max pool), to scale rocprofv3's FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -174,6 +191,20 @@ def main():
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
     ok = verify_sample(loaded)
     loaded.close()
+    if args.copy_calibration:
+        # a 1x1 stride-1 max pool over the whole int8 range is a plain copy: 256 MiB read, 256 MiB written
+        prog = pkg.Program()
+        shape = (1, 4096, 4096, 16)
+        src = prog.binding(0, shape)
+        prog.maxpool2d(src, input_zp=-128, output_min=-128, output_max=127, stride=(1, 1), pad=(0, 0, 0, 0), kernel=(1, 1),
+                       init=prog.binding(1, shape), nhwc_input=True)
+        exe = pkg.Executable(dev, prog.serialize())
+        host = np.zeros(shape, dtype=np.int8)
+        ptrs = [dev.upload(host), dev.upload(host)]
+        exe.time_device(ptrs, [host.nbytes, host.nbytes], 3)
+        exe.close()
+        for ptr in ptrs:
+            dev.free(ptr)
 
     per_op = {}
     if not args.no_others:
@@ -220,7 +251,7 @@ def main():
         "data": "synthetic",
         "config": {"workload": args.workload, "kernels": kernels, "parity_checked": ok,
                    "algorithmic_ops": wl.ops, "algorithmic_bytes": wl.bytes},
-        "roofline": dict(roofline(wl, bound, ev_ms), kernel=kernels[0], kernel_ms=round(ev_ms, 5)),
+        "roofline": dict(roofline(wl, bound, ev_ms, args.workload), kernel=kernels[0], kernel_ms=round(ev_ms, 5)),
     }
     if not args.no_cpu and args.workload.startswith("fc_"):
         result["cpu_baseline"] = cpu_baseline(wl)

@@ -76,6 +76,15 @@ def test_dense_igemm_every_tile_variant(device, variant, monkeypatch):
     check(device, w.conv2d_workload(N=2, H=28, W=28, C=192, O=32, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True))
 
 
+@pytest.mark.parametrize("variant", [4, 7, 9])
+def test_dense_igemm_staged_epilogue(device, variant, monkeypatch):
+    """The LDS-staged epilogue with the 32-bit requant tail (the in-register one normally takes these shapes)."""
+    monkeypatch.setenv("THIP_IGEMM_DENSE_VARIANT", str(variant))
+    monkeypatch.setenv("THIP_NO_DIRECT_EPILOGUE", "1")
+    check(device, w.fully_connected_workload(300, 192, 528, realistic=True), kernel="igemm_dense_i8")
+    check(device, w.fully_connected_workload(257, 80, 48, realistic=True), kernel="igemm_dense_i8")
+
+
 def test_stream_igemm(device, monkeypatch):
     """The pixel-streaming kernel (weights resident in LDS): every accumulator width, ragged M, k-step
     counts around the prefetch ring, N ending in half a 32-channel block, both requant tails."""

@@ -214,6 +214,53 @@ __device__ __forceinline__ void igemmEpilogue(v16i (&acc)[WTN / 32][WTM / 32], i
     }
 }
 
+// The same epilogue without the LDS round trip, for int8 outputs with N % 16 == 0 and the 32-bit
+// requant tail: each accumulator tile is requantised in place, two v_permlane32_swap exchange
+// register groups between the wave halves so that a lane owns 16 consecutive channels of its row
+// (see igemm_stream_i8), and the lane stores them as one 128-bit word.  Only the (bias, scale)
+// vectors pass through LDS.
+template <int WTM, int WTN, int NW, int BN>
+__device__ __forceinline__ void igemmEpilogueDirect(v16i (&acc)[WTN / 32][WTM / 32], int8_t *smem, const IgemmArgs &p, int m0,
+                                                    int n0, int wm, int wn, int32_t myBias, int32_t myScale) {
+    blockBarrier();
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    const int tid = threadIdx.x, lane = tid & 63, fr = lane & 31, half = lane >> 5;
+    int32_t *ldsBias = (int32_t *)smem, *ldsScale = ldsBias + BN;
+    if (tid < BN) {
+        ldsBias[tid] = myBias;
+        ldsScale[tid] = myScale;
+    }
+    __syncthreads();
+    const WideRequant wrq = wideRequant(p.rq);
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const int nl = wn * WTN + j * 32;  // first channel of this tile column, relative to n0
+        v4i b4[4], s4[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            b4[q] = *(const v4i *)(ldsBias + nl + 8 * q + 4 * half);
+            s4[q] = *(const v4i *)(ldsScale + nl + 8 * q + 4 * half);
+        }
+        const int n = n0 + nl + 16 * half;
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            uint32_t d4[4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                int32_t v[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) v[e] = requantWideShift(acc[j][i][4 * q + e], b4[q][e], s4[q][e], wrq);
+                d4[q] = packBytes(v[0], v[1], v[2], v[3]);
+            }
+            const auto s02 = __builtin_amdgcn_permlane32_swap(d4[0], d4[2], false, false);
+            const auto s13 = __builtin_amdgcn_permlane32_swap(d4[1], d4[3], false, false);
+            const v4i outv = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
+            const int m = m0 + wm * WTM + i * 32 + fr;
+            if (m < p.M && n < p.N) *(v4i *)((int8_t *)p.out + (size_t)m * p.N + n) = outv;
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------
 // igemm_i8
 // ---------------------------------------------------------------------------
@@ -516,7 +563,9 @@ __device__ __forceinline__ void waitVmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU>
+// DIRECT selects the epilogue: in registers (int8 output, N % 16 == 0, 32-bit requant tail: the launcher
+// checks) or staged through LDS (everything else).
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, bool DIRECT>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_dense_i8(IgemmArgs p) {
     constexpr int BK = 64;
     constexpr int NW = WAVES_M * WAVES_N;
@@ -712,7 +761,11 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
     for (; kt + STAGES < KT - 1; kt++) step(kt, std::true_type{});
     for (; kt < KT; kt++) step(kt, std::false_type{});
 
-    igemmEpilogue<WTM, WTN, NW, BN>(acc, smem, p, m0, n0, wm, wn, myBias, myScale);
+    if (DIRECT) {
+        igemmEpilogueDirect<WTM, WTN, NW, BN>(acc, smem, p, m0, n0, wm, wn, myBias, myScale);
+    } else {
+        igemmEpilogue<WTM, WTN, NW, BN>(acc, smem, p, m0, n0, wm, wn, myBias, myScale);
+    }
 }
 
 
@@ -968,14 +1021,14 @@ static hipError_t launchIgemmLoader(const IgemmArgs &a, hipStream_t stream) {
     }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU>
-static hipError_t launchIgemmDense(const IgemmArgs &a, hipStream_t stream) {
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, bool DIRECT>
+static hipError_t launchIgemmDenseE(const IgemmArgs &a, hipStream_t stream) {
     // the stage ring, reused by the epilogue as staging slices (one per wave) plus bias/scale
     constexpr size_t ring = (size_t)STAGES * (BM + BN) * 64;
     constexpr size_t epilogue = (size_t)(BM / WAVES_M) * (WAVES_M * WAVES_N) * (32 * 4 + 16) + 2 * BN * 4;
     constexpr size_t smem = ring > epilogue ? ring : epilogue;
     static_assert(smem * BLOCKS_PER_CU <= 160 * 1024, "LDS of one CU");
-    auto kernel = igemm_dense_i8<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU>;
+    auto kernel = igemm_dense_i8<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, DIRECT>;
     static bool configured = false;
     if (!configured) {
         hipError_t err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -986,6 +1039,14 @@ static hipError_t launchIgemmDense(const IgemmArgs &a, hipStream_t stream) {
     const int tilesN = a.Np / BN;
     hipLaunchKernelGGL(kernel, dim3((unsigned)(tilesM * tilesN)), dim3(WAVES_M * WAVES_N * 64), smem, stream, a);
     return hipGetLastError();
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU>
+static hipError_t launchIgemmDense(const IgemmArgs &a, hipStream_t stream) {
+    const bool direct = a.out_dtype == kDtypeI8 && a.N % 16 == 0 && ((uintptr_t)a.out & 15) == 0 &&
+                        a.rq.shift + a.rq.pre_shift >= 33 && !getenv("THIP_NO_DIRECT_EPILOGUE");
+    return direct ? launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, true>(a, stream)
+                  : launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, false>(a, stream);
 }
 
 hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, hipStream_t stream) {
@@ -1475,10 +1536,13 @@ hipError_t launchDepthwise(const DepthwiseArgs &a, hipStream_t stream) {
         if (!tileOff) {
             if (a.SW == 1 && a.SH == 1 && (tileOn || outputs >= 8 * 4 * 65536)) return launchDepthwiseTile<4, 2, 1>(a, stream);
         }
-        if (a.SW == 1 && outputs >= 4 * 65536) return launchDepthwiseDot4<4, 1>(a, stream);
-        if (a.SW == 2 && outputs >= 4 * 65536) return launchDepthwiseDot4<4, 2>(a, stream);
-        if (a.SW == 1 && outputs >= 2 * 65536) return launchDepthwiseDot4<2, 1>(a, stream);
-        if (a.SW == 2 && outputs >= 2 * 65536) return launchDepthwiseDot4<2, 2>(a, stream);
+        // pixels per thread (THIP_DEPTHWISE_P forces 1, 2 or 4, for tuning)
+        int pix = outputs >= 4 * 65536 ? 4 : outputs >= 2 * 65536 ? 2 : 1;
+        if (const char *env = getenv("THIP_DEPTHWISE_P")) pix = atoi(env);
+        if (a.SW == 1 && pix == 4) return launchDepthwiseDot4<4, 1>(a, stream);
+        if (a.SW == 2 && pix == 4) return launchDepthwiseDot4<4, 2>(a, stream);
+        if (a.SW == 1 && pix == 2) return launchDepthwiseDot4<2, 1>(a, stream);
+        if (a.SW == 2 && pix == 2) return launchDepthwiseDot4<2, 2>(a, stream);
         return launchDepthwiseDot4<1, 0>(a, stream);
     }
     if (a.variant != kDepthwiseGeneric) return hipErrorInvalidValue;
