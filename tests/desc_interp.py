@@ -16,7 +16,7 @@ HEADER = np.dtype([("magic", "<u4"), ("version", "<u4"), ("arch", "<u4"), ("flag
                    ("consts_offset", "<u8"), ("data_offset", "<u8"), ("total_size", "<u8")])
 _I32 = ["out_dtype", "input_zp", "output_zp", "output_min", "output_max", "shift",
         "N", "H", "W", "C", "OH", "OW", "OC", "KH", "KW", "SH", "SW", "PL", "PR", "PT", "PB",
-        "M", "K", "Kp", "Nn", "Np", "w0", "w1", "bias0", "scale0", "TB", "TR", "TS", "pre_shift", "r1", "r2"]
+        "M", "K", "Kp", "Nn", "Np", "w0", "w1", "bias0", "scale0", "TB", "TR", "TS", "pre_shift", "t0_clamp", "r2"]
 OP = np.dtype([("kind", "<u4"), ("variant", "<u4"), ("loader", "<u4"), ("gran", "<u4")] +
               [(n, "<i4") for n in _I32] +
               [(n, REF) for n in ["in0", "in1", "weights", "bias", "scale", "table", "out"]])
@@ -45,9 +45,12 @@ class Descriptor:
         return self.blob[start:start + int(c["size"])]
 
 
-def _requant_vec(acc, bias, scale, shift, zp, mn, mx, pre=0):
+def _requant_vec(acc, bias, scale, shift, zp, mn, mx, pre=0, t0_clamp=0):
     t0 = (acc.astype(np.int64) + bias.astype(np.int64))
     t0 = ((t0 + (1 << 31)) % (1 << 32)) - (1 << 31)  # int32 wrap
+    if t0_clamp:
+        assert pre and t0_clamp < (1 << (31 - pre))
+        t0 = np.clip(t0, -t0_clamp, t0_clamp)
     if pre:
         # the kernels' 32-bit tail: (mulhi(t0 << pre, scale) + 1) >> 1, valid only if the shift loses no bit
         assert shift + pre == 33 and np.all(np.abs(t0) < (1 << (31 - pre))), "pre_shift overflows acc + bias"
@@ -133,7 +136,7 @@ def run(blob, binding_arrays):
                     A[..., e * g:(e + 1) * g] = vals
                 A = A.reshape(M, Kp)
             acc = A @ Wp.T  # M x Np
-            q = _requant_vec(acc[:, :N], bias[None, :N], scale[None, :N], sh, zp, mn, mx, int(op["pre_shift"]))
+            q = _requant_vec(acc[:, :N], bias[None, :N], scale[None, :N], sh, zp, mn, mx, int(op["pre_shift"]), int(op["t0_clamp"]))
             odt = OUT_NP[int(op["out_dtype"])]
             out = view(op["out"], M * N * np.dtype(odt).itemsize).view(odt)
             out[:] = q.astype(odt).reshape(-1)
@@ -156,7 +159,7 @@ def run(blob, binding_arrays):
                                        pad=[int(op["PL"]), int(op["PR"]), int(op["PT"]), int(op["PB"])],
                                        stride=[int(op["SH"]), int(op["SW"])], layout=orc.NHWC)
             assert res.shape == (Nimg, OH, OW, C)
-            if int(op["pre_shift"]):
+            if int(op["pre_shift"]) and not int(op["t0_clamp"]):
                 bound = 128 * np.abs(wpk.astype(np.int64)).sum(axis=(0, 1)) + np.abs(sb[0::2].astype(np.int64))
                 assert sh + int(op["pre_shift"]) == 33 and np.all(bound < (1 << (31 - int(op["pre_shift"]))))
             view(op["out"], res.size)[:] = res.reshape(-1).view(np.uint8)

@@ -296,7 +296,40 @@ def test_pre_shift_identity_and_emitter_bound():
     # emitter: small-K op with shift 24 gets pre_shift 9; a large bias or a tiny shift gets none
     wl = w.fully_connected_workload(64, 64, 32, shift=24)
     assert int(desc_interp.Descriptor(wl.program.serialize()).ops[0]["pre_shift"]) == 9
+    # K too large for the bound: acc + bias is clamped instead, to a range where every channel is saturated
     wl = w.fully_connected_workload(64, 4096, 32, shift=24)
-    assert int(desc_interp.Descriptor(wl.program.serialize()).ops[0]["pre_shift"]) == 0
+    op = desc_interp.Descriptor(wl.program.serialize()).ops[0]
+    assert int(op["pre_shift"]) == 9 and int(op["t0_clamp"]) == (1 << 22) - 1
+    out = np.zeros(wl.outputs[0][0], dtype=wl.outputs[0][1])
+    desc_interp.run(wl.program.serialize(), list(wl.inputs) + [out])
+    assert_bit_exact(out, oracle_eval(wl)[0], "clamped pre-shift")
     wl = w.fully_connected_workload(64, 64, 32, shift=2)
     assert int(desc_interp.Descriptor(wl.program.serialize()).ops[0]["pre_shift"]) == 0
+
+
+@pytest.mark.parametrize("shift,scale_bits", [(10, 14), (10, 9), (6, 31), (20, 22), (3, 4), (32, 30)])
+def test_t0_clamp_keeps_results(shift, scale_bits):
+    """Small shifts with scales of either sign (and zero): where the emitter clamps acc + bias the 32-bit tail
+    still gives the oracle's bytes, in range and saturated; where a channel would not be saturated it must not clamp."""
+    rng = np.random.default_rng(shift * 100 + scale_bits)
+    M, K, N = 40, 256, 48
+    x = rng.integers(-128, 128, size=(M, K)).astype(np.int8)
+    wt = rng.integers(-127, 128, size=(N, K)).astype(np.int8)
+    wt[:, K // 2:] = 0
+    wt[::3] = rng.integers(-2, 3, size=wt[::3].shape)  # some channels with small accumulators: unsaturated results
+    sb = np.zeros(2 * N, dtype=np.int32)
+    sb[0::2] = rng.integers(-3000, 3000, size=N)
+    lim = (1 << scale_bits) - 1
+    sb[1::2] = rng.integers(-lim, lim, size=N, endpoint=True)
+    sb[1] = 0
+    p = Program()
+    out_b = p.binding(1, (M, N))
+    p.fully_connected(p.binding(0, (M, K)), wt, sb, init=out_b, output_zp=-5, output_min=-128, output_max=127, shift_factor=shift)
+    want = orc.fully_connected(x, wt, sb, output_zp=-5, output_min=-128, output_max=127, shift_factor=shift)
+    out = np.zeros((M, N), dtype=np.int8)
+    d = desc_interp.run(p.serialize(), [x, out])
+    assert_bit_exact(out, want, "fc shift %d" % shift)
+    op = d.ops[0]
+    if int(op["t0_clamp"]):
+        assert int(op["pre_shift"]) == 33 - shift
+    assert scale_bits > 24 or len(np.unique(want)) > 3  # not everything saturated

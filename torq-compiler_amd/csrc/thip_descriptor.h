@@ -108,7 +108,11 @@ struct DescOp {
     // igemm / depthwise: left shift of (acc + bias) the emitter proved lossless, with shift + pre_shift == 33
     // (0 = none); lets the kernels requantise with 32-bit arithmetic
     int32_t pre_shift;
-    int32_t reserved[2];
+    // with pre_shift: clamp (acc + bias) to [-t0_clamp, t0_clamp] first (0 = no clamp).  The emitter sets it
+    // when the bound of |acc + bias| is too large for pre_shift but every channel's result already saturates
+    // at +-t0_clamp, so the clamp cannot change a result.
+    int32_t t0_clamp;
+    int32_t reserved[1];
     DescRef in0;
     DescRef in1;
     DescRef weights;  // packed weights

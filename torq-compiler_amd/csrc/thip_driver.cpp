@@ -164,6 +164,9 @@ static thip_status_t checkOpFootprint(const thip_executable_t *e, uint32_t i) {
                               (op.kind != kKindIgemm && op.kind != kKindDepthwise))) {
         return fail(THIP_INVALID_ARGUMENT, "op %u: pre_shift %d does not complete shift %d to 33", i, op.pre_shift, op.shift);
     }
+    if (op.t0_clamp != 0 && (op.t0_clamp < 0 || op.pre_shift <= 0 || op.pre_shift > 30 || op.t0_clamp >= (1 << (31 - op.pre_shift)))) {
+        return fail(THIP_INVALID_ARGUMENT, "op %u: t0_clamp %d does not fit pre_shift %d", i, op.t0_clamp, op.pre_shift);
+    }
     switch (op.kind) {
     case kKindTranspose: {
         if (!positive({op.TB, op.TR, op.TS})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad transpose extents", i);
@@ -282,7 +285,7 @@ static uint8_t *resolve(const thip_executable_t *e, const DescRef &r, uint8_t *c
 
 static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *bp) {
     const DescOp &op = e->ops[i];
-    const Requant rq{op.shift, op.output_zp, op.output_min, op.output_max, op.pre_shift};
+    const Requant rq{op.shift, op.output_zp, op.output_min, op.output_max, op.pre_shift, op.t0_clamp};
     hipError_t err = hipSuccess;
     switch (op.kind) {
     case kKindTranspose: {

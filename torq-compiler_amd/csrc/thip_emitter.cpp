@@ -343,18 +343,39 @@ class Emitter {
 
     // Left shift of (acc + bias) that lifts a shift below 33 to 33 without losing a bit, or 0 when
     // there is no such shift.  Activations are int8, so |acc| <= 128 * sum |w| per output channel;
-    // with the bias that bounds |acc + bias|, which has to stay below 2^(31 - pre).  The kernels then
-    // requantise with their 32-bit tail; the result is the same number.  THIP_NO_PRE_SHIFT turns it off.
-    int32_t planPreShift(int32_t shift, const std::vector<int64_t> &absWeightSum, DescRef bias) const {
-        if (shift >= 33 || shift < 3 || getenv("THIP_NO_PRE_SHIFT")) return 0;
+    // with the bias that bounds |acc + bias|, which has to stay below 2^(31 - pre).  If the bound is
+    // too large, (acc + bias) may still be clamped to +-(2^(31 - pre) - 1) first, provided every
+    // channel's result at those two values already lies at or beyond the output clamp: the result is
+    // monotonic in acc + bias, so the clamp then changes nothing.  The kernels requantise such ops with
+    // their 32-bit tail; the result is the same number.  THIP_NO_PRE_SHIFT turns it off.
+    void planPreShift(DescOp *op, const std::vector<int64_t> &absWeightSum) const {
+        op->pre_shift = 0;
+        op->t0_clamp = 0;
+        const int32_t shift = op->shift;
+        if (shift >= 33 || shift < 3 || getenv("THIP_NO_PRE_SHIFT")) return;
         const int32_t pre = 33 - shift;
-        const int32_t *b = (const int32_t *)consts_[bias.index].data();
+        const int32_t *b = (const int32_t *)consts_[op->bias.index].data();
+        const int32_t *sc = (const int32_t *)consts_[op->scale.index].data();
         const int64_t limit = (1LL << 31) >> pre;
-        for (size_t n = 0; n < absWeightSum.size(); n++) {
-            const int64_t bound = 128 * absWeightSum[n] + std::llabs((long long)b[n]);
-            if (bound >= limit) return 0;
+        bool fits = true;
+        for (size_t n = 0; n < absWeightSum.size() && fits; n++) {
+            fits = 128 * absWeightSum[n] + std::llabs((long long)b[n]) < limit;
         }
-        return pre;
+        if (fits) {
+            op->pre_shift = pre;
+            return;
+        }
+        const int64_t bound = limit - 1;
+        const int64_t lo = (int64_t)op->output_min - op->output_zp, hi = (int64_t)op->output_max - op->output_zp;
+        auto result = [&](int64_t t0, int64_t scale) { return (t0 * scale + (1LL << (shift - 1))) >> shift; };
+        for (size_t n = 0; n < absWeightSum.size(); n++) {
+            const int64_t scale = sc[n];
+            if (scale == 0) continue;  // the result does not depend on acc + bias
+            const int64_t top = result(scale > 0 ? bound : -bound, scale), bottom = result(scale > 0 ? -bound : bound, scale);
+            if (top < hi || bottom > lo) return;
+        }
+        op->pre_shift = pre;
+        op->t0_clamp = (int32_t)bound;
     }
 
     // Tile choice.  THIP_IGEMM_VARIANT / THIP_IGEMM_DENSE_VARIANT force one (for tuning runs).
@@ -412,7 +433,7 @@ class Emitter {
                 absSum[(size_t)n] += wv < 0 ? -(int64_t)wv : wv;
             }
         }
-        base.pre_shift = planPreShift(base.shift, absSum, base.bias);
+        planPreShift(&base, absSum);
         base.kind = kKindIgemm;
         base.variant = variant;
         base.loader = loader;
@@ -594,7 +615,7 @@ thip_status_t Emitter::emitDepthwise(const thip_hl_depthwise_conv2d_t &c) {
     op.output_min = c.output_min;
     op.output_max = c.output_max;
     op.shift = c.shift_factor;
-    op.pre_shift = planPreShift(op.shift, absSum, op.bias);
+    planPreShift(&op, absSum);
     op.N = (int32_t)d.N; op.H = (int32_t)d.H; op.W = (int32_t)d.W; op.C = (int32_t)Cp;
     op.OH = (int32_t)OH; op.OW = (int32_t)OW; op.OC = (int32_t)Cp;
     op.KH = (int32_t)KH; op.KW = (int32_t)KW; op.SH = (int32_t)c.stride[0]; op.SW = (int32_t)c.stride[1];

@@ -18,6 +18,9 @@ struct Requant {
     // 0, or 33 - shift for a shift below 33 when (acc + bias) << pre_shift is known to fit 32 bits:
     // the MFMA and 3x3 depthwise kernels then take their 32-bit tail (the result is the same).
     int32_t pre_shift;
+    // > 0 with pre_shift: (acc + bias) is clamped to [-t0_clamp, t0_clamp] before the shift; whoever sets it has
+    // checked that every channel's result is already saturated at those values
+    int32_t t0_clamp;
 };
 
 struct IgemmArgs {

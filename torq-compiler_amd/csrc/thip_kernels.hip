@@ -48,11 +48,14 @@ __device__ __forceinline__ int32_t requant(int32_t acc, int32_t bias, int32_t sc
 // carry an integer across a multiple of 2^(shift-32).  |H| <= 2^30 and r <= 2^29: no overflow.
 // A smaller shift gets there through rq.pre_shift = 33 - shift: t0 * 2^pre * scale >> (shift + pre)
 // is the same number, provided t0 * 2^pre still fits 32 bits; whoever fills rq.pre_shift has
-// bounded |t0| from the weights and the bias to make sure of that.
+// bounded |t0| from the weights and the bias to make sure of that, or passes rq.t0_clamp: t0 is
+// then clamped to a range that fits, chosen so wide that every result outside it is saturated by
+// the output clamp anyway (the result is monotonic in t0).
 struct WideRequant {
     bool on;  // rq.shift + rq.pre_shift >= 33
     int pre, shiftMinus32;
     int32_t rnd, lo, hi, zp;
+    int32_t t0lo, t0hi;  // clamp of acc + bias (the whole int32 range when rq.t0_clamp == 0)
 };
 __device__ __forceinline__ WideRequant wideRequant(const Requant &rq) {
     WideRequant w;
@@ -65,6 +68,8 @@ __device__ __forceinline__ WideRequant wideRequant(const Requant &rq) {
     w.lo = (int32_t)(lo64 < INT32_MIN ? INT32_MIN : lo64);
     w.hi = (int32_t)(hi64 > INT32_MAX ? INT32_MAX : hi64);
     w.zp = rq.out_zp;
+    w.t0lo = rq.t0_clamp > 0 ? -rq.t0_clamp : INT32_MIN;
+    w.t0hi = rq.t0_clamp > 0 ? rq.t0_clamp : INT32_MAX;
     // ((H + r) >> s) + zp == (H + r + zp * 2^s) >> s: fold the zero point into the rounding term
     // where that cannot overflow (|H| <= 2^30, r <= 2^29, so |zp| * 2^s up to 2^29 is safe)
     if (w.on && w.shiftMinus32 <= 13 && rq.out_zp >= -32768 && rq.out_zp <= 32767 && rq.out_min <= rq.out_max) {
@@ -81,7 +86,7 @@ __device__ __forceinline__ int32_t med3(int32_t v, int32_t lo, int32_t hi) {
     return r;
 }
 __device__ __forceinline__ int32_t requantWideShift(int32_t acc, int32_t bias, int32_t scale, const WideRequant &w) {
-    const int32_t t0 = (int32_t)(((uint32_t)acc + (uint32_t)bias) << w.pre);
+    const int32_t t0 = (int32_t)((uint32_t)med3((int32_t)((uint32_t)acc + (uint32_t)bias), w.t0lo, w.t0hi) << w.pre);
     const int32_t t3 = med3((__mulhi(t0, scale) + w.rnd) >> w.shiftMinus32, w.lo, w.hi);  // lo <= hi
     return (int32_t)((uint32_t)t3 + (uint32_t)w.zp);
 }
