@@ -165,6 +165,16 @@ def test_fully_connected_geometries(device, mkn):
     check(device, w.fully_connected_workload(*mkn, realistic=True))
 
 
+@pytest.mark.parametrize("dot4", [False, True])
+def test_fully_connected_skinny_kernels(device, dot4, monkeypatch):
+    """At most 16 rows: the MFMA kernel (3 rows and up) and the dot-product kernel, K and N with ragged ends."""
+    if dot4:
+        monkeypatch.setenv("THIP_SKINNY_DOT4", "1")
+    for mkn in [(3, 16, 16), (5, 48, 20), (16, 272, 1000), (9, 1040, 37), (4, 256, 64), (2, 512, 32), (16, 2048, 8192), (7, 4096, 130)]:
+        check(device, w.fully_connected_workload(*mkn, realistic=True), kernel="fc_skinny")
+    check(device, w.fully_connected_workload(12, 528, 100, shift=7), kernel="fc_skinny")
+
+
 def test_fully_connected_without_skinny_kernel(device, monkeypatch):
     monkeypatch.setenv("THIP_NO_SKINNY", "1")
     check(device, w.fully_connected_workload(16, 2048, 512, realistic=True), kernel="igemm_")

@@ -1166,6 +1166,68 @@ __global__ __launch_bounds__(256) void fc_skinny(FcSkinnyArgs p) {
     }
 }
 
+// fc_skinny_mfma: the same op for 3 .. 16 rows on v_mfma_i32_16x16x64_i8.  A block owns 16 output
+// columns; its four waves split K and add their partial sums through LDS.  Per 256 bytes of K a lane
+// loads 64 contiguous bytes of one weight row and of one activation row (lane l: row l & 15, bytes
+// 64 (l >> 4) .. + 63 of the 256), and MFMA step s takes 16-byte piece s of every lane: the k order
+// inside the 256 bytes is permuted, identically for both operands, so that every load instruction
+// of a wave covers whole 256-byte stretches of 16 rows.  The weights are the MFMA's first operand:
+// lane l then holds out[m = l & 15][n0 + 4 (l >> 4) + r], r = 0 .. 3: four consecutive columns.
+__global__ __launch_bounds__(256) void fc_skinny_mfma(FcSkinnyArgs p) {
+    __shared__ int32_t partial[3][4][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, kg = lane >> 4;
+    const int n0 = blockIdx.x * 16;
+    const int nrow = n0 + r < p.N ? n0 + r : p.N - 1;  // clamped: such columns are never stored
+    const int mrow = r < p.M ? r : p.M - 1;
+    const int8_t *wrow = p.w + (size_t)nrow * p.K;
+    const int8_t *xrow = p.x + (size_t)mrow * p.K;
+    // this wave's share of K, in whole 256-byte steps
+    const int steps = (p.K + 255) / 256, per = (steps + 3) / 4;
+    const int sBeg = wave * per, sEnd = (sBeg + per) < steps ? (sBeg + per) : steps;
+    v4i acc = {0, 0, 0, 0};
+    for (int s = sBeg; s < sEnd; s++) {
+        const int k = s * 256 + 64 * kg;
+        v4i wv[4], xv[4];
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const bool in = k + 16 * c < p.K;  // K % 16 == 0: a piece is inside K or outside
+            wv[c] = in ? *(const v4i *)(wrow + k + 16 * c) : v4i{0, 0, 0, 0};
+            xv[c] = in ? *(const v4i *)(xrow + k + 16 * c) : v4i{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int c = 0; c < 4; c++) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wv[c], xv[c], acc, 0, 0, 0);
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) partial[wave - 1][e][lane] = acc[e];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 0; w < 3; w++) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) acc[e] += partial[w][e][lane];
+    }
+    const int m = r, n = n0 + 4 * kg;
+    if (m >= p.M || n >= p.N) return;
+    const long long rnd = roundTerm(p.rq.shift);
+    int32_t q[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const int ne = n + e < p.N ? n + e : p.N - 1;
+        q[e] = requant(acc[e], p.bias[ne], p.scale[ne], rnd, p.rq);
+    }
+    if (p.out_dtype == kDtypeI8 && (p.N & 3) == 0) {
+        *(uint32_t *)((int8_t *)p.out + (size_t)m * p.N + n) = packBytes(q[0], q[1], q[2], q[3]);
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            if (n + e < p.N) storeElem(p.out, (size_t)m * p.N + n + e, q[e], p.out_dtype);
+        }
+    }
+}
+
 template <int MR, int NW>
 static hipError_t launchFcSkinnyT(const FcSkinnyArgs &a, hipStream_t stream) {
     const int waves = (a.N + NW - 1) / NW;
@@ -1182,6 +1244,10 @@ hipError_t launchFcSkinny(const FcSkinnyArgs &a, hipStream_t stream) {
     if ((((uintptr_t)a.x) | ((uintptr_t)a.w)) & 15) return hipErrorInvalidValue;
     if (a.out_dtype < kDtypeI8 || a.out_dtype > kDtypeI32) return hipErrorInvalidValue;
     if (a.M == 1) return launchFcSkinnyT<1, 4>(a, stream);
+    if (a.M >= 3 && ((uintptr_t)a.out & 3) == 0 && !getenv("THIP_SKINNY_DOT4")) {
+        hipLaunchKernelGGL(fc_skinny_mfma, dim3((unsigned)((a.N + 15) / 16)), dim3(256), 0, stream, a);
+        return hipGetLastError();
+    }
     if (a.M <= 4) return launchFcSkinnyT<4, 4>(a, stream);
     if (a.M <= 8) return launchFcSkinnyT<8, 2>(a, stream);
     return launchFcSkinnyT<16, 2>(a, stream);
