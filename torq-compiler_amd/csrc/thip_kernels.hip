@@ -56,6 +56,7 @@ struct WideRequant {
     int pre, shiftMinus32;
     int32_t rnd, lo, hi, zp;
     int32_t t0lo, t0hi;  // clamp of acc + bias (the whole int32 range when rq.t0_clamp == 0)
+    bool plain;          // on, pre == 0, no clamp of t0, zero point folded: requantWideT0<true> applies
 };
 __device__ __forceinline__ WideRequant wideRequant(const Requant &rq) {
     WideRequant w;
@@ -78,6 +79,7 @@ __device__ __forceinline__ WideRequant wideRequant(const Requant &rq) {
         w.hi = rq.out_max;
         w.zp = 0;
     }
+    w.plain = w.on && w.pre == 0 && rq.t0_clamp <= 0 && w.zp == 0;
     return w;
 }
 __device__ __forceinline__ int32_t med3(int32_t v, int32_t lo, int32_t hi) {
@@ -85,10 +87,34 @@ __device__ __forceinline__ int32_t med3(int32_t v, int32_t lo, int32_t hi) {
     asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "v"(lo), "v"(hi));
     return r;
 }
-__device__ __forceinline__ int32_t requantWideShift(int32_t acc, int32_t bias, int32_t scale, const WideRequant &w) {
-    const int32_t t0 = (int32_t)((uint32_t)med3((int32_t)((uint32_t)acc + (uint32_t)bias), w.t0lo, w.t0hi) << w.pre);
+// `t0` is acc + bias (with int32 wrap).  PLAIN: no pre-shift, no clamp of t0, zero point folded into the
+// rounding term (WideRequant::plain), which is the usual case and four instructions shorter.
+template <bool PLAIN>
+__device__ __forceinline__ int32_t requantWideT0(int32_t t0, int32_t scale, const WideRequant &w) {
+    if (PLAIN) return med3((__mulhi(t0, scale) + w.rnd) >> w.shiftMinus32, w.lo, w.hi);
+    t0 = (int32_t)((uint32_t)med3(t0, w.t0lo, w.t0hi) << w.pre);
     const int32_t t3 = med3((__mulhi(t0, scale) + w.rnd) >> w.shiftMinus32, w.lo, w.hi);  // lo <= hi
     return (int32_t)((uint32_t)t3 + (uint32_t)w.zp);
+}
+__device__ __forceinline__ int32_t requantWideShift(int32_t acc, int32_t bias, int32_t scale, const WideRequant &w) {
+    return requantWideT0<false>((int32_t)((uint32_t)acc + (uint32_t)bias), scale, w);
+}
+// The three requant tails as a compile-time choice made once per kernel: f(tag) with tag::value
+// 0 = generic 64-bit, 1 = 32-bit, 2 = 32-bit plain.
+template <typename F>
+__device__ __forceinline__ void withRequantMode(const WideRequant &w, F &&f) {
+    if (!w.on) {
+        f(std::integral_constant<int, 0>{});
+    } else if (!w.plain) {
+        f(std::integral_constant<int, 1>{});
+    } else {
+        f(std::integral_constant<int, 2>{});
+    }
+}
+template <int MODE>
+__device__ __forceinline__ int32_t requantT0(int32_t t0, int32_t scale, long long rnd, const Requant &rq, const WideRequant &w) {
+    if (MODE == 0) return requant(t0, 0, scale, rnd, rq);
+    return requantWideT0<MODE == 2>(t0, scale, w);
 }
 // Four requantised values (each within int8 after the clamp) as the bytes of one dword.
 __device__ __forceinline__ uint32_t packBytes(int32_t a, int32_t b, int32_t c, int32_t d) {
@@ -237,32 +263,42 @@ __device__ __forceinline__ void igemmEpilogueDirect(v16i (&acc)[WTN / 32][WTM / 
     }
     __syncthreads();
     const WideRequant wrq = wideRequant(p.rq);
+    auto tiles = [&](auto plainTag) {
+        constexpr bool kPlain = decltype(plainTag)::value;
 #pragma unroll
-    for (int j = 0; j < TN; j++) {
-        const int nl = wn * WTN + j * 32;  // first channel of this tile column, relative to n0
-        v4i b4[4], s4[4];
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-            b4[q] = *(const v4i *)(ldsBias + nl + 8 * q + 4 * half);
-            s4[q] = *(const v4i *)(ldsScale + nl + 8 * q + 4 * half);
-        }
-        const int n = n0 + nl + 16 * half;
-#pragma unroll
-        for (int i = 0; i < TM; i++) {
-            uint32_t d4[4];
+        for (int j = 0; j < TN; j++) {
+            const int nl = wn * WTN + j * 32;  // first channel of this tile column, relative to n0
+            v4i b4[4], s4[4];
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-                int32_t v[4];
-#pragma unroll
-                for (int e = 0; e < 4; e++) v[e] = requantWideShift(acc[j][i][4 * q + e], b4[q][e], s4[q][e], wrq);
-                d4[q] = packBytes(v[0], v[1], v[2], v[3]);
+                b4[q] = *(const v4i *)(ldsBias + nl + 8 * q + 4 * half);
+                s4[q] = *(const v4i *)(ldsScale + nl + 8 * q + 4 * half);
             }
-            const auto s02 = __builtin_amdgcn_permlane32_swap(d4[0], d4[2], false, false);
-            const auto s13 = __builtin_amdgcn_permlane32_swap(d4[1], d4[3], false, false);
-            const v4i outv = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
-            const int m = m0 + wm * WTM + i * 32 + fr;
-            if (m < p.M && n < p.N) *(v4i *)((int8_t *)p.out + (size_t)m * p.N + n) = outv;
+            const int n = n0 + nl + 16 * half;
+#pragma unroll
+            for (int i = 0; i < TM; i++) {
+                uint32_t d4[4];
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    int32_t v[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        v[e] = requantWideT0<kPlain>((int32_t)((uint32_t)acc[j][i][4 * q + e] + (uint32_t)b4[q][e]), s4[q][e], wrq);
+                    }
+                    d4[q] = packBytes(v[0], v[1], v[2], v[3]);
+                }
+                const auto s02 = __builtin_amdgcn_permlane32_swap(d4[0], d4[2], false, false);
+                const auto s13 = __builtin_amdgcn_permlane32_swap(d4[1], d4[3], false, false);
+                const v4i outv = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
+                const int m = m0 + wm * WTM + i * 32 + fr;
+                if (m < p.M && n < p.N) *(v4i *)((int8_t *)p.out + (size_t)m * p.N + n) = outv;
+            }
         }
+    };
+    if (wrq.plain) {
+        tiles(std::true_type{});
+    } else {
+        tiles(std::false_type{});
     }
 }
 
@@ -860,11 +896,18 @@ __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArg
     for (int d = 0; d < RING; d++) ring[d] = fetch(g, d, here);
     for (; g < groups; g += stride) {
         const Pos next = locate(g + stride < groups ? g + stride : g);
+        // accumulators start at the bias: register 4 q + e of block j holds channel 32 j + 8 q + 4 half + e
         v16i acc[NB];
 #pragma unroll
         for (int j = 0; j < NB; j++) {
+            if (j < nblocks) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) acc[j][r] = 0;
+                for (int q = 0; q < 4; q++) {
+                    const v4i b4 = *(const v4i *)(ldsBias + j * 32 + 8 * q + 4 * half);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc[j][4 * q + e] = b4[e];
+                }
+            }
         }
         for (int s0 = 0; s0 < kstepsRing; s0 += RING) {
 #pragma unroll
@@ -887,23 +930,18 @@ __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArg
             }
         }
         const int m = g * 32 + fr;
-        auto finish = [&](auto wideShiftTag) {
-            constexpr bool kWideShift = decltype(wideShiftTag)::value;
+        withRequantMode(wrq, [&](auto mode) {
+            constexpr int kMode = decltype(mode)::value;
 #pragma unroll
             for (int j = 0; j < NB; j++) {
                 if (j < nblocks) {
                     uint32_t d4[4];
 #pragma unroll
                     for (int q = 0; q < 4; q++) {
-                        const int ch = j * 32 + 8 * q + 4 * half;
-                        const v4i b4 = *(const v4i *)(ldsBias + ch);
-                        const v4i s4 = *(const v4i *)(ldsScale + ch);
+                        const v4i s4 = *(const v4i *)(ldsScale + j * 32 + 8 * q + 4 * half);
                         int32_t v[4];
 #pragma unroll
-                        for (int e = 0; e < 4; e++) {
-                            v[e] = kWideShift ? requantWideShift(acc[j][4 * q + e], b4[e], s4[e], wrq)
-                                              : requant(acc[j][4 * q + e], b4[e], s4[e], rnd, p.rq);
-                        }
+                        for (int e = 0; e < 4; e++) v[e] = requantT0<kMode>(acc[j][4 * q + e], s4[e], rnd, p.rq, wrq);
                         d4[q] = packBytes(v[0], v[1], v[2], v[3]);
                     }
                     // lower half lanes: channels 0-3, 8-11, 16-19, 24-27; upper half: 4-7, 12-15, 20-23, 28-31.
@@ -916,12 +954,7 @@ __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArg
                     if (m < p.M && n < p.N) *(v4i *)((int8_t *)p.out + (size_t)m * p.N + n) = outv;
                 }
             }
-        };
-        if (wrq.on) {
-            finish(std::true_type{});
-        } else {
-            finish(std::false_type{});
-        }
+        });
         here = next;
     }
 }
@@ -1394,22 +1427,23 @@ __global__ __launch_bounds__(256) void depthwise3x3_dot4_i8(DepthwiseArgs p) {
     const WideRequant wrq = wideRequant(p.rq);
     const long long rnd = roundTerm(p.rq.shift);
     v4i o[P];
+    withRequantMode(wrq, [&](auto mode) {
+        constexpr int kMode = decltype(mode)::value;
 #pragma unroll
-    for (int g = 0; g < 4; g++) {
-        const v4i b4 = *(const v4i *)(p.bias + c0 + 4 * g);
-        const v4i s4 = *(const v4i *)(p.scale + c0 + 4 * g);
+        for (int g = 0; g < 4; g++) {
+            const v4i b4 = *(const v4i *)(p.bias + c0 + 4 * g);
+            const v4i s4 = *(const v4i *)(p.scale + c0 + 4 * g);
 #pragma unroll
-        for (int q = 0; q < P; q++) {
-            uint32_t w = 0;
+            for (int q = 0; q < P; q++) {
+                int32_t v[4];
 #pragma unroll
-            for (int c = 0; c < 4; c++) {
-                const int32_t r = wrq.on ? requantWideShift(acc[q][4 * g + c], b4[c], s4[c], wrq)
-                                            : requant(acc[q][4 * g + c], b4[c], s4[c], rnd, p.rq);
-                w |= (uint32_t)(r & 0xff) << (8 * c);
+                for (int c = 0; c < 4; c++) {
+                    v[c] = requantT0<kMode>((int32_t)((uint32_t)acc[q][4 * g + c] + (uint32_t)b4[c]), s4[c], rnd, p.rq, wrq);
+                }
+                o[q][g] = (int)packBytes(v[0], v[1], v[2], v[3]);
             }
-            o[q][g] = (int)w;
         }
-    }
+    });
 #pragma unroll
     for (int q = 0; q < P; q++) {
         if (ox0 + q < p.OW) *(v4i *)(p.out + (((size_t)n * p.OH + oy) * p.OW + ox0 + q) * p.C + c0) = o[q];
@@ -1478,13 +1512,15 @@ __global__ __launch_bounds__(256) void depthwise3x3_tile_i8(DepthwiseArgs p) {
     const long long rnd = roundTerm(p.rq.shift);
     const uint32_t *wrow = (const uint32_t *)p.wpk + c0;
     v4i o[R][P];
-    auto channels = [&](auto wideShiftTag) {
-        constexpr bool kWideShift = decltype(wideShiftTag)::value;
+    withRequantMode(wrq, [&](auto mode) {
+        constexpr int kMode = decltype(mode)::value;
 #pragma unroll
         for (int g = 0; g < 4; g++) {
             v4i wk[3];
 #pragma unroll
             for (int kh = 0; kh < 3; kh++) wk[kh] = *(const v4i *)(wrow + (size_t)kh * p.C + 4 * g);
+            const v4i b4 = *(const v4i *)(p.bias + c0 + 4 * g);
+            const v4i s4 = *(const v4i *)(p.scale + c0 + 4 * g);
             int32_t acc[R][P][4];
 #pragma unroll
             for (int r = 0; r < R; r++) {
@@ -1522,8 +1558,6 @@ __global__ __launch_bounds__(256) void depthwise3x3_tile_i8(DepthwiseArgs p) {
                     }
                 }
             }
-            const v4i b4 = *(const v4i *)(p.bias + c0 + 4 * g);
-            const v4i s4 = *(const v4i *)(p.scale + c0 + 4 * g);
 #pragma unroll
             for (int r = 0; r < R; r++) {
 #pragma unroll
@@ -1531,19 +1565,13 @@ __global__ __launch_bounds__(256) void depthwise3x3_tile_i8(DepthwiseArgs p) {
                     int32_t v[4];
 #pragma unroll
                     for (int c = 0; c < 4; c++) {
-                        v[c] = kWideShift ? requantWideShift(acc[r][q][c], b4[c], s4[c], wrq)
-                                          : requant(acc[r][q][c], b4[c], s4[c], rnd, p.rq);
+                        v[c] = requantT0<kMode>((int32_t)((uint32_t)acc[r][q][c] + (uint32_t)b4[c]), s4[c], rnd, p.rq, wrq);
                     }
                     o[r][q][g] = (int)packBytes(v[0], v[1], v[2], v[3]);
                 }
             }
         }
-    };
-    if (wrq.on) {
-        channels(std::true_type{});
-    } else {
-        channels(std::false_type{});
-    }
+    });
 #pragma unroll
     for (int r = 0; r < R; r++) {
 #pragma unroll
