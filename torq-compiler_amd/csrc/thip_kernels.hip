@@ -1465,18 +1465,44 @@ static hipError_t launchDepthwiseDot4(const DepthwiseArgs &a, hipStream_t stream
 // gives the window row at the block's first column and, for stride 1, with [0, w0, w1, w2] the
 // one at its second column.  That is about one permute and three dot products per output instead
 // of six and three.
-template <int P, int R, int S>
+template <int G>
+struct DwordVec {
+    typedef v4i type;
+};
+template <>
+struct DwordVec<2> {
+    typedef v2i type;
+};
+template <>
+struct DwordVec<1> {
+    typedef int type;
+};
+template <int G>
+__device__ __forceinline__ void loadDwords(const int8_t *src, int (&dst)[G]) {
+    union {
+        typename DwordVec<G>::type v;
+        int w[G];
+    } u;
+    u.v = *(const typename DwordVec<G>::type *)src;
+#pragma unroll
+    for (int g = 0; g < G; g++) dst[g] = u.w[g];
+}
+
+// G = channels per thread / 4.  Fewer channels per thread mean fewer registers and more waves per SIMD
+// (the loads stay coalesced: neighbouring lanes hold neighbouring channel groups).
+template <int P, int R, int S, int G>
 __global__ __launch_bounds__(256) void depthwise3x3_tile_i8(DepthwiseArgs p) {
     static_assert(S == 1 || S == 2, "stride 1 or 2");
     static_assert(S == 2 || P % 2 == 0, "stride 1 pairs the pixels of a block");
     constexpr int NC = (P - 1) * S + 3, NR = (R - 1) * S + 3;
     constexpr int NBK = S == 1 ? P / 2 : P;  // blocks of four columns per row; block b starts at column 2 b
-    const int cg = p.C / 16;
+    constexpr int CV = 4 * G;
+    const int cg = p.C / CV;
     const int oxGroups = (p.OW + P - 1) / P, oyGroups = (p.OH + R - 1) / R;
     const long long total = (long long)p.N * oyGroups * oxGroups * cg;
     const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
     if (t >= total) return;
-    const int c0 = (int)(t % cg) * 16;
+    const int c0 = (int)(t % cg) * CV;
     long long pix = t / cg;
     const int ox0 = (int)(pix % oxGroups) * P;
     pix /= oxGroups;
@@ -1485,13 +1511,13 @@ __global__ __launch_bounds__(256) void depthwise3x3_tile_i8(DepthwiseArgs p) {
     const int iy0 = oy0 * S - p.PT, ix0 = ox0 * S - p.PL;
     const int8_t *img = p.in + (size_t)n * p.H * p.W * p.C + c0;
     const int zp4 = (int)((uint32_t)(p.input_zp & 0xff) * 0x01010101u);
-    v4i d[NR][NC];
+    int d[NR][NC][G];
     if (iy0 >= 0 && iy0 + NR <= p.H && ix0 >= 0 && ix0 + NC <= p.W) {
         const int8_t *base = img + ((size_t)iy0 * p.W + ix0) * p.C;
 #pragma unroll
         for (int i = 0; i < NR; i++) {
 #pragma unroll
-            for (int j = 0; j < NC; j++) d[i][j] = *(const v4i *)(base + ((size_t)i * p.W + j) * p.C);
+            for (int j = 0; j < NC; j++) loadDwords<G>(base + ((size_t)i * p.W + j) * p.C, d[i][j]);
         }
     } else {
 #pragma unroll
@@ -1502,20 +1528,21 @@ __global__ __launch_bounds__(256) void depthwise3x3_tile_i8(DepthwiseArgs p) {
             for (int j = 0; j < NC; j++) {
                 const int ix = ix0 + j;
                 const int ixc = ix < 0 ? 0 : ix >= p.W ? p.W - 1 : ix;
-                const v4i v = *(const v4i *)(img + ((size_t)iyc * p.W + ixc) * p.C);
+                loadDwords<G>(img + ((size_t)iyc * p.W + ixc) * p.C, d[i][j]);
                 const bool inside = iy == iyc && ix == ixc;
-                d[i][j] = inside ? v : v4i{zp4, zp4, zp4, zp4};
+#pragma unroll
+                for (int g = 0; g < G; g++) d[i][j][g] = inside ? d[i][j][g] : zp4;
             }
         }
     }
     const WideRequant wrq = wideRequant(p.rq);
     const long long rnd = roundTerm(p.rq.shift);
     const uint32_t *wrow = (const uint32_t *)p.wpk + c0;
-    v4i o[R][P];
+    int o[R][P][G];
     withRequantMode(wrq, [&](auto mode) {
         constexpr int kMode = decltype(mode)::value;
 #pragma unroll
-        for (int g = 0; g < 4; g++) {
+        for (int g = 0; g < G; g++) {
             v4i wk[3];
 #pragma unroll
             for (int kh = 0; kh < 3; kh++) wk[kh] = *(const v4i *)(wrow + (size_t)kh * p.C + 4 * g);
@@ -1577,16 +1604,22 @@ __global__ __launch_bounds__(256) void depthwise3x3_tile_i8(DepthwiseArgs p) {
 #pragma unroll
         for (int q = 0; q < P; q++) {
             if (oy0 + r < p.OH && ox0 + q < p.OW) {
-                *(v4i *)(p.out + (((size_t)n * p.OH + oy0 + r) * p.OW + ox0 + q) * p.C + c0) = o[r][q];
+                union {
+                    typename DwordVec<G>::type v;
+                    int w[G];
+                } u;
+#pragma unroll
+                for (int g = 0; g < G; g++) u.w[g] = o[r][q][g];
+                *(typename DwordVec<G>::type *)(p.out + (((size_t)n * p.OH + oy0 + r) * p.OW + ox0 + q) * p.C + c0) = u.v;
             }
         }
     }
 }
 
-template <int P, int R, int S>
+template <int P, int R, int S, int G>
 static hipError_t launchDepthwiseTile(const DepthwiseArgs &a, hipStream_t stream) {
-    const long long total = (long long)a.N * ((a.OH + R - 1) / R) * ((a.OW + P - 1) / P) * (a.C / 16);
-    hipLaunchKernelGGL((depthwise3x3_tile_i8<P, R, S>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a);
+    const long long total = (long long)a.N * ((a.OH + R - 1) / R) * ((a.OW + P - 1) / P) * (a.C / (4 * G));
+    hipLaunchKernelGGL((depthwise3x3_tile_i8<P, R, S, G>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a);
     return hipGetLastError();
 }
 
@@ -1633,7 +1666,8 @@ hipError_t launchDepthwise(const DepthwiseArgs &a, hipStream_t stream) {
         const char *tileEnv = getenv("THIP_DEPTHWISE_TILE");
         const bool tileOff = tileEnv && tileEnv[0] == '0', tileOn = tileEnv && tileEnv[0] == '1';
         if (!tileOff) {
-            if (a.SW == 1 && a.SH == 1 && (tileOn || outputs >= 8 * 4 * 65536)) return launchDepthwiseTile<4, 2, 1>(a, stream);
+            // 16 channels per thread: 8 or 4 (more waves, fewer registers) measured 5 % and 12 % slower
+            if (a.SW == 1 && a.SH == 1 && (tileOn || outputs >= 8 * 4 * 65536)) return launchDepthwiseTile<4, 2, 1, 4>(a, stream);
         }
         // pixels per thread (THIP_DEPTHWISE_P forces 1, 2 or 4, for tuning)
         int pix = outputs >= 4 * 65536 ? 4 : outputs >= 2 * 65536 ? 2 : 1;
