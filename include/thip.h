@@ -66,7 +66,8 @@ typedef struct thip_program_t thip_program_t;
 /* A tensor value of the program (index into the program's value table). */
 typedef int32_t thip_value_t;
 
-enum { THIP_DTYPE_I8 = 1, THIP_DTYPE_I16 = 2, THIP_DTYPE_I32 = 3 };
+/* BF16 values are bfloat16 bit patterns (16 bits); F32 is used for the bias of the bf16 ops. */
+enum { THIP_DTYPE_I8 = 1, THIP_DTYPE_I16 = 2, THIP_DTYPE_I32 = 3, THIP_DTYPE_BF16 = 4, THIP_DTYPE_F32 = 5 };
 
 #define THIP_MAX_RANK 4
 
@@ -146,7 +147,12 @@ typedef struct thip_hl_depthwise_conv2d_t {
 } thip_hl_depthwise_conv2d_t;
 
 /* torq_hl.fully_connected -- TorqHLOps.td:172-190.  input M,K; weights N,K;
- * scale_bias int32[2*N]. */
+ * scale_bias int32[2*N].
+ * bf16 form (input, weights and init BF16): the ACT stage has no scale and no shift
+ * (compiler/torq/Utils/Kernel.h:626-632): scale_bias is F32[N] (bias only), shift_factor and the
+ * zero points must be 0, output_min / output_max are float bit patterns (0xff800000 / 0x7f800000
+ * when there is no clamp, compiler/torq/Utils/ConversionUtils.cpp:33-39); fp32 accumulate,
+ * result rounded to bf16.  K must be a multiple of 8. */
 typedef struct thip_hl_fully_connected_t {
     thip_value_t init;
     int32_t input_zp;
@@ -162,7 +168,9 @@ typedef struct thip_hl_fully_connected_t {
 } thip_hl_fully_connected_t;
 
 /* torq_hl.matmul -- TorqHLOps.td:85-99.  input1 [B,]M,K; input2 [B,]K,N; one
- * (bias, scale) pair in scale_bias; a batch of 1 broadcasts. */
+ * (bias, scale) pair in scale_bias; a batch of 1 broadcasts.
+ * bf16 form (both inputs and init BF16): scale_bias is F32 with one bias value, shift and output_zp
+ * 0, output_min / output_max float bit patterns, as for fully_connected. */
 typedef struct thip_hl_matmul_t {
     thip_value_t init;
     int32_t output_zp;

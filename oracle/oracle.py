@@ -168,6 +168,60 @@ def matmul(input1, input2, scale_bias, *, output_zp, output_min, output_max, shi
     return out
 
 
+NO_CLAMP_MIN, NO_CLAMP_MAX = -8388608, 0x7f800000  # float bit patterns of -inf / +inf as int32 attributes
+
+
+def to_bf16(values):
+    """float32 array -> bfloat16 bit patterns (uint16), round to nearest even."""
+    f = np.ascontiguousarray(values, dtype=np.float32)
+    out = np.empty(f.shape, dtype=np.uint16)
+    flat_in, flat_out = f.reshape(-1), out.reshape(-1)
+    u = flat_in.view(np.uint32).astype(np.uint64)
+    r = ((u + 0x7fff + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    nan = (u & 0x7fffffff) > 0x7f800000
+    r[nan] = ((u[nan] >> 16) | 0x40).astype(np.uint16)
+    flat_out[:] = r
+    return out
+
+
+def from_bf16(bits):
+    """bfloat16 bit patterns (uint16) -> float32."""
+    b = np.ascontiguousarray(bits, dtype=np.uint16)
+    return (b.astype(np.uint32) << 16).view(np.float32)
+
+
+def fully_connected_bf16(input, weights, bias, *, output_min=NO_CLAMP_MIN, output_max=NO_CLAMP_MAX):
+    """torq_hl.fully_connected on bf16 bit patterns; input M,K, weights N,K, bias N float32."""
+    x = _c(input, np.uint16)
+    w = _c(weights, np.uint16)
+    b = _c(bias, np.float32)
+    M, K = x.shape
+    N, K2 = w.shape
+    assert K == K2 and b.size == N
+    out = np.empty((M, N), dtype=np.uint16)
+    rc = lib().torq_fully_connected_bf16(_p(x), _p(w), _p(b), _p(out), M, K, N, int(output_min), int(output_max))
+    assert rc == 0
+    return out
+
+
+def matmul_bf16(input1, input2, bias, *, output_min=NO_CLAMP_MIN, output_max=NO_CLAMP_MAX):
+    """torq_hl.matmul on bf16 bit patterns; input1 [B,]M,K  input2 [B,]K,N; one float32 bias."""
+    a = _c(input1, np.uint16)
+    b = _c(input2, np.uint16)
+    bias = _c(bias, np.float32)
+    a3 = a.reshape((-1,) + a.shape[-2:])
+    b3 = b.reshape((-1,) + b.shape[-2:])
+    B = max(a3.shape[0], b3.shape[0])
+    _, M, K = a3.shape
+    _, K2, N = b3.shape
+    assert K == K2 and bias.size >= 1
+    out = np.empty((B, M, N), dtype=np.uint16)
+    rc = lib().torq_matmul_bf16(_p(a3), _p(b3), _p(bias), _p(out), B, M, K, N, int(a3.shape[0] == 1 and B > 1),
+                                int(b3.shape[0] == 1 and B > 1), int(output_min), int(output_max))
+    assert rc == 0
+    return out
+
+
 def maxpool2d(input, *, input_zp, output_min, output_max, stride, pad, kernel, layout=NCHW):
     """torq_hl.maxpool2d."""
     x = _c(input, np.int8)

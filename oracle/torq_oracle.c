@@ -237,6 +237,83 @@ int torq_matmul(const int8_t *input1, const int8_t *input2, const int32_t *scale
 }
 
 /*
+ * bf16 rows.  With floating-point partials the ACT stage has no scale and no shift
+ * (compiler/torq/Utils/Kernel.h:626-632):
+ *     float t0 = pdata + bias;   float t1 = t0 < clipMin ? clipMin : t0 > clipMax ? clipMax : t0;   qdata = t1
+ * with the clamp bounds given as float bit patterns (compiler/torq/Utils/ConversionUtils.cpp:33-39: -inf / +inf
+ * when there is no clamp).  The products of two bf16 values are exact in fp32; they are accumulated in fp32 in
+ * k order (the ALU's scalarProductAccumulate loop, compiler/torq/Conversions/TorqHLToTorqHW/MatMulPattern.cpp:66-78)
+ * and the result is rounded to bf16 to nearest even, which is what the reference's own expected values use
+ * (python/torq/testing/numpy.py:42-53, float32 matmul cast to the output type).
+ */
+float torq_bf16_to_f32(uint16_t h) {
+    union {
+        uint32_t u;
+        float f;
+    } v;
+    v.u = (uint32_t)h << 16;
+    return v.f;
+}
+
+uint16_t torq_f32_to_bf16(float f) {
+    union {
+        uint32_t u;
+        float f;
+    } v;
+    v.f = f;
+    if ((v.u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((v.u >> 16) | 0x0040u); /* NaN stays NaN */
+    return (uint16_t)((v.u + 0x7fffu + ((v.u >> 16) & 1u)) >> 16);
+}
+
+static float float_from_bits(int32_t bits) {
+    union {
+        int32_t i;
+        float f;
+    } v;
+    v.i = bits;
+    return v.f;
+}
+
+static uint16_t act_float(float acc, float bias, float lo, float hi) {
+    float t0 = acc + bias;
+    float t1 = t0 < lo ? lo : (t0 > hi ? hi : t0);
+    return torq_f32_to_bf16(t1);
+}
+
+int torq_fully_connected_bf16(const uint16_t *input, const uint16_t *weights, const float *bias,
+                              uint16_t *out, int M, int K, int N, int32_t clip_min, int32_t clip_max) {
+    const float lo = float_from_bits(clip_min), hi = float_from_bits(clip_max);
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int m = 0; m < M; m++) {
+        for (int n = 0; n < N; n++) {
+            const uint16_t *x = input + (size_t)m * K, *w = weights + (size_t)n * K;
+            float acc = 0.0f;
+            for (int k = 0; k < K; k++) acc += torq_bf16_to_f32(x[k]) * torq_bf16_to_f32(w[k]);
+            out[(size_t)m * N + n] = act_float(acc, bias[n], lo, hi);
+        }
+    }
+    return 0;
+}
+
+int torq_matmul_bf16(const uint16_t *input1, const uint16_t *input2, const float *bias, uint16_t *out,
+                     int B, int M, int K, int N, int bcast1, int bcast2, int32_t clip_min, int32_t clip_max) {
+    const float lo = float_from_bits(clip_min), hi = float_from_bits(clip_max);
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int b = 0; b < B; b++) {
+        for (int m = 0; m < M; m++) {
+            const uint16_t *a = input1 + (bcast1 ? 0 : (size_t)b * M * K) + (size_t)m * K;
+            const uint16_t *bm = input2 + (bcast2 ? 0 : (size_t)b * K * N);
+            for (int n = 0; n < N; n++) {
+                float acc = 0.0f;
+                for (int k = 0; k < K; k++) acc += torq_bf16_to_f32(a[k]) * torq_bf16_to_f32(bm[(size_t)k * N + n]);
+                out[((size_t)b * M + m) * N + n] = act_float(acc, bias[0], lo, hi);
+            }
+        }
+    }
+    return 0;
+}
+
+/*
  * torq_hl.maxpool2d -- signature TorqHLOps.td:435-453; created
  * compiler/torq/Conversions/LinalgToTorqHL/PoolingPattern.cpp:199-236 (pad value
  * becomes input_zp, output_min/max = element type range); executed

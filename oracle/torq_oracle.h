@@ -76,6 +76,21 @@ int torq_matmul(const int8_t *input1, const int8_t *input2, const int32_t *scale
                 int B, int M, int K, int N, int bcast1, int bcast2, const torq_requant_t *rq,
                 int out_elem_bytes);
 
+/* ---- bf16 rows (floating-point partials: bias only, no scale, no shift) ---- */
+
+/* bfloat16 <-> float: the upper 16 bits of the IEEE single; to bf16 rounds to nearest, ties to even. */
+float torq_bf16_to_f32(uint16_t h);
+uint16_t torq_f32_to_bf16(float f);
+
+/* torq_hl.fully_connected on bf16: input M x K, weights N x K (bf16 bit patterns), bias N floats.
+ * clip_min / clip_max are float bit patterns (0xff800000 / 0x7f800000 = no clamp). */
+int torq_fully_connected_bf16(const uint16_t *input, const uint16_t *weights, const float *bias,
+                              uint16_t *out, int M, int K, int N, int32_t clip_min, int32_t clip_max);
+
+/* torq_hl.matmul on bf16: input1 B x M x K, input2 B x K x N, ONE float bias. */
+int torq_matmul_bf16(const uint16_t *input1, const uint16_t *input2, const float *bias, uint16_t *out,
+                     int B, int M, int K, int N, int bcast1, int bcast2, int32_t clip_min, int32_t clip_max);
+
 /* torq_hl.maxpool2d.  No rescale; padding value is input_zp; result is
  * clamped to [output_min, output_max]. */
 int torq_maxpool2d(const int8_t *input, int8_t *out, int N, int C, int H, int W, int KH, int KW,

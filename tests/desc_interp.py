@@ -24,7 +24,7 @@ BINDING = np.dtype([("id", "<u4"), ("flags", "<u4"), ("size", "<u8")])
 TEMP = np.dtype([("size", "<u8")])
 CONST = np.dtype([("offset", "<u8"), ("size", "<u8")])
 
-K_TRANSPOSE, K_IGEMM, K_FC_SKINNY, K_DW, K_MAXPOOL, K_AVGPOOL, K_ADD = 1, 2, 3, 4, 5, 6, 7
+K_TRANSPOSE, K_IGEMM, K_FC_SKINNY, K_DW, K_MAXPOOL, K_AVGPOOL, K_ADD, K_FC_BF16 = 1, 2, 3, 4, 5, 6, 7, 8
 OUT_NP = {1: np.int8, 2: np.int16, 3: np.int32}
 
 
@@ -81,6 +81,10 @@ def run(blob, binding_arrays):
         sh, zp, mn, mx = int(op["shift"]), int(op["output_zp"]), int(op["output_min"]), int(op["output_max"])
         if kind == K_TRANSPOSE:
             B, R, S = int(op["TB"]), int(op["TR"]), int(op["TS"])
+            if int(op["gran"]) == 2:
+                src = view(op["in0"], B * R * S * 2).view(np.uint16).reshape(B, R, S)
+                view(op["out"], B * R * S * 2).view(np.uint16)[:] = np.ascontiguousarray(src.transpose(0, 2, 1)).reshape(-1)
+                continue
             src = view(op["in0"], B * R * S).reshape(B, R, S)
             view(op["out"], B * R * S)[:] = np.ascontiguousarray(src.transpose(0, 2, 1)).reshape(-1)
         elif kind in (K_IGEMM, K_FC_SKINNY):
@@ -186,6 +190,13 @@ def run(blob, binding_arrays):
                           np.array([op["bias0"], op["scale0"]], dtype=np.int32), output_zp=zp, output_min=mn,
                           output_max=mx, shift_factor=sh)
             view(op["out"], n)[:] = res.view(np.uint8)
+        elif kind == K_FC_BF16:
+            M, K, N = int(op["M"]), int(op["K"]), int(op["Nn"])
+            x = view(op["in0"], M * K * 2).view(np.uint16).reshape(M, K)
+            wt = view(op["weights"], N * K * 2).view(np.uint16).reshape(N, K)
+            bias = view(op["bias"], N * 4).view(np.float32)
+            res = orc.fully_connected_bf16(x, wt, bias, output_min=mn, output_max=mx)
+            view(op["out"], M * N * 2).view(np.uint16)[:] = res.reshape(-1)
         else:
             raise AssertionError("unknown kernel kind %d" % kind)
     return d

@@ -20,6 +20,11 @@ def oracle_eval(wl):
     if kind == "fully":
         w, sb = a.pop("weights"), a.pop("scale_bias")
         return [orc.fully_connected(x, w, sb, **a)]
+    if kind == "fcbf16":
+        return [orc.fully_connected_bf16(x, a["weights"], a["bias"], output_min=a["output_min"], output_max=a["output_max"])]
+    if kind == "matmulbf16":
+        res = orc.matmul_bf16(x, a["input2"], a["bias"])
+        return [res.reshape(wl.outputs[0][0])]
     if kind == "maxpool":
         layout = orc.NHWC if a.pop("nhwc") else orc.NCHW
         return [orc.maxpool2d(x, layout=layout, **a)]
@@ -63,6 +68,30 @@ def assert_bit_exact(got, want, what=""):
         first = tuple(bad[0])
         raise AssertionError("%s: %d of %d elements differ; first at %s: got %d want %d"
                              % (what, len(bad), got.size, first, int(got[first]), int(want[first])))
+
+
+def bf16_ordered(bits):
+    """bf16 bit patterns -> integers whose order and spacing are those of the values (one step = one ULP)."""
+    b = np.asarray(bits, dtype=np.uint16).astype(np.int32)
+    return np.where(b < 0x8000, b, 0x8000 - b)
+
+
+def assert_bf16_close(got, want, what="", ulps=1, magnitude=None):
+    """The bf16 rows are tolerance rows: at most `ulps` bf16 steps from the oracle per element.
+
+    `magnitude` (sum of |products| + |bias| per element) admits, for sums that cancel, the error a different
+    order of fp32 additions can make: 2^-17 of it (a bf16 step is 2^-8 of the result, so where nothing cancels the
+    ULP bound is the binding one)."""
+    assert got.shape == want.shape and got.dtype == np.uint16 and want.dtype == np.uint16, (what, got.shape, want.shape)
+    bad = np.abs(bf16_ordered(got) - bf16_ordered(want)) > ulps
+    if magnitude is not None:
+        gf = (got.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+        wf = (want.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+        bad &= ~(np.abs(gf - wf) <= np.asarray(magnitude, dtype=np.float64).reshape(got.shape) * 2.0 ** -17)
+    if bad.any():
+        first = tuple(np.argwhere(bad)[0])
+        raise AssertionError("%s: %d of %d elements differ by more than %d bf16 ULP; first at %s: got 0x%04x want 0x%04x"
+                             % (what, int(bad.sum()), got.size, ulps, first, int(got[first]), int(want[first])))
 
 
 def oracle_network(wl, return_all=False):

@@ -1,0 +1,140 @@
+"""bf16 rows of fully_connected / matmul: the oracle's pins, the emitter, and (on a GPU) the kernel, which is a
+tolerance row: at most one bf16 ULP from the oracle per element."""
+import numpy as np
+import pytest
+
+import desc_interp
+from helpers import assert_bf16_close, assert_bit_exact, bf16_ordered, oracle_eval, run_on_gpu
+from oracle import oracle as orc
+from torq_compiler_amd import Executable, Program, ThipError, runtime, workloads as w
+
+
+# ---- oracle pins ---------------------------------------------------------------------------------
+def test_bf16_conversion_matches_torch_and_is_nearest_even():
+    import torch
+    rng = np.random.default_rng(1)
+    vals = np.concatenate([rng.standard_normal(5000).astype(np.float32) * 10.0 ** rng.integers(-30, 30, 5000),
+                           np.array([0.0, -0.0, 1.0, 1.00390625, 1.01171875, 3.3e38, -3.4e38, 1e-40, np.inf, -np.inf], dtype=np.float32)])
+    got = orc.to_bf16(vals)
+    want = torch.tensor(vals).to(torch.bfloat16).view(torch.int16).numpy().astype(np.uint16)
+    assert np.array_equal(got, want)
+    # ties: 1 + 2^-8 is exactly between 1 and 1 + 2^-7 -> even mantissa (1.0); 1 + 3*2^-8 -> 1 + 2^-6
+    assert orc.to_bf16(np.float32(1 + 2.0 ** -8)) == 0x3f80 and orc.to_bf16(np.float32(1 + 3 * 2.0 ** -8)) == 0x3f82
+    assert np.array_equal(orc.from_bf16(got[:5000]).view(np.uint32) & 0xffff, np.zeros(5000, dtype=np.uint32))
+    assert np.isnan(orc.from_bf16(orc.to_bf16(np.float32(np.nan))))
+
+
+def test_bf16_fully_connected_closed_forms():
+    # small integers: every product and sum is exact, so the result is the integer matmul plus the bias
+    rng = np.random.default_rng(2)
+    xi, wi = rng.integers(-8, 9, size=(5, 24)), rng.integers(-8, 9, size=(7, 24))
+    bias = rng.integers(-4, 5, size=7).astype(np.float32)
+    out = orc.fully_connected_bf16(orc.to_bf16(xi), orc.to_bf16(wi), bias)
+    want = (xi @ wi.T + bias).astype(np.float32)
+    assert np.array_equal(out, orc.to_bf16(want))
+    # clamp to [0, 6] (a ReLU6) with float bit patterns; bias only, no scale
+    out = orc.fully_connected_bf16(orc.to_bf16(xi), orc.to_bf16(wi), bias, output_min=w.float_bits(0.0), output_max=w.float_bits(6.0))
+    assert np.array_equal(out, orc.to_bf16(np.clip(want, 0.0, 6.0)))
+    # a transposed operand or a dropped bias would show
+    assert not np.array_equal(orc.fully_connected_bf16(orc.to_bf16(xi), orc.to_bf16(wi), 0 * bias), orc.to_bf16(want))
+
+
+def test_bf16_oracle_against_float64():
+    rng = np.random.default_rng(3)
+    for M, K, N in [(3, 64, 5), (9, 1152, 33), (2, 6912, 8)]:
+        x, wt = orc.to_bf16(rng.standard_normal((M, K))), orc.to_bf16(rng.standard_normal((N, K)) / np.sqrt(K))
+        bias = rng.standard_normal(N).astype(np.float32)
+        got = orc.fully_connected_bf16(x, wt, bias)
+        exact = orc.from_bf16(x).astype(np.float64) @ orc.from_bf16(wt).astype(np.float64).T + bias
+        assert_bf16_close(got, orc.to_bf16(exact.astype(np.float32)), "fp32 accumulate vs float64")
+        # matmul is the same arithmetic with input2 = weights^T and one bias
+        mm = orc.matmul_bf16(x, np.ascontiguousarray(wt.T), np.array([0.25], dtype=np.float32))
+        fc = orc.fully_connected_bf16(x, wt, np.full(N, 0.25, dtype=np.float32))
+        assert np.array_equal(mm.reshape(M, N), fc)
+
+
+def test_bf16_matmul_batches_broadcast():
+    rng = np.random.default_rng(4)
+    a, b = orc.to_bf16(rng.standard_normal((4, 3, 16))), orc.to_bf16(rng.standard_normal((1, 16, 10)))
+    out = orc.matmul_bf16(a, b, np.zeros(1, dtype=np.float32))
+    for i in range(4):
+        assert np.array_equal(out[i], orc.matmul_bf16(a[i], b[0], np.zeros(1, dtype=np.float32))[0])
+
+
+# ---- emitter ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("make", [lambda: w.fully_connected_bf16_workload(5, 64, 40), lambda: w.fully_connected_bf16_workload(33, 1152, 7, clamp=(-0.5, 0.75)),
+                                  lambda: w.matmul_bf16_workload(4, 1, 256, 96, batch2=False), lambda: w.matmul_bf16_workload(3, 2, 64, 24),
+                                  lambda: w.matmul_bf16_workload(1, 6, 32, 20, batch1=False, batch2=False, constant_rhs=True, bias=0.5),
+                                  lambda: w.matmul_bf16_workload(2, 5, 16, 12, batch1=False, constant_rhs=True)])
+def test_bf16_descriptor(make):
+    wl = make()
+    outs = [np.zeros(s, dtype=dt) for s, dt in wl.outputs]
+    d = desc_interp.run(wl.program.serialize(), list(wl.inputs) + outs)
+    assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)
+    assert desc_interp.K_FC_BF16 in [int(o["kind"]) for o in d.ops]
+
+
+def test_bf16_rejections():
+    def expect(code, build):
+        p = Program()
+        with pytest.raises(ThipError) as e:
+            build(p)
+            p.serialize()
+        assert e.value.code == code, e.value
+
+    wt = np.zeros((8, 16), dtype=np.uint16)
+    bias = np.zeros(8, dtype=np.float32)
+    ok = dict(output_zp=0, output_min=w.NO_CLAMP[0], output_max=w.NO_CLAMP[1], shift_factor=0, input_zp=0)
+    expect(runtime.INVALID_ARGUMENT, lambda p: p.fully_connected(p.binding(0, (2, 16), np.uint16), wt, bias, init=p.binding(1, (2, 8), np.uint16), **dict(ok, shift_factor=3)))
+    expect(runtime.INVALID_ARGUMENT, lambda p: p.fully_connected(p.binding(0, (2, 16), np.uint16), wt, bias, init=p.binding(1, (2, 8), np.uint16), **dict(ok, output_zp=1)))
+    expect(runtime.INVALID_ARGUMENT, lambda p: p.fully_connected(p.binding(0, (2, 16), np.uint16), wt, bias[:4], init=p.binding(1, (2, 8), np.uint16), **ok))
+    expect(runtime.UNIMPLEMENTED, lambda p: p.fully_connected(p.binding(0, (2, 12), np.uint16), wt[:, :12].copy(), bias, init=p.binding(1, (2, 8), np.uint16), **ok))
+    # int8 weights under a bf16 input
+    expect(runtime.INVALID_ARGUMENT, lambda p: p.fully_connected(p.binding(0, (2, 16), np.uint16), np.zeros((8, 16), dtype=np.int8), bias, init=p.binding(1, (2, 8), np.uint16), **ok))
+
+
+# ---- GPU ------------------------------------------------------------------------------------------------
+def _magnitude(wl):
+    """Per output element: sum of |x * w| + |bias|, what the fp32 rounding errors scale with."""
+    f = lambda bits: np.abs(orc.from_bf16(bits).astype(np.float64))
+    if wl.name.startswith("fcbf16"):
+        return f(wl.inputs[0]) @ f(wl.attrs["weights"]).T + np.abs(wl.attrs["bias"])
+    return np.matmul(f(wl.inputs[0]), f(wl.attrs["input2"])) + abs(float(wl.attrs["bias"][0]))
+
+
+def _check_gpu(device, wl, via="host"):
+    print("[gpu-case]", wl.name, flush=True)
+    got, kernels = run_on_gpu(device, wl, via=via)
+    assert_bf16_close(got[0], oracle_eval(wl)[0], wl.name, magnitude=_magnitude(wl))
+    assert any("fc_bf16" in k for k in kernels), kernels
+    return got[0]
+
+
+@pytest.mark.gpu
+def test_gpu_bf16_fully_connected(device):
+    """Decoder linear shapes at 1 and 32 tokens, ragged M / N / K, a clamp; exact on small integers."""
+    for M, K, N in [(1, 1152, 1024), (32, 1152, 256), (1, 1152, 6912), (32, 6912, 1152), (5, 64, 40), (33, 1152, 7), (70, 24, 130), (3, 8, 2)]:
+        _check_gpu(device, w.fully_connected_bf16_workload(M, K, N))
+    _check_gpu(device, w.fully_connected_bf16_workload(9, 200, 44, clamp=(-0.25, 0.5)), via="device")
+    rng = np.random.default_rng(5)
+    xi, wi = rng.integers(-8, 9, size=(6, 48)), rng.integers(-8, 9, size=(20, 48))
+    bias = rng.integers(-4, 5, size=20).astype(np.float32)
+    p = Program()
+    p.fully_connected(p.binding(0, (6, 48), np.uint16), w.to_bf16(wi), bias, init=p.binding(1, (6, 20), np.uint16), output_zp=0,
+                      output_min=w.NO_CLAMP[0], output_max=w.NO_CLAMP[1], shift_factor=0, input_zp=0)
+    exe = Executable(device, p.serialize())
+    out = np.zeros((6, 20), dtype=np.uint16)
+    exe.run_host([w.to_bf16(xi), out])
+    exe.close()
+    assert_bit_exact(out, w.to_bf16((xi @ wi.T + bias).astype(np.float32)), "exact small integers")
+
+
+@pytest.mark.gpu
+def test_gpu_bf16_matmul(device):
+    """Attention-shaped matmuls (4 query heads sharing one K / V, length 1024, head size 256) with a run-time input2,
+    per-batch input2, and a constant input2."""
+    _check_gpu(device, w.matmul_bf16_workload(4, 1, 256, 1024, batch2=False))
+    _check_gpu(device, w.matmul_bf16_workload(4, 1, 1024, 256, batch2=False))
+    _check_gpu(device, w.matmul_bf16_workload(3, 2, 64, 24))
+    _check_gpu(device, w.matmul_bf16_workload(2, 5, 16, 12, batch1=False, constant_rhs=True))
+    _check_gpu(device, w.matmul_bf16_workload(1, 6, 32, 20, batch1=False, batch2=False, constant_rhs=True, bias=0.5))

@@ -62,13 +62,14 @@ struct DescConst {
 
 // Kernel kinds.  One record = one kernel launch.
 enum Kind : uint32_t {
-    kKindTranspose = 1,  // [B, R, S] -> [B, S, R] bytes (NCHW <-> NHWC)
+    kKindTranspose = 1,  // [B, R, S] -> [B, S, R] elements of `gran` bytes (0 or 1: bytes; 2: bf16)
     kKindIgemm = 2,      // conv2d / fully_connected / matmul on MFMA
     kKindFcSkinny = 3,   // fully_connected with few rows: weight streaming
     kKindDepthwise = 4,
     kKindMaxPool = 5,
     kKindAvgPool = 6,
     kKindAdd = 7,
+    kKindFcBf16 = 8,     // bf16 fully_connected / matmul: fp32 accumulate, float bias, float clamp (output_min/max bits)
 };
 
 // Variants of kKindIgemm: how the A (activation) tile is gathered.

@@ -170,7 +170,8 @@ static thip_status_t checkOpFootprint(const thip_executable_t *e, uint32_t i) {
     switch (op.kind) {
     case kKindTranspose: {
         if (!positive({op.TB, op.TR, op.TS})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad transpose extents", i);
-        const uint64_t bytes = (uint64_t)op.TB * op.TR * op.TS;
+        if (op.gran > 2) return fail(THIP_INVALID_ARGUMENT, "op %u: transpose element size %u", i, op.gran);
+        const uint64_t bytes = (uint64_t)op.TB * op.TR * op.TS * (op.gran == 2 ? 2 : 1);
         if ((s = need(op.in0, bytes, "in"))) return s;
         return need(op.out, bytes, "out");
     }
@@ -249,6 +250,13 @@ static thip_status_t checkOpFootprint(const thip_executable_t *e, uint32_t i) {
         if ((s = need(op.in1, (uint64_t)op.C, "in2"))) return s;
         return need(op.out, (uint64_t)op.C, "out");
     }
+    case kKindFcBf16: {
+        if (!positive({op.M, op.K, op.Nn}) || op.K % 8 != 0) return fail(THIP_INVALID_ARGUMENT, "op %u: bad bf16 fully_connected extents", i);
+        if ((s = need(op.in0, (uint64_t)op.M * op.K * 2, "in"))) return s;
+        if ((s = need(op.weights, (uint64_t)op.Nn * op.K * 2, "weights"))) return s;
+        if ((s = need(op.bias, (uint64_t)op.Nn * 4, "bias"))) return s;
+        return need(op.out, (uint64_t)op.M * op.Nn * 2, "out");
+    }
     default: return fail(THIP_INVALID_ARGUMENT, "op %u has unknown kind %u", i, op.kind);
     }
 }
@@ -262,6 +270,7 @@ static const char *opKernelName(const DescOp &op) {
     case kKindMaxPool: return "maxpool_i8";
     case kKindAvgPool: return "avgpool_i8";
     case kKindAdd: return "add_i8";
+    case kKindFcBf16: return "fc_bf16";
     default: return "unknown";
     }
 }
@@ -289,7 +298,7 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
     hipError_t err = hipSuccess;
     switch (op.kind) {
     case kKindTranspose: {
-        TransposeArgs a{(const int8_t *)resolve(e, op.in0, bp), (int8_t *)resolve(e, op.out, bp), op.TB, op.TR, op.TS};
+        TransposeArgs a{(const int8_t *)resolve(e, op.in0, bp), (int8_t *)resolve(e, op.out, bp), op.TB, op.TR, op.TS, op.gran == 2 ? 2 : 1};
         err = launchTranspose(a, e->stream);
         break;
     }
@@ -345,6 +354,15 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
         AddArgs a{(const int8_t *)resolve(e, op.in0, bp), (const int8_t *)resolve(e, op.in1, bp),
                   (int8_t *)resolve(e, op.out, bp), (int64_t)op.C, op.w0, op.w1, op.bias0, op.scale0, rq};
         err = launchAdd(a, e->stream);
+        break;
+    }
+    case kKindFcBf16: {
+        float lo, hi;
+        memcpy(&lo, &op.output_min, 4);
+        memcpy(&hi, &op.output_max, 4);
+        FcBf16Args a{(const uint16_t *)resolve(e, op.in0, bp), (const uint16_t *)resolve(e, op.weights, bp),
+                     (const float *)resolve(e, op.bias, bp), (uint16_t *)resolve(e, op.out, bp), op.M, op.K, op.Nn, lo, hi};
+        err = launchFcBf16(a, e->stream);
         break;
     }
     default: return fail(THIP_INTERNAL, "op %u has unknown kind %u", i, op.kind);

@@ -75,6 +75,8 @@ static size_t elemSize(int32_t dtype) {
     case THIP_DTYPE_I8: return 1;
     case THIP_DTYPE_I16: return 2;
     case THIP_DTYPE_I32: return 4;
+    case THIP_DTYPE_BF16: return 2;
+    case THIP_DTYPE_F32: return 4;
     default: return 0;
     }
 }
@@ -173,10 +175,11 @@ class Emitter {
         return THIP_OK;
     }
 
-    void emitTranspose(DescRef in, DescRef out, int64_t B, int64_t R, int64_t S) {
+    void emitTranspose(DescRef in, DescRef out, int64_t B, int64_t R, int64_t S, uint32_t elem = 1) {
         DescOp op;
         memset(&op, 0, sizeof(op));
         op.kind = kKindTranspose;
+        op.gran = elem;
         op.TB = (int32_t)B;
         op.TR = (int32_t)R;
         op.TS = (int32_t)S;
@@ -476,6 +479,8 @@ class Emitter {
     thip_status_t emitDepthwise(const thip_hl_depthwise_conv2d_t &c);
     thip_status_t emitFullyConnected(const thip_hl_fully_connected_t &c);
     thip_status_t emitMatmul(const thip_hl_matmul_t &c);
+    thip_status_t emitFullyConnectedBf16(const thip_hl_fully_connected_t &c);
+    thip_status_t emitMatmulBf16(const thip_hl_matmul_t &c);
     thip_status_t emitMaxPool(const thip_hl_maxpool2d_t &c);
     thip_status_t emitAvgPool(const thip_hl_avg_pool2d_t &c);
     thip_status_t emitAdd(const thip_hl_add_t &c);
@@ -645,6 +650,11 @@ thip_status_t Emitter::emitDepthwise(const thip_hl_depthwise_conv2d_t &c) {
 
 thip_status_t Emitter::emitFullyConnected(const thip_hl_fully_connected_t &c) {
     const char *what = "torq_hl.fully_connected";
+    {
+        const Value *xin;
+        if (thip_status_t s = checkValue(c.input, "torq_hl.fully_connected input", &xin)) return s;
+        if (xin->dtype == THIP_DTYPE_BF16) return emitFullyConnectedBf16(c);
+    }
     if (c.weight_zp != 0) return fail(THIP_UNIMPLEMENTED, "%s: weight_zp must be 0", what);
     const Value *w;
     if (thip_status_t s = constantData(c.weights, "torq_hl.fully_connected weights", THIP_DTYPE_I8, &w)) return s;
@@ -652,7 +662,7 @@ thip_status_t Emitter::emitFullyConnected(const thip_hl_fully_connected_t &c) {
     const int64_t N = w->shape[0], K = w->shape[1];
     const Value *x;
     if (thip_status_t s = checkValue(c.input, "torq_hl.fully_connected input", &x)) return s;
-    if (x->dtype != THIP_DTYPE_I8) return fail(THIP_UNIMPLEMENTED, "%s: only int8 inputs", what);
+    if (x->dtype != THIP_DTYPE_I8) return fail(THIP_UNIMPLEMENTED, "%s: only int8 and bf16 inputs", what);
     if (x->rank < 1 || x->shape[x->rank - 1] != K) {
         // a flattened N,C,1,1 / N,1,1,C activation is accepted as M,K too
         if (K <= 0 || x->numel() % K != 0) return fail(THIP_INVALID_ARGUMENT, "%s: input does not end in K=%lld", what, (long long)K);
@@ -702,6 +712,7 @@ thip_status_t Emitter::emitMatmul(const thip_hl_matmul_t &c) {
     if (thip_status_t s = checkValue(c.input1, "torq_hl.matmul input1", &a)) return s;
     if (thip_status_t s = checkValue(c.input2, "torq_hl.matmul input2", &b)) return s;
     if (thip_status_t s = checkValue(c.init, "torq_hl.matmul init", &init)) return s;
+    if (a->dtype == THIP_DTYPE_BF16) return emitMatmulBf16(c);
     if (a->dtype != THIP_DTYPE_I8 || b->dtype != THIP_DTYPE_I8) return fail(THIP_UNIMPLEMENTED, "%s: only int8 inputs", what);
     if (a->rank < 2 || a->rank > 3 || b->rank < 2 || b->rank > 3) return fail(THIP_UNIMPLEMENTED, "%s: operands must have rank 2 or 3", what);
     if (state_[c.input1].nhwcOfNchw || state_[c.input2].nhwcOfNchw) return fail(THIP_UNIMPLEMENTED, "%s: N,C,H,W intermediates are not accepted", what);
@@ -777,6 +788,119 @@ thip_status_t Emitter::emitMatmul(const thip_hl_matmul_t &c) {
         o.weights = packed[(size_t)(Bb == 1 ? 0 : batch)];
         if (thip_status_t s = splitScaleBias(c.scale_bias, "torq_hl.matmul scale_bias", N, Np, true, &o.bias, &o.scale)) return s;
         ops_.push_back(o);
+    }
+    return THIP_OK;
+}
+
+
+// bf16 rows (compiler/torq/Utils/Kernel.h:626-632): float bias, no scale, no shift, float clamp.
+static thip_status_t checkFloatAct(const char *what, int32_t shift, int32_t zpA, int32_t zpB, int32_t zpOut) {
+    if (shift != 0) return fail(THIP_INVALID_ARGUMENT, "%s: bf16 has no rescale: shift must be 0", what);
+    if (zpA != 0 || zpB != 0 || zpOut != 0) return fail(THIP_INVALID_ARGUMENT, "%s: bf16 has no zero points", what);
+    return THIP_OK;
+}
+
+thip_status_t Emitter::emitFullyConnectedBf16(const thip_hl_fully_connected_t &c) {
+    const char *what = "torq_hl.fully_connected (bf16)";
+    if (thip_status_t s = checkFloatAct(what, c.shift_factor, c.input_zp, c.weight_zp, c.output_zp)) return s;
+    const Value *w, *x, *init, *b;
+    if (thip_status_t s = constantData(c.weights, "torq_hl.fully_connected weights", THIP_DTYPE_BF16, &w)) return s;
+    if (w->rank != 2) return fail(THIP_INVALID_ARGUMENT, "%s: weights must be N,K", what);
+    const int64_t N = w->shape[0], K = w->shape[1];
+    if (thip_status_t s = checkValue(c.input, "torq_hl.fully_connected input", &x)) return s;
+    if (K <= 0 || x->numel() % K != 0 || x->numel() == 0) return fail(THIP_INVALID_ARGUMENT, "%s: input does not end in K=%lld", what, (long long)K);
+    if (K % 8 != 0) return fail(THIP_UNIMPLEMENTED, "%s: K must be a multiple of 8", what);
+    if (state_[c.input].nhwcOfNchw) return fail(THIP_UNIMPLEMENTED, "%s: N,C,H,W intermediates are not accepted", what);
+    const int64_t M = x->numel() / K;
+    if (thip_status_t s = checkValue(c.init, "torq_hl.fully_connected init", &init)) return s;
+    if (init->dtype != THIP_DTYPE_BF16) return fail(THIP_INVALID_ARGUMENT, "%s: init must be bf16", what);
+    if (thip_status_t s = constantData(c.scale_bias, "torq_hl.fully_connected scale_bias", THIP_DTYPE_F32, &b)) return s;
+    if (b->numel() < N) return fail(THIP_INVALID_ARGUMENT, "%s: scale_bias holds %lld floats, %lld needed", what, (long long)b->numel(), (long long)N);
+    if (!fitsInt32(M) || !fitsInt32(K) || !fitsInt32(N) || !fitsInt32(M * N) || !fitsInt32(M * K)) {
+        return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
+    }
+    DescOp op;
+    memset(&op, 0, sizeof(op));
+    op.kind = kKindFcBf16;
+    if (thip_status_t s = literalInput(c.input, "torq_hl.fully_connected input", &op.in0)) return s;
+    if (thip_status_t s = literalOutput(c.init, "torq_hl.fully_connected init", THIP_DTYPE_BF16, M * N, &op.out)) return s;
+    op.out_dtype = THIP_DTYPE_BF16;
+    op.output_min = c.output_min;
+    op.output_max = c.output_max;
+    op.M = (int32_t)M; op.K = (int32_t)K; op.Kp = (int32_t)K; op.Nn = (int32_t)N; op.Np = (int32_t)N;
+    op.weights = newConst(w->data);
+    std::vector<uint8_t> bias(b->data.begin(), b->data.begin() + (size_t)N * 4);
+    op.bias = newConst(bias);
+    ops_.push_back(op);
+    return THIP_OK;
+}
+
+thip_status_t Emitter::emitMatmulBf16(const thip_hl_matmul_t &c) {
+    const char *what = "torq_hl.matmul (bf16)";
+    if (thip_status_t s = checkFloatAct(what, c.shift, 0, 0, c.output_zp)) return s;
+    const Value *a, *b, *init, *bv;
+    if (thip_status_t s = checkValue(c.input1, "torq_hl.matmul input1", &a)) return s;
+    if (thip_status_t s = checkValue(c.input2, "torq_hl.matmul input2", &b)) return s;
+    if (thip_status_t s = checkValue(c.init, "torq_hl.matmul init", &init)) return s;
+    if (b->dtype != THIP_DTYPE_BF16 || init->dtype != THIP_DTYPE_BF16) return fail(THIP_INVALID_ARGUMENT, "%s: input2 and init must be bf16", what);
+    if (a->rank < 2 || a->rank > 3 || b->rank < 2 || b->rank > 3) return fail(THIP_UNIMPLEMENTED, "%s: operands must have rank 2 or 3", what);
+    if (state_[c.input1].nhwcOfNchw || state_[c.input2].nhwcOfNchw) return fail(THIP_UNIMPLEMENTED, "%s: N,C,H,W intermediates are not accepted", what);
+    const int64_t Ba = a->rank == 3 ? a->shape[0] : 1, Bb = b->rank == 3 ? b->shape[0] : 1;
+    const int64_t M = a->shape[a->rank - 2], K = a->shape[a->rank - 1];
+    const int64_t K2 = b->shape[b->rank - 2], N = b->shape[b->rank - 1];
+    if (K != K2) return fail(THIP_INVALID_ARGUMENT, "%s: inner dimensions differ (%lld vs %lld)", what, (long long)K, (long long)K2);
+    if (K % 8 != 0) return fail(THIP_UNIMPLEMENTED, "%s: K must be a multiple of 8", what);
+    const int64_t B = std::max(Ba, Bb);
+    if ((Ba != B && Ba != 1) || (Bb != B && Bb != 1)) return fail(THIP_INVALID_ARGUMENT, "%s: batch dimensions do not broadcast", what);
+    if (thip_status_t s = constantData(c.scale_bias, "torq_hl.matmul scale_bias", THIP_DTYPE_F32, &bv)) return s;
+    if (bv->numel() < 1) return fail(THIP_INVALID_ARGUMENT, "%s: scale_bias is empty", what);
+    if (!fitsInt32(B * M * N) || !fitsInt32(B * M * K) || !fitsInt32(B * K * N)) return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
+    const float bias0 = ((const float *)bv->data.data())[0];
+    DescRef biasRef = newConst(std::vector<float>((size_t)N, bias0));
+    DescRef aRef, outRef;
+    if (thip_status_t s = literalInput(c.input1, "torq_hl.matmul input1", &aRef)) return s;
+    if (thip_status_t s = literalOutput(c.init, "torq_hl.matmul init", THIP_DTYPE_BF16, B * M * N, &outRef)) return s;
+    // input2 as [N][K] per batch: transposed here when it is a constant, by a kernel when it is not
+    std::vector<DescRef> wrefs;
+    const int64_t wcount = Bb == 1 ? 1 : B;
+    if (b->kind == kValueConstant) {
+        const uint16_t *bd = (const uint16_t *)b->data.data();
+        for (int64_t r = 0; r < wcount; r++) {
+            std::vector<uint16_t> t((size_t)(N * K));
+            for (int64_t k = 0; k < K; k++) {
+                for (int64_t n = 0; n < N; n++) t[(size_t)(n * K + k)] = bd[(size_t)(r * K * N + k * N + n)];
+            }
+            wrefs.push_back(newConst(t));
+        }
+    } else {
+        DescRef bRef;
+        if (thip_status_t s = literalInput(c.input2, "torq_hl.matmul input2", &bRef)) return s;
+        for (int64_t r = 0; r < wcount; r++) {
+            DescRef t = newTemp((uint64_t)(N * K) * 2);
+            DescRef src = bRef;
+            src.offset += (uint64_t)(r * K * N) * 2;
+            emitTranspose(src, t, 1, K, N, 2);
+            wrefs.push_back(t);
+        }
+    }
+    // one record per batch, or a single one over all rows when input2 is shared
+    const bool merge = Bb == 1;
+    for (int64_t r = 0; r < (merge ? 1 : B); r++) {
+        DescOp op;
+        memset(&op, 0, sizeof(op));
+        op.kind = kKindFcBf16;
+        op.out_dtype = THIP_DTYPE_BF16;
+        op.output_min = c.output_min;
+        op.output_max = c.output_max;
+        const int64_t rows = merge ? (Ba == 1 ? M : B * M) : M;
+        op.M = (int32_t)rows; op.K = (int32_t)K; op.Kp = (int32_t)K; op.Nn = (int32_t)N; op.Np = (int32_t)N;
+        op.in0 = aRef;
+        op.in0.offset += (uint64_t)(Ba == 1 ? 0 : r * M * K) * 2;
+        op.out = outRef;
+        op.out.offset += (uint64_t)(r * M * N) * 2;
+        op.weights = wrefs[(size_t)(merge ? 0 : r)];
+        op.bias = biasRef;
+        ops_.push_back(op);
     }
     return THIP_OK;
 }

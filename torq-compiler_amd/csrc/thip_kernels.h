@@ -93,6 +93,17 @@ struct FcSkinnyArgs {
 constexpr int kFcSkinnyMaxRows = 16;
 hipError_t launchFcSkinny(const FcSkinnyArgs &a, hipStream_t stream);
 
+// bf16 fully_connected: out[m][n] = bf16(clamp(sum_k x[m][k] * w[n][k] + bias[n])), fp32 accumulate.
+struct FcBf16Args {
+    const uint16_t *x;  // [M][K] bf16 bit patterns
+    const uint16_t *w;  // [N][K]
+    const float *bias;  // [N]
+    uint16_t *out;      // [M][N]
+    int32_t M, K, N;
+    float lo, hi;       // clamp (-inf / +inf for none)
+};
+hipError_t launchFcBf16(const FcBf16Args &a, hipStream_t stream);
+
 struct DepthwiseArgs {
     const int8_t *in;     // NHWC
     const int8_t *wpk;    // variant 0: [KH][KW][C] bytes; variant 1: [KH][C] dwords, byte kw of a dword = tap kw
@@ -141,6 +152,7 @@ struct TransposeArgs {
     const int8_t *in;  // [B][R][S]
     int8_t *out;       // [B][S][R]
     int32_t B, R, S;
+    int32_t elem;      // element size in bytes: 1 or 2
 };
 hipError_t launchTranspose(const TransposeArgs &a, hipStream_t stream);
 

@@ -1854,8 +1854,9 @@ hipError_t launchAdd(const AddArgs &a, hipStream_t stream) {
 }
 
 // Batched byte transpose [B][R][S] -> [B][S][R] through a 64 x 64 LDS tile.
+template <typename T>
 __global__ __launch_bounds__(256) void transpose_i8(TransposeArgs p) {
-    __shared__ int8_t tile[64][65];
+    __shared__ T tile[64][65];
     const int tilesS = (p.S + 63) / 64, tilesR = (p.R + 63) / 64;
     int bid = (int)blockIdx.x;
     const int ts = bid % tilesS;
@@ -1863,8 +1864,8 @@ __global__ __launch_bounds__(256) void transpose_i8(TransposeArgs p) {
     const int tr = bid % tilesR;
     const int b = bid / tilesR;
     const int r0 = tr * 64, s0 = ts * 64;
-    const int8_t *src = p.in + (size_t)b * p.R * p.S;
-    int8_t *dst = p.out + (size_t)b * p.R * p.S;
+    const T *src = (const T *)p.in + (size_t)b * p.R * p.S;
+    T *dst = (T *)p.out + (size_t)b * p.R * p.S;
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
     for (int r = ty; r < 64; r += 4) {
         if (r0 + r < p.R && s0 + tx < p.S) tile[r][tx] = src[(size_t)(r0 + r) * p.S + s0 + tx];
@@ -1876,10 +1877,107 @@ __global__ __launch_bounds__(256) void transpose_i8(TransposeArgs p) {
 }
 
 hipError_t launchTranspose(const TransposeArgs &a, hipStream_t stream) {
-    if (a.B <= 0 || a.R <= 0 || a.S <= 0 || !a.in || !a.out) return hipErrorInvalidValue;
+    if (!a.in || !a.out || a.B <= 0 || a.R <= 0 || a.S <= 0 || (a.elem != 1 && a.elem != 2)) return hipErrorInvalidValue;
+    if (a.elem == 2 && ((((uintptr_t)a.in) | ((uintptr_t)a.out)) & 1)) return hipErrorInvalidValue;
     const long long blocks = (long long)a.B * ((a.R + 63) / 64) * ((a.S + 63) / 64);
     if (blocks >= (1LL << 31)) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(transpose_i8, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+    if (a.elem == 2) {
+        hipLaunchKernelGGL(transpose_i8<uint16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+    } else {
+        hipLaunchKernelGGL(transpose_i8<int8_t>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+    }
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------
+// fc_bf16: bf16 fully_connected / matmul with the weights streamed once per 32 rows of the input
+// (decode-shaped: few rows, weight traffic dominates).  A block owns 32 output columns of 32 input
+// rows; its four waves split K and add their fp32 partial sums through LDS.
+// v_mfma_f32_32x32x16_bf16, weights as the first operand: register r of lane l ends up with
+// out[m = l & 31][n = 8 (r / 4) + 4 (l >> 5) + (r & 3)].  Per 64 elements of K a lane loads 64
+// contiguous bytes of one weight row and of one input row (lane l: row l & 31, elements
+// 32 (l >> 5) .. + 31 of the 64) and MFMA step c takes 16-byte piece c of every lane: the k order
+// inside the 64 is permuted, identically for both operands, so that a wave's loads cover whole
+// 128-byte stretches of 32 rows.  fp32 products of bf16 values are exact; only the order of the
+// additions differs from a sequential sum.  K % 8 == 0.
+// ---------------------------------------------------------------------------
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ uint16_t bf16Bits(float f) {
+    const uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);  // NaN stays NaN
+    return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);                      // nearest, ties to even
+}
+
+__global__ __launch_bounds__(256) void fc_bf16(FcBf16Args p) {
+    __shared__ float partial[3][16][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 31, h = lane >> 5;
+    const int n0 = blockIdx.x * 32, m0 = blockIdx.y * 32;
+    const int nrow = n0 + r < p.N ? n0 + r : p.N - 1;  // clamped rows are never stored
+    const int mrow = m0 + r < p.M ? m0 + r : p.M - 1;
+    const uint16_t *wrow = p.w + (size_t)nrow * p.K;
+    const uint16_t *xrow = p.x + (size_t)mrow * p.K;
+    const int steps = (p.K + 63) / 64, per = (steps + 3) / 4;
+    const int sBeg = wave * per, sEnd = (sBeg + per) < steps ? (sBeg + per) : steps;
+    v16f acc;
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[e] = 0.0f;
+    for (int s = sBeg; s < sEnd; s++) {
+        const int k = s * 64 + 32 * h;
+        v4i wv[4], xv[4];
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const bool in = k + 8 * c < p.K;  // K % 8 == 0: a piece is inside K or outside
+            wv[c] = in ? *(const v4i *)(wrow + k + 8 * c) : v4i{0, 0, 0, 0};
+            xv[c] = in ? *(const v4i *)(xrow + k + 8 * c) : v4i{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, wv[c]), __builtin_bit_cast(v8bf, xv[c]), acc, 0, 0, 0);
+        }
+    }
+    if (wave > 0) {
+#pragma unroll
+        for (int e = 0; e < 16; e++) partial[wave - 1][e][lane] = acc[e];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 0; w < 3; w++) {
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[e] += partial[w][e][lane];
+    }
+    const int m = m0 + r;
+    if (m >= p.M) return;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int n = n0 + 8 * q + 4 * h;
+        uint16_t o[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int ne = n + e < p.N ? n + e : p.N - 1;
+            const float t0 = acc[4 * q + e] + p.bias[ne];
+            o[e] = bf16Bits(t0 < p.lo ? p.lo : (t0 > p.hi ? p.hi : t0));
+        }
+        if ((p.N & 3) == 0 && n + 3 < p.N) {
+            *(v2i *)(p.out + (size_t)m * p.N + n) = v2i{(int)((uint32_t)o[0] | ((uint32_t)o[1] << 16)), (int)((uint32_t)o[2] | ((uint32_t)o[3] << 16))};
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                if (n + e < p.N) p.out[(size_t)m * p.N + n + e] = o[e];
+            }
+        }
+    }
+}
+
+hipError_t launchFcBf16(const FcBf16Args &a, hipStream_t stream) {
+    if (!a.x || !a.w || !a.bias || !a.out || a.M <= 0 || a.N <= 0 || a.K <= 0 || a.K % 8 != 0) return hipErrorInvalidValue;
+    if (((((uintptr_t)a.x) | ((uintptr_t)a.w)) & 15) || (((uintptr_t)a.out) & (a.N % 4 == 0 ? 7 : 1)) || (((uintptr_t)a.bias) & 3)) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)((a.N + 31) / 32), (unsigned)((a.M + 31) / 32));
+    if (grid.y > 65535) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(fc_bf16, grid, dim3(256), 0, stream, a);
     return hipGetLastError();
 }
 

@@ -27,8 +27,10 @@ STATUS_NAMES = {
     UNIMPLEMENTED: "UNIMPLEMENTED", INTERNAL: "INTERNAL", UNAVAILABLE: "UNAVAILABLE",
 }
 
-DTYPE_I8, DTYPE_I16, DTYPE_I32 = 1, 2, 3
-_NP_TO_DTYPE = {np.dtype(np.int8): DTYPE_I8, np.dtype(np.int16): DTYPE_I16, np.dtype(np.int32): DTYPE_I32}
+DTYPE_I8, DTYPE_I16, DTYPE_I32, DTYPE_BF16, DTYPE_F32 = 1, 2, 3, 4, 5
+# numpy has no bfloat16: uint16 arrays carry bf16 bit patterns
+_NP_TO_DTYPE = {np.dtype(np.int8): DTYPE_I8, np.dtype(np.int16): DTYPE_I16, np.dtype(np.int32): DTYPE_I32,
+                np.dtype(np.uint16): DTYPE_BF16, np.dtype(np.float32): DTYPE_F32}
 _DTYPE_TO_NP = {v: k for k, v in _NP_TO_DTYPE.items()}
 
 BINDING_HOST, BINDING_DEVICE = 0, 1

@@ -143,6 +143,8 @@ class Program:
         scale_bias = self._as_value(scale_bias)
         N, K = weights.shape
         M = int(np.prod(input.shape)) // K
+        if input.dtype == np.uint16:  # bf16 bit patterns in, bf16 out
+            out_dtype = np.uint16
         init = self._init_or_new(init, (M, N), out_dtype)
         op = rt.HlFullyConnected(init.index, input_zp, weight_zp, output_zp, output_min, output_max,
                                  shift_factor, vectorization_mode, weights.index, scale_bias.index,
@@ -160,6 +162,8 @@ class Program:
             b2 = input2.shape[0] if len(input2.shape) == 3 else 1
             batch = (max(b1, b2),)
         shape = batch + (input1.shape[-2], input2.shape[-1])
+        if input1.dtype == np.uint16:  # bf16 bit patterns in, bf16 out
+            out_dtype = np.uint16
         init = self._init_or_new(init, shape, out_dtype)
         op = rt.HlMatmul(init.index, output_zp, output_min, output_max, shift, scale_bias.index,
                          input1.index, input2.index)

@@ -108,6 +108,63 @@ def fully_connected_workload(M, K, N, realistic=False, output_zp=5, output_min=-
                     bytes_, attrs)
 
 
+def to_bf16(values):
+    """float32 array -> bfloat16 bit patterns (uint16), round to nearest even."""
+    f = np.ascontiguousarray(values, dtype=np.float32)
+    u = f.reshape(-1).view(np.uint32).astype(np.uint64)
+    r = ((u + 0x7fff + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    nan = (u & 0x7fffffff) > 0x7f800000
+    r[nan] = ((u[nan] >> 16) | 0x40).astype(np.uint16)
+    return r.reshape(f.shape)
+
+
+NO_CLAMP = (-8388608, 0x7f800000)  # float bit patterns of -inf / +inf, as the int32 attributes carry them
+
+
+def float_bits(value):
+    """The int32 attribute that carries a float clamp bound."""
+    return int(np.array([value], dtype=np.float32).view(np.int32)[0])
+
+
+def fully_connected_bf16_workload(M, K, N, seed=1010, clamp=None):
+    """bf16 fully_connected (a linear layer of a decoder at M tokens): fp32 accumulate, float bias, bf16 out."""
+    rng = np.random.default_rng(seed)
+    x = to_bf16(rng.standard_normal((M, K)))
+    w = to_bf16(rng.standard_normal((N, K)) / np.sqrt(K))
+    bias = rng.standard_normal(N).astype(np.float32)
+    lo, hi = NO_CLAMP if clamp is None else (float_bits(clamp[0]), float_bits(clamp[1]))
+    attrs = dict(output_min=lo, output_max=hi)
+    p = Program()
+    inp = p.binding(0, (M, K), np.uint16)
+    out = p.binding(1, (M, N), np.uint16)
+    p.fully_connected(inp, w, bias, init=out, output_zp=0, shift_factor=0, input_zp=0, **attrs)
+    bytes_ = x.nbytes + w.nbytes + bias.nbytes + 2 * M * N
+    attrs.update(weights=w, bias=bias)
+    return Workload("fcbf16_%dx%dx%d" % (M, K, N), p, [x], [((M, N), np.uint16)], 2 * M * K * N, bytes_, attrs)
+
+
+def matmul_bf16_workload(B, M, K, N, batch1=True, batch2=True, constant_rhs=False, seed=1011, bias=0.0):
+    """bf16 matmul [B,]M,K x [B,]K,N with one float bias; input2 a run-time binding unless constant_rhs."""
+    rng = np.random.default_rng(seed)
+    a = to_bf16(rng.standard_normal((B, M, K) if batch1 else (M, K)))
+    b = to_bf16(rng.standard_normal((B, K, N) if batch2 else (K, N)) / np.sqrt(K))
+    bv = np.array([bias], dtype=np.float32)
+    p = Program()
+    ia = p.binding(0, a.shape, np.uint16)
+    inputs = [a]
+    if constant_rhs:
+        ib = b
+    else:
+        ib = p.binding(1, b.shape, np.uint16)
+        inputs.append(b)
+    oshape = ((B,) if (batch1 or batch2) else ()) + (M, N)
+    out = p.binding(len(inputs), oshape, np.uint16)
+    p.matmul(ia, ib, bv, init=out, output_zp=0, output_min=NO_CLAMP[0], output_max=NO_CLAMP[1], shift=0)
+    attrs = dict(input2=b, bias=bv)
+    return Workload("matmulbf16_%dx%dx%dx%d" % (B, M, K, N), p, inputs, [(oshape, np.uint16)], 2 * B * M * K * N,
+                    a.nbytes + b.nbytes + 2 * int(np.prod(oshape)), attrs)
+
+
 def depthwise_workload(N=1, H=56, W=56, C=144, KH=3, KW=3, stride=(2, 2), pad=(0, 1, 0, 1), input_zp=-3,
                        output_zp=5, output_min=-128, output_max=127, realistic=True, nhwc=True, seed=1002):
     """BASELINE config 2a: depthwise 3x3 stride 2 SAME on 56x56x144."""
