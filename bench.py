@@ -48,6 +48,10 @@ def workload_table(pkg):
         "avgpool_b1": (lambda: w.avgpool_workload(N=1), "hbm"),
         "add_b64": (lambda: w.add_workload(N=64), "hbm"),
         "add_b1": (lambda: w.add_workload(N=1), "hbm"),
+        # bf16 linears of a decoder layer (hidden 1152, MLP 6912) at 1 and 32 tokens: weight streaming
+        "fcbf16_1x1152x6912": (lambda: w.fully_connected_bf16_workload(1, 1152, 6912), "hbm"),
+        "fcbf16_32x1152x6912": (lambda: w.fully_connected_bf16_workload(32, 1152, 6912), "hbm"),
+        "fcbf16_32x6912x1152": (lambda: w.fully_connected_bf16_workload(32, 6912, 1152), "hbm"),
     }
 
 
@@ -125,6 +129,16 @@ def verify_sample(loaded):
         rows = np.unique(np.r_[0:16, M // 2:M // 2 + 16, M - 16:M])
         want = orc.fully_connected(wl.inputs[0][rows], wts, sb, **a)
         return bool(np.array_equal(got[rows], want))
+    if wl.name.startswith("fcbf16"):
+        # tolerance row: one bf16 ULP, or the fp32 reordering error where the sum cancels
+        from helpers import assert_bf16_close
+        f = lambda bits: np.abs(orc.from_bf16(bits).astype(np.float64))
+        mag = f(wl.inputs[0]) @ f(wl.attrs["weights"]).T + np.abs(wl.attrs["bias"])
+        try:
+            assert_bf16_close(got, oracle_eval(wl)[0], wl.name, magnitude=mag)
+        except AssertionError:
+            return False
+        return True
     return bool(np.array_equal(got, oracle_eval(wl)[0]))
 
 
@@ -247,7 +261,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "int8",
+        "dtype": "bf16" if args.workload.startswith("fcbf16") else "int8",
         "data": "synthetic",
         "config": {"workload": args.workload, "kernels": kernels, "parity_checked": ok,
                    "algorithmic_ops": wl.ops, "algorithmic_bytes": wl.bytes},

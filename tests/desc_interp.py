@@ -193,7 +193,14 @@ def run(blob, binding_arrays):
         elif kind == K_FC_BF16:
             M, K, N = int(op["M"]), int(op["K"]), int(op["Nn"])
             x = view(op["in0"], M * K * 2).view(np.uint16).reshape(M, K)
-            wt = view(op["weights"], N * K * 2).view(np.uint16).reshape(N, K)
+            if int(op["loader"]) == 1:  # fragment order: [column block][k step][piece][lane] x 8 elements
+                steps, nbk = (K + 63) // 64, (N + 31) // 32
+                frag = view(op["weights"], nbk * 32 * steps * 64 * 2).view(np.uint16).reshape(nbk, steps, 4, 2, 32, 8)
+                full = frag.transpose(0, 4, 1, 3, 2, 5).reshape(nbk * 32, steps * 64)  # [nb, r][s, h, c, e]
+                assert not full[N:].any() and not full[:, K:].any()
+                wt = np.ascontiguousarray(full[:N, :K])
+            else:
+                wt = view(op["weights"], N * K * 2).view(np.uint16).reshape(N, K)
             bias = view(op["bias"], N * 4).view(np.float32)
             res = orc.fully_connected_bf16(x, wt, bias, output_min=mn, output_max=mx)
             view(op["out"], M * N * 2).view(np.uint16)[:] = res.reshape(-1)

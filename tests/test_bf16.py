@@ -130,6 +130,23 @@ def test_gpu_bf16_fully_connected(device):
 
 
 @pytest.mark.gpu
+def test_gpu_bf16_split_k_is_deterministic(device):
+    """Few output tiles and a long K: K is split over blocks whose partial sums the last block to arrive adds in a
+    fixed order; repeated dispatches give the same bits, and the counters are back at zero for the next one."""
+    wl = w.fully_connected_bf16_workload(32, 6912, 1152)
+    d = desc_interp.Descriptor(wl.program.serialize())
+    assert int(d.ops[0]["w0"]) > 1
+    first = _check_gpu(device, wl, via="device")
+    exe = Executable(device, wl.program.serialize())
+    for _ in range(5):
+        out = np.zeros_like(first)
+        exe.run_host([wl.inputs[0], out])
+        assert np.array_equal(out, first)
+    exe.close()
+    _check_gpu(device, w.fully_connected_bf16_workload(3, 1152, 40))
+
+
+@pytest.mark.gpu
 def test_gpu_bf16_matmul(device):
     """Attention-shaped matmuls (4 query heads sharing one K / V, length 1024, head size 256) with a run-time input2,
     per-batch input2, and a constant input2."""

@@ -253,8 +253,15 @@ static thip_status_t checkOpFootprint(const thip_executable_t *e, uint32_t i) {
     case kKindFcBf16: {
         if (!positive({op.M, op.K, op.Nn}) || op.K % 8 != 0) return fail(THIP_INVALID_ARGUMENT, "op %u: bad bf16 fully_connected extents", i);
         if ((s = need(op.in0, (uint64_t)op.M * op.K * 2, "in"))) return s;
-        if ((s = need(op.weights, (uint64_t)op.Nn * op.K * 2, "weights"))) return s;
+        if (op.loader > 1) return fail(THIP_INVALID_ARGUMENT, "op %u: unknown bf16 weight layout %u", i, op.loader);
+        const uint64_t wBytes = op.loader == 1 ? (uint64_t)((op.Nn + 31) / 32 * 32) * ((op.K + 63) / 64 * 64) * 2 : (uint64_t)op.Nn * op.K * 2;
+        if ((s = need(op.weights, wBytes, "weights"))) return s;
         if ((s = need(op.bias, (uint64_t)op.Nn * 4, "bias"))) return s;
+        if (op.w0 > 1) {
+            // K split over blocks: counters and partial sums live in an intermediate (zero-filled at creation)
+            if (op.w0 > 64 || op.in1.space != kSpaceTemp) return fail(THIP_INVALID_ARGUMENT, "op %u: bad split-K workspace", i);
+            if ((s = need(op.in1, fcBf16WorkspaceBytes(op.M, op.Nn, op.w0), "workspace"))) return s;
+        }
         return need(op.out, (uint64_t)op.M * op.Nn * 2, "out");
     }
     default: return fail(THIP_INVALID_ARGUMENT, "op %u has unknown kind %u", i, op.kind);
@@ -361,7 +368,8 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
         memcpy(&lo, &op.output_min, 4);
         memcpy(&hi, &op.output_max, 4);
         FcBf16Args a{(const uint16_t *)resolve(e, op.in0, bp), (const uint16_t *)resolve(e, op.weights, bp),
-                     (const float *)resolve(e, op.bias, bp), (uint16_t *)resolve(e, op.out, bp), op.M, op.K, op.Nn, lo, hi};
+                     (const float *)resolve(e, op.bias, bp), (uint16_t *)resolve(e, op.out, bp), op.M, op.K, op.Nn, lo, hi,
+                     op.w0 > 1 ? op.w0 : 1, op.w0 > 1 ? (void *)resolve(e, op.in1, bp) : nullptr, (int32_t)op.loader};
         err = launchFcBf16(a, e->stream);
         break;
     }

@@ -479,6 +479,28 @@ class Emitter {
     thip_status_t emitDepthwise(const thip_hl_depthwise_conv2d_t &c);
     thip_status_t emitFullyConnected(const thip_hl_fully_connected_t &c);
     thip_status_t emitMatmul(const thip_hl_matmul_t &c);
+    // Few output tiles and a long K: split K over several blocks per tile; their partial sums and the
+    // tile counters live in an intermediate of the record's own (THIP_NO_SPLIT_K turns it off).
+    void planFcBf16Split(DescOp *op) {
+        const int split = getenv("THIP_NO_SPLIT_K") ? 1 : fcBf16PreferredSplit(op->M, op->Nn, op->K);
+        op->w0 = split;
+        if (split > 1) op->in1 = newTemp(fcBf16WorkspaceBytes(op->M, op->Nn, split));
+    }
+    // Constant bf16 weights [N][K] in the order the kernel's wave loads read them (THIP_BF16_ROW_MAJOR keeps rows).
+    void packBf16Weights(DescOp *op, const uint16_t *w, int64_t N, int64_t K) {
+        if (getenv("THIP_BF16_ROW_MAJOR")) {
+            op->loader = 0;
+            op->weights = newConst(std::vector<uint16_t>(w, w + N * K));
+            return;
+        }
+        const int steps = (int)((K + 63) / 64);
+        std::vector<uint8_t> packed((size_t)roundUp(N, 32) * (size_t)steps * 64 * 2, 0);
+        for (int64_t n = 0; n < N; n++) {
+            for (int64_t k = 0; k < K; k++) memcpy(&packed[fcBf16FragmentOffset((int)n, (int)k, steps)], &w[n * K + k], 2);
+        }
+        op->loader = 1;
+        op->weights = newConst(packed);
+    }
     thip_status_t emitFullyConnectedBf16(const thip_hl_fully_connected_t &c);
     thip_status_t emitMatmulBf16(const thip_hl_matmul_t &c);
     thip_status_t emitMaxPool(const thip_hl_maxpool2d_t &c);
@@ -828,9 +850,10 @@ thip_status_t Emitter::emitFullyConnectedBf16(const thip_hl_fully_connected_t &c
     op.output_min = c.output_min;
     op.output_max = c.output_max;
     op.M = (int32_t)M; op.K = (int32_t)K; op.Kp = (int32_t)K; op.Nn = (int32_t)N; op.Np = (int32_t)N;
-    op.weights = newConst(w->data);
+    packBf16Weights(&op, (const uint16_t *)w->data.data(), N, K);
     std::vector<uint8_t> bias(b->data.begin(), b->data.begin() + (size_t)N * 4);
     op.bias = newConst(bias);
+    planFcBf16Split(&op);
     ops_.push_back(op);
     return THIP_OK;
 }
@@ -862,6 +885,7 @@ thip_status_t Emitter::emitMatmulBf16(const thip_hl_matmul_t &c) {
     if (thip_status_t s = literalOutput(c.init, "torq_hl.matmul init", THIP_DTYPE_BF16, B * M * N, &outRef)) return s;
     // input2 as [N][K] per batch: transposed here when it is a constant, by a kernel when it is not
     std::vector<DescRef> wrefs;
+    std::vector<std::vector<uint16_t>> wconst;
     const int64_t wcount = Bb == 1 ? 1 : B;
     if (b->kind == kValueConstant) {
         const uint16_t *bd = (const uint16_t *)b->data.data();
@@ -870,7 +894,7 @@ thip_status_t Emitter::emitMatmulBf16(const thip_hl_matmul_t &c) {
             for (int64_t k = 0; k < K; k++) {
                 for (int64_t n = 0; n < N; n++) t[(size_t)(n * K + k)] = bd[(size_t)(r * K * N + k * N + n)];
             }
-            wrefs.push_back(newConst(t));
+            wconst.push_back(std::move(t));
         }
     } else {
         DescRef bRef;
@@ -898,8 +922,13 @@ thip_status_t Emitter::emitMatmulBf16(const thip_hl_matmul_t &c) {
         op.in0.offset += (uint64_t)(Ba == 1 ? 0 : r * M * K) * 2;
         op.out = outRef;
         op.out.offset += (uint64_t)(r * M * N) * 2;
-        op.weights = wrefs[(size_t)(merge ? 0 : r)];
+        if (!wconst.empty()) {
+            packBf16Weights(&op, wconst[(size_t)(merge ? 0 : r)].data(), N, K);
+        } else {
+            op.weights = wrefs[(size_t)(merge ? 0 : r)];
+        }
         op.bias = biasRef;
+        planFcBf16Split(&op);
         ops_.push_back(op);
     }
     return THIP_OK;

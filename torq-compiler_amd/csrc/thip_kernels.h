@@ -96,12 +96,41 @@ hipError_t launchFcSkinny(const FcSkinnyArgs &a, hipStream_t stream);
 // bf16 fully_connected: out[m][n] = bf16(clamp(sum_k x[m][k] * w[n][k] + bias[n])), fp32 accumulate.
 struct FcBf16Args {
     const uint16_t *x;  // [M][K] bf16 bit patterns
-    const uint16_t *w;  // [N][K]
+    const uint16_t *w;  // [N][K], or in fragment order (w_fragments)
     const float *bias;  // [N]
     uint16_t *out;      // [M][N]
     int32_t M, K, N;
     float lo, hi;       // clamp (-inf / +inf for none)
+    // K split over `ksplit` blocks per output tile (1 = no split).  workspace: one int32 counter per tile
+    // (zero before the first launch; the kernel leaves them zero), padded to 256 bytes, then
+    // tiles * ksplit * 1024 floats of partial sums.
+    int32_t ksplit;
+    void *workspace;
+    // weights in fragment order: for column block nb (32 columns), k-step s (64 elements) and piece c (0..3),
+    // 64 lanes x 16 bytes, lane l = column l & 31, elements 32 (l >> 5) + 8 c .. + 7 of the step; zero padded
+    // to whole blocks and steps.  One wave load is then 1 KiB of consecutive memory.
+    int32_t w_fragments;
 };
+// Byte offset of element (n, k) in the fragment order, for K padded to `steps` steps of 64.
+inline size_t fcBf16FragmentOffset(int n, int k, int steps) {
+    const int nb = n >> 5, r = n & 31, s = k >> 6, kk = k & 63, h = kk >> 5, c = (kk & 31) >> 3, e = kk & 7;
+    return ((((size_t)nb * steps + s) * 4 + c) * 64 + (size_t)(h * 32 + r)) * 16 + (size_t)e * 2;
+}
+// Bytes of workspace a launch with this split needs.
+inline size_t fcBf16WorkspaceBytes(int M, int N, int ksplit) {
+    const size_t tiles = (size_t)((N + 31) / 32) * ((M + 31) / 32);
+    return ksplit <= 1 ? 0 : (tiles * 4 + 255) / 256 * 256 + tiles * ksplit * 1024 * 4;
+}
+// The split the launcher's heuristics would like for this shape (the emitter allocates the workspace for it).
+inline int fcBf16PreferredSplit(int M, int N, int K) {
+    const long long tiles = (long long)((N + 31) / 32) * ((M + 31) / 32);
+    const int steps = (K + 63) / 64;
+    if (tiles >= 128 || steps < 8) return 1;
+    long long split = 256 / tiles;  // at most one block per CU: a second round would double the time
+    if (split > steps / 4) split = steps / 4;
+    if (split > 16) split = 16;
+    return split < 2 ? 1 : (int)split;
+}
 hipError_t launchFcBf16(const FcBf16Args &a, hipStream_t stream);
 
 struct DepthwiseArgs {

@@ -1910,8 +1910,9 @@ __device__ __forceinline__ uint16_t bf16Bits(float f) {
     return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);                      // nearest, ties to even
 }
 
-__global__ __launch_bounds__(256) void fc_bf16(FcBf16Args p) {
-    __shared__ float partial[3][16][64];
+template <int NWAVES>  // waves of a block = ways K is split
+__global__ __launch_bounds__(NWAVES * 64) void fc_bf16(FcBf16Args p) {
+    __shared__ float partial[NWAVES - 1][16][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, h = lane >> 5;
     const int n0 = blockIdx.x * 32, m0 = blockIdx.y * 32;
@@ -1919,23 +1920,40 @@ __global__ __launch_bounds__(256) void fc_bf16(FcBf16Args p) {
     const int mrow = m0 + r < p.M ? m0 + r : p.M - 1;
     const uint16_t *wrow = p.w + (size_t)nrow * p.K;
     const uint16_t *xrow = p.x + (size_t)mrow * p.K;
-    const int steps = (p.K + 63) / 64, per = (steps + 3) / 4;
-    const int sBeg = wave * per, sEnd = (sBeg + per) < steps ? (sBeg + per) : steps;
+    // this block's slice of K (blockIdx.z of ksplit), then this wave's share of the slice
+    const int steps = (p.K + 63) / 64;
+    const int zBeg = (int)((long long)steps * blockIdx.z / p.ksplit), zEnd = (int)((long long)steps * (blockIdx.z + 1) / p.ksplit);
+    const int per = (zEnd - zBeg + NWAVES - 1) / NWAVES;
+    const int sBeg = zBeg + wave * per, sEnd = (sBeg + per) < zEnd ? (sBeg + per) : zEnd;
     v16f acc;
 #pragma unroll
     for (int e = 0; e < 16; e++) acc[e] = 0.0f;
-    for (int s = sBeg; s < sEnd; s++) {
-        const int k = s * 64 + 32 * h;
-        v4i wv[4], xv[4];
+    // UNR steps of loads are issued before their MFMAs: one memory round trip per UNR * 64 elements of K
+    constexpr int UNR = NWAVES > 4 ? 2 : 4;
+    for (int s0 = sBeg; s0 < sEnd; s0 += UNR) {
+        v4i wv[UNR][4], xv[UNR][4];
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            const bool in = k + 8 * c < p.K;  // K % 8 == 0: a piece is inside K or outside
-            wv[c] = in ? *(const v4i *)(wrow + k + 8 * c) : v4i{0, 0, 0, 0};
-            xv[c] = in ? *(const v4i *)(xrow + k + 8 * c) : v4i{0, 0, 0, 0};
+        for (int u = 0; u < UNR; u++) {
+            const int k = (s0 + u) * 64 + 32 * h;
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const bool in = s0 + u < sEnd && k + 8 * c < p.K;  // K % 8 == 0: a piece is inside K or outside
+                if (p.w_fragments) {
+                    // whole (zero padded) steps: every lane of the wave loads, 1 KiB in a row
+                    const int8_t *frag = (const int8_t *)p.w + ((((size_t)blockIdx.x * steps + (s0 + u)) * 4 + c) * 64 + lane) * 16;
+                    wv[u][c] = s0 + u < sEnd ? *(const v4i *)frag : v4i{0, 0, 0, 0};
+                } else {
+                    wv[u][c] = in ? *(const v4i *)(wrow + k + 8 * c) : v4i{0, 0, 0, 0};
+                }
+                xv[u][c] = in ? *(const v4i *)(xrow + k + 8 * c) : v4i{0, 0, 0, 0};
+            }
         }
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, wv[c]), __builtin_bit_cast(v8bf, xv[c]), acc, 0, 0, 0);
+        for (int u = 0; u < UNR; u++) {
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, wv[u][c]), __builtin_bit_cast(v8bf, xv[u][c]), acc, 0, 0, 0);
+            }
         }
     }
     if (wave > 0) {
@@ -1944,10 +1962,34 @@ __global__ __launch_bounds__(256) void fc_bf16(FcBf16Args p) {
     }
     __syncthreads();
     if (wave > 0) return;
-#pragma unroll
-    for (int w = 0; w < 3; w++) {
+    for (int w = 0; w < NWAVES - 1; w++) {
 #pragma unroll
         for (int e = 0; e < 16; e++) acc[e] += partial[w][e][lane];
+    }
+    if (p.ksplit > 1) {
+        // K split over blocks: every block leaves its partial tile in the workspace; the block that arrives
+        // last at the tile's counter adds them up in slice order (so the result does not depend on who was
+        // last), finishes the tile and puts the counter back to zero.  Nobody waits for anybody.
+        const int tile = blockIdx.y * gridDim.x + blockIdx.x, tiles = gridDim.x * gridDim.y;
+        int *counters = (int *)p.workspace;
+        float *parts = (float *)((char *)p.workspace + ((size_t)tiles * 4 + 255) / 256 * 256);
+        float *mine = parts + ((size_t)tile * p.ksplit + blockIdx.z) * 1024;
+#pragma unroll
+        for (int e = 0; e < 16; e++) mine[e * 64 + lane] = acc[e];
+        __threadfence();
+        int arrived = 0;
+        if (lane == 0) arrived = atomicAdd(&counters[tile], 1);
+        arrived = __shfl(arrived, 0, 64);
+        if (arrived != p.ksplit - 1) return;
+        __threadfence();
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[e] = 0.0f;
+        for (int z = 0; z < p.ksplit; z++) {
+            const float *part = parts + ((size_t)tile * p.ksplit + z) * 1024;
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[e] += __builtin_nontemporal_load(part + e * 64 + lane);
+        }
+        if (lane == 0) counters[tile] = 0;
     }
     const int m = m0 + r;
     if (m >= p.M) return;
@@ -1975,9 +2017,10 @@ __global__ __launch_bounds__(256) void fc_bf16(FcBf16Args p) {
 hipError_t launchFcBf16(const FcBf16Args &a, hipStream_t stream) {
     if (!a.x || !a.w || !a.bias || !a.out || a.M <= 0 || a.N <= 0 || a.K <= 0 || a.K % 8 != 0) return hipErrorInvalidValue;
     if (((((uintptr_t)a.x) | ((uintptr_t)a.w)) & 15) || (((uintptr_t)a.out) & (a.N % 4 == 0 ? 7 : 1)) || (((uintptr_t)a.bias) & 3)) return hipErrorInvalidValue;
-    const dim3 grid((unsigned)((a.N + 31) / 32), (unsigned)((a.M + 31) / 32));
+    if (a.ksplit < 1 || a.ksplit > 64 || (a.ksplit > 1 && (!a.workspace || ((uintptr_t)a.workspace & 255)))) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)((a.N + 31) / 32), (unsigned)((a.M + 31) / 32), (unsigned)a.ksplit);
     if (grid.y > 65535) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(fc_bf16, grid, dim3(256), 0, stream, a);
+    hipLaunchKernelGGL(fc_bf16<4>, grid, dim3(256), 0, stream, a);
     return hipGetLastError();
 }
 
