@@ -303,6 +303,56 @@ __device__ __forceinline__ void igemmEpilogueDirect(v16i (&acc)[WTN / 32][WTM / 
 }
 
 // ---------------------------------------------------------------------------
+// Linear work index -> (channel group, x, y, image).  A 64-bit division by a run-time divisor costs a
+// couple of hundred instructions, more than the whole body of a pooling thread, so the launchers
+// precompute multipliers: for n < 2^31 and a divisor d with s = ceil(log2 d),
+// n / d == umulhi(n, ceil(2^(31+s) / d)) >> (s - 1) (the multiplier fits 32 bits because
+// d > 2^(s-1)).  Work counts of 2^31 and more take the plain 64-bit path.
+// ---------------------------------------------------------------------------
+struct FastDiv {
+    uint32_t mul;    // 0: the divisor is 1
+    uint32_t shift;  // s - 1
+    uint32_t d;
+};
+static FastDiv makeFastDiv(uint32_t d) {
+    FastDiv f{0, 0, d};
+    if (d <= 1) return f;
+    uint32_t s = 0;
+    while ((1ull << s) < d) s++;
+    f.mul = (uint32_t)((((unsigned long long)1 << (31 + s)) + d - 1) / d);
+    f.shift = s - 1;
+    return f;
+}
+struct WorkSplit {
+    FastDiv cg, xs, ys;  // channel groups, x positions, y positions per image
+    int wide;            // the work count does not fit 31 bits
+};
+static WorkSplit makeWorkSplit(long long total, int cg, int xs, int ys) {
+    return WorkSplit{makeFastDiv((uint32_t)cg), makeFastDiv((uint32_t)xs), makeFastDiv((uint32_t)ys), total >= (1LL << 31)};
+}
+__device__ __forceinline__ uint32_t fastDiv(uint32_t n, const FastDiv &f) { return f.mul ? __umulhi(n, f.mul) >> f.shift : n; }
+__device__ __forceinline__ void splitWork(long long t, const WorkSplit &w, int &c, int &x, int &y, int &n) {
+    if (!w.wide) {
+        uint32_t u = (uint32_t)t, q = fastDiv(u, w.cg);
+        c = (int)(u - q * w.cg.d);
+        u = q;
+        q = fastDiv(u, w.xs);
+        x = (int)(u - q * w.xs.d);
+        u = q;
+        q = fastDiv(u, w.ys);
+        y = (int)(u - q * w.ys.d);
+        n = (int)q;
+    } else {
+        c = (int)(t % w.cg.d);
+        long long pix = t / w.cg.d;
+        x = (int)(pix % w.xs.d);
+        pix /= w.xs.d;
+        y = (int)(pix % w.ys.d);
+        n = (int)(pix / w.ys.d);
+    }
+}
+
+// ---------------------------------------------------------------------------
 // igemm_i8
 // ---------------------------------------------------------------------------
 //
@@ -1316,17 +1366,14 @@ union Pack {
 };
 
 template <int VEC, int KS>  // KS > 0: square KS x KS window known at compile time
-__global__ __launch_bounds__(256) void depthwise_i8(DepthwiseArgs p) {
+__global__ __launch_bounds__(256) void depthwise_i8(DepthwiseArgs p, WorkSplit ws) {
     const int cg = p.C / VEC;
     const long long total = (long long)p.N * p.OH * p.OW * cg;
     const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
     if (t >= total) return;
-    const int c0 = (int)(t % cg) * VEC;
-    long long pix = t / cg;
-    const int ox = (int)(pix % p.OW);
-    pix /= p.OW;
-    const int oy = (int)(pix % p.OH);
-    const int n = (int)(pix / p.OH);
+    int cgi, ox, oy, n;
+    splitWork(t, ws, cgi, ox, oy, n);
+    const int c0 = cgi * VEC;
     const int KH = KS > 0 ? KS : p.KH, KW = KS > 0 ? KS : p.KW;
     const int iy0 = oy * p.SH - p.PT, ix0 = ox * p.SW - p.PL;
     const int8_t *img = p.in + (size_t)n * p.H * p.W * p.C + c0;
@@ -1369,7 +1416,7 @@ __global__ __launch_bounds__(256) void depthwise_i8(DepthwiseArgs p) {
 // the kernel is bound by the traffic through the vector L1, not by arithmetic.
 // SWT is the horizontal stride when it is 1 or 2 (P > 1 needs it at compile time), 0 = run time.
 template <int P, int SWT>
-__global__ __launch_bounds__(256) void depthwise3x3_dot4_i8(DepthwiseArgs p) {
+__global__ __launch_bounds__(256) void depthwise3x3_dot4_i8(DepthwiseArgs p, WorkSplit ws) {
     static_assert(P == 1 || SWT > 0, "several pixels per thread need a compile-time stride");
     const int SW = SWT > 0 ? SWT : p.SW;
     constexpr int NC = SWT > 0 ? (P - 1) * SWT + 3 : 3;  // input columns one window row of the thread spans
@@ -1378,12 +1425,9 @@ __global__ __launch_bounds__(256) void depthwise3x3_dot4_i8(DepthwiseArgs p) {
     const long long total = (long long)p.N * p.OH * oxGroups * cg;
     const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
     if (t >= total) return;
-    const int c0 = (int)(t % cg) * 16;
-    long long pix = t / cg;
-    const int ox0 = (int)(pix % oxGroups) * P;
-    pix /= oxGroups;
-    const int oy = (int)(pix % p.OH);
-    const int n = (int)(pix / p.OH);
+    int cgi, oxg, oy, n;
+    splitWork(t, ws, cgi, oxg, oy, n);
+    const int c0 = cgi * 16, ox0 = oxg * P;
     const int iy0 = oy * p.SH - p.PT, ix0 = ox0 * SW - p.PL;
     const int8_t *img = p.in + (size_t)n * p.H * p.W * p.C + c0;
     const uint32_t zp4 = (uint32_t)(p.input_zp & 0xff) * 0x01010101u;
@@ -1453,7 +1497,8 @@ __global__ __launch_bounds__(256) void depthwise3x3_dot4_i8(DepthwiseArgs p) {
 template <int P, int SWT>
 static hipError_t launchDepthwiseDot4(const DepthwiseArgs &a, hipStream_t stream) {
     const long long total = (long long)a.N * a.OH * ((a.OW + P - 1) / P) * (a.C / 16);
-    hipLaunchKernelGGL((depthwise3x3_dot4_i8<P, SWT>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a);
+    const WorkSplit ws = makeWorkSplit(total, a.C / 16, (a.OW + P - 1) / P, a.OH);
+    hipLaunchKernelGGL((depthwise3x3_dot4_i8<P, SWT>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a, ws);
     return hipGetLastError();
 }
 
@@ -1491,7 +1536,7 @@ __device__ __forceinline__ void loadDwords(const int8_t *src, int (&dst)[G]) {
 // G = channels per thread / 4.  Fewer channels per thread mean fewer registers and more waves per SIMD
 // (the loads stay coalesced: neighbouring lanes hold neighbouring channel groups).
 template <int P, int R, int S, int G>
-__global__ __launch_bounds__(256) void depthwise3x3_tile_i8(DepthwiseArgs p) {
+__global__ __launch_bounds__(256) void depthwise3x3_tile_i8(DepthwiseArgs p, WorkSplit ws) {
     static_assert(S == 1 || S == 2, "stride 1 or 2");
     static_assert(S == 2 || P % 2 == 0, "stride 1 pairs the pixels of a block");
     constexpr int NC = (P - 1) * S + 3, NR = (R - 1) * S + 3;
@@ -1502,12 +1547,9 @@ __global__ __launch_bounds__(256) void depthwise3x3_tile_i8(DepthwiseArgs p) {
     const long long total = (long long)p.N * oyGroups * oxGroups * cg;
     const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
     if (t >= total) return;
-    const int c0 = (int)(t % cg) * CV;
-    long long pix = t / cg;
-    const int ox0 = (int)(pix % oxGroups) * P;
-    pix /= oxGroups;
-    const int oy0 = (int)(pix % oyGroups) * R;
-    const int n = (int)(pix / oyGroups);
+    int cgi, oxg, oyg, n;
+    splitWork(t, ws, cgi, oxg, oyg, n);
+    const int c0 = cgi * CV, ox0 = oxg * P, oy0 = oyg * R;
     const int iy0 = oy0 * S - p.PT, ix0 = ox0 * S - p.PL;
     const int8_t *img = p.in + (size_t)n * p.H * p.W * p.C + c0;
     const int zp4 = (int)((uint32_t)(p.input_zp & 0xff) * 0x01010101u);
@@ -1619,7 +1661,8 @@ __global__ __launch_bounds__(256) void depthwise3x3_tile_i8(DepthwiseArgs p) {
 template <int P, int R, int S, int G>
 static hipError_t launchDepthwiseTile(const DepthwiseArgs &a, hipStream_t stream) {
     const long long total = (long long)a.N * ((a.OH + R - 1) / R) * ((a.OW + P - 1) / P) * (a.C / (4 * G));
-    hipLaunchKernelGGL((depthwise3x3_tile_i8<P, R, S, G>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a);
+    const WorkSplit ws = makeWorkSplit(total, a.C / (4 * G), (a.OW + P - 1) / P, (a.OH + R - 1) / R);
+    hipLaunchKernelGGL((depthwise3x3_tile_i8<P, R, S, G>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a, ws);
     return hipGetLastError();
 }
 
@@ -1642,10 +1685,11 @@ template <int VEC>
 static hipError_t launchDepthwiseV(const DepthwiseArgs &a, hipStream_t stream) {
     const long long total = (long long)a.N * a.OH * a.OW * (a.C / VEC);
     const dim3 grid((unsigned)((total + 255) / 256));
+    const WorkSplit ws = makeWorkSplit(total, a.C / VEC, a.OW, a.OH);
     if (a.KH == 3 && a.KW == 3) {
-        hipLaunchKernelGGL((depthwise_i8<VEC, 3>), grid, dim3(256), 0, stream, a);
+        hipLaunchKernelGGL((depthwise_i8<VEC, 3>), grid, dim3(256), 0, stream, a, ws);
     } else {
-        hipLaunchKernelGGL((depthwise_i8<VEC, 0>), grid, dim3(256), 0, stream, a);
+        hipLaunchKernelGGL((depthwise_i8<VEC, 0>), grid, dim3(256), 0, stream, a, ws);
     }
     return hipGetLastError();
 }
@@ -1688,17 +1732,14 @@ hipError_t launchDepthwise(const DepthwiseArgs &a, hipStream_t stream) {
 }
 
 template <int VEC>
-__global__ __launch_bounds__(256) void maxpool_i8(MaxPoolArgs p) {
+__global__ __launch_bounds__(256) void maxpool_i8(MaxPoolArgs p, WorkSplit ws) {
     const int cg = p.C / VEC;
     const long long total = (long long)p.N * p.OH * p.OW * cg;
     const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
     if (t >= total) return;
-    const int c0 = (int)(t % cg) * VEC;
-    long long pix = t / cg;
-    const int ox = (int)(pix % p.OW);
-    pix /= p.OW;
-    const int oy = (int)(pix % p.OH);
-    const int n = (int)(pix / p.OH);
+    int cgi, ox, oy, n;
+    splitWork(t, ws, cgi, ox, oy, n);
+    const int c0 = cgi * VEC;
     const int iy0 = oy * p.SH - p.PT, ix0 = ox * p.SW - p.PL;
     const int8_t *img = p.in + (size_t)n * p.H * p.W * p.C + c0;
     int32_t best[VEC];
@@ -1735,7 +1776,8 @@ template <int VEC>
 static hipError_t launchMaxPoolV(const MaxPoolArgs &a, hipStream_t stream) {
     const long long total = (long long)a.N * a.OH * a.OW * (a.C / VEC);
     const dim3 grid((unsigned)((total + 255) / 256));
-    hipLaunchKernelGGL((maxpool_i8<VEC>), grid, dim3(256), 0, stream, a);
+    const WorkSplit ws = makeWorkSplit(total, a.C / VEC, a.OW, a.OH);
+    hipLaunchKernelGGL((maxpool_i8<VEC>), grid, dim3(256), 0, stream, a, ws);
     return hipGetLastError();
 }
 
