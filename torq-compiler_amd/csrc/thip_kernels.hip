@@ -245,8 +245,8 @@ __device__ __forceinline__ void igemmEpilogue(v16i (&acc)[WTN / 32][WTM / 32], i
     }
 }
 
-// The same epilogue without the LDS round trip, for int8 outputs with N % 16 == 0 and the 32-bit
-// requant tail: each accumulator tile is requantised in place, two v_permlane32_swap exchange
+// The same epilogue without the LDS round trip, for int8 outputs with N % 16 == 0 and the plain
+// 32-bit requant tail (no pre-shift, zero point folded into the rounding term): each accumulator tile is requantised in place, two v_permlane32_swap exchange
 // register groups between the wave halves so that a lane owns 16 consecutive channels of its row
 // (see igemm_stream_i8), and the lane stores them as one 128-bit word.  Only the (bias, scale)
 // vectors pass through LDS.
@@ -262,43 +262,35 @@ __device__ __forceinline__ void igemmEpilogueDirect(v16i (&acc)[WTN / 32][WTM / 
         ldsScale[tid] = myScale;
     }
     __syncthreads();
-    const WideRequant wrq = wideRequant(p.rq);
-    auto tiles = [&](auto plainTag) {
-        constexpr bool kPlain = decltype(plainTag)::value;
+    const WideRequant wrq = wideRequant(p.rq);  // plain (the launcher checks): no pre-shift, zero point folded
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
-            const int nl = wn * WTN + j * 32;  // first channel of this tile column, relative to n0
-            v4i b4[4], s4[4];
+    for (int j = 0; j < TN; j++) {
+        const int nl = wn * WTN + j * 32;  // first channel of this tile column, relative to n0
+        v4i b4[4], s4[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            b4[q] = *(const v4i *)(ldsBias + nl + 8 * q + 4 * half);
+            s4[q] = *(const v4i *)(ldsScale + nl + 8 * q + 4 * half);
+        }
+        const int n = n0 + nl + 16 * half;
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            uint32_t d4[4];
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-                b4[q] = *(const v4i *)(ldsBias + nl + 8 * q + 4 * half);
-                s4[q] = *(const v4i *)(ldsScale + nl + 8 * q + 4 * half);
-            }
-            const int n = n0 + nl + 16 * half;
+                int32_t v[4];
 #pragma unroll
-            for (int i = 0; i < TM; i++) {
-                uint32_t d4[4];
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    int32_t v[4];
-#pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        v[e] = requantWideT0<kPlain>((int32_t)((uint32_t)acc[j][i][4 * q + e] + (uint32_t)b4[q][e]), s4[q][e], wrq);
-                    }
-                    d4[q] = packBytes(v[0], v[1], v[2], v[3]);
+                for (int e = 0; e < 4; e++) {
+                    v[e] = requantWideT0<true>((int32_t)((uint32_t)acc[j][i][4 * q + e] + (uint32_t)b4[q][e]), s4[q][e], wrq);
                 }
-                const auto s02 = __builtin_amdgcn_permlane32_swap(d4[0], d4[2], false, false);
-                const auto s13 = __builtin_amdgcn_permlane32_swap(d4[1], d4[3], false, false);
-                const v4i outv = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
-                const int m = m0 + wm * WTM + i * 32 + fr;
-                if (m < p.M && n < p.N) *(v4i *)((int8_t *)p.out + (size_t)m * p.N + n) = outv;
+                d4[q] = packBytes(v[0], v[1], v[2], v[3]);
             }
+            const auto s02 = __builtin_amdgcn_permlane32_swap(d4[0], d4[2], false, false);
+            const auto s13 = __builtin_amdgcn_permlane32_swap(d4[1], d4[3], false, false);
+            const v4i outv = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
+            const int m = m0 + wm * WTM + i * 32 + fr;
+            if (m < p.M && n < p.N) *(v4i *)((int8_t *)p.out + (size_t)m * p.N + n) = outv;
         }
-    };
-    if (wrq.plain) {
-        tiles(std::true_type{});
-    } else {
-        tiles(std::false_type{});
     }
 }
 
@@ -654,7 +646,7 @@ __device__ __forceinline__ void waitVmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
-// DIRECT selects the epilogue: in registers (int8 output, N % 16 == 0, 32-bit requant tail: the launcher
+// DIRECT selects the epilogue: in registers (int8 output, N % 16 == 0, plain 32-bit requant tail: the launcher
 // checks) or staged through LDS (everything else).
 template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, bool DIRECT>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_dense_i8(IgemmArgs p) {
@@ -1131,8 +1123,11 @@ static hipError_t launchIgemmDenseE(const IgemmArgs &a, hipStream_t stream) {
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU>
 static hipError_t launchIgemmDense(const IgemmArgs &a, hipStream_t stream) {
-    const bool direct = a.out_dtype == kDtypeI8 && a.N % 16 == 0 && ((uintptr_t)a.out & 15) == 0 &&
-                        a.rq.shift + a.rq.pre_shift >= 33 && !getenv("THIP_NO_DIRECT_EPILOGUE");
+    // the in-register epilogue takes the plain 32-bit tail only (what wideRequant() calls plain)
+    const bool plain = a.rq.shift >= 33 && a.rq.shift <= 45 && a.rq.pre_shift == 0 && a.rq.t0_clamp == 0 &&
+                       a.rq.out_zp >= -32768 && a.rq.out_zp <= 32767 && a.rq.out_min <= a.rq.out_max;
+    const bool direct = a.out_dtype == kDtypeI8 && a.N % 16 == 0 && ((uintptr_t)a.out & 15) == 0 && plain &&
+                        !getenv("THIP_NO_DIRECT_EPILOGUE");
     return direct ? launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, true>(a, stream)
                   : launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, false>(a, stream);
 }
