@@ -215,7 +215,9 @@ typedef struct thip_hl_avg_pool2d_t {
 } thip_hl_avg_pool2d_t;
 
 /* torq_hl.add -- TorqHLOps.td:48-69.  weights int16[2]; scale_bias int32[2];
- * `name` is "add" or "sub" (the sign already lives in weights[1]). */
+ * `name` is "add" or "sub" (the sign already lives in weights[1]).
+ * bf16 form (inputs and init BF16): weights BF16[2], scale_bias F32[1] (bias only), shift_factor and
+ * zero points 0, output_min / output_max float bit patterns. */
 typedef struct thip_hl_add_t {
     thip_value_t init;
     const char *name;

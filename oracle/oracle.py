@@ -222,6 +222,20 @@ def matmul_bf16(input1, input2, bias, *, output_min=NO_CLAMP_MIN, output_max=NO_
     return out
 
 
+def add_bf16(input1, input2, weights, bias, *, output_min=NO_CLAMP_MIN, output_max=NO_CLAMP_MAX):
+    """torq_hl.add on bf16 bit patterns: two bf16 weights, one float32 bias."""
+    a = _c(input1, np.uint16)
+    b = _c(input2, np.uint16)
+    assert a.shape == b.shape
+    w = _c(weights, np.uint16)
+    bias = _c(bias, np.float32)
+    assert w.size >= 2 and bias.size >= 1
+    out = np.empty(a.shape, dtype=np.uint16)
+    rc = lib().torq_add_bf16(_p(a), _p(b), _p(w), _p(bias), _p(out), ctypes.c_size_t(a.size), int(output_min), int(output_max))
+    assert rc == 0
+    return out
+
+
 def maxpool2d(input, *, input_zp, output_min, output_max, stride, pad, kernel, layout=NCHW):
     """torq_hl.maxpool2d."""
     x = _c(input, np.int8)

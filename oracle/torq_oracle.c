@@ -314,6 +314,24 @@ int torq_matmul_bf16(const uint16_t *input1, const uint16_t *input2, const float
 }
 
 /*
+ * torq_hl.add on bf16 -- compiler/torq/Conversions/TorqHLToTorqHW/AddPattern.cpp:262-281 with floating-point
+ * partials: the two products (exact in fp32) are accumulated in tensor order, then the float ACT stage
+ * (one bias: biasScaleWidth is 1 for bf16, AddPattern.cpp:118-121,197-200).
+ */
+int torq_add_bf16(const uint16_t *input1, const uint16_t *input2, const uint16_t weights[2], const float *bias,
+                  uint16_t *out, size_t count, int32_t clip_min, int32_t clip_max) {
+    const float lo = float_from_bits(clip_min), hi = float_from_bits(clip_max);
+    const float w0 = torq_bf16_to_f32(weights[0]), w1 = torq_bf16_to_f32(weights[1]);
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < count; i++) {
+        float acc = torq_bf16_to_f32(input1[i]) * w0;
+        acc += torq_bf16_to_f32(input2[i]) * w1;
+        out[i] = act_float(acc, bias[0], lo, hi);
+    }
+    return 0;
+}
+
+/*
  * torq_hl.maxpool2d -- signature TorqHLOps.td:435-453; created
  * compiler/torq/Conversions/LinalgToTorqHL/PoolingPattern.cpp:199-236 (pad value
  * becomes input_zp, output_min/max = element type range); executed

@@ -91,6 +91,10 @@ int torq_fully_connected_bf16(const uint16_t *input, const uint16_t *weights, co
 int torq_matmul_bf16(const uint16_t *input1, const uint16_t *input2, const float *bias, uint16_t *out,
                      int B, int M, int K, int N, int bcast1, int bcast2, int32_t clip_min, int32_t clip_max);
 
+/* torq_hl.add on bf16: out = bf16(clamp(in1 * w[0] + in2 * w[1] + bias)), two bf16 weights, ONE float bias. */
+int torq_add_bf16(const uint16_t *input1, const uint16_t *input2, const uint16_t weights[2], const float *bias,
+                  uint16_t *out, size_t count, int32_t clip_min, int32_t clip_max);
+
 /* torq_hl.maxpool2d.  No rescale; padding value is input_zp; result is
  * clamped to [output_min, output_max]. */
 int torq_maxpool2d(const int8_t *input, int8_t *out, int N, int C, int H, int W, int KH, int KW,

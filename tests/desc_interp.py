@@ -24,7 +24,7 @@ BINDING = np.dtype([("id", "<u4"), ("flags", "<u4"), ("size", "<u8")])
 TEMP = np.dtype([("size", "<u8")])
 CONST = np.dtype([("offset", "<u8"), ("size", "<u8")])
 
-K_TRANSPOSE, K_IGEMM, K_FC_SKINNY, K_DW, K_MAXPOOL, K_AVGPOOL, K_ADD, K_FC_BF16 = 1, 2, 3, 4, 5, 6, 7, 8
+K_TRANSPOSE, K_IGEMM, K_FC_SKINNY, K_DW, K_MAXPOOL, K_AVGPOOL, K_ADD, K_FC_BF16, K_ADD_BF16 = 1, 2, 3, 4, 5, 6, 7, 8, 9
 OUT_NP = {1: np.int8, 2: np.int16, 3: np.int32}
 
 
@@ -190,6 +190,13 @@ def run(blob, binding_arrays):
                           np.array([op["bias0"], op["scale0"]], dtype=np.int32), output_zp=zp, output_min=mn,
                           output_max=mx, shift_factor=sh)
             view(op["out"], n)[:] = res.view(np.uint8)
+        elif kind == K_ADD_BF16:
+            n = int(op["C"])
+            a = view(op["in0"], 2 * n).view(np.uint16)
+            b = view(op["in1"], 2 * n).view(np.uint16)
+            res = orc.add_bf16(a, b, np.array([op["w0"], op["w1"]], dtype=np.uint16),
+                               np.array([op["bias0"]], dtype=np.int32).view(np.float32), output_min=mn, output_max=mx)
+            view(op["out"], 2 * n).view(np.uint16)[:] = res
         elif kind == K_FC_BF16:
             M, K, N = int(op["M"]), int(op["K"]), int(op["Nn"])
             x = view(op["in0"], M * K * 2).view(np.uint16).reshape(M, K)

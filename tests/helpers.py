@@ -22,6 +22,8 @@ def oracle_eval(wl):
         return [orc.fully_connected(x, w, sb, **a)]
     if kind == "fcbf16":
         return [orc.fully_connected_bf16(x, a["weights"], a["bias"], output_min=a["output_min"], output_max=a["output_max"])]
+    if kind == "addbf16":
+        return [orc.add_bf16(wl.inputs[0], wl.inputs[1], a["weights"], a["bias"], output_min=a["output_min"], output_max=a["output_max"])]
     if kind == "matmulbf16":
         res = orc.matmul_bf16(x, a["input2"], a["bias"])
         return [res.reshape(wl.outputs[0][0])]

@@ -61,17 +61,38 @@ def test_bf16_matmul_batches_broadcast():
         assert np.array_equal(out[i], orc.matmul_bf16(a[i], b[0], np.zeros(1, dtype=np.float32))[0])
 
 
+def test_bf16_add_closed_forms():
+    # weights 1 and -1 on equal inputs cancel exactly: the bias alone remains; small integers are exact
+    rng = np.random.default_rng(6)
+    x = orc.to_bf16(rng.standard_normal(1000))
+    out = orc.add_bf16(x, x, orc.to_bf16(np.array([1.0, -1.0], dtype=np.float32)), np.array([0.375], dtype=np.float32))
+    assert np.array_equal(out, np.full(1000, orc.to_bf16(np.float32(0.375)), dtype=np.uint16))
+    ai, bi = rng.integers(-20, 21, size=500), rng.integers(-20, 21, size=500)
+    out = orc.add_bf16(orc.to_bf16(ai), orc.to_bf16(bi), orc.to_bf16(np.array([2.0, 3.0], dtype=np.float32)), np.array([-1.0], dtype=np.float32),
+                       output_min=w.float_bits(-10.0), output_max=w.float_bits(40.0))
+    assert np.array_equal(out, orc.to_bf16(np.clip(2.0 * ai + 3.0 * bi - 1.0, -10.0, 40.0).astype(np.float32)))
+    # against float64 on random data: one bf16 step at most (two fp32 roundings before the bf16 one)
+    a, b = orc.to_bf16(rng.standard_normal(4000)), orc.to_bf16(rng.standard_normal(4000))
+    wts = orc.to_bf16(np.array([0.7, 1.3], dtype=np.float32))
+    got = orc.add_bf16(a, b, wts, np.array([0.1], dtype=np.float32))
+    wf = orc.from_bf16(wts).astype(np.float64)
+    exact = orc.from_bf16(a).astype(np.float64) * wf[0] + orc.from_bf16(b).astype(np.float64) * wf[1] + np.float64(np.float32(0.1))
+    assert_bf16_close(got, orc.to_bf16(exact.astype(np.float32)), "bf16 add vs float64")
+
+
 # ---- emitter ------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("make", [lambda: w.fully_connected_bf16_workload(5, 64, 40), lambda: w.fully_connected_bf16_workload(33, 1152, 7, clamp=(-0.5, 0.75)),
                                   lambda: w.matmul_bf16_workload(4, 1, 256, 96, batch2=False), lambda: w.matmul_bf16_workload(3, 2, 64, 24),
                                   lambda: w.matmul_bf16_workload(1, 6, 32, 20, batch1=False, batch2=False, constant_rhs=True, bias=0.5),
-                                  lambda: w.matmul_bf16_workload(2, 5, 16, 12, batch1=False, constant_rhs=True)])
+                                  lambda: w.matmul_bf16_workload(2, 5, 16, 12, batch1=False, constant_rhs=True),
+                                  lambda: w.add_bf16_workload(), lambda: w.add_bf16_workload((3, 5, 7), 0.5, -1.25, 0.125, clamp=(-1.0, 2.0))])
 def test_bf16_descriptor(make):
     wl = make()
     outs = [np.zeros(s, dtype=dt) for s, dt in wl.outputs]
     d = desc_interp.run(wl.program.serialize(), list(wl.inputs) + outs)
     assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)
-    assert desc_interp.K_FC_BF16 in [int(o["kind"]) for o in d.ops]
+    kinds = [int(o["kind"]) for o in d.ops]
+    assert desc_interp.K_FC_BF16 in kinds or desc_interp.K_ADD_BF16 in kinds
 
 
 def test_bf16_rejections():
@@ -127,6 +148,17 @@ def test_gpu_bf16_fully_connected(device):
     exe.run_host([w.to_bf16(xi), out])
     exe.close()
     assert_bit_exact(out, w.to_bf16((xi @ wi.T + bias).astype(np.float32)), "exact small integers")
+
+
+@pytest.mark.gpu
+def test_gpu_bf16_add(device):
+    """Elementwise: the kernel does the oracle's three fp32 operations in the oracle's order, so it is bit-exact."""
+    for wl in [w.add_bf16_workload(), w.add_bf16_workload((3, 5, 7), 0.5, -1.25, 0.125, clamp=(-1.0, 2.0)),
+               w.add_bf16_workload((64, 56, 56, 24), 0.7, 1.3, -0.01)]:
+        print("[gpu-case]", wl.name, flush=True)
+        got, kernels = run_on_gpu(device, wl, via="device")
+        assert_bit_exact(got[0], oracle_eval(wl)[0], wl.name)
+        assert kernels == ["add_bf16"]
 
 
 @pytest.mark.gpu

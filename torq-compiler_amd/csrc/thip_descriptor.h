@@ -69,6 +69,7 @@ enum Kind : uint32_t {
     kKindMaxPool = 5,
     kKindAvgPool = 6,
     kKindAdd = 7,
+    kKindAddBf16 = 9,    // bf16 add: w0 / w1 bf16 bits, bias0 / output_min / output_max float bits, C = element count
     kKindFcBf16 = 8,     // bf16 fully_connected / matmul: fp32 accumulate, float bias, float clamp (output_min/max bits)
 };
 

@@ -250,6 +250,12 @@ static thip_status_t checkOpFootprint(const thip_executable_t *e, uint32_t i) {
         if ((s = need(op.in1, (uint64_t)op.C, "in2"))) return s;
         return need(op.out, (uint64_t)op.C, "out");
     }
+    case kKindAddBf16: {
+        if (!positive({op.C})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad add extent", i);
+        if ((s = need(op.in0, (uint64_t)op.C * 2, "in1"))) return s;
+        if ((s = need(op.in1, (uint64_t)op.C * 2, "in2"))) return s;
+        return need(op.out, (uint64_t)op.C * 2, "out");
+    }
     case kKindFcBf16: {
         if (!positive({op.M, op.K, op.Nn}) || op.K % 8 != 0) return fail(THIP_INVALID_ARGUMENT, "op %u: bad bf16 fully_connected extents", i);
         if ((s = need(op.in0, (uint64_t)op.M * op.K * 2, "in"))) return s;
@@ -278,6 +284,7 @@ static const char *opKernelName(const DescOp &op) {
     case kKindAvgPool: return "avgpool_i8";
     case kKindAdd: return "add_i8";
     case kKindFcBf16: return "fc_bf16";
+    case kKindAddBf16: return "add_bf16";
     default: return "unknown";
     }
 }
@@ -361,6 +368,18 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
         AddArgs a{(const int8_t *)resolve(e, op.in0, bp), (const int8_t *)resolve(e, op.in1, bp),
                   (int8_t *)resolve(e, op.out, bp), (int64_t)op.C, op.w0, op.w1, op.bias0, op.scale0, rq};
         err = launchAdd(a, e->stream);
+        break;
+    }
+    case kKindAddBf16: {
+        auto asFloat = [](int32_t bits) {
+            float f;
+            memcpy(&f, &bits, 4);
+            return f;
+        };
+        AddBf16Args a{(const uint16_t *)resolve(e, op.in0, bp), (const uint16_t *)resolve(e, op.in1, bp),
+                      (uint16_t *)resolve(e, op.out, bp), (int64_t)op.C, asFloat(op.w0 << 16), asFloat(op.w1 << 16),
+                      asFloat(op.bias0), asFloat(op.output_min), asFloat(op.output_max)};
+        err = launchAddBf16(a, e->stream);
         break;
     }
     case kKindFcBf16: {

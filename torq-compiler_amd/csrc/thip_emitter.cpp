@@ -1005,10 +1005,40 @@ thip_status_t Emitter::emitAdd(const thip_hl_add_t &c) {
     if (thip_status_t s = checkValue(c.input1, "torq_hl.add input1", &a)) return s;
     if (thip_status_t s = checkValue(c.input2, "torq_hl.add input2", &b)) return s;
     if (thip_status_t s = checkValue(c.init, "torq_hl.add init", &init)) return s;
-    if (a->dtype != THIP_DTYPE_I8 || b->dtype != THIP_DTYPE_I8 || init->dtype != THIP_DTYPE_I8) return fail(THIP_UNIMPLEMENTED, "%s: only int8 tensors", what);
+    const bool bf16 = a->dtype == THIP_DTYPE_BF16;
+    if (bf16 ? (b->dtype != THIP_DTYPE_BF16 || init->dtype != THIP_DTYPE_BF16)
+             : (a->dtype != THIP_DTYPE_I8 || b->dtype != THIP_DTYPE_I8 || init->dtype != THIP_DTYPE_I8)) {
+        return fail(THIP_UNIMPLEMENTED, "%s: int8 tensors, or bf16 tensors, only", what);
+    }
     if (a->rank != b->rank || a->rank != init->rank) return fail(THIP_INVALID_ARGUMENT, "%s: operand ranks differ (broadcast is materialised by the patterns)", what);
     for (int i = 0; i < a->rank; i++) {
         if (a->shape[i] != b->shape[i] || a->shape[i] != init->shape[i]) return fail(THIP_INVALID_ARGUMENT, "%s: operand shapes differ", what);
+    }
+    if (bf16) {
+        // floating-point partials: two bf16 weights, one float bias, no rescale
+        // (compiler/torq/Conversions/TorqHLToTorqHW/AddPattern.cpp:118-121,262-281)
+        if (thip_status_t s = checkFloatAct(what, c.shift_factor, c.input_zp, 0, c.output_zp)) return s;
+        if (thip_status_t s = constantData(c.weights, "torq_hl.add weights", THIP_DTYPE_BF16, &w)) return s;
+        if (thip_status_t s = constantData(c.scale_bias, "torq_hl.add scale_bias", THIP_DTYPE_F32, &sb)) return s;
+        if (w->numel() < 2 || sb->numel() < 1) return fail(THIP_INVALID_ARGUMENT, "%s: weights / scale_bias too short", what);
+        if (state_[c.input1].nhwcOfNchw || state_[c.input2].nhwcOfNchw) return fail(THIP_UNIMPLEMENTED, "%s: N,C,H,W intermediates are not accepted", what);
+        if (!fitsInt32(a->numel())) return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
+        DescOp op;
+        memset(&op, 0, sizeof(op));
+        op.kind = kKindAddBf16;
+        op.out_dtype = THIP_DTYPE_BF16;
+        op.output_min = c.output_min;
+        op.output_max = c.output_max;
+        op.w0 = ((const uint16_t *)w->data.data())[0];
+        op.w1 = ((const uint16_t *)w->data.data())[1];
+        memcpy(&op.bias0, sb->data.data(), 4);
+        if (thip_status_t s = literalInput(c.input1, "torq_hl.add input1", &op.in0)) return s;
+        if (thip_status_t s = literalInput(c.input2, "torq_hl.add input2", &op.in1)) return s;
+        if (thip_status_t s = literalOutput(c.init, "torq_hl.add init", THIP_DTYPE_BF16, a->numel(), &op.out)) return s;
+        op.N = 1; op.H = 1; op.W = 1;
+        op.C = (int32_t)a->numel();
+        ops_.push_back(op);
+        return THIP_OK;
     }
     if (thip_status_t s = constantData(c.weights, "torq_hl.add weights", THIP_DTYPE_I16, &w)) return s;
     if (thip_status_t s = constantData(c.scale_bias, "torq_hl.add scale_bias", THIP_DTYPE_I32, &sb)) return s;

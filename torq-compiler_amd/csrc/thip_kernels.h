@@ -177,6 +177,16 @@ struct AddArgs {
 };
 hipError_t launchAdd(const AddArgs &a, hipStream_t stream);
 
+// bf16 add: out = bf16(clamp(in0 * w0 + in1 * w1 + bias)) in fp32.
+struct AddBf16Args {
+    const uint16_t *in0;
+    const uint16_t *in1;
+    uint16_t *out;
+    int64_t count;
+    float w0, w1, bias, lo, hi;
+};
+hipError_t launchAddBf16(const AddBf16Args &a, hipStream_t stream);
+
 struct TransposeArgs {
     const int8_t *in;  // [B][R][S]
     int8_t *out;       // [B][S][R]

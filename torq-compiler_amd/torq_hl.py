@@ -204,7 +204,7 @@ class Program:
             rhs_is_scalar=False):
         weights = self._as_value(weights)
         scale_bias = self._as_value(scale_bias)
-        init = self._init_or_new(init, input1.shape, np.int8)
+        init = self._init_or_new(init, input1.shape, input1.dtype)
         op = rt.HlAdd(init.index, name.encode(), input_zp, output_zp, output_min, output_max,
                       shift_factor, weights.index, scale_bias.index, input1.index, input2.index,
                       int(segment_output), int(rhs_is_scalar))

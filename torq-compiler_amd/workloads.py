@@ -165,6 +165,23 @@ def matmul_bf16_workload(B, M, K, N, batch1=True, batch2=True, constant_rhs=Fals
                     a.nbytes + b.nbytes + 2 * int(np.prod(oshape)), attrs)
 
 
+def add_bf16_workload(shape=(1, 32, 1152), w0=1.0, w1=1.0, bias=0.0, clamp=None, seed=1012):
+    """bf16 add (a residual connection of a decoder layer): in1 * w0 + in2 * w1 + bias in fp32."""
+    rng = np.random.default_rng(seed)
+    a = to_bf16(rng.standard_normal(shape))
+    b = to_bf16(rng.standard_normal(shape))
+    wts = to_bf16(np.array([w0, w1], dtype=np.float32))
+    bv = np.array([bias], dtype=np.float32)
+    lo, hi = NO_CLAMP if clamp is None else (float_bits(clamp[0]), float_bits(clamp[1]))
+    p = Program()
+    out = p.binding(2, shape, np.uint16)
+    p.add(p.binding(0, shape, np.uint16), p.binding(1, shape, np.uint16), wts, bv, init=out, output_zp=0, output_min=lo,
+          output_max=hi, shift_factor=0)
+    n = int(np.prod(shape))
+    return Workload("addbf16_" + "x".join(str(d) for d in shape), p, [a, b], [(shape, np.uint16)], 3 * n, 6 * n,
+                    dict(weights=wts, bias=bv, output_min=lo, output_max=hi))
+
+
 def depthwise_workload(N=1, H=56, W=56, C=144, KH=3, KW=3, stride=(2, 2), pad=(0, 1, 0, 1), input_zp=-3,
                        output_zp=5, output_min=-128, output_max=127, realistic=True, nhwc=True, seed=1002):
     """BASELINE config 2a: depthwise 3x3 stride 2 SAME on 56x56x144."""
