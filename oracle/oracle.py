@@ -222,6 +222,44 @@ def matmul_bf16(input1, input2, bias, *, output_min=NO_CLAMP_MIN, output_max=NO_
     return out
 
 
+def conv2d_bf16(input, weights, bias, *, pad, stride, output_min=NO_CLAMP_MIN, output_max=NO_CLAMP_MAX, layout=NCHW):
+    """torq_hl.conv2d on bf16 bit patterns; weights O,I,KH,KW; bias O float32; zero padding."""
+    x = _c(input, np.uint16)
+    w = _c(weights, np.uint16)
+    b = _c(bias, np.float32)
+    if layout == NHWC:
+        N, H, W, C = x.shape
+    else:
+        N, C, H, W = x.shape
+    O, I, KH, KW = w.shape
+    assert I == C and b.size == O
+    OH, OW = _out_hw(H, W, KH, KW, pad, stride)
+    out = np.empty((N, OH, OW, O) if layout == NHWC else (N, O, OH, OW), dtype=np.uint16)
+    rc = lib().torq_conv2d_bf16(_p(x), _p(w), _p(b), _p(out), N, C, H, W, O, KH, KW, _i64x(pad), _i64x(stride),
+                                int(output_min), int(output_max), layout)
+    assert rc == 0
+    return out
+
+
+def depthwise_conv2d_bf16(input, weights, bias, *, pad, stride, output_min=NO_CLAMP_MIN, output_max=NO_CLAMP_MAX, layout=NCHW):
+    """torq_hl.depthwise_conv2d on bf16 bit patterns; weights C,1,KH,KW; bias C float32."""
+    x = _c(input, np.uint16)
+    w = _c(weights, np.uint16)
+    b = _c(bias, np.float32)
+    if layout == NHWC:
+        N, H, W, C = x.shape
+    else:
+        N, C, H, W = x.shape
+    C2, one, KH, KW = w.shape
+    assert C2 == C and one == 1 and b.size == C
+    OH, OW = _out_hw(H, W, KH, KW, pad, stride)
+    out = np.empty((N, OH, OW, C) if layout == NHWC else (N, C, OH, OW), dtype=np.uint16)
+    rc = lib().torq_depthwise_conv2d_bf16(_p(x), _p(w), _p(b), _p(out), N, C, H, W, KH, KW, _i64x(pad), _i64x(stride),
+                                          int(output_min), int(output_max), layout)
+    assert rc == 0
+    return out
+
+
 def add_bf16(input1, input2, weights, bias, *, output_min=NO_CLAMP_MIN, output_max=NO_CLAMP_MAX):
     """torq_hl.add on bf16 bit patterns: two bf16 weights, one float32 bias."""
     a = _c(input1, np.uint16)

@@ -314,6 +314,80 @@ int torq_matmul_bf16(const uint16_t *input1, const uint16_t *input2, const float
 }
 
 /*
+ * torq_hl.conv2d / depthwise_conv2d on bf16 -- the loop nests of the int8 ops
+ * (compiler/torq/Conversions/TorqHLToTorqHW/Conv2DToHw.cpp:150-186, DWToHw.cpp:223-251) with bf16 operands
+ * (Conv2DPattern.cpp:96-106: alu_format = act_format = BF, 4-byte bias, no scale), fp32 accumulation over
+ * (kh, kw, ic), and the float ACT stage.  The padding value is the op's input_zp, which is 0 for bf16 tensors:
+ * positions outside the image contribute nothing.
+ */
+int torq_conv2d_bf16(const uint16_t *input, const uint16_t *weights, const float *bias, uint16_t *out,
+                     int N, int C, int H, int W, int O, int KH, int KW, const int64_t pad[4],
+                     const int64_t stride[2], int32_t clip_min, int32_t clip_max, int layout) {
+    const float lo = float_from_bits(clip_min), hi = float_from_bits(clip_max);
+    const int64_t pl = pad[0], pr = pad[1], pt = pad[2], pb = pad[3];
+    const int64_t sh = stride[0], sw = stride[1];
+    const int OH = out_dim(H, KH, pt, pb, sh), OW = out_dim(W, KW, pl, pr, sw);
+    const strides4_t is = act_strides(layout, C, H, W);
+    const strides4_t os = act_strides(layout, O, OH, OW);
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int n = 0; n < N; n++) {
+        for (int oy = 0; oy < OH; oy++) {
+            for (int ox = 0; ox < OW; ox++) {
+                for (int o = 0; o < O; o++) {
+                    float acc = 0.0f;
+                    for (int kh = 0; kh < KH; kh++) {
+                        const int64_t iy = (int64_t)oy * sh - pt + kh;
+                        for (int kw = 0; kw < KW; kw++) {
+                            const int64_t ix = (int64_t)ox * sw - pl + kw;
+                            if (iy < 0 || iy >= H || ix < 0 || ix >= W) continue;
+                            const uint16_t *wp = weights + (((size_t)o * C) * KH + kh) * KW + kw;
+                            const uint16_t *ip = input + n * is.n + (size_t)iy * is.h + (size_t)ix * is.w;
+                            for (int ic = 0; ic < C; ic++) {
+                                acc += torq_bf16_to_f32(ip[ic * is.c]) * torq_bf16_to_f32(wp[(size_t)ic * KH * KW]);
+                            }
+                        }
+                    }
+                    out[n * os.n + (size_t)o * os.c + (size_t)oy * os.h + (size_t)ox * os.w] = act_float(acc, bias[o], lo, hi);
+                }
+            }
+        }
+    }
+    return 0;
+}
+
+int torq_depthwise_conv2d_bf16(const uint16_t *input, const uint16_t *weights, const float *bias, uint16_t *out,
+                               int N, int C, int H, int W, int KH, int KW, const int64_t pad[4],
+                               const int64_t stride[2], int32_t clip_min, int32_t clip_max, int layout) {
+    const float lo = float_from_bits(clip_min), hi = float_from_bits(clip_max);
+    const int64_t pl = pad[0], pr = pad[1], pt = pad[2], pb = pad[3];
+    const int64_t sh = stride[0], sw = stride[1];
+    const int OH = out_dim(H, KH, pt, pb, sh), OW = out_dim(W, KW, pl, pr, sw);
+    const strides4_t is = act_strides(layout, C, H, W);
+    const strides4_t os = act_strides(layout, C, OH, OW);
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int n = 0; n < N; n++) {
+        for (int oy = 0; oy < OH; oy++) {
+            for (int ox = 0; ox < OW; ox++) {
+                for (int c = 0; c < C; c++) {
+                    float acc = 0.0f;
+                    for (int kh = 0; kh < KH; kh++) {
+                        const int64_t iy = (int64_t)oy * sh - pt + kh;
+                        for (int kw = 0; kw < KW; kw++) {
+                            const int64_t ix = (int64_t)ox * sw - pl + kw;
+                            if (iy < 0 || iy >= H || ix < 0 || ix >= W) continue;
+                            acc += torq_bf16_to_f32(input[n * is.n + (size_t)c * is.c + (size_t)iy * is.h + (size_t)ix * is.w]) *
+                                   torq_bf16_to_f32(weights[((size_t)c * KH + kh) * KW + kw]);
+                        }
+                    }
+                    out[n * os.n + (size_t)c * os.c + (size_t)oy * os.h + (size_t)ox * os.w] = act_float(acc, bias[c], lo, hi);
+                }
+            }
+        }
+    }
+    return 0;
+}
+
+/*
  * torq_hl.add on bf16 -- compiler/torq/Conversions/TorqHLToTorqHW/AddPattern.cpp:262-281 with floating-point
  * partials: the two products (exact in fp32) are accumulated in tensor order, then the float ACT stage
  * (one bias: biasScaleWidth is 1 for bf16, AddPattern.cpp:118-121,197-200).

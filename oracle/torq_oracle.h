@@ -91,6 +91,17 @@ int torq_fully_connected_bf16(const uint16_t *input, const uint16_t *weights, co
 int torq_matmul_bf16(const uint16_t *input1, const uint16_t *input2, const float *bias, uint16_t *out,
                      int B, int M, int K, int N, int bcast1, int bcast2, int32_t clip_min, int32_t clip_max);
 
+/* torq_hl.conv2d on bf16: weights O x I x KH x KW (bf16), bias O floats, padding with +0.0;
+ * layout as for the int8 op. */
+int torq_conv2d_bf16(const uint16_t *input, const uint16_t *weights, const float *bias, uint16_t *out,
+                     int N, int C, int H, int W, int O, int KH, int KW, const int64_t pad[4],
+                     const int64_t stride[2], int32_t clip_min, int32_t clip_max, int layout);
+
+/* torq_hl.depthwise_conv2d on bf16: weights C x 1 x KH x KW, bias C floats. */
+int torq_depthwise_conv2d_bf16(const uint16_t *input, const uint16_t *weights, const float *bias, uint16_t *out,
+                               int N, int C, int H, int W, int KH, int KW, const int64_t pad[4],
+                               const int64_t stride[2], int32_t clip_min, int32_t clip_max, int layout);
+
 /* torq_hl.add on bf16: out = bf16(clamp(in1 * w[0] + in2 * w[1] + bias)), two bf16 weights, ONE float bias. */
 int torq_add_bf16(const uint16_t *input1, const uint16_t *input2, const uint16_t weights[2], const float *bias,
                   uint16_t *out, size_t count, int32_t clip_min, int32_t clip_max);

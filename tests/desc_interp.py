@@ -24,7 +24,7 @@ BINDING = np.dtype([("id", "<u4"), ("flags", "<u4"), ("size", "<u8")])
 TEMP = np.dtype([("size", "<u8")])
 CONST = np.dtype([("offset", "<u8"), ("size", "<u8")])
 
-K_TRANSPOSE, K_IGEMM, K_FC_SKINNY, K_DW, K_MAXPOOL, K_AVGPOOL, K_ADD, K_FC_BF16, K_ADD_BF16 = 1, 2, 3, 4, 5, 6, 7, 8, 9
+K_TRANSPOSE, K_IGEMM, K_FC_SKINNY, K_DW, K_MAXPOOL, K_AVGPOOL, K_ADD, K_FC_BF16, K_ADD_BF16, K_IM2COL_BF16, K_DW_BF16 = 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11
 OUT_NP = {1: np.int8, 2: np.int16, 3: np.int32}
 
 
@@ -190,6 +190,31 @@ def run(blob, binding_arrays):
                           np.array([op["bias0"], op["scale0"]], dtype=np.int32), output_zp=zp, output_min=mn,
                           output_max=mx, shift_factor=sh)
             view(op["out"], n)[:] = res.view(np.uint8)
+        elif kind == K_IM2COL_BF16:
+            Nimg, H, W, C, OH, OW, KH, KW = (int(op[k]) for k in ["N", "H", "W", "C", "OH", "OW", "KH", "KW"])
+            SH, SW, PT, PL, Kp = (int(op[k]) for k in ["SH", "SW", "PT", "PL", "Kp"])
+            x = view(op["in0"], Nimg * H * W * C * 2).view(np.uint16).reshape(Nimg, H, W, C)
+            A = np.zeros((Nimg, OH, OW, Kp), dtype=np.uint16)
+            oy = np.arange(OH)[:, None] * SH - PT
+            ox = np.arange(OW)[None, :] * SW - PL
+            for kh in range(KH):
+                for kw in range(KW):
+                    iy, ix = oy + kh, ox + kw
+                    inside = (iy >= 0) & (iy < H) & (ix >= 0) & (ix < W)
+                    vals = x[:, np.clip(iy, 0, H - 1), np.clip(ix, 0, W - 1), :]
+                    k0 = (kh * KW + kw) * C
+                    A[..., k0:k0 + C] = np.where(inside[None, :, :, None], vals, 0)
+            view(op["out"], A.size * 2).view(np.uint16)[:] = A.reshape(-1)
+        elif kind == K_DW_BF16:
+            Nimg, H, W, C, OH, OW, KH, KW = (int(op[k]) for k in ["N", "H", "W", "C", "OH", "OW", "KH", "KW"])
+            x = view(op["in0"], Nimg * H * W * C * 2).view(np.uint16).reshape(Nimg, H, W, C)
+            wpk = view(op["weights"], KH * KW * C * 2).view(np.uint16).reshape(KH, KW, C)
+            bias = view(op["bias"], C * 4).view(np.float32)
+            res = orc.depthwise_conv2d_bf16(x, np.ascontiguousarray(wpk.transpose(2, 0, 1))[:, None], bias,
+                                            pad=[int(op["PL"]), int(op["PR"]), int(op["PT"]), int(op["PB"])],
+                                            stride=[int(op["SH"]), int(op["SW"])], output_min=mn, output_max=mx, layout=orc.NHWC)
+            assert res.shape == (Nimg, OH, OW, C)
+            view(op["out"], res.size * 2).view(np.uint16)[:] = res.reshape(-1)
         elif kind == K_ADD_BF16:
             n = int(op["C"])
             a = view(op["in0"], 2 * n).view(np.uint16)

@@ -22,6 +22,10 @@ def oracle_eval(wl):
         return [orc.fully_connected(x, w, sb, **a)]
     if kind == "fcbf16":
         return [orc.fully_connected_bf16(x, a["weights"], a["bias"], output_min=a["output_min"], output_max=a["output_max"])]
+    if kind in ("convbf16", "dwbf16"):
+        fn = orc.conv2d_bf16 if kind == "convbf16" else orc.depthwise_conv2d_bf16
+        return [fn(x, a["weights"], a["bias"], pad=a["pad"], stride=a["stride"], output_min=a["output_min"], output_max=a["output_max"],
+                   layout=orc.NHWC if a["nhwc"] else orc.NCHW)]
     if kind == "addbf16":
         return [orc.add_bf16(wl.inputs[0], wl.inputs[1], a["weights"], a["bias"], output_min=a["output_min"], output_max=a["output_max"])]
     if kind == "matmulbf16":

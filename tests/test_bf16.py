@@ -61,6 +61,38 @@ def test_bf16_matmul_batches_broadcast():
         assert np.array_equal(out[i], orc.matmul_bf16(a[i], b[0], np.zeros(1, dtype=np.float32))[0])
 
 
+def test_bf16_conv_oracle_pins():
+    """conv2d / depthwise_conv2d on bf16: exact on small integers (vs an integer convolution), within one bf16 ULP of
+    torch's float64 convolution on random data, both layouts, asymmetric padding and strides."""
+    import torch
+    import torch.nn.functional as F
+    rng = np.random.default_rng(7)
+    for (N, C, H, W, O, KH, KW, pad, stride) in [(2, 5, 9, 8, 6, 3, 3, (1, 0, 2, 1), (2, 1)), (1, 8, 7, 7, 4, 1, 1, (0, 0, 0, 0), (1, 1)),
+                                                 (1, 3, 12, 10, 7, 5, 2, (0, 1, 2, 2), (3, 2))]:
+        xi = rng.integers(-6, 7, size=(N, C, H, W))
+        wi = rng.integers(-6, 7, size=(O, C, KH, KW))
+        bi = rng.integers(-9, 10, size=O).astype(np.float32)
+        padded = F.pad(torch.tensor(xi, dtype=torch.float64), (pad[0], pad[1], pad[2], pad[3]))
+        want = F.conv2d(padded, torch.tensor(wi, dtype=torch.float64), torch.tensor(bi, dtype=torch.float64), stride=stride).numpy()
+        got = orc.conv2d_bf16(orc.to_bf16(xi), orc.to_bf16(wi), bi, pad=pad, stride=stride)
+        assert np.array_equal(got, orc.to_bf16(want.astype(np.float32)))
+        nhwc = orc.conv2d_bf16(orc.to_bf16(xi.transpose(0, 2, 3, 1)), orc.to_bf16(wi), bi, pad=pad, stride=stride, layout=orc.NHWC)
+        assert np.array_equal(nhwc.transpose(0, 3, 1, 2), got)
+        x = orc.to_bf16(rng.standard_normal((N, C, H, W)))
+        wt = orc.to_bf16(rng.standard_normal((O, C, KH, KW)) / np.sqrt(C * KH * KW))
+        b = rng.standard_normal(O).astype(np.float32)
+        padded = F.pad(torch.tensor(orc.from_bf16(x), dtype=torch.float64), (pad[0], pad[1], pad[2], pad[3]))
+        exact = F.conv2d(padded, torch.tensor(orc.from_bf16(wt), dtype=torch.float64), torch.tensor(b, dtype=torch.float64), stride=stride).numpy()
+        got = orc.conv2d_bf16(x, wt, b, pad=pad, stride=stride, output_min=w.float_bits(-0.5), output_max=w.float_bits(1.0))
+        assert_bf16_close(got, orc.to_bf16(np.clip(exact, -0.5, 1.0).astype(np.float32)), "conv2d bf16 vs float64")
+        # depthwise = grouped convolution with one input channel per group
+        wd = orc.to_bf16(rng.standard_normal((C, 1, KH, KW)) / np.sqrt(KH * KW))
+        bd = rng.standard_normal(C).astype(np.float32)
+        exact = F.conv2d(padded, torch.tensor(orc.from_bf16(wd), dtype=torch.float64), torch.tensor(bd, dtype=torch.float64), stride=stride, groups=C).numpy()
+        got = orc.depthwise_conv2d_bf16(x, wd, bd, pad=pad, stride=stride)
+        assert_bf16_close(got, orc.to_bf16(exact.astype(np.float32)), "depthwise bf16 vs float64")
+
+
 def test_bf16_add_closed_forms():
     # weights 1 and -1 on equal inputs cancel exactly: the bias alone remains; small integers are exact
     rng = np.random.default_rng(6)
@@ -85,6 +117,10 @@ def test_bf16_add_closed_forms():
                                   lambda: w.matmul_bf16_workload(4, 1, 256, 96, batch2=False), lambda: w.matmul_bf16_workload(3, 2, 64, 24),
                                   lambda: w.matmul_bf16_workload(1, 6, 32, 20, batch1=False, batch2=False, constant_rhs=True, bias=0.5),
                                   lambda: w.matmul_bf16_workload(2, 5, 16, 12, batch1=False, constant_rhs=True),
+                                  lambda: w.conv2d_bf16_workload(), lambda: w.conv2d_bf16_workload(N=2, H=9, W=11, C=5, O=7, KH=2, KW=3, stride=(2, 1), pad=(0, 2, 1, 0), nhwc=False),
+                                  lambda: w.conv2d_bf16_workload(N=2, H=6, W=6, C=16, O=40, KH=1, KW=1, pad=(0, 0, 0, 0)),
+                                  lambda: w.conv2d_bf16_workload(depthwise=True, C=12, stride=(2, 2), pad=(0, 1, 0, 1), clamp=(-0.5, 0.5)),
+                                  lambda: w.conv2d_bf16_workload(depthwise=True, N=2, C=5, H=7, W=9, nhwc=False),
                                   lambda: w.add_bf16_workload(), lambda: w.add_bf16_workload((3, 5, 7), 0.5, -1.25, 0.125, clamp=(-1.0, 2.0))])
 def test_bf16_descriptor(make):
     wl = make()
@@ -92,7 +128,7 @@ def test_bf16_descriptor(make):
     d = desc_interp.run(wl.program.serialize(), list(wl.inputs) + outs)
     assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)
     kinds = [int(o["kind"]) for o in d.ops]
-    assert desc_interp.K_FC_BF16 in kinds or desc_interp.K_ADD_BF16 in kinds
+    assert {desc_interp.K_FC_BF16, desc_interp.K_ADD_BF16, desc_interp.K_DW_BF16} & set(kinds)
 
 
 def test_bf16_rejections():
@@ -148,6 +184,32 @@ def test_gpu_bf16_fully_connected(device):
     exe.run_host([w.to_bf16(xi), out])
     exe.close()
     assert_bit_exact(out, w.to_bf16((xi @ wi.T + bias).astype(np.float32)), "exact small integers")
+
+
+@pytest.mark.gpu
+def test_gpu_bf16_conv2d_and_depthwise(device):
+    """conv2d as patch matrix + GEMM (tolerance row), pointwise conv2d straight on the image, depthwise (same order of
+    fp32 operations as the oracle: bit-exact), N,C,H,W bindings through the 16-bit transpose."""
+    for wl in [w.conv2d_bf16_workload(), w.conv2d_bf16_workload(N=2, H=9, W=11, C=5, O=7, KH=2, KW=3, stride=(2, 1), pad=(0, 2, 1, 0), nhwc=False),
+               w.conv2d_bf16_workload(N=2, H=28, W=28, C=32, O=64, KH=1, KW=1, pad=(0, 0, 0, 0)),
+               w.conv2d_bf16_workload(N=1, H=56, W=56, C=24, O=48, stride=(2, 2), pad=(0, 1, 0, 1), clamp=(0.0, 6.0))]:
+        print("[gpu-case]", wl.name, flush=True)
+        got, kernels = run_on_gpu(device, wl)
+        f = lambda bits: np.abs(orc.from_bf16(bits).astype(np.float64))
+        # sum of |products| per output: a convolution of magnitudes (through the oracle's own loop nest in float64 is
+        # overkill; bound it by |x|max * sum|w| + |b|)
+        wabs = f(wl.attrs["weights"]).reshape(wl.attrs["weights"].shape[0], -1).sum(axis=1) * f(wl.inputs[0]).max() + np.abs(wl.attrs["bias"])
+        shape = [1, 1, 1, 1]
+        shape[3 if wl.attrs["nhwc"] else 1] = -1
+        assert_bf16_close(got[0], oracle_eval(wl)[0], wl.name, magnitude=np.broadcast_to(wabs.reshape(shape), got[0].shape))
+        assert "fc_bf16" in kernels
+    for wl in [w.conv2d_bf16_workload(depthwise=True, C=12, stride=(2, 2), pad=(0, 1, 0, 1), clamp=(-0.5, 0.5)),
+               w.conv2d_bf16_workload(depthwise=True, N=2, C=5, H=7, W=9, nhwc=False),
+               w.conv2d_bf16_workload(depthwise=True, N=4, C=144, H=56, W=56)]:
+        print("[gpu-case]", wl.name, flush=True)
+        got, kernels = run_on_gpu(device, wl, via="device")
+        assert_bit_exact(got[0], oracle_eval(wl)[0], wl.name)
+        assert "depthwise_bf16" in kernels
 
 
 @pytest.mark.gpu

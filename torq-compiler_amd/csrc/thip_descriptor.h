@@ -70,6 +70,8 @@ enum Kind : uint32_t {
     kKindAvgPool = 6,
     kKindAdd = 7,
     kKindAddBf16 = 9,    // bf16 add: w0 / w1 bf16 bits, bias0 / output_min / output_max float bits, C = element count
+    kKindIm2colBf16 = 10,     // bf16 N,H,W,C image -> [M][Kp] patch matrix, k = (kh * KW + kw) * C + ci, zero padded
+    kKindDepthwiseBf16 = 11,  // bf16 depthwise: weights [KH][KW][C] bf16, bias f32[C]
     kKindFcBf16 = 8,     // bf16 fully_connected / matmul: fp32 accumulate, float bias, float clamp (output_min/max bits)
 };
 

@@ -250,6 +250,20 @@ static thip_status_t checkOpFootprint(const thip_executable_t *e, uint32_t i) {
         if ((s = need(op.in1, (uint64_t)op.C, "in2"))) return s;
         return need(op.out, (uint64_t)op.C, "out");
     }
+    case kKindIm2colBf16: {
+        if (!positive({op.N, op.H, op.W, op.C, op.OH, op.OW, op.KH, op.KW, op.Kp}) || op.Kp < op.KH * op.KW * op.C) {
+            return fail(THIP_INVALID_ARGUMENT, "op %u: bad im2col extents", i);
+        }
+        if ((s = need(op.in0, (uint64_t)op.N * op.H * op.W * op.C * 2, "in"))) return s;
+        return need(op.out, (uint64_t)op.N * op.OH * op.OW * op.Kp * 2, "out");
+    }
+    case kKindDepthwiseBf16: {
+        if (!positive({op.N, op.H, op.W, op.C, op.OH, op.OW, op.KH, op.KW})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad depthwise extents", i);
+        if ((s = need(op.in0, (uint64_t)op.N * op.H * op.W * op.C * 2, "in"))) return s;
+        if ((s = need(op.weights, (uint64_t)op.KH * op.KW * op.C * 2, "weights"))) return s;
+        if ((s = need(op.bias, (uint64_t)op.C * 4, "bias"))) return s;
+        return need(op.out, (uint64_t)op.N * op.OH * op.OW * op.C * 2, "out");
+    }
     case kKindAddBf16: {
         if (!positive({op.C})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad add extent", i);
         if ((s = need(op.in0, (uint64_t)op.C * 2, "in1"))) return s;
@@ -285,6 +299,8 @@ static const char *opKernelName(const DescOp &op) {
     case kKindAdd: return "add_i8";
     case kKindFcBf16: return "fc_bf16";
     case kKindAddBf16: return "add_bf16";
+    case kKindIm2colBf16: return "im2col_bf16";
+    case kKindDepthwiseBf16: return "depthwise_bf16";
     default: return "unknown";
     }
 }
@@ -368,6 +384,22 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
         AddArgs a{(const int8_t *)resolve(e, op.in0, bp), (const int8_t *)resolve(e, op.in1, bp),
                   (int8_t *)resolve(e, op.out, bp), (int64_t)op.C, op.w0, op.w1, op.bias0, op.scale0, rq};
         err = launchAdd(a, e->stream);
+        break;
+    }
+    case kKindIm2colBf16: {
+        Im2colBf16Args a{(const uint16_t *)resolve(e, op.in0, bp), (uint16_t *)resolve(e, op.out, bp), op.N, op.H, op.W, op.C,
+                         op.OH, op.OW, op.KH, op.KW, op.SH, op.SW, op.PT, op.PL, op.Kp};
+        err = launchIm2colBf16(a, e->stream);
+        break;
+    }
+    case kKindDepthwiseBf16: {
+        float lo, hi;
+        memcpy(&lo, &op.output_min, 4);
+        memcpy(&hi, &op.output_max, 4);
+        DepthwiseBf16Args a{(const uint16_t *)resolve(e, op.in0, bp), (const uint16_t *)resolve(e, op.weights, bp),
+                            (const float *)resolve(e, op.bias, bp), (uint16_t *)resolve(e, op.out, bp), op.N, op.H, op.W, op.C,
+                            op.OH, op.OW, op.KH, op.KW, op.SH, op.SW, op.PT, op.PL, lo, hi};
+        err = launchDepthwiseBf16(a, e->stream);
         break;
     }
     case kKindAddBf16: {

@@ -189,11 +189,12 @@ class Emitter {
     }
 
     // A 4-D int8 activation operand, delivered to the kernel as NHWC.
-    thip_status_t nhwcInput(thip_value_t id, bool declaredNhwc, const char *what, Dims4 *dims, DescRef *out) {
+    thip_status_t nhwcInput(thip_value_t id, bool declaredNhwc, const char *what, Dims4 *dims, DescRef *out,
+                            int32_t dtype = THIP_DTYPE_I8) {
         const Value *v;
         if (thip_status_t s = checkValue(id, what, &v)) return s;
         if (v->rank != 4) return fail(THIP_INVALID_ARGUMENT, "%s: expected a rank-4 tensor, got rank %d", what, v->rank);
-        if (v->dtype != THIP_DTYPE_I8) return fail(THIP_UNIMPLEMENTED, "%s: only int8 activations are supported", what);
+        if (v->dtype != dtype) return fail(THIP_UNIMPLEMENTED, "%s: activation element type not supported here", what);
         if (declaredNhwc) {
             *dims = Dims4{v->shape[0], v->shape[3], v->shape[1], v->shape[2]};
         } else {
@@ -213,8 +214,8 @@ class Emitter {
             return THIP_OK;
         }
         // literal NCHW in memory: transpose [N][C][HW] -> [N][HW][C]
-        DescRef t = newTemp((uint64_t)v->numel());
-        emitTranspose(lit, t, dims->N, dims->C, dims->H * dims->W);
+        DescRef t = newTemp((uint64_t)v->numel() * elemSize(dtype));
+        emitTranspose(lit, t, dims->N, dims->C, dims->H * dims->W, (uint32_t)elemSize(dtype));
         *out = t;
         return THIP_OK;
     }
@@ -226,6 +227,7 @@ class Emitter {
         bool needed = false;
         DescRef from, to;
         int64_t B = 0, R = 0, S = 0;
+        uint32_t elem = 1;
     };
     thip_status_t nhwcOutput(thip_value_t id, bool declaredNhwc, const char *what, int32_t dtype, int64_t N,
                              int64_t C, int64_t H, int64_t W, DescRef *out, Pending *post) {
@@ -255,10 +257,11 @@ class Emitter {
             *out = b;
             return THIP_OK;
         }
-        if (elemSize(dtype) != 1) {
-            return fail(THIP_UNIMPLEMENTED, "%s: N,C,H,W outputs wider than 8 bits need nhwc_input", what);
+        if (elemSize(dtype) != 1 && dtype != THIP_DTYPE_BF16) {
+            return fail(THIP_UNIMPLEMENTED, "%s: N,C,H,W integer outputs wider than 8 bits need nhwc_input", what);
         }
         DescRef t = newTemp(bytes);
+        post->elem = (uint32_t)elemSize(dtype);
         post->needed = true;
         post->from = t;
         post->to = b;
@@ -269,7 +272,7 @@ class Emitter {
         return THIP_OK;
     }
     void finishOutput(const Pending &post) {
-        if (post.needed) emitTranspose(post.from, post.to, post.B, post.R, post.S);
+        if (post.needed) emitTranspose(post.from, post.to, post.B, post.R, post.S, post.elem);
     }
 
     // An output written in its declared order (FC, matmul, avg pool).
@@ -501,6 +504,8 @@ class Emitter {
         op->loader = 1;
         op->weights = newConst(packed);
     }
+    thip_status_t emitConv2dBf16(const thip_hl_conv2d_t &c);
+    thip_status_t emitDepthwiseBf16(const thip_hl_depthwise_conv2d_t &c);
     thip_status_t emitFullyConnectedBf16(const thip_hl_fully_connected_t &c);
     thip_status_t emitMatmulBf16(const thip_hl_matmul_t &c);
     thip_status_t emitMaxPool(const thip_hl_maxpool2d_t &c);
@@ -527,6 +532,11 @@ static bool fitsInt32(int64_t v) { return v > 0 && v < (1LL << 31); }
 
 thip_status_t Emitter::emitConv2d(const thip_hl_conv2d_t &c) {
     const char *what = "torq_hl.conv2d";
+    {
+        const Value *xin;
+        if (thip_status_t s = checkValue(c.input, "torq_hl.conv2d input", &xin)) return s;
+        if (xin->dtype == THIP_DTYPE_BF16) return emitConv2dBf16(c);
+    }
     if (c.groups != 1) return fail(THIP_UNIMPLEMENTED, "%s: groups must be 1", what);
     if (c.weight_zp != 0) return fail(THIP_UNIMPLEMENTED, "%s: weight_zp must be 0 (the patterns fold it into the weights)", what);
     if (c.dilation[0] != 1 || c.dilation[1] != 1) return fail(THIP_UNIMPLEMENTED, "%s: dilation must be [1,1] (the patterns fold it into the weights)", what);
@@ -596,6 +606,11 @@ thip_status_t Emitter::emitConv2d(const thip_hl_conv2d_t &c) {
 
 thip_status_t Emitter::emitDepthwise(const thip_hl_depthwise_conv2d_t &c) {
     const char *what = "torq_hl.depthwise_conv2d";
+    {
+        const Value *xin;
+        if (thip_status_t s = checkValue(c.input, "torq_hl.depthwise_conv2d input", &xin)) return s;
+        if (xin->dtype == THIP_DTYPE_BF16) return emitDepthwiseBf16(c);
+    }
     if (c.weight_zp != 0) return fail(THIP_UNIMPLEMENTED, "%s: weight_zp must be 0", what);
     if (c.dilation[0] != 1 || c.dilation[1] != 1) return fail(THIP_UNIMPLEMENTED, "%s: dilation must be [1,1]", what);
     if (c.segment_output) return fail(THIP_UNIMPLEMENTED, "%s: segment_output is an NPU memory layout", what);
@@ -819,6 +834,127 @@ thip_status_t Emitter::emitMatmul(const thip_hl_matmul_t &c) {
 static thip_status_t checkFloatAct(const char *what, int32_t shift, int32_t zpA, int32_t zpB, int32_t zpOut) {
     if (shift != 0) return fail(THIP_INVALID_ARGUMENT, "%s: bf16 has no rescale: shift must be 0", what);
     if (zpA != 0 || zpB != 0 || zpOut != 0) return fail(THIP_INVALID_ARGUMENT, "%s: bf16 has no zero points", what);
+    return THIP_OK;
+}
+
+thip_status_t Emitter::emitConv2dBf16(const thip_hl_conv2d_t &c) {
+    const char *what = "torq_hl.conv2d (bf16)";
+    if (c.groups != 1) return fail(THIP_UNIMPLEMENTED, "%s: groups must be 1", what);
+    if (c.dilation[0] != 1 || c.dilation[1] != 1) return fail(THIP_UNIMPLEMENTED, "%s: dilation must be [1,1]", what);
+    if (c.segment_output) return fail(THIP_UNIMPLEMENTED, "%s: segment_output is an NPU memory layout", what);
+    if (thip_status_t s = checkFloatAct(what, c.shift_factor, c.input_zp, c.weight_zp, c.output_zp)) return s;
+    const Value *w, *init, *b;
+    if (thip_status_t s = constantData(c.weights, "torq_hl.conv2d weights", THIP_DTYPE_BF16, &w)) return s;
+    if (w->rank != 4) return fail(THIP_INVALID_ARGUMENT, "%s: weights must be O,I,KH,KW", what);
+    if (thip_status_t s = checkValue(c.init, "torq_hl.conv2d init", &init)) return s;
+    if (init->dtype != THIP_DTYPE_BF16) return fail(THIP_INVALID_ARGUMENT, "%s: init must be bf16", what);
+    Dims4 d;
+    DescRef in;
+    if (thip_status_t s = nhwcInput(c.input, c.nhwc_input != 0, "torq_hl.conv2d input", &d, &in, THIP_DTYPE_BF16)) return s;
+    const int64_t O = w->shape[0], I = w->shape[1], KH = w->shape[2], KW = w->shape[3];
+    if (I != d.C) return fail(THIP_INVALID_ARGUMENT, "%s: weights expect %lld input channels, input has %lld", what, (long long)I, (long long)d.C);
+    if (thip_status_t s = constantData(c.scale_bias, "torq_hl.conv2d scale_bias", THIP_DTYPE_F32, &b)) return s;
+    if (b->numel() < O) return fail(THIP_INVALID_ARGUMENT, "%s: scale_bias holds %lld floats, %lld needed", what, (long long)b->numel(), (long long)O);
+    int64_t OH, OW;
+    if (thip_status_t s = windowGeometry(what, d.H, d.W, KH, KW, c.pad, c.stride, &OH, &OW)) return s;
+    const int64_t M = d.N * OH * OW, K = KH * KW * d.C, Kp = roundUp(K, 8);
+    if (!fitsInt32(M) || !fitsInt32(Kp) || !fitsInt32(M * O) || !fitsInt32(M * Kp) || !fitsInt32(d.N * d.H * d.W * d.C)) {
+        return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
+    }
+    DescRef out;
+    Pending post;
+    if (thip_status_t s = nhwcOutput(c.init, c.nhwc_input != 0, "torq_hl.conv2d init", THIP_DTYPE_BF16, d.N, O, OH, OW, &out, &post)) return s;
+    // the GEMM operand: the image itself for a pointwise convolution, its patch matrix otherwise
+    const bool pointwise = KH == 1 && KW == 1 && c.stride[0] == 1 && c.stride[1] == 1 && c.pad[0] == 0 && c.pad[1] == 0 &&
+                           c.pad[2] == 0 && c.pad[3] == 0 && d.C % 8 == 0;
+    DescRef a = in;
+    if (!pointwise) {
+        DescOp g;
+        memset(&g, 0, sizeof(g));
+        g.kind = kKindIm2colBf16;
+        g.N = (int32_t)d.N; g.H = (int32_t)d.H; g.W = (int32_t)d.W; g.C = (int32_t)d.C;
+        g.OH = (int32_t)OH; g.OW = (int32_t)OW; g.KH = (int32_t)KH; g.KW = (int32_t)KW;
+        g.SH = (int32_t)c.stride[0]; g.SW = (int32_t)c.stride[1]; g.PL = (int32_t)c.pad[0]; g.PT = (int32_t)c.pad[2];
+        g.Kp = (int32_t)Kp;
+        g.in0 = in;
+        a = newTemp((uint64_t)(M * Kp) * 2);
+        g.out = a;
+        ops_.push_back(g);
+    }
+    // weights as [O][Kp], k = (kh * KW + kw) * C + ci
+    const uint16_t *wd = (const uint16_t *)w->data.data();
+    std::vector<uint16_t> wk((size_t)(O * Kp), 0);
+    for (int64_t o = 0; o < O; o++) {
+        for (int64_t kh = 0; kh < KH; kh++) {
+            for (int64_t kw = 0; kw < KW; kw++) {
+                for (int64_t ci = 0; ci < d.C; ci++) {
+                    wk[(size_t)(o * Kp + (kh * KW + kw) * d.C + ci)] = wd[((o * d.C + ci) * KH + kh) * KW + kw];
+                }
+            }
+        }
+    }
+    DescOp op;
+    memset(&op, 0, sizeof(op));
+    op.kind = kKindFcBf16;
+    op.out_dtype = THIP_DTYPE_BF16;
+    op.output_min = c.output_min;
+    op.output_max = c.output_max;
+    op.M = (int32_t)M; op.K = (int32_t)Kp; op.Kp = (int32_t)Kp; op.Nn = (int32_t)O; op.Np = (int32_t)O;
+    op.in0 = a;
+    op.out = out;
+    packBf16Weights(&op, wk.data(), O, Kp);
+    op.bias = newConst(std::vector<uint8_t>(b->data.begin(), b->data.begin() + (size_t)O * 4));
+    planFcBf16Split(&op);
+    ops_.push_back(op);
+    finishOutput(post);
+    return THIP_OK;
+}
+
+thip_status_t Emitter::emitDepthwiseBf16(const thip_hl_depthwise_conv2d_t &c) {
+    const char *what = "torq_hl.depthwise_conv2d (bf16)";
+    if (c.dilation[0] != 1 || c.dilation[1] != 1) return fail(THIP_UNIMPLEMENTED, "%s: dilation must be [1,1]", what);
+    if (c.segment_output) return fail(THIP_UNIMPLEMENTED, "%s: segment_output is an NPU memory layout", what);
+    if (c.is_dw1d_stride1) return fail(THIP_UNIMPLEMENTED, "%s: is_dw1d_stride1 is the 1-D special case", what);
+    if (thip_status_t s = checkFloatAct(what, c.shift_factor, c.input_zp, c.weight_zp, c.output_zp)) return s;
+    const Value *w, *init, *b;
+    if (thip_status_t s = constantData(c.weights, "torq_hl.depthwise_conv2d weights", THIP_DTYPE_BF16, &w)) return s;
+    if (w->rank != 4 || w->shape[1] != 1) return fail(THIP_INVALID_ARGUMENT, "%s: weights must be C,1,KH,KW", what);
+    if (thip_status_t s = checkValue(c.init, "torq_hl.depthwise_conv2d init", &init)) return s;
+    if (init->dtype != THIP_DTYPE_BF16) return fail(THIP_INVALID_ARGUMENT, "%s: init must be bf16", what);
+    Dims4 d;
+    DescRef in;
+    if (thip_status_t s = nhwcInput(c.input, c.nhwc_input != 0, "torq_hl.depthwise_conv2d input", &d, &in, THIP_DTYPE_BF16)) return s;
+    const int64_t C = w->shape[0], KH = w->shape[2], KW = w->shape[3];
+    if (C != d.C) return fail(THIP_INVALID_ARGUMENT, "%s: weights have %lld channels, input has %lld", what, (long long)C, (long long)d.C);
+    if (thip_status_t s = constantData(c.scale_bias, "torq_hl.depthwise_conv2d scale_bias", THIP_DTYPE_F32, &b)) return s;
+    if (b->numel() < C) return fail(THIP_INVALID_ARGUMENT, "%s: scale_bias holds %lld floats, %lld needed", what, (long long)b->numel(), (long long)C);
+    int64_t OH, OW;
+    if (thip_status_t s = windowGeometry(what, d.H, d.W, KH, KW, c.pad, c.stride, &OH, &OW)) return s;
+    if (!fitsInt32(d.N * OH * OW * C) || !fitsInt32(d.N * d.H * d.W * C)) return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
+    DescOp op;
+    memset(&op, 0, sizeof(op));
+    DescRef out;
+    Pending post;
+    if (thip_status_t s = nhwcOutput(c.init, c.nhwc_input != 0, "torq_hl.depthwise_conv2d init", THIP_DTYPE_BF16, d.N, C, OH, OW, &out, &post)) return s;
+    const uint16_t *wd = (const uint16_t *)w->data.data();
+    std::vector<uint16_t> wpk((size_t)(KH * KW * C));
+    for (int64_t ch = 0; ch < C; ch++) {
+        for (int64_t k = 0; k < KH * KW; k++) wpk[(size_t)(k * C + ch)] = wd[ch * KH * KW + k];
+    }
+    op.kind = kKindDepthwiseBf16;
+    op.out_dtype = THIP_DTYPE_BF16;
+    op.output_min = c.output_min;
+    op.output_max = c.output_max;
+    op.N = (int32_t)d.N; op.H = (int32_t)d.H; op.W = (int32_t)d.W; op.C = (int32_t)C;
+    op.OH = (int32_t)OH; op.OW = (int32_t)OW; op.OC = (int32_t)C;
+    op.KH = (int32_t)KH; op.KW = (int32_t)KW; op.SH = (int32_t)c.stride[0]; op.SW = (int32_t)c.stride[1];
+    op.PL = (int32_t)c.pad[0]; op.PR = (int32_t)c.pad[1]; op.PT = (int32_t)c.pad[2]; op.PB = (int32_t)c.pad[3];
+    op.in0 = in;
+    op.out = out;
+    op.weights = newConst(wpk);
+    op.bias = newConst(std::vector<uint8_t>(b->data.begin(), b->data.begin() + (size_t)C * 4));
+    ops_.push_back(op);
+    finishOutput(post);
     return THIP_OK;
 }
 

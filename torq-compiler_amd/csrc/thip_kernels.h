@@ -177,6 +177,26 @@ struct AddArgs {
 };
 hipError_t launchAdd(const AddArgs &a, hipStream_t stream);
 
+// bf16 patch matrix of a convolution: out[m][k] with m = (n * OH + oy) * OW + ox and k = (kh * KW + kw) * C + ci,
+// rows padded with zeros to Kp; positions outside the image are zero.
+struct Im2colBf16Args {
+    const uint16_t *in;  // NHWC
+    uint16_t *out;       // [M][Kp]
+    int32_t N, H, W, C, OH, OW, KH, KW, SH, SW, PT, PL, Kp;
+};
+hipError_t launchIm2colBf16(const Im2colBf16Args &a, hipStream_t stream);
+
+// bf16 depthwise convolution: fp32 accumulation over (kh, kw), float bias and clamp.
+struct DepthwiseBf16Args {
+    const uint16_t *in;   // NHWC
+    const uint16_t *wpk;  // [KH][KW][C]
+    const float *bias;    // [C]
+    uint16_t *out;        // NHWC
+    int32_t N, H, W, C, OH, OW, KH, KW, SH, SW, PT, PL;
+    float lo, hi;
+};
+hipError_t launchDepthwiseBf16(const DepthwiseBf16Args &a, hipStream_t stream);
+
 // bf16 add: out = bf16(clamp(in0 * w0 + in1 * w1 + bias)) in fp32.
 struct AddBf16Args {
     const uint16_t *in0;

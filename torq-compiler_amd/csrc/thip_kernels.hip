@@ -1897,7 +1897,69 @@ hipError_t launchAdd(const AddArgs &a, hipStream_t stream) {
     return hipGetLastError();
 }
 
-// Batched byte transpose [B][R][S] -> [B][S][R] through a 64 x 64 LDS tile.
+// Patch matrix of a bf16 convolution (the GEMM that follows streams it like any other input): one
+// thread per element.  Not a fast path: the int8 convolutions gather inside the GEMM instead.
+__global__ __launch_bounds__(256) void im2col_bf16(Im2colBf16Args p, long long total) {
+    const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (t >= total) return;
+    const int k = (int)(t % p.Kp);
+    const long long m = t / p.Kp;
+    uint16_t v = 0;
+    if (k < p.KH * p.KW * p.C) {
+        const int ci = k % p.C, pos = k / p.C, kw = pos % p.KW, kh = pos / p.KW;
+        const int ox = (int)(m % p.OW);
+        const long long r = m / p.OW;
+        const int oy = (int)(r % p.OH), n = (int)(r / p.OH);
+        const int iy = oy * p.SH - p.PT + kh, ix = ox * p.SW - p.PL + kw;
+        if ((unsigned)iy < (unsigned)p.H && (unsigned)ix < (unsigned)p.W) v = p.in[(((size_t)n * p.H + iy) * p.W + ix) * p.C + ci];
+    }
+    p.out[t] = v;
+}
+
+hipError_t launchIm2colBf16(const Im2colBf16Args &a, hipStream_t stream) {
+    if (!a.in || !a.out || !poolGeometryOk(a.N, a.H, a.W, a.C, a.OH, a.OW, a.KH, a.KW, a.SH, a.SW, a.PT, a.PL)) return hipErrorInvalidValue;
+    if (a.Kp < a.KH * a.KW * a.C) return hipErrorInvalidValue;
+    const long long total = (long long)a.N * a.OH * a.OW * a.Kp;
+    if (total >= (1LL << 39)) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(im2col_bf16, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a, total);
+    return hipGetLastError();
+}
+
+// bf16 depthwise: one thread per output element, taps accumulated in (kh, kw) order in fp32 (the
+// products are exact, so a fused multiply-add gives the same sums as a multiply and an add).
+__global__ __launch_bounds__(256) void depthwise_bf16(DepthwiseBf16Args p, long long total) {
+    const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (t >= total) return;
+    const int c = (int)(t % p.C);
+    long long r = t / p.C;
+    const int ox = (int)(r % p.OW);
+    r /= p.OW;
+    const int oy = (int)(r % p.OH), n = (int)(r / p.OH);
+    float acc = 0.0f;
+    for (int kh = 0; kh < p.KH; kh++) {
+        const int iy = oy * p.SH - p.PT + kh;
+        if ((unsigned)iy >= (unsigned)p.H) continue;
+        for (int kw = 0; kw < p.KW; kw++) {
+            const int ix = ox * p.SW - p.PL + kw;
+            if ((unsigned)ix >= (unsigned)p.W) continue;
+            const float x = __uint_as_float((uint32_t)p.in[(((size_t)n * p.H + iy) * p.W + ix) * p.C + c] << 16);
+            const float w = __uint_as_float((uint32_t)p.wpk[((size_t)kh * p.KW + kw) * p.C + c] << 16);
+            acc = __fadd_rn(acc, __fmul_rn(x, w));
+        }
+    }
+    const float t0 = __fadd_rn(acc, p.bias[c]);
+    p.out[t] = bf16Bits(t0 < p.lo ? p.lo : (t0 > p.hi ? p.hi : t0));
+}
+
+hipError_t launchDepthwiseBf16(const DepthwiseBf16Args &a, hipStream_t stream) {
+    if (!a.in || !a.wpk || !a.bias || !a.out) return hipErrorInvalidValue;
+    if (!poolGeometryOk(a.N, a.H, a.W, a.C, a.OH, a.OW, a.KH, a.KW, a.SH, a.SW, a.PT, a.PL)) return hipErrorInvalidValue;
+    const long long total = (long long)a.N * a.OH * a.OW * a.C;
+    if (total >= (1LL << 39)) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(depthwise_bf16, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a, total);
+    return hipGetLastError();
+}
+
 // bf16 add: 8 elements (16 bytes) per thread when the tensors allow it.  No fused multiply-add: the second
 // product is added to the first (both exact in fp32), then the bias, as the ACT stage does.
 template <int VEC>
@@ -1944,6 +2006,7 @@ hipError_t launchAddBf16(const AddBf16Args &a, hipStream_t stream) {
     return hipGetLastError();
 }
 
+// Batched transpose [B][R][S] -> [B][S][R] of 1- or 2-byte elements through a 64 x 64 LDS tile.
 template <typename T>
 __global__ __launch_bounds__(256) void transpose_i8(TransposeArgs p) {
     __shared__ T tile[64][65];

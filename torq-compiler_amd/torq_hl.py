@@ -104,6 +104,8 @@ class Program:
         OH = _window_out(H, KH, pad[2], pad[3], stride[0])
         OW = _window_out(W, KW, pad[0], pad[1], stride[1])
         shape = (N, OH, OW, O) if nhwc_input else (N, O, OH, OW)
+        if input.dtype == np.uint16:  # bf16 bit patterns in, bf16 out
+            out_dtype = np.uint16
         init = self._init_or_new(init, shape, out_dtype)
         op = rt.HlConv2d(init.index, input_zp, weight_zp, output_zp, output_min, output_max, shift_factor,
                          groups, (ctypes.c_int64 * 4)(*pad), (ctypes.c_int64 * 2)(*stride),
@@ -126,7 +128,7 @@ class Program:
         OH = _window_out(H, KH, pad[2], pad[3], stride[0])
         OW = _window_out(W, KW, pad[0], pad[1], stride[1])
         shape = (N, OH, OW, C) if nhwc_input else (N, C, OH, OW)
-        init = self._init_or_new(init, shape, np.int8)
+        init = self._init_or_new(init, shape, np.uint16 if input.dtype == np.uint16 else np.int8)
         op = rt.HlDepthwiseConv2d(init.index, input_zp, weight_zp, output_zp, output_min, output_max,
                                   shift_factor, C if groups is None else groups,
                                   (ctypes.c_int64 * 4)(*pad), (ctypes.c_int64 * 2)(*stride),
@@ -179,7 +181,7 @@ class Program:
         OH = _window_out(H, kernel[0], pad[2], pad[3], stride[0])
         OW = _window_out(W, kernel[1], pad[0], pad[1], stride[1])
         shape = (N, OH, OW, C) if nhwc_input else (N, C, OH, OW)
-        init = self._init_or_new(init, shape, np.int8)
+        init = self._init_or_new(init, shape, np.uint16 if input.dtype == np.uint16 else np.int8)
         widx = self._as_value(weights).index if weights is not None else -1
         sidx = self._as_value(scale_bias).index if scale_bias is not None else -1
         op = rt.HlMaxPool2d(init.index, input_zp, output_min, output_max, (ctypes.c_int64 * 2)(*stride),

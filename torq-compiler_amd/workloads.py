@@ -165,6 +165,35 @@ def matmul_bf16_workload(B, M, K, N, batch1=True, batch2=True, constant_rhs=Fals
                     a.nbytes + b.nbytes + 2 * int(np.prod(oshape)), attrs)
 
 
+def conv2d_bf16_workload(N=1, H=14, W=14, C=16, O=24, KH=3, KW=3, stride=(1, 1), pad=(1, 1, 1, 1), nhwc=True, clamp=None,
+                         depthwise=False, seed=1013):
+    """bf16 conv2d (or depthwise_conv2d, O = C): fp32 accumulate, float bias, zero padding."""
+    rng = np.random.default_rng(seed)
+    x = to_bf16(rng.standard_normal((N, H, W, C)))
+    if depthwise:
+        O = C
+        wts = to_bf16(rng.standard_normal((C, 1, KH, KW)) / np.sqrt(KH * KW))
+    else:
+        wts = to_bf16(rng.standard_normal((O, C, KH, KW)) / np.sqrt(C * KH * KW))
+    bias = rng.standard_normal(O).astype(np.float32)
+    lo, hi = NO_CLAMP if clamp is None else (float_bits(clamp[0]), float_bits(clamp[1]))
+    if not nhwc:
+        x = np.ascontiguousarray(x.transpose(0, 3, 1, 2))
+    OH = (H + pad[2] + pad[3] - KH) // stride[0] + 1
+    OW = (W + pad[0] + pad[1] - KW) // stride[1] + 1
+    oshape = (N, OH, OW, O) if nhwc else (N, O, OH, OW)
+    p = Program()
+    inp = p.binding(0, x.shape, np.uint16)
+    out = p.binding(1, oshape, np.uint16)
+    fn = p.depthwise_conv2d if depthwise else p.conv2d
+    fn(inp, wts, bias, init=out, input_zp=0, output_zp=0, output_min=lo, output_max=hi, shift_factor=0, pad=tuple(pad),
+       stride=tuple(stride), nhwc_input=nhwc)
+    macs = N * OH * OW * O * KH * KW * (1 if depthwise else C)
+    attrs = dict(weights=wts, bias=bias, output_min=lo, output_max=hi, pad=tuple(pad), stride=tuple(stride), nhwc=nhwc)
+    name = "%sbf16_%dx%dx%dx%d_o%d_k%dx%d_s%d" % ("dw" if depthwise else "conv", N, H, W, C, O, KH, KW, stride[0])
+    return Workload(name, p, [x], [(oshape, np.uint16)], 2 * macs, x.nbytes + wts.nbytes + bias.nbytes + 2 * int(np.prod(oshape)), attrs)
+
+
 def add_bf16_workload(shape=(1, 32, 1152), w0=1.0, w1=1.0, bias=0.0, clamp=None, seed=1012):
     """bf16 add (a residual connection of a decoder layer): in1 * w0 + in2 * w1 + bias in fp32."""
     rng = np.random.default_rng(seed)
