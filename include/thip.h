@@ -201,7 +201,10 @@ typedef struct thip_hl_maxpool2d_t {
 } thip_hl_maxpool2d_t;
 
 /* torq_hl.avg_pool2d -- TorqHLOps.td:192-208.  Global: input N,H,W,C (NHWC),
- * init N,1,1,C; weights one int8; pair 0 of scale_bias applies to every channel. */
+ * init N,1,1,C; weights one int8; pair 0 of scale_bias applies to every channel.
+ * bf16 form (compiler/torq/Conversions/LinalgToTorqHL/PoolingPattern.cpp:448-457): weights one BF16 (1.0 or a
+ * folded multiplier), scale_bias F32[1] (bias only), shift_factor and zero points 0, output_min / output_max
+ * float bit patterns; the frame is summed in order in fp32. */
 typedef struct thip_hl_avg_pool2d_t {
     thip_value_t init;
     int32_t input_zp;
@@ -245,6 +248,24 @@ typedef struct thip_hl_transpose_t {
     thip_value_t input;
 } thip_hl_transpose_t;
 
+/* torq_hl.expand_weights -- TorqHLOps.td:943-957 (fields in the op's order); the block-quantized right-hand
+ * side of a bf16 matmul (compiler/torq/Conversions/LinalgToTorqHL/MatmulPattern.cpp:596-680).  input int8
+ * K,N; scale BF16 K/block_size,N; scale_bias F32 K/block_size,cols with cols >= N (the float bias
+ * -zero_point * scale, columns rounded up to even, MatmulPattern.cpp:322-400); init BF16 K,N or 1,K,N:
+ * init = bf16(clamp(input * scale + scale_bias)), output_min / output_max float bit patterns.  When every
+ * operand is a constant and the only reader of init is input2 of a bf16 torq_hl.matmul, no kernel is
+ * emitted: the matmul streams the int8 weights and expands them in registers (few rows), or reads weights
+ * expanded at serialisation (many rows). */
+typedef struct thip_hl_expand_weights_t {
+    thip_value_t init;
+    thip_value_t scale_bias;
+    int32_t output_min;
+    int32_t output_max;
+    thip_value_t scale;
+    thip_value_t input;
+    int32_t block_size;
+} thip_hl_expand_weights_t;
+
 thip_status_t thip_hl_conv2d(thip_program_t *program, const thip_hl_conv2d_t *op);
 thip_status_t thip_hl_depthwise_conv2d(thip_program_t *program,
                                        const thip_hl_depthwise_conv2d_t *op);
@@ -255,6 +276,7 @@ thip_status_t thip_hl_maxpool2d(thip_program_t *program, const thip_hl_maxpool2d
 thip_status_t thip_hl_avg_pool2d(thip_program_t *program, const thip_hl_avg_pool2d_t *op);
 thip_status_t thip_hl_add(thip_program_t *program, const thip_hl_add_t *op);
 thip_status_t thip_hl_transpose(thip_program_t *program, const thip_hl_transpose_t *op);
+thip_status_t thip_hl_expand_weights(thip_program_t *program, const thip_hl_expand_weights_t *op);
 
 /* Serialises the program (role of TargetBackend::serializeExecutable,
  * compiler/torq/Target/TorqTarget.cpp:115-151, and serializeTorqHW,

@@ -274,6 +274,34 @@ def add_bf16(input1, input2, weights, bias, *, output_min=NO_CLAMP_MIN, output_m
     return out
 
 
+def avg_pool2d_bf16(input, weight, bias, *, output_min=NO_CLAMP_MIN, output_max=NO_CLAMP_MAX):
+    """torq_hl.avg_pool2d on bf16 bit patterns (N,H,W,C): one bf16 weight, one float32 bias; result N,1,1,C."""
+    x = _c(input, np.uint16)
+    N, H, W, C = x.shape
+    w = _c(weight, np.uint16).reshape(-1)
+    bias = _c(bias, np.float32).reshape(-1)
+    assert w.size >= 1 and bias.size >= 1
+    out = np.empty((N, 1, 1, C), dtype=np.uint16)
+    rc = lib().torq_avg_pool2d_bf16(_p(x), ctypes.c_uint16(int(w[0])), _p(bias), _p(out), N, H, W, C, int(output_min), int(output_max))
+    assert rc == 0
+    return out
+
+
+def expand_weights(weights, scale, bias, *, block_size, output_min=NO_CLAMP_MIN, output_max=NO_CLAMP_MAX):
+    """torq_hl.expand_weights: int8 weights [K, N], bf16 scales [K / block_size, N], float32 biases
+    [K / block_size, >= N]; result bf16 bit patterns [K, N]."""
+    w = _c(weights, np.int8)
+    K, N = w.shape
+    sc = _c(scale, np.uint16)
+    b = _c(bias, np.float32)
+    G = K // block_size
+    assert G * block_size == K and sc.shape == (G, N) and b.shape[0] == G and b.shape[1] >= N
+    out = np.empty((K, N), dtype=np.uint16)
+    rc = lib().torq_expand_weights(_p(w), _p(sc), _p(b), _p(out), K, N, int(block_size), int(b.shape[1]), int(output_min), int(output_max))
+    assert rc == 0
+    return out
+
+
 def maxpool2d(input, *, input_zp, output_min, output_max, stride, pad, kernel, layout=NCHW):
     """torq_hl.maxpool2d."""
     x = _c(input, np.int8)

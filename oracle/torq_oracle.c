@@ -406,6 +406,53 @@ int torq_add_bf16(const uint16_t *input1, const uint16_t *input2, const uint16_t
 }
 
 /*
+ * torq_hl.avg_pool2d on bf16 -- created compiler/torq/Conversions/LinalgToTorqHL/PoolingPattern.cpp:448-457
+ * (ONE bf16 weight: 1.0, or the constant of a mulf/divf that follows the pool, folded in; scale_bias is a
+ * single float bias 0.0; clamp at -inf/+inf); executed by the same slice program as the int8 op
+ * (compiler/torq/Conversions/TorqHLToTorqHW/AvgpoolPattern.cpp:67-83): for each channel the products
+ * x[u] * w are accumulated over the frame u = 0 .. H*W-1 in order, in fp32, then the float ACT stage.
+ */
+int torq_avg_pool2d_bf16(const uint16_t *input, uint16_t weight, const float *bias, uint16_t *out,
+                         int N, int H, int W, int C, int32_t clip_min, int32_t clip_max) {
+    const float lo = float_from_bits(clip_min), hi = float_from_bits(clip_max);
+    const float w = torq_bf16_to_f32(weight);
+    const size_t HW = (size_t)H * W;
+#pragma omp parallel for collapse(2) schedule(static)
+    for (int n = 0; n < N; n++) {
+        for (int c = 0; c < C; c++) {
+            float acc = 0.0f;
+            for (size_t u = 0; u < HW; u++) acc += torq_bf16_to_f32(input[((size_t)n * HW + u) * C + c]) * w;
+            out[(size_t)n * C + c] = act_float(acc, bias[0], lo, hi);
+        }
+    }
+    return 0;
+}
+
+/*
+ * torq_hl.expand_weights -- signature TorqHLOps.td:943-957; created for the right-hand side of a matmul by
+ * compiler/torq/Conversions/LinalgToTorqHL/MatmulPattern.cpp:596-680 (weights [G, B, N] flattened to [K, N],
+ * scales [G, N], scale_bias = the float bias -zero_point * scale, [G, cols rounded up to even]
+ * MatmulPattern.cpp:322-400; clamp = the float range -inf/+inf); executed
+ * compiler/torq/Conversions/TorqHLToTorqHW/ExpandWeightsPattern.cpp:42-98: per block of `block_size` rows
+ * one scale and one bias per column, out = weight * scale (elementwise product in fp32, exact for an 8-bit
+ * weight and a bf16 scale) then the float ACT stage (+ bias, clamp, round to bf16).
+ */
+int torq_expand_weights(const int8_t *weights, const uint16_t *scale, const float *bias, uint16_t *out,
+                        int K, int N, int block_size, int bias_cols, int32_t clip_min, int32_t clip_max) {
+    const float lo = float_from_bits(clip_min), hi = float_from_bits(clip_max);
+    if (block_size <= 0 || K % block_size != 0 || bias_cols < N) return -1;
+#pragma omp parallel for schedule(static)
+    for (int k = 0; k < K; k++) {
+        const size_t g = (size_t)(k / block_size);
+        for (int n = 0; n < N; n++) {
+            const float p = (float)weights[(size_t)k * N + n] * torq_bf16_to_f32(scale[g * N + n]);
+            out[(size_t)k * N + n] = act_float(p, bias[g * bias_cols + n], lo, hi);
+        }
+    }
+    return 0;
+}
+
+/*
  * torq_hl.maxpool2d -- signature TorqHLOps.td:435-453; created
  * compiler/torq/Conversions/LinalgToTorqHL/PoolingPattern.cpp:199-236 (pad value
  * becomes input_zp, output_min/max = element type range); executed

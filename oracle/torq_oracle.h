@@ -106,6 +106,16 @@ int torq_depthwise_conv2d_bf16(const uint16_t *input, const uint16_t *weights, c
 int torq_add_bf16(const uint16_t *input1, const uint16_t *input2, const uint16_t weights[2], const float *bias,
                   uint16_t *out, size_t count, int32_t clip_min, int32_t clip_max);
 
+/* torq_hl.avg_pool2d (global) on bf16: out[n][c] = bf16(clamp(sum_u x[n][u][c] * weight + bias[0])), summed
+ * over the frame in order, in fp32. */
+int torq_avg_pool2d_bf16(const uint16_t *input, uint16_t weight, const float *bias, uint16_t *out,
+                         int N, int H, int W, int C, int32_t clip_min, int32_t clip_max);
+
+/* torq_hl.expand_weights: int8 weights K x N, bf16 scales and float biases per block of block_size rows
+ * (bias rows are bias_cols >= N wide): out = bf16(clamp(weight * scale + bias)). */
+int torq_expand_weights(const int8_t *weights, const uint16_t *scale, const float *bias, uint16_t *out,
+                        int K, int N, int block_size, int bias_cols, int32_t clip_min, int32_t clip_max);
+
 /* torq_hl.maxpool2d.  No rescale; padding value is input_zp; result is
  * clamped to [output_min, output_max]. */
 int torq_maxpool2d(const int8_t *input, int8_t *out, int N, int C, int H, int W, int KH, int KW,

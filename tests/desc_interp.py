@@ -25,6 +25,7 @@ TEMP = np.dtype([("size", "<u8")])
 CONST = np.dtype([("offset", "<u8"), ("size", "<u8")])
 
 K_TRANSPOSE, K_IGEMM, K_FC_SKINNY, K_DW, K_MAXPOOL, K_AVGPOOL, K_ADD, K_FC_BF16, K_ADD_BF16, K_IM2COL_BF16, K_DW_BF16 = 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11
+K_AVGPOOL_BF16, K_EXPAND = 12, 13
 OUT_NP = {1: np.int8, 2: np.int16, 3: np.int32}
 
 
@@ -225,7 +226,18 @@ def run(blob, binding_arrays):
         elif kind == K_FC_BF16:
             M, K, N = int(op["M"]), int(op["K"]), int(op["Nn"])
             x = view(op["in0"], M * K * 2).view(np.uint16).reshape(M, K)
-            if int(op["loader"]) == 1:  # fragment order: [column block][k step][piece][lane] x 8 elements
+            if int(op["loader"]) == 2:  # block-quantized int8: [column block][k step][half][lane] x 16 bytes, tables [G][Np]
+                steps, nbk = (K + 63) // 64, (N + 31) // 32
+                block, cols = int(op["gran"]), int(op["Np"])
+                G = K // block
+                frag = view(op["weights"], nbk * 32 * steps * 64).view(np.int8).reshape(nbk, steps, 2, 2, 32, 16)  # [nb][s][h2][h][r][e]
+                full = frag.transpose(0, 4, 1, 3, 2, 5).reshape(nbk * 32, steps * 64)  # [nb, r][s, h, h2, e]
+                assert not full[N:].any() and not full[:, K:].any()
+                sc = view(op["scale"], G * cols * 2).view(np.uint16).reshape(G, cols)
+                bi = view(op["table"], G * cols * 4).view(np.float32).reshape(G, cols)
+                wt = np.ascontiguousarray(orc.expand_weights(np.ascontiguousarray(full[:N, :K].T), sc[:, :N], bi, block_size=block,
+                                                             output_min=int(op["bias0"]), output_max=int(op["scale0"])).T)
+            elif int(op["loader"]) == 1:  # fragment order: [column block][k step][piece][lane] x 8 elements
                 steps, nbk = (K + 63) // 64, (N + 31) // 32
                 frag = view(op["weights"], nbk * 32 * steps * 64 * 2).view(np.uint16).reshape(nbk, steps, 4, 2, 32, 8)
                 full = frag.transpose(0, 4, 1, 3, 2, 5).reshape(nbk * 32, steps * 64)  # [nb, r][s, h, c, e]
@@ -236,6 +248,20 @@ def run(blob, binding_arrays):
             bias = view(op["bias"], N * 4).view(np.float32)
             res = orc.fully_connected_bf16(x, wt, bias, output_min=mn, output_max=mx)
             view(op["out"], M * N * 2).view(np.uint16)[:] = res.reshape(-1)
+        elif kind == K_AVGPOOL_BF16:
+            Nimg, H, W, C = (int(op[k]) for k in ["N", "H", "W", "C"])
+            x = view(op["in0"], Nimg * H * W * C * 2).view(np.uint16).reshape(Nimg, H, W, C)
+            res = orc.avg_pool2d_bf16(x, np.array([op["w0"]], dtype=np.uint16), np.array([op["bias0"]], dtype=np.int32).view(np.float32),
+                                      output_min=mn, output_max=mx)
+            view(op["out"], Nimg * C * 2).view(np.uint16)[:] = res.reshape(-1)
+        elif kind == K_EXPAND:
+            K, N, block, cols = int(op["K"]), int(op["Nn"]), int(op["gran"]), int(op["Np"])
+            G = K // block
+            wq = view(op["in0"], K * N).view(np.int8).reshape(K, N)
+            sc = view(op["scale"], G * N * 2).view(np.uint16).reshape(G, N)
+            bi = view(op["bias"], G * cols * 4).view(np.float32).reshape(G, cols)
+            res = orc.expand_weights(wq, sc, bi, block_size=block, output_min=mn, output_max=mx)
+            view(op["out"], K * N * 2).view(np.uint16)[:] = res.reshape(-1)
         else:
             raise AssertionError("unknown kernel kind %d" % kind)
     return d

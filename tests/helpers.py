@@ -26,6 +26,13 @@ def oracle_eval(wl):
         fn = orc.conv2d_bf16 if kind == "convbf16" else orc.depthwise_conv2d_bf16
         return [fn(x, a["weights"], a["bias"], pad=a["pad"], stride=a["stride"], output_min=a["output_min"], output_max=a["output_max"],
                    layout=orc.NHWC if a["nhwc"] else orc.NCHW)]
+    if kind == "avgpoolbf16":
+        return [orc.avg_pool2d_bf16(x, a["weights"], a["bias"], output_min=a["output_min"], output_max=a["output_max"])]
+    if kind == "expandmm":
+        w16 = orc.expand_weights(a["weights"], a["scale"], a["qbias"], block_size=a["block"], output_min=a["expand_min"],
+                                 output_max=a["expand_max"])
+        res = [orc.matmul_bf16(x, w16, a["bias"], output_min=a["output_min"], output_max=a["output_max"])]
+        return res if a["fold"] else res + [w16[None]]
     if kind == "addbf16":
         return [orc.add_bf16(wl.inputs[0], wl.inputs[1], a["weights"], a["bias"], output_min=a["output_min"], output_max=a["output_max"])]
     if kind == "matmulbf16":

@@ -1,5 +1,7 @@
 """bf16 rows of fully_connected / matmul: the oracle's pins, the emitter, and (on a GPU) the kernel, which is a
 tolerance row: at most one bf16 ULP from the oracle per element."""
+import os
+
 import numpy as np
 import pytest
 
@@ -93,6 +95,37 @@ def test_bf16_conv_oracle_pins():
         assert_bf16_close(got, orc.to_bf16(exact.astype(np.float32)), "depthwise bf16 vs float64")
 
 
+def test_bf16_avg_pool_and_expand_weights_oracle_pins():
+    """Global average pool: exact on small integers with a power-of-two weight, within one ULP of the float64 mean.
+    expand_weights: exact when scale and bias are small integers (and equal to (w - zp) * scale, the dequantisation the
+    op stands for), within one ULP of float64 otherwise, clamp, padded bias rows."""
+    rng = np.random.default_rng(11)
+    xi = rng.integers(-8, 9, size=(3, 4, 4, 10))
+    got = orc.avg_pool2d_bf16(orc.to_bf16(xi), orc.to_bf16(np.array([1.0 / 16])), np.array([2.0], dtype=np.float32))
+    assert np.array_equal(got.reshape(3, 10), orc.to_bf16((xi.sum(axis=(1, 2)) / 16.0 + 2.0).astype(np.float32)))
+    x = orc.to_bf16(rng.standard_normal((2, 7, 7, 33)) + 0.5)
+    wt = orc.to_bf16(np.array([1.0 / 49]))
+    exact = orc.from_bf16(x).astype(np.float64).sum(axis=(1, 2)) * float(orc.from_bf16(wt)[0])
+    got = orc.avg_pool2d_bf16(x, wt, np.zeros(1, dtype=np.float32), output_min=w.float_bits(0.0), output_max=w.float_bits(0.75))
+    mag = np.abs(orc.from_bf16(x).astype(np.float64)).sum(axis=(1, 2)) * float(orc.from_bf16(wt)[0])
+    assert_bf16_close(got.reshape(2, 33), orc.to_bf16(np.clip(exact, 0.0, 0.75).astype(np.float32)), "avgpool bf16 vs float64", magnitude=mag)
+
+    K, N, block = 64, 10, 32
+    wq = rng.integers(-128, 128, size=(K, N), dtype=np.int8)
+    sci = rng.integers(1, 4, size=(2, N))
+    zp = rng.integers(-5, 6, size=(2, N))
+    qb = np.zeros((2, N + 2), dtype=np.float32)
+    qb[:, :N] = -zp * sci
+    got = orc.expand_weights(wq, orc.to_bf16(sci), qb, block_size=block)
+    want = (wq.astype(np.int64) - np.repeat(zp, block, axis=0)) * np.repeat(sci, block, axis=0)
+    assert np.array_equal(got, orc.to_bf16(want.astype(np.float32)))
+    sc = orc.to_bf16(rng.uniform(0.001, 0.02, size=(2, N)))
+    qb = rng.standard_normal((2, N)).astype(np.float32)
+    exact = wq.astype(np.float64) * np.repeat(orc.from_bf16(sc).astype(np.float64), block, axis=0) + np.repeat(qb.astype(np.float64), block, axis=0)
+    got = orc.expand_weights(wq, sc, qb, block_size=block, output_min=w.float_bits(-1.0), output_max=w.float_bits(1.5))
+    assert_bf16_close(got, orc.to_bf16(np.clip(exact, -1.0, 1.5).astype(np.float32)), "expand_weights vs float64", magnitude=np.abs(exact) + 1)
+
+
 def test_bf16_add_closed_forms():
     # weights 1 and -1 on equal inputs cancel exactly: the bias alone remains; small integers are exact
     rng = np.random.default_rng(6)
@@ -121,14 +154,40 @@ def test_bf16_add_closed_forms():
                                   lambda: w.conv2d_bf16_workload(N=2, H=6, W=6, C=16, O=40, KH=1, KW=1, pad=(0, 0, 0, 0)),
                                   lambda: w.conv2d_bf16_workload(depthwise=True, C=12, stride=(2, 2), pad=(0, 1, 0, 1), clamp=(-0.5, 0.5)),
                                   lambda: w.conv2d_bf16_workload(depthwise=True, N=2, C=5, H=7, W=9, nhwc=False),
+                                  lambda: w.avg_pool2d_bf16_workload(), lambda: w.avg_pool2d_bf16_workload(N=3, H=5, W=4, C=7, weight=1.0, clamp=(-1.0, 1.0)),
+                                  lambda: w.expand_weights_workload(), lambda: w.expand_weights_workload(M=70, K=128, N=40, block=64, clamp=(-2.0, 2.0)),
+                                  lambda: w.expand_weights_workload(M=3, K=96, N=20, block=48, bias_pad=2),
+                                  lambda: w.expand_weights_workload(M=2, K=64, N=33, fold=False, expand_clamp=(-0.01, 0.02), bias_pad=1),
                                   lambda: w.add_bf16_workload(), lambda: w.add_bf16_workload((3, 5, 7), 0.5, -1.25, 0.125, clamp=(-1.0, 2.0))])
 def test_bf16_descriptor(make):
     wl = make()
     outs = [np.zeros(s, dtype=dt) for s, dt in wl.outputs]
     d = desc_interp.run(wl.program.serialize(), list(wl.inputs) + outs)
-    assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)
+    for got, want in zip(outs, oracle_eval(wl)):
+        assert_bit_exact(got, want.reshape(got.shape), wl.name)
     kinds = [int(o["kind"]) for o in d.ops]
-    assert {desc_interp.K_FC_BF16, desc_interp.K_ADD_BF16, desc_interp.K_DW_BF16} & set(kinds)
+    assert {desc_interp.K_FC_BF16, desc_interp.K_ADD_BF16, desc_interp.K_DW_BF16, desc_interp.K_AVGPOOL_BF16} & set(kinds)
+
+
+def test_expand_weights_folding():
+    """An expansion that only feeds a bf16 matmul emits no kernel: few rows take the int8 weights (layout 2), many rows
+    or a block size the kernel does not take get weights expanded at serialisation; an expansion that is also an
+    output, or THIP_NO_EXPAND_FOLD, stays a kernel of its own followed by the transpose of a run-time input2."""
+    def kinds_loader(wl):
+        d = desc_interp.Descriptor(wl.program.serialize())
+        return [int(o["kind"]) for o in d.ops], [int(o["loader"]) for o in d.ops if int(o["kind"]) == desc_interp.K_FC_BF16]
+
+    assert kinds_loader(w.expand_weights_workload()) == ([desc_interp.K_FC_BF16], [2])
+    assert kinds_loader(w.expand_weights_workload(M=70, K=128, N=40, block=64)) == ([desc_interp.K_FC_BF16], [1])
+    assert kinds_loader(w.expand_weights_workload(M=3, K=96, N=20, block=48)) == ([desc_interp.K_FC_BF16], [1])
+    kinds, loaders = kinds_loader(w.expand_weights_workload(fold=False))
+    assert kinds == [desc_interp.K_EXPAND, desc_interp.K_TRANSPOSE, desc_interp.K_FC_BF16] and loaders == [0]
+    os.environ["THIP_NO_EXPAND_FOLD"] = "1"
+    try:
+        kinds, _ = kinds_loader(w.expand_weights_workload())
+    finally:
+        del os.environ["THIP_NO_EXPAND_FOLD"]
+    assert kinds == [desc_interp.K_EXPAND, desc_interp.K_TRANSPOSE, desc_interp.K_FC_BF16]
 
 
 def test_bf16_rejections():
@@ -210,6 +269,40 @@ def test_gpu_bf16_conv2d_and_depthwise(device):
         got, kernels = run_on_gpu(device, wl, via="device")
         assert_bit_exact(got[0], oracle_eval(wl)[0], wl.name)
         assert "depthwise_bf16" in kernels
+
+
+@pytest.mark.gpu
+def test_gpu_bf16_avg_pool(device):
+    """The kernel walks the frame in the oracle's order: bit-exact."""
+    for wl in [w.avg_pool2d_bf16_workload(), w.avg_pool2d_bf16_workload(N=64), w.avg_pool2d_bf16_workload(N=3, H=5, W=4, C=7, weight=1.0, clamp=(-1.0, 1.0)),
+               w.avg_pool2d_bf16_workload(N=1, H=14, W=14, C=96, weight=0.0078125)]:
+        print("[gpu-case]", wl.name, flush=True)
+        got, kernels = run_on_gpu(device, wl, via="device")
+        assert_bit_exact(got[0], oracle_eval(wl)[0], wl.name)
+        assert kernels == ["avgpool_bf16"]
+
+
+@pytest.mark.gpu
+def test_gpu_expand_weights(device):
+    """Block-quantized weights: expanded in registers by the matmul (decoder shapes at 1 and 32 tokens, split K, ragged
+    N, an expansion clamp), expanded at serialisation (many rows), and as a kernel of its own, whose result is bit-exact."""
+    f = lambda bits: np.abs(orc.from_bf16(bits).astype(np.float64))
+    cases = [(w.expand_weights_workload(), "q8"), (w.expand_weights_workload(M=1, K=1152, N=1024, block=128), "q8"),
+             (w.expand_weights_workload(M=32, K=6912, N=1152, block=64), "q8"), (w.expand_weights_workload(M=5, K=192, N=45, block=96, bias_pad=1), "q8"),
+             (w.expand_weights_workload(M=7, K=128, N=70, expand_clamp=(-0.004, 0.006), clamp=(-0.05, 0.05)), "q8"),
+             (w.expand_weights_workload(M=70, K=128, N=40, block=64), "folded"), (w.expand_weights_workload(M=2, K=64, N=33, fold=False, bias_pad=1), "own")]
+    for wl, how in cases:
+        print("[gpu-case]", wl.name, how, flush=True)
+        got, kernels = run_on_gpu(device, wl)
+        want = oracle_eval(wl)
+        w16 = orc.expand_weights(wl.attrs["weights"], wl.attrs["scale"], wl.attrs["qbias"], block_size=wl.attrs["block"],
+                                 output_min=wl.attrs["expand_min"], output_max=wl.attrs["expand_max"])
+        assert_bf16_close(got[0], want[0].reshape(got[0].shape), wl.name, magnitude=f(wl.inputs[0]) @ f(w16))
+        if how == "own":
+            assert_bit_exact(got[1], want[1], wl.name + " expansion")
+            assert kernels == ["expand_weights_bf16", "transpose_i8", "fc_bf16"], kernels
+        else:
+            assert kernels == ["fc_bf16"], kernels
 
 
 @pytest.mark.gpu

@@ -72,7 +72,14 @@ enum Kind : uint32_t {
     kKindAddBf16 = 9,    // bf16 add: w0 / w1 bf16 bits, bias0 / output_min / output_max float bits, C = element count
     kKindIm2colBf16 = 10,     // bf16 N,H,W,C image -> [M][Kp] patch matrix, k = (kh * KW + kw) * C + ci, zero padded
     kKindDepthwiseBf16 = 11,  // bf16 depthwise: weights [KH][KW][C] bf16, bias f32[C]
-    kKindFcBf16 = 8,     // bf16 fully_connected / matmul: fp32 accumulate, float bias, float clamp (output_min/max bits)
+    // bf16 fully_connected / matmul: fp32 accumulate, float bias, float clamp (output_min/max bits).  loader: weight
+    // layout, 0 rows, 1 fragment order, 2 block-quantized int8 in fragment order (a folded torq_hl.expand_weights):
+    // scale = bf16 scales [K / gran][Np], table = float biases [K / gran][Np], gran = rows per block, bias0 / scale0
+    // = float bits of the expansion's clamp.
+    kKindFcBf16 = 8,
+    kKindAvgPoolBf16 = 12,    // bf16 global average pool: w0 = bf16 bits of the weight, bias0 = float bits of the bias
+    // torq_hl.expand_weights: in0 int8 [K][Nn], scale bf16 [K / gran][Nn], bias float [K / gran][Np], out bf16 [K][Nn]
+    kKindExpandWeights = 13,
 };
 
 // Variants of kKindIgemm: how the A (activation) tile is gathered.

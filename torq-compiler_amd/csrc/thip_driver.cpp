@@ -264,6 +264,19 @@ static thip_status_t checkOpFootprint(const thip_executable_t *e, uint32_t i) {
         if ((s = need(op.bias, (uint64_t)op.C * 4, "bias"))) return s;
         return need(op.out, (uint64_t)op.N * op.OH * op.OW * op.C * 2, "out");
     }
+    case kKindAvgPoolBf16: {
+        if (!positive({op.N, op.H, op.W, op.C})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad avgpool extents", i);
+        if ((s = need(op.in0, (uint64_t)op.N * op.H * op.W * op.C * 2, "in"))) return s;
+        return need(op.out, (uint64_t)op.N * op.C * 2, "out");
+    }
+    case kKindExpandWeights: {
+        const int32_t block = (int32_t)op.gran;
+        if (!positive({op.K, op.Nn, block}) || op.K % block != 0 || op.Np < op.Nn) return fail(THIP_INVALID_ARGUMENT, "op %u: bad expand_weights extents", i);
+        if ((s = need(op.in0, (uint64_t)op.K * op.Nn, "weights"))) return s;
+        if ((s = need(op.scale, (uint64_t)(op.K / block) * op.Nn * 2, "scale"))) return s;
+        if ((s = need(op.bias, (uint64_t)(op.K / block) * op.Np * 4, "bias"))) return s;
+        return need(op.out, (uint64_t)op.K * op.Nn * 2, "out");
+    }
     case kKindAddBf16: {
         if (!positive({op.C})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad add extent", i);
         if ((s = need(op.in0, (uint64_t)op.C * 2, "in1"))) return s;
@@ -273,9 +286,18 @@ static thip_status_t checkOpFootprint(const thip_executable_t *e, uint32_t i) {
     case kKindFcBf16: {
         if (!positive({op.M, op.K, op.Nn}) || op.K % 8 != 0) return fail(THIP_INVALID_ARGUMENT, "op %u: bad bf16 fully_connected extents", i);
         if ((s = need(op.in0, (uint64_t)op.M * op.K * 2, "in"))) return s;
-        if (op.loader > 1) return fail(THIP_INVALID_ARGUMENT, "op %u: unknown bf16 weight layout %u", i, op.loader);
-        const uint64_t wBytes = op.loader == 1 ? (uint64_t)((op.Nn + 31) / 32 * 32) * ((op.K + 63) / 64 * 64) * 2 : (uint64_t)op.Nn * op.K * 2;
+        if (op.loader > 2) return fail(THIP_INVALID_ARGUMENT, "op %u: unknown bf16 weight layout %u", i, op.loader);
+        const uint64_t padded = (uint64_t)((op.Nn + 31) / 32 * 32) * ((op.K + 63) / 64 * 64);
+        const uint64_t wBytes = op.loader == 2 ? padded : op.loader == 1 ? padded * 2 : (uint64_t)op.Nn * op.K * 2;
         if ((s = need(op.weights, wBytes, "weights"))) return s;
+        if (op.loader == 2) {
+            const int32_t block = (int32_t)op.gran;
+            if (block < 32 || block % 32 != 0 || op.K % block != 0 || op.Np < (op.Nn + 31) / 32 * 32 || op.Np % 32 != 0) {
+                return fail(THIP_INVALID_ARGUMENT, "op %u: bad block-quantized weight tables", i);
+            }
+            if ((s = need(op.scale, (uint64_t)(op.K / block) * op.Np * 2, "block scales"))) return s;
+            if ((s = need(op.table, (uint64_t)(op.K / block) * op.Np * 4, "block biases"))) return s;
+        }
         if ((s = need(op.bias, (uint64_t)op.Nn * 4, "bias"))) return s;
         if (op.w0 > 1) {
             // K split over blocks: counters and partial sums live in an intermediate (zero-filled at creation)
@@ -301,6 +323,8 @@ static const char *opKernelName(const DescOp &op) {
     case kKindAddBf16: return "add_bf16";
     case kKindIm2colBf16: return "im2col_bf16";
     case kKindDepthwiseBf16: return "depthwise_bf16";
+    case kKindAvgPoolBf16: return "avgpool_bf16";
+    case kKindExpandWeights: return "expand_weights_bf16";
     default: return "unknown";
     }
 }
@@ -420,8 +444,37 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
         memcpy(&hi, &op.output_max, 4);
         FcBf16Args a{(const uint16_t *)resolve(e, op.in0, bp), (const uint16_t *)resolve(e, op.weights, bp),
                      (const float *)resolve(e, op.bias, bp), (uint16_t *)resolve(e, op.out, bp), op.M, op.K, op.Nn, lo, hi,
-                     op.w0 > 1 ? op.w0 : 1, op.w0 > 1 ? (void *)resolve(e, op.in1, bp) : nullptr, (int32_t)op.loader};
+                     op.w0 > 1 ? op.w0 : 1, op.w0 > 1 ? (void *)resolve(e, op.in1, bp) : nullptr, (int32_t)op.loader,
+                     nullptr, nullptr, 0, 0, 0.0f, 0.0f};
+        if (op.loader == 2) {
+            a.qscale = (const uint16_t *)resolve(e, op.scale, bp);
+            a.qbias = (const float *)resolve(e, op.table, bp);
+            a.qblock = (int32_t)op.gran;
+            a.qcols = op.Np;
+            memcpy(&a.qlo, &op.bias0, 4);
+            memcpy(&a.qhi, &op.scale0, 4);
+        }
         err = launchFcBf16(a, e->stream);
+        break;
+    }
+    case kKindAvgPoolBf16: {
+        AvgPoolBf16Args a{(const uint16_t *)resolve(e, op.in0, bp), (uint16_t *)resolve(e, op.out, bp), op.N, op.H * op.W, op.C,
+                          0.0f, 0.0f, 0.0f, 0.0f};
+        const uint32_t wbits = (uint32_t)op.w0 << 16;
+        memcpy(&a.weight, &wbits, 4);
+        memcpy(&a.bias, &op.bias0, 4);
+        memcpy(&a.lo, &op.output_min, 4);
+        memcpy(&a.hi, &op.output_max, 4);
+        err = launchAvgPoolBf16(a, e->stream);
+        break;
+    }
+    case kKindExpandWeights: {
+        ExpandWeightsArgs a{(const int8_t *)resolve(e, op.in0, bp), (const uint16_t *)resolve(e, op.scale, bp),
+                            (const float *)resolve(e, op.bias, bp), (uint16_t *)resolve(e, op.out, bp), op.K, op.Nn,
+                            (int32_t)op.gran, op.Np, 0.0f, 0.0f};
+        memcpy(&a.lo, &op.output_min, 4);
+        memcpy(&a.hi, &op.output_max, 4);
+        err = launchExpandWeights(a, e->stream);
         break;
     }
     default: return fail(THIP_INTERNAL, "op %u has unknown kind %u", i, op.kind);

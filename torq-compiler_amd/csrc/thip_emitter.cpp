@@ -44,7 +44,7 @@ struct Value {
     }
 };
 
-enum HlKind { kHlConv2d, kHlDepthwise, kHlFullyConnected, kHlMatmul, kHlMaxPool, kHlAvgPool, kHlAdd, kHlTranspose };
+enum HlKind { kHlConv2d, kHlDepthwise, kHlFullyConnected, kHlMatmul, kHlMaxPool, kHlAvgPool, kHlAdd, kHlTranspose, kHlExpandWeights };
 
 struct HlOp {
     HlKind kind;
@@ -57,6 +57,7 @@ struct HlOp {
         thip_hl_avg_pool2d_t ap;
         thip_hl_add_t add;
         thip_hl_transpose_t tr;
+        thip_hl_expand_weights_t ew;
     } u;
     std::string name;
 };
@@ -123,6 +124,11 @@ class Emitter {
         return cpad_[id] ? n / cdeclared_[id] * cpad_[id] : n;
     }
     void planChannelPadding();
+    // torq_hl.expand_weights ops that emit no kernel: every operand a constant and the result read once, as
+    // input2 of a bf16 matmul, which then takes the block-quantized weights itself (value id of the result ->
+    // the op).  THIP_NO_EXPAND_FOLD keeps every expand_weights a kernel of its own.
+    std::map<thip_value_t, const thip_hl_expand_weights_t *> foldedExpand_;
+    void planExpandFolding();
 
     thip_status_t checkValue(thip_value_t v, const char *what, const Value **out) const {
         if (v < 0 || (size_t)v >= prog_.values.size()) {
@@ -512,7 +518,40 @@ class Emitter {
     thip_status_t emitAvgPool(const thip_hl_avg_pool2d_t &c);
     thip_status_t emitAdd(const thip_hl_add_t &c);
     thip_status_t emitTransposeOp(const thip_hl_transpose_t &c);
+    thip_status_t emitExpandWeights(const thip_hl_expand_weights_t &c);
+    thip_status_t emitAvgPoolBf16(const thip_hl_avg_pool2d_t &c);
+    // Operands of an expand_weights checked and measured.
+    struct ExpandShape {
+        const Value *w, *scale, *bias, *init;
+        int64_t K, N, G, block, biasCols;
+    };
+    thip_status_t checkExpandWeights(const thip_hl_expand_weights_t &c, ExpandShape *out);
 };
+
+// Round-to-nearest-even bf16 bits of a float (NaN stays NaN).
+static uint16_t bf16FromFloat(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40);
+    return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1)) >> 16);
+}
+static float floatFromBf16(uint16_t b) {
+    const uint32_t u = (uint32_t)b << 16;
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+static float floatFromBits(int32_t bits) {
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+// One expanded weight, as the kernels compute it: the product of an 8-bit weight and a bf16 scale is exact in
+// fp32, so it does not matter whether the compiler fuses the multiply and the add.
+static uint16_t expandWeight(int8_t w, uint16_t scale, float bias, float lo, float hi) {
+    const float t0 = (float)w * floatFromBf16(scale) + bias;
+    return bf16FromFloat(t0 < lo ? lo : (t0 > hi ? hi : t0));
+}
 
 static thip_status_t windowGeometry(const char *what, int64_t H, int64_t W, int64_t KH, int64_t KW, const int64_t pad[4],
                                     const int64_t stride[2], int64_t *OH, int64_t *OW) {
@@ -1023,7 +1062,31 @@ thip_status_t Emitter::emitMatmulBf16(const thip_hl_matmul_t &c) {
     std::vector<DescRef> wrefs;
     std::vector<std::vector<uint16_t>> wconst;
     const int64_t wcount = Bb == 1 ? 1 : B;
-    if (b->kind == kValueConstant) {
+    // a folded torq_hl.expand_weights: few rows stream the int8 weights and expand them in registers (half the
+    // weight traffic), many rows read weights expanded here, once
+    const auto folded = foldedExpand_.find(c.input2);
+    ExpandShape ex{};
+    bool q8 = false;
+    if (folded != foldedExpand_.end()) {
+        if (thip_status_t s = checkExpandWeights(*folded->second, &ex)) return s;
+        const int64_t rows = Ba == 1 ? M : B * M;
+        const char *lim = getenv("THIP_EXPAND_INLINE_ROWS");
+        q8 = ex.block % 32 == 0 && rows <= (lim ? atoll(lim) : 64);
+        if (!q8) {
+            const float lo = floatFromBits(folded->second->output_min), hi = floatFromBits(folded->second->output_max);
+            const int8_t *wd = (const int8_t *)ex.w->data.data();
+            const uint16_t *sd = (const uint16_t *)ex.scale->data.data();
+            const float *bd = (const float *)ex.bias->data.data();
+            std::vector<uint16_t> t((size_t)(N * K));
+            for (int64_t k = 0; k < K; k++) {
+                const int64_t g = k / ex.block;
+                for (int64_t n = 0; n < N; n++) {
+                    t[(size_t)(n * K + k)] = expandWeight(wd[k * N + n], sd[g * N + n], bd[g * ex.biasCols + n], lo, hi);
+                }
+            }
+            wconst.push_back(std::move(t));
+        }
+    } else if (b->kind == kValueConstant) {
         const uint16_t *bd = (const uint16_t *)b->data.data();
         for (int64_t r = 0; r < wcount; r++) {
             std::vector<uint16_t> t((size_t)(N * K));
@@ -1058,7 +1121,29 @@ thip_status_t Emitter::emitMatmulBf16(const thip_hl_matmul_t &c) {
         op.in0.offset += (uint64_t)(Ba == 1 ? 0 : r * M * K) * 2;
         op.out = outRef;
         op.out.offset += (uint64_t)(r * M * N) * 2;
-        if (!wconst.empty()) {
+        if (q8) {
+            const int steps = (int)((K + 63) / 64);
+            const int64_t cols = roundUp(N, 32);
+            const int8_t *wd = (const int8_t *)ex.w->data.data();
+            std::vector<int8_t> packed((size_t)cols * (size_t)steps * 64, 0);
+            for (int64_t k = 0; k < K; k++) {
+                for (int64_t n = 0; n < N; n++) packed[fcBf16Q8FragmentOffset((int)n, (int)k, steps)] = wd[k * N + n];
+            }
+            std::vector<uint16_t> sc((size_t)(ex.G * cols), 0);
+            std::vector<float> bi((size_t)(ex.G * cols), 0.0f);
+            for (int64_t g = 0; g < ex.G; g++) {
+                memcpy(&sc[(size_t)(g * cols)], (const uint16_t *)ex.scale->data.data() + g * N, (size_t)N * 2);
+                memcpy(&bi[(size_t)(g * cols)], (const float *)ex.bias->data.data() + g * ex.biasCols, (size_t)N * 4);
+            }
+            op.loader = 2;
+            op.weights = newConst(packed);
+            op.scale = newConst(sc);
+            op.table = newConst(bi);
+            op.gran = (uint32_t)ex.block;
+            op.Np = (int32_t)cols;
+            op.bias0 = folded->second->output_min;
+            op.scale0 = folded->second->output_max;
+        } else if (!wconst.empty()) {
             packBf16Weights(&op, wconst[(size_t)(merge ? 0 : r)].data(), N, K);
         } else {
             op.weights = wrefs[(size_t)(merge ? 0 : r)];
@@ -1107,6 +1192,7 @@ thip_status_t Emitter::emitAvgPool(const thip_hl_avg_pool2d_t &c) {
     const char *what = "torq_hl.avg_pool2d";
     const Value *x, *w, *sb;
     if (thip_status_t s = checkValue(c.input, "torq_hl.avg_pool2d input", &x)) return s;
+    if (x->dtype == THIP_DTYPE_BF16) return emitAvgPoolBf16(c);
     if (x->rank != 4 || x->dtype != THIP_DTYPE_I8) return fail(THIP_INVALID_ARGUMENT, "%s: input must be an int8 N,H,W,C tensor", what);
     if (state_[c.input].nhwcOfNchw) return fail(THIP_INVALID_ARGUMENT, "%s: input %d is declared N,C,H,W; insert torq_hl.transpose [0,2,3,1]", what, (int)c.input);
     if (thip_status_t s = constantData(c.weights, "torq_hl.avg_pool2d weights", THIP_DTYPE_I8, &w)) return s;
@@ -1129,6 +1215,84 @@ thip_status_t Emitter::emitAvgPool(const thip_hl_avg_pool2d_t &c) {
     op.w0 = ((const int8_t *)w->data.data())[0];
     op.bias0 = ((const int32_t *)sb->data.data())[0];
     op.scale0 = ((const int32_t *)sb->data.data())[1];
+    ops_.push_back(op);
+    return THIP_OK;
+}
+
+thip_status_t Emitter::emitAvgPoolBf16(const thip_hl_avg_pool2d_t &c) {
+    // one bf16 weight and one float bias for every channel, no rescale
+    // (compiler/torq/Conversions/LinalgToTorqHL/PoolingPattern.cpp:448-457)
+    const char *what = "torq_hl.avg_pool2d (bf16)";
+    if (thip_status_t s = checkFloatAct(what, c.shift_factor, c.input_zp, 0, c.output_zp)) return s;
+    const Value *x, *w, *sb, *init;
+    if (thip_status_t s = checkValue(c.input, "torq_hl.avg_pool2d input", &x)) return s;
+    if (thip_status_t s = checkValue(c.init, "torq_hl.avg_pool2d init", &init)) return s;
+    if (x->rank != 4 || init->dtype != THIP_DTYPE_BF16) return fail(THIP_INVALID_ARGUMENT, "%s: input must be N,H,W,C and init bf16", what);
+    if (state_[c.input].nhwcOfNchw) return fail(THIP_INVALID_ARGUMENT, "%s: input %d is declared N,C,H,W; insert torq_hl.transpose [0,2,3,1]", what, (int)c.input);
+    if (thip_status_t s = constantData(c.weights, "torq_hl.avg_pool2d weights", THIP_DTYPE_BF16, &w)) return s;
+    if (thip_status_t s = constantData(c.scale_bias, "torq_hl.avg_pool2d scale_bias", THIP_DTYPE_F32, &sb)) return s;
+    if (w->numel() < 1 || sb->numel() < 1) return fail(THIP_INVALID_ARGUMENT, "%s: weights / scale_bias too short", what);
+    const int64_t N = x->shape[0], H = x->shape[1], W = x->shape[2], C = x->shape[3];
+    if (!fitsInt32(N * H * W * C)) return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
+    DescOp op;
+    memset(&op, 0, sizeof(op));
+    if (thip_status_t s = literalInput(c.input, "torq_hl.avg_pool2d input", &op.in0)) return s;
+    if (thip_status_t s = literalOutput(c.init, "torq_hl.avg_pool2d init", THIP_DTYPE_BF16, N * C, &op.out)) return s;
+    op.kind = kKindAvgPoolBf16;
+    op.out_dtype = THIP_DTYPE_BF16;
+    op.output_min = c.output_min;
+    op.output_max = c.output_max;
+    op.N = (int32_t)N; op.H = (int32_t)H; op.W = (int32_t)W; op.C = (int32_t)C;
+    op.w0 = ((const uint16_t *)w->data.data())[0];
+    memcpy(&op.bias0, sb->data.data(), 4);
+    ops_.push_back(op);
+    return THIP_OK;
+}
+
+thip_status_t Emitter::checkExpandWeights(const thip_hl_expand_weights_t &c, ExpandShape *out) {
+    const char *what = "torq_hl.expand_weights";
+    ExpandShape e;
+    if (thip_status_t s = checkValue(c.input, "torq_hl.expand_weights input", &e.w)) return s;
+    if (thip_status_t s = checkValue(c.scale, "torq_hl.expand_weights scale", &e.scale)) return s;
+    if (thip_status_t s = checkValue(c.scale_bias, "torq_hl.expand_weights scale_bias", &e.bias)) return s;
+    if (thip_status_t s = checkValue(c.init, "torq_hl.expand_weights init", &e.init)) return s;
+    if (e.w->dtype != THIP_DTYPE_I8) return fail(THIP_UNIMPLEMENTED, "%s: only int8 weights (4-bit and fp8 inputs are not on this path)", what);
+    if (e.scale->dtype != THIP_DTYPE_BF16 || e.bias->dtype != THIP_DTYPE_F32 || e.init->dtype != THIP_DTYPE_BF16) {
+        return fail(THIP_UNIMPLEMENTED, "%s: scale and init must be bf16 and scale_bias float32", what);
+    }
+    if (e.w->rank != 2) return fail(THIP_INVALID_ARGUMENT, "%s: input must be K,N", what);
+    e.K = e.w->shape[0];
+    e.N = e.w->shape[1];
+    e.block = c.block_size;
+    if (e.block <= 0 || e.K % e.block != 0) return fail(THIP_INVALID_ARGUMENT, "%s: block_size %lld does not divide K=%lld", what, (long long)e.block, (long long)e.K);
+    e.G = e.K / e.block;
+    const bool initOk = (e.init->rank == 2 && e.init->shape[0] == e.K && e.init->shape[1] == e.N) ||
+                        (e.init->rank == 3 && e.init->shape[0] == 1 && e.init->shape[1] == e.K && e.init->shape[2] == e.N);
+    if (!initOk) return fail(THIP_INVALID_ARGUMENT, "%s: init must be K,N or 1,K,N", what);
+    if (e.scale->numel() != e.G * e.N) return fail(THIP_INVALID_ARGUMENT, "%s: scale must hold K/block_size x N values", what);
+    if (e.bias->numel() % e.G != 0 || e.bias->numel() / e.G < e.N) return fail(THIP_INVALID_ARGUMENT, "%s: scale_bias must hold K/block_size rows of at least N values", what);
+    e.biasCols = e.bias->numel() / e.G;
+    if (!fitsInt32(e.K * e.N)) return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
+    *out = e;
+    return THIP_OK;
+}
+
+thip_status_t Emitter::emitExpandWeights(const thip_hl_expand_weights_t &c) {
+    ExpandShape e;
+    if (thip_status_t s = checkExpandWeights(c, &e)) return s;
+    if (foldedExpand_.count(c.init)) return THIP_OK;  // the matmul that reads it takes the quantized weights
+    DescOp op;
+    memset(&op, 0, sizeof(op));
+    op.kind = kKindExpandWeights;
+    op.out_dtype = THIP_DTYPE_BF16;
+    op.output_min = c.output_min;
+    op.output_max = c.output_max;
+    op.K = (int32_t)e.K; op.Nn = (int32_t)e.N; op.Np = (int32_t)e.biasCols; op.gran = (uint32_t)e.block;
+    op.M = 1; op.Kp = (int32_t)e.K;
+    if (thip_status_t s = literalInput(c.input, "torq_hl.expand_weights input", &op.in0)) return s;
+    if (thip_status_t s = literalInput(c.scale, "torq_hl.expand_weights scale", &op.scale)) return s;
+    if (thip_status_t s = literalInput(c.scale_bias, "torq_hl.expand_weights scale_bias", &op.bias)) return s;
+    if (thip_status_t s = literalOutput(c.init, "torq_hl.expand_weights init", THIP_DTYPE_BF16, e.K * e.N, &op.out)) return s;
     ops_.push_back(op);
     return THIP_OK;
 }
@@ -1344,6 +1508,7 @@ void Emitter::planChannelPadding() {
         case kHlMatmul: bar(op.u.mm.input1); bar(op.u.mm.input2); bar(op.u.mm.init); break;
         case kHlAvgPool: bar(op.u.ap.input); bar(op.u.ap.init); break;
         case kHlTranspose: bar(op.u.tr.input); bar(op.u.tr.init); break;
+        case kHlExpandWeights: bar(op.u.ew.input); bar(op.u.ew.init); break;
         }
     }
     // one verdict per group: every member an int8 rank-4 intermediate, all uses agreeing on C
@@ -1366,8 +1531,47 @@ void Emitter::planChannelPadding() {
     }
 }
 
+void Emitter::planExpandFolding() {
+    foldedExpand_.clear();
+    if (getenv("THIP_NO_EXPAND_FOLD")) return;
+    const size_t n = prog_.values.size();
+    std::vector<int> reads(n, 0), asMatmulRhs(n, 0);
+    auto read = [&](thip_value_t v) {
+        if (v >= 0 && (size_t)v < n) reads[(size_t)v]++;
+    };
+    for (const HlOp &op : prog_.ops) {
+        switch (op.kind) {
+        case kHlConv2d: read(op.u.conv.input); break;
+        case kHlDepthwise: read(op.u.dw.input); break;
+        case kHlFullyConnected: read(op.u.fc.input); break;
+        case kHlMatmul:
+            read(op.u.mm.input1);
+            read(op.u.mm.input2);
+            if (op.u.mm.input2 >= 0 && (size_t)op.u.mm.input2 < n && op.u.mm.input1 >= 0 && (size_t)op.u.mm.input1 < n &&
+                prog_.values[(size_t)op.u.mm.input1].dtype == THIP_DTYPE_BF16) {
+                asMatmulRhs[(size_t)op.u.mm.input2]++;
+            }
+            break;
+        case kHlMaxPool: read(op.u.mp.input); break;
+        case kHlAvgPool: read(op.u.ap.input); break;
+        case kHlAdd: read(op.u.add.input1); read(op.u.add.input2); break;
+        case kHlTranspose: read(op.u.tr.input); break;
+        case kHlExpandWeights: read(op.u.ew.input); read(op.u.ew.scale); read(op.u.ew.scale_bias); break;
+        }
+    }
+    auto constant = [&](thip_value_t v) { return v >= 0 && (size_t)v < n && prog_.values[(size_t)v].kind == kValueConstant; };
+    for (const HlOp &op : prog_.ops) {
+        if (op.kind != kHlExpandWeights) continue;
+        const thip_hl_expand_weights_t &c = op.u.ew;
+        if (c.init < 0 || (size_t)c.init >= n || prog_.values[(size_t)c.init].kind != kValueTensor) continue;
+        if (!constant(c.input) || !constant(c.scale) || !constant(c.scale_bias)) continue;
+        if (reads[(size_t)c.init] == 1 && asMatmulRhs[(size_t)c.init] == 1) foldedExpand_[c.init] = &c;
+    }
+}
+
 thip_status_t Emitter::run(void **outBlob, size_t *outSize) {
     planChannelPadding();
+    planExpandFolding();
     for (const HlOp &op : prog_.ops) {
         thip_status_t s = THIP_OK;
         switch (op.kind) {
@@ -1379,6 +1583,7 @@ thip_status_t Emitter::run(void **outBlob, size_t *outSize) {
         case kHlAvgPool: s = emitAvgPool(op.u.ap); break;
         case kHlAdd: s = emitAdd(op.u.add); break;
         case kHlTranspose: s = emitTransposeOp(op.u.tr); break;
+        case kHlExpandWeights: s = emitExpandWeights(op.u.ew); break;
         }
         if (s != THIP_OK) return s;
     }
@@ -1511,6 +1716,7 @@ THIP_DEFINE_HL(thip_hl_matmul, thip_hl_matmul_t, kHlMatmul, mm)
 THIP_DEFINE_HL(thip_hl_maxpool2d, thip_hl_maxpool2d_t, kHlMaxPool, mp)
 THIP_DEFINE_HL(thip_hl_avg_pool2d, thip_hl_avg_pool2d_t, kHlAvgPool, ap)
 THIP_DEFINE_HL(thip_hl_transpose, thip_hl_transpose_t, kHlTranspose, tr)
+THIP_DEFINE_HL(thip_hl_expand_weights, thip_hl_expand_weights_t, kHlExpandWeights, ew)
 
 thip_status_t thip_hl_add(thip_program_t *program, const thip_hl_add_t *op) {
     if (!program || !op) return fail(THIP_INVALID_ARGUMENT, "thip_hl_add: null argument");

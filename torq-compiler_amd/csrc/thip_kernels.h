@@ -109,8 +109,22 @@ struct FcBf16Args {
     // weights in fragment order: for column block nb (32 columns), k-step s (64 elements) and piece c (0..3),
     // 64 lanes x 16 bytes, lane l = column l & 31, elements 32 (l >> 5) + 8 c .. + 7 of the step; zero padded
     // to whole blocks and steps.  One wave load is then 1 KiB of consecutive memory.
+    // 2: block-quantized int8 weights expanded while they are loaded (torq_hl.expand_weights folded into the
+    // matmul that consumes it): w then holds int8 in the same order, 64 lanes x 16 bytes per half h2 (0..1) of
+    // a step, byte e of lane l = element 32 (l >> 5) + 16 h2 + e; weight (n, k) stands for
+    // bf16(clamp(w * qscale[k / qblock][n] + qbias[k / qblock][n], qlo, qhi)).  qblock % 32 == 0; the two
+    // tables are qcols (a multiple of 32, >= N) wide.
     int32_t w_fragments;
+    const uint16_t *qscale;
+    const float *qbias;
+    int32_t qblock, qcols;
+    float qlo, qhi;
 };
+// Byte offset of int8 weight (n, k) in the block-quantized fragment order.
+inline size_t fcBf16Q8FragmentOffset(int n, int k, int steps) {
+    const int nb = n >> 5, r = n & 31, s = k >> 6, kk = k & 63, h = kk >> 5, h2 = (kk & 31) >> 4, e = kk & 15;
+    return ((((size_t)nb * steps + s) * 2 + h2) * 64 + (size_t)(h * 32 + r)) * 16 + (size_t)e;
+}
 // Byte offset of element (n, k) in the fragment order, for K padded to `steps` steps of 64.
 inline size_t fcBf16FragmentOffset(int n, int k, int steps) {
     const int nb = n >> 5, r = n & 31, s = k >> 6, kk = k & 63, h = kk >> 5, c = (kk & 31) >> 3, e = kk & 7;
@@ -132,6 +146,27 @@ inline int fcBf16PreferredSplit(int M, int N, int K) {
     return split < 2 ? 1 : (int)split;
 }
 hipError_t launchFcBf16(const FcBf16Args &a, hipStream_t stream);
+
+// bf16 global average pool: out[n][c] = bf16(clamp(sum_u in[n][u][c] * weight + bias)), summed over the frame
+// in order, in fp32.
+struct AvgPoolBf16Args {
+    const uint16_t *in;  // [N][HW][C]
+    uint16_t *out;       // [N][C]
+    int32_t N, HW, C;
+    float weight, bias, lo, hi;
+};
+hipError_t launchAvgPoolBf16(const AvgPoolBf16Args &a, hipStream_t stream);
+
+// torq_hl.expand_weights: out[k][n] = bf16(clamp(w[k][n] * scale[k / block][n] + bias[k / block][n])).
+struct ExpandWeightsArgs {
+    const int8_t *w;        // [K][N]
+    const uint16_t *scale;  // [K / block][N] bf16
+    const float *bias;      // [K / block][bias_cols]
+    uint16_t *out;          // [K][N]
+    int32_t K, N, block, bias_cols;
+    float lo, hi;
+};
+hipError_t launchExpandWeights(const ExpandWeightsArgs &a, hipStream_t stream);
 
 struct DepthwiseArgs {
     const int8_t *in;     // NHWC

@@ -2057,8 +2057,26 @@ hipError_t launchTranspose(const TransposeArgs &a, hipStream_t stream) {
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-template <int NWAVES>  // waves of a block = ways K is split
-__global__ __launch_bounds__(NWAVES * 64) void fc_bf16(FcBf16Args p) {
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+
+// Four int8 weights of a dword to bf16 pairs: w * scale + bias in fp32 (the product of an 8-bit weight and a
+// bf16 scale is exact, so the fused multiply-add rounds once, like a multiply followed by an add), optional
+// clamp, round to nearest even.
+template <bool CLAMP>
+__device__ __forceinline__ void expandQ8(int d, float sc, float bi, float lo, float hi, int *o0, int *o1) {
+    float f[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        f[j] = __builtin_fmaf((float)(int8_t)(d >> (8 * j)), sc, bi);
+        if (CLAMP) f[j] = f[j] < lo ? lo : (f[j] > hi ? hi : f[j]);
+    }
+    *o0 = __builtin_bit_cast(int, __builtin_convertvector((v2f){f[0], f[1]}, v2bf));
+    *o1 = __builtin_bit_cast(int, __builtin_convertvector((v2f){f[2], f[3]}, v2bf));
+}
+
+template <int NWAVES, int Q8>  // waves of a block = ways K is split; Q8: 0 bf16 weights, 1 int8 expanded, 2 with clamp
+__global__ __launch_bounds__(NWAVES * 64) void fc_bf16(FcBf16Args p, FastDiv qblk) {
     __shared__ float partial[NWAVES - 1][16][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, h = lane >> 5;
@@ -2078,19 +2096,35 @@ __global__ __launch_bounds__(NWAVES * 64) void fc_bf16(FcBf16Args p) {
     // UNR steps of loads are issued before their MFMAs: one memory round trip per UNR * 64 elements of K
     constexpr int UNR = NWAVES > 4 ? 2 : 4;
     for (int s0 = sBeg; s0 < sEnd; s0 += UNR) {
-        v4i wv[UNR][4], xv[UNR][4];
+        v4i wv[Q8 ? 1 : UNR][4], xv[UNR][4];
+        v4i wq[Q8 ? UNR : 1][2];
+        float qs[Q8 ? UNR : 1], qb[Q8 ? UNR : 1];
 #pragma unroll
         for (int u = 0; u < UNR; u++) {
             const int k = (s0 + u) * 64 + 32 * h;
+            if (Q8) {
+                // the lane's 32 weights of this step lie in one block: one scale, one bias
+                const bool live = s0 + u < sEnd;
+                const size_t g = fastDiv((uint32_t)(live && k < p.K ? k : 0), qblk);  // beyond K the input rows are zero
+                qs[u] = __uint_as_float((uint32_t)p.qscale[g * p.qcols + n0 + r] << 16);
+                qb[u] = p.qbias[g * p.qcols + n0 + r];
+#pragma unroll
+                for (int h2 = 0; h2 < 2; h2++) {
+                    const int8_t *frag = (const int8_t *)p.w + ((((size_t)blockIdx.x * steps + (s0 + u)) * 2 + h2) * 64 + lane) * 16;
+                    wq[u][h2] = live ? *(const v4i *)frag : v4i{0, 0, 0, 0};
+                }
+                if (!live) qs[u] = qb[u] = 0.0f;  // a step past the end multiplies zeros
+            }
 #pragma unroll
             for (int c = 0; c < 4; c++) {
                 const bool in = s0 + u < sEnd && k + 8 * c < p.K;  // K % 8 == 0: a piece is inside K or outside
-                if (p.w_fragments) {
+                if (Q8) {
+                } else if (p.w_fragments) {
                     // whole (zero padded) steps: every lane of the wave loads, 1 KiB in a row
                     const int8_t *frag = (const int8_t *)p.w + ((((size_t)blockIdx.x * steps + (s0 + u)) * 4 + c) * 64 + lane) * 16;
-                    wv[u][c] = s0 + u < sEnd ? *(const v4i *)frag : v4i{0, 0, 0, 0};
+                    wv[Q8 ? 0 : u][c] = s0 + u < sEnd ? *(const v4i *)frag : v4i{0, 0, 0, 0};
                 } else {
-                    wv[u][c] = in ? *(const v4i *)(wrow + k + 8 * c) : v4i{0, 0, 0, 0};
+                    wv[Q8 ? 0 : u][c] = in ? *(const v4i *)(wrow + k + 8 * c) : v4i{0, 0, 0, 0};
                 }
                 xv[u][c] = in ? *(const v4i *)(xrow + k + 8 * c) : v4i{0, 0, 0, 0};
             }
@@ -2099,7 +2133,17 @@ __global__ __launch_bounds__(NWAVES * 64) void fc_bf16(FcBf16Args p) {
         for (int u = 0; u < UNR; u++) {
 #pragma unroll
             for (int c = 0; c < 4; c++) {
-                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, wv[u][c]), __builtin_bit_cast(v8bf, xv[u][c]), acc, 0, 0, 0);
+                v4i wpiece;
+                if (Q8) {
+                    // piece c = bytes 8 (c & 1) .. + 7 of half c >> 1; the k rows beyond K are zero in the input
+                    int o[4];
+                    expandQ8<Q8 == 2>(wq[u][c >> 1][2 * (c & 1)], qs[u], qb[u], p.qlo, p.qhi, &o[0], &o[1]);
+                    expandQ8<Q8 == 2>(wq[u][c >> 1][2 * (c & 1) + 1], qs[u], qb[u], p.qlo, p.qhi, &o[2], &o[3]);
+                    wpiece = v4i{o[0], o[1], o[2], o[3]};
+                } else {
+                    wpiece = wv[u][c];
+                }
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, wpiece), __builtin_bit_cast(v8bf, xv[u][c]), acc, 0, 0, 0);
             }
         }
     }
@@ -2167,7 +2211,85 @@ hipError_t launchFcBf16(const FcBf16Args &a, hipStream_t stream) {
     if (a.ksplit < 1 || a.ksplit > 64 || (a.ksplit > 1 && (!a.workspace || ((uintptr_t)a.workspace & 255)))) return hipErrorInvalidValue;
     const dim3 grid((unsigned)((a.N + 31) / 32), (unsigned)((a.M + 31) / 32), (unsigned)a.ksplit);
     if (grid.y > 65535) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(fc_bf16<4>, grid, dim3(256), 0, stream, a);
+    if (a.w_fragments == 2) {
+        if (!a.qscale || !a.qbias || a.qblock < 32 || a.qblock % 32 != 0 || a.qcols < (a.N + 31) / 32 * 32 || a.qcols % 32 != 0) return hipErrorInvalidValue;
+        if ((((uintptr_t)a.qscale) & 1) || (((uintptr_t)a.qbias) & 3)) return hipErrorInvalidValue;
+        const FastDiv blk = makeFastDiv((uint32_t)a.qblock);
+        const bool clamp = !(a.qlo == -INFINITY && a.qhi == INFINITY);
+        if (clamp) hipLaunchKernelGGL((fc_bf16<4, 2>), grid, dim3(256), 0, stream, a, blk);
+        else hipLaunchKernelGGL((fc_bf16<4, 1>), grid, dim3(256), 0, stream, a, blk);
+        return hipGetLastError();
+    }
+    hipLaunchKernelGGL((fc_bf16<4, 0>), grid, dim3(256), 0, stream, a, makeFastDiv(1));
+    return hipGetLastError();
+}
+
+// bf16 global average pool: a thread owns VEC neighbouring channels of one image and walks the frame in
+// order (the sums then equal a sequential fp32 accumulation bit for bit); a wave's loads cover 64 * VEC
+// neighbouring channels of one pixel.
+template <int VEC>
+__global__ __launch_bounds__(256) void avgpool_bf16(AvgPoolBf16Args p) {
+    const int cgroups = p.C / VEC;
+    const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (t >= (long long)p.N * cgroups) return;
+    const int n = (int)(t / cgroups), c0 = (int)(t % cgroups) * VEC;
+    const uint16_t *src = p.in + (size_t)n * p.HW * p.C + c0;
+    float acc[VEC];
+#pragma unroll
+    for (int v = 0; v < VEC; v++) acc[v] = 0.0f;
+#pragma unroll 8
+    for (int u = 0; u < p.HW; u++) {
+        uint16_t x[VEC];
+        if (VEC == 2) {
+            const uint32_t d = *(const uint32_t *)(src + (size_t)u * p.C);
+            x[0] = (uint16_t)d;
+            x[VEC - 1] = (uint16_t)(d >> 16);
+        } else {
+            x[0] = src[(size_t)u * p.C];
+        }
+#pragma unroll
+        for (int v = 0; v < VEC; v++) acc[v] = __fadd_rn(acc[v], __fmul_rn(__uint_as_float((uint32_t)x[v] << 16), p.weight));
+    }
+#pragma unroll
+    for (int v = 0; v < VEC; v++) {
+        const float t0 = __fadd_rn(acc[v], p.bias);
+        p.out[(size_t)n * p.C + c0 + v] = bf16Bits(t0 < p.lo ? p.lo : (t0 > p.hi ? p.hi : t0));
+    }
+}
+
+hipError_t launchAvgPoolBf16(const AvgPoolBf16Args &a, hipStream_t stream) {
+    if (a.N <= 0 || a.HW <= 0 || a.C <= 0 || !a.in || !a.out) return hipErrorInvalidValue;
+    const bool pairs = a.C % 2 == 0 && (((uintptr_t)a.in) & 3) == 0;
+    const long long threads = (long long)a.N * (pairs ? a.C / 2 : a.C);
+    const dim3 grid((unsigned)((threads + 255) / 256));
+    if (pairs) hipLaunchKernelGGL(avgpool_bf16<2>, grid, dim3(256), 0, stream, a);
+    else hipLaunchKernelGGL(avgpool_bf16<1>, grid, dim3(256), 0, stream, a);
+    return hipGetLastError();
+}
+
+// torq_hl.expand_weights as an op of its own (the result is a binding, or has several readers): a thread
+// expands four neighbouring columns of one row.
+__global__ __launch_bounds__(256) void expand_weights_bf16(ExpandWeightsArgs p, FastDiv blk, int quads) {
+    const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (t >= (long long)p.K * quads) return;
+    const int k = (int)(t / quads), n0 = (int)(t % quads) * 4;
+    const size_t g = fastDiv((uint32_t)k, blk);
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const int n = n0 + e;
+        if (n >= p.N) break;
+        const float sc = __uint_as_float((uint32_t)p.scale[g * p.N + n] << 16);
+        const float t0 = __fadd_rn(__fmul_rn((float)p.w[(size_t)k * p.N + n], sc), p.bias[g * p.bias_cols + n]);
+        p.out[(size_t)k * p.N + n] = bf16Bits(t0 < p.lo ? p.lo : (t0 > p.hi ? p.hi : t0));
+    }
+}
+
+hipError_t launchExpandWeights(const ExpandWeightsArgs &a, hipStream_t stream) {
+    if (!a.w || !a.scale || !a.bias || !a.out || a.K <= 0 || a.N <= 0 || a.block <= 0 || a.K % a.block != 0 || a.bias_cols < a.N) return hipErrorInvalidValue;
+    const int quads = (a.N + 3) / 4;
+    const long long threads = (long long)a.K * quads;
+    if (threads >= (1LL << 39)) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(expand_weights_bf16, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, a, makeFastDiv((uint32_t)a.block), quads);
     return hipGetLastError();
 }
 

@@ -40,7 +40,7 @@ EXPORTED_SYMBOLS = [
     "thip_status_message", "thip_version", "thip_descriptor_version",
     "thip_program_create", "thip_program_destroy", "thip_program_binding", "thip_program_constant",
     "thip_program_tensor", "thip_hl_conv2d", "thip_hl_depthwise_conv2d", "thip_hl_fully_connected",
-    "thip_hl_matmul", "thip_hl_maxpool2d", "thip_hl_avg_pool2d", "thip_hl_add", "thip_hl_transpose",
+    "thip_hl_matmul", "thip_hl_maxpool2d", "thip_hl_avg_pool2d", "thip_hl_add", "thip_hl_transpose", "thip_hl_expand_weights",
     "thip_program_serialize", "thip_blob_free",
     "thip_device_create", "thip_device_destroy", "thip_device_name", "thip_device_alloc",
     "thip_device_free", "thip_device_h2d", "thip_device_d2h", "thip_device_synchronize",
@@ -120,6 +120,14 @@ class HlAvgPool2d(ctypes.Structure):
     ]
 
 
+class HlExpandWeights(ctypes.Structure):
+    _fields_ = [
+        ("init", ctypes.c_int32), ("scale_bias", ctypes.c_int32), ("output_min", ctypes.c_int32),
+        ("output_max", ctypes.c_int32), ("scale", ctypes.c_int32), ("input", ctypes.c_int32),
+        ("block_size", ctypes.c_int32),
+    ]
+
+
 class HlAdd(ctypes.Structure):
     _fields_ = [
         ("init", ctypes.c_int32), ("name", ctypes.c_char_p), ("input_zp", ctypes.c_int32),
@@ -167,7 +175,8 @@ def lib():
     for name, st in [("thip_hl_conv2d", HlConv2d), ("thip_hl_depthwise_conv2d", HlDepthwiseConv2d),
                      ("thip_hl_fully_connected", HlFullyConnected), ("thip_hl_matmul", HlMatmul),
                      ("thip_hl_maxpool2d", HlMaxPool2d), ("thip_hl_avg_pool2d", HlAvgPool2d),
-                     ("thip_hl_add", HlAdd), ("thip_hl_transpose", HlTranspose)]:
+                     ("thip_hl_add", HlAdd), ("thip_hl_transpose", HlTranspose),
+                     ("thip_hl_expand_weights", HlExpandWeights)]:
         getattr(L, name).argtypes = [vp, P(st)]
     L.thip_program_serialize.argtypes = [vp, P(vp), P(sz)]
     L.thip_blob_free.argtypes = [vp]

@@ -195,7 +195,7 @@ class Program:
         weights = self._as_value(weights)
         scale_bias = self._as_value(scale_bias)
         N, _, _, C = input.shape
-        init = self._init_or_new(init, (N, 1, 1, C), np.int8)
+        init = self._init_or_new(init, (N, 1, 1, C), np.uint16 if input.dtype == np.uint16 else np.int8)
         op = rt.HlAvgPool2d(init.index, input_zp, output_zp, output_min, output_max, shift_factor,
                             weights.index, scale_bias.index, input.index)
         rt.check(rt.lib().thip_hl_avg_pool2d(self._h, ctypes.byref(op)))
@@ -211,6 +211,18 @@ class Program:
                       shift_factor, weights.index, scale_bias.index, input1.index, input2.index,
                       int(segment_output), int(rhs_is_scalar))
         rt.check(rt.lib().thip_hl_add(self._h, ctypes.byref(op)))
+        return init
+
+    def expand_weights(self, input, scale, scale_bias, *, block_size, output_min, output_max, init=None):
+        """torq_hl.expand_weights: int8 weights K,N times per-block bf16 scales plus float biases -> bf16 1,K,N."""
+        input = self._as_value(input)
+        scale = self._as_value(scale)
+        scale_bias = self._as_value(scale_bias)
+        K, N = input.shape
+        init = self._init_or_new(init, (1, K, N), np.uint16)
+        op = rt.HlExpandWeights(init.index, scale_bias.index, output_min, output_max, scale.index, input.index,
+                                block_size)
+        rt.check(rt.lib().thip_hl_expand_weights(self._h, ctypes.byref(op)))
         return init
 
     def transpose(self, input, perm, init=None):

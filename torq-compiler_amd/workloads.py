@@ -194,6 +194,58 @@ def conv2d_bf16_workload(N=1, H=14, W=14, C=16, O=24, KH=3, KW=3, stride=(1, 1),
     return Workload(name, p, [x], [(oshape, np.uint16)], 2 * macs, x.nbytes + wts.nbytes + bias.nbytes + 2 * int(np.prod(oshape)), attrs)
 
 
+def avg_pool2d_bf16_workload(N=2, H=7, W=7, C=1280, weight=None, clamp=None, seed=1014):
+    """bf16 global average pool: one bf16 weight (1 / (H W) by default, the folded divide), bias 0."""
+    rng = np.random.default_rng(seed)
+    x = to_bf16(rng.standard_normal((N, H, W, C)) + 0.25)
+    wt = to_bf16(np.array([1.0 / (H * W) if weight is None else weight]))
+    bias = np.zeros(1, dtype=np.float32)
+    lo, hi = NO_CLAMP if clamp is None else (float_bits(clamp[0]), float_bits(clamp[1]))
+    p = Program()
+    inp = p.binding(0, x.shape, np.uint16)
+    out = p.binding(1, (N, 1, 1, C), np.uint16)
+    p.avg_pool2d(inp, wt, bias, init=out, input_zp=0, output_zp=0, output_min=lo, output_max=hi, shift_factor=0)
+    attrs = dict(weights=wt, bias=bias, output_min=lo, output_max=hi)
+    return Workload("avgpoolbf16_%dx%dx%dx%d" % (N, H, W, C), p, [x], [((N, 1, 1, C), np.uint16)], 2 * x.size,
+                    x.nbytes + 2 * N * C, attrs)
+
+
+def expand_weights_workload(M=4, K=256, N=96, block=32, fold=True, clamp=None, expand_clamp=None, bias_pad=0, seed=1015):
+    """Block-quantized int8 weights -> torq_hl.expand_weights -> bf16 matmul (fold=True: the expansion feeds only the
+    matmul; False: it is also an output of the program, so it must run as an op of its own)."""
+    rng = np.random.default_rng(seed)
+    G = K // block
+    x = to_bf16(rng.standard_normal((M, K)))
+    wq = rng.integers(-128, 128, size=(K, N), dtype=np.int8)
+    scale = to_bf16(rng.uniform(0.5, 1.5, size=(G, N)) / (64.0 * np.sqrt(K)))
+    zp = rng.integers(-8, 9, size=(G, N))
+    cols = N + bias_pad
+    qbias = np.zeros((G, cols), dtype=np.float32)
+    qbias[:, :N] = (-zp).astype(np.float32) * from_bf16_np(scale)
+    mm_bias = np.zeros(1, dtype=np.float32)
+    lo, hi = NO_CLAMP if clamp is None else (float_bits(clamp[0]), float_bits(clamp[1]))
+    elo, ehi = NO_CLAMP if expand_clamp is None else (float_bits(expand_clamp[0]), float_bits(expand_clamp[1]))
+    p = Program()
+    inp = p.binding(0, x.shape, np.uint16)
+    out = p.binding(1, (M, N), np.uint16)
+    outputs = [((M, N), np.uint16)]
+    if fold:
+        w16 = p.expand_weights(wq, scale, qbias, block_size=block, output_min=elo, output_max=ehi)
+    else:
+        wout = p.binding(2, (1, K, N), np.uint16)
+        w16 = p.expand_weights(wq, scale, qbias, block_size=block, output_min=elo, output_max=ehi, init=wout)
+        outputs.append(((1, K, N), np.uint16))
+    p.matmul(inp, w16, mm_bias, init=out, output_zp=0, output_min=lo, output_max=hi, shift=0)
+    attrs = dict(weights=wq, scale=scale, qbias=qbias, block=block, bias=mm_bias, output_min=lo, output_max=hi,
+                 expand_min=elo, expand_max=ehi, fold=fold)
+    return Workload("expandmm_%dx%dx%d_b%d%s" % (M, K, N, block, "" if fold else "_out"), p, [x], outputs, 2 * M * K * N,
+                    x.nbytes + wq.nbytes + scale.nbytes + qbias.nbytes + 2 * M * N, attrs)
+
+
+def from_bf16_np(bits):
+    return (np.asarray(bits, dtype=np.uint16).astype(np.uint32) << 16).view(np.float32)
+
+
 def add_bf16_workload(shape=(1, 32, 1152), w0=1.0, w1=1.0, bias=0.0, clamp=None, seed=1012):
     """bf16 add (a residual connection of a decoder layer): in1 * w0 + in2 * w1 + bias in fp32."""
     rng = np.random.default_rng(seed)
