@@ -56,6 +56,11 @@ def workload_table(pkg):
         "fcbf16_1x1152x6912": (lambda: w.fully_connected_bf16_workload(1, 1152, 6912), "hbm"),
         "fcbf16_32x1152x6912": (lambda: w.fully_connected_bf16_workload(32, 1152, 6912), "hbm"),
         "fcbf16_32x6912x1152": (lambda: w.fully_connected_bf16_workload(32, 6912, 1152), "hbm"),
+        # a quarter of the vocabulary projection (1152 -> 262144) with bf16 weights, and with block-quantized int8
+        # weights (torq_hl.expand_weights folded into the matmul: the int8 bytes are what is streamed)
+        "fcbf16_1x1152x65536": (lambda: w.fully_connected_bf16_workload(1, 1152, 65536), "hbm"),
+        "expandmm_1x1152x65536": (lambda: w.expand_weights_workload(M=1, K=1152, N=65536, block=128), "hbm"),
+        "expandmm_32x1152x65536": (lambda: w.expand_weights_workload(M=32, K=1152, N=65536, block=128), "hbm"),
     }
 
 
@@ -90,16 +95,16 @@ class Loaded:
             self.dev.free(p)
 
 
-# HBM bytes per launch of each workload's kernel, from rocprofv3 counters: FETCH_SIZE * 1.9993 + WRITE_SIZE * 1.0
+# HBM bytes per launch of each workload's kernel, from rocprofv3 counters: FETCH_SIZE * 1.9995 + WRITE_SIZE * 1.0
 # (KiB per dispatch; the factors are what the same counters read for a plain 256 MiB copy, --copy-calibration).
 MEASURED_TRAFFIC = {
-    "fc_4096x4096x4096": (49396.2 * 1.9993 + 16569.0) * 1024,
-    "fc_512x4096x4096": (16452.6 * 1.9993 + 2048.0) * 1024,
-    "fc_16x2048x8192": (8553.6 * 1.9993 + 512.0) * 1024,
-    "conv_112x112x32_o64_3x3": (359.4 * 1.9993 + 784.0) * 1024,
-    "depthwise_b64": (17042.9 * 1.9993 + 7105.0) * 1024,
-    "avgpool_b64": (1991.6 * 1.9993 + 80.0) * 1024,
-    "add_b64": (4727.1 * 1.9993 + 4704.0) * 1024,
+    "fc_4096x4096x4096": (49386.7 * 1.9995 + 16565.3) * 1024,
+    "fc_512x4096x4096": (16445.6 * 1.9995 + 2048.0) * 1024,
+    "fc_16x2048x8192": (8408.1 * 1.9995 + 256.0) * 1024,
+    "conv_112x112x32_o64_3x3": (350.4 * 1.9995 + 784.0) * 1024,
+    "depthwise_b64": (17051.3 * 1.9995 + 7105.0) * 1024,
+    "avgpool_b64": (1991.5 * 1.9995 + 80.0) * 1024,
+    "add_b64": (4727.1 * 1.9995 + 4704.0) * 1024,
 }
 
 
@@ -133,13 +138,19 @@ def verify_sample(loaded):
         rows = np.unique(np.r_[0:16, M // 2:M // 2 + 16, M - 16:M])
         want = orc.fully_connected(wl.inputs[0][rows], wts, sb, **a)
         return bool(np.array_equal(got[rows], want))
-    if wl.name.startswith("fcbf16"):
+    if wl.name.startswith("fcbf16") or wl.name.startswith("expandmm"):
         # tolerance row: one bf16 ULP, or the fp32 reordering error where the sum cancels
         from helpers import assert_bf16_close
         f = lambda bits: np.abs(orc.from_bf16(bits).astype(np.float64))
-        mag = f(wl.inputs[0]) @ f(wl.attrs["weights"]).T + np.abs(wl.attrs["bias"])
+        if wl.name.startswith("expandmm"):
+            a = wl.attrs
+            w16 = orc.expand_weights(a["weights"], a["scale"], a["qbias"], block_size=a["block"], output_min=a["expand_min"], output_max=a["expand_max"])
+            mag = f(wl.inputs[0]) @ f(w16)
+            got = got.reshape(mag.shape)
+        else:
+            mag = f(wl.inputs[0]) @ f(wl.attrs["weights"]).T + np.abs(wl.attrs["bias"])
         try:
-            assert_bf16_close(got, oracle_eval(wl)[0], wl.name, magnitude=mag)
+            assert_bf16_close(got, oracle_eval(wl)[0].reshape(got.shape), wl.name, magnitude=mag)
         except AssertionError:
             return False
         return True
@@ -269,7 +280,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16" if args.workload.startswith("fcbf16") else "int8",
+        "dtype": "bf16" if args.workload.startswith(("fcbf16", "expandmm")) else "int8",
         "data": "synthetic",
         "config": {"workload": args.workload, "kernels": kernels, "parity_checked": ok,
                    "algorithmic_ops": wl.ops, "algorithmic_bytes": wl.bytes},
