@@ -52,6 +52,9 @@ def workload_table(pkg):
         "avgpool_b1": (lambda: w.avgpool_workload(N=1), "hbm"),
         "add_b64": (lambda: w.add_workload(N=64), "hbm"),
         "add_b1": (lambda: w.add_workload(N=1), "hbm"),
+        # integer elementwise ops next to the convolution path, at the shape of the add row
+        "rescale_b64": (lambda: w.fma_workload((64, 56, 56, 24)), "hbm"),
+        "mul_b64": (lambda: w.mul_workload((64, 56, 56, 24)), "hbm"),
         # bf16 linears of a decoder layer (hidden 1152, MLP 6912) at 1 and 32 tokens: weight streaming
         "fcbf16_1x1152x6912": (lambda: w.fully_connected_bf16_workload(1, 1152, 6912), "hbm"),
         "fcbf16_32x1152x6912": (lambda: w.fully_connected_bf16_workload(32, 1152, 6912), "hbm"),

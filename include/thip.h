@@ -266,6 +266,53 @@ typedef struct thip_hl_expand_weights_t {
     int32_t block_size;
 } thip_hl_expand_weights_t;
 
+/* torq_hl.fma -- TorqHLOps.td:926-941: the stand-alone rescale
+ * (compiler/torq/Conversions/LinalgToTorqHL/Patterns.cpp:1896-1946: weight 1, bias = -input_zp, scale = the
+ * multiplier).  input and init int8 / int16 / int32 of the same element count; weights ONE int8 (or int16) value;
+ * scale_bias int32[2] = [bias, scale]: init = R1(input * weights[0]). */
+typedef struct thip_hl_fma_t {
+    thip_value_t init;
+    int32_t output_zp;
+    int32_t output_min;
+    int32_t output_max;
+    int32_t shift_factor;
+    thip_value_t weights;
+    thip_value_t scale_bias;
+    thip_value_t input;
+} thip_hl_fma_t;
+
+/* torq_hl.mul -- TorqHLOps.td:101-117.  input1 / input2 int8 or int16 (the same type), of init's element count or of
+ * one element (broadcast); scale_bias int32[2] = [bias, scale]: init = R1(input1 * input2) with shift `shift`. */
+typedef struct thip_hl_mul_t {
+    thip_value_t init;
+    int32_t output_zp;
+    int32_t output_min;
+    int32_t output_max;
+    thip_value_t scale_bias;
+    int32_t shift;
+    thip_value_t input1;
+    thip_value_t input2;
+} thip_hl_mul_t;
+
+/* torq_hl.act -- TorqHLOps.td:291-309, integer tensors.  name: "clamp" (clip to [min_int, max_int]), "abs",
+ * "negate" (both clipped to the range of init's element type; the zero-point attributes are carried but, as in
+ * compiler/torq/Conversions/TorqHLToTorqHW/ActPattern.cpp:60-140, not used), "i2i" (conversion by truncation).
+ * weights (the unsigned-cast multiplier) must be THIP_NO_VALUE; the float names (ceil, floor, i2f, f2i, f2f, clz)
+ * are not on this path. */
+#define THIP_NO_VALUE (-1)
+typedef struct thip_hl_act_t {
+    thip_value_t init;
+    const char *name;
+    int32_t input_zp;
+    int32_t output_zp;
+    int64_t min_int;
+    int64_t max_int;
+    float min_fp;
+    float max_fp;
+    thip_value_t input;
+    thip_value_t weights;
+} thip_hl_act_t;
+
 thip_status_t thip_hl_conv2d(thip_program_t *program, const thip_hl_conv2d_t *op);
 thip_status_t thip_hl_depthwise_conv2d(thip_program_t *program,
                                        const thip_hl_depthwise_conv2d_t *op);
@@ -277,6 +324,9 @@ thip_status_t thip_hl_avg_pool2d(thip_program_t *program, const thip_hl_avg_pool
 thip_status_t thip_hl_add(thip_program_t *program, const thip_hl_add_t *op);
 thip_status_t thip_hl_transpose(thip_program_t *program, const thip_hl_transpose_t *op);
 thip_status_t thip_hl_expand_weights(thip_program_t *program, const thip_hl_expand_weights_t *op);
+thip_status_t thip_hl_fma(thip_program_t *program, const thip_hl_fma_t *op);
+thip_status_t thip_hl_mul(thip_program_t *program, const thip_hl_mul_t *op);
+thip_status_t thip_hl_act(thip_program_t *program, const thip_hl_act_t *op);
 
 /* Serialises the program (role of TargetBackend::serializeExecutable,
  * compiler/torq/Target/TorqTarget.cpp:115-151, and serializeTorqHW,

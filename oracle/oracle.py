@@ -348,6 +348,54 @@ def add(input1, input2, weights, scale_bias, *, output_zp, output_min, output_ma
     return out
 
 
+_INT_TYPES = (np.int8, np.int16, np.int32)
+ACT_MODES = {"clamp": 0, "abs": 1, "negate": 2, "i2i": 3}
+
+
+def _int_array(a):
+    a = np.ascontiguousarray(a)
+    assert a.dtype in [np.dtype(t) for t in _INT_TYPES], a.dtype
+    return a
+
+
+def fma(input, weights, scale_bias, *, output_zp, output_min, output_max, shift_factor, out_dtype=np.int8):
+    """torq_hl.fma (stand-alone rescale): one scalar weight, one [bias, scale] pair."""
+    x = _int_array(input)
+    w = np.asarray(weights).reshape(-1)
+    sb = _c(scale_bias, np.int32)
+    out = np.empty(x.shape, dtype=out_dtype)
+    rq = Requant(shift_factor, output_zp, output_min, output_max)
+    rc = lib().torq_fma(_p(x), x.itemsize, ctypes.c_int32(int(w[0])), _p(sb), _p(out), out.itemsize, ctypes.c_size_t(x.size), ctypes.byref(rq))
+    assert rc == 0
+    return out
+
+
+def mul(input1, input2, scale_bias, *, output_zp, output_min, output_max, shift, out_dtype=np.int8):
+    """torq_hl.mul: elementwise product (a one-element input is broadcast), one [bias, scale] pair."""
+    a = _int_array(input1)
+    b = _int_array(input2)
+    assert a.dtype == b.dtype
+    shape = a.shape if a.size >= b.size else b.shape
+    count = max(a.size, b.size)
+    sb = _c(scale_bias, np.int32)
+    out = np.empty(shape, dtype=out_dtype)
+    rq = Requant(shift, output_zp, output_min, output_max)
+    rc = lib().torq_mul(_p(a), ctypes.c_size_t(a.size), _p(b), ctypes.c_size_t(b.size), a.itemsize, _p(sb), _p(out), out.itemsize,
+                        ctypes.c_size_t(count), ctypes.byref(rq))
+    assert rc == 0
+    return out
+
+
+def act(input, name, *, min_int=0, max_int=0, out_dtype=None):
+    """torq_hl.act on integers: name in clamp / abs / negate / i2i."""
+    x = _int_array(input)
+    out = np.empty(x.shape, dtype=x.dtype if out_dtype is None else out_dtype)
+    rc = lib().torq_act(_p(x), x.itemsize, _p(out), out.itemsize, ctypes.c_size_t(x.size), ACT_MODES[name], ctypes.c_int64(int(min_int)),
+                        ctypes.c_int64(int(max_int)))
+    assert rc == 0
+    return out
+
+
 def per_channel_sum(weights):
     w = _c(weights, np.int8)
     ch = w.shape[0]

@@ -534,6 +534,81 @@ int torq_add(const int8_t *input1, const int8_t *input2, const int16_t weights[2
     return 0;
 }
 
+static inline int64_t load_elem(const void *in, size_t idx, int bytes) {
+    switch (bytes) {
+    case 1: return ((const int8_t *)in)[idx];
+    case 2: return ((const int16_t *)in)[idx];
+    default: return ((const int32_t *)in)[idx];
+    }
+}
+
+/*
+ * torq_hl.fma -- signature TorqHLOps.td:926-941; the stand-alone rescale, created
+ * compiler/torq/Conversions/LinalgToTorqHL/Patterns.cpp:1896-1946 (weight 1, bias = -input_zp, scale = the
+ * multiplier, shift_factor = the shift); executed compiler/torq/Conversions/TorqHLToTorqHW/FMAPattern.cpp:19-50:
+ * acc = input * weights[0] (one scalar weight), rescaleClamp with ONE (bias, scale) pair.
+ */
+int torq_fma(const void *input, int in_bytes, int32_t weight, const int32_t scale_bias[2], void *out, int out_bytes,
+             size_t count, const torq_requant_t *rq) {
+    if (bad_out_bytes(in_bytes) || bad_out_bytes(out_bytes)) return -1;
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < count; i++) {
+        const int32_t acc = (int32_t)((uint32_t)load_elem(input, i, in_bytes) * (uint32_t)weight);
+        store_elem(out, i, torq_act_rescale_clamp(acc, scale_bias[0], scale_bias[1], rq), out_bytes);
+    }
+    return 0;
+}
+
+/*
+ * torq_hl.mul -- signature TorqHLOps.td:101-117; created
+ * compiler/torq/Conversions/LinalgToTorqHL/MulPattern.cpp:178-212,354-378 (no input zero points: bias 0 or the
+ * folded constant, one scale, `shift`); executed compiler/torq/Conversions/TorqHLToTorqHW/MulPattern.cpp:19-62:
+ * the inputs broadcast to the output, acc = input1 * input2 elementwise, rescaleClamp with ONE pair.
+ * count1 / count2: elements of each input, `count` or 1 (a one-element tensor is broadcast).
+ */
+int torq_mul(const void *input1, size_t count1, const void *input2, size_t count2, int in_bytes,
+             const int32_t scale_bias[2], void *out, int out_bytes, size_t count, const torq_requant_t *rq) {
+    if (bad_out_bytes(in_bytes) || bad_out_bytes(out_bytes)) return -1;
+    if ((count1 != count && count1 != 1) || (count2 != count && count2 != 1)) return -1;
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < count; i++) {
+        const int64_t a = load_elem(input1, count1 == 1 ? 0 : i, in_bytes), b = load_elem(input2, count2 == 1 ? 0 : i, in_bytes);
+        const int32_t acc = (int32_t)((uint32_t)(int32_t)a * (uint32_t)(int32_t)b);
+        store_elem(out, i, torq_act_rescale_clamp(acc, scale_bias[0], scale_bias[1], rq), out_bytes);
+    }
+    return 0;
+}
+
+/*
+ * torq_hl.act on integers -- signature TorqHLOps.td:291-309; executed
+ * compiler/torq/Conversions/TorqHLToTorqHW/ActPattern.cpp:60-140,196-212: the ALU passes the input through and
+ * the ACT unit applies `mode`, then clips: "clamp" clips to [min_int, max_int]; "abs" and "negate" clip to the
+ * range of the output type (abs(-128) is 127 in int8; the zero-point attributes are not read by the lowering);
+ * "i2i" clips to the int32 range, i.e. converts by truncation.
+ * mode: 0 clamp, 1 abs, 2 negate, 3 i2i.
+ */
+int torq_act(const void *input, int in_bytes, void *out, int out_bytes, size_t count, int mode, int64_t min_int,
+             int64_t max_int) {
+    if (bad_out_bytes(in_bytes) || bad_out_bytes(out_bytes) || mode < 0 || mode > 3) return -1;
+    int64_t lo = min_int, hi = max_int;
+    if (mode == 1 || mode == 2) {
+        lo = out_bytes == 1 ? INT8_MIN : out_bytes == 2 ? INT16_MIN : INT32_MIN;
+        hi = out_bytes == 1 ? INT8_MAX : out_bytes == 2 ? INT16_MAX : INT32_MAX;
+    } else if (mode == 3) {
+        lo = INT32_MIN;
+        hi = INT32_MAX;
+    }
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < count; i++) {
+        int64_t v = load_elem(input, i, in_bytes);
+        if (mode == 1) v = v < 0 ? -v : v;
+        if (mode == 2) v = -v;
+        v = v < lo ? lo : (v > hi ? hi : v);
+        store_elem(out, i, v, out_bytes);
+    }
+    return 0;
+}
+
 /* ---- R2 ---- */
 
 /* compiler/torq/Utils/ConversionUtils.cpp:122-141 (per_channel_sum). */

@@ -132,6 +132,20 @@ int torq_avg_pool2d(const int8_t *input, int8_t weight, const int32_t *scale_bia
 int torq_add(const int8_t *input1, const int8_t *input2, const int16_t weights[2],
              const int32_t scale_bias[2], int8_t *out, size_t count, const torq_requant_t *rq);
 
+/* torq_hl.fma (the stand-alone rescale): out = R1(input * weight) with one [bias, scale] pair; int8 / int16 /
+ * int32 elements (in_bytes, out_bytes = 1, 2, 4). */
+int torq_fma(const void *input, int in_bytes, int32_t weight, const int32_t scale_bias[2], void *out, int out_bytes,
+             size_t count, const torq_requant_t *rq);
+
+/* torq_hl.mul: out = R1(input1 * input2) with one [bias, scale] pair; an input of one element is broadcast. */
+int torq_mul(const void *input1, size_t count1, const void *input2, size_t count2, int in_bytes,
+             const int32_t scale_bias[2], void *out, int out_bytes, size_t count, const torq_requant_t *rq);
+
+/* torq_hl.act on integers; mode 0 clamp [min_int, max_int], 1 abs, 2 negate (both clipped to the output type),
+ * 3 i2i (truncating conversion). */
+int torq_act(const void *input, int in_bytes, void *out, int out_bytes, size_t count, int mode, int64_t min_int,
+             int64_t max_int);
+
 /* ---- R2: compile-side parameter derivations ---- */
 
 /* Conv / depthwise / FC: per-channel TOSA (multiplier, shift) -> one global

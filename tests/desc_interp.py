@@ -25,7 +25,8 @@ TEMP = np.dtype([("size", "<u8")])
 CONST = np.dtype([("offset", "<u8"), ("size", "<u8")])
 
 K_TRANSPOSE, K_IGEMM, K_FC_SKINNY, K_DW, K_MAXPOOL, K_AVGPOOL, K_ADD, K_FC_BF16, K_ADD_BF16, K_IM2COL_BF16, K_DW_BF16 = 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11
-K_AVGPOOL_BF16, K_EXPAND = 12, 13
+K_AVGPOOL_BF16, K_EXPAND, K_ELTWISE = 12, 13, 14
+INT_BY_SIZE = {1: np.int8, 2: np.int16, 4: np.int32}
 OUT_NP = {1: np.int8, 2: np.int16, 3: np.int32}
 
 
@@ -44,6 +45,9 @@ class Descriptor:
         c = self.consts[index]
         start = int(self.header["data_offset"] + c["offset"])
         return self.blob[start:start + int(c["size"])]
+
+
+_TYPE_RANGE = {np.int8: (-128, 127), np.int16: (-32768, 32767), np.int32: (-2 ** 31, 2 ** 31 - 1)}
 
 
 def _requant_vec(acc, bias, scale, shift, zp, mn, mx, pre=0, t0_clamp=0):
@@ -254,6 +258,24 @@ def run(blob, binding_arrays):
             res = orc.avg_pool2d_bf16(x, np.array([op["w0"]], dtype=np.uint16), np.array([op["bias0"]], dtype=np.int32).view(np.float32),
                                       output_min=mn, output_max=mx)
             view(op["out"], Nimg * C * 2).view(np.uint16)[:] = res.reshape(-1)
+        elif kind == K_ELTWISE:
+            n, variant, bcast = int(op["C"]), int(op["variant"]), int(op["w1"])
+            tin, tout = INT_BY_SIZE[int(op["gran"])], OUT_NP[int(op["out_dtype"])]
+            esz, osz = np.dtype(tin).itemsize, np.dtype(tout).itemsize
+            a = view(op["in0"], (1 if bcast == 1 else n) * esz).view(tin)
+            if variant == 0:
+                res = orc.fma(a, [int(op["w0"])], [int(op["bias0"]), int(op["scale0"])], output_zp=zp, output_min=mn, output_max=mx,
+                              shift_factor=sh, out_dtype=tout)
+            elif variant == 1:
+                b = view(op["in1"], (1 if bcast == 2 else n) * esz).view(tin)
+                res = orc.mul(a, b, [int(op["bias0"]), int(op["scale0"])], output_zp=zp, output_min=mn, output_max=mx, shift=sh, out_dtype=tout)
+            else:
+                name = {2: "clamp", 3: "abs", 4: "negate", 5: "i2i"}[variant]
+                if name != "clamp":  # the record carries the clip range the op implies
+                    want = {"abs": _TYPE_RANGE[tout], "negate": _TYPE_RANGE[tout], "i2i": _TYPE_RANGE[np.int32]}[name]
+                    assert (mn, mx) == want, (name, mn, mx)
+                res = orc.act(a, name, min_int=mn, max_int=mx, out_dtype=tout)
+            view(op["out"], n * osz).view(tout)[:] = res.reshape(-1)
         elif kind == K_EXPAND:
             K, N, block, cols = int(op["K"]), int(op["Nn"]), int(op["gran"]), int(op["Np"])
             G = K // block

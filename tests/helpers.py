@@ -26,6 +26,12 @@ def oracle_eval(wl):
         fn = orc.conv2d_bf16 if kind == "convbf16" else orc.depthwise_conv2d_bf16
         return [fn(x, a["weights"], a["bias"], pad=a["pad"], stride=a["stride"], output_min=a["output_min"], output_max=a["output_max"],
                    layout=orc.NHWC if a["nhwc"] else orc.NCHW)]
+    if kind == "fma":
+        return [orc.fma(x, a.pop("weights"), a.pop("scale_bias"), **a)]
+    if kind == "mul":
+        return [orc.mul(x, wl.inputs[1], a.pop("scale_bias"), **a)]
+    if kind == "act":
+        return [orc.act(x, a["name"], min_int=a["min_int"], max_int=a["max_int"], out_dtype=a["out_dtype"])]
     if kind == "avgpoolbf16":
         return [orc.avg_pool2d_bf16(x, a["weights"], a["bias"], output_min=a["output_min"], output_max=a["output_max"])]
     if kind == "expandmm":

@@ -1,0 +1,155 @@
+"""Integer elementwise ops next to the convolution path: torq_hl.fma (the stand-alone rescale), torq_hl.mul and
+torq_hl.act (clamp / abs / negate / i2i).  Oracle pins, the emitter, and (on a GPU) the kernel, bit-exact."""
+import numpy as np
+import pytest
+
+import desc_interp
+from helpers import assert_bit_exact, oracle_eval, run_on_gpu
+from oracle import oracle as orc
+from torq_compiler_amd import Program, ThipError, runtime, workloads as w
+
+
+def _r1_exact(acc, bias, scale, shift, zp, lo, hi):
+    """The ACT stage with Python integers: floor((t0 * scale) / 2^shift + 1/2) as an exact rational."""
+    t1 = (int(acc) + int(bias)) * int(scale)
+    t3 = (2 * t1 + (1 << shift)) // (1 << (shift + 1)) if shift > 0 else t1
+    return min(max(t3 + zp, lo), hi)
+
+
+# ---- oracle pins ----------------------------------------------------------------------------------------
+def test_fma_is_the_exact_rescale():
+    """Every int8 input (and a sweep of int16 / int32 ones) against exact integer arithmetic; scale = 2^shift with
+    weight 1 is x - input_zp + output_zp."""
+    x8 = np.arange(-128, 128, dtype=np.int8)
+    for shift, scale, bias, zp, weight in [(31, 1 << 30, 3, -2, 1), (38, 1518500250, -7, 11, 1), (12, 2896, 0, 0, -3), (0, 5, 1, 0, 2), (45, 2 ** 31 - 1, 100, -128, 1)]:
+        got = orc.fma(x8, [weight], [bias, scale], output_zp=zp, output_min=-128, output_max=127, shift_factor=shift)
+        want = [_r1_exact(int(v) * weight, bias, scale, shift, zp, -128, 127) for v in x8]
+        assert got.tolist() == want, (shift, scale)
+    got = orc.fma(x8, [1], [5, 1 << 20], output_zp=-9, output_min=-2 ** 31, output_max=2 ** 31 - 1, shift_factor=20, out_dtype=np.int32)
+    assert np.array_equal(got, x8.astype(np.int32) + 5 - 9)
+    rng = np.random.default_rng(3)
+    x32 = rng.integers(-2 ** 20, 2 ** 20, size=500).astype(np.int32)
+    got = orc.fma(x32, [1], [-17, 1330000000], output_zp=3, output_min=-32768, output_max=32767, shift_factor=37, out_dtype=np.int16)
+    assert got.tolist() == [_r1_exact(int(v), -17, 1330000000, 37, 3, -32768, 32767) for v in x32]
+    x16 = rng.integers(-32768, 32768, size=500).astype(np.int16)
+    got = orc.fma(x16, [1], [128, 1 << 30], output_zp=-128, output_min=-128, output_max=127, shift_factor=38)
+    assert got.tolist() == [_r1_exact(int(v), 128, 1 << 30, 38, -128, -128, 127) for v in x16]
+
+
+def test_mul_against_exact_products():
+    """All 65 536 int8 pairs, random int16 pairs, and both broadcasts."""
+    a, b = np.meshgrid(np.arange(-128, 128, dtype=np.int8), np.arange(-128, 128, dtype=np.int8))
+    for shift, scale, bias, zp in [(37, 1503238554, 0, -4), (20, 1 << 13, 9, 0), (33, 2 ** 31 - 1, -300, 7)]:
+        got = orc.mul(a, b, [bias, scale], output_zp=zp, output_min=-128, output_max=127, shift=shift)
+        t1 = (a.astype(np.int64) * b.astype(np.int64) + bias) * scale
+        want = np.clip(((t1 + (1 << (shift - 1))) >> shift) + zp, -128, 127)  # int64 cannot overflow at these sizes
+        assert np.array_equal(got, want.astype(np.int8)), (shift, scale)
+        sample = [(5, 77), (200, 13), (255, 255), (0, 0), (128, 64)]
+        assert [int(got[i, j]) for i, j in sample] == [_r1_exact(int(a[i, j]) * int(b[i, j]), bias, scale, shift, zp, -128, 127) for i, j in sample]
+    rng = np.random.default_rng(4)
+    x, y = rng.integers(-32768, 32768, size=400).astype(np.int16), rng.integers(-32768, 32768, size=400).astype(np.int16)
+    got = orc.mul(x, y, [0, 1 << 30], output_zp=0, output_min=-32768, output_max=32767, shift=45, out_dtype=np.int16)
+    assert got.tolist() == [_r1_exact(int(p) * int(q), 0, 1 << 30, 45, 0, -32768, 32767) for p, q in zip(x, y)]
+    one = np.array([-7], dtype=np.int16)
+    assert np.array_equal(orc.mul(x, one, [0, 1], output_zp=0, output_min=-2 ** 31, output_max=2 ** 31 - 1, shift=0, out_dtype=np.int32), x.astype(np.int32) * -7)
+    assert np.array_equal(orc.mul(one, x, [0, 1], output_zp=0, output_min=-2 ** 31, output_max=2 ** 31 - 1, shift=0, out_dtype=np.int32), x.astype(np.int32) * -7)
+
+
+def test_act_modes():
+    x = np.arange(-128, 128, dtype=np.int8)
+    assert np.array_equal(orc.act(x, "clamp", min_int=-20, max_int=90), np.clip(x, -20, 90))
+    assert np.array_equal(orc.act(x, "abs"), np.minimum(np.abs(x.astype(np.int32)), 127).astype(np.int8))      # |-128| saturates
+    assert np.array_equal(orc.act(x, "negate"), np.minimum(-x.astype(np.int32), 127).astype(np.int8))
+    assert np.array_equal(orc.act(x, "abs", out_dtype=np.int16), np.abs(x.astype(np.int16)))                    # the wider type holds 128
+    wide = np.array([-2 ** 31, -70000, -129, -1, 0, 127, 128, 65535, 2 ** 31 - 1], dtype=np.int32)
+    assert np.array_equal(orc.act(wide, "i2i", out_dtype=np.int8), wide.astype(np.int8))                        # truncation, no clipping
+    assert np.array_equal(orc.act(wide, "i2i", out_dtype=np.int16), wide.astype(np.int16))
+    assert np.array_equal(orc.act(x, "i2i", out_dtype=np.int32), x.astype(np.int32))
+    assert np.array_equal(orc.act(wide, "negate"), np.clip(-wide.astype(np.int64), -2 ** 31, 2 ** 31 - 1).astype(np.int32))
+    assert np.array_equal(orc.act(wide, "clamp", min_int=-100, max_int=100, out_dtype=np.int8), np.clip(wide, -100, 100).astype(np.int8))
+
+
+# ---- emitter ----------------------------------------------------------------------------------------------
+CASES = [lambda: w.fma_workload(), lambda: w.fma_workload((3, 5, 7), np.int16, np.int8, input_zp=11, scale=0.004, output_zp=-128),
+         lambda: w.fma_workload((1000,), np.int32, np.int16, scale=0.0021, output_zp=0), lambda: w.fma_workload((37,), np.int8, np.int32, scale=3.7, weight=-2),
+         lambda: w.fma_workload((4, 33), np.int8, np.int16, scale=2.0 ** -20),
+         lambda: w.mul_workload(), lambda: w.mul_workload((2, 9, 13), np.int16, np.int8, scale=2.0 ** -22, output_zp=3),
+         lambda: w.mul_workload((129,), np.int8, np.int32, scale=0.5, bias=-5), lambda: w.mul_workload((5, 17), np.int16, np.int16, scale=2.0 ** -15, broadcast=2),
+         lambda: w.mul_workload((64,), np.int8, np.int8, scale=0.02, broadcast=1),
+         lambda: w.act_workload("clamp"), lambda: w.act_workload("abs"), lambda: w.act_workload("negate", (77,), np.int16),
+         lambda: w.act_workload("i2i", (5, 9), np.int32, np.int8), lambda: w.act_workload("i2i", (50,), np.int8, np.int32),
+         lambda: w.act_workload("abs", (19,), np.int8, np.int16), lambda: w.act_workload("clamp", (300,), np.int32, np.int16, min_int=-32768, max_int=1000)]
+
+
+@pytest.mark.parametrize("make", CASES)
+def test_eltwise_descriptor(make):
+    wl = make()
+    outs = [np.zeros(s, dtype=dt) for s, dt in wl.outputs]
+    d = desc_interp.run(wl.program.serialize(), list(wl.inputs) + outs)
+    assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)
+    assert [int(o["kind"]) for o in d.ops] == [desc_interp.K_ELTWISE]
+
+
+def test_eltwise_in_a_program():
+    """conv2d -> act(clamp) -> fma -> mul with the conv's own output: intermediates, not bindings."""
+    conv = w.conv2d_workload(N=1, H=12, W=12, C=16, O=32, nhwc=True)
+    rng = np.random.default_rng(8)
+    x = conv.inputs[0]
+    p = Program()
+    inp = p.binding(0, x.shape)
+    a = conv.attrs
+    y = p.conv2d(inp, a["weights"], a["scale_bias"], input_zp=a["input_zp"], output_zp=a["output_zp"], output_min=a["output_min"], output_max=a["output_max"],
+                 shift_factor=a["shift_factor"], pad=a["pad"], stride=a["stride"], nhwc_input=True)
+    c = p.act(y, "clamp", min_int=-50, max_int=60)
+    r = p.fma(c, np.array([1], dtype=np.int8), np.array([7, 1 << 30], dtype=np.int32), output_zp=-1, output_min=-128, output_max=127, shift_factor=31)
+    out = p.binding(1, y.shape)
+    p.mul(r, y, np.array([0, 1 << 24], dtype=np.int32), output_zp=2, output_min=-128, output_max=127, shift=30, init=out)
+    got = np.zeros(y.shape, dtype=np.int8)
+    d = desc_interp.run(p.serialize(), [x, got])
+    y0 = oracle_eval(conv)[0]
+    c0 = orc.act(y0, "clamp", min_int=-50, max_int=60)
+    r0 = orc.fma(c0, [1], [7, 1 << 30], output_zp=-1, output_min=-128, output_max=127, shift_factor=31)
+    want = orc.mul(r0, y0, [0, 1 << 24], output_zp=2, output_min=-128, output_max=127, shift=30)
+    assert_bit_exact(got, want, "conv -> clamp -> fma -> mul")
+    assert [int(o["kind"]) for o in d.ops][-3:] == [desc_interp.K_ELTWISE] * 3
+    del rng
+
+
+def test_eltwise_rejections():
+    def expect(code, build):
+        p = Program()
+        with pytest.raises(ThipError) as e:
+            build(p)
+            p.serialize()
+        assert e.value.code == code, e.value
+
+    sb = np.array([0, 1], dtype=np.int32)
+    one = np.array([1], dtype=np.int8)
+    ok = dict(output_zp=0, output_min=-128, output_max=127)
+    expect(runtime.INVALID_ARGUMENT, lambda p: p.fma(p.binding(0, (8,)), one, sb, init=p.binding(1, (9,)), shift_factor=1, **ok))
+    expect(runtime.INVALID_ARGUMENT, lambda p: p.fma(p.binding(0, (8,)), one, sb, init=p.binding(1, (8,)), shift_factor=64, **ok))
+    expect(runtime.INVALID_ARGUMENT, lambda p: p.fma(p.binding(0, (8,)), one, sb, init=p.binding(1, (8,)), shift_factor=1, output_zp=0, output_min=-129, output_max=127))
+    expect(runtime.UNIMPLEMENTED, lambda p: p.fma(p.binding(0, (8,), np.uint16), one, sb, init=p.binding(1, (8,)), shift_factor=1, **ok))
+    expect(runtime.UNIMPLEMENTED, lambda p: p.mul(p.binding(0, (8,)), p.binding(1, (8,), np.int16), sb, init=p.binding(2, (8,)), shift=1, **ok))
+    expect(runtime.UNIMPLEMENTED, lambda p: p.mul(p.binding(0, (8,)), p.binding(1, (4,)), sb, init=p.binding(2, (8,)), shift=1, **ok))
+    expect(runtime.UNIMPLEMENTED, lambda p: p.act(p.binding(0, (8,)), "ceil", init=p.binding(1, (8,))))
+    expect(runtime.UNIMPLEMENTED, lambda p: p.act(p.binding(0, (8,)), "i2i", init=p.binding(1, (8,)), weights=one))
+    expect(runtime.INVALID_ARGUMENT, lambda p: p.act(p.binding(0, (8,)), "clamp", min_int=-200, max_int=5, init=p.binding(1, (8,))))
+    expect(runtime.INVALID_ARGUMENT, lambda p: p.act(p.binding(0, (8,)), "clamp", min_int=6, max_int=5, init=p.binding(1, (8,))))
+
+
+# ---- GPU ---------------------------------------------------------------------------------------------------
+@pytest.mark.gpu
+def test_gpu_eltwise(device):
+    """Every case of the emitter test, plus sizes that exercise whole vectors, the ragged tail and both requant tails
+    (shift below and above 33)."""
+    extra = [lambda: w.fma_workload((64, 56, 56, 24)), lambda: w.fma_workload((100003,), np.int16, np.int8, scale=0.0009, output_zp=-7),
+             lambda: w.fma_workload((4099,), np.int8, np.int8, scale=2.0 ** -3), lambda: w.mul_workload((64, 56, 56, 24)),
+             lambda: w.mul_workload((70001,), np.int16, np.int8, scale=2.0 ** -21, broadcast=2), lambda: w.mul_workload((1031,), np.int8, np.int16, scale=0.3),
+             lambda: w.act_workload("abs", (64, 56, 56, 24)), lambda: w.act_workload("i2i", (9999,), np.int32, np.int8)]
+    for make in CASES + extra:
+        wl = make()
+        print("[gpu-case]", wl.name, flush=True)
+        got, kernels = run_on_gpu(device, wl, via="device" if wl.inputs[0].size > 5000 else "host")
+        assert_bit_exact(got[0], oracle_eval(wl)[0], wl.name)
+        assert kernels == ["eltwise_int"]

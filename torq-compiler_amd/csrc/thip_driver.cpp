@@ -277,6 +277,16 @@ static thip_status_t checkOpFootprint(const thip_executable_t *e, uint32_t i) {
         if ((s = need(op.bias, (uint64_t)(op.K / block) * op.Np * 4, "bias"))) return s;
         return need(op.out, (uint64_t)op.K * op.Nn * 2, "out");
     }
+    case kKindEltwise: {
+        const uint64_t inElem = op.gran, outElem = op.out_dtype == THIP_DTYPE_I8 ? 1 : op.out_dtype == THIP_DTYPE_I16 ? 2 : op.out_dtype == THIP_DTYPE_I32 ? 4 : 0;
+        if (!positive({op.C}) || !(inElem == 1 || inElem == 2 || inElem == 4) || outElem == 0 || op.variant > kEltCast || op.w1 < 0 || op.w1 > 2 ||
+            (op.variant != kEltMul && op.w1 != 0)) {
+            return fail(THIP_INVALID_ARGUMENT, "op %u: bad elementwise record", i);
+        }
+        if ((s = need(op.in0, (op.w1 == 1 ? 1 : (uint64_t)op.C) * inElem, "in1"))) return s;
+        if (op.variant == kEltMul && (s = need(op.in1, (op.w1 == 2 ? 1 : (uint64_t)op.C) * inElem, "in2"))) return s;
+        return need(op.out, (uint64_t)op.C * outElem, "out");
+    }
     case kKindAddBf16: {
         if (!positive({op.C})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad add extent", i);
         if ((s = need(op.in0, (uint64_t)op.C * 2, "in1"))) return s;
@@ -325,6 +335,7 @@ static const char *opKernelName(const DescOp &op) {
     case kKindDepthwiseBf16: return "depthwise_bf16";
     case kKindAvgPoolBf16: return "avgpool_bf16";
     case kKindExpandWeights: return "expand_weights_bf16";
+    case kKindEltwise: return "eltwise_int";
     default: return "unknown";
     }
 }
@@ -466,6 +477,13 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
         memcpy(&a.lo, &op.output_min, 4);
         memcpy(&a.hi, &op.output_max, 4);
         err = launchAvgPoolBf16(a, e->stream);
+        break;
+    }
+    case kKindEltwise: {
+        EltwiseArgs a{resolve(e, op.in0, bp), op.variant == kEltMul ? resolve(e, op.in1, bp) : nullptr, resolve(e, op.out, bp), (int64_t)op.C,
+                      (int32_t)op.variant, (int32_t)op.gran, op.out_dtype == THIP_DTYPE_I8 ? 1 : op.out_dtype == THIP_DTYPE_I16 ? 2 : 4, op.w1,
+                      op.w0, op.bias0, op.scale0, op.output_min, op.output_max, rq};
+        err = launchEltwise(a, e->stream);
         break;
     }
     case kKindExpandWeights: {

@@ -44,7 +44,7 @@ struct Value {
     }
 };
 
-enum HlKind { kHlConv2d, kHlDepthwise, kHlFullyConnected, kHlMatmul, kHlMaxPool, kHlAvgPool, kHlAdd, kHlTranspose, kHlExpandWeights };
+enum HlKind { kHlConv2d, kHlDepthwise, kHlFullyConnected, kHlMatmul, kHlMaxPool, kHlAvgPool, kHlAdd, kHlTranspose, kHlExpandWeights, kHlFma, kHlMul, kHlAct };
 
 struct HlOp {
     HlKind kind;
@@ -58,6 +58,9 @@ struct HlOp {
         thip_hl_add_t add;
         thip_hl_transpose_t tr;
         thip_hl_expand_weights_t ew;
+        thip_hl_fma_t fma;
+        thip_hl_mul_t mul;
+        thip_hl_act_t act;
     } u;
     std::string name;
 };
@@ -519,6 +522,11 @@ class Emitter {
     thip_status_t emitAdd(const thip_hl_add_t &c);
     thip_status_t emitTransposeOp(const thip_hl_transpose_t &c);
     thip_status_t emitExpandWeights(const thip_hl_expand_weights_t &c);
+    thip_status_t emitFma(const thip_hl_fma_t &c);
+    thip_status_t emitMul(const thip_hl_mul_t &c);
+    thip_status_t emitAct(const thip_hl_act_t &c, const std::string &name);
+    // Operands of an integer elementwise op: element types, and the record's common fields.
+    thip_status_t eltwiseCommon(const char *what, thip_value_t input, thip_value_t init, DescOp *op);
     thip_status_t emitAvgPoolBf16(const thip_hl_avg_pool2d_t &c);
     // Operands of an expand_weights checked and measured.
     struct ExpandShape {
@@ -1297,6 +1305,131 @@ thip_status_t Emitter::emitExpandWeights(const thip_hl_expand_weights_t &c) {
     return THIP_OK;
 }
 
+static bool isIntDtype(int32_t d) { return d == THIP_DTYPE_I8 || d == THIP_DTYPE_I16 || d == THIP_DTYPE_I32; }
+
+thip_status_t Emitter::eltwiseCommon(const char *what, thip_value_t input, thip_value_t init, DescOp *op) {
+    const Value *x, *o;
+    if (thip_status_t s = checkValue(input, what, &x)) return s;
+    if (thip_status_t s = checkValue(init, what, &o)) return s;
+    if (!isIntDtype(x->dtype) || !isIntDtype(o->dtype)) return fail(THIP_UNIMPLEMENTED, "%s: int8 / int16 / int32 tensors only", what);
+    if (x->numel() != o->numel() || x->numel() <= 0) return fail(THIP_INVALID_ARGUMENT, "%s: input and init differ in element count", what);
+    if (state_[input].nhwcOfNchw) return fail(THIP_UNIMPLEMENTED, "%s: N,C,H,W intermediates are not accepted", what);
+    if (!fitsInt32(x->numel())) return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
+    memset(op, 0, sizeof(*op));
+    op->kind = kKindEltwise;
+    op->gran = (uint32_t)elemSize(x->dtype);
+    op->out_dtype = o->dtype;
+    op->N = 1; op->H = 1; op->W = 1;
+    op->C = (int32_t)x->numel();
+    if (thip_status_t s = literalInput(input, what, &op->in0)) return s;
+    return literalOutput(init, what, o->dtype, x->numel(), &op->out);
+}
+
+thip_status_t Emitter::emitFma(const thip_hl_fma_t &c) {
+    const char *what = "torq_hl.fma";
+    const Value *w, *sb, *init;
+    if (thip_status_t s = checkValue(c.init, what, &init)) return s;
+    if (thip_status_t s = checkRequant(what, c.shift_factor, c.output_zp, c.output_min, c.output_max, init->dtype)) return s;
+    if (thip_status_t s = checkValue(c.weights, "torq_hl.fma weights", &w)) return s;
+    if (w->kind != kValueConstant || (w->dtype != THIP_DTYPE_I8 && w->dtype != THIP_DTYPE_I16) || w->numel() < 1) {
+        return fail(THIP_UNIMPLEMENTED, "%s: weights must be a constant int8 / int16 scalar", what);
+    }
+    if (thip_status_t s = constantData(c.scale_bias, "torq_hl.fma scale_bias", THIP_DTYPE_I32, &sb)) return s;
+    if (sb->numel() < 2) return fail(THIP_INVALID_ARGUMENT, "%s: scale_bias too short", what);
+    DescOp op;
+    if (thip_status_t s = eltwiseCommon(what, c.input, c.init, &op)) return s;
+    op.variant = kEltFma;
+    op.w0 = w->dtype == THIP_DTYPE_I8 ? (int32_t)((const int8_t *)w->data.data())[0] : (int32_t)((const int16_t *)w->data.data())[0];
+    op.bias0 = ((const int32_t *)sb->data.data())[0];
+    op.scale0 = ((const int32_t *)sb->data.data())[1];
+    op.shift = c.shift_factor;
+    op.output_zp = c.output_zp;
+    op.output_min = c.output_min;
+    op.output_max = c.output_max;
+    ops_.push_back(op);
+    return THIP_OK;
+}
+
+thip_status_t Emitter::emitMul(const thip_hl_mul_t &c) {
+    const char *what = "torq_hl.mul";
+    const Value *a, *b, *init, *sb;
+    if (thip_status_t s = checkValue(c.input1, "torq_hl.mul input1", &a)) return s;
+    if (thip_status_t s = checkValue(c.input2, "torq_hl.mul input2", &b)) return s;
+    if (thip_status_t s = checkValue(c.init, "torq_hl.mul init", &init)) return s;
+    if (a->dtype != b->dtype || (a->dtype != THIP_DTYPE_I8 && a->dtype != THIP_DTYPE_I16)) {
+        return fail(THIP_UNIMPLEMENTED, "%s: inputs must both be int8 or both int16 (the bf16 form is not on this path)", what);
+    }
+    if (!isIntDtype(init->dtype)) return fail(THIP_UNIMPLEMENTED, "%s: init must be int8 / int16 / int32", what);
+    if (thip_status_t s = checkRequant(what, c.shift, c.output_zp, c.output_min, c.output_max, init->dtype)) return s;
+    const int64_t count = init->numel();
+    if ((a->numel() != count && a->numel() != 1) || (b->numel() != count && b->numel() != 1) || count <= 0) {
+        return fail(THIP_UNIMPLEMENTED, "%s: an input must have init's element count or one element", what);
+    }
+    if (state_[c.input1].nhwcOfNchw || state_[c.input2].nhwcOfNchw) return fail(THIP_UNIMPLEMENTED, "%s: N,C,H,W intermediates are not accepted", what);
+    if (!fitsInt32(count)) return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
+    if (thip_status_t s = constantData(c.scale_bias, "torq_hl.mul scale_bias", THIP_DTYPE_I32, &sb)) return s;
+    if (sb->numel() < 2) return fail(THIP_INVALID_ARGUMENT, "%s: scale_bias too short", what);
+    DescOp op;
+    memset(&op, 0, sizeof(op));
+    op.kind = kKindEltwise;
+    op.variant = kEltMul;
+    op.gran = (uint32_t)elemSize(a->dtype);
+    op.out_dtype = init->dtype;
+    op.N = 1; op.H = 1; op.W = 1;
+    op.C = (int32_t)count;
+    op.w1 = count == 1 ? 0 : a->numel() == 1 ? 1 : b->numel() == 1 ? 2 : 0;
+    if (thip_status_t s = literalInput(c.input1, "torq_hl.mul input1", &op.in0)) return s;
+    if (thip_status_t s = literalInput(c.input2, "torq_hl.mul input2", &op.in1)) return s;
+    if (thip_status_t s = literalOutput(c.init, "torq_hl.mul init", init->dtype, count, &op.out)) return s;
+    op.bias0 = ((const int32_t *)sb->data.data())[0];
+    op.scale0 = ((const int32_t *)sb->data.data())[1];
+    op.shift = c.shift;
+    op.output_zp = c.output_zp;
+    op.output_min = c.output_min;
+    op.output_max = c.output_max;
+    ops_.push_back(op);
+    return THIP_OK;
+}
+
+thip_status_t Emitter::emitAct(const thip_hl_act_t &c, const std::string &name) {
+    const char *what = "torq_hl.act";
+    if (c.weights != THIP_NO_VALUE) return fail(THIP_UNIMPLEMENTED, "%s: weights (the unsigned cast) are not on this path", what);
+    const Value *init;
+    if (thip_status_t s = checkValue(c.init, what, &init)) return s;
+    int64_t lo, hi;
+    switch (init->dtype) {
+    case THIP_DTYPE_I8: lo = -128; hi = 127; break;
+    case THIP_DTYPE_I16: lo = -32768; hi = 32767; break;
+    default: lo = INT32_MIN; hi = INT32_MAX; break;
+    }
+    uint32_t variant;
+    if (name == "clamp") {
+        variant = kEltClamp;
+        if (c.min_int > c.max_int) return fail(THIP_INVALID_ARGUMENT, "%s: min_int > max_int", what);
+        // a clip range beyond the output type would leave the order of clip and truncation to decide the result
+        if (c.min_int < lo || c.max_int > hi) return fail(THIP_INVALID_ARGUMENT, "%s: clamp range exceeds the output element type", what);
+        lo = c.min_int;
+        hi = c.max_int;
+    } else if (name == "abs") {
+        variant = kEltAbs;
+    } else if (name == "negate") {
+        variant = kEltNegate;
+    } else if (name == "i2i") {
+        variant = kEltCast;
+        lo = INT32_MIN;
+        hi = INT32_MAX;
+    } else {
+        return fail(THIP_UNIMPLEMENTED, "%s: \"%s\" is not on this path (clamp, abs, negate, i2i on integers are)", what, name.c_str());
+    }
+    DescOp op;
+    if (thip_status_t s = eltwiseCommon(what, c.input, c.init, &op)) return s;
+    op.variant = variant;
+    op.output_min = (int32_t)lo;
+    op.output_max = (int32_t)hi;
+    ops_.push_back(op);
+    return THIP_OK;
+}
+
 thip_status_t Emitter::emitAdd(const thip_hl_add_t &c) {
     const char *what = "torq_hl.add";
     if (c.segment_output) return fail(THIP_UNIMPLEMENTED, "%s: segment_output is an NPU memory layout", what);
@@ -1509,6 +1642,9 @@ void Emitter::planChannelPadding() {
         case kHlAvgPool: bar(op.u.ap.input); bar(op.u.ap.init); break;
         case kHlTranspose: bar(op.u.tr.input); bar(op.u.tr.init); break;
         case kHlExpandWeights: bar(op.u.ew.input); bar(op.u.ew.init); break;
+        case kHlFma: bar(op.u.fma.input); bar(op.u.fma.init); break;
+        case kHlMul: bar(op.u.mul.input1); bar(op.u.mul.input2); bar(op.u.mul.init); break;
+        case kHlAct: bar(op.u.act.input); bar(op.u.act.init); break;
         }
     }
     // one verdict per group: every member an int8 rank-4 intermediate, all uses agreeing on C
@@ -1557,6 +1693,9 @@ void Emitter::planExpandFolding() {
         case kHlAdd: read(op.u.add.input1); read(op.u.add.input2); break;
         case kHlTranspose: read(op.u.tr.input); break;
         case kHlExpandWeights: read(op.u.ew.input); read(op.u.ew.scale); read(op.u.ew.scale_bias); break;
+        case kHlFma: read(op.u.fma.input); break;
+        case kHlMul: read(op.u.mul.input1); read(op.u.mul.input2); break;
+        case kHlAct: read(op.u.act.input); break;
         }
     }
     auto constant = [&](thip_value_t v) { return v >= 0 && (size_t)v < n && prog_.values[(size_t)v].kind == kValueConstant; };
@@ -1584,6 +1723,9 @@ thip_status_t Emitter::run(void **outBlob, size_t *outSize) {
         case kHlAdd: s = emitAdd(op.u.add); break;
         case kHlTranspose: s = emitTransposeOp(op.u.tr); break;
         case kHlExpandWeights: s = emitExpandWeights(op.u.ew); break;
+        case kHlFma: s = emitFma(op.u.fma); break;
+        case kHlMul: s = emitMul(op.u.mul); break;
+        case kHlAct: s = emitAct(op.u.act, op.name); break;
         }
         if (s != THIP_OK) return s;
     }
@@ -1717,6 +1859,20 @@ THIP_DEFINE_HL(thip_hl_maxpool2d, thip_hl_maxpool2d_t, kHlMaxPool, mp)
 THIP_DEFINE_HL(thip_hl_avg_pool2d, thip_hl_avg_pool2d_t, kHlAvgPool, ap)
 THIP_DEFINE_HL(thip_hl_transpose, thip_hl_transpose_t, kHlTranspose, tr)
 THIP_DEFINE_HL(thip_hl_expand_weights, thip_hl_expand_weights_t, kHlExpandWeights, ew)
+THIP_DEFINE_HL(thip_hl_fma, thip_hl_fma_t, kHlFma, fma)
+THIP_DEFINE_HL(thip_hl_mul, thip_hl_mul_t, kHlMul, mul)
+
+thip_status_t thip_hl_act(thip_program_t *program, const thip_hl_act_t *op) {
+    if (!program || !op || !op->name) return fail(THIP_INVALID_ARGUMENT, "thip_hl_act: null argument");
+    HlOp h;
+    memset((void *)&h.u, 0, sizeof(h.u));
+    h.kind = kHlAct;
+    h.u.act = *op;
+    h.name = op->name;  // the caller's string need not outlive this call
+    h.u.act.name = nullptr;
+    program->ops.push_back(h);
+    return THIP_OK;
+}
 
 thip_status_t thip_hl_add(thip_program_t *program, const thip_hl_add_t *op) {
     if (!program || !op) return fail(THIP_INVALID_ARGUMENT, "thip_hl_add: null argument");

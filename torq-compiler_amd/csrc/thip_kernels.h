@@ -147,6 +147,24 @@ inline int fcBf16PreferredSplit(int M, int N, int K) {
 }
 hipError_t launchFcBf16(const FcBf16Args &a, hipStream_t stream);
 
+// Integer elementwise ops with the ACT stage behind them.  fma: out = R1(in0 * w0); mul: out = R1(in0 * in1) (an
+// input of one element is broadcast); both with ONE (bias, scale) pair.  clamp / abs / negate / i2i: the input
+// passed through the mode, then clipped to [lo, hi] and truncated to the output type.
+enum EltwiseOp : int32_t { kEltFma = 0, kEltMul = 1, kEltClamp = 2, kEltAbs = 3, kEltNegate = 4, kEltCast = 5 };
+struct EltwiseArgs {
+    const void *in0;
+    const void *in1;  // mul only
+    void *out;
+    int64_t count;
+    int32_t op;
+    int32_t in_bytes, out_bytes;  // 1, 2 or 4 (int8 / int16 / int32)
+    int32_t bcast;                // mul: 0 none, 1 in0 has one element, 2 in1 has one element
+    int32_t w0, bias, scale;
+    int32_t lo, hi;               // clamp / abs / negate / i2i
+    Requant rq;                   // fma / mul
+};
+hipError_t launchEltwise(const EltwiseArgs &a, hipStream_t stream);
+
 // bf16 global average pool: out[n][c] = bf16(clamp(sum_u in[n][u][c] * weight + bias)), summed over the frame
 // in order, in fp32.
 struct AvgPoolBf16Args {

@@ -2006,6 +2006,100 @@ hipError_t launchAddBf16(const AddBf16Args &a, hipStream_t stream) {
     return hipGetLastError();
 }
 
+// Integer elementwise ops: a thread owns VEC neighbouring elements (one wide load per input, one wide store).
+template <typename T, int VEC>
+struct alignas(sizeof(T) * VEC) EltVec {
+    T e[VEC];
+};
+template <typename TIN, typename TOUT, int VEC>
+__global__ __launch_bounds__(256) void eltwise_int(EltwiseArgs p) {
+    const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * VEC;
+    if (i0 >= p.count) return;
+    const TIN *in0 = (const TIN *)p.in0, *in1 = (const TIN *)p.in1;
+    TOUT *out = (TOUT *)p.out;
+    const bool whole = i0 + VEC <= p.count;
+    EltVec<TIN, VEC> a, b;
+    EltVec<TOUT, VEC> o;
+    if (whole && p.bcast != 1) {
+        a = *(const EltVec<TIN, VEC> *)(in0 + i0);
+    } else {
+#pragma unroll
+        for (int v = 0; v < VEC; v++) a.e[v] = p.bcast == 1 ? in0[0] : (i0 + v < p.count ? in0[i0 + v] : (TIN)0);
+    }
+    if (p.op == kEltMul) {
+        if (whole && p.bcast != 2) {
+            b = *(const EltVec<TIN, VEC> *)(in1 + i0);
+        } else {
+#pragma unroll
+            for (int v = 0; v < VEC; v++) b.e[v] = p.bcast == 2 ? in1[0] : (i0 + v < p.count ? in1[i0 + v] : (TIN)0);
+        }
+    }
+    if (p.op == kEltFma || p.op == kEltMul) {
+        const WideRequant wrq = wideRequant(p.rq);
+        const long long rnd = roundTerm(p.rq.shift);
+        withRequantMode(wrq, [&](auto mode) {
+            constexpr int kMode = decltype(mode)::value;
+#pragma unroll
+            for (int v = 0; v < VEC; v++) {
+                const uint32_t rhs = p.op == kEltMul ? (uint32_t)(int32_t)b.e[v] : (uint32_t)p.w0;
+                const int32_t t0 = (int32_t)((uint32_t)(int32_t)a.e[v] * rhs + (uint32_t)p.bias);
+                o.e[v] = (TOUT)requantT0<kMode>(t0, p.scale, rnd, p.rq, wrq);
+            }
+        });
+    } else {
+#pragma unroll
+        for (int v = 0; v < VEC; v++) {
+            long long x = (long long)a.e[v];
+            if (p.op == kEltAbs) x = x < 0 ? -x : x;
+            if (p.op == kEltNegate) x = -x;
+            x = x < p.lo ? (long long)p.lo : (x > p.hi ? (long long)p.hi : x);
+            o.e[v] = (TOUT)x;
+        }
+    }
+    if (whole) {
+        *(EltVec<TOUT, VEC> *)(out + i0) = o;
+    } else {
+#pragma unroll
+        for (int v = 0; v < VEC; v++) {
+            if (i0 + v < p.count) out[i0 + v] = o.e[v];
+        }
+    }
+}
+
+template <typename TIN, typename TOUT>
+static hipError_t launchEltwiseT(const EltwiseArgs &a, hipStream_t stream) {
+    constexpr int VEC = sizeof(TIN) == 1 && sizeof(TOUT) == 1 ? 16 : 8;
+    const uintptr_t bits = (uintptr_t)a.in0 | (a.op == kEltMul ? (uintptr_t)a.in1 : 0);
+    const bool aligned = (bits & (sizeof(TIN) * VEC - 1)) == 0 && (((uintptr_t)a.out) & (sizeof(TOUT) * VEC - 1)) == 0;
+    if (aligned) {
+        const long long threads = (a.count + VEC - 1) / VEC;
+        hipLaunchKernelGGL((eltwise_int<TIN, TOUT, VEC>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, a);
+    } else {
+        hipLaunchKernelGGL((eltwise_int<TIN, TOUT, 1>), dim3((unsigned)((a.count + 255) / 256)), dim3(256), 0, stream, a);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launchEltwise(const EltwiseArgs &a, hipStream_t stream) {
+    if (!a.in0 || !a.out || a.count <= 0 || a.count >= (1LL << 39) || a.op < kEltFma || a.op > kEltCast) return hipErrorInvalidValue;
+    if (a.op == kEltMul && (!a.in1 || a.bcast < 0 || a.bcast > 2)) return hipErrorInvalidValue;
+    if (a.op != kEltMul && a.bcast != 0) return hipErrorInvalidValue;
+    if ((((uintptr_t)a.in0) & (a.in_bytes - 1)) || (((uintptr_t)a.out) & (a.out_bytes - 1))) return hipErrorInvalidValue;
+    if (a.op == kEltMul && (((uintptr_t)a.in1) & (a.in_bytes - 1))) return hipErrorInvalidValue;
+    switch (a.in_bytes * 8 + a.out_bytes) {
+    case 1 * 8 + 1: return launchEltwiseT<int8_t, int8_t>(a, stream);
+    case 1 * 8 + 2: return launchEltwiseT<int8_t, int16_t>(a, stream);
+    case 1 * 8 + 4: return launchEltwiseT<int8_t, int32_t>(a, stream);
+    case 2 * 8 + 1: return launchEltwiseT<int16_t, int8_t>(a, stream);
+    case 2 * 8 + 2: return launchEltwiseT<int16_t, int16_t>(a, stream);
+    case 2 * 8 + 4: return launchEltwiseT<int16_t, int32_t>(a, stream);
+    case 4 * 8 + 1: return launchEltwiseT<int32_t, int8_t>(a, stream);
+    case 4 * 8 + 2: return launchEltwiseT<int32_t, int16_t>(a, stream);
+    case 4 * 8 + 4: return launchEltwiseT<int32_t, int32_t>(a, stream);
+    default: return hipErrorInvalidValue;
+    }
+}
+
 // Batched transpose [B][R][S] -> [B][S][R] of 1- or 2-byte elements through a 64 x 64 LDS tile.
 template <typename T>
 __global__ __launch_bounds__(256) void transpose_i8(TransposeArgs p) {

@@ -41,6 +41,7 @@ EXPORTED_SYMBOLS = [
     "thip_program_create", "thip_program_destroy", "thip_program_binding", "thip_program_constant",
     "thip_program_tensor", "thip_hl_conv2d", "thip_hl_depthwise_conv2d", "thip_hl_fully_connected",
     "thip_hl_matmul", "thip_hl_maxpool2d", "thip_hl_avg_pool2d", "thip_hl_add", "thip_hl_transpose", "thip_hl_expand_weights",
+    "thip_hl_fma", "thip_hl_mul", "thip_hl_act",
     "thip_program_serialize", "thip_blob_free",
     "thip_device_create", "thip_device_destroy", "thip_device_name", "thip_device_alloc",
     "thip_device_free", "thip_device_h2d", "thip_device_d2h", "thip_device_synchronize",
@@ -128,6 +129,34 @@ class HlExpandWeights(ctypes.Structure):
     ]
 
 
+class HlFma(ctypes.Structure):
+    _fields_ = [
+        ("init", ctypes.c_int32), ("output_zp", ctypes.c_int32), ("output_min", ctypes.c_int32),
+        ("output_max", ctypes.c_int32), ("shift_factor", ctypes.c_int32), ("weights", ctypes.c_int32),
+        ("scale_bias", ctypes.c_int32), ("input", ctypes.c_int32),
+    ]
+
+
+class HlMul(ctypes.Structure):
+    _fields_ = [
+        ("init", ctypes.c_int32), ("output_zp", ctypes.c_int32), ("output_min", ctypes.c_int32),
+        ("output_max", ctypes.c_int32), ("scale_bias", ctypes.c_int32), ("shift", ctypes.c_int32),
+        ("input1", ctypes.c_int32), ("input2", ctypes.c_int32),
+    ]
+
+
+class HlAct(ctypes.Structure):
+    _fields_ = [
+        ("init", ctypes.c_int32), ("name", ctypes.c_char_p), ("input_zp", ctypes.c_int32),
+        ("output_zp", ctypes.c_int32), ("min_int", ctypes.c_int64), ("max_int", ctypes.c_int64),
+        ("min_fp", ctypes.c_float), ("max_fp", ctypes.c_float), ("input", ctypes.c_int32),
+        ("weights", ctypes.c_int32),
+    ]
+
+
+NO_VALUE = -1
+
+
 class HlAdd(ctypes.Structure):
     _fields_ = [
         ("init", ctypes.c_int32), ("name", ctypes.c_char_p), ("input_zp", ctypes.c_int32),
@@ -176,7 +205,8 @@ def lib():
                      ("thip_hl_fully_connected", HlFullyConnected), ("thip_hl_matmul", HlMatmul),
                      ("thip_hl_maxpool2d", HlMaxPool2d), ("thip_hl_avg_pool2d", HlAvgPool2d),
                      ("thip_hl_add", HlAdd), ("thip_hl_transpose", HlTranspose),
-                     ("thip_hl_expand_weights", HlExpandWeights)]:
+                     ("thip_hl_expand_weights", HlExpandWeights), ("thip_hl_fma", HlFma), ("thip_hl_mul", HlMul),
+                     ("thip_hl_act", HlAct)]:
         getattr(L, name).argtypes = [vp, P(st)]
     L.thip_program_serialize.argtypes = [vp, P(vp), P(sz)]
     L.thip_blob_free.argtypes = [vp]

@@ -225,6 +225,40 @@ class Program:
         rt.check(rt.lib().thip_hl_expand_weights(self._h, ctypes.byref(op)))
         return init
 
+    def fma(self, input, weights, scale_bias, *, output_zp, output_min, output_max, shift_factor, init=None,
+            out_dtype=np.int8):
+        """torq_hl.fma, the stand-alone rescale: init = R1(input * weights[0])."""
+        weights = self._as_value(weights)
+        scale_bias = self._as_value(scale_bias)
+        init = self._init_or_new(init, input.shape, out_dtype)
+        op = rt.HlFma(init.index, output_zp, output_min, output_max, shift_factor, weights.index, scale_bias.index,
+                      input.index)
+        rt.check(rt.lib().thip_hl_fma(self._h, ctypes.byref(op)))
+        return init
+
+    def mul(self, input1, input2, scale_bias, *, output_zp, output_min, output_max, shift, init=None,
+            out_dtype=np.int8):
+        """torq_hl.mul: init = R1(input1 * input2); an input of one element is broadcast."""
+        input1 = self._as_value(input1)
+        input2 = self._as_value(input2)
+        scale_bias = self._as_value(scale_bias)
+        shape = input1.shape if int(np.prod(input1.shape)) >= int(np.prod(input2.shape)) else input2.shape
+        init = self._init_or_new(init, shape, out_dtype)
+        op = rt.HlMul(init.index, output_zp, output_min, output_max, scale_bias.index, shift, input1.index,
+                      input2.index)
+        rt.check(rt.lib().thip_hl_mul(self._h, ctypes.byref(op)))
+        return init
+
+    def act(self, input, name, *, min_int=0, max_int=0, min_fp=0.0, max_fp=0.0, input_zp=0, output_zp=0, init=None,
+            out_dtype=None, weights=None):
+        """torq_hl.act on integers: name in clamp / abs / negate / i2i."""
+        init = self._init_or_new(init, input.shape, input.dtype if out_dtype is None else out_dtype)
+        w = rt.NO_VALUE if weights is None else self._as_value(weights).index
+        op = rt.HlAct(init.index, name.encode(), input_zp, output_zp, int(min_int), int(max_int), min_fp, max_fp,
+                      input.index, w)
+        rt.check(rt.lib().thip_hl_act(self._h, ctypes.byref(op)))
+        return init
+
     def transpose(self, input, perm, init=None):
         shape = tuple(input.shape[p] for p in perm)
         init = self._init_or_new(init, shape, input.dtype)

@@ -355,6 +355,69 @@ def add_workload(N=1, H=56, W=56, C=24, zp0=-3, zp1=7, m0=0.71838506, m1=1.3 * 0
                     attrs)
 
 
+_INT_RANGE = {np.dtype(np.int8): (-128, 127), np.dtype(np.int16): (-32768, 32767), np.dtype(np.int32): (-2 ** 31, 2 ** 31 - 1)}
+
+
+def _random_ints(rng, shape, dtype, limit=None):
+    lo, hi = _INT_RANGE[np.dtype(dtype)]
+    if limit is not None:
+        lo, hi = max(lo, -limit), min(hi, limit)
+    return rng.integers(lo, hi, size=shape, endpoint=True, dtype=np.int64).astype(dtype)
+
+
+def fma_workload(shape=(1, 56, 56, 24), in_dtype=np.int8, out_dtype=np.int8, input_zp=-3, scale=0.37, output_zp=5, weight=1, seed=1016):
+    """Stand-alone rescale (tosa.rescale -> torq_hl.fma): weight 1, bias = -input_zp, TFLite multiplier / shift."""
+    rng = np.random.default_rng(seed)
+    x = _random_ints(rng, shape, in_dtype, limit=1 << 20)
+    mult, sh = quantize_multiplier(scale)
+    sb = np.array([-input_zp, int(mult)], dtype=np.int32)
+    lo, hi = _INT_RANGE[np.dtype(out_dtype)]
+    attrs = dict(output_zp=output_zp, output_min=lo, output_max=hi, shift_factor=int(sh))
+    wts = np.array([weight], dtype=np.int8)
+    p = Program()
+    inp = p.binding(0, x.shape, in_dtype)
+    out = p.binding(1, x.shape, out_dtype)
+    p.fma(inp, wts, sb, init=out, **attrs)
+    attrs.update(weights=wts, scale_bias=sb, out_dtype=out_dtype)
+    nbytes = x.nbytes + x.size * np.dtype(out_dtype).itemsize
+    return Workload("fma_%s_%s_%d" % (np.dtype(in_dtype).name, np.dtype(out_dtype).name, x.size), p, [x], [(x.shape, out_dtype)], 2 * x.size, nbytes, attrs)
+
+
+def mul_workload(shape=(1, 56, 56, 24), in_dtype=np.int8, out_dtype=np.int8, scale=0.011, output_zp=-4, bias=0, broadcast=0, seed=1017):
+    """Quantised multiply: inputs already zero-point free; one multiplier / shift.  broadcast 1 / 2: that input has one element."""
+    rng = np.random.default_rng(seed)
+    a = _random_ints(rng, (1,) if broadcast == 1 else shape, in_dtype)
+    b = _random_ints(rng, (1,) if broadcast == 2 else shape, in_dtype)
+    mult, sh = quantize_multiplier(scale)
+    sb = np.array([bias, int(mult)], dtype=np.int32)
+    lo, hi = _INT_RANGE[np.dtype(out_dtype)]
+    attrs = dict(output_zp=output_zp, output_min=lo, output_max=hi, shift=int(sh))
+    p = Program()
+    i0 = p.binding(0, a.shape, in_dtype)
+    i1 = p.binding(1, b.shape, in_dtype)
+    out = p.binding(2, shape, out_dtype)
+    p.mul(i0, i1, sb, init=out, **attrs)
+    attrs.update(scale_bias=sb, out_dtype=out_dtype)
+    count = int(np.prod(shape))
+    nbytes = a.nbytes + b.nbytes + count * np.dtype(out_dtype).itemsize
+    return Workload("mul_%s_%s_%d_b%d" % (np.dtype(in_dtype).name, np.dtype(out_dtype).name, count, broadcast), p, [a, b], [(shape, out_dtype)], 3 * count, nbytes, attrs)
+
+
+def act_workload(name="clamp", shape=(1, 56, 56, 24), in_dtype=np.int8, out_dtype=None, min_int=-20, max_int=90, seed=1018):
+    """torq_hl.act on integers: clamp / abs / negate / i2i."""
+    rng = np.random.default_rng(seed)
+    out_dtype = in_dtype if out_dtype is None else out_dtype
+    x = _random_ints(rng, shape, in_dtype)
+    x.reshape(-1)[:2] = _INT_RANGE[np.dtype(in_dtype)]  # the extremes: abs / negate of the most negative value saturate
+    p = Program()
+    inp = p.binding(0, x.shape, in_dtype)
+    out = p.binding(1, x.shape, out_dtype)
+    p.act(inp, name, min_int=min_int, max_int=max_int, init=out)
+    attrs = dict(name=name, min_int=min_int, max_int=max_int, out_dtype=out_dtype)
+    nbytes = x.nbytes + x.size * np.dtype(out_dtype).itemsize
+    return Workload("act_%s_%s_%s_%d" % (name, np.dtype(in_dtype).name, np.dtype(out_dtype).name, x.size), p, [x], [(x.shape, out_dtype)], x.size, nbytes, attrs)
+
+
 # ---------------------------------------------------------------------------------------------
 # MobileNetV2-1.0 int8 (BASELINE config 3)
 # ---------------------------------------------------------------------------------------------
