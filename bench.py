@@ -68,7 +68,7 @@ def workload_table(pkg):
 
 
 def network_table(pkg):
-    """Whole-network workloads (BASELINE config 3); selectable with --workload, reported as images/s."""
+    """Whole-network workloads (benchmark configuration 3); selectable with --workload, reported as images/s."""
     w = pkg.workloads
     return {"mbv2_b%d" % b: (lambda b=b: w.mobilenet_v2_workload(batch=b), "mfma") for b in (1, 32, 256)}
 

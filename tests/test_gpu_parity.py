@@ -32,7 +32,7 @@ def check(device, wl, via="host", kernel=None):
 
 # ---- conv2d ---------------------------------------------------------------------------------
 def test_conv2d_config0_literal(device):
-    """BASELINE config 0 with its literal (saturating) requant ranges."""
+    """benchmark configuration 0 with its literal (saturating) requant ranges."""
     check(device, w.conv2d_workload(), kernel="igemm_i8")
 
 
@@ -63,7 +63,7 @@ def test_conv2d_every_tile_variant(device, variant, monkeypatch):
     check(device, w.fully_connected_workload(300, 192, 520, realistic=True))
 
 
-@pytest.mark.parametrize("variant", [4, 5, 6, 7, 8, 9, 10])
+@pytest.mark.parametrize("variant", [4, 5, 6, 7, 8, 9, 10, 12, 13])
 def test_dense_igemm_every_tile_variant(device, variant, monkeypatch):
     """The LDS-DMA kernel: whole tiles, ragged M / N / K tails, K shorter than the stage ring."""
     monkeypatch.setenv("THIP_IGEMM_DENSE_VARIANT", str(variant))
@@ -76,7 +76,7 @@ def test_dense_igemm_every_tile_variant(device, variant, monkeypatch):
     check(device, w.conv2d_workload(N=2, H=28, W=28, C=192, O=32, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True))
 
 
-@pytest.mark.parametrize("variant", [4, 7, 9])
+@pytest.mark.parametrize("variant", [4, 7, 9, 13])
 def test_dense_igemm_staged_epilogue(device, variant, monkeypatch):
     """The LDS-staged epilogue with the 32-bit requant tail (the in-register one normally takes these shapes)."""
     monkeypatch.setenv("THIP_IGEMM_DENSE_VARIANT", str(variant))
@@ -265,7 +265,7 @@ def test_padded_channel_chain(device, nhwc):
 
 @pytest.mark.parametrize("batch", [1, 3])
 def test_mobilenet_v2_full(device, batch):
-    """BASELINE config 3: the whole 64-op network as one program, final logits bit-exact."""
+    """benchmark configuration 3: the whole 64-op network as one program, final logits bit-exact."""
     wl = w.mobilenet_v2_workload(batch=batch)
     announce(wl.name)
     got, kernels = run_on_gpu(device, wl, via="device")

@@ -414,8 +414,10 @@ class Emitter {
                 return N <= 32 ? kIgemmDense256x32 : N <= 64 ? kIgemmDense256x64 : kIgemmDense256x128;
             }
             // otherwise the largest tile that still gives (nearly) every CU a tile
-            const uint32_t order[] = {kIgemmDense256x256, kIgemmDense128x256, kIgemmDense128x128};
+            const uint32_t order[] = {kIgemmDense256x256, kIgemmDense128x256, kIgemmDense128x128, kIgemmDense64x128};
             for (uint32_t v : order) {
+                // the wide-N tile only where N nearly fills whole tiles (padded columns are computed too)
+                if (v == kIgemmDense64x128 && ((roundUp(N, 128) - N) * 8 > N || getenv("THIP_NO_64X128"))) continue;
                 if (tiles(v) >= 224) return v;
             }
             return kIgemmDense64x64;

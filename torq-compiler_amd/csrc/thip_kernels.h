@@ -56,7 +56,9 @@ enum IgemmVariant : uint32_t {
     kIgemmDense256x32 = 10,
     // dense operand, weights of at most 64 KiB resident in LDS, N <= 256, int8 output: streams the pixels
     kIgemmStream = 11,
-    kIgemmVariantCount = 12,
+    kIgemmDense128x64 = 12,  // mid-sized problems: enough tiles to fill the chip at a better ratio of loads to MFMAs than 64x64
+    kIgemmDense64x128 = 13,
+    kIgemmVariantCount = 14,
 };
 struct IgemmTile {
     int bm, bn, bk;

@@ -669,7 +669,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
     // waves) is loaded redundantly, several waves writing the same bytes to the same place
     static_assert(BM % (16 * NW) == 0 && BN % 16 == 0 && (BWL % NW == 0 || BWL < NW), "unbalanced DMA loads");
     static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the MFMA tile");
-    static_assert(STAGES >= 2 && STAGES <= 5 && LPT * (STAGES - 1) < 64, "vmcnt is a 6-bit counter");
+    static_assert(STAGES >= 2 && STAGES <= 8 && LPT * (STAGES - 1) < 64, "vmcnt is a 6-bit counter");
 
     extern __shared__ __align__(16) int8_t smem[];
     const unsigned ldsBase = (unsigned)(uintptr_t)(__attribute__((address_space(3))) int8_t *)smem;
@@ -819,7 +819,13 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
             waitVmcnt<LPT *(STAGES - 2)>();
         } else if (more) {
             const int inFlight = (KT - 2 - kt) < (STAGES - 2) ? (KT - 2 - kt) : (STAGES - 2);
-            if (inFlight >= 3) {
+            if (inFlight >= 6) {
+                waitVmcnt<(LPT * 6 < 64 ? LPT * 6 : 0)>();
+            } else if (inFlight == 5) {
+                waitVmcnt<(LPT * 5 < 64 ? LPT * 5 : 0)>();
+            } else if (inFlight == 4) {
+                waitVmcnt<(LPT * 4 < 64 ? LPT * 4 : 0)>();
+            } else if (inFlight == 3) {
                 waitVmcnt<LPT * 3>();
             } else if (inFlight == 2) {
                 waitVmcnt<LPT * 2>();
@@ -1063,6 +1069,8 @@ static const IgemmTile kTiles[kIgemmVariantCount] = {
     {256, 64, 64, "igemm_dense_i8_256x64x64"},
     {256, 32, 64, "igemm_dense_i8_256x32x64"},
     {32, 32, 32, "igemm_stream_i8"},
+    {128, 64, 64, "igemm_dense_i8_128x64x64"},
+    {64, 128, 64, "igemm_dense_i8_64x128x64"},
 };
 
 const IgemmTile &igemmTile(uint32_t variant) {
@@ -1178,6 +1186,8 @@ hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, hipStream_t stream)
     case kIgemmDense256x64: return launchIgemmDense<256, 64, 4, 1, 3, 2>(a, stream);
     case kIgemmDense256x32: return launchIgemmDense<256, 32, 4, 1, 3, 2>(a, stream);
     case kIgemmStream: return launchIgemmStream(a, stream);
+    case kIgemmDense128x64: return launchIgemmDense<128, 64, 2, 2, 4, 2>(a, stream);
+    case kIgemmDense64x128: return launchIgemmDense<64, 128, 2, 2, 4, 2>(a, stream);
     default: return hipErrorInvalidValue;
     }
 }

@@ -55,7 +55,7 @@ def random_requant(rng, channels, realistic):
 def conv2d_workload(N=1, H=112, W=112, C=32, O=64, KH=3, KW=3, stride=(1, 1), pad=(1, 1, 1, 1),
                     input_zp=-3, output_zp=5, output_min=5, output_max=127, realistic=False,
                     nhwc=True, seed=1000):
-    """BASELINE config 0 by default: NHWC 1x112x112x32 -> 1x112x112x64, 3x3, SAME."""
+    """benchmark configuration 0 by default: NHWC 1x112x112x32 -> 1x112x112x64, 3x3, SAME."""
     rng = np.random.default_rng(seed)
     x = rng.integers(-128, 127, size=(N, H, W, C), endpoint=True, dtype=np.int8)
     w_hwio = rng.integers(-127, 127, size=(KH, KW, C, O), endpoint=True, dtype=np.int8)
@@ -83,7 +83,7 @@ def conv2d_workload(N=1, H=112, W=112, C=32, O=64, KH=3, KW=3, stride=(1, 1), pa
 
 def fully_connected_workload(M, K, N, realistic=False, output_zp=5, output_min=-128, output_max=127,
                              seed=1001, shift=None):
-    """BASELINE config 1: int8 [M,K] x [N,K]^T with per-column requant.
+    """benchmark configuration 1: int8 [M,K] x [N,K]^T with per-column requant.
 
     `shift` forces one shift_factor for every column (multipliers drawn so that outputs still spread)."""
     rng = np.random.default_rng(seed)
@@ -265,7 +265,7 @@ def add_bf16_workload(shape=(1, 32, 1152), w0=1.0, w1=1.0, bias=0.0, clamp=None,
 
 def depthwise_workload(N=1, H=56, W=56, C=144, KH=3, KW=3, stride=(2, 2), pad=(0, 1, 0, 1), input_zp=-3,
                        output_zp=5, output_min=-128, output_max=127, realistic=True, nhwc=True, seed=1002):
-    """BASELINE config 2a: depthwise 3x3 stride 2 SAME on 56x56x144."""
+    """benchmark configuration 2a: depthwise 3x3 stride 2 SAME on 56x56x144."""
     rng = np.random.default_rng(seed)
     x = rng.integers(-128, 127, size=(N, H, W, C), endpoint=True, dtype=np.int8)
     w = rng.integers(-127, 127, size=(C, 1, KH, KW), endpoint=True, dtype=np.int8)
@@ -294,7 +294,7 @@ def depthwise_workload(N=1, H=56, W=56, C=144, KH=3, KW=3, stride=(2, 2), pad=(0
 
 def maxpool_workload(N=1, H=112, W=112, C=64, kernel=(2, 2), stride=(2, 2), pad=(0, 0, 0, 0), input_zp=-128,
                      nhwc=True, seed=1003):
-    """BASELINE config 2b: maxpool 2x2 stride 2 on 112x112x64."""
+    """benchmark configuration 2b: maxpool 2x2 stride 2 on 112x112x64."""
     rng = np.random.default_rng(seed)
     x = rng.integers(-128, 127, size=(N, H, W, C), endpoint=True, dtype=np.int8)
     attrs = dict(input_zp=input_zp, output_min=-128, output_max=127, stride=tuple(stride), pad=tuple(pad),
@@ -314,7 +314,7 @@ def maxpool_workload(N=1, H=112, W=112, C=64, kernel=(2, 2), stride=(2, 2), pad=
 
 
 def avgpool_workload(N=1, H=7, W=7, C=1280, input_zp=-3, output_zp=5, seed=1004):
-    """BASELINE config 2c: global average pool on 7x7x1280 (NHWC), scale = floor(2^20 / 49)."""
+    """benchmark configuration 2c: global average pool on 7x7x1280 (NHWC), scale = floor(2^20 / 49)."""
     rng = np.random.default_rng(seed)
     x = rng.integers(-128, 127, size=(N, H, W, C), endpoint=True, dtype=np.int8)
     # compiler/torq/Conversions/LinalgToTorqHL/PoolingPattern.cpp:325-328
@@ -339,7 +339,7 @@ def add_params(m0, m1, zp0, zp1, sign=1):
 
 
 def add_workload(N=1, H=56, W=56, C=24, zp0=-3, zp1=7, m0=0.71838506, m1=1.3 * 0.5, output_zp=-2, seed=1005):
-    """BASELINE config 2d: quantised add of two 56x56x24 tensors with distinct zero points and scales."""
+    """benchmark configuration 2d: quantised add of two 56x56x24 tensors with distinct zero points and scales."""
     rng = np.random.default_rng(seed)
     a = rng.integers(-128, 127, size=(N, H, W, C), endpoint=True, dtype=np.int8)
     b = rng.integers(-128, 127, size=(N, H, W, C), endpoint=True, dtype=np.int8)
@@ -419,7 +419,7 @@ def act_workload(name="clamp", shape=(1, 56, 56, 24), in_dtype=np.int8, out_dtyp
 
 
 # ---------------------------------------------------------------------------------------------
-# MobileNetV2-1.0 int8 (BASELINE config 3)
+# MobileNetV2-1.0 int8 (benchmark configuration 3)
 # ---------------------------------------------------------------------------------------------
 MBV2_BLOCKS = [(1, 16, 1, 1), (6, 24, 2, 2), (6, 32, 3, 2), (6, 64, 4, 2), (6, 96, 3, 1), (6, 160, 3, 2), (6, 320, 1, 1)]
 
@@ -546,7 +546,7 @@ def mobilenet_v2_layers(resolution=224, classes=1000, seed=1006, width=1.0):
 
 
 def mobilenet_v2_workload(batch=1, resolution=224, classes=1000, seed=1006, nhwc=True, width=1.0):
-    """BASELINE config 3 as ONE program: 52 convs, 17 depthwise, 10 adds, global average pool, FC.
+    """benchmark configuration 3 as ONE program: 52 convs, 17 depthwise, 10 adds, global average pool, FC.
 
     nhwc=True declares every tensor N,H,W,C (the layout the kernels run); nhwc=False declares the ops
     N,C,H,W as the reference's patterns emit them, with the torq_hl.transpose the reference places in
