@@ -272,6 +272,23 @@ def test_gpu_bf16_conv2d_and_depthwise(device):
 
 
 @pytest.mark.gpu
+def test_gpu_bf16_wide_n(device):
+    """A vocabulary-sized N with a short K: every wave streams its own columns through two register buffers
+    (bf16 weights, block-quantized weights with and without the expansion clamp, ragged N and K, two row tiles)."""
+    for wl in [w.fully_connected_bf16_workload(3, 200, 32800), w.fully_connected_bf16_workload(40, 1152, 32768, clamp=(-0.5, 0.75))]:
+        _check_gpu(device, wl, via="device")
+    f = lambda bits: np.abs(orc.from_bf16(bits).astype(np.float64))
+    for wl in [w.expand_weights_workload(M=5, K=192, N=32808, block=64), w.expand_weights_workload(M=33, K=1152, N=32768, block=128),
+               w.expand_weights_workload(M=2, K=320, N=32768, block=32, expand_clamp=(-0.002, 0.003))]:
+        print("[gpu-case]", wl.name, flush=True)
+        got, kernels = run_on_gpu(device, wl, via="device")
+        w16 = orc.expand_weights(wl.attrs["weights"], wl.attrs["scale"], wl.attrs["qbias"], block_size=wl.attrs["block"],
+                                 output_min=wl.attrs["expand_min"], output_max=wl.attrs["expand_max"])
+        assert_bf16_close(got[0], oracle_eval(wl)[0].reshape(got[0].shape), wl.name, magnitude=f(wl.inputs[0]) @ f(w16))
+        assert kernels == ["fc_bf16"], kernels
+
+
+@pytest.mark.gpu
 def test_gpu_bf16_avg_pool(device):
     """The kernel walks the frame in the oracle's order: bit-exact."""
     for wl in [w.avg_pool2d_bf16_workload(), w.avg_pool2d_bf16_workload(N=64), w.avg_pool2d_bf16_workload(N=3, H=5, W=4, C=7, weight=1.0, clamp=(-1.0, 1.0)),

@@ -2179,6 +2179,32 @@ __device__ __forceinline__ void expandQ8(int d, float sc, float bi, float lo, fl
     *o1 = __builtin_bit_cast(int, __builtin_convertvector((v2f){f[2], f[3]}, v2bf));
 }
 
+// Bias, clamp, round to bf16 and store one 32 x 32 accumulator tile: register 4 q + e of lane (r, h) is
+// out[m0 + r][n0 + 8 q + 4 h + e].
+__device__ __forceinline__ void fcBf16Store(const FcBf16Args &p, const v16f &acc, int m0, int n0, int r, int h) {
+    const int m = m0 + r;
+    if (m >= p.M) return;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int n = n0 + 8 * q + 4 * h;
+        uint16_t o[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int ne = n + e < p.N ? n + e : p.N - 1;
+            const float t0 = acc[4 * q + e] + p.bias[ne];
+            o[e] = bf16Bits(t0 < p.lo ? p.lo : (t0 > p.hi ? p.hi : t0));
+        }
+        if ((p.N & 3) == 0 && n + 3 < p.N) {
+            *(v2i *)(p.out + (size_t)m * p.N + n) = v2i{(int)((uint32_t)o[0] | ((uint32_t)o[1] << 16)), (int)((uint32_t)o[2] | ((uint32_t)o[3] << 16))};
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                if (n + e < p.N) p.out[(size_t)m * p.N + n + e] = o[e];
+            }
+        }
+    }
+}
+
 template <int NWAVES, int Q8>  // waves of a block = ways K is split; Q8: 0 bf16 weights, 1 int8 expanded, 2 with clamp
 __global__ __launch_bounds__(NWAVES * 64) void fc_bf16(FcBf16Args p, FastDiv qblk) {
     __shared__ float partial[NWAVES - 1][16][64];
@@ -2202,22 +2228,22 @@ __global__ __launch_bounds__(NWAVES * 64) void fc_bf16(FcBf16Args p, FastDiv qbl
     for (int s0 = sBeg; s0 < sEnd; s0 += UNR) {
         v4i wv[Q8 ? 1 : UNR][4], xv[UNR][4];
         v4i wq[Q8 ? UNR : 1][2];
-        float qs[Q8 ? UNR : 1], qb[Q8 ? UNR : 1];
+        uint16_t qs[Q8 ? UNR : 1];  // raw bf16 bits: converting here would wait for the load, and for every older one
+        float qb[Q8 ? UNR : 1];
 #pragma unroll
         for (int u = 0; u < UNR; u++) {
             const int k = (s0 + u) * 64 + 32 * h;
             if (Q8) {
-                // the lane's 32 weights of this step lie in one block: one scale, one bias
-                const bool live = s0 + u < sEnd;
-                const size_t g = fastDiv((uint32_t)(live && k < p.K ? k : 0), qblk);  // beyond K the input rows are zero
-                qs[u] = __uint_as_float((uint32_t)p.qscale[g * p.qcols + n0 + r] << 16);
+                // the lane's 32 weights of this step lie in one block: one scale, one bias.  Loads only, no branch:
+                // a step past the end re-reads the last one and meets zero input rows
+                const int sq = s0 + u < sEnd ? s0 + u : sEnd - 1, kq = sq * 64 + 32 * h;
+                const size_t g = fastDiv((uint32_t)(kq < p.K ? kq : 0), qblk);  // beyond K the input rows are zero
+                qs[u] = p.qscale[g * p.qcols + n0 + r];
                 qb[u] = p.qbias[g * p.qcols + n0 + r];
 #pragma unroll
                 for (int h2 = 0; h2 < 2; h2++) {
-                    const int8_t *frag = (const int8_t *)p.w + ((((size_t)blockIdx.x * steps + (s0 + u)) * 2 + h2) * 64 + lane) * 16;
-                    wq[u][h2] = live ? *(const v4i *)frag : v4i{0, 0, 0, 0};
+                    wq[u][h2] = *(const v4i *)((const int8_t *)p.w + ((((size_t)blockIdx.x * steps + sq) * 2 + h2) * 64 + lane) * 16);
                 }
-                if (!live) qs[u] = qb[u] = 0.0f;  // a step past the end multiplies zeros
             }
 #pragma unroll
             for (int c = 0; c < 4; c++) {
@@ -2241,8 +2267,9 @@ __global__ __launch_bounds__(NWAVES * 64) void fc_bf16(FcBf16Args p, FastDiv qbl
                 if (Q8) {
                     // piece c = bytes 8 (c & 1) .. + 7 of half c >> 1; the k rows beyond K are zero in the input
                     int o[4];
-                    expandQ8<Q8 == 2>(wq[u][c >> 1][2 * (c & 1)], qs[u], qb[u], p.qlo, p.qhi, &o[0], &o[1]);
-                    expandQ8<Q8 == 2>(wq[u][c >> 1][2 * (c & 1) + 1], qs[u], qb[u], p.qlo, p.qhi, &o[2], &o[3]);
+                    const float sc = __uint_as_float((uint32_t)qs[u] << 16);
+                    expandQ8<Q8 == 2>(wq[u][c >> 1][2 * (c & 1)], sc, qb[u], p.qlo, p.qhi, &o[0], &o[1]);
+                    expandQ8<Q8 == 2>(wq[u][c >> 1][2 * (c & 1) + 1], sc, qb[u], p.qlo, p.qhi, &o[2], &o[3]);
                     wpiece = v4i{o[0], o[1], o[2], o[3]};
                 } else {
                     wpiece = wv[u][c];
@@ -2286,27 +2313,119 @@ __global__ __launch_bounds__(NWAVES * 64) void fc_bf16(FcBf16Args p, FastDiv qbl
         }
         if (lane == 0) counters[tile] = 0;
     }
-    const int m = m0 + r;
-    if (m >= p.M) return;
+    fcBf16Store(p, acc, m0, n0, r, h);
+}
+
+// fc_bf16_wide: the same product for a very wide N and a short K (a vocabulary projection): a wave owns a
+// column block for the whole of K, so nothing is reduced across waves, and it streams the weights through two
+// register buffers, the loads of one in flight while the other feeds the MFMAs.  The input rows of the block
+// (at most 32, and one slot of zeros for the lanes of rows it does not have) sit in LDS in fragment order, read
+// 16 bytes per lane right before each MFMA: with few rows that is a few KiB, and registers set the occupancy.
+// Weights in fragment order only (layouts 1 and 2).
+constexpr int kFcBf16WideMaxSteps = 24;  // 99 KiB of LDS for 32 input rows
+template <int Q8, int U>  // U: k-steps per register buffer
+__global__ __launch_bounds__(256) void fc_bf16_wide(FcBf16Args p, FastDiv qblk) {
+    extern __shared__ __attribute__((aligned(16))) int8_t xs[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 31, h = lane >> 5;
+    const int steps = (p.K + 63) / 64;
+    const int m0 = blockIdx.y * 32;
+    // rows the block really has, plus one slot of zeros that the lanes of the missing rows all read
+    const int mt = p.M - m0 < 32 ? p.M - m0 : 32, slots = 2 * (mt + 1);
+    for (int i = threadIdx.x; i < steps * 4 * slots; i += 256) {
+        const int slot = i % slots, sc = i / slots, c = sc & 3, s = sc >> 2;
+        const int hh = slot / (mt + 1), rr = slot - hh * (mt + 1);
+        const int k = s * 64 + 32 * hh + 8 * c;
+        v4i v = {0, 0, 0, 0};
+        if (rr < mt && k < p.K) v = *(const v4i *)(p.x + (size_t)(m0 + rr) * p.K + k);
+        *(v4i *)(xs + (size_t)i * 16) = v;
+    }
+    __syncthreads();
+    const int xslot = (h * (mt + 1) + (r < mt ? r : mt)) * 16;
+    const int nb = blockIdx.x * 4 + wave;
+    if (nb >= (p.N + 31) / 32) return;
+    const int n0 = nb * 32;
+    constexpr int PIECES = Q8 ? 2 : 4;  // 16-byte loads per lane per step
+    const int8_t *wbase = (const int8_t *)p.w + (size_t)nb * steps * (PIECES * 1024) + lane * 16;
+    struct Buf {
+        v4i w[U][PIECES];
+        uint16_t qs[U];  // raw bf16 bits: converting here would wait for the load, and with it for every older one
+        float qb[U];
+    };
+    // Loads only, no use of a loaded value and no branch: the steps past the end re-read the last one (never used).
+    auto loadGroup = [&](int s0, Buf &b) {
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-        const int n = n0 + 8 * q + 4 * h;
-        uint16_t o[4];
+        for (int u = 0; u < U; u++) {
+            const int s = s0 + u < steps ? s0 + u : steps - 1;
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const int ne = n + e < p.N ? n + e : p.N - 1;
-            const float t0 = acc[4 * q + e] + p.bias[ne];
-            o[e] = bf16Bits(t0 < p.lo ? p.lo : (t0 > p.hi ? p.hi : t0));
-        }
-        if ((p.N & 3) == 0 && n + 3 < p.N) {
-            *(v2i *)(p.out + (size_t)m * p.N + n) = v2i{(int)((uint32_t)o[0] | ((uint32_t)o[1] << 16)), (int)((uint32_t)o[2] | ((uint32_t)o[3] << 16))};
-        } else {
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                if (n + e < p.N) p.out[(size_t)m * p.N + n + e] = o[e];
+            for (int c = 0; c < PIECES; c++) b.w[u][c] = *(const v4i *)(wbase + ((size_t)s * PIECES + c) * 1024);
+            if (Q8) {
+                const int k = s * 64 + 32 * h;
+                const size_t g = fastDiv((uint32_t)(k < p.K ? k : 0), qblk);  // beyond K the input rows are zero
+                b.qs[u] = p.qscale[g * p.qcols + n0 + r];
+                b.qb[u] = p.qbias[g * p.qcols + n0 + r];
             }
         }
+    };
+    v16f acc;
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[e] = 0.0f;
+    auto compute = [&](int s0, const Buf &b) {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int s = s0 + u;
+            if (s >= steps) break;
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const v4i xpiece = *(const v4i *)(xs + (size_t)(s * 4 + c) * slots * 16 + xslot);
+                v4i wpiece;
+                if (Q8) {
+                    int o[4];
+                    const float sc = __uint_as_float((uint32_t)b.qs[u] << 16);
+                    expandQ8<Q8 == 2>(b.w[u][c >> 1][2 * (c & 1)], sc, b.qb[u], p.qlo, p.qhi, &o[0], &o[1]);
+                    expandQ8<Q8 == 2>(b.w[u][c >> 1][2 * (c & 1) + 1], sc, b.qb[u], p.qlo, p.qhi, &o[2], &o[3]);
+                    wpiece = v4i{o[0], o[1], o[2], o[3]};
+                } else {
+                    wpiece = b.w[u][c & (PIECES - 1)];
+                }
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, wpiece), __builtin_bit_cast(v8bf, xpiece), acc, 0, 0, 0);
+            }
+        }
+    };
+    Buf b0, b1;
+    loadGroup(0, b0);
+    for (int s0 = 0; s0 < steps; s0 += 2 * U) {
+        loadGroup(s0 + U, b1);
+        compute(s0, b0);
+        loadGroup(s0 + 2 * U, b0);
+        compute(s0 + U, b1);
     }
+    fcBf16Store(p, acc, m0, n0, r, h);
+}
+
+template <int Q8, int U>
+static hipError_t launchFcBf16WideU(const FcBf16Args &a, FastDiv blk, hipStream_t stream) {
+    auto kernel = fc_bf16_wide<Q8, U>;
+    static bool configured = false;
+    if (!configured) {
+        hipError_t err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kFcBf16WideMaxSteps * 4 * 66 * 16);
+        if (err != hipSuccess) return err;
+        configured = true;
+    }
+    const int steps = (a.K + 63) / 64, nblocks = (a.N + 31) / 32;
+    const dim3 grid((unsigned)((nblocks + 3) / 4), (unsigned)((a.M + 31) / 32));
+    const int mt = a.M < 32 ? a.M : 32;
+    hipLaunchKernelGGL(kernel, grid, dim3(256), (size_t)steps * 4 * 2 * (mt + 1) * 16, stream, a, blk);
+    return hipGetLastError();
+}
+
+template <int Q8>
+static hipError_t launchFcBf16Wide(const FcBf16Args &a, FastDiv blk, hipStream_t stream) {
+    const char *e = getenv("THIP_FC_WIDE_U");
+    const int u = e ? atoi(e) : (Q8 ? 4 : 2);
+    if (u == 8 && Q8) return launchFcBf16WideU<Q8, 8>(a, blk, stream);
+    if (u == 4) return launchFcBf16WideU<Q8, 4>(a, blk, stream);
+    return launchFcBf16WideU<Q8, Q8 ? 4 : 2>(a, blk, stream);
 }
 
 hipError_t launchFcBf16(const FcBf16Args &a, hipStream_t stream) {
@@ -2315,15 +2434,20 @@ hipError_t launchFcBf16(const FcBf16Args &a, hipStream_t stream) {
     if (a.ksplit < 1 || a.ksplit > 64 || (a.ksplit > 1 && (!a.workspace || ((uintptr_t)a.workspace & 255)))) return hipErrorInvalidValue;
     const dim3 grid((unsigned)((a.N + 31) / 32), (unsigned)((a.M + 31) / 32), (unsigned)a.ksplit);
     if (grid.y > 65535) return hipErrorInvalidValue;
+    // a very wide N with a short K and no K split: every wave streams its own columns (THIP_NO_FC_WIDE: off)
+    const bool wide = a.w_fragments >= 1 && a.ksplit == 1 && (a.K + 63) / 64 <= kFcBf16WideMaxSteps && (a.N + 31) / 32 >= 1024 &&
+                      !getenv("THIP_NO_FC_WIDE");
     if (a.w_fragments == 2) {
         if (!a.qscale || !a.qbias || a.qblock < 32 || a.qblock % 32 != 0 || a.qcols < (a.N + 31) / 32 * 32 || a.qcols % 32 != 0) return hipErrorInvalidValue;
         if ((((uintptr_t)a.qscale) & 1) || (((uintptr_t)a.qbias) & 3)) return hipErrorInvalidValue;
         const FastDiv blk = makeFastDiv((uint32_t)a.qblock);
         const bool clamp = !(a.qlo == -INFINITY && a.qhi == INFINITY);
+        if (wide) return clamp ? launchFcBf16Wide<2>(a, blk, stream) : launchFcBf16Wide<1>(a, blk, stream);
         if (clamp) hipLaunchKernelGGL((fc_bf16<4, 2>), grid, dim3(256), 0, stream, a, blk);
         else hipLaunchKernelGGL((fc_bf16<4, 1>), grid, dim3(256), 0, stream, a, blk);
         return hipGetLastError();
     }
+    if (wide) return launchFcBf16Wide<0>(a, makeFastDiv(1), stream);
     hipLaunchKernelGGL((fc_bf16<4, 0>), grid, dim3(256), 0, stream, a, makeFastDiv(1));
     return hipGetLastError();
 }
