@@ -57,6 +57,7 @@ struct WideRequant {
     int32_t rnd, lo, hi, zp;
     int32_t t0lo, t0hi;  // clamp of acc + bias (the whole int32 range when rq.t0_clamp == 0)
     bool plain;          // on, pre == 0, no clamp of t0, zero point folded: requantWideT0<true> applies
+    bool preOnly;        // on, pre > 0, no clamp of t0, zero point folded: requantPreShift applies
 };
 __device__ __forceinline__ WideRequant wideRequant(const Requant &rq) {
     WideRequant w;
@@ -80,6 +81,7 @@ __device__ __forceinline__ WideRequant wideRequant(const Requant &rq) {
         w.zp = 0;
     }
     w.plain = w.on && w.pre == 0 && rq.t0_clamp <= 0 && w.zp == 0;
+    w.preOnly = w.on && w.pre > 0 && rq.t0_clamp <= 0 && w.zp == 0;
     return w;
 }
 __device__ __forceinline__ int32_t med3(int32_t v, int32_t lo, int32_t hi) {
@@ -96,24 +98,32 @@ __device__ __forceinline__ int32_t requantWideT0(int32_t t0, int32_t scale, cons
     const int32_t t3 = med3((__mulhi(t0, scale) + w.rnd) >> w.shiftMinus32, w.lo, w.hi);  // lo <= hi
     return (int32_t)((uint32_t)t3 + (uint32_t)w.zp);
 }
+// The pre-shifted tail without the clamp of t0 and with the zero point folded (WideRequant::preOnly): what a
+// layer with a shift below 33 and a proven bound on |acc + bias| takes; two instructions shorter than the general one.
+__device__ __forceinline__ int32_t requantPreShift(int32_t t0, int32_t scale, const WideRequant &w) {
+    return med3((__mulhi((int32_t)((uint32_t)t0 << w.pre), scale) + w.rnd) >> w.shiftMinus32, w.lo, w.hi);
+}
 __device__ __forceinline__ int32_t requantWideShift(int32_t acc, int32_t bias, int32_t scale, const WideRequant &w) {
     return requantWideT0<false>((int32_t)((uint32_t)acc + (uint32_t)bias), scale, w);
 }
-// The three requant tails as a compile-time choice made once per kernel: f(tag) with tag::value
-// 0 = generic 64-bit, 1 = 32-bit, 2 = 32-bit plain.
+// The requant tails as a compile-time choice made once per kernel: f(tag) with tag::value
+// 0 = generic 64-bit, 1 = 32-bit general, 2 = 32-bit plain, 3 = 32-bit pre-shifted only.
 template <typename F>
 __device__ __forceinline__ void withRequantMode(const WideRequant &w, F &&f) {
     if (!w.on) {
         f(std::integral_constant<int, 0>{});
-    } else if (!w.plain) {
-        f(std::integral_constant<int, 1>{});
-    } else {
+    } else if (w.plain) {
         f(std::integral_constant<int, 2>{});
+    } else if (w.preOnly) {
+        f(std::integral_constant<int, 3>{});
+    } else {
+        f(std::integral_constant<int, 1>{});
     }
 }
 template <int MODE>
 __device__ __forceinline__ int32_t requantT0(int32_t t0, int32_t scale, long long rnd, const Requant &rq, const WideRequant &w) {
     if (MODE == 0) return requant(t0, 0, scale, rnd, rq);
+    if (MODE == 3) return requantPreShift(t0, scale, w);
     return requantWideT0<MODE == 2>(t0, scale, w);
 }
 // Four requantised values (each within int8 after the clamp) as the bytes of one dword.
