@@ -55,6 +55,7 @@ struct WideRequant {
     bool on;  // rq.shift + rq.pre_shift >= 33
     int pre, shiftMinus32;
     int32_t rnd, lo, hi, zp;
+    long long rnd64;     // rnd * 2^32: added to the 64-bit product, it adds rnd to the product's high word
     int32_t t0lo, t0hi;  // clamp of acc + bias (the whole int32 range when rq.t0_clamp == 0)
     bool plain;          // on, pre == 0, no clamp of t0, zero point folded: requantWideT0<true> applies
     bool preOnly;        // on, pre > 0, no clamp of t0, zero point folded: requantPreShift applies
@@ -80,6 +81,7 @@ __device__ __forceinline__ WideRequant wideRequant(const Requant &rq) {
         w.hi = rq.out_max;
         w.zp = 0;
     }
+    w.rnd64 = (long long)w.rnd * 4294967296LL;  // rnd may be negative (a folded negative zero point)
     w.plain = w.on && w.pre == 0 && rq.t0_clamp <= 0 && w.zp == 0;
     w.preOnly = w.on && w.pre > 0 && rq.t0_clamp <= 0 && w.zp == 0;
     return w;
@@ -89,19 +91,24 @@ __device__ __forceinline__ int32_t med3(int32_t v, int32_t lo, int32_t hi) {
     asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "v"(lo), "v"(hi));
     return r;
 }
+// High word of t0 * scale, plus the rounding term: one v_mad_i64_i32 (full rate) instead of a v_mul_hi_i32 and an
+// add.  |t0 * scale| < 2^62 and rnd * 2^32 < 2^62: the sum cannot overflow.
+__device__ __forceinline__ int32_t mulhiPlusRnd(int32_t t0, int32_t scale, const WideRequant &w) {
+    return (int32_t)(((long long)t0 * (long long)scale + w.rnd64) >> 32);
+}
 // `t0` is acc + bias (with int32 wrap).  PLAIN: no pre-shift, no clamp of t0, zero point folded into the
 // rounding term (WideRequant::plain), which is the usual case and four instructions shorter.
 template <bool PLAIN>
 __device__ __forceinline__ int32_t requantWideT0(int32_t t0, int32_t scale, const WideRequant &w) {
-    if (PLAIN) return med3((__mulhi(t0, scale) + w.rnd) >> w.shiftMinus32, w.lo, w.hi);
+    if (PLAIN) return med3(mulhiPlusRnd(t0, scale, w) >> w.shiftMinus32, w.lo, w.hi);
     t0 = (int32_t)((uint32_t)med3(t0, w.t0lo, w.t0hi) << w.pre);
-    const int32_t t3 = med3((__mulhi(t0, scale) + w.rnd) >> w.shiftMinus32, w.lo, w.hi);  // lo <= hi
+    const int32_t t3 = med3(mulhiPlusRnd(t0, scale, w) >> w.shiftMinus32, w.lo, w.hi);  // lo <= hi
     return (int32_t)((uint32_t)t3 + (uint32_t)w.zp);
 }
 // The pre-shifted tail without the clamp of t0 and with the zero point folded (WideRequant::preOnly): what a
 // layer with a shift below 33 and a proven bound on |acc + bias| takes; two instructions shorter than the general one.
 __device__ __forceinline__ int32_t requantPreShift(int32_t t0, int32_t scale, const WideRequant &w) {
-    return med3((__mulhi((int32_t)((uint32_t)t0 << w.pre), scale) + w.rnd) >> w.shiftMinus32, w.lo, w.hi);
+    return med3(mulhiPlusRnd((int32_t)((uint32_t)t0 << w.pre), scale, w) >> w.shiftMinus32, w.lo, w.hi);
 }
 __device__ __forceinline__ int32_t requantWideShift(int32_t acc, int32_t bias, int32_t scale, const WideRequant &w) {
     return requantWideT0<false>((int32_t)((uint32_t)acc + (uint32_t)bias), scale, w);
