@@ -147,8 +147,17 @@ def run(blob, binding_arrays):
             acc = A @ Wp.T  # M x Np
             q = _requant_vec(acc[:, :N], bias[None, :N], scale[None, :N], sh, zp, mn, mx, int(op["pre_shift"]), int(op["t0_clamp"]))
             odt = OUT_NP[int(op["out_dtype"])]
+            res = q.astype(odt).reshape(-1)
+            if kind == K_IGEMM and int(op["in1"]["space"]) != 0:
+                # a residual add folded into the epilogue: the other operand from in1, the add's parameters from `table`
+                assert int(op["variant"]) == 11 and int(op["loader"]) == 0 and odt == np.int8
+                ap = view(op["table"], 48).view(np.int32)
+                other = view(op["in1"], M * N).view(np.int8)
+                a, b = (other, res) if int(ap[8]) else (res, other)
+                res = orc.add(a, b, np.array([ap[0], ap[1]], dtype=np.int16), np.array([ap[2], ap[3]], dtype=np.int32), output_zp=int(ap[5]),
+                              output_min=int(ap[6]), output_max=int(ap[7]), shift_factor=int(ap[4]))
             out = view(op["out"], M * N * np.dtype(odt).itemsize).view(odt)
-            out[:] = q.astype(odt).reshape(-1)
+            out[:] = res
         elif kind == K_DW:
             Nimg, H, W, C, OH, OW = (int(op[k]) for k in ["N", "H", "W", "C", "OH", "OW"])
             KH, KW = int(op["KH"]), int(op["KW"])

@@ -26,6 +26,11 @@ def oracle_eval(wl):
         fn = orc.conv2d_bf16 if kind == "convbf16" else orc.depthwise_conv2d_bf16
         return [fn(x, a["weights"], a["bias"], pad=a["pad"], stride=a["stride"], output_min=a["output_min"], output_max=a["output_max"],
                    layout=orc.NHWC if a["nhwc"] else orc.NCHW)]
+    if kind == "pwadd":
+        wp, sbp, pa = a["pw"]
+        aw, asb, aa = a["add"]
+        y = orc.conv2d(x, wp, sbp, layout=orc.NHWC, **pa)
+        return [orc.add(wl.inputs[1], y, aw, asb, **aa) if a["other_first"] else orc.add(y, wl.inputs[1], aw, asb, **aa)]
     if kind == "fma":
         return [orc.fma(x, a.pop("weights"), a.pop("scale_bias"), **a)]
     if kind == "mul":

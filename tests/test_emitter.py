@@ -333,3 +333,34 @@ def test_t0_clamp_keeps_results(shift, scale_bits):
     if int(op["t0_clamp"]):
         assert int(op["pre_shift"]) == 33 - shift
     assert scale_bits > 24 or len(np.unique(want)) > 3  # not everything saturated
+
+
+# ---- residual add folded into the pointwise convolution --------------------------------------------------
+@pytest.mark.parametrize("kw", [dict(), dict(other_first=True), dict(N=1, H=65, W=66, C=32, O=16), dict(N=3, H=40, W=40, C=144, O=48, other_first=True)])
+def test_residual_add_folds_into_the_streaming_convolution(kw):
+    wl = w.pointwise_add_workload(**kw)
+    outs = [np.zeros(s, dtype=dt) for s, dt in wl.outputs]
+    d = desc_interp.run(wl.program.serialize(), list(wl.inputs) + outs)
+    assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)
+    assert [int(o["kind"]) for o in d.ops] == [desc_interp.K_IGEMM] and int(d.ops[0]["in1"]["space"]) != 0
+    assert all(int(t["size"]) == 0 for t in d.temps)  # the convolution's own result is never materialised
+
+
+def test_residual_add_stays_apart_when_it_must(monkeypatch):
+    def kinds(p):
+        return [int(o["kind"]) for o in desc_interp.Descriptor(p.serialize()).ops]
+
+    monkeypatch.setenv("THIP_NO_ADD_FUSION", "1")
+    assert kinds(w.pointwise_add_workload().program) == [desc_interp.K_IGEMM, desc_interp.K_ADD]
+    monkeypatch.delenv("THIP_NO_ADD_FUSION")
+    # few rows: a tile kernel, not the streaming one
+    assert kinds(w.pointwise_add_workload(N=1, H=8, W=8).program) == [desc_interp.K_IGEMM, desc_interp.K_ADD]
+    # the convolution's result has a second reader
+    wl = w.pointwise_add_workload()
+    wp, sbp, pa = wl.attrs["pw"]
+    aw, asb, aa = wl.attrs["add"]
+    p = Program()
+    t = p.conv2d(p.binding(0, wl.inputs[0].shape), wp, sbp, nhwc_input=True, **pa)
+    s1 = p.add(t, p.binding(1, wl.inputs[1].shape), aw, asb, init=p.binding(2, wl.inputs[1].shape), **aa)
+    p.add(t, s1, aw, asb, init=p.binding(3, wl.inputs[1].shape), **aa)
+    assert kinds(p) == [desc_interp.K_IGEMM, desc_interp.K_ADD, desc_interp.K_ADD]

@@ -63,7 +63,9 @@ struct DescConst {
 // Kernel kinds.  One record = one kernel launch.
 enum Kind : uint32_t {
     kKindTranspose = 1,  // [B, R, S] -> [B, S, R] elements of `gran` bytes (0 or 1: bytes; 2: bf16)
-    kKindIgemm = 2,      // conv2d / fully_connected / matmul on MFMA
+    // conv2d / fully_connected / matmul on MFMA.  A residual add fused by the emitter (pixel-streaming variant, dense
+    // loader, int8): in1 = the add's other operand, table = ResidualAddParams (in1.space none: no add)
+    kKindIgemm = 2,
     kKindFcSkinny = 3,   // fully_connected with few rows: weight streaming
     kKindDepthwise = 4,
     kKindMaxPool = 5,
@@ -97,6 +99,15 @@ enum IgemmLoader : uint32_t {
     // kh in bits 24..30, run length KW * C in bits 0..15.
     kLoaderRuns = 2,
 };
+
+// torq_hl.add folded into the epilogue of the convolution that produces one of its operands.
+struct ResidualAddParams {
+    int32_t w0, w1, bias, scale;             // the add's weights and its one (bias, scale) pair
+    int32_t shift, output_zp, output_min, output_max;
+    int32_t other_first;                     // the operand read from memory is the add's input1
+    int32_t reserved[3];
+};
+static_assert(sizeof(ResidualAddParams) == 48, "ResidualAddParams layout");
 
 struct DescOp {
     uint32_t kind;

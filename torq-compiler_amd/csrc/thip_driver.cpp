@@ -215,6 +215,18 @@ static thip_status_t checkOpFootprint(const thip_executable_t *e, uint32_t i) {
                 if (kh >= op.KH || kw >= op.KW || ci + (int)op.gran > op.C) return fail(THIP_INVALID_ARGUMENT, "op %u: table entry %u is outside the window", i, t);
             }
         }
+        if (op.in1.space != kSpaceNone) {  // fused residual add
+            if (op.variant != kIgemmStream || op.loader != kLoaderDense || op.out_dtype != THIP_DTYPE_I8 || op.table.space != kSpaceConst) {
+                return fail(THIP_INVALID_ARGUMENT, "op %u: a residual add needs the streaming int8 kernel", i);
+            }
+            if ((s = need(op.in1, (uint64_t)op.M * op.Nn, "residual"))) return s;
+            if ((s = need(op.table, sizeof(ResidualAddParams), "residual parameters"))) return s;
+            ResidualAddParams ap;
+            memcpy(&ap, e->blob.data() + e->header.data_offset + e->consts[op.table.index].offset + op.table.offset, sizeof(ap));
+            if (ap.shift < 0 || ap.shift > 63 || ap.output_min > ap.output_max || ap.output_min < -128 || ap.output_max > 127) {
+                return fail(THIP_INVALID_ARGUMENT, "op %u: bad residual add parameters", i);
+            }
+        }
         return need(op.out, (uint64_t)op.M * op.Nn * outElem, "out");
     }
     case kKindFcSkinny: {
@@ -385,6 +397,14 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
         a.loader = op.loader;
         a.gran = op.gran;
         a.rq = rq;
+        if (op.in1.space != kSpaceNone) {
+            ResidualAddParams ap;
+            memcpy(&ap, e->blob.data() + e->header.data_offset + e->consts[op.table.index].offset + op.table.offset, sizeof(ap));
+            a.skip = (const int8_t *)resolve(e, op.in1, bp);
+            a.add_skip_first = ap.other_first;
+            a.add_w0 = ap.w0; a.add_w1 = ap.w1; a.add_bias = ap.bias; a.add_scale = ap.scale;
+            a.arq = Requant{ap.shift, ap.output_zp, ap.output_min, ap.output_max, 0, 0};
+        }
         err = launchIgemm(a, op.variant, e->stream);
         break;
     }

@@ -132,6 +132,9 @@ class Emitter {
     // the op).  THIP_NO_EXPAND_FOLD keeps every expand_weights a kernel of its own.
     std::map<thip_value_t, const thip_hl_expand_weights_t *> foldedExpand_;
     void planExpandFolding();
+    // Folds a torq_hl.add record into the pixel-streaming convolution record right before it that produces one of
+    // its operands, when nobody else reads that operand (THIP_NO_ADD_FUSION leaves them apart).
+    void fuseResidualAdd();
 
     thip_status_t checkValue(thip_value_t v, const char *what, const Value **out) const {
         if (v < 0 || (size_t)v >= prog_.values.size()) {
@@ -1710,6 +1713,40 @@ void Emitter::planExpandFolding() {
     }
 }
 
+void Emitter::fuseResidualAdd() {
+    if (getenv("THIP_NO_ADD_FUSION")) return;
+    auto same = [](const DescRef &a, const DescRef &b) { return a.space == b.space && a.index == b.index && a.offset == b.offset; };
+    for (size_t i = 0; i + 1 < ops_.size(); i++) {
+        const DescOp conv = ops_[i], add = ops_[i + 1];
+        if (conv.kind != kKindIgemm || conv.variant != kIgemmStream || conv.loader != kLoaderDense || conv.out_dtype != THIP_DTYPE_I8) continue;
+        if (conv.in1.space != kSpaceNone || conv.out.space != kSpaceTemp || conv.out.offset != 0 || add.kind != kKindAdd) continue;
+        const bool first = same(add.in0, conv.out), second = same(add.in1, conv.out);
+        if (first == second || add.C != (int64_t)conv.M * conv.Nn) continue;
+        // nobody else may touch the convolution's result
+        bool shared = false;
+        for (size_t k = 0; k < ops_.size() && !shared; k++) {
+            if (k == i || k == i + 1) continue;
+            const DescRef *refs[] = {&ops_[k].in0, &ops_[k].in1, &ops_[k].weights, &ops_[k].bias, &ops_[k].scale, &ops_[k].table, &ops_[k].out};
+            for (const DescRef *r : refs) shared = shared || (r->space == kSpaceTemp && r->index == conv.out.index);
+        }
+        if (shared) continue;
+        ResidualAddParams ap;
+        memset(&ap, 0, sizeof(ap));
+        ap.w0 = add.w0; ap.w1 = add.w1; ap.bias = add.bias0; ap.scale = add.scale0;
+        ap.shift = add.shift; ap.output_zp = add.output_zp; ap.output_min = add.output_min; ap.output_max = add.output_max;
+        ap.other_first = second;  // the convolution's result is input2: the operand read from memory is input1
+        std::vector<uint8_t> blob(sizeof(ap));
+        memcpy(blob.data(), &ap, sizeof(ap));
+        DescOp f = conv;
+        f.in1 = second ? add.in0 : add.in1;
+        f.table = newConst(blob);
+        f.out = add.out;
+        temps_[conv.out.index] = 0;  // never materialised
+        ops_[i] = f;
+        ops_.erase(ops_.begin() + (long)i + 1);
+    }
+}
+
 thip_status_t Emitter::run(void **outBlob, size_t *outSize) {
     planChannelPadding();
     planExpandFolding();
@@ -1732,6 +1769,7 @@ thip_status_t Emitter::run(void **outBlob, size_t *outSize) {
         if (s != THIP_OK) return s;
     }
     if (ops_.empty()) return fail(THIP_INVALID_ARGUMENT, "program has no ops");
+    fuseResidualAdd();
 
     // Binding ids must be dense 0..n-1 so the dispatch's binding table indexes directly.
     uint32_t bindingCount = 0;

@@ -38,6 +38,11 @@ struct IgemmArgs {
     uint32_t loader;
     uint32_t gran;
     Requant rq;
+    // a residual add fused behind the requant (pixel-streaming kernel only; null: none): the other operand, laid
+    // out like out, and the parameters of torq_hl.add.  add_skip_first: the other operand is the add's input1.
+    const int8_t *skip;
+    int32_t add_skip_first, add_w0, add_w1, add_bias, add_scale;
+    Requant arq;
 };
 
 // Tile configurations of the igemm kernel.

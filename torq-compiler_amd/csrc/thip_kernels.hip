@@ -883,6 +883,43 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
 
 
 // ---------------------------------------------------------------------------
+// torq_hl.add on 16 requantised bytes and 16 bytes of the other operand.  The patterns give an add scale 1 and shift
+// 12: then bias, rounding term and zero point fold into one 32-bit constant `folded` and a value costs two
+// multiply-adds, a shift and a clamp (FAST; the launcher proves that nothing overflows).  Anything else takes the
+// generic 64-bit ACT stage.
+template <bool FAST>
+__device__ __forceinline__ v4i residualAdd16(v4i mine, v4i other, bool otherFirst, int32_t w0, int32_t w1, int32_t bias, int32_t scale,
+                                             long long rnd, const Requant &rq, int32_t folded) {
+    v4i r;
+    const int32_t wm = otherFirst ? w1 : w0, wo = otherFirst ? w0 : w1;
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        int32_t v[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int32_t a = (int32_t)(int8_t)((uint32_t)mine[g] >> (8 * e)), b = (int32_t)(int8_t)((uint32_t)other[g] >> (8 * e));
+            if (FAST) {
+                v[e] = med3((a * wm + b * wo + folded) >> rq.shift, rq.out_min, rq.out_max);
+            } else {
+                v[e] = requant(a * wm + b * wo, bias, scale, rnd, rq);
+            }
+        }
+        r[g] = (int)packBytes(v[0], v[1], v[2], v[3]);
+    }
+    return r;
+}
+// Whether the FAST form applies, and its constant: ((sum + bias) + 2^(shift-1)) >> shift, + zp, clamp equals
+// (sum + bias + 2^(shift-1) + zp * 2^shift) >> shift, clamp, as long as the 32-bit sum cannot overflow.
+__host__ __device__ inline bool residualAddFolded(int32_t w0, int32_t w1, int32_t bias, int32_t scale, const Requant &rq, int32_t *folded) {
+    if (scale != 1 || rq.shift < 1 || rq.shift > 20 || rq.out_min > rq.out_max) return false;
+    const long long aw0 = w0 < 0 ? -(long long)w0 : w0, aw1 = w1 < 0 ? -(long long)w1 : w1;
+    const long long c = (long long)bias + (1LL << (rq.shift - 1)) + (long long)rq.out_zp * (1LL << rq.shift);
+    const long long bound = 128 * (aw0 + aw1) + (c < 0 ? -c : c);
+    if (bound >= (1LL << 31)) return false;
+    *folded = (int32_t)c;
+    return true;
+}
+
 // igemm_stream_i8: pointwise convolution / fully_connected with a small weight matrix
 // (Np * Kp of at most 64 KiB, N <= 256), the shape of the expand and project convolutions of
 // mobile networks at high resolution.  These are bandwidth-bound: a tile kernel spends its time
@@ -898,7 +935,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
 constexpr int kStreamRing = 4;
 constexpr size_t kStreamMaxLds = 64 * 1024;
 
-template <int NB, int LOADER>
+template <int NB, int LOADER, bool ADD>  // ADD: a residual add behind the requant (its code costs the others registers)
 __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArgs p) {
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
     constexpr int RING = kStreamRing;
@@ -959,7 +996,9 @@ __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArg
         return *(const v4i *)(p.A + (size_t)m * p.K + k);
     };
     const WideRequant wrq = wideRequant(p.rq);
-    const long long rnd = roundTerm(p.rq.shift);
+    const long long rnd = roundTerm(p.rq.shift), addRnd = roundTerm(p.arq.shift);
+    int32_t addFolded = 0;
+    const bool addFast = ADD && residualAddFolded(p.add_w0, p.add_w1, p.add_bias, p.add_scale, p.arq, &addFolded);
 
     int g = blockIdx.x * 4 + wave;
     v4i ring[RING];
@@ -1021,9 +1060,16 @@ __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArg
                     // then {d4[0], d4[2], d4[1], d4[3]} are 16 consecutive channels, 0-15 below, 16-31 above.
                     const auto s02 = __builtin_amdgcn_permlane32_swap(d4[0], d4[2], false, false);
                     const auto s13 = __builtin_amdgcn_permlane32_swap(d4[1], d4[3], false, false);
-                    const v4i outv = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
+                    v4i outv = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
                     const int n = n0 + j * 32 + 16 * half;
-                    if (m < p.M && n < p.N) *(v4i *)((int8_t *)p.out + (size_t)m * p.N + n) = outv;
+                    if (m < p.M && n < p.N) {
+                        if (ADD) {
+                            const v4i other = *(const v4i *)(p.skip + (size_t)m * p.N + n);
+                            outv = addFast ? residualAdd16<true>(outv, other, p.add_skip_first != 0, p.add_w0, p.add_w1, p.add_bias, p.add_scale, addRnd, p.arq, addFolded)
+                                           : residualAdd16<false>(outv, other, p.add_skip_first != 0, p.add_w0, p.add_w1, p.add_bias, p.add_scale, addRnd, p.arq, 0);
+                        }
+                        *(v4i *)((int8_t *)p.out + (size_t)m * p.N + n) = outv;
+                    }
                 }
             }
         });
@@ -1031,9 +1077,9 @@ __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArg
     }
 }
 
-template <int NB, int LOADER>
-static hipError_t launchIgemmStreamT(const IgemmArgs &a, size_t smem, hipStream_t stream) {
-    auto kernel = igemm_stream_i8<NB, LOADER>;
+template <int NB, int LOADER, bool ADD>
+static hipError_t launchIgemmStreamA(const IgemmArgs &a, size_t smem, hipStream_t stream) {
+    auto kernel = igemm_stream_i8<NB, LOADER, ADD>;
     static bool configured = false;
     if (!configured) {
         hipError_t err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kStreamMaxLds);
@@ -1052,9 +1098,18 @@ static hipError_t launchIgemmStreamT(const IgemmArgs &a, size_t smem, hipStream_
     return hipGetLastError();
 }
 
+template <int NB, int LOADER>
+static hipError_t launchIgemmStreamT(const IgemmArgs &a, size_t smem, hipStream_t stream) {
+    if (a.skip != nullptr) {
+        if (LOADER != kLoaderDense) return hipErrorInvalidValue;
+        return launchIgemmStreamA<NB, kLoaderDense, true>(a, smem, stream);
+    }
+    return launchIgemmStreamA<NB, LOADER, false>(a, smem, stream);
+}
+
 static hipError_t launchIgemmStream(const IgemmArgs &a, hipStream_t stream) {
     if ((a.loader != kLoaderDense && a.loader != kLoaderRuns) || a.out_dtype != kDtypeI8) return hipErrorInvalidValue;
-    if (a.N % 16 != 0 || ((uintptr_t)a.out & 15) != 0) return hipErrorInvalidValue;
+    if (a.N % 16 != 0 || ((uintptr_t)a.out & 15) != 0 || ((uintptr_t)a.skip & 15) != 0) return hipErrorInvalidValue;
     const int chunk = igemmStreamChunk(a.Np);
     const size_t smem = (size_t)chunk * a.Kp + 8 * (size_t)chunk + (a.loader == kLoaderRuns ? (size_t)a.Kp / 16 * 4 : 0);
     if (chunk > 256 || smem > kStreamMaxLds) return hipErrorInvalidValue;
@@ -1190,6 +1245,7 @@ hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, hipStream_t stream)
     }
     if (((uintptr_t)a.Bp & 15) != 0) return hipErrorInvalidValue;
     if (a.out_dtype < kDtypeI8 || a.out_dtype > kDtypeI32) return hipErrorInvalidValue;
+    if (a.skip != nullptr && variant != kIgemmStream) return hipErrorInvalidValue;  // only the streaming kernel adds a residual
     switch (variant) {
     case kIgemm128x128x64: return launchIgemmLoader<128, 128, 64>(a, stream);
     case kIgemm256x256x64: return launchIgemmLoader<256, 256, 64>(a, stream);

@@ -355,6 +355,31 @@ def add_workload(N=1, H=56, W=56, C=24, zp0=-3, zp1=7, m0=0.71838506, m1=1.3 * 0
                     attrs)
 
 
+def pointwise_add_workload(N=2, H=48, W=48, C=96, O=32, other_first=False, seed=1020):
+    """The end of an inverted-residual block: 1x1 convolution -> add with a second input (the block's input)."""
+    rng = np.random.default_rng(seed)
+    x = rng.integers(-128, 127, size=(N, H, W, C), endpoint=True, dtype=np.int8)
+    skip = rng.integers(-128, 127, size=(N, H, W, O), endpoint=True, dtype=np.int8)
+    wp = rng.integers(-127, 127, size=(O, C, 1, 1), endpoint=True, dtype=np.int8)
+    mult, shift = random_requant(rng, O, True)
+    sbp, sfp = derive_scale_bias(mult, shift, rng.integers(-(1 << 15), 1 << 15, size=O, endpoint=True, dtype=np.int64), wp, 5)
+    pattrs = dict(input_zp=5, output_zp=-7, output_min=-128, output_max=127, shift_factor=sfp, pad=(0, 0, 0, 0), stride=(1, 1))
+    aw, asb, asf = add_params(0.71838506, 0.65, -3, -7) if other_first else add_params(0.65, 0.71838506, -7, -3)
+    aattrs = dict(output_zp=-2, output_min=-128, output_max=127, shift_factor=asf)
+    p = Program()
+    inp = p.binding(0, x.shape)
+    sk = p.binding(1, skip.shape)
+    out = p.binding(2, skip.shape)
+    t = p.conv2d(inp, wp, sbp, nhwc_input=True, **pattrs)
+    if other_first:
+        p.add(sk, t, aw, asb, init=out, **aattrs)
+    else:
+        p.add(t, sk, aw, asb, init=out, **aattrs)
+    attrs = dict(pw=(wp, sbp, pattrs), add=(aw, asb, aattrs), other_first=other_first)
+    return Workload("pwadd_%dx%dx%dx%d_o%d_%d" % (N, H, W, C, O, int(other_first)), p, [x, skip], [(skip.shape, np.int8)],
+                    2 * N * H * W * C * O, x.nbytes + 2 * skip.nbytes + wp.nbytes, attrs)
+
+
 _INT_RANGE = {np.dtype(np.int8): (-128, 127), np.dtype(np.int16): (-32768, 32767), np.dtype(np.int32): (-2 ** 31, 2 ** 31 - 1)}
 
 
