@@ -1517,11 +1517,17 @@ __global__ __launch_bounds__(256) void depthwise3x3_dot4_i8(DepthwiseArgs p, Wor
     const int8_t *img = p.in + (size_t)n * p.H * p.W * p.C + c0;
     const uint32_t zp4 = (uint32_t)(p.input_zp & 0xff) * 0x01010101u;
     const uint32_t *wrow = (const uint32_t *)p.wpk + c0;
+    // the accumulators start at the bias: the first dot product takes it as its addend, which saves clearing the
+    // accumulator and adding the bias afterwards (int32 wrap-around is the same in either order)
     int32_t acc[P][16];
 #pragma unroll
-    for (int q = 0; q < P; q++) {
+    for (int g = 0; g < 4; g++) {
+        const v4i b4 = *(const v4i *)(p.bias + c0 + 4 * g);
 #pragma unroll
-        for (int v = 0; v < 16; v++) acc[q][v] = 0;
+        for (int q = 0; q < P; q++) {
+#pragma unroll
+            for (int c = 0; c < 4; c++) acc[q][4 * g + c] = b4[c];
+        }
     }
 #pragma unroll
     for (int kh = 0; kh < 3; kh++) {
@@ -1560,15 +1566,12 @@ __global__ __launch_bounds__(256) void depthwise3x3_dot4_i8(DepthwiseArgs p, Wor
         constexpr int kMode = decltype(mode)::value;
 #pragma unroll
         for (int g = 0; g < 4; g++) {
-            const v4i b4 = *(const v4i *)(p.bias + c0 + 4 * g);
             const v4i s4 = *(const v4i *)(p.scale + c0 + 4 * g);
 #pragma unroll
             for (int q = 0; q < P; q++) {
                 int32_t v[4];
 #pragma unroll
-                for (int c = 0; c < 4; c++) {
-                    v[c] = requantT0<kMode>((int32_t)((uint32_t)acc[q][4 * g + c] + (uint32_t)b4[c]), s4[c], rnd, p.rq, wrq);
-                }
+                for (int c = 0; c < 4; c++) v[c] = requantT0<kMode>(acc[q][4 * g + c], s4[c], rnd, p.rq, wrq);
                 o[q][g] = (int)packBytes(v[0], v[1], v[2], v[3]);
             }
         }
