@@ -150,7 +150,7 @@ def run(blob, binding_arrays):
             res = q.astype(odt).reshape(-1)
             if kind == K_IGEMM and int(op["in1"]["space"]) != 0:
                 # a residual add folded into the epilogue: the other operand from in1, the add's parameters from `table`
-                assert int(op["variant"]) == 11 and int(op["loader"]) == 0 and odt == np.int8
+                assert int(op["variant"]) in (7, 11) and int(op["loader"]) == 0 and odt == np.int8
                 ap = view(op["table"], 48).view(np.int32)
                 other = view(op["in1"], M * N).view(np.int8)
                 a, b = (other, res) if int(ap[8]) else (res, other)

@@ -336,8 +336,10 @@ def test_t0_clamp_keeps_results(shift, scale_bits):
 
 
 # ---- residual add folded into the pointwise convolution --------------------------------------------------
-@pytest.mark.parametrize("kw", [dict(), dict(other_first=True), dict(N=1, H=65, W=66, C=32, O=16), dict(N=3, H=40, W=40, C=144, O=48, other_first=True)])
+@pytest.mark.parametrize("kw", [dict(), dict(other_first=True), dict(N=1, H=65, W=66, C=32, O=16), dict(N=3, H=40, W=40, C=144, O=48, other_first=True),
+                                dict(N=1, H=8, W=8), dict(N=1, H=14, W=14, C=384, O=64, other_first=True), dict(N=2, H=7, W=7, C=960, O=160)])
 def test_residual_add_folds_into_the_streaming_convolution(kw):
+    """Many pixels: the pixel-streaming kernel; few: the 64x64 dense tile with its in-register epilogue."""
     wl = w.pointwise_add_workload(**kw)
     outs = [np.zeros(s, dtype=dt) for s, dt in wl.outputs]
     d = desc_interp.run(wl.program.serialize(), list(wl.inputs) + outs)
@@ -353,8 +355,8 @@ def test_residual_add_stays_apart_when_it_must(monkeypatch):
     monkeypatch.setenv("THIP_NO_ADD_FUSION", "1")
     assert kinds(w.pointwise_add_workload().program) == [desc_interp.K_IGEMM, desc_interp.K_ADD]
     monkeypatch.delenv("THIP_NO_ADD_FUSION")
-    # few rows: a tile kernel, not the streaming one
-    assert kinds(w.pointwise_add_workload(N=1, H=8, W=8).program) == [desc_interp.K_IGEMM, desc_interp.K_ADD]
+    # output channels that are not a multiple of 16: neither kernel that can add a residual takes them
+    assert kinds(w.pointwise_add_workload(O=24).program) == [desc_interp.K_IGEMM, desc_interp.K_ADD]
     # the convolution's result has a second reader
     wl = w.pointwise_add_workload()
     wp, sbp, pa = wl.attrs["pw"]

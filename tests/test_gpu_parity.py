@@ -395,6 +395,14 @@ def test_residual_add_in_the_streaming_epilogue(device, monkeypatch):
         got, kernels = run_on_gpu(device, wl, via="device")
         assert kernels == ["igemm_stream_i8"], kernels
         assert_bit_exact(got[0], oracle_eval(wl)[0], wl.name)
+    # few pixels: the small dense tile adds the residual in its in-register epilogue
+    for kw in [dict(N=1, H=8, W=8), dict(N=1, H=14, W=14, C=384, O=64, other_first=True), dict(N=2, H=7, W=7, C=960, O=160), dict(N=1, H=28, W=28, C=192, O=32),
+               dict(N=1, H=9, W=7, C=48, O=80, other_first=True)]:
+        wl = w.pointwise_add_workload(**kw)
+        print("[gpu-case]", wl.name, flush=True)
+        got, kernels = run_on_gpu(device, wl, via="device")
+        assert kernels == ["igemm_dense_i8_64x64x64"], kernels
+        assert_bit_exact(got[0], oracle_eval(wl)[0], wl.name)
     folded, kernels = run_on_gpu(device, w.mobilenet_v2_workload(batch=8), via="device")
     monkeypatch.setenv("THIP_NO_ADD_FUSION", "1")
     apart, kernels_apart = run_on_gpu(device, w.mobilenet_v2_workload(batch=8), via="device")

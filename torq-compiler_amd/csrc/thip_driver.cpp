@@ -216,8 +216,9 @@ static thip_status_t checkOpFootprint(const thip_executable_t *e, uint32_t i) {
             }
         }
         if (op.in1.space != kSpaceNone) {  // fused residual add
-            if (op.variant != kIgemmStream || op.loader != kLoaderDense || op.out_dtype != THIP_DTYPE_I8 || op.table.space != kSpaceConst) {
-                return fail(THIP_INVALID_ARGUMENT, "op %u: a residual add needs the streaming int8 kernel", i);
+            if ((op.variant != kIgemmStream && op.variant != kIgemmDense64x64) || op.loader != kLoaderDense || op.out_dtype != THIP_DTYPE_I8 ||
+                op.table.space != kSpaceConst) {
+                return fail(THIP_INVALID_ARGUMENT, "op %u: a residual add needs the streaming or the small-tile int8 kernel", i);
             }
             if ((s = need(op.in1, (uint64_t)op.M * op.Nn, "residual"))) return s;
             if ((s = need(op.table, sizeof(ResidualAddParams), "residual parameters"))) return s;

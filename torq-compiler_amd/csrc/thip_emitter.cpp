@@ -1718,7 +1718,11 @@ void Emitter::fuseResidualAdd() {
     auto same = [](const DescRef &a, const DescRef &b) { return a.space == b.space && a.index == b.index && a.offset == b.offset; };
     for (size_t i = 0; i + 1 < ops_.size(); i++) {
         const DescOp conv = ops_[i], add = ops_[i + 1];
-        if (conv.kind != kKindIgemm || conv.variant != kIgemmStream || conv.loader != kLoaderDense || conv.out_dtype != THIP_DTYPE_I8) continue;
+        if (conv.kind != kKindIgemm || conv.loader != kLoaderDense || conv.out_dtype != THIP_DTYPE_I8) continue;
+        // the pixel-streaming kernel, or the small dense tile when it will run its in-register epilogue
+        const bool inRegister = conv.variant == kIgemmDense64x64 && conv.Nn % 16 == 0 && conv.shift >= 33 && conv.shift <= 45 &&
+                                conv.pre_shift == 0 && conv.t0_clamp == 0 && conv.output_min <= conv.output_max && !getenv("THIP_NO_DIRECT_EPILOGUE");
+        if (conv.variant != kIgemmStream && !inRegister) continue;
         if (conv.in1.space != kSpaceNone || conv.out.space != kSpaceTemp || conv.out.offset != 0 || add.kind != kKindAdd) continue;
         const bool first = same(add.in0, conv.out), second = same(add.in1, conv.out);
         if (first == second || add.C != (int64_t)conv.M * conv.Nn) continue;

@@ -269,12 +269,49 @@ __device__ __forceinline__ void igemmEpilogue(v16i (&acc)[WTN / 32][WTM / 32], i
     }
 }
 
+// torq_hl.add on 16 requantised bytes and 16 bytes of the other operand.  The patterns give an add scale 1 and shift
+// 12: then bias, rounding term and zero point fold into one 32-bit constant `folded` and a value costs two
+// multiply-adds, a shift and a clamp (FAST; the launcher proves that nothing overflows).  Anything else takes the
+// generic 64-bit ACT stage.
+template <bool FAST>
+__device__ __forceinline__ v4i residualAdd16(v4i mine, v4i other, bool otherFirst, int32_t w0, int32_t w1, int32_t bias, int32_t scale,
+                                             long long rnd, const Requant &rq, int32_t folded) {
+    v4i r;
+    const int32_t wm = otherFirst ? w1 : w0, wo = otherFirst ? w0 : w1;
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        int32_t v[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int32_t a = (int32_t)(int8_t)((uint32_t)mine[g] >> (8 * e)), b = (int32_t)(int8_t)((uint32_t)other[g] >> (8 * e));
+            if (FAST) {
+                v[e] = med3((a * wm + b * wo + folded) >> rq.shift, rq.out_min, rq.out_max);
+            } else {
+                v[e] = requant(a * wm + b * wo, bias, scale, rnd, rq);
+            }
+        }
+        r[g] = (int)packBytes(v[0], v[1], v[2], v[3]);
+    }
+    return r;
+}
+// Whether the FAST form applies, and its constant: ((sum + bias) + 2^(shift-1)) >> shift, + zp, clamp equals
+// (sum + bias + 2^(shift-1) + zp * 2^shift) >> shift, clamp, as long as the 32-bit sum cannot overflow.
+__host__ __device__ inline bool residualAddFolded(int32_t w0, int32_t w1, int32_t bias, int32_t scale, const Requant &rq, int32_t *folded) {
+    if (scale != 1 || rq.shift < 1 || rq.shift > 20 || rq.out_min > rq.out_max) return false;
+    const long long aw0 = w0 < 0 ? -(long long)w0 : w0, aw1 = w1 < 0 ? -(long long)w1 : w1;
+    const long long c = (long long)bias + (1LL << (rq.shift - 1)) + (long long)rq.out_zp * (1LL << rq.shift);
+    const long long bound = 128 * (aw0 + aw1) + (c < 0 ? -c : c);
+    if (bound >= (1LL << 31)) return false;
+    *folded = (int32_t)c;
+    return true;
+}
+
 // The same epilogue without the LDS round trip, for int8 outputs with N % 16 == 0 and the plain
 // 32-bit requant tail (no pre-shift, zero point folded into the rounding term): each accumulator tile is requantised in place, two v_permlane32_swap exchange
 // register groups between the wave halves so that a lane owns 16 consecutive channels of its row
 // (see igemm_stream_i8), and the lane stores them as one 128-bit word.  Only the (bias, scale)
 // vectors pass through LDS.
-template <int WTM, int WTN, int NW, int BN>
+template <int WTM, int WTN, int NW, int BN, bool ADD>  // ADD: a residual add behind the requant (IgemmArgs::skip)
 __device__ __forceinline__ void igemmEpilogueDirect(v16i (&acc)[WTN / 32][WTM / 32], int8_t *smem, const IgemmArgs &p, int m0,
                                                     int n0, int wm, int wn, int32_t myBias, int32_t myScale) {
     blockBarrier();
@@ -287,6 +324,9 @@ __device__ __forceinline__ void igemmEpilogueDirect(v16i (&acc)[WTN / 32][WTM / 
     }
     __syncthreads();
     const WideRequant wrq = wideRequant(p.rq);  // plain (the launcher checks): no pre-shift, zero point folded
+    const long long addRnd = roundTerm(p.arq.shift);
+    int32_t addFolded = 0;
+    const bool addFast = ADD && residualAddFolded(p.add_w0, p.add_w1, p.add_bias, p.add_scale, p.arq, &addFolded);
 #pragma unroll
     for (int j = 0; j < TN; j++) {
         const int nl = wn * WTN + j * 32;  // first channel of this tile column, relative to n0
@@ -311,9 +351,16 @@ __device__ __forceinline__ void igemmEpilogueDirect(v16i (&acc)[WTN / 32][WTM / 
             }
             const auto s02 = __builtin_amdgcn_permlane32_swap(d4[0], d4[2], false, false);
             const auto s13 = __builtin_amdgcn_permlane32_swap(d4[1], d4[3], false, false);
-            const v4i outv = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
+            v4i outv = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
             const int m = m0 + wm * WTM + i * 32 + fr;
-            if (m < p.M && n < p.N) *(v4i *)((int8_t *)p.out + (size_t)m * p.N + n) = outv;
+            if (m < p.M && n < p.N) {
+                if (ADD) {
+                    const v4i other = *(const v4i *)(p.skip + (size_t)m * p.N + n);
+                    outv = addFast ? residualAdd16<true>(outv, other, p.add_skip_first != 0, p.add_w0, p.add_w1, p.add_bias, p.add_scale, addRnd, p.arq, addFolded)
+                                   : residualAdd16<false>(outv, other, p.add_skip_first != 0, p.add_w0, p.add_w1, p.add_bias, p.add_scale, addRnd, p.arq, 0);
+                }
+                *(v4i *)((int8_t *)p.out + (size_t)m * p.N + n) = outv;
+            }
         }
     }
 }
@@ -672,7 +719,7 @@ __device__ __forceinline__ void waitVmcnt() {
 
 // DIRECT selects the epilogue: in registers (int8 output, N % 16 == 0, plain 32-bit requant tail: the launcher
 // checks) or staged through LDS (everything else).
-template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, bool DIRECT>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, bool DIRECT, bool ADD = false>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_dense_i8(IgemmArgs p) {
     constexpr int BK = 64;
     constexpr int NW = WAVES_M * WAVES_N;
@@ -875,7 +922,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
     for (; kt < KT; kt++) step(kt, std::false_type{});
 
     if (DIRECT) {
-        igemmEpilogueDirect<WTM, WTN, NW, BN>(acc, smem, p, m0, n0, wm, wn, myBias, myScale);
+        igemmEpilogueDirect<WTM, WTN, NW, BN, ADD>(acc, smem, p, m0, n0, wm, wn, myBias, myScale);
     } else {
         igemmEpilogue<WTM, WTN, NW, BN>(acc, smem, p, m0, n0, wm, wn, myBias, myScale);
     }
@@ -883,43 +930,6 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
 
 
 // ---------------------------------------------------------------------------
-// torq_hl.add on 16 requantised bytes and 16 bytes of the other operand.  The patterns give an add scale 1 and shift
-// 12: then bias, rounding term and zero point fold into one 32-bit constant `folded` and a value costs two
-// multiply-adds, a shift and a clamp (FAST; the launcher proves that nothing overflows).  Anything else takes the
-// generic 64-bit ACT stage.
-template <bool FAST>
-__device__ __forceinline__ v4i residualAdd16(v4i mine, v4i other, bool otherFirst, int32_t w0, int32_t w1, int32_t bias, int32_t scale,
-                                             long long rnd, const Requant &rq, int32_t folded) {
-    v4i r;
-    const int32_t wm = otherFirst ? w1 : w0, wo = otherFirst ? w0 : w1;
-#pragma unroll
-    for (int g = 0; g < 4; g++) {
-        int32_t v[4];
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const int32_t a = (int32_t)(int8_t)((uint32_t)mine[g] >> (8 * e)), b = (int32_t)(int8_t)((uint32_t)other[g] >> (8 * e));
-            if (FAST) {
-                v[e] = med3((a * wm + b * wo + folded) >> rq.shift, rq.out_min, rq.out_max);
-            } else {
-                v[e] = requant(a * wm + b * wo, bias, scale, rnd, rq);
-            }
-        }
-        r[g] = (int)packBytes(v[0], v[1], v[2], v[3]);
-    }
-    return r;
-}
-// Whether the FAST form applies, and its constant: ((sum + bias) + 2^(shift-1)) >> shift, + zp, clamp equals
-// (sum + bias + 2^(shift-1) + zp * 2^shift) >> shift, clamp, as long as the 32-bit sum cannot overflow.
-__host__ __device__ inline bool residualAddFolded(int32_t w0, int32_t w1, int32_t bias, int32_t scale, const Requant &rq, int32_t *folded) {
-    if (scale != 1 || rq.shift < 1 || rq.shift > 20 || rq.out_min > rq.out_max) return false;
-    const long long aw0 = w0 < 0 ? -(long long)w0 : w0, aw1 = w1 < 0 ? -(long long)w1 : w1;
-    const long long c = (long long)bias + (1LL << (rq.shift - 1)) + (long long)rq.out_zp * (1LL << rq.shift);
-    const long long bound = 128 * (aw0 + aw1) + (c < 0 ? -c : c);
-    if (bound >= (1LL << 31)) return false;
-    *folded = (int32_t)c;
-    return true;
-}
-
 // igemm_stream_i8: pointwise convolution / fully_connected with a small weight matrix
 // (Np * Kp of at most 64 KiB, N <= 256), the shape of the expand and project convolutions of
 // mobile networks at high resolution.  These are bandwidth-bound: a tile kernel spends its time
@@ -1188,14 +1198,14 @@ static hipError_t launchIgemmLoader(const IgemmArgs &a, hipStream_t stream) {
     }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, bool DIRECT>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, bool DIRECT, bool ADD = false>
 static hipError_t launchIgemmDenseE(const IgemmArgs &a, hipStream_t stream) {
     // the stage ring, reused by the epilogue as staging slices (one per wave) plus bias/scale
     constexpr size_t ring = (size_t)STAGES * (BM + BN) * 64;
     constexpr size_t epilogue = (size_t)(BM / WAVES_M) * (WAVES_M * WAVES_N) * (32 * 4 + 16) + 2 * BN * 4;
     constexpr size_t smem = ring > epilogue ? ring : epilogue;
     static_assert(smem * BLOCKS_PER_CU <= 160 * 1024, "LDS of one CU");
-    auto kernel = igemm_dense_i8<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, DIRECT>;
+    auto kernel = igemm_dense_i8<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, DIRECT, ADD>;
     static bool configured = false;
     if (!configured) {
         hipError_t err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
@@ -1215,6 +1225,15 @@ static hipError_t launchIgemmDense(const IgemmArgs &a, hipStream_t stream) {
                        a.rq.out_zp >= -32768 && a.rq.out_zp <= 32767 && a.rq.out_min <= a.rq.out_max;
     const bool direct = a.out_dtype == kDtypeI8 && a.N % 16 == 0 && ((uintptr_t)a.out & 15) == 0 && plain &&
                         !getenv("THIP_NO_DIRECT_EPILOGUE");
+    if (a.skip != nullptr) {
+        // a residual add: the in-register epilogue of the small tile only (what a network's late, small layers take)
+        if constexpr (BM == 64 && BN == 64) {
+            if (!direct || ((uintptr_t)a.skip & 15) != 0) return hipErrorInvalidValue;
+            return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, true, true>(a, stream);
+        } else {
+            return hipErrorInvalidValue;
+        }
+    }
     return direct ? launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, true>(a, stream)
                   : launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, false>(a, stream);
 }
@@ -1245,7 +1264,7 @@ hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, hipStream_t stream)
     }
     if (((uintptr_t)a.Bp & 15) != 0) return hipErrorInvalidValue;
     if (a.out_dtype < kDtypeI8 || a.out_dtype > kDtypeI32) return hipErrorInvalidValue;
-    if (a.skip != nullptr && variant != kIgemmStream) return hipErrorInvalidValue;  // only the streaming kernel adds a residual
+    if (a.skip != nullptr && variant != kIgemmStream && variant != kIgemmDense64x64) return hipErrorInvalidValue;  // the kernels that can add a residual
     switch (variant) {
     case kIgemm128x128x64: return launchIgemmLoader<128, 128, 64>(a, stream);
     case kIgemm256x256x64: return launchIgemmLoader<256, 256, 64>(a, stream);
