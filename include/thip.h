@@ -313,6 +313,18 @@ typedef struct thip_hl_act_t {
     thip_value_t weights;
 } thip_hl_act_t;
 
+/* torq_hl.elementwisebinary -- TorqHLOps.td:248-260.  op_type: the reference's ElementwiseOpEnum value
+ * (TorqHLAttrs.td:219-235); on this path BITWISE_AND 0, BITWISE_OR 1, BITWISE_XOR 2, MINIMUM 4, MAXIMUM 5.  input1,
+ * input2 and init: int8 / int16 / int32 tensors of one type and shape; is_unsigned (16-bit only) makes MINIMUM /
+ * MAXIMUM compare as unsigned.  The comparisons, logical ops and the int32 ADD / SUB are not on this path. */
+typedef struct thip_hl_elementwisebinary_t {
+    thip_value_t init;
+    int32_t op_type;
+    thip_value_t input1;
+    thip_value_t input2;
+    int32_t is_unsigned;
+} thip_hl_elementwisebinary_t;
+
 thip_status_t thip_hl_conv2d(thip_program_t *program, const thip_hl_conv2d_t *op);
 thip_status_t thip_hl_depthwise_conv2d(thip_program_t *program,
                                        const thip_hl_depthwise_conv2d_t *op);
@@ -327,6 +339,7 @@ thip_status_t thip_hl_expand_weights(thip_program_t *program, const thip_hl_expa
 thip_status_t thip_hl_fma(thip_program_t *program, const thip_hl_fma_t *op);
 thip_status_t thip_hl_mul(thip_program_t *program, const thip_hl_mul_t *op);
 thip_status_t thip_hl_act(thip_program_t *program, const thip_hl_act_t *op);
+thip_status_t thip_hl_elementwisebinary(thip_program_t *program, const thip_hl_elementwisebinary_t *op);
 
 /* Serialises the program (role of TargetBackend::serializeExecutable,
  * compiler/torq/Target/TorqTarget.cpp:115-151, and serializeTorqHW,

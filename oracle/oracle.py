@@ -396,6 +396,20 @@ def act(input, name, *, min_int=0, max_int=0, out_dtype=None):
     return out
 
 
+BINARY_MODES = {"and": 0, "or": 1, "xor": 2, "minimum": 4, "maximum": 5}
+
+
+def elementwise_binary(op_type, input1, input2, *, is_unsigned=False):
+    """torq_hl.elementwisebinary: and / or / xor / minimum / maximum on two integer tensors of one type."""
+    a = _int_array(input1)
+    b = _int_array(input2)
+    assert a.dtype == b.dtype and a.shape == b.shape
+    out = np.empty(a.shape, dtype=a.dtype)
+    rc = lib().torq_elementwise_binary(BINARY_MODES[op_type], _p(a), _p(b), a.itemsize, int(bool(is_unsigned)), _p(out), ctypes.c_size_t(a.size))
+    assert rc == 0
+    return out
+
+
 def per_channel_sum(weights):
     w = _c(weights, np.int8)
     ch = w.shape[0]

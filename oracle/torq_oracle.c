@@ -609,6 +609,34 @@ int torq_act(const void *input, int in_bytes, void *out, int out_bytes, size_t c
     return 0;
 }
 
+/*
+ * torq_hl.elementwisebinary -- signature TorqHLOps.td:248-260, modes TorqHLAttrs.td:219-235; executed
+ * compiler/torq/Conversions/TorqHLToTorqHW/ElementWiseBinaryPattern.cpp:93-107 (ALU op1 modes BAND / BOR / BXOR /
+ * MIN / MAX on two tensors of one element type, no ACT rescale) and :70-84 (16-bit operands compare as unsigned
+ * when is_unsigned is set).  mode: 0 and, 1 or, 2 xor, 4 minimum, 5 maximum (the enum's values).
+ */
+int torq_elementwise_binary(int mode, const void *input1, const void *input2, int bytes, int is_unsigned, void *out, size_t count) {
+    if (bad_out_bytes(bytes) || !(mode == 0 || mode == 1 || mode == 2 || mode == 4 || mode == 5)) return -1;
+    if (is_unsigned && bytes != 2) return -1;
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < count; i++) {
+        const int64_t a = load_elem(input1, i, bytes), b = load_elem(input2, i, bytes);
+        int64_t r;
+        switch (mode) {
+        case 0: r = a & b; break;
+        case 1: r = a | b; break;
+        case 2: r = a ^ b; break;
+        default: {
+            const int64_t ka = is_unsigned ? (a & 0xffff) : a, kb = is_unsigned ? (b & 0xffff) : b;
+            r = (mode == 4) == (ka < kb) ? a : b;
+            break;
+        }
+        }
+        store_elem(out, i, r, bytes);
+    }
+    return 0;
+}
+
 /* ---- R2 ---- */
 
 /* compiler/torq/Utils/ConversionUtils.cpp:122-141 (per_channel_sum). */

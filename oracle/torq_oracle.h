@@ -146,6 +146,10 @@ int torq_mul(const void *input1, size_t count1, const void *input2, size_t count
 int torq_act(const void *input, int in_bytes, void *out, int out_bytes, size_t count, int mode, int64_t min_int,
              int64_t max_int);
 
+/* torq_hl.elementwisebinary: mode 0 and, 1 or, 2 xor, 4 minimum, 5 maximum; both inputs and the output of one integer
+ * type (bytes = 1, 2, 4); is_unsigned (16-bit only) compares as unsigned. */
+int torq_elementwise_binary(int mode, const void *input1, const void *input2, int bytes, int is_unsigned, void *out, size_t count);
+
 /* ---- R2: compile-side parameter derivations ---- */
 
 /* Conv / depthwise / FC: per-channel TOSA (multiplier, shift) -> one global

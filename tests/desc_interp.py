@@ -278,6 +278,10 @@ def run(blob, binding_arrays):
             elif variant == 1:
                 b = view(op["in1"], (1 if bcast == 2 else n) * esz).view(tin)
                 res = orc.mul(a, b, [int(op["bias0"]), int(op["scale0"])], output_zp=zp, output_min=mn, output_max=mx, shift=sh, out_dtype=tout)
+            elif variant >= 6:
+                b = view(op["in1"], n * esz).view(tin)
+                assert tin == tout
+                res = orc.elementwise_binary({6: "and", 7: "or", 8: "xor", 9: "minimum", 10: "maximum"}[variant], a, b, is_unsigned=bool(int(op["w0"])))
             else:
                 name = {2: "clamp", 3: "abs", 4: "negate", 5: "i2i"}[variant]
                 if name != "clamp":  # the record carries the clip range the op implies

@@ -35,6 +35,8 @@ def oracle_eval(wl):
         return [orc.fma(x, a.pop("weights"), a.pop("scale_bias"), **a)]
     if kind == "mul":
         return [orc.mul(x, wl.inputs[1], a.pop("scale_bias"), **a)]
+    if kind == "binary":
+        return [orc.elementwise_binary(a["op_type"], x, wl.inputs[1], is_unsigned=a["is_unsigned"])]
     if kind == "act":
         return [orc.act(x, a["name"], min_int=a["min_int"], max_int=a["max_int"], out_dtype=a["out_dtype"])]
     if kind == "avgpoolbf16":

@@ -69,6 +69,23 @@ def test_act_modes():
     assert np.array_equal(orc.act(wide, "clamp", min_int=-100, max_int=100, out_dtype=np.int8), np.clip(wide, -100, 100).astype(np.int8))
 
 
+def test_elementwise_binary_modes():
+    rng = np.random.default_rng(6)
+    for dt in (np.int8, np.int16, np.int32):
+        info = np.iinfo(dt)
+        a = rng.integers(info.min, info.max, size=300, endpoint=True).astype(dt)
+        b = rng.integers(info.min, info.max, size=300, endpoint=True).astype(dt)
+        a[:3], b[:3] = [info.min, info.max, -1], [info.max, info.min, 0]
+        assert np.array_equal(orc.elementwise_binary("and", a, b), a & b)
+        assert np.array_equal(orc.elementwise_binary("or", a, b), a | b)
+        assert np.array_equal(orc.elementwise_binary("xor", a, b), a ^ b)
+        assert np.array_equal(orc.elementwise_binary("minimum", a, b), np.minimum(a, b))
+        assert np.array_equal(orc.elementwise_binary("maximum", a, b), np.maximum(a, b))
+    a16, b16 = a.astype(np.int16), b.astype(np.int16)
+    assert np.array_equal(orc.elementwise_binary("minimum", a16, b16, is_unsigned=True).view(np.uint16), np.minimum(a16.view(np.uint16), b16.view(np.uint16)))
+    assert np.array_equal(orc.elementwise_binary("maximum", a16, b16, is_unsigned=True).view(np.uint16), np.maximum(a16.view(np.uint16), b16.view(np.uint16)))
+
+
 # ---- emitter ----------------------------------------------------------------------------------------------
 CASES = [lambda: w.fma_workload(), lambda: w.fma_workload((3, 5, 7), np.int16, np.int8, input_zp=11, scale=0.004, output_zp=-128),
          lambda: w.fma_workload((1000,), np.int32, np.int16, scale=0.0021, output_zp=0), lambda: w.fma_workload((37,), np.int8, np.int32, scale=3.7, weight=-2),
@@ -78,7 +95,10 @@ CASES = [lambda: w.fma_workload(), lambda: w.fma_workload((3, 5, 7), np.int16, n
          lambda: w.mul_workload((64,), np.int8, np.int8, scale=0.02, broadcast=1),
          lambda: w.act_workload("clamp"), lambda: w.act_workload("abs"), lambda: w.act_workload("negate", (77,), np.int16),
          lambda: w.act_workload("i2i", (5, 9), np.int32, np.int8), lambda: w.act_workload("i2i", (50,), np.int8, np.int32),
-         lambda: w.act_workload("abs", (19,), np.int8, np.int16), lambda: w.act_workload("clamp", (300,), np.int32, np.int16, min_int=-32768, max_int=1000)]
+         lambda: w.act_workload("abs", (19,), np.int8, np.int16), lambda: w.act_workload("clamp", (300,), np.int32, np.int16, min_int=-32768, max_int=1000),
+         lambda: w.binary_workload(0), lambda: w.binary_workload(1, (77,), np.int16), lambda: w.binary_workload(2, (5, 9), np.int32),
+         lambda: w.binary_workload(4), lambda: w.binary_workload(5, (1000,), np.int16, is_unsigned=True), lambda: w.binary_workload(4, (333,), np.int16, is_unsigned=True),
+         lambda: w.binary_workload(5, (4099,), np.int32)]
 
 
 @pytest.mark.parametrize("make", CASES)
@@ -136,6 +156,10 @@ def test_eltwise_rejections():
     expect(runtime.UNIMPLEMENTED, lambda p: p.act(p.binding(0, (8,)), "i2i", init=p.binding(1, (8,)), weights=one))
     expect(runtime.INVALID_ARGUMENT, lambda p: p.act(p.binding(0, (8,)), "clamp", min_int=-200, max_int=5, init=p.binding(1, (8,))))
     expect(runtime.INVALID_ARGUMENT, lambda p: p.act(p.binding(0, (8,)), "clamp", min_int=6, max_int=5, init=p.binding(1, (8,))))
+    expect(runtime.UNIMPLEMENTED, lambda p: p.elementwisebinary(6, p.binding(0, (8,)), p.binding(1, (8,)), init=p.binding(2, (8,))))   # GREATER
+    expect(runtime.UNIMPLEMENTED, lambda p: p.elementwisebinary(runtime.MINIMUM, p.binding(0, (8,)), p.binding(1, (8,)), is_unsigned=True, init=p.binding(2, (8,))))
+    expect(runtime.UNIMPLEMENTED, lambda p: p.elementwisebinary(runtime.MAXIMUM, p.binding(0, (8,)), p.binding(1, (8,), np.int16), init=p.binding(2, (8,))))
+    expect(runtime.INVALID_ARGUMENT, lambda p: p.elementwisebinary(runtime.MAXIMUM, p.binding(0, (8,)), p.binding(1, (9,)), init=p.binding(2, (8,))))
 
 
 # ---- GPU ---------------------------------------------------------------------------------------------------

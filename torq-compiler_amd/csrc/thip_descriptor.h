@@ -82,7 +82,8 @@ enum Kind : uint32_t {
     kKindAvgPoolBf16 = 12,    // bf16 global average pool: w0 = bf16 bits of the weight, bias0 = float bits of the bias
     // torq_hl.expand_weights: in0 int8 [K][Nn], scale bf16 [K / gran][Nn], bias float [K / gran][Np], out bf16 [K][Nn]
     kKindExpandWeights = 13,
-    // integer elementwise ops: variant = EltwiseOp (0 fma, 1 mul, 2 clamp, 3 abs, 4 negate, 5 i2i), C = element
+    // integer elementwise ops: variant = EltwiseOp (0 fma, 1 mul, 2 clamp, 3 abs, 4 negate, 5 i2i, 6 and, 7 or, 8 xor,
+    // 9 min, 10 max: two inputs of the output's type, w0 = compare as unsigned), C = element
     // count, gran = input element size, out_dtype, w0 = fma weight, w1 = mul broadcast (1: in0, 2: in1 has one
     // element), bias0 / scale0 / shift / output_zp / output_min / output_max = the ACT stage (fma, mul) or
     // output_min / output_max = the clip range (the others)

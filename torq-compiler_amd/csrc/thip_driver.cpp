@@ -292,12 +292,12 @@ static thip_status_t checkOpFootprint(const thip_executable_t *e, uint32_t i) {
     }
     case kKindEltwise: {
         const uint64_t inElem = op.gran, outElem = op.out_dtype == THIP_DTYPE_I8 ? 1 : op.out_dtype == THIP_DTYPE_I16 ? 2 : op.out_dtype == THIP_DTYPE_I32 ? 4 : 0;
-        if (!positive({op.C}) || !(inElem == 1 || inElem == 2 || inElem == 4) || outElem == 0 || op.variant > kEltCast || op.w1 < 0 || op.w1 > 2 ||
+        if (!positive({op.C}) || !(inElem == 1 || inElem == 2 || inElem == 4) || outElem == 0 || op.variant > kEltMax || op.w1 < 0 || op.w1 > 2 ||
             (op.variant != kEltMul && op.w1 != 0)) {
             return fail(THIP_INVALID_ARGUMENT, "op %u: bad elementwise record", i);
         }
         if ((s = need(op.in0, (op.w1 == 1 ? 1 : (uint64_t)op.C) * inElem, "in1"))) return s;
-        if (op.variant == kEltMul && (s = need(op.in1, (op.w1 == 2 ? 1 : (uint64_t)op.C) * inElem, "in2"))) return s;
+        if ((op.variant == kEltMul || op.variant >= kEltAnd) && (s = need(op.in1, (op.w1 == 2 ? 1 : (uint64_t)op.C) * inElem, "in2"))) return s;
         return need(op.out, (uint64_t)op.C * outElem, "out");
     }
     case kKindAddBf16: {
@@ -501,7 +501,7 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
         break;
     }
     case kKindEltwise: {
-        EltwiseArgs a{resolve(e, op.in0, bp), op.variant == kEltMul ? resolve(e, op.in1, bp) : nullptr, resolve(e, op.out, bp), (int64_t)op.C,
+        EltwiseArgs a{resolve(e, op.in0, bp), (op.variant == kEltMul || op.variant >= kEltAnd) ? resolve(e, op.in1, bp) : nullptr, resolve(e, op.out, bp), (int64_t)op.C,
                       (int32_t)op.variant, (int32_t)op.gran, op.out_dtype == THIP_DTYPE_I8 ? 1 : op.out_dtype == THIP_DTYPE_I16 ? 2 : 4, op.w1,
                       op.w0, op.bias0, op.scale0, op.output_min, op.output_max, rq};
         err = launchEltwise(a, e->stream);

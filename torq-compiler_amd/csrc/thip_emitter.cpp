@@ -44,7 +44,7 @@ struct Value {
     }
 };
 
-enum HlKind { kHlConv2d, kHlDepthwise, kHlFullyConnected, kHlMatmul, kHlMaxPool, kHlAvgPool, kHlAdd, kHlTranspose, kHlExpandWeights, kHlFma, kHlMul, kHlAct };
+enum HlKind { kHlConv2d, kHlDepthwise, kHlFullyConnected, kHlMatmul, kHlMaxPool, kHlAvgPool, kHlAdd, kHlTranspose, kHlExpandWeights, kHlFma, kHlMul, kHlAct, kHlBinary };
 
 struct HlOp {
     HlKind kind;
@@ -61,6 +61,7 @@ struct HlOp {
         thip_hl_fma_t fma;
         thip_hl_mul_t mul;
         thip_hl_act_t act;
+        thip_hl_elementwisebinary_t bin;
     } u;
     std::string name;
 };
@@ -530,6 +531,7 @@ class Emitter {
     thip_status_t emitFma(const thip_hl_fma_t &c);
     thip_status_t emitMul(const thip_hl_mul_t &c);
     thip_status_t emitAct(const thip_hl_act_t &c, const std::string &name);
+    thip_status_t emitBinary(const thip_hl_elementwisebinary_t &c);
     // Operands of an integer elementwise op: element types, and the record's common fields.
     thip_status_t eltwiseCommon(const char *what, thip_value_t input, thip_value_t init, DescOp *op);
     thip_status_t emitAvgPoolBf16(const thip_hl_avg_pool2d_t &c);
@@ -1396,6 +1398,34 @@ thip_status_t Emitter::emitMul(const thip_hl_mul_t &c) {
     return THIP_OK;
 }
 
+thip_status_t Emitter::emitBinary(const thip_hl_elementwisebinary_t &c) {
+    const char *what = "torq_hl.elementwisebinary";
+    uint32_t variant;
+    switch (c.op_type) {  // ElementwiseOpEnum, compiler/torq/Dialect/TorqHL/TorqHLAttrs.td:219-235
+    case 0: variant = kEltAnd; break;
+    case 1: variant = kEltOr; break;
+    case 2: variant = kEltXor; break;
+    case 4: variant = kEltMin; break;
+    case 5: variant = kEltMax; break;
+    default: return fail(THIP_UNIMPLEMENTED, "%s: op_type %d is not on this path (bitwise and / or / xor, minimum, maximum are)", what, (int)c.op_type);
+    }
+    const Value *a, *b, *init;
+    if (thip_status_t s = checkValue(c.input1, "torq_hl.elementwisebinary input1", &a)) return s;
+    if (thip_status_t s = checkValue(c.input2, "torq_hl.elementwisebinary input2", &b)) return s;
+    if (thip_status_t s = checkValue(c.init, "torq_hl.elementwisebinary init", &init)) return s;
+    if (!isIntDtype(a->dtype) || a->dtype != b->dtype || a->dtype != init->dtype) return fail(THIP_UNIMPLEMENTED, "%s: inputs and init must share one integer type", what);
+    if (a->numel() != b->numel() || a->numel() != init->numel()) return fail(THIP_INVALID_ARGUMENT, "%s: operand shapes differ (broadcast is materialised by the patterns)", what);
+    if (c.is_unsigned && a->dtype != THIP_DTYPE_I16) return fail(THIP_UNIMPLEMENTED, "%s: is_unsigned applies to 16-bit operands only", what);
+    if (state_[c.input2].nhwcOfNchw) return fail(THIP_UNIMPLEMENTED, "%s: N,C,H,W intermediates are not accepted", what);
+    DescOp op;
+    if (thip_status_t s = eltwiseCommon(what, c.input1, c.init, &op)) return s;
+    if (thip_status_t s = literalInput(c.input2, "torq_hl.elementwisebinary input2", &op.in1)) return s;
+    op.variant = variant;
+    op.w0 = c.is_unsigned ? 1 : 0;
+    ops_.push_back(op);
+    return THIP_OK;
+}
+
 thip_status_t Emitter::emitAct(const thip_hl_act_t &c, const std::string &name) {
     const char *what = "torq_hl.act";
     if (c.weights != THIP_NO_VALUE) return fail(THIP_UNIMPLEMENTED, "%s: weights (the unsigned cast) are not on this path", what);
@@ -1650,6 +1680,7 @@ void Emitter::planChannelPadding() {
         case kHlFma: bar(op.u.fma.input); bar(op.u.fma.init); break;
         case kHlMul: bar(op.u.mul.input1); bar(op.u.mul.input2); bar(op.u.mul.init); break;
         case kHlAct: bar(op.u.act.input); bar(op.u.act.init); break;
+        case kHlBinary: bar(op.u.bin.input1); bar(op.u.bin.input2); bar(op.u.bin.init); break;
         }
     }
     // one verdict per group: every member an int8 rank-4 intermediate, all uses agreeing on C
@@ -1701,6 +1732,7 @@ void Emitter::planExpandFolding() {
         case kHlFma: read(op.u.fma.input); break;
         case kHlMul: read(op.u.mul.input1); read(op.u.mul.input2); break;
         case kHlAct: read(op.u.act.input); break;
+        case kHlBinary: read(op.u.bin.input1); read(op.u.bin.input2); break;
         }
     }
     auto constant = [&](thip_value_t v) { return v >= 0 && (size_t)v < n && prog_.values[(size_t)v].kind == kValueConstant; };
@@ -1769,6 +1801,7 @@ thip_status_t Emitter::run(void **outBlob, size_t *outSize) {
         case kHlFma: s = emitFma(op.u.fma); break;
         case kHlMul: s = emitMul(op.u.mul); break;
         case kHlAct: s = emitAct(op.u.act, op.name); break;
+        case kHlBinary: s = emitBinary(op.u.bin); break;
         }
         if (s != THIP_OK) return s;
     }
@@ -1905,6 +1938,7 @@ THIP_DEFINE_HL(thip_hl_transpose, thip_hl_transpose_t, kHlTranspose, tr)
 THIP_DEFINE_HL(thip_hl_expand_weights, thip_hl_expand_weights_t, kHlExpandWeights, ew)
 THIP_DEFINE_HL(thip_hl_fma, thip_hl_fma_t, kHlFma, fma)
 THIP_DEFINE_HL(thip_hl_mul, thip_hl_mul_t, kHlMul, mul)
+THIP_DEFINE_HL(thip_hl_elementwisebinary, thip_hl_elementwisebinary_t, kHlBinary, bin)
 
 thip_status_t thip_hl_act(thip_program_t *program, const thip_hl_act_t *op) {
     if (!program || !op || !op->name) return fail(THIP_INVALID_ARGUMENT, "thip_hl_act: null argument");

@@ -157,10 +157,15 @@ hipError_t launchFcBf16(const FcBf16Args &a, hipStream_t stream);
 // Integer elementwise ops with the ACT stage behind them.  fma: out = R1(in0 * w0); mul: out = R1(in0 * in1) (an
 // input of one element is broadcast); both with ONE (bias, scale) pair.  clamp / abs / negate / i2i: the input
 // passed through the mode, then clipped to [lo, hi] and truncated to the output type.
-enum EltwiseOp : int32_t { kEltFma = 0, kEltMul = 1, kEltClamp = 2, kEltAbs = 3, kEltNegate = 4, kEltCast = 5 };
+// and / or / xor / min / max: two inputs and the output of one type, no ACT stage; w0 != 0 (16-bit only): min / max
+// compare as unsigned.
+enum EltwiseOp : int32_t {
+    kEltFma = 0, kEltMul = 1, kEltClamp = 2, kEltAbs = 3, kEltNegate = 4, kEltCast = 5,
+    kEltAnd = 6, kEltOr = 7, kEltXor = 8, kEltMin = 9, kEltMax = 10,
+};
 struct EltwiseArgs {
     const void *in0;
-    const void *in1;  // mul only
+    const void *in1;  // mul and the two-input ops
     void *out;
     int64_t count;
     int32_t op;

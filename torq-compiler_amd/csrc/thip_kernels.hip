@@ -2131,7 +2131,7 @@ __global__ __launch_bounds__(256) void eltwise_int(EltwiseArgs p) {
 #pragma unroll
         for (int v = 0; v < VEC; v++) a.e[v] = p.bcast == 1 ? in0[0] : (i0 + v < p.count ? in0[i0 + v] : (TIN)0);
     }
-    if (p.op == kEltMul) {
+    if (p.op == kEltMul || p.op >= kEltAnd) {
         if (whole && p.bcast != 2) {
             b = *(const EltVec<TIN, VEC> *)(in1 + i0);
         } else {
@@ -2151,6 +2151,15 @@ __global__ __launch_bounds__(256) void eltwise_int(EltwiseArgs p) {
                 o.e[v] = (TOUT)requantT0<kMode>(t0, p.scale, rnd, p.rq, wrq);
             }
         });
+    } else if (p.op >= kEltAnd) {
+        const int32_t mask = p.w0 ? 0xffff : -1;  // unsigned 16-bit comparison
+#pragma unroll
+        for (int v = 0; v < VEC; v++) {
+            const int32_t x = (int32_t)a.e[v], y = (int32_t)b.e[v];
+            const bool less = p.w0 ? (x & mask) < (y & mask) : x < y;
+            const int32_t r = p.op == kEltAnd ? (x & y) : p.op == kEltOr ? (x | y) : p.op == kEltXor ? (x ^ y) : (p.op == kEltMin) == less ? x : y;
+            o.e[v] = (TOUT)r;
+        }
     } else {
 #pragma unroll
         for (int v = 0; v < VEC; v++) {
@@ -2174,7 +2183,7 @@ __global__ __launch_bounds__(256) void eltwise_int(EltwiseArgs p) {
 template <typename TIN, typename TOUT>
 static hipError_t launchEltwiseT(const EltwiseArgs &a, hipStream_t stream) {
     constexpr int VEC = sizeof(TIN) == 1 && sizeof(TOUT) == 1 ? 16 : 8;
-    const uintptr_t bits = (uintptr_t)a.in0 | (a.op == kEltMul ? (uintptr_t)a.in1 : 0);
+    const uintptr_t bits = (uintptr_t)a.in0 | ((a.op == kEltMul || a.op >= kEltAnd) ? (uintptr_t)a.in1 : 0);
     const bool aligned = (bits & (sizeof(TIN) * VEC - 1)) == 0 && (((uintptr_t)a.out) & (sizeof(TOUT) * VEC - 1)) == 0;
     if (aligned) {
         const long long threads = (a.count + VEC - 1) / VEC;
@@ -2186,11 +2195,13 @@ static hipError_t launchEltwiseT(const EltwiseArgs &a, hipStream_t stream) {
 }
 
 hipError_t launchEltwise(const EltwiseArgs &a, hipStream_t stream) {
-    if (!a.in0 || !a.out || a.count <= 0 || a.count >= (1LL << 39) || a.op < kEltFma || a.op > kEltCast) return hipErrorInvalidValue;
-    if (a.op == kEltMul && (!a.in1 || a.bcast < 0 || a.bcast > 2)) return hipErrorInvalidValue;
+    if (!a.in0 || !a.out || a.count <= 0 || a.count >= (1LL << 39) || a.op < kEltFma || a.op > kEltMax) return hipErrorInvalidValue;
+    const bool two = a.op == kEltMul || a.op >= kEltAnd;
+    if (two && (!a.in1 || a.bcast < 0 || a.bcast > 2)) return hipErrorInvalidValue;
     if (a.op != kEltMul && a.bcast != 0) return hipErrorInvalidValue;
+    if (a.op >= kEltAnd && (a.in_bytes != a.out_bytes || (a.w0 != 0 && a.in_bytes != 2))) return hipErrorInvalidValue;
     if ((((uintptr_t)a.in0) & (a.in_bytes - 1)) || (((uintptr_t)a.out) & (a.out_bytes - 1))) return hipErrorInvalidValue;
-    if (a.op == kEltMul && (((uintptr_t)a.in1) & (a.in_bytes - 1))) return hipErrorInvalidValue;
+    if (two && (((uintptr_t)a.in1) & (a.in_bytes - 1))) return hipErrorInvalidValue;
     switch (a.in_bytes * 8 + a.out_bytes) {
     case 1 * 8 + 1: return launchEltwiseT<int8_t, int8_t>(a, stream);
     case 1 * 8 + 2: return launchEltwiseT<int8_t, int16_t>(a, stream);

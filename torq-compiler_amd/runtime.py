@@ -41,7 +41,7 @@ EXPORTED_SYMBOLS = [
     "thip_program_create", "thip_program_destroy", "thip_program_binding", "thip_program_constant",
     "thip_program_tensor", "thip_hl_conv2d", "thip_hl_depthwise_conv2d", "thip_hl_fully_connected",
     "thip_hl_matmul", "thip_hl_maxpool2d", "thip_hl_avg_pool2d", "thip_hl_add", "thip_hl_transpose", "thip_hl_expand_weights",
-    "thip_hl_fma", "thip_hl_mul", "thip_hl_act",
+    "thip_hl_fma", "thip_hl_mul", "thip_hl_act", "thip_hl_elementwisebinary",
     "thip_program_serialize", "thip_blob_free",
     "thip_device_create", "thip_device_destroy", "thip_device_name", "thip_device_alloc",
     "thip_device_free", "thip_device_h2d", "thip_device_d2h", "thip_device_synchronize",
@@ -154,7 +154,16 @@ class HlAct(ctypes.Structure):
     ]
 
 
+class HlElementwiseBinary(ctypes.Structure):
+    _fields_ = [
+        ("init", ctypes.c_int32), ("op_type", ctypes.c_int32), ("input1", ctypes.c_int32), ("input2", ctypes.c_int32),
+        ("is_unsigned", ctypes.c_int32),
+    ]
+
+
 NO_VALUE = -1
+# torq_hl.elementwisebinary op_type values on this path (the reference's ElementwiseOpEnum)
+BITWISE_AND, BITWISE_OR, BITWISE_XOR, MINIMUM, MAXIMUM = 0, 1, 2, 4, 5
 
 
 class HlAdd(ctypes.Structure):
@@ -206,7 +215,7 @@ def lib():
                      ("thip_hl_maxpool2d", HlMaxPool2d), ("thip_hl_avg_pool2d", HlAvgPool2d),
                      ("thip_hl_add", HlAdd), ("thip_hl_transpose", HlTranspose),
                      ("thip_hl_expand_weights", HlExpandWeights), ("thip_hl_fma", HlFma), ("thip_hl_mul", HlMul),
-                     ("thip_hl_act", HlAct)]:
+                     ("thip_hl_act", HlAct), ("thip_hl_elementwisebinary", HlElementwiseBinary)]:
         getattr(L, name).argtypes = [vp, P(st)]
     L.thip_program_serialize.argtypes = [vp, P(vp), P(sz)]
     L.thip_blob_free.argtypes = [vp]

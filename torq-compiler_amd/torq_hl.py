@@ -259,6 +259,14 @@ class Program:
         rt.check(rt.lib().thip_hl_act(self._h, ctypes.byref(op)))
         return init
 
+    def elementwisebinary(self, op_type, input1, input2, *, is_unsigned=False, init=None):
+        """torq_hl.elementwisebinary: op_type one of runtime.BITWISE_AND / _OR / _XOR / MINIMUM / MAXIMUM."""
+        input2 = self._as_value(input2)
+        init = self._init_or_new(init, input1.shape, input1.dtype)
+        op = rt.HlElementwiseBinary(init.index, int(op_type), input1.index, input2.index, int(bool(is_unsigned)))
+        rt.check(rt.lib().thip_hl_elementwisebinary(self._h, ctypes.byref(op)))
+        return init
+
     def transpose(self, input, perm, init=None):
         shape = tuple(input.shape[p] for p in perm)
         init = self._init_or_new(init, shape, input.dtype)

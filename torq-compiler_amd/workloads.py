@@ -428,6 +428,21 @@ def mul_workload(shape=(1, 56, 56, 24), in_dtype=np.int8, out_dtype=np.int8, sca
     return Workload("mul_%s_%s_%d_b%d" % (np.dtype(in_dtype).name, np.dtype(out_dtype).name, count, broadcast), p, [a, b], [(shape, out_dtype)], 3 * count, nbytes, attrs)
 
 
+def binary_workload(op_type=4, shape=(1, 56, 56, 24), dtype=np.int8, is_unsigned=False, seed=1021):
+    """torq_hl.elementwisebinary: op_type 0 and, 1 or, 2 xor, 4 minimum, 5 maximum."""
+    rng = np.random.default_rng(seed)
+    a = _random_ints(rng, shape, dtype)
+    b = _random_ints(rng, shape, dtype)
+    p = Program()
+    i0 = p.binding(0, shape, dtype)
+    i1 = p.binding(1, shape, dtype)
+    out = p.binding(2, shape, dtype)
+    p.elementwisebinary(op_type, i0, i1, is_unsigned=is_unsigned, init=out)
+    attrs = dict(op_type={0: "and", 1: "or", 2: "xor", 4: "minimum", 5: "maximum"}[op_type], is_unsigned=is_unsigned)
+    return Workload("binary_%s_%s_%d_u%d" % (attrs["op_type"], np.dtype(dtype).name, a.size, int(is_unsigned)), p, [a, b], [(shape, dtype)], a.size,
+                    3 * a.nbytes, attrs)
+
+
 def act_workload(name="clamp", shape=(1, 56, 56, 24), in_dtype=np.int8, out_dtype=None, min_int=-20, max_int=90, seed=1018):
     """torq_hl.act on integers: clamp / abs / negate / i2i."""
     rng = np.random.default_rng(seed)
