@@ -441,8 +441,12 @@ thip_status_t thip_executable_binding_count(thip_executable_t *executable, uint3
 thip_status_t thip_executable_binding_size(thip_executable_t *executable, uint32_t binding,
                                            size_t *out_size);
 
-/* Per-dispatch event log (role of TorqEventLog, runtime/torq_hw/inc/TorqEventLog.h:19-46):
- * when a path is set every run appends BEGIN/END rows per op as CSV. */
+/* Per-dispatch event log (role of TorqEventLog, runtime/torq_hw/inc/TorqEventLog.h:19-46, .cpp:48,97-101): when a
+ * path is set every dispatch appends rows in the reference's runtime CSV columns (doc/user-manual/profiling.md:53-63)
+ * dispatch_name, invocation_id, action_id, timestamp_us, event -- event an EventType name plus _BEGIN / _END:
+ * DISPATCH, DISPATCH_SYNC_BINDINGS_IN / _OUT, DISPATCH_EXECUTE_ACTIONS, NSS_START per kernel launch (action_id = the
+ * op's index), NSS_WAIT -- and a sixth column, kernel, naming the kernel of a launch row.  An empty path closes the
+ * log.  While a log is open dispatches are not replayed as graphs. */
 thip_status_t thip_device_set_event_log(thip_device_t *device, const char *csv_path);
 
 #ifdef __cplusplus

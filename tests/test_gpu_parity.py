@@ -375,9 +375,24 @@ def test_event_log_and_timing(device, tmp_path):
     ms = exe.time_device([pin, pout], [x.nbytes, int(np.prod(wl.outputs[0][0]))], 5)
     device.set_event_log("")
     assert ms > 0
-    rows = log.read_text().strip().splitlines()
-    assert rows[0] == "time_us,op,kernel,phase" and len(rows) == 1 + 2 * 5
-    assert "maxpool_i8,BEGIN" in rows[1] and "maxpool_i8,END" in rows[2]
+    # the reference's runtime CSV columns, plus the kernel name
+    import csv
+    rows = list(csv.DictReader(log.open()))
+    assert list(rows[0].keys()) == ["dispatch_name", "invocation_id", "action_id", "timestamp_us", "event", "kernel"]
+    assert len(rows) == 2 * 5 and [r["event"] for r in rows[:2]] == ["NSS_START_BEGIN", "NSS_START_END"]
+    assert all(r["kernel"] == "maxpool_i8" and r["action_id"] == "0" for r in rows)
+    assert [int(r["invocation_id"]) for r in rows] == [i // 2 for i in range(10)]
+    assert all(int(a["timestamp_us"]) <= int(b["timestamp_us"]) for a, b in zip(rows, rows[1:]))
+    # a blocking run on host buffers logs the whole dispatch
+    device.set_event_log(str(log))
+    host_out = np.zeros(wl.outputs[0][0], dtype=np.int8)
+    exe.run_host([x, host_out])
+    device.set_event_log("")
+    events = [r["event"] for r in csv.DictReader(log.open())]
+    assert events == ["DISPATCH_BEGIN", "DISPATCH_SYNC_BINDINGS_IN_BEGIN", "DISPATCH_SYNC_BINDINGS_IN_END", "DISPATCH_EXECUTE_ACTIONS_BEGIN",
+                      "NSS_START_BEGIN", "NSS_START_END", "DISPATCH_EXECUTE_ACTIONS_END", "DISPATCH_SYNC_BINDINGS_OUT_BEGIN", "NSS_WAIT_BEGIN",
+                      "NSS_WAIT_END", "DISPATCH_SYNC_BINDINGS_OUT_END", "DISPATCH_END"]
+    assert_bit_exact(host_out, oracle_eval(wl)[0], "logged run")
     got = device.download(pout, wl.outputs[0][0], np.int8)
     assert_bit_exact(got, oracle_eval(wl)[0], "timed maxpool")
     device.free(pin)

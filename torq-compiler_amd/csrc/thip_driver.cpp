@@ -59,6 +59,7 @@ struct thip_executable_t {
     hipGraph_t graph = nullptr;
     hipGraphExec_t graphExec = nullptr;
     bool graphsDisabled = false;
+    uint64_t invocation = 0;             // dispatches so far (the event log's invocation_id)
 };
 
 static thip_status_t hipFail(hipError_t e, const char *what) {
@@ -353,11 +354,14 @@ static const char *opKernelName(const DescOp &op) {
     }
 }
 
-static void logEvent(thip_device_t *d, uint32_t opIndex, const char *name, const char *phase) {
+// One row of the event log, in the reference's runtime CSV columns (doc/user-manual/profiling.md:53-63, written by
+// runtime/torq_hw/src/TorqEventLog.cpp:48,97-101): dispatch_name, invocation_id, action_id, timestamp_us, event
+// (an EventType name + _BEGIN / _END), plus one column of this backend's own: the kernel of a launch row.
+static void logEvent(thip_device_t *d, uint64_t invocation, int32_t action, const char *event, const char *phase, const char *kernel) {
     if (!d->eventLog) return;
     std::lock_guard<std::mutex> lock(d->logMutex);
     const auto us = std::chrono::duration_cast<std::chrono::microseconds>(std::chrono::steady_clock::now() - d->t0).count();
-    fprintf(d->eventLog, "%lld,%u,%s,%s\n", (long long)us, opIndex, name, phase);
+    fprintf(d->eventLog, "thip_dispatch,%llu,%d,%lld,%s_%s,%s\n", (unsigned long long)invocation, action, (long long)us, event, phase, kernel);
 }
 
 // Resolves an operand reference against the buffers of this dispatch.
@@ -556,9 +560,10 @@ static thip_status_t checkState(const thip_executable_t *e, const thip_dispatch_
 // Enqueues every kernel record of the program.  `bp` holds one device pointer per binding.
 static thip_status_t enqueueOps(thip_executable_t *e, uint8_t *const *bp) {
     for (uint32_t i = 0; i < e->header.op_count; i++) {
-        logEvent(e->device, i, opKernelName(e->ops[i]), "BEGIN");
+        // a kernel launch is what starting an NSS task is on the reference's hardware
+        logEvent(e->device, e->invocation, (int32_t)i, "NSS_START", "BEGIN", opKernelName(e->ops[i]));
         if (thip_status_t s = launchOp(e, i, bp)) return s;
-        logEvent(e->device, i, opKernelName(e->ops[i]), "END");
+        logEvent(e->device, e->invocation, (int32_t)i, "NSS_START", "END", opKernelName(e->ops[i]));
     }
     return THIP_OK;
 }
@@ -692,7 +697,7 @@ thip_status_t thip_device_set_event_log(thip_device_t *device, const char *csv_p
     if (csv_path && csv_path[0]) {
         device->eventLog = fopen(csv_path, "w");
         if (!device->eventLog) return fail(THIP_INVALID_ARGUMENT, "cannot open event log %s", csv_path);
-        fprintf(device->eventLog, "time_us,op,kernel,phase\n");
+        fprintf(device->eventLog, "dispatch_name,invocation_id,action_id,timestamp_us,event,kernel\n");
     }
     return THIP_OK;
 }
@@ -777,6 +782,9 @@ thip_status_t thip_executable_create(thip_device_t *device, const void *blob, si
 static thip_status_t runLocked(thip_executable_t *e, const thip_dispatch_state_t *st) {
     THIP_HIP(hipSetDevice(e->device->ordinal), "hipSetDevice");
     uint8_t *bp[64] = {nullptr};
+    const int32_t lastOp = (int32_t)e->header.op_count - 1;
+    logEvent(e->device, e->invocation, 0, "DISPATCH", "BEGIN", "");
+    logEvent(e->device, e->invocation, 0, "DISPATCH_SYNC_BINDINGS_IN", "BEGIN", "");
     // writeInputs: host bindings are staged into device memory (TorqExecutable::writeInputs)
     for (uint32_t i = 0; i < e->header.binding_count; i++) {
         if (e->bindings[i].flags == 0) continue;
@@ -793,21 +801,32 @@ static thip_status_t runLocked(thip_executable_t *e, const thip_dispatch_state_t
             THIP_HIP(hipMemcpyAsync(bp[i], st->binding_ptrs[i], e->bindings[i].size, hipMemcpyHostToDevice, e->stream), "staging a binding");
         }
     }
+    logEvent(e->device, e->invocation, 0, "DISPATCH_SYNC_BINDINGS_IN", "END", "");
     bool allDevice = true;
     for (uint32_t i = 0; i < e->header.binding_count; i++) {
         if (e->bindings[i].flags != 0 && !(st->binding_flags && (st->binding_flags[i] & THIP_BINDING_DEVICE))) allDevice = false;
     }
+    logEvent(e->device, e->invocation, 0, "DISPATCH_EXECUTE_ACTIONS", "BEGIN", "");
     if (thip_status_t s = allDevice ? enqueueDevice(e, bp) : enqueueOps(e, bp)) {
         (void)hipStreamSynchronize(e->stream);
+        e->invocation++;
         return s;
     }
+    logEvent(e->device, e->invocation, lastOp, "DISPATCH_EXECUTE_ACTIONS", "END", "");
+    logEvent(e->device, e->invocation, lastOp, "DISPATCH_SYNC_BINDINGS_OUT", "BEGIN", "");
     // readOutputs (TorqExecutable::readOutputs, runtime/driver/TorqExecutable.cc:860-918)
     for (uint32_t i = 0; i < e->header.binding_count; i++) {
         const bool isDevice = st->binding_flags && (st->binding_flags[i] & THIP_BINDING_DEVICE);
         if (isDevice || !(e->bindings[i].flags & kBindingWritten)) continue;
         THIP_HIP(hipMemcpyAsync(st->binding_ptrs[i], bp[i], e->bindings[i].size, hipMemcpyDeviceToHost, e->stream), "reading back a binding");
     }
-    THIP_HIP(hipStreamSynchronize(e->stream), "waiting for the dispatch");
+    logEvent(e->device, e->invocation, lastOp, "NSS_WAIT", "BEGIN", "");
+    const hipError_t waited = hipStreamSynchronize(e->stream);
+    logEvent(e->device, e->invocation, lastOp, "NSS_WAIT", "END", "");
+    logEvent(e->device, e->invocation, lastOp, "DISPATCH_SYNC_BINDINGS_OUT", "END", "");
+    logEvent(e->device, e->invocation, lastOp, "DISPATCH", "END", "");
+    e->invocation++;
+    THIP_HIP(waited, "waiting for the dispatch");
     return THIP_OK;
 }
 
@@ -825,7 +844,9 @@ thip_status_t thip_executable_enqueue(thip_executable_t *e, const thip_dispatch_
     THIP_HIP(hipSetDevice(e->device->ordinal), "hipSetDevice");
     uint8_t *bp[64] = {nullptr};
     for (uint32_t i = 0; i < e->header.binding_count; i++) bp[i] = (uint8_t *)st->binding_ptrs[i];
-    return enqueueDevice(e, bp);
+    const thip_status_t s = enqueueDevice(e, bp);
+    e->invocation++;
+    return s;
 }
 
 thip_status_t thip_executable_wait(thip_executable_t *e) {
@@ -844,7 +865,9 @@ thip_status_t thip_executable_time(thip_executable_t *e, const thip_dispatch_sta
     for (uint32_t i = 0; i < e->header.binding_count; i++) bp[i] = (uint8_t *)st->binding_ptrs[i];
     THIP_HIP(hipEventRecord(e->evStart, e->stream), "hipEventRecord");
     for (int32_t it = 0; it < iterations; it++) {
-        if (thip_status_t s = enqueueDevice(e, bp)) {
+        const thip_status_t s = enqueueDevice(e, bp);
+        e->invocation++;
+        if (s != THIP_OK) {
             (void)hipStreamSynchronize(e->stream);
             return s;
         }
