@@ -162,7 +162,45 @@ def test_eltwise_rejections():
     expect(runtime.INVALID_ARGUMENT, lambda p: p.elementwisebinary(runtime.MAXIMUM, p.binding(0, (8,)), p.binding(1, (9,)), init=p.binding(2, (8,))))
 
 
+TRANSPOSES = [((5, 9), (1, 0), np.int8), ((70, 130), (1, 0), np.uint16), ((3, 33, 65), (0, 2, 1), np.int16), ((2, 5, 6, 7), (0, 2, 3, 1), np.int8),
+              ((2, 6, 7, 5), (0, 3, 1, 2), np.uint16), ((1, 24, 56, 56), (0, 2, 3, 1), np.int8)]
+
+
+def _transpose_program(shape, perm, dtype, seed=9):
+    rng = np.random.default_rng(seed)
+    info = np.iinfo(dtype)
+    x = rng.integers(info.min, info.max, size=shape, endpoint=True).astype(dtype)
+    p = Program()
+    out_shape = tuple(shape[i] for i in perm)
+    p.transpose(p.binding(0, shape, dtype), perm, init=p.binding(1, out_shape, dtype))
+    return p, x, np.ascontiguousarray(x.transpose(perm))
+
+
+@pytest.mark.parametrize("shape,perm,dtype", TRANSPOSES)
+def test_transpose_op_descriptor(shape, perm, dtype):
+    """torq_hl.transpose between bindings, 8- and 16-bit elements (bf16 bit patterns travel as uint16)."""
+    p, x, want = _transpose_program(shape, perm, dtype)
+    got = np.zeros(want.shape, dtype=dtype)
+    d = desc_interp.run(p.serialize(), [x, got])
+    assert np.array_equal(got, want)
+    assert [int(o["kind"]) for o in d.ops] == [desc_interp.K_TRANSPOSE]
+
+
 # ---- GPU ---------------------------------------------------------------------------------------------------
+@pytest.mark.gpu
+def test_gpu_transpose_op(device):
+    from torq_compiler_amd import Executable
+    for shape, perm, dtype in TRANSPOSES + [((4, 144, 28, 28), (0, 2, 3, 1), np.uint16), ((1000, 3000), (1, 0), np.int8)]:
+        p, x, want = _transpose_program(shape, perm, dtype)
+        print("[gpu-case] transpose", shape, perm, np.dtype(dtype).name, flush=True)
+        exe = Executable(device, p.serialize())
+        got = np.zeros(want.shape, dtype=dtype)
+        exe.run_host([x, got])
+        exe.close()
+        assert np.array_equal(got, want)
+
+
+
 @pytest.mark.gpu
 def test_gpu_eltwise(device):
     """Every case of the emitter test, plus sizes that exercise whole vectors, the ragged tail and both requant tails

@@ -1554,7 +1554,9 @@ thip_status_t Emitter::emitTransposeOp(const thip_hl_transpose_t &c) {
     const Value *x, *init;
     if (thip_status_t s = checkValue(c.input, "torq_hl.transpose input", &x)) return s;
     if (thip_status_t s = checkValue(c.init, "torq_hl.transpose init", &init)) return s;
-    if (x->dtype != THIP_DTYPE_I8 || init->dtype != THIP_DTYPE_I8) return fail(THIP_UNIMPLEMENTED, "%s: only int8 tensors", what);
+    const uint32_t elem = (uint32_t)elemSize(x->dtype);
+    if (x->dtype != init->dtype || (elem != 1 && elem != 2)) return fail(THIP_UNIMPLEMENTED, "%s: 8- and 16-bit tensors of one type only", what);
+    const int32_t dt = x->dtype;
     if (c.rank != x->rank || c.rank != init->rank) return fail(THIP_INVALID_ARGUMENT, "%s: rank mismatch", what);
     for (int i = 0; i < c.rank; i++) {
         if (c.perm[i] < 0 || c.perm[i] >= c.rank || init->shape[i] != x->shape[c.perm[i]]) {
@@ -1599,15 +1601,15 @@ thip_status_t Emitter::emitTransposeOp(const thip_hl_transpose_t &c) {
             // bytes are already N,H,W,C: copy through a double transpose is wasteful, but
             // a binding destination needs its own bytes; use add-free copy = transpose with R == 1
             DescRef out;
-            if (thip_status_t s = literalOutput(c.init, "torq_hl.transpose init", THIP_DTYPE_I8, x->numel(), &out)) return s;
-            emitTranspose(in, out, 1, 1, x->numel());
+            if (thip_status_t s = literalOutput(c.init, "torq_hl.transpose init", dt, x->numel(), &out)) return s;
+            emitTranspose(in, out, 1, 1, x->numel(), elem);
             return THIP_OK;
         }
         return fail(THIP_UNIMPLEMENTED, "%s: permutation of an N,C,H,W intermediate other than [0,2,3,1]", what);
     }
     DescRef out;
-    if (thip_status_t s = literalOutput(c.init, "torq_hl.transpose init", THIP_DTYPE_I8, x->numel(), &out)) return s;
-    emitTranspose(in, out, B, R, S);
+    if (thip_status_t s = literalOutput(c.init, "torq_hl.transpose init", dt, x->numel(), &out)) return s;
+    emitTranspose(in, out, B, R, S, elem);
     return THIP_OK;
 }
 
