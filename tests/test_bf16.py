@@ -305,7 +305,7 @@ def test_gpu_expand_weights(device):
     N, an expansion clamp), expanded at serialisation (many rows), and as a kernel of its own, whose result is bit-exact."""
     f = lambda bits: np.abs(orc.from_bf16(bits).astype(np.float64))
     cases = [(w.expand_weights_workload(), "q8"), (w.expand_weights_workload(M=1, K=1152, N=1024, block=128), "q8"),
-             (w.expand_weights_workload(M=32, K=6912, N=1152, block=64), "q8"), (w.expand_weights_workload(M=5, K=192, N=45, block=96, bias_pad=1), "q8"),
+             (w.expand_weights_workload(M=32, K=6912, N=1152, block=64), "q8"), (w.expand_weights_workload(M=9, K=6912, N=200, block=128), "q8"), (w.expand_weights_workload(M=5, K=192, N=45, block=96, bias_pad=1), "q8"),
              (w.expand_weights_workload(M=7, K=128, N=70, expand_clamp=(-0.004, 0.006), clamp=(-0.05, 0.05)), "q8"),
              (w.expand_weights_workload(M=70, K=128, N=40, block=64), "folded"), (w.expand_weights_workload(M=2, K=64, N=33, fold=False, bias_pad=1), "own")]
     for wl, how in cases:
@@ -337,9 +337,10 @@ def test_gpu_bf16_add(device):
 def test_gpu_bf16_split_k_is_deterministic(device):
     """Few output tiles and a long K: K is split over blocks whose partial sums the last block to arrive adds in a
     fixed order; repeated dispatches give the same bits, and the counters are back at zero for the next one."""
-    wl = w.fully_connected_bf16_workload(32, 6912, 1152)
+    wl = w.fully_connected_bf16_workload(32, 6912, 256)
     d = desc_interp.Descriptor(wl.program.serialize())
     assert int(d.ops[0]["w0"]) > 1
+    assert int(desc_interp.Descriptor(w.fully_connected_bf16_workload(32, 6912, 1152).program.serialize()).ops[0]["w0"]) == 1  # enough tiles: no split
     first = _check_gpu(device, wl, via="device")
     exe = Executable(device, wl.program.serialize())
     for _ in range(5):

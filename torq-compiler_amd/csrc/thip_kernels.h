@@ -146,7 +146,9 @@ inline size_t fcBf16WorkspaceBytes(int M, int N, int ksplit) {
 inline int fcBf16PreferredSplit(int M, int N, int K) {
     const long long tiles = (long long)((N + 31) / 32) * ((M + 31) / 32);
     const int steps = (K + 63) / 64;
-    if (tiles >= 128 || steps < 8) return 1;
+    // the fenced write-back / counter / read-back chain costs 4-7 us: it only pays when a handful of tiles would
+    // otherwise walk a long K alone (6912 -> 256: 12 us split, 16-21 us not; 6912 -> 1152 and everything shorter: even or worse)
+    if (tiles > 16 || steps < 64) return 1;
     long long split = 256 / tiles;  // at most one block per CU: a second round would double the time
     if (split > steps / 4) split = steps / 4;
     if (split > 16) split = 16;

@@ -2311,7 +2311,9 @@ __device__ __forceinline__ void fcBf16Store(const FcBf16Args &p, const v16f &acc
     }
 }
 
-template <int NWAVES, int Q8>  // waves of a block = ways K is split; Q8: 0 bf16 weights, 1 int8 expanded, 2 with clamp
+// waves of a block = ways K is split; Q8: 0 bf16 weights, 1 int8 expanded, 2 with clamp; UNR: k-steps whose loads are
+// in flight together (6 for the small grids of a decoder's linears: a wave's whole share of K <= 1536 in one round trip)
+template <int NWAVES, int Q8, int UNR = 4>
 __global__ __launch_bounds__(NWAVES * 64) void fc_bf16(FcBf16Args p, FastDiv qblk) {
     __shared__ float partial[NWAVES - 1][16][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -2330,7 +2332,6 @@ __global__ __launch_bounds__(NWAVES * 64) void fc_bf16(FcBf16Args p, FastDiv qbl
 #pragma unroll
     for (int e = 0; e < 16; e++) acc[e] = 0.0f;
     // UNR steps of loads are issued before their MFMAs: one memory round trip per UNR * 64 elements of K
-    constexpr int UNR = NWAVES > 4 ? 2 : 4;
     for (int s0 = sBeg; s0 < sEnd; s0 += UNR) {
         v4i wv[Q8 ? 1 : UNR][4], xv[UNR][4];
         v4i wq[Q8 ? UNR : 1][2];
@@ -2540,6 +2541,9 @@ hipError_t launchFcBf16(const FcBf16Args &a, hipStream_t stream) {
     if (a.ksplit < 1 || a.ksplit > 64 || (a.ksplit > 1 && (!a.workspace || ((uintptr_t)a.workspace & 255)))) return hipErrorInvalidValue;
     const dim3 grid((unsigned)((a.N + 31) / 32), (unsigned)((a.M + 31) / 32), (unsigned)a.ksplit);
     if (grid.y > 65535) return hipErrorInvalidValue;
+    // few blocks (registers do not limit anything then) and 5 or 6 k-steps per wave: one deeper round of loads instead of two
+    const int stepsPerWave = (((a.K + 63) / 64 + a.ksplit - 1) / a.ksplit + 3) / 4;
+    const bool deep = (long long)grid.x * grid.y * grid.z <= 512 && stepsPerWave > 4 && stepsPerWave <= 6 && !getenv("THIP_NO_FC_DEEP");
     // a very wide N with a short K and no K split: every wave streams its own columns (THIP_NO_FC_WIDE: off)
     const bool wide = a.w_fragments >= 1 && a.ksplit == 1 && (a.K + 63) / 64 <= kFcBf16WideMaxSteps && (a.N + 31) / 32 >= 1024 &&
                       !getenv("THIP_NO_FC_WIDE");
@@ -2550,11 +2554,13 @@ hipError_t launchFcBf16(const FcBf16Args &a, hipStream_t stream) {
         const bool clamp = !(a.qlo == -INFINITY && a.qhi == INFINITY);
         if (wide) return clamp ? launchFcBf16Wide<2>(a, blk, stream) : launchFcBf16Wide<1>(a, blk, stream);
         if (clamp) hipLaunchKernelGGL((fc_bf16<4, 2>), grid, dim3(256), 0, stream, a, blk);
+        else if (deep) hipLaunchKernelGGL((fc_bf16<4, 1, 6>), grid, dim3(256), 0, stream, a, blk);
         else hipLaunchKernelGGL((fc_bf16<4, 1>), grid, dim3(256), 0, stream, a, blk);
         return hipGetLastError();
     }
     if (wide) return launchFcBf16Wide<0>(a, makeFastDiv(1), stream);
-    hipLaunchKernelGGL((fc_bf16<4, 0>), grid, dim3(256), 0, stream, a, makeFastDiv(1));
+    if (deep) hipLaunchKernelGGL((fc_bf16<4, 0, 6>), grid, dim3(256), 0, stream, a, makeFastDiv(1));
+    else hipLaunchKernelGGL((fc_bf16<4, 0>), grid, dim3(256), 0, stream, a, makeFastDiv(1));
     return hipGetLastError();
 }
 
