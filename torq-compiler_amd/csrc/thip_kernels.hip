@@ -1818,7 +1818,9 @@ hipError_t launchDepthwise(const DepthwiseArgs &a, hipStream_t stream) {
         const bool tileOff = tileEnv && tileEnv[0] == '0', tileOn = tileEnv && tileEnv[0] == '1';
         if (!tileOff) {
             // 16 channels per thread: 8 or 4 (more waves, fewer registers) measured 5 % and 12 % slower
-            if (a.SW == 1 && a.SH == 1 && (tileOn || outputs >= 8 * 4 * 65536)) return launchDepthwiseTile<4, 2, 1, 4>(a, stream);
+            const char *thr = getenv("THIP_DEPTHWISE_TILE_MIN");
+            const long long tileMin = thr ? atoll(thr) : 8 * 65536;  // measured on a mobile network at batch 32 and 256: even or ahead from about half a million thread-outputs
+            if (a.SW == 1 && a.SH == 1 && (tileOn || outputs >= tileMin)) return launchDepthwiseTile<4, 2, 1, 4>(a, stream);
         }
         // pixels per thread (THIP_DEPTHWISE_P forces 1, 2 or 4, for tuning)
         int pix = outputs >= 4 * 65536 ? 4 : outputs >= 2 * 65536 ? 2 : 1;
