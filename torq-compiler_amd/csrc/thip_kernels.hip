@@ -377,7 +377,7 @@ struct FastDiv {
     uint32_t shift;  // s - 1
     uint32_t d;
 };
-static FastDiv makeFastDiv(uint32_t d) {
+__host__ __device__ static inline FastDiv makeFastDiv(uint32_t d) {
     FastDiv f{0, 0, d};
     if (d <= 1) return f;
     uint32_t s = 0;
@@ -985,13 +985,16 @@ __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArg
         int iy0, ix0;
         size_t base;
     };
+    // pixel index -> (image, row, column) with multiply-shift divisions (M < 2^31): two run-time integer divisions
+    // per group cost this loader about a fifth of its instructions
+    const FastDiv divPlane = makeFastDiv(LOADER == kLoaderRuns ? (uint32_t)(p.OH * p.OW) : 1u), divOw = makeFastDiv(LOADER == kLoaderRuns ? (uint32_t)p.OW : 1u);
     auto locate = [&](int g) -> Pos {
         if (LOADER != kLoaderRuns) return Pos{0, 0, 0};
         int m = g * 32 + fr;
         m = m < p.M ? m : p.M - 1;
         const int plane = p.OH * p.OW;
-        const int img = m / plane, rem = m - img * plane;
-        const int oy = rem / p.OW, ox = rem - oy * p.OW;
+        const int img = (int)fastDiv((uint32_t)m, divPlane), rem = m - img * plane;
+        const int oy = (int)fastDiv((uint32_t)rem, divOw), ox = rem - oy * p.OW;
         return Pos{oy * p.SH - p.PT, ox * p.SW - p.PL, (size_t)img * p.H * p.W * p.C};
     };
     const uint32_t zpb = (uint32_t)(p.input_zp & 0xff);
