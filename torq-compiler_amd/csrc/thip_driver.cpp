@@ -161,7 +161,7 @@ static thip_status_t checkOpFootprint(const thip_executable_t *e, uint32_t i) {
     };
     const uint64_t outElem = op.out_dtype == THIP_DTYPE_I32 ? 4 : op.out_dtype == THIP_DTYPE_I16 ? 2 : 1;
     thip_status_t s = THIP_OK;
-    if (op.pre_shift != 0 && (op.pre_shift < 0 || op.shift + op.pre_shift != 33 ||
+    if (op.pre_shift != 0 && (op.pre_shift < 0 || op.pre_shift > 30 || op.shift + op.pre_shift != 33 ||
                               (op.kind != kKindIgemm && op.kind != kKindDepthwise))) {
         return fail(THIP_INVALID_ARGUMENT, "op %u: pre_shift %d does not complete shift %d to 33", i, op.pre_shift, op.shift);
     }

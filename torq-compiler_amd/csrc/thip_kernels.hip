@@ -50,29 +50,37 @@ __device__ __forceinline__ int32_t requant(int32_t acc, int32_t bias, int32_t sc
 // is the same number, provided t0 * 2^pre still fits 32 bits; whoever fills rq.pre_shift has
 // bounded |t0| from the weights and the bias to make sure of that, or passes rq.t0_clamp: t0 is
 // then clamped to a range that fits, chosen so wide that every result outside it is saturated by
-// the output clamp anyway (the result is monotonic in t0).
+// the output clamp anyway (the result is monotonic in t0).  Where no clamp is needed the kernels do not shift
+// at all: the bound says that the result fits 32 bits, so it is read out of the 64-bit sum directly
+// (requantPreShift).  shift == 32 needs neither: the result is the high word of product + 2^31.
 struct WideRequant {
-    bool on;  // rq.shift + rq.pre_shift >= 33
+    bool on;  // rq.shift + rq.pre_shift >= 33, or rq.shift == 32
     int pre, shiftMinus32;
     int32_t rnd, lo, hi, zp;
-    long long rnd64;     // rnd * 2^32: added to the 64-bit product, it adds rnd to the product's high word
+    long long rnd64;     // added to the 64-bit product: rnd * 2^32 adds rnd to the product's high word
     int32_t t0lo, t0hi;  // clamp of acc + bias (the whole int32 range when rq.t0_clamp == 0)
     bool plain;          // on, pre == 0, no clamp of t0, zero point folded: requantWideT0<true> applies
     bool preOnly;        // on, pre > 0, no clamp of t0, zero point folded: requantPreShift applies
+    int alignShift;      // preOnly: rq.shift (3..31)
+    long long rndAlign;  // preOnly: 2^(shift-1) + zp * 2^shift, added to the product before its bits [shift, shift+32) are taken
 };
 __device__ __forceinline__ WideRequant wideRequant(const Requant &rq) {
     WideRequant w;
-    const int sh = rq.shift + rq.pre_shift;
-    w.on = sh >= 33;
-    w.pre = rq.pre_shift;
+    // shift == 32: the result is the high word of product + 2^31, exact for every acc + bias; a pre-shift or a clamp
+    // of acc + bias that the op carries is not needed (either changes nothing in the result)
+    const bool whole = rq.shift == 32;
+    const int sh = whole ? 32 : rq.shift + rq.pre_shift;
+    w.on = sh >= 32;
+    w.pre = whole ? 0 : rq.pre_shift;
     w.shiftMinus32 = sh - 32;
-    w.rnd = w.on ? (int32_t)(1u << (sh - 33)) : 0;
+    w.rnd = sh >= 33 ? (int32_t)(1u << (sh - 33)) : 0;
     const long long lo64 = (long long)rq.out_min - rq.out_zp, hi64 = (long long)rq.out_max - rq.out_zp;
     w.lo = (int32_t)(lo64 < INT32_MIN ? INT32_MIN : lo64);
     w.hi = (int32_t)(hi64 > INT32_MAX ? INT32_MAX : hi64);
     w.zp = rq.out_zp;
-    w.t0lo = rq.t0_clamp > 0 ? -rq.t0_clamp : INT32_MIN;
-    w.t0hi = rq.t0_clamp > 0 ? rq.t0_clamp : INT32_MAX;
+    const bool clampT0 = !whole && rq.t0_clamp > 0;
+    w.t0lo = clampT0 ? -rq.t0_clamp : INT32_MIN;
+    w.t0hi = clampT0 ? rq.t0_clamp : INT32_MAX;
     // ((H + r) >> s) + zp == (H + r + zp * 2^s) >> s: fold the zero point into the rounding term
     // where that cannot overflow (|H| <= 2^30, r <= 2^29, so |zp| * 2^s up to 2^29 is safe)
     if (w.on && w.shiftMinus32 <= 13 && rq.out_zp >= -32768 && rq.out_zp <= 32767 && rq.out_min <= rq.out_max) {
@@ -81,11 +89,16 @@ __device__ __forceinline__ WideRequant wideRequant(const Requant &rq) {
         w.hi = rq.out_max;
         w.zp = 0;
     }
-    w.rnd64 = (long long)w.rnd * 4294967296LL;  // rnd may be negative (a folded negative zero point)
-    w.plain = w.on && w.pre == 0 && rq.t0_clamp <= 0 && w.zp == 0;
-    w.preOnly = w.on && w.pre > 0 && rq.t0_clamp <= 0 && w.zp == 0;
+    w.rnd64 = (long long)w.rnd * 4294967296LL + (whole ? 2147483648LL : 0LL);  // rnd may be negative (a folded negative zero point)
+    w.plain = w.on && w.pre == 0 && !clampT0 && w.zp == 0;
+    w.preOnly = w.on && w.pre > 0 && !clampT0 && w.zp == 0;
+    w.alignShift = rq.shift & 31;
+    w.rndAlign = (w.preOnly ? 1LL << (w.alignShift - 1) : 0LL) + (long long)rq.out_zp * (1LL << w.alignShift);
     return w;
 }
+// `v` has to be the result of an ordinary VALU instruction the compiler emitted (every caller passes a shift's):
+// the compiler does not look into the asm for the wait states that the result of a dot-product instruction needs
+// before another kind of VALU instruction may read it, and a v_med3 issued right behind a v_dot4c reads a stale value.
 __device__ __forceinline__ int32_t med3(int32_t v, int32_t lo, int32_t hi) {
     int32_t r;
     asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(v), "v"(lo), "v"(hi));
@@ -101,14 +114,20 @@ __device__ __forceinline__ int32_t mulhiPlusRnd(int32_t t0, int32_t scale, const
 template <bool PLAIN>
 __device__ __forceinline__ int32_t requantWideT0(int32_t t0, int32_t scale, const WideRequant &w) {
     if (PLAIN) return med3(mulhiPlusRnd(t0, scale, w) >> w.shiftMinus32, w.lo, w.hi);
-    t0 = (int32_t)((uint32_t)med3(t0, w.t0lo, w.t0hi) << w.pre);
+    // t0 may come straight out of a dot product (accumulators that start at the bias): clamp it with compiler-visible code
+    t0 = t0 < w.t0lo ? w.t0lo : t0;
+    t0 = t0 > w.t0hi ? w.t0hi : t0;
+    t0 = (int32_t)((uint32_t)t0 << w.pre);
     const int32_t t3 = med3(mulhiPlusRnd(t0, scale, w) >> w.shiftMinus32, w.lo, w.hi);  // lo <= hi
     return (int32_t)((uint32_t)t3 + (uint32_t)w.zp);
 }
-// The pre-shifted tail without the clamp of t0 and with the zero point folded (WideRequant::preOnly): what a
-// layer with a shift below 33 and a proven bound on |acc + bias| takes; two instructions shorter than the general one.
+// The tail of an op with a shift below 32 and a proven bound |acc + bias| < 2^(31 - pre) = 2^(shift - 2), no clamp of
+// t0 and the zero point folded (WideRequant::preOnly).  |t0 * scale| < 2^(shift + 29), so the rounded, shifted sum
+// fits 32 bits and is bits [shift, shift + 32) of the 64-bit sum: one v_mad_i64_i32 and one v_alignbit_b32, the
+// same number as shifting t0 left by pre first and the high word right afterwards, two instructions shorter.
 __device__ __forceinline__ int32_t requantPreShift(int32_t t0, int32_t scale, const WideRequant &w) {
-    return med3(mulhiPlusRnd((int32_t)((uint32_t)t0 << w.pre), scale, w) >> w.shiftMinus32, w.lo, w.hi);
+    const long long sum = (long long)t0 * (long long)scale + w.rndAlign;
+    return med3((int32_t)__builtin_amdgcn_alignbit((uint32_t)(sum >> 32), (uint32_t)sum, (uint32_t)w.alignShift), w.lo, w.hi);
 }
 __device__ __forceinline__ int32_t requantWideShift(int32_t acc, int32_t bias, int32_t scale, const WideRequant &w) {
     return requantWideT0<false>((int32_t)((uint32_t)acc + (uint32_t)bias), scale, w);
@@ -1776,6 +1795,201 @@ static hipError_t launchDepthwiseTile(const DepthwiseArgs &a, hipStream_t stream
     return hipGetLastError();
 }
 
+// 3x3 depthwise as a rolling window: a thread owns 4 G channels of P adjacent output columns and walks down a
+// segment of `seg` output rows.  Every input row is loaded once per thread, transposed once (the byte transposes
+// of depthwise3x3_tile_i8) into a ring of three rows held in registers, and then serves the three output rows
+// whose windows contain it.  The loads for the next output row are issued before the arithmetic of the current
+// one, so a wave overlaps its own memory latency with its own arithmetic instead of relying on the other waves
+// of the SIMD for that; weights, bias and scale stay in registers for the whole segment.
+// The row loop is unrolled three times so that the ring slots are compile-time indices.  S is the stride (1 or
+// 2, both directions); OCC is the number of waves per SIMD the register allocation aims for.
+template <int P, int S, int G, int OCC>
+__global__ __launch_bounds__(256, OCC) void depthwise3x3_strip_i8(DepthwiseArgs p, WorkSplit ws, int seg) {
+    static_assert(S == 1 || S == 2, "stride 1 or 2");
+    static_assert(S == 2 || P % 2 == 0, "stride 1 pairs the pixels of a block");
+    constexpr int NC = (P - 1) * S + 3;      // input columns under the thread's P windows
+    constexpr int NBK = S == 1 ? P / 2 : P;  // blocks of four columns per row; block b starts at column 2 b
+    constexpr int CV = 4 * G;
+    constexpr int NEW = S;                   // input rows that enter the window per output row
+    const int cg = p.C / CV;
+    const int oxGroups = (p.OW + P - 1) / P, nseg = (p.OH + seg - 1) / seg;
+    const long long total = (long long)p.N * nseg * oxGroups * cg;
+    const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (t >= total) return;
+    int cgi, oxg, sg, n;
+    splitWork(t, ws, cgi, oxg, sg, n);
+    const int c0 = cgi * CV, ox0 = oxg * P, oy0 = sg * seg;
+    const int oyEnd = oy0 + seg < p.OH ? oy0 + seg : p.OH;
+    const int ix0 = ox0 * S - p.PL;
+    const int8_t *img = p.in + (size_t)n * p.H * p.W * p.C + c0;
+    int8_t *outImg = p.out + (size_t)n * p.OH * p.OW * p.C + c0;
+    const int zp4 = (int)((uint32_t)(p.input_zp & 0xff) * 0x01010101u);
+    // every load is in bounds: coordinates are clamped and what the clamp moved is replaced by the zero point
+    int colOff[NC];
+    bool colIn[NC];
+#pragma unroll
+    for (int j = 0; j < NC; j++) {
+        const int ix = ix0 + j;
+        const int ixc = ix < 0 ? 0 : ix >= p.W ? p.W - 1 : ix;
+        colOff[j] = ixc * p.C;
+        colIn[j] = ix == ixc;
+    }
+    const int rowBytes = p.W * p.C;
+    auto issue = [&](int iy, int (&raw)[NC][G]) {
+        const int iyc = iy < 0 ? 0 : iy >= p.H ? p.H - 1 : iy;
+        const int8_t *row = img + (size_t)iyc * rowBytes;
+#pragma unroll
+        for (int j = 0; j < NC; j++) loadDwords<G>(row + colOff[j], raw[j]);
+    };
+    auto settle = [&](int iy, const int (&raw)[NC][G], uint32_t (&tr)[NBK][G][4]) {
+        const bool rowIn = (unsigned)iy < (unsigned)p.H;
+        uint32_t x[NC][G];
+#pragma unroll
+        for (int j = 0; j < NC; j++) {
+            const bool in = rowIn && colIn[j];
+#pragma unroll
+            for (int g = 0; g < G; g++) x[j][g] = in ? (uint32_t)raw[j][g] : (uint32_t)zp4;
+        }
+#pragma unroll
+        for (int b = 0; b < NBK; b++) {
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                // the last block of a stride-2 row has no fourth column; its weight is zero
+                const uint32_t x0 = x[2 * b][g], x1 = x[2 * b + 1][g], x2 = x[2 * b + 2][g], x3 = x[2 * b + 3 < NC ? 2 * b + 3 : NC - 1][g];
+                // 4 x 4 byte transpose: tr[c] = channel c at columns 2b .. 2b+3
+                const uint32_t lo01 = __builtin_amdgcn_perm(x1, x0, 0x05010400u), hi01 = __builtin_amdgcn_perm(x1, x0, 0x07030602u);
+                const uint32_t lo23 = __builtin_amdgcn_perm(x3, x2, 0x05010400u), hi23 = __builtin_amdgcn_perm(x3, x2, 0x07030602u);
+                tr[b][g][0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);
+                tr[b][g][1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+                tr[b][g][2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
+                tr[b][g][3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+            }
+        }
+    };
+    const WideRequant wrq = wideRequant(p.rq);
+    const long long rnd = roundTerm(p.rq.shift);
+    const uint32_t *wrow = (const uint32_t *)p.wpk + c0;
+    // wk = [w0, w1, w2, 0] serves the window at a block's first column, wks = [0, w0, w1, w2] the one at its second
+    int wk[G][3][4], wks[G][3][4], bs[G][4], sc[G][4];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+#pragma unroll
+        for (int kh = 0; kh < 3; kh++) {
+            const v4i w4 = *(const v4i *)(wrow + (size_t)kh * p.C + 4 * g);
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                wk[g][kh][c] = w4[c];
+                wks[g][kh][c] = (int)((uint32_t)w4[c] << 8);
+            }
+        }
+        const v4i b4 = *(const v4i *)(p.bias + c0 + 4 * g);
+        const v4i s4 = *(const v4i *)(p.scale + c0 + 4 * g);
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            bs[g][c] = b4[c];
+            sc[g][c] = s4[c];
+        }
+    }
+    uint32_t ring[3][NBK][G][4];  // window row kh of the J-th output row of a round of three sits in slot (J S + kh) % 3
+    int raw[NEW][NC][G];
+    const int iyFirst = oy0 * S - p.PT;
+#pragma unroll
+    for (int kh = 0; kh < 3 - NEW; kh++) {
+        issue(iyFirst + kh, raw[0]);
+        settle(iyFirst + kh, raw[0], ring[kh]);
+    }
+#pragma unroll
+    for (int e = 0; e < NEW; e++) issue(iyFirst + 3 - NEW + e, raw[e]);
+    withRequantMode(wrq, [&](auto mode) {
+        constexpr int kMode = decltype(mode)::value;
+        auto step = [&](auto round, int oy) {
+            constexpr int J = decltype(round)::value;
+            constexpr int slots[3] = {(J * S) % 3, (J * S + 1) % 3, (J * S + 2) % 3};
+            const int base = oy * S - p.PT;
+#pragma unroll
+            for (int e = 0; e < NEW; e++) settle(base + 3 - NEW + e, raw[e], ring[slots[3 - NEW + e]]);
+            // the rows the next output row adds (clamped: past the segment's end they are loaded and not used)
+#pragma unroll
+            for (int e = 0; e < NEW; e++) issue(base + S + 3 - NEW + e, raw[e]);
+            int o[P][G];
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                int32_t acc[P][4];  // starts at the bias (int32 wrap-around is the same in either order)
+#pragma unroll
+                for (int q = 0; q < P; q++) {
+#pragma unroll
+                    for (int c = 0; c < 4; c++) acc[q][c] = bs[g][c];
+                }
+#pragma unroll
+                for (int kh = 0; kh < 3; kh++) {
+#pragma unroll
+                    for (int b = 0; b < NBK; b++) {
+#pragma unroll
+                        for (int c = 0; c < 4; c++) {
+                            const int x = (int)ring[slots[kh]][b][g][c];
+                            if (S == 1) {
+                                acc[2 * b][c] = __builtin_amdgcn_sdot4(x, wk[g][kh][c], acc[2 * b][c], false);
+                                acc[2 * b + 1][c] = __builtin_amdgcn_sdot4(x, wks[g][kh][c], acc[2 * b + 1][c], false);
+                            } else {
+                                acc[b][c] = __builtin_amdgcn_sdot4(x, wk[g][kh][c], acc[b][c], false);
+                            }
+                        }
+                    }
+                }
+#pragma unroll
+                for (int q = 0; q < P; q++) {
+                    int32_t v[4];
+#pragma unroll
+                    for (int c = 0; c < 4; c++) v[c] = requantT0<kMode>(acc[q][c], sc[g][c], rnd, p.rq, wrq);
+                    o[q][g] = (int)packBytes(v[0], v[1], v[2], v[3]);
+                }
+            }
+            if (oy < oyEnd) {
+                int8_t *orow = outImg + ((size_t)oy * p.OW + ox0) * p.C;
+#pragma unroll
+                for (int q = 0; q < P; q++) {
+                    if (ox0 + q < p.OW) {
+                        union {
+                            typename DwordVec<G>::type v;
+                            int w[G];
+                        } u;
+#pragma unroll
+                        for (int g = 0; g < G; g++) u.w[g] = o[q][g];
+                        *(typename DwordVec<G>::type *)(orow + (size_t)q * p.C) = u.v;
+                    }
+                }
+            }
+        };
+        // the same trip count for every thread (rows past a short last segment are computed and not stored)
+        for (int oy = oy0; oy < oy0 + seg; oy += 3) {
+            step(std::integral_constant<int, 0>{}, oy);
+            step(std::integral_constant<int, 1>{}, oy + 1);
+            step(std::integral_constant<int, 2>{}, oy + 2);
+        }
+    });
+}
+
+// Rows per segment: enough segments that every SIMD gets several waves (they hide what the prefetch does not),
+// segments of at least six rows (each one re-reads two rows of its neighbour and reloads the weights).
+static int depthwiseStripSegment(const DepthwiseArgs &a, int P, int G, long long *waves) {
+    const long long stripWaves = ((long long)a.N * ((a.OW + P - 1) / P) * (a.C / (4 * G)) + 63) / 64;
+    long long nseg = (6 * 1024 + stripWaves - 1) / stripWaves;
+    const long long most = a.OH / 6 > 0 ? a.OH / 6 : 1;
+    nseg = nseg < 1 ? 1 : nseg > most ? most : nseg;
+    const int seg = (int)((a.OH + nseg - 1) / nseg);
+    *waves = stripWaves * ((a.OH + seg - 1) / seg);
+    return seg;
+}
+
+template <int P, int S, int G, int OCC>
+static hipError_t launchDepthwiseStrip(const DepthwiseArgs &a, int seg, hipStream_t stream) {
+    const int nseg = (a.OH + seg - 1) / seg, xs = (a.OW + P - 1) / P;
+    const long long total = (long long)a.N * nseg * xs * (a.C / (4 * G));
+    const WorkSplit ws = makeWorkSplit(total, a.C / (4 * G), xs, nseg);
+    hipLaunchKernelGGL((depthwise3x3_strip_i8<P, S, G, OCC>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a, ws, seg);
+    return hipGetLastError();
+}
+
 static int pickVec(int C, const void *a, const void *b, const void *c) {
     const uintptr_t bits = (uintptr_t)a | (uintptr_t)b | (uintptr_t)c;
     if (C % 16 == 0 && (bits & 15) == 0) return 16;
@@ -1817,6 +2031,16 @@ hipError_t launchDepthwise(const DepthwiseArgs &a, hipStream_t stream) {
         const long long outputs = (long long)a.N * a.OH * a.OW * (a.C / 16);
         // a register tile of outputs per thread where that still leaves every CU several blocks
         // (THIP_DEPTHWISE_TILE=0 / 1 switches that kernel off / on for every size, for tests and tuning)
+        // the rolling-window kernel where it has at least a wave (stride 1) or 2.5 waves (stride 2) per SIMD
+        // (THIP_DEPTHWISE_STRIP=0 / 1 switches it off / on for every size, for tests and tuning)
+        const char *stripEnv = getenv("THIP_DEPTHWISE_STRIP");
+        const bool stripOff = stripEnv && stripEnv[0] == '0', stripOn = stripEnv && stripEnv[0] == '1';
+        if (!stripOff && a.SH == a.SW && (a.SW == 1 || a.SW == 2) && (long long)a.W * a.C < (1LL << 24)) {
+            long long waves = 0;
+            const int seg = depthwiseStripSegment(a, 2, 1, &waves);
+            if (a.SW == 1 && (stripOn || (a.OH >= 12 && waves >= 1024))) return launchDepthwiseStrip<2, 1, 1, 4>(a, seg, stream);
+            if (a.SW == 2 && (stripOn || (a.OH >= 12 && 2 * waves >= 5 * 1024))) return launchDepthwiseStrip<2, 2, 1, 3>(a, seg, stream);
+        }
         const char *tileEnv = getenv("THIP_DEPTHWISE_TILE");
         const bool tileOff = tileEnv && tileEnv[0] == '0', tileOn = tileEnv && tileEnv[0] == '1';
         if (!tileOff) {

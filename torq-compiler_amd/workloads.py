@@ -264,15 +264,22 @@ def add_bf16_workload(shape=(1, 32, 1152), w0=1.0, w1=1.0, bias=0.0, clamp=None,
 
 
 def depthwise_workload(N=1, H=56, W=56, C=144, KH=3, KW=3, stride=(2, 2), pad=(0, 1, 0, 1), input_zp=-3,
-                       output_zp=5, output_min=-128, output_max=127, realistic=True, nhwc=True, seed=1002):
-    """benchmark configuration 2a: depthwise 3x3 stride 2 SAME on 56x56x144."""
+                       output_zp=5, output_min=-128, output_max=127, realistic=True, nhwc=True, seed=1002, shift=None):
+    """benchmark configuration 2a: depthwise 3x3 stride 2 SAME on 56x56x144.
+
+    `shift` forces one shift_factor for every channel (multipliers drawn so that outputs still spread)."""
     rng = np.random.default_rng(seed)
     x = rng.integers(-128, 127, size=(N, H, W, C), endpoint=True, dtype=np.int8)
     w = rng.integers(-127, 127, size=(C, 1, KH, KW), endpoint=True, dtype=np.int8)
     tosa_bias = rng.integers(-(1 << 15), 1 << 15, size=C, endpoint=True, dtype=np.int64)
-    mult, shift = random_requant(rng, C, realistic)
-    if realistic:
-        shift = (shift - 4).astype(np.int8)  # only 9 taps: keep outputs spread over the int8 range
+    if shift is not None:
+        top = min(max(int(shift) - 10, 1), 31)
+        mult = rng.integers(1 << (top - 1), (1 << top) - 1, size=C, endpoint=True, dtype=np.int64).astype(np.int32)
+        shift = np.full(C, int(shift), dtype=np.int8)
+    else:
+        mult, shift = random_requant(rng, C, realistic)
+        if realistic:
+            shift = (shift - 4).astype(np.int8)  # only 9 taps: keep outputs spread over the int8 range
     sb, sf = derive_scale_bias(mult, shift, tosa_bias, w, input_zp)
     attrs = dict(input_zp=input_zp, output_zp=output_zp, output_min=output_min, output_max=output_max,
                  shift_factor=sf, pad=tuple(pad), stride=tuple(stride))
