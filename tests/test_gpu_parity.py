@@ -196,13 +196,14 @@ def test_depthwise_geometries(device, kw, nhwc):
     check(device, w.depthwise_workload(nhwc=nhwc, **kw))
 
 
-@pytest.mark.parametrize("which", ["rows", "tile", "strip"])
+@pytest.mark.parametrize("which", ["rows", "tile", "strip", "strip1"])
 def test_depthwise_3x3_kernels(device, which, monkeypatch):
     """The three 3x3 kernels (one window row of pixels per thread, a register tile of outputs per thread, a rolling
-    window down a segment of rows) on images whose sizes are no multiples of the tiles or segments, with and
-    without padding, stride 1 and 2, with one and with several row segments."""
+    window down a segment of rows, with two columns or, at stride 2, one column per thread) on images whose sizes
+    are no multiples of the tiles or segments, with and without padding, stride 1 and 2, with one and with several
+    row segments."""
     monkeypatch.setenv("THIP_DEPTHWISE_TILE", "1" if which == "tile" else "0")
-    monkeypatch.setenv("THIP_DEPTHWISE_STRIP", "1" if which == "strip" else "0")
+    monkeypatch.setenv("THIP_DEPTHWISE_STRIP", {"strip": "1", "strip1": "2"}.get(which, "0"))
     for kw in [dict(N=2, H=13, W=15, C=16, stride=(1, 1), pad=(1, 1, 1, 1)), dict(N=1, H=14, W=14, C=48, stride=(1, 1), pad=(0, 0, 0, 0)),
                dict(N=1, H=9, W=31, C=32, stride=(1, 1), pad=(1, 1, 1, 1)), dict(N=2, H=21, W=22, C=16, stride=(2, 2), pad=(0, 1, 0, 1)),
                dict(N=1, H=15, W=13, C=80, stride=(2, 2), pad=(1, 1, 1, 1)), dict(N=1, H=3, W=3, C=16, stride=(1, 1), pad=(0, 0, 0, 0)),
@@ -216,16 +217,17 @@ def test_depthwise_3x3_kernels(device, which, monkeypatch):
         check(device, w.depthwise_workload(**kw), kernel="depthwise3x3_dot4_i8")
 
 
-@pytest.mark.parametrize("which", ["rows", "tile", "strip"])
+@pytest.mark.parametrize("which", ["rows", "tile", "strip", "strip1"])
 def test_depthwise_shift_boundaries(device, which, monkeypatch):
     """Every requant tail of the 3x3 kernels: the generic 64-bit one, the bits of the sum read directly (a shift below
     32 with a proven bound), with a clamp of acc + bias (a large bias breaks the bound), the high word itself
     (shift 32) and the shifted high word (33 and up); zero points of either sign."""
     monkeypatch.setenv("THIP_DEPTHWISE_TILE", "1" if which == "tile" else "0")
-    monkeypatch.setenv("THIP_DEPTHWISE_STRIP", "1" if which == "strip" else "0")
+    monkeypatch.setenv("THIP_DEPTHWISE_STRIP", {"strip": "1", "strip1": "2"}.get(which, "0"))
+    stride = (2, 2) if which == "strip1" else (1, 1)
     for shift in [0, 2, 3, 12, 24, 31, 32, 33, 34, 40, 62]:
         for zp in (-7, 100):
-            check(device, w.depthwise_workload(N=1, H=12, W=10, C=32, stride=(1, 1), pad=(1, 1, 1, 1), shift=shift, output_zp=zp),
+            check(device, w.depthwise_workload(N=1, H=12, W=10, C=32, stride=stride, pad=(1, 1, 1, 1), shift=shift, output_zp=zp),
                   kernel="depthwise3x3_dot4_i8")
     check(device, w.depthwise_workload(N=1, H=12, W=10, C=32, stride=(2, 2), pad=(1, 1, 1, 1), shift=31, output_zp=-128),
           kernel="depthwise3x3_dot4_i8")

@@ -1802,9 +1802,11 @@ static hipError_t launchDepthwiseTile(const DepthwiseArgs &a, hipStream_t stream
 // one, so a wave overlaps its own memory latency with its own arithmetic instead of relying on the other waves
 // of the SIMD for that; weights, bias and scale stay in registers for the whole segment.
 // The row loop is unrolled three times so that the ring slots are compile-time indices.  S is the stride (1 or
-// 2, both directions); OCC is the number of waves per SIMD the register allocation aims for.
-template <int P, int S, int G, int OCC>
+// 2, both directions); OCC is the number of waves per SIMD the register allocation aims for; D (1 or 3) is how
+// many output rows ahead the loads run.
+template <int P, int S, int G, int OCC, int D>
 __global__ __launch_bounds__(256, OCC) void depthwise3x3_strip_i8(DepthwiseArgs p, WorkSplit ws, int seg) {
+    static_assert(D == 1 || D == 3, "the prefetch buffers rotate with the row loop's unrolling");
     static_assert(S == 1 || S == 2, "stride 1 or 2");
     static_assert(S == 2 || P % 2 == 0, "stride 1 pairs the pixels of a block");
     constexpr int NC = (P - 1) * S + 3;      // input columns under the thread's P windows
@@ -1891,15 +1893,18 @@ __global__ __launch_bounds__(256, OCC) void depthwise3x3_strip_i8(DepthwiseArgs 
         }
     }
     uint32_t ring[3][NBK][G][4];  // window row kh of the J-th output row of a round of three sits in slot (J S + kh) % 3
-    int raw[NEW][NC][G];
+    int raw[D][NEW][NC][G];
     const int iyFirst = oy0 * S - p.PT;
 #pragma unroll
     for (int kh = 0; kh < 3 - NEW; kh++) {
-        issue(iyFirst + kh, raw[0]);
-        settle(iyFirst + kh, raw[0], ring[kh]);
+        issue(iyFirst + kh, raw[0][0]);
+        settle(iyFirst + kh, raw[0][0], ring[kh]);
     }
 #pragma unroll
-    for (int e = 0; e < NEW; e++) issue(iyFirst + 3 - NEW + e, raw[e]);
+    for (int d = 0; d < D; d++) {
+#pragma unroll
+        for (int e = 0; e < NEW; e++) issue(iyFirst + d * S + 3 - NEW + e, raw[d][e]);
+    }
     withRequantMode(wrq, [&](auto mode) {
         constexpr int kMode = decltype(mode)::value;
         auto step = [&](auto round, int oy) {
@@ -1907,10 +1912,10 @@ __global__ __launch_bounds__(256, OCC) void depthwise3x3_strip_i8(DepthwiseArgs 
             constexpr int slots[3] = {(J * S) % 3, (J * S + 1) % 3, (J * S + 2) % 3};
             const int base = oy * S - p.PT;
 #pragma unroll
-            for (int e = 0; e < NEW; e++) settle(base + 3 - NEW + e, raw[e], ring[slots[3 - NEW + e]]);
-            // the rows the next output row adds (clamped: past the segment's end they are loaded and not used)
+            for (int e = 0; e < NEW; e++) settle(base + 3 - NEW + e, raw[J % D][e], ring[slots[3 - NEW + e]]);
+            // the rows that output row oy + D adds (clamped: past the segment's end they are loaded and not used)
 #pragma unroll
-            for (int e = 0; e < NEW; e++) issue(base + S + 3 - NEW + e, raw[e]);
+            for (int e = 0; e < NEW; e++) issue(base + D * S + 3 - NEW + e, raw[J % D][e]);
             int o[P][G];
 #pragma unroll
             for (int g = 0; g < G; g++) {
@@ -1981,12 +1986,12 @@ static int depthwiseStripSegment(const DepthwiseArgs &a, int P, int G, long long
     return seg;
 }
 
-template <int P, int S, int G, int OCC>
+template <int P, int S, int G, int OCC, int D>
 static hipError_t launchDepthwiseStrip(const DepthwiseArgs &a, int seg, hipStream_t stream) {
     const int nseg = (a.OH + seg - 1) / seg, xs = (a.OW + P - 1) / P;
     const long long total = (long long)a.N * nseg * xs * (a.C / (4 * G));
     const WorkSplit ws = makeWorkSplit(total, a.C / (4 * G), xs, nseg);
-    hipLaunchKernelGGL((depthwise3x3_strip_i8<P, S, G, OCC>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a, ws, seg);
+    hipLaunchKernelGGL((depthwise3x3_strip_i8<P, S, G, OCC, D>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a, ws, seg);
     return hipGetLastError();
 }
 
@@ -2032,14 +2037,22 @@ hipError_t launchDepthwise(const DepthwiseArgs &a, hipStream_t stream) {
         // a register tile of outputs per thread where that still leaves every CU several blocks
         // (THIP_DEPTHWISE_TILE=0 / 1 switches that kernel off / on for every size, for tests and tuning)
         // the rolling-window kernel where it has at least a wave (stride 1) or 2.5 waves (stride 2) per SIMD
-        // (THIP_DEPTHWISE_STRIP=0 / 1 switches it off / on for every size, for tests and tuning)
+        // (THIP_DEPTHWISE_STRIP=0 / 1 / 2 switches it off / on / on with one column per thread at stride 2, for every
+        // size, for tests and tuning)
         const char *stripEnv = getenv("THIP_DEPTHWISE_STRIP");
-        const bool stripOff = stripEnv && stripEnv[0] == '0', stripOn = stripEnv && stripEnv[0] == '1';
+        const bool stripOff = stripEnv && stripEnv[0] == '0', stripOn = stripEnv && (stripEnv[0] == '1' || stripEnv[0] == '2');
+        const bool stripOne = stripEnv && stripEnv[0] == '2';
         if (!stripOff && a.SH == a.SW && (a.SW == 1 || a.SW == 2) && (long long)a.W * a.C < (1LL << 24)) {
             long long waves = 0;
             const int seg = depthwiseStripSegment(a, 2, 1, &waves);
-            if (a.SW == 1 && (stripOn || (a.OH >= 12 && waves >= 1024))) return launchDepthwiseStrip<2, 1, 1, 4>(a, seg, stream);
-            if (a.SW == 2 && (stripOn || (a.OH >= 12 && 2 * waves >= 5 * 1024))) return launchDepthwiseStrip<2, 2, 1, 3>(a, seg, stream);
+            if (a.SW == 1 && (stripOn || (a.OH >= 12 && waves >= 1024))) return launchDepthwiseStrip<2, 1, 1, 4, 3>(a, seg, stream);
+            if (a.SW == 2 && (stripOne || (!stripOn && a.OH >= 12))) {
+                // with plenty of work, one column per thread, more waves and the deeper prefetch measured 7-10 % ahead
+                long long waves1 = 0;
+                const int seg1 = depthwiseStripSegment(a, 1, 1, &waves1);
+                if (stripOne || waves1 >= 7 * 1024) return launchDepthwiseStrip<1, 2, 1, 4, 3>(a, seg1, stream);
+            }
+            if (a.SW == 2 && (stripOn || (a.OH >= 12 && 2 * waves >= 5 * 1024))) return launchDepthwiseStrip<2, 2, 1, 3, 1>(a, seg, stream);
         }
         const char *tileEnv = getenv("THIP_DEPTHWISE_TILE");
         const bool tileOff = tileEnv && tileEnv[0] == '0', tileOn = tileEnv && tileEnv[0] == '1';
