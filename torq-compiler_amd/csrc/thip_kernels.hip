@@ -1533,6 +1533,14 @@ __global__ __launch_bounds__(256) void depthwise_i8(DepthwiseArgs p, WorkSplit w
     *(typename ByteVec<VEC>::type *)(p.out + (((size_t)n * p.OH + oy) * p.OW + ox) * p.C + c0) = o.v;
 }
 
+// Blocks are handed to the eight XCDs in turn (block b runs on XCD b % 8), each with an L2 of its own.  This
+// renumbering gives every XCD one contiguous eighth of the blocks, so that blocks whose threads read the same input
+// (neighbouring column strips share two of four columns) find it in their own L2 instead of fetching it eight times.
+__device__ __forceinline__ unsigned xcdContiguousBlock() {
+    const unsigned nb = gridDim.x, x = blockIdx.x & 7u, i = blockIdx.x >> 3, per = nb >> 3, rem = nb & 7u;
+    return x * per + (x < rem ? x : rem) + i;
+}
+
 // 3x3 depthwise with the window row as the dot dimension.  A thread owns 16 channels of P
 // horizontally adjacent output pixels.  The three taps of a window row are brought together per
 // channel with two byte permutes ([x(kw0), x(kw1), x(kw2), 0] in one register) and multiplied by the
@@ -1549,7 +1557,7 @@ __global__ __launch_bounds__(256) void depthwise3x3_dot4_i8(DepthwiseArgs p, Wor
     const int cg = p.C / 16;
     const int oxGroups = (p.OW + P - 1) / P;
     const long long total = (long long)p.N * p.OH * oxGroups * cg;
-    const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+    const long long t = (long long)xcdContiguousBlock() * 256 + threadIdx.x;
     if (t >= total) return;
     int cgi, oxg, oy, n;
     splitWork(t, ws, cgi, oxg, oy, n);
@@ -1674,7 +1682,7 @@ __global__ __launch_bounds__(256) void depthwise3x3_tile_i8(DepthwiseArgs p, Wor
     const int cg = p.C / CV;
     const int oxGroups = (p.OW + P - 1) / P, oyGroups = (p.OH + R - 1) / R;
     const long long total = (long long)p.N * oyGroups * oxGroups * cg;
-    const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+    const long long t = (long long)xcdContiguousBlock() * 256 + threadIdx.x;
     if (t >= total) return;
     int cgi, oxg, oyg, n;
     splitWork(t, ws, cgi, oxg, oyg, n);
@@ -1816,7 +1824,7 @@ __global__ __launch_bounds__(256, OCC) void depthwise3x3_strip_i8(DepthwiseArgs 
     const int cg = p.C / CV;
     const int oxGroups = (p.OW + P - 1) / P, nseg = (p.OH + seg - 1) / seg;
     const long long total = (long long)p.N * nseg * oxGroups * cg;
-    const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+    const long long t = (long long)xcdContiguousBlock() * 256 + threadIdx.x;
     if (t >= total) return;
     int cgi, oxg, sg, n;
     splitWork(t, ws, cgi, oxg, sg, n);
