@@ -43,6 +43,7 @@ struct IgemmArgs {
     const int8_t *skip;
     int32_t add_skip_first, add_w0, add_w1, add_bias, add_scale;
     Requant arq;
+    int32_t stream_guarded;  // pixel-streaming kernel: keep every load and store under its bounds check (tests, tuning)
 };
 
 // Tile configurations of the igemm kernel.

@@ -964,8 +964,12 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
 constexpr int kStreamRing = 4;
 constexpr size_t kStreamMaxLds = 64 * 1024;
 
-template <int NB, int LOADER, bool ADD>  // ADD: a residual add behind the requant (its code costs the others registers)
+// KS: 0, or the number of k-steps (1 or 2) when that is known at compile time and divides the ring: the ring then
+// runs over RING / KS pixel groups instead of one, so that loads stay RING k-steps ahead of the MFMAs even where a
+// group has only one or two of them (the expanding pointwise convolutions of a mobile network: K = 16 .. 64).
+template <int NB, int LOADER, bool ADD, int KS>  // ADD: a residual add behind the requant (its code costs the others registers)
 __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArgs p) {
+    static_assert(KS == 0 || (kStreamRing % KS == 0 && LOADER == kLoaderDense), "the ring holds whole groups");
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
     constexpr int RING = kStreamRing;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -1032,15 +1036,8 @@ __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArg
     int32_t addFolded = 0;
     const bool addFast = ADD && residualAddFolded(p.add_w0, p.add_w1, p.add_bias, p.add_scale, p.arq, &addFolded);
 
-    int g = blockIdx.x * 4 + wave;
-    v4i ring[RING];
-    Pos here = locate(g);
-#pragma unroll
-    for (int d = 0; d < RING; d++) ring[d] = fetch(g, d, here);
-    for (; g < groups; g += stride) {
-        const Pos next = locate(g + stride < groups ? g + stride : g);
-        // accumulators start at the bias: register 4 q + e of block j holds channel 32 j + 8 q + 4 half + e
-        v16i acc[NB];
+    // accumulators start at the bias: register 4 q + e of block j holds channel 32 j + 8 q + 4 half + e
+    auto initAcc = [&](v16i (&acc)[NB]) {
 #pragma unroll
         for (int j = 0; j < NB; j++) {
             if (j < nblocks) {
@@ -1052,26 +1049,18 @@ __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArg
                 }
             }
         }
-        for (int s0 = 0; s0 < kstepsRing; s0 += RING) {
+    };
+    auto multiply = [&](int s, const v4i &a, v16i (&acc)[NB]) {
+        const int8_t *wfrag = smem + ((size_t)(s * nblocks) * 64 + lane) * 16;
 #pragma unroll
-            for (int d = 0; d < RING; d++) {
-                const int s = s0 + d;
-                const v4i a = ring[d];
-                // slot d next holds k-step s + RING of this group, or the same slot of the next group
-                const bool wrap = s + RING >= kstepsRing;
-                ring[d] = fetch(wrap ? g + stride : g, wrap ? s + RING - kstepsRing : s + RING, wrap ? next : here);
-                if (s < ksteps) {
-                    const int8_t *wfrag = smem + ((size_t)(s * nblocks) * 64 + lane) * 16;
-#pragma unroll
-                    for (int j = 0; j < NB; j++) {
-                        if (j < nblocks) {
-                            const v4i w = *(const v4i *)(wfrag + j * 1024);
-                            acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w, a, acc[j], 0, 0, 0);
-                        }
-                    }
-                }
+        for (int j = 0; j < NB; j++) {
+            if (j < nblocks) {
+                const v4i w = *(const v4i *)(wfrag + j * 1024);
+                acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w, a, acc[j], 0, 0, 0);
             }
         }
+    };
+    auto epilogue = [&](int g, v16i (&acc)[NB]) {
         const int m = g * 32 + fr;
         withRequantMode(wrq, [&](auto mode) {
             constexpr int kMode = decltype(mode)::value;
@@ -1105,13 +1094,174 @@ __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArg
                 }
             }
         });
+    };
+
+    int g = blockIdx.x * 4 + wave;
+    v4i ring[RING];
+    // The steady state of the dense loader: every load and every store unconditional and branch-free, so that the
+    // compiler's s_waitcnt before an MFMA counts exactly the memory operations issued after the load it needs (a
+    // load or a store under a branch counts as zero, and the wait then drains the whole queue, prefetches included).
+    // A row past M reads row M - 1 and bytes past the end of A the last 16: they meet zero weights (K..Kp) or
+    // belong to rows that are not stored.  Full groups only; what is left goes through the guarded code below.
+    if (LOADER == kLoaderDense && !ADD && nblocks == NB && !p.stream_guarded) {
+        const long long lastRun = (long long)p.M * p.K - 16;
+        auto fetchDense = [&](int gq, int sq) -> v4i {
+            int m = gq * 32 + fr;
+            m = m < p.M ? m : p.M - 1;
+            long long off = (long long)m * p.K + (sq < ksteps ? sq : 0) * 32 + half * 16;
+            off = off < lastRun ? off : lastRun;
+            return *(const v4i *)(p.A + off);
+        };
+        const int groupsFull = p.M / 32;
+        const bool ragged = p.N - n0 < NB * 32;  // the upper 16 channels of the last block do not exist (N % 16 == 0)
+        // bias and scale are read from LDS again for every group: kept in registers across the loop (where the compiler
+        // hoists loop-invariant loads to) they would be 32 registers per block of channels and spill; an offset of
+        // zero that the compiler cannot see through keeps the reads where they are
+        auto perGroupZero = [] {
+            int zero = 0;
+            asm volatile("" : "+v"(zero));
+            return zero;
+        };
+        auto initAll = [&](v16i (&acc)[NB]) {
+            const int32_t *bias = ldsBias + perGroupZero();
+#pragma unroll
+            for (int j = 0; j < NB; j++) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const v4i b4 = *(const v4i *)(bias + j * 32 + 8 * q + 4 * half);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) acc[j][4 * q + e] = b4[e];
+                }
+            }
+        };
+        auto multiplyAll = [&](int sq, const v4i &a, v16i (&acc)[NB]) {
+            const int8_t *wfrag = smem + ((size_t)(sq * NB) * 64 + lane) * 16;
+#pragma unroll
+            for (int j = 0; j < NB; j++) {
+                const v4i w = *(const v4i *)(wfrag + j * 1024);
+                acc[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w, a, acc[j], 0, 0, 0);
+            }
+        };
+        withRequantMode(wrq, [&](auto mode) {
+            constexpr int kMode = decltype(mode)::value;
+            auto storeFull = [&](int gq, v16i (&acc)[NB]) {
+                int8_t *orow = (int8_t *)p.out + (size_t)(gq * 32 + fr) * p.N + n0 + 16 * half;
+                const int32_t *scale = ldsScale + perGroupZero();
+#pragma unroll
+                for (int j = 0; j < NB; j++) {
+                    uint32_t d4[4];
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        const v4i s4 = *(const v4i *)(scale + j * 32 + 8 * q + 4 * half);
+                        int32_t v[4];
+#pragma unroll
+                        for (int e = 0; e < 4; e++) v[e] = requantT0<kMode>(acc[j][4 * q + e], s4[e], rnd, p.rq, wrq);
+                        d4[q] = packBytes(v[0], v[1], v[2], v[3]);
+                    }
+                    const auto s02 = __builtin_amdgcn_permlane32_swap(d4[0], d4[2], false, false);
+                    const auto s13 = __builtin_amdgcn_permlane32_swap(d4[1], d4[3], false, false);
+                    v4i outv = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
+                    if (j == NB - 1 && ragged) {
+                        // ragged last block: its 16 channels sit in the lower half lanes; the upper half lanes take over
+                        // the second 8 of them, so that every lane stores (one store on either side of this branch)
+                        const auto hi0 = __builtin_amdgcn_permlane32_swap((uint32_t)outv[2], (uint32_t)outv[2], false, false);
+                        const auto hi1 = __builtin_amdgcn_permlane32_swap((uint32_t)outv[3], (uint32_t)outv[3], false, false);
+                        const v2i part = {half ? (int)hi0[0] : outv[0], half ? (int)hi1[0] : outv[1]};
+                        *(v2i *)(orow + j * 32 - 8 * half) = part;
+                    } else {
+                        *(v4i *)(orow + j * 32) = outv;
+                    }
+                }
+            };
+            if (KS > 0) {
+                // slot d holds k-step d % KS of group g + (d / KS) * stride; a revolution of the ring covers GPI groups
+                constexpr int KSS = KS > 0 ? KS : 1, GPI = RING / KSS;
+#pragma unroll
+                for (int d = 0; d < RING; d++) ring[d] = fetchDense(g + (d / KSS) * stride, d % KSS);
+                for (; g + (GPI - 1) * stride < groupsFull; g += GPI * stride) {
+#pragma unroll
+                    for (int gi = 0; gi < GPI; gi++) {
+                        const int gd = g + gi * stride;
+                        v16i acc[NB];
+                        initAll(acc);
+#pragma unroll
+                        for (int ks = 0; ks < KSS; ks++) {
+                            // the MFMAs read the slot before its next load is issued: the slot keeps its registers
+                            multiplyAll(ks, ring[gi * KSS + ks], acc);
+                            ring[gi * KSS + ks] = fetchDense(gd + GPI * stride, ks);
+                        }
+                        storeFull(gd, acc);
+                    }
+                }
+                // the wave's last groups (fewer than a revolution, the last one perhaps short): their data is in the ring
+#pragma unroll
+                for (int gi = 0; gi < GPI; gi++) {
+                    const int gd = g + gi * stride;
+                    if (gd < groups) {
+                        v16i acc[NB];
+                        initAcc(acc);
+#pragma unroll
+                        for (int ks = 0; ks < KSS; ks++) multiply(ks, ring[gi * KSS + ks], acc);
+                        epilogue(gd, acc);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int d = 0; d < RING; d++) ring[d] = fetchDense(g, d);
+                auto revolve = [&](int gq, v16i (&acc)[NB]) {
+                    for (int s0 = 0; s0 < kstepsRing; s0 += RING) {
+#pragma unroll
+                        for (int d = 0; d < RING; d++) {
+                            const int sq = s0 + d;
+                            if (sq < ksteps) multiplyAll(sq, ring[d], acc);
+                            // slot d next holds k-step s + RING of this group, or the same slot of the next group
+                            const bool wrap = sq + RING >= kstepsRing;
+                            ring[d] = fetchDense(wrap ? gq + stride : gq, wrap ? sq + RING - kstepsRing : sq + RING);
+                        }
+                    }
+                };
+                for (; g < groupsFull; g += stride) {
+                    v16i acc[NB];
+                    initAll(acc);
+                    revolve(g, acc);
+                    storeFull(g, acc);
+                }
+                if (g < groups) {  // the short last group
+                    v16i acc[NB];
+                    initAcc(acc);
+                    revolve(g, acc);
+                    epilogue(g, acc);
+                }
+            }
+        });
+        return;
+    }
+    Pos here = locate(g);
+#pragma unroll
+    for (int d = 0; d < RING; d++) ring[d] = fetch(g, d, here);
+    for (; g < groups; g += stride) {
+        const Pos next = locate(g + stride < groups ? g + stride : g);
+        v16i acc[NB];
+        initAcc(acc);
+        for (int s0 = 0; s0 < kstepsRing; s0 += RING) {
+#pragma unroll
+            for (int d = 0; d < RING; d++) {
+                const int s = s0 + d;
+                const v4i a = ring[d];
+                // slot d next holds k-step s + RING of this group, or the same slot of the next group
+                const bool wrap = s + RING >= kstepsRing;
+                ring[d] = fetch(wrap ? g + stride : g, wrap ? s + RING - kstepsRing : s + RING, wrap ? next : here);
+                if (s < ksteps) multiply(s, a, acc);
+            }
+        }
+        epilogue(g, acc);
         here = next;
     }
 }
 
-template <int NB, int LOADER, bool ADD>
+template <int NB, int LOADER, bool ADD, int KS>
 static hipError_t launchIgemmStreamA(const IgemmArgs &a, size_t smem, hipStream_t stream) {
-    auto kernel = igemm_stream_i8<NB, LOADER, ADD>;
+    auto kernel = igemm_stream_i8<NB, LOADER, ADD, KS>;
     static bool configured = false;
     if (!configured) {
         hipError_t err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kStreamMaxLds);
@@ -1120,9 +1270,19 @@ static hipError_t launchIgemmStreamA(const IgemmArgs &a, size_t smem, hipStream_
     }
     // every block copies the weights into LDS once, then strides over the pixel groups:
     // one resident set of blocks, each with several groups where the image is large
-    // blocks one CU holds: by registers (7, 5, 4, 3, 2 waves per SIMD for NB = 1, 2, 4, 6, 8) and by LDS
-    const int byRegs = NB <= 1 ? 7 : NB <= 2 ? 5 : NB <= 4 ? 4 : NB <= 6 ? 3 : 2;
-    const int perCu = (int)std::min<size_t>(byRegs, (160 * 1024) / smem);
+    // blocks one CU holds (registers and LDS), asked once per LDS size
+    static size_t askedSmem = 0;
+    static int perCuAsked = 0;
+    if (askedSmem != smem || perCuAsked <= 0) {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void *)kernel, 256, smem) != hipSuccess || n <= 0) {
+            (void)hipGetLastError();
+            n = (int)std::min<size_t>(NB <= 1 ? 7 : NB <= 2 ? 5 : NB <= 4 ? 4 : NB <= 6 ? 3 : 2, (160 * 1024) / smem);
+        }
+        perCuAsked = n;
+        askedSmem = smem;
+    }
+    const int perCu = std::min(perCuAsked, 8);
     const int groups = (a.M + 31) / 32;
     const int chunk = igemmStreamChunk(a.Np), chunks = (a.Np + chunk - 1) / chunk;
     const int blocks = std::min((groups + 3) / 4, std::max(1, 256 * perCu / chunks));
@@ -1134,9 +1294,13 @@ template <int NB, int LOADER>
 static hipError_t launchIgemmStreamT(const IgemmArgs &a, size_t smem, hipStream_t stream) {
     if (a.skip != nullptr) {
         if (LOADER != kLoaderDense) return hipErrorInvalidValue;
-        return launchIgemmStreamA<NB, kLoaderDense, true>(a, smem, stream);
+        return launchIgemmStreamA<NB, kLoaderDense, true, 0>(a, smem, stream);
     }
-    return launchIgemmStreamA<NB, LOADER, false>(a, smem, stream);
+    // one or two k-steps per pixel group: the ring runs over several groups (THIP_NO_STREAM_DEEP: never)
+    if (LOADER == kLoaderDense && a.Kp <= 64 && !getenv("THIP_NO_STREAM_DEEP")) {
+        return a.Kp <= 32 ? launchIgemmStreamA<NB, kLoaderDense, false, 1>(a, smem, stream) : launchIgemmStreamA<NB, kLoaderDense, false, 2>(a, smem, stream);
+    }
+    return launchIgemmStreamA<NB, LOADER, false, 0>(a, smem, stream);
 }
 
 static hipError_t launchIgemmStream(const IgemmArgs &a, hipStream_t stream) {
@@ -1152,6 +1316,21 @@ static hipError_t launchIgemmStream(const IgemmArgs &a, hipStream_t stream) {
         if (nb <= 2) return launchIgemmStreamT<2, kLoaderRuns>(a, smem, stream);
         if (nb <= 4) return launchIgemmStreamT<4, kLoaderRuns>(a, smem, stream);
         return hipErrorInvalidValue;
+    }
+    if (a.skip == nullptr) {
+        // the branch-free steady state needs the block count at compile time (THIP_STREAM_GUARDED: the guarded loop only)
+        IgemmArgs b = a;
+        b.stream_guarded = getenv("THIP_STREAM_GUARDED") != nullptr;
+        switch (nb) {
+        case 1: return launchIgemmStreamT<1, kLoaderDense>(b, smem, stream);
+        case 2: return launchIgemmStreamT<2, kLoaderDense>(b, smem, stream);
+        case 3: return launchIgemmStreamT<3, kLoaderDense>(b, smem, stream);
+        case 4: return launchIgemmStreamT<4, kLoaderDense>(b, smem, stream);
+        case 5: return launchIgemmStreamT<5, kLoaderDense>(b, smem, stream);
+        case 6: return launchIgemmStreamT<6, kLoaderDense>(b, smem, stream);
+        case 7: return launchIgemmStreamT<7, kLoaderDense>(b, smem, stream);
+        default: return launchIgemmStreamT<8, kLoaderDense>(b, smem, stream);
+        }
     }
     if (nb <= 1) return launchIgemmStreamT<1, kLoaderDense>(a, smem, stream);
     if (nb <= 2) return launchIgemmStreamT<2, kLoaderDense>(a, smem, stream);
