@@ -1293,8 +1293,12 @@ static hipError_t launchIgemmStreamA(const IgemmArgs &a, size_t smem, hipStream_
 template <int NB, int LOADER>
 static hipError_t launchIgemmStreamT(const IgemmArgs &a, size_t smem, hipStream_t stream) {
     if (a.skip != nullptr) {
-        if (LOADER != kLoaderDense) return hipErrorInvalidValue;
-        return launchIgemmStreamA<NB, kLoaderDense, true, 0>(a, smem, stream);
+        // the residual add comes with the accumulator widths 1, 2, 4, 6, 8 only (its caller rounds up)
+        if constexpr (LOADER == kLoaderDense && (NB <= 2 || NB % 2 == 0)) {
+            return launchIgemmStreamA<NB, kLoaderDense, true, 0>(a, smem, stream);
+        } else {
+            return hipErrorInvalidValue;
+        }
     }
     // one or two k-steps per pixel group: the ring runs over several groups (THIP_NO_STREAM_DEEP: never)
     if (LOADER == kLoaderDense && a.Kp <= 64 && !getenv("THIP_NO_STREAM_DEEP")) {
