@@ -2227,7 +2227,7 @@ hipError_t launchDepthwise(const DepthwiseArgs &a, hipStream_t stream) {
         const long long outputs = (long long)a.N * a.OH * a.OW * (a.C / 16);
         // a register tile of outputs per thread where that still leaves every CU several blocks
         // (THIP_DEPTHWISE_TILE=0 / 1 switches that kernel off / on for every size, for tests and tuning)
-        // the rolling-window kernel where it has at least a wave (stride 1) or 2.5 waves (stride 2) per SIMD
+        // the rolling-window kernel where it has at least a wave (stride 1) or 1.9 waves (stride 2) per SIMD
         // (THIP_DEPTHWISE_STRIP=0 / 1 / 2 switches it off / on / on with one column per thread at stride 2, for every
         // size, for tests and tuning)
         const char *stripEnv = getenv("THIP_DEPTHWISE_STRIP");
@@ -2243,7 +2243,7 @@ hipError_t launchDepthwise(const DepthwiseArgs &a, hipStream_t stream) {
                 const int seg1 = depthwiseStripSegment(a, 1, 1, &waves1);
                 if (stripOne || waves1 >= 7 * 1024) return launchDepthwiseStrip<1, 2, 1, 4, 3>(a, seg1, stream);
             }
-            if (a.SW == 2 && (stripOn || (a.OH >= 12 && 2 * waves >= 5 * 1024))) return launchDepthwiseStrip<2, 2, 1, 3, 1>(a, seg, stream);
+            if (a.SW == 2 && (stripOn || (a.OH >= 12 && 10 * waves >= 19 * 1024))) return launchDepthwiseStrip<2, 2, 1, 3, 1>(a, seg, stream);
         }
         const char *tileEnv = getenv("THIP_DEPTHWISE_TILE");
         const bool tileOff = tileEnv && tileEnv[0] == '0', tileOn = tileEnv && tileEnv[0] == '1';
