@@ -85,14 +85,16 @@ def test_dense_igemm_staged_epilogue(device, variant, monkeypatch):
     check(device, w.fully_connected_workload(257, 80, 48, realistic=True), kernel="igemm_dense_i8")
 
 
-@pytest.mark.parametrize("guarded", [False, True])
+@pytest.mark.parametrize("guarded", [False, True, "staged"])
 def test_stream_igemm(device, guarded, monkeypatch):
     """The pixel-streaming kernel (weights resident in LDS): every accumulator width, ragged M (also fewer rows than
     one group), k-step counts around the prefetch ring (one and two k-steps take a ring over several groups), N
     ending in half a 32-channel block, both requant tails; with the branch-free steady state and with every load
-    and store under its bounds check."""
+    and store under its bounds check, and with the results leaving through the per-wave LDS slices wherever these fit."""
     monkeypatch.setenv("THIP_IGEMM_DENSE_VARIANT", "11")
-    if guarded:
+    if guarded == "staged":
+        monkeypatch.setenv("THIP_STREAM_STAGE", "1")
+    elif guarded:
         monkeypatch.setenv("THIP_STREAM_GUARDED", "1")
     for M, K, N in [(17, 16, 16), (31, 64, 80), (32, 32, 96), (65, 48, 32), (4096 + 5, 64, 224)]:
         check(device, w.fully_connected_workload(M, K, N, realistic=True), kernel="igemm_stream_i8")

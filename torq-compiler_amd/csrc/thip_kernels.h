@@ -44,6 +44,7 @@ struct IgemmArgs {
     int32_t add_skip_first, add_w0, add_w1, add_bias, add_scale;
     Requant arq;
     int32_t stream_guarded;  // pixel-streaming kernel: keep every load and store under its bounds check (tests, tuning)
+    int32_t stream_stage;    // pixel-streaming kernel: results leave through a per-wave LDS slice as whole rows (its launcher sets it)
 };
 
 // Tile configurations of the igemm kernel.

@@ -963,6 +963,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
 // ---------------------------------------------------------------------------
 constexpr int kStreamRing = 4;
 constexpr size_t kStreamMaxLds = 64 * 1024;
+// LDS of the streaming kernel: weights [chunk][Kp], bias and scale [chunk] each, the run table, then (16-byte
+// aligned) the staging slices of the four waves: 32 rows of chunk + 16 bytes each (the 16 keep the 128-bit writes
+// of 16 lanes, one row each, on distinct banks)
+__host__ __device__ inline size_t igemmStreamStageOffset(int chunk, int Kp, bool runs) {
+    const size_t used = (size_t)chunk * Kp + 8 * (size_t)chunk + (runs ? (size_t)Kp / 16 * 4 : 0);
+    return (used + 15) & ~(size_t)15;
+}
+__host__ __device__ inline size_t igemmStreamStageBytes(int chunk) { return (size_t)4 * 32 * (chunk + 16); }
 
 // KS: 0, or the number of k-steps (1 or 2) when that is known at compile time and divides the ring: the ring then
 // runs over RING / KS pixel groups instead of one, so that loads stay RING k-steps ahead of the MFMAs even where a
@@ -1114,6 +1122,30 @@ __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArg
         };
         const int groupsFull = p.M / 32;
         const bool ragged = p.N - n0 < NB * 32;  // the upper 16 channels of the last block do not exist (N % 16 == 0)
+        // Staged stores: a group's 32 rows of this chunk go through the wave's LDS slice and leave as 16-byte pieces in
+        // row order, consecutive lanes taking consecutive pieces, so that a store instruction writes whole pixel rows
+        // (1 KiB of consecutive bytes where the chunk is the whole row) instead of 32 bytes per pixel: with 32-byte
+        // pieces the partly written lines of the output do not survive in L2 next to the activation reads.
+        // Piece q = i * 64 + lane of a group is the same for every group: its LDS and global offsets are computed once.
+        const bool stage = p.stream_stage != 0;
+        const int pitch = chunk + 16;
+        int8_t *slice = smem + igemmStreamStageOffset(chunk, p.Kp, false) + (size_t)wave * 32 * pitch;
+        const int piecesPerRow = (p.N - n0 < chunkN ? p.N - n0 : chunkN) >> 4;
+        int pieceLds[NB], pieceOut[NB];
+        {
+            const FastDiv divPieces = makeFastDiv((uint32_t)piecesPerRow);
+#pragma unroll
+            for (int i = 0; i < NB; i++) {
+                const int q = i * 64 + lane;
+                int row = (int)fastDiv((uint32_t)q, divPieces);
+                const int c = q - row * piecesPerRow;
+                // the last instruction may run past the 32 rows: those lanes write their first piece again (with one
+                // piece per row and one instruction, the piece of the lane 32 below)
+                if (i == 0) row = row < 32 ? row : row - 32;
+                pieceLds[i] = row < 32 ? row * pitch + c * 16 : pieceLds[0];
+                pieceOut[i] = row < 32 ? row * p.N + c * 16 : pieceOut[0];
+            }
+        }
         // bias and scale are read from LDS again for every group: kept in registers across the loop (where the compiler
         // hoists loop-invariant loads to) they would be 32 registers per block of channels and spill; an offset of
         // zero that the compiler cannot see through keeps the reads where they are
@@ -1161,7 +1193,9 @@ __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArg
                     const auto s02 = __builtin_amdgcn_permlane32_swap(d4[0], d4[2], false, false);
                     const auto s13 = __builtin_amdgcn_permlane32_swap(d4[1], d4[3], false, false);
                     v4i outv = {(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
-                    if (j == NB - 1 && ragged) {
+                    if (stage) {
+                        *(v4i *)(slice + fr * pitch + j * 32 + 16 * half) = outv;
+                    } else if (j == NB - 1 && ragged) {
                         // ragged last block: its 16 channels sit in the lower half lanes; the upper half lanes take over
                         // the second 8 of them, so that every lane stores (one store on either side of this branch)
                         const auto hi0 = __builtin_amdgcn_permlane32_swap((uint32_t)outv[2], (uint32_t)outv[2], false, false);
@@ -1171,6 +1205,13 @@ __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArg
                     } else {
                         *(v4i *)(orow + j * 32) = outv;
                     }
+                }
+                if (stage) {
+                    // LDS operations of a wave complete in order: the reads see the writes above, and the next group's
+                    // writes come behind these reads
+                    int8_t *obase = (int8_t *)p.out + (size_t)gq * 32 * p.N + n0;
+#pragma unroll
+                    for (int i = 0; i < NB; i++) *(v4i *)(obase + pieceOut[i]) = *(const v4i *)(slice + pieceLds[i]);
                 }
             };
             if (KS > 0) {
@@ -1311,7 +1352,7 @@ static hipError_t launchIgemmStream(const IgemmArgs &a, hipStream_t stream) {
     if ((a.loader != kLoaderDense && a.loader != kLoaderRuns) || a.out_dtype != kDtypeI8) return hipErrorInvalidValue;
     if (a.N % 16 != 0 || ((uintptr_t)a.out & 15) != 0 || ((uintptr_t)a.skip & 15) != 0) return hipErrorInvalidValue;
     const int chunk = igemmStreamChunk(a.Np);
-    const size_t smem = (size_t)chunk * a.Kp + 8 * (size_t)chunk + (a.loader == kLoaderRuns ? (size_t)a.Kp / 16 * 4 : 0);
+    size_t smem = (size_t)chunk * a.Kp + 8 * (size_t)chunk + (a.loader == kLoaderRuns ? (size_t)a.Kp / 16 * 4 : 0);
     if (chunk > 256 || smem > kStreamMaxLds) return hipErrorInvalidValue;
     const int nb = chunk / 32;
     if (a.loader == kLoaderRuns) {
@@ -1325,6 +1366,13 @@ static hipError_t launchIgemmStream(const IgemmArgs &a, hipStream_t stream) {
         // the branch-free steady state needs the block count at compile time (THIP_STREAM_GUARDED: the guarded loop only)
         IgemmArgs b = a;
         b.stream_guarded = getenv("THIP_STREAM_GUARDED") != nullptr;
+        // staged stores where the slices fit beside the weights, the stores outweigh the loads and the output is far larger than
+        // the caches (measured on a mobile network at batch 256: ahead from about 100 MB of output, behind at 40 MB);
+        // THIP_STREAM_STAGE=0 / 1: never / wherever they fit
+        const size_t staged = igemmStreamStageOffset(chunk, a.Kp, false) + igemmStreamStageBytes(chunk);
+        const char *stageEnv = getenv("THIP_STREAM_STAGE");
+        b.stream_stage = staged <= kStreamMaxLds && a.skip == nullptr && (stageEnv ? stageEnv[0] == '1' : a.N >= 2 * a.K && a.N >= 32 && (long long)a.M * a.N >= (64LL << 20));
+        if (b.stream_stage) smem = staged;
         switch (nb) {
         case 1: return launchIgemmStreamT<1, kLoaderDense>(b, smem, stream);
         case 2: return launchIgemmStreamT<2, kLoaderDense>(b, smem, stream);
