@@ -1127,7 +1127,7 @@ __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArg
         // (1 KiB of consecutive bytes where the chunk is the whole row) instead of 32 bytes per pixel: with 32-byte
         // pieces the partly written lines of the output do not survive in L2 next to the activation reads.
         // Piece q = i * 64 + lane of a group is the same for every group: its LDS and global offsets are computed once.
-        const bool stage = p.stream_stage != 0;
+        const bool stage = KS > 0 && p.stream_stage != 0;  // (the widths with more k-steps would pay for the offsets with a wave per SIMD)
         const int pitch = chunk + 16;
         int8_t *slice = smem + igemmStreamStageOffset(chunk, p.Kp, false) + (size_t)wave * 32 * pitch;
         const int piecesPerRow = (p.N - n0 < chunkN ? p.N - n0 : chunkN) >> 4;
@@ -1371,7 +1371,7 @@ static hipError_t launchIgemmStream(const IgemmArgs &a, hipStream_t stream) {
         // THIP_STREAM_STAGE=0 / 1: never / wherever they fit
         const size_t staged = igemmStreamStageOffset(chunk, a.Kp, false) + igemmStreamStageBytes(chunk);
         const char *stageEnv = getenv("THIP_STREAM_STAGE");
-        b.stream_stage = staged <= kStreamMaxLds && a.skip == nullptr && (stageEnv ? stageEnv[0] == '1' : a.N >= 2 * a.K && a.N >= 32 && (long long)a.M * a.N >= (64LL << 20));
+        b.stream_stage = staged <= kStreamMaxLds && a.skip == nullptr && (stageEnv ? stageEnv[0] == '1' : a.N >= 2 * a.K && a.N >= 32 && (long long)a.M * a.N >= (64LL << 20)) && a.Kp <= 64;
         if (b.stream_stage) smem = staged;
         switch (nb) {
         case 1: return launchIgemmStreamT<1, kLoaderDense>(b, smem, stream);
