@@ -101,14 +101,14 @@ class Loaded:
 # HBM bytes per launch of each workload's kernel, from rocprofv3 counters: FETCH_SIZE * 1.9995 + WRITE_SIZE * 1.0
 # (KiB per dispatch; the factors are what the same counters read for a plain 256 MiB copy, --copy-calibration).
 MEASURED_TRAFFIC = {
-    "fc_4096x4096x4096": (49382.7 * 1.9995 + 16553.8) * 1024,
-    "fc_512x4096x4096": (16479.1 * 1.9995 + 2048.0) * 1024,
-    "fc_16x2048x8192": (8401.1 * 1.9995 + 256.0) * 1024,
-    "conv_112x112x32_o64_3x3": (355.9 * 1.9995 + 784.0) * 1024,
-    "depthwise_b64": (14274.5 * 1.9995 + 7056.9) * 1024,
-    "depthwise_s1_b256": (63666.6 * 1.9995 + 113077.6) * 1024,
-    "avgpool_b64": (1991.5 * 1.9995 + 80.0) * 1024,
-    "add_b64": (4727.2 * 1.9995 + 4704.0) * 1024,
+    "fc_4096x4096x4096": (49392.2 * 1.9995 + 16566.1) * 1024,
+    "fc_512x4096x4096": (16481.0 * 1.9995 + 2048.0) * 1024,
+    "fc_16x2048x8192": (8408.1 * 1.9995 + 256.0) * 1024,
+    "conv_112x112x32_o64_3x3": (354.9 * 1.9995 + 784.0) * 1024,
+    "depthwise_b64": (15240.6 * 1.9995 + 7064.0) * 1024,
+    "depthwise_s1_b256": (63656.6 * 1.9995 + 113084.5) * 1024,
+    "avgpool_b64": (1991.6 * 1.9995 + 80.0) * 1024,
+    "add_b64": (4722.6 * 1.9995 + 4704.0) * 1024,
 }
 
 
