@@ -1311,19 +1311,17 @@ static hipError_t launchIgemmStreamA(const IgemmArgs &a, size_t smem, hipStream_
     }
     // every block copies the weights into LDS once, then strides over the pixel groups:
     // one resident set of blocks, each with several groups where the image is large
-    // blocks one CU holds (registers and LDS), asked once per LDS size
-    static size_t askedSmem = 0;
-    static int perCuAsked = 0;
-    if (askedSmem != smem || perCuAsked <= 0) {
+    // blocks one CU holds: by registers (asked once per kernel, with no LDS in the way) and by LDS
+    static int byRegs = 0;
+    if (byRegs <= 0) {
         int n = 0;
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void *)kernel, 256, smem) != hipSuccess || n <= 0) {
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void *)kernel, 256, 0) != hipSuccess || n <= 0) {
             (void)hipGetLastError();
-            n = (int)std::min<size_t>(NB <= 1 ? 7 : NB <= 2 ? 5 : NB <= 4 ? 4 : NB <= 6 ? 3 : 2, (160 * 1024) / smem);
+            n = NB <= 1 ? 7 : NB <= 2 ? 5 : NB <= 4 ? 4 : NB <= 6 ? 3 : 2;
         }
-        perCuAsked = n;
-        askedSmem = smem;
+        byRegs = n;
     }
-    const int perCu = std::min(perCuAsked, 8);
+    const int perCu = (int)std::min<size_t>((size_t)std::min(byRegs, 8), (160 * 1024) / ((smem + 1023) / 1024 * 1024));
     const int groups = (a.M + 31) / 32;
     const int chunk = igemmStreamChunk(a.Np), chunks = (a.Np + chunk - 1) / chunk;
     const int blocks = std::min((groups + 3) / 4, std::max(1, 256 * perCu / chunks));
