@@ -16,6 +16,7 @@ else here touches it.
 Prints ONE JSON line.
 """
 import argparse
+import hashlib
 import json
 import os
 import sys
@@ -28,6 +29,10 @@ sys.path.insert(0, ROOT)
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, TOP/s
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s
+# bandwidth rows are timed on buffer sets that together exceed this many bytes (twice the 256 MiB last-level cache),
+# dispatch i on set i mod n, so that every dispatch finds its operands in HBM
+COLD_WORKING_SET = 512 << 20
+MAX_BUFFER_SETS = 160
 
 
 def import_package():
@@ -88,6 +93,22 @@ class Loaded:
         """Returns mean ms per dispatch from HIP events on the executable's stream."""
         return self.exe.time_device(self.ptrs, self.lens, iterations)
 
+    def run_cold(self, iterations):
+        """The same on rotating copies of every binding (see COLD_WORKING_SET); returns (ms per dispatch, sets)."""
+        per_set = sum(self.lens)
+        sets = int(min(MAX_BUFFER_SETS, max(2, -(-COLD_WORKING_SET // per_set))))
+        hosts = list(self.wl.inputs) + self.outs
+        extra = [[self.dev.upload(h) for h in hosts] for _ in range(sets - 1)]
+        try:
+            all_sets = [self.ptrs] + extra
+            self.exe.time_device_rotating(all_sets, self.lens, sets)  # every set once: first touch
+            ms = self.exe.time_device_rotating(all_sets, self.lens, max(iterations, 2 * sets))
+        finally:
+            for ptrs in extra:
+                for p in ptrs:
+                    self.dev.free(p)
+        return ms, sets
+
     def output(self, i=0):
         o = self.outs[i]
         return self.dev.download(self.ptrs[len(self.wl.inputs) + i], o.shape, o.dtype)
@@ -100,6 +121,9 @@ class Loaded:
 
 # HBM bytes per launch of each workload's kernel, from rocprofv3 counters: FETCH_SIZE * 1.9995 + WRITE_SIZE * 1.0
 # (KiB per dispatch; the factors are what the same counters read for a plain 256 MiB copy, --copy-calibration).
+# They belong to the kernels as they were when the counters were read: TRAFFIC_KERNELS_SHA256 is the hash of
+# torq-compiler_amd/csrc/thip_kernels.hip at that time, and a run on other kernel sources reports traffic null.
+TRAFFIC_KERNELS_SHA256 = "unset"
 MEASURED_TRAFFIC = {
     "fc_4096x4096x4096": (49392.2 * 1.9995 + 16566.1) * 1024,
     "fc_512x4096x4096": (16481.0 * 1.9995 + 2048.0) * 1024,
@@ -112,8 +136,13 @@ MEASURED_TRAFFIC = {
 }
 
 
+def kernels_sha256():
+    with open(os.path.join(ROOT, "torq-compiler_amd", "csrc", "thip_kernels.hip"), "rb") as f:
+        return hashlib.sha256(f.read()).hexdigest()
+
+
 def roofline(wl, bound, ms, name=None):
-    traffic = MEASURED_TRAFFIC.get(name)
+    traffic = MEASURED_TRAFFIC.get(name) if kernels_sha256() == TRAFFIC_KERNELS_SHA256 else None
     traffic = None if traffic is None else int(round(traffic))
     if bound == "mfma":
         achieved = wl.ops / (ms * 1e-3) / 1e12
@@ -161,30 +190,42 @@ def verify_sample(loaded):
     return bool(np.array_equal(got, oracle_eval(wl)[0]))
 
 
-def cpu_baseline(wl, target_seconds=12.0):
-    """Times the CPU oracle on a bounded sample of the default workload on this host's cores."""
+def cpu_baseline(wl, target_seconds=10.0, single_thread_seconds=6.0):
+    """Times the CPU oracle on a bounded sample of the default workload on this host's cores: with every core
+    (`value`, `cores`) and with one thread (`single_thread`)."""
     from oracle import oracle as orc
     a = dict(wl.attrs)
     wts, sb = a.pop("weights"), a.pop("scale_bias")
     x = wl.inputs[0]
     M, K = x.shape
     N = wts.shape[0]
-    rows = min(M, 8)
-    t0 = time.perf_counter()
-    orc.fully_connected(x[:rows], wts, sb, **a)
-    dt = max(time.perf_counter() - t0, 1e-4)
-    rows = int(min(M, max(rows, rows * 2.0 / dt)))  # about 2 s per pass
-    passes, dt = 0, 0.0
-    t0 = time.perf_counter()
-    while dt < target_seconds:
+
+    def timed(seconds):
+        rows = min(M, 4)
+        t0 = time.perf_counter()
         orc.fully_connected(x[:rows], wts, sb, **a)
-        passes += 1
-        dt = time.perf_counter() - t0
-    rows_total = rows * passes
-    gops = 2.0 * rows_total * K * N / dt / 1e9
-    return {"value": round(gops, 2), "unit": "GOP/s", "cores": orc.threads(), "kind": "port",
-            "sample": "%d passes over the first %d of %d rows of the same (M,K,N)=(%d,%d,%d) fully_connected, %.1f s, C oracle with OpenMP"
-                      % (passes, rows, M, M, K, N, dt)}
+        dt = max(time.perf_counter() - t0, 1e-4)
+        rows = int(min(M, max(rows, rows * 2.0 / dt)))  # about 2 s per pass
+        passes, dt = 0, 0.0
+        t0 = time.perf_counter()
+        while dt < seconds:
+            orc.fully_connected(x[:rows], wts, sb, **a)
+            passes += 1
+            dt = time.perf_counter() - t0
+        return 2.0 * rows * passes * K * N / dt / 1e9, passes, rows, dt
+
+    cores = orc.threads()
+    gops, passes, rows, dt = timed(target_seconds)
+    orc.set_threads(1)
+    try:
+        gops1, passes1, rows1, dt1 = timed(single_thread_seconds)
+    finally:
+        orc.set_threads(cores)
+    what = "%d passes over the first %d of %d rows of the same (M,K,N)=(%d,%d,%d) fully_connected, %.1f s, C oracle"
+    return {"value": round(gops, 2), "unit": "GOP/s", "cores": cores, "kind": "port",
+            "sample": (what + " with OpenMP") % (passes, rows, M, M, K, N, dt),
+            "single_thread": {"value": round(gops1, 2), "unit": "GOP/s", "cores": 1,
+                              "sample": (what + ", one thread") % (passes1, rows1, M, M, K, N, dt1)}}
 
 
 def main():
@@ -247,11 +288,23 @@ def main():
                 continue
             o = Loaded(pkg, dev, mk())
             o.run(5)
-            ms = o.run(50)
+            warm = o.run(50)
+            names = o.exe.op_kernels()
+            row = {"kernel": names[-1 if "transpose" in names[0] else 0], "bound": bnd}
+            if bnd == "hbm":
+                # what the roofline fraction is quoted on: operands cold in every dispatch; the repeated dispatch of one
+                # buffer set (served by the last-level cache where it fits) is reported next to it
+                ms, sets = o.run_cold(50)
+                row.update({"us": round(ms * 1e3, 2), "us_cache_warm": round(warm * 1e3, 2), "buffer_sets": sets})
+            else:
+                ms = warm
+                row["us"] = round(ms * 1e3, 2)
             r = roofline(o.wl, bnd, ms)
-            per_op[name] = {"us": round(ms * 1e3, 2), "kernel": o.exe.op_kernels()[-1 if "transpose" in o.exe.op_kernels()[0] else 0],
-                            "GOP/s": round(o.wl.ops / (ms * 1e-3) / 1e9, 1), "GB/s": round(o.wl.bytes / (ms * 1e-3) / 1e9, 1),
-                            "bound": bnd, "frac": r["frac"]}
+            row.update({"GOP/s": round(o.wl.ops / (ms * 1e-3) / 1e9, 1), "GB/s": round(o.wl.bytes / (ms * 1e-3) / 1e9, 1), "frac": r["frac"]})
+            if not args.no_cpu:
+                row["parity_checked"] = verify_sample(o)
+                ok = ok and row["parity_checked"]
+            per_op[name] = row
             o.close()
 
     mbv2 = {}

@@ -432,9 +432,19 @@ thip_status_t thip_executable_time(thip_executable_t *executable,
                                    const thip_dispatch_state_t *state, int32_t iterations,
                                    float *out_ms_per_dispatch);
 
+/* Same measurement with dispatch i taking states[i % state_count]: with enough distinct buffer sets the working
+ * set exceeds the last-level cache and a bandwidth-bound program is timed on memory that is cold in every
+ * dispatch.  Device bindings only.  (No counterpart in the reference; benchmark support like the one above.) */
+thip_status_t thip_executable_time_rotating(thip_executable_t *executable,
+                                            const thip_dispatch_state_t *states, uint32_t state_count,
+                                            int32_t iterations, float *out_ms_per_dispatch);
+
 /* Introspection used by the harness and the tests. */
 thip_status_t thip_executable_op_count(thip_executable_t *executable, uint32_t *out_count);
-/* Name of the kernel chosen for op `index` (e.g. "igemm_i8_128x128x64"). */
+/* Name of the kernel that op `index` launches, as a profiler shows it without namespace and argument list
+ * (e.g. "igemm_dense_i8<256,256,2,2,4,1,1,0>", "depthwise3x3_strip_i8<2,2,1,3,1>").  It is settled when the
+ * executable is created (from the record, the alignment of its operands and the THIP_* environment switches as
+ * they are then) and does not change afterwards. */
 thip_status_t thip_executable_op_kernel(thip_executable_t *executable, uint32_t index,
                                         char *name, size_t capacity);
 thip_status_t thip_executable_binding_count(thip_executable_t *executable, uint32_t *out_count);

@@ -16,7 +16,7 @@ HEADER = np.dtype([("magic", "<u4"), ("version", "<u4"), ("arch", "<u4"), ("flag
                    ("consts_offset", "<u8"), ("data_offset", "<u8"), ("total_size", "<u8")])
 _I32 = ["out_dtype", "input_zp", "output_zp", "output_min", "output_max", "shift",
         "N", "H", "W", "C", "OH", "OW", "OC", "KH", "KW", "SH", "SW", "PL", "PR", "PT", "PB",
-        "M", "K", "Kp", "Nn", "Np", "w0", "w1", "bias0", "scale0", "TB", "TR", "TS", "pre_shift", "t0_clamp", "r2"]
+        "M", "K", "Kp", "Nn", "Np", "w0", "w1", "bias0", "scale0", "TB", "TR", "TS", "pre_shift", "t0_clamp", "TP"]
 OP = np.dtype([("kind", "<u4"), ("variant", "<u4"), ("loader", "<u4"), ("gran", "<u4")] +
               [(n, "<i4") for n in _I32] +
               [(n, REF) for n in ["in0", "in1", "weights", "bias", "scale", "table", "out"]])
@@ -86,12 +86,14 @@ def run(blob, binding_arrays):
         sh, zp, mn, mx = int(op["shift"]), int(op["output_zp"]), int(op["output_min"]), int(op["output_max"])
         if kind == K_TRANSPOSE:
             B, R, S = int(op["TB"]), int(op["TR"]), int(op["TS"])
+            pitch = int(op["TP"]) or R  # output rows `pitch` elements apart; what lies beyond R is left alone
+            assert pitch >= R
             if int(op["gran"]) == 2:
                 src = view(op["in0"], B * R * S * 2).view(np.uint16).reshape(B, R, S)
-                view(op["out"], B * R * S * 2).view(np.uint16)[:] = np.ascontiguousarray(src.transpose(0, 2, 1)).reshape(-1)
+                view(op["out"], B * S * pitch * 2).view(np.uint16).reshape(B, S, pitch)[:, :, :R] = src.transpose(0, 2, 1)
                 continue
             src = view(op["in0"], B * R * S).reshape(B, R, S)
-            view(op["out"], B * R * S)[:] = np.ascontiguousarray(src.transpose(0, 2, 1)).reshape(-1)
+            view(op["out"], B * S * pitch).reshape(B, S, pitch)[:, :, :R] = src.transpose(0, 2, 1)
         elif kind in (K_IGEMM, K_FC_SKINNY):
             M, K, Kp, N, Np = (int(op[k]) for k in ["M", "K", "Kp", "Nn", "Np"])
             Wp = view(op["weights"], Np * Kp).view(np.int8).reshape(Np, Kp).astype(np.int64)

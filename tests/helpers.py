@@ -48,6 +48,10 @@ def oracle_eval(wl):
         return res if a["fold"] else res + [w16[None]]
     if kind == "addbf16":
         return [orc.add_bf16(wl.inputs[0], wl.inputs[1], a["weights"], a["bias"], output_min=a["output_min"], output_max=a["output_max"])]
+    if kind == "matmul":
+        res = orc.matmul(x, a["input2"], a["scale_bias"], output_zp=a["output_zp"], output_min=a["output_min"], output_max=a["output_max"],
+                         shift=a["shift"], out_dtype=a["out_dtype"])
+        return [res.reshape(wl.outputs[0][0])]
     if kind == "matmulbf16":
         res = orc.matmul_bf16(x, a["input2"], a["bias"])
         return [res.reshape(wl.outputs[0][0])]
@@ -85,6 +89,11 @@ def run_on_gpu(device, wl, via="host"):
         return outs, exe.op_kernels()
     finally:
         exe.close()
+
+
+def families(kernels):
+    """Kernel names without their template arguments: "maxpool_i8<16>" -> "maxpool_i8"."""
+    return [k.split("<")[0] for k in kernels]
 
 
 def assert_bit_exact(got, want, what=""):

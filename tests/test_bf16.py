@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 
 import desc_interp
-from helpers import assert_bf16_close, assert_bit_exact, bf16_ordered, oracle_eval, run_on_gpu
+from helpers import assert_bf16_close, assert_bit_exact, bf16_ordered, families, oracle_eval, run_on_gpu
 from oracle import oracle as orc
 from torq_compiler_amd import Executable, Program, ThipError, runtime, workloads as w
 
@@ -261,14 +261,14 @@ def test_gpu_bf16_conv2d_and_depthwise(device):
         shape = [1, 1, 1, 1]
         shape[3 if wl.attrs["nhwc"] else 1] = -1
         assert_bf16_close(got[0], oracle_eval(wl)[0], wl.name, magnitude=np.broadcast_to(wabs.reshape(shape), got[0].shape))
-        assert "fc_bf16" in kernels
+        assert "fc_bf16" in families(kernels)
     for wl in [w.conv2d_bf16_workload(depthwise=True, C=12, stride=(2, 2), pad=(0, 1, 0, 1), clamp=(-0.5, 0.5)),
                w.conv2d_bf16_workload(depthwise=True, N=2, C=5, H=7, W=9, nhwc=False),
                w.conv2d_bf16_workload(depthwise=True, N=4, C=144, H=56, W=56)]:
         print("[gpu-case]", wl.name, flush=True)
         got, kernels = run_on_gpu(device, wl, via="device")
         assert_bit_exact(got[0], oracle_eval(wl)[0], wl.name)
-        assert "depthwise_bf16" in kernels
+        assert "depthwise_bf16" in families(kernels)
 
 
 @pytest.mark.gpu
@@ -285,7 +285,7 @@ def test_gpu_bf16_wide_n(device):
         w16 = orc.expand_weights(wl.attrs["weights"], wl.attrs["scale"], wl.attrs["qbias"], block_size=wl.attrs["block"],
                                  output_min=wl.attrs["expand_min"], output_max=wl.attrs["expand_max"])
         assert_bf16_close(got[0], oracle_eval(wl)[0].reshape(got[0].shape), wl.name, magnitude=f(wl.inputs[0]) @ f(w16))
-        assert kernels == ["fc_bf16"], kernels
+        assert families(kernels) == ["fc_bf16_wide"], kernels  # >= 1024 column blocks, short K: every wave streams its own columns
 
 
 @pytest.mark.gpu
@@ -296,7 +296,7 @@ def test_gpu_bf16_avg_pool(device):
         print("[gpu-case]", wl.name, flush=True)
         got, kernels = run_on_gpu(device, wl, via="device")
         assert_bit_exact(got[0], oracle_eval(wl)[0], wl.name)
-        assert kernels == ["avgpool_bf16"]
+        assert families(kernels) == ["avgpool_bf16"]
 
 
 @pytest.mark.gpu
@@ -317,9 +317,9 @@ def test_gpu_expand_weights(device):
         assert_bf16_close(got[0], want[0].reshape(got[0].shape), wl.name, magnitude=f(wl.inputs[0]) @ f(w16))
         if how == "own":
             assert_bit_exact(got[1], want[1], wl.name + " expansion")
-            assert kernels == ["expand_weights_bf16", "transpose_i8", "fc_bf16"], kernels
+            assert families(kernels) == ["expand_weights_bf16", "transpose_i8", "fc_bf16"], kernels
         else:
-            assert kernels == ["fc_bf16"], kernels
+            assert families(kernels) == ["fc_bf16"], kernels
 
 
 @pytest.mark.gpu
@@ -330,7 +330,7 @@ def test_gpu_bf16_add(device):
         print("[gpu-case]", wl.name, flush=True)
         got, kernels = run_on_gpu(device, wl, via="device")
         assert_bit_exact(got[0], oracle_eval(wl)[0], wl.name)
-        assert kernels == ["add_bf16"]
+        assert families(kernels) == ["add_bf16"]
 
 
 @pytest.mark.gpu

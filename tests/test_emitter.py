@@ -68,6 +68,50 @@ def test_fully_connected_descriptor(mkn):
     assert int(d.ops[0]["kind"]) == want_kind
 
 
+# int8 torq_hl.matmul.  The first five are the shapes of the reference's own fixtures:
+# tests/testdata/tosa_ops/matmul-in-int8-out-int16-{1024x128x1024,64x128x2048}.mlir and
+# tests/testdata/linalg_ops/{matmul-in-int8-out-int16-noalign,batch-matmul-in-int8-out-int16,matvec-in-int8-out-int16}.mlir
+# (12x56x168 has K % 16 != 0; the matrix-vector product is N = 1).  Then: batch broadcast on either side, constant
+# and run-time input2, every result type, a real rescale, ragged K and N.
+MATMUL = [
+    dict(B=1, M=1024, K=128, N=1024),
+    dict(B=1, M=64, K=128, N=2048),
+    dict(B=1, M=12, K=56, N=168, batch1=False, batch2=False),
+    dict(B=1, M=64, K=128, N=256),
+    dict(B=1, M=128, K=64, N=1, batch1=False, batch2=False),
+    dict(B=3, M=20, K=64, N=48, batch1=False),
+    dict(B=3, M=20, K=64, N=48, batch2=False),
+    dict(B=3, M=20, K=64, N=48, batch1=False, constant_rhs=True),
+    dict(B=2, M=33, K=96, N=40, batch2=False, constant_rhs=True),
+    dict(B=2, M=33, K=96, N=40, constant_rhs=True, out_dtype=np.int32),
+    dict(B=2, M=9, K=61, N=37, out_dtype=np.int32),
+    dict(B=2, M=9, K=61, N=37, constant_rhs=True, out_dtype=np.int8, bias=-77, scale=(1 << 30) + 12345, shift=41, output_zp=3),
+    dict(B=1, M=300, K=80, N=130, out_dtype=np.int8, bias=1234, scale=(1 << 30) + 999, shift=42, output_zp=-5, clamp=(-100, 90)),
+    dict(B=2, M=5, K=7, N=3, bias=5, scale=3, shift=1),
+]
+
+
+def matmul_id(kw):
+    return "-".join("%s%s" % (k[:2], getattr(v, "__name__", v)) for k, v in kw.items())
+
+
+@pytest.mark.parametrize("kw", MATMUL, ids=matmul_id)
+def test_matmul_descriptor(kw):
+    wl = w.matmul_workload(**kw)
+    outs, d = interp(wl)
+    want = oracle_eval(wl)[0]
+    assert_bit_exact(outs[0], want, wl.name)
+    kinds = [int(o["kind"]) for o in d.ops]
+    Bb = kw["B"] if kw.get("batch2", True) else 1
+    if kw.get("constant_rhs"):
+        assert kinds == [desc_interp.K_IGEMM] * Bb  # one record per weight matrix; a broadcast input2 takes all rows at once
+    else:
+        assert kinds == [desc_interp.K_TRANSPOSE] * Bb + [desc_interp.K_IGEMM] * kw["B"]
+        assert all(int(o["TP"]) == int(d.ops[-1]["Kp"]) for o in d.ops[:Bb])  # transposed into zero-padded rows of Kp
+    if kw.get("out_dtype", np.int16) == np.int16 and kw["K"] >= 64 and "scale" not in kw:
+        assert (want == 32767).any() or (want == -32768).any() or kw["K"] < 128  # int16 results of a long K saturate: the clamp is exercised
+
+
 @pytest.mark.parametrize("kw", [dict(H=8, W=8, C=4), dict(H=32, W=32, C=64, kernel=(3, 3), pad=(1, 1, 1, 1)), dict(H=10, W=10, C=4, kernel=(5, 5), stride=(1, 1)),
                                 dict(H=10, W=10, C=4, kernel=(1, 3), stride=(1, 3), pad=(0, 2, 0, 0), input_zp=-7)])
 @pytest.mark.parametrize("nhwc", [True, False])

@@ -8,8 +8,8 @@ import sys
 import numpy as np
 import pytest
 
-from helpers import assert_bit_exact, oracle_eval, oracle_network, run_on_gpu
-from test_emitter import CONV, _chain_program, _padded_chain
+from helpers import assert_bit_exact, families, oracle_eval, oracle_network, run_on_gpu
+from test_emitter import CONV, MATMUL, _chain_program, _padded_chain, matmul_id
 from torq_compiler_amd import Executable, ThipError, runtime, workloads as w
 
 pytestmark = pytest.mark.gpu
@@ -26,7 +26,12 @@ def check(device, wl, via="host", kernel=None):
     want = oracle_eval(wl)
     assert_bit_exact(got[0], want[0], wl.name)
     if kernel is not None:
-        assert any(kernel in k for k in kernels), (kernels, kernel)
+        # `kernel` names what rocprof would show for the op: a whole instantiation ("name<args>") must match exactly,
+        # a bare name must be the name in front of the template arguments
+        if "<" in kernel:
+            assert kernel in kernels, (kernels, kernel)
+        else:
+            assert kernel in families(kernels), (kernels, kernel)
     return kernels
 
 
@@ -43,7 +48,7 @@ def test_conv2d_config0_realistic(device):
 def test_conv2d_config0_nchw_boundary(device):
     """Same op with the reference's literal N,C,H,W boundary: transposes at the bindings."""
     kernels = check(device, w.conv2d_workload(realistic=True, nhwc=False))
-    assert kernels[0] == "transpose_i8" and kernels[-1] == "transpose_i8"
+    assert kernels[0] == "transpose_i8<1>" and kernels[-1] == "transpose_i8<1>"
 
 
 @pytest.mark.parametrize("kw", CONV)
@@ -57,8 +62,8 @@ def test_conv2d_every_tile_variant(device, variant, monkeypatch):
     monkeypatch.setenv("THIP_IGEMM_VARIANT", str(variant))
     k = check(device, w.conv2d_workload(N=2, H=28, W=28, C=32, O=96, realistic=True))
     assert runtime.lib()  # the variant is baked into the descriptor at serialize time
-    names = ["128x128", "256x256", "64x64", "256x128"]
-    assert names[variant] in k[0]
+    names = ["igemm_i8<128,128,64,", "igemm_i8<256,256,64,", "igemm_i8<64,64,64,", "igemm_i8<256,128,64,"]
+    assert k[0].startswith(names[variant]), k
     check(device, w.conv2d_workload(N=1, H=15, W=17, C=24, O=40, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True))
     check(device, w.fully_connected_workload(300, 192, 520, realistic=True))
 
@@ -67,9 +72,11 @@ def test_conv2d_every_tile_variant(device, variant, monkeypatch):
 def test_dense_igemm_every_tile_variant(device, variant, monkeypatch):
     """The LDS-DMA kernel: whole tiles, ragged M / N / K tails, K shorter than the stage ring."""
     monkeypatch.setenv("THIP_IGEMM_DENSE_VARIANT", str(variant))
+    tile = {4: (256, 256), 5: (128, 128), 6: (128, 256), 7: (64, 64), 8: (256, 128), 9: (256, 64), 10: (256, 32), 12: (128, 64), 13: (64, 128)}[variant]
     k = check(device, w.fully_connected_workload(300, 192, 520, realistic=True))
-    assert "igemm_dense_i8" in k[0]
-    check(device, w.fully_connected_workload(512, 1024, 512, realistic=True))
+    assert k[0].startswith("igemm_dense_i8<%d,%d," % tile) and k[0].endswith(",0,0>"), k  # N % 16 != 0: results leave through LDS
+    k = check(device, w.fully_connected_workload(512, 1024, 512, realistic=True))
+    assert k[0].startswith("igemm_dense_i8<%d,%d," % tile) and k[0].endswith(",1,0>"), k  # N % 16 == 0, shift >= 33: the in-register epilogue
     check(device, w.fully_connected_workload(257, 80, 48, realistic=True))
     check(device, w.fully_connected_workload(33, 16, 1000, realistic=True))
     check(device, w.fully_connected_workload(1000, 4096, 272, realistic=True))
@@ -81,8 +88,9 @@ def test_dense_igemm_staged_epilogue(device, variant, monkeypatch):
     """The LDS-staged epilogue with the 32-bit requant tail (the in-register one normally takes these shapes)."""
     monkeypatch.setenv("THIP_IGEMM_DENSE_VARIANT", str(variant))
     monkeypatch.setenv("THIP_NO_DIRECT_EPILOGUE", "1")
-    check(device, w.fully_connected_workload(300, 192, 528, realistic=True), kernel="igemm_dense_i8")
-    check(device, w.fully_connected_workload(257, 80, 48, realistic=True), kernel="igemm_dense_i8")
+    for mkn in [(300, 192, 528), (257, 80, 48)]:
+        k = check(device, w.fully_connected_workload(*mkn, realistic=True), kernel="igemm_dense_i8")
+        assert k[0].endswith(",0,0>"), k  # the staged epilogue
 
 
 @pytest.mark.parametrize("guarded", [False, True, "staged"])
@@ -121,9 +129,9 @@ def test_stream_igemm(device, guarded, monkeypatch):
 @pytest.mark.parametrize("shift", [0, 1, 6, 31, 32, 33, 34, 40, 62])
 def test_igemm_shift_boundaries(device, shift):
     """Both epilogue tails of the MFMA kernels (generic 64-bit, and 32-bit for shift >= 33) around their switch."""
-    check(device, w.fully_connected_workload(200, 256, 144, shift=shift), kernel="igemm_dense")
+    check(device, w.fully_connected_workload(200, 256, 144, shift=shift), kernel="igemm_dense_i8")
     check(device, w.fully_connected_workload(40, 72, 20, shift=shift, output_zp=-7), kernel="igemm_i8")
-    check(device, w.fully_connected_workload(3, 64, 40, shift=shift), kernel="fc_skinny")
+    check(device, w.fully_connected_workload(3, 64, 40, shift=shift), kernel="fc_skinny_mfma")
 
 
 def test_conv2d_mbv2_layer_shapes(device):
@@ -161,7 +169,7 @@ def test_conv2d_int32_output(device):
 def test_fully_connected_config1(device, mkn):
     M = mkn[0]
     check(device, w.fully_connected_workload(*mkn, realistic=True), via="device",
-          kernel="fc_skinny" if M <= 16 else "igemm_")
+          kernel=("fc_skinny<1,4>" if M == 1 else "fc_skinny_mfma") if M <= 16 else ("igemm_dense_i8" if M >= 512 else None))
 
 
 def test_fully_connected_config1_literal_ranges(device):
@@ -179,20 +187,38 @@ def test_fully_connected_skinny_kernels(device, dot4, monkeypatch):
     """At most 16 rows: the MFMA kernel (3 rows and up) and the dot-product kernel, K and N with ragged ends."""
     if dot4:
         monkeypatch.setenv("THIP_SKINNY_DOT4", "1")
-    for mkn in [(3, 16, 16), (5, 48, 20), (16, 272, 1000), (9, 1040, 37), (4, 256, 64), (2, 512, 32), (16, 2048, 8192), (7, 4096, 130)]:
-        check(device, w.fully_connected_workload(*mkn, realistic=True), kernel="fc_skinny")
-    check(device, w.fully_connected_workload(12, 528, 100, shift=7), kernel="fc_skinny")
+    def expected(M):
+        if M >= 3 and not dot4:
+            return "fc_skinny_mfma"
+        return "fc_skinny<1,4>" if M == 1 else "fc_skinny<4,4>" if M <= 4 else "fc_skinny<8,2>" if M <= 8 else "fc_skinny<16,2>"
+    for mkn in [(3, 16, 16), (5, 48, 20), (16, 272, 1000), (9, 1040, 37), (4, 256, 64), (2, 512, 32), (16, 2048, 8192), (7, 4096, 130), (1, 64, 48)]:
+        check(device, w.fully_connected_workload(*mkn, realistic=True), kernel=expected(mkn[0]))
+    check(device, w.fully_connected_workload(12, 528, 100, shift=7), kernel=expected(12))
 
 
 def test_fully_connected_without_skinny_kernel(device, monkeypatch):
     monkeypatch.setenv("THIP_NO_SKINNY", "1")
-    check(device, w.fully_connected_workload(16, 2048, 512, realistic=True), kernel="igemm_")
+    check(device, w.fully_connected_workload(16, 2048, 512, realistic=True), kernel="igemm_dense_i8")
+
+
+# ---- matmul (int8) ----------------------------------------------------------------------------
+@pytest.mark.parametrize("kw", MATMUL, ids=matmul_id)
+def test_matmul_int8(device, kw):
+    """torq_hl.matmul with ONE (bias, scale) pair (compiler/torq/Conversions/TorqHLToTorqHW/MatMulPattern.cpp:66-86): the
+    reference's fixture shapes, batch broadcast on either side, constant and run-time input2, every result type."""
+    wl = w.matmul_workload(**kw)
+    kernels = check(device, wl, via="device" if kw["M"] >= 64 else "host")
+    if not kw.get("constant_rhs"):
+        assert kernels[0] == "transpose_i8<1>"
+    assert any(k.startswith("igemm") for k in kernels)
 
 
 # ---- bandwidth ops ---------------------------------------------------------------------------
-@pytest.mark.parametrize("batch", [1, 8])
+@pytest.mark.parametrize("batch", [1, 8, 64])
 def test_depthwise_config2a(device, batch):
-    check(device, w.depthwise_workload(N=batch), via="device", kernel="depthwise3x3_dot4_i8")
+    """56x56x144 stride 2 at the benchmark's batch sizes; batch 64 has enough waves for the rolling-window kernel."""
+    check(device, w.depthwise_workload(N=batch), via="device",
+          kernel="depthwise3x3_strip_i8<2,2,1,3,1>" if batch == 64 else "depthwise3x3_dot4_i8<1,0>")
 
 
 @pytest.mark.parametrize("kw", [
@@ -213,6 +239,7 @@ def test_depthwise_3x3_kernels(device, which, monkeypatch):
     row segments."""
     monkeypatch.setenv("THIP_DEPTHWISE_TILE", "1" if which == "tile" else "0")
     monkeypatch.setenv("THIP_DEPTHWISE_STRIP", {"strip": "1", "strip1": "2"}.get(which, "0"))
+    seen = set()
     for kw in [dict(N=2, H=13, W=15, C=16, stride=(1, 1), pad=(1, 1, 1, 1)), dict(N=1, H=14, W=14, C=48, stride=(1, 1), pad=(0, 0, 0, 0)),
                dict(N=1, H=9, W=31, C=32, stride=(1, 1), pad=(1, 1, 1, 1)), dict(N=2, H=21, W=22, C=16, stride=(2, 2), pad=(0, 1, 0, 1)),
                dict(N=1, H=15, W=13, C=80, stride=(2, 2), pad=(1, 1, 1, 1)), dict(N=1, H=3, W=3, C=16, stride=(1, 1), pad=(0, 0, 0, 0)),
@@ -223,7 +250,19 @@ def test_depthwise_3x3_kernels(device, which, monkeypatch):
                dict(N=1, H=45, W=7, C=32, stride=(2, 2), pad=(1, 1, 1, 1), input_zp=3),
                dict(N=1, H=1, W=5, C=16, stride=(1, 1), pad=(1, 1, 1, 1)),
                dict(N=2, H=112, W=112, C=32, stride=(2, 2), pad=(0, 1, 0, 1), input_zp=-128)]:
-        check(device, w.depthwise_workload(**kw), kernel="depthwise3x3_dot4_i8")
+        seen.add(check(device, w.depthwise_workload(**kw), kernel=depthwise_kernel(which, kw["stride"][0]))[0])
+    assert len(seen) >= (1 if which == "rows" else 2), seen  # both strides took a kernel of their own
+
+
+def depthwise_kernel(which, stride):
+    """The 3x3 depthwise kernel the switches of test_depthwise_3x3_kernels select at this stride."""
+    if which == "tile":
+        return "depthwise3x3_tile_i8<4,2,1,4>" if stride == 1 else "depthwise3x3_dot4_i8"
+    if which == "strip":
+        return "depthwise3x3_strip_i8<2,1,1,4,3>" if stride == 1 else "depthwise3x3_strip_i8<2,2,1,3,1>"
+    if which == "strip1":
+        return "depthwise3x3_strip_i8<2,1,1,4,3>" if stride == 1 else "depthwise3x3_strip_i8<1,2,1,4,3>"
+    return "depthwise3x3_dot4_i8"
 
 
 @pytest.mark.parametrize("which", ["rows", "tile", "strip", "strip1"])
@@ -237,16 +276,16 @@ def test_depthwise_shift_boundaries(device, which, monkeypatch):
     for shift in [0, 2, 3, 12, 24, 31, 32, 33, 34, 40, 62]:
         for zp in (-7, 100):
             check(device, w.depthwise_workload(N=1, H=12, W=10, C=32, stride=stride, pad=(1, 1, 1, 1), shift=shift, output_zp=zp),
-                  kernel="depthwise3x3_dot4_i8")
+                  kernel=depthwise_kernel(which, stride[0]))
     check(device, w.depthwise_workload(N=1, H=12, W=10, C=32, stride=(2, 2), pad=(1, 1, 1, 1), shift=31, output_zp=-128),
-          kernel="depthwise3x3_dot4_i8")
+          kernel=depthwise_kernel(which, 2))
     monkeypatch.setenv("THIP_NO_PRE_SHIFT", "1")
-    check(device, w.depthwise_workload(N=1, H=12, W=10, C=32, stride=(1, 1), pad=(1, 1, 1, 1), shift=24), kernel="depthwise3x3_dot4_i8")
+    check(device, w.depthwise_workload(N=1, H=12, W=10, C=32, stride=(1, 1), pad=(1, 1, 1, 1), shift=24), kernel=depthwise_kernel(which, 1))
 
 
-@pytest.mark.parametrize("batch", [1, 8])
+@pytest.mark.parametrize("batch", [1, 8, 64])
 def test_maxpool_config2b(device, batch):
-    check(device, w.maxpool_workload(N=batch), via="device", kernel="maxpool_i8")
+    check(device, w.maxpool_workload(N=batch), via="device", kernel="maxpool_i8<16>")
 
 
 @pytest.mark.parametrize("kw", [dict(H=8, W=8, C=4), dict(H=8, W=8, C=1), dict(H=32, W=32, C=64, kernel=(3, 3), pad=(1, 1, 1, 1)),
@@ -296,15 +335,37 @@ def test_padded_channel_chain(device, nhwc):
     assert_bit_exact(out, want, "padded chain")
 
 
-@pytest.mark.parametrize("batch", [1, 3])
+@pytest.mark.parametrize("batch", [1, 3, 32])
 def test_mobilenet_v2_full(device, batch):
-    """benchmark configuration 3: the whole 64-op network as one program, final logits bit-exact."""
+    """benchmark configuration 3: the whole 64-op network as one program, final logits of every image bit-exact."""
     wl = w.mobilenet_v2_workload(batch=batch)
     announce(wl.name)
     got, kernels = run_on_gpu(device, wl, via="device")
     assert_bit_exact(got[0], oracle_network(wl), wl.name)
     # 64 ops; a residual add behind a streaming convolution (enough pixels) is folded into it
-    assert 54 <= len(kernels) <= 64 and "transpose_i8" not in kernels
+    assert 54 <= len(kernels) <= 64 and "transpose_i8" not in families(kernels)
+
+
+def test_mobilenet_v2_batch256(device):
+    """benchmark configuration 3 at its largest batch: the first and the last four images against the oracle, and every
+    image independent of its neighbours (copies of an image at other batch positions give copies of its logits)."""
+    wl = w.mobilenet_v2_workload(batch=256)
+    announce(wl.name)
+    x = wl.inputs[0]
+    x[100] = x[0]
+    x[201] = x[255]
+    x[77] = x[130]
+    got, kernels = run_on_gpu(device, wl, via="device")
+    got = got[0]
+    ends = w.mobilenet_v2_workload(batch=8)  # same seed: the same weights
+    ends.inputs[0][:4] = x[:4]
+    ends.inputs[0][4:] = x[-4:]
+    want = oracle_network(ends)
+    assert_bit_exact(got[:4], want[:4], "first four images")
+    assert_bit_exact(got[-4:], want[4:], "last four images")
+    assert np.array_equal(got[100], got[0]) and np.array_equal(got[201], got[255]) and np.array_equal(got[77], got[130])
+    assert len(np.unique(got, axis=0)) >= 200  # the logits do depend on the image
+    assert "transpose_i8" not in families(kernels)
 
 
 def test_mobilenet_v2_nchw_declared(device):
@@ -313,7 +374,7 @@ def test_mobilenet_v2_nchw_declared(device):
     announce(wl.name, "nchw")
     got, kernels = run_on_gpu(device, wl)
     assert_bit_exact(got[0], oracle_network(wl), wl.name)
-    assert kernels.count("transpose_i8") == 1 and kernels[0] == "transpose_i8"
+    assert families(kernels).count("transpose_i8") == 1 and kernels[0] == "transpose_i8<1>"
 
 
 def test_graph_replay_matches_oracle_every_time(device):
@@ -413,7 +474,7 @@ def test_event_log_and_timing(device, tmp_path):
     rows = list(csv.DictReader(log.open()))
     assert list(rows[0].keys()) == ["dispatch_name", "invocation_id", "action_id", "timestamp_us", "event", "kernel"]
     assert len(rows) == 2 * 5 and [r["event"] for r in rows[:2]] == ["NSS_START_BEGIN", "NSS_START_END"]
-    assert all(r["kernel"] == "maxpool_i8" and r["action_id"] == "0" for r in rows)
+    assert all(r["kernel"] == "maxpool_i8<16>" and r["action_id"] == "0" for r in rows)
     assert [int(r["invocation_id"]) for r in rows] == [i // 2 for i in range(10)]
     assert all(int(a["timestamp_us"]) <= int(b["timestamp_us"]) for a, b in zip(rows, rows[1:]))
     # a blocking run on host buffers logs the whole dispatch
@@ -441,7 +502,7 @@ def test_residual_add_in_the_streaming_epilogue(device, monkeypatch):
         wl = w.pointwise_add_workload(**kw)
         print("[gpu-case]", wl.name, flush=True)
         got, kernels = run_on_gpu(device, wl, via="device")
-        assert kernels == ["igemm_stream_i8"], kernels
+        assert families(kernels) == ["igemm_stream_i8"] and kernels[0].split(",")[2] == "1", kernels  # the instantiation with the add
         assert_bit_exact(got[0], oracle_eval(wl)[0], wl.name)
     # few pixels: the small dense tile adds the residual in its in-register epilogue
     for kw in [dict(N=1, H=8, W=8), dict(N=1, H=14, W=14, C=384, O=64, other_first=True), dict(N=2, H=7, W=7, C=960, O=160), dict(N=1, H=28, W=28, C=192, O=32),
@@ -449,7 +510,7 @@ def test_residual_add_in_the_streaming_epilogue(device, monkeypatch):
         wl = w.pointwise_add_workload(**kw)
         print("[gpu-case]", wl.name, flush=True)
         got, kernels = run_on_gpu(device, wl, via="device")
-        assert kernels == ["igemm_dense_i8_64x64x64"], kernels
+        assert kernels == ["igemm_dense_i8<64,64,2,2,4,4,1,1>"], kernels
         assert_bit_exact(got[0], oracle_eval(wl)[0], wl.name)
     folded, kernels = run_on_gpu(device, w.mobilenet_v2_workload(batch=8), via="device")
     monkeypatch.setenv("THIP_NO_ADD_FUSION", "1")

@@ -62,7 +62,7 @@ struct DescConst {
 
 // Kernel kinds.  One record = one kernel launch.
 enum Kind : uint32_t {
-    kKindTranspose = 1,  // [B, R, S] -> [B, S, R] elements of `gran` bytes (0 or 1: bytes; 2: bf16)
+    kKindTranspose = 1,  // [B, R, S] -> [B, S, R] elements of `gran` bytes (0 or 1: bytes; 2: bf16), output rows TP elements apart
     // conv2d / fully_connected / matmul on MFMA.  A residual add fused by the emitter (pixel-streaming variant, dense
     // loader, int8): in1 = the add's other operand, table = ResidualAddParams (in1.space none: no add)
     kKindIgemm = 2,
@@ -140,7 +140,9 @@ struct DescOp {
     // when the bound of |acc + bias| is too large for pre_shift but every channel's result already saturates
     // at +-t0_clamp, so the clamp cannot change a result.
     int32_t t0_clamp;
-    int32_t reserved[1];
+    // transpose: elements from one output row to the next (0: TR, rows packed); a wider pitch leaves the rest of
+    // each row as it was (the zero padding of a run-time matmul operand)
+    int32_t TP;
     DescRef in0;
     DescRef in1;
     DescRef weights;  // packed weights

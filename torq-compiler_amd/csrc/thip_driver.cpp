@@ -60,6 +60,8 @@ struct thip_executable_t {
     hipGraphExec_t graphExec = nullptr;
     bool graphsDisabled = false;
     uint64_t invocation = 0;             // dispatches so far (the event log's invocation_id)
+    Tuning tuning;                       // the environment's switches as they were when the executable was created
+    std::vector<std::string> kernelNames;  // per record: the kernel its launcher resolved at creation
 };
 
 static thip_status_t hipFail(hipError_t e, const char *what) {
@@ -172,9 +174,10 @@ static thip_status_t checkOpFootprint(const thip_executable_t *e, uint32_t i) {
     case kKindTranspose: {
         if (!positive({op.TB, op.TR, op.TS})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad transpose extents", i);
         if (op.gran > 2) return fail(THIP_INVALID_ARGUMENT, "op %u: transpose element size %u", i, op.gran);
-        const uint64_t bytes = (uint64_t)op.TB * op.TR * op.TS * (op.gran == 2 ? 2 : 1);
-        if ((s = need(op.in0, bytes, "in"))) return s;
-        return need(op.out, bytes, "out");
+        if (op.TP != 0 && op.TP < op.TR) return fail(THIP_INVALID_ARGUMENT, "op %u: transpose pitch %d is below its row length %d", i, op.TP, op.TR);
+        const uint64_t elem = op.gran == 2 ? 2 : 1, pitch = op.TP ? (uint64_t)op.TP : (uint64_t)op.TR;
+        if ((s = need(op.in0, (uint64_t)op.TB * op.TR * op.TS * elem, "in"))) return s;
+        return need(op.out, (uint64_t)op.TB * op.TS * pitch * elem, "out");
     }
     case kKindIgemm: {
         if (!positive({op.M, op.K, op.Kp, op.Nn, op.Np, op.N, op.H, op.W, op.C, op.OH, op.OW})) {
@@ -334,6 +337,7 @@ static thip_status_t checkOpFootprint(const thip_executable_t *e, uint32_t i) {
     }
 }
 
+// The kernel family of a record (error messages before the launcher has named the instantiation).
 static const char *opKernelName(const DescOp &op) {
     switch (op.kind) {
     case kKindTranspose: return "transpose_i8";
@@ -374,14 +378,15 @@ static uint8_t *resolve(const thip_executable_t *e, const DescRef &r, uint8_t *c
     }
 }
 
-static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *bp) {
+// Launches record i, or (ctx.name set) only asks its launcher which kernel it takes for these operands.
+static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *bp, const LaunchCtx &ctx) {
     const DescOp &op = e->ops[i];
     const Requant rq{op.shift, op.output_zp, op.output_min, op.output_max, op.pre_shift, op.t0_clamp};
     hipError_t err = hipSuccess;
     switch (op.kind) {
     case kKindTranspose: {
-        TransposeArgs a{(const int8_t *)resolve(e, op.in0, bp), (int8_t *)resolve(e, op.out, bp), op.TB, op.TR, op.TS, op.gran == 2 ? 2 : 1};
-        err = launchTranspose(a, e->stream);
+        TransposeArgs a{(const int8_t *)resolve(e, op.in0, bp), (int8_t *)resolve(e, op.out, bp), op.TB, op.TR, op.TS, op.gran == 2 ? 2 : 1, op.TP ? op.TP : op.TR};
+        err = launchTranspose(a, ctx);
         break;
     }
     case kKindIgemm: {
@@ -410,14 +415,14 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
             a.add_w0 = ap.w0; a.add_w1 = ap.w1; a.add_bias = ap.bias; a.add_scale = ap.scale;
             a.arq = Requant{ap.shift, ap.output_zp, ap.output_min, ap.output_max, 0, 0};
         }
-        err = launchIgemm(a, op.variant, e->stream);
+        err = launchIgemm(a, op.variant, ctx);
         break;
     }
     case kKindFcSkinny: {
         FcSkinnyArgs a{(const int8_t *)resolve(e, op.in0, bp), (const int8_t *)resolve(e, op.weights, bp),
                        (const int32_t *)resolve(e, op.bias, bp), (const int32_t *)resolve(e, op.scale, bp),
                        resolve(e, op.out, bp), op.M, op.Nn, op.K, op.out_dtype, rq};
-        err = launchFcSkinny(a, e->stream);
+        err = launchFcSkinny(a, ctx);
         break;
     }
     case kKindDepthwise: {
@@ -425,31 +430,31 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
                         (const int32_t *)resolve(e, op.bias, bp), (const int32_t *)resolve(e, op.scale, bp),
                         (int8_t *)resolve(e, op.out, bp), op.N, op.H, op.W, op.C, op.OH, op.OW, op.KH, op.KW,
                         op.SH, op.SW, op.PT, op.PL, op.input_zp, op.variant, rq};
-        err = launchDepthwise(a, e->stream);
+        err = launchDepthwise(a, ctx);
         break;
     }
     case kKindMaxPool: {
         MaxPoolArgs a{(const int8_t *)resolve(e, op.in0, bp), (int8_t *)resolve(e, op.out, bp), op.N, op.H, op.W, op.C,
                       op.OH, op.OW, op.KH, op.KW, op.SH, op.SW, op.PT, op.PL, op.input_zp, op.output_min, op.output_max};
-        err = launchMaxPool(a, e->stream);
+        err = launchMaxPool(a, ctx);
         break;
     }
     case kKindAvgPool: {
         AvgPoolArgs a{(const int8_t *)resolve(e, op.in0, bp), (int8_t *)resolve(e, op.out, bp), op.N, op.H * op.W, op.C,
                       op.w0, op.bias0, op.scale0, rq};
-        err = launchAvgPool(a, e->stream);
+        err = launchAvgPool(a, ctx);
         break;
     }
     case kKindAdd: {
         AddArgs a{(const int8_t *)resolve(e, op.in0, bp), (const int8_t *)resolve(e, op.in1, bp),
                   (int8_t *)resolve(e, op.out, bp), (int64_t)op.C, op.w0, op.w1, op.bias0, op.scale0, rq};
-        err = launchAdd(a, e->stream);
+        err = launchAdd(a, ctx);
         break;
     }
     case kKindIm2colBf16: {
         Im2colBf16Args a{(const uint16_t *)resolve(e, op.in0, bp), (uint16_t *)resolve(e, op.out, bp), op.N, op.H, op.W, op.C,
                          op.OH, op.OW, op.KH, op.KW, op.SH, op.SW, op.PT, op.PL, op.Kp};
-        err = launchIm2colBf16(a, e->stream);
+        err = launchIm2colBf16(a, ctx);
         break;
     }
     case kKindDepthwiseBf16: {
@@ -459,7 +464,7 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
         DepthwiseBf16Args a{(const uint16_t *)resolve(e, op.in0, bp), (const uint16_t *)resolve(e, op.weights, bp),
                             (const float *)resolve(e, op.bias, bp), (uint16_t *)resolve(e, op.out, bp), op.N, op.H, op.W, op.C,
                             op.OH, op.OW, op.KH, op.KW, op.SH, op.SW, op.PT, op.PL, lo, hi};
-        err = launchDepthwiseBf16(a, e->stream);
+        err = launchDepthwiseBf16(a, ctx);
         break;
     }
     case kKindAddBf16: {
@@ -471,7 +476,7 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
         AddBf16Args a{(const uint16_t *)resolve(e, op.in0, bp), (const uint16_t *)resolve(e, op.in1, bp),
                       (uint16_t *)resolve(e, op.out, bp), (int64_t)op.C, asFloat(op.w0 << 16), asFloat(op.w1 << 16),
                       asFloat(op.bias0), asFloat(op.output_min), asFloat(op.output_max)};
-        err = launchAddBf16(a, e->stream);
+        err = launchAddBf16(a, ctx);
         break;
     }
     case kKindFcBf16: {
@@ -490,7 +495,7 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
             memcpy(&a.qlo, &op.bias0, 4);
             memcpy(&a.qhi, &op.scale0, 4);
         }
-        err = launchFcBf16(a, e->stream);
+        err = launchFcBf16(a, ctx);
         break;
     }
     case kKindAvgPoolBf16: {
@@ -501,14 +506,14 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
         memcpy(&a.bias, &op.bias0, 4);
         memcpy(&a.lo, &op.output_min, 4);
         memcpy(&a.hi, &op.output_max, 4);
-        err = launchAvgPoolBf16(a, e->stream);
+        err = launchAvgPoolBf16(a, ctx);
         break;
     }
     case kKindEltwise: {
         EltwiseArgs a{resolve(e, op.in0, bp), (op.variant == kEltMul || op.variant >= kEltAnd) ? resolve(e, op.in1, bp) : nullptr, resolve(e, op.out, bp), (int64_t)op.C,
                       (int32_t)op.variant, (int32_t)op.gran, op.out_dtype == THIP_DTYPE_I8 ? 1 : op.out_dtype == THIP_DTYPE_I16 ? 2 : 4, op.w1,
                       op.w0, op.bias0, op.scale0, op.output_min, op.output_max, rq};
-        err = launchEltwise(a, e->stream);
+        err = launchEltwise(a, ctx);
         break;
     }
     case kKindExpandWeights: {
@@ -517,13 +522,13 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
                             (int32_t)op.gran, op.Np, 0.0f, 0.0f};
         memcpy(&a.lo, &op.output_min, 4);
         memcpy(&a.hi, &op.output_max, 4);
-        err = launchExpandWeights(a, e->stream);
+        err = launchExpandWeights(a, ctx);
         break;
     }
     default: return fail(THIP_INTERNAL, "op %u has unknown kind %u", i, op.kind);
     }
     if (err != hipSuccess) {
-        return fail(THIP_INTERNAL, "op %u (%s): launch failed: %s", i, opKernelName(op), hipGetErrorString(err));
+        return fail(THIP_INTERNAL, "op %u (%s): launch failed: %s", i, ctx.name ? opKernelName(op) : e->kernelNames[i].c_str(), hipGetErrorString(err));
     }
     return THIP_OK;
 }
@@ -561,9 +566,9 @@ static thip_status_t checkState(const thip_executable_t *e, const thip_dispatch_
 static thip_status_t enqueueOps(thip_executable_t *e, uint8_t *const *bp) {
     for (uint32_t i = 0; i < e->header.op_count; i++) {
         // a kernel launch is what starting an NSS task is on the reference's hardware
-        logEvent(e->device, e->invocation, (int32_t)i, "NSS_START", "BEGIN", opKernelName(e->ops[i]));
-        if (thip_status_t s = launchOp(e, i, bp)) return s;
-        logEvent(e->device, e->invocation, (int32_t)i, "NSS_START", "END", opKernelName(e->ops[i]));
+        logEvent(e->device, e->invocation, (int32_t)i, "NSS_START", "BEGIN", e->kernelNames[i].c_str());
+        if (thip_status_t s = launchOp(e, i, bp, LaunchCtx{e->stream, &e->tuning, nullptr, 0})) return s;
+        logEvent(e->device, e->invocation, (int32_t)i, "NSS_START", "END", e->kernelNames[i].c_str());
     }
     return THIP_OK;
 }
@@ -775,6 +780,21 @@ thip_status_t thip_executable_create(thip_device_t *device, const void *blob, si
     }
     e->staging.assign(h.binding_count, nullptr);
     e->graphsDisabled = getenv("THIP_NO_GRAPH") != nullptr;
+    // Which kernel each record runs is settled now, from the record, the alignment of its operands and the
+    // environment's switches, and kept: the launchers are asked in naming mode (they also configure their kernels,
+    // which must not happen later inside a stream capture).  Bindings stand in as aligned placeholder addresses:
+    // device bindings must be 16-byte aligned and staged host bindings are, so a dispatch resolves the same way.
+    e->tuning = tuningFromEnvironment();
+    e->kernelNames.assign(h.op_count, std::string());
+    {
+        uint8_t *placeholder[64];
+        for (auto &ptr : placeholder) ptr = (uint8_t *)(uintptr_t)0x1000000;
+        for (uint32_t i = 0; i < h.op_count; i++) {
+            char name[96] = "";
+            if (thip_status_t st = launchOp(e, i, placeholder, LaunchCtx{nullptr, &e->tuning, name, sizeof(name)})) return bail(st);
+            e->kernelNames[i] = name[0] ? name : opKernelName(e->ops[i]);
+        }
+    }
     *out_executable = e;
     return THIP_OK;
 }
@@ -880,6 +900,35 @@ thip_status_t thip_executable_time(thip_executable_t *e, const thip_dispatch_sta
     return THIP_OK;
 }
 
+thip_status_t thip_executable_time_rotating(thip_executable_t *e, const thip_dispatch_state_t *states, uint32_t state_count,
+                                            int32_t iterations, float *out_ms) {
+    if (!e || !out_ms || !states) return fail(THIP_INVALID_ARGUMENT, "null argument");
+    if (iterations <= 0 || state_count == 0) return fail(THIP_INVALID_ARGUMENT, "iterations and state_count must be positive");
+    for (uint32_t s = 0; s < state_count; s++) {
+        if (thip_status_t st = checkState(e, &states[s], true)) return st;
+    }
+    std::lock_guard<std::mutex> lock(e->mutex);
+    THIP_HIP(hipSetDevice(e->device->ordinal), "hipSetDevice");
+    THIP_HIP(hipEventRecord(e->evStart, e->stream), "hipEventRecord");
+    for (int32_t it = 0; it < iterations; it++) {
+        const thip_dispatch_state_t &st = states[(uint32_t)it % state_count];
+        uint8_t *bp[64] = {nullptr};
+        for (uint32_t i = 0; i < e->header.binding_count; i++) bp[i] = (uint8_t *)st.binding_ptrs[i];
+        const thip_status_t s = enqueueDevice(e, bp);
+        e->invocation++;
+        if (s != THIP_OK) {
+            (void)hipStreamSynchronize(e->stream);
+            return s;
+        }
+    }
+    THIP_HIP(hipEventRecord(e->evStop, e->stream), "hipEventRecord");
+    THIP_HIP(hipEventSynchronize(e->evStop), "hipEventSynchronize");
+    float ms = 0.f;
+    THIP_HIP(hipEventElapsedTime(&ms, e->evStart, e->evStop), "hipEventElapsedTime");
+    *out_ms = ms / (float)iterations;
+    return THIP_OK;
+}
+
 thip_status_t thip_executable_op_count(thip_executable_t *e, uint32_t *out_count) {
     if (!e || !out_count) return fail(THIP_INVALID_ARGUMENT, "null argument");
     *out_count = e->header.op_count;
@@ -889,7 +938,7 @@ thip_status_t thip_executable_op_count(thip_executable_t *e, uint32_t *out_count
 thip_status_t thip_executable_op_kernel(thip_executable_t *e, uint32_t index, char *name, size_t capacity) {
     if (!e || !name || capacity == 0) return fail(THIP_INVALID_ARGUMENT, "null argument");
     if (index >= e->header.op_count) return fail(THIP_OUT_OF_RANGE, "op %u of %u", index, e->header.op_count);
-    snprintf(name, capacity, "%s", opKernelName(e->ops[index]));
+    snprintf(name, capacity, "%s", e->kernelNames[index].c_str());
     return THIP_OK;
 }
 

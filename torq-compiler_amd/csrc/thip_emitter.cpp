@@ -188,7 +188,7 @@ class Emitter {
         return THIP_OK;
     }
 
-    void emitTranspose(DescRef in, DescRef out, int64_t B, int64_t R, int64_t S, uint32_t elem = 1) {
+    void emitTranspose(DescRef in, DescRef out, int64_t B, int64_t R, int64_t S, uint32_t elem = 1, int64_t outPitch = 0) {
         DescOp op;
         memset(&op, 0, sizeof(op));
         op.kind = kKindTranspose;
@@ -196,6 +196,7 @@ class Emitter {
         op.TB = (int32_t)B;
         op.TR = (int32_t)R;
         op.TS = (int32_t)S;
+        op.TP = (int32_t)outPitch;
         op.in0 = in;
         op.out = out;
         ops_.push_back(op);
@@ -454,7 +455,17 @@ class Emitter {
                 absSum[(size_t)n] += wv < 0 ? -(int64_t)wv : wv;
             }
         }
-        planPreShift(&base, absSum);
+        base.weights = newConst(packed);
+        finishIgemm(base, M, N, K, loader, variant, absSum);
+    }
+
+    // The record of an igemm whose [Np][Kp] weight matrix (base.weights) is in place: requant plan, extents, k-table.
+    // absWeightSum[n] bounds sum_k |w[n][k]|.
+    void finishIgemm(DescOp base, int64_t M, int64_t N, int64_t K, uint32_t loader, uint32_t variant, const std::vector<int64_t> &absWeightSum) {
+        const IgemmTile &t = igemmTile(variant);
+        const int64_t Kp = roundUp(K, t.bk), Np = roundUp(N, t.bn);
+        const bool dense = loader == kLoaderDense;
+        planPreShift(&base, absWeightSum);
         base.kind = kKindIgemm;
         base.variant = variant;
         base.loader = loader;
@@ -463,7 +474,6 @@ class Emitter {
         base.Kp = (int32_t)Kp;
         base.Nn = (int32_t)N;
         base.Np = (int32_t)Np;
-        base.weights = newConst(packed);
         if (dense) {
             base.gran = 16;
         } else if (loader == kLoaderRuns) {
@@ -848,37 +858,35 @@ thip_status_t Emitter::emitMatmul(const thip_hl_matmul_t &c) {
     }
     // input2 produced at run time: transpose each batch into a zero-padded
     // [Np][Kp] buffer (intermediates are zero-filled when the executable is
-    // created and the padding is never written), then run the dense igemm.
+    // created and the padding is never written), then run the igemm on it: the dense loader
+    // when the rows of input1 are whole 16-byte chunks, the gather loader (K as the channel axis
+    // of a 1x1 window) otherwise.
     DescRef bRef;
     if (thip_status_t s = literalInput(c.input2, "torq_hl.matmul input2", &bRef)) return s;
-    if (K % 16 != 0) return fail(THIP_UNIMPLEMENTED, "%s: a run-time input2 needs K %% 16 == 0", what);
-    const uint32_t variant = chooseIgemmVariant(M, N, true);
+    const uint32_t loader = K % 16 == 0 ? kLoaderDense : kLoaderGather;
+    const uint32_t variant = chooseIgemmVariant(M, N, loader == kLoaderDense, K, init->dtype);
     const IgemmTile &t = igemmTile(variant);
     const int64_t Kp = roundUp(K, t.bk), Np = roundUp(N, t.bn);
-    if (Kp != K) return fail(THIP_UNIMPLEMENTED, "%s: a run-time input2 needs K %% %d == 0", what, t.bk);
     std::vector<DescRef> packed;
     for (int64_t r = 0; r < (Bb == 1 ? 1 : B); r++) {
         DescRef t2 = newTemp((uint64_t)(Np * Kp));
         DescRef src = bRef;
         src.offset += (uint64_t)(r * K * N);
-        emitTranspose(src, t2, 1, K, N);
+        emitTranspose(src, t2, 1, K, N, 1, Kp);
         packed.push_back(t2);
     }
+    // nothing is known about the values of a run-time operand: every |w| may be 128
+    const std::vector<int64_t> absSum((size_t)N, 128 * K);
     for (int64_t batch = 0; batch < B; batch++) {
         DescOp o = op;
-        o.kind = kKindIgemm;
-        o.variant = variant;
-        o.loader = kLoaderDense;
-        o.gran = 16;
         o.N = (int32_t)M;
-        o.M = (int32_t)M; o.K = (int32_t)K; o.Kp = (int32_t)Kp; o.Nn = (int32_t)N; o.Np = (int32_t)Np;
         o.in0 = aRef;
         o.in0.offset += (uint64_t)(Ba == 1 ? 0 : batch * M * K);
         o.out = outRef;
         o.out.offset += (uint64_t)(batch * M * N) * outElem;
         o.weights = packed[(size_t)(Bb == 1 ? 0 : batch)];
-        if (thip_status_t s = splitScaleBias(c.scale_bias, "torq_hl.matmul scale_bias", N, Np, true, &o.bias, &o.scale)) return s;
-        ops_.push_back(o);
+        if (thip_status_t s = splitScaleBias(c.scale_bias, "torq_hl.matmul scale_bias", N, roundUp(N, 256), true, &o.bias, &o.scale)) return s;
+        finishIgemm(o, M, N, K, loader, variant, absSum);
     }
     return THIP_OK;
 }

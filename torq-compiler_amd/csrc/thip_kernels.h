@@ -23,6 +23,34 @@ struct Requant {
     int32_t t0_clamp;
 };
 
+// Tuning and test switches, read from the environment once per executable (when it is created), never on the launch
+// path: a record keeps the kernel it was given for as long as its executable lives.
+struct Tuning {
+    bool noStreamDeep = false;      // THIP_NO_STREAM_DEEP: pixel-streaming GEMM, no ring over several pixel groups
+    bool streamGuarded = false;     // THIP_STREAM_GUARDED: pixel-streaming GEMM, the bounds-checked loop only
+    int streamStage = -1;           // THIP_STREAM_STAGE=0 / 1: staged stores never / wherever they fit (-1: by size)
+    bool noDirectEpilogue = false;  // THIP_NO_DIRECT_EPILOGUE: dense GEMM, results through LDS
+    bool skinnyDot4 = false;        // THIP_SKINNY_DOT4: few-row fully_connected on v_dot4 only
+    int depthwiseStrip = -1;        // THIP_DEPTHWISE_STRIP=0 / 1 / 2: rolling-window kernel off / on / on with one column per thread at stride 2
+    int depthwiseTile = -1;         // THIP_DEPTHWISE_TILE=0 / 1: register-tile kernel off / on
+    long long depthwiseTileMin = 0; // THIP_DEPTHWISE_TILE_MIN: thread-outputs from which the tile kernel is taken
+    int depthwisePixels = 0;        // THIP_DEPTHWISE_P: pixels per thread of the window-row kernel
+    int fcWideU = 0;                // THIP_FC_WIDE_U: k-steps per register buffer of the wide bf16 kernel
+    bool noFcDeep = false;          // THIP_NO_FC_DEEP
+    bool noFcWide = false;          // THIP_NO_FC_WIDE
+};
+Tuning tuningFromEnvironment();
+
+// How a launcher is called.  name == nullptr: enqueue the kernel on `stream`.  Otherwise: validate the arguments,
+// configure the kernel it would launch (dynamic LDS limit, occupancy query: things that must not happen inside a
+// stream capture), write that kernel's name ("kernel<template arguments>") to `name` and enqueue nothing.
+struct LaunchCtx {
+    hipStream_t stream;
+    const Tuning *tuning;
+    char *name;
+    size_t name_capacity;
+};
+
 struct IgemmArgs {
     const int8_t *A;        // activations: NHWC image batch, or dense [M, K]
     const int8_t *Bp;       // packed weights [Np][Kp], K contiguous, zero padded
@@ -87,7 +115,7 @@ inline bool igemmStreamFits(int64_t N, int64_t K, int32_t out_dtype) {
     const int64_t chunk = igemmStreamChunk((int)Np), chunks = (Np + chunk - 1) / chunk;
     return chunk * Kp + 8 * chunk + Kp / 4 <= 64 * 1024 && (chunks - 1) * K <= N;
 }
-hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, hipStream_t stream);
+hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, const LaunchCtx &ctx);
 
 struct FcSkinnyArgs {
     const int8_t *x;      // [M][K]
@@ -100,7 +128,7 @@ struct FcSkinnyArgs {
     Requant rq;
 };
 constexpr int kFcSkinnyMaxRows = 16;
-hipError_t launchFcSkinny(const FcSkinnyArgs &a, hipStream_t stream);
+hipError_t launchFcSkinny(const FcSkinnyArgs &a, const LaunchCtx &ctx);
 
 // bf16 fully_connected: out[m][n] = bf16(clamp(sum_k x[m][k] * w[n][k] + bias[n])), fp32 accumulate.
 struct FcBf16Args {
@@ -156,7 +184,7 @@ inline int fcBf16PreferredSplit(int M, int N, int K) {
     if (split > 16) split = 16;
     return split < 2 ? 1 : (int)split;
 }
-hipError_t launchFcBf16(const FcBf16Args &a, hipStream_t stream);
+hipError_t launchFcBf16(const FcBf16Args &a, const LaunchCtx &ctx);
 
 // Integer elementwise ops with the ACT stage behind them.  fma: out = R1(in0 * w0); mul: out = R1(in0 * in1) (an
 // input of one element is broadcast); both with ONE (bias, scale) pair.  clamp / abs / negate / i2i: the input
@@ -179,7 +207,7 @@ struct EltwiseArgs {
     int32_t lo, hi;               // clamp / abs / negate / i2i
     Requant rq;                   // fma / mul
 };
-hipError_t launchEltwise(const EltwiseArgs &a, hipStream_t stream);
+hipError_t launchEltwise(const EltwiseArgs &a, const LaunchCtx &ctx);
 
 // bf16 global average pool: out[n][c] = bf16(clamp(sum_u in[n][u][c] * weight + bias)), summed over the frame
 // in order, in fp32.
@@ -189,7 +217,7 @@ struct AvgPoolBf16Args {
     int32_t N, HW, C;
     float weight, bias, lo, hi;
 };
-hipError_t launchAvgPoolBf16(const AvgPoolBf16Args &a, hipStream_t stream);
+hipError_t launchAvgPoolBf16(const AvgPoolBf16Args &a, const LaunchCtx &ctx);
 
 // torq_hl.expand_weights: out[k][n] = bf16(clamp(w[k][n] * scale[k / block][n] + bias[k / block][n])).
 struct ExpandWeightsArgs {
@@ -200,7 +228,7 @@ struct ExpandWeightsArgs {
     int32_t K, N, block, bias_cols;
     float lo, hi;
 };
-hipError_t launchExpandWeights(const ExpandWeightsArgs &a, hipStream_t stream);
+hipError_t launchExpandWeights(const ExpandWeightsArgs &a, const LaunchCtx &ctx);
 
 struct DepthwiseArgs {
     const int8_t *in;     // NHWC
@@ -217,7 +245,7 @@ enum DepthwiseVariant : uint32_t {
     kDepthwiseGeneric = 0,  // any window, any channel count
     kDepthwiseDot4Rows = 1, // 3x3 window, C % 16 == 0: one v_dot4 per window row and channel
 };
-hipError_t launchDepthwise(const DepthwiseArgs &a, hipStream_t stream);
+hipError_t launchDepthwise(const DepthwiseArgs &a, const LaunchCtx &ctx);
 
 struct MaxPoolArgs {
     const int8_t *in;  // NHWC
@@ -225,7 +253,7 @@ struct MaxPoolArgs {
     int32_t N, H, W, C, OH, OW, KH, KW, SH, SW, PT, PL;
     int32_t input_zp, out_min, out_max;
 };
-hipError_t launchMaxPool(const MaxPoolArgs &a, hipStream_t stream);
+hipError_t launchMaxPool(const MaxPoolArgs &a, const LaunchCtx &ctx);
 
 struct AvgPoolArgs {
     const int8_t *in;  // [N][HW][C]
@@ -234,7 +262,7 @@ struct AvgPoolArgs {
     int32_t weight, bias, scale;
     Requant rq;
 };
-hipError_t launchAvgPool(const AvgPoolArgs &a, hipStream_t stream);
+hipError_t launchAvgPool(const AvgPoolArgs &a, const LaunchCtx &ctx);
 
 struct AddArgs {
     const int8_t *in0;
@@ -244,7 +272,7 @@ struct AddArgs {
     int32_t w0, w1, bias, scale;
     Requant rq;
 };
-hipError_t launchAdd(const AddArgs &a, hipStream_t stream);
+hipError_t launchAdd(const AddArgs &a, const LaunchCtx &ctx);
 
 // bf16 patch matrix of a convolution: out[m][k] with m = (n * OH + oy) * OW + ox and k = (kh * KW + kw) * C + ci,
 // rows padded with zeros to Kp; positions outside the image are zero.
@@ -253,7 +281,7 @@ struct Im2colBf16Args {
     uint16_t *out;       // [M][Kp]
     int32_t N, H, W, C, OH, OW, KH, KW, SH, SW, PT, PL, Kp;
 };
-hipError_t launchIm2colBf16(const Im2colBf16Args &a, hipStream_t stream);
+hipError_t launchIm2colBf16(const Im2colBf16Args &a, const LaunchCtx &ctx);
 
 // bf16 depthwise convolution: fp32 accumulation over (kh, kw), float bias and clamp.
 struct DepthwiseBf16Args {
@@ -264,7 +292,7 @@ struct DepthwiseBf16Args {
     int32_t N, H, W, C, OH, OW, KH, KW, SH, SW, PT, PL;
     float lo, hi;
 };
-hipError_t launchDepthwiseBf16(const DepthwiseBf16Args &a, hipStream_t stream);
+hipError_t launchDepthwiseBf16(const DepthwiseBf16Args &a, const LaunchCtx &ctx);
 
 // bf16 add: out = bf16(clamp(in0 * w0 + in1 * w1 + bias)) in fp32.
 struct AddBf16Args {
@@ -274,14 +302,15 @@ struct AddBf16Args {
     int64_t count;
     float w0, w1, bias, lo, hi;
 };
-hipError_t launchAddBf16(const AddBf16Args &a, hipStream_t stream);
+hipError_t launchAddBf16(const AddBf16Args &a, const LaunchCtx &ctx);
 
 struct TransposeArgs {
     const int8_t *in;  // [B][R][S]
     int8_t *out;       // [B][S][R]
     int32_t B, R, S;
     int32_t elem;      // element size in bytes: 1 or 2
+    int32_t out_pitch; // elements between output rows (>= R); the batch stride of the output is S * out_pitch
 };
-hipError_t launchTranspose(const TransposeArgs &a, hipStream_t stream);
+hipError_t launchTranspose(const TransposeArgs &a, const LaunchCtx &ctx);
 
 }  // namespace thip

@@ -15,7 +15,11 @@
 #include "thip_kernels.h"
 
 #include <algorithm>
+#include <cstdio>
 #include <cstdlib>
+#include <initializer_list>
+#include <mutex>
+#include <string>
 #include <type_traits>
 
 #include "thip_descriptor.h"
@@ -27,6 +31,30 @@ typedef int v2i __attribute__((ext_vector_type(2)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
 constexpr int kDtypeI8 = 1, kDtypeI16 = 2, kDtypeI32 = 3;
+
+// "name<a,b,...>": the kernel instantiation as a profiler shows it (without its namespace and argument list).
+static std::string kernelLabel(const char *name, std::initializer_list<int> params) {
+    std::string s = name;
+    char sep = '<';
+    for (int v : params) {
+        s += sep;
+        s += std::to_string(v);
+        sep = ',';
+    }
+    return s + ">";
+}
+static const char *labelText(const char *s) { return s; }
+static const char *labelText(const std::string &s) { return s.c_str(); }
+// A launch site.  With ctx.name set the launcher is only asked which kernel it would launch for these arguments (the
+// driver asks once per record when an executable is created): the name is written and nothing is enqueued.
+#define THIP_ENQUEUE(ctx, label, kernel, grid, block, lds, ...)                           \
+    do {                                                                                  \
+        if ((ctx).name) {                                                                 \
+            snprintf((ctx).name, (ctx).name_capacity, "%s", labelText(label));            \
+        } else {                                                                          \
+            hipLaunchKernelGGL(kernel, grid, block, lds, (ctx).stream, __VA_ARGS__);      \
+        }                                                                                 \
+    } while (0)
 
 __device__ __forceinline__ int32_t requant(int32_t acc, int32_t bias, int32_t scale, long long rnd,
                                            const Requant &rq) {
@@ -1301,52 +1329,50 @@ __global__ __launch_bounds__(256, NB <= 2 ? 4 : 2) void igemm_stream_i8(IgemmArg
 }
 
 template <int NB, int LOADER, bool ADD, int KS>
-static hipError_t launchIgemmStreamA(const IgemmArgs &a, size_t smem, hipStream_t stream) {
+static hipError_t launchIgemmStreamA(const IgemmArgs &a, size_t smem, const LaunchCtx &ctx) {
     auto kernel = igemm_stream_i8<NB, LOADER, ADD, KS>;
-    static bool configured = false;
-    if (!configured) {
-        hipError_t err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kStreamMaxLds);
-        if (err != hipSuccess) return err;
-        configured = true;
-    }
     // every block copies the weights into LDS once, then strides over the pixel groups:
     // one resident set of blocks, each with several groups where the image is large
     // blocks one CU holds: by registers (asked once per kernel, with no LDS in the way) and by LDS
+    static std::once_flag once;
+    static hipError_t configured = hipSuccess;
     static int byRegs = 0;
-    if (byRegs <= 0) {
+    std::call_once(once, [&] {
+        configured = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kStreamMaxLds);
         int n = 0;
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void *)kernel, 256, 0) != hipSuccess || n <= 0) {
             (void)hipGetLastError();
             n = NB <= 1 ? 7 : NB <= 2 ? 5 : NB <= 4 ? 4 : NB <= 6 ? 3 : 2;
         }
         byRegs = n;
-    }
+    });
+    if (configured != hipSuccess) return configured;
     const int perCu = (int)std::min<size_t>((size_t)std::min(byRegs, 8), (160 * 1024) / ((smem + 1023) / 1024 * 1024));
     const int groups = (a.M + 31) / 32;
     const int chunk = igemmStreamChunk(a.Np), chunks = (a.Np + chunk - 1) / chunk;
     const int blocks = std::min((groups + 3) / 4, std::max(1, 256 * perCu / chunks));
-    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)chunks), dim3(256), smem, stream, a);
+    THIP_ENQUEUE(ctx, kernelLabel("igemm_stream_i8", {NB, LOADER, ADD, KS}), kernel, dim3((unsigned)blocks, (unsigned)chunks), dim3(256), smem, a);
     return hipGetLastError();
 }
 
 template <int NB, int LOADER>
-static hipError_t launchIgemmStreamT(const IgemmArgs &a, size_t smem, hipStream_t stream) {
+static hipError_t launchIgemmStreamT(const IgemmArgs &a, size_t smem, const LaunchCtx &ctx) {
     if (a.skip != nullptr) {
         // the residual add comes with the accumulator widths 1, 2, 4, 6, 8 only (its caller rounds up)
         if constexpr (LOADER == kLoaderDense && (NB <= 2 || NB % 2 == 0)) {
-            return launchIgemmStreamA<NB, kLoaderDense, true, 0>(a, smem, stream);
+            return launchIgemmStreamA<NB, kLoaderDense, true, 0>(a, smem, ctx);
         } else {
             return hipErrorInvalidValue;
         }
     }
     // one or two k-steps per pixel group: the ring runs over several groups (THIP_NO_STREAM_DEEP: never)
-    if (LOADER == kLoaderDense && a.Kp <= 64 && !getenv("THIP_NO_STREAM_DEEP")) {
-        return a.Kp <= 32 ? launchIgemmStreamA<NB, kLoaderDense, false, 1>(a, smem, stream) : launchIgemmStreamA<NB, kLoaderDense, false, 2>(a, smem, stream);
+    if (LOADER == kLoaderDense && a.Kp <= 64 && !ctx.tuning->noStreamDeep) {
+        return a.Kp <= 32 ? launchIgemmStreamA<NB, kLoaderDense, false, 1>(a, smem, ctx) : launchIgemmStreamA<NB, kLoaderDense, false, 2>(a, smem, ctx);
     }
-    return launchIgemmStreamA<NB, LOADER, false, 0>(a, smem, stream);
+    return launchIgemmStreamA<NB, LOADER, false, 0>(a, smem, ctx);
 }
 
-static hipError_t launchIgemmStream(const IgemmArgs &a, hipStream_t stream) {
+static hipError_t launchIgemmStream(const IgemmArgs &a, const LaunchCtx &ctx) {
     if ((a.loader != kLoaderDense && a.loader != kLoaderRuns) || a.out_dtype != kDtypeI8) return hipErrorInvalidValue;
     if (a.N % 16 != 0 || ((uintptr_t)a.out & 15) != 0 || ((uintptr_t)a.skip & 15) != 0) return hipErrorInvalidValue;
     const int chunk = igemmStreamChunk(a.Np);
@@ -1355,38 +1381,38 @@ static hipError_t launchIgemmStream(const IgemmArgs &a, hipStream_t stream) {
     const int nb = chunk / 32;
     if (a.loader == kLoaderRuns) {
         // the first layer of an image network: few output channels
-        if (nb <= 1) return launchIgemmStreamT<1, kLoaderRuns>(a, smem, stream);
-        if (nb <= 2) return launchIgemmStreamT<2, kLoaderRuns>(a, smem, stream);
-        if (nb <= 4) return launchIgemmStreamT<4, kLoaderRuns>(a, smem, stream);
+        if (nb <= 1) return launchIgemmStreamT<1, kLoaderRuns>(a, smem, ctx);
+        if (nb <= 2) return launchIgemmStreamT<2, kLoaderRuns>(a, smem, ctx);
+        if (nb <= 4) return launchIgemmStreamT<4, kLoaderRuns>(a, smem, ctx);
         return hipErrorInvalidValue;
     }
     if (a.skip == nullptr) {
         // the branch-free steady state needs the block count at compile time (THIP_STREAM_GUARDED: the guarded loop only)
         IgemmArgs b = a;
-        b.stream_guarded = getenv("THIP_STREAM_GUARDED") != nullptr;
+        b.stream_guarded = ctx.tuning->streamGuarded;
         // staged stores where the slices fit beside the weights, the stores outweigh the loads and the output is far larger than
         // the caches (measured on a mobile network at batch 256: ahead from about 100 MB of output, behind at 40 MB);
         // THIP_STREAM_STAGE=0 / 1: never / wherever they fit
         const size_t staged = igemmStreamStageOffset(chunk, a.Kp, false) + igemmStreamStageBytes(chunk);
-        const char *stageEnv = getenv("THIP_STREAM_STAGE");
-        b.stream_stage = staged <= kStreamMaxLds && a.skip == nullptr && (stageEnv ? stageEnv[0] == '1' : a.N >= 2 * a.K && a.N >= 32 && (long long)a.M * a.N >= (64LL << 20)) && a.Kp <= 64;
+        const int stageMode = ctx.tuning->streamStage;
+        b.stream_stage = staged <= kStreamMaxLds && a.skip == nullptr && (stageMode >= 0 ? stageMode == 1 : a.N >= 2 * a.K && a.N >= 32 && (long long)a.M * a.N >= (64LL << 20)) && a.Kp <= 64;
         if (b.stream_stage) smem = staged;
         switch (nb) {
-        case 1: return launchIgemmStreamT<1, kLoaderDense>(b, smem, stream);
-        case 2: return launchIgemmStreamT<2, kLoaderDense>(b, smem, stream);
-        case 3: return launchIgemmStreamT<3, kLoaderDense>(b, smem, stream);
-        case 4: return launchIgemmStreamT<4, kLoaderDense>(b, smem, stream);
-        case 5: return launchIgemmStreamT<5, kLoaderDense>(b, smem, stream);
-        case 6: return launchIgemmStreamT<6, kLoaderDense>(b, smem, stream);
-        case 7: return launchIgemmStreamT<7, kLoaderDense>(b, smem, stream);
-        default: return launchIgemmStreamT<8, kLoaderDense>(b, smem, stream);
+        case 1: return launchIgemmStreamT<1, kLoaderDense>(b, smem, ctx);
+        case 2: return launchIgemmStreamT<2, kLoaderDense>(b, smem, ctx);
+        case 3: return launchIgemmStreamT<3, kLoaderDense>(b, smem, ctx);
+        case 4: return launchIgemmStreamT<4, kLoaderDense>(b, smem, ctx);
+        case 5: return launchIgemmStreamT<5, kLoaderDense>(b, smem, ctx);
+        case 6: return launchIgemmStreamT<6, kLoaderDense>(b, smem, ctx);
+        case 7: return launchIgemmStreamT<7, kLoaderDense>(b, smem, ctx);
+        default: return launchIgemmStreamT<8, kLoaderDense>(b, smem, ctx);
         }
     }
-    if (nb <= 1) return launchIgemmStreamT<1, kLoaderDense>(a, smem, stream);
-    if (nb <= 2) return launchIgemmStreamT<2, kLoaderDense>(a, smem, stream);
-    if (nb <= 4) return launchIgemmStreamT<4, kLoaderDense>(a, smem, stream);
-    if (nb <= 6) return launchIgemmStreamT<6, kLoaderDense>(a, smem, stream);
-    return launchIgemmStreamT<8, kLoaderDense>(a, smem, stream);
+    if (nb <= 1) return launchIgemmStreamT<1, kLoaderDense>(a, smem, ctx);
+    if (nb <= 2) return launchIgemmStreamT<2, kLoaderDense>(a, smem, ctx);
+    if (nb <= 4) return launchIgemmStreamT<4, kLoaderDense>(a, smem, ctx);
+    if (nb <= 6) return launchIgemmStreamT<6, kLoaderDense>(a, smem, ctx);
+    return launchIgemmStreamT<8, kLoaderDense>(a, smem, ctx);
 }
 
 static const IgemmTile kTiles[kIgemmVariantCount] = {
@@ -1411,85 +1437,81 @@ const IgemmTile &igemmTile(uint32_t variant) {
 }
 
 template <int BM, int BN, int BK, int LOADER, int G>
-static hipError_t launchIgemmTile(const IgemmArgs &a, hipStream_t stream) {
+static hipError_t launchIgemmTile(const IgemmArgs &a, const LaunchCtx &ctx) {
     constexpr int LDK = BK + 16;
     constexpr size_t tiles = (size_t)2 * (BM + BN) * LDK;
     constexpr size_t epilogue = igemmEpilogueLds<BM / 2, 4, BN>();
     constexpr size_t smem = tiles > epilogue ? tiles : epilogue;
     auto kernel = igemm_i8<BM, BN, BK, LOADER, G>;
-    // once per kernel: later launches may sit inside a stream capture, where only stream work belongs
-    static bool configured = false;
-    if (!configured) {
-        hipError_t err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (err != hipSuccess) return err;
-        configured = true;
-    }
+    // once per kernel, when an executable that uses it is created: launches may sit inside a stream capture, where only stream work belongs
+    static std::once_flag once;
+    static hipError_t configured = hipSuccess;
+    std::call_once(once, [&] { configured = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); });
+    if (configured != hipSuccess) return configured;
     const int tilesM = (a.M + BM - 1) / BM;
     const int tilesN = a.Np / BN;
     const dim3 grid((unsigned)(tilesM * tilesN));
-    hipLaunchKernelGGL(kernel, grid, dim3(256), smem, stream, a);
+    THIP_ENQUEUE(ctx, kernelLabel("igemm_i8", {BM, BN, BK, LOADER, G}), kernel, grid, dim3(256), smem, a);
     return hipGetLastError();
 }
 
 template <int BM, int BN, int BK>
-static hipError_t launchIgemmLoader(const IgemmArgs &a, hipStream_t stream) {
+static hipError_t launchIgemmLoader(const IgemmArgs &a, const LaunchCtx &ctx) {
     if (a.loader == kLoaderDense) {
-        return launchIgemmTile<BM, BN, BK, kLoaderDense, 16>(a, stream);
+        return launchIgemmTile<BM, BN, BK, kLoaderDense, 16>(a, ctx);
     }
     if (a.loader == kLoaderRuns) {
-        return launchIgemmTile<BM, BN, BK, kLoaderRuns, 16>(a, stream);
+        return launchIgemmTile<BM, BN, BK, kLoaderRuns, 16>(a, ctx);
     }
     switch (a.gran) {
-    case 16: return launchIgemmTile<BM, BN, BK, kLoaderGather, 16>(a, stream);
-    case 8: return launchIgemmTile<BM, BN, BK, kLoaderGather, 8>(a, stream);
-    case 4: return launchIgemmTile<BM, BN, BK, kLoaderGather, 4>(a, stream);
-    case 2: return launchIgemmTile<BM, BN, BK, kLoaderGather, 2>(a, stream);
-    case 1: return launchIgemmTile<BM, BN, BK, kLoaderGather, 1>(a, stream);
+    case 16: return launchIgemmTile<BM, BN, BK, kLoaderGather, 16>(a, ctx);
+    case 8: return launchIgemmTile<BM, BN, BK, kLoaderGather, 8>(a, ctx);
+    case 4: return launchIgemmTile<BM, BN, BK, kLoaderGather, 4>(a, ctx);
+    case 2: return launchIgemmTile<BM, BN, BK, kLoaderGather, 2>(a, ctx);
+    case 1: return launchIgemmTile<BM, BN, BK, kLoaderGather, 1>(a, ctx);
     default: return hipErrorInvalidValue;
     }
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, bool DIRECT, bool ADD = false>
-static hipError_t launchIgemmDenseE(const IgemmArgs &a, hipStream_t stream) {
+static hipError_t launchIgemmDenseE(const IgemmArgs &a, const LaunchCtx &ctx) {
     // the stage ring, reused by the epilogue as staging slices (one per wave) plus bias/scale
     constexpr size_t ring = (size_t)STAGES * (BM + BN) * 64;
     constexpr size_t epilogue = (size_t)(BM / WAVES_M) * (WAVES_M * WAVES_N) * (32 * 4 + 16) + 2 * BN * 4;
     constexpr size_t smem = ring > epilogue ? ring : epilogue;
     static_assert(smem * BLOCKS_PER_CU <= 160 * 1024, "LDS of one CU");
     auto kernel = igemm_dense_i8<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, DIRECT, ADD>;
-    static bool configured = false;
-    if (!configured) {
-        hipError_t err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-        if (err != hipSuccess) return err;
-        configured = true;
-    }
+    static std::once_flag once;
+    static hipError_t configured = hipSuccess;
+    std::call_once(once, [&] { configured = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); });
+    if (configured != hipSuccess) return configured;
     const int tilesM = (a.M + BM - 1) / BM;
     const int tilesN = a.Np / BN;
-    hipLaunchKernelGGL(kernel, dim3((unsigned)(tilesM * tilesN)), dim3(WAVES_M * WAVES_N * 64), smem, stream, a);
+    THIP_ENQUEUE(ctx, kernelLabel("igemm_dense_i8", {BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, DIRECT, ADD}), kernel, dim3((unsigned)(tilesM * tilesN)), dim3(WAVES_M * WAVES_N * 64), smem, a);
     return hipGetLastError();
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU>
-static hipError_t launchIgemmDense(const IgemmArgs &a, hipStream_t stream) {
+static hipError_t launchIgemmDense(const IgemmArgs &a, const LaunchCtx &ctx) {
     // the in-register epilogue takes the plain 32-bit tail only (what wideRequant() calls plain)
     const bool plain = a.rq.shift >= 33 && a.rq.shift <= 45 && a.rq.pre_shift == 0 && a.rq.t0_clamp == 0 &&
                        a.rq.out_zp >= -32768 && a.rq.out_zp <= 32767 && a.rq.out_min <= a.rq.out_max;
     const bool direct = a.out_dtype == kDtypeI8 && a.N % 16 == 0 && ((uintptr_t)a.out & 15) == 0 && plain &&
-                        !getenv("THIP_NO_DIRECT_EPILOGUE");
+                        !ctx.tuning->noDirectEpilogue;
     if (a.skip != nullptr) {
         // a residual add: the in-register epilogue of the small tile only (what a network's late, small layers take)
         if constexpr (BM == 64 && BN == 64) {
             if (!direct || ((uintptr_t)a.skip & 15) != 0) return hipErrorInvalidValue;
-            return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, true, true>(a, stream);
+            return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, true, true>(a, ctx);
         } else {
             return hipErrorInvalidValue;
         }
     }
-    return direct ? launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, true>(a, stream)
-                  : launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, false>(a, stream);
+    return direct ? launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, true>(a, ctx)
+                  : launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, false>(a, ctx);
 }
 
-hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, hipStream_t stream) {
+hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, const LaunchCtx &ctx) {
     if (variant >= kIgemmVariantCount) return hipErrorInvalidValue;
     const IgemmTile &t = kTiles[variant];
     // What the kernel assumes: padded sizes are whole tiles, the real sizes fit
@@ -1517,20 +1539,20 @@ hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, hipStream_t stream)
     if (a.out_dtype < kDtypeI8 || a.out_dtype > kDtypeI32) return hipErrorInvalidValue;
     if (a.skip != nullptr && variant != kIgemmStream && variant != kIgemmDense64x64) return hipErrorInvalidValue;  // the kernels that can add a residual
     switch (variant) {
-    case kIgemm128x128x64: return launchIgemmLoader<128, 128, 64>(a, stream);
-    case kIgemm256x256x64: return launchIgemmLoader<256, 256, 64>(a, stream);
-    case kIgemm64x64x64: return launchIgemmLoader<64, 64, 64>(a, stream);
-    case kIgemm256x128x64: return launchIgemmLoader<256, 128, 64>(a, stream);
-    case kIgemmDense256x256: return launchIgemmDense<256, 256, 2, 2, 4, 1>(a, stream);
-    case kIgemmDense128x128: return launchIgemmDense<128, 128, 2, 2, 4, 2>(a, stream);
-    case kIgemmDense128x256: return launchIgemmDense<128, 256, 2, 2, 3, 2>(a, stream);
-    case kIgemmDense64x64: return launchIgemmDense<64, 64, 2, 2, 4, 4>(a, stream);
-    case kIgemmDense256x128: return launchIgemmDense<256, 128, 2, 2, 3, 2>(a, stream);
-    case kIgemmDense256x64: return launchIgemmDense<256, 64, 4, 1, 3, 2>(a, stream);
-    case kIgemmDense256x32: return launchIgemmDense<256, 32, 4, 1, 3, 2>(a, stream);
-    case kIgemmStream: return launchIgemmStream(a, stream);
-    case kIgemmDense128x64: return launchIgemmDense<128, 64, 2, 2, 4, 2>(a, stream);
-    case kIgemmDense64x128: return launchIgemmDense<64, 128, 2, 2, 4, 2>(a, stream);
+    case kIgemm128x128x64: return launchIgemmLoader<128, 128, 64>(a, ctx);
+    case kIgemm256x256x64: return launchIgemmLoader<256, 256, 64>(a, ctx);
+    case kIgemm64x64x64: return launchIgemmLoader<64, 64, 64>(a, ctx);
+    case kIgemm256x128x64: return launchIgemmLoader<256, 128, 64>(a, ctx);
+    case kIgemmDense256x256: return launchIgemmDense<256, 256, 2, 2, 4, 1>(a, ctx);
+    case kIgemmDense128x128: return launchIgemmDense<128, 128, 2, 2, 4, 2>(a, ctx);
+    case kIgemmDense128x256: return launchIgemmDense<128, 256, 2, 2, 3, 2>(a, ctx);
+    case kIgemmDense64x64: return launchIgemmDense<64, 64, 2, 2, 4, 4>(a, ctx);
+    case kIgemmDense256x128: return launchIgemmDense<256, 128, 2, 2, 3, 2>(a, ctx);
+    case kIgemmDense256x64: return launchIgemmDense<256, 64, 4, 1, 3, 2>(a, ctx);
+    case kIgemmDense256x32: return launchIgemmDense<256, 32, 4, 1, 3, 2>(a, ctx);
+    case kIgemmStream: return launchIgemmStream(a, ctx);
+    case kIgemmDense128x64: return launchIgemmDense<128, 64, 2, 2, 4, 2>(a, ctx);
+    case kIgemmDense64x128: return launchIgemmDense<64, 128, 2, 2, 4, 2>(a, ctx);
     default: return hipErrorInvalidValue;
     }
 }
@@ -1667,28 +1689,28 @@ __global__ __launch_bounds__(256) void fc_skinny_mfma(FcSkinnyArgs p) {
 }
 
 template <int MR, int NW>
-static hipError_t launchFcSkinnyT(const FcSkinnyArgs &a, hipStream_t stream) {
+static hipError_t launchFcSkinnyT(const FcSkinnyArgs &a, const LaunchCtx &ctx) {
     const int waves = (a.N + NW - 1) / NW;
     const dim3 grid((unsigned)((waves + 3) / 4));
-    hipLaunchKernelGGL((fc_skinny<MR, NW>), grid, dim3(256), 0, stream, a);
+    THIP_ENQUEUE(ctx, kernelLabel("fc_skinny", {MR, NW}), (fc_skinny<MR, NW>), grid, dim3(256), 0, a);
     return hipGetLastError();
 }
 
-hipError_t launchFcSkinny(const FcSkinnyArgs &a, hipStream_t stream) {
+hipError_t launchFcSkinny(const FcSkinnyArgs &a, const LaunchCtx &ctx) {
     if (a.M <= 0 || a.M > kFcSkinnyMaxRows || a.N <= 0 || a.K <= 0 || a.K % 16 != 0) {
         return hipErrorInvalidValue;
     }
     if (!a.x || !a.w || !a.bias || !a.scale || !a.out) return hipErrorInvalidValue;
     if ((((uintptr_t)a.x) | ((uintptr_t)a.w)) & 15) return hipErrorInvalidValue;
     if (a.out_dtype < kDtypeI8 || a.out_dtype > kDtypeI32) return hipErrorInvalidValue;
-    if (a.M == 1) return launchFcSkinnyT<1, 4>(a, stream);
-    if (a.M >= 3 && ((uintptr_t)a.out & 3) == 0 && !getenv("THIP_SKINNY_DOT4")) {
-        hipLaunchKernelGGL(fc_skinny_mfma, dim3((unsigned)((a.N + 15) / 16)), dim3(256), 0, stream, a);
+    if (a.M == 1) return launchFcSkinnyT<1, 4>(a, ctx);
+    if (a.M >= 3 && ((uintptr_t)a.out & 3) == 0 && !ctx.tuning->skinnyDot4) {
+        THIP_ENQUEUE(ctx, "fc_skinny_mfma", fc_skinny_mfma, dim3((unsigned)((a.N + 15) / 16)), dim3(256), 0, a);
         return hipGetLastError();
     }
-    if (a.M <= 4) return launchFcSkinnyT<4, 4>(a, stream);
-    if (a.M <= 8) return launchFcSkinnyT<8, 2>(a, stream);
-    return launchFcSkinnyT<16, 2>(a, stream);
+    if (a.M <= 4) return launchFcSkinnyT<4, 4>(a, ctx);
+    if (a.M <= 8) return launchFcSkinnyT<8, 2>(a, ctx);
+    return launchFcSkinnyT<16, 2>(a, ctx);
 }
 
 // ---------------------------------------------------------------------------
@@ -1861,10 +1883,10 @@ __global__ __launch_bounds__(256) void depthwise3x3_dot4_i8(DepthwiseArgs p, Wor
 }
 
 template <int P, int SWT>
-static hipError_t launchDepthwiseDot4(const DepthwiseArgs &a, hipStream_t stream) {
+static hipError_t launchDepthwiseDot4(const DepthwiseArgs &a, const LaunchCtx &ctx) {
     const long long total = (long long)a.N * a.OH * ((a.OW + P - 1) / P) * (a.C / 16);
     const WorkSplit ws = makeWorkSplit(total, a.C / 16, (a.OW + P - 1) / P, a.OH);
-    hipLaunchKernelGGL((depthwise3x3_dot4_i8<P, SWT>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a, ws);
+    THIP_ENQUEUE(ctx, kernelLabel("depthwise3x3_dot4_i8", {P, SWT}), (depthwise3x3_dot4_i8<P, SWT>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, a, ws);
     return hipGetLastError();
 }
 
@@ -2025,10 +2047,10 @@ __global__ __launch_bounds__(256) void depthwise3x3_tile_i8(DepthwiseArgs p, Wor
 }
 
 template <int P, int R, int S, int G>
-static hipError_t launchDepthwiseTile(const DepthwiseArgs &a, hipStream_t stream) {
+static hipError_t launchDepthwiseTile(const DepthwiseArgs &a, const LaunchCtx &ctx) {
     const long long total = (long long)a.N * ((a.OH + R - 1) / R) * ((a.OW + P - 1) / P) * (a.C / (4 * G));
     const WorkSplit ws = makeWorkSplit(total, a.C / (4 * G), (a.OW + P - 1) / P, (a.OH + R - 1) / R);
-    hipLaunchKernelGGL((depthwise3x3_tile_i8<P, R, S, G>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a, ws);
+    THIP_ENQUEUE(ctx, kernelLabel("depthwise3x3_tile_i8", {P, R, S, G}), (depthwise3x3_tile_i8<P, R, S, G>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, a, ws);
     return hipGetLastError();
 }
 
@@ -2224,11 +2246,11 @@ static int depthwiseStripSegment(const DepthwiseArgs &a, int P, int G, long long
 }
 
 template <int P, int S, int G, int OCC, int D>
-static hipError_t launchDepthwiseStrip(const DepthwiseArgs &a, int seg, hipStream_t stream) {
+static hipError_t launchDepthwiseStrip(const DepthwiseArgs &a, int seg, const LaunchCtx &ctx) {
     const int nseg = (a.OH + seg - 1) / seg, xs = (a.OW + P - 1) / P;
     const long long total = (long long)a.N * nseg * xs * (a.C / (4 * G));
     const WorkSplit ws = makeWorkSplit(total, a.C / (4 * G), xs, nseg);
-    hipLaunchKernelGGL((depthwise3x3_strip_i8<P, S, G, OCC, D>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a, ws, seg);
+    THIP_ENQUEUE(ctx, kernelLabel("depthwise3x3_strip_i8", {P, S, G, OCC, D}), (depthwise3x3_strip_i8<P, S, G, OCC, D>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, a, ws, seg);
     return hipGetLastError();
 }
 
@@ -2248,19 +2270,19 @@ static bool poolGeometryOk(int N, int H, int W, int C, int OH, int OW, int KH, i
 }
 
 template <int VEC>
-static hipError_t launchDepthwiseV(const DepthwiseArgs &a, hipStream_t stream) {
+static hipError_t launchDepthwiseV(const DepthwiseArgs &a, const LaunchCtx &ctx) {
     const long long total = (long long)a.N * a.OH * a.OW * (a.C / VEC);
     const dim3 grid((unsigned)((total + 255) / 256));
     const WorkSplit ws = makeWorkSplit(total, a.C / VEC, a.OW, a.OH);
     if (a.KH == 3 && a.KW == 3) {
-        hipLaunchKernelGGL((depthwise_i8<VEC, 3>), grid, dim3(256), 0, stream, a, ws);
+        THIP_ENQUEUE(ctx, kernelLabel("depthwise_i8", {VEC, 3}), (depthwise_i8<VEC, 3>), grid, dim3(256), 0, a, ws);
     } else {
-        hipLaunchKernelGGL((depthwise_i8<VEC, 0>), grid, dim3(256), 0, stream, a, ws);
+        THIP_ENQUEUE(ctx, kernelLabel("depthwise_i8", {VEC, 0}), (depthwise_i8<VEC, 0>), grid, dim3(256), 0, a, ws);
     }
     return hipGetLastError();
 }
 
-hipError_t launchDepthwise(const DepthwiseArgs &a, hipStream_t stream) {
+hipError_t launchDepthwise(const DepthwiseArgs &a, const LaunchCtx &ctx) {
     if (!poolGeometryOk(a.N, a.H, a.W, a.C, a.OH, a.OW, a.KH, a.KW, a.SH, a.SW, a.PT, a.PL)) {
         return hipErrorInvalidValue;
     }
@@ -2276,44 +2298,42 @@ hipError_t launchDepthwise(const DepthwiseArgs &a, hipStream_t stream) {
         // the rolling-window kernel where it has at least a wave (stride 1) or 1.9 waves (stride 2) per SIMD
         // (THIP_DEPTHWISE_STRIP=0 / 1 / 2 switches it off / on / on with one column per thread at stride 2, for every
         // size, for tests and tuning)
-        const char *stripEnv = getenv("THIP_DEPTHWISE_STRIP");
-        const bool stripOff = stripEnv && stripEnv[0] == '0', stripOn = stripEnv && (stripEnv[0] == '1' || stripEnv[0] == '2');
-        const bool stripOne = stripEnv && stripEnv[0] == '2';
+        const int stripMode = ctx.tuning->depthwiseStrip;
+        const bool stripOff = stripMode == 0, stripOn = stripMode == 1 || stripMode == 2;
+        const bool stripOne = stripMode == 2;
         if (!stripOff && a.SH == a.SW && (a.SW == 1 || a.SW == 2) && (long long)a.W * a.C < (1LL << 24)) {
             long long waves = 0;
             const int seg = depthwiseStripSegment(a, 2, 1, &waves);
-            if (a.SW == 1 && (stripOn || (a.OH >= 12 && waves >= 1024))) return launchDepthwiseStrip<2, 1, 1, 4, 3>(a, seg, stream);
+            if (a.SW == 1 && (stripOn || (a.OH >= 12 && waves >= 1024))) return launchDepthwiseStrip<2, 1, 1, 4, 3>(a, seg, ctx);
             if (a.SW == 2 && (stripOne || (!stripOn && a.OH >= 12))) {
                 // with plenty of work, one column per thread, more waves and the deeper prefetch measured 7-10 % ahead
                 long long waves1 = 0;
                 const int seg1 = depthwiseStripSegment(a, 1, 1, &waves1);
-                if (stripOne || waves1 >= 7 * 1024) return launchDepthwiseStrip<1, 2, 1, 4, 3>(a, seg1, stream);
+                if (stripOne || waves1 >= 7 * 1024) return launchDepthwiseStrip<1, 2, 1, 4, 3>(a, seg1, ctx);
             }
-            if (a.SW == 2 && (stripOn || (a.OH >= 12 && 10 * waves >= 19 * 1024))) return launchDepthwiseStrip<2, 2, 1, 3, 1>(a, seg, stream);
+            if (a.SW == 2 && (stripOn || (a.OH >= 12 && 10 * waves >= 19 * 1024))) return launchDepthwiseStrip<2, 2, 1, 3, 1>(a, seg, ctx);
         }
-        const char *tileEnv = getenv("THIP_DEPTHWISE_TILE");
-        const bool tileOff = tileEnv && tileEnv[0] == '0', tileOn = tileEnv && tileEnv[0] == '1';
+        const bool tileOff = ctx.tuning->depthwiseTile == 0, tileOn = ctx.tuning->depthwiseTile == 1;
         if (!tileOff) {
             // 16 channels per thread: 8 or 4 (more waves, fewer registers) measured 5 % and 12 % slower
-            const char *thr = getenv("THIP_DEPTHWISE_TILE_MIN");
-            const long long tileMin = thr ? atoll(thr) : 8 * 65536;  // measured on a mobile network at batch 32 and 256: even or ahead from about half a million thread-outputs
-            if (a.SW == 1 && a.SH == 1 && (tileOn || outputs >= tileMin)) return launchDepthwiseTile<4, 2, 1, 4>(a, stream);
+            const long long tileMin = ctx.tuning->depthwiseTileMin > 0 ? ctx.tuning->depthwiseTileMin : 8 * 65536;  // measured on a mobile network at batch 32 and 256: even or ahead from about half a million thread-outputs
+            if (a.SW == 1 && a.SH == 1 && (tileOn || outputs >= tileMin)) return launchDepthwiseTile<4, 2, 1, 4>(a, ctx);
         }
         // pixels per thread (THIP_DEPTHWISE_P forces 1, 2 or 4, for tuning)
         int pix = outputs >= 4 * 65536 ? 4 : outputs >= 2 * 65536 ? 2 : 1;
-        if (const char *env = getenv("THIP_DEPTHWISE_P")) pix = atoi(env);
-        if (a.SW == 1 && pix == 4) return launchDepthwiseDot4<4, 1>(a, stream);
-        if (a.SW == 2 && pix == 4) return launchDepthwiseDot4<4, 2>(a, stream);
-        if (a.SW == 1 && pix == 2) return launchDepthwiseDot4<2, 1>(a, stream);
-        if (a.SW == 2 && pix == 2) return launchDepthwiseDot4<2, 2>(a, stream);
-        return launchDepthwiseDot4<1, 0>(a, stream);
+        if (ctx.tuning->depthwisePixels > 0) pix = ctx.tuning->depthwisePixels;
+        if (a.SW == 1 && pix == 4) return launchDepthwiseDot4<4, 1>(a, ctx);
+        if (a.SW == 2 && pix == 4) return launchDepthwiseDot4<4, 2>(a, ctx);
+        if (a.SW == 1 && pix == 2) return launchDepthwiseDot4<2, 1>(a, ctx);
+        if (a.SW == 2 && pix == 2) return launchDepthwiseDot4<2, 2>(a, ctx);
+        return launchDepthwiseDot4<1, 0>(a, ctx);
     }
     if (a.variant != kDepthwiseGeneric) return hipErrorInvalidValue;
     switch (pickVec(a.C, a.in, a.out, a.wpk)) {
-    case 16: return launchDepthwiseV<16>(a, stream);
-    case 8: return launchDepthwiseV<8>(a, stream);
-    case 4: return launchDepthwiseV<4>(a, stream);
-    default: return launchDepthwiseV<1>(a, stream);
+    case 16: return launchDepthwiseV<16>(a, ctx);
+    case 8: return launchDepthwiseV<8>(a, ctx);
+    case 4: return launchDepthwiseV<4>(a, ctx);
+    default: return launchDepthwiseV<1>(a, ctx);
     }
 }
 
@@ -2359,25 +2379,25 @@ __global__ __launch_bounds__(256) void maxpool_i8(MaxPoolArgs p, WorkSplit ws) {
 }
 
 template <int VEC>
-static hipError_t launchMaxPoolV(const MaxPoolArgs &a, hipStream_t stream) {
+static hipError_t launchMaxPoolV(const MaxPoolArgs &a, const LaunchCtx &ctx) {
     const long long total = (long long)a.N * a.OH * a.OW * (a.C / VEC);
     const dim3 grid((unsigned)((total + 255) / 256));
     const WorkSplit ws = makeWorkSplit(total, a.C / VEC, a.OW, a.OH);
-    hipLaunchKernelGGL((maxpool_i8<VEC>), grid, dim3(256), 0, stream, a, ws);
+    THIP_ENQUEUE(ctx, kernelLabel("maxpool_i8", {VEC}), (maxpool_i8<VEC>), grid, dim3(256), 0, a, ws);
     return hipGetLastError();
 }
 
-hipError_t launchMaxPool(const MaxPoolArgs &a, hipStream_t stream) {
+hipError_t launchMaxPool(const MaxPoolArgs &a, const LaunchCtx &ctx) {
     if (!poolGeometryOk(a.N, a.H, a.W, a.C, a.OH, a.OW, a.KH, a.KW, a.SH, a.SW, a.PT, a.PL)) {
         return hipErrorInvalidValue;
     }
     if (!a.in || !a.out) return hipErrorInvalidValue;
     if ((long long)a.N * a.OH * a.OW * a.C >= (1LL << 40)) return hipErrorInvalidValue;
     switch (pickVec(a.C, a.in, a.out, nullptr)) {
-    case 16: return launchMaxPoolV<16>(a, stream);
-    case 8: return launchMaxPoolV<8>(a, stream);
-    case 4: return launchMaxPoolV<4>(a, stream);
-    default: return launchMaxPoolV<1>(a, stream);
+    case 16: return launchMaxPoolV<16>(a, ctx);
+    case 8: return launchMaxPoolV<8>(a, ctx);
+    case 4: return launchMaxPoolV<4>(a, ctx);
+    default: return launchMaxPoolV<1>(a, ctx);
     }
 }
 
@@ -2426,22 +2446,22 @@ __global__ __launch_bounds__(256) void avgpool_i8(AvgPoolArgs p) {
 }
 
 template <int VEC>
-static hipError_t launchAvgPoolV(const AvgPoolArgs &a, hipStream_t stream) {
+static hipError_t launchAvgPoolV(const AvgPoolArgs &a, const LaunchCtx &ctx) {
     constexpr int CC = 4;
     const int cgroups = a.C / VEC;
     const long long waves = (long long)a.N * ((cgroups + CC - 1) / CC);
     const dim3 grid((unsigned)((waves + 3) / 4));
-    hipLaunchKernelGGL((avgpool_i8<VEC, CC>), grid, dim3(256), 0, stream, a);
+    THIP_ENQUEUE(ctx, kernelLabel("avgpool_i8", {VEC, CC}), (avgpool_i8<VEC, CC>), grid, dim3(256), 0, a);
     return hipGetLastError();
 }
 
-hipError_t launchAvgPool(const AvgPoolArgs &a, hipStream_t stream) {
+hipError_t launchAvgPool(const AvgPoolArgs &a, const LaunchCtx &ctx) {
     if (a.N <= 0 || a.HW <= 0 || a.C <= 0 || !a.in || !a.out) return hipErrorInvalidValue;
     switch (pickVec(a.C, a.in, a.out, nullptr)) {
-    case 16: return launchAvgPoolV<16>(a, stream);
-    case 8: return launchAvgPoolV<8>(a, stream);
-    case 4: return launchAvgPoolV<4>(a, stream);
-    default: return launchAvgPoolV<1>(a, stream);
+    case 16: return launchAvgPoolV<16>(a, ctx);
+    case 8: return launchAvgPoolV<8>(a, ctx);
+    case 4: return launchAvgPoolV<4>(a, ctx);
+    default: return launchAvgPoolV<1>(a, ctx);
     }
 }
 
@@ -2469,14 +2489,14 @@ __global__ __launch_bounds__(256) void add_i8(AddArgs p) {
     }
 }
 
-hipError_t launchAdd(const AddArgs &a, hipStream_t stream) {
+hipError_t launchAdd(const AddArgs &a, const LaunchCtx &ctx) {
     if (a.count <= 0 || !a.in0 || !a.in1 || !a.out) return hipErrorInvalidValue;
     const uintptr_t bits = (uintptr_t)a.in0 | (uintptr_t)a.in1 | (uintptr_t)a.out;
     if ((bits & 15) == 0) {
         const long long threads = (a.count + 15) / 16;
-        hipLaunchKernelGGL((add_i8<16>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, a);
+        THIP_ENQUEUE(ctx, "add_i8<16>", (add_i8<16>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, a);
     } else {
-        hipLaunchKernelGGL((add_i8<1>), dim3((unsigned)((a.count + 255) / 256)), dim3(256), 0, stream, a);
+        THIP_ENQUEUE(ctx, "add_i8<1>", (add_i8<1>), dim3((unsigned)((a.count + 255) / 256)), dim3(256), 0, a);
     }
     return hipGetLastError();
 }
@@ -2500,12 +2520,12 @@ __global__ __launch_bounds__(256) void im2col_bf16(Im2colBf16Args p, long long t
     p.out[t] = v;
 }
 
-hipError_t launchIm2colBf16(const Im2colBf16Args &a, hipStream_t stream) {
+hipError_t launchIm2colBf16(const Im2colBf16Args &a, const LaunchCtx &ctx) {
     if (!a.in || !a.out || !poolGeometryOk(a.N, a.H, a.W, a.C, a.OH, a.OW, a.KH, a.KW, a.SH, a.SW, a.PT, a.PL)) return hipErrorInvalidValue;
     if (a.Kp < a.KH * a.KW * a.C) return hipErrorInvalidValue;
     const long long total = (long long)a.N * a.OH * a.OW * a.Kp;
     if (total >= (1LL << 39)) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(im2col_bf16, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a, total);
+    THIP_ENQUEUE(ctx, "im2col_bf16", im2col_bf16, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, a, total);
     return hipGetLastError();
 }
 
@@ -2535,12 +2555,12 @@ __global__ __launch_bounds__(256) void depthwise_bf16(DepthwiseBf16Args p, long 
     p.out[t] = bf16Bits(t0 < p.lo ? p.lo : (t0 > p.hi ? p.hi : t0));
 }
 
-hipError_t launchDepthwiseBf16(const DepthwiseBf16Args &a, hipStream_t stream) {
+hipError_t launchDepthwiseBf16(const DepthwiseBf16Args &a, const LaunchCtx &ctx) {
     if (!a.in || !a.wpk || !a.bias || !a.out) return hipErrorInvalidValue;
     if (!poolGeometryOk(a.N, a.H, a.W, a.C, a.OH, a.OW, a.KH, a.KW, a.SH, a.SW, a.PT, a.PL)) return hipErrorInvalidValue;
     const long long total = (long long)a.N * a.OH * a.OW * a.C;
     if (total >= (1LL << 39)) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(depthwise_bf16, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, a, total);
+    THIP_ENQUEUE(ctx, "depthwise_bf16", depthwise_bf16, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, a, total);
     return hipGetLastError();
 }
 
@@ -2576,16 +2596,16 @@ __global__ __launch_bounds__(256) void add_bf16(AddBf16Args p) {
     }
 }
 
-hipError_t launchAddBf16(const AddBf16Args &a, hipStream_t stream) {
+hipError_t launchAddBf16(const AddBf16Args &a, const LaunchCtx &ctx) {
     if (!a.in0 || !a.in1 || !a.out || a.count <= 0) return hipErrorInvalidValue;
     const bool vec = a.count % 8 == 0 && ((((uintptr_t)a.in0) | ((uintptr_t)a.in1) | ((uintptr_t)a.out)) & 15) == 0;
     const int64_t threads = vec ? a.count / 8 : a.count;
     if (threads >= (1LL << 39)) return hipErrorInvalidValue;
     const dim3 grid((unsigned)((threads + 255) / 256));
     if (vec) {
-        hipLaunchKernelGGL(add_bf16<8>, grid, dim3(256), 0, stream, a);
+        THIP_ENQUEUE(ctx, "add_bf16<8>", add_bf16<8>, grid, dim3(256), 0, a);
     } else {
-        hipLaunchKernelGGL(add_bf16<1>, grid, dim3(256), 0, stream, a);
+        THIP_ENQUEUE(ctx, "add_bf16<1>", add_bf16<1>, grid, dim3(256), 0, a);
     }
     return hipGetLastError();
 }
@@ -2660,20 +2680,20 @@ __global__ __launch_bounds__(256) void eltwise_int(EltwiseArgs p) {
 }
 
 template <typename TIN, typename TOUT>
-static hipError_t launchEltwiseT(const EltwiseArgs &a, hipStream_t stream) {
+static hipError_t launchEltwiseT(const EltwiseArgs &a, const LaunchCtx &ctx) {
     constexpr int VEC = sizeof(TIN) == 1 && sizeof(TOUT) == 1 ? 16 : 8;
     const uintptr_t bits = (uintptr_t)a.in0 | ((a.op == kEltMul || a.op >= kEltAnd) ? (uintptr_t)a.in1 : 0);
     const bool aligned = (bits & (sizeof(TIN) * VEC - 1)) == 0 && (((uintptr_t)a.out) & (sizeof(TOUT) * VEC - 1)) == 0;
     if (aligned) {
         const long long threads = (a.count + VEC - 1) / VEC;
-        hipLaunchKernelGGL((eltwise_int<TIN, TOUT, VEC>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, a);
+        THIP_ENQUEUE(ctx, kernelLabel("eltwise_int", {(int)sizeof(TIN), (int)sizeof(TOUT), VEC}), (eltwise_int<TIN, TOUT, VEC>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, a);
     } else {
-        hipLaunchKernelGGL((eltwise_int<TIN, TOUT, 1>), dim3((unsigned)((a.count + 255) / 256)), dim3(256), 0, stream, a);
+        THIP_ENQUEUE(ctx, kernelLabel("eltwise_int", {(int)sizeof(TIN), (int)sizeof(TOUT), 1}), (eltwise_int<TIN, TOUT, 1>), dim3((unsigned)((a.count + 255) / 256)), dim3(256), 0, a);
     }
     return hipGetLastError();
 }
 
-hipError_t launchEltwise(const EltwiseArgs &a, hipStream_t stream) {
+hipError_t launchEltwise(const EltwiseArgs &a, const LaunchCtx &ctx) {
     if (!a.in0 || !a.out || a.count <= 0 || a.count >= (1LL << 39) || a.op < kEltFma || a.op > kEltMax) return hipErrorInvalidValue;
     const bool two = a.op == kEltMul || a.op >= kEltAnd;
     if (two && (!a.in1 || a.bcast < 0 || a.bcast > 2)) return hipErrorInvalidValue;
@@ -2682,20 +2702,21 @@ hipError_t launchEltwise(const EltwiseArgs &a, hipStream_t stream) {
     if ((((uintptr_t)a.in0) & (a.in_bytes - 1)) || (((uintptr_t)a.out) & (a.out_bytes - 1))) return hipErrorInvalidValue;
     if (two && (((uintptr_t)a.in1) & (a.in_bytes - 1))) return hipErrorInvalidValue;
     switch (a.in_bytes * 8 + a.out_bytes) {
-    case 1 * 8 + 1: return launchEltwiseT<int8_t, int8_t>(a, stream);
-    case 1 * 8 + 2: return launchEltwiseT<int8_t, int16_t>(a, stream);
-    case 1 * 8 + 4: return launchEltwiseT<int8_t, int32_t>(a, stream);
-    case 2 * 8 + 1: return launchEltwiseT<int16_t, int8_t>(a, stream);
-    case 2 * 8 + 2: return launchEltwiseT<int16_t, int16_t>(a, stream);
-    case 2 * 8 + 4: return launchEltwiseT<int16_t, int32_t>(a, stream);
-    case 4 * 8 + 1: return launchEltwiseT<int32_t, int8_t>(a, stream);
-    case 4 * 8 + 2: return launchEltwiseT<int32_t, int16_t>(a, stream);
-    case 4 * 8 + 4: return launchEltwiseT<int32_t, int32_t>(a, stream);
+    case 1 * 8 + 1: return launchEltwiseT<int8_t, int8_t>(a, ctx);
+    case 1 * 8 + 2: return launchEltwiseT<int8_t, int16_t>(a, ctx);
+    case 1 * 8 + 4: return launchEltwiseT<int8_t, int32_t>(a, ctx);
+    case 2 * 8 + 1: return launchEltwiseT<int16_t, int8_t>(a, ctx);
+    case 2 * 8 + 2: return launchEltwiseT<int16_t, int16_t>(a, ctx);
+    case 2 * 8 + 4: return launchEltwiseT<int16_t, int32_t>(a, ctx);
+    case 4 * 8 + 1: return launchEltwiseT<int32_t, int8_t>(a, ctx);
+    case 4 * 8 + 2: return launchEltwiseT<int32_t, int16_t>(a, ctx);
+    case 4 * 8 + 4: return launchEltwiseT<int32_t, int32_t>(a, ctx);
     default: return hipErrorInvalidValue;
     }
 }
 
-// Batched transpose [B][R][S] -> [B][S][R] of 1- or 2-byte elements through a 64 x 64 LDS tile.
+// Batched transpose [B][R][S] -> [B][S][R] of 1- or 2-byte elements through a 64 x 64 LDS tile; output rows are
+// out_pitch elements apart (what lies between R and the pitch is not written).
 template <typename T>
 __global__ __launch_bounds__(256) void transpose_i8(TransposeArgs p) {
     __shared__ T tile[64][65];
@@ -2707,26 +2728,26 @@ __global__ __launch_bounds__(256) void transpose_i8(TransposeArgs p) {
     const int b = bid / tilesR;
     const int r0 = tr * 64, s0 = ts * 64;
     const T *src = (const T *)p.in + (size_t)b * p.R * p.S;
-    T *dst = (T *)p.out + (size_t)b * p.R * p.S;
+    T *dst = (T *)p.out + (size_t)b * p.S * p.out_pitch;
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
     for (int r = ty; r < 64; r += 4) {
         if (r0 + r < p.R && s0 + tx < p.S) tile[r][tx] = src[(size_t)(r0 + r) * p.S + s0 + tx];
     }
     __syncthreads();
     for (int s = ty; s < 64; s += 4) {
-        if (s0 + s < p.S && r0 + tx < p.R) dst[(size_t)(s0 + s) * p.R + r0 + tx] = tile[tx][s];
+        if (s0 + s < p.S && r0 + tx < p.R) dst[(size_t)(s0 + s) * p.out_pitch + r0 + tx] = tile[tx][s];
     }
 }
 
-hipError_t launchTranspose(const TransposeArgs &a, hipStream_t stream) {
-    if (!a.in || !a.out || a.B <= 0 || a.R <= 0 || a.S <= 0 || (a.elem != 1 && a.elem != 2)) return hipErrorInvalidValue;
+hipError_t launchTranspose(const TransposeArgs &a, const LaunchCtx &ctx) {
+    if (!a.in || !a.out || a.B <= 0 || a.R <= 0 || a.S <= 0 || (a.elem != 1 && a.elem != 2) || a.out_pitch < a.R) return hipErrorInvalidValue;
     if (a.elem == 2 && ((((uintptr_t)a.in) | ((uintptr_t)a.out)) & 1)) return hipErrorInvalidValue;
     const long long blocks = (long long)a.B * ((a.R + 63) / 64) * ((a.S + 63) / 64);
     if (blocks >= (1LL << 31)) return hipErrorInvalidValue;
     if (a.elem == 2) {
-        hipLaunchKernelGGL(transpose_i8<uint16_t>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+        THIP_ENQUEUE(ctx, "transpose_i8<2>", transpose_i8<uint16_t>, dim3((unsigned)blocks), dim3(256), 0, a);
     } else {
-        hipLaunchKernelGGL(transpose_i8<int8_t>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+        THIP_ENQUEUE(ctx, "transpose_i8<1>", transpose_i8<int8_t>, dim3((unsigned)blocks), dim3(256), 0, a);
     }
     return hipGetLastError();
 }
@@ -2990,31 +3011,28 @@ __global__ __launch_bounds__(256) void fc_bf16_wide(FcBf16Args p, FastDiv qblk) 
 }
 
 template <int Q8, int U>
-static hipError_t launchFcBf16WideU(const FcBf16Args &a, FastDiv blk, hipStream_t stream) {
+static hipError_t launchFcBf16WideU(const FcBf16Args &a, FastDiv blk, const LaunchCtx &ctx) {
     auto kernel = fc_bf16_wide<Q8, U>;
-    static bool configured = false;
-    if (!configured) {
-        hipError_t err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kFcBf16WideMaxSteps * 4 * 66 * 16);
-        if (err != hipSuccess) return err;
-        configured = true;
-    }
+    static std::once_flag once;
+    static hipError_t configured = hipSuccess;
+    std::call_once(once, [&] { configured = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kFcBf16WideMaxSteps * 4 * 66 * 16); });
+    if (configured != hipSuccess) return configured;
     const int steps = (a.K + 63) / 64, nblocks = (a.N + 31) / 32;
     const dim3 grid((unsigned)((nblocks + 3) / 4), (unsigned)((a.M + 31) / 32));
     const int mt = a.M < 32 ? a.M : 32;
-    hipLaunchKernelGGL(kernel, grid, dim3(256), (size_t)steps * 4 * 2 * (mt + 1) * 16, stream, a, blk);
+    THIP_ENQUEUE(ctx, kernelLabel("fc_bf16_wide", {Q8, U}), kernel, grid, dim3(256), (size_t)steps * 4 * 2 * (mt + 1) * 16, a, blk);
     return hipGetLastError();
 }
 
 template <int Q8>
-static hipError_t launchFcBf16Wide(const FcBf16Args &a, FastDiv blk, hipStream_t stream) {
-    const char *e = getenv("THIP_FC_WIDE_U");
-    const int u = e ? atoi(e) : (Q8 ? 4 : 2);
-    if (u == 8 && Q8) return launchFcBf16WideU<Q8, 8>(a, blk, stream);
-    if (u == 4) return launchFcBf16WideU<Q8, 4>(a, blk, stream);
-    return launchFcBf16WideU<Q8, Q8 ? 4 : 2>(a, blk, stream);
+static hipError_t launchFcBf16Wide(const FcBf16Args &a, FastDiv blk, const LaunchCtx &ctx) {
+    const int u = ctx.tuning->fcWideU > 0 ? ctx.tuning->fcWideU : (Q8 ? 4 : 2);
+    if (u == 8 && Q8) return launchFcBf16WideU<Q8, 8>(a, blk, ctx);
+    if (u == 4) return launchFcBf16WideU<Q8, 4>(a, blk, ctx);
+    return launchFcBf16WideU<Q8, Q8 ? 4 : 2>(a, blk, ctx);
 }
 
-hipError_t launchFcBf16(const FcBf16Args &a, hipStream_t stream) {
+hipError_t launchFcBf16(const FcBf16Args &a, const LaunchCtx &ctx) {
     if (!a.x || !a.w || !a.bias || !a.out || a.M <= 0 || a.N <= 0 || a.K <= 0 || a.K % 8 != 0) return hipErrorInvalidValue;
     if (((((uintptr_t)a.x) | ((uintptr_t)a.w)) & 15) || (((uintptr_t)a.out) & (a.N % 4 == 0 ? 7 : 1)) || (((uintptr_t)a.bias) & 3)) return hipErrorInvalidValue;
     if (a.ksplit < 1 || a.ksplit > 64 || (a.ksplit > 1 && (!a.workspace || ((uintptr_t)a.workspace & 255)))) return hipErrorInvalidValue;
@@ -3022,24 +3040,24 @@ hipError_t launchFcBf16(const FcBf16Args &a, hipStream_t stream) {
     if (grid.y > 65535) return hipErrorInvalidValue;
     // few blocks (registers do not limit anything then) and 5 or 6 k-steps per wave: one deeper round of loads instead of two
     const int stepsPerWave = (((a.K + 63) / 64 + a.ksplit - 1) / a.ksplit + 3) / 4;
-    const bool deep = (long long)grid.x * grid.y * grid.z <= 512 && stepsPerWave > 4 && stepsPerWave <= 6 && !getenv("THIP_NO_FC_DEEP");
+    const bool deep = (long long)grid.x * grid.y * grid.z <= 512 && stepsPerWave > 4 && stepsPerWave <= 6 && !ctx.tuning->noFcDeep;
     // a very wide N with a short K and no K split: every wave streams its own columns (THIP_NO_FC_WIDE: off)
     const bool wide = a.w_fragments >= 1 && a.ksplit == 1 && (a.K + 63) / 64 <= kFcBf16WideMaxSteps && (a.N + 31) / 32 >= 1024 &&
-                      !getenv("THIP_NO_FC_WIDE");
+                      !ctx.tuning->noFcWide;
     if (a.w_fragments == 2) {
         if (!a.qscale || !a.qbias || a.qblock < 32 || a.qblock % 32 != 0 || a.qcols < (a.N + 31) / 32 * 32 || a.qcols % 32 != 0) return hipErrorInvalidValue;
         if ((((uintptr_t)a.qscale) & 1) || (((uintptr_t)a.qbias) & 3)) return hipErrorInvalidValue;
         const FastDiv blk = makeFastDiv((uint32_t)a.qblock);
         const bool clamp = !(a.qlo == -INFINITY && a.qhi == INFINITY);
-        if (wide) return clamp ? launchFcBf16Wide<2>(a, blk, stream) : launchFcBf16Wide<1>(a, blk, stream);
-        if (clamp) hipLaunchKernelGGL((fc_bf16<4, 2>), grid, dim3(256), 0, stream, a, blk);
-        else if (deep) hipLaunchKernelGGL((fc_bf16<4, 1, 6>), grid, dim3(256), 0, stream, a, blk);
-        else hipLaunchKernelGGL((fc_bf16<4, 1>), grid, dim3(256), 0, stream, a, blk);
+        if (wide) return clamp ? launchFcBf16Wide<2>(a, blk, ctx) : launchFcBf16Wide<1>(a, blk, ctx);
+        if (clamp) THIP_ENQUEUE(ctx, "fc_bf16<4,2,4>", (fc_bf16<4, 2>), grid, dim3(256), 0, a, blk);
+        else if (deep) THIP_ENQUEUE(ctx, "fc_bf16<4,1,6>", (fc_bf16<4, 1, 6>), grid, dim3(256), 0, a, blk);
+        else THIP_ENQUEUE(ctx, "fc_bf16<4,1,4>", (fc_bf16<4, 1>), grid, dim3(256), 0, a, blk);
         return hipGetLastError();
     }
-    if (wide) return launchFcBf16Wide<0>(a, makeFastDiv(1), stream);
-    if (deep) hipLaunchKernelGGL((fc_bf16<4, 0, 6>), grid, dim3(256), 0, stream, a, makeFastDiv(1));
-    else hipLaunchKernelGGL((fc_bf16<4, 0>), grid, dim3(256), 0, stream, a, makeFastDiv(1));
+    if (wide) return launchFcBf16Wide<0>(a, makeFastDiv(1), ctx);
+    if (deep) THIP_ENQUEUE(ctx, "fc_bf16<4,0,6>", (fc_bf16<4, 0, 6>), grid, dim3(256), 0, a, makeFastDiv(1));
+    else THIP_ENQUEUE(ctx, "fc_bf16<4,0,4>", (fc_bf16<4, 0>), grid, dim3(256), 0, a, makeFastDiv(1));
     return hipGetLastError();
 }
 
@@ -3076,13 +3094,13 @@ __global__ __launch_bounds__(256) void avgpool_bf16(AvgPoolBf16Args p) {
     }
 }
 
-hipError_t launchAvgPoolBf16(const AvgPoolBf16Args &a, hipStream_t stream) {
+hipError_t launchAvgPoolBf16(const AvgPoolBf16Args &a, const LaunchCtx &ctx) {
     if (a.N <= 0 || a.HW <= 0 || a.C <= 0 || !a.in || !a.out) return hipErrorInvalidValue;
     const bool pairs = a.C % 2 == 0 && (((uintptr_t)a.in) & 3) == 0;
     const long long threads = (long long)a.N * (pairs ? a.C / 2 : a.C);
     const dim3 grid((unsigned)((threads + 255) / 256));
-    if (pairs) hipLaunchKernelGGL(avgpool_bf16<2>, grid, dim3(256), 0, stream, a);
-    else hipLaunchKernelGGL(avgpool_bf16<1>, grid, dim3(256), 0, stream, a);
+    if (pairs) THIP_ENQUEUE(ctx, "avgpool_bf16<2>", avgpool_bf16<2>, grid, dim3(256), 0, a);
+    else THIP_ENQUEUE(ctx, "avgpool_bf16<1>", avgpool_bf16<1>, grid, dim3(256), 0, a);
     return hipGetLastError();
 }
 
@@ -3103,13 +3121,42 @@ __global__ __launch_bounds__(256) void expand_weights_bf16(ExpandWeightsArgs p, 
     }
 }
 
-hipError_t launchExpandWeights(const ExpandWeightsArgs &a, hipStream_t stream) {
+hipError_t launchExpandWeights(const ExpandWeightsArgs &a, const LaunchCtx &ctx) {
     if (!a.w || !a.scale || !a.bias || !a.out || a.K <= 0 || a.N <= 0 || a.block <= 0 || a.K % a.block != 0 || a.bias_cols < a.N) return hipErrorInvalidValue;
     const int quads = (a.N + 3) / 4;
     const long long threads = (long long)a.K * quads;
     if (threads >= (1LL << 39)) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(expand_weights_bf16, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, stream, a, makeFastDiv((uint32_t)a.block), quads);
+    THIP_ENQUEUE(ctx, "expand_weights_bf16", expand_weights_bf16, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, a, makeFastDiv((uint32_t)a.block), quads);
     return hipGetLastError();
+}
+
+}  // namespace thip
+
+namespace thip {
+
+Tuning tuningFromEnvironment() {
+    Tuning t;
+    auto flag = [](const char *name) { return getenv(name) != nullptr; };
+    auto digit = [](const char *name, int unset) {
+        const char *v = getenv(name);
+        return v && v[0] >= '0' && v[0] <= '9' ? v[0] - '0' : unset;
+    };
+    t.noStreamDeep = flag("THIP_NO_STREAM_DEEP");
+    t.streamGuarded = flag("THIP_STREAM_GUARDED");
+    t.streamStage = digit("THIP_STREAM_STAGE", -1);
+    if (t.streamStage > 1) t.streamStage = -1;
+    t.noDirectEpilogue = flag("THIP_NO_DIRECT_EPILOGUE");
+    t.skinnyDot4 = flag("THIP_SKINNY_DOT4");
+    t.depthwiseStrip = digit("THIP_DEPTHWISE_STRIP", -1);
+    if (t.depthwiseStrip > 2) t.depthwiseStrip = -1;
+    t.depthwiseTile = digit("THIP_DEPTHWISE_TILE", -1);
+    if (t.depthwiseTile > 1) t.depthwiseTile = -1;
+    if (const char *v = getenv("THIP_DEPTHWISE_TILE_MIN")) t.depthwiseTileMin = atoll(v);
+    if (const char *v = getenv("THIP_DEPTHWISE_P")) t.depthwisePixels = atoi(v);
+    if (const char *v = getenv("THIP_FC_WIDE_U")) t.fcWideU = atoi(v);
+    t.noFcDeep = flag("THIP_NO_FC_DEEP");
+    t.noFcWide = flag("THIP_NO_FC_WIDE");
+    return t;
 }
 
 }  // namespace thip

@@ -47,7 +47,7 @@ EXPORTED_SYMBOLS = [
     "thip_device_free", "thip_device_h2d", "thip_device_d2h", "thip_device_synchronize",
     "thip_device_set_event_log", "thip_infer_format",
     "thip_executable_create", "thip_executable_destroy", "thip_executable_run",
-    "thip_executable_enqueue", "thip_executable_wait", "thip_executable_time",
+    "thip_executable_enqueue", "thip_executable_wait", "thip_executable_time", "thip_executable_time_rotating",
     "thip_executable_op_count", "thip_executable_op_kernel", "thip_executable_binding_count",
     "thip_executable_binding_size",
 ]
@@ -238,6 +238,7 @@ def lib():
     L.thip_executable_enqueue.argtypes = [vp, P(DispatchState)]
     L.thip_executable_wait.argtypes = [vp]
     L.thip_executable_time.argtypes = [vp, P(DispatchState), i32, P(ctypes.c_float)]
+    L.thip_executable_time_rotating.argtypes = [vp, P(DispatchState), u32, i32, P(ctypes.c_float)]
     L.thip_executable_op_count.argtypes = [vp, P(u32)]
     L.thip_executable_op_kernel.argtypes = [vp, u32, ctypes.c_char_p, sz]
     L.thip_executable_binding_count.argtypes = [vp, P(u32)]
@@ -394,6 +395,15 @@ class Executable:
         ms = ctypes.c_float()
         check(lib().thip_executable_time(self._h, ctypes.byref(st), int(iterations), ctypes.byref(ms)))
         del keep
+        return ms.value
+
+    def time_device_rotating(self, ptr_sets, lengths, iterations):
+        """Like time_device, with dispatch i on ptr_sets[i % len(ptr_sets)] (a working set larger than the caches)."""
+        made = [make_state(ptrs, lengths, [BINDING_DEVICE] * len(ptrs)) for ptrs in ptr_sets]
+        states = (DispatchState * len(made))(*[m[0] for m in made])
+        ms = ctypes.c_float()
+        check(lib().thip_executable_time_rotating(self._h, states, len(made), int(iterations), ctypes.byref(ms)))
+        del made
         return ms.value
 
     def close(self):

@@ -108,6 +108,34 @@ def fully_connected_workload(M, K, N, realistic=False, output_zp=5, output_min=-
                     bytes_, attrs)
 
 
+def matmul_workload(B, M, K, N, batch1=True, batch2=True, constant_rhs=False, out_dtype=np.int16, bias=0, scale=1, shift=0,
+                    output_zp=0, clamp=None, seed=1022):
+    """int8 torq_hl.matmul [B,]M,K x [B,]K,N with ONE (bias, scale) pair and an int8 / int16 / int32 result; input2 is a
+    run-time binding unless constant_rhs.  The defaults are what the matmul patterns produce (bias 0, scale 1, shift 0,
+    the clamp = the range of the result type; compiler/torq/Conversions/LinalgToTorqHL/MatmulPattern.cpp:925-994)."""
+    rng = np.random.default_rng(seed)
+    a = rng.integers(-128, 127, size=(B, M, K) if batch1 else (M, K), endpoint=True, dtype=np.int8)
+    b = rng.integers(-128, 127, size=(B, K, N) if batch2 else (K, N), endpoint=True, dtype=np.int8)
+    sb = np.array([bias, scale], dtype=np.int32)
+    info = np.iinfo(out_dtype)
+    lo, hi = (int(info.min), int(info.max)) if clamp is None else clamp
+    p = Program()
+    ia = p.binding(0, a.shape)
+    inputs = [a]
+    if constant_rhs:
+        ib = b
+    else:
+        ib = p.binding(1, b.shape)
+        inputs.append(b)
+    oshape = ((B,) if (batch1 or batch2) else ()) + (M, N)
+    out = p.binding(len(inputs), oshape, out_dtype)
+    attrs = dict(output_zp=output_zp, output_min=lo, output_max=hi, shift=shift)
+    p.matmul(ia, ib, sb, init=out, out_dtype=out_dtype, **attrs)
+    attrs.update(input2=b, scale_bias=sb, out_dtype=out_dtype)
+    return Workload("matmul_%dx%dx%dx%d" % (B, M, K, N), p, inputs, [(oshape, np.dtype(out_dtype).type)], 2 * B * M * K * N,
+                    a.nbytes + b.nbytes + int(np.prod(oshape)) * np.dtype(out_dtype).itemsize, attrs)
+
+
 def to_bf16(values):
     """float32 array -> bfloat16 bit patterns (uint16), round to nearest even."""
     f = np.ascontiguousarray(values, dtype=np.float32)
