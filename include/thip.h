@@ -424,6 +424,19 @@ thip_status_t thip_executable_enqueue(thip_executable_t *executable,
                                       const thip_dispatch_state_t *state);
 thip_status_t thip_executable_wait(thip_executable_t *executable);
 
+/* thip_executable_enqueue for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid it).  It has no counterpart in the reference.  The dispatch is enqueued
+ * kernel by kernel (no graph is built), on device bindings only, and makes no hipMalloc / hipFree or allocating
+ * library call: the scratch memory of the program's kernels (the partial sums and tile counters of a bf16
+ * fully_connected / matmul whose K is split over blocks) is taken from an array that is part of the library's
+ * device image instead of the executable's intermediates.  The results are those of thip_executable_enqueue.
+ * A program whose kernels need more scratch than the array holds (2 MiB) is refused with
+ * THIP_RESOURCE_EXHAUSTED.  Each GPU has one such array, shared by every executable and kept until the process
+ * ends: calls that overlap in time on one GPU (from different executables, whose streams differ) race on it, so
+ * wait for one to finish before enqueueing the next.  Pair with thip_executable_wait. */
+thip_status_t thip_executable_enqueue_noalloc(thip_executable_t *executable,
+                                              const thip_dispatch_state_t *state);
+
 /* Enqueues the dispatch `iterations` times between two HIP events recorded on
  * the executable's stream and returns the mean time of one dispatch in
  * milliseconds (role of the per-dispatch profile scopes,

@@ -35,6 +35,7 @@ struct thip_device_t {
     std::mutex logMutex;
     FILE *eventLog = nullptr;
     std::chrono::steady_clock::time_point t0 = std::chrono::steady_clock::now();
+    uint8_t *staticScratch = nullptr;    // this GPU's copy of the library's scratch array (kStaticScratchBytes)
 };
 
 struct thip_executable_t {
@@ -62,6 +63,10 @@ struct thip_executable_t {
     uint64_t invocation = 0;             // dispatches so far (the event log's invocation_id)
     Tuning tuning;                       // the environment's switches as they were when the executable was created
     std::vector<std::string> kernelNames;  // per record: the kernel its launcher resolved at creation
+    // thip_executable_enqueue_noalloc: where each record's scratch (a K-split workspace) sits in the static array,
+    // how much of it has to be zero before the launch, and the program's total
+    std::vector<uint64_t> scratchOffset, scratchZeroBytes;
+    uint64_t scratchBytes = 0;
 };
 
 static thip_status_t hipFail(hipError_t e, const char *what) {
@@ -379,7 +384,8 @@ static uint8_t *resolve(const thip_executable_t *e, const DescRef &r, uint8_t *c
 }
 
 // Launches record i, or (ctx.name set) only asks its launcher which kernel it takes for these operands.
-static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *bp, const LaunchCtx &ctx) {
+// `scratch` (or null): the static scratch array, which then stands in for the record's workspace intermediate.
+static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *bp, const LaunchCtx &ctx, uint8_t *scratch = nullptr) {
     const DescOp &op = e->ops[i];
     const Requant rq{op.shift, op.output_zp, op.output_min, op.output_max, op.pre_shift, op.t0_clamp};
     hipError_t err = hipSuccess;
@@ -485,7 +491,7 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
         memcpy(&hi, &op.output_max, 4);
         FcBf16Args a{(const uint16_t *)resolve(e, op.in0, bp), (const uint16_t *)resolve(e, op.weights, bp),
                      (const float *)resolve(e, op.bias, bp), (uint16_t *)resolve(e, op.out, bp), op.M, op.K, op.Nn, lo, hi,
-                     op.w0 > 1 ? op.w0 : 1, op.w0 > 1 ? (void *)resolve(e, op.in1, bp) : nullptr, (int32_t)op.loader,
+                     op.w0 > 1 ? op.w0 : 1, op.w0 > 1 ? (void *)(scratch ? scratch + e->scratchOffset[i] : resolve(e, op.in1, bp)) : nullptr, (int32_t)op.loader,
                      nullptr, nullptr, 0, 0, 0.0f, 0.0f};
         if (op.loader == 2) {
             a.qscale = (const uint16_t *)resolve(e, op.scale, bp);
@@ -644,6 +650,16 @@ thip_status_t thip_device_create(int32_t ordinal, thip_device_t **out_device) {
     if (!d) return fail(THIP_RESOURCE_EXHAUSTED, "out of memory");
     d->ordinal = ordinal;
     d->arch = arch;
+    {
+        // the address of this device's copy of the scratch array (the device is current)
+        void *ptr = nullptr;
+        const hipError_t se = staticScratchAddress(&ptr);
+        if (se != hipSuccess) {
+            delete d;
+            return hipFail(se, "locating the static scratch array");
+        }
+        d->staticScratch = (uint8_t *)ptr;
+    }
     *out_device = d;
     return THIP_OK;
 }
@@ -784,6 +800,15 @@ thip_status_t thip_executable_create(thip_device_t *device, const void *blob, si
     // environment's switches, and kept: the launchers are asked in naming mode (they also configure their kernels,
     // which must not happen later inside a stream capture).  Bindings stand in as aligned placeholder addresses:
     // device bindings must be 16-byte aligned and staged host bindings are, so a dispatch resolves the same way.
+    e->scratchOffset.assign(h.op_count, 0);
+    e->scratchZeroBytes.assign(h.op_count, 0);
+    for (uint32_t i = 0; i < h.op_count; i++) {
+        const DescOp &op = e->ops[i];
+        if (op.kind != kKindFcBf16 || op.w0 <= 1) continue;
+        e->scratchOffset[i] = e->scratchBytes;
+        e->scratchZeroBytes[i] = fcBf16WorkspaceCounterBytes(op.M, op.Nn, op.w0);
+        e->scratchBytes += (fcBf16WorkspaceBytes(op.M, op.Nn, op.w0) + 255) / 256 * 256;
+    }
     e->tuning = tuningFromEnvironment();
     e->kernelNames.assign(h.op_count, std::string());
     {
@@ -867,6 +892,33 @@ thip_status_t thip_executable_enqueue(thip_executable_t *e, const thip_dispatch_
     const thip_status_t s = enqueueDevice(e, bp);
     e->invocation++;
     return s;
+}
+
+thip_status_t thip_executable_enqueue_noalloc(thip_executable_t *e, const thip_dispatch_state_t *st) {
+    if (!e) return fail(THIP_INVALID_ARGUMENT, "null executable");
+    if (thip_status_t s = checkState(e, st, true)) return s;
+    if (e->scratchBytes > kStaticScratchBytes) {
+        return fail(THIP_RESOURCE_EXHAUSTED, "the program's kernels need %llu bytes of scratch, the static array holds %llu",
+                    (unsigned long long)e->scratchBytes, (unsigned long long)kStaticScratchBytes);
+    }
+    std::lock_guard<std::mutex> lock(e->mutex);
+    THIP_HIP(hipSetDevice(e->device->ordinal), "hipSetDevice");
+    uint8_t *scratch = e->device->staticScratch;  // the address hipGetSymbolAddress gave for this device
+    if (!scratch) return fail(THIP_INTERNAL, "the static scratch array was not located");
+    uint8_t *bp[64] = {nullptr};
+    for (uint32_t i = 0; i < e->header.binding_count; i++) bp[i] = (uint8_t *)st->binding_ptrs[i];
+    const LaunchCtx ctx{e->stream, &e->tuning, nullptr, 0};
+    thip_status_t result = THIP_OK;
+    for (uint32_t i = 0; i < e->header.op_count && result == THIP_OK; i++) {
+        // the array keeps what the last call left there, whoever made it: what has to start at zero is cleared
+        if (e->scratchZeroBytes[i]) {
+            const hipError_t ze = launchZeroFill(scratch + e->scratchOffset[i], (size_t)e->scratchZeroBytes[i], e->stream);
+            if (ze != hipSuccess) result = hipFail(ze, "clearing the scratch counters");
+        }
+        if (result == THIP_OK) result = launchOp(e, i, bp, ctx, scratch);
+    }
+    e->invocation++;
+    return result;
 }
 
 thip_status_t thip_executable_wait(thip_executable_t *e) {

@@ -185,6 +185,17 @@ inline int fcBf16PreferredSplit(int M, int N, int K) {
     return split < 2 ? 1 : (int)split;
 }
 hipError_t launchFcBf16(const FcBf16Args &a, const LaunchCtx &ctx);
+// Bytes of a K-split workspace that must be zero before a launch (the tile counters, padded to 256).
+inline size_t fcBf16WorkspaceCounterBytes(int M, int N, int ksplit) {
+    const size_t tiles = (size_t)((N + 31) / 32) * ((M + 31) / 32);
+    return ksplit <= 1 ? 0 : (tiles * 4 + 255) / 256 * 256;
+}
+
+// The library's static scratch array (device memory that needs no allocation): its size, its address on the
+// current device (ask once per device, with that device current), and a zero fill that is a kernel.
+constexpr size_t kStaticScratchBytes = 2u << 20;
+hipError_t staticScratchAddress(void **out);
+hipError_t launchZeroFill(void *dst, size_t bytes, hipStream_t stream);
 
 // Integer elementwise ops with the ACT stage behind them.  fma: out = R1(in0 * w0); mul: out = R1(in0 * in1) (an
 // input of one element is broadcast); both with ONE (bias, scale) pair.  clamp / abs / negate / i2i: the input

@@ -3134,6 +3134,47 @@ hipError_t launchExpandWeights(const ExpandWeightsArgs &a, const LaunchCtx &ctx)
 
 namespace thip {
 
+// ---------------------------------------------------------------------------
+// Scratch memory that exists without any allocation: a device array of the library's image.  Every GPU the
+// library runs on holds its own copy, at its own address, until the process ends.  In host code the array's name
+// is only a handle for hipGetSymbolAddress; the address that call returns is what kernels, fills and copies take.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+hipError_t staticScratchAddress(void **out) {
+    // asked once per device, with that device current; kept for the life of the process
+    static std::mutex mutex;
+    static void *known[64] = {nullptr};
+    int device = -1;
+    hipError_t err = hipGetDevice(&device);
+    if (err != hipSuccess) return err;
+    if (device < 0 || device >= 64) return hipErrorInvalidDevice;
+    std::lock_guard<std::mutex> lock(mutex);
+    if (!known[device]) {
+        void *ptr = nullptr;
+        err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (err != hipSuccess) return err;
+        if (!ptr || ((uintptr_t)ptr & 255) != 0) return hipErrorInvalidSymbol;
+        known[device] = ptr;
+    }
+    *out = known[device];
+    return hipSuccess;
+}
+
+// Zero fill by a kernel (a memset node recorded into a captured graph is not reliable on this platform).
+__global__ __launch_bounds__(256) void zero_fill(v4i *dst, size_t count) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < count) dst[i] = v4i{0, 0, 0, 0};
+}
+
+hipError_t launchZeroFill(void *dst, size_t bytes, hipStream_t stream) {
+    if (!dst || bytes == 0 || (bytes & 15) != 0 || ((uintptr_t)dst & 15) != 0) return hipErrorInvalidValue;
+    const size_t count = bytes / 16;
+    if ((count + 255) / 256 >= (1ull << 31)) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(zero_fill, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, (v4i *)dst, count);
+    return hipGetLastError();
+}
+
 Tuning tuningFromEnvironment() {
     Tuning t;
     auto flag = [](const char *name) { return getenv(name) != nullptr; };

@@ -47,7 +47,7 @@ EXPORTED_SYMBOLS = [
     "thip_device_free", "thip_device_h2d", "thip_device_d2h", "thip_device_synchronize",
     "thip_device_set_event_log", "thip_infer_format",
     "thip_executable_create", "thip_executable_destroy", "thip_executable_run",
-    "thip_executable_enqueue", "thip_executable_wait", "thip_executable_time", "thip_executable_time_rotating",
+    "thip_executable_enqueue", "thip_executable_enqueue_noalloc", "thip_executable_wait", "thip_executable_time", "thip_executable_time_rotating",
     "thip_executable_op_count", "thip_executable_op_kernel", "thip_executable_binding_count",
     "thip_executable_binding_size",
 ]
@@ -236,6 +236,7 @@ def lib():
     L.thip_executable_destroy.restype = None
     L.thip_executable_run.argtypes = [vp, P(DispatchState)]
     L.thip_executable_enqueue.argtypes = [vp, P(DispatchState)]
+    L.thip_executable_enqueue_noalloc.argtypes = [vp, P(DispatchState)]
     L.thip_executable_wait.argtypes = [vp]
     L.thip_executable_time.argtypes = [vp, P(DispatchState), i32, P(ctypes.c_float)]
     L.thip_executable_time_rotating.argtypes = [vp, P(DispatchState), u32, i32, P(ctypes.c_float)]
@@ -384,6 +385,12 @@ class Executable:
     def enqueue_device(self, ptrs, lengths):
         st, keep = make_state(ptrs, lengths, [BINDING_DEVICE] * len(ptrs))
         check(lib().thip_executable_enqueue(self._h, ctypes.byref(st)))
+        del keep
+
+    def enqueue_device_noalloc(self, ptrs, lengths):
+        """thip_executable_enqueue_noalloc: the dispatch without any device allocation (scratch from the static array)."""
+        st, keep = make_state(ptrs, lengths, [BINDING_DEVICE] * len(ptrs))
+        check(lib().thip_executable_enqueue_noalloc(self._h, ctypes.byref(st)))
         del keep
 
     def wait(self):
