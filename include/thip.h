@@ -375,11 +375,27 @@ thip_status_t thip_device_d2h(thip_device_t *device, void *dst_host, const void 
                               size_t size);
 thip_status_t thip_device_synchronize(thip_device_t *device);
 
-/* Validates the header of a descriptor blob and writes the format string
+/* Debug dumps, the roles of the reference's --torq_dump_io_data_dir and --torq_dump_buffers_dir
+ * (runtime/driver/TorqDump.cc:34-35,329-428).  io_data_dir: every blocking dispatch writes the raw bytes of its
+ * host bindings to <io_data_dir>/thip_dispatch/npu.{in,out}.host_binding.<i>.torq_binding.<i>.bin (the reference's
+ * file names).  buffers_dir: dispatches run one kernel record at a time and after record <a> the buffer it wrote
+ * is saved as <buffers_dir>/thip_dispatch/action<a>/buffer<id>.npy (a NumPy array; id = binding<k> or temp<k>;
+ * activations are N,H,W,C as the kernels hold them), with an index buffers.csv in the reference's columns.
+ * NULL or "" switches a dump off.  Dumps are for debugging: they serialise the GPU and copy every result back. */
+thip_status_t thip_device_set_dump_dirs(thip_device_t *device, const char *io_data_dir,
+                                        const char *buffers_dir);
+
+/* Validates a descriptor blob and writes the format string
  * ("thip-gfx950") -- iree_hal_torq_native_executable_infer_format,
  * runtime/driver/native_executable.cc:151-178. */
 thip_status_t thip_infer_format(const void *blob, size_t size, size_t format_capacity,
                                 char *format, size_t *out_inferred_size);
+
+/* Everything thip_executable_create checks about a blob before it touches the GPU: header (magic, version,
+ * target), table extents, every operand reference and every kernel record's footprint inside the buffer it
+ * names, k-table entries inside their windows.  Needs no device.  The blob must be 8-byte aligned.  (The
+ * reference verifies its flatbuffer the same way before use, runtime/driver/native_executable.cc:151-170.) */
+thip_status_t thip_descriptor_validate(const void *blob, size_t size);
 
 /* Creates an executable from a descriptor: copies the blob, uploads its
  * constant segments, allocates intermediates --
@@ -423,6 +439,14 @@ thip_status_t thip_executable_run(thip_executable_t *executable,
 thip_status_t thip_executable_enqueue(thip_executable_t *executable,
                                       const thip_dispatch_state_t *state);
 thip_status_t thip_executable_wait(thip_executable_t *executable);
+
+/* Every wait for the GPU (run, wait, time) gives up after this many milliseconds (default 120 000, or the
+ * environment's THIP_WAIT_TIMEOUT_MS when the executable is created; <= 0: no limit) and returns THIP_INTERNAL,
+ * as the reference turns a hardware wait that exceeds its timeout into IREE_STATUS_INTERNAL
+ * (runtime/torq_hw/src/TorqHw.cpp:172-186, runtime/driver/TorqExecutable.cc:640-643).  The executable is then
+ * abandoned: its kernels may still be running, every later call on it fails with THIP_FAILED_PRECONDITION, and
+ * destroying it leaves its device memory in place.  The process itself stays usable. */
+thip_status_t thip_executable_set_wait_timeout(thip_executable_t *executable, int64_t milliseconds);
 
 /* thip_executable_enqueue for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid it).  It has no counterpart in the reference.  The dispatch is enqueued

@@ -13,7 +13,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libthip.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
-SOURCES = ["thip_kernels.hip", "thip_driver.cpp", "thip_emitter.cpp", "thip_status.cpp"]
+SOURCES = ["thip_kernels.hip", "thip_driver.cpp", "thip_emitter.cpp", "thip_validate.cpp", "thip_status.cpp"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",

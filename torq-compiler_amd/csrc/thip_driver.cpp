@@ -17,15 +17,20 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <errno.h>
+#include <sys/stat.h>
+
 #include <chrono>
 #include <mutex>
 #include <new>
 #include <string>
+#include <thread>
 #include <vector>
 
 #include "thip_descriptor.h"
 #include "thip_kernels.h"
 #include "thip_status.h"
+#include "thip_validate.h"
 
 using namespace thip;
 
@@ -36,6 +41,8 @@ struct thip_device_t {
     FILE *eventLog = nullptr;
     std::chrono::steady_clock::time_point t0 = std::chrono::steady_clock::now();
     uint8_t *staticScratch = nullptr;    // this GPU's copy of the library's scratch array (kStaticScratchBytes)
+    // dump directories (empty: off): bindings of every blocking dispatch / every buffer a kernel record wrote
+    std::string dumpIoDir, dumpBuffersDir;
 };
 
 struct thip_executable_t {
@@ -51,7 +58,11 @@ struct thip_executable_t {
     std::vector<uint8_t *> tempPtrs;     // device intermediates
     std::vector<uint8_t *> staging;      // device staging of host bindings
     hipStream_t stream = nullptr;
-    hipEvent_t evStart = nullptr, evStop = nullptr;
+    hipEvent_t evStart = nullptr, evStop = nullptr, evDone = nullptr;
+    // A wait for the GPU gives up after this long (the reference turns a wait that exceeds its timeout into
+    // IREE_STATUS_INTERNAL, runtime/torq_hw/src/TorqHw.cpp:172-186).  <= 0: no limit.
+    int64_t waitTimeoutMs = 120000;
+    bool abandoned = false;              // a wait timed out: work may still be running, the executable is unusable
     std::mutex mutex;                    // one dispatch at a time
     // Multi-kernel programs on device bindings are replayed as a HIP graph: the first dispatch on a
     // set of binding pointers runs eagerly, the second is captured, later ones are one graph launch.
@@ -79,268 +90,6 @@ static thip_status_t hipFail(hipError_t e, const char *what) {
         hipError_t e_ = (call);                       \
         if (e_ != hipSuccess) return hipFail(e_, what); \
     } while (0)
-
-static thip_status_t validateDescriptor(const uint8_t *p, size_t size, DescHeader *out) {
-    if (!p || size < sizeof(DescHeader)) return fail(THIP_INVALID_ARGUMENT, "descriptor is smaller than its header");
-    DescHeader h;
-    memcpy(&h, p, sizeof(h));
-    if (h.magic != kMagic) return fail(THIP_INVALID_ARGUMENT, "descriptor magic 0x%08x is not THIP", h.magic);
-    // same gate as `runtime_version != 2 -> UNAVAILABLE`, runtime/driver/TorqExecutable.cc:663-667
-    if (h.version != kDescriptorVersion) {
-        return fail(THIP_UNAVAILABLE, "descriptor version %u, this runtime reads version %u", h.version, kDescriptorVersion);
-    }
-    // same gate as isHwCompatible(hwId), runtime/driver/TorqExecutable.cc:701-705
-    if (h.arch != kArchGfx950) return fail(THIP_UNAVAILABLE, "descriptor targets arch %u, this runtime drives gfx950", h.arch);
-    if (h.total_size > size) return fail(THIP_INVALID_ARGUMENT, "descriptor says %llu bytes, %zu given", (unsigned long long)h.total_size, size);
-    auto inside = [&](uint64_t off, uint64_t count, uint64_t each) {
-        return off <= h.total_size && count * each <= h.total_size - off;
-    };
-    if (!inside(h.ops_offset, h.op_count, sizeof(DescOp)) || !inside(h.bindings_offset, h.binding_count, sizeof(DescBinding)) ||
-        !inside(h.temps_offset, h.temp_count, sizeof(DescTemp)) || !inside(h.consts_offset, h.const_count, sizeof(DescConst)) ||
-        h.data_offset > h.total_size) {
-        return fail(THIP_INVALID_ARGUMENT, "descriptor tables run past its end");
-    }
-    if (h.op_count == 0) return fail(THIP_INVALID_ARGUMENT, "descriptor holds no ops");
-    if (h.binding_count > 64) return fail(THIP_INVALID_ARGUMENT, "descriptor declares %u bindings (max 64)", h.binding_count);
-    const DescConst *consts = (const DescConst *)(p + h.consts_offset);
-    for (uint32_t i = 0; i < h.const_count; i++) {
-        if (consts[i].offset > h.total_size - h.data_offset || consts[i].size > h.total_size - h.data_offset - consts[i].offset) {
-            return fail(THIP_INVALID_ARGUMENT, "constant segment %u runs past the descriptor", i);
-        }
-    }
-    // every operand reference must name an existing buffer and stay inside it
-    const DescOp *ops = (const DescOp *)(p + h.ops_offset);
-    const DescBinding *bindings = (const DescBinding *)(p + h.bindings_offset);
-    const DescTemp *temps = (const DescTemp *)(p + h.temps_offset);
-    for (uint32_t i = 0; i < h.op_count; i++) {
-        const DescRef *refs[] = {&ops[i].in0, &ops[i].in1, &ops[i].weights, &ops[i].bias, &ops[i].scale, &ops[i].table, &ops[i].out};
-        for (const DescRef *r : refs) {
-            uint64_t limit = 0;
-            switch (r->space) {
-            case kSpaceNone: continue;
-            case kSpaceBinding:
-                if (r->index >= h.binding_count) return fail(THIP_INVALID_ARGUMENT, "op %u names binding %u of %u", i, r->index, h.binding_count);
-                limit = bindings[r->index].size;
-                break;
-            case kSpaceTemp:
-                if (r->index >= h.temp_count) return fail(THIP_INVALID_ARGUMENT, "op %u names intermediate %u of %u", i, r->index, h.temp_count);
-                limit = temps[r->index].size;
-                break;
-            case kSpaceConst:
-                if (r->index >= h.const_count) return fail(THIP_INVALID_ARGUMENT, "op %u names constant %u of %u", i, r->index, h.const_count);
-                limit = consts[r->index].size;
-                break;
-            default: return fail(THIP_INVALID_ARGUMENT, "op %u has an operand in unknown space %u", i, r->space);
-            }
-            if (r->offset > limit) return fail(THIP_INVALID_ARGUMENT, "op %u operand offset %llu is past its buffer (%llu)", i, (unsigned long long)r->offset, (unsigned long long)limit);
-        }
-    }
-    *out = h;
-    return THIP_OK;
-}
-
-// Bytes an operand reference can still address.
-static uint64_t refRoom(const thip_executable_t *e, const DescRef &r) {
-    switch (r.space) {
-    case kSpaceBinding: return e->bindings[r.index].size - r.offset;
-    case kSpaceTemp: return e->temps[r.index].size - r.offset;
-    case kSpaceConst: return e->consts[r.index].size - r.offset;
-    default: return 0;
-    }
-}
-
-// Checks, once at creation, that every kernel record stays inside the buffers it names.
-static thip_status_t checkOpFootprint(const thip_executable_t *e, uint32_t i) {
-    const DescOp &op = e->ops[i];
-    auto need = [&](const DescRef &r, uint64_t bytes, const char *name) -> thip_status_t {
-        if (r.space == kSpaceNone) return fail(THIP_INVALID_ARGUMENT, "op %u: operand %s is missing", i, name);
-        if (refRoom(e, r) < bytes) {
-            return fail(THIP_INVALID_ARGUMENT, "op %u: operand %s needs %llu bytes, its buffer has %llu", i, name,
-                        (unsigned long long)bytes, (unsigned long long)refRoom(e, r));
-        }
-        return THIP_OK;
-    };
-    auto positive = [&](std::initializer_list<int32_t> vals) {
-        for (int32_t v : vals) {
-            if (v <= 0) return false;
-        }
-        return true;
-    };
-    const uint64_t outElem = op.out_dtype == THIP_DTYPE_I32 ? 4 : op.out_dtype == THIP_DTYPE_I16 ? 2 : 1;
-    thip_status_t s = THIP_OK;
-    if (op.pre_shift != 0 && (op.pre_shift < 0 || op.pre_shift > 30 || op.shift + op.pre_shift != 33 ||
-                              (op.kind != kKindIgemm && op.kind != kKindDepthwise))) {
-        return fail(THIP_INVALID_ARGUMENT, "op %u: pre_shift %d does not complete shift %d to 33", i, op.pre_shift, op.shift);
-    }
-    if (op.t0_clamp != 0 && (op.t0_clamp < 0 || op.pre_shift <= 0 || op.pre_shift > 30 || op.t0_clamp >= (1 << (31 - op.pre_shift)))) {
-        return fail(THIP_INVALID_ARGUMENT, "op %u: t0_clamp %d does not fit pre_shift %d", i, op.t0_clamp, op.pre_shift);
-    }
-    switch (op.kind) {
-    case kKindTranspose: {
-        if (!positive({op.TB, op.TR, op.TS})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad transpose extents", i);
-        if (op.gran > 2) return fail(THIP_INVALID_ARGUMENT, "op %u: transpose element size %u", i, op.gran);
-        if (op.TP != 0 && op.TP < op.TR) return fail(THIP_INVALID_ARGUMENT, "op %u: transpose pitch %d is below its row length %d", i, op.TP, op.TR);
-        const uint64_t elem = op.gran == 2 ? 2 : 1, pitch = op.TP ? (uint64_t)op.TP : (uint64_t)op.TR;
-        if ((s = need(op.in0, (uint64_t)op.TB * op.TR * op.TS * elem, "in"))) return s;
-        return need(op.out, (uint64_t)op.TB * op.TS * pitch * elem, "out");
-    }
-    case kKindIgemm: {
-        if (!positive({op.M, op.K, op.Kp, op.Nn, op.Np, op.N, op.H, op.W, op.C, op.OH, op.OW})) {
-            return fail(THIP_INVALID_ARGUMENT, "op %u: bad igemm extents", i);
-        }
-        if (op.variant >= kIgemmVariantCount) return fail(THIP_INVALID_ARGUMENT, "op %u: unknown igemm variant %u", i, op.variant);
-        const uint64_t inBytes = op.loader == kLoaderDense ? (uint64_t)op.M * op.K : (uint64_t)op.N * op.H * op.W * op.C;
-        if (op.loader != kLoaderDense && (uint64_t)op.N * op.OH * op.OW != (uint64_t)op.M) {
-            return fail(THIP_INVALID_ARGUMENT, "op %u: igemm rows do not match the output pixels", i);
-        }
-        if ((s = need(op.in0, inBytes, "in"))) return s;
-        if ((s = need(op.weights, (uint64_t)op.Np * op.Kp, "weights"))) return s;
-        if ((s = need(op.bias, (uint64_t)op.Np * 4, "bias"))) return s;
-        if ((s = need(op.scale, (uint64_t)op.Np * 4, "scale"))) return s;
-        if (op.loader > kLoaderRuns) return fail(THIP_INVALID_ARGUMENT, "op %u: unknown igemm loader %u", i, op.loader);
-        if (op.loader == kLoaderRuns) {
-            if (op.KW * op.C > 16 || op.Kp % 16 != 0) return fail(THIP_INVALID_ARGUMENT, "op %u: window row of %d bytes does not fit a 16-byte run", i, op.KW * op.C);
-            if ((s = need(op.table, (uint64_t)op.Kp / 16 * 4, "table"))) return s;
-            if (op.table.space != kSpaceConst) return fail(THIP_INVALID_ARGUMENT, "op %u: table must be a constant", i);
-            const uint8_t *base = e->blob.data() + e->header.data_offset + e->consts[op.table.index].offset + op.table.offset;
-            for (uint32_t t = 0; t < (uint32_t)op.Kp / 16; t++) {
-                uint32_t ent;
-                memcpy(&ent, base + 4ull * t, 4);
-                if (ent & kKEntryInvalid) continue;
-                if ((int)((ent >> 24) & 0x7f) >= op.KH || (int)(ent & 0xffff) != op.KW * op.C) return fail(THIP_INVALID_ARGUMENT, "op %u: run table entry %u is outside the window", i, t);
-            }
-        }
-        if (op.loader == kLoaderGather) {
-            if (op.gran == 0 || (op.gran & (op.gran - 1)) || op.gran > 16) return fail(THIP_INVALID_ARGUMENT, "op %u: bad gather granularity", i);
-            if ((s = need(op.table, (uint64_t)op.Kp / op.gran * 4, "table"))) return s;
-            // every valid table entry must stay inside the window and the channel axis
-            const uint8_t *base = e->blob.data() + e->header.data_offset + e->consts[op.table.index].offset + op.table.offset;
-            if (op.table.space != kSpaceConst) return fail(THIP_INVALID_ARGUMENT, "op %u: table must be a constant", i);
-            for (uint32_t t = 0; t < (uint32_t)op.Kp / op.gran; t++) {
-                uint32_t ent;
-                memcpy(&ent, base + 4ull * t, 4);
-                if (ent & kKEntryInvalid) continue;
-                const int kh = (ent >> 24) & 0x7f, kw = (ent >> 16) & 0xff, ci = ent & 0xffff;
-                if (kh >= op.KH || kw >= op.KW || ci + (int)op.gran > op.C) return fail(THIP_INVALID_ARGUMENT, "op %u: table entry %u is outside the window", i, t);
-            }
-        }
-        if (op.in1.space != kSpaceNone) {  // fused residual add
-            if ((op.variant != kIgemmStream && op.variant != kIgemmDense64x64) || op.loader != kLoaderDense || op.out_dtype != THIP_DTYPE_I8 ||
-                op.table.space != kSpaceConst) {
-                return fail(THIP_INVALID_ARGUMENT, "op %u: a residual add needs the streaming or the small-tile int8 kernel", i);
-            }
-            if ((s = need(op.in1, (uint64_t)op.M * op.Nn, "residual"))) return s;
-            if ((s = need(op.table, sizeof(ResidualAddParams), "residual parameters"))) return s;
-            ResidualAddParams ap;
-            memcpy(&ap, e->blob.data() + e->header.data_offset + e->consts[op.table.index].offset + op.table.offset, sizeof(ap));
-            if (ap.shift < 0 || ap.shift > 63 || ap.output_min > ap.output_max || ap.output_min < -128 || ap.output_max > 127) {
-                return fail(THIP_INVALID_ARGUMENT, "op %u: bad residual add parameters", i);
-            }
-        }
-        return need(op.out, (uint64_t)op.M * op.Nn * outElem, "out");
-    }
-    case kKindFcSkinny: {
-        if (!positive({op.M, op.K, op.Nn})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad fc extents", i);
-        if ((s = need(op.in0, (uint64_t)op.M * op.K, "in"))) return s;
-        if ((s = need(op.weights, (uint64_t)op.Nn * op.K, "weights"))) return s;
-        if ((s = need(op.bias, (uint64_t)op.Nn * 4, "bias"))) return s;
-        if ((s = need(op.scale, (uint64_t)op.Nn * 4, "scale"))) return s;
-        return need(op.out, (uint64_t)op.M * op.Nn * outElem, "out");
-    }
-    case kKindDepthwise: {
-        if (!positive({op.N, op.H, op.W, op.C, op.OH, op.OW, op.KH, op.KW})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad depthwise extents", i);
-        if ((s = need(op.in0, (uint64_t)op.N * op.H * op.W * op.C, "in"))) return s;
-        if (op.variant > kDepthwiseDot4Rows) return fail(THIP_INVALID_ARGUMENT, "op %u: unknown depthwise variant %u", i, op.variant);
-        if ((s = need(op.weights, op.variant == kDepthwiseDot4Rows ? (uint64_t)op.KH * op.C * 4 : (uint64_t)op.KH * op.KW * op.C, "weights"))) return s;
-        if ((s = need(op.bias, (uint64_t)op.C * 4, "bias"))) return s;
-        if ((s = need(op.scale, (uint64_t)op.C * 4, "scale"))) return s;
-        return need(op.out, (uint64_t)op.N * op.OH * op.OW * op.C, "out");
-    }
-    case kKindMaxPool: {
-        if (!positive({op.N, op.H, op.W, op.C, op.OH, op.OW, op.KH, op.KW})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad maxpool extents", i);
-        if ((s = need(op.in0, (uint64_t)op.N * op.H * op.W * op.C, "in"))) return s;
-        return need(op.out, (uint64_t)op.N * op.OH * op.OW * op.C, "out");
-    }
-    case kKindAvgPool: {
-        if (!positive({op.N, op.H, op.W, op.C})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad avgpool extents", i);
-        if ((s = need(op.in0, (uint64_t)op.N * op.H * op.W * op.C, "in"))) return s;
-        return need(op.out, (uint64_t)op.N * op.C, "out");
-    }
-    case kKindAdd: {
-        if (!positive({op.C})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad add extent", i);
-        if ((s = need(op.in0, (uint64_t)op.C, "in1"))) return s;
-        if ((s = need(op.in1, (uint64_t)op.C, "in2"))) return s;
-        return need(op.out, (uint64_t)op.C, "out");
-    }
-    case kKindIm2colBf16: {
-        if (!positive({op.N, op.H, op.W, op.C, op.OH, op.OW, op.KH, op.KW, op.Kp}) || op.Kp < op.KH * op.KW * op.C) {
-            return fail(THIP_INVALID_ARGUMENT, "op %u: bad im2col extents", i);
-        }
-        if ((s = need(op.in0, (uint64_t)op.N * op.H * op.W * op.C * 2, "in"))) return s;
-        return need(op.out, (uint64_t)op.N * op.OH * op.OW * op.Kp * 2, "out");
-    }
-    case kKindDepthwiseBf16: {
-        if (!positive({op.N, op.H, op.W, op.C, op.OH, op.OW, op.KH, op.KW})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad depthwise extents", i);
-        if ((s = need(op.in0, (uint64_t)op.N * op.H * op.W * op.C * 2, "in"))) return s;
-        if ((s = need(op.weights, (uint64_t)op.KH * op.KW * op.C * 2, "weights"))) return s;
-        if ((s = need(op.bias, (uint64_t)op.C * 4, "bias"))) return s;
-        return need(op.out, (uint64_t)op.N * op.OH * op.OW * op.C * 2, "out");
-    }
-    case kKindAvgPoolBf16: {
-        if (!positive({op.N, op.H, op.W, op.C})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad avgpool extents", i);
-        if ((s = need(op.in0, (uint64_t)op.N * op.H * op.W * op.C * 2, "in"))) return s;
-        return need(op.out, (uint64_t)op.N * op.C * 2, "out");
-    }
-    case kKindExpandWeights: {
-        const int32_t block = (int32_t)op.gran;
-        if (!positive({op.K, op.Nn, block}) || op.K % block != 0 || op.Np < op.Nn) return fail(THIP_INVALID_ARGUMENT, "op %u: bad expand_weights extents", i);
-        if ((s = need(op.in0, (uint64_t)op.K * op.Nn, "weights"))) return s;
-        if ((s = need(op.scale, (uint64_t)(op.K / block) * op.Nn * 2, "scale"))) return s;
-        if ((s = need(op.bias, (uint64_t)(op.K / block) * op.Np * 4, "bias"))) return s;
-        return need(op.out, (uint64_t)op.K * op.Nn * 2, "out");
-    }
-    case kKindEltwise: {
-        const uint64_t inElem = op.gran, outElem = op.out_dtype == THIP_DTYPE_I8 ? 1 : op.out_dtype == THIP_DTYPE_I16 ? 2 : op.out_dtype == THIP_DTYPE_I32 ? 4 : 0;
-        if (!positive({op.C}) || !(inElem == 1 || inElem == 2 || inElem == 4) || outElem == 0 || op.variant > kEltMax || op.w1 < 0 || op.w1 > 2 ||
-            (op.variant != kEltMul && op.w1 != 0)) {
-            return fail(THIP_INVALID_ARGUMENT, "op %u: bad elementwise record", i);
-        }
-        if ((s = need(op.in0, (op.w1 == 1 ? 1 : (uint64_t)op.C) * inElem, "in1"))) return s;
-        if ((op.variant == kEltMul || op.variant >= kEltAnd) && (s = need(op.in1, (op.w1 == 2 ? 1 : (uint64_t)op.C) * inElem, "in2"))) return s;
-        return need(op.out, (uint64_t)op.C * outElem, "out");
-    }
-    case kKindAddBf16: {
-        if (!positive({op.C})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad add extent", i);
-        if ((s = need(op.in0, (uint64_t)op.C * 2, "in1"))) return s;
-        if ((s = need(op.in1, (uint64_t)op.C * 2, "in2"))) return s;
-        return need(op.out, (uint64_t)op.C * 2, "out");
-    }
-    case kKindFcBf16: {
-        if (!positive({op.M, op.K, op.Nn}) || op.K % 8 != 0) return fail(THIP_INVALID_ARGUMENT, "op %u: bad bf16 fully_connected extents", i);
-        if ((s = need(op.in0, (uint64_t)op.M * op.K * 2, "in"))) return s;
-        if (op.loader > 2) return fail(THIP_INVALID_ARGUMENT, "op %u: unknown bf16 weight layout %u", i, op.loader);
-        const uint64_t padded = (uint64_t)((op.Nn + 31) / 32 * 32) * ((op.K + 63) / 64 * 64);
-        const uint64_t wBytes = op.loader == 2 ? padded : op.loader == 1 ? padded * 2 : (uint64_t)op.Nn * op.K * 2;
-        if ((s = need(op.weights, wBytes, "weights"))) return s;
-        if (op.loader == 2) {
-            const int32_t block = (int32_t)op.gran;
-            if (block < 32 || block % 32 != 0 || op.K % block != 0 || op.Np < (op.Nn + 31) / 32 * 32 || op.Np % 32 != 0) {
-                return fail(THIP_INVALID_ARGUMENT, "op %u: bad block-quantized weight tables", i);
-            }
-            if ((s = need(op.scale, (uint64_t)(op.K / block) * op.Np * 2, "block scales"))) return s;
-            if ((s = need(op.table, (uint64_t)(op.K / block) * op.Np * 4, "block biases"))) return s;
-        }
-        if ((s = need(op.bias, (uint64_t)op.Nn * 4, "bias"))) return s;
-        if (op.w0 > 1) {
-            // K split over blocks: counters and partial sums live in an intermediate (zero-filled at creation)
-            if (op.w0 > 64 || op.in1.space != kSpaceTemp) return fail(THIP_INVALID_ARGUMENT, "op %u: bad split-K workspace", i);
-            if ((s = need(op.in1, fcBf16WorkspaceBytes(op.M, op.Nn, op.w0), "workspace"))) return s;
-        }
-        return need(op.out, (uint64_t)op.M * op.Nn * 2, "out");
-    }
-    default: return fail(THIP_INVALID_ARGUMENT, "op %u has unknown kind %u", i, op.kind);
-    }
-}
 
 // The kernel family of a record (error messages before the launcher has named the instantiation).
 static const char *opKernelName(const DescOp &op) {
@@ -568,6 +317,123 @@ static thip_status_t checkState(const thip_executable_t *e, const thip_dispatch_
     return THIP_OK;
 }
 
+// Waits for everything enqueued on the executable's stream, at most waitTimeoutMs.  On expiry the executable is
+// marked abandoned (kernels may still be running on its buffers: later calls are refused and destruction does not
+// free them) and THIP_INTERNAL comes back; the process goes on and can report the failure.
+static thip_status_t waitBounded(thip_executable_t *e, const char *what) {
+    if (e->waitTimeoutMs <= 0) {
+        THIP_HIP(hipStreamSynchronize(e->stream), what);
+        return THIP_OK;
+    }
+    THIP_HIP(hipEventRecord(e->evDone, e->stream), "hipEventRecord");
+    const auto start = std::chrono::steady_clock::now();
+    const auto deadline = start + std::chrono::milliseconds(e->waitTimeoutMs);
+    for (;;) {
+        const hipError_t q = hipEventQuery(e->evDone);
+        if (q == hipSuccess) return THIP_OK;
+        if (q != hipErrorNotReady) return hipFail(q, what);
+        (void)hipGetLastError();  // not-ready is no error
+        const auto now = std::chrono::steady_clock::now();
+        if (now >= deadline) {
+            e->abandoned = true;
+            return fail(THIP_INTERNAL, "%s: the GPU did not finish within %lld ms; the executable is abandoned", what, (long long)e->waitTimeoutMs);
+        }
+        // poll hard at first (dispatches are microseconds long), then back off
+        if (now - start > std::chrono::microseconds(500)) std::this_thread::sleep_for(std::chrono::microseconds(50));
+    }
+}
+
+static bool makeDirs(const std::string &path) {
+    for (size_t i = 1; i <= path.size(); i++) {
+        if (i == path.size() || path[i] == '/') {
+            const std::string part = path.substr(0, i);
+            if (mkdir(part.c_str(), 0777) != 0 && errno != EEXIST) return false;
+        }
+    }
+    return true;
+}
+
+static const char *kDispatchName = "thip_dispatch";  // the executable name in file paths and in the event log
+
+// Raw bytes of a binding, named as the reference names them (runtime/driver/TorqDump.cc:329-339):
+// <dir>/<executable>/npu.{in,out}.host_binding.<i>.torq_binding.<i>.bin
+static void dumpBinding(const thip_device_t *d, uint32_t binding, const void *host, size_t size, bool isInput) {
+    if (d->dumpIoDir.empty()) return;
+    const std::string dir = d->dumpIoDir + "/" + kDispatchName;
+    if (!makeDirs(dir)) return;
+    const std::string n = std::to_string(binding);
+    const std::string path = dir + "/npu" + (isInput ? ".in" : ".out") + ".host_binding." + n + ".torq_binding." + n + ".bin";
+    if (FILE *f = fopen(path.c_str(), "wb")) {
+        fwrite(host, 1, size, f);
+        fclose(f);
+    }
+}
+
+// What record i wrote, as a NumPy array file <dir>/<executable>/action<i>/buffer<id>.npy (the reference writes one
+// .npy per live buffer per action, runtime/driver/TorqDump.cc:341-428), id = "binding<k>" or "temp<k>", plus one
+// line of <dir>/<executable>/buffers.csv in the reference's columns.  The record's kernels must have finished.
+static thip_status_t dumpOpOutput(thip_executable_t *e, uint32_t i, uint8_t *const *bp) {
+    const thip_device_t *d = e->device;
+    const DescOp &op = e->ops[i];
+    std::vector<int64_t> shape;
+    const char *descr = "|i1", *typeName = "i8";
+    size_t elem = 1;
+    auto outType = [&]() {
+        if (op.out_dtype == THIP_DTYPE_I32) { descr = "<i4"; typeName = "i32"; elem = 4; }
+        else if (op.out_dtype == THIP_DTYPE_I16) { descr = "<i2"; typeName = "i16"; elem = 2; }
+    };
+    auto bf16 = [&]() { descr = "<u2"; typeName = "bf16"; elem = 2; };  // bf16 bit patterns, as uint16
+    switch (op.kind) {
+    case kKindTranspose: shape = {op.TB, op.TS, op.TP ? op.TP : op.TR}; if (op.gran == 2) bf16(); break;
+    case kKindIgemm: case kKindFcSkinny: shape = {op.M, op.Nn}; outType(); break;
+    case kKindDepthwise: case kKindMaxPool: shape = {op.N, op.OH, op.OW, op.C}; break;
+    case kKindAvgPool: shape = {op.N, op.C}; break;
+    case kKindAdd: shape = {op.C}; break;
+    case kKindEltwise: shape = {op.C}; outType(); break;
+    case kKindFcBf16: shape = {op.M, op.Nn}; bf16(); break;
+    case kKindAddBf16: shape = {op.C}; bf16(); break;
+    case kKindIm2colBf16: shape = {op.N, op.OH, op.OW, op.Kp}; bf16(); break;
+    case kKindDepthwiseBf16: shape = {op.N, op.OH, op.OW, op.C}; bf16(); break;
+    case kKindAvgPoolBf16: shape = {op.N, op.C}; bf16(); break;
+    case kKindExpandWeights: shape = {op.K, op.Nn}; bf16(); break;
+    default: return THIP_OK;
+    }
+    size_t count = 1;
+    for (int64_t v : shape) count *= (size_t)v;
+    if (count == 0 || op.out.space == kSpaceNone) return THIP_OK;  // e.g. a convolution whose result only feeds its fused add
+    std::vector<uint8_t> host(count * elem);
+    THIP_HIP(hipMemcpy(host.data(), resolve(e, op.out, bp), host.size(), hipMemcpyDeviceToHost), "reading a buffer back for the dump");
+    const std::string base = d->dumpBuffersDir + "/" + kDispatchName, dir = base + "/action" + std::to_string(i);
+    if (!makeDirs(dir)) return fail(THIP_INVALID_ARGUMENT, "cannot create dump directory %s", dir.c_str());
+    const std::string id = (op.out.space == kSpaceBinding ? "binding" : "temp") + std::to_string(op.out.index);
+    std::string dims, dimsX;
+    for (size_t k = 0; k < shape.size(); k++) {
+        dims += std::to_string(shape[k]) + ",";
+        dimsX += std::to_string(shape[k]) + "x";
+    }
+    std::string header = std::string("{'descr': '") + descr + "', 'fortran_order': False, 'shape': (" + dims + "), }";
+    while ((10 + header.size() + 1) % 64 != 0) header += ' ';
+    header += '\n';
+    FILE *f = fopen((dir + "/buffer" + id + ".npy").c_str(), "wb");
+    if (!f) return fail(THIP_INVALID_ARGUMENT, "cannot write into dump directory %s", dir.c_str());
+    const uint8_t magic[10] = {0x93, 'N', 'U', 'M', 'P', 'Y', 1, 0, (uint8_t)(header.size() & 0xff), (uint8_t)(header.size() >> 8)};
+    fwrite(magic, 1, sizeof(magic), f);
+    fwrite(header.data(), 1, header.size(), f);
+    fwrite(host.data(), 1, host.size(), f);
+    fclose(f);
+    // index of the buffers, one line per record output; started afresh by the first record of every dispatch
+    if (FILE *csv = fopen((base + "/buffers.csv").c_str(), i == 0 ? "w" : "a")) {
+        if (i == 0) {
+            fprintf(csv, "id;type;shape;strides;address;size;allocation_action;last_use_action;deallocation_action;"
+                         "allocation_location;last_use_location;deallocation_location\n");
+        }
+        fprintf(csv, "%s;%s;%s%s;;%llu;%zu;%u;%u;%u;%s;;\n", id.c_str(), op.out.space == kSpaceBinding ? "BINDING" : "INTERMEDIATE", dimsX.c_str(),
+                typeName, (unsigned long long)op.out.offset, host.size(), i, i, e->header.op_count - 1, e->kernelNames[i].c_str());
+        fclose(csv);
+    }
+    return THIP_OK;
+}
+
 // Enqueues every kernel record of the program.  `bp` holds one device pointer per binding.
 static thip_status_t enqueueOps(thip_executable_t *e, uint8_t *const *bp) {
     for (uint32_t i = 0; i < e->header.op_count; i++) {
@@ -575,6 +441,11 @@ static thip_status_t enqueueOps(thip_executable_t *e, uint8_t *const *bp) {
         logEvent(e->device, e->invocation, (int32_t)i, "NSS_START", "BEGIN", e->kernelNames[i].c_str());
         if (thip_status_t s = launchOp(e, i, bp, LaunchCtx{e->stream, &e->tuning, nullptr, 0})) return s;
         logEvent(e->device, e->invocation, (int32_t)i, "NSS_START", "END", e->kernelNames[i].c_str());
+        if (!e->device->dumpBuffersDir.empty()) {
+            // buffer dumps: each record runs to its end and what it wrote is read back before the next one starts
+            if (thip_status_t s = waitBounded(e, "waiting for a record before its dump")) return s;
+            if (thip_status_t s = dumpOpOutput(e, i, bp)) return s;
+        }
     }
     return THIP_OK;
 }
@@ -592,7 +463,7 @@ static void dropGraph(thip_executable_t *e) {
 // Enqueues one dispatch on device bindings, through the graph when there is one.
 static thip_status_t enqueueDevice(thip_executable_t *e, uint8_t *const *bp) {
     const uint32_t nb = e->header.binding_count;
-    const bool eligible = !e->graphsDisabled && e->header.op_count >= kGraphMinOps && !e->device->eventLog;
+    const bool eligible = !e->graphsDisabled && e->header.op_count >= kGraphMinOps && !e->device->eventLog && e->device->dumpBuffersDir.empty();
     if (!eligible) return enqueueOps(e, bp);
     std::vector<uint8_t *> key(bp, bp + nb);
     if (e->graphExec && key == e->graphPtrs) {
@@ -723,18 +594,34 @@ thip_status_t thip_device_set_event_log(thip_device_t *device, const char *csv_p
     return THIP_OK;
 }
 
-thip_status_t thip_infer_format(const void *blob, size_t size, size_t format_capacity, char *format, size_t *out_inferred_size) {
-    DescHeader h;
-    if (thip_status_t s = validateDescriptor((const uint8_t *)blob, size, &h)) return s;
-    static const char kFormat[] = "thip-gfx950";
-    if (!format || format_capacity < sizeof(kFormat)) return fail(THIP_OUT_OF_RANGE, "format buffer too small");
-    memcpy(format, kFormat, sizeof(kFormat));
-    if (out_inferred_size) *out_inferred_size = (size_t)h.total_size;
+thip_status_t thip_device_set_dump_dirs(thip_device_t *device, const char *io_data_dir, const char *buffers_dir) {
+    if (!device) return fail(THIP_INVALID_ARGUMENT, "null device");
+    const std::string io = io_data_dir ? io_data_dir : "", buffers = buffers_dir ? buffers_dir : "";
+    for (const std::string *dir : {&io, &buffers}) {
+        if (!dir->empty() && !makeDirs(*dir)) return fail(THIP_INVALID_ARGUMENT, "cannot create dump directory %s", dir->c_str());
+    }
+    device->dumpIoDir = io;
+    device->dumpBuffersDir = buffers;
+    return THIP_OK;
+}
+
+thip_status_t thip_executable_set_wait_timeout(thip_executable_t *e, int64_t milliseconds) {
+    if (!e) return fail(THIP_INVALID_ARGUMENT, "null executable");
+    std::lock_guard<std::mutex> lock(e->mutex);
+    e->waitTimeoutMs = milliseconds;
     return THIP_OK;
 }
 
 void thip_executable_destroy(thip_executable_t *e) {
     if (!e) return;
+    if (e->abandoned) {
+        // a wait on this executable timed out.  If its work has finished since, clean up as usual; if not, kernels may
+        // still be using its buffers: leave everything in place (the caller is expected to end the process)
+        if (!e->stream || hipStreamQuery(e->stream) != hipSuccess) {
+            (void)hipGetLastError();
+            return;
+        }
+    }
     if (e->stream) (void)hipStreamSynchronize(e->stream);
     dropGraph(e);
     for (uint8_t *p : e->tempPtrs) {
@@ -746,6 +633,7 @@ void thip_executable_destroy(thip_executable_t *e) {
     if (e->constData) (void)hipFree(e->constData);
     if (e->evStart) (void)hipEventDestroy(e->evStart);
     if (e->evStop) (void)hipEventDestroy(e->evStop);
+    if (e->evDone) (void)hipEventDestroy(e->evDone);
     if (e->stream) (void)hipStreamDestroy(e->stream);
     delete e;
 }
@@ -769,7 +657,10 @@ thip_status_t thip_executable_create(thip_device_t *device, const void *blob, si
     e->temps = (const DescTemp *)(e->blob.data() + h.temps_offset);
     e->consts = (const DescConst *)(e->blob.data() + h.consts_offset);
     thip_status_t s = THIP_OK;
-    for (uint32_t i = 0; i < h.op_count && s == THIP_OK; i++) s = checkOpFootprint(e, i);
+    {
+        const DescriptorView view{e->blob.data(), h, e->ops, e->bindings, e->temps, e->consts};
+        for (uint32_t i = 0; i < h.op_count && s == THIP_OK; i++) s = checkOpFootprint(&view, i);
+    }
     auto bail = [&](thip_status_t code) {
         thip_executable_destroy(e);
         return code;
@@ -779,6 +670,7 @@ thip_status_t thip_executable_create(thip_device_t *device, const void *blob, si
     if (err == hipSuccess) err = hipStreamCreate(&e->stream);  // default priority
     if (err == hipSuccess) err = hipEventCreate(&e->evStart);
     if (err == hipSuccess) err = hipEventCreate(&e->evStop);
+    if (err == hipSuccess) err = hipEventCreateWithFlags(&e->evDone, hipEventDisableTiming);
     if (err != hipSuccess) return bail(hipFail(err, "creating the stream"));
     const uint64_t dataSize = h.total_size - h.data_offset;
     if (dataSize) {
@@ -796,6 +688,7 @@ thip_status_t thip_executable_create(thip_device_t *device, const void *blob, si
     }
     e->staging.assign(h.binding_count, nullptr);
     e->graphsDisabled = getenv("THIP_NO_GRAPH") != nullptr;
+    if (const char *t = getenv("THIP_WAIT_TIMEOUT_MS")) e->waitTimeoutMs = atoll(t);
     // Which kernel each record runs is settled now, from the record, the alignment of its operands and the
     // environment's switches, and kept: the launchers are asked in naming mode (they also configure their kernels,
     // which must not happen later inside a stream capture).  Bindings stand in as aligned placeholder addresses:
@@ -824,7 +717,13 @@ thip_status_t thip_executable_create(thip_device_t *device, const void *blob, si
     return THIP_OK;
 }
 
+static thip_status_t refuseAbandoned(const thip_executable_t *e) {
+    if (!e->abandoned) return THIP_OK;
+    return fail(THIP_FAILED_PRECONDITION, "an earlier wait on this executable timed out; it cannot be used any more");
+}
+
 static thip_status_t runLocked(thip_executable_t *e, const thip_dispatch_state_t *st) {
+    if (thip_status_t s = refuseAbandoned(e)) return s;
     THIP_HIP(hipSetDevice(e->device->ordinal), "hipSetDevice");
     uint8_t *bp[64] = {nullptr};
     const int32_t lastOp = (int32_t)e->header.op_count - 1;
@@ -843,6 +742,7 @@ static thip_status_t runLocked(thip_executable_t *e, const thip_dispatch_state_t
         }
         bp[i] = e->staging[i];
         if (e->bindings[i].flags & kBindingRead) {
+            dumpBinding(e->device, i, st->binding_ptrs[i], e->bindings[i].size, true);
             THIP_HIP(hipMemcpyAsync(bp[i], st->binding_ptrs[i], e->bindings[i].size, hipMemcpyHostToDevice, e->stream), "staging a binding");
         }
     }
@@ -853,9 +753,11 @@ static thip_status_t runLocked(thip_executable_t *e, const thip_dispatch_state_t
     }
     logEvent(e->device, e->invocation, 0, "DISPATCH_EXECUTE_ACTIONS", "BEGIN", "");
     if (thip_status_t s = allDevice ? enqueueDevice(e, bp) : enqueueOps(e, bp)) {
-        (void)hipStreamSynchronize(e->stream);
+        // what was enqueued before the failure still runs: wait for it (bounded; the launch error is what is reported)
+        std::string message = thip_status_message();
+        if (!e->abandoned) (void)waitBounded(e, "waiting after a failed launch");
         e->invocation++;
-        return s;
+        return fail(s, "%s", message.c_str());
     }
     logEvent(e->device, e->invocation, lastOp, "DISPATCH_EXECUTE_ACTIONS", "END", "");
     logEvent(e->device, e->invocation, lastOp, "DISPATCH_SYNC_BINDINGS_OUT", "BEGIN", "");
@@ -866,12 +768,17 @@ static thip_status_t runLocked(thip_executable_t *e, const thip_dispatch_state_t
         THIP_HIP(hipMemcpyAsync(st->binding_ptrs[i], bp[i], e->bindings[i].size, hipMemcpyDeviceToHost, e->stream), "reading back a binding");
     }
     logEvent(e->device, e->invocation, lastOp, "NSS_WAIT", "BEGIN", "");
-    const hipError_t waited = hipStreamSynchronize(e->stream);
+    const thip_status_t waited = waitBounded(e, "waiting for the dispatch");
+    const std::string waitMessage = waited == THIP_OK ? std::string() : std::string(thip_status_message());
     logEvent(e->device, e->invocation, lastOp, "NSS_WAIT", "END", "");
     logEvent(e->device, e->invocation, lastOp, "DISPATCH_SYNC_BINDINGS_OUT", "END", "");
     logEvent(e->device, e->invocation, lastOp, "DISPATCH", "END", "");
     e->invocation++;
-    THIP_HIP(waited, "waiting for the dispatch");
+    if (waited != THIP_OK) return fail(waited, "%s", waitMessage.c_str());
+    for (uint32_t i = 0; i < e->header.binding_count; i++) {
+        const bool isDevice = st->binding_flags && (st->binding_flags[i] & THIP_BINDING_DEVICE);
+        if (!isDevice && (e->bindings[i].flags & kBindingWritten)) dumpBinding(e->device, i, st->binding_ptrs[i], e->bindings[i].size, false);
+    }
     return THIP_OK;
 }
 
@@ -886,6 +793,7 @@ thip_status_t thip_executable_enqueue(thip_executable_t *e, const thip_dispatch_
     if (!e) return fail(THIP_INVALID_ARGUMENT, "null executable");
     if (thip_status_t s = checkState(e, st, true)) return s;
     std::lock_guard<std::mutex> lock(e->mutex);
+    if (thip_status_t s = refuseAbandoned(e)) return s;
     THIP_HIP(hipSetDevice(e->device->ordinal), "hipSetDevice");
     uint8_t *bp[64] = {nullptr};
     for (uint32_t i = 0; i < e->header.binding_count; i++) bp[i] = (uint8_t *)st->binding_ptrs[i];
@@ -902,6 +810,7 @@ thip_status_t thip_executable_enqueue_noalloc(thip_executable_t *e, const thip_d
                     (unsigned long long)e->scratchBytes, (unsigned long long)kStaticScratchBytes);
     }
     std::lock_guard<std::mutex> lock(e->mutex);
+    if (thip_status_t s = refuseAbandoned(e)) return s;
     THIP_HIP(hipSetDevice(e->device->ordinal), "hipSetDevice");
     uint8_t *scratch = e->device->staticScratch;  // the address hipGetSymbolAddress gave for this device
     if (!scratch) return fail(THIP_INTERNAL, "the static scratch array was not located");
@@ -923,8 +832,9 @@ thip_status_t thip_executable_enqueue_noalloc(thip_executable_t *e, const thip_d
 
 thip_status_t thip_executable_wait(thip_executable_t *e) {
     if (!e) return fail(THIP_INVALID_ARGUMENT, "null executable");
-    THIP_HIP(hipStreamSynchronize(e->stream), "waiting for the dispatch");
-    return THIP_OK;
+    std::lock_guard<std::mutex> lock(e->mutex);
+    if (thip_status_t s = refuseAbandoned(e)) return s;
+    return waitBounded(e, "waiting for the dispatch");
 }
 
 thip_status_t thip_executable_time(thip_executable_t *e, const thip_dispatch_state_t *st, int32_t iterations, float *out_ms) {
@@ -932,6 +842,7 @@ thip_status_t thip_executable_time(thip_executable_t *e, const thip_dispatch_sta
     if (iterations <= 0) return fail(THIP_INVALID_ARGUMENT, "iterations must be positive");
     if (thip_status_t s = checkState(e, st, true)) return s;
     std::lock_guard<std::mutex> lock(e->mutex);
+    if (thip_status_t as = refuseAbandoned(e)) return as;
     THIP_HIP(hipSetDevice(e->device->ordinal), "hipSetDevice");
     uint8_t *bp[64] = {nullptr};
     for (uint32_t i = 0; i < e->header.binding_count; i++) bp[i] = (uint8_t *)st->binding_ptrs[i];
@@ -945,7 +856,7 @@ thip_status_t thip_executable_time(thip_executable_t *e, const thip_dispatch_sta
         }
     }
     THIP_HIP(hipEventRecord(e->evStop, e->stream), "hipEventRecord");
-    THIP_HIP(hipEventSynchronize(e->evStop), "hipEventSynchronize");
+    if (thip_status_t ws = waitBounded(e, "waiting for the timed dispatches")) return ws;
     float ms = 0.f;
     THIP_HIP(hipEventElapsedTime(&ms, e->evStart, e->evStop), "hipEventElapsedTime");
     *out_ms = ms / (float)iterations;
@@ -960,6 +871,7 @@ thip_status_t thip_executable_time_rotating(thip_executable_t *e, const thip_dis
         if (thip_status_t st = checkState(e, &states[s], true)) return st;
     }
     std::lock_guard<std::mutex> lock(e->mutex);
+    if (thip_status_t as = refuseAbandoned(e)) return as;
     THIP_HIP(hipSetDevice(e->device->ordinal), "hipSetDevice");
     THIP_HIP(hipEventRecord(e->evStart, e->stream), "hipEventRecord");
     for (int32_t it = 0; it < iterations; it++) {
@@ -974,7 +886,7 @@ thip_status_t thip_executable_time_rotating(thip_executable_t *e, const thip_dis
         }
     }
     THIP_HIP(hipEventRecord(e->evStop, e->stream), "hipEventRecord");
-    THIP_HIP(hipEventSynchronize(e->evStop), "hipEventSynchronize");
+    if (thip_status_t ws = waitBounded(e, "waiting for the timed dispatches")) return ws;
     float ms = 0.f;
     THIP_HIP(hipEventElapsedTime(&ms, e->evStart, e->evStop), "hipEventElapsedTime");
     *out_ms = ms / (float)iterations;

@@ -1415,27 +1415,6 @@ static hipError_t launchIgemmStream(const IgemmArgs &a, const LaunchCtx &ctx) {
     return launchIgemmStreamT<8, kLoaderDense>(a, smem, ctx);
 }
 
-static const IgemmTile kTiles[kIgemmVariantCount] = {
-    {128, 128, 64, "igemm_i8_128x128x64"},
-    {256, 256, 64, "igemm_i8_256x256x64"},
-    {64, 64, 64, "igemm_i8_64x64x64"},
-    {256, 128, 64, "igemm_i8_256x128x64"},
-    {256, 256, 64, "igemm_dense_i8_256x256x64"},
-    {128, 128, 64, "igemm_dense_i8_128x128x64"},
-    {128, 256, 64, "igemm_dense_i8_128x256x64"},
-    {64, 64, 64, "igemm_dense_i8_64x64x64"},
-    {256, 128, 64, "igemm_dense_i8_256x128x64"},
-    {256, 64, 64, "igemm_dense_i8_256x64x64"},
-    {256, 32, 64, "igemm_dense_i8_256x32x64"},
-    {32, 32, 32, "igemm_stream_i8"},
-    {128, 64, 64, "igemm_dense_i8_128x64x64"},
-    {64, 128, 64, "igemm_dense_i8_64x128x64"},
-};
-
-const IgemmTile &igemmTile(uint32_t variant) {
-    return kTiles[variant < kIgemmVariantCount ? variant : 0];
-}
-
 template <int BM, int BN, int BK, int LOADER, int G>
 static hipError_t launchIgemmTile(const IgemmArgs &a, const LaunchCtx &ctx) {
     constexpr int LDK = BK + 16;
@@ -1513,7 +1492,7 @@ static hipError_t launchIgemmDense(const IgemmArgs &a, const LaunchCtx &ctx) {
 
 hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, const LaunchCtx &ctx) {
     if (variant >= kIgemmVariantCount) return hipErrorInvalidValue;
-    const IgemmTile &t = kTiles[variant];
+    const IgemmTile &t = igemmTile(variant);
     // What the kernel assumes: padded sizes are whole tiles, the real sizes fit
     // inside them, the dense loader reads whole 16-byte chunks of each row.
     if (a.M <= 0 || a.N <= 0 || a.K <= 0) return hipErrorInvalidValue;

@@ -1,0 +1,344 @@
+// Validation of a dispatch descriptor: everything that can be checked without a GPU.  The driver runs it when an
+// executable is created (and thip_infer_format / thip_descriptor_validate on their own); nothing here calls HIP, so
+// the same code is fuzzed on the host under sanitizers.
+#include "thip_validate.h"
+
+#include <string.h>
+
+#include <initializer_list>
+
+#include "thip_kernels.h"
+#include "thip_status.h"
+
+namespace thip {
+
+// Tile geometry of the igemm variants (what the emitter pads to and the launchers launch).
+static const IgemmTile kTiles[kIgemmVariantCount] = {
+    {128, 128, 64, "igemm_i8_128x128x64"},
+    {256, 256, 64, "igemm_i8_256x256x64"},
+    {64, 64, 64, "igemm_i8_64x64x64"},
+    {256, 128, 64, "igemm_i8_256x128x64"},
+    {256, 256, 64, "igemm_dense_i8_256x256x64"},
+    {128, 128, 64, "igemm_dense_i8_128x128x64"},
+    {128, 256, 64, "igemm_dense_i8_128x256x64"},
+    {64, 64, 64, "igemm_dense_i8_64x64x64"},
+    {256, 128, 64, "igemm_dense_i8_256x128x64"},
+    {256, 64, 64, "igemm_dense_i8_256x64x64"},
+    {256, 32, 64, "igemm_dense_i8_256x32x64"},
+    {32, 32, 32, "igemm_stream_i8"},
+    {128, 64, 64, "igemm_dense_i8_128x64x64"},
+    {64, 128, 64, "igemm_dense_i8_64x128x64"},
+};
+
+const IgemmTile &igemmTile(uint32_t variant) {
+    return kTiles[variant < kIgemmVariantCount ? variant : 0];
+}
+
+// Product of non-negative extents, saturating (a corrupt record must not wrap around to a small number).
+template <typename... T>
+static uint64_t mul(T... factors) {
+    unsigned __int128 p = 1;
+    for (int64_t f : {(int64_t)factors...}) {
+        if (f < 0) return ~0ull >> 8;
+        p *= (uint64_t)f;
+        if (p > (~0ull >> 8)) return ~0ull >> 8;
+    }
+    return (uint64_t)p;
+}
+
+thip_status_t validateDescriptor(const uint8_t *p, size_t size, DescHeader *out) {
+    if (!p || size < sizeof(DescHeader)) return fail(THIP_INVALID_ARGUMENT, "descriptor is smaller than its header");
+    DescHeader h;
+    memcpy(&h, p, sizeof(h));
+    if (h.magic != kMagic) return fail(THIP_INVALID_ARGUMENT, "descriptor magic 0x%08x is not THIP", h.magic);
+    // same gate as `runtime_version != 2 -> UNAVAILABLE`, runtime/driver/TorqExecutable.cc:663-667
+    if (h.version != kDescriptorVersion) {
+        return fail(THIP_UNAVAILABLE, "descriptor version %u, this runtime reads version %u", h.version, kDescriptorVersion);
+    }
+    // same gate as isHwCompatible(hwId), runtime/driver/TorqExecutable.cc:701-705
+    if (h.arch != kArchGfx950) return fail(THIP_UNAVAILABLE, "descriptor targets arch %u, this runtime drives gfx950", h.arch);
+    if (h.total_size > size) return fail(THIP_INVALID_ARGUMENT, "descriptor says %llu bytes, %zu given", (unsigned long long)h.total_size, size);
+    auto inside = [&](uint64_t off, uint64_t count, uint64_t each) {
+        return off <= h.total_size && count * each <= h.total_size - off;
+    };
+    if (!inside(h.ops_offset, h.op_count, sizeof(DescOp)) || !inside(h.bindings_offset, h.binding_count, sizeof(DescBinding)) ||
+        !inside(h.temps_offset, h.temp_count, sizeof(DescTemp)) || !inside(h.consts_offset, h.const_count, sizeof(DescConst)) ||
+        h.data_offset > h.total_size) {
+        return fail(THIP_INVALID_ARGUMENT, "descriptor tables run past its end");
+    }
+    if ((h.ops_offset | h.bindings_offset | h.temps_offset | h.consts_offset) & 7) return fail(THIP_INVALID_ARGUMENT, "descriptor tables are misaligned");
+    if (((uintptr_t)p & 7) != 0) return fail(THIP_INVALID_ARGUMENT, "descriptor must be 8-byte aligned in memory");
+    if (h.op_count == 0) return fail(THIP_INVALID_ARGUMENT, "descriptor holds no ops");
+    if (h.binding_count > 64) return fail(THIP_INVALID_ARGUMENT, "descriptor declares %u bindings (max 64)", h.binding_count);
+    const DescConst *consts = (const DescConst *)(p + h.consts_offset);
+    for (uint32_t i = 0; i < h.const_count; i++) {
+        if (consts[i].offset > h.total_size - h.data_offset || consts[i].size > h.total_size - h.data_offset - consts[i].offset) {
+            return fail(THIP_INVALID_ARGUMENT, "constant segment %u runs past the descriptor", i);
+        }
+    }
+    // every operand reference must name an existing buffer and stay inside it
+    const DescOp *ops = (const DescOp *)(p + h.ops_offset);
+    const DescBinding *bindings = (const DescBinding *)(p + h.bindings_offset);
+    const DescTemp *temps = (const DescTemp *)(p + h.temps_offset);
+    for (uint32_t i = 0; i < h.op_count; i++) {
+        const DescRef *refs[] = {&ops[i].in0, &ops[i].in1, &ops[i].weights, &ops[i].bias, &ops[i].scale, &ops[i].table, &ops[i].out};
+        for (const DescRef *r : refs) {
+            uint64_t limit = 0;
+            switch (r->space) {
+            case kSpaceNone: continue;
+            case kSpaceBinding:
+                if (r->index >= h.binding_count) return fail(THIP_INVALID_ARGUMENT, "op %u names binding %u of %u", i, r->index, h.binding_count);
+                limit = bindings[r->index].size;
+                break;
+            case kSpaceTemp:
+                if (r->index >= h.temp_count) return fail(THIP_INVALID_ARGUMENT, "op %u names intermediate %u of %u", i, r->index, h.temp_count);
+                limit = temps[r->index].size;
+                break;
+            case kSpaceConst:
+                if (r->index >= h.const_count) return fail(THIP_INVALID_ARGUMENT, "op %u names constant %u of %u", i, r->index, h.const_count);
+                limit = consts[r->index].size;
+                break;
+            default: return fail(THIP_INVALID_ARGUMENT, "op %u has an operand in unknown space %u", i, r->space);
+            }
+            if (r->offset > limit) return fail(THIP_INVALID_ARGUMENT, "op %u operand offset %llu is past its buffer (%llu)", i, (unsigned long long)r->offset, (unsigned long long)limit);
+        }
+    }
+    *out = h;
+    return THIP_OK;
+}
+
+// Bytes an operand reference can still address.
+static uint64_t refRoom(const DescriptorView *e, const DescRef &r) {
+    switch (r.space) {
+    case kSpaceBinding: return e->bindings[r.index].size - r.offset;
+    case kSpaceTemp: return e->temps[r.index].size - r.offset;
+    case kSpaceConst: return e->consts[r.index].size - r.offset;
+    default: return 0;
+    }
+}
+
+// Checks, once at creation, that every kernel record stays inside the buffers it names.
+thip_status_t checkOpFootprint(const DescriptorView *e, uint32_t i) {
+    const DescOp &op = e->ops[i];
+    auto need = [&](const DescRef &r, uint64_t bytes, const char *name) -> thip_status_t {
+        if (r.space == kSpaceNone) return fail(THIP_INVALID_ARGUMENT, "op %u: operand %s is missing", i, name);
+        if (bytes >= (1ull << 48)) return fail(THIP_INVALID_ARGUMENT, "op %u: operand %s has an absurd extent", i, name);
+        if (refRoom(e, r) < bytes) {
+            return fail(THIP_INVALID_ARGUMENT, "op %u: operand %s needs %llu bytes, its buffer has %llu", i, name,
+                        (unsigned long long)bytes, (unsigned long long)refRoom(e, r));
+        }
+        return THIP_OK;
+    };
+    auto positive = [&](std::initializer_list<int32_t> vals) {
+        for (int32_t v : vals) {
+            if (v <= 0) return false;
+        }
+        return true;
+    };
+    const uint64_t outElem = op.out_dtype == THIP_DTYPE_I32 ? 4 : op.out_dtype == THIP_DTYPE_I16 ? 2 : 1;
+    thip_status_t s = THIP_OK;
+    if (op.shift < 0 || op.shift > 63) return fail(THIP_INVALID_ARGUMENT, "op %u: shift %d is outside 0..63", i, op.shift);
+    if (op.pre_shift != 0 && (op.pre_shift < 0 || op.pre_shift > 30 || (int64_t)op.shift + op.pre_shift != 33 || op.shift < 0 || op.shift > 63 ||
+                              (op.kind != kKindIgemm && op.kind != kKindDepthwise))) {
+        return fail(THIP_INVALID_ARGUMENT, "op %u: pre_shift %d does not complete shift %d to 33", i, op.pre_shift, op.shift);
+    }
+    if (op.t0_clamp != 0 && (op.t0_clamp < 0 || op.pre_shift <= 0 || op.pre_shift > 30 || op.t0_clamp >= (1 << (31 - op.pre_shift)))) {
+        return fail(THIP_INVALID_ARGUMENT, "op %u: t0_clamp %d does not fit pre_shift %d", i, op.t0_clamp, op.pre_shift);
+    }
+    switch (op.kind) {
+    case kKindTranspose: {
+        if (!positive({op.TB, op.TR, op.TS})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad transpose extents", i);
+        if (op.gran > 2) return fail(THIP_INVALID_ARGUMENT, "op %u: transpose element size %u", i, op.gran);
+        if (op.TP != 0 && op.TP < op.TR) return fail(THIP_INVALID_ARGUMENT, "op %u: transpose pitch %d is below its row length %d", i, op.TP, op.TR);
+        const uint64_t elem = op.gran == 2 ? 2 : 1, pitch = op.TP ? (uint64_t)op.TP : (uint64_t)op.TR;
+        if ((s = need(op.in0, mul(op.TB, op.TR, op.TS) * elem, "in"))) return s;
+        return need(op.out, mul(op.TB, op.TS) * pitch * elem, "out");
+    }
+    case kKindIgemm: {
+        if (!positive({op.M, op.K, op.Kp, op.Nn, op.Np, op.N, op.H, op.W, op.C, op.OH, op.OW})) {
+            return fail(THIP_INVALID_ARGUMENT, "op %u: bad igemm extents", i);
+        }
+        if (op.variant >= kIgemmVariantCount) return fail(THIP_INVALID_ARGUMENT, "op %u: unknown igemm variant %u", i, op.variant);
+        const uint64_t inBytes = op.loader == kLoaderDense ? mul(op.M, op.K) : mul(op.N, op.H, op.W, op.C);
+        if (op.loader != kLoaderDense && mul(op.N, op.OH, op.OW) != (uint64_t)op.M) {
+            return fail(THIP_INVALID_ARGUMENT, "op %u: igemm rows do not match the output pixels", i);
+        }
+        if (op.loader == kLoaderDense && mul(op.N, op.H, op.W, op.C) != mul(op.M, op.K)) {
+            return fail(THIP_INVALID_ARGUMENT, "op %u: the dense operand's image view is not its M x K matrix", i);
+        }
+        if ((s = need(op.in0, inBytes, "in"))) return s;
+        if ((s = need(op.weights, mul(op.Np, op.Kp), "weights"))) return s;
+        if ((s = need(op.bias, (uint64_t)op.Np * 4, "bias"))) return s;
+        if ((s = need(op.scale, (uint64_t)op.Np * 4, "scale"))) return s;
+        if (op.loader > kLoaderRuns) return fail(THIP_INVALID_ARGUMENT, "op %u: unknown igemm loader %u", i, op.loader);
+        if (op.loader == kLoaderRuns) {
+            if (!positive({op.KH, op.KW}) || (int64_t)op.KW * op.C > 16 || op.Kp % 16 != 0) return fail(THIP_INVALID_ARGUMENT, "op %u: a window row of %d x %d bytes does not fit a 16-byte run", i, op.KW, op.C);
+            if (op.table.space != kSpaceConst) return fail(THIP_INVALID_ARGUMENT, "op %u: table must be a constant", i);
+            if ((s = need(op.table, (uint64_t)op.Kp / 16 * 4, "table"))) return s;
+            const uint8_t *base = e->blob + e->header.data_offset + e->consts[op.table.index].offset + op.table.offset;
+            for (uint32_t t = 0; t < (uint32_t)op.Kp / 16; t++) {
+                uint32_t ent;
+                memcpy(&ent, base + 4ull * t, 4);
+                if (ent & kKEntryInvalid) continue;
+                if ((int)((ent >> 24) & 0x7f) >= op.KH || (int)(ent & 0xffff) != op.KW * op.C) return fail(THIP_INVALID_ARGUMENT, "op %u: run table entry %u is outside the window", i, t);
+            }
+        }
+        if (op.loader == kLoaderGather) {
+            if (op.gran == 0 || (op.gran & (op.gran - 1)) || op.gran > 16) return fail(THIP_INVALID_ARGUMENT, "op %u: bad gather granularity", i);
+            if (op.table.space != kSpaceConst) return fail(THIP_INVALID_ARGUMENT, "op %u: table must be a constant", i);
+            if ((s = need(op.table, (uint64_t)op.Kp / op.gran * 4, "table"))) return s;
+            // every valid table entry must stay inside the window and the channel axis
+            const uint8_t *base = e->blob + e->header.data_offset + e->consts[op.table.index].offset + op.table.offset;
+            for (uint32_t t = 0; t < (uint32_t)op.Kp / op.gran; t++) {
+                uint32_t ent;
+                memcpy(&ent, base + 4ull * t, 4);
+                if (ent & kKEntryInvalid) continue;
+                const int kh = (ent >> 24) & 0x7f, kw = (ent >> 16) & 0xff, ci = ent & 0xffff;
+                if (kh >= op.KH || kw >= op.KW || ci + (int)op.gran > op.C) return fail(THIP_INVALID_ARGUMENT, "op %u: table entry %u is outside the window", i, t);
+            }
+        }
+        if (op.in1.space != kSpaceNone) {  // fused residual add
+            if ((op.variant != kIgemmStream && op.variant != kIgemmDense64x64) || op.loader != kLoaderDense || op.out_dtype != THIP_DTYPE_I8 ||
+                op.table.space != kSpaceConst) {
+                return fail(THIP_INVALID_ARGUMENT, "op %u: a residual add needs the streaming or the small-tile int8 kernel", i);
+            }
+            if ((s = need(op.in1, mul(op.M, op.Nn), "residual"))) return s;
+            if ((s = need(op.table, sizeof(ResidualAddParams), "residual parameters"))) return s;
+            ResidualAddParams ap;
+            memcpy(&ap, e->blob + e->header.data_offset + e->consts[op.table.index].offset + op.table.offset, sizeof(ap));
+            if (ap.shift < 0 || ap.shift > 63 || ap.output_min > ap.output_max || ap.output_min < -128 || ap.output_max > 127) {
+                return fail(THIP_INVALID_ARGUMENT, "op %u: bad residual add parameters", i);
+            }
+        }
+        return need(op.out, mul(op.M, op.Nn) * outElem, "out");
+    }
+    case kKindFcSkinny: {
+        if (!positive({op.M, op.K, op.Nn})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad fc extents", i);
+        if ((s = need(op.in0, mul(op.M, op.K), "in"))) return s;
+        if ((s = need(op.weights, mul(op.Nn, op.K), "weights"))) return s;
+        if ((s = need(op.bias, (uint64_t)op.Nn * 4, "bias"))) return s;
+        if ((s = need(op.scale, (uint64_t)op.Nn * 4, "scale"))) return s;
+        return need(op.out, mul(op.M, op.Nn) * outElem, "out");
+    }
+    case kKindDepthwise: {
+        if (!positive({op.N, op.H, op.W, op.C, op.OH, op.OW, op.KH, op.KW})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad depthwise extents", i);
+        if ((s = need(op.in0, mul(op.N, op.H, op.W, op.C), "in"))) return s;
+        if (op.variant > kDepthwiseDot4Rows) return fail(THIP_INVALID_ARGUMENT, "op %u: unknown depthwise variant %u", i, op.variant);
+        if ((s = need(op.weights, op.variant == kDepthwiseDot4Rows ? mul(op.KH, op.C) * 4 : mul(op.KH, op.KW, op.C), "weights"))) return s;
+        if ((s = need(op.bias, (uint64_t)op.C * 4, "bias"))) return s;
+        if ((s = need(op.scale, (uint64_t)op.C * 4, "scale"))) return s;
+        return need(op.out, mul(op.N, op.OH, op.OW, op.C), "out");
+    }
+    case kKindMaxPool: {
+        if (!positive({op.N, op.H, op.W, op.C, op.OH, op.OW, op.KH, op.KW})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad maxpool extents", i);
+        if ((s = need(op.in0, mul(op.N, op.H, op.W, op.C), "in"))) return s;
+        return need(op.out, mul(op.N, op.OH, op.OW, op.C), "out");
+    }
+    case kKindAvgPool: {
+        if (!positive({op.N, op.H, op.W, op.C})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad avgpool extents", i);
+        if ((s = need(op.in0, mul(op.N, op.H, op.W, op.C), "in"))) return s;
+        return need(op.out, mul(op.N, op.C), "out");
+    }
+    case kKindAdd: {
+        if (!positive({op.C})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad add extent", i);
+        if ((s = need(op.in0, (uint64_t)op.C, "in1"))) return s;
+        if ((s = need(op.in1, (uint64_t)op.C, "in2"))) return s;
+        return need(op.out, (uint64_t)op.C, "out");
+    }
+    case kKindIm2colBf16: {
+        if (!positive({op.N, op.H, op.W, op.C, op.OH, op.OW, op.KH, op.KW, op.Kp}) || (uint64_t)op.Kp < mul(op.KH, op.KW, op.C)) {
+            return fail(THIP_INVALID_ARGUMENT, "op %u: bad im2col extents", i);
+        }
+        if ((s = need(op.in0, mul(op.N, op.H, op.W, op.C) * 2, "in"))) return s;
+        return need(op.out, mul(op.N, op.OH, op.OW, op.Kp) * 2, "out");
+    }
+    case kKindDepthwiseBf16: {
+        if (!positive({op.N, op.H, op.W, op.C, op.OH, op.OW, op.KH, op.KW})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad depthwise extents", i);
+        if ((s = need(op.in0, mul(op.N, op.H, op.W, op.C) * 2, "in"))) return s;
+        if ((s = need(op.weights, mul(op.KH, op.KW, op.C) * 2, "weights"))) return s;
+        if ((s = need(op.bias, (uint64_t)op.C * 4, "bias"))) return s;
+        return need(op.out, mul(op.N, op.OH, op.OW, op.C) * 2, "out");
+    }
+    case kKindAvgPoolBf16: {
+        if (!positive({op.N, op.H, op.W, op.C})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad avgpool extents", i);
+        if ((s = need(op.in0, mul(op.N, op.H, op.W, op.C) * 2, "in"))) return s;
+        return need(op.out, mul(op.N, op.C) * 2, "out");
+    }
+    case kKindExpandWeights: {
+        const int32_t block = (int32_t)op.gran;
+        if (!positive({op.K, op.Nn, block}) || op.K % block != 0 || op.Np < op.Nn) return fail(THIP_INVALID_ARGUMENT, "op %u: bad expand_weights extents", i);
+        if ((s = need(op.in0, mul(op.K, op.Nn), "weights"))) return s;
+        if ((s = need(op.scale, (uint64_t)(op.K / block) * op.Nn * 2, "scale"))) return s;
+        if ((s = need(op.bias, (uint64_t)(op.K / block) * op.Np * 4, "bias"))) return s;
+        return need(op.out, mul(op.K, op.Nn) * 2, "out");
+    }
+    case kKindEltwise: {
+        const uint64_t inElem = op.gran, outElem = op.out_dtype == THIP_DTYPE_I8 ? 1 : op.out_dtype == THIP_DTYPE_I16 ? 2 : op.out_dtype == THIP_DTYPE_I32 ? 4 : 0;
+        if (!positive({op.C}) || !(inElem == 1 || inElem == 2 || inElem == 4) || outElem == 0 || op.variant > kEltMax || op.w1 < 0 || op.w1 > 2 ||
+            (op.variant != kEltMul && op.w1 != 0)) {
+            return fail(THIP_INVALID_ARGUMENT, "op %u: bad elementwise record", i);
+        }
+        if ((s = need(op.in0, (op.w1 == 1 ? 1 : (uint64_t)op.C) * inElem, "in1"))) return s;
+        if ((op.variant == kEltMul || op.variant >= kEltAnd) && (s = need(op.in1, (op.w1 == 2 ? 1 : (uint64_t)op.C) * inElem, "in2"))) return s;
+        return need(op.out, (uint64_t)op.C * outElem, "out");
+    }
+    case kKindAddBf16: {
+        if (!positive({op.C})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad add extent", i);
+        if ((s = need(op.in0, (uint64_t)op.C * 2, "in1"))) return s;
+        if ((s = need(op.in1, (uint64_t)op.C * 2, "in2"))) return s;
+        return need(op.out, (uint64_t)op.C * 2, "out");
+    }
+    case kKindFcBf16: {
+        if (!positive({op.M, op.K, op.Nn}) || op.K % 8 != 0) return fail(THIP_INVALID_ARGUMENT, "op %u: bad bf16 fully_connected extents", i);
+        if ((s = need(op.in0, mul(op.M, op.K) * 2, "in"))) return s;
+        if (op.loader > 2) return fail(THIP_INVALID_ARGUMENT, "op %u: unknown bf16 weight layout %u", i, op.loader);
+        const uint64_t padded = (((uint64_t)op.Nn + 31) / 32 * 32) * (((uint64_t)op.K + 63) / 64 * 64);
+        const uint64_t wBytes = op.loader == 2 ? padded : op.loader == 1 ? padded * 2 : mul(op.Nn, op.K) * 2;
+        if ((s = need(op.weights, wBytes, "weights"))) return s;
+        if (op.loader == 2) {
+            const int32_t block = (int32_t)op.gran;
+            if (block < 32 || block % 32 != 0 || op.K % block != 0 || (int64_t)op.Np < ((int64_t)op.Nn + 31) / 32 * 32 || op.Np % 32 != 0) {
+                return fail(THIP_INVALID_ARGUMENT, "op %u: bad block-quantized weight tables", i);
+            }
+            if ((s = need(op.scale, (uint64_t)(op.K / block) * op.Np * 2, "block scales"))) return s;
+            if ((s = need(op.table, (uint64_t)(op.K / block) * op.Np * 4, "block biases"))) return s;
+        }
+        if ((s = need(op.bias, (uint64_t)op.Nn * 4, "bias"))) return s;
+        if (op.w0 > 1) {
+            // K split over blocks: counters and partial sums live in an intermediate (zero-filled at creation)
+            if (op.w0 > 64 || op.in1.space != kSpaceTemp) return fail(THIP_INVALID_ARGUMENT, "op %u: bad split-K workspace", i);
+            if ((s = need(op.in1, fcBf16WorkspaceBytes(op.M, op.Nn, op.w0), "workspace"))) return s;
+        }
+        return need(op.out, mul(op.M, op.Nn) * 2, "out");
+    }
+    default: return fail(THIP_INVALID_ARGUMENT, "op %u has unknown kind %u", i, op.kind);
+    }
+}
+
+thip_status_t validateWhole(const uint8_t *blob, size_t size, DescHeader *out) {
+    DescHeader h;
+    if (thip_status_t s = validateDescriptor(blob, size, &h)) return s;
+    const DescriptorView v{blob, h, (const DescOp *)(blob + h.ops_offset), (const DescBinding *)(blob + h.bindings_offset),
+                           (const DescTemp *)(blob + h.temps_offset), (const DescConst *)(blob + h.consts_offset)};
+    for (uint32_t i = 0; i < h.op_count; i++) {
+        if (thip_status_t s = checkOpFootprint(&v, i)) return s;
+    }
+    if (out) *out = h;
+    return THIP_OK;
+}
+
+}  // namespace thip
+
+extern "C" thip_status_t thip_descriptor_validate(const void *blob, size_t size) {
+    return thip::validateWhole((const uint8_t *)blob, size, nullptr);
+}
+
+extern "C" thip_status_t thip_infer_format(const void *blob, size_t size, size_t format_capacity, char *format, size_t *out_inferred_size) {
+    thip::DescHeader h;
+    if (thip_status_t s = thip::validateWhole((const uint8_t *)blob, size, &h)) return s;
+    static const char kFormat[] = "thip-gfx950";
+    if (!format || format_capacity < sizeof(kFormat)) return thip::fail(THIP_OUT_OF_RANGE, "format buffer too small");
+    memcpy(format, kFormat, sizeof(kFormat));
+    if (out_inferred_size) *out_inferred_size = (size_t)h.total_size;
+    return THIP_OK;
+}

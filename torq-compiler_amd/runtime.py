@@ -45,9 +45,9 @@ EXPORTED_SYMBOLS = [
     "thip_program_serialize", "thip_blob_free",
     "thip_device_create", "thip_device_destroy", "thip_device_name", "thip_device_alloc",
     "thip_device_free", "thip_device_h2d", "thip_device_d2h", "thip_device_synchronize",
-    "thip_device_set_event_log", "thip_infer_format",
+    "thip_device_set_event_log", "thip_device_set_dump_dirs", "thip_infer_format", "thip_descriptor_validate",
     "thip_executable_create", "thip_executable_destroy", "thip_executable_run",
-    "thip_executable_enqueue", "thip_executable_enqueue_noalloc", "thip_executable_wait", "thip_executable_time", "thip_executable_time_rotating",
+    "thip_executable_enqueue", "thip_executable_enqueue_noalloc", "thip_executable_wait", "thip_executable_set_wait_timeout", "thip_executable_time", "thip_executable_time_rotating",
     "thip_executable_op_count", "thip_executable_op_kernel", "thip_executable_binding_count",
     "thip_executable_binding_size",
 ]
@@ -230,7 +230,9 @@ def lib():
     L.thip_device_d2h.argtypes = [vp, vp, vp, sz]
     L.thip_device_synchronize.argtypes = [vp]
     L.thip_device_set_event_log.argtypes = [vp, ctypes.c_char_p]
+    L.thip_device_set_dump_dirs.argtypes = [vp, ctypes.c_char_p, ctypes.c_char_p]
     L.thip_infer_format.argtypes = [vp, sz, sz, ctypes.c_char_p, P(sz)]
+    L.thip_descriptor_validate.argtypes = [vp, sz]
     L.thip_executable_create.argtypes = [vp, vp, sz, P(u32), sz, P(vp)]
     L.thip_executable_destroy.argtypes = [vp]
     L.thip_executable_destroy.restype = None
@@ -238,6 +240,7 @@ def lib():
     L.thip_executable_enqueue.argtypes = [vp, P(DispatchState)]
     L.thip_executable_enqueue_noalloc.argtypes = [vp, P(DispatchState)]
     L.thip_executable_wait.argtypes = [vp]
+    L.thip_executable_set_wait_timeout.argtypes = [vp, ctypes.c_int64]
     L.thip_executable_time.argtypes = [vp, P(DispatchState), i32, P(ctypes.c_float)]
     L.thip_executable_time_rotating.argtypes = [vp, P(DispatchState), u32, i32, P(ctypes.c_float)]
     L.thip_executable_op_count.argtypes = [vp, P(u32)]
@@ -298,6 +301,11 @@ class Device:
 
     def set_event_log(self, path):
         check(lib().thip_device_set_event_log(self._h, path.encode() if path else None))
+
+    def set_dump_dirs(self, io_data_dir=None, buffers_dir=None):
+        """Debug dumps of the bindings of blocking dispatches / of every buffer a kernel record wrote (None: off)."""
+        check(lib().thip_device_set_dump_dirs(self._h, io_data_dir.encode() if io_data_dir else None,
+                                              buffers_dir.encode() if buffers_dir else None))
 
     def close(self):
         if self._h:
@@ -395,6 +403,10 @@ class Executable:
 
     def wait(self):
         check(lib().thip_executable_wait(self._h))
+
+    def set_wait_timeout(self, milliseconds):
+        """Waits for the GPU give up after this long (THIP_INTERNAL; the executable is abandoned); <= 0: no limit."""
+        check(lib().thip_executable_set_wait_timeout(self._h, int(milliseconds)))
 
     def time_device(self, ptrs, lengths, iterations):
         """Mean milliseconds per dispatch over `iterations`, HIP events on the executable's stream."""
