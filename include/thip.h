@@ -82,6 +82,11 @@ void thip_program_destroy(thip_program_t *program);
 /* Declares the tensor carried by dispatch binding `binding` (the
  * hal.interface.binding of the dispatch; table entry of
  * runtime/schemas/torq_executable_def.fbs:29-48). */
+/* Name of the hal.executable.export the program comes from (the reference keeps it as
+ * ExecutableDef.executable_name, runtime/schemas/torq_executable_def.fbs:172-173, and names its dump directories
+ * and profile rows after it).  1..63 characters of [A-Za-z0-9_.$-]; "thip_dispatch" when never set. */
+thip_status_t thip_program_set_name(thip_program_t *program, const char *name);
+
 thip_status_t thip_program_binding(thip_program_t *program, uint32_t binding, int32_t dtype,
                                    int32_t rank, const int64_t *shape, thip_value_t *out_value);
 
@@ -374,6 +379,42 @@ thip_status_t thip_device_h2d(thip_device_t *device, void *dst_device, const voi
 thip_status_t thip_device_d2h(thip_device_t *device, void *dst_host, const void *src_device,
                               size_t size);
 thip_status_t thip_device_synchronize(thip_device_t *device);
+
+/* What a descriptor blob holds, in the terms of the reference's executable schema
+ * (runtime/schemas/torq_executable_def.fbs): ExecutableDef :168-197, Binding :28-48, Segment :13-24.  These read
+ * the blob only (no device) and validate it first, like thip_descriptor_validate. */
+typedef struct thip_descriptor_info_t {
+    char executable_name[64];     /* ExecutableDef.executable_name */
+    uint32_t runtime_version;     /* ExecutableDef.runtime_version: the descriptor version the runtime gates on */
+    uint32_t hw_id;               /* ExecutableDef.hw_id: 950 = gfx950 */
+    uint32_t action_count;        /* ExecutableDef.actions: here one kernel record each */
+    uint32_t binding_count;       /* ExecutableDef.bindings */
+    uint32_t segment_count;       /* ExecutableDef.code: the constant segments uploaded once at create */
+    uint32_t intermediate_count;  /* device buffers the executable allocates for itself */
+    uint64_t intermediate_bytes;
+    uint64_t total_size;
+} thip_descriptor_info_t;
+thip_status_t thip_descriptor_info(const void *blob, size_t size, thip_descriptor_info_t *out_info);
+
+typedef struct thip_binding_info_t {
+    uint32_t id;            /* Binding.id: index into the dispatch's binding table */
+    uint64_t address;       /* Binding.address: always 0 (bindings arrive as pointers with each dispatch) */
+    uint64_t offset;        /* Binding.offset: always 0 */
+    uint64_t size;          /* Binding.size: bytes of the binding the program touches */
+    uint8_t is_read_only;   /* Binding.is_read_only */
+    uint8_t is_write_only;  /* Binding.is_write_only */
+    uint8_t is_used;        /* 0: the id is declared but no kernel touches it */
+} thip_binding_info_t;
+thip_status_t thip_descriptor_binding(const void *blob, size_t size, uint32_t index,
+                                      thip_binding_info_t *out_binding);
+
+typedef struct thip_segment_info_t {
+    uint64_t address;     /* Segment.xram_address: here the offset inside the executable's constant buffer */
+    uint64_t size;        /* Segment.size */
+    const uint8_t *data;  /* Segment.data: points into the blob */
+} thip_segment_info_t;
+thip_status_t thip_descriptor_segment(const void *blob, size_t size, uint32_t index,
+                                      thip_segment_info_t *out_segment);
 
 /* Debug dumps, the roles of the reference's --torq_dump_io_data_dir and --torq_dump_buffers_dir
  * (runtime/driver/TorqDump.cc:34-35,329-428).  io_data_dir: every blocking dispatch writes the raw bytes of its

@@ -13,7 +13,7 @@ REF = np.dtype([("space", "<u4"), ("index", "<u4"), ("offset", "<u8")])
 HEADER = np.dtype([("magic", "<u4"), ("version", "<u4"), ("arch", "<u4"), ("flags", "<u4"),
                    ("op_count", "<u4"), ("binding_count", "<u4"), ("temp_count", "<u4"), ("const_count", "<u4"),
                    ("ops_offset", "<u8"), ("bindings_offset", "<u8"), ("temps_offset", "<u8"),
-                   ("consts_offset", "<u8"), ("data_offset", "<u8"), ("total_size", "<u8")])
+                   ("consts_offset", "<u8"), ("data_offset", "<u8"), ("total_size", "<u8"), ("name", "S64")])
 _I32 = ["out_dtype", "input_zp", "output_zp", "output_min", "output_max", "shift",
         "N", "H", "W", "C", "OH", "OW", "OC", "KH", "KW", "SH", "SW", "PL", "PR", "PT", "PB",
         "M", "K", "Kp", "Nn", "Np", "w0", "w1", "bias0", "scale0", "TB", "TR", "TS", "pre_shift", "t0_clamp", "TP"]

@@ -27,7 +27,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_version_and_status_message():
     lib = runtime.lib()
-    assert lib.thip_descriptor_version() == 1
+    assert lib.thip_descriptor_version() == 2
     assert lib.thip_version() >= 1
     p = ctypes.c_void_p()
     assert lib.thip_program_create(ctypes.byref(p)) == runtime.OK
@@ -57,3 +57,23 @@ def test_device_create_without_gpu_is_unavailable_or_ok():
         return
     assert dev.name() == "gfx950"
     dev.close()
+
+
+def test_iree_glue_covers_every_op_entry_point():
+    """The plugin-side serialiser (iree_glue/, built only inside the reference's tree) forwards every TorqHL op the
+    C-ABI declares, and the HAL-side files call the run-side entry points they stand in front of."""
+    import re
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    header = open(os.path.join(root, "include", "thip.h")).read()
+    glue = open(os.path.join(root, "iree_glue", "ThipSerialization.cpp")).read()
+    ops = sorted(set(re.findall(r"thip_status_t (thip_hl_\w+)\(", header)))
+    assert len(ops) >= 13
+    for name in ops:
+        assert name + "(program_" in glue, name + " is not forwarded by iree_glue/ThipSerialization.cpp"
+        assert name + "_t s = {}" in glue
+    for name in ("thip_program_create", "thip_program_set_name", "thip_program_binding", "thip_program_constant", "thip_program_tensor",
+                 "thip_program_serialize", "thip_blob_free", "thip_descriptor_validate"):
+        assert name + "(" in glue, name
+    hal = open(os.path.join(root, "iree_glue", "thip_native_executable.cc")).read() + open(os.path.join(root, "iree_glue", "thip_driver_module.c")).read()
+    for name in ("thip_executable_create", "thip_executable_run", "thip_executable_destroy", "thip_infer_format", "thip_device_create", "thip_device_destroy"):
+        assert name + "(" in hal, name

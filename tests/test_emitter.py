@@ -410,3 +410,41 @@ def test_residual_add_stays_apart_when_it_must(monkeypatch):
     s1 = p.add(t, p.binding(1, wl.inputs[1].shape), aw, asb, init=p.binding(2, wl.inputs[1].shape), **aa)
     p.add(t, s1, aw, asb, init=p.binding(3, wl.inputs[1].shape), **aa)
     assert kinds(p) == [desc_interp.K_IGEMM, desc_interp.K_ADD, desc_interp.K_ADD]
+
+
+def test_descriptor_in_the_terms_of_the_reference_schema():
+    """The blob read back as the reference's ExecutableDef concepts (runtime/schemas/torq_executable_def.fbs:13-48,168-197):
+    executable name, runtime version / hardware id gates, the binding table {id, address, offset, size, is_read_only,
+    is_write_only}, the constant segments."""
+    p, x, want_fc, want_sum = _chain_program(True)
+    p.set_name("main_dispatch_0_conv2d")
+    blob = p.serialize()
+    info, bindings, segments = runtime.describe_blob(blob)
+    d = desc_interp.Descriptor(blob)
+    assert info["executable_name"] == "main_dispatch_0_conv2d" and info["runtime_version"] == 2 and info["hw_id"] == 950
+    assert info["action_count"] == len(d.ops) and info["total_size"] == len(blob)
+    assert info["intermediate_count"] == len(d.temps) and info["intermediate_bytes"] == int(d.temps["size"].sum())
+    # binding 0 is the input (read only), bindings 1 and 2 are results (write only); sizes are the bytes touched
+    assert [b["id"] for b in bindings] == [0, 1, 2]
+    assert [(b["is_read_only"], b["is_write_only"]) for b in bindings] == [(True, False), (False, True), (False, True)]
+    assert [b["size"] for b in bindings] == [x.nbytes, want_fc.nbytes, want_sum.nbytes]
+    assert all(b["address"] == 0 and b["offset"] == 0 and b["is_used"] for b in bindings)
+    # segments: what create uploads once; they tile the data region without overlap, 256-byte aligned
+    assert len(segments) == len(d.consts) and segments
+    end = 0
+    for s, c in zip(segments, d.consts):
+        assert s["address"] == int(c["offset"]) and s["size"] == int(c["size"]) and s["address"] % 256 == 0 and s["address"] >= end
+        end = s["address"] + s["size"]
+    assert all(s["data"] == bytes(d.const_bytes(i)) for i, s in enumerate(segments))
+    # a binding that is both read and written is neither read-only nor write-only
+    q = Program()
+    a = q.binding(0, (1, 8, 8, 16))
+    q.maxpool2d(a, input_zp=-128, output_min=-128, output_max=127, stride=(1, 1), pad=(0, 0, 0, 0), kernel=(1, 1), init=q.binding(1, (1, 8, 8, 16)), nhwc_input=True)
+    q.maxpool2d(q.binding(1, (1, 8, 8, 16)), input_zp=-128, output_min=-128, output_max=127, stride=(1, 1), pad=(0, 0, 0, 0), kernel=(1, 1),
+                init=q.binding(2, (1, 8, 8, 16)), nhwc_input=True)
+    _, b2, _ = runtime.describe_blob(q.serialize())
+    assert (b2[1]["is_read_only"], b2[1]["is_write_only"]) == (False, False)
+    # names that would not survive as a directory or a CSV column are refused
+    for bad in ["", "a/b", "x,y", "..", "n" * 64]:
+        with pytest.raises(ThipError):
+            Program().set_name(bad)

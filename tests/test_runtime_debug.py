@@ -23,6 +23,7 @@ def test_buffer_and_binding_dumps(device, tmp_path, monkeypatch):
     sys.stdout.flush()
     tensors = oracle_network(wl, return_all=True)
     io_dir, buf_dir = str(tmp_path / "io"), str(tmp_path / "buffers")
+    wl.program.set_name("mbv2_small")  # the directory the dumps go to
     exe = Executable(device, wl.program.serialize())
     out = np.zeros(wl.outputs[0][0], dtype=np.int8)
     device.set_dump_dirs(io_dir, buf_dir)
@@ -34,7 +35,7 @@ def test_buffer_and_binding_dumps(device, tmp_path, monkeypatch):
     exe.close()
     assert_bit_exact(out, tensors[-1], "logits with dumps on")
     assert len(kernels) == len(tensors) - 1
-    base = os.path.join(buf_dir, "thip_dispatch")
+    base = os.path.join(buf_dir, "mbv2_small")
     for i in range(len(kernels)):
         files = os.listdir(os.path.join(base, "action%d" % i))
         assert len(files) == 1 and files[0].startswith("buffer") and files[0].endswith(".npy"), files
@@ -45,7 +46,7 @@ def test_buffer_and_binding_dumps(device, tmp_path, monkeypatch):
     index = open(os.path.join(base, "buffers.csv")).read().splitlines()
     assert index[0].startswith("id;type;shape;strides;address;size;allocation_action;last_use_action;deallocation_action")
     assert len(index) == 1 + len(kernels) and index[-1].startswith("binding1;BINDING;2x40xi8;")
-    io = os.path.join(io_dir, "thip_dispatch")
+    io = os.path.join(io_dir, "mbv2_small")
     assert np.array_equal(np.fromfile(os.path.join(io, "npu.in.host_binding.0.torq_binding.0.bin"), dtype=np.int8), wl.inputs[0].reshape(-1))
     assert np.array_equal(np.fromfile(os.path.join(io, "npu.out.host_binding.1.torq_binding.1.bin"), dtype=np.int8), out.reshape(-1))
     # dumps off again: nothing new is written

@@ -13,7 +13,7 @@
 namespace thip {
 
 constexpr uint32_t kMagic = 0x50494854u;  // "THIP"
-constexpr uint32_t kDescriptorVersion = 1;
+constexpr uint32_t kDescriptorVersion = 2;
 constexpr uint32_t kArchGfx950 = 950;
 constexpr uint64_t kDataAlign = 256;
 
@@ -41,6 +41,9 @@ struct DescHeader {
     uint64_t consts_offset;
     uint64_t data_offset;
     uint64_t total_size;
+    // name of the hal.executable.export this program was made from (the reference's ExecutableDef.executable_name,
+    // runtime/schemas/torq_executable_def.fbs:172-173), NUL-terminated and NUL-padded
+    char name[64];
 };
 
 enum BindingFlags : uint32_t { kBindingRead = 1, kBindingWritten = 2 };

@@ -115,11 +115,12 @@ static const char *opKernelName(const DescOp &op) {
 // One row of the event log, in the reference's runtime CSV columns (doc/user-manual/profiling.md:53-63, written by
 // runtime/torq_hw/src/TorqEventLog.cpp:48,97-101): dispatch_name, invocation_id, action_id, timestamp_us, event
 // (an EventType name + _BEGIN / _END), plus one column of this backend's own: the kernel of a launch row.
-static void logEvent(thip_device_t *d, uint64_t invocation, int32_t action, const char *event, const char *phase, const char *kernel) {
+static void logEvent(const thip_executable_t *e, uint64_t invocation, int32_t action, const char *event, const char *phase, const char *kernel) {
+    thip_device_t *d = e->device;
     if (!d->eventLog) return;
     std::lock_guard<std::mutex> lock(d->logMutex);
     const auto us = std::chrono::duration_cast<std::chrono::microseconds>(std::chrono::steady_clock::now() - d->t0).count();
-    fprintf(d->eventLog, "thip_dispatch,%llu,%d,%lld,%s_%s,%s\n", (unsigned long long)invocation, action, (long long)us, event, phase, kernel);
+    fprintf(d->eventLog, "%s,%llu,%d,%lld,%s_%s,%s\n", e->header.name, (unsigned long long)invocation, action, (long long)us, event, phase, kernel);
 }
 
 // Resolves an operand reference against the buffers of this dispatch.
@@ -353,13 +354,12 @@ static bool makeDirs(const std::string &path) {
     return true;
 }
 
-static const char *kDispatchName = "thip_dispatch";  // the executable name in file paths and in the event log
-
 // Raw bytes of a binding, named as the reference names them (runtime/driver/TorqDump.cc:329-339):
 // <dir>/<executable>/npu.{in,out}.host_binding.<i>.torq_binding.<i>.bin
-static void dumpBinding(const thip_device_t *d, uint32_t binding, const void *host, size_t size, bool isInput) {
+static void dumpBinding(const thip_executable_t *e, uint32_t binding, const void *host, size_t size, bool isInput) {
+    const thip_device_t *d = e->device;
     if (d->dumpIoDir.empty()) return;
-    const std::string dir = d->dumpIoDir + "/" + kDispatchName;
+    const std::string dir = d->dumpIoDir + "/" + e->header.name;
     if (!makeDirs(dir)) return;
     const std::string n = std::to_string(binding);
     const std::string path = dir + "/npu" + (isInput ? ".in" : ".out") + ".host_binding." + n + ".torq_binding." + n + ".bin";
@@ -403,7 +403,7 @@ static thip_status_t dumpOpOutput(thip_executable_t *e, uint32_t i, uint8_t *con
     if (count == 0 || op.out.space == kSpaceNone) return THIP_OK;  // e.g. a convolution whose result only feeds its fused add
     std::vector<uint8_t> host(count * elem);
     THIP_HIP(hipMemcpy(host.data(), resolve(e, op.out, bp), host.size(), hipMemcpyDeviceToHost), "reading a buffer back for the dump");
-    const std::string base = d->dumpBuffersDir + "/" + kDispatchName, dir = base + "/action" + std::to_string(i);
+    const std::string base = d->dumpBuffersDir + "/" + e->header.name, dir = base + "/action" + std::to_string(i);
     if (!makeDirs(dir)) return fail(THIP_INVALID_ARGUMENT, "cannot create dump directory %s", dir.c_str());
     const std::string id = (op.out.space == kSpaceBinding ? "binding" : "temp") + std::to_string(op.out.index);
     std::string dims, dimsX;
@@ -438,9 +438,9 @@ static thip_status_t dumpOpOutput(thip_executable_t *e, uint32_t i, uint8_t *con
 static thip_status_t enqueueOps(thip_executable_t *e, uint8_t *const *bp) {
     for (uint32_t i = 0; i < e->header.op_count; i++) {
         // a kernel launch is what starting an NSS task is on the reference's hardware
-        logEvent(e->device, e->invocation, (int32_t)i, "NSS_START", "BEGIN", e->kernelNames[i].c_str());
+        logEvent(e, e->invocation, (int32_t)i, "NSS_START", "BEGIN", e->kernelNames[i].c_str());
         if (thip_status_t s = launchOp(e, i, bp, LaunchCtx{e->stream, &e->tuning, nullptr, 0})) return s;
-        logEvent(e->device, e->invocation, (int32_t)i, "NSS_START", "END", e->kernelNames[i].c_str());
+        logEvent(e, e->invocation, (int32_t)i, "NSS_START", "END", e->kernelNames[i].c_str());
         if (!e->device->dumpBuffersDir.empty()) {
             // buffer dumps: each record runs to its end and what it wrote is read back before the next one starts
             if (thip_status_t s = waitBounded(e, "waiting for a record before its dump")) return s;
@@ -727,8 +727,8 @@ static thip_status_t runLocked(thip_executable_t *e, const thip_dispatch_state_t
     THIP_HIP(hipSetDevice(e->device->ordinal), "hipSetDevice");
     uint8_t *bp[64] = {nullptr};
     const int32_t lastOp = (int32_t)e->header.op_count - 1;
-    logEvent(e->device, e->invocation, 0, "DISPATCH", "BEGIN", "");
-    logEvent(e->device, e->invocation, 0, "DISPATCH_SYNC_BINDINGS_IN", "BEGIN", "");
+    logEvent(e, e->invocation, 0, "DISPATCH", "BEGIN", "");
+    logEvent(e, e->invocation, 0, "DISPATCH_SYNC_BINDINGS_IN", "BEGIN", "");
     // writeInputs: host bindings are staged into device memory (TorqExecutable::writeInputs)
     for (uint32_t i = 0; i < e->header.binding_count; i++) {
         if (e->bindings[i].flags == 0) continue;
@@ -742,16 +742,16 @@ static thip_status_t runLocked(thip_executable_t *e, const thip_dispatch_state_t
         }
         bp[i] = e->staging[i];
         if (e->bindings[i].flags & kBindingRead) {
-            dumpBinding(e->device, i, st->binding_ptrs[i], e->bindings[i].size, true);
+            dumpBinding(e, i, st->binding_ptrs[i], e->bindings[i].size, true);
             THIP_HIP(hipMemcpyAsync(bp[i], st->binding_ptrs[i], e->bindings[i].size, hipMemcpyHostToDevice, e->stream), "staging a binding");
         }
     }
-    logEvent(e->device, e->invocation, 0, "DISPATCH_SYNC_BINDINGS_IN", "END", "");
+    logEvent(e, e->invocation, 0, "DISPATCH_SYNC_BINDINGS_IN", "END", "");
     bool allDevice = true;
     for (uint32_t i = 0; i < e->header.binding_count; i++) {
         if (e->bindings[i].flags != 0 && !(st->binding_flags && (st->binding_flags[i] & THIP_BINDING_DEVICE))) allDevice = false;
     }
-    logEvent(e->device, e->invocation, 0, "DISPATCH_EXECUTE_ACTIONS", "BEGIN", "");
+    logEvent(e, e->invocation, 0, "DISPATCH_EXECUTE_ACTIONS", "BEGIN", "");
     if (thip_status_t s = allDevice ? enqueueDevice(e, bp) : enqueueOps(e, bp)) {
         // what was enqueued before the failure still runs: wait for it (bounded; the launch error is what is reported)
         std::string message = thip_status_message();
@@ -759,25 +759,25 @@ static thip_status_t runLocked(thip_executable_t *e, const thip_dispatch_state_t
         e->invocation++;
         return fail(s, "%s", message.c_str());
     }
-    logEvent(e->device, e->invocation, lastOp, "DISPATCH_EXECUTE_ACTIONS", "END", "");
-    logEvent(e->device, e->invocation, lastOp, "DISPATCH_SYNC_BINDINGS_OUT", "BEGIN", "");
+    logEvent(e, e->invocation, lastOp, "DISPATCH_EXECUTE_ACTIONS", "END", "");
+    logEvent(e, e->invocation, lastOp, "DISPATCH_SYNC_BINDINGS_OUT", "BEGIN", "");
     // readOutputs (TorqExecutable::readOutputs, runtime/driver/TorqExecutable.cc:860-918)
     for (uint32_t i = 0; i < e->header.binding_count; i++) {
         const bool isDevice = st->binding_flags && (st->binding_flags[i] & THIP_BINDING_DEVICE);
         if (isDevice || !(e->bindings[i].flags & kBindingWritten)) continue;
         THIP_HIP(hipMemcpyAsync(st->binding_ptrs[i], bp[i], e->bindings[i].size, hipMemcpyDeviceToHost, e->stream), "reading back a binding");
     }
-    logEvent(e->device, e->invocation, lastOp, "NSS_WAIT", "BEGIN", "");
+    logEvent(e, e->invocation, lastOp, "NSS_WAIT", "BEGIN", "");
     const thip_status_t waited = waitBounded(e, "waiting for the dispatch");
     const std::string waitMessage = waited == THIP_OK ? std::string() : std::string(thip_status_message());
-    logEvent(e->device, e->invocation, lastOp, "NSS_WAIT", "END", "");
-    logEvent(e->device, e->invocation, lastOp, "DISPATCH_SYNC_BINDINGS_OUT", "END", "");
-    logEvent(e->device, e->invocation, lastOp, "DISPATCH", "END", "");
+    logEvent(e, e->invocation, lastOp, "NSS_WAIT", "END", "");
+    logEvent(e, e->invocation, lastOp, "DISPATCH_SYNC_BINDINGS_OUT", "END", "");
+    logEvent(e, e->invocation, lastOp, "DISPATCH", "END", "");
     e->invocation++;
     if (waited != THIP_OK) return fail(waited, "%s", waitMessage.c_str());
     for (uint32_t i = 0; i < e->header.binding_count; i++) {
         const bool isDevice = st->binding_flags && (st->binding_flags[i] & THIP_BINDING_DEVICE);
-        if (!isDevice && (e->bindings[i].flags & kBindingWritten)) dumpBinding(e->device, i, st->binding_ptrs[i], e->bindings[i].size, false);
+        if (!isDevice && (e->bindings[i].flags & kBindingWritten)) dumpBinding(e, i, st->binding_ptrs[i], e->bindings[i].size, false);
     }
     return THIP_OK;
 }

@@ -71,6 +71,7 @@ struct HlOp {
 struct thip_program_t {
     std::vector<thip::Value> values;
     std::vector<thip::HlOp> ops;
+    std::string name = "thip_dispatch";
 };
 
 namespace thip {
@@ -1834,6 +1835,7 @@ thip_status_t Emitter::run(void **outBlob, size_t *outSize) {
     h.binding_count = bindingCount;
     h.temp_count = (uint32_t)temps_.size();
     h.const_count = (uint32_t)consts_.size();
+    snprintf(h.name, sizeof(h.name), "%s", prog_.name.c_str());
     uint64_t off = sizeof(DescHeader);
     h.ops_offset = off;
     off += sizeof(DescOp) * ops_.size();
@@ -1910,6 +1912,21 @@ thip_status_t thip_program_create(thip_program_t **out_program) {
 }
 
 void thip_program_destroy(thip_program_t *program) { delete program; }
+
+thip_status_t thip_program_set_name(thip_program_t *program, const char *name) {
+    if (!program || !name) return fail(THIP_INVALID_ARGUMENT, "null argument");
+    const size_t n = strlen(name);
+    if (n == 0 || n >= sizeof(DescHeader::name)) return fail(THIP_INVALID_ARGUMENT, "an executable name has 1..%zu characters", sizeof(DescHeader::name) - 1);
+    for (size_t i = 0; i < n; i++) {
+        const char c = name[i];
+        // the name becomes a directory of the dumps and a CSV column: keep it to what is safe in both
+        if (!((c >= 'a' && c <= 'z') || (c >= 'A' && c <= 'Z') || (c >= '0' && c <= '9') || c == '_' || c == '-' || c == '.' || c == '$') || (i == 0 && c == '.')) {
+            return fail(THIP_INVALID_ARGUMENT, "executable name has a character outside [A-Za-z0-9_.$-]");
+        }
+    }
+    program->name = name;
+    return THIP_OK;
+}
 
 thip_status_t thip_program_binding(thip_program_t *program, uint32_t binding, int32_t dtype, int32_t rank,
                                    const int64_t *shape, thip_value_t *out_value) {

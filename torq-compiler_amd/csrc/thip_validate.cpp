@@ -69,6 +69,16 @@ thip_status_t validateDescriptor(const uint8_t *p, size_t size, DescHeader *out)
     if ((h.ops_offset | h.bindings_offset | h.temps_offset | h.consts_offset) & 7) return fail(THIP_INVALID_ARGUMENT, "descriptor tables are misaligned");
     if (((uintptr_t)p & 7) != 0) return fail(THIP_INVALID_ARGUMENT, "descriptor must be 8-byte aligned in memory");
     if (h.op_count == 0) return fail(THIP_INVALID_ARGUMENT, "descriptor holds no ops");
+    {
+        size_t n = 0;
+        while (n < sizeof(h.name) && h.name[n]) n++;
+        if (n == 0 || n == sizeof(h.name)) return fail(THIP_INVALID_ARGUMENT, "descriptor has no terminated executable name");
+        for (size_t k = 0; k < sizeof(h.name); k++) {
+            const char c = h.name[k];
+            const bool ok = k >= n ? c == 0 : ((c >= 'a' && c <= 'z') || (c >= 'A' && c <= 'Z') || (c >= '0' && c <= '9') || c == '_' || c == '-' || (c == '.' && k > 0) || c == '$');
+            if (!ok) return fail(THIP_INVALID_ARGUMENT, "descriptor's executable name is malformed");
+        }
+    }
     if (h.binding_count > 64) return fail(THIP_INVALID_ARGUMENT, "descriptor declares %u bindings (max 64)", h.binding_count);
     const DescConst *consts = (const DescConst *)(p + h.consts_offset);
     for (uint32_t i = 0; i < h.const_count; i++) {
@@ -331,6 +341,53 @@ thip_status_t validateWhole(const uint8_t *blob, size_t size, DescHeader *out) {
 
 extern "C" thip_status_t thip_descriptor_validate(const void *blob, size_t size) {
     return thip::validateWhole((const uint8_t *)blob, size, nullptr);
+}
+
+extern "C" thip_status_t thip_descriptor_info(const void *blob, size_t size, thip_descriptor_info_t *out) {
+    if (!out) return thip::fail(THIP_INVALID_ARGUMENT, "null result pointer");
+    thip::DescHeader h;
+    if (thip_status_t s = thip::validateWhole((const uint8_t *)blob, size, &h)) return s;
+    memset(out, 0, sizeof(*out));
+    memcpy(out->executable_name, h.name, sizeof(h.name));
+    out->runtime_version = h.version;
+    out->hw_id = h.arch;
+    out->action_count = h.op_count;
+    out->binding_count = h.binding_count;
+    out->segment_count = h.const_count;
+    out->intermediate_count = h.temp_count;
+    const thip::DescTemp *temps = (const thip::DescTemp *)((const uint8_t *)blob + h.temps_offset);
+    for (uint32_t i = 0; i < h.temp_count; i++) out->intermediate_bytes += temps[i].size;
+    out->total_size = h.total_size;
+    return THIP_OK;
+}
+
+extern "C" thip_status_t thip_descriptor_binding(const void *blob, size_t size, uint32_t index, thip_binding_info_t *out) {
+    if (!out) return thip::fail(THIP_INVALID_ARGUMENT, "null result pointer");
+    thip::DescHeader h;
+    if (thip_status_t s = thip::validateWhole((const uint8_t *)blob, size, &h)) return s;
+    if (index >= h.binding_count) return thip::fail(THIP_OUT_OF_RANGE, "binding %u of %u", index, h.binding_count);
+    const thip::DescBinding &b = ((const thip::DescBinding *)((const uint8_t *)blob + h.bindings_offset))[index];
+    memset(out, 0, sizeof(*out));
+    out->id = b.id;
+    out->address = 0;  // bindings are passed as pointers with each dispatch; nothing is mapped at a fixed address
+    out->offset = 0;   // always from the start of the binding's buffer
+    out->size = b.size;
+    out->is_read_only = (b.flags & thip::kBindingRead) && !(b.flags & thip::kBindingWritten);
+    out->is_write_only = (b.flags & thip::kBindingWritten) && !(b.flags & thip::kBindingRead);
+    out->is_used = b.flags != 0;
+    return THIP_OK;
+}
+
+extern "C" thip_status_t thip_descriptor_segment(const void *blob, size_t size, uint32_t index, thip_segment_info_t *out) {
+    if (!out) return thip::fail(THIP_INVALID_ARGUMENT, "null result pointer");
+    thip::DescHeader h;
+    if (thip_status_t s = thip::validateWhole((const uint8_t *)blob, size, &h)) return s;
+    if (index >= h.const_count) return thip::fail(THIP_OUT_OF_RANGE, "segment %u of %u", index, h.const_count);
+    const thip::DescConst &c = ((const thip::DescConst *)((const uint8_t *)blob + h.consts_offset))[index];
+    out->address = c.offset;
+    out->size = c.size;
+    out->data = (const uint8_t *)blob + h.data_offset + c.offset;
+    return THIP_OK;
 }
 
 extern "C" thip_status_t thip_infer_format(const void *blob, size_t size, size_t format_capacity, char *format, size_t *out_inferred_size) {

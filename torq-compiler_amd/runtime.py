@@ -38,14 +38,14 @@ BINDING_HOST, BINDING_DEVICE = 0, 1
 # every symbol include/thip.h declares
 EXPORTED_SYMBOLS = [
     "thip_status_message", "thip_version", "thip_descriptor_version",
-    "thip_program_create", "thip_program_destroy", "thip_program_binding", "thip_program_constant",
+    "thip_program_create", "thip_program_destroy", "thip_program_set_name", "thip_program_binding", "thip_program_constant",
     "thip_program_tensor", "thip_hl_conv2d", "thip_hl_depthwise_conv2d", "thip_hl_fully_connected",
     "thip_hl_matmul", "thip_hl_maxpool2d", "thip_hl_avg_pool2d", "thip_hl_add", "thip_hl_transpose", "thip_hl_expand_weights",
     "thip_hl_fma", "thip_hl_mul", "thip_hl_act", "thip_hl_elementwisebinary",
     "thip_program_serialize", "thip_blob_free",
     "thip_device_create", "thip_device_destroy", "thip_device_name", "thip_device_alloc",
     "thip_device_free", "thip_device_h2d", "thip_device_d2h", "thip_device_synchronize",
-    "thip_device_set_event_log", "thip_device_set_dump_dirs", "thip_infer_format", "thip_descriptor_validate",
+    "thip_device_set_event_log", "thip_device_set_dump_dirs", "thip_infer_format", "thip_descriptor_validate", "thip_descriptor_info", "thip_descriptor_binding", "thip_descriptor_segment",
     "thip_executable_create", "thip_executable_destroy", "thip_executable_run",
     "thip_executable_enqueue", "thip_executable_enqueue_noalloc", "thip_executable_wait", "thip_executable_set_wait_timeout", "thip_executable_time", "thip_executable_time_rotating",
     "thip_executable_op_count", "thip_executable_op_kernel", "thip_executable_binding_count",
@@ -58,6 +58,41 @@ class ThipError(RuntimeError):
         super().__init__("%s: %s" % (STATUS_NAMES.get(code, str(code)), message))
         self.code = code
         self.message = message
+
+
+class DescriptorInfo(ctypes.Structure):
+    _fields_ = [("executable_name", ctypes.c_char * 64), ("runtime_version", ctypes.c_uint32), ("hw_id", ctypes.c_uint32),
+                ("action_count", ctypes.c_uint32), ("binding_count", ctypes.c_uint32), ("segment_count", ctypes.c_uint32),
+                ("intermediate_count", ctypes.c_uint32), ("intermediate_bytes", ctypes.c_uint64), ("total_size", ctypes.c_uint64)]
+
+
+class BindingInfo(ctypes.Structure):
+    _fields_ = [("id", ctypes.c_uint32), ("address", ctypes.c_uint64), ("offset", ctypes.c_uint64), ("size", ctypes.c_uint64),
+                ("is_read_only", ctypes.c_uint8), ("is_write_only", ctypes.c_uint8), ("is_used", ctypes.c_uint8)]
+
+
+class SegmentInfo(ctypes.Structure):
+    _fields_ = [("address", ctypes.c_uint64), ("size", ctypes.c_uint64), ("data", ctypes.POINTER(ctypes.c_uint8))]
+
+
+def describe_blob(blob):
+    """What a descriptor blob holds in the terms of the reference's executable schema: (info, bindings, segments)."""
+    buf = ctypes.create_string_buffer(bytes(blob), len(blob))
+    info = DescriptorInfo()
+    check(lib().thip_descriptor_info(buf, len(blob), ctypes.byref(info)))
+    bindings, segments = [], []
+    for i in range(info.binding_count):
+        b = BindingInfo()
+        check(lib().thip_descriptor_binding(buf, len(blob), i, ctypes.byref(b)))
+        bindings.append(dict(id=b.id, address=b.address, offset=b.offset, size=b.size, is_read_only=bool(b.is_read_only),
+                             is_write_only=bool(b.is_write_only), is_used=bool(b.is_used)))
+    for i in range(info.segment_count):
+        s = SegmentInfo()
+        check(lib().thip_descriptor_segment(buf, len(blob), i, ctypes.byref(s)))
+        segments.append(dict(address=s.address, size=s.size, data=bytes(ctypes.string_at(s.data, s.size))))
+    return dict(executable_name=info.executable_name.decode(), runtime_version=info.runtime_version, hw_id=info.hw_id,
+                action_count=info.action_count, intermediate_count=info.intermediate_count, intermediate_bytes=info.intermediate_bytes,
+                total_size=info.total_size), bindings, segments
 
 
 class DispatchState(ctypes.Structure):
@@ -233,6 +268,10 @@ def lib():
     L.thip_device_set_dump_dirs.argtypes = [vp, ctypes.c_char_p, ctypes.c_char_p]
     L.thip_infer_format.argtypes = [vp, sz, sz, ctypes.c_char_p, P(sz)]
     L.thip_descriptor_validate.argtypes = [vp, sz]
+    L.thip_descriptor_info.argtypes = [vp, sz, vp]
+    L.thip_descriptor_binding.argtypes = [vp, sz, u32, vp]
+    L.thip_descriptor_segment.argtypes = [vp, sz, u32, vp]
+    L.thip_program_set_name.argtypes = [vp, ctypes.c_char_p]
     L.thip_executable_create.argtypes = [vp, vp, sz, P(u32), sz, P(vp)]
     L.thip_executable_destroy.argtypes = [vp]
     L.thip_executable_destroy.restype = None

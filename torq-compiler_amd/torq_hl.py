@@ -59,6 +59,10 @@ class Program:
         except KeyError:
             raise rt.ThipError(rt.UNIMPLEMENTED, "element type %s is not supported" % np.dtype(dtype))
 
+    def set_name(self, name):
+        """Name of the hal.executable.export the program stands for (dump directories and profile rows carry it)."""
+        rt.check(rt.lib().thip_program_set_name(self._h, name.encode()))
+
     def binding(self, index, shape, dtype=np.int8):
         v = ctypes.c_int32()
         rt.check(rt.lib().thip_program_binding(self._h, int(index), self._dtype_code(dtype), len(shape),
