@@ -57,6 +57,11 @@ def workload_table(pkg):
         "avgpool_b1": (lambda: w.avgpool_workload(N=1), "hbm"),
         "add_b64": (lambda: w.add_workload(N=64), "hbm"),
         "add_b1": (lambda: w.add_workload(N=1), "hbm"),
+        # what a kernel with no arithmetic reaches: plain copies (1x1 max pool) of 18 + 18 MiB (the size of the
+        # depthwise row), 32 + 32 MiB (the max pool row) and 128 + 128 MiB
+        "copy_18MiB": (lambda: w.copy_workload(18 << 20), "hbm"),
+        "copy_32MiB": (lambda: w.copy_workload(32 << 20), "hbm"),
+        "copy_128MiB": (lambda: w.copy_workload(128 << 20), "hbm"),
         # integer elementwise ops next to the convolution path, at the shape of the add row
         "rescale_b64": (lambda: w.fma_workload((64, 56, 56, 24)), "hbm"),
         "mul_b64": (lambda: w.mul_workload((64, 56, 56, 24)), "hbm"),
@@ -228,6 +233,46 @@ def cpu_baseline(wl, target_seconds=10.0, single_thread_seconds=6.0):
                               "sample": (what + ", one thread") % (passes1, rows1, M, M, K, N, dt1)}}
 
 
+def mfma_calibration(pkg, dev, wl, args):
+    """What bounds the headline GEMM on this card, measured in this run (TOP/s, 1 multiply-add = 2 ops)."""
+    out = {"unit": "TOP/s", "published_peak": PEAK_INT8_TOPS}
+    # the matrix cores with nothing else going on: every CU busy (256 workgroups of 4 waves), and 32 workgroups only
+    # (an eighth of the chip: far below the power limit, so this is the clock-limited rate of one CU)
+    out["mfma_only_constant_operands"] = round(dev.mfma_rate(False, 256, 12000), 1)
+    out["mfma_only_random_operands"] = round(dev.mfma_rate(True, 256, 12000), 1)
+    out["mfma_only_random_operands_32_of_256_cus_scaled"] = round(dev.mfma_rate(True, 32, 12000) * 8, 1)
+    # the same GEMM kernel on all-zero operands (nothing toggles) against the benchmark's uniform random bytes
+    M, K = wl.inputs[0].shape
+    N = wl.attrs["weights"].shape[0]
+    for label, zeros in (("gemm_random_data", False), ("gemm_zero_data", True)):
+        o = Loaded(pkg, dev, pkg.workloads.fully_connected_workload(M, K, N, zeros=zeros))
+        o.run(args.warmup)
+        ms = o.run(args.steps)
+        out[label] = {"us": round(ms * 1e3, 2), "TOP/s": round(o.wl.ops / (ms * 1e-3) / 1e12, 1), "kernel": o.exe.op_kernels()[0]}
+        o.close()
+    out["gemm_over_mfma_only_random"] = round(out["gemm_random_data"]["TOP/s"] / out["mfma_only_random_operands"], 3)
+    if args.library_gemm:
+        try:
+            import torch
+            a = torch.randint(-128, 128, (M, K), dtype=torch.int8, device="cuda:0")
+            bt = torch.randint(-128, 128, (N, K), dtype=torch.int8, device="cuda:0").t()
+            for _ in range(args.warmup):
+                torch._int_mm(a, bt)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(args.steps):
+                torch._int_mm(a, bt)
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / args.steps
+            out["library_int_mm_random_data"] = {"us": round(ms * 1e3, 2), "TOP/s": round(2.0 * M * K * N / (ms * 1e-3) / 1e12, 1),
+                                                 "what": "torch._int_mm (hipBLASLt), int32 result, no requant, [N,K] weights like ours"}
+        except Exception as ex:  # the comparison is optional
+            out["library_int_mm_random_data"] = "unavailable: %r" % (ex,)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -236,6 +281,10 @@ def main():
     ap.add_argument("--workload", default="fc_4096x4096x4096")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-others", action="store_true", help="skip the brief per-op measurements")
+    ap.add_argument("--mfma-calibration", action="store_true",
+                    help="also measure what bounds the int8 GEMM on this card: the matrix cores alone on constant and on random operands, "
+                         "the same GEMM on all-zero data, and (with --library-gemm) the vendor library's int8 GEMM")
+    ap.add_argument("--library-gemm", action="store_true", help="with --mfma-calibration: time torch._int_mm (hipBLASLt) on the same shape")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (a 1x1 max pool), to scale rocprofv3's FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
@@ -280,6 +329,10 @@ def main():
         exe.close()
         for ptr in ptrs:
             dev.free(ptr)
+
+    calibration = None
+    if args.mfma_calibration:
+        calibration = mfma_calibration(pkg, dev, wl, args)
 
     per_op = {}
     if not args.no_others:
@@ -345,6 +398,8 @@ def main():
     }
     if not args.no_cpu and args.workload.startswith("fc_"):
         result["cpu_baseline"] = cpu_baseline(wl)
+    if calibration:
+        result["mfma_calibration"] = calibration
     if per_op:
         result["per_op"] = per_op
     if mbv2:

@@ -67,7 +67,8 @@ typedef struct thip_program_t thip_program_t;
 typedef int32_t thip_value_t;
 
 /* BF16 values are bfloat16 bit patterns (16 bits); F32 is used for the bias of the bf16 ops. */
-enum { THIP_DTYPE_I8 = 1, THIP_DTYPE_I16 = 2, THIP_DTYPE_I32 = 3, THIP_DTYPE_BF16 = 4, THIP_DTYPE_F32 = 5 };
+/* THIP_DTYPE_I1: a truth value (MLIR's i1), one byte per element holding 0 or 1. */
+enum { THIP_DTYPE_I8 = 1, THIP_DTYPE_I16 = 2, THIP_DTYPE_I32 = 3, THIP_DTYPE_BF16 = 4, THIP_DTYPE_F32 = 5, THIP_DTYPE_I1 = 6 };
 
 #define THIP_MAX_RANK 4
 
@@ -319,9 +320,11 @@ typedef struct thip_hl_act_t {
 } thip_hl_act_t;
 
 /* torq_hl.elementwisebinary -- TorqHLOps.td:248-260.  op_type: the reference's ElementwiseOpEnum value
- * (TorqHLAttrs.td:219-235); on this path BITWISE_AND 0, BITWISE_OR 1, BITWISE_XOR 2, MINIMUM 4, MAXIMUM 5.  input1,
- * input2 and init: int8 / int16 / int32 tensors of one type and shape; is_unsigned (16-bit only) makes MINIMUM /
- * MAXIMUM compare as unsigned.  The comparisons, logical ops and the int32 ADD / SUB are not on this path. */
+ * (TorqHLAttrs.td:219-235).  BITWISE_AND 0, BITWISE_OR 1, BITWISE_XOR 2, MINIMUM 4, MAXIMUM 5: input1, input2 and
+ * init are int8 / int16 / int32 tensors of one type and shape.  GREATER 6, GREATER_EQUAL 7, EQUAL 8: inputs of one
+ * such type, init an i1 tensor (THIP_DTYPE_I1).  LOGICAL_AND 9, LOGICAL_OR 10, LOGICAL_XOR 11: i1 in, i1 out.
+ * is_unsigned (16-bit operands only) makes MINIMUM / MAXIMUM and the comparisons read their operands as unsigned.
+ * The int32 ADD / SUB through the 48-bit accumulator (13, 14) are not on this path. */
 typedef struct thip_hl_elementwisebinary_t {
     thip_value_t init;
     int32_t op_type;
@@ -329,6 +332,25 @@ typedef struct thip_hl_elementwisebinary_t {
     thip_value_t input2;
     int32_t is_unsigned;
 } thip_hl_elementwisebinary_t;
+
+/* torq_hl.elementwiseunary -- TorqHLOps.td:262-273.  op_type (ElementwiseOpEnum): 3 BITWISE_NOT on int8 / int16 /
+ * int32 (init of the same type), 12 LOGICAL_NOT on i1 (init i1). */
+typedef struct thip_hl_elementwiseunary_t {
+    thip_value_t init;
+    int32_t op_type;
+    thip_value_t input;
+} thip_hl_elementwiseunary_t;
+
+/* torq_hl.elementwiseshift -- TorqHLOps.td:275-289.  op_type (ShiftModeEnum, TorqHLAttrs.td:239-246): 0 LSR, 1 LSL,
+ * 2 ASR (3 ASL is refused, as the reference's lowering refuses it).  input1, input2 (the per-element shift counts)
+ * and init share one type of int8 / int16 / int32 and one element count.  round: right shifts round half up. */
+typedef struct thip_hl_elementwiseshift_t {
+    thip_value_t init;
+    int32_t op_type;
+    int32_t round;
+    thip_value_t input1;
+    thip_value_t input2;
+} thip_hl_elementwiseshift_t;
 
 thip_status_t thip_hl_conv2d(thip_program_t *program, const thip_hl_conv2d_t *op);
 thip_status_t thip_hl_depthwise_conv2d(thip_program_t *program,
@@ -343,6 +365,8 @@ thip_status_t thip_hl_transpose(thip_program_t *program, const thip_hl_transpose
 thip_status_t thip_hl_expand_weights(thip_program_t *program, const thip_hl_expand_weights_t *op);
 thip_status_t thip_hl_fma(thip_program_t *program, const thip_hl_fma_t *op);
 thip_status_t thip_hl_mul(thip_program_t *program, const thip_hl_mul_t *op);
+thip_status_t thip_hl_elementwiseunary(thip_program_t *program, const thip_hl_elementwiseunary_t *op);
+thip_status_t thip_hl_elementwiseshift(thip_program_t *program, const thip_hl_elementwiseshift_t *op);
 thip_status_t thip_hl_act(thip_program_t *program, const thip_hl_act_t *op);
 thip_status_t thip_hl_elementwisebinary(thip_program_t *program, const thip_hl_elementwisebinary_t *op);
 
@@ -379,6 +403,13 @@ thip_status_t thip_device_h2d(thip_device_t *device, void *dst_device, const voi
 thip_status_t thip_device_d2h(thip_device_t *device, void *dst_host, const void *src_device,
                               size_t size);
 thip_status_t thip_device_synchronize(thip_device_t *device);
+
+/* Calibration for the benchmark (no counterpart in the reference): the rate, in TOP/s with 1 multiply-add = 2 ops,
+ * that `workgroups` workgroups of four waves sustain when they issue v_mfma_i32_32x32x32_i8 back to back on
+ * register operands and touch no memory.  random_operands != 0: uniformly random operand bytes; 0: every byte 1.
+ * The card runs against a power limit, so the two differ: it is the ceiling of any int8 GEMM on such data. */
+thip_status_t thip_device_mfma_rate(thip_device_t *device, int32_t random_operands, int32_t workgroups,
+                                    int32_t iterations, double *out_tops);
 
 /* What a descriptor blob holds, in the terms of the reference's executable schema
  * (runtime/schemas/torq_executable_def.fbs): ExecutableDef :168-197, Binding :28-48, Segment :13-24.  These read

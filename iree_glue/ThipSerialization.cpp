@@ -32,6 +32,7 @@ namespace {
 
 // Element type of a tensor / memref in the C-ABI's numbering; -1 when the path does not carry it.
 int32_t dtypeOf(Type elementType) {
+    if (elementType.isInteger(1)) return THIP_DTYPE_I1;  // stored as one byte of 0 / 1
     if (elementType.isInteger(8)) return THIP_DTYPE_I8;
     if (elementType.isInteger(16)) return THIP_DTYPE_I16;
     if (elementType.isInteger(32)) return THIP_DTYPE_I32;
@@ -270,6 +271,21 @@ class ProgramBuilder {
                 s.op_type = (int32_t)c.getOpType(); s.is_unsigned = c.getIsUnsigned();
                 LogicalResult r = withOperands(op, {{c.getInit(), &s.init}, {c.getInput1(), &s.input1}, {c.getInput2(), &s.input2}},
                                                [&] { return thip_hl_elementwisebinary(program_, &s); });
+                aliasResult(op, s.init);
+                return r;
+            })
+            .Case<torq_hl::ElementWiseUnaryOp>([&](torq_hl::ElementWiseUnaryOp c) {
+                thip_hl_elementwiseunary_t s = {};
+                s.op_type = (int32_t)c.getOpType();
+                LogicalResult r = withOperands(op, {{c.getInit(), &s.init}, {c.getInput(), &s.input}}, [&] { return thip_hl_elementwiseunary(program_, &s); });
+                aliasResult(op, s.init);
+                return r;
+            })
+            .Case<torq_hl::ElementWiseShiftOp>([&](torq_hl::ElementWiseShiftOp c) {
+                thip_hl_elementwiseshift_t s = {};
+                s.op_type = (int32_t)c.getOpType(); s.round = c.getRound();
+                LogicalResult r = withOperands(op, {{c.getInit(), &s.init}, {c.getInput1(), &s.input1}, {c.getInput2(), &s.input2}},
+                                               [&] { return thip_hl_elementwiseshift(program_, &s); });
                 aliasResult(op, s.init);
                 return r;
             })

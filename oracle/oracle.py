@@ -352,8 +352,12 @@ _INT_TYPES = (np.int8, np.int16, np.int32)
 ACT_MODES = {"clamp": 0, "abs": 1, "negate": 2, "i2i": 3}
 
 
-def _int_array(a):
+def _int_array(a, truth_values=False):
+    """int8 / int16 / int32 data; with truth_values also uint8 arrays of 0 / 1 (i1 tensors, one byte per element)."""
     a = np.ascontiguousarray(a)
+    if truth_values and a.dtype == np.uint8:
+        assert a.size == 0 or int(a.max()) <= 1, "an i1 tensor holds 0 or 1"
+        return a
     assert a.dtype in [np.dtype(t) for t in _INT_TYPES], a.dtype
     return a
 
@@ -406,6 +410,37 @@ def elementwise_binary(op_type, input1, input2, *, is_unsigned=False):
     assert a.dtype == b.dtype and a.shape == b.shape
     out = np.empty(a.shape, dtype=a.dtype)
     rc = lib().torq_elementwise_binary(BINARY_MODES[op_type], _p(a), _p(b), a.itemsize, int(bool(is_unsigned)), _p(out), ctypes.c_size_t(a.size))
+    assert rc == 0
+    return out
+
+
+def elementwise_compare(op_type, input1, input2, *, is_unsigned=False):
+    """torq_hl.elementwisebinary, comparison / logical modes (the enum's values 6..11): an i1 result as uint8 0 / 1."""
+    a = _int_array(input1, truth_values=True)
+    b = _int_array(input2, truth_values=True)
+    assert a.dtype == b.dtype and a.shape == b.shape
+    out = np.empty(a.shape, dtype=np.uint8)
+    rc = lib().torq_elementwise_compare(int(op_type), _p(a), _p(b), a.itemsize, int(bool(is_unsigned)), _p(out), ctypes.c_size_t(a.size))
+    assert rc == 0
+    return out
+
+
+def elementwise_unary(op_type, input):
+    """torq_hl.elementwiseunary: 3 bitwise not, 12 logical not (on i1 bytes)."""
+    a = _int_array(input, truth_values=True)
+    out = np.empty(a.shape, dtype=a.dtype)
+    rc = lib().torq_elementwise_unary(int(op_type), _p(a), a.itemsize, _p(out), ctypes.c_size_t(a.size))
+    assert rc == 0
+    return out
+
+
+def elementwise_shift(op_type, input1, input2, *, round=False):
+    """torq_hl.elementwiseshift: 0 logical right, 1 logical left, 2 arithmetic right; counts per element in input2."""
+    a = _int_array(input1)
+    b = _int_array(input2)
+    assert a.dtype == b.dtype and a.shape == b.shape
+    out = np.empty(a.shape, dtype=a.dtype)
+    rc = lib().torq_elementwise_shift(int(op_type), int(bool(round)), _p(a), _p(b), a.itemsize, _p(out), ctypes.c_size_t(a.size))
     assert rc == 0
     return out
 

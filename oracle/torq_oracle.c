@@ -637,6 +637,87 @@ int torq_elementwise_binary(int mode, const void *input1, const void *input2, in
     return 0;
 }
 
+/*
+ * The comparisons and logical modes of torq_hl.elementwisebinary (TorqHLAttrs.td:226-231: GREATER 6, GREATER_EQUAL 7,
+ * EQUAL 8, LOGICAL_AND 9, LOGICAL_OR 10, LOGICAL_XOR 11), created from arith.cmpi / cmpf and i1 and / or / xor
+ * (compiler/torq/Conversions/LinalgToTorqHL/ArithToTorqHLPattern.cpp:104-131,181-222; a "less" predicate arrives
+ * with its inputs swapped, "not equal" as EQUAL followed by LOGICAL_NOT :239-251).  The result is an i1 tensor:
+ * one byte per element holding 0 or 1.  What pins the values is the arith op each mode replaces; the NPU's own
+ * encoding of a truth value before its right shift by 16 (ElementWiseBinaryPattern.cpp:108-119) is internal to it.
+ * Logical modes read i1 bytes (any non-zero byte is true).  is_unsigned (16-bit operands only, as :70-79).
+ */
+int torq_elementwise_compare(int mode, const void *input1, const void *input2, int bytes, int is_unsigned, uint8_t *out, size_t count) {
+    if (bad_out_bytes(bytes) || mode < 6 || mode > 11) return -1;
+    if (is_unsigned && bytes != 2) return -1;
+    if (mode >= 9 && bytes != 1) return -1;
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < count; i++) {
+        int64_t a = load_elem(input1, i, bytes), b = load_elem(input2, i, bytes);
+        if (is_unsigned) {
+            a &= 0xffff;
+            b &= 0xffff;
+        }
+        int r;
+        switch (mode) {
+        case 6: r = a > b; break;
+        case 7: r = a >= b; break;
+        case 8: r = a == b; break;
+        case 9: r = (a != 0) && (b != 0); break;
+        case 10: r = (a != 0) || (b != 0); break;
+        default: r = (a != 0) != (b != 0); break;
+        }
+        out[i] = (uint8_t)r;
+    }
+    return 0;
+}
+
+/*
+ * torq_hl.elementwiseunary -- signature TorqHLOps.td:262-273; modes BITWISE_NOT (3) and LOGICAL_NOT (12), created
+ * from arith.xori with an all-ones constant (ArithToTorqHLPattern.cpp:322-340: LOGICAL_NOT when the result is i1);
+ * executed ElementWiseUnaryPattern.cpp:31-36 (ALU op1 BNOT / NOT).  BITWISE_NOT complements every bit of an
+ * int8 / int16 / int32 element; LOGICAL_NOT maps an i1 byte to 1 if it is zero, else 0.
+ */
+int torq_elementwise_unary(int mode, const void *input, int bytes, void *out, size_t count) {
+    if (bad_out_bytes(bytes) || !(mode == 3 || mode == 12) || (mode == 12 && bytes != 1)) return -1;
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < count; i++) {
+        const int64_t a = load_elem(input, i, bytes);
+        store_elem(out, i, mode == 3 ? ~a : (int64_t)(a == 0), bytes);
+    }
+    return 0;
+}
+
+/*
+ * torq_hl.elementwiseshift -- signature TorqHLOps.td:275-289, modes TorqHLAttrs.td:239-246 (LSR 0, LSL 1, ASR 2; ASL
+ * is refused by the lowering, ElementWiseShiftPattern.cpp:77-90); both inputs and the result share one integer type,
+ * input2 holds the shift count of each element.  `round` selects the ACT rounding mode NTP (:91-93); the op stands
+ * for exactly this arithmetic (ArithToTorqHLPattern.cpp:367-379, the linalg body RoundingRightShiftPattern matches):
+ *     r = x >> s;  if (s > 0 && ((x >> (s - 1)) & 1)) r += 1
+ * i.e. round half up, on the signed value for ASR and on the unsigned bit pattern for LSR.  LSL drops the bits
+ * shifted out.  Counts must lie in 0 .. bits-1 (arith.shrsi / shli are undefined beyond); here they are clamped.
+ */
+int torq_elementwise_shift(int mode, int round, const void *input1, const void *input2, int bytes, void *out, size_t count) {
+    if (bad_out_bytes(bytes) || mode < 0 || mode > 2) return -1;
+    const int bits = 8 * bytes;
+    const uint64_t mask = bits == 32 ? 0xffffffffull : ((1ull << bits) - 1);
+#pragma omp parallel for schedule(static)
+    for (size_t i = 0; i < count; i++) {
+        const int64_t x = load_elem(input1, i, bytes);
+        int64_t s = load_elem(input2, i, bytes);
+        s = s < 0 ? 0 : (s > bits - 1 ? bits - 1 : s);
+        int64_t r;
+        if (mode == 1) {
+            r = (int64_t)(((uint64_t)x << s) & mask);
+        } else {
+            const int64_t v = mode == 2 ? x : (int64_t)((uint64_t)x & mask);
+            r = v >> s;
+            if (round && s > 0 && ((v >> (s - 1)) & 1)) r += 1;
+        }
+        store_elem(out, i, r, bytes);  /* keeps the low `bits` bits */
+    }
+    return 0;
+}
+
 /* ---- R2 ---- */
 
 /* compiler/torq/Utils/ConversionUtils.cpp:122-141 (per_channel_sum). */

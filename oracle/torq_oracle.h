@@ -150,6 +150,17 @@ int torq_act(const void *input, int in_bytes, void *out, int out_bytes, size_t c
  * type (bytes = 1, 2, 4); is_unsigned (16-bit only) compares as unsigned. */
 int torq_elementwise_binary(int mode, const void *input1, const void *input2, int bytes, int is_unsigned, void *out, size_t count);
 
+/* torq_hl.elementwisebinary, comparison and logical modes (6 greater, 7 greater-equal, 8 equal on int8 / int16 /
+ * int32; 9 and, 10 or, 11 xor on i1 bytes): the result is an i1 tensor, one byte of 0 or 1 per element. */
+int torq_elementwise_compare(int mode, const void *input1, const void *input2, int bytes, int is_unsigned, uint8_t *out, size_t count);
+
+/* torq_hl.elementwiseunary: 3 bitwise not (int8 / int16 / int32), 12 logical not (i1 bytes). */
+int torq_elementwise_unary(int mode, const void *input, int bytes, void *out, size_t count);
+
+/* torq_hl.elementwiseshift: 0 logical right, 1 logical left, 2 arithmetic right; round: half up on right shifts;
+ * input2 holds each element's count. */
+int torq_elementwise_shift(int mode, int round, const void *input1, const void *input2, int bytes, void *out, size_t count);
+
 /* ---- R2: compile-side parameter derivations ---- */
 
 /* Conv / depthwise / FC: per-channel TOSA (multiplier, shift) -> one global

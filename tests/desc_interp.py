@@ -280,6 +280,20 @@ def run(blob, binding_arrays):
             elif variant == 1:
                 b = view(op["in1"], (1 if bcast == 2 else n) * esz).view(tin)
                 res = orc.mul(a, b, [int(op["bias0"]), int(op["scale0"])], output_zp=zp, output_min=mn, output_max=mx, shift=sh, out_dtype=tout)
+            elif variant in (11, 18):  # bitwise / logical not
+                assert tin == tout
+                res = orc.elementwise_unary(3 if variant == 11 else 12, a.view(np.uint8) if variant == 18 else a)
+                res = res.view(tout)
+            elif 12 <= variant <= 17:  # comparisons and logical ops: a byte of 0 / 1 per element
+                b = view(op["in1"], n * esz).view(tin)
+                assert tout == np.int8
+                if variant >= 15:
+                    a, b = a.view(np.uint8), b.view(np.uint8)
+                res = orc.elementwise_compare(variant - 6, a, b, is_unsigned=bool(int(op["w0"]))).view(np.int8)
+            elif variant >= 19:  # shifts
+                b = view(op["in1"], n * esz).view(tin)
+                assert tin == tout
+                res = orc.elementwise_shift(variant - 19, a, b, round=bool(int(op["w0"])))
             elif variant >= 6:
                 b = view(op["in1"], n * esz).view(tin)
                 assert tin == tout

@@ -37,6 +37,12 @@ def oracle_eval(wl):
         return [orc.mul(x, wl.inputs[1], a.pop("scale_bias"), **a)]
     if kind == "binary":
         return [orc.elementwise_binary(a["op_type"], x, wl.inputs[1], is_unsigned=a["is_unsigned"])]
+    if kind == "compare":
+        return [orc.elementwise_compare(a["op_type"], x, wl.inputs[1], is_unsigned=a["is_unsigned"])]
+    if kind == "unary":
+        return [orc.elementwise_unary(a["op_type"], x)]
+    if kind == "shift":
+        return [orc.elementwise_shift(a["op_type"], x, wl.inputs[1], round=a["round"])]
     if kind == "act":
         return [orc.act(x, a["name"], min_int=a["min_int"], max_int=a["max_int"], out_dtype=a["out_dtype"])]
     if kind == "avgpoolbf16":

@@ -215,3 +215,108 @@ def test_gpu_eltwise(device):
         got, kernels = run_on_gpu(device, wl, via="device" if wl.inputs[0].size > 5000 else "host")
         assert_bit_exact(got[0], oracle_eval(wl)[0], wl.name)
         assert families(kernels) == ["eltwise_int"]
+
+
+# ---- comparisons, logical ops, bitwise not, shifts ------------------------------------------------------------------
+def test_oracle_compare_logical_and_not():
+    """What pins them is the arith op each mode replaces (ArithToTorqHLPattern.cpp:104-131,181-251): numpy's comparison /
+    logical functions on every int8 pair, on int16 / int32 extremes, and on the unsigned views of 16-bit operands."""
+    a8, b8 = np.meshgrid(np.arange(-128, 128, dtype=np.int8), np.arange(-128, 128, dtype=np.int8))
+    for mode, fn in [(6, np.greater), (7, np.greater_equal), (8, np.equal)]:
+        assert np.array_equal(orc.elementwise_compare(mode, a8, b8), fn(a8, b8).astype(np.uint8))
+        for dt in (np.int16, np.int32):
+            info = np.iinfo(dt)
+            x = np.array([info.min, info.max, -1, 0, 1, info.min, 7, -7], dtype=dt)
+            y = np.array([info.max, info.min, 0, -1, 1, info.min, -7, 7], dtype=dt)
+            assert np.array_equal(orc.elementwise_compare(mode, x, y), fn(x, y).astype(np.uint8))
+        x = np.array([-1, 0, 1, -32768, 32767, 5], dtype=np.int16)
+        y = np.array([1, -1, 1, 32767, -32768, 5], dtype=np.int16)
+        assert np.array_equal(orc.elementwise_compare(mode, x, y, is_unsigned=True), fn(x.view(np.uint16), y.view(np.uint16)).astype(np.uint8))
+    t = np.array([0, 0, 1, 1], dtype=np.uint8)
+    u = np.array([0, 1, 0, 1], dtype=np.uint8)
+    assert orc.elementwise_compare(9, t, u).tolist() == [0, 0, 0, 1]
+    assert orc.elementwise_compare(10, t, u).tolist() == [0, 1, 1, 1]
+    assert orc.elementwise_compare(11, t, u).tolist() == [0, 1, 1, 0]
+    assert orc.elementwise_unary(12, t).tolist() == [1, 1, 0, 0]
+    for dt in (np.int8, np.int16, np.int32):
+        info = np.iinfo(dt)
+        x = np.array([info.min, info.max, -1, 0, 1, 85], dtype=dt)
+        assert np.array_equal(orc.elementwise_unary(3, x), np.invert(x))
+        assert np.array_equal(orc.elementwise_unary(3, orc.elementwise_unary(3, x)), x)
+
+
+def test_oracle_shifts():
+    """The rounding right shift is the linalg body the reference's pattern matches (ArithToTorqHLPattern.cpp:367-379):
+    (x >> s) + (s > 0 and bit s-1 of x); checked against exact rationals floor(x / 2^s + 1/2) with Python integers, the
+    logical forms on the unsigned bit patterns, the left shift modulo the width."""
+    for dt, bits in ((np.int8, 8), (np.int16, 16), (np.int32, 32)):
+        info = np.iinfo(dt)
+        rng = np.random.default_rng(bits)
+        xs = np.concatenate([np.array([info.min, info.max, -1, 0, 1, -3, 3, -2, 2, -5, 5], dtype=dt),
+                             rng.integers(info.min, info.max, size=300, endpoint=True, dtype=np.int64).astype(dt)])
+        for s in list(range(bits)):
+            sv = np.full(xs.shape, s, dtype=dt)
+            px = [int(v) for v in xs]
+            ux = [v & ((1 << bits) - 1) for v in px]
+            wrap = lambda v: ((v + (1 << (bits - 1))) % (1 << bits)) - (1 << (bits - 1))
+            assert orc.elementwise_shift(2, xs, sv, round=False).tolist() == [v >> s for v in px]
+            assert orc.elementwise_shift(2, xs, sv, round=True).tolist() == [wrap((2 * v + (1 << s)) >> (s + 1)) if s else v for v in px]
+            assert orc.elementwise_shift(0, xs, sv, round=False).tolist() == [wrap(v >> s) for v in ux]
+            assert orc.elementwise_shift(0, xs, sv, round=True).tolist() == [wrap((2 * v + (1 << s)) >> (s + 1)) if s else wrap(v) for v in ux]
+            assert orc.elementwise_shift(1, xs, sv).tolist() == [wrap((v << s) & ((1 << bits) - 1)) for v in ux]
+    # the matched body itself, on int32
+    x = np.array([5, -5, 6, -6, 7, -7, 2 ** 31 - 1, -2 ** 31], dtype=np.int64)
+    for s in (1, 2, 5, 31):
+        body = (x >> s) + (((x >> (s - 1)) & 1) if s > 0 else 0)
+        got = orc.elementwise_shift(2, x.astype(np.int32), np.full(8, s, dtype=np.int32), round=True)
+        assert got.tolist() == [int(((v + 2 ** 31) % 2 ** 32) - 2 ** 31) for v in body]
+
+
+NEW_ELTWISE = [lambda: w.compare_workload(6), lambda: w.compare_workload(7, dtype=np.int16), lambda: w.compare_workload(8, dtype=np.int32),
+               lambda: w.compare_workload(6, dtype=np.int16, is_unsigned=True), lambda: w.compare_workload(7, shape=(3, 7, 11), dtype=np.int8),
+               lambda: w.compare_workload(9), lambda: w.compare_workload(10, shape=(5, 13)), lambda: w.compare_workload(11),
+               lambda: w.unary_workload(3), lambda: w.unary_workload(3, dtype=np.int16, shape=(3, 5, 7)), lambda: w.unary_workload(3, dtype=np.int32),
+               lambda: w.unary_workload(12),
+               lambda: w.shift_workload(2, round=True), lambda: w.shift_workload(2, dtype=np.int16, round=False), lambda: w.shift_workload(0, dtype=np.int8, round=True),
+               lambda: w.shift_workload(0, dtype=np.int32, round=False), lambda: w.shift_workload(1, dtype=np.int16, shape=(7, 9)), lambda: w.shift_workload(1)]
+
+
+@pytest.mark.parametrize("make", NEW_ELTWISE)
+def test_new_eltwise_descriptors(make):
+    wl = make()
+    blob = wl.program.serialize()
+    outs = [np.zeros(s, dtype=dt) for s, dt in wl.outputs]
+    d = desc_interp.run(blob, list(wl.inputs) + outs)
+    assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)
+    assert [int(o["kind"]) for o in d.ops] == [desc_interp.K_ELTWISE]
+
+
+def test_new_eltwise_rejections():
+    p = Program()
+    a = p.binding(0, (4, 4), np.int8)
+    with pytest.raises(ThipError):
+        p.elementwiseshift(3, a, p.binding(1, (4, 4), np.int8), init=p.binding(2, (4, 4), np.int8))  # ASL is not lowered
+        p.serialize()
+    p = Program()
+    a = p.binding(0, (4, 4), np.int8)
+    with pytest.raises(ThipError):
+        p.elementwisebinary(6, a, p.binding(1, (4, 4), np.int8), init=p.binding(2, (4, 4), np.int8))  # a comparison gives i1
+        p.serialize()
+    p = Program()
+    with pytest.raises(ThipError):
+        p.elementwiseunary(12, p.binding(0, (4, 4), np.int8), init=p.binding(1, (4, 4), np.int8))  # LOGICAL_NOT is for i1
+        p.serialize()
+    p = Program()
+    with pytest.raises(ThipError):
+        p.elementwisebinary(13, p.binding(0, (4,), np.int32), p.binding(1, (4,), np.int32), init=p.binding(2, (4,), np.int32))  # 48-bit SUB
+        p.serialize()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("make", NEW_ELTWISE + [lambda: w.compare_workload(6, shape=(64, 56, 56, 24)), lambda: w.shift_workload(2, shape=(8, 56, 56, 24), round=True)])
+def test_gpu_new_eltwise(device, make):
+    wl = make()
+    print("[gpu-case]", wl.name, flush=True)
+    got, kernels = run_on_gpu(device, wl, via="device" if wl.inputs[0].size > 10000 else "host")
+    assert_bit_exact(got[0], oracle_eval(wl)[0], wl.name)
+    assert families(kernels) == ["eltwise_int"]

@@ -284,8 +284,28 @@ def test_depthwise_shift_boundaries(device, which, monkeypatch):
 
 
 @pytest.mark.parametrize("batch", [1, 8, 64])
-def test_maxpool_config2b(device, batch):
-    check(device, w.maxpool_workload(N=batch), via="device", kernel="maxpool_i8<16>")
+def test_maxpool_config2b(device, batch, monkeypatch):
+    """112x112x64, 2x2 stride 2, at the benchmark's batch sizes: the dedicated 2x2 kernel, and the any-window one."""
+    check(device, w.maxpool_workload(N=batch), via="device", kernel="maxpool2x2_i8")
+    if batch == 8:
+        monkeypatch.setenv("THIP_MAXPOOL_GENERIC", "1")
+        check(device, w.maxpool_workload(N=batch), via="device", kernel="maxpool_i8<16>")
+
+
+def test_maxpool_2x2_kernel_edges(device):
+    """The 2x2 kernel's packed byte maxima on the extremes (-128 and 127 next to each other in every byte position),
+    odd image sizes (the last row / column is never read), and the shapes it must leave to the general kernel."""
+    wl = w.maxpool_workload(N=2, H=9, W=11, C=32)
+    x = wl.inputs[0]
+    x[...] = np.array([-128, 127, -1, 0, 1, -127, 126, -2], dtype=np.int8)[np.arange(x.size).reshape(x.shape) % 8]
+    x[0, ::2, ::2, ::3] = -128
+    x[1, 1::2, :, 1::2] = 127
+    check(device, wl, kernel="maxpool2x2_i8")
+    check(device, w.maxpool_workload(N=1, H=16, W=16, C=16), kernel="maxpool2x2_i8")
+    check(device, w.maxpool_workload(N=1, H=16, W=16, C=16, pad=(0, 1, 0, 1)), kernel="maxpool2x2_i8")    # declared, never reached
+    check(device, w.maxpool_workload(N=1, H=15, W=15, C=16, pad=(0, 1, 0, 1)), kernel="maxpool_i8<16>")   # padding is touched
+    check(device, w.maxpool_workload(N=1, H=16, W=16, C=24), kernel="maxpool_i8<8>")                       # C % 16 != 0
+    check(device, w.maxpool_workload(N=1, H=16, W=16, C=16, kernel=(3, 3), stride=(2, 2)), kernel="maxpool_i8<16>")
 
 
 @pytest.mark.parametrize("kw", [dict(H=8, W=8, C=4), dict(H=8, W=8, C=1), dict(H=32, W=32, C=64, kernel=(3, 3), pad=(1, 1, 1, 1)),
@@ -302,8 +322,11 @@ def test_avgpool(device, kw):
 
 
 @pytest.mark.parametrize("kw", [dict(N=1), dict(N=64), dict(N=1, H=4, W=4, C=1), dict(N=1, H=6, W=8, C=4, zp0=127, zp1=-128), dict(N=1, H=7, W=7, C=33)])
-def test_add(device, kw):
-    check(device, w.add_workload(**kw), via="device", kernel="add_i8")
+def test_add(device, kw, monkeypatch):
+    """The quantised add with the patterns' scale 1 / shift 12 (one folded 32-bit constant), and through the 64-bit ACT stage."""
+    check(device, w.add_workload(**kw), via="device", kernel="add_i8<16,1>")
+    monkeypatch.setenv("THIP_ADD_GENERIC", "1")
+    check(device, w.add_workload(**kw), via="device", kernel="add_i8<16,0>")
 
 
 # ---- programs, properties, error paths ------------------------------------------------------------
@@ -474,7 +497,7 @@ def test_event_log_and_timing(device, tmp_path):
     rows = list(csv.DictReader(log.open()))
     assert list(rows[0].keys()) == ["dispatch_name", "invocation_id", "action_id", "timestamp_us", "event", "kernel"]
     assert len(rows) == 2 * 5 and [r["event"] for r in rows[:2]] == ["NSS_START_BEGIN", "NSS_START_END"]
-    assert all(r["kernel"] == "maxpool_i8<16>" and r["action_id"] == "0" for r in rows)
+    assert all(r["kernel"] == "maxpool2x2_i8" and r["action_id"] == "0" for r in rows)
     assert [int(r["invocation_id"]) for r in rows] == [i // 2 for i in range(10)]
     assert all(int(a["timestamp_us"]) <= int(b["timestamp_us"]) for a, b in zip(rows, rows[1:]))
     # a blocking run on host buffers logs the whole dispatch

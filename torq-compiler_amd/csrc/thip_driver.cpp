@@ -266,7 +266,7 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
         break;
     }
     case kKindEltwise: {
-        EltwiseArgs a{resolve(e, op.in0, bp), (op.variant == kEltMul || op.variant >= kEltAnd) ? resolve(e, op.in1, bp) : nullptr, resolve(e, op.out, bp), (int64_t)op.C,
+        EltwiseArgs a{resolve(e, op.in0, bp), eltwiseTwoInputs((int32_t)op.variant) ? resolve(e, op.in1, bp) : nullptr, resolve(e, op.out, bp), (int64_t)op.C,
                       (int32_t)op.variant, (int32_t)op.gran, op.out_dtype == THIP_DTYPE_I8 ? 1 : op.out_dtype == THIP_DTYPE_I16 ? 2 : 4, op.w1,
                       op.w0, op.bias0, op.scale0, op.output_min, op.output_max, rq};
         err = launchEltwise(a, ctx);
@@ -591,6 +591,14 @@ thip_status_t thip_device_set_event_log(thip_device_t *device, const char *csv_p
         if (!device->eventLog) return fail(THIP_INVALID_ARGUMENT, "cannot open event log %s", csv_path);
         fprintf(device->eventLog, "dispatch_name,invocation_id,action_id,timestamp_us,event,kernel\n");
     }
+    return THIP_OK;
+}
+
+thip_status_t thip_device_mfma_rate(thip_device_t *device, int32_t random_operands, int32_t workgroups, int32_t iterations, double *out_tops) {
+    if (!device || !out_tops) return fail(THIP_INVALID_ARGUMENT, "null argument");
+    if (workgroups <= 0 || iterations <= 0) return fail(THIP_INVALID_ARGUMENT, "workgroups and iterations must be positive");
+    THIP_HIP(hipSetDevice(device->ordinal), "hipSetDevice");
+    THIP_HIP(measureMfmaRate(random_operands, workgroups, iterations, nullptr, out_tops), "measuring the MFMA rate");
     return THIP_OK;
 }
 

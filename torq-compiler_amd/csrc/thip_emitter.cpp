@@ -44,7 +44,7 @@ struct Value {
     }
 };
 
-enum HlKind { kHlConv2d, kHlDepthwise, kHlFullyConnected, kHlMatmul, kHlMaxPool, kHlAvgPool, kHlAdd, kHlTranspose, kHlExpandWeights, kHlFma, kHlMul, kHlAct, kHlBinary };
+enum HlKind { kHlConv2d, kHlDepthwise, kHlFullyConnected, kHlMatmul, kHlMaxPool, kHlAvgPool, kHlAdd, kHlTranspose, kHlExpandWeights, kHlFma, kHlMul, kHlAct, kHlBinary, kHlUnary, kHlShift };
 
 struct HlOp {
     HlKind kind;
@@ -62,6 +62,8 @@ struct HlOp {
         thip_hl_mul_t mul;
         thip_hl_act_t act;
         thip_hl_elementwisebinary_t bin;
+        thip_hl_elementwiseunary_t un;
+        thip_hl_elementwiseshift_t sh;
     } u;
     std::string name;
 };
@@ -83,6 +85,7 @@ static size_t elemSize(int32_t dtype) {
     case THIP_DTYPE_I32: return 4;
     case THIP_DTYPE_BF16: return 2;
     case THIP_DTYPE_F32: return 4;
+    case THIP_DTYPE_I1: return 1;
     default: return 0;
     }
 }
@@ -543,6 +546,8 @@ class Emitter {
     thip_status_t emitMul(const thip_hl_mul_t &c);
     thip_status_t emitAct(const thip_hl_act_t &c, const std::string &name);
     thip_status_t emitBinary(const thip_hl_elementwisebinary_t &c);
+    thip_status_t emitUnary(const thip_hl_elementwiseunary_t &c);
+    thip_status_t emitShift(const thip_hl_elementwiseshift_t &c);
     // Operands of an integer elementwise op: element types, and the record's common fields.
     thip_status_t eltwiseCommon(const char *what, thip_value_t input, thip_value_t init, DescOp *op);
     thip_status_t emitAvgPoolBf16(const thip_hl_avg_pool2d_t &c);
@@ -1327,14 +1332,15 @@ thip_status_t Emitter::eltwiseCommon(const char *what, thip_value_t input, thip_
     const Value *x, *o;
     if (thip_status_t s = checkValue(input, what, &x)) return s;
     if (thip_status_t s = checkValue(init, what, &o)) return s;
-    if (!isIntDtype(x->dtype) || !isIntDtype(o->dtype)) return fail(THIP_UNIMPLEMENTED, "%s: int8 / int16 / int32 tensors only", what);
+    auto carried = [](int32_t d) { return isIntDtype(d) || d == THIP_DTYPE_I1; };
+    if (!carried(x->dtype) || !carried(o->dtype)) return fail(THIP_UNIMPLEMENTED, "%s: int8 / int16 / int32 / i1 tensors only", what);
     if (x->numel() != o->numel() || x->numel() <= 0) return fail(THIP_INVALID_ARGUMENT, "%s: input and init differ in element count", what);
     if (state_[input].nhwcOfNchw) return fail(THIP_UNIMPLEMENTED, "%s: N,C,H,W intermediates are not accepted", what);
     if (!fitsInt32(x->numel())) return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
     memset(op, 0, sizeof(*op));
     op->kind = kKindEltwise;
     op->gran = (uint32_t)elemSize(x->dtype);
-    op->out_dtype = o->dtype;
+    op->out_dtype = o->dtype == THIP_DTYPE_I1 ? THIP_DTYPE_I8 : o->dtype;  // a truth value is a byte to the kernel
     op->N = 1; op->H = 1; op->W = 1;
     op->C = (int32_t)x->numel();
     if (thip_status_t s = literalInput(input, what, &op->in0)) return s;
@@ -1416,21 +1422,75 @@ thip_status_t Emitter::emitBinary(const thip_hl_elementwisebinary_t &c) {
     case 2: variant = kEltXor; break;
     case 4: variant = kEltMin; break;
     case 5: variant = kEltMax; break;
-    default: return fail(THIP_UNIMPLEMENTED, "%s: op_type %d is not on this path (bitwise and / or / xor, minimum, maximum are)", what, (int)c.op_type);
+    case 6: variant = kEltGreater; break;
+    case 7: variant = kEltGreaterEqual; break;
+    case 8: variant = kEltEqual; break;
+    case 9: variant = kEltLogicalAnd; break;
+    case 10: variant = kEltLogicalOr; break;
+    case 11: variant = kEltLogicalXor; break;
+    default: return fail(THIP_UNIMPLEMENTED, "%s: op_type %d is not on this path (bitwise, minimum / maximum, comparisons and logical ops are)", what, (int)c.op_type);
     }
     const Value *a, *b, *init;
     if (thip_status_t s = checkValue(c.input1, "torq_hl.elementwisebinary input1", &a)) return s;
     if (thip_status_t s = checkValue(c.input2, "torq_hl.elementwisebinary input2", &b)) return s;
     if (thip_status_t s = checkValue(c.init, "torq_hl.elementwisebinary init", &init)) return s;
-    if (!isIntDtype(a->dtype) || a->dtype != b->dtype || a->dtype != init->dtype) return fail(THIP_UNIMPLEMENTED, "%s: inputs and init must share one integer type", what);
+    const bool compares = variant >= kEltGreater && variant <= kEltEqual, logical = variant >= kEltLogicalAnd;
+    if (a->dtype != b->dtype) return fail(THIP_UNIMPLEMENTED, "%s: the inputs must share one type", what);
+    if (logical) {
+        if (a->dtype != THIP_DTYPE_I1 || init->dtype != THIP_DTYPE_I1) return fail(THIP_UNIMPLEMENTED, "%s: logical ops take and give i1 tensors", what);
+    } else if (compares) {
+        if (!isIntDtype(a->dtype) || init->dtype != THIP_DTYPE_I1) return fail(THIP_UNIMPLEMENTED, "%s: a comparison takes int8 / int16 / int32 tensors and gives an i1 tensor", what);
+    } else if (!isIntDtype(a->dtype) || a->dtype != init->dtype) {
+        return fail(THIP_UNIMPLEMENTED, "%s: inputs and init must share one integer type", what);
+    }
     if (a->numel() != b->numel() || a->numel() != init->numel()) return fail(THIP_INVALID_ARGUMENT, "%s: operand shapes differ (broadcast is materialised by the patterns)", what);
-    if (c.is_unsigned && a->dtype != THIP_DTYPE_I16) return fail(THIP_UNIMPLEMENTED, "%s: is_unsigned applies to 16-bit operands only", what);
+    if (c.is_unsigned && (a->dtype != THIP_DTYPE_I16 || logical || variant <= kEltXor)) return fail(THIP_UNIMPLEMENTED, "%s: is_unsigned applies to 16-bit minimum / maximum / comparisons only", what);
     if (state_[c.input2].nhwcOfNchw) return fail(THIP_UNIMPLEMENTED, "%s: N,C,H,W intermediates are not accepted", what);
     DescOp op;
     if (thip_status_t s = eltwiseCommon(what, c.input1, c.init, &op)) return s;
     if (thip_status_t s = literalInput(c.input2, "torq_hl.elementwisebinary input2", &op.in1)) return s;
     op.variant = variant;
     op.w0 = c.is_unsigned ? 1 : 0;
+    ops_.push_back(op);
+    return THIP_OK;
+}
+
+thip_status_t Emitter::emitUnary(const thip_hl_elementwiseunary_t &c) {
+    const char *what = "torq_hl.elementwiseunary";
+    if (c.op_type != 3 && c.op_type != 12) return fail(THIP_UNIMPLEMENTED, "%s: op_type %d is not a unary mode (BITWISE_NOT 3 and LOGICAL_NOT 12 are)", what, (int)c.op_type);
+    const Value *x, *init;
+    if (thip_status_t s = checkValue(c.input, "torq_hl.elementwiseunary input", &x)) return s;
+    if (thip_status_t s = checkValue(c.init, "torq_hl.elementwiseunary init", &init)) return s;
+    if (x->dtype != init->dtype) return fail(THIP_UNIMPLEMENTED, "%s: input and init must share one type", what);
+    if (c.op_type == 3 ? !isIntDtype(x->dtype) : x->dtype != THIP_DTYPE_I1) return fail(THIP_UNIMPLEMENTED, "%s: BITWISE_NOT takes integers, LOGICAL_NOT i1", what);
+    DescOp op;
+    if (thip_status_t s = eltwiseCommon(what, c.input, c.init, &op)) return s;
+    op.variant = c.op_type == 3 ? kEltNot : kEltLogicalNot;
+    ops_.push_back(op);
+    return THIP_OK;
+}
+
+thip_status_t Emitter::emitShift(const thip_hl_elementwiseshift_t &c) {
+    const char *what = "torq_hl.elementwiseshift";
+    uint32_t variant;
+    switch (c.op_type) {  // ShiftModeEnum, compiler/torq/Dialect/TorqHL/TorqHLAttrs.td:239-246
+    case 0: variant = kEltLsr; break;
+    case 1: variant = kEltLsl; break;
+    case 2: variant = kEltAsr; break;
+    default: return fail(THIP_UNIMPLEMENTED, "%s: shift mode %d is not lowered (LSR 0, LSL 1 and ASR 2 are)", what, (int)c.op_type);
+    }
+    const Value *a, *b, *init;
+    if (thip_status_t s = checkValue(c.input1, "torq_hl.elementwiseshift input1", &a)) return s;
+    if (thip_status_t s = checkValue(c.input2, "torq_hl.elementwiseshift input2", &b)) return s;
+    if (thip_status_t s = checkValue(c.init, "torq_hl.elementwiseshift init", &init)) return s;
+    if (!isIntDtype(a->dtype) || a->dtype != b->dtype || a->dtype != init->dtype) return fail(THIP_UNIMPLEMENTED, "%s: inputs and init must share one integer type", what);
+    if (a->numel() != b->numel() || a->numel() != init->numel()) return fail(THIP_INVALID_ARGUMENT, "%s: operand shapes differ", what);
+    if (state_[c.input2].nhwcOfNchw) return fail(THIP_UNIMPLEMENTED, "%s: N,C,H,W intermediates are not accepted", what);
+    DescOp op;
+    if (thip_status_t s = eltwiseCommon(what, c.input1, c.init, &op)) return s;
+    if (thip_status_t s = literalInput(c.input2, "torq_hl.elementwiseshift input2", &op.in1)) return s;
+    op.variant = variant;
+    op.w0 = c.round ? 1 : 0;
     ops_.push_back(op);
     return THIP_OK;
 }
@@ -1692,6 +1752,8 @@ void Emitter::planChannelPadding() {
         case kHlMul: bar(op.u.mul.input1); bar(op.u.mul.input2); bar(op.u.mul.init); break;
         case kHlAct: bar(op.u.act.input); bar(op.u.act.init); break;
         case kHlBinary: bar(op.u.bin.input1); bar(op.u.bin.input2); bar(op.u.bin.init); break;
+        case kHlUnary: bar(op.u.un.input); bar(op.u.un.init); break;
+        case kHlShift: bar(op.u.sh.input1); bar(op.u.sh.input2); bar(op.u.sh.init); break;
         }
     }
     // one verdict per group: every member an int8 rank-4 intermediate, all uses agreeing on C
@@ -1744,6 +1806,8 @@ void Emitter::planExpandFolding() {
         case kHlMul: read(op.u.mul.input1); read(op.u.mul.input2); break;
         case kHlAct: read(op.u.act.input); break;
         case kHlBinary: read(op.u.bin.input1); read(op.u.bin.input2); break;
+        case kHlUnary: read(op.u.un.input); break;
+        case kHlShift: read(op.u.sh.input1); read(op.u.sh.input2); break;
         }
     }
     auto constant = [&](thip_value_t v) { return v >= 0 && (size_t)v < n && prog_.values[(size_t)v].kind == kValueConstant; };
@@ -1813,6 +1877,8 @@ thip_status_t Emitter::run(void **outBlob, size_t *outSize) {
         case kHlMul: s = emitMul(op.u.mul); break;
         case kHlAct: s = emitAct(op.u.act, op.name); break;
         case kHlBinary: s = emitBinary(op.u.bin); break;
+        case kHlUnary: s = emitUnary(op.u.un); break;
+        case kHlShift: s = emitShift(op.u.sh); break;
         }
         if (s != THIP_OK) return s;
     }
@@ -1966,6 +2032,8 @@ THIP_DEFINE_HL(thip_hl_expand_weights, thip_hl_expand_weights_t, kHlExpandWeight
 THIP_DEFINE_HL(thip_hl_fma, thip_hl_fma_t, kHlFma, fma)
 THIP_DEFINE_HL(thip_hl_mul, thip_hl_mul_t, kHlMul, mul)
 THIP_DEFINE_HL(thip_hl_elementwisebinary, thip_hl_elementwisebinary_t, kHlBinary, bin)
+THIP_DEFINE_HL(thip_hl_elementwiseunary, thip_hl_elementwiseunary_t, kHlUnary, un)
+THIP_DEFINE_HL(thip_hl_elementwiseshift, thip_hl_elementwiseshift_t, kHlShift, sh)
 
 thip_status_t thip_hl_act(thip_program_t *program, const thip_hl_act_t *op) {
     if (!program || !op || !op->name) return fail(THIP_INVALID_ARGUMENT, "thip_hl_act: null argument");

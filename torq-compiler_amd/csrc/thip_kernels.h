@@ -38,6 +38,8 @@ struct Tuning {
     int fcWideU = 0;                // THIP_FC_WIDE_U: k-steps per register buffer of the wide bf16 kernel
     bool noFcDeep = false;          // THIP_NO_FC_DEEP
     bool noFcWide = false;          // THIP_NO_FC_WIDE
+    bool addGeneric = false;        // THIP_ADD_GENERIC: the quantised add always through the 64-bit ACT stage
+    bool maxpoolGeneric = false;    // THIP_MAXPOOL_GENERIC: the any-window max pool kernel also for 2 x 2 stride 2
 };
 Tuning tuningFromEnvironment();
 
@@ -193,6 +195,10 @@ inline size_t fcBf16WorkspaceCounterBytes(int M, int N, int ksplit) {
 
 // The library's static scratch array (device memory that needs no allocation): its size, its address on the
 // current device (ask once per device, with that device current), and a zero fill that is a kernel.
+// Sustained v_mfma_i32_32x32x32_i8 rate (TOP/s, 1 multiply-add = 2 ops) of `blocks` workgroups of four waves that
+// do nothing else, on constant or on random operand bytes.  Allocates and frees its own few KiB.
+hipError_t measureMfmaRate(int randomOperands, int blocks, int iterations, hipStream_t stream, double *outTops);
+
 constexpr size_t kStaticScratchBytes = 2u << 20;
 hipError_t staticScratchAddress(void **out);
 hipError_t launchZeroFill(void *dst, size_t bytes, hipStream_t stream);
@@ -201,11 +207,25 @@ hipError_t launchZeroFill(void *dst, size_t bytes, hipStream_t stream);
 // input of one element is broadcast); both with ONE (bias, scale) pair.  clamp / abs / negate / i2i: the input
 // passed through the mode, then clipped to [lo, hi] and truncated to the output type.
 // and / or / xor / min / max: two inputs and the output of one type, no ACT stage; w0 != 0 (16-bit only): min / max
-// compare as unsigned.
+// compare as unsigned.  not: bitwise complement.  greater / greater-equal / equal: two inputs of one integer type
+// (w0 != 0, 16-bit only: unsigned), the result one byte of 0 or 1 per element; logical and / or / xor / not: such
+// bytes in (non-zero = true), such bytes out.  lsr / lsl / asr: in0 shifted by the counts in in1 (clamped to
+// 0 .. bits-1), same type out; w0 != 0: right shifts round half up.
 enum EltwiseOp : int32_t {
     kEltFma = 0, kEltMul = 1, kEltClamp = 2, kEltAbs = 3, kEltNegate = 4, kEltCast = 5,
     kEltAnd = 6, kEltOr = 7, kEltXor = 8, kEltMin = 9, kEltMax = 10,
+    kEltNot = 11, kEltGreater = 12, kEltGreaterEqual = 13, kEltEqual = 14,
+    kEltLogicalAnd = 15, kEltLogicalOr = 16, kEltLogicalXor = 17, kEltLogicalNot = 18,
+    kEltLsr = 19, kEltLsl = 20, kEltAsr = 21,
+    kEltLast = kEltAsr,
 };
+// Ops that read a second tensor, and those whose result has the inputs' element type.
+__host__ __device__ inline bool eltwiseTwoInputs(int32_t op) {
+    return op == kEltMul || (op >= kEltAnd && op <= kEltMax) || (op >= kEltGreater && op <= kEltLogicalXor) || op >= kEltLsr;
+}
+__host__ __device__ inline bool eltwiseSameType(int32_t op) {
+    return (op >= kEltAnd && op <= kEltNot) || (op >= kEltLogicalAnd && op <= kEltLogicalNot) || op >= kEltLsr;
+}
 struct EltwiseArgs {
     const void *in0;
     const void *in1;  // mul and the two-input ops

@@ -358,7 +358,7 @@ __host__ __device__ inline bool residualAddFolded(int32_t w0, int32_t w1, int32_
 // register groups between the wave halves so that a lane owns 16 consecutive channels of its row
 // (see igemm_stream_i8), and the lane stores them as one 128-bit word.  Only the (bias, scale)
 // vectors pass through LDS.
-template <int WTM, int WTN, int NW, int BN, bool ADD>  // ADD: a residual add behind the requant (IgemmArgs::skip)
+template <int WTM, int WTN, int NW, int BN, bool ADD, bool PLAIN>  // ADD: a residual add behind the requant (IgemmArgs::skip); PLAIN: see requantWideT0
 __device__ __forceinline__ void igemmEpilogueDirect(v16i (&acc)[WTN / 32][WTM / 32], int8_t *smem, const IgemmArgs &p, int m0,
                                                     int n0, int wm, int wn, int32_t myBias, int32_t myScale) {
     blockBarrier();
@@ -370,7 +370,7 @@ __device__ __forceinline__ void igemmEpilogueDirect(v16i (&acc)[WTN / 32][WTM / 
         ldsScale[tid] = myScale;
     }
     __syncthreads();
-    const WideRequant wrq = wideRequant(p.rq);  // plain (the launcher checks): no pre-shift, zero point folded
+    const WideRequant wrq = wideRequant(p.rq);  // a 32-bit tail applies (the launcher checks); PLAIN: no pre-shift, no clamp of acc + bias, zero point folded
     const long long addRnd = roundTerm(p.arq.shift);
     int32_t addFolded = 0;
     const bool addFast = ADD && residualAddFolded(p.add_w0, p.add_w1, p.add_bias, p.add_scale, p.arq, &addFolded);
@@ -392,7 +392,7 @@ __device__ __forceinline__ void igemmEpilogueDirect(v16i (&acc)[WTN / 32][WTM / 
                 int32_t v[4];
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    v[e] = requantWideT0<true>((int32_t)((uint32_t)acc[j][i][4 * q + e] + (uint32_t)b4[q][e]), s4[q][e], wrq);
+                    v[e] = requantWideT0<PLAIN>((int32_t)((uint32_t)acc[j][i][4 * q + e] + (uint32_t)b4[q][e]), s4[q][e], wrq);
                 }
                 d4[q] = packBytes(v[0], v[1], v[2], v[3]);
             }
@@ -764,9 +764,11 @@ __device__ __forceinline__ void waitVmcnt() {
     asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
 }
 
-// DIRECT selects the epilogue: in registers (int8 output, N % 16 == 0, plain 32-bit requant tail: the launcher
-// checks) or staged through LDS (everything else).
-template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, bool DIRECT, bool ADD = false>
+// DIRECT selects the epilogue: 0 staged through LDS (any output type, ragged N, the 64-bit requant tail), or in
+// registers (int8 output, N % 16 == 0: the launcher checks) with 1 the plain 32-bit tail or 2 the general 32-bit tail
+// (a pre-shift, a clamp of acc + bias or a zero point that does not fold: e.g. small shifts under large scales,
+// where every result beyond a small |acc + bias| saturates).
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, int DIRECT, bool ADD = false>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_dense_i8(IgemmArgs p) {
     constexpr int BK = 64;
     constexpr int NW = WAVES_M * WAVES_N;
@@ -969,7 +971,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
     for (; kt < KT; kt++) step(kt, std::false_type{});
 
     if (DIRECT) {
-        igemmEpilogueDirect<WTM, WTN, NW, BN, ADD>(acc, smem, p, m0, n0, wm, wn, myBias, myScale);
+        igemmEpilogueDirect<WTM, WTN, NW, BN, ADD, DIRECT == 1>(acc, smem, p, m0, n0, wm, wn, myBias, myScale);
     } else {
         igemmEpilogue<WTM, WTN, NW, BN>(acc, smem, p, m0, n0, wm, wn, myBias, myScale);
     }
@@ -1452,7 +1454,7 @@ static hipError_t launchIgemmLoader(const IgemmArgs &a, const LaunchCtx &ctx) {
     }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, bool DIRECT, bool ADD = false>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, int DIRECT, bool ADD = false>
 static hipError_t launchIgemmDenseE(const IgemmArgs &a, const LaunchCtx &ctx) {
     // the stage ring, reused by the epilogue as staging slices (one per wave) plus bias/scale
     constexpr size_t ring = (size_t)STAGES * (BM + BN) * 64;
@@ -1472,22 +1474,27 @@ static hipError_t launchIgemmDenseE(const IgemmArgs &a, const LaunchCtx &ctx) {
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU>
 static hipError_t launchIgemmDense(const IgemmArgs &a, const LaunchCtx &ctx) {
-    // the in-register epilogue takes the plain 32-bit tail only (what wideRequant() calls plain)
+    // the in-register epilogue takes the 32-bit requant tails: the plain one (what wideRequant() calls plain), or, on
+    // the large tiles, the general one (any shift of 32 and up, or a smaller one that the record's pre_shift lifts to 33)
     const bool plain = a.rq.shift >= 33 && a.rq.shift <= 45 && a.rq.pre_shift == 0 && a.rq.t0_clamp == 0 &&
                        a.rq.out_zp >= -32768 && a.rq.out_zp <= 32767 && a.rq.out_min <= a.rq.out_max;
-    const bool direct = a.out_dtype == kDtypeI8 && a.N % 16 == 0 && ((uintptr_t)a.out & 15) == 0 && plain &&
-                        !ctx.tuning->noDirectEpilogue;
+    const bool wide = (a.rq.shift >= 32 || (a.rq.pre_shift > 0 && a.rq.shift + a.rq.pre_shift == 33)) && a.rq.out_min <= a.rq.out_max;
+    const bool inRegisters = a.out_dtype == kDtypeI8 && a.N % 16 == 0 && ((uintptr_t)a.out & 15) == 0 && !ctx.tuning->noDirectEpilogue;
+    const bool direct = inRegisters && plain;
     if (a.skip != nullptr) {
         // a residual add: the in-register epilogue of the small tile only (what a network's late, small layers take)
         if constexpr (BM == 64 && BN == 64) {
             if (!direct || ((uintptr_t)a.skip & 15) != 0) return hipErrorInvalidValue;
-            return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, true, true>(a, ctx);
+            return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, 1, true>(a, ctx);
         } else {
             return hipErrorInvalidValue;
         }
     }
-    return direct ? launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, true>(a, ctx)
-                  : launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, false>(a, ctx);
+    if (direct) return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, 1>(a, ctx);
+    if constexpr (BM * BN >= 128 * 128) {
+        if (inRegisters && wide) return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, 2>(a, ctx);
+    }
+    return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, 0>(a, ctx);
 }
 
 hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, const LaunchCtx &ctx) {
@@ -2357,6 +2364,45 @@ __global__ __launch_bounds__(256) void maxpool_i8(MaxPoolArgs p, WorkSplit ws) {
     *(typename ByteVec<VEC>::type *)(p.out + (((size_t)n * p.OH + oy) * p.OW + ox) * p.C + c0) = o.v;
 }
 
+// Signed maximum of the four bytes of two dwords.  Bytes 0 and 2 move to the upper byte of their 16-bit half (a byte
+// permute), bytes 1 and 3 are masked in place; a packed 16-bit signed maximum then orders each pair exactly as the
+// bytes order (the lower byte of every half is zero on both sides).  Halves stay split between calls.
+struct SplitBytes {
+    uint32_t even, odd;  // [0, b0, 0, b2] and [0, b1, 0, b3] as bytes 0..3
+};
+__device__ __forceinline__ SplitBytes splitBytes(uint32_t x) {
+    return SplitBytes{__builtin_amdgcn_perm(x, x, 0x020c000cu), x & 0xff00ff00u};
+}
+typedef short v2s __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pkMaxI16(uint32_t a, uint32_t b) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(v2s, a), __builtin_bit_cast(v2s, b)));
+}
+__device__ __forceinline__ SplitBytes maxSplit(SplitBytes a, SplitBytes b) { return SplitBytes{pkMaxI16(a.even, b.even), pkMaxI16(a.odd, b.odd)}; }
+__device__ __forceinline__ uint32_t joinBytes(SplitBytes m) { return __builtin_amdgcn_perm(m.odd, m.even, 0x07030501u); }
+
+// The common pooling window as its own kernel: 2 x 2, stride 2, no padding touched, C % 16 == 0, no clamp beyond the
+// int8 range.  A thread owns 16 channels of one output pixel: its four 128-bit loads are issued together (the
+// general kernel walks a run-time window, one load in flight per thread) and the maxima are taken on packed bytes.
+__global__ __launch_bounds__(256) void maxpool2x2_i8(MaxPoolArgs p, WorkSplit ws) {
+    const int cg = p.C / 16;
+    const long long total = (long long)p.N * p.OH * p.OW * cg;
+    const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (t >= total) return;
+    int cgi, ox, oy, n;
+    splitWork(t, ws, cgi, ox, oy, n);
+    const int8_t *src = p.in + (((size_t)n * p.H + 2 * oy) * p.W + 2 * ox) * p.C + cgi * 16;
+    const size_t row = (size_t)p.W * p.C;
+    const v4i a = *(const v4i *)src, b = *(const v4i *)(src + p.C), c = *(const v4i *)(src + row), d = *(const v4i *)(src + row + p.C);
+    v4i o;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const SplitBytes m = maxSplit(maxSplit(splitBytes((uint32_t)a[q]), splitBytes((uint32_t)b[q])),
+                                      maxSplit(splitBytes((uint32_t)c[q]), splitBytes((uint32_t)d[q])));
+        o[q] = (int)joinBytes(m);
+    }
+    *(v4i *)(p.out + (((size_t)n * p.OH + oy) * p.OW + ox) * p.C + cgi * 16) = o;
+}
+
 template <int VEC>
 static hipError_t launchMaxPoolV(const MaxPoolArgs &a, const LaunchCtx &ctx) {
     const long long total = (long long)a.N * a.OH * a.OW * (a.C / VEC);
@@ -2372,7 +2418,15 @@ hipError_t launchMaxPool(const MaxPoolArgs &a, const LaunchCtx &ctx) {
     }
     if (!a.in || !a.out) return hipErrorInvalidValue;
     if ((long long)a.N * a.OH * a.OW * a.C >= (1LL << 40)) return hipErrorInvalidValue;
-    switch (pickVec(a.C, a.in, a.out, nullptr)) {
+    const int vec = pickVec(a.C, a.in, a.out, nullptr);
+    if (vec == 16 && a.KH == 2 && a.KW == 2 && a.SH == 2 && a.SW == 2 && a.PT == 0 && a.PL == 0 && 2 * a.OH <= a.H && 2 * a.OW <= a.W &&
+        a.out_min <= -128 && a.out_max >= 127 && !ctx.tuning->maxpoolGeneric) {
+        const long long total = (long long)a.N * a.OH * a.OW * (a.C / 16);
+        const WorkSplit ws = makeWorkSplit(total, a.C / 16, a.OW, a.OH);
+        THIP_ENQUEUE(ctx, "maxpool2x2_i8", maxpool2x2_i8, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, a, ws);
+        return hipGetLastError();
+    }
+    switch (vec) {
     case 16: return launchMaxPoolV<16>(a, ctx);
     case 8: return launchMaxPoolV<8>(a, ctx);
     case 4: return launchMaxPoolV<4>(a, ctx);
@@ -2444,22 +2498,29 @@ hipError_t launchAvgPool(const AvgPoolArgs &a, const LaunchCtx &ctx) {
     }
 }
 
-template <int VEC>
-__global__ __launch_bounds__(256) void add_i8(AddArgs p) {
+// FAST (16 bytes per thread only): the add's scale is 1 and its 32-bit sum cannot overflow, so bias, rounding term
+// and zero point are one constant and a value costs two multiply-adds, a shift and a clamp (residualAdd16).
+template <int VEC, bool FAST>
+__global__ __launch_bounds__(256) void add_i8(AddArgs p, int32_t folded) {
     const long long t = (long long)blockIdx.x * 256 + threadIdx.x;
     const long long i0 = t * VEC;
     if (i0 >= p.count) return;
     const long long rnd = roundTerm(p.rq.shift);
     if (i0 + VEC <= p.count) {
-        Pack<VEC> a, b, o;
-        a.v = *(const typename ByteVec<VEC>::type *)(p.in0 + i0);
-        b.v = *(const typename ByteVec<VEC>::type *)(p.in1 + i0);
+        if constexpr (FAST && VEC == 16) {
+            const v4i a = *(const v4i *)(p.in0 + i0), b = *(const v4i *)(p.in1 + i0);
+            *(v4i *)(p.out + i0) = residualAdd16<true>(a, b, false, p.w0, p.w1, p.bias, p.scale, rnd, p.rq, folded);
+        } else {
+            Pack<VEC> a, b, o;
+            a.v = *(const typename ByteVec<VEC>::type *)(p.in0 + i0);
+            b.v = *(const typename ByteVec<VEC>::type *)(p.in1 + i0);
 #pragma unroll
-        for (int v = 0; v < VEC; v++) {
-            const int32_t acc = (int32_t)a.b[v] * p.w0 + (int32_t)b.b[v] * p.w1;
-            o.b[v] = (int8_t)requant(acc, p.bias, p.scale, rnd, p.rq);
+            for (int v = 0; v < VEC; v++) {
+                const int32_t acc = (int32_t)a.b[v] * p.w0 + (int32_t)b.b[v] * p.w1;
+                o.b[v] = (int8_t)requant(acc, p.bias, p.scale, rnd, p.rq);
+            }
+            *(typename ByteVec<VEC>::type *)(p.out + i0) = o.v;
         }
-        *(typename ByteVec<VEC>::type *)(p.out + i0) = o.v;
     } else {
         for (long long i = i0; i < p.count; i++) {
             const int32_t acc = (int32_t)p.in0[i] * p.w0 + (int32_t)p.in1[i] * p.w1;
@@ -2473,9 +2534,16 @@ hipError_t launchAdd(const AddArgs &a, const LaunchCtx &ctx) {
     const uintptr_t bits = (uintptr_t)a.in0 | (uintptr_t)a.in1 | (uintptr_t)a.out;
     if ((bits & 15) == 0) {
         const long long threads = (a.count + 15) / 16;
-        THIP_ENQUEUE(ctx, "add_i8<16>", (add_i8<16>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, a);
+        const dim3 grid((unsigned)((threads + 255) / 256));
+        int32_t folded = 0;
+        // what the patterns emit (scale 1, shift 12, int8 clamp) folds; anything else takes the 64-bit ACT stage
+        if (a.rq.out_min >= -128 && a.rq.out_max <= 127 && residualAddFolded(a.w0, a.w1, a.bias, a.scale, a.rq, &folded) && !ctx.tuning->addGeneric) {
+            THIP_ENQUEUE(ctx, "add_i8<16,1>", (add_i8<16, true>), grid, dim3(256), 0, a, folded);
+        } else {
+            THIP_ENQUEUE(ctx, "add_i8<16,0>", (add_i8<16, false>), grid, dim3(256), 0, a, 0);
+        }
     } else {
-        THIP_ENQUEUE(ctx, "add_i8<1>", (add_i8<1>), dim3((unsigned)((a.count + 255) / 256)), dim3(256), 0, a);
+        THIP_ENQUEUE(ctx, "add_i8<1,0>", (add_i8<1, false>), dim3((unsigned)((a.count + 255) / 256)), dim3(256), 0, a, 0);
     }
     return hipGetLastError();
 }
@@ -2603,13 +2671,15 @@ __global__ __launch_bounds__(256) void eltwise_int(EltwiseArgs p) {
     const bool whole = i0 + VEC <= p.count;
     EltVec<TIN, VEC> a, b;
     EltVec<TOUT, VEC> o;
+#pragma unroll
+    for (int v = 0; v < VEC; v++) b.e[v] = (TIN)0;  // the one-input ops never look at it
     if (whole && p.bcast != 1) {
         a = *(const EltVec<TIN, VEC> *)(in0 + i0);
     } else {
 #pragma unroll
         for (int v = 0; v < VEC; v++) a.e[v] = p.bcast == 1 ? in0[0] : (i0 + v < p.count ? in0[i0 + v] : (TIN)0);
     }
-    if (p.op == kEltMul || p.op >= kEltAnd) {
+    if (eltwiseTwoInputs(p.op)) {
         if (whole && p.bcast != 2) {
             b = *(const EltVec<TIN, VEC> *)(in1 + i0);
         } else {
@@ -2629,6 +2699,35 @@ __global__ __launch_bounds__(256) void eltwise_int(EltwiseArgs p) {
                 o.e[v] = (TOUT)requantT0<kMode>(t0, p.scale, rnd, p.rq, wrq);
             }
         });
+    } else if (p.op >= kEltNot) {
+        constexpr int BITS = 8 * (int)sizeof(TIN);
+        const uint32_t typeMask = BITS == 32 ? 0xffffffffu : ((1u << BITS) - 1u);
+#pragma unroll
+        for (int v = 0; v < VEC; v++) {
+            const int32_t x = (int32_t)a.e[v], y = (int32_t)b.e[v];
+            int32_t r;
+            if (p.op == kEltNot) {
+                r = ~x;
+            } else if (p.op <= kEltEqual) {
+                const int32_t kx = p.w0 ? (x & 0xffff) : x, ky = p.w0 ? (y & 0xffff) : y;
+                r = p.op == kEltGreater ? kx > ky : p.op == kEltGreaterEqual ? kx >= ky : kx == ky;
+            } else if (p.op <= kEltLogicalNot) {
+                const bool tx = x != 0, ty = y != 0;
+                r = p.op == kEltLogicalAnd ? (tx && ty) : p.op == kEltLogicalOr ? (tx || ty) : p.op == kEltLogicalXor ? (tx != ty) : !tx;
+            } else {
+                int32_t s = y < 0 ? 0 : (y > BITS - 1 ? BITS - 1 : y);
+                if (p.op == kEltLsl) {
+                    r = (int32_t)((uint32_t)x << s);
+                } else {
+                    // arithmetic: the sign-extended value; logical: the element's own bits, zero-extended
+                    const long long val = p.op == kEltAsr ? (long long)x : (long long)((uint32_t)x & typeMask);
+                    long long q = val >> s;
+                    if (p.w0 && s > 0 && ((val >> (s - 1)) & 1)) q += 1;
+                    r = (int32_t)q;
+                }
+            }
+            o.e[v] = (TOUT)r;
+        }
     } else if (p.op >= kEltAnd) {
         const int32_t mask = p.w0 ? 0xffff : -1;  // unsigned 16-bit comparison
 #pragma unroll
@@ -2661,7 +2760,7 @@ __global__ __launch_bounds__(256) void eltwise_int(EltwiseArgs p) {
 template <typename TIN, typename TOUT>
 static hipError_t launchEltwiseT(const EltwiseArgs &a, const LaunchCtx &ctx) {
     constexpr int VEC = sizeof(TIN) == 1 && sizeof(TOUT) == 1 ? 16 : 8;
-    const uintptr_t bits = (uintptr_t)a.in0 | ((a.op == kEltMul || a.op >= kEltAnd) ? (uintptr_t)a.in1 : 0);
+    const uintptr_t bits = (uintptr_t)a.in0 | (eltwiseTwoInputs(a.op) ? (uintptr_t)a.in1 : 0);
     const bool aligned = (bits & (sizeof(TIN) * VEC - 1)) == 0 && (((uintptr_t)a.out) & (sizeof(TOUT) * VEC - 1)) == 0;
     if (aligned) {
         const long long threads = (a.count + VEC - 1) / VEC;
@@ -2673,11 +2772,14 @@ static hipError_t launchEltwiseT(const EltwiseArgs &a, const LaunchCtx &ctx) {
 }
 
 hipError_t launchEltwise(const EltwiseArgs &a, const LaunchCtx &ctx) {
-    if (!a.in0 || !a.out || a.count <= 0 || a.count >= (1LL << 39) || a.op < kEltFma || a.op > kEltMax) return hipErrorInvalidValue;
-    const bool two = a.op == kEltMul || a.op >= kEltAnd;
+    if (!a.in0 || !a.out || a.count <= 0 || a.count >= (1LL << 39) || a.op < kEltFma || a.op > kEltLast) return hipErrorInvalidValue;
+    const bool two = eltwiseTwoInputs(a.op);
     if (two && (!a.in1 || a.bcast < 0 || a.bcast > 2)) return hipErrorInvalidValue;
     if (a.op != kEltMul && a.bcast != 0) return hipErrorInvalidValue;
-    if (a.op >= kEltAnd && (a.in_bytes != a.out_bytes || (a.w0 != 0 && a.in_bytes != 2))) return hipErrorInvalidValue;
+    if (eltwiseSameType(a.op) && a.in_bytes != a.out_bytes) return hipErrorInvalidValue;
+    if (a.op >= kEltAnd && a.op <= kEltEqual && a.w0 != 0 && a.in_bytes != 2) return hipErrorInvalidValue;  // unsigned: 16-bit only
+    if (a.op >= kEltGreater && a.op <= kEltEqual && a.out_bytes != 1) return hipErrorInvalidValue;            // a truth value is one byte
+    if (a.op >= kEltLogicalAnd && a.op <= kEltLogicalNot && a.in_bytes != 1) return hipErrorInvalidValue;
     if ((((uintptr_t)a.in0) & (a.in_bytes - 1)) || (((uintptr_t)a.out) & (a.out_bytes - 1))) return hipErrorInvalidValue;
     if (two && (((uintptr_t)a.in1) & (a.in_bytes - 1))) return hipErrorInvalidValue;
     switch (a.in_bytes * 8 + a.out_bytes) {
@@ -3154,6 +3256,85 @@ hipError_t launchZeroFill(void *dst, size_t bytes, hipStream_t stream) {
     return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// Calibration: what the matrix cores sustain on this GPU with nothing else going on.  Every wave owns a 4 x 4 grid of
+// 32 x 32 accumulators (the register layout of the 256 x 256 GEMM tile) and issues v_mfma_i32_32x32x32_i8 back to
+// back on operands it loaded once; no memory traffic inside the loop.  The rate depends on the operand VALUES: the
+// card runs against a power limit, and random bytes toggle far more of the datapath than constants do.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void mfma_rate_i8(int iterations, const v4i *__restrict__ operands, int *__restrict__ sink) {
+    v16i acc[4][4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[j][i][r] = 0;
+        }
+    }
+    v4i a[4], b[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        a[i] = operands[threadIdx.x + 256 * i];
+        b[i] = operands[threadIdx.x + 256 * (4 + i)];
+    }
+    for (int it = 0; it < iterations; it++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(b[j], a[i], acc[j][i], 0, 0, 0);
+        }
+        // the operands stay live and opaque, so the loop is not folded
+        asm volatile("" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
+    }
+    int s = 0;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) s += acc[j][i][r];
+        }
+    }
+    sink[blockIdx.x * 256 + threadIdx.x] = s;
+}
+
+hipError_t measureMfmaRate(int randomOperands, int blocks, int iterations, hipStream_t stream, double *outTops) {
+    if (blocks <= 0 || blocks > 65536 || iterations <= 0 || !outTops) return hipErrorInvalidValue;
+    constexpr size_t kOperandBytes = 256 * 8 * 16;
+    uint8_t host[kOperandBytes];
+    uint32_t x = 0x9e3779b9u;
+    for (size_t i = 0; i < kOperandBytes; i++) {
+        x ^= x << 13; x ^= x >> 17; x ^= x << 5;  // xorshift: any uniform bytes will do
+        host[i] = randomOperands ? (uint8_t)(x >> 11) : (uint8_t)1;
+    }
+    v4i *operands = nullptr;
+    int *sink = nullptr;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipError_t err = hipMalloc((void **)&operands, kOperandBytes);
+    if (err == hipSuccess) err = hipMalloc((void **)&sink, (size_t)blocks * 256 * 4);
+    if (err == hipSuccess) err = hipMemcpy(operands, host, kOperandBytes, hipMemcpyHostToDevice);
+    if (err == hipSuccess) err = hipEventCreate(&e0);
+    if (err == hipSuccess) err = hipEventCreate(&e1);
+    if (err == hipSuccess) {
+        hipLaunchKernelGGL(mfma_rate_i8, dim3((unsigned)blocks), dim3(256), 0, stream, iterations / 20 + 1, operands, sink);  // warm-up
+        err = hipEventRecord(e0, stream);
+        hipLaunchKernelGGL(mfma_rate_i8, dim3((unsigned)blocks), dim3(256), 0, stream, iterations, operands, sink);
+        if (err == hipSuccess) err = hipGetLastError();
+        if (err == hipSuccess) err = hipEventRecord(e1, stream);
+        if (err == hipSuccess) err = hipEventSynchronize(e1);
+        float ms = 0.f;
+        if (err == hipSuccess) err = hipEventElapsedTime(&ms, e0, e1);
+        // per wave and iteration: 16 MFMAs of 32 x 32 x 32 multiply-adds, 2 ops each
+        if (err == hipSuccess) *outTops = (double)blocks * 4 * iterations * 16 * 32768.0 * 2 / ((double)ms * 1e-3) / 1e12;
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (operands) (void)hipFree(operands);
+    if (sink) (void)hipFree(sink);
+    return err;
+}
+
 Tuning tuningFromEnvironment() {
     Tuning t;
     auto flag = [](const char *name) { return getenv(name) != nullptr; };
@@ -3176,6 +3357,8 @@ Tuning tuningFromEnvironment() {
     if (const char *v = getenv("THIP_FC_WIDE_U")) t.fcWideU = atoi(v);
     t.noFcDeep = flag("THIP_NO_FC_DEEP");
     t.noFcWide = flag("THIP_NO_FC_WIDE");
+    t.maxpoolGeneric = flag("THIP_MAXPOOL_GENERIC");
+    t.addGeneric = flag("THIP_ADD_GENERIC");
     return t;
 }
 

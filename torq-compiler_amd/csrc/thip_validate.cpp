@@ -284,12 +284,12 @@ thip_status_t checkOpFootprint(const DescriptorView *e, uint32_t i) {
     }
     case kKindEltwise: {
         const uint64_t inElem = op.gran, outElem = op.out_dtype == THIP_DTYPE_I8 ? 1 : op.out_dtype == THIP_DTYPE_I16 ? 2 : op.out_dtype == THIP_DTYPE_I32 ? 4 : 0;
-        if (!positive({op.C}) || !(inElem == 1 || inElem == 2 || inElem == 4) || outElem == 0 || op.variant > kEltMax || op.w1 < 0 || op.w1 > 2 ||
+        if (!positive({op.C}) || !(inElem == 1 || inElem == 2 || inElem == 4) || outElem == 0 || op.variant > kEltLast || op.w1 < 0 || op.w1 > 2 ||
             (op.variant != kEltMul && op.w1 != 0)) {
             return fail(THIP_INVALID_ARGUMENT, "op %u: bad elementwise record", i);
         }
         if ((s = need(op.in0, (op.w1 == 1 ? 1 : (uint64_t)op.C) * inElem, "in1"))) return s;
-        if ((op.variant == kEltMul || op.variant >= kEltAnd) && (s = need(op.in1, (op.w1 == 2 ? 1 : (uint64_t)op.C) * inElem, "in2"))) return s;
+        if (eltwiseTwoInputs((int32_t)op.variant) && (s = need(op.in1, (op.w1 == 2 ? 1 : (uint64_t)op.C) * inElem, "in2"))) return s;
         return need(op.out, (uint64_t)op.C * outElem, "out");
     }
     case kKindAddBf16: {

@@ -27,10 +27,10 @@ STATUS_NAMES = {
     UNIMPLEMENTED: "UNIMPLEMENTED", INTERNAL: "INTERNAL", UNAVAILABLE: "UNAVAILABLE",
 }
 
-DTYPE_I8, DTYPE_I16, DTYPE_I32, DTYPE_BF16, DTYPE_F32 = 1, 2, 3, 4, 5
-# numpy has no bfloat16: uint16 arrays carry bf16 bit patterns
+DTYPE_I8, DTYPE_I16, DTYPE_I32, DTYPE_BF16, DTYPE_F32, DTYPE_I1 = 1, 2, 3, 4, 5, 6
+# numpy has no bfloat16: uint16 arrays carry bf16 bit patterns; uint8 arrays of 0 / 1 carry i1 truth values
 _NP_TO_DTYPE = {np.dtype(np.int8): DTYPE_I8, np.dtype(np.int16): DTYPE_I16, np.dtype(np.int32): DTYPE_I32,
-                np.dtype(np.uint16): DTYPE_BF16, np.dtype(np.float32): DTYPE_F32}
+                np.dtype(np.uint16): DTYPE_BF16, np.dtype(np.float32): DTYPE_F32, np.dtype(np.uint8): DTYPE_I1}
 _DTYPE_TO_NP = {v: k for k, v in _NP_TO_DTYPE.items()}
 
 BINDING_HOST, BINDING_DEVICE = 0, 1
@@ -41,11 +41,11 @@ EXPORTED_SYMBOLS = [
     "thip_program_create", "thip_program_destroy", "thip_program_set_name", "thip_program_binding", "thip_program_constant",
     "thip_program_tensor", "thip_hl_conv2d", "thip_hl_depthwise_conv2d", "thip_hl_fully_connected",
     "thip_hl_matmul", "thip_hl_maxpool2d", "thip_hl_avg_pool2d", "thip_hl_add", "thip_hl_transpose", "thip_hl_expand_weights",
-    "thip_hl_fma", "thip_hl_mul", "thip_hl_act", "thip_hl_elementwisebinary",
+    "thip_hl_fma", "thip_hl_mul", "thip_hl_act", "thip_hl_elementwisebinary", "thip_hl_elementwiseunary", "thip_hl_elementwiseshift",
     "thip_program_serialize", "thip_blob_free",
     "thip_device_create", "thip_device_destroy", "thip_device_name", "thip_device_alloc",
     "thip_device_free", "thip_device_h2d", "thip_device_d2h", "thip_device_synchronize",
-    "thip_device_set_event_log", "thip_device_set_dump_dirs", "thip_infer_format", "thip_descriptor_validate", "thip_descriptor_info", "thip_descriptor_binding", "thip_descriptor_segment",
+    "thip_device_set_event_log", "thip_device_set_dump_dirs", "thip_device_mfma_rate", "thip_infer_format", "thip_descriptor_validate", "thip_descriptor_info", "thip_descriptor_binding", "thip_descriptor_segment",
     "thip_executable_create", "thip_executable_destroy", "thip_executable_run",
     "thip_executable_enqueue", "thip_executable_enqueue_noalloc", "thip_executable_wait", "thip_executable_set_wait_timeout", "thip_executable_time", "thip_executable_time_rotating",
     "thip_executable_op_count", "thip_executable_op_kernel", "thip_executable_binding_count",
@@ -180,6 +180,15 @@ class HlMul(ctypes.Structure):
     ]
 
 
+class HlElementwiseUnary(ctypes.Structure):
+    _fields_ = [("init", ctypes.c_int32), ("op_type", ctypes.c_int32), ("input", ctypes.c_int32)]
+
+
+class HlElementwiseShift(ctypes.Structure):
+    _fields_ = [("init", ctypes.c_int32), ("op_type", ctypes.c_int32), ("round", ctypes.c_int32), ("input1", ctypes.c_int32),
+                ("input2", ctypes.c_int32)]
+
+
 class HlAct(ctypes.Structure):
     _fields_ = [
         ("init", ctypes.c_int32), ("name", ctypes.c_char_p), ("input_zp", ctypes.c_int32),
@@ -266,6 +275,7 @@ def lib():
     L.thip_device_synchronize.argtypes = [vp]
     L.thip_device_set_event_log.argtypes = [vp, ctypes.c_char_p]
     L.thip_device_set_dump_dirs.argtypes = [vp, ctypes.c_char_p, ctypes.c_char_p]
+    L.thip_device_mfma_rate.argtypes = [vp, i32, i32, i32, P(ctypes.c_double)]
     L.thip_infer_format.argtypes = [vp, sz, sz, ctypes.c_char_p, P(sz)]
     L.thip_descriptor_validate.argtypes = [vp, sz]
     L.thip_descriptor_info.argtypes = [vp, sz, vp]
@@ -340,6 +350,12 @@ class Device:
 
     def set_event_log(self, path):
         check(lib().thip_device_set_event_log(self._h, path.encode() if path else None))
+
+    def mfma_rate(self, random_operands, workgroups=256, iterations=10000):
+        """Sustained int8 MFMA rate in TOP/s of `workgroups` workgroups doing nothing else (benchmark calibration)."""
+        tops = ctypes.c_double()
+        check(lib().thip_device_mfma_rate(self._h, int(bool(random_operands)), int(workgroups), int(iterations), ctypes.byref(tops)))
+        return tops.value
 
     def set_dump_dirs(self, io_data_dir=None, buffers_dir=None):
         """Debug dumps of the bindings of blocking dispatches / of every buffer a kernel record wrote (None: off)."""

@@ -263,10 +263,27 @@ class Program:
         rt.check(rt.lib().thip_hl_act(self._h, ctypes.byref(op)))
         return init
 
-    def elementwisebinary(self, op_type, input1, input2, *, is_unsigned=False, init=None):
-        """torq_hl.elementwisebinary: op_type one of runtime.BITWISE_AND / _OR / _XOR / MINIMUM / MAXIMUM."""
+    def elementwiseunary(self, op_type, input, *, init=None):
+        """torq_hl.elementwiseunary: op_type 3 BITWISE_NOT (integers) or 12 LOGICAL_NOT (i1, carried as uint8 0 / 1)."""
+        init = self._init_or_new(init, input.shape, input.dtype)
+        op = rt.HlElementwiseUnary(init.index, int(op_type), input.index)
+        rt.check(rt.lib().thip_hl_elementwiseunary(self._h, ctypes.byref(op)))
+        return init
+
+    def elementwiseshift(self, op_type, input1, input2, *, round=False, init=None):
+        """torq_hl.elementwiseshift: op_type 0 LSR, 1 LSL, 2 ASR; input2 holds the per-element counts."""
         input2 = self._as_value(input2)
         init = self._init_or_new(init, input1.shape, input1.dtype)
+        op = rt.HlElementwiseShift(init.index, int(op_type), int(bool(round)), input1.index, input2.index)
+        rt.check(rt.lib().thip_hl_elementwiseshift(self._h, ctypes.byref(op)))
+        return init
+
+    def elementwisebinary(self, op_type, input1, input2, *, is_unsigned=False, init=None):
+        """torq_hl.elementwisebinary: op_type is the reference's ElementwiseOpEnum value: 0 and, 1 or, 2 xor, 4 minimum,
+        5 maximum (result of the inputs' type); 6 greater, 7 greater-equal, 8 equal, 9..11 logical and / or / xor (an i1
+        result, carried as uint8 0 / 1)."""
+        input2 = self._as_value(input2)
+        init = self._init_or_new(init, input1.shape, np.uint8 if int(op_type) >= 6 else input1.dtype)
         op = rt.HlElementwiseBinary(init.index, int(op_type), input1.index, input2.index, int(bool(is_unsigned)))
         rt.check(rt.lib().thip_hl_elementwisebinary(self._h, ctypes.byref(op)))
         return init

@@ -82,13 +82,17 @@ def conv2d_workload(N=1, H=112, W=112, C=32, O=64, KH=3, KW=3, stride=(1, 1), pa
 
 
 def fully_connected_workload(M, K, N, realistic=False, output_zp=5, output_min=-128, output_max=127,
-                             seed=1001, shift=None):
+                             seed=1001, shift=None, zeros=False):
     """benchmark configuration 1: int8 [M,K] x [N,K]^T with per-column requant.
 
-    `shift` forces one shift_factor for every column (multipliers drawn so that outputs still spread)."""
+    `shift` forces one shift_factor for every column (multipliers drawn so that outputs still spread).
+    `zeros`: both operands all zero (the same work on data that toggles nothing: a power calibration)."""
     rng = np.random.default_rng(seed)
     x = rng.integers(-128, 127, size=(M, K), endpoint=True, dtype=np.int8)
     w = rng.integers(-128, 127, size=(N, K), endpoint=True, dtype=np.int8)
+    if zeros:
+        x[...] = 0
+        w[...] = 0
     tosa_bias = rng.integers(-(1 << 15), 1 << 15, size=N, endpoint=True, dtype=np.int64)
     if shift is None:
         mult, shift = random_requant(rng, N, realistic)
@@ -348,6 +352,22 @@ def maxpool_workload(N=1, H=112, W=112, C=64, kernel=(2, 2), stride=(2, 2), pad=
                     N * OH * OW * C * kernel[0] * kernel[1], x.nbytes + N * OH * OW * C, attrs)
 
 
+def copy_workload(nbytes=32 << 20, seed=1023):
+    """A plain device copy through this library: a 1x1 stride-1 max pool over the whole int8 range (what a streaming
+    kernel with no arithmetic reaches on this memory system; `nbytes` read and `nbytes` written)."""
+    rng = np.random.default_rng(seed)
+    pixels = nbytes // 64
+    shape = (1, pixels // 1024, 1024, 64)
+    x = rng.integers(-128, 127, size=shape, endpoint=True, dtype=np.int8)
+    p = Program()
+    inp = p.binding(0, shape)
+    out = p.binding(1, shape)
+    attrs = dict(input_zp=-128, output_min=-128, output_max=127, stride=(1, 1), pad=(0, 0, 0, 0), kernel=(1, 1))
+    p.maxpool2d(inp, init=out, nhwc_input=True, **attrs)
+    attrs.update(nhwc=True)
+    return Workload("maxpool_copy_%dMiB" % (nbytes >> 20), p, [x], [(shape, np.int8)], x.size, 2 * x.nbytes, attrs)
+
+
 def avgpool_workload(N=1, H=7, W=7, C=1280, input_zp=-3, output_zp=5, seed=1004):
     """benchmark configuration 2c: global average pool on 7x7x1280 (NHWC), scale = floor(2^20 / 49)."""
     rng = np.random.default_rng(seed)
@@ -476,6 +496,59 @@ def binary_workload(op_type=4, shape=(1, 56, 56, 24), dtype=np.int8, is_unsigned
     attrs = dict(op_type={0: "and", 1: "or", 2: "xor", 4: "minimum", 5: "maximum"}[op_type], is_unsigned=is_unsigned)
     return Workload("binary_%s_%s_%d_u%d" % (attrs["op_type"], np.dtype(dtype).name, a.size, int(is_unsigned)), p, [a, b], [(shape, dtype)], a.size,
                     3 * a.nbytes, attrs)
+
+
+def compare_workload(op_type=6, shape=(1, 56, 56, 24), dtype=np.int8, is_unsigned=False, seed=1024):
+    """torq_hl.elementwisebinary, comparison and logical modes: 6 greater, 7 greater-equal, 8 equal (integers in), 9 and,
+    10 or, 11 xor (i1 in: uint8 0 / 1); the result is i1."""
+    rng = np.random.default_rng(seed)
+    if op_type >= 9:
+        dtype = np.uint8
+        a = rng.integers(0, 2, size=shape, dtype=np.uint8)
+        b = rng.integers(0, 2, size=shape, dtype=np.uint8)
+    else:
+        a = _random_ints(rng, shape, dtype, limit=5)  # a narrow range: equal pairs do occur
+        b = _random_ints(rng, shape, dtype, limit=5)
+        a.reshape(-1)[:4] = [np.iinfo(dtype).min, np.iinfo(dtype).max, -1, 0]
+        b.reshape(-1)[:4] = [np.iinfo(dtype).max, np.iinfo(dtype).min, 0, -1]
+    p = Program()
+    i0 = p.binding(0, shape, dtype)
+    i1 = p.binding(1, shape, dtype)
+    out = p.binding(2, shape, np.uint8)
+    p.elementwisebinary(op_type, i0, i1, is_unsigned=is_unsigned, init=out)
+    attrs = dict(op_type=op_type, is_unsigned=is_unsigned)
+    return Workload("compare_%d_%s_%d_u%d" % (op_type, np.dtype(dtype).name, a.size, int(is_unsigned)), p, [a, b], [(shape, np.uint8)], a.size,
+                    2 * a.nbytes + a.size, attrs)
+
+
+def unary_workload(op_type=3, shape=(1, 56, 56, 24), dtype=np.int8, seed=1025):
+    """torq_hl.elementwiseunary: 3 bitwise not (integers), 12 logical not (i1: uint8 0 / 1)."""
+    rng = np.random.default_rng(seed)
+    if op_type == 12:
+        dtype = np.uint8
+        a = rng.integers(0, 2, size=shape, dtype=np.uint8)
+    else:
+        a = _random_ints(rng, shape, dtype)
+    p = Program()
+    out = p.binding(1, shape, dtype)
+    p.elementwiseunary(op_type, p.binding(0, shape, dtype), init=out)
+    return Workload("unary_%d_%s_%d" % (op_type, np.dtype(dtype).name, a.size), p, [a], [(shape, np.dtype(dtype).type)], a.size, 2 * a.nbytes,
+                    dict(op_type=op_type))
+
+
+def shift_workload(op_type=2, shape=(1, 56, 56, 24), dtype=np.int32, round=True, seed=1026):
+    """torq_hl.elementwiseshift: 0 logical right, 1 logical left, 2 arithmetic right; counts 0 .. bits-1 per element."""
+    rng = np.random.default_rng(seed)
+    a = _random_ints(rng, shape, dtype)
+    bits = 8 * np.dtype(dtype).itemsize
+    s = rng.integers(0, bits, size=shape).astype(dtype)
+    a.reshape(-1)[:6] = [np.iinfo(dtype).min, np.iinfo(dtype).max, -1, 1, -3, 3]
+    s.reshape(-1)[:6] = [bits - 1, bits - 1, 1, 1, 1, 1]
+    p = Program()
+    out = p.binding(2, shape, dtype)
+    p.elementwiseshift(op_type, p.binding(0, shape, dtype), p.binding(1, shape, dtype), round=round, init=out)
+    return Workload("shift_%d_%s_%d_r%d" % (op_type, np.dtype(dtype).name, a.size, int(round)), p, [a, s], [(shape, np.dtype(dtype).type)], a.size,
+                    3 * a.nbytes, dict(op_type=op_type, round=round))
 
 
 def act_workload(name="clamp", shape=(1, 56, 56, 24), in_dtype=np.int8, out_dtype=None, min_int=-20, max_int=90, seed=1018):
