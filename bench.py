@@ -57,11 +57,6 @@ def workload_table(pkg):
         "avgpool_b1": (lambda: w.avgpool_workload(N=1), "hbm"),
         "add_b64": (lambda: w.add_workload(N=64), "hbm"),
         "add_b1": (lambda: w.add_workload(N=1), "hbm"),
-        # what a kernel with no arithmetic reaches: plain copies (1x1 max pool) of 18 + 18 MiB (the size of the
-        # depthwise row), 32 + 32 MiB (the max pool row) and 128 + 128 MiB
-        "copy_18MiB": (lambda: w.copy_workload(18 << 20), "hbm"),
-        "copy_32MiB": (lambda: w.copy_workload(32 << 20), "hbm"),
-        "copy_128MiB": (lambda: w.copy_workload(128 << 20), "hbm"),
         # integer elementwise ops next to the convolution path, at the shape of the add row
         "rescale_b64": (lambda: w.fma_workload((64, 56, 56, 24)), "hbm"),
         "mul_b64": (lambda: w.mul_workload((64, 56, 56, 24)), "hbm"),
@@ -144,6 +139,15 @@ MEASURED_TRAFFIC = {
 def kernels_sha256():
     with open(os.path.join(ROOT, "torq-compiler_amd", "csrc", "thip_kernels.hip"), "rb") as f:
         return hashlib.sha256(f.read()).hexdigest()
+
+
+# The traffic shape of the benchmark's bandwidth rows for the streaming-floor calibration: 16-byte reads per 16-byte
+# write (1, 2 or 4) and bytes written per launch.  The floor is what a kernel with next to no arithmetic takes for
+# the same bytes on the same buffers-larger-than-cache rotation: no op of that size can be faster on this card.
+STREAM_SHAPES = {
+    "depthwise_b64": (4, 64 * 28 * 28 * 144), "depthwise_s1_b256": (1, 256 * 56 * 56 * 144), "maxpool_b64": (4, 64 * 56 * 56 * 64),
+    "add_b64": (2, 64 * 56 * 56 * 24), "rescale_b64": (1, 64 * 56 * 56 * 24), "mul_b64": (2, 64 * 56 * 56 * 24),
+}
 
 
 def roofline(wl, bound, ms, name=None):
@@ -252,22 +256,24 @@ def mfma_calibration(pkg, dev, wl, args):
         o.close()
     out["gemm_over_mfma_only_random"] = round(out["gemm_random_data"]["TOP/s"] / out["mfma_only_random_operands"], 3)
     if args.library_gemm:
+        # in a process of its own: PyTorch brings its own HIP runtime, which does not share a process with this library's
+        import subprocess
+        script = ("import torch, json\n"
+                  "M, K, N, W, S = %d, %d, %d, %d, %d\n"
+                  "a = torch.randint(-128, 128, (M, K), dtype=torch.int8, device='cuda:0')\n"
+                  "bt = torch.randint(-128, 128, (N, K), dtype=torch.int8, device='cuda:0').t()\n"
+                  "for _ in range(W): torch._int_mm(a, bt)\n"
+                  "torch.cuda.synchronize()\n"
+                  "e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)\n"
+                  "e0.record()\n"
+                  "for _ in range(S): torch._int_mm(a, bt)\n"
+                  "e1.record(); torch.cuda.synchronize()\n"
+                  "print(json.dumps({'ms': e0.elapsed_time(e1) / S}))\n") % (M, K, N, max(args.warmup, 5), args.steps)
         try:
-            import torch
-            a = torch.randint(-128, 128, (M, K), dtype=torch.int8, device="cuda:0")
-            bt = torch.randint(-128, 128, (N, K), dtype=torch.int8, device="cuda:0").t()
-            for _ in range(args.warmup):
-                torch._int_mm(a, bt)
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for _ in range(args.steps):
-                torch._int_mm(a, bt)
-            e1.record()
-            torch.cuda.synchronize()
-            ms = e0.elapsed_time(e1) / args.steps
+            done = subprocess.run([sys.executable, "-c", script], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+            ms = json.loads(done.stdout.strip().splitlines()[-1])["ms"]
             out["library_int_mm_random_data"] = {"us": round(ms * 1e3, 2), "TOP/s": round(2.0 * M * K * N / (ms * 1e-3) / 1e12, 1),
-                                                 "what": "torch._int_mm (hipBLASLt), int32 result, no requant, [N,K] weights like ours"}
+                                                 "what": "torch._int_mm (hipBLASLt) in a child process: int32 result, no requant, [N,K] weights like ours"}
         except Exception as ex:  # the comparison is optional
             out["library_int_mm_random_data"] = "unavailable: %r" % (ex,)
     return out
@@ -349,6 +355,12 @@ def main():
                 # buffer set (served by the last-level cache where it fits) is reported next to it
                 ms, sets = o.run_cold(50)
                 row.update({"us": round(ms * 1e3, 2), "us_cache_warm": round(warm * 1e3, 2), "buffer_sets": sets})
+                if name in STREAM_SHAPES:
+                    rd, wbytes = STREAM_SHAPES[name]
+                    wbytes = wbytes // 16 * 16
+                    floor_us = dev.stream_floor(rd, wbytes, cold=True)
+                    row["streaming_floor_us"] = round(floor_us, 2)
+                    row["frac_of_streaming_floor"] = round(floor_us / (ms * 1e3), 3)
             else:
                 ms = warm
                 row["us"] = round(ms * 1e3, 2)

@@ -411,6 +411,13 @@ thip_status_t thip_device_synchronize(thip_device_t *device);
 thip_status_t thip_device_mfma_rate(thip_device_t *device, int32_t random_operands, int32_t workgroups,
                                     int32_t iterations, double *out_tops);
 
+/* Calibration for the benchmark (no counterpart in the reference): microseconds per launch of a kernel with next to
+ * no arithmetic that reads reads_per_write (1, 2 or 4) 16-byte pieces for every 16 bytes it writes, write_bytes
+ * written per launch: what this memory system gives a bandwidth-bound op of that size and read/write mix.
+ * cold != 0: every launch on other buffers, more of them than the last-level cache holds. */
+thip_status_t thip_device_stream_floor(thip_device_t *device, int32_t reads_per_write, size_t write_bytes,
+                                       int32_t cold, double *out_microseconds);
+
 /* What a descriptor blob holds, in the terms of the reference's executable schema
  * (runtime/schemas/torq_executable_def.fbs): ExecutableDef :168-197, Binding :28-48, Segment :13-24.  These read
  * the blob only (no device) and validate it first, like thip_descriptor_validate. */

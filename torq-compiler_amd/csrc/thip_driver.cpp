@@ -602,6 +602,15 @@ thip_status_t thip_device_mfma_rate(thip_device_t *device, int32_t random_operan
     return THIP_OK;
 }
 
+thip_status_t thip_device_stream_floor(thip_device_t *device, int32_t reads_per_write, size_t write_bytes, int32_t cold, double *out_microseconds) {
+    if (!device || !out_microseconds) return fail(THIP_INVALID_ARGUMENT, "null argument");
+    THIP_HIP(hipSetDevice(device->ordinal), "hipSetDevice");
+    const hipError_t err = measureStreamRate(reads_per_write, write_bytes, cold, nullptr, out_microseconds);
+    if (err == hipErrorInvalidValue) return fail(THIP_INVALID_ARGUMENT, "reads_per_write is 1, 2 or 4; write_bytes a multiple of 16 from 4 KiB to 2 GiB");
+    THIP_HIP(err, "measuring the streaming floor");
+    return THIP_OK;
+}
+
 thip_status_t thip_device_set_dump_dirs(thip_device_t *device, const char *io_data_dir, const char *buffers_dir) {
     if (!device) return fail(THIP_INVALID_ARGUMENT, "null device");
     const std::string io = io_data_dir ? io_data_dir : "", buffers = buffers_dir ? buffers_dir : "";

@@ -199,6 +199,11 @@ inline size_t fcBf16WorkspaceCounterBytes(int M, int N, int ksplit) {
 // do nothing else, on constant or on random operand bytes.  Allocates and frees its own few KiB.
 hipError_t measureMfmaRate(int randomOperands, int blocks, int iterations, hipStream_t stream, double *outTops);
 
+// Microseconds per launch of a streaming kernel with next to no arithmetic that reads readsPerWrite (1, 2 or 4)
+// 16-byte pieces per 16 bytes written, writeBytes written per launch; cold: on rotating buffer sets larger than the
+// last-level cache.  Allocates and frees its buffers.
+hipError_t measureStreamRate(int readsPerWrite, size_t writeBytes, int cold, hipStream_t stream, double *outMicroseconds);
+
 constexpr size_t kStaticScratchBytes = 2u << 20;
 hipError_t staticScratchAddress(void **out);
 hipError_t launchZeroFill(void *dst, size_t bytes, hipStream_t stream);

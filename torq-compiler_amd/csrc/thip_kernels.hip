@@ -21,6 +21,7 @@
 #include <mutex>
 #include <string>
 #include <type_traits>
+#include <vector>
 
 #include "thip_descriptor.h"
 
@@ -2140,15 +2141,19 @@ __global__ __launch_bounds__(256, OCC) void depthwise3x3_strip_i8(DepthwiseArgs 
     uint32_t ring[3][NBK][G][4];  // window row kh of the J-th output row of a round of three sits in slot (J S + kh) % 3
     int raw[D][NEW][NC][G];
     const int iyFirst = oy0 * S - p.PT;
+    {
+        // every load of the prologue goes out before the first one is waited for: the rows that complete the first
+        // window and the D rows of prefetch cost one memory round trip together, not one each
+        int first[3 - NEW][NC][G];
 #pragma unroll
-    for (int kh = 0; kh < 3 - NEW; kh++) {
-        issue(iyFirst + kh, raw[0][0]);
-        settle(iyFirst + kh, raw[0][0], ring[kh]);
-    }
+        for (int kh = 0; kh < 3 - NEW; kh++) issue(iyFirst + kh, first[kh]);
 #pragma unroll
-    for (int d = 0; d < D; d++) {
+        for (int d = 0; d < D; d++) {
 #pragma unroll
-        for (int e = 0; e < NEW; e++) issue(iyFirst + d * S + 3 - NEW + e, raw[d][e]);
+            for (int e = 0; e < NEW; e++) issue(iyFirst + d * S + 3 - NEW + e, raw[d][e]);
+        }
+#pragma unroll
+        for (int kh = 0; kh < 3 - NEW; kh++) settle(iyFirst + kh, first[kh], ring[kh]);
     }
     withRequantMode(wrq, [&](auto mode) {
         constexpr int kMode = decltype(mode)::value;
@@ -3332,6 +3337,74 @@ hipError_t measureMfmaRate(int randomOperands, int blocks, int iterations, hipSt
     if (e1) (void)hipEventDestroy(e1);
     if (operands) (void)hipFree(operands);
     if (sink) (void)hipFree(sink);
+    return err;
+}
+
+// Calibration: what a kernel with no arithmetic to speak of reaches on this memory system for a transfer of a given
+// size: every thread reads RD 16-byte pieces (from RD separate streams, perfectly coalesced), combines them with one
+// instruction each and writes 16 bytes.  RD = 1 is a plain copy, RD = 2 the traffic shape of an elementwise add,
+// RD = 4 that of a 2 x 2 pooling or a stride-2 3 x 3 depthwise convolution.
+template <int RD>
+__global__ __launch_bounds__(256) void stream_floor(const v4i *__restrict__ in, v4i *__restrict__ out, size_t items) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= items) return;
+    v4i v[RD];
+#pragma unroll
+    for (int r = 0; r < RD; r++) v[r] = in[(size_t)r * items + i];
+    v4i m = v[0];
+#pragma unroll
+    for (int r = 1; r < RD; r++) {
+        m[0] ^= v[r][0];
+        m[1] ^= v[r][1];
+        m[2] ^= v[r][2];
+        m[3] ^= v[r][3];
+    }
+    out[i] = m;
+}
+
+hipError_t measureStreamRate(int readsPerWrite, size_t writeBytes, int cold, hipStream_t stream, double *outMicroseconds) {
+    if ((readsPerWrite != 1 && readsPerWrite != 2 && readsPerWrite != 4) || writeBytes < 4096 || writeBytes % 16 != 0 || writeBytes > (1ull << 31) ||
+        !outMicroseconds) {
+        return hipErrorInvalidValue;
+    }
+    const size_t items = writeBytes / 16, perSet = writeBytes * (size_t)(readsPerWrite + 1);
+    // cold: dispatch i works on buffer set i mod n, the sets together twice the size of the 256 MiB last-level cache
+    int sets = cold ? (int)((512ull << 20) / perSet) + 1 : 1;
+    sets = sets < (cold ? 2 : 1) ? 2 : (sets > 160 ? 160 : sets);
+    std::vector<v4i *> in((size_t)sets, nullptr), out((size_t)sets, nullptr);
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipError_t err = hipSuccess;
+    for (int s = 0; s < sets && err == hipSuccess; s++) {
+        err = hipMalloc((void **)&in[(size_t)s], writeBytes * (size_t)readsPerWrite);
+        if (err == hipSuccess) err = hipMalloc((void **)&out[(size_t)s], writeBytes);
+        if (err == hipSuccess) err = hipMemsetAsync(in[(size_t)s], s + 1, writeBytes * (size_t)readsPerWrite, stream);
+    }
+    auto launch = [&](int s) {
+        const dim3 grid((unsigned)((items + 255) / 256));
+        if (readsPerWrite == 1) hipLaunchKernelGGL(stream_floor<1>, grid, dim3(256), 0, stream, in[(size_t)s], out[(size_t)s], items);
+        else if (readsPerWrite == 2) hipLaunchKernelGGL(stream_floor<2>, grid, dim3(256), 0, stream, in[(size_t)s], out[(size_t)s], items);
+        else hipLaunchKernelGGL(stream_floor<4>, grid, dim3(256), 0, stream, in[(size_t)s], out[(size_t)s], items);
+    };
+    if (err == hipSuccess) err = hipEventCreate(&e0);
+    if (err == hipSuccess) err = hipEventCreate(&e1);
+    if (err == hipSuccess) {
+        for (int s = 0; s < sets; s++) launch(s);  // first touch
+        const int iterations = sets * 3 > 30 ? sets * 3 : 30;
+        err = hipEventRecord(e0, stream);
+        for (int i = 0; i < iterations; i++) launch(i % sets);
+        if (err == hipSuccess) err = hipGetLastError();
+        if (err == hipSuccess) err = hipEventRecord(e1, stream);
+        if (err == hipSuccess) err = hipEventSynchronize(e1);
+        float ms = 0.f;
+        if (err == hipSuccess) err = hipEventElapsedTime(&ms, e0, e1);
+        if (err == hipSuccess) *outMicroseconds = (double)ms * 1e3 / iterations;
+    }
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    for (int s = 0; s < sets; s++) {
+        if (in[(size_t)s]) (void)hipFree(in[(size_t)s]);
+        if (out[(size_t)s]) (void)hipFree(out[(size_t)s]);
+    }
     return err;
 }
 
