@@ -352,6 +352,27 @@ typedef struct thip_hl_elementwiseshift_t {
     thip_value_t input2;
 } thip_hl_elementwiseshift_t;
 
+/* torq_hl.table -- TorqHLOps.td:311-327, in the forms the lookup patterns produce
+ * (compiler/torq/Conversions/LinalgToTorqHL/ExtractPattern.cpp:30-62,285-298,432-545): a 256-entry table of segment
+ * words (slope << 16) | (base & 0xFFFF) and scale_bias = int32[2] = [-128, 128].  That scale puts the input into
+ * the ACT unit's 9.7 fixed point with a zero fraction, so the slope never contributes and the op is the lookup its
+ * source program states: init[i] = value(table[int8(input[i]) + 128]) with value = base >> 8 for an int8 init (the
+ * words are sext(lut[i]) << 8; a base whose low byte is not zero is refused) and value = base for an int16 init
+ * (the words are zext(lut[i])).  input int8, or int16 of which the low byte is taken as the patterns' trunci does.
+ * The table comes either as static_table (static_table_count entries, the attribute a later reference pass folds
+ * it into) or as dynamic_table, which must then be a constant int32 tensor (THIP_NO_VALUE when absent); a run-time
+ * table is torq_hl.gather in the reference and is not on this path.  Any other scale_bias (the interpolating
+ * tables of the bf16 activation functions) is refused: how the ACT unit rounds an interpolated value is not in the
+ * sources present. */
+typedef struct thip_hl_table_t {
+    thip_value_t init;
+    thip_value_t scale_bias;
+    thip_value_t input;
+    thip_value_t dynamic_table;
+    const int32_t *static_table;
+    int32_t static_table_count;
+} thip_hl_table_t;
+
 thip_status_t thip_hl_conv2d(thip_program_t *program, const thip_hl_conv2d_t *op);
 thip_status_t thip_hl_depthwise_conv2d(thip_program_t *program,
                                        const thip_hl_depthwise_conv2d_t *op);
@@ -367,6 +388,7 @@ thip_status_t thip_hl_fma(thip_program_t *program, const thip_hl_fma_t *op);
 thip_status_t thip_hl_mul(thip_program_t *program, const thip_hl_mul_t *op);
 thip_status_t thip_hl_elementwiseunary(thip_program_t *program, const thip_hl_elementwiseunary_t *op);
 thip_status_t thip_hl_elementwiseshift(thip_program_t *program, const thip_hl_elementwiseshift_t *op);
+thip_status_t thip_hl_table(thip_program_t *program, const thip_hl_table_t *op);
 thip_status_t thip_hl_act(thip_program_t *program, const thip_hl_act_t *op);
 thip_status_t thip_hl_elementwisebinary(thip_program_t *program, const thip_hl_elementwisebinary_t *op);
 

@@ -289,8 +289,24 @@ class ProgramBuilder {
                 aliasResult(op, s.init);
                 return r;
             })
+            .Case<torq_hl::TableOp>([&](torq_hl::TableOp c) {
+                // the plain lookups only (scale_bias = [-128, 128]); the interpolating tables of the bf16 activation
+                // functions come back as THIP_UNIMPLEMENTED and stay on the NPU target
+                thip_hl_table_t s = {};
+                SmallVector<int32_t> words;
+                if (auto attr = c.getStaticTableAttr()) {
+                    words.assign(attr.asArrayRef().begin(), attr.asArrayRef().end());
+                    s.static_table = words.data();
+                    s.static_table_count = (int32_t)words.size();
+                }
+                LogicalResult r = withOperands(op, {{c.getInit(), &s.init}, {c.getScaleBias(), &s.scale_bias}, {c.getInput(), &s.input},
+                                                    {c.getDynamicTable(), &s.dynamic_table}},
+                                               [&] { return thip_hl_table(program_, &s); });
+                aliasResult(op, s.init);
+                return r;
+            })
             .Default([&](Operation *other) {
-                // everything else the pattern set can produce (table, reduce, gather, ...) stays on the NPU target
+                // everything else the pattern set can produce (reduce, gather, argmax, ...) stays on the NPU target
                 return LogicalResult(other->emitError("MI355X backend: ") << other->getName() << " is outside the quantized operator path this target covers");
             });
     }

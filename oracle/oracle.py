@@ -445,6 +445,18 @@ def elementwise_shift(op_type, input1, input2, *, round=False):
     return out
 
 
+def table(input, words, out_dtype, *, bias=-128, scale=128):
+    """torq_hl.table with segment words `words` (int32): the plain lookup the extract patterns produce."""
+    x = _int_array(input)
+    assert x.dtype in (np.int8, np.int16)
+    w = _c(words, np.int32)
+    out = np.empty(x.shape, dtype=out_dtype)
+    rc = lib().torq_table(_p(x), x.itemsize, _p(w), int(w.size), int(bias), int(scale), _p(out), out.itemsize, ctypes.c_size_t(x.size))
+    if rc != 0:
+        raise ValueError("torq_table: an input needs an interpolated or out-of-table entry, which the oracle does not define")
+    return out
+
+
 def per_channel_sum(weights):
     w = _c(weights, np.int8)
     ch = w.shape[0]

@@ -718,6 +718,42 @@ int torq_elementwise_shift(int mode, int round, const void *input1, const void *
     return 0;
 }
 
+/*
+ * torq_hl.table -- signature and segment-word format TorqHLOps.td:311-327: word = (slope << 16) | (base & 0xFFFF).
+ * The ACT stage first applies the one (bias, scale) pair (TablePattern.cpp:58-63: rescaleClamp with shift 0), which
+ * yields a 16-bit 9.7 fixed-point number; its upper nine bits, read as signed, select the entry (-256 .. 255 ->
+ * 0 .. 511) and its lower seven are the fraction the slope is multiplied with (TablePattern.cpp:20-27).  The lookup
+ * patterns (LinalgToTorqHL/ExtractPattern.cpp:56-62) pass bias -128 and scale 128, so the fraction is zero, the
+ * slope contributes nothing and the selected entry is int8(x) + 128 of a 256-entry table: the op then equals the
+ * program it replaced, out = lut[x + 128] (ExtractPattern.cpp:285-298 for an int8 table packed as sext(v) << 8,
+ * :432-545 for an int16 table packed as zext(v); an int16 input is truncated to int8 first, :485-497).  The value
+ * of an entry is base >> 8 for an int8 result and base for an int16 result.
+ * How an interpolated value (non-zero fraction) is rounded is not in the sources present: such an input returns -1,
+ * as does an int8 result from a base with a non-zero low byte and an index beyond the table.
+ */
+int torq_table(const void *input, int in_bytes, const int32_t *table, int table_count, int32_t bias, int32_t scale, void *out, int out_bytes, size_t count) {
+    if ((in_bytes != 1 && in_bytes != 2) || (out_bytes != 1 && out_bytes != 2) || table_count <= 0) return -1;
+    int bad = 0;
+#pragma omp parallel for schedule(static) reduction(| : bad)
+    for (size_t i = 0; i < count; i++) {
+        const int64_t x = (int8_t)(load_elem(input, i, in_bytes) & 0xff);
+        const int64_t t = (x + bias) * (int64_t)scale;
+        const int16_t fixed = (int16_t)(uint16_t)((uint64_t)t & 0xffffu);
+        const int frac = fixed & 127, index = (fixed >> 7) + 256;
+        if (frac != 0 || index < 0 || index >= table_count) {
+            bad |= 1;
+            continue;
+        }
+        const int16_t base = (int16_t)(uint16_t)((uint32_t)table[index] & 0xffffu);
+        if (out_bytes == 1 && (base & 0xff)) {
+            bad |= 1;
+            continue;
+        }
+        store_elem(out, i, out_bytes == 1 ? base >> 8 : base, out_bytes);
+    }
+    return bad ? -1 : 0;
+}
+
 /* ---- R2 ---- */
 
 /* compiler/torq/Utils/ConversionUtils.cpp:122-141 (per_channel_sum). */

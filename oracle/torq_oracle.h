@@ -161,6 +161,11 @@ int torq_elementwise_unary(int mode, const void *input, int bytes, void *out, si
  * input2 holds each element's count. */
 int torq_elementwise_shift(int mode, int round, const void *input1, const void *input2, int bytes, void *out, size_t count);
 
+/* torq_hl.table as the lookup patterns use it: the (bias, scale) pair turns each input (its low byte, signed) into
+ * 9.7 fixed point, the integer part selects one of table_count segment words, the result is the word's base
+ * (>> 8 for a 1-byte result).  Returns -1 where an interpolation would be needed (non-zero fraction). */
+int torq_table(const void *input, int in_bytes, const int32_t *table, int table_count, int32_t bias, int32_t scale, void *out, int out_bytes, size_t count);
+
 /* ---- R2: compile-side parameter derivations ---- */
 
 /* Conv / depthwise / FC: per-channel TOSA (multiplier, shift) -> one global

@@ -290,6 +290,10 @@ def run(blob, binding_arrays):
                 if variant >= 15:
                     a, b = a.view(np.uint8), b.view(np.uint8)
                 res = orc.elementwise_compare(variant - 6, a, b, is_unsigned=bool(int(op["w0"]))).view(np.int8)
+            elif variant == 22:  # table: the record holds the 256 values in the output's type
+                lut = view(op["in1"], 256 * osz).view(tout)
+                assert osz >= esz and osz <= 2
+                res = lut[(a.astype(np.int64) & 0xFF) ^ 0x80]
             elif variant >= 19:  # shifts
                 b = view(op["in1"], n * esz).view(tin)
                 assert tin == tout

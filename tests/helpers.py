@@ -43,6 +43,8 @@ def oracle_eval(wl):
         return [orc.elementwise_unary(a["op_type"], x)]
     if kind == "shift":
         return [orc.elementwise_shift(a["op_type"], x, wl.inputs[1], round=a["round"])]
+    if kind == "table":
+        return [orc.table(x, a["words"], a["out_dtype"])]
     if kind == "act":
         return [orc.act(x, a["name"], min_int=a["min_int"], max_int=a["max_int"], out_dtype=a["out_dtype"])]
     if kind == "avgpoolbf16":
@@ -117,6 +119,11 @@ def bf16_ordered(bits):
     return np.where(b < 0x8000, b, 0x8000 - b)
 
 
+# Tally of the bf16 comparisons of this process: per call, (what, elements compared, elements beyond `ulps` steps that
+# only the cancellation bound admitted).  tests/test_bf16.py reports and bounds it after its GPU cases.
+BF16_TALLY = []
+
+
 def assert_bf16_close(got, want, what="", ulps=1, magnitude=None):
     """The bf16 rows are tolerance rows: at most `ulps` bf16 steps from the oracle per element.
 
@@ -128,7 +135,11 @@ def assert_bf16_close(got, want, what="", ulps=1, magnitude=None):
     if magnitude is not None:
         gf = (got.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
         wf = (want.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+        beyond = int(bad.sum())
         bad &= ~(np.abs(gf - wf) <= np.asarray(magnitude, dtype=np.float64).reshape(got.shape) * 2.0 ** -17)
+        BF16_TALLY.append((what, int(got.size), beyond - int(bad.sum())))
+    else:
+        BF16_TALLY.append((what, int(got.size), 0))
     if bad.any():
         first = tuple(np.argwhere(bad)[0])
         raise AssertionError("%s: %d of %d elements differ by more than %d bf16 ULP; first at %s: got 0x%04x want 0x%04x"

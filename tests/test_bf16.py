@@ -221,7 +221,7 @@ def _magnitude(wl):
 def _check_gpu(device, wl, via="host"):
     print("[gpu-case]", wl.name, flush=True)
     got, kernels = run_on_gpu(device, wl, via=via)
-    assert_bf16_close(got[0], oracle_eval(wl)[0], wl.name, magnitude=_magnitude(wl))
+    assert_bf16_close(got[0], oracle_eval(wl)[0], wl.name + " (gpu)", magnitude=_magnitude(wl))
     assert any("fc_bf16" in k for k in kernels), kernels
     return got[0]
 
@@ -260,7 +260,7 @@ def test_gpu_bf16_conv2d_and_depthwise(device):
         wabs = f(wl.attrs["weights"]).reshape(wl.attrs["weights"].shape[0], -1).sum(axis=1) * f(wl.inputs[0]).max() + np.abs(wl.attrs["bias"])
         shape = [1, 1, 1, 1]
         shape[3 if wl.attrs["nhwc"] else 1] = -1
-        assert_bf16_close(got[0], oracle_eval(wl)[0], wl.name, magnitude=np.broadcast_to(wabs.reshape(shape), got[0].shape))
+        assert_bf16_close(got[0], oracle_eval(wl)[0], wl.name + " (gpu)", magnitude=np.broadcast_to(wabs.reshape(shape), got[0].shape))
         assert "fc_bf16" in families(kernels)
     for wl in [w.conv2d_bf16_workload(depthwise=True, C=12, stride=(2, 2), pad=(0, 1, 0, 1), clamp=(-0.5, 0.5)),
                w.conv2d_bf16_workload(depthwise=True, N=2, C=5, H=7, W=9, nhwc=False),
@@ -284,7 +284,7 @@ def test_gpu_bf16_wide_n(device):
         got, kernels = run_on_gpu(device, wl, via="device")
         w16 = orc.expand_weights(wl.attrs["weights"], wl.attrs["scale"], wl.attrs["qbias"], block_size=wl.attrs["block"],
                                  output_min=wl.attrs["expand_min"], output_max=wl.attrs["expand_max"])
-        assert_bf16_close(got[0], oracle_eval(wl)[0].reshape(got[0].shape), wl.name, magnitude=f(wl.inputs[0]) @ f(w16))
+        assert_bf16_close(got[0], oracle_eval(wl)[0].reshape(got[0].shape), wl.name + " (gpu)", magnitude=f(wl.inputs[0]) @ f(w16))
         assert families(kernels) == ["fc_bf16_wide"], kernels  # >= 1024 column blocks, short K: every wave streams its own columns
 
 
@@ -314,7 +314,7 @@ def test_gpu_expand_weights(device):
         want = oracle_eval(wl)
         w16 = orc.expand_weights(wl.attrs["weights"], wl.attrs["scale"], wl.attrs["qbias"], block_size=wl.attrs["block"],
                                  output_min=wl.attrs["expand_min"], output_max=wl.attrs["expand_max"])
-        assert_bf16_close(got[0], want[0].reshape(got[0].shape), wl.name, magnitude=f(wl.inputs[0]) @ f(w16))
+        assert_bf16_close(got[0], want[0].reshape(got[0].shape), wl.name + " (gpu)", magnitude=f(wl.inputs[0]) @ f(w16))
         if how == "own":
             assert_bit_exact(got[1], want[1], wl.name + " expansion")
             assert families(kernels) == ["expand_weights_bf16", "transpose_i8", "fc_bf16"], kernels
@@ -360,3 +360,22 @@ def test_gpu_bf16_matmul(device):
     _check_gpu(device, w.matmul_bf16_workload(3, 2, 64, 24))
     _check_gpu(device, w.matmul_bf16_workload(2, 5, 16, 12, batch1=False, constant_rhs=True))
     _check_gpu(device, w.matmul_bf16_workload(1, 6, 32, 20, batch1=False, batch2=False, constant_rhs=True, bias=0.5))
+
+
+@pytest.mark.gpu
+def test_gpu_bf16_tolerance_tally(device):
+    """Which elements needed more than one bf16 step.  Every tolerance comparison of this process is tallied by
+    assert_bf16_close; the elements that differ from the oracle by more than one step and pass only because their sum
+    cancelled (|difference| <= 2^-17 of sum |x w| + |bias|) are counted, printed per case, and must stay a small
+    minority: the one-step bound is the binding one wherever nothing cancels."""
+    import helpers
+    gpu_cases = [t for t in helpers.BF16_TALLY if t[0].endswith("(gpu)")]
+    if not gpu_cases:
+        pytest.skip("no bf16 GPU comparison ran in this process before this test")
+    compared = sum(n for _, n, _ in gpu_cases)
+    widened = sum(k for _, _, k in gpu_cases)
+    for what, n, k in gpu_cases:
+        if k:
+            print("[bf16-tolerance] %s: %d of %d elements beyond one step, admitted by the cancellation bound" % (what, k, n), flush=True)
+    print("[bf16-tolerance] total: %d of %d elements (%.4f %%) in %d comparisons" % (widened, compared, 100.0 * widened / compared, len(gpu_cases)), flush=True)
+    assert widened <= compared * 1e-4

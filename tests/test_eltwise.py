@@ -320,3 +320,90 @@ def test_gpu_new_eltwise(device, make):
     got, kernels = run_on_gpu(device, wl, via="device" if wl.inputs[0].size > 10000 else "host")
     assert_bit_exact(got[0], oracle_eval(wl)[0], wl.name)
     assert families(kernels) == ["eltwise_int"]
+
+
+# ---- torq_hl.table: the plain lookups the extract patterns produce --------------------------------------------------
+
+def test_oracle_table_is_the_lookup_of_the_program_it_replaces():
+    """The reference rewrites `extract(lut, index_cast(x) + 128)` into torq_hl.table with the words of
+    ExtractPattern.cpp:30-54 and scale_bias [-128, 128] (:56-62), so the op must give lut[x + 128]: checked for every
+    int8 input against plain indexing, for int8 and int16 tables, and for int16 inputs through their low byte
+    (the trunci of :485-497)."""
+    rng = np.random.default_rng(7)
+    x8 = np.arange(-128, 128, dtype=np.int8)
+    for dtype in (np.int8, np.int16):
+        info = np.iinfo(dtype)
+        lut = rng.integers(info.min, info.max, size=256, endpoint=True).astype(dtype)
+        lut[:2] = [info.min, info.max]
+        words = w.pack_table_words(lut)
+        # the packing itself, against the pattern's arithmetic written out
+        want_words = [(int(v) << 8) & 0xFFFFFFFF if dtype == np.int8 else int(v) & 0xFFFF for v in lut]
+        assert [int(t) & 0xFFFFFFFF for t in words] == want_words
+        np.testing.assert_array_equal(orc.table(x8, words, dtype), lut[x8.astype(np.int64) + 128])
+    x16 = rng.integers(-32768, 32767, size=4096, endpoint=True).astype(np.int16)
+    np.testing.assert_array_equal(orc.table(x16, words, np.int16), lut[x16.astype(np.int8).astype(np.int64) + 128])
+    # the slope half of a word never contributes while the fraction is zero
+    noisy = (words.astype(np.int64) & 0xFFFF | (rng.integers(0, 1 << 16, size=256) << 16)).astype(np.uint32).view(np.int32)
+    np.testing.assert_array_equal(orc.table(x8, noisy, np.int16), lut[x8.astype(np.int64) + 128])
+
+
+def test_oracle_table_refuses_what_the_sources_do_not_define():
+    words = w.pack_table_words(np.arange(-128, 128, dtype=np.int8))
+    x = np.arange(-128, 128, dtype=np.int8)
+    with pytest.raises(ValueError):
+        orc.table(x, words, np.int8, bias=0, scale=1)  # a 9.7 input with a fraction: interpolation
+    with pytest.raises(ValueError):
+        orc.table(x, words + 1, np.int8)  # an int8 result from a base with a low byte
+    with pytest.raises(ValueError):
+        orc.table(x, words, np.int8, bias=128, scale=128)  # entries 256 .. 511 of a 256-entry table
+
+
+TABLES = [lambda: w.table_workload(), lambda: w.table_workload(static=True), lambda: w.table_workload(out_dtype=np.int16, shape=(3, 7, 11)),
+          lambda: w.table_workload(in_dtype=np.int16, out_dtype=np.int16, static=True), lambda: w.table_workload(shape=(1, 1, 1, 5))]
+
+
+@pytest.mark.parametrize("make", TABLES)
+def test_table_descriptor(make):
+    wl = make()
+    blob = wl.program.serialize()
+    outs = [np.zeros(s, dtype=dt) for s, dt in wl.outputs]
+    d = desc_interp.run(blob, list(wl.inputs) + outs)
+    assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)
+    np.testing.assert_array_equal(outs[0], wl.attrs["lut"][(wl.inputs[0].astype(np.int64) & 0xFF) ^ 0x80])
+    assert [(int(o["kind"]), int(o["variant"])) for o in d.ops] == [(desc_interp.K_ELTWISE, 22)]
+
+
+def test_table_rejections():
+    words = w.pack_table_words(np.arange(-128, 128, dtype=np.int8))
+
+    def build(scale_bias=(-128, 128), in_dtype=np.int8, out_dtype=np.int8, **table):
+        p = Program()
+        p.table(p.binding(0, (4, 4), in_dtype), list(scale_bias), init=p.binding(1, (4, 4), out_dtype), **table)
+        return p.serialize()
+
+    build(dynamic_table=words)
+    for bad in (dict(scale_bias=(0, 1), dynamic_table=words),          # an interpolated lookup
+                dict(dynamic_table=words[:128]),                       # not 256 entries
+                dict(dynamic_table=words + 3),                         # int8 result from a base with a low byte
+                dict(in_dtype=np.int16, dynamic_table=words),          # int16 -> int8 is not a form the patterns produce
+                dict(out_dtype=np.int32, dynamic_table=words),
+                dict(dynamic_table=words, static_table=words),         # both forms at once
+                dict()):                                               # no table
+        with pytest.raises(ThipError):
+            build(**bad)
+    p = Program()
+    with pytest.raises(ThipError):  # a run-time table is torq_hl.gather in the reference
+        op = runtime.HlTable(p.binding(1, (4, 4), np.int8).index, p.constant(np.array([-128, 128], dtype=np.int32)).index,
+                             p.binding(0, (4, 4), np.int8).index, p.binding(2, (256,), np.int32).index, None, 0)
+        runtime.check(runtime.lib().thip_hl_table(p._h, __import__("ctypes").byref(op)))
+        p.serialize()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("make", TABLES + [lambda: w.table_workload(shape=(64, 56, 56, 24)), lambda: w.table_workload(shape=(8, 56, 56, 24), out_dtype=np.int16)])
+def test_gpu_table(device, make):
+    wl = make()
+    print("[gpu-case]", wl.name, flush=True)
+    got, kernels = run_on_gpu(device, wl, via="device" if wl.inputs[0].size > 10000 else "host")
+    assert_bit_exact(got[0], oracle_eval(wl)[0], wl.name)
+    assert families(kernels) == ["table_lookup"]

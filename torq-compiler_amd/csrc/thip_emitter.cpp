@@ -44,7 +44,7 @@ struct Value {
     }
 };
 
-enum HlKind { kHlConv2d, kHlDepthwise, kHlFullyConnected, kHlMatmul, kHlMaxPool, kHlAvgPool, kHlAdd, kHlTranspose, kHlExpandWeights, kHlFma, kHlMul, kHlAct, kHlBinary, kHlUnary, kHlShift };
+enum HlKind { kHlConv2d, kHlDepthwise, kHlFullyConnected, kHlMatmul, kHlMaxPool, kHlAvgPool, kHlAdd, kHlTranspose, kHlExpandWeights, kHlFma, kHlMul, kHlAct, kHlBinary, kHlUnary, kHlShift, kHlTable };
 
 struct HlOp {
     HlKind kind;
@@ -64,8 +64,10 @@ struct HlOp {
         thip_hl_elementwisebinary_t bin;
         thip_hl_elementwiseunary_t un;
         thip_hl_elementwiseshift_t sh;
+        thip_hl_table_t tab;
     } u;
     std::string name;
+    std::vector<int32_t> staticTable;  // torq_hl.table: the caller's static_table, copied
 };
 
 }  // namespace thip
@@ -548,6 +550,7 @@ class Emitter {
     thip_status_t emitBinary(const thip_hl_elementwisebinary_t &c);
     thip_status_t emitUnary(const thip_hl_elementwiseunary_t &c);
     thip_status_t emitShift(const thip_hl_elementwiseshift_t &c);
+    thip_status_t emitTable(const thip_hl_table_t &c, const std::vector<int32_t> &staticTable);
     // Operands of an integer elementwise op: element types, and the record's common fields.
     thip_status_t eltwiseCommon(const char *what, thip_value_t input, thip_value_t init, DescOp *op);
     thip_status_t emitAvgPoolBf16(const thip_hl_avg_pool2d_t &c);
@@ -1495,6 +1498,59 @@ thip_status_t Emitter::emitShift(const thip_hl_elementwiseshift_t &c) {
     return THIP_OK;
 }
 
+// torq_hl.table in the forms the lookup patterns produce (compiler/torq/Conversions/LinalgToTorqHL/
+// ExtractPattern.cpp:30-62,285-298,432-545): scale_bias = [-128, 128] turns the input into a 9.7 fixed-point index
+// with a zero fraction (compiler/torq/Conversions/TorqHLToTorqHW/TablePattern.cpp:20-27), so only the base half of a
+// segment word is ever used and the op is out = lut[int8(x) + 128], the statement of the program it replaced.  The
+// record carries the 256 values in the output's type.
+thip_status_t Emitter::emitTable(const thip_hl_table_t &c, const std::vector<int32_t> &staticTable) {
+    const char *what = "torq_hl.table";
+    const Value *x, *init, *sb;
+    if (thip_status_t s = checkValue(c.input, "torq_hl.table input", &x)) return s;
+    if (thip_status_t s = checkValue(c.init, "torq_hl.table init", &init)) return s;
+    if (thip_status_t s = constantData(c.scale_bias, "torq_hl.table scale_bias", THIP_DTYPE_I32, &sb)) return s;
+    if (sb->numel() < 2) return fail(THIP_INVALID_ARGUMENT, "%s: scale_bias too short", what);
+    const int32_t *sbd = (const int32_t *)sb->data.data();
+    if (sbd[0] != -128 || sbd[1] != 128) {
+        return fail(THIP_UNIMPLEMENTED, "%s: scale_bias [%d, %d] asks for an interpolated lookup; only the plain lookup [-128, 128] is on this path", what, (int)sbd[0], (int)sbd[1]);
+    }
+    const bool out8 = init->dtype == THIP_DTYPE_I8, out16 = init->dtype == THIP_DTYPE_I16;
+    if (!(out8 && x->dtype == THIP_DTYPE_I8) && !(out16 && (x->dtype == THIP_DTYPE_I8 || x->dtype == THIP_DTYPE_I16))) {
+        return fail(THIP_UNIMPLEMENTED, "%s: int8 -> int8, int8 -> int16 and int16 -> int16 lookups only", what);
+    }
+    const int32_t *words = nullptr;
+    int64_t count = 0;
+    if (c.static_table_count > 0) {
+        if (c.dynamic_table != THIP_NO_VALUE) return fail(THIP_INVALID_ARGUMENT, "%s: both static_table and dynamic_table given", what);
+        words = staticTable.data();
+        count = (int64_t)staticTable.size();
+    } else {
+        const Value *t;
+        if (thip_status_t s = checkValue(c.dynamic_table, "torq_hl.table dynamic_table", &t)) return s;
+        if (t->kind != kValueConstant) return fail(THIP_UNIMPLEMENTED, "%s: a run-time table is torq_hl.gather in the reference and is not on this path", what);
+        if (t->dtype != THIP_DTYPE_I32) return fail(THIP_INVALID_ARGUMENT, "%s: the table must be int32 segment words", what);
+        words = (const int32_t *)t->data.data();
+        count = t->numel();
+    }
+    if (count != 256) return fail(THIP_UNIMPLEMENTED, "%s: the lookup patterns produce 256 entries, this table has %lld", what, (long long)count);
+    std::vector<uint8_t> lut(out8 ? 256 : 512);
+    for (int i = 0; i < 256; i++) {
+        const int16_t base = (int16_t)(uint16_t)((uint32_t)words[i] & 0xffffu);
+        if (out8) {
+            if (base & 0xff) return fail(THIP_UNIMPLEMENTED, "%s: entry %d has a base that is not an int8 value shifted left by 8", what, i);
+            lut[(size_t)i] = (uint8_t)(int8_t)(base >> 8);
+        } else {
+            memcpy(&lut[(size_t)i * 2], &base, 2);
+        }
+    }
+    DescOp op;
+    if (thip_status_t s = eltwiseCommon(what, c.input, c.init, &op)) return s;
+    op.variant = kEltTable;
+    op.in1 = newConst(lut);
+    ops_.push_back(op);
+    return THIP_OK;
+}
+
 thip_status_t Emitter::emitAct(const thip_hl_act_t &c, const std::string &name) {
     const char *what = "torq_hl.act";
     if (c.weights != THIP_NO_VALUE) return fail(THIP_UNIMPLEMENTED, "%s: weights (the unsigned cast) are not on this path", what);
@@ -1754,6 +1810,7 @@ void Emitter::planChannelPadding() {
         case kHlBinary: bar(op.u.bin.input1); bar(op.u.bin.input2); bar(op.u.bin.init); break;
         case kHlUnary: bar(op.u.un.input); bar(op.u.un.init); break;
         case kHlShift: bar(op.u.sh.input1); bar(op.u.sh.input2); bar(op.u.sh.init); break;
+        case kHlTable: bar(op.u.tab.input); bar(op.u.tab.init); break;
         }
     }
     // one verdict per group: every member an int8 rank-4 intermediate, all uses agreeing on C
@@ -1808,6 +1865,7 @@ void Emitter::planExpandFolding() {
         case kHlBinary: read(op.u.bin.input1); read(op.u.bin.input2); break;
         case kHlUnary: read(op.u.un.input); break;
         case kHlShift: read(op.u.sh.input1); read(op.u.sh.input2); break;
+        case kHlTable: read(op.u.tab.input); break;
         }
     }
     auto constant = [&](thip_value_t v) { return v >= 0 && (size_t)v < n && prog_.values[(size_t)v].kind == kValueConstant; };
@@ -1879,6 +1937,7 @@ thip_status_t Emitter::run(void **outBlob, size_t *outSize) {
         case kHlBinary: s = emitBinary(op.u.bin); break;
         case kHlUnary: s = emitUnary(op.u.un); break;
         case kHlShift: s = emitShift(op.u.sh); break;
+        case kHlTable: s = emitTable(op.u.tab, op.staticTable); break;
         }
         if (s != THIP_OK) return s;
     }
@@ -2034,6 +2093,21 @@ THIP_DEFINE_HL(thip_hl_mul, thip_hl_mul_t, kHlMul, mul)
 THIP_DEFINE_HL(thip_hl_elementwisebinary, thip_hl_elementwisebinary_t, kHlBinary, bin)
 THIP_DEFINE_HL(thip_hl_elementwiseunary, thip_hl_elementwiseunary_t, kHlUnary, un)
 THIP_DEFINE_HL(thip_hl_elementwiseshift, thip_hl_elementwiseshift_t, kHlShift, sh)
+
+thip_status_t thip_hl_table(thip_program_t *program, const thip_hl_table_t *op) {
+    if (!program || !op) return fail(THIP_INVALID_ARGUMENT, "thip_hl_table: null argument");
+    if (op->static_table_count < 0 || (op->static_table_count > 0 && !op->static_table) || op->static_table_count > 65536) {
+        return fail(THIP_INVALID_ARGUMENT, "thip_hl_table: bad static_table");
+    }
+    HlOp h;
+    memset((void *)&h.u, 0, sizeof(h.u));
+    h.kind = kHlTable;
+    h.u.tab = *op;
+    if (op->static_table_count > 0) h.staticTable.assign(op->static_table, op->static_table + op->static_table_count);
+    h.u.tab.static_table = nullptr;  // the copy is what the serialiser reads
+    program->ops.push_back(h);
+    return THIP_OK;
+}
 
 thip_status_t thip_hl_act(thip_program_t *program, const thip_hl_act_t *op) {
     if (!program || !op || !op->name) return fail(THIP_INVALID_ARGUMENT, "thip_hl_act: null argument");

@@ -215,21 +215,23 @@ hipError_t launchZeroFill(void *dst, size_t bytes, hipStream_t stream);
 // compare as unsigned.  not: bitwise complement.  greater / greater-equal / equal: two inputs of one integer type
 // (w0 != 0, 16-bit only: unsigned), the result one byte of 0 or 1 per element; logical and / or / xor / not: such
 // bytes in (non-zero = true), such bytes out.  lsr / lsl / asr: in0 shifted by the counts in in1 (clamped to
-// 0 .. bits-1), same type out; w0 != 0: right shifts round half up.
+// 0 .. bits-1), same type out; w0 != 0: right shifts round half up.  table: out = lut[int8(in0) + 128], in1 = the
+// 256 entries of the output's type (int8 or int16); in0 int8 or int16 (its low byte).
 enum EltwiseOp : int32_t {
     kEltFma = 0, kEltMul = 1, kEltClamp = 2, kEltAbs = 3, kEltNegate = 4, kEltCast = 5,
     kEltAnd = 6, kEltOr = 7, kEltXor = 8, kEltMin = 9, kEltMax = 10,
     kEltNot = 11, kEltGreater = 12, kEltGreaterEqual = 13, kEltEqual = 14,
     kEltLogicalAnd = 15, kEltLogicalOr = 16, kEltLogicalXor = 17, kEltLogicalNot = 18,
     kEltLsr = 19, kEltLsl = 20, kEltAsr = 21,
-    kEltLast = kEltAsr,
+    kEltTable = 22,
+    kEltLast = kEltTable,
 };
 // Ops that read a second tensor, and those whose result has the inputs' element type.
 __host__ __device__ inline bool eltwiseTwoInputs(int32_t op) {
     return op == kEltMul || (op >= kEltAnd && op <= kEltMax) || (op >= kEltGreater && op <= kEltLogicalXor) || op >= kEltLsr;
 }
 __host__ __device__ inline bool eltwiseSameType(int32_t op) {
-    return (op >= kEltAnd && op <= kEltNot) || (op >= kEltLogicalAnd && op <= kEltLogicalNot) || op >= kEltLsr;
+    return (op >= kEltAnd && op <= kEltNot) || (op >= kEltLogicalAnd && op <= kEltLogicalNot) || (op >= kEltLsr && op <= kEltAsr);
 }
 struct EltwiseArgs {
     const void *in0;

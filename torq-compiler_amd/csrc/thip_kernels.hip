@@ -2297,10 +2297,11 @@ hipError_t launchDepthwise(const DepthwiseArgs &a, const LaunchCtx &ctx) {
             const int seg = depthwiseStripSegment(a, 2, 1, &waves);
             if (a.SW == 1 && (stripOn || (a.OH >= 12 && waves >= 1024))) return launchDepthwiseStrip<2, 1, 1, 4, 3>(a, seg, ctx);
             if (a.SW == 2 && (stripOne || (!stripOn && a.OH >= 12))) {
-                // with plenty of work, one column per thread, more waves and the deeper prefetch measured 7-10 % ahead
+                // with plenty of work (the six waves per SIMD that the segment length aims for), one column per thread, more
+                // waves and the deeper prefetch measured 7-11 % ahead
                 long long waves1 = 0;
                 const int seg1 = depthwiseStripSegment(a, 1, 1, &waves1);
-                if (stripOne || waves1 >= 7 * 1024) return launchDepthwiseStrip<1, 2, 1, 4, 3>(a, seg1, ctx);
+                if (stripOne || waves1 >= 6 * 1024) return launchDepthwiseStrip<1, 2, 1, 4, 3>(a, seg1, ctx);
             }
             if (a.SW == 2 && (stripOn || (a.OH >= 12 && 10 * waves >= 19 * 1024))) return launchDepthwiseStrip<2, 2, 1, 3, 1>(a, seg, ctx);
         }
@@ -2762,6 +2763,51 @@ __global__ __launch_bounds__(256) void eltwise_int(EltwiseArgs p) {
     }
 }
 
+// torq_hl.table as a plain lookup: the block copies the 256 entries into LDS, a thread looks up VEC neighbouring
+// elements by the low byte of each input (read as signed, plus 128).
+template <typename TIN, typename TOUT, int VEC>
+__global__ __launch_bounds__(256) void table_lookup(EltwiseArgs p) {
+    __shared__ TOUT lut[256];
+    lut[threadIdx.x] = ((const TOUT *)p.in1)[threadIdx.x];
+    __syncthreads();
+    const int64_t i0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * VEC;
+    if (i0 >= p.count) return;
+    const TIN *in0 = (const TIN *)p.in0;
+    TOUT *out = (TOUT *)p.out;
+    const bool whole = i0 + VEC <= p.count;
+    EltVec<TIN, VEC> a;
+    EltVec<TOUT, VEC> o;
+    if (whole) {
+        a = *(const EltVec<TIN, VEC> *)(in0 + i0);
+    } else {
+#pragma unroll
+        for (int v = 0; v < VEC; v++) a.e[v] = i0 + v < p.count ? in0[i0 + v] : (TIN)0;
+    }
+#pragma unroll
+    for (int v = 0; v < VEC; v++) o.e[v] = lut[((uint32_t)(int32_t)a.e[v] & 0xffu) ^ 0x80u];
+    if (whole) {
+        *(EltVec<TOUT, VEC> *)(out + i0) = o;
+    } else {
+#pragma unroll
+        for (int v = 0; v < VEC; v++) {
+            if (i0 + v < p.count) out[i0 + v] = o.e[v];
+        }
+    }
+}
+
+template <typename TIN, typename TOUT>
+static hipError_t launchTableT(const EltwiseArgs &a, const LaunchCtx &ctx) {
+    constexpr int VEC = sizeof(TIN) == 1 && sizeof(TOUT) == 1 ? 16 : 8;
+    const bool aligned = (((uintptr_t)a.in0) & (sizeof(TIN) * VEC - 1)) == 0 && (((uintptr_t)a.out) & (sizeof(TOUT) * VEC - 1)) == 0;
+    if (aligned) {
+        const long long threads = (a.count + VEC - 1) / VEC;
+        THIP_ENQUEUE(ctx, kernelLabel("table_lookup", {(int)sizeof(TIN), (int)sizeof(TOUT), VEC}), (table_lookup<TIN, TOUT, VEC>), dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, a);
+    } else {
+        THIP_ENQUEUE(ctx, kernelLabel("table_lookup", {(int)sizeof(TIN), (int)sizeof(TOUT), 1}), (table_lookup<TIN, TOUT, 1>), dim3((unsigned)((a.count + 255) / 256)), dim3(256), 0, a);
+    }
+    return hipGetLastError();
+}
+
 template <typename TIN, typename TOUT>
 static hipError_t launchEltwiseT(const EltwiseArgs &a, const LaunchCtx &ctx) {
     constexpr int VEC = sizeof(TIN) == 1 && sizeof(TOUT) == 1 ? 16 : 8;
@@ -2786,6 +2832,12 @@ hipError_t launchEltwise(const EltwiseArgs &a, const LaunchCtx &ctx) {
     if (a.op >= kEltGreater && a.op <= kEltEqual && a.out_bytes != 1) return hipErrorInvalidValue;            // a truth value is one byte
     if (a.op >= kEltLogicalAnd && a.op <= kEltLogicalNot && a.in_bytes != 1) return hipErrorInvalidValue;
     if ((((uintptr_t)a.in0) & (a.in_bytes - 1)) || (((uintptr_t)a.out) & (a.out_bytes - 1))) return hipErrorInvalidValue;
+    if (a.op == kEltTable) {
+        // the 256 entries have the output's type; an int8 table serves int8 inputs only
+        if ((((uintptr_t)a.in1) & (a.out_bytes - 1)) || a.in_bytes > 2 || a.out_bytes > 2 || a.out_bytes < a.in_bytes) return hipErrorInvalidValue;
+        if (a.in_bytes == 1) return a.out_bytes == 1 ? launchTableT<int8_t, int8_t>(a, ctx) : launchTableT<int8_t, int16_t>(a, ctx);
+        return launchTableT<int16_t, int16_t>(a, ctx);
+    }
     if (two && (((uintptr_t)a.in1) & (a.in_bytes - 1))) return hipErrorInvalidValue;
     switch (a.in_bytes * 8 + a.out_bytes) {
     case 1 * 8 + 1: return launchEltwiseT<int8_t, int8_t>(a, ctx);

@@ -289,6 +289,11 @@ thip_status_t checkOpFootprint(const DescriptorView *e, uint32_t i) {
             return fail(THIP_INVALID_ARGUMENT, "op %u: bad elementwise record", i);
         }
         if ((s = need(op.in0, (op.w1 == 1 ? 1 : (uint64_t)op.C) * inElem, "in1"))) return s;
+        if (op.variant == kEltTable) {
+            if (inElem > 2 || outElem > 2 || outElem < inElem || op.in1.space != kSpaceConst) return fail(THIP_INVALID_ARGUMENT, "op %u: bad table record", i);
+            if ((s = need(op.in1, 256 * outElem, "table"))) return s;
+            return need(op.out, (uint64_t)op.C * outElem, "out");
+        }
         if (eltwiseTwoInputs((int32_t)op.variant) && (s = need(op.in1, (op.w1 == 2 ? 1 : (uint64_t)op.C) * inElem, "in2"))) return s;
         return need(op.out, (uint64_t)op.C * outElem, "out");
     }

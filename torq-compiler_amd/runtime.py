@@ -41,7 +41,7 @@ EXPORTED_SYMBOLS = [
     "thip_program_create", "thip_program_destroy", "thip_program_set_name", "thip_program_binding", "thip_program_constant",
     "thip_program_tensor", "thip_hl_conv2d", "thip_hl_depthwise_conv2d", "thip_hl_fully_connected",
     "thip_hl_matmul", "thip_hl_maxpool2d", "thip_hl_avg_pool2d", "thip_hl_add", "thip_hl_transpose", "thip_hl_expand_weights",
-    "thip_hl_fma", "thip_hl_mul", "thip_hl_act", "thip_hl_elementwisebinary", "thip_hl_elementwiseunary", "thip_hl_elementwiseshift",
+    "thip_hl_fma", "thip_hl_mul", "thip_hl_act", "thip_hl_elementwisebinary", "thip_hl_elementwiseunary", "thip_hl_elementwiseshift", "thip_hl_table",
     "thip_program_serialize", "thip_blob_free",
     "thip_device_create", "thip_device_destroy", "thip_device_name", "thip_device_alloc",
     "thip_device_free", "thip_device_h2d", "thip_device_d2h", "thip_device_synchronize",
@@ -182,6 +182,11 @@ class HlMul(ctypes.Structure):
 
 class HlElementwiseUnary(ctypes.Structure):
     _fields_ = [("init", ctypes.c_int32), ("op_type", ctypes.c_int32), ("input", ctypes.c_int32)]
+
+
+class HlTable(ctypes.Structure):
+    _fields_ = [("init", ctypes.c_int32), ("scale_bias", ctypes.c_int32), ("input", ctypes.c_int32), ("dynamic_table", ctypes.c_int32),
+                ("static_table", ctypes.POINTER(ctypes.c_int32)), ("static_table_count", ctypes.c_int32)]
 
 
 class HlElementwiseShift(ctypes.Structure):

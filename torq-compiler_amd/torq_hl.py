@@ -270,6 +270,21 @@ class Program:
         rt.check(rt.lib().thip_hl_elementwiseunary(self._h, ctypes.byref(op)))
         return init
 
+    def table(self, input, scale_bias, *, dynamic_table=None, static_table=None, init=None, out_dtype=None):
+        """torq_hl.table: 256 int32 segment words, either as a constant tensor (dynamic_table) or as the static_table
+        attribute; scale_bias = [-128, 128] (the plain lookup)."""
+        init = self._init_or_new(init, input.shape, input.dtype if out_dtype is None else out_dtype)
+        sb = self._as_value(np.asarray(scale_bias, dtype=np.int32))
+        dyn = rt.NO_VALUE if dynamic_table is None else self._as_value(np.asarray(dynamic_table, dtype=np.int32)).index
+        if static_table is None:
+            words, count = None, 0
+        else:
+            arr = np.ascontiguousarray(static_table, dtype=np.int32)
+            words, count = arr.ctypes.data_as(ctypes.POINTER(ctypes.c_int32)), int(arr.size)
+        op = rt.HlTable(init.index, sb.index, input.index, dyn, words, count)
+        rt.check(rt.lib().thip_hl_table(self._h, ctypes.byref(op)))
+        return init
+
     def elementwiseshift(self, op_type, input1, input2, *, round=False, init=None):
         """torq_hl.elementwiseshift: op_type 0 LSR, 1 LSL, 2 ASR; input2 holds the per-element counts."""
         input2 = self._as_value(input2)

@@ -551,6 +551,32 @@ def shift_workload(op_type=2, shape=(1, 56, 56, 24), dtype=np.int32, round=True,
                     3 * a.nbytes, dict(op_type=op_type, round=round))
 
 
+def pack_table_words(lut):
+    """Segment words of a 256-entry lookup table as the extract patterns build them
+    (compiler/torq/Conversions/LinalgToTorqHL/ExtractPattern.cpp:30-54): sext(v) << 8 for int8, zext(v) for int16."""
+    lut = np.asarray(lut)
+    if lut.dtype == np.int8:
+        return (lut.astype(np.int32) << 8).astype(np.int32)
+    assert lut.dtype == np.int16
+    return lut.view(np.uint16).astype(np.int32)
+
+
+def table_workload(shape=(1, 56, 56, 24), in_dtype=np.int8, out_dtype=np.int8, static=False, seed=1027):
+    """torq_hl.table: a random 256-entry lookup table of the output's type, as a constant operand or as the attribute."""
+    rng = np.random.default_rng(seed)
+    x = _random_ints(rng, shape, in_dtype)
+    x.reshape(-1)[:4] = [-128, 127, 0, -1]
+    lut = _random_ints(rng, (256,), out_dtype)
+    lut[[0, 255]] = _INT_RANGE[np.dtype(out_dtype)]
+    words = pack_table_words(lut)
+    p = Program()
+    out = p.binding(1, shape, out_dtype)
+    p.table(p.binding(0, shape, in_dtype), [-128, 128], init=out, **({"static_table": words} if static else {"dynamic_table": words}))
+    nbytes = x.nbytes + x.size * np.dtype(out_dtype).itemsize
+    return Workload("table_%s_%s_%d_%s" % (np.dtype(in_dtype).name, np.dtype(out_dtype).name, x.size, "attr" if static else "operand"), p, [x],
+                    [(shape, np.dtype(out_dtype).type)], x.size, nbytes, dict(words=words, lut=lut, out_dtype=out_dtype))
+
+
 def act_workload(name="clamp", shape=(1, 56, 56, 24), in_dtype=np.int8, out_dtype=None, min_int=-20, max_int=90, seed=1018):
     """torq_hl.act on integers: clamp / abs / negate / i2i."""
     rng = np.random.default_rng(seed)
