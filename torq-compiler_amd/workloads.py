@@ -656,7 +656,7 @@ def mobilenet_v2_layers(resolution=224, classes=1000, seed=1006, width=1.0):
         xp = torch.nn.functional.pad(calib[src], (pl, pr, pt, pb))  # x - zp is 0 in the padding
         acc = torch.nn.functional.conv2d(xp, torch.from_numpy(w.astype(np.float64)), stride=s, groups=C if depthwise else 1)
         acc = acc + torch.from_numpy(tosa_bias.astype(np.float64)).reshape(1, -1, 1, 1)
-        spread = acc.std(dim=(0, 2, 3)).numpy() + 1.0
+        spread = acc.std(dim=(0, 2, 3), unbiased=False).numpy() + 1.0  # a 1x1 frame has a spread of 0, not NaN
         # ReLU6 layers keep the positive half: give it most of the range; linear layers are centred
         eff = (60.0 if relu6 else 40.0) / spread * rng.uniform(0.8, 1.25, size=O_)
         mult, shift = quantize_multiplier(eff)
