@@ -2461,11 +2461,21 @@ __global__ __launch_bounds__(256) void avgpool_i8(AvgPoolArgs p) {
     for (int v = 0; v < VEC; v++) acc[v] = 0;
     if (active) {
         const int8_t *src = p.in + (size_t)n * p.HW * p.C + c0;
-        for (int u = pg; u < p.HW; u += PG) {
-            Pack<VEC> x;
-            x.v = *(const typename ByteVec<VEC>::type *)(src + (size_t)u * p.C);
+        // four pixels per round, all four loads issued before the first is used (a pixel past the frame re-reads the
+        // lane's first one and is weighted 0): a 7 x 7 frame costs one memory round trip instead of four
+        for (int u0 = pg; u0 < p.HW; u0 += 4 * PG) {
+            Pack<VEC> x[4];
 #pragma unroll
-            for (int v = 0; v < VEC; v++) acc[v] += (int32_t)x.b[v] * p.weight;
+            for (int j = 0; j < 4; j++) {
+                const int u = u0 + j * PG;
+                x[j].v = *(const typename ByteVec<VEC>::type *)(src + (size_t)(u < p.HW ? u : pg) * p.C);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int32_t wj = u0 + j * PG < p.HW ? p.weight : 0;
+#pragma unroll
+                for (int v = 0; v < VEC; v++) acc[v] += (int32_t)x[j].b[v] * wj;
+            }
         }
     }
 #pragma unroll
