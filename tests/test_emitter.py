@@ -47,6 +47,38 @@ def test_conv2d_descriptor(kw, nhwc):
         assert kinds[0] == desc_interp.K_TRANSPOSE and kinds[1] == desc_interp.K_IGEMM
 
 
+# Convolutions over whole 64-channel k-tiles with at least 2048 output pixels: the LDS-DMA ring kernel addresses the window.
+WINDOW_RING = [
+    dict(N=2, H=32, W=32, C=64, O=64),                                            # M = 2048: the smallest taken; one tile column
+    dict(N=10, H=29, W=31, C=64, O=96, stride=(2, 2), pad=(0, 1, 0, 1)),          # odd frame, stride 2, one-sided padding, ragged M
+    dict(N=2, H=40, W=36, C=128, O=160, pad=(1, 1, 1, 1)),                        # two k-tiles per tap, N not a multiple of any tile
+    dict(N=1, H=50, W=50, C=64, O=72, KH=5, KW=5, pad=(2, 2, 2, 2)),              # 25 taps; N % 16 != 0: the staged epilogue
+    dict(N=2, H=34, W=66, C=64, O=256, KH=1, KW=3, pad=(1, 1, 0, 0)),             # a flat window
+    dict(N=8, H=24, W=24, C=192, O=128, KH=3, KW=3, stride=(1, 2), pad=(2, 0, 1, 2)),  # three k-tiles per tap, mixed strides, lopsided pads
+    dict(N=8, H=33, W=33, C=64, O=64, KH=1, KW=1, stride=(2, 2), pad=(0, 0, 0, 0)),    # a strided pointwise convolution
+]
+
+
+def test_conv2d_window_loader_records():
+    """Whole 64-channel k-tiles and enough rows: the record asks for the ring kernel's window addressing (loader 3, a
+    64-byte zero-point page as its table); fewer rows, other channel counts or the switch keep the gather loader."""
+    import os
+    for kw in WINDOW_RING:
+        wl = w.conv2d_workload(realistic=True, **kw)
+        outs, d = interp(wl)
+        assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)
+        assert [(int(o["kind"]), int(o["loader"])) for o in d.ops] == [(desc_interp.K_IGEMM, 3)], wl.name
+        assert int(d.ops[0]["Kp"]) == int(d.ops[0]["K"])
+    for kw in (dict(N=1, H=32, W=32, C=64, O=64), dict(N=2, H=32, W=32, C=96, O=64), dict(N=2, H=32, W=32, C=64, O=16)):
+        d = interp(w.conv2d_workload(realistic=True, **kw))[1]
+        assert int(d.ops[0]["loader"]) == 1, kw
+    os.environ["THIP_NO_WINDOW_RING"] = "1"
+    try:
+        assert int(interp(w.conv2d_workload(realistic=True, **WINDOW_RING[0]))[1].ops[0]["loader"]) == 1
+    finally:
+        del os.environ["THIP_NO_WINDOW_RING"]
+
+
 @pytest.mark.parametrize("kw", [
     dict(N=1, H=6, W=42, C=16), dict(N=1, H=6, W=6, C=2, pad=(0, 0, 0, 0)), dict(N=1, H=13, W=15, C=8, stride=(1, 1), pad=(1, 1, 1, 1)),
     dict(N=1, H=27, W=27, C=128, KH=4, KW=4, stride=(2, 2), pad=(1, 2, 1, 2)), dict(N=2, H=21, W=21, C=5, stride=(2, 2), pad=(1, 1, 1, 1)),

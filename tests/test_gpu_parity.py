@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 from helpers import assert_bit_exact, families, oracle_eval, oracle_network, run_on_gpu
-from test_emitter import CONV, MATMUL, _chain_program, _padded_chain, matmul_id
+from test_emitter import CONV, MATMUL, WINDOW_RING, _chain_program, _padded_chain, matmul_id
 from torq_compiler_amd import Executable, ThipError, runtime, workloads as w
 
 pytestmark = pytest.mark.gpu
@@ -66,6 +66,34 @@ def test_conv2d_every_tile_variant(device, variant, monkeypatch):
     assert k[0].startswith(names[variant]), k
     check(device, w.conv2d_workload(N=1, H=15, W=17, C=24, O=40, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True))
     check(device, w.fully_connected_workload(300, 192, 520, realistic=True))
+
+
+@pytest.mark.parametrize("kw", WINDOW_RING, ids=lambda kw: "x".join(str(kw[k]) for k in ("N", "H", "W", "C", "O")))
+def test_conv2d_window_ring(device, kw):
+    """Convolutions over whole 64-channel k-tiles: the LDS-DMA ring kernel addresses the window itself."""
+    k = check(device, w.conv2d_workload(realistic=True, **kw), via="device")
+    assert families(k) == ["igemm_dense_conv_i8"], k
+    k = check(device, w.conv2d_workload(realistic=False, nhwc=False, **kw))  # the literal requant range, N,C,H,W bindings
+    assert "igemm_dense_conv_i8" in families(k), k
+
+
+@pytest.mark.parametrize("variant", [4, 5, 6, 8, 9])
+def test_conv2d_window_ring_every_tile(device, variant, monkeypatch):
+    monkeypatch.setenv("THIP_WINDOW_VARIANT", str(variant))
+    names = {4: "igemm_dense_conv_i8<256,256,", 5: "igemm_dense_conv_i8<128,128,", 6: "igemm_dense_conv_i8<128,256,", 8: "igemm_dense_conv_i8<256,128,",
+             9: "igemm_dense_conv_i8<256,64,"}
+    for kw in (dict(N=2, H=33, W=35, C=64, O=80, pad=(1, 1, 1, 1)), dict(N=5, H=47, W=45, C=128, O=48, stride=(2, 2), pad=(1, 0, 1, 0), output_zp=-7, output_min=-128)):
+        k = check(device, w.conv2d_workload(realistic=True, **kw), via="device")
+        assert k[0].startswith(names[variant]), k
+    # an int32 result and a requant shift on the 64-bit tail: the staged epilogue
+    k = check(device, w.conv2d_workload(N=2, H=32, W=32, C=64, O=64, realistic=False))
+    assert k[0].startswith(names[variant]), k
+
+
+def test_conv2d_window_ring_switch(device, monkeypatch):
+    monkeypatch.setenv("THIP_NO_WINDOW_RING", "1")
+    k = check(device, w.conv2d_workload(N=2, H=32, W=32, C=64, O=64, realistic=True))
+    assert families(k) == ["igemm_i8"], k
 
 
 @pytest.mark.parametrize("variant", [4, 5, 6, 7, 8, 9, 10, 12, 13])

@@ -102,6 +102,9 @@ enum IgemmLoader : uint32_t {
     // (what it reads past the KW * C bytes meets zero weights).  Table: one entry per group,
     // kh in bits 24..30, run length KW * C in bits 0..15.
     kLoaderRuns = 2,
+    // a convolution window over an image with C % 64 == 0, addressed by the LDS-DMA ring kernel itself: a k-tile is 64
+    // channels of one tap, K = Kp = KH * KW * C.  Table: 64 bytes of input_zp (what a tap outside the image reads).
+    kLoaderWindow = 3,
 };
 
 // torq_hl.add folded into the epilogue of the convolution that produces one of its operands.

@@ -157,6 +157,7 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
         a.M = op.M; a.N = op.Nn; a.K = op.K; a.Kp = op.Kp; a.Np = op.Np;
         a.H = op.H; a.W = op.W; a.C = op.C; a.OH = op.OH; a.OW = op.OW;
         a.SH = op.SH; a.SW = op.SW; a.PT = op.PT; a.PL = op.PL;
+        a.KH = op.KH; a.KW = op.KW;
         a.input_zp = op.input_zp;
         a.out_dtype = op.out_dtype;
         a.a_bytes = (int64_t)op.N * op.H * op.W * op.C;

@@ -427,6 +427,9 @@ class Emitter {
             // otherwise the largest tile that still gives (nearly) every CU a tile
             const uint32_t order[] = {kIgemmDense256x256, kIgemmDense128x256, kIgemmDense128x128, kIgemmDense64x128};
             for (uint32_t v : order) {
+                // a short K leaves a 256 x 256 tile (one block per CU) mostly prologue and epilogue; two blocks per CU
+                // of half the size overlap them (256 -> 1024 channels at 56 x 56, batch 32: 75 -> 54 us)
+                if (v == kIgemmDense256x256 && K > 0 && K <= 512) continue;
                 // the wide-N tile only where N nearly fills whole tiles (padded columns are computed too)
                 if (v == kIgemmDense64x128 && ((roundUp(N, 128) - N) * 8 > N || getenv("THIP_NO_64X128"))) continue;
                 if (tiles(v) >= 224) return v;
@@ -444,12 +447,32 @@ class Emitter {
         return kIgemm64x64x64;
     }
 
+    // Tile of the ring kernel with window addressing: one tile column for few output channels (the image is read
+    // once), else the largest tile that still gives every CU a tile, two blocks per CU where there are many.
+    static uint32_t chooseWindowVariant(int64_t M, int64_t N) {
+        if (const char *env = getenv("THIP_WINDOW_VARIANT")) {
+            const long v = strtol(env, nullptr, 10);
+            if (v == kIgemmDense256x256 || v == kIgemmDense128x256 || v == kIgemmDense128x128 || v == kIgemmDense256x128 || v == kIgemmDense256x64) return (uint32_t)v;
+        }
+        auto tiles = [&](uint32_t v) {
+            const IgemmTile &t = igemmTile(v);
+            return ((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn);
+        };
+        if (N <= 64) return kIgemmDense256x64;
+        if (N <= 128) return kIgemmDense256x128;
+        // measured on 3x3 convolutions of 64 .. 512 channels at batch 32: the largest tile wins as soon as half the CUs
+        // get one (a long K per tile amortises its prologue and epilogue)
+        if (tiles(kIgemmDense256x256) >= 128) return kIgemmDense256x256;
+        if (tiles(kIgemmDense128x256) >= 128) return kIgemmDense128x256;
+        return kIgemmDense128x128;
+    }
+
     // conv2d / fully_connected / matmul as one igemm record.  `wAt(n, k)` returns
     // weight (n, k) with k = (kh * KW + kw) * C + ci.
     template <typename WeightAt>
     void emitIgemm(DescOp base, int64_t M, int64_t N, int64_t K, uint32_t loader, WeightAt wAt) {
         const bool dense = loader == kLoaderDense;
-        const uint32_t variant = chooseIgemmVariant(M, N, dense, K, base.out_dtype, loader == kLoaderRuns);
+        const uint32_t variant = loader == kLoaderWindow ? chooseWindowVariant(M, N) : chooseIgemmVariant(M, N, dense, K, base.out_dtype, loader == kLoaderRuns);
         const IgemmTile &t = igemmTile(variant);
         const int64_t Kp = roundUp(K, t.bk), Np = roundUp(N, t.bn);
         std::vector<int8_t> packed((size_t)(Np * Kp), 0);
@@ -482,6 +505,9 @@ class Emitter {
         base.Np = (int32_t)Np;
         if (dense) {
             base.gran = 16;
+        } else if (loader == kLoaderWindow) {
+            base.gran = 16;
+            base.table = newConst(std::vector<int8_t>(64, (int8_t)base.input_zp));
         } else if (loader == kLoaderRuns) {
             // K = KH groups of 16 bytes; entry: kh and the run length KW * C
             base.gran = 16;
@@ -666,7 +692,10 @@ thip_status_t Emitter::emitConv2d(const thip_hl_conv2d_t &c) {
             return wd[((n * C + b % C) * KH + kh) * KW + b / C];
         });
     } else {
-        emitIgemm(op, M, Oout, K, (pointwise && K % 16 == 0) ? kLoaderDense : kLoaderGather, [&](int64_t n, int64_t k) -> int8_t {
+        // a window over whole 64-channel k-tiles with enough rows for the large tiles: the LDS-DMA ring kernel addresses
+        // the window itself (THIP_NO_WINDOW_RING keeps such convolutions on the gather kernel, for tests and tuning)
+        const bool ring = !pointwise && Cin % 64 == 0 && M >= 2048 && Oout >= 32 && d.N * d.H * d.W * Cin < (1LL << 32) && !getenv("THIP_NO_WINDOW_RING");
+        emitIgemm(op, M, Oout, K, (pointwise && K % 16 == 0) ? kLoaderDense : ring ? kLoaderWindow : kLoaderGather, [&](int64_t n, int64_t k) -> int8_t {
             const int64_t pos = k / Cin, ci = k % Cin;
             const int64_t kh = pos / KW, kw = pos % KW;
             if (ci >= C || n >= O) return 0;  // padded channels meet zero weights

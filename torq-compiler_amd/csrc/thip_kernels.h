@@ -62,6 +62,7 @@ struct IgemmArgs {
     void *out;              // [M][N] elements of out_dtype
     int32_t M, N, K, Kp, Np;
     int32_t H, W, C, OH, OW, SH, SW, PT, PL;
+    int32_t KH, KW;         // window loader only
     int32_t input_zp;
     int32_t out_dtype;
     int64_t a_bytes;        // size of A in bytes (the run loader keeps its 16-byte loads inside it)

@@ -769,7 +769,14 @@ __device__ __forceinline__ void waitVmcnt() {
 // registers (int8 output, N % 16 == 0: the launcher checks) with 1 the plain 32-bit tail or 2 the general 32-bit tail
 // (a pre-shift, a clamp of acc + bias or a zero point that does not fold: e.g. small shifts under large scales,
 // where every result beyond a small |acc + bias| saturates).
-template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, int DIRECT, bool ADD = false>
+//
+// CONV: the activation operand is not a dense matrix but the patch matrix of a convolution over an N,H,W,C image
+// with C % 64 == 0, so that a k-tile is 64 consecutive channels of ONE window tap (kh, kw) and its chunk order is
+// the dense one.  Row m of the patch matrix is output pixel (n, oy, ox); the lane that loads it keeps the pixel's
+// window origin and, per k-tile, adds the tap's offset (wave-uniform, advanced with scalar selects: no division
+// and no branch in the loop).  A tap outside the image reads a 64-byte page of input_zp bytes instead (p.ktab):
+// the same number of loads whatever the padding, as the hand-counted waits need.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, int DIRECT, bool ADD = false, bool CONV = false>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_dense_i8(IgemmArgs p) {
     constexpr int BK = 64;
     constexpr int NW = WAVES_M * WAVES_N;
@@ -817,15 +824,30 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
     const int lchunk = (lane & 3) ^ ((lane >> 4) & 3);
     // per-lane byte offsets from the tile origins (rows past M are clamped to the last row: their
     // results are never stored, and every wave must issue the same number of loads)
-    const int8_t *aTile = p.A + (size_t)m0 * p.K;
+    const int8_t *aTile = CONV ? p.A : p.A + (size_t)m0 * p.K;
     const int8_t *bTile = p.Bp + (size_t)n0 * p.Kp;
     uint32_t aOff[LA], bOff[LB];
+    int winY[CONV ? LA : 1], winX[CONV ? LA : 1];  // CONV: input row / column of tap (0, 0) of the lane's output pixels
 #pragma unroll
     for (int i = 0; i < LA; i++) {
         int r = 16 * (wave + NW * i) + lrow;
         r = m0 + r < p.M ? r : p.M - 1 - m0;
-        aOff[i] = (uint32_t)r * (uint32_t)p.K + (uint32_t)lchunk * 16u;
+        if constexpr (CONV) {
+            const int m = m0 + r, frame = p.OH * p.OW;
+            const int n = m / frame, rem = m - n * frame;
+            const int oy = rem / p.OW, ox = rem - oy * p.OW;
+            winY[i] = oy * p.SH - p.PT;
+            winX[i] = ox * p.SW - p.PL;
+            // byte offset of the window origin (modulo 2^32: it may lie before the image; origin + tap does not)
+            aOff[i] = ((uint32_t)(n * p.H + winY[i]) * (uint32_t)p.W + (uint32_t)winX[i]) * (uint32_t)p.C + (uint32_t)lchunk * 16u;
+        } else {
+            aOff[i] = (uint32_t)r * (uint32_t)p.K + (uint32_t)lchunk * 16u;
+        }
     }
+    // CONV: the tap of the next k-tile to be issued and its byte offset from a window origin, all wave-uniform
+    int tapH = 0, tapW = 0, tapC = 0;
+    uint32_t tapOff = 0;
+    const int8_t *zpPage = CONV ? (const int8_t *)p.ktab + lchunk * 16 : nullptr;
 #pragma unroll
     for (int i = 0; i < LB; i++) {
         bOff[i] = (uint32_t)(16 * ((wave + NW * i) % BWL) + lrow) * (uint32_t)p.Kp + (uint32_t)lchunk * 16u;
@@ -876,9 +898,27 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
         for (int x = 0; x < LPT; x++) {
             if (x * parts / LPT != part) continue;
             if (x < LA) {
-                dmaLoad16(aBase, aOff[x] - back, stage + (unsigned)(wave + NW * x) * 1024u);
+                if constexpr (CONV) {
+                    const int y = winY[x] + tapH, xx = winX[x] + tapW;
+                    const bool inside = (unsigned)y < (unsigned)p.H && (unsigned)xx < (unsigned)p.W;
+                    const int8_t *src = inside ? p.A + (size_t)(uint32_t)(aOff[x] + tapOff) : zpPage;
+                    dmaLoad16(src, stage + (unsigned)(wave + NW * x) * 1024u);
+                } else {
+                    dmaLoad16(aBase, aOff[x] - back, stage + (unsigned)(wave + NW * x) * 1024u);
+                }
             } else {
                 dmaLoad16(bBase, bOff[x - LA], stage + A_STAGE + (unsigned)((wave + NW * (x - LA)) % BWL) * 1024u);
+            }
+        }
+        if constexpr (CONV) {
+            if (part == parts - 1) {
+                // on to the tap of tile kt + 1: 64 channels further, then the next column, then the next row of the window
+                const bool endC = tapC + 64 == p.C;
+                tapC = endC ? 0 : tapC + 64;
+                const bool endW = endC && tapW + 1 == p.KW;
+                tapW = endC ? (endW ? 0 : tapW + 1) : tapW;
+                tapH += endW ? 1 : 0;
+                tapOff = ((uint32_t)tapH * (uint32_t)p.W + (uint32_t)tapW) * (uint32_t)p.C + (uint32_t)tapC;
             }
         }
     };
@@ -1455,25 +1495,25 @@ static hipError_t launchIgemmLoader(const IgemmArgs &a, const LaunchCtx &ctx) {
     }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, int DIRECT, bool ADD = false>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, int DIRECT, bool ADD = false, bool CONV = false>
 static hipError_t launchIgemmDenseE(const IgemmArgs &a, const LaunchCtx &ctx) {
     // the stage ring, reused by the epilogue as staging slices (one per wave) plus bias/scale
     constexpr size_t ring = (size_t)STAGES * (BM + BN) * 64;
     constexpr size_t epilogue = (size_t)(BM / WAVES_M) * (WAVES_M * WAVES_N) * (32 * 4 + 16) + 2 * BN * 4;
     constexpr size_t smem = ring > epilogue ? ring : epilogue;
     static_assert(smem * BLOCKS_PER_CU <= 160 * 1024, "LDS of one CU");
-    auto kernel = igemm_dense_i8<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, DIRECT, ADD>;
+    auto kernel = igemm_dense_i8<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, DIRECT, ADD, CONV>;
     static std::once_flag once;
     static hipError_t configured = hipSuccess;
     std::call_once(once, [&] { configured = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); });
     if (configured != hipSuccess) return configured;
     const int tilesM = (a.M + BM - 1) / BM;
     const int tilesN = a.Np / BN;
-    THIP_ENQUEUE(ctx, kernelLabel("igemm_dense_i8", {BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, DIRECT, ADD}), kernel, dim3((unsigned)(tilesM * tilesN)), dim3(WAVES_M * WAVES_N * 64), smem, a);
+    THIP_ENQUEUE(ctx, kernelLabel(CONV ? "igemm_dense_conv_i8" : "igemm_dense_i8", {BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, DIRECT, ADD}), kernel, dim3((unsigned)(tilesM * tilesN)), dim3(WAVES_M * WAVES_N * 64), smem, a);
     return hipGetLastError();
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, bool CONV = false>
 static hipError_t launchIgemmDense(const IgemmArgs &a, const LaunchCtx &ctx) {
     // the in-register epilogue takes the 32-bit requant tails: the plain one (what wideRequant() calls plain), or, on
     // the large tiles, the general one (any shift of 32 and up, or a smaller one that the record's pre_shift lifts to 33)
@@ -1484,18 +1524,18 @@ static hipError_t launchIgemmDense(const IgemmArgs &a, const LaunchCtx &ctx) {
     const bool direct = inRegisters && plain;
     if (a.skip != nullptr) {
         // a residual add: the in-register epilogue of the small tile only (what a network's late, small layers take)
-        if constexpr (BM == 64 && BN == 64) {
+        if constexpr (BM == 64 && BN == 64 && !CONV) {
             if (!direct || ((uintptr_t)a.skip & 15) != 0) return hipErrorInvalidValue;
             return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, 1, true>(a, ctx);
         } else {
             return hipErrorInvalidValue;
         }
     }
-    if (direct) return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, 1>(a, ctx);
+    if (direct) return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, 1, false, CONV>(a, ctx);
     if constexpr (BM * BN >= 128 * 128) {
-        if (inRegisters && wide) return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, 2>(a, ctx);
+        if (inRegisters && wide) return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, 2, false, CONV>(a, ctx);
     }
-    return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, 0>(a, ctx);
+    return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, 0, false, CONV>(a, ctx);
 }
 
 hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, const LaunchCtx &ctx) {
@@ -1516,6 +1556,22 @@ hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, const LaunchCtx &ct
         if (!a.ktab || a.C <= 0 || a.C % (int)a.gran != 0) return hipErrorInvalidValue;
         if (a.OH <= 0 || a.OW <= 0 || a.M % (a.OH * a.OW) != 0) return hipErrorInvalidValue;
         if (((uintptr_t)a.A & (a.gran - 1)) != 0) return hipErrorInvalidValue;
+    } else if (a.loader == kLoaderWindow) {
+        // the ring kernel's window addressing: whole k-tiles per tap, 32-bit byte offsets into the image, a page of
+        // zero-point bytes behind ktab, every tap offset non-negative once the tap lies inside the image
+        if (!a.ktab || ((uintptr_t)a.ktab & 15) != 0 || a.C <= 0 || a.C % 64 != 0 || a.KH <= 0 || a.KW <= 0) return hipErrorInvalidValue;
+        if (a.H <= 0 || a.W <= 0 || a.OH <= 0 || a.OW <= 0 || a.SH <= 0 || a.SW <= 0 || a.PT < 0 || a.PL < 0) return hipErrorInvalidValue;
+        if (a.M % (a.OH * a.OW) != 0 || (long long)a.K != (long long)a.KH * a.KW * a.C || a.Kp != a.K) return hipErrorInvalidValue;
+        if (a.a_bytes != (long long)(a.M / (a.OH * a.OW)) * a.H * a.W * a.C || a.a_bytes >= (1LL << 32)) return hipErrorInvalidValue;
+        if (((uintptr_t)a.A & 15) != 0 || a.skip != nullptr) return hipErrorInvalidValue;
+        switch (variant) {
+        case kIgemmDense256x256: return launchIgemmDense<256, 256, 2, 2, 4, 1, true>(a, ctx);
+        case kIgemmDense128x256: return launchIgemmDense<128, 256, 2, 2, 3, 2, true>(a, ctx);
+        case kIgemmDense128x128: return launchIgemmDense<128, 128, 2, 2, 4, 2, true>(a, ctx);
+        case kIgemmDense256x128: return launchIgemmDense<256, 128, 2, 2, 3, 2, true>(a, ctx);
+        case kIgemmDense256x64: return launchIgemmDense<256, 64, 4, 1, 3, 2, true>(a, ctx);
+        default: return hipErrorInvalidValue;
+        }
     } else {
         return hipErrorInvalidValue;
     }

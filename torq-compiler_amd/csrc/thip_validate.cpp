@@ -180,7 +180,23 @@ thip_status_t checkOpFootprint(const DescriptorView *e, uint32_t i) {
         if ((s = need(op.weights, mul(op.Np, op.Kp), "weights"))) return s;
         if ((s = need(op.bias, (uint64_t)op.Np * 4, "bias"))) return s;
         if ((s = need(op.scale, (uint64_t)op.Np * 4, "scale"))) return s;
-        if (op.loader > kLoaderRuns) return fail(THIP_INVALID_ARGUMENT, "op %u: unknown igemm loader %u", i, op.loader);
+        if (op.loader > kLoaderWindow) return fail(THIP_INVALID_ARGUMENT, "op %u: unknown igemm loader %u", i, op.loader);
+        if (op.loader == kLoaderWindow) {
+            if (!positive({op.KH, op.KW, op.SH, op.SW}) || op.PT < 0 || op.PL < 0 || op.C % 64 != 0 || mul(op.KH, op.KW, op.C) != (uint64_t)op.K || op.Kp != op.K) {
+                return fail(THIP_INVALID_ARGUMENT, "op %u: the window loader needs whole 64-channel k-tiles per tap", i);
+            }
+            if (inBytes >= (1ull << 32)) return fail(THIP_INVALID_ARGUMENT, "op %u: image too large for the window loader", i);
+            switch (op.variant) {
+            case kIgemmDense256x256: case kIgemmDense128x256: case kIgemmDense128x128: case kIgemmDense256x128: case kIgemmDense256x64: break;
+            default: return fail(THIP_INVALID_ARGUMENT, "op %u: the window loader has no kernel for tile variant %u", i, op.variant);
+            }
+            if (op.table.space != kSpaceConst) return fail(THIP_INVALID_ARGUMENT, "op %u: table must be a constant", i);
+            if ((s = need(op.table, 64, "zero-point page"))) return s;
+            const uint8_t *page = e->blob + e->header.data_offset + e->consts[op.table.index].offset + op.table.offset;
+            for (int b = 0; b < 64; b++) {
+                if ((int8_t)page[b] != (int8_t)op.input_zp) return fail(THIP_INVALID_ARGUMENT, "op %u: the zero-point page does not hold input_zp", i);
+            }
+        }
         if (op.loader == kLoaderRuns) {
             if (!positive({op.KH, op.KW}) || (int64_t)op.KW * op.C > 16 || op.Kp % 16 != 0) return fail(THIP_INVALID_ARGUMENT, "op %u: a window row of %d x %d bytes does not fit a 16-byte run", i, op.KW, op.C);
             if (op.table.space != kSpaceConst) return fail(THIP_INVALID_ARGUMENT, "op %u: table must be a constant", i);
