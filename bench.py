@@ -48,6 +48,11 @@ def workload_table(pkg):
         "fc_16x2048x8192": (lambda: w.fully_connected_workload(16, 2048, 8192), "hbm"),
         "fc_1x2048x2048": (lambda: w.fully_connected_workload(1, 2048, 2048), "hbm"),
         "conv_112x112x32_o64_3x3": (lambda: w.conv2d_workload(), "mfma"),
+        # large convolutions (the benchmark's own convolution is 0.46 GOP): 3x3 over 256 / 512 channels at batch 32, 118 GOP each,
+        # and a pointwise expansion whose K is short
+        "conv3x3_56x56x256_o256_b32": (lambda: w.conv2d_workload(N=32, H=56, W=56, C=256, O=256, realistic=True), "mfma"),
+        "conv3x3_28x28x512_o512_b32": (lambda: w.conv2d_workload(N=32, H=28, W=28, C=512, O=512, realistic=True), "mfma"),
+        "conv1x1_56x56x256_o1024_b32": (lambda: w.conv2d_workload(N=32, H=56, W=56, C=256, O=1024, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True), "mfma"),
         "depthwise_b64": (lambda: w.depthwise_workload(N=64), "hbm"),
         "depthwise_b1": (lambda: w.depthwise_workload(N=1), "hbm"),
         "depthwise_s1_b256": (lambda: w.depthwise_workload(N=256, stride=(1, 1), pad=(1, 1, 1, 1)), "hbm"),
