@@ -128,16 +128,18 @@ class Loaded:
 # (KiB per dispatch; the factors are what the same counters read for a plain 256 MiB copy, --copy-calibration).
 # They belong to the kernels as they were when the counters were read: TRAFFIC_KERNELS_SHA256 is the hash of
 # torq-compiler_amd/csrc/thip_kernels.hip at that time, and a run on other kernel sources reports traffic null.
-TRAFFIC_KERNELS_SHA256 = "unset"
+TRAFFIC_KERNELS_SHA256 = "61bc9c8507c66e983329eebd70b7a98a43bbff9833d79ce92b0d614a9e1f0f30"
 MEASURED_TRAFFIC = {
-    "fc_4096x4096x4096": (49392.2 * 1.9995 + 16566.1) * 1024,
-    "fc_512x4096x4096": (16481.0 * 1.9995 + 2048.0) * 1024,
-    "fc_16x2048x8192": (8408.1 * 1.9995 + 256.0) * 1024,
-    "conv_112x112x32_o64_3x3": (354.9 * 1.9995 + 784.0) * 1024,
-    "depthwise_b64": (15240.6 * 1.9995 + 7064.0) * 1024,
-    "depthwise_s1_b256": (63656.6 * 1.9995 + 113084.5) * 1024,
-    "avgpool_b64": (1991.6 * 1.9995 + 80.0) * 1024,
-    "add_b64": (4722.6 * 1.9995 + 4704.0) * 1024,
+    "fc_4096x4096x4096": (49377.5 * 1.9995 + 16597.5 * 1.0000) * 1024,
+    "fc_512x4096x4096": (16477.0 * 1.9995 + 2048.0 * 1.0000) * 1024,
+    "fc_16x2048x8192": (8408.0 * 1.9995 + 256.0 * 1.0000) * 1024,
+    "conv_112x112x32_o64_3x3": (358.9 * 1.9995 + 784.0 * 1.0000) * 1024,
+    "conv3x3_56x56x256_o256_b32": (17231.9 * 1.9995 + 25977.5 * 1.0000) * 1024,
+    "depthwise_b64": (15498.8 * 1.9995 + 7063.5 * 1.0000) * 1024,
+    "depthwise_s1_b256": (63711.9 * 1.9995 + 113170.4 * 1.0000) * 1024,
+    "maxpool_b64": (25112.3 * 1.9995 + 12544.0 * 1.0000) * 1024,
+    "avgpool_b64": (1998.5 * 1.9995 + 80.0 * 1.0000) * 1024,
+    "add_b64": (4723.0 * 1.9995 + 4704.0 * 1.0000) * 1024,
 }
 
 
@@ -378,8 +380,10 @@ def main():
             else:
                 ms = warm
                 row["us"] = round(ms * 1e3, 2)
-            r = roofline(o.wl, bnd, ms)
+            r = roofline(o.wl, bnd, ms, name)
             row.update({"GOP/s": round(o.wl.ops / (ms * 1e-3) / 1e9, 1), "GB/s": round(o.wl.bytes / (ms * 1e-3) / 1e9, 1), "frac": r["frac"]})
+            if r["traffic"] is not None:
+                row["traffic"] = r["traffic"]  # HBM bytes per launch from the rocprofv3 counters (MEASURED_TRAFFIC)
             if not args.no_cpu:
                 row["parity_checked"] = verify_sample(o)
                 ok = ok and row["parity_checked"]
