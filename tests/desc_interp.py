@@ -128,8 +128,9 @@ def run(blob, binding_arrays):
             elif int(op["loader"]) == 3:  # the ring kernel's own window addressing: k-tile t is 64 channels of tap t * 64 // C
                 Nimg, H, W, C = (int(op[k]) for k in ["N", "H", "W", "C"])
                 OH, OW, SH, SW, PT, PL, KH, KW = (int(op[k]) for k in ["OH", "OW", "SH", "SW", "PT", "PL", "KH", "KW"])
-                assert C % 64 == 0 and K == Kp == KH * KW * C and int(op["variant"]) in (4, 5, 6, 8, 9)
-                page = view(op["table"], 64).view(np.int8)
+                assert C % 64 == 0 and K == Kp == KH * KW * C and int(op["variant"]) in (4, 5, 6, 8, 9, 14)
+                assert int(op["variant"]) != 14 or C % 128 == 0
+                page = view(op["table"], 128).view(np.int8)
                 assert (page == int(op["input_zp"])).all()
                 x = view(op["in0"], Nimg * H * W * C).view(np.int8).reshape(Nimg, H, W, C)
                 A = np.zeros((Nimg, OH, OW, Kp), dtype=np.int64)
@@ -164,7 +165,9 @@ def run(blob, binding_arrays):
                     vals = np.where(inside[None, :, :, None], vals, int(op["input_zp"]))
                     A[..., e * g:(e + 1) * g] = vals
                 A = A.reshape(M, Kp)
-            acc = A @ Wp.T  # M x Np
+            # M x Np; as float64 through BLAS where that is exact (|acc| <= Kp * 2^14 < 2^53 always holds for int8 operands)
+            assert Kp < (1 << 38)
+            acc = np.rint(A.astype(np.float64) @ Wp.T.astype(np.float64)).astype(np.int64)
             q = _requant_vec(acc[:, :N], bias[None, :N], scale[None, :N], sh, zp, mn, mx, int(op["pre_shift"]), int(op["t0_clamp"]))
             odt = OUT_NP[int(op["out_dtype"])]
             res = q.astype(odt).reshape(-1)

@@ -59,6 +59,23 @@ WINDOW_RING = [
 ]
 
 
+def test_dense_k128_records(monkeypatch):
+    """A long K with enough 256 x 256 tiles takes the variant with 128-byte k-tiles: K padded to 128, same results."""
+    wl = w.fully_connected_workload(3584, 1040, 4096, realistic=True)
+    outs, d = interp(wl)
+    assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)
+    assert int(d.ops[0]["variant"]) == 14 and int(d.ops[0]["Kp"]) == 1152
+    monkeypatch.setenv("THIP_NO_K128", "1")
+    assert int(interp(wl)[1].ops[0]["variant"]) == 4
+    monkeypatch.delenv("THIP_NO_K128")
+    monkeypatch.setenv("THIP_IGEMM_DENSE_VARIANT", "14")
+    for mkn in ((300, 48, 272), (33, 400, 40), (257, 128, 520)):
+        wl = w.fully_connected_workload(*mkn, realistic=True)
+        outs, d = interp(wl)
+        assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)
+        assert int(d.ops[0]["variant"]) == 14 and int(d.ops[0]["Kp"]) % 128 == 0
+
+
 def test_conv2d_window_loader_records():
     """Whole 64-channel k-tiles and enough rows: the record asks for the ring kernel's window addressing (loader 3, a
     64-byte zero-point page as its table); fewer rows, other channel counts or the switch keep the gather loader."""

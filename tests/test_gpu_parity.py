@@ -90,6 +90,21 @@ def test_conv2d_window_ring_every_tile(device, variant, monkeypatch):
     assert k[0].startswith(names[variant]), k
 
 
+def test_conv2d_window_ring_k128(device, monkeypatch):
+    """C % 128 == 0 and at least 128 tiles of 256 x 256: k-tiles of 128 channels of one tap."""
+    k = check(device, w.conv2d_workload(N=8, H=64, W=64, C=128, O=256, realistic=True), via="device")
+    assert k[0] == "igemm_dense_conv_i8<256,256,2,2,2,1,1,0>", k
+    monkeypatch.setenv("THIP_WINDOW_VARIANT", "14")
+    for kw in (dict(N=2, H=33, W=35, C=128, O=80, pad=(1, 1, 1, 1)), dict(N=5, H=47, W=45, C=256, O=48, stride=(2, 2), pad=(1, 0, 1, 0), output_zp=-7, output_min=-128),
+               dict(N=3, H=30, W=30, C=384, O=40, KH=2, KW=5, pad=(3, 1, 0, 1))):
+        k = check(device, w.conv2d_workload(realistic=True, **kw), via="device")
+        assert k[0].startswith("igemm_dense_conv_i8<256,256,2,2,2,1,"), k
+    k = check(device, w.conv2d_workload(N=2, H=32, W=32, C=128, O=64, realistic=False))  # the literal requant range
+    assert k[0].startswith("igemm_dense_conv_i8<256,256,2,2,2,1,"), k
+    k = check(device, w.conv2d_workload(N=2, H=32, W=32, C=64, O=64, realistic=True))    # C % 128 != 0: the switch does not apply
+    assert k[0].startswith("igemm_dense_conv_i8<256,64,"), k
+
+
 def test_conv2d_window_ring_switch(device, monkeypatch):
     monkeypatch.setenv("THIP_NO_WINDOW_RING", "1")
     k = check(device, w.conv2d_workload(N=2, H=32, W=32, C=64, O=64, realistic=True))
@@ -109,6 +124,30 @@ def test_dense_igemm_every_tile_variant(device, variant, monkeypatch):
     check(device, w.fully_connected_workload(33, 16, 1000, realistic=True))
     check(device, w.fully_connected_workload(1000, 4096, 272, realistic=True))
     check(device, w.conv2d_workload(N=2, H=28, W=28, C=192, O=32, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True))
+
+
+def test_dense_igemm_k128(device, monkeypatch):
+    """k-tiles of 128 bytes (whole cache lines per tile row, four MFMA phases, two ring stages): taken by itself for a
+    long K with enough tiles, forced here on ragged M / N, K tails that end inside a k-tile (at every 16-byte chunk),
+    K shorter than one k-tile and than the ring, every epilogue."""
+    k = check(device, w.fully_connected_workload(4096, 1024, 4096, realistic=True), via="device")
+    assert k[0] == "igemm_dense_k128_i8<256,256,2,2,2,1,1,0>", k       # chosen without a switch
+    k = check(device, w.fully_connected_workload(4096, 1024, 4096), via="device")
+    assert k[0] == "igemm_dense_k128_i8<256,256,2,2,2,1,2,0>", k       # the literal requant range: the general 32-bit tail
+    monkeypatch.setenv("THIP_IGEMM_DENSE_VARIANT", "14")
+    for K in (16, 48, 112, 128, 144, 240, 256, 272, 400, 1024 + 64, 2048 + 16):
+        k = check(device, w.fully_connected_workload(300, K, 272, realistic=True))
+        assert k[0].startswith("igemm_dense_k128_i8<256,256,2,2,2,1,"), k
+    k = check(device, w.fully_connected_workload(300, 192, 520, realistic=True))
+    assert k[0].endswith(",0,0>"), k                                    # N % 16 != 0: the staged epilogue
+    check(device, w.fully_connected_workload(513, 1024, 515, realistic=True))
+    check(device, w.fully_connected_workload(17, 4096, 16, realistic=True))
+    check(device, w.conv2d_workload(N=2, H=28, W=28, C=192, O=32, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True))
+    check(device, w.matmul_workload(2, 70, 200, 90))                    # run-time input2: transposed into rows of Kp = 256
+    monkeypatch.setenv("THIP_NO_K128", "1")
+    monkeypatch.delenv("THIP_IGEMM_DENSE_VARIANT")
+    k = check(device, w.fully_connected_workload(4096, 1024, 4096, realistic=True), via="device")
+    assert k[0] == "igemm_dense_i8<256,256,2,2,4,1,1,0>", k
 
 
 @pytest.mark.parametrize("variant", [4, 7, 9, 13])

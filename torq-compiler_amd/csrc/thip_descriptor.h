@@ -103,7 +103,8 @@ enum IgemmLoader : uint32_t {
     // kh in bits 24..30, run length KW * C in bits 0..15.
     kLoaderRuns = 2,
     // a convolution window over an image with C % 64 == 0, addressed by the LDS-DMA ring kernel itself: a k-tile is 64
-    // channels of one tap, K = Kp = KH * KW * C.  Table: 64 bytes of input_zp (what a tap outside the image reads).
+    // channels of one tap (128 with C % 128 == 0 on the 128-byte variant), K = Kp = KH * KW * C.  Table: 128 bytes of input_zp
+    // (what a tap outside the image reads).
     kLoaderWindow = 3,
 };
 

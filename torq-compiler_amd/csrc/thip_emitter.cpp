@@ -426,6 +426,8 @@ class Emitter {
             }
             // otherwise the largest tile that still gives (nearly) every CU a tile
             const uint32_t order[] = {kIgemmDense256x256, kIgemmDense128x256, kIgemmDense128x128, kIgemmDense64x128};
+            // a long K on the largest tile: k-tiles of 128 bytes, whole cache lines per row (THIP_NO_K128 keeps 64)
+            if (K >= 1024 && tiles(kIgemmDense256x256) >= 224 && !getenv("THIP_NO_K128")) return kIgemmDense256x256K128;
             for (uint32_t v : order) {
                 // a short K leaves a 256 x 256 tile (one block per CU) mostly prologue and epilogue; two blocks per CU
                 // of half the size overlap them (256 -> 1024 channels at 56 x 56, batch 32: 75 -> 54 us)
@@ -449,10 +451,11 @@ class Emitter {
 
     // Tile of the ring kernel with window addressing: one tile column for few output channels (the image is read
     // once), else the largest tile that still gives every CU a tile, two blocks per CU where there are many.
-    static uint32_t chooseWindowVariant(int64_t M, int64_t N) {
+    static uint32_t chooseWindowVariant(int64_t M, int64_t N, int64_t C) {
         if (const char *env = getenv("THIP_WINDOW_VARIANT")) {
             const long v = strtol(env, nullptr, 10);
             if (v == kIgemmDense256x256 || v == kIgemmDense128x256 || v == kIgemmDense128x128 || v == kIgemmDense256x128 || v == kIgemmDense256x64) return (uint32_t)v;
+            if (v == kIgemmDense256x256K128 && C % 128 == 0) return (uint32_t)v;
         }
         auto tiles = [&](uint32_t v) {
             const IgemmTile &t = igemmTile(v);
@@ -462,7 +465,7 @@ class Emitter {
         if (N <= 128) return kIgemmDense256x128;
         // measured on 3x3 convolutions of 64 .. 512 channels at batch 32: the largest tile wins as soon as half the CUs
         // get one (a long K per tile amortises its prologue and epilogue)
-        if (tiles(kIgemmDense256x256) >= 128) return kIgemmDense256x256;
+        if (tiles(kIgemmDense256x256) >= 128) return (C % 128 == 0 && !getenv("THIP_NO_K128")) ? kIgemmDense256x256K128 : kIgemmDense256x256;
         if (tiles(kIgemmDense128x256) >= 128) return kIgemmDense128x256;
         return kIgemmDense128x128;
     }
@@ -472,7 +475,7 @@ class Emitter {
     template <typename WeightAt>
     void emitIgemm(DescOp base, int64_t M, int64_t N, int64_t K, uint32_t loader, WeightAt wAt) {
         const bool dense = loader == kLoaderDense;
-        const uint32_t variant = loader == kLoaderWindow ? chooseWindowVariant(M, N) : chooseIgemmVariant(M, N, dense, K, base.out_dtype, loader == kLoaderRuns);
+        const uint32_t variant = loader == kLoaderWindow ? chooseWindowVariant(M, N, base.C) : chooseIgemmVariant(M, N, dense, K, base.out_dtype, loader == kLoaderRuns);
         const IgemmTile &t = igemmTile(variant);
         const int64_t Kp = roundUp(K, t.bk), Np = roundUp(N, t.bn);
         std::vector<int8_t> packed((size_t)(Np * Kp), 0);
@@ -507,7 +510,7 @@ class Emitter {
             base.gran = 16;
         } else if (loader == kLoaderWindow) {
             base.gran = 16;
-            base.table = newConst(std::vector<int8_t>(64, (int8_t)base.input_zp));
+            base.table = newConst(std::vector<int8_t>(128, (int8_t)base.input_zp));
         } else if (loader == kLoaderRuns) {
             // K = KH groups of 16 bytes; entry: kh and the run length KW * C
             base.gran = 16;

@@ -96,7 +96,8 @@ enum IgemmVariant : uint32_t {
     kIgemmStream = 11,
     kIgemmDense128x64 = 12,  // mid-sized problems: enough tiles to fill the chip at a better ratio of loads to MFMAs than 64x64
     kIgemmDense64x128 = 13,
-    kIgemmVariantCount = 14,
+    kIgemmDense256x256K128 = 14,  // k-tiles of 128 bytes: whole cache lines per tile row, two stages
+    kIgemmVariantCount = 15,
 };
 struct IgemmTile {
     int bm, bn, bk;

@@ -771,24 +771,34 @@ __device__ __forceinline__ void waitVmcnt() {
 // where every result beyond a small |acc + bias| saturates).
 //
 // CONV: the activation operand is not a dense matrix but the patch matrix of a convolution over an N,H,W,C image
-// with C % 64 == 0, so that a k-tile is 64 consecutive channels of ONE window tap (kh, kw) and its chunk order is
+// with C % BK == 0, so that a k-tile is BK consecutive channels of ONE window tap (kh, kw) and its chunk order is
 // the dense one.  Row m of the patch matrix is output pixel (n, oy, ox); the lane that loads it keeps the pixel's
 // window origin and, per k-tile, adds the tap's offset (wave-uniform, advanced with scalar selects: no division
-// and no branch in the loop).  A tap outside the image reads a 64-byte page of input_zp bytes instead (p.ktab):
+// and no branch in the loop).  A tap outside the image reads a 128-byte page of input_zp bytes instead (p.ktab):
 // the same number of loads whatever the padding, as the hand-counted waits need.
-template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, int DIRECT, bool ADD = false, bool CONV = false>
+//
+// BK = 128: a k-tile is 128 bytes of K, so that the eight lanes that load one tile row fetch a whole 128-byte line
+// (with BK = 64 every request to L2 is half a line, and the path L2 -> LDS is bound by requests, not bytes: the bare
+// DMA stream of a 4096^3 problem takes 44 us in half lines and 30 us in whole ones).  One DMA instruction then covers
+// 8 rows, slot p of row r holds chunk p ^ ((r >> 1) & 7) (row pitch 128 bytes = 32 banks: the 16 rows of a ds_read_b128
+// phase again fall into 16 distinct bank groups), and a k-tile is four MFMA phases.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, int DIRECT, bool ADD = false, bool CONV = false, int BK = 64>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_dense_i8(IgemmArgs p) {
-    constexpr int BK = 64;
+    static_assert(BK == 64 || BK == 128, "k-tile of 64 or 128 bytes");
+    constexpr int CH = BK / 16;    // 16-byte chunks per tile row
+    constexpr int RPI = 64 / CH;   // tile rows one DMA instruction covers
+    constexpr int NP = BK / 32;    // MFMA phases per k-tile
     constexpr int NW = WAVES_M * WAVES_N;
     constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
     constexpr int TM = WTM / 32, TN = WTN / 32;
-    constexpr int BWL = BN / 16;                          // wave-loads (16 rows each) that make up the B tile
-    constexpr int LA = BM / 16 / NW, LB = (BWL + NW - 1) / NW;  // DMA instructions per wave per k-tile
+    constexpr int BWL = BN / RPI;                          // wave-loads (RPI rows each) that make up the B tile
+    constexpr int LA = BM / RPI / NW, LB = (BWL + NW - 1) / NW;  // DMA instructions per wave per k-tile
     constexpr int LPT = LA + LB;
     constexpr int A_STAGE = BM * BK, B_STAGE = BN * BK, STAGE = A_STAGE + B_STAGE;
     // every wave must issue the same number of loads: a narrow B tile (fewer wave-loads than
     // waves) is loaded redundantly, several waves writing the same bytes to the same place
-    static_assert(BM % (16 * NW) == 0 && BN % 16 == 0 && (BWL % NW == 0 || BWL < NW), "unbalanced DMA loads");
+    static_assert(BM % (RPI * NW) == 0 && BN % RPI == 0 && (BWL % NW == 0 || BWL < NW), "unbalanced DMA loads");
+    static_assert(BK == 64 || (NW % 2 == 0 && BWL % 2 == 0), "the 128-byte swizzle takes the parity of a wave-load from the wave");
     static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tile must be a multiple of the MFMA tile");
     static_assert(STAGES >= 2 && STAGES <= 8 && LPT * (STAGES - 1) < 64, "vmcnt is a 6-bit counter");
 
@@ -820,8 +830,10 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
 
     // DMA source pointers: lane l of a wave-load covers row l / 4 of its 16 rows and
     // fetches the logical chunk that belongs at slot l % 4 of that row.
-    const int lrow = lane >> 2;
-    const int lchunk = (lane & 3) ^ ((lane >> 4) & 3);
+    const int lrow = lane / CH;
+    // the swizzle of the row a lane loads: (row >> 2) & 3 for 64-byte rows; (row >> 1) & 7 for 128-byte rows, where
+    // row = 8 * (wave-load index) + lrow and the index has the wave's parity (NW and BWL are even)
+    const int lchunk = BK == 64 ? ((lane & 3) ^ ((lane >> 4) & 3)) : ((lane & 7) ^ ((((wave & 1) << 2) + (lrow >> 1)) & 7));
     // per-lane byte offsets from the tile origins (rows past M are clamped to the last row: their
     // results are never stored, and every wave must issue the same number of loads)
     const int8_t *aTile = CONV ? p.A : p.A + (size_t)m0 * p.K;
@@ -830,7 +842,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
     int winY[CONV ? LA : 1], winX[CONV ? LA : 1];  // CONV: input row / column of tap (0, 0) of the lane's output pixels
 #pragma unroll
     for (int i = 0; i < LA; i++) {
-        int r = 16 * (wave + NW * i) + lrow;
+        int r = RPI * (wave + NW * i) + lrow;
         r = m0 + r < p.M ? r : p.M - 1 - m0;
         if constexpr (CONV) {
             const int m = m0 + r, frame = p.OH * p.OW;
@@ -850,7 +862,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
     const int8_t *zpPage = CONV ? (const int8_t *)p.ktab + lchunk * 16 : nullptr;
 #pragma unroll
     for (int i = 0; i < LB; i++) {
-        bOff[i] = (uint32_t)(16 * ((wave + NW * i) % BWL) + lrow) * (uint32_t)p.Kp + (uint32_t)lchunk * 16u;
+        bOff[i] = (uint32_t)(RPI * ((wave + NW * i) % BWL) + lrow) * (uint32_t)p.Kp + (uint32_t)lchunk * 16u;
     }
     v16i acc[TN][TM];
 #pragma unroll
@@ -864,8 +876,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
 
     // Fragment addresses: row (l & 31) of a 32-row MFMA tile, logical chunk 2 * kk + (l >> 5).
     const int fr = lane & 31;
-    const int swz = (fr >> 2) & 3;
-    const int off0 = (((lane >> 5)) ^ swz) * 16;  // kk = 0; kk = 1 is off0 ^ 32
+    const int swz = BK == 64 ? ((fr >> 2) & 3) : ((fr >> 1) & 7);
+    const int off0 = (((lane >> 5)) ^ swz) * 16;  // phase kk = 0; phase kk is off0 ^ (32 kk)
     const int aFrag = (wm * WTM + fr) * BK + off0;
     const int bFrag = A_STAGE + (wn * WTN + fr) * BK + off0;
 
@@ -879,7 +891,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
     const int KT = p.Kp / BK;
 
     // Software pipeline.  The ring holds tiles kt+1 .. kt+STAGES while tile kt is computed.
-    // Each k-tile is two MFMA phases (k halves of 32).  While phase 0 runs, the fragments
+    // Each k-tile is NP MFMA phases (k slices of 32; described here for two).  While phase 0 runs, the fragments
     // of phase 1 are read from LDS; then the wave waits for tile kt+1, meets the block at the
     // barrier, and while phase 1 runs it refills the stage it just finished with tile
     // kt+STAGES and reads phase 0 of tile kt+1.  LDS latency and the DMA issue thus hide
@@ -913,8 +925,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
         if constexpr (CONV) {
             if (part == parts - 1) {
                 // on to the tap of tile kt + 1: 64 channels further, then the next column, then the next row of the window
-                const bool endC = tapC + 64 == p.C;
-                tapC = endC ? 0 : tapC + 64;
+                const bool endC = tapC + BK == p.C;
+                tapC = endC ? 0 : tapC + BK;
                 const bool endW = endC && tapW + 1 == p.KW;
                 tapW = endC ? (endW ? 0 : tapW + 1) : tapW;
                 tapH += endW ? 1 : 0;
@@ -953,19 +965,26 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
         constexpr bool kSteady = decltype(steady)::value;
         const int8_t *st = smem + (kt % STAGES) * STAGE;
         const int8_t *stNext = smem + ((kt + 1) % STAGES) * STAGE;
-        // phase 0: MFMAs on (af0, bf0); the reads of (af1, bf1) go out behind the first weight row
-        // (so that the wait in front of that row only covers reads issued a phase ago) and
+        // every phase but the last: MFMAs on the current fragments; the reads of the next phase's go out behind the
+        // first weight row (so that the wait in front of that row only covers reads issued a phase ago) and
         // complete under the remaining rows
+        auto phase = [&](v4i(&afC)[TM], v4i(&bfC)[TN], v4i(&afN)[TM], v4i(&bfN)[TN], int kkNext) {
 #pragma unroll
-        for (int j = 0; j < TN; j++) {
+            for (int j = 0; j < TN; j++) {
 #pragma unroll
-            for (int i = 0; i < TM; i++) acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf0[j], af0[i], acc[j][i], 0, 0, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            if (j == 0) {
-#pragma unroll
-                for (int x = 0; x < NF; x++) readFrag(st, 1, x, af1, bf1);
+                for (int i = 0; i < TM; i++) acc[j][i] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bfC[j], afC[i], acc[j][i], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
+                if (j == 0) {
+#pragma unroll
+                    for (int x = 0; x < NF; x++) readFrag(st, kkNext, x, afN, bfN);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
+        };
+        phase(af0, bf0, af1, bf1, 1);
+        if constexpr (NP == 4) {
+            phase(af1, bf1, af0, bf0, 2);
+            phase(af0, bf0, af1, bf1, 3);
         }
         // tile kt+1 must have landed; tiles kt+2 .. kt+STAGES-1 may stay in flight
         const bool more = kSteady || kt + 1 < KT;
@@ -992,7 +1011,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
         asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");  // this wave's reads of tile kt are complete
         blockBarrier();  // tile kt+1 is visible to everyone, and nobody reads stage kt % STAGES any more
         const bool refill = kSteady || kt + STAGES < KT;
-        // phase 1: MFMAs on (af1, bf1), the reads of the next phase 0 behind the first weight row,
+        // last phase: MFMAs on (af1, bf1), the reads of the next phase 0 behind the first weight row,
         // the refill of the freed stage spread between the rows
 #pragma unroll
         for (int j = 0; j < TN; j++) {
@@ -1495,25 +1514,25 @@ static hipError_t launchIgemmLoader(const IgemmArgs &a, const LaunchCtx &ctx) {
     }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, int DIRECT, bool ADD = false, bool CONV = false>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, int DIRECT, bool ADD = false, bool CONV = false, int BK = 64>
 static hipError_t launchIgemmDenseE(const IgemmArgs &a, const LaunchCtx &ctx) {
     // the stage ring, reused by the epilogue as staging slices (one per wave) plus bias/scale
-    constexpr size_t ring = (size_t)STAGES * (BM + BN) * 64;
+    constexpr size_t ring = (size_t)STAGES * (BM + BN) * BK;
     constexpr size_t epilogue = (size_t)(BM / WAVES_M) * (WAVES_M * WAVES_N) * (32 * 4 + 16) + 2 * BN * 4;
     constexpr size_t smem = ring > epilogue ? ring : epilogue;
     static_assert(smem * BLOCKS_PER_CU <= 160 * 1024, "LDS of one CU");
-    auto kernel = igemm_dense_i8<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, DIRECT, ADD, CONV>;
+    auto kernel = igemm_dense_i8<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, DIRECT, ADD, CONV, BK>;
     static std::once_flag once;
     static hipError_t configured = hipSuccess;
     std::call_once(once, [&] { configured = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem); });
     if (configured != hipSuccess) return configured;
     const int tilesM = (a.M + BM - 1) / BM;
     const int tilesN = a.Np / BN;
-    THIP_ENQUEUE(ctx, kernelLabel(CONV ? "igemm_dense_conv_i8" : "igemm_dense_i8", {BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, DIRECT, ADD}), kernel, dim3((unsigned)(tilesM * tilesN)), dim3(WAVES_M * WAVES_N * 64), smem, a);
+    THIP_ENQUEUE(ctx, kernelLabel(CONV ? "igemm_dense_conv_i8" : BK == 128 ? "igemm_dense_k128_i8" : "igemm_dense_i8", {BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, DIRECT, ADD}), kernel, dim3((unsigned)(tilesM * tilesN)), dim3(WAVES_M * WAVES_N * 64), smem, a);
     return hipGetLastError();
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, bool CONV = false>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int STAGES, int BLOCKS_PER_CU, bool CONV = false, int BK = 64>
 static hipError_t launchIgemmDense(const IgemmArgs &a, const LaunchCtx &ctx) {
     // the in-register epilogue takes the 32-bit requant tails: the plain one (what wideRequant() calls plain), or, on
     // the large tiles, the general one (any shift of 32 and up, or a smaller one that the record's pre_shift lifts to 33)
@@ -1531,11 +1550,11 @@ static hipError_t launchIgemmDense(const IgemmArgs &a, const LaunchCtx &ctx) {
             return hipErrorInvalidValue;
         }
     }
-    if (direct) return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, 1, false, CONV>(a, ctx);
+    if (direct) return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, 1, false, CONV, BK>(a, ctx);
     if constexpr (BM * BN >= 128 * 128) {
-        if (inRegisters && wide) return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, 2, false, CONV>(a, ctx);
+        if (inRegisters && wide) return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, 2, false, CONV, BK>(a, ctx);
     }
-    return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, 0, false, CONV>(a, ctx);
+    return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, 0, false, CONV, BK>(a, ctx);
 }
 
 hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, const LaunchCtx &ctx) {
@@ -1559,7 +1578,7 @@ hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, const LaunchCtx &ct
     } else if (a.loader == kLoaderWindow) {
         // the ring kernel's window addressing: whole k-tiles per tap, 32-bit byte offsets into the image, a page of
         // zero-point bytes behind ktab, every tap offset non-negative once the tap lies inside the image
-        if (!a.ktab || ((uintptr_t)a.ktab & 15) != 0 || a.C <= 0 || a.C % 64 != 0 || a.KH <= 0 || a.KW <= 0) return hipErrorInvalidValue;
+        if (!a.ktab || ((uintptr_t)a.ktab & 15) != 0 || a.C <= 0 || a.C % t.bk != 0 || a.KH <= 0 || a.KW <= 0) return hipErrorInvalidValue;
         if (a.H <= 0 || a.W <= 0 || a.OH <= 0 || a.OW <= 0 || a.SH <= 0 || a.SW <= 0 || a.PT < 0 || a.PL < 0) return hipErrorInvalidValue;
         if (a.M % (a.OH * a.OW) != 0 || (long long)a.K != (long long)a.KH * a.KW * a.C || a.Kp != a.K) return hipErrorInvalidValue;
         if (a.a_bytes != (long long)(a.M / (a.OH * a.OW)) * a.H * a.W * a.C || a.a_bytes >= (1LL << 32)) return hipErrorInvalidValue;
@@ -1570,6 +1589,7 @@ hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, const LaunchCtx &ct
         case kIgemmDense128x128: return launchIgemmDense<128, 128, 2, 2, 4, 2, true>(a, ctx);
         case kIgemmDense256x128: return launchIgemmDense<256, 128, 2, 2, 3, 2, true>(a, ctx);
         case kIgemmDense256x64: return launchIgemmDense<256, 64, 4, 1, 3, 2, true>(a, ctx);
+        case kIgemmDense256x256K128: return launchIgemmDense<256, 256, 2, 2, 2, 1, true, 128>(a, ctx);  // C % 128 == 0 (checked above): 128 channels of one tap per k-tile
         default: return hipErrorInvalidValue;
         }
     } else {
@@ -1596,6 +1616,7 @@ hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, const LaunchCtx &ct
     case kIgemmStream: return launchIgemmStream(a, ctx);
     case kIgemmDense128x64: return launchIgemmDense<128, 64, 2, 2, 4, 2>(a, ctx);
     case kIgemmDense64x128: return launchIgemmDense<64, 128, 2, 2, 4, 2>(a, ctx);
+    case kIgemmDense256x256K128: return launchIgemmDense<256, 256, 2, 2, 2, 1, false, 128>(a, ctx);
     default: return hipErrorInvalidValue;
     }
 }

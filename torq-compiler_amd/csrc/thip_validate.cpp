@@ -28,6 +28,7 @@ static const IgemmTile kTiles[kIgemmVariantCount] = {
     {32, 32, 32, "igemm_stream_i8"},
     {128, 64, 64, "igemm_dense_i8_128x64x64"},
     {64, 128, 64, "igemm_dense_i8_64x128x64"},
+    {256, 256, 128, "igemm_dense_i8_256x256x128"},
 };
 
 const IgemmTile &igemmTile(uint32_t variant) {
@@ -182,18 +183,19 @@ thip_status_t checkOpFootprint(const DescriptorView *e, uint32_t i) {
         if ((s = need(op.scale, (uint64_t)op.Np * 4, "scale"))) return s;
         if (op.loader > kLoaderWindow) return fail(THIP_INVALID_ARGUMENT, "op %u: unknown igemm loader %u", i, op.loader);
         if (op.loader == kLoaderWindow) {
-            if (!positive({op.KH, op.KW, op.SH, op.SW}) || op.PT < 0 || op.PL < 0 || op.C % 64 != 0 || mul(op.KH, op.KW, op.C) != (uint64_t)op.K || op.Kp != op.K) {
+            const int32_t bk = igemmTile(op.variant).bk;
+            if (!positive({op.KH, op.KW, op.SH, op.SW}) || op.PT < 0 || op.PL < 0 || op.C % bk != 0 || mul(op.KH, op.KW, op.C) != (uint64_t)op.K || op.Kp != op.K) {
                 return fail(THIP_INVALID_ARGUMENT, "op %u: the window loader needs whole 64-channel k-tiles per tap", i);
             }
             if (inBytes >= (1ull << 32)) return fail(THIP_INVALID_ARGUMENT, "op %u: image too large for the window loader", i);
             switch (op.variant) {
-            case kIgemmDense256x256: case kIgemmDense128x256: case kIgemmDense128x128: case kIgemmDense256x128: case kIgemmDense256x64: break;
+            case kIgemmDense256x256: case kIgemmDense128x256: case kIgemmDense128x128: case kIgemmDense256x128: case kIgemmDense256x64: case kIgemmDense256x256K128: break;
             default: return fail(THIP_INVALID_ARGUMENT, "op %u: the window loader has no kernel for tile variant %u", i, op.variant);
             }
             if (op.table.space != kSpaceConst) return fail(THIP_INVALID_ARGUMENT, "op %u: table must be a constant", i);
-            if ((s = need(op.table, 64, "zero-point page"))) return s;
+            if ((s = need(op.table, 128, "zero-point page"))) return s;
             const uint8_t *page = e->blob + e->header.data_offset + e->consts[op.table.index].offset + op.table.offset;
-            for (int b = 0; b < 64; b++) {
+            for (int b = 0; b < 128; b++) {
                 if ((int8_t)page[b] != (int8_t)op.input_zp) return fail(THIP_INVALID_ARGUMENT, "op %u: the zero-point page does not hold input_zp", i);
             }
         }
