@@ -128,17 +128,17 @@ class Loaded:
 # (KiB per dispatch; the factors are what the same counters read for a plain 256 MiB copy, --copy-calibration).
 # They belong to the kernels as they were when the counters were read: TRAFFIC_KERNELS_SHA256 is the hash of
 # torq-compiler_amd/csrc/thip_kernels.hip at that time, and a run on other kernel sources reports traffic null.
-TRAFFIC_KERNELS_SHA256 = "61bc9c8507c66e983329eebd70b7a98a43bbff9833d79ce92b0d614a9e1f0f30"
+TRAFFIC_KERNELS_SHA256 = "0acbf3416db5afe163a399bdcfd009399c32ede9781ee36ec2ecf8fbfcee2c18"
 MEASURED_TRAFFIC = {
-    "fc_4096x4096x4096": (49377.5 * 1.9995 + 16597.5 * 1.0000) * 1024,
-    "fc_512x4096x4096": (16477.0 * 1.9995 + 2048.0 * 1.0000) * 1024,
+    "fc_4096x4096x4096": (49380.0 * 1.9995 + 16590.7 * 1.0000) * 1024,
+    "fc_512x4096x4096": (16473.0 * 1.9995 + 2048.0 * 1.0000) * 1024,
     "fc_16x2048x8192": (8408.0 * 1.9995 + 256.0 * 1.0000) * 1024,
-    "conv_112x112x32_o64_3x3": (358.9 * 1.9995 + 784.0 * 1.0000) * 1024,
-    "conv3x3_56x56x256_o256_b32": (17231.9 * 1.9995 + 25977.5 * 1.0000) * 1024,
-    "depthwise_b64": (15498.8 * 1.9995 + 7063.5 * 1.0000) * 1024,
-    "depthwise_s1_b256": (63711.9 * 1.9995 + 113170.4 * 1.0000) * 1024,
-    "maxpool_b64": (25112.3 * 1.9995 + 12544.0 * 1.0000) * 1024,
-    "avgpool_b64": (1998.5 * 1.9995 + 80.0 * 1.0000) * 1024,
+    "conv_112x112x32_o64_3x3": (352.4 * 1.9995 + 784.0 * 1.0000) * 1024,
+    "conv3x3_56x56x256_o256_b32": (17237.2 * 1.9995 + 25987.5 * 1.0000) * 1024,
+    "depthwise_b64": (15512.5 * 1.9995 + 7063.4 * 1.0000) * 1024,
+    "depthwise_s1_b256": (63707.3 * 1.9995 + 113147.9 * 1.0000) * 1024,
+    "maxpool_b64": (25114.3 * 1.9995 + 12544.0 * 1.0000) * 1024,
+    "avgpool_b64": (2000.5 * 1.9995 + 80.0 * 1.0000) * 1024,
     "add_b64": (4723.0 * 1.9995 + 4704.0 * 1.0000) * 1024,
 }
 
@@ -325,9 +325,9 @@ def main():
         loaded.run(args.warmup)
     dev.synchronize()
     t0 = time.perf_counter()
-    sets = 1
+    main_sets = 1
     if args.cold:
-        ev_ms, sets = loaded.run_cold(args.steps)
+        ev_ms, main_sets = loaded.run_cold(args.steps)
     else:
         ev_ms = loaded.run(args.steps)      # HIP events on the executable's stream around the K dispatches
     dev.synchronize()
@@ -423,7 +423,7 @@ def main():
         "dtype": "bf16" if args.workload.startswith(("fcbf16", "expandmm")) else "int8",
         "data": "synthetic",
         "config": {"workload": args.workload, "kernels": kernels, "parity_checked": ok,
-                   "algorithmic_ops": wl.ops, "algorithmic_bytes": wl.bytes, "buffer_sets": sets},
+                   "algorithmic_ops": wl.ops, "algorithmic_bytes": wl.bytes, "buffer_sets": main_sets},
         "roofline": dict(roofline(wl, bound, ev_ms, args.workload), kernel=kernels[0], kernel_ms=round(ev_ms, 5)),
     }
     if not args.no_cpu and args.workload.startswith("fc_"):
