@@ -411,7 +411,7 @@ class Emitter {
             return ((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn);
         };
         if (dense) {
-            if (const char *env = getenv("THIP_IGEMM_DENSE_VARIANT")) {
+            if (const char *env = getenv("THIP_IGEMM_DENSE_VARIANT"); env && *env) {
                 const long v = strtol(env, nullptr, 10);
                 if (v >= 0 && v < (long)kIgemmVariantCount && (v != (long)kIgemmStream || igemmStreamFits(N, K, outDtype))) {
                     return (uint32_t)v;
@@ -438,7 +438,7 @@ class Emitter {
             }
             return kIgemmDense64x64;
         }
-        if (const char *env = getenv("THIP_IGEMM_VARIANT")) {
+        if (const char *env = getenv("THIP_IGEMM_VARIANT"); env && *env) {
             const long v = strtol(env, nullptr, 10);
             if (v >= 0 && v < (long)kIgemmDense256x256) return (uint32_t)v;
         }
@@ -452,7 +452,7 @@ class Emitter {
     // Tile of the ring kernel with window addressing: one tile column for few output channels (the image is read
     // once), else the largest tile that still gives every CU a tile, two blocks per CU where there are many.
     static uint32_t chooseWindowVariant(int64_t M, int64_t N, int64_t C) {
-        if (const char *env = getenv("THIP_WINDOW_VARIANT")) {
+        if (const char *env = getenv("THIP_WINDOW_VARIANT"); env && *env) {
             const long v = strtol(env, nullptr, 10);
             if (v == kIgemmDense256x256 || v == kIgemmDense128x256 || v == kIgemmDense128x128 || v == kIgemmDense256x128 || v == kIgemmDense256x64) return (uint32_t)v;
             if (v == kIgemmDense256x256K128 && C % 128 == 0) return (uint32_t)v;
