@@ -59,6 +59,19 @@ WINDOW_RING = [
 ]
 
 
+def test_conv2d_on_images_smaller_than_one_load():
+    """An image of fewer than 16 bytes cannot feed the window-row loader (16-byte loads kept inside the image): such
+    convolutions take the gather loader.  (Found by a long run of the random sweep: the launcher refused them.)"""
+    for kw in (dict(N=1, H=2, W=6, C=1, O=3, KH=2, KW=1, pad=(0, 0, 1, 0)), dict(N=1, H=11, W=1, C=1, O=15, KH=3, KW=1, pad=(0, 0, 1, 1)),
+               dict(N=2, H=1, W=1, C=4, O=3, KH=1, KW=1, pad=(0, 0, 0, 0)), dict(N=1, H=2, W=2, C=3, O=24, KH=2, KW=1, pad=(0, 0, 0, 1)),
+               dict(N=1, H=4, W=4, C=1, O=5, KH=3, KW=3)):
+        wl = w.conv2d_workload(realistic=True, **kw)
+        outs, d = interp(wl)
+        assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)
+        small = kw["N"] * kw["H"] * kw["W"] * kw["C"] < 16
+        assert int(d.ops[-1]["loader"]) == (1 if small else 2), (kw, int(d.ops[-1]["loader"]))
+
+
 def test_dense_k128_records(monkeypatch):
     """A long K with enough 256 x 256 tiles takes the variant with 128-byte k-tiles: K padded to 128, same results."""
     wl = w.fully_connected_workload(3584, 1040, 4096, realistic=True)

@@ -209,6 +209,13 @@ def test_conv2d_mbv2_layer_shapes(device):
     check(device, w.conv2d_workload(N=2, H=7, W=7, C=320, O=1280, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True))
 
 
+def test_conv2d_on_images_smaller_than_one_load(device):
+    for kw in (dict(N=1, H=2, W=6, C=1, O=3, KH=2, KW=1, pad=(0, 0, 1, 0)), dict(N=1, H=11, W=1, C=1, O=15, KH=3, KW=1, pad=(0, 0, 1, 1)),
+               dict(N=2, H=1, W=1, C=4, O=3, KH=1, KW=1, pad=(0, 0, 0, 0)), dict(N=1, H=2, W=2, C=3, O=24, KH=2, KW=1, pad=(0, 0, 0, 1)),
+               dict(N=1, H=4, W=4, C=1, O=5, KH=3, KW=3), dict(N=1, H=1, W=1, C=1, O=1, KH=1, KW=1, pad=(0, 0, 0, 0))):
+        check(device, w.conv2d_workload(realistic=True, **kw), kernel="igemm_i8")
+
+
 def test_conv2d_int32_output(device):
     wl = w.conv2d_workload(N=1, H=9, W=9, C=16, O=8, realistic=True)
     # same op, int32 init and full-range clamp: exposes the un-narrowed requant result

@@ -687,7 +687,8 @@ thip_status_t Emitter::emitConv2d(const thip_hl_conv2d_t &c) {
     const bool pointwise = KH == 1 && KW == 1 && c.stride[0] == 1 && c.stride[1] == 1 && c.pad[0] == 0 &&
                            c.pad[1] == 0 && c.pad[2] == 0 && c.pad[3] == 0;
     const int64_t C = d.C;
-    if (KW * Cin <= 16 && Cin % 16 != 0 && !getenv("THIP_NO_RUN_LOADER")) {
+    // (its 16-byte loads stay inside the image by stepping back from its end, so the image must hold 16 bytes)
+    if (KW * Cin <= 16 && Cin % 16 != 0 && d.N * d.H * d.W * Cin >= 16 && !getenv("THIP_NO_RUN_LOADER")) {
         // few input channels (the first layer of an image network): one 16-byte run per window row
         emitIgemm(op, M, Oout, KH * 16, kLoaderRuns, [&](int64_t n, int64_t k) -> int8_t {
             const int64_t kh = k / 16, b = k % 16;

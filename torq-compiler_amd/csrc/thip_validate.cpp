@@ -201,6 +201,7 @@ thip_status_t checkOpFootprint(const DescriptorView *e, uint32_t i) {
         }
         if (op.loader == kLoaderRuns) {
             if (!positive({op.KH, op.KW}) || (int64_t)op.KW * op.C > 16 || op.Kp % 16 != 0) return fail(THIP_INVALID_ARGUMENT, "op %u: a window row of %d x %d bytes does not fit a 16-byte run", i, op.KW, op.C);
+            if (inBytes < 16) return fail(THIP_INVALID_ARGUMENT, "op %u: the run loader reads 16 bytes at a time, the image has %llu", i, (unsigned long long)inBytes);
             if (op.table.space != kSpaceConst) return fail(THIP_INVALID_ARGUMENT, "op %u: table must be a constant", i);
             if ((s = need(op.table, (uint64_t)op.Kp / 16 * 4, "table"))) return s;
             const uint8_t *base = e->blob + e->header.data_offset + e->consts[op.table.index].offset + op.table.offset;
