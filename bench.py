@@ -3,7 +3,9 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu] [--no-others]
 
-A "step" is one dispatch of the workload's program (inputs resident in HBM).  The default workload
+A "step" is one dispatch of the workload's program (inputs resident in HBM).  Before the W warm-up steps of every
+workload the card is kept busy with it for --precondition-ms (200 by default, untimed, reported in the JSON): an idle
+card sits at its lowest clocks, and a few milliseconds of timed steps right after that measure the ramp.  The default workload
 is the int8 fully_connected (4096, 4096, 4096) with fused per-column requant, the largest
 single-GPU case of the benchmark's matmul configuration; its metric is int8 GOP/s (1 MAC = 2 ops)
 against the dense int8 MFMA peak.  The other benchmark shapes are measured briefly in the same run
@@ -98,7 +100,17 @@ class Loaded:
         """Returns mean ms per dispatch from HIP events on the executable's stream."""
         return self.exe.time_device(self.ptrs, self.lens, iterations)
 
-    def run_cold(self, iterations):
+    def precondition(self, milliseconds, dispatch=None):
+        """Keeps the card busy with this workload for `milliseconds` of wall time, untimed: an idle card sits at its
+        lowest clocks and takes some 100 ms of work to reach the ones it sustains, and a measurement of a few
+        milliseconds taken before that reads 10-20 % slow."""
+        dispatch = dispatch or self.run
+        n, t0 = 20, time.perf_counter()
+        while (time.perf_counter() - t0) * 1e3 < milliseconds:
+            ms = dispatch(n)
+            n = int(min(5000, max(20, 2.0 / max(ms, 1e-4))))  # about 2 ms of work between synchronisations
+
+    def run_cold(self, iterations, precondition_ms=0.0):
         """The same on rotating copies of every binding (see COLD_WORKING_SET); returns (ms per dispatch, sets)."""
         per_set = sum(self.lens)
         sets = int(min(MAX_BUFFER_SETS, max(2, -(-COLD_WORKING_SET // per_set))))
@@ -107,6 +119,7 @@ class Loaded:
         try:
             all_sets = [self.ptrs] + extra
             self.exe.time_device_rotating(all_sets, self.lens, sets)  # every set once: first touch
+            self.precondition(precondition_ms, lambda n: self.exe.time_device_rotating(all_sets, self.lens, n))
             ms = self.exe.time_device_rotating(all_sets, self.lens, max(iterations, 2 * sets))
         finally:
             for ptrs in extra:
@@ -244,45 +257,125 @@ def cpu_baseline(wl, target_seconds=10.0, single_thread_seconds=6.0):
                               "sample": (what + ", one thread") % (passes1, rows1, M, M, K, N, dt1)}}
 
 
+class PowerMeter:
+    """Samples the card's power sensor (hwmon `power1_average` / `power1_input`, microwatts) from a thread.  A machine that
+    does not show the sensor gives None everywhere.  With several cards present the busiest one is reported."""
+
+    def __init__(self, period=0.005):
+        import glob
+        self.paths = sorted(p for name in ("power1_average", "power1_input")
+                            for p in glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/" + name))
+        self.period = period
+        self.samples = []   # (time.time(), [watts per sensor])
+        self.thread = None
+
+    def cap_watts(self):
+        caps = []
+        for p in self.paths:
+            try:
+                caps.append(int(open(os.path.join(os.path.dirname(p), "power1_cap")).read()) / 1e6)
+            except (OSError, ValueError):
+                pass
+        return max(caps) if caps else None
+
+    def _loop(self):
+        while self.running:
+            row = []
+            for p in self.paths:
+                try:
+                    row.append(int(open(p).read()) / 1e6)
+                except (OSError, ValueError):
+                    row.append(0.0)
+            self.samples.append((time.time(), row))
+            time.sleep(self.period)
+
+    def __enter__(self):
+        import threading
+        self.samples, self.running = [], bool(self.paths)
+        if self.running:
+            self.thread = threading.Thread(target=self._loop, daemon=True)
+            self.thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self.running = False
+        if self.thread:
+            self.thread.join()
+
+    def mean_watts(self, t0, t1):
+        """Mean over the second half of [t0, t1] (the sensor itself averages over a while)."""
+        rows = [r for t, r in self.samples if t0 + 0.5 * (t1 - t0) <= t <= t1]
+        if not rows:
+            return None
+        return round(max(float(np.mean([r[i] for r in rows])) for i in range(len(self.paths))), 1)
+
+
 def mfma_calibration(pkg, dev, wl, args):
-    """What bounds the headline GEMM on this card, measured in this run (TOP/s, 1 multiply-add = 2 ops)."""
+    """What bounds the headline GEMM on this card, measured in this run (TOP/s, 1 multiply-add = 2 ops), and what
+    the card draws meanwhile: every leg is repeated for `leg_seconds` under the power sensor."""
     out = {"unit": "TOP/s", "published_peak": PEAK_INT8_TOPS}
+    meter = PowerMeter()
+    leg_seconds = max(0.0, args.leg_seconds)
+    power = {"unit": "W", "sensor": meter.paths[0] if meter.paths else None, "cap": meter.cap_watts(), "leg_seconds": leg_seconds}
+
+    def leg(label, fn):
+        """Median of fn() over the leg; the power goes into power[label]."""
+        results = []
+        with meter:
+            t0 = time.time()
+            results.append(fn())
+            while time.time() - t0 < leg_seconds:
+                results.append(fn())
+            t1 = time.time()
+        power[label] = meter.mean_watts(t0, t1)
+        return float(np.median(results))
+
+    leg("idle", lambda: time.sleep(0.05) or 0.0)
     # the matrix cores with nothing else going on: every CU busy (256 workgroups of 4 waves), and 32 workgroups only
     # (an eighth of the chip: far below the power limit, so this is the clock-limited rate of one CU)
-    out["mfma_only_constant_operands"] = round(dev.mfma_rate(False, 256, 12000), 1)
-    out["mfma_only_random_operands"] = round(dev.mfma_rate(True, 256, 12000), 1)
-    out["mfma_only_random_operands_32_of_256_cus_scaled"] = round(dev.mfma_rate(True, 32, 12000) * 8, 1)
+    out["mfma_only_constant_operands"] = round(leg("mfma_only_constant_operands", lambda: dev.mfma_rate(False, 256, 12000)), 1)
+    out["mfma_only_random_operands"] = round(leg("mfma_only_random_operands", lambda: dev.mfma_rate(True, 256, 12000)), 1)
+    out["mfma_only_random_operands_32_of_256_cus_scaled"] = round(
+        leg("mfma_only_random_operands_32_of_256_cus", lambda: dev.mfma_rate(True, 32, 12000)) * 8, 1)
     # the same GEMM kernel on all-zero operands (nothing toggles) against the benchmark's uniform random bytes
     M, K = wl.inputs[0].shape
     N = wl.attrs["weights"].shape[0]
     for label, zeros in (("gemm_random_data", False), ("gemm_zero_data", True)):
         o = Loaded(pkg, dev, pkg.workloads.fully_connected_workload(M, K, N, zeros=zeros))
         o.run(args.warmup)
-        ms = o.run(args.steps)
+        ms = leg(label, lambda: o.run(args.steps))
         out[label] = {"us": round(ms * 1e3, 2), "TOP/s": round(o.wl.ops / (ms * 1e-3) / 1e12, 1), "kernel": o.exe.op_kernels()[0]}
         o.close()
     out["gemm_over_mfma_only_random"] = round(out["gemm_random_data"]["TOP/s"] / out["mfma_only_random_operands"], 3)
     if args.library_gemm:
         # in a process of its own: PyTorch brings its own HIP runtime, which does not share a process with this library's
         import subprocess
-        script = ("import torch, json\n"
-                  "M, K, N, W, S = %d, %d, %d, %d, %d\n"
+        script = ("import torch, json, time\n"
+                  "M, K, N, W, S, T = %d, %d, %d, %d, %d, %f\n"
                   "a = torch.randint(-128, 128, (M, K), dtype=torch.int8, device='cuda:0')\n"
                   "bt = torch.randint(-128, 128, (N, K), dtype=torch.int8, device='cuda:0').t()\n"
                   "for _ in range(W): torch._int_mm(a, bt)\n"
                   "torch.cuda.synchronize()\n"
                   "e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)\n"
-                  "e0.record()\n"
-                  "for _ in range(S): torch._int_mm(a, bt)\n"
-                  "e1.record(); torch.cuda.synchronize()\n"
-                  "print(json.dumps({'ms': e0.elapsed_time(e1) / S}))\n") % (M, K, N, max(args.warmup, 5), args.steps)
+                  "t0, ms = time.time(), []\n"
+                  "while not ms or time.time() - t0 < T:\n"
+                  "    e0.record()\n"
+                  "    for _ in range(S): torch._int_mm(a, bt)\n"
+                  "    e1.record(); torch.cuda.synchronize()\n"
+                  "    ms.append(e0.elapsed_time(e1) / S)\n"
+                  "ms.sort()\n"
+                  "print(json.dumps({'ms': ms[len(ms) // 2], 't0': t0, 't1': time.time()}))\n") % (M, K, N, max(args.warmup, 5), args.steps, leg_seconds)
         try:
-            done = subprocess.run([sys.executable, "-c", script], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
-            ms = json.loads(done.stdout.strip().splitlines()[-1])["ms"]
+            with meter:
+                done = subprocess.run([sys.executable, "-c", script], stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+            res = json.loads(done.stdout.strip().splitlines()[-1])
+            ms = res["ms"]
+            power["library_int_mm_random_data"] = meter.mean_watts(res["t0"], res["t1"])
             out["library_int_mm_random_data"] = {"us": round(ms * 1e3, 2), "TOP/s": round(2.0 * M * K * N / (ms * 1e-3) / 1e12, 1),
                                                  "what": "torch._int_mm (hipBLASLt) in a child process: int32 result, no requant, [N,K] weights like ours"}
         except Exception as ex:  # the comparison is optional
             out["library_int_mm_random_data"] = "unavailable: %r" % (ex,)
+    out["power"] = power
     return out
 
 
@@ -292,11 +385,17 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="fc_4096x4096x4096")
+    ap.add_argument("--precondition-ms", type=float, default=200.0,
+                    help="untimed dispatches of the workload for this long before its warm-up steps, so that the card has left its idle "
+                         "clocks when the timed steps start (0 switches it off); reported as config.clock_preconditioning_ms")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-others", action="store_true", help="skip the brief per-op measurements")
     ap.add_argument("--mfma-calibration", action="store_true",
                     help="also measure what bounds the int8 GEMM on this card: the matrix cores alone on constant and on random operands, "
                          "the same GEMM on all-zero data, and (with --library-gemm) the vendor library's int8 GEMM")
+    ap.add_argument("--leg-seconds", type=float, default=1.5,
+                    help="with --mfma-calibration: every measurement is repeated for this long (the clocks settle, the power sensor "
+                         "averages); 0 = once each, for a short run under a profiler")
     ap.add_argument("--library-gemm", action="store_true", help="with --mfma-calibration: time torch._int_mm (hipBLASLt) on the same shape")
     ap.add_argument("--cold", action="store_true",
                     help="time --workload on rotating copies of its buffers (together larger than the last-level cache), as the "
@@ -321,13 +420,15 @@ def main():
     wl = make()
     loaded = Loaded(pkg, dev, wl)
     kernels = loaded.exe.op_kernels()
+    pre_ms = max(0.0, args.precondition_ms)
+    loaded.precondition(pre_ms)
     if args.warmup > 0:
         loaded.run(args.warmup)
     dev.synchronize()
     t0 = time.perf_counter()
     main_sets = 1
     if args.cold:
-        ev_ms, main_sets = loaded.run_cold(args.steps)
+        ev_ms, main_sets = loaded.run_cold(args.steps, pre_ms)
     else:
         ev_ms = loaded.run(args.steps)      # HIP events on the executable's stream around the K dispatches
     dev.synchronize()
@@ -362,6 +463,7 @@ def main():
             if name == args.workload:
                 continue
             o = Loaded(pkg, dev, mk())
+            o.precondition(pre_ms)
             o.run(5)
             warm = o.run(50)
             names = o.exe.op_kernels()
@@ -369,12 +471,12 @@ def main():
             if bnd == "hbm":
                 # what the roofline fraction is quoted on: operands cold in every dispatch; the repeated dispatch of one
                 # buffer set (served by the last-level cache where it fits) is reported next to it
-                ms, sets = o.run_cold(50)
+                ms, sets = o.run_cold(50, pre_ms)
                 row.update({"us": round(ms * 1e3, 2), "us_cache_warm": round(warm * 1e3, 2), "buffer_sets": sets})
                 if name in STREAM_SHAPES:
                     rd, wbytes = STREAM_SHAPES[name]
                     wbytes = wbytes // 16 * 16
-                    floor_us = dev.stream_floor(rd, wbytes, cold=True)
+                    floor_us = min(dev.stream_floor(rd, wbytes, cold=True) for _ in range(3))  # the first call meets a card that has idled
                     row["streaming_floor_us"] = round(floor_us, 2)
                     row["frac_of_streaming_floor"] = round(floor_us / (ms * 1e3), 3)
             else:
@@ -397,6 +499,7 @@ def main():
             from helpers import oracle_network
         for batch in (1, 32, 256):
             o = Loaded(pkg, dev, pkg.workloads.mobilenet_v2_workload(batch=batch))
+            o.precondition(pre_ms)
             o.run(2)
             ms = o.run(10 if batch > 1 else 30)
             same = None
@@ -423,7 +526,8 @@ def main():
         "dtype": "bf16" if args.workload.startswith(("fcbf16", "expandmm")) else "int8",
         "data": "synthetic",
         "config": {"workload": args.workload, "kernels": kernels, "parity_checked": ok,
-                   "algorithmic_ops": wl.ops, "algorithmic_bytes": wl.bytes, "buffer_sets": main_sets},
+                   "algorithmic_ops": wl.ops, "algorithmic_bytes": wl.bytes, "buffer_sets": main_sets,
+                   "clock_preconditioning_ms": pre_ms},
         "roofline": dict(roofline(wl, bound, ev_ms, args.workload), kernel=kernels[0], kernel_ms=round(ev_ms, 5)),
     }
     if not args.no_cpu and args.workload.startswith("fc_"):

@@ -340,8 +340,9 @@ static thip_status_t waitBounded(thip_executable_t *e, const char *what) {
             e->abandoned = true;
             return fail(THIP_INTERNAL, "%s: the GPU did not finish within %lld ms; the executable is abandoned", what, (long long)e->waitTimeoutMs);
         }
-        // poll hard at first (dispatches are microseconds long), then back off
-        if (now - start > std::chrono::microseconds(500)) std::this_thread::sleep_for(std::chrono::microseconds(50));
+        // poll hard at first (dispatches are microseconds to a few milliseconds long, and a sleep of any length costs
+        // some 100 us before the thread runs again), then back off
+        if (now - start > std::chrono::microseconds(3000)) std::this_thread::sleep_for(std::chrono::microseconds(50));
     }
 }
 
