@@ -143,14 +143,14 @@ class Loaded:
 # torq-compiler_amd/csrc/thip_kernels.hip at that time, and a run on other kernel sources reports traffic null.
 TRAFFIC_KERNELS_SHA256 = "0acbf3416db5afe163a399bdcfd009399c32ede9781ee36ec2ecf8fbfcee2c18"
 MEASURED_TRAFFIC = {
-    "fc_4096x4096x4096": (49380.0 * 1.9995 + 16590.7 * 1.0000) * 1024,
+    "fc_4096x4096x4096": (49380.0 * 1.9995 + 16579.3 * 1.0000) * 1024,
     "fc_512x4096x4096": (16473.0 * 1.9995 + 2048.0 * 1.0000) * 1024,
     "fc_16x2048x8192": (8408.0 * 1.9995 + 256.0 * 1.0000) * 1024,
     "conv_112x112x32_o64_3x3": (352.4 * 1.9995 + 784.0 * 1.0000) * 1024,
-    "conv3x3_56x56x256_o256_b32": (17237.2 * 1.9995 + 25987.5 * 1.0000) * 1024,
-    "depthwise_b64": (15512.5 * 1.9995 + 7063.4 * 1.0000) * 1024,
-    "depthwise_s1_b256": (63707.3 * 1.9995 + 113147.9 * 1.0000) * 1024,
-    "maxpool_b64": (25114.3 * 1.9995 + 12544.0 * 1.0000) * 1024,
+    "conv3x3_56x56x256_o256_b32": (17237.1 * 1.9995 + 25305.1 * 1.0000) * 1024,
+    "depthwise_b64": (15505.0 * 1.9995 + 7063.5 * 1.0000) * 1024,
+    "depthwise_s1_b256": (63709.0 * 1.9995 + 113137.1 * 1.0000) * 1024,
+    "maxpool_b64": (25114.1 * 1.9995 + 12544.0 * 1.0000) * 1024,
     "avgpool_b64": (2000.5 * 1.9995 + 80.0 * 1.0000) * 1024,
     "add_b64": (4723.0 * 1.9995 + 4704.0 * 1.0000) * 1024,
 }
