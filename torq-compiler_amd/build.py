@@ -19,14 +19,17 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
           "--offload-arch=gfx950",
           # packed FP32 instruction selection stays off for every device pass
-          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+          # no v_dot4c_i32_i8: its accumulator is tied to the destination, so every dot-product chain that starts from
+          # a value it must keep (the bias) costs a v_mov per output; v_dot4_i32_i8 takes the addend as a third operand
+          "-Xclang", "-target-feature", "-Xclang", "-dot6-insts"]
 
 
 def _compile(src, extra):
     obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
     cmd = [HIPCC] + COMMON + extra + ["-c", os.path.join(CSRC, src), "-o", obj]
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l)
+    out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l and "dot6-insts" not in l)
     if proc.returncode != 0:
         raise RuntimeError("hipcc failed for %s:\n%s" % (src, out))
     return obj, out
