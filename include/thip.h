@@ -552,7 +552,7 @@ thip_status_t thip_executable_set_wait_timeout(thip_executable_t *executable, in
 /* thip_executable_enqueue for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid it).  It has no counterpart in the reference.  The dispatch is enqueued
  * kernel by kernel (no graph is built), on device bindings only, and makes no hipMalloc / hipFree or allocating
- * library call: the scratch memory of the program's kernels (the partial sums and tile counters of a bf16
+ * library call: the scratch memory of the program's kernels (the partial sums of a bf16
  * fully_connected / matmul whose K is split over blocks) is taken from an array that is part of the library's
  * device image instead of the executable's intermediates.  The results are those of thip_executable_enqueue.
  * A program whose kernels need more scratch than the array holds (2 MiB) is refused with

@@ -335,12 +335,14 @@ def test_gpu_bf16_add(device):
 
 @pytest.mark.gpu
 def test_gpu_bf16_split_k_is_deterministic(device):
-    """Few output tiles and a long K: K is split over blocks whose partial sums the last block to arrive adds in a
-    fixed order; repeated dispatches give the same bits, and the counters are back at zero for the next one."""
+    """A long K over fewer output tiles than CUs: K is split over blocks whose partial sums a second kernel adds in
+    slice order; repeated dispatches give the same bits."""
     wl = w.fully_connected_bf16_workload(32, 6912, 256)
-    d = desc_interp.Descriptor(wl.program.serialize())
-    assert int(d.ops[0]["w0"]) > 1
-    assert int(desc_interp.Descriptor(w.fully_connected_bf16_workload(32, 6912, 1152).program.serialize()).ops[0]["w0"]) == 1  # enough tiles: no split
+    split = lambda M, K, N: int(desc_interp.Descriptor(w.fully_connected_bf16_workload(M, K, N).program.serialize()).ops[0]["w0"])
+    assert split(32, 6912, 256) == 9      # about 12 k-steps of 64 per block
+    assert split(32, 6912, 1152) == 7     # 36 tiles: at most one block per CU
+    assert split(32, 1152, 6912) == 1     # a short K: the second launch costs more than it saves
+    assert split(200, 6912, 1152) == 1    # enough tiles already
     first = _check_gpu(device, wl, via="device")
     exe = Executable(device, wl.program.serialize())
     for _ in range(5):

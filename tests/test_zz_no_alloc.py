@@ -1,7 +1,7 @@
 """thip_executable_enqueue_noalloc: the dispatch that allocates nothing, against thip_executable_enqueue.
 
 The kernels with scratch memory are the bf16 fully_connected / matmul records whose K is split over blocks (partial
-sums and tile counters).  The no-allocation entry point takes that memory from the library's static device array,
+sums).  The no-allocation entry point takes that memory from the library's static device array,
 which every call on the GPU shares and which keeps the last call's contents: two calls in a row, the second on a
 smaller problem, must each give exactly what the ordinary entry point gives.
 """
@@ -49,10 +49,10 @@ def _both_ways(device, wl):
 
 def test_noalloc_matches_enqueue_twice_in_a_row(device):
     f = lambda bits: np.abs(orc.from_bf16(bits).astype(np.float64))
-    # a long K over a handful of output tiles: K split 16 ways; then a smaller problem, split as well
-    for M, K, N in [(1, 6912, 256), (3, 4096, 128)]:
+    # a long K over a handful of output tiles: K split 9 ways; then a smaller problem, split 5 ways
+    for (M, K, N), split in [((1, 6912, 256), 9), ((3, 4096, 128), 5)]:
         wl = w.fully_connected_bf16_workload(M, K, N)
-        assert _split_of(wl) == [16], "the workload must take the K-split kernel (scratch: partial sums and counters)"
+        assert _split_of(wl) == [split], "the workload must take the K-split kernels (scratch: partial sums)"
         (plain, first, again), kernels = _both_ways(device, wl)
         assert families(kernels) == ["fc_bf16"]
         assert_bit_exact(first, plain, wl.name + ": no-allocation entry point against thip_executable_enqueue")
@@ -70,20 +70,20 @@ def test_noalloc_without_scratch_and_on_a_whole_network(device):
 
 
 def test_noalloc_refuses_what_does_not_fit_and_host_bindings(device):
-    # three K-split linears of 16 tiles x 16 slices each: 3 MiB of partial sums, the array holds 2 MiB
+    # four K-split linears of 16 tiles x 9 slices each: 2.25 MiB of partial sums, the array holds 2 MiB
     rng = np.random.default_rng(3)
     p = Program()
     x = p.binding(0, (32, 6912), np.uint16)
-    weights = [w.to_bf16(rng.standard_normal((512, 6912)) / 83.0) for _ in range(3)]
+    weights = [w.to_bf16(rng.standard_normal((512, 6912)) / 83.0) for _ in range(4)]
     for i, wt in enumerate(weights):
         p.fully_connected(x, wt, np.zeros(512, dtype=np.float32), init=p.binding(1 + i, (32, 512), np.uint16), output_zp=0, shift_factor=0,
                           input_zp=0, output_min=w.NO_CLAMP[0], output_max=w.NO_CLAMP[1])
     blob = p.serialize()
-    assert [int(o["w0"]) for o in desc_interp.Descriptor(blob).ops] == [16, 16, 16]
+    assert [int(o["w0"]) for o in desc_interp.Descriptor(blob).ops] == [9, 9, 9, 9]
     exe = Executable(device, blob)
     xin = w.to_bf16(rng.standard_normal((32, 6912)))
-    ptrs = [device.upload(xin)] + [device.upload(np.zeros((32, 512), dtype=np.uint16)) for _ in range(3)]
-    lens = [xin.nbytes] + [32 * 512 * 2] * 3
+    ptrs = [device.upload(xin)] + [device.upload(np.zeros((32, 512), dtype=np.uint16)) for _ in range(4)]
+    lens = [xin.nbytes] + [32 * 512 * 2] * 4
     try:
         with pytest.raises(ThipError) as err:
             exe.enqueue_device_noalloc(ptrs, lens)

@@ -75,8 +75,8 @@ struct thip_executable_t {
     Tuning tuning;                       // the environment's switches as they were when the executable was created
     std::vector<std::string> kernelNames;  // per record: the kernel its launcher resolved at creation
     // thip_executable_enqueue_noalloc: where each record's scratch (a K-split workspace) sits in the static array,
-    // how much of it has to be zero before the launch, and the program's total
-    std::vector<uint64_t> scratchOffset, scratchZeroBytes;
+    // and the program's total
+    std::vector<uint64_t> scratchOffset;
     uint64_t scratchBytes = 0;
 };
 
@@ -713,12 +713,10 @@ thip_status_t thip_executable_create(thip_device_t *device, const void *blob, si
     // which must not happen later inside a stream capture).  Bindings stand in as aligned placeholder addresses:
     // device bindings must be 16-byte aligned and staged host bindings are, so a dispatch resolves the same way.
     e->scratchOffset.assign(h.op_count, 0);
-    e->scratchZeroBytes.assign(h.op_count, 0);
     for (uint32_t i = 0; i < h.op_count; i++) {
         const DescOp &op = e->ops[i];
         if (op.kind != kKindFcBf16 || op.w0 <= 1) continue;
         e->scratchOffset[i] = e->scratchBytes;
-        e->scratchZeroBytes[i] = fcBf16WorkspaceCounterBytes(op.M, op.Nn, op.w0);
         e->scratchBytes += (fcBf16WorkspaceBytes(op.M, op.Nn, op.w0) + 255) / 256 * 256;
     }
     e->tuning = tuningFromEnvironment();
@@ -838,11 +836,8 @@ thip_status_t thip_executable_enqueue_noalloc(thip_executable_t *e, const thip_d
     const LaunchCtx ctx{e->stream, &e->tuning, nullptr, 0};
     thip_status_t result = THIP_OK;
     for (uint32_t i = 0; i < e->header.op_count && result == THIP_OK; i++) {
-        // the array keeps what the last call left there, whoever made it: what has to start at zero is cleared
-        if (e->scratchZeroBytes[i]) {
-            const hipError_t ze = launchZeroFill(scratch + e->scratchOffset[i], (size_t)e->scratchZeroBytes[i], e->stream);
-            if (ze != hipSuccess) result = hipFail(ze, "clearing the scratch counters");
-        }
+        // the array keeps what the last call left there, whoever made it; nothing in a K-split workspace has to start
+        // at zero (every slot that is read has been written by the same dispatch)
         if (result == THIP_OK) result = launchOp(e, i, bp, ctx, scratch);
     }
     e->invocation++;

@@ -545,7 +545,12 @@ class Emitter {
     // Few output tiles and a long K: split K over several blocks per tile; their partial sums and the
     // tile counters live in an intermediate of the record's own (THIP_NO_SPLIT_K turns it off).
     void planFcBf16Split(DescOp *op) {
-        const int split = getenv("THIP_NO_SPLIT_K") ? 1 : fcBf16PreferredSplit(op->M, op->Nn, op->K);
+        int split = getenv("THIP_NO_SPLIT_K") ? 1 : fcBf16PreferredSplit(op->M, op->Nn, op->K);
+        // THIP_FC_SPLIT forces a split of 1 .. 16 where K has that many k-steps (for tuning runs)
+        if (const char *env = getenv("THIP_FC_SPLIT"); env && *env) {
+            const long v = strtol(env, nullptr, 10);
+            if (v >= 1 && v <= 16 && v <= (op->K + 63) / 64) split = (int)v;
+        }
         op->w0 = split;
         if (split > 1) op->in1 = newTemp(fcBf16WorkspaceBytes(op->M, op->Nn, split));
     }

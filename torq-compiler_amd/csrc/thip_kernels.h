@@ -142,9 +142,8 @@ struct FcBf16Args {
     uint16_t *out;      // [M][N]
     int32_t M, K, N;
     float lo, hi;       // clamp (-inf / +inf for none)
-    // K split over `ksplit` blocks per output tile (1 = no split).  workspace: one int32 counter per tile
-    // (zero before the first launch; the kernel leaves them zero), padded to 256 bytes, then
-    // tiles * ksplit * 1024 floats of partial sums.
+    // K split over `ksplit` blocks per output tile (1 = no split): the blocks leave their partial tiles in
+    // `workspace` (tiles * ksplit * 1024 floats; nothing in it has to be initialised) and a second kernel adds them.
     int32_t ksplit;
     void *workspace;
     // weights in fragment order: for column block nb (32 columns), k-step s (64 elements) and piece c (0..3),
@@ -174,29 +173,24 @@ inline size_t fcBf16FragmentOffset(int n, int k, int steps) {
 // Bytes of workspace a launch with this split needs.
 inline size_t fcBf16WorkspaceBytes(int M, int N, int ksplit) {
     const size_t tiles = (size_t)((N + 31) / 32) * ((M + 31) / 32);
-    return ksplit <= 1 ? 0 : (tiles * 4 + 255) / 256 * 256 + tiles * ksplit * 1024 * 4;
+    return ksplit <= 1 ? 0 : tiles * ksplit * 1024 * 4;
 }
 // The split the launcher's heuristics would like for this shape (the emitter allocates the workspace for it).
 inline int fcBf16PreferredSplit(int M, int N, int K) {
     const long long tiles = (long long)((N + 31) / 32) * ((M + 31) / 32);
     const int steps = (K + 63) / 64;
-    // the fenced write-back / counter / read-back chain costs 4-7 us: it only pays when a handful of tiles would
-    // otherwise walk a long K alone (6912 -> 256: 12 us split, 16-21 us not; 6912 -> 1152 and everything shorter: even or worse)
-    if (tiles > 16 || steps < 64) return 1;
-    long long split = 256 / tiles;  // at most one block per CU: a second round would double the time
-    if (split > steps / 4) split = steps / 4;
+    // The second kernel costs a dependent launch (2-3 us): the split pays where a block would otherwise walk a long
+    // K alone while most CUs idle (a CU streams 30-50 GB/s whatever its waves do).  About 12 k-steps per block, at
+    // most one block per CU (a second round would double the time); measured: 32 x 6912 -> 1152 21.0 us whole, 10.7
+    // split 7 ways; 6912 -> 256 20.7 / 9.8; 4096 -> 1024 11.7 / 8.7; 2048 -> 2048 10.4 / 8.8; K = 1152 and 1024: 7.0-7.4
+    // whole, 8.4-8.7 split.
+    if (steps < 32) return 1;
+    long long split = 256 / tiles;
+    if (split > (steps + 6) / 12) split = (steps + 6) / 12;
     if (split > 16) split = 16;
     return split < 2 ? 1 : (int)split;
 }
 hipError_t launchFcBf16(const FcBf16Args &a, const LaunchCtx &ctx);
-// Bytes of a K-split workspace that must be zero before a launch (the tile counters, padded to 256).
-inline size_t fcBf16WorkspaceCounterBytes(int M, int N, int ksplit) {
-    const size_t tiles = (size_t)((N + 31) / 32) * ((M + 31) / 32);
-    return ksplit <= 1 ? 0 : (tiles * 4 + 255) / 256 * 256;
-}
-
-// The library's static scratch array (device memory that needs no allocation): its size, its address on the
-// current device (ask once per device, with that device current), and a zero fill that is a kernel.
 // Sustained v_mfma_i32_32x32x32_i8 rate (TOP/s, 1 multiply-add = 2 ops) of `blocks` workgroups of four waves that
 // do nothing else, on constant or on random operand bytes.  Allocates and frees its own few KiB.
 hipError_t measureMfmaRate(int randomOperands, int blocks, int iterations, hipStream_t stream, double *outTops);
@@ -206,9 +200,10 @@ hipError_t measureMfmaRate(int randomOperands, int blocks, int iterations, hipSt
 // last-level cache.  Allocates and frees its buffers.
 hipError_t measureStreamRate(int readsPerWrite, size_t writeBytes, int cold, hipStream_t stream, double *outMicroseconds);
 
+// The library's static scratch array (device memory that needs no allocation): its size and its address on the
+// current device (ask once per device, with that device current).
 constexpr size_t kStaticScratchBytes = 2u << 20;
 hipError_t staticScratchAddress(void **out);
-hipError_t launchZeroFill(void *dst, size_t bytes, hipStream_t stream);
 
 // Integer elementwise ops with the ACT stage behind them.  fma: out = R1(in0 * w0); mul: out = R1(in0 * in1) (an
 // input of one element is broadcast); both with ONE (bias, scale) pair.  clamp / abs / negate / i2i: the input

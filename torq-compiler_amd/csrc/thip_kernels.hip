@@ -3121,31 +3121,32 @@ __global__ __launch_bounds__(NWAVES * 64) void fc_bf16(FcBf16Args p, FastDiv qbl
         for (int e = 0; e < 16; e++) acc[e] += partial[w][e][lane];
     }
     if (p.ksplit > 1) {
-        // K split over blocks: every block leaves its partial tile in the workspace; the block that arrives
-        // last at the tile's counter adds them up in slice order (so the result does not depend on who was
-        // last), finishes the tile and puts the counter back to zero.  Nobody waits for anybody.
-        const int tile = blockIdx.y * gridDim.x + blockIdx.x, tiles = gridDim.x * gridDim.y;
-        int *counters = (int *)p.workspace;
-        float *parts = (float *)((char *)p.workspace + ((size_t)tiles * 4 + 255) / 256 * 256);
-        float *mine = parts + ((size_t)tile * p.ksplit + blockIdx.z) * 1024;
+        // K split over blocks: every block leaves its partial tile in the workspace and fc_bf16_reduce, launched
+        // behind this kernel, adds the slices in slice order.  (One kernel with a fence, a counter per tile and the
+        // last block to arrive doing the sum measured 5-7 us slower: the fence writes the XCD's L2 back.)
+        const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+        float *mine = (float *)p.workspace + ((size_t)tile * p.ksplit + blockIdx.z) * 1024;
 #pragma unroll
         for (int e = 0; e < 16; e++) mine[e * 64 + lane] = acc[e];
-        __threadfence();
-        int arrived = 0;
-        if (lane == 0) arrived = atomicAdd(&counters[tile], 1);
-        arrived = __shfl(arrived, 0, 64);
-        if (arrived != p.ksplit - 1) return;
-        __threadfence();
-#pragma unroll
-        for (int e = 0; e < 16; e++) acc[e] = 0.0f;
-        for (int z = 0; z < p.ksplit; z++) {
-            const float *part = parts + ((size_t)tile * p.ksplit + z) * 1024;
-#pragma unroll
-            for (int e = 0; e < 16; e++) acc[e] += __builtin_nontemporal_load(part + e * 64 + lane);
-        }
-        if (lane == 0) counters[tile] = 0;
+        return;
     }
     fcBf16Store(p, acc, m0, n0, r, h);
+}
+
+// Second kernel of a K split: one wave per output tile adds the slices' partial tiles in slice order and finishes
+// the tile (bias, clamp, bf16).
+__global__ __launch_bounds__(64) void fc_bf16_reduce(FcBf16Args p) {
+    const int lane = threadIdx.x, r = lane & 31, h = lane >> 5;
+    const int tile = blockIdx.y * gridDim.x + blockIdx.x;
+    const float *parts = (const float *)p.workspace + (size_t)tile * p.ksplit * 1024;
+    v16f acc;
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[e] = 0.0f;
+    for (int z = 0; z < p.ksplit; z++) {
+#pragma unroll
+        for (int e = 0; e < 16; e++) acc[e] += parts[(size_t)z * 1024 + e * 64 + lane];
+    }
+    fcBf16Store(p, acc, blockIdx.y * 32, blockIdx.x * 32, r, h);
 }
 
 // fc_bf16_wide: the same product for a very wide N and a short K (a vocabulary projection): a wave owns a
@@ -3278,11 +3279,13 @@ hipError_t launchFcBf16(const FcBf16Args &a, const LaunchCtx &ctx) {
         if (clamp) THIP_ENQUEUE(ctx, "fc_bf16<4,2,4>", (fc_bf16<4, 2>), grid, dim3(256), 0, a, blk);
         else if (deep) THIP_ENQUEUE(ctx, "fc_bf16<4,1,6>", (fc_bf16<4, 1, 6>), grid, dim3(256), 0, a, blk);
         else THIP_ENQUEUE(ctx, "fc_bf16<4,1,4>", (fc_bf16<4, 1>), grid, dim3(256), 0, a, blk);
+        if (a.ksplit > 1 && !ctx.name) hipLaunchKernelGGL(fc_bf16_reduce, dim3(grid.x, grid.y), dim3(64), 0, ctx.stream, a);
         return hipGetLastError();
     }
     if (wide) return launchFcBf16Wide<0>(a, makeFastDiv(1), ctx);
     if (deep) THIP_ENQUEUE(ctx, "fc_bf16<4,0,6>", (fc_bf16<4, 0, 6>), grid, dim3(256), 0, a, makeFastDiv(1));
     else THIP_ENQUEUE(ctx, "fc_bf16<4,0,4>", (fc_bf16<4, 0>), grid, dim3(256), 0, a, makeFastDiv(1));
+    if (a.ksplit > 1 && !ctx.name) hipLaunchKernelGGL(fc_bf16_reduce, dim3(grid.x, grid.y), dim3(64), 0, ctx.stream, a);
     return hipGetLastError();
 }
 
@@ -3384,20 +3387,6 @@ hipError_t staticScratchAddress(void **out) {
     }
     *out = known[device];
     return hipSuccess;
-}
-
-// Zero fill by a kernel (a memset node recorded into a captured graph is not reliable on this platform).
-__global__ __launch_bounds__(256) void zero_fill(v4i *dst, size_t count) {
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < count) dst[i] = v4i{0, 0, 0, 0};
-}
-
-hipError_t launchZeroFill(void *dst, size_t bytes, hipStream_t stream) {
-    if (!dst || bytes == 0 || (bytes & 15) != 0 || ((uintptr_t)dst & 15) != 0) return hipErrorInvalidValue;
-    const size_t count = bytes / 16;
-    if ((count + 255) / 256 >= (1ull << 31)) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(zero_fill, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, (v4i *)dst, count);
-    return hipGetLastError();
 }
 
 // ---------------------------------------------------------------------------
