@@ -181,9 +181,9 @@ inline int fcBf16PreferredSplit(int M, int N, int K) {
     const int steps = (K + 63) / 64;
     // The second kernel costs a dependent launch (2-3 us): the split pays where a block would otherwise walk a long
     // K alone while most CUs idle (a CU streams 30-50 GB/s whatever its waves do).  About 12 k-steps per block, at
-    // most one block per CU (a second round would double the time); measured: 32 x 6912 -> 1152 21.0 us whole, 10.7
-    // split 7 ways; 6912 -> 256 20.7 / 9.8; 4096 -> 1024 11.7 / 8.7; 2048 -> 2048 10.4 / 8.8; K = 1152 and 1024: 7.0-7.4
-    // whole, 8.4-8.7 split.
+    // most one block per CU (a second round would double the time); measured: 32 x 6912 -> 1152 20.7 us whole, 8.1
+    // split 7 ways; 6912 -> 256 20.5 / 7.2; 4096 -> 1024 10.8 / 7.9; 2048 -> 2048 9.4 / 7.1; K = 1152 and 1024: 7.0-7.4
+    // whole, 6.7-7.1 split.
     if (steps < 32) return 1;
     long long split = 256 / tiles;
     if (split > (steps + 6) / 12) split = (steps + 6) / 12;

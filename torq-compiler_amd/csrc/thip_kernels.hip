@@ -3011,28 +3011,32 @@ __device__ __forceinline__ void expandQ8(int d, float sc, float bi, float lo, fl
 }
 
 // Bias, clamp, round to bf16 and store one 32 x 32 accumulator tile: register 4 q + e of lane (r, h) is
-// out[m0 + r][n0 + 8 q + 4 h + e].
-__device__ __forceinline__ void fcBf16Store(const FcBf16Args &p, const v16f &acc, int m0, int n0, int r, int h) {
+// out[m0 + r][n0 + 8 q + 4 h + e].  fcBf16StoreQuad stores the four registers of one q.
+__device__ __forceinline__ void fcBf16StoreQuad(const FcBf16Args &p, const float (&a)[4], int m0, int n0, int r, int h, int q) {
     const int m = m0 + r;
     if (m >= p.M) return;
+    const int n = n0 + 8 * q + 4 * h;
+    uint16_t o[4];
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-        const int n = n0 + 8 * q + 4 * h;
-        uint16_t o[4];
+    for (int e = 0; e < 4; e++) {
+        const int ne = n + e < p.N ? n + e : p.N - 1;
+        const float t0 = a[e] + p.bias[ne];
+        o[e] = bf16Bits(t0 < p.lo ? p.lo : (t0 > p.hi ? p.hi : t0));
+    }
+    if ((p.N & 3) == 0 && n + 3 < p.N) {
+        *(v2i *)(p.out + (size_t)m * p.N + n) = v2i{(int)((uint32_t)o[0] | ((uint32_t)o[1] << 16)), (int)((uint32_t)o[2] | ((uint32_t)o[3] << 16))};
+    } else {
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            const int ne = n + e < p.N ? n + e : p.N - 1;
-            const float t0 = acc[4 * q + e] + p.bias[ne];
-            o[e] = bf16Bits(t0 < p.lo ? p.lo : (t0 > p.hi ? p.hi : t0));
+            if (n + e < p.N) p.out[(size_t)m * p.N + n + e] = o[e];
         }
-        if ((p.N & 3) == 0 && n + 3 < p.N) {
-            *(v2i *)(p.out + (size_t)m * p.N + n) = v2i{(int)((uint32_t)o[0] | ((uint32_t)o[1] << 16)), (int)((uint32_t)o[2] | ((uint32_t)o[3] << 16))};
-        } else {
+    }
+}
+__device__ __forceinline__ void fcBf16Store(const FcBf16Args &p, const v16f &acc, int m0, int n0, int r, int h) {
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                if (n + e < p.N) p.out[(size_t)m * p.N + n + e] = o[e];
-            }
-        }
+    for (int q = 0; q < 4; q++) {
+        const float a[4] = {acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]};
+        fcBf16StoreQuad(p, a, m0, n0, r, h, q);
     }
 }
 
@@ -3133,20 +3137,27 @@ __global__ __launch_bounds__(NWAVES * 64) void fc_bf16(FcBf16Args p, FastDiv qbl
     fcBf16Store(p, acc, m0, n0, r, h);
 }
 
-// Second kernel of a K split: one wave per output tile adds the slices' partial tiles in slice order and finishes
-// the tile (bias, clamp, bf16).
-__global__ __launch_bounds__(64) void fc_bf16_reduce(FcBf16Args p) {
-    const int lane = threadIdx.x, r = lane & 31, h = lane >> 5;
+// Second kernel of a K split: a block per output tile adds the slices' partial tiles in slice order and finishes the
+// tile (bias, clamp, bf16).  Wave q owns registers 4 q .. 4 q + 3 of the tile's accumulator layout; the loads of
+// every slice (at most 16) are issued before the first addition, so the kernel is one memory round trip.
+__global__ __launch_bounds__(256) void fc_bf16_reduce(FcBf16Args p) {
+    const int lane = threadIdx.x & 63, q = threadIdx.x >> 6, r = lane & 31, h = lane >> 5;
     const int tile = blockIdx.y * gridDim.x + blockIdx.x;
-    const float *parts = (const float *)p.workspace + (size_t)tile * p.ksplit * 1024;
-    v16f acc;
+    const float *parts = (const float *)p.workspace + (size_t)tile * p.ksplit * 1024 + (size_t)(4 * q) * 64 + lane;
+    float v[16][4];
 #pragma unroll
-    for (int e = 0; e < 16; e++) acc[e] = 0.0f;
-    for (int z = 0; z < p.ksplit; z++) {
+    for (int z = 0; z < 16; z++) {
+        const int zc = z < p.ksplit ? z : p.ksplit - 1;  // loads only, no branch: slices past the split re-read the last one
 #pragma unroll
-        for (int e = 0; e < 16; e++) acc[e] += parts[(size_t)z * 1024 + e * 64 + lane];
+        for (int e = 0; e < 4; e++) v[z][e] = parts[(size_t)zc * 1024 + e * 64];
     }
-    fcBf16Store(p, acc, blockIdx.y * 32, blockIdx.x * 32, r, h);
+    float a[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int z = 0; z < 16; z++) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) a[e] += z < p.ksplit ? v[z][e] : 0.0f;
+    }
+    fcBf16StoreQuad(p, a, blockIdx.y * 32, blockIdx.x * 32, r, h, q);
 }
 
 // fc_bf16_wide: the same product for a very wide N and a short K (a vocabulary projection): a wave owns a
@@ -3261,7 +3272,7 @@ static hipError_t launchFcBf16Wide(const FcBf16Args &a, FastDiv blk, const Launc
 hipError_t launchFcBf16(const FcBf16Args &a, const LaunchCtx &ctx) {
     if (!a.x || !a.w || !a.bias || !a.out || a.M <= 0 || a.N <= 0 || a.K <= 0 || a.K % 8 != 0) return hipErrorInvalidValue;
     if (((((uintptr_t)a.x) | ((uintptr_t)a.w)) & 15) || (((uintptr_t)a.out) & (a.N % 4 == 0 ? 7 : 1)) || (((uintptr_t)a.bias) & 3)) return hipErrorInvalidValue;
-    if (a.ksplit < 1 || a.ksplit > 64 || (a.ksplit > 1 && (!a.workspace || ((uintptr_t)a.workspace & 255)))) return hipErrorInvalidValue;
+    if (a.ksplit < 1 || a.ksplit > 16 || (a.ksplit > 1 && (!a.workspace || ((uintptr_t)a.workspace & 255)))) return hipErrorInvalidValue;
     const dim3 grid((unsigned)((a.N + 31) / 32), (unsigned)((a.M + 31) / 32), (unsigned)a.ksplit);
     if (grid.y > 65535) return hipErrorInvalidValue;
     // few blocks (registers do not limit anything then) and 5 or 6 k-steps per wave: one deeper round of loads instead of two
@@ -3279,13 +3290,13 @@ hipError_t launchFcBf16(const FcBf16Args &a, const LaunchCtx &ctx) {
         if (clamp) THIP_ENQUEUE(ctx, "fc_bf16<4,2,4>", (fc_bf16<4, 2>), grid, dim3(256), 0, a, blk);
         else if (deep) THIP_ENQUEUE(ctx, "fc_bf16<4,1,6>", (fc_bf16<4, 1, 6>), grid, dim3(256), 0, a, blk);
         else THIP_ENQUEUE(ctx, "fc_bf16<4,1,4>", (fc_bf16<4, 1>), grid, dim3(256), 0, a, blk);
-        if (a.ksplit > 1 && !ctx.name) hipLaunchKernelGGL(fc_bf16_reduce, dim3(grid.x, grid.y), dim3(64), 0, ctx.stream, a);
+        if (a.ksplit > 1 && !ctx.name) hipLaunchKernelGGL(fc_bf16_reduce, dim3(grid.x, grid.y), dim3(256), 0, ctx.stream, a);
         return hipGetLastError();
     }
     if (wide) return launchFcBf16Wide<0>(a, makeFastDiv(1), ctx);
     if (deep) THIP_ENQUEUE(ctx, "fc_bf16<4,0,6>", (fc_bf16<4, 0, 6>), grid, dim3(256), 0, a, makeFastDiv(1));
     else THIP_ENQUEUE(ctx, "fc_bf16<4,0,4>", (fc_bf16<4, 0>), grid, dim3(256), 0, a, makeFastDiv(1));
-    if (a.ksplit > 1 && !ctx.name) hipLaunchKernelGGL(fc_bf16_reduce, dim3(grid.x, grid.y), dim3(64), 0, ctx.stream, a);
+    if (a.ksplit > 1 && !ctx.name) hipLaunchKernelGGL(fc_bf16_reduce, dim3(grid.x, grid.y), dim3(256), 0, ctx.stream, a);
     return hipGetLastError();
 }
 
