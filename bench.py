@@ -141,17 +141,17 @@ class Loaded:
 # (KiB per dispatch; the factors are what the same counters read for a plain 256 MiB copy, --copy-calibration).
 # They belong to the kernels as they were when the counters were read: TRAFFIC_KERNELS_SHA256 is the hash of
 # torq-compiler_amd/csrc/thip_kernels.hip at that time, and a run on other kernel sources reports traffic null.
-TRAFFIC_KERNELS_SHA256 = "0acbf3416db5afe163a399bdcfd009399c32ede9781ee36ec2ecf8fbfcee2c18"
+TRAFFIC_KERNELS_SHA256 = "7daad0415b7cd414e17f94e0560977efef096b004140aba8f97a666b8284ebe5"
 MEASURED_TRAFFIC = {
-    "fc_4096x4096x4096": (49380.0 * 1.9995 + 16579.3 * 1.0000) * 1024,
-    "fc_512x4096x4096": (16473.0 * 1.9995 + 2048.0 * 1.0000) * 1024,
+    "fc_4096x4096x4096": (49384.0 * 1.9995 + 16584.3 * 1.0000) * 1024,
+    "fc_512x4096x4096": (16472.0 * 1.9995 + 2048.0 * 1.0000) * 1024,
     "fc_16x2048x8192": (8408.0 * 1.9995 + 256.0 * 1.0000) * 1024,
-    "conv_112x112x32_o64_3x3": (352.4 * 1.9995 + 784.0 * 1.0000) * 1024,
-    "conv3x3_56x56x256_o256_b32": (17237.1 * 1.9995 + 25305.1 * 1.0000) * 1024,
-    "depthwise_b64": (15505.0 * 1.9995 + 7063.5 * 1.0000) * 1024,
-    "depthwise_s1_b256": (63709.0 * 1.9995 + 113137.1 * 1.0000) * 1024,
-    "maxpool_b64": (25114.1 * 1.9995 + 12544.0 * 1.0000) * 1024,
-    "avgpool_b64": (2000.5 * 1.9995 + 80.0 * 1.0000) * 1024,
+    "conv_112x112x32_o64_3x3": (356.4 * 1.9995 + 784.0 * 1.0000) * 1024,
+    "conv3x3_56x56x256_o256_b32": (17236.8 * 1.9995 + 25302.9 * 1.0000) * 1024,
+    "depthwise_b64": (15426.1 * 1.9995 + 7063.2 * 1.0000) * 1024,
+    "depthwise_s1_b256": (63724.4 * 1.9995 + 113184.0 * 1.0000) * 1024,
+    "maxpool_b64": (25119.8 * 1.9995 + 12544.0 * 1.0000) * 1024,
+    "avgpool_b64": (1998.5 * 1.9995 + 80.0 * 1.0000) * 1024,
     "add_b64": (4723.0 * 1.9995 + 4704.0 * 1.0000) * 1024,
 }
 
