@@ -407,3 +407,32 @@ def test_gpu_table(device, make):
     got, kernels = run_on_gpu(device, wl, via="device" if wl.inputs[0].size > 10000 else "host")
     assert_bit_exact(got[0], oracle_eval(wl)[0], wl.name)
     assert families(kernels) == ["table_lookup"]
+
+
+# ---- tensors of one to five elements --------------------------------------------------------------------------------
+
+TINY = [lambda sh=sh, f=f: f(sh) for sh in [(1,), (2,), (3,), (5,), (1, 1, 3)] for f in (
+    lambda sh: w.shift_workload(0, shape=sh, dtype=np.int16, round=True, seed=1),
+    lambda sh: w.binary_workload(4, shape=sh, dtype=np.int8, seed=2),
+    lambda sh: w.compare_workload(7, shape=sh, dtype=np.int32, seed=3),
+    lambda sh: w.table_workload(shape=sh, seed=4),
+    lambda sh: w.act_workload("abs", shape=sh, in_dtype=np.int8, min_int=-5, max_int=90, seed=5),
+    lambda sh: w.fma_workload(sh, in_dtype=np.int8, out_dtype=np.int16, input_zp=3, scale=0.7, output_zp=-4, seed=6))]
+
+
+@pytest.mark.parametrize("make", TINY)
+def test_tiny_tensors_descriptor(make):
+    """The generators plant their edge values into as many elements as the tensor has; the record covers the ragged tail."""
+    wl = make()
+    outs = [np.zeros(s, dtype=dt) for s, dt in wl.outputs]
+    desc_interp.run(wl.program.serialize(), list(wl.inputs) + outs)
+    assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)
+
+
+@pytest.mark.gpu
+def test_gpu_tiny_tensors(device):
+    for make in TINY:
+        wl = make()
+        print("[gpu-case]", wl.name, wl.inputs[0].shape, flush=True)
+        got, _ = run_on_gpu(device, wl, via="host")
+        assert_bit_exact(got[0], oracle_eval(wl)[0], wl.name)

@@ -509,8 +509,8 @@ def compare_workload(op_type=6, shape=(1, 56, 56, 24), dtype=np.int8, is_unsigne
     else:
         a = _random_ints(rng, shape, dtype, limit=5)  # a narrow range: equal pairs do occur
         b = _random_ints(rng, shape, dtype, limit=5)
-        a.reshape(-1)[:4] = [np.iinfo(dtype).min, np.iinfo(dtype).max, -1, 0]
-        b.reshape(-1)[:4] = [np.iinfo(dtype).max, np.iinfo(dtype).min, 0, -1]
+        _plant(a, [np.iinfo(dtype).min, np.iinfo(dtype).max, -1, 0])
+        _plant(b, [np.iinfo(dtype).max, np.iinfo(dtype).min, 0, -1])
     p = Program()
     i0 = p.binding(0, shape, dtype)
     i1 = p.binding(1, shape, dtype)
@@ -542,13 +542,20 @@ def shift_workload(op_type=2, shape=(1, 56, 56, 24), dtype=np.int32, round=True,
     a = _random_ints(rng, shape, dtype)
     bits = 8 * np.dtype(dtype).itemsize
     s = rng.integers(0, bits, size=shape).astype(dtype)
-    a.reshape(-1)[:6] = [np.iinfo(dtype).min, np.iinfo(dtype).max, -1, 1, -3, 3]
-    s.reshape(-1)[:6] = [bits - 1, bits - 1, 1, 1, 1, 1]
+    _plant(a, [np.iinfo(dtype).min, np.iinfo(dtype).max, -1, 1, -3, 3])
+    _plant(s, [bits - 1, bits - 1, 1, 1, 1, 1])
     p = Program()
     out = p.binding(2, shape, dtype)
     p.elementwiseshift(op_type, p.binding(0, shape, dtype), p.binding(1, shape, dtype), round=round, init=out)
     return Workload("shift_%d_%s_%d_r%d" % (op_type, np.dtype(dtype).name, a.size, int(round)), p, [a, s], [(shape, np.dtype(dtype).type)], a.size,
                     3 * a.nbytes, dict(op_type=op_type, round=round))
+
+
+def _plant(a, values):
+    """Writes the edge values into the first elements of `a` (as many as it has)."""
+    flat = a.reshape(-1)
+    n = min(flat.size, len(values))
+    flat[:n] = values[:n]
 
 
 def pack_table_words(lut):
@@ -565,7 +572,7 @@ def table_workload(shape=(1, 56, 56, 24), in_dtype=np.int8, out_dtype=np.int8, s
     """torq_hl.table: a random 256-entry lookup table of the output's type, as a constant operand or as the attribute."""
     rng = np.random.default_rng(seed)
     x = _random_ints(rng, shape, in_dtype)
-    x.reshape(-1)[:4] = [-128, 127, 0, -1]
+    _plant(x, [-128, 127, 0, -1])
     lut = _random_ints(rng, (256,), out_dtype)
     lut[[0, 255]] = _INT_RANGE[np.dtype(out_dtype)]
     words = pack_table_words(lut)
@@ -582,7 +589,7 @@ def act_workload(name="clamp", shape=(1, 56, 56, 24), in_dtype=np.int8, out_dtyp
     rng = np.random.default_rng(seed)
     out_dtype = in_dtype if out_dtype is None else out_dtype
     x = _random_ints(rng, shape, in_dtype)
-    x.reshape(-1)[:2] = _INT_RANGE[np.dtype(in_dtype)]  # the extremes: abs / negate of the most negative value saturate
+    _plant(x, list(_INT_RANGE[np.dtype(in_dtype)]))  # the extremes: abs / negate of the most negative value saturate
     p = Program()
     inp = p.binding(0, x.shape, in_dtype)
     out = p.binding(1, x.shape, out_dtype)
