@@ -31,6 +31,10 @@ def oracle_eval(wl):
         aw, asb, aa = a["add"]
         y = orc.conv2d(x, wp, sbp, layout=orc.NHWC, **pa)
         return [orc.add(wl.inputs[1], y, aw, asb, **aa) if a["other_first"] else orc.add(y, wl.inputs[1], aw, asb, **aa)]
+    if kind == "branches":
+        ya, yb, yc = [orc.fully_connected(x, wt, sb, **at) for wt, sb, at in a["fcs"]]
+        (w0, sb0, a0), (w1, sb1, a1) = a["adds"]
+        return [orc.add(orc.add(ya, yb, w0, sb0, **a0), yc, w1, sb1, **a1)]
     if kind == "fma":
         return [orc.fma(x, a.pop("weights"), a.pop("scale_bias"), **a)]
     if kind == "mul":

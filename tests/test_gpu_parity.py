@@ -506,6 +506,28 @@ def test_graph_replay_matches_oracle_every_time(device):
     exe.close()
 
 
+def test_program_with_independent_records(device):
+    """Three fully_connected records on one input joined by two adds (no path between the first three): the eager
+    dispatch, the capture and every replay must give the oracle's bytes, with fresh inputs in between."""
+    for M, K, N in [(64, 256, 128), (300, 1024, 512)]:
+        wl = w.branches_workload(M, K, N)
+        announce(wl.name, "independent records")
+        exe = Executable(device, wl.program.serialize())
+        x = wl.inputs[0]
+        rng = np.random.default_rng(11)
+        pin, pout = device.upload(x), device.upload(np.zeros((M, N), dtype=np.int8))
+        for it in range(5):
+            if it:
+                x[...] = rng.integers(-128, 128, size=x.shape).astype(np.int8)
+                runtime.check(runtime.lib().thip_device_h2d(device.handle, pin, x.ctypes.data, x.nbytes))
+                device.synchronize()
+            exe.run_device([pin, pout], [x.nbytes, M * N])
+            assert_bit_exact(device.download(pout, (M, N), np.int8), oracle_eval(wl)[0], "dispatch %d" % it)
+        exe.close()
+        for ptr in (pin, pout):
+            device.free(ptr)
+
+
 def test_full_size_gemm_properties(device):
     """(4096,4096,4096) is too slow for the oracle in a test: check rows the oracle can afford plus a
     structural property (each output row depends on its own input row only)."""

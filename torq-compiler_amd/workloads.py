@@ -410,6 +410,32 @@ def add_workload(N=1, H=56, W=56, C=24, zp0=-3, zp1=7, m0=0.71838506, m1=1.3 * 0
                     attrs)
 
 
+def branches_workload(M=64, K=256, N=128, seed=1030):
+    """Three fully_connected records that read the same input and do not depend on each other, joined by two adds:
+    out = add(add(fc_a(x), fc_b(x)), fc_c(x)).  A program with independent records (the shape of q / k / v projections
+    or of a block with a projection shortcut)."""
+    rng = np.random.default_rng(seed)
+    x = rng.integers(-128, 127, size=(M, K), endpoint=True, dtype=np.int8)
+    fcs = []
+    for _ in range(3):
+        wt = rng.integers(-128, 127, size=(N, K), endpoint=True, dtype=np.int8)
+        mult, shift = random_requant(rng, N, True)
+        sb, sf = derive_scale_bias(mult, shift, rng.integers(-(1 << 15), 1 << 15, size=N, endpoint=True, dtype=np.int64), wt, 0)
+        fcs.append((wt, sb, dict(output_zp=int(rng.integers(-10, 10)), output_min=-128, output_max=127, shift_factor=sf)))
+    adds = []
+    for zp0, zp1 in ((fcs[0][2]["output_zp"], fcs[1][2]["output_zp"]), (-2, fcs[2][2]["output_zp"])):
+        aw, asb, asf = add_params(0.71838506, 0.65, zp0, zp1)
+        adds.append((aw, asb, dict(output_zp=-2, output_min=-128, output_max=127, shift_factor=asf)))
+    p = Program()
+    inp = p.binding(0, x.shape)
+    out = p.binding(1, (M, N))
+    ya, yb, yc = [p.fully_connected(inp, wt, sb, **at) for wt, sb, at in fcs]
+    t = p.add(ya, yb, adds[0][0], adds[0][1], **adds[0][2])
+    p.add(t, yc, adds[1][0], adds[1][1], init=out, **adds[1][2])
+    return Workload("branches_%dx%dx%d" % (M, K, N), p, [x], [((M, N), np.int8)], 6 * M * K * N, x.nbytes + 3 * N * K + M * N,
+                    dict(fcs=fcs, adds=adds))
+
+
 def pointwise_add_workload(N=2, H=48, W=48, C=96, O=32, other_first=False, seed=1020):
     """The end of an inverted-residual block: 1x1 convolution -> add with a second input (the block's input)."""
     rng = np.random.default_rng(seed)
