@@ -510,4 +510,3 @@ def test_descriptor_in_the_terms_of_the_reference_schema():
     for bad in ["", "a/b", "x,y", "..", "n" * 64]:
         with pytest.raises(ThipError):
             Program().set_name(bad)
-

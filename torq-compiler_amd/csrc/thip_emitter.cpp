@@ -542,8 +542,8 @@ class Emitter {
     thip_status_t emitDepthwise(const thip_hl_depthwise_conv2d_t &c);
     thip_status_t emitFullyConnected(const thip_hl_fully_connected_t &c);
     thip_status_t emitMatmul(const thip_hl_matmul_t &c);
-    // Few output tiles and a long K: split K over several blocks per tile; their partial sums and the
-    // tile counters live in an intermediate of the record's own (THIP_NO_SPLIT_K turns it off).
+    // A long K over fewer output tiles than CUs: split K over several blocks per tile; their partial sums live in
+    // an intermediate of the record's own (THIP_NO_SPLIT_K turns it off).
     void planFcBf16Split(DescOp *op) {
         int split = getenv("THIP_NO_SPLIT_K") ? 1 : fcBf16PreferredSplit(op->M, op->Nn, op->K);
         // THIP_FC_SPLIT forces a split of 1 .. 16 where K has that many k-steps (for tuning runs)

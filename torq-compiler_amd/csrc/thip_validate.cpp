@@ -339,7 +339,7 @@ thip_status_t checkOpFootprint(const DescriptorView *e, uint32_t i) {
         }
         if ((s = need(op.bias, (uint64_t)op.Nn * 4, "bias"))) return s;
         if (op.w0 > 1) {
-            // K split over blocks: counters and partial sums live in an intermediate (zero-filled at creation)
+            // K split over blocks: the partial sums live in an intermediate of the record's own
             if (op.w0 > 16 || op.in1.space != kSpaceTemp) return fail(THIP_INVALID_ARGUMENT, "op %u: bad split-K workspace", i);
             if ((s = need(op.in1, fcBf16WorkspaceBytes(op.M, op.Nn, op.w0), "workspace"))) return s;
         }
