@@ -91,3 +91,41 @@ def test_wait_timeout_becomes_a_status(device):
     exe2.close()
     assert_bit_exact(res, oracle_eval(other)[0], other.name)
     assert got.shape == (4096, 4096)
+
+
+def test_dispatches_from_two_threads(device):
+    """The run-side contract of the reference (one dispatch at a time per executable behind a mutex, callers on any
+    thread: runtime/driver/TorqExecutable.cc:1045): two threads dispatch two executables at the same time, then both
+    dispatch the same one; every result is the oracle's."""
+    import threading
+    wls = [w.conv2d_workload(N=2, H=28, W=28, C=32, O=64, realistic=True), w.branches_workload(64, 256, 128)]
+    wants = [oracle_eval(wl)[0] for wl in wls]
+    exes = [Executable(device, wl.program.serialize()) for wl in wls]
+    print("[gpu-case] two threads,", wls[0].name, "and", wls[1].name, flush=True)
+    sys.stdout.flush()
+    errors = []
+
+    def worker(which, rounds):
+        try:
+            wl, want, exe = wls[which], wants[which], exes[which]
+            for _ in range(rounds):
+                out = np.zeros(wl.outputs[0][0], dtype=np.int8)
+                exe.run_host(list(wl.inputs) + [out])   # blocking; the library call runs without the interpreter lock
+                if not np.array_equal(out, want):
+                    errors.append("%s differs" % wl.name)
+                    return
+        except Exception as ex:  # reported by the main thread
+            errors.append(repr(ex))
+
+    try:
+        for pair in ((0, 1), (0, 0), (1, 1)):
+            threads = [threading.Thread(target=worker, args=(which, 40)) for which in pair]
+            for t in threads:
+                t.start()
+            for t in threads:
+                t.join(timeout=100)
+            assert not any(t.is_alive() for t in threads), "a dispatching thread did not finish"
+            assert not errors, errors
+    finally:
+        for exe in exes:
+            exe.close()
