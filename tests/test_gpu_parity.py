@@ -179,9 +179,14 @@ def test_stream_igemm(device, guarded, monkeypatch):
         check(device, w.fully_connected_workload(M, K, N, realistic=True), kernel="igemm_stream_i8")
     for shift in [0, 1, 31, 32, 33, 34, 62]:
         check(device, w.fully_connected_workload(500, 48, 80, shift=shift, output_zp=-7), kernel="igemm_stream_i8")
-    # chosen without forcing for a pointwise convolution over a large image; not when the weights outgrow LDS
+    # chosen without forcing for an expanding pointwise convolution from 40 000 pixels, for one with at most four k-steps
+    # from 200 000; not below that, not for a projecting one with a long K, and not when the weights outgrow LDS
     monkeypatch.delenv("THIP_IGEMM_DENSE_VARIANT")
-    check(device, w.conv2d_workload(N=4, H=56, W=56, C=32, O=144, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True), kernel="igemm_stream_i8")
+    check(device, w.conv2d_workload(N=13, H=56, W=56, C=32, O=144, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True), kernel="igemm_stream_i8")
+    check(device, w.conv2d_workload(N=4, H=56, W=56, C=32, O=144, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True), kernel="igemm_dense_i8")
+    check(device, w.conv2d_workload(N=13, H=56, W=56, C=96, O=32, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True), kernel="igemm_dense_i8")
+    check(device, w.conv2d_workload(N=70, H=56, W=56, C=96, O=32, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True), kernel="igemm_stream_i8")
+    check(device, w.conv2d_workload(N=70, H=56, W=56, C=144, O=32, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True), kernel="igemm_dense_i8")
     check(device, w.fully_connected_workload(8192, 256, 256, realistic=True), kernel="igemm_dense_i8")
     # few input channels: the streaming kernel gathers one run per window row (also across the image border)
     for kw in [dict(N=2, H=224, W=224, C=3, O=32, stride=(2, 2), pad=(0, 1, 0, 1), input_zp=-1),
@@ -616,16 +621,22 @@ def test_event_log_and_timing(device, tmp_path):
 def test_residual_add_in_the_streaming_epilogue(device, monkeypatch):
     """The add folded behind the requant of the pixel-streaming convolution: both operand orders, ragged rows,
     every accumulator width; and the whole network with and without the folding gives the same bits."""
+    # the streaming kernel takes such a convolution on its own from some hundred thousand pixels (the last case); the
+    # smaller ones are forced onto it so that every accumulator width of the instantiation with the add runs
+    monkeypatch.setenv("THIP_IGEMM_DENSE_VARIANT", "11")
     for kw in [dict(), dict(other_first=True), dict(N=1, H=65, W=66, C=32, O=16), dict(N=3, H=40, W=40, C=144, O=48, other_first=True),
-               dict(N=2, H=56, W=56, C=144, O=32), dict(N=4, H=36, W=36, C=64, O=208, other_first=True), dict(N=8, H=28, W=28, C=192, O=64)]:
+               dict(N=2, H=56, W=56, C=144, O=32), dict(N=4, H=36, W=36, C=64, O=208, other_first=True), dict(N=8, H=28, W=28, C=192, O=64),
+               dict(N=130, H=56, W=56, C=96, O=32)]:
+        if kw.get("N") == 130:
+            monkeypatch.delenv("THIP_IGEMM_DENSE_VARIANT")
         wl = w.pointwise_add_workload(**kw)
         print("[gpu-case]", wl.name, flush=True)
         got, kernels = run_on_gpu(device, wl, via="device")
         assert families(kernels) == ["igemm_stream_i8"] and kernels[0].split(",")[2] == "1", kernels  # the instantiation with the add
         assert_bit_exact(got[0], oracle_eval(wl)[0], wl.name)
-    # few pixels: the small dense tile adds the residual in its in-register epilogue
+    # fewer pixels: the small dense tile adds the residual in its in-register epilogue
     for kw in [dict(N=1, H=8, W=8), dict(N=1, H=14, W=14, C=384, O=64, other_first=True), dict(N=2, H=7, W=7, C=960, O=160), dict(N=1, H=28, W=28, C=192, O=32),
-               dict(N=1, H=9, W=7, C=48, O=80, other_first=True)]:
+               dict(N=1, H=9, W=7, C=48, O=80, other_first=True), dict(N=8, H=28, W=28, C=192, O=64), dict(N=32, H=14, W=14, C=576, O=96)]:
         wl = w.pointwise_add_workload(**kw)
         print("[gpu-case]", wl.name, flush=True)
         got, kernels = run_on_gpu(device, wl, via="device")

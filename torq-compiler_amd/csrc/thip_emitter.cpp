@@ -122,6 +122,8 @@ class Emitter {
     std::map<uint32_t, DescBinding> bindings_;
     // Physical channel count of an intermediate whose channels are padded to a multiple of 16
     // (0 = stored as declared).  See planChannelPadding.
+    std::vector<int> valueReads_;  // per value: how many op inputs name it (planExpandFolding fills it)
+    bool addFollows_ = false;      // the convolution being emitted is read by one op only, the torq_hl.add right behind it
     std::vector<int64_t> cpad_;
     std::vector<int64_t> cdeclared_;  // declared channel count of a padded intermediate
 
@@ -404,8 +406,9 @@ class Emitter {
         op->t0_clamp = (int32_t)bound;
     }
 
-    // Tile choice.  THIP_IGEMM_VARIANT / THIP_IGEMM_DENSE_VARIANT force one (for tuning runs).
-    static uint32_t chooseIgemmVariant(int64_t M, int64_t N, bool dense, int64_t K = 0, int32_t outDtype = 0, bool runs = false) {
+    // Tile choice.  THIP_IGEMM_VARIANT / THIP_IGEMM_DENSE_VARIANT force one (for tuning runs).  addFollows: the
+    // record's only reader is a torq_hl.add right behind it, which the streaming kernel and the 64 x 64 tile can fold.
+    static uint32_t chooseIgemmVariant(int64_t M, int64_t N, bool dense, int64_t K = 0, int32_t outDtype = 0, bool runs = false, bool addFollows = false) {
         auto tiles = [&](uint32_t v) {
             const IgemmTile &t = igemmTile(v);
             return ((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn);
@@ -417,24 +420,44 @@ class Emitter {
                     return (uint32_t)v;
                 }
             }
-            // a small weight matrix over many pixels: keep it in LDS and stream the pixels
-            if (M >= 4096 && igemmStreamFits(N, K, outDtype) && !getenv("THIP_NO_STREAM")) return kIgemmStream;
+            // A small weight matrix over many pixels: keep it in LDS and stream the pixels.  Measured against the dense
+            // tiles on pointwise shapes of 16 .. 960 channels over 12 544 .. 802 816 pixels: with at most four k-steps
+            // per pixel group (the depth of its prefetch ring) it is ahead from about 200 000 pixels, and from 40 000
+            // where N >= 2 K (the output dominates: the expanding convolutions); with a longer K only where N >= 2 K,
+            // up to 2^28 outputs (beyond that its passes over the activations, one per 256 channels, cost more), or
+            // where an add follows a very large image (the fused add saves more than the dense tile gains); below
+            // those sizes a dense tile is 10-50 % faster.
+            if (M >= 4096 && igemmStreamFits(N, K, outDtype) && !getenv("THIP_NO_STREAM")) {
+                const bool expanding = N >= 2 * K;
+                const bool take = K <= 128 ? (M >= 200000 || (expanding && M >= 40000))
+                                           : ((expanding && M >= 25000 && M * N < (1LL << 28)) || (addFollows && M >= 400000));
+                if (take) return kIgemmStream;
+            }
+            // an add behind it: the small tile folds the add into its epilogue, which beats a larger tile plus an add kernel
+            if (addFollows && outDtype == THIP_DTYPE_I8 && N % 16 == 0) return kIgemmDense64x64;
             // N narrower than a tile: one tile column of the narrowest tile that covers N, so the
             // activations are streamed once (these shapes are bandwidth-bound, padded MFMA work is free)
-            if (N <= 128 && M >= 4096) {
+            if (N <= 128 && M >= 16384) {
                 return N <= 32 ? kIgemmDense256x32 : N <= 64 ? kIgemmDense256x64 : kIgemmDense256x128;
             }
-            // otherwise the largest tile that still gives (nearly) every CU a tile
-            const uint32_t order[] = {kIgemmDense256x256, kIgemmDense128x256, kIgemmDense128x128, kIgemmDense64x128};
             // a long K on the largest tile: k-tiles of 128 bytes, whole cache lines per row (THIP_NO_K128 keeps 64)
             if (K >= 1024 && tiles(kIgemmDense256x256) >= 224 && !getenv("THIP_NO_K128")) return kIgemmDense256x256K128;
-            for (uint32_t v : order) {
+            // otherwise the largest tile that still gives (nearly) every CU a tile and does not pad N by more than an
+            // eighth where a narrower tile that fills the chip would not (padded columns are computed too)
+            const uint32_t order[] = {kIgemmDense256x256, kIgemmDense128x256, kIgemmDense128x128, kIgemmDense64x128, kIgemmDense128x64};
+            auto enough = [&](uint32_t v) { return tiles(v) >= (v == kIgemmDense128x128 || v == kIgemmDense128x64 ? 192 : 224); };
+            auto wasteful = [&](uint32_t v) { return (roundUp(N, igemmTile(v).bn) - N) * 8 > N; };
+            for (size_t i = 0; i < sizeof(order) / sizeof(order[0]); i++) {
+                const uint32_t v = order[i];
                 // a short K leaves a 256 x 256 tile (one block per CU) mostly prologue and epilogue; two blocks per CU
                 // of half the size overlap them (256 -> 1024 channels at 56 x 56, batch 32: 75 -> 54 us)
                 if (v == kIgemmDense256x256 && K > 0 && K <= 512) continue;
-                // the wide-N tile only where N nearly fills whole tiles (padded columns are computed too)
-                if (v == kIgemmDense64x128 && ((roundUp(N, 128) - N) * 8 > N || getenv("THIP_NO_64X128"))) continue;
-                if (tiles(v) >= 224) return v;
+                if (v == kIgemmDense64x128 && (wasteful(v) || getenv("THIP_NO_64X128"))) continue;
+                if (!enough(v)) continue;
+                bool better = false;
+                for (size_t j = i + 1; j < sizeof(order) / sizeof(order[0]) && wasteful(v); j++) better = better || (!wasteful(order[j]) && enough(order[j]));
+                if (better) continue;
+                return v;
             }
             return kIgemmDense64x64;
         }
@@ -475,7 +498,8 @@ class Emitter {
     template <typename WeightAt>
     void emitIgemm(DescOp base, int64_t M, int64_t N, int64_t K, uint32_t loader, WeightAt wAt) {
         const bool dense = loader == kLoaderDense;
-        const uint32_t variant = loader == kLoaderWindow ? chooseWindowVariant(M, N, base.C) : chooseIgemmVariant(M, N, dense, K, base.out_dtype, loader == kLoaderRuns);
+        const uint32_t variant = loader == kLoaderWindow ? chooseWindowVariant(M, N, base.C)
+                                                         : chooseIgemmVariant(M, N, dense, K, base.out_dtype, loader == kLoaderRuns, addFollows_);
         const IgemmTile &t = igemmTile(variant);
         const int64_t Kp = roundUp(K, t.bk), Np = roundUp(N, t.bn);
         std::vector<int8_t> packed((size_t)(Np * Kp), 0);
@@ -1873,7 +1897,6 @@ void Emitter::planChannelPadding() {
 
 void Emitter::planExpandFolding() {
     foldedExpand_.clear();
-    if (getenv("THIP_NO_EXPAND_FOLD")) return;
     const size_t n = prog_.values.size();
     std::vector<int> reads(n, 0), asMatmulRhs(n, 0);
     auto read = [&](thip_value_t v) {
@@ -1906,6 +1929,8 @@ void Emitter::planExpandFolding() {
         case kHlTable: read(op.u.tab.input); break;
         }
     }
+    valueReads_ = reads;
+    if (getenv("THIP_NO_EXPAND_FOLD")) return;
     auto constant = [&](thip_value_t v) { return v >= 0 && (size_t)v < n && prog_.values[(size_t)v].kind == kValueConstant; };
     for (const HlOp &op : prog_.ops) {
         if (op.kind != kHlExpandWeights) continue;
@@ -1957,8 +1982,15 @@ void Emitter::fuseResidualAdd() {
 thip_status_t Emitter::run(void **outBlob, size_t *outSize) {
     planChannelPadding();
     planExpandFolding();
-    for (const HlOp &op : prog_.ops) {
+    for (size_t at = 0; at < prog_.ops.size(); at++) {
+        const HlOp &op = prog_.ops[at];
         thip_status_t s = THIP_OK;
+        addFollows_ = false;
+        if (op.kind == kHlConv2d && at + 1 < prog_.ops.size() && prog_.ops[at + 1].kind == kHlAdd && !getenv("THIP_NO_ADD_FUSION")) {
+            const thip_value_t y = op.u.conv.init;
+            const thip_hl_add_t &next = prog_.ops[at + 1].u.add;
+            addFollows_ = y >= 0 && (size_t)y < valueReads_.size() && valueReads_[(size_t)y] == 1 && ((next.input1 == y) != (next.input2 == y));
+        }
         switch (op.kind) {
         case kHlConv2d: s = emitConv2d(op.u.conv); break;
         case kHlDepthwise: s = emitDepthwise(op.u.dw); break;
