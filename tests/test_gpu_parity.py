@@ -102,7 +102,12 @@ def test_conv2d_window_ring_k128(device, monkeypatch):
     k = check(device, w.conv2d_workload(N=2, H=32, W=32, C=128, O=64, realistic=False))  # the literal requant range
     assert k[0].startswith("igemm_dense_conv_i8<256,256,2,2,2,1,"), k
     k = check(device, w.conv2d_workload(N=2, H=32, W=32, C=64, O=64, realistic=True))    # C % 128 != 0: the switch does not apply
+    assert k[0].startswith("igemm_dense_conv_i8<128,128,"), k  # 8 row tiles: too few for the one-column tile
+    monkeypatch.delenv("THIP_WINDOW_VARIANT")
+    k = check(device, w.conv2d_workload(N=30, H=48, W=48, C=64, O=64, realistic=True), via="device")  # 270 row tiles: one tile column
     assert k[0].startswith("igemm_dense_conv_i8<256,64,"), k
+    k = check(device, w.conv2d_workload(N=1, H=14, W=14, C=256, O=256, realistic=True))  # few pixels, a long K: still the ring kernel
+    assert k[0].startswith("igemm_dense_conv_i8<128,128,"), k
 
 
 def test_conv2d_window_ring_switch(device, monkeypatch):

@@ -484,12 +484,18 @@ class Emitter {
             const IgemmTile &t = igemmTile(v);
             return ((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn);
         };
-        if (N <= 64) return kIgemmDense256x64;
-        if (N <= 128) return kIgemmDense256x128;
-        // measured on 3x3 convolutions of 64 .. 512 channels at batch 32: the largest tile wins as soon as half the CUs
-        // get one (a long K per tile amortises its prologue and epilogue)
-        if (tiles(kIgemmDense256x256) >= 128) return (C % 128 == 0 && !getenv("THIP_NO_K128")) ? kIgemmDense256x256K128 : kIgemmDense256x256;
-        if (tiles(kIgemmDense128x256) >= 128) return kIgemmDense128x256;
+        auto wasteful = [&](uint32_t v) { return (roundUp(N, igemmTile(v).bn) - N) * 8 > N; };
+        // few output channels over many pixels: one tile column, the image is read once (64 -> 64 at 112 x 112, batch 32:
+        // 27.8 us against 41.1 with 128 x 128 tiles); with fewer than a tile per CU the smaller tile wins (128 -> 128 at
+        // 28 x 28, batch 8: 8.5 us against 12.4)
+        if (N <= 64 && tiles(kIgemmDense256x64) >= 224) return kIgemmDense256x64;
+        if (N <= 128 && tiles(kIgemmDense256x128) >= 224) return kIgemmDense256x128;
+        // measured on 3x3 convolutions of 64 .. 512 channels at batch 1 .. 64: the largest tile wins as soon as half the CUs
+        // get one (a long K per tile amortises its prologue and epilogue), unless it pads N by more than an eighth
+        if (tiles(kIgemmDense256x256) >= 128 && !wasteful(kIgemmDense256x256)) {
+            return (C % 128 == 0 && !getenv("THIP_NO_K128")) ? kIgemmDense256x256K128 : kIgemmDense256x256;
+        }
+        if (tiles(kIgemmDense128x256) >= 128 && !wasteful(kIgemmDense128x256)) return kIgemmDense128x256;
         return kIgemmDense128x128;
     }
 
@@ -725,9 +731,10 @@ thip_status_t Emitter::emitConv2d(const thip_hl_conv2d_t &c) {
             return wd[((n * C + b % C) * KH + kh) * KW + b / C];
         });
     } else {
-        // a window over whole 64-channel k-tiles with enough rows for the large tiles: the LDS-DMA ring kernel addresses
+        // a window over whole 64-channel k-tiles with enough rows for the large tiles, or with a long K at any size
+        // (256 -> 256 at 14 x 14, one image: 12.6 us against 15.4 on the gather kernel): the LDS-DMA ring kernel addresses
         // the window itself (THIP_NO_WINDOW_RING keeps such convolutions on the gather kernel, for tests and tuning)
-        const bool ring = !pointwise && Cin % 64 == 0 && M >= 2048 && Oout >= 32 && d.N * d.H * d.W * Cin < (1LL << 32) && !getenv("THIP_NO_WINDOW_RING");
+        const bool ring = !pointwise && Cin % 64 == 0 && (M >= 2048 || K >= 1024) && Oout >= 32 && d.N * d.H * d.W * Cin < (1LL << 32) && !getenv("THIP_NO_WINDOW_RING");
         emitIgemm(op, M, Oout, K, (pointwise && K % 16 == 0) ? kLoaderDense : ring ? kLoaderWindow : kLoaderGather, [&](int64_t n, int64_t k) -> int8_t {
             const int64_t pos = k / Cin, ci = k % Cin;
             const int64_t kh = pos / KW, kw = pos % KW;
