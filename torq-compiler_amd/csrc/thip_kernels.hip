@@ -2363,7 +2363,7 @@ hipError_t launchDepthwise(const DepthwiseArgs &a, const LaunchCtx &ctx) {
         const long long outputs = (long long)a.N * a.OH * a.OW * (a.C / 16);
         // a register tile of outputs per thread where that still leaves every CU several blocks
         // (THIP_DEPTHWISE_TILE=0 / 1 switches that kernel off / on for every size, for tests and tuning)
-        // the rolling-window kernel where it has at least a wave (stride 1) or 1.9 waves (stride 2) per SIMD
+        // the rolling-window kernel where it has at least 0.6 waves (stride 1) or 1.9 waves (stride 2) per SIMD
         // (THIP_DEPTHWISE_STRIP=0 / 1 / 2 switches it off / on / on with one column per thread at stride 2, for every
         // size, for tests and tuning)
         const int stripMode = ctx.tuning->depthwiseStrip;
@@ -2372,7 +2372,7 @@ hipError_t launchDepthwise(const DepthwiseArgs &a, const LaunchCtx &ctx) {
         if (!stripOff && a.SH == a.SW && (a.SW == 1 || a.SW == 2) && (long long)a.W * a.C < (1LL << 24)) {
             long long waves = 0;
             const int seg = depthwiseStripSegment(a, 2, 1, &waves);
-            if (a.SW == 1 && (stripOn || (a.OH >= 12 && waves >= 1024))) return launchDepthwiseStrip<2, 1, 1, 4, 3>(a, seg, ctx);
+            if (a.SW == 1 && (stripOn || (a.OH >= 6 && waves >= 640))) return launchDepthwiseStrip<2, 1, 1, 4, 3>(a, seg, ctx);
             if (a.SW == 2 && (stripOne || (!stripOn && a.OH >= 12))) {
                 // with plenty of work (the six waves per SIMD that the segment length aims for), one column per thread, more
                 // waves and the deeper prefetch measured 7-11 % ahead
@@ -2381,6 +2381,13 @@ hipError_t launchDepthwise(const DepthwiseArgs &a, const LaunchCtx &ctx) {
                 if (stripOne || waves1 >= 6 * 1024) return launchDepthwiseStrip<1, 2, 1, 4, 3>(a, seg1, ctx);
             }
             if (a.SW == 2 && (stripOn || (a.OH >= 12 && 10 * waves >= 19 * 1024))) return launchDepthwiseStrip<2, 2, 1, 3, 1>(a, seg, ctx);
+            // too few waves for two columns per thread, enough for one (112 x 112 x 96 at batch 8: 6.8 us against 7.7 for
+            // the window-row kernel; 56 x 56 x 144 at batch 32: 7.2 against 8.2)
+            if (a.SW == 2 && !stripOn && a.OH >= 12) {
+                long long waves1 = 0;
+                const int seg1 = depthwiseStripSegment(a, 1, 1, &waves1);
+                if (waves1 >= 1280) return launchDepthwiseStrip<1, 2, 1, 4, 3>(a, seg1, ctx);
+            }
         }
         const bool tileOff = ctx.tuning->depthwiseTile == 0, tileOn = ctx.tuning->depthwiseTile == 1;
         if (!tileOff) {
