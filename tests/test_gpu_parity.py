@@ -268,11 +268,11 @@ def test_fully_connected_geometries(device, mkn):
 
 @pytest.mark.parametrize("dot4", [False, True])
 def test_fully_connected_skinny_kernels(device, dot4, monkeypatch):
-    """At most 16 rows: the MFMA kernel (3 rows and up) and the dot-product kernel, K and N with ragged ends."""
+    """At most 16 rows: the MFMA kernel (2 rows and up) and the dot-product kernel, K and N with ragged ends."""
     if dot4:
         monkeypatch.setenv("THIP_SKINNY_DOT4", "1")
     def expected(M):
-        if M >= 3 and not dot4:
+        if M >= 2 and not dot4:
             return "fc_skinny_mfma"
         return "fc_skinny<1,4>" if M == 1 else "fc_skinny<4,4>" if M <= 4 else "fc_skinny<8,2>" if M <= 8 else "fc_skinny<16,2>"
     for mkn in [(3, 16, 16), (5, 48, 20), (16, 272, 1000), (9, 1040, 37), (4, 256, 64), (2, 512, 32), (16, 2048, 8192), (7, 4096, 130), (1, 64, 48)]:
