@@ -125,24 +125,29 @@ def run(blob, binding_arrays):
                     # bytes beyond the run are whatever memory holds: they must meet zero weights
                     A[..., e * 16 + length:(e + 1) * 16] = 77
                 A = A.reshape(M, Kp)
-            elif int(op["loader"]) == 3:  # the ring kernel's own window addressing: k-tile t is 64 channels of tap t * 64 // C
+            elif int(op["loader"]) == 3:  # the ring kernel's own window addressing: 16-byte chunk e holds channels (16 e) % C .. of tap 16 e // C
                 Nimg, H, W, C = (int(op[k]) for k in ["N", "H", "W", "C"])
                 OH, OW, SH, SW, PT, PL, KH, KW = (int(op[k]) for k in ["OH", "OW", "SH", "SW", "PT", "PL", "KH", "KW"])
-                assert C % 64 == 0 and K == Kp == KH * KW * C and int(op["variant"]) in (4, 5, 6, 8, 9, 14)
-                assert int(op["variant"]) != 14 or C % 128 == 0
+                bk = 128 if int(op["variant"]) == 14 else 64
+                assert int(op["variant"]) in (4, 5, 6, 8, 9, 14)
+                assert C % 16 == 0 and C >= bk and K == KH * KW * C and Kp == -(-K // bk) * bk
                 page = view(op["table"], 128).view(np.int8)
                 assert (page == int(op["input_zp"])).all()
                 x = view(op["in0"], Nimg * H * W * C).view(np.int8).reshape(Nimg, H, W, C)
                 A = np.zeros((Nimg, OH, OW, Kp), dtype=np.int64)
                 oy = np.arange(OH)[:, None] * SH - PT
                 ox = np.arange(OW)[None, :] * SW - PL
-                for t in range(Kp // 64):
-                    tap, ci = (t * 64) // C, (t * 64) % C
+                for e in range(Kp // 16):
+                    tap, ci = (e * 16) // C, (e * 16) % C
+                    if tap >= KH * KW:
+                        # chunks of the last k-tile beyond K are whatever the walk reads: they must meet zero weights
+                        A[..., e * 16:(e + 1) * 16] = 77
+                        continue
                     kh, kw = tap // KW, tap % KW
                     iy, ix = oy + kh, ox + kw
                     inside = (iy >= 0) & (iy < H) & (ix >= 0) & (ix < W)
-                    vals = x[:, np.clip(iy, 0, H - 1), np.clip(ix, 0, W - 1), ci:ci + 64].astype(np.int64)
-                    A[..., t * 64:(t + 1) * 64] = np.where(inside[None, :, :, None], vals, int(page[0]))
+                    vals = x[:, np.clip(iy, 0, H - 1), np.clip(ix, 0, W - 1), ci:ci + 16].astype(np.int64)
+                    A[..., e * 16:(e + 1) * 16] = np.where(inside[None, :, :, None], vals, int(page[0]))
                 A = A.reshape(M, Kp)
             else:
                 Nimg, H, W, C = (int(op[k]) for k in ["N", "H", "W", "C"])

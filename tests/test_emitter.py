@@ -47,7 +47,8 @@ def test_conv2d_descriptor(kw, nhwc):
         assert kinds[0] == desc_interp.K_TRANSPOSE and kinds[1] == desc_interp.K_IGEMM
 
 
-# Convolutions over whole 64-channel k-tiles with at least 2048 output pixels: the LDS-DMA ring kernel addresses the window.
+# Convolutions over a multiple of 16 channels (64 at least) with at least 2048 output pixels or a long K: the LDS-DMA ring
+# kernel addresses the window.
 WINDOW_RING = [
     dict(N=2, H=32, W=32, C=64, O=64),                                            # M = 2048: the smallest taken; one tile column
     dict(N=10, H=29, W=31, C=64, O=96, stride=(2, 2), pad=(0, 1, 0, 1)),          # odd frame, stride 2, one-sided padding, ragged M
@@ -56,6 +57,11 @@ WINDOW_RING = [
     dict(N=2, H=34, W=66, C=64, O=256, KH=1, KW=3, pad=(1, 1, 0, 0)),             # a flat window
     dict(N=8, H=24, W=24, C=192, O=128, KH=3, KW=3, stride=(1, 2), pad=(2, 0, 1, 2)),  # three k-tiles per tap, mixed strides, lopsided pads
     dict(N=8, H=33, W=33, C=64, O=64, KH=1, KW=1, stride=(2, 2), pad=(0, 0, 0, 0)),    # a strided pointwise convolution
+    dict(N=3, H=31, W=30, C=80, O=96, pad=(1, 1, 1, 1)),                          # k-tiles straddle taps; K = 720 ends inside the last k-tile
+    dict(N=4, H=36, W=34, C=96, O=40, KH=3, KW=3, stride=(2, 1), pad=(0, 2, 1, 0), input_zp=-77),  # K = 864, Kp = 896
+    dict(N=2, H=33, W=37, C=144, O=144, KH=2, KW=3, pad=(1, 1, 0, 1), input_zp=55),                # K = 864: taps of 2.25 k-tiles
+    dict(N=1, H=60, W=44, C=208, O=64, KH=1, KW=3, pad=(1, 1, 0, 0)),                              # K = 624, Kp = 640
+    dict(N=1, H=16, W=16, C=112, O=112, KH=5, KW=5, pad=(2, 2, 2, 2)),                             # few pixels, K = 2800 -> 2816
 ]
 
 
@@ -90,16 +96,18 @@ def test_dense_k128_records(monkeypatch):
 
 
 def test_conv2d_window_loader_records():
-    """Whole 64-channel k-tiles and enough rows: the record asks for the ring kernel's window addressing (loader 3, a
-    64-byte zero-point page as its table); fewer rows, other channel counts or the switch keep the gather loader."""
+    """A multiple of 16 channels (64 or more) and enough rows: the record asks for the ring kernel's window addressing
+    (loader 3, a page of zero-point bytes as its table, K rounded up to whole k-tiles); fewer rows, other channel counts
+    or the switch keep the gather loader."""
     import os
     for kw in WINDOW_RING:
         wl = w.conv2d_workload(realistic=True, **kw)
         outs, d = interp(wl)
         assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)
         assert [(int(o["kind"]), int(o["loader"])) for o in d.ops] == [(desc_interp.K_IGEMM, 3)], wl.name
-        assert int(d.ops[0]["Kp"]) == int(d.ops[0]["K"])
-    for kw in (dict(N=1, H=32, W=32, C=64, O=64), dict(N=2, H=32, W=32, C=96, O=64), dict(N=2, H=32, W=32, C=64, O=16)):
+        bk = 128 if int(d.ops[0]["variant"]) == 14 else 64
+        assert int(d.ops[0]["Kp"]) == -(-int(d.ops[0]["K"]) // bk) * bk
+    for kw in (dict(N=1, H=32, W=32, C=64, O=64), dict(N=2, H=32, W=32, C=72, O=64), dict(N=2, H=32, W=32, C=48, O=64), dict(N=2, H=32, W=32, C=64, O=16)):
         d = interp(w.conv2d_workload(realistic=True, **kw))[1]
         assert int(d.ops[0]["loader"]) == 1, kw
     os.environ["THIP_NO_WINDOW_RING"] = "1"

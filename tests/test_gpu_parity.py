@@ -70,7 +70,7 @@ def test_conv2d_every_tile_variant(device, variant, monkeypatch):
 
 @pytest.mark.parametrize("kw", WINDOW_RING, ids=lambda kw: "x".join(str(kw[k]) for k in ("N", "H", "W", "C", "O")))
 def test_conv2d_window_ring(device, kw):
-    """Convolutions over whole 64-channel k-tiles: the LDS-DMA ring kernel addresses the window itself."""
+    """Convolutions over a multiple of 16 channels, 64 or more: the LDS-DMA ring kernel addresses the window itself."""
     k = check(device, w.conv2d_workload(realistic=True, **kw), via="device")
     assert families(k) == ["igemm_dense_conv_i8"], k
     k = check(device, w.conv2d_workload(realistic=False, nhwc=False, **kw))  # the literal requant range, N,C,H,W bindings
@@ -82,7 +82,8 @@ def test_conv2d_window_ring_every_tile(device, variant, monkeypatch):
     monkeypatch.setenv("THIP_WINDOW_VARIANT", str(variant))
     names = {4: "igemm_dense_conv_i8<256,256,", 5: "igemm_dense_conv_i8<128,128,", 6: "igemm_dense_conv_i8<128,256,", 8: "igemm_dense_conv_i8<256,128,",
              9: "igemm_dense_conv_i8<256,64,"}
-    for kw in (dict(N=2, H=33, W=35, C=64, O=80, pad=(1, 1, 1, 1)), dict(N=5, H=47, W=45, C=128, O=48, stride=(2, 2), pad=(1, 0, 1, 0), output_zp=-7, output_min=-128)):
+    for kw in (dict(N=2, H=33, W=35, C=64, O=80, pad=(1, 1, 1, 1)), dict(N=5, H=47, W=45, C=128, O=48, stride=(2, 2), pad=(1, 0, 1, 0), output_zp=-7, output_min=-128),
+               dict(N=3, H=29, W=31, C=80, O=72, pad=(1, 1, 1, 1), input_zp=-90), dict(N=4, H=40, W=33, C=176, O=130, KH=2, KW=2, stride=(1, 2), pad=(0, 1, 1, 0))):
         k = check(device, w.conv2d_workload(realistic=True, **kw), via="device")
         assert k[0].startswith(names[variant]), k
     # an int32 result and a requant shift on the 64-bit tail: the staged epilogue
@@ -91,12 +92,14 @@ def test_conv2d_window_ring_every_tile(device, variant, monkeypatch):
 
 
 def test_conv2d_window_ring_k128(device, monkeypatch):
-    """C % 128 == 0 and at least 128 tiles of 256 x 256: k-tiles of 128 channels of one tap."""
+    """C % 128 == 0 and at least 128 tiles of 256 x 256: k-tiles of 128 channels of one tap (asked for by hand, of any
+    128 channels or more)."""
     k = check(device, w.conv2d_workload(N=8, H=64, W=64, C=128, O=256, realistic=True), via="device")
     assert k[0] == "igemm_dense_conv_i8<256,256,2,2,2,1,1,0>", k
     monkeypatch.setenv("THIP_WINDOW_VARIANT", "14")
     for kw in (dict(N=2, H=33, W=35, C=128, O=80, pad=(1, 1, 1, 1)), dict(N=5, H=47, W=45, C=256, O=48, stride=(2, 2), pad=(1, 0, 1, 0), output_zp=-7, output_min=-128),
-               dict(N=3, H=30, W=30, C=384, O=40, KH=2, KW=5, pad=(3, 1, 0, 1))):
+               dict(N=3, H=30, W=30, C=384, O=40, KH=2, KW=5, pad=(3, 1, 0, 1)), dict(N=2, H=34, W=31, C=144, O=96, pad=(1, 1, 1, 1), input_zp=101),
+               dict(N=4, H=31, W=35, C=208, O=300, KH=1, KW=3, stride=(2, 1), pad=(1, 0, 0, 0))):
         k = check(device, w.conv2d_workload(realistic=True, **kw), via="device")
         assert k[0].startswith("igemm_dense_conv_i8<256,256,2,2,2,1,"), k
     k = check(device, w.conv2d_workload(N=2, H=32, W=32, C=128, O=64, realistic=False))  # the literal requant range

@@ -478,13 +478,18 @@ class Emitter {
         if (const char *env = getenv("THIP_WINDOW_VARIANT"); env && *env) {
             const long v = strtol(env, nullptr, 10);
             if (v == kIgemmDense256x256 || v == kIgemmDense128x256 || v == kIgemmDense128x128 || v == kIgemmDense256x128 || v == kIgemmDense256x64) return (uint32_t)v;
-            if (v == kIgemmDense256x256K128 && C % 128 == 0) return (uint32_t)v;
+            if (v == kIgemmDense256x256K128 && C >= 128) return (uint32_t)v;
         }
         auto tiles = [&](uint32_t v) {
             const IgemmTile &t = igemmTile(v);
             return ((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn);
         };
-        auto wasteful = [&](uint32_t v) { return (roundUp(N, igemmTile(v).bn) - N) * 8 > N; };
+        // padding N by more than an eighth counts against a wide tile only where the 128-wide fallback pads less
+        // (144 channels are 256 either way: 144 -> 144 at 56 x 56, batch 32, 45.1 us on 256 x 256 against 48.3 on 128 x 128)
+        auto wasteful = [&](uint32_t v) {
+            const int64_t np = roundUp(N, igemmTile(v).bn);
+            return np > roundUp(N, 128) && (np - N) * 8 > N;
+        };
         // few output channels over many pixels: one tile column, the image is read once (64 -> 64 at 112 x 112, batch 32:
         // 27.8 us against 41.1 with 128 x 128 tiles); with fewer than a tile per CU the smaller tile wins (128 -> 128 at
         // 28 x 28, batch 8: 8.5 us against 12.4)
@@ -734,7 +739,7 @@ thip_status_t Emitter::emitConv2d(const thip_hl_conv2d_t &c) {
         // a window over whole 64-channel k-tiles with enough rows for the large tiles, or with a long K at any size
         // (256 -> 256 at 14 x 14, one image: 12.6 us against 15.4 on the gather kernel): the LDS-DMA ring kernel addresses
         // the window itself (THIP_NO_WINDOW_RING keeps such convolutions on the gather kernel, for tests and tuning)
-        const bool ring = !pointwise && Cin % 64 == 0 && (M >= 2048 || K >= 1024) && Oout >= 32 && d.N * d.H * d.W * Cin < (1LL << 32) && !getenv("THIP_NO_WINDOW_RING");
+        const bool ring = !pointwise && Cin % 16 == 0 && Cin >= 64 && (M >= 2048 || K >= 1024) && Oout >= 32 && d.N * d.H * d.W * Cin < (1LL << 32) && !getenv("THIP_NO_WINDOW_RING");
         emitIgemm(op, M, Oout, K, (pointwise && K % 16 == 0) ? kLoaderDense : ring ? kLoaderWindow : kLoaderGather, [&](int64_t n, int64_t k) -> int8_t {
             const int64_t pos = k / Cin, ci = k % Cin;
             const int64_t kh = pos / KW, kw = pos % KW;
