@@ -64,6 +64,19 @@ WINDOW_RING = [
     dict(N=1, H=16, W=16, C=112, O=112, KH=5, KW=5, pad=(2, 2, 2, 2)),                             # few pixels, K = 2800 -> 2816
 ]
 
+# Fewer channels than a k-tile: the chunks of one k-tile span several taps, up to four window rows (1 x 1 x 16).
+WINDOW_RING_FEW_CHANNELS = [
+    dict(N=3, H=31, W=30, C=32, O=96, pad=(1, 1, 1, 1)),
+    dict(N=4, H=36, W=34, C=16, O=40, KH=3, KW=3, stride=(2, 1), pad=(0, 2, 1, 0), input_zp=-77),
+    dict(N=2, H=33, W=37, C=48, O=144, KH=2, KW=3, pad=(1, 1, 0, 1), input_zp=55),
+    dict(N=1, H=60, W=44, C=16, O=64, KH=1, KW=3, pad=(1, 1, 0, 0)),
+    dict(N=1, H=50, W=50, C=32, O=72, KH=5, KW=5, pad=(2, 2, 2, 2)),
+    dict(N=2, H=40, W=40, C=16, O=33, KH=7, KW=7, pad=(3, 3, 3, 3)),
+    dict(N=2, H=40, W=40, C=16, O=64, KH=1, KW=2, pad=(0, 1, 0, 0)),
+    dict(N=24, H=20, W=20, C=48, O=64, KH=4, KW=1, stride=(2, 2), pad=(0, 0, 1, 2)),
+    dict(N=2, H=40, W=40, C=16, O=64, KH=3, KW=1, pad=(0, 0, 1, 1)),
+]
+
 
 def test_conv2d_on_images_smaller_than_one_load():
     """An image of fewer than 16 bytes cannot feed the window-row loader (16-byte loads kept inside the image): such
@@ -115,6 +128,19 @@ def test_conv2d_window_loader_records():
         assert int(interp(w.conv2d_workload(realistic=True, **WINDOW_RING[0]))[1].ops[0]["loader"]) == 1
     finally:
         del os.environ["THIP_NO_WINDOW_RING"]
+
+
+@pytest.mark.parametrize("variant", [None, 14])
+def test_conv2d_window_loader_few_channels(variant, monkeypatch):
+    """16, 32 and 48 channels on the window loader (THIP_RING_MIN_C lowers the channel count from which it is taken)."""
+    monkeypatch.setenv("THIP_RING_MIN_C", "16")
+    if variant is not None:
+        monkeypatch.setenv("THIP_WINDOW_VARIANT", str(variant))
+    for kw in WINDOW_RING_FEW_CHANNELS:
+        wl = w.conv2d_workload(realistic=True, **kw)
+        outs, d = interp(wl)
+        assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)
+        assert [(int(o["kind"]), int(o["loader"])) for o in d.ops] == [(desc_interp.K_IGEMM, 3)], wl.name
 
 
 @pytest.mark.parametrize("kw", [

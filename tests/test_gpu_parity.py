@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 from helpers import assert_bit_exact, families, oracle_eval, oracle_network, run_on_gpu
-from test_emitter import CONV, MATMUL, WINDOW_RING, _chain_program, _padded_chain, matmul_id
+from test_emitter import CONV, MATMUL, WINDOW_RING, WINDOW_RING_FEW_CHANNELS, _chain_program, _padded_chain, matmul_id
 from torq_compiler_amd import Executable, ThipError, runtime, workloads as w
 
 pytestmark = pytest.mark.gpu
@@ -104,13 +104,26 @@ def test_conv2d_window_ring_k128(device, monkeypatch):
         assert k[0].startswith("igemm_dense_conv_i8<256,256,2,2,2,1,"), k
     k = check(device, w.conv2d_workload(N=2, H=32, W=32, C=128, O=64, realistic=False))  # the literal requant range
     assert k[0].startswith("igemm_dense_conv_i8<256,256,2,2,2,1,"), k
-    k = check(device, w.conv2d_workload(N=2, H=32, W=32, C=64, O=64, realistic=True))    # C % 128 != 0: the switch does not apply
-    assert k[0].startswith("igemm_dense_conv_i8<128,128,"), k  # 8 row tiles: too few for the one-column tile
+    k = check(device, w.conv2d_workload(N=2, H=32, W=32, C=64, O=64, realistic=True))    # half a k-tile per tap
+    assert k[0].startswith("igemm_dense_conv_i8<256,256,2,2,2,1,"), k
     monkeypatch.delenv("THIP_WINDOW_VARIANT")
+    k = check(device, w.conv2d_workload(N=2, H=32, W=32, C=64, O=64, realistic=True))
+    assert k[0].startswith("igemm_dense_conv_i8<128,128,"), k  # 8 row tiles: too few for the one-column tile
     k = check(device, w.conv2d_workload(N=30, H=48, W=48, C=64, O=64, realistic=True), via="device")  # 270 row tiles: one tile column
     assert k[0].startswith("igemm_dense_conv_i8<256,64,"), k
     k = check(device, w.conv2d_workload(N=1, H=14, W=14, C=256, O=256, realistic=True))  # few pixels, a long K: still the ring kernel
     assert k[0].startswith("igemm_dense_conv_i8<128,128,"), k
+
+
+@pytest.mark.parametrize("variant", [None, 14, 9])
+def test_conv2d_window_ring_few_channels(device, variant, monkeypatch):
+    """Fewer channels than a k-tile: the chunks of one k-tile span several taps and window rows."""
+    monkeypatch.setenv("THIP_RING_MIN_C", "16")
+    if variant is not None:
+        monkeypatch.setenv("THIP_WINDOW_VARIANT", str(variant))
+    for kw in WINDOW_RING_FEW_CHANNELS:
+        k = check(device, w.conv2d_workload(realistic=True, **kw), via="device")
+        assert families(k) == ["igemm_dense_conv_i8"], (kw, k)
 
 
 def test_conv2d_window_ring_switch(device, monkeypatch):

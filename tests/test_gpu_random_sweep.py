@@ -105,16 +105,16 @@ def _add(seed):
                           output_zp=int(rng.integers(-128, 128)), seed=seed)
 
 
-def _conv_ring(seed, channels=(64, 64, 128, 192)):
+def _conv_ring(seed, channels=(64, 64, 128, 192), images=(3, 6), extent=(30, 50)):
     """A multiple of 16 channels, 64 or more, and at least 2048 output pixels: the ring kernel's window addressing."""
     rng = np.random.default_rng(seed)
     KH, KW = int(rng.integers(1, 5)), int(rng.integers(1, 5))
     stride = (int(rng.integers(1, 3)), int(rng.integers(1, 3)))
-    H, W = int(rng.integers(30, 50)) * stride[0], int(rng.integers(30, 50)) * stride[1]
+    H, W = int(rng.integers(*extent)) * stride[0], int(rng.integers(*extent)) * stride[1]
     pad = (int(rng.integers(0, KW)), int(rng.integers(0, KW)), int(rng.integers(0, KH)), int(rng.integers(0, KH)))
     zp = int(rng.integers(-128, 128))
     lo, hi = _clamp(rng, zp)
-    return w.conv2d_workload(N=int(rng.integers(3, 6)), H=H, W=W, C=int(rng.choice(channels)), O=int(rng.choice([32, 48, 64, 72, 96, 160, 272])), KH=KH, KW=KW,
+    return w.conv2d_workload(N=int(rng.integers(*images)), H=H, W=W, C=int(rng.choice(channels)), O=int(rng.choice([32, 48, 64, 72, 96, 160, 272])), KH=KH, KW=KW,
                              stride=stride, pad=pad, input_zp=int(rng.integers(-128, 128)), output_zp=zp, output_min=lo, output_max=hi,
                              realistic=bool(rng.integers(0, 4)), nhwc=bool(rng.integers(0, 2)), seed=seed)
 
@@ -124,9 +124,15 @@ def _conv_ring16(seed):
     return _conv_ring(seed, channels=(80, 96, 112, 144, 160, 176, 208, 240, 272))
 
 
+def _conv_ring_few(seed):
+    """Fewer channels than a k-tile over at least 20 000 output pixels: several taps per k-tile."""
+    return _conv_ring(seed, channels=(16, 32, 48), images=(10, 15), extent=(50, 60))
+
+
 SWEEP = ([("conv2d", _conv, s, {"igemm_i8", "igemm_dense_i8", "igemm_stream_i8", "igemm_dense_conv_i8"}) for s in range(5000, 5200)] +
          [("conv2d_ring", _conv_ring, s, {"igemm_dense_conv_i8"}) for s in range(5500, 5530)] +
          [("conv2d_ring16", _conv_ring16, s, {"igemm_dense_conv_i8"}) for s in range(5600, 5640)] +
+         [("conv2d_ring_few", _conv_ring_few, s, {"igemm_dense_conv_i8"}) for s in range(5700, 5730)] +
          [("depthwise", _depthwise, s, {"depthwise3x3_strip_i8", "depthwise3x3_tile_i8", "depthwise3x3_dot4_i8", "depthwise_i8"}) for s in range(6000, 6200)] +
          [("fully_connected", _fully_connected, s, {"igemm_i8", "igemm_dense_i8", "igemm_stream_i8", "fc_skinny", "fc_skinny_mfma"}) for s in range(7000, 7150)] +
          [("matmul", _matmul, s, {"igemm_i8", "igemm_dense_i8", "igemm_stream_i8", "fc_skinny", "fc_skinny_mfma"}) for s in range(8000, 8100)] +

@@ -478,7 +478,7 @@ class Emitter {
         if (const char *env = getenv("THIP_WINDOW_VARIANT"); env && *env) {
             const long v = strtol(env, nullptr, 10);
             if (v == kIgemmDense256x256 || v == kIgemmDense128x256 || v == kIgemmDense128x128 || v == kIgemmDense256x128 || v == kIgemmDense256x64) return (uint32_t)v;
-            if (v == kIgemmDense256x256K128 && C >= 128) return (uint32_t)v;
+            if (v == kIgemmDense256x256K128) return (uint32_t)v;
         }
         auto tiles = [&](uint32_t v) {
             const IgemmTile &t = igemmTile(v);
@@ -736,10 +736,14 @@ thip_status_t Emitter::emitConv2d(const thip_hl_conv2d_t &c) {
             return wd[((n * C + b % C) * KH + kh) * KW + b / C];
         });
     } else {
-        // a window over whole 64-channel k-tiles with enough rows for the large tiles, or with a long K at any size
+        // a window over a multiple of 16 channels with enough rows for the large tiles, or with a long K at any size
         // (256 -> 256 at 14 x 14, one image: 12.6 us against 15.4 on the gather kernel): the LDS-DMA ring kernel addresses
-        // the window itself (THIP_NO_WINDOW_RING keeps such convolutions on the gather kernel, for tests and tuning)
-        const bool ring = !pointwise && Cin % 16 == 0 && Cin >= 64 && (M >= 2048 || K >= 1024) && Oout >= 32 && d.N * d.H * d.W * Cin < (1LL << 32) && !getenv("THIP_NO_WINDOW_RING");
+        // the window itself.  Fewer than 64 channels (several taps per k-tile) pay from about 20 000 output pixels
+        // (32 -> 64 at 112 x 112: 8.6 us against 10.6 at batch 8, 5.8 against 4.8 for one image).  THIP_NO_WINDOW_RING
+        // keeps such convolutions on the gather kernel and THIP_RING_MIN_C sets the channel count alone, for tests and tuning.
+        const char *minC = getenv("THIP_RING_MIN_C");
+        const bool channelsFit = Cin % 16 == 0 && (minC && *minC ? Cin >= atoi(minC) : (Cin >= 64 || M >= 20000));
+        const bool ring = !pointwise && channelsFit && (M >= 2048 || K >= 1024) && Oout >= 32 && d.N * d.H * d.W * Cin < (1LL << 32) && !getenv("THIP_NO_WINDOW_RING");
         emitIgemm(op, M, Oout, K, (pointwise && K % 16 == 0) ? kLoaderDense : ring ? kLoaderWindow : kLoaderGather, [&](int64_t n, int64_t k) -> int8_t {
             const int64_t pos = k / Cin, ci = k % Cin;
             const int64_t kh = pos / KW, kw = pos % KW;

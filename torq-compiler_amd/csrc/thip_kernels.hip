@@ -858,11 +858,26 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
     }
     // CONV: the tap the lane's 16-byte chunk of the next k-tile to be issued belongs to, the chunk's first channel and
     // its byte offset from a window origin.  C is a multiple of 16, so a chunk never straddles two taps, but the chunks
-    // of one tile row may (C need not be a multiple of BK): the state is per lane.  Chunks of the last tile past
+    // of one tile row may (C need not be a multiple of BK, and may be less): the state is per lane.  Chunks of the last tile past
     // KH * KW * C carry on into row KH of the window: inside the image they read valid bytes, which meet zero weights.
     int tapH = 0, tapW = 0, tapC = CONV ? lchunk * 16 : 0;
     uint32_t tapOff = (uint32_t)tapC;
     const uint32_t rowJump = CONV ? ((uint32_t)p.W - (uint32_t)p.KW) * (uint32_t)p.C : 0u;
+    // brings tapC back below C once: on to the next column of the window, at the end of a window row on to the next row
+    auto tapWrap = [&]() {
+        const bool endC = tapC >= p.C;
+        tapC -= endC ? p.C : 0;
+        const bool endW = endC && tapW + 1 == p.KW;
+        tapW = endC ? (endW ? 0 : tapW + 1) : tapW;
+        tapH += endW ? 1 : 0;
+        tapOff += endW ? rowJump : 0u;
+    };
+    if constexpr (CONV) {
+        if (p.C < BK) {  // the chunks of the first k-tile already span several taps
+#pragma unroll
+            for (int extra = 1; extra < CH; extra++) tapWrap();
+        }
+    }
     const int8_t *zpPage = CONV ? (const int8_t *)p.ktab + lchunk * 16 : nullptr;
 #pragma unroll
     for (int i = 0; i < LB; i++) {
@@ -928,19 +943,20 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64, BLOCKS_PER_CU) void igemm_de
         }
         if constexpr (CONV) {
             if (part == parts - 1) {
-                // on to tile kt + 1: BK channels further (BK <= C: at most one wrap), then the next column, then the
-                // next row of the window
-                const bool endC = tapC + BK >= p.C;
-                tapC = endC ? tapC + BK - p.C : tapC + BK;
-                const bool endW = endC && tapW + 1 == p.KW;
-                tapW = endC ? (endW ? 0 : tapW + 1) : tapW;
-                tapH += endW ? 1 : 0;
-                // channels and columns of one window row are contiguous in the image: BK bytes on, and at the end of
-                // a window row the rest of the image row as well (modulo 2^32 where the window is wider than the image).
+                // on to tile kt + 1: BK bytes further along the window.  Channels and columns of one window row are
+                // contiguous in the image, so the offset moves on by BK, and by the rest of the image row as well
+                // wherever a window row ends (modulo 2^32 where the window is wider than the image).  With C >= BK
+                // that is one wrap of the channel at most; fewer channels wrap up to BK / 16 times.
                 // (Recomputing (tapH * W + tapW) * C + tapC instead becomes a 64-bit multiply-add whose unused upper
                 // addend lands in a register with a load in flight, and the compiler then drains vmcnt in every
                 // k-tile: 17.0 us against 12.8 for 256 -> 256 channels at 14 x 14.)
-                tapOff += (uint32_t)BK + (endW ? rowJump : 0u);
+                tapC += BK;
+                tapOff += (uint32_t)BK;
+                tapWrap();
+                if (p.C < BK) {
+#pragma unroll
+                    for (int extra = 1; extra < CH; extra++) tapWrap();
+                }
             }
         }
     };
@@ -1586,10 +1602,10 @@ hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, const LaunchCtx &ct
         if (a.OH <= 0 || a.OW <= 0 || a.M % (a.OH * a.OW) != 0) return hipErrorInvalidValue;
         if (((uintptr_t)a.A & (a.gran - 1)) != 0) return hipErrorInvalidValue;
     } else if (a.loader == kLoaderWindow) {
-        // the ring kernel's window addressing: whole 16-byte chunks per tap, a k-tile no longer than a tap (the walk
-        // wraps once per tile at most), 32-bit byte offsets into the image, a page of zero-point bytes behind ktab,
+        // the ring kernel's window addressing: whole 16-byte chunks per tap (so the walk wraps the channel at most
+        // bk / 16 times per k-tile), 32-bit byte offsets into the image, a page of zero-point bytes behind ktab,
         // every tap offset non-negative once the tap lies inside the image, K rounded up to whole k-tiles
-        if (!a.ktab || ((uintptr_t)a.ktab & 15) != 0 || a.C < t.bk || a.C % 16 != 0 || a.KH <= 0 || a.KW <= 0) return hipErrorInvalidValue;
+        if (!a.ktab || ((uintptr_t)a.ktab & 15) != 0 || a.C < 16 || a.C % 16 != 0 || a.KH <= 0 || a.KW <= 0) return hipErrorInvalidValue;
         if (a.H <= 0 || a.W <= 0 || a.OH <= 0 || a.OW <= 0 || a.SH <= 0 || a.SW <= 0 || a.PT < 0 || a.PL < 0) return hipErrorInvalidValue;
         if (a.M % (a.OH * a.OW) != 0 || (long long)a.K != (long long)a.KH * a.KW * a.C || a.Kp != (a.K + t.bk - 1) / t.bk * t.bk) return hipErrorInvalidValue;
         if (a.a_bytes != (long long)(a.M / (a.OH * a.OW)) * a.H * a.W * a.C || a.a_bytes >= (1LL << 32)) return hipErrorInvalidValue;
@@ -1600,7 +1616,7 @@ hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, const LaunchCtx &ct
         case kIgemmDense128x128: return launchIgemmDense<128, 128, 2, 2, 4, 2, true>(a, ctx);
         case kIgemmDense256x128: return launchIgemmDense<256, 128, 2, 2, 3, 2, true>(a, ctx);
         case kIgemmDense256x64: return launchIgemmDense<256, 64, 4, 1, 3, 2, true>(a, ctx);
-        case kIgemmDense256x256K128: return launchIgemmDense<256, 256, 2, 2, 2, 1, true, 128>(a, ctx);  // C >= 128 (checked above): 128 channels per k-tile
+        case kIgemmDense256x256K128: return launchIgemmDense<256, 256, 2, 2, 2, 1, true, 128>(a, ctx);  // 128 channels per k-tile
         default: return hipErrorInvalidValue;
         }
     } else {

@@ -184,8 +184,8 @@ thip_status_t checkOpFootprint(const DescriptorView *e, uint32_t i) {
         if (op.loader > kLoaderWindow) return fail(THIP_INVALID_ARGUMENT, "op %u: unknown igemm loader %u", i, op.loader);
         if (op.loader == kLoaderWindow) {
             const int32_t bk = igemmTile(op.variant).bk;
-            if (!positive({op.KH, op.KW, op.SH, op.SW}) || op.PT < 0 || op.PL < 0 || op.C < bk || op.C % 16 != 0 || mul(op.KH, op.KW, op.C) != (uint64_t)op.K || op.Kp != (op.K + bk - 1) / bk * bk) {
-                return fail(THIP_INVALID_ARGUMENT, "op %u: the window loader needs a multiple of 16 channels, at least one k-tile of them, and K rounded up to whole k-tiles", i);
+            if (!positive({op.KH, op.KW, op.SH, op.SW}) || op.PT < 0 || op.PL < 0 || op.C < 16 || op.C % 16 != 0 || mul(op.KH, op.KW, op.C) != (uint64_t)op.K || op.Kp != (op.K + bk - 1) / bk * bk) {
+                return fail(THIP_INVALID_ARGUMENT, "op %u: the window loader needs a multiple of 16 channels and K rounded up to whole k-tiles", i);
             }
             if (inBytes >= (1ull << 32)) return fail(THIP_INVALID_ARGUMENT, "op %u: image too large for the window loader", i);
             switch (op.variant) {
