@@ -54,6 +54,8 @@ def workload_table(pkg):
         # and a pointwise expansion whose K is short
         "conv3x3_56x56x256_o256_b32": (lambda: w.conv2d_workload(N=32, H=56, W=56, C=256, O=256, realistic=True), "mfma"),
         "conv3x3_28x28x512_o512_b32": (lambda: w.conv2d_workload(N=32, H=28, W=28, C=512, O=512, realistic=True), "mfma"),
+        # a channel count that is no multiple of the 64-byte k-tile: k-tiles straddle the window's taps
+        "conv3x3_56x56x96_o96_b32": (lambda: w.conv2d_workload(N=32, H=56, W=56, C=96, O=96, realistic=True), "mfma"),
         "conv1x1_56x56x256_o1024_b32": (lambda: w.conv2d_workload(N=32, H=56, W=56, C=256, O=1024, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True), "mfma"),
         "depthwise_b64": (lambda: w.depthwise_workload(N=64), "hbm"),
         "depthwise_b1": (lambda: w.depthwise_workload(N=1), "hbm"),

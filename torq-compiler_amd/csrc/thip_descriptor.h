@@ -102,9 +102,9 @@ enum IgemmLoader : uint32_t {
     // (what it reads past the KW * C bytes meets zero weights).  Table: one entry per group,
     // kh in bits 24..30, run length KW * C in bits 0..15.
     kLoaderRuns = 2,
-    // a convolution window over an image with C % 64 == 0, addressed by the LDS-DMA ring kernel itself: a k-tile is 64
-    // channels of one tap (128 with C % 128 == 0 on the 128-byte variant), K = Kp = KH * KW * C.  Table: 128 bytes of input_zp
-    // (what a tap outside the image reads).
+    // a convolution window over an image with C % 16 == 0, addressed by the LDS-DMA ring kernel itself: every 16-byte
+    // chunk of a k-tile is 16 channels of one tap, K = KH * KW * C, Kp = K rounded up to whole k-tiles (zero weights
+    // beyond K).  Table: 128 bytes of input_zp (what a tap outside the image reads).
     kLoaderWindow = 3,
 };
 
