@@ -47,8 +47,7 @@ def test_conv2d_descriptor(kw, nhwc):
         assert kinds[0] == desc_interp.K_TRANSPOSE and kinds[1] == desc_interp.K_IGEMM
 
 
-# Convolutions over a multiple of 16 channels (64 at least) with at least 2048 output pixels or a long K: the LDS-DMA ring
-# kernel addresses the window.
+# Convolutions over a multiple of 16 channels: the LDS-DMA ring kernel addresses the window.
 WINDOW_RING = [
     dict(N=2, H=32, W=32, C=64, O=64),                                            # M = 2048: the smallest taken; one tile column
     dict(N=10, H=29, W=31, C=64, O=96, stride=(2, 2), pad=(0, 1, 0, 1)),          # odd frame, stride 2, one-sided padding, ragged M
@@ -109,9 +108,9 @@ def test_dense_k128_records(monkeypatch):
 
 
 def test_conv2d_window_loader_records():
-    """A multiple of 16 channels (64 or more) and enough rows: the record asks for the ring kernel's window addressing
-    (loader 3, a page of zero-point bytes as its table, K rounded up to whole k-tiles); fewer rows, other channel counts
-    or the switch keep the gather loader."""
+    """A multiple of 16 channels: the record asks for the ring kernel's window addressing (loader 3, a page of
+    zero-point bytes as its table, K rounded up to whole k-tiles); other channel counts, few output channels or the
+    switch keep the gather loader."""
     import os
     for kw in WINDOW_RING:
         wl = w.conv2d_workload(realistic=True, **kw)
@@ -120,9 +119,16 @@ def test_conv2d_window_loader_records():
         assert [(int(o["kind"]), int(o["loader"])) for o in d.ops] == [(desc_interp.K_IGEMM, 3)], wl.name
         bk = 128 if int(d.ops[0]["variant"]) == 14 else 64
         assert int(d.ops[0]["Kp"]) == -(-int(d.ops[0]["K"]) // bk) * bk
-    for kw in (dict(N=1, H=32, W=32, C=64, O=64), dict(N=2, H=32, W=32, C=72, O=64), dict(N=2, H=32, W=32, C=48, O=64), dict(N=2, H=32, W=32, C=64, O=16)):
+    for kw in (dict(N=2, H=32, W=32, C=72, O=64), dict(N=2, H=32, W=32, C=40, O=64), dict(N=2, H=32, W=32, C=64, O=16)):
         d = interp(w.conv2d_workload(realistic=True, **kw))[1]
         assert int(d.ops[0]["loader"]) == 1, kw
+    # small convolutions take the 64 x 64 tile (up to 512 of them)
+    for kw, variant in ((dict(N=1, H=32, W=32, C=64, O=64), 7), (dict(N=1, H=7, W=7, C=160, O=160), 7), (dict(N=1, H=28, W=28, C=32, O=32), 7),
+                        (dict(N=16, H=14, W=14, C=512, O=512), 7), (dict(N=32, H=14, W=14, C=512, O=512), 5)):
+        wl = w.conv2d_workload(realistic=True, **kw)
+        outs, d = interp(wl)
+        assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)
+        assert (int(d.ops[0]["loader"]), int(d.ops[0]["variant"])) == (3, variant), kw
     os.environ["THIP_NO_WINDOW_RING"] = "1"
     try:
         assert int(interp(w.conv2d_workload(realistic=True, **WINDOW_RING[0]))[1].ops[0]["loader"]) == 1
@@ -132,8 +138,7 @@ def test_conv2d_window_loader_records():
 
 @pytest.mark.parametrize("variant", [None, 14])
 def test_conv2d_window_loader_few_channels(variant, monkeypatch):
-    """16, 32 and 48 channels on the window loader (THIP_RING_MIN_C lowers the channel count from which it is taken)."""
-    monkeypatch.setenv("THIP_RING_MIN_C", "16")
+    """16, 32 and 48 channels on the window loader: several taps per k-tile."""
     if variant is not None:
         monkeypatch.setenv("THIP_WINDOW_VARIANT", str(variant))
     for kw in WINDOW_RING_FEW_CHANNELS:

@@ -38,11 +38,11 @@ def check(device, wl, via="host", kernel=None):
 # ---- conv2d ---------------------------------------------------------------------------------
 def test_conv2d_config0_literal(device):
     """benchmark configuration 0 with its literal (saturating) requant ranges."""
-    check(device, w.conv2d_workload(), kernel="igemm_i8")
+    check(device, w.conv2d_workload(), kernel="igemm_dense_conv_i8")
 
 
 def test_conv2d_config0_realistic(device):
-    check(device, w.conv2d_workload(realistic=True), via="device", kernel="igemm_i8")
+    check(device, w.conv2d_workload(realistic=True), via="device", kernel="igemm_dense_conv_i8")
 
 
 def test_conv2d_config0_nchw_boundary(device):
@@ -60,7 +60,7 @@ def test_conv2d_geometries(device, kw, nhwc):
 @pytest.mark.parametrize("variant", [0, 1, 2, 3])
 def test_conv2d_every_tile_variant(device, variant, monkeypatch):
     monkeypatch.setenv("THIP_IGEMM_VARIANT", str(variant))
-    k = check(device, w.conv2d_workload(N=2, H=28, W=28, C=32, O=96, realistic=True))
+    k = check(device, w.conv2d_workload(N=2, H=28, W=28, C=24, O=96, realistic=True))  # 24 channels: the gather kernel
     assert runtime.lib()  # the variant is baked into the descriptor at serialize time
     names = ["igemm_i8<128,128,64,", "igemm_i8<256,256,64,", "igemm_i8<64,64,64,", "igemm_i8<256,128,64,"]
     assert k[0].startswith(names[variant]), k
@@ -77,11 +77,11 @@ def test_conv2d_window_ring(device, kw):
     assert "igemm_dense_conv_i8" in families(k), k
 
 
-@pytest.mark.parametrize("variant", [4, 5, 6, 8, 9])
+@pytest.mark.parametrize("variant", [4, 5, 6, 7, 8, 9])
 def test_conv2d_window_ring_every_tile(device, variant, monkeypatch):
     monkeypatch.setenv("THIP_WINDOW_VARIANT", str(variant))
-    names = {4: "igemm_dense_conv_i8<256,256,", 5: "igemm_dense_conv_i8<128,128,", 6: "igemm_dense_conv_i8<128,256,", 8: "igemm_dense_conv_i8<256,128,",
-             9: "igemm_dense_conv_i8<256,64,"}
+    names = {4: "igemm_dense_conv_i8<256,256,", 5: "igemm_dense_conv_i8<128,128,", 6: "igemm_dense_conv_i8<128,256,", 7: "igemm_dense_conv_i8<64,64,",
+             8: "igemm_dense_conv_i8<256,128,", 9: "igemm_dense_conv_i8<256,64,"}
     for kw in (dict(N=2, H=33, W=35, C=64, O=80, pad=(1, 1, 1, 1)), dict(N=5, H=47, W=45, C=128, O=48, stride=(2, 2), pad=(1, 0, 1, 0), output_zp=-7, output_min=-128),
                dict(N=3, H=29, W=31, C=80, O=72, pad=(1, 1, 1, 1), input_zp=-90), dict(N=4, H=40, W=33, C=176, O=130, KH=2, KW=2, stride=(1, 2), pad=(0, 1, 1, 0))):
         k = check(device, w.conv2d_workload(realistic=True, **kw), via="device")
@@ -108,17 +108,20 @@ def test_conv2d_window_ring_k128(device, monkeypatch):
     assert k[0].startswith("igemm_dense_conv_i8<256,256,2,2,2,1,"), k
     monkeypatch.delenv("THIP_WINDOW_VARIANT")
     k = check(device, w.conv2d_workload(N=2, H=32, W=32, C=64, O=64, realistic=True))
-    assert k[0].startswith("igemm_dense_conv_i8<128,128,"), k  # 8 row tiles: too few for the one-column tile
+    assert k[0].startswith("igemm_dense_conv_i8<64,64,2,2,5,4,"), k   # 32 small tiles
+    k = check(device, w.conv2d_workload(N=20, H=32, W=32, C=64, O=128, realistic=True))
+    assert k[0].startswith("igemm_dense_conv_i8<128,128,"), k         # 640 small tiles would be too many, 160 of 128 x 128
     k = check(device, w.conv2d_workload(N=30, H=48, W=48, C=64, O=64, realistic=True), via="device")  # 270 row tiles: one tile column
     assert k[0].startswith("igemm_dense_conv_i8<256,64,"), k
-    k = check(device, w.conv2d_workload(N=1, H=14, W=14, C=256, O=256, realistic=True))  # few pixels, a long K: still the ring kernel
-    assert k[0].startswith("igemm_dense_conv_i8<128,128,"), k
+    k = check(device, w.conv2d_workload(N=1, H=14, W=14, C=256, O=256, realistic=True))  # few pixels, a long K: the small tile
+    assert k[0].startswith("igemm_dense_conv_i8<64,64,2,2,5,4,"), k
+    k = check(device, w.conv2d_workload(N=1, H=14, W=14, C=256, O=250, realistic=False))  # the small tile's staged epilogue
+    assert k[0].startswith("igemm_dense_conv_i8<64,64,2,2,5,4,0,"), k
 
 
 @pytest.mark.parametrize("variant", [None, 14, 9])
 def test_conv2d_window_ring_few_channels(device, variant, monkeypatch):
     """Fewer channels than a k-tile: the chunks of one k-tile span several taps and window rows."""
-    monkeypatch.setenv("THIP_RING_MIN_C", "16")
     if variant is not None:
         monkeypatch.setenv("THIP_WINDOW_VARIANT", str(variant))
     for kw in WINDOW_RING_FEW_CHANNELS:

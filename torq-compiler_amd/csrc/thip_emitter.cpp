@@ -477,7 +477,7 @@ class Emitter {
     static uint32_t chooseWindowVariant(int64_t M, int64_t N, int64_t C) {
         if (const char *env = getenv("THIP_WINDOW_VARIANT"); env && *env) {
             const long v = strtol(env, nullptr, 10);
-            if (v == kIgemmDense256x256 || v == kIgemmDense128x256 || v == kIgemmDense128x128 || v == kIgemmDense256x128 || v == kIgemmDense256x64) return (uint32_t)v;
+            if (v == kIgemmDense256x256 || v == kIgemmDense128x256 || v == kIgemmDense128x128 || v == kIgemmDense256x128 || v == kIgemmDense256x64 || v == kIgemmDense64x64) return (uint32_t)v;
             if (v == kIgemmDense256x256K128) return (uint32_t)v;
         }
         auto tiles = [&](uint32_t v) {
@@ -490,6 +490,10 @@ class Emitter {
             const int64_t np = roundUp(N, igemmTile(v).bn);
             return np > roundUp(N, 128) && (np - N) * 8 > N;
         };
+        // up to two small tiles per CU: the 64 x 64 tile (five stages deep, four blocks per CU) spreads a small
+        // convolution over the chip (256 -> 256 at 14 x 14: 10.8 us against 13.7 on 7 tiles of 128 x 128; 512 -> 512 at
+        // 14 x 14, batch 16, 392 tiles: 20.0 against 24.2; at 784 tiles the 128 x 128 tile is ahead, 14.5 against 21.0)
+        if (tiles(kIgemmDense64x64) <= 512) return kIgemmDense64x64;
         // few output channels over many pixels: one tile column, the image is read once (64 -> 64 at 112 x 112, batch 32:
         // 27.8 us against 41.1 with 128 x 128 tiles); with fewer than a tile per CU the smaller tile wins (128 -> 128 at
         // 28 x 28, batch 8: 8.5 us against 12.4)
@@ -736,14 +740,14 @@ thip_status_t Emitter::emitConv2d(const thip_hl_conv2d_t &c) {
             return wd[((n * C + b % C) * KH + kh) * KW + b / C];
         });
     } else {
-        // a window over a multiple of 16 channels with enough rows for the large tiles, or with a long K at any size
-        // (256 -> 256 at 14 x 14, one image: 12.6 us against 15.4 on the gather kernel): the LDS-DMA ring kernel addresses
-        // the window itself.  Fewer than 64 channels (several taps per k-tile) pay from about 20 000 output pixels
-        // (32 -> 64 at 112 x 112: 8.6 us against 10.6 at batch 8, 5.8 against 4.8 for one image).  THIP_NO_WINDOW_RING
-        // keeps such convolutions on the gather kernel and THIP_RING_MIN_C sets the channel count alone, for tests and tuning.
-        const char *minC = getenv("THIP_RING_MIN_C");
-        const bool channelsFit = Cin % 16 == 0 && (minC && *minC ? Cin >= atoi(minC) : (Cin >= 64 || M >= 20000));
-        const bool ring = !pointwise && channelsFit && (M >= 2048 || K >= 1024) && Oout >= 32 && d.N * d.H * d.W * Cin < (1LL << 32) && !getenv("THIP_NO_WINDOW_RING");
+        // a window over a multiple of 16 channels: the LDS-DMA ring kernel addresses the window itself, at every size
+        // (256 -> 256 at 14 x 14, one image: 10.8 us against 15.3 on the gather kernel; 32 -> 32 at 28 x 28: 4.4
+        // against 4.8; 96 -> 96 at 56 x 56, batch 32: 17.3 against 29.4).  THIP_NO_WINDOW_RING keeps such convolutions
+        // on the gather kernel; THIP_RING_MIN_C and THIP_RING_MIN_M raise the channel and pixel counts from which the
+        // ring kernel is taken (tests and tuning).
+        const char *minC = getenv("THIP_RING_MIN_C"), *minM = getenv("THIP_RING_MIN_M");
+        const bool ring = !pointwise && Cin % 16 == 0 && Cin >= (minC && *minC ? atoi(minC) : 16) && M >= (minM && *minM ? atoi(minM) : 1) && Oout >= 32 &&
+                          d.N * d.H * d.W * Cin < (1LL << 32) && !getenv("THIP_NO_WINDOW_RING");
         emitIgemm(op, M, Oout, K, (pointwise && K % 16 == 0) ? kLoaderDense : ring ? kLoaderWindow : kLoaderGather, [&](int64_t n, int64_t k) -> int8_t {
             const int64_t pos = k / Cin, ci = k % Cin;
             const int64_t kh = pos / KW, kw = pos % KW;
