@@ -108,15 +108,15 @@ def test_conv2d_window_ring_k128(device, monkeypatch):
     assert k[0].startswith("igemm_dense_conv_i8<256,256,2,2,2,1,"), k
     monkeypatch.delenv("THIP_WINDOW_VARIANT")
     k = check(device, w.conv2d_workload(N=2, H=32, W=32, C=64, O=64, realistic=True))
-    assert k[0].startswith("igemm_dense_conv_i8<64,64,2,2,5,4,"), k   # 32 small tiles
+    assert k[0].startswith("igemm_dense_conv_i8<64,64,2,2,4,4,"), k   # 32 small tiles
     k = check(device, w.conv2d_workload(N=20, H=32, W=32, C=64, O=128, realistic=True))
     assert k[0].startswith("igemm_dense_conv_i8<128,128,"), k         # 640 small tiles would be too many, 160 of 128 x 128
     k = check(device, w.conv2d_workload(N=30, H=48, W=48, C=64, O=64, realistic=True), via="device")  # 270 row tiles: one tile column
     assert k[0].startswith("igemm_dense_conv_i8<256,64,"), k
     k = check(device, w.conv2d_workload(N=1, H=14, W=14, C=256, O=256, realistic=True))  # few pixels, a long K: the small tile
-    assert k[0].startswith("igemm_dense_conv_i8<64,64,2,2,5,4,"), k
+    assert k[0].startswith("igemm_dense_conv_i8<64,64,2,2,4,4,"), k
     k = check(device, w.conv2d_workload(N=1, H=14, W=14, C=256, O=250, realistic=False))  # the small tile's staged epilogue
-    assert k[0].startswith("igemm_dense_conv_i8<64,64,2,2,5,4,0,"), k
+    assert k[0].startswith("igemm_dense_conv_i8<64,64,2,2,4,4,0,"), k
 
 
 @pytest.mark.parametrize("variant", [None, 14, 9])

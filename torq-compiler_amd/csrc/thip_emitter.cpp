@@ -490,9 +490,9 @@ class Emitter {
             const int64_t np = roundUp(N, igemmTile(v).bn);
             return np > roundUp(N, 128) && (np - N) * 8 > N;
         };
-        // up to two small tiles per CU: the 64 x 64 tile (five stages deep, four blocks per CU) spreads a small
-        // convolution over the chip (256 -> 256 at 14 x 14: 10.8 us against 13.7 on 7 tiles of 128 x 128; 512 -> 512 at
-        // 14 x 14, batch 16, 392 tiles: 20.0 against 24.2; at 784 tiles the 128 x 128 tile is ahead, 14.5 against 21.0)
+        // up to two small tiles per CU: the 64 x 64 tile (four blocks per CU) spreads a small convolution over the chip
+        // (256 -> 256 at 14 x 14: 10.3 us against 13.7 on 7 tiles of 128 x 128; 512 -> 512 at 14 x 14, batch 16, 392
+        // tiles: 17.8 against 24.2; at 784 tiles the 128 x 128 tile is ahead, 14.5 against 19.8)
         if (tiles(kIgemmDense64x64) <= 512) return kIgemmDense64x64;
         // few output channels over many pixels: one tile column, the image is read once (64 -> 64 at 112 x 112, batch 32:
         // 27.8 us against 41.1 with 128 x 128 tiles); with fewer than a tile per CU the smaller tile wins (128 -> 128 at
@@ -741,7 +741,7 @@ thip_status_t Emitter::emitConv2d(const thip_hl_conv2d_t &c) {
         });
     } else {
         // a window over a multiple of 16 channels: the LDS-DMA ring kernel addresses the window itself, at every size
-        // (256 -> 256 at 14 x 14, one image: 10.8 us against 15.3 on the gather kernel; 32 -> 32 at 28 x 28: 4.4
+        // (256 -> 256 at 14 x 14, one image: 10.3 us against 15.3 on the gather kernel; 32 -> 32 at 28 x 28: 4.3
         // against 4.8; 96 -> 96 at 56 x 56, batch 32: 17.3 against 29.4).  THIP_NO_WINDOW_RING keeps such convolutions
         // on the gather kernel; THIP_RING_MIN_C and THIP_RING_MIN_M raise the channel and pixel counts from which the
         // ring kernel is taken (tests and tuning).
