@@ -494,10 +494,12 @@ class Emitter {
         // (256 -> 256 at 14 x 14: 10.3 us against 13.7 on 7 tiles of 128 x 128; 512 -> 512 at 14 x 14, batch 16, 392
         // tiles: 17.8 against 24.2; at 784 tiles the 128 x 128 tile is ahead, 14.5 against 19.8)
         if (tiles(kIgemmDense64x64) <= 512) return kIgemmDense64x64;
-        // few output channels over many pixels: one tile column, the image is read once (64 -> 64 at 112 x 112, batch 32:
-        // 27.8 us against 41.1 with 128 x 128 tiles); with fewer than a tile per CU the smaller tile wins (128 -> 128 at
-        // 28 x 28, batch 8: 8.5 us against 12.4)
-        if (N <= 64 && tiles(kIgemmDense256x64) >= 224) return kIgemmDense256x64;
+        // few output channels: one tile column, the image is read once (64 -> 64 at 112 x 112, batch 32: 27.8 us against
+        // 41.1 with 128 x 128 tiles).  At most 64 output channels never take a wider tile (32 -> 64 at 112 x 112, batch
+        // 3 / 4: 6.2 / 7.2 us on 588 / 784 small tiles, 6.5 / 6.6 on one column of 256 x 64, 7.0 / 7.1 on 128 x 128); up
+        // to 128 take theirs with a tile per CU, below that the 128 x 128 tile wins (128 -> 128 at 28 x 28, batch 8: 8.5 us
+        // against 12.4)
+        if (N <= 64) return tiles(kIgemmDense64x64) <= 640 ? kIgemmDense64x64 : kIgemmDense256x64;
         if (N <= 128 && tiles(kIgemmDense256x128) >= 224) return kIgemmDense256x128;
         // measured on 3x3 convolutions of 64 .. 512 channels at batch 1 .. 64: the largest tile wins as soon as half the CUs
         // get one (a long K per tile amortises its prologue and epilogue), unless it pads N by more than an eighth

@@ -1577,7 +1577,7 @@ static hipError_t launchIgemmDense(const IgemmArgs &a, const LaunchCtx &ctx) {
         }
     }
     if (direct) return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, 1, false, CONV, BK>(a, ctx);
-    if constexpr (BM * BN >= 128 * 128) {
+    if constexpr (BM * BN >= 128 * 128 || CONV) {  // and the small window tile: the benchmark's own convolution with its literal requant range, 4.9 -> 4.5 us
         if (inRegisters && wide) return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, 2, false, CONV, BK>(a, ctx);
     }
     return launchIgemmDenseE<BM, BN, WAVES_M, WAVES_N, STAGES, BLOCKS_PER_CU, 0, false, CONV, BK>(a, ctx);
