@@ -144,6 +144,11 @@ def test_dense_igemm_every_tile_variant(device, variant, monkeypatch):
     assert k[0].startswith("igemm_dense_i8<%d,%d," % tile) and k[0].endswith(",0,0>"), k  # N % 16 != 0: results leave through LDS
     k = check(device, w.fully_connected_workload(512, 1024, 512, realistic=True))
     assert k[0].startswith("igemm_dense_i8<%d,%d," % tile) and k[0].endswith(",1,0>"), k  # N % 16 == 0, shift >= 33: the in-register epilogue
+    k = check(device, w.fully_connected_workload(300, 320, 528))
+    assert k[0].startswith("igemm_dense_i8<%d,%d," % tile) and k[0].endswith(",2,0>"), k  # the literal requant range: the general 32-bit tail, in registers
+    for shift in (32, 40, 50, 62):
+        k = check(device, w.fully_connected_workload(130, 96, 64, shift=shift, output_zp=-7))
+        assert k[0].endswith(",2,0>" if shift > 45 or shift == 32 else ",1,0>"), (shift, k)
     check(device, w.fully_connected_workload(257, 80, 48, realistic=True))
     check(device, w.fully_connected_workload(33, 16, 1000, realistic=True))
     check(device, w.fully_connected_workload(1000, 4096, 272, realistic=True))
