@@ -144,17 +144,17 @@ class Loaded:
 # (KiB per dispatch; the factors are what the same counters read for a plain 256 MiB copy, --copy-calibration).
 # They belong to the kernels as they were when the counters were read: TRAFFIC_KERNELS_SHA256 is the hash of
 # torq-compiler_amd/csrc/thip_kernels.hip at that time, and a run on other kernel sources reports traffic null.
-TRAFFIC_KERNELS_SHA256 = "566202ce933049d85a94b6da2b9a5aea48d738abdba70619d0c0aa13020b6819"
+TRAFFIC_KERNELS_SHA256 = "2929b1e29a0eceaed4b5222ad00c941bca9dbea14c0b5102394e73af94b1737d"
 MEASURED_TRAFFIC = {
-    "fc_4096x4096x4096": (49384.0 * 1.9995 + 16595.8 * 1.0000) * 1024,
-    "fc_512x4096x4096": (16472.0 * 1.9995 + 2048.0 * 1.0000) * 1024,
-    "fc_16x2048x8192": (8408.0 * 1.9995 + 256.0 * 1.0000) * 1024,
-    "conv_112x112x32_o64_3x3": (363.7 * 1.9995 + 784.0 * 1.0000) * 1024,
-    "conv3x3_56x56x256_o256_b32": (17260.7 * 1.9995 + 26020.8 * 1.0000) * 1024,
-    "depthwise_b64": (15437.8 * 1.9995 + 7063.3 * 1.0000) * 1024,
-    "depthwise_s1_b256": (63702.4 * 1.9995 + 113170.7 * 1.0000) * 1024,
-    "maxpool_b64": (25117.1 * 1.9995 + 12544.0 * 1.0000) * 1024,
-    "avgpool_b64": (1998.5 * 1.9995 + 80.0 * 1.0000) * 1024,
+    "fc_4096x4096x4096": (49381.0 * 1.9995 + 16592.8 * 1.0000) * 1024,
+    "fc_512x4096x4096": (16444.0 * 1.9995 + 2048.0 * 1.0000) * 1024,
+    "fc_16x2048x8192": (8406.0 * 1.9995 + 256.0 * 1.0000) * 1024,
+    "conv_112x112x32_o64_3x3": (370.7 * 1.9995 + 784.0 * 1.0000) * 1024,
+    "conv3x3_56x56x256_o256_b32": (17261.1 * 1.9995 + 26014.2 * 1.0000) * 1024,
+    "depthwise_b64": (15436.6 * 1.9995 + 7063.3 * 1.0000) * 1024,
+    "depthwise_s1_b256": (63704.9 * 1.9995 + 113194.1 * 1.0000) * 1024,
+    "maxpool_b64": (25110.9 * 1.9995 + 12544.0 * 1.0000) * 1024,
+    "avgpool_b64": (2001.0 * 1.9995 + 80.0 * 1.0000) * 1024,
     "add_b64": (4723.0 * 1.9995 + 4704.0 * 1.0000) * 1024,
 }
 
