@@ -289,6 +289,28 @@ def test_gpu_bf16_wide_n(device):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("waves", [4, 8, 16])
+def test_gpu_bf16_wide_n_waves_per_block(device, waves, monkeypatch):
+    """The waves of a block share its input rows in LDS: four, eight or sixteen of them, every one with columns of its
+    own; the last block has waves without columns."""
+    monkeypatch.setenv("THIP_FC_WIDE_WAVES", str(waves))
+    for wl, label in [(w.fully_connected_bf16_workload(33, 200, 32800 + 96), "fc_bf16_wide<0,2,%d>" % waves),
+                      (w.expand_weights_workload(M=7, K=320, N=32768 + 160, block=64), "fc_bf16_wide<1,4,%d>" % waves),
+                      (w.expand_weights_workload(M=40, K=192, N=32768, block=32, expand_clamp=(-0.002, 0.003)), "fc_bf16_wide<2,4,%d>" % waves)]:
+        print("[gpu-case]", wl.name, flush=True)
+        got, kernels = run_on_gpu(device, wl, via="device")
+        if "qbias" in wl.attrs:
+            f = lambda bits: np.abs(orc.from_bf16(bits).astype(np.float64))
+            w16 = orc.expand_weights(wl.attrs["weights"], wl.attrs["scale"], wl.attrs["qbias"], block_size=wl.attrs["block"],
+                                     output_min=wl.attrs["expand_min"], output_max=wl.attrs["expand_max"])
+            magnitude = f(wl.inputs[0]) @ f(w16)
+        else:
+            magnitude = _magnitude(wl)
+        assert_bf16_close(got[0], oracle_eval(wl)[0].reshape(got[0].shape), wl.name + " (gpu)", magnitude=magnitude)
+        assert label in kernels, (label, kernels)
+
+
+@pytest.mark.gpu
 def test_gpu_bf16_avg_pool(device):
     """The kernel walks the frame in the oracle's order: bit-exact."""
     for wl in [w.avg_pool2d_bf16_workload(), w.avg_pool2d_bf16_workload(N=64), w.avg_pool2d_bf16_workload(N=3, H=5, W=4, C=7, weight=1.0, clamp=(-1.0, 1.0)),

@@ -36,6 +36,7 @@ struct Tuning {
     long long depthwiseTileMin = 0; // THIP_DEPTHWISE_TILE_MIN: thread-outputs from which the tile kernel is taken
     int depthwisePixels = 0;        // THIP_DEPTHWISE_P: pixels per thread of the window-row kernel
     int fcWideU = 0;                // THIP_FC_WIDE_U: k-steps per register buffer of the wide bf16 kernel
+    int fcWideWaves = 0;            // THIP_FC_WIDE_WAVES=4 / 8 / 16: waves per block of the wide bf16 kernel (0: by weight format and rows)
     bool noFcDeep = false;          // THIP_NO_FC_DEEP
     bool noFcWide = false;          // THIP_NO_FC_WIDE
     bool addGeneric = false;        // THIP_ADD_GENERIC: the quantised add always through the 64-bit ACT stage

@@ -3201,8 +3201,8 @@ __global__ __launch_bounds__(256) void fc_bf16_reduce(FcBf16Args p) {
 // 16 bytes per lane right before each MFMA: with few rows that is a few KiB, and registers set the occupancy.
 // Weights in fragment order only (layouts 1 and 2).
 constexpr int kFcBf16WideMaxSteps = 24;  // 99 KiB of LDS for 32 input rows
-template <int Q8, int U>  // U: k-steps per register buffer
-__global__ __launch_bounds__(256) void fc_bf16_wide(FcBf16Args p, FastDiv qblk) {
+template <int Q8, int U, int W = 4>  // U: k-steps per register buffer; W: waves per block (they share the block's input rows in LDS)
+__global__ __launch_bounds__(64 * W) void fc_bf16_wide(FcBf16Args p, FastDiv qblk) {
     extern __shared__ __attribute__((aligned(16))) int8_t xs[];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int r = lane & 31, h = lane >> 5;
@@ -3210,7 +3210,7 @@ __global__ __launch_bounds__(256) void fc_bf16_wide(FcBf16Args p, FastDiv qblk) 
     const int m0 = blockIdx.y * 32;
     // rows the block really has, plus one slot of zeros that the lanes of the missing rows all read
     const int mt = p.M - m0 < 32 ? p.M - m0 : 32, slots = 2 * (mt + 1);
-    for (int i = threadIdx.x; i < steps * 4 * slots; i += 256) {
+    for (int i = threadIdx.x; i < steps * 4 * slots; i += 64 * W) {
         const int slot = i % slots, sc = i / slots, c = sc & 3, s = sc >> 2;
         const int hh = slot / (mt + 1), rr = slot - hh * (mt + 1);
         const int k = s * 64 + 32 * hh + 8 * c;
@@ -3220,7 +3220,7 @@ __global__ __launch_bounds__(256) void fc_bf16_wide(FcBf16Args p, FastDiv qblk) 
     }
     __syncthreads();
     const int xslot = (h * (mt + 1) + (r < mt ? r : mt)) * 16;
-    const int nb = blockIdx.x * 4 + wave;
+    const int nb = blockIdx.x * W + wave;
     if (nb >= (p.N + 31) / 32) return;
     const int n0 = nb * 32;
     constexpr int PIECES = Q8 ? 2 : 4;  // 16-byte loads per lane per step
@@ -3281,18 +3281,34 @@ __global__ __launch_bounds__(256) void fc_bf16_wide(FcBf16Args p, FastDiv qblk) 
     fcBf16Store(p, acc, m0, n0, r, h);
 }
 
-template <int Q8, int U>
-static hipError_t launchFcBf16WideU(const FcBf16Args &a, FastDiv blk, const LaunchCtx &ctx) {
-    auto kernel = fc_bf16_wide<Q8, U>;
+template <int Q8, int U, int W>
+static hipError_t launchFcBf16WideUW(const FcBf16Args &a, FastDiv blk, const LaunchCtx &ctx) {
+    auto kernel = fc_bf16_wide<Q8, U, W>;
     static std::once_flag once;
     static hipError_t configured = hipSuccess;
     std::call_once(once, [&] { configured = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, kFcBf16WideMaxSteps * 4 * 66 * 16); });
     if (configured != hipSuccess) return configured;
     const int steps = (a.K + 63) / 64, nblocks = (a.N + 31) / 32;
-    const dim3 grid((unsigned)((nblocks + 3) / 4), (unsigned)((a.M + 31) / 32));
+    const dim3 grid((unsigned)((nblocks + W - 1) / W), (unsigned)((a.M + 31) / 32));
     const int mt = a.M < 32 ? a.M : 32;
-    THIP_ENQUEUE(ctx, kernelLabel("fc_bf16_wide", {Q8, U}), kernel, grid, dim3(256), (size_t)steps * 4 * 2 * (mt + 1) * 16, a, blk);
+    THIP_ENQUEUE(ctx, kernelLabel("fc_bf16_wide", {Q8, U, W}), kernel, grid, dim3(64 * W), (size_t)steps * 4 * 2 * (mt + 1) * 16, a, blk);
     return hipGetLastError();
+}
+
+template <int Q8, int U>
+static hipError_t launchFcBf16WideU(const FcBf16Args &a, FastDiv blk, const LaunchCtx &ctx) {
+    // Waves per block: they share one copy of the block's input rows in LDS (up to 99 KiB, read from L2 once per block),
+    // so more waves mean fewer copies and more waves per CU.  Measured at K = 1152, N = 65536, 1 / 32 / 64 rows, in us:
+    // bf16 weights 26.3 / 34.4 / 64.8 with four waves, 26.0 / 30.3 / 53.0 with eight, 26.6 / 29.3 / 30.2 with sixteen;
+    // block-scaled int8 weights 19.7 / 27.6 / 50.4, 19.4 / 23.5 / 34.3 and 23.9 / 26.2 / 28.6 (one block of sixteen
+    // waves per CU: its prologue overlaps with nothing).  THIP_FC_WIDE_WAVES forces a count.
+    constexpr bool fitsSixteen = U <= (Q8 ? 4 : 2);  // beyond that 128 registers per lane are not enough
+    int waves = ctx.tuning->fcWideWaves;
+    if (waves != 4 && waves != 8 && waves != 16) waves = (!Q8 || a.M > 32) ? 16 : 8;
+    if constexpr (fitsSixteen) {
+        if (waves == 16) return launchFcBf16WideUW<Q8, U, 16>(a, blk, ctx);
+    }
+    return waves == 4 ? launchFcBf16WideUW<Q8, U, 4>(a, blk, ctx) : launchFcBf16WideUW<Q8, U, 8>(a, blk, ctx);
 }
 
 template <int Q8>
@@ -3601,6 +3617,7 @@ Tuning tuningFromEnvironment() {
     if (const char *v = getenv("THIP_DEPTHWISE_TILE_MIN")) t.depthwiseTileMin = atoll(v);
     if (const char *v = getenv("THIP_DEPTHWISE_P")) t.depthwisePixels = atoi(v);
     if (const char *v = getenv("THIP_FC_WIDE_U")) t.fcWideU = atoi(v);
+    if (const char *v = getenv("THIP_FC_WIDE_WAVES")) t.fcWideWaves = atoi(v);
     t.noFcDeep = flag("THIP_NO_FC_DEEP");
     t.noFcWide = flag("THIP_NO_FC_WIDE");
     t.maxpoolGeneric = flag("THIP_MAXPOOL_GENERIC");
