@@ -474,7 +474,7 @@ class Emitter {
 
     // Tile of the ring kernel with window addressing: one tile column for few output channels (the image is read
     // once), else the largest tile that still gives every CU a tile, two blocks per CU where there are many.
-    static uint32_t chooseWindowVariant(int64_t M, int64_t N, int64_t C) {
+    static uint32_t chooseWindowVariant(int64_t M, int64_t N, int64_t C, int64_t K) {
         if (const char *env = getenv("THIP_WINDOW_VARIANT"); env && *env) {
             const long v = strtol(env, nullptr, 10);
             if (v == kIgemmDense256x256 || v == kIgemmDense128x256 || v == kIgemmDense128x128 || v == kIgemmDense256x128 || v == kIgemmDense256x64 || v == kIgemmDense64x64) return (uint32_t)v;
@@ -503,7 +503,9 @@ class Emitter {
         if (N <= 128 && tiles(kIgemmDense256x128) >= 224) return kIgemmDense256x128;
         // measured on 3x3 convolutions of 64 .. 512 channels at batch 1 .. 64: the largest tile wins as soon as half the CUs
         // get one (a long K per tile amortises its prologue and epilogue), unless it pads N by more than an eighth
-        if (tiles(kIgemmDense256x256) >= 128 && !wasteful(kIgemmDense256x256)) {
+        // (a short K leaves the largest tile mostly prologue and epilogue, as in the dense choice: 64 -> 256 at 56 x 56,
+        // batch 32, K = 576: 24.7 us on 128 x 256 against 27.5)
+        if (K > 640 && tiles(kIgemmDense256x256) >= 128 && !wasteful(kIgemmDense256x256)) {
             return (C % 128 == 0 && !getenv("THIP_NO_K128")) ? kIgemmDense256x256K128 : kIgemmDense256x256;
         }
         if (tiles(kIgemmDense128x256) >= 128 && !wasteful(kIgemmDense128x256)) return kIgemmDense128x256;
@@ -515,7 +517,7 @@ class Emitter {
     template <typename WeightAt>
     void emitIgemm(DescOp base, int64_t M, int64_t N, int64_t K, uint32_t loader, WeightAt wAt) {
         const bool dense = loader == kLoaderDense;
-        const uint32_t variant = loader == kLoaderWindow ? chooseWindowVariant(M, N, base.C)
+        const uint32_t variant = loader == kLoaderWindow ? chooseWindowVariant(M, N, base.C, K)
                                                          : chooseIgemmVariant(M, N, dense, K, base.out_dtype, loader == kLoaderRuns, addFollows_);
         const IgemmTile &t = igemmTile(variant);
         const int64_t Kp = roundUp(K, t.bk), Np = roundUp(N, t.bn);
