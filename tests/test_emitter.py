@@ -109,8 +109,8 @@ def test_dense_k128_records(monkeypatch):
 
 def test_conv2d_window_loader_records():
     """A multiple of 16 channels: the record asks for the ring kernel's window addressing (loader 3, a page of
-    zero-point bytes as its table, K rounded up to whole k-tiles); other channel counts, few output channels or the
-    switch keep the gather loader."""
+    zero-point bytes as its table, K rounded up to whole k-tiles); other channel counts or the switch keep the gather
+    loader."""
     import os
     for kw in WINDOW_RING:
         wl = w.conv2d_workload(realistic=True, **kw)
@@ -119,12 +119,13 @@ def test_conv2d_window_loader_records():
         assert [(int(o["kind"]), int(o["loader"])) for o in d.ops] == [(desc_interp.K_IGEMM, 3)], wl.name
         bk = 128 if int(d.ops[0]["variant"]) == 14 else 64
         assert int(d.ops[0]["Kp"]) == -(-int(d.ops[0]["K"]) // bk) * bk
-    for kw in (dict(N=2, H=32, W=32, C=72, O=64), dict(N=2, H=32, W=32, C=40, O=64), dict(N=2, H=32, W=32, C=64, O=16)):
+    for kw in (dict(N=2, H=32, W=32, C=72, O=64), dict(N=2, H=32, W=32, C=40, O=64)):
         d = interp(w.conv2d_workload(realistic=True, **kw))[1]
         assert int(d.ops[0]["loader"]) == 1, kw
     # small convolutions take the 64 x 64 tile (up to 512 of them)
     for kw, variant in ((dict(N=1, H=32, W=32, C=64, O=64), 7), (dict(N=1, H=7, W=7, C=160, O=160), 7), (dict(N=1, H=28, W=28, C=32, O=32), 7),
-                        (dict(N=16, H=14, W=14, C=512, O=512), 7), (dict(N=32, H=14, W=14, C=512, O=512), 5)):
+                        (dict(N=16, H=14, W=14, C=512, O=512), 7), (dict(N=32, H=14, W=14, C=512, O=512), 5),
+                        (dict(N=2, H=32, W=32, C=64, O=16), 7), (dict(N=1, H=28, W=28, C=64, O=8), 7), (dict(N=48, H=32, W=32, C=16, O=24), 9)):
         wl = w.conv2d_workload(realistic=True, **kw)
         outs, d = interp(wl)
         assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)

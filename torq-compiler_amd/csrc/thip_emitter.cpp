@@ -747,10 +747,12 @@ thip_status_t Emitter::emitConv2d(const thip_hl_conv2d_t &c) {
         // a window over a multiple of 16 channels: the LDS-DMA ring kernel addresses the window itself, at every size
         // (256 -> 256 at 14 x 14, one image: 10.3 us against 15.3 on the gather kernel; 32 -> 32 at 28 x 28: 4.3
         // against 4.8; 96 -> 96 at 56 x 56, batch 32: 17.3 against 29.4).  THIP_NO_WINDOW_RING keeps such convolutions
-        // on the gather kernel; THIP_RING_MIN_C and THIP_RING_MIN_M raise the channel and pixel counts from which the
-        // ring kernel is taken (tests and tuning).
-        const char *minC = getenv("THIP_RING_MIN_C"), *minM = getenv("THIP_RING_MIN_M");
-        const bool ring = !pointwise && Cin % 16 == 0 && Cin >= (minC && *minC ? atoi(minC) : 16) && M >= (minM && *minM ? atoi(minM) : 1) && Oout >= 32 &&
+        // on the gather kernel; THIP_RING_MIN_C, THIP_RING_MIN_M and THIP_RING_MIN_O raise the input channel, pixel and
+        // output channel counts from which the ring kernel is taken (tests and tuning).  Few output channels pay as
+        // well, padded to a 64-wide tile as on the gather kernel (16 -> 16 at 32 x 32: 3.6 us against 4.2, batch 128: 6.5
+        // against 9.8; 32 -> 16 at 112 x 112, batch 32: 22.3 against 28.9).
+        const char *minC = getenv("THIP_RING_MIN_C"), *minM = getenv("THIP_RING_MIN_M"), *minO = getenv("THIP_RING_MIN_O");
+        const bool ring = !pointwise && Cin % 16 == 0 && Cin >= (minC && *minC ? atoi(minC) : 16) && M >= (minM && *minM ? atoi(minM) : 1) && Oout >= (minO && *minO ? atoi(minO) : 1) &&
                           d.N * d.H * d.W * Cin < (1LL << 32) && !getenv("THIP_NO_WINDOW_RING");
         emitIgemm(op, M, Oout, K, (pointwise && K % 16 == 0) ? kLoaderDense : ring ? kLoaderWindow : kLoaderGather, [&](int64_t n, int64_t k) -> int8_t {
             const int64_t pos = k / Cin, ci = k % Cin;
