@@ -129,7 +129,7 @@ def run(blob, binding_arrays):
                 Nimg, H, W, C = (int(op[k]) for k in ["N", "H", "W", "C"])
                 OH, OW, SH, SW, PT, PL, KH, KW = (int(op[k]) for k in ["OH", "OW", "SH", "SW", "PT", "PL", "KH", "KW"])
                 bk = 128 if int(op["variant"]) == 14 else 64
-                assert int(op["variant"]) in (4, 5, 6, 7, 8, 9, 14)
+                assert int(op["variant"]) in (4, 5, 6, 7, 8, 9, 10, 14)
                 assert C % 16 == 0 and K == KH * KW * C and Kp == -(-K // bk) * bk
                 page = view(op["table"], 128).view(np.int8)
                 assert (page == int(op["input_zp"])).all()

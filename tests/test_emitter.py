@@ -125,7 +125,7 @@ def test_conv2d_window_loader_records():
     # small convolutions take the 64 x 64 tile (up to 512 of them)
     for kw, variant in ((dict(N=1, H=32, W=32, C=64, O=64), 7), (dict(N=1, H=7, W=7, C=160, O=160), 7), (dict(N=1, H=28, W=28, C=32, O=32), 7),
                         (dict(N=16, H=14, W=14, C=512, O=512), 7), (dict(N=32, H=14, W=14, C=512, O=512), 5),
-                        (dict(N=2, H=32, W=32, C=64, O=16), 7), (dict(N=1, H=28, W=28, C=64, O=8), 7), (dict(N=48, H=32, W=32, C=16, O=24), 9)):
+                        (dict(N=2, H=32, W=32, C=64, O=16), 7), (dict(N=1, H=28, W=28, C=64, O=8), 7), (dict(N=48, H=32, W=32, C=16, O=24), 10), (dict(N=48, H=32, W=32, C=16, O=40), 9)):
         wl = w.conv2d_workload(realistic=True, **kw)
         outs, d = interp(wl)
         assert_bit_exact(outs[0], oracle_eval(wl)[0], wl.name)

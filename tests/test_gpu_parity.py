@@ -77,11 +77,11 @@ def test_conv2d_window_ring(device, kw):
     assert "igemm_dense_conv_i8" in families(k), k
 
 
-@pytest.mark.parametrize("variant", [4, 5, 6, 7, 8, 9])
+@pytest.mark.parametrize("variant", [4, 5, 6, 7, 8, 9, 10])
 def test_conv2d_window_ring_every_tile(device, variant, monkeypatch):
     monkeypatch.setenv("THIP_WINDOW_VARIANT", str(variant))
     names = {4: "igemm_dense_conv_i8<256,256,", 5: "igemm_dense_conv_i8<128,128,", 6: "igemm_dense_conv_i8<128,256,", 7: "igemm_dense_conv_i8<64,64,",
-             8: "igemm_dense_conv_i8<256,128,", 9: "igemm_dense_conv_i8<256,64,"}
+             8: "igemm_dense_conv_i8<256,128,", 9: "igemm_dense_conv_i8<256,64,", 10: "igemm_dense_conv_i8<256,32,"}
     for kw in (dict(N=2, H=33, W=35, C=64, O=80, pad=(1, 1, 1, 1)), dict(N=5, H=47, W=45, C=128, O=48, stride=(2, 2), pad=(1, 0, 1, 0), output_zp=-7, output_min=-128),
                dict(N=3, H=29, W=31, C=80, O=72, pad=(1, 1, 1, 1), input_zp=-90), dict(N=4, H=40, W=33, C=176, O=130, KH=2, KW=2, stride=(1, 2), pad=(0, 1, 1, 0))):
         k = check(device, w.conv2d_workload(realistic=True, **kw), via="device")

@@ -477,7 +477,7 @@ class Emitter {
     static uint32_t chooseWindowVariant(int64_t M, int64_t N, int64_t C, int64_t K) {
         if (const char *env = getenv("THIP_WINDOW_VARIANT"); env && *env) {
             const long v = strtol(env, nullptr, 10);
-            if (v == kIgemmDense256x256 || v == kIgemmDense128x256 || v == kIgemmDense128x128 || v == kIgemmDense256x128 || v == kIgemmDense256x64 || v == kIgemmDense64x64) return (uint32_t)v;
+            if (v == kIgemmDense256x256 || v == kIgemmDense128x256 || v == kIgemmDense128x128 || v == kIgemmDense256x128 || v == kIgemmDense256x64 || v == kIgemmDense64x64 || v == kIgemmDense256x32) return (uint32_t)v;
             if (v == kIgemmDense256x256K128) return (uint32_t)v;
         }
         auto tiles = [&](uint32_t v) {
@@ -499,7 +499,8 @@ class Emitter {
         // 3 / 4: 6.2 / 7.2 us on 588 / 784 small tiles, 6.5 / 6.6 on one column of 256 x 64, 7.0 / 7.1 on 128 x 128); up
         // to 128 take theirs with a tile per CU, below that the 128 x 128 tile wins (128 -> 128 at 28 x 28, batch 8: 8.5 us
         // against 12.4)
-        if (N <= 64) return tiles(kIgemmDense64x64) <= 640 ? kIgemmDense64x64 : kIgemmDense256x64;
+        // (and at most 32 take the 32-wide column: 32 -> 16 at 112 x 112, batch 32: 19.2 us against 22.4)
+        if (N <= 64) return tiles(kIgemmDense64x64) <= 640 ? kIgemmDense64x64 : N <= 32 ? kIgemmDense256x32 : kIgemmDense256x64;
         if (N <= 128 && tiles(kIgemmDense256x128) >= 224) return kIgemmDense256x128;
         // measured on 3x3 convolutions of 64 .. 512 channels at batch 1 .. 64: the largest tile wins as soon as half the CUs
         // get one (a long K per tile amortises its prologue and epilogue), unless it pads N by more than an eighth

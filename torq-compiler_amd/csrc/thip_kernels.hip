@@ -1616,6 +1616,7 @@ hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, const LaunchCtx &ct
         case kIgemmDense256x128: return launchIgemmDense<256, 128, 2, 2, 3, 2, true>(a, ctx);
         case kIgemmDense256x64: return launchIgemmDense<256, 64, 4, 1, 3, 2, true>(a, ctx);
         case kIgemmDense64x64: return launchIgemmDense<64, 64, 2, 2, 4, 4, true>(a, ctx);  // four stages: measured against three and five
+        case kIgemmDense256x32: return launchIgemmDense<256, 32, 4, 1, 3, 2, true>(a, ctx);
         case kIgemmDense256x256K128: return launchIgemmDense<256, 256, 2, 2, 2, 1, true, 128>(a, ctx);  // 128 channels per k-tile
         default: return hipErrorInvalidValue;
         }

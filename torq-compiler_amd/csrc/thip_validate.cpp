@@ -189,7 +189,7 @@ thip_status_t checkOpFootprint(const DescriptorView *e, uint32_t i) {
             }
             if (inBytes >= (1ull << 32)) return fail(THIP_INVALID_ARGUMENT, "op %u: image too large for the window loader", i);
             switch (op.variant) {
-            case kIgemmDense256x256: case kIgemmDense128x256: case kIgemmDense128x128: case kIgemmDense256x128: case kIgemmDense256x64: case kIgemmDense64x64: case kIgemmDense256x256K128: break;
+            case kIgemmDense256x256: case kIgemmDense128x256: case kIgemmDense128x128: case kIgemmDense256x128: case kIgemmDense256x64: case kIgemmDense64x64: case kIgemmDense256x32: case kIgemmDense256x256K128: break;
             default: return fail(THIP_INVALID_ARGUMENT, "op %u: the window loader has no kernel for tile variant %u", i, op.variant);
             }
             if (op.table.space != kSpaceConst) return fail(THIP_INVALID_ARGUMENT, "op %u: table must be a constant", i);
