@@ -155,6 +155,26 @@ def test_dense_igemm_every_tile_variant(device, variant, monkeypatch):
     check(device, w.conv2d_workload(N=2, H=28, W=28, C=192, O=32, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True))
 
 
+def test_dense_igemm_short_k(device, monkeypatch):
+    """Up to six k-tiles over at least two 128 x 128 tiles per CU: two ring stages, four blocks per CU (K of one to six
+    k-tiles, ragged M / N / K, every epilogue); fewer tiles or a longer K keep the deeper ring."""
+    for K in (16, 64, 100 // 4 * 4 + 12, 192, 256, 320, 384):
+        k = check(device, w.fully_connected_workload(16500, K, 512, realistic=True), via="device")
+        assert k[0] == "igemm_dense_i8<128,128,2,2,2,4,1,0>", (K, k)
+    k = check(device, w.fully_connected_workload(16500, 256, 512))                      # the literal requant range
+    assert k[0] == "igemm_dense_i8<128,128,2,2,2,4,2,0>", k
+    monkeypatch.setenv("THIP_IGEMM_DENSE_VARIANT", "5")
+    k = check(device, w.fully_connected_workload(16390, 208, 520, realistic=True))      # N % 16 != 0: staged epilogue
+    assert k[0] == "igemm_dense_i8<128,128,2,2,2,4,0,0>", k
+    k = check(device, w.fully_connected_workload(16390, 448, 512, realistic=True))      # seven k-tiles
+    assert k[0] == "igemm_dense_i8<128,128,2,2,4,2,1,0>", k
+    k = check(device, w.fully_connected_workload(8000, 256, 512, realistic=True))       # 252 tiles
+    assert k[0] == "igemm_dense_i8<128,128,2,2,4,2,1,0>", k
+    monkeypatch.setenv("THIP_DENSE_SHORT_K", "0")
+    k = check(device, w.fully_connected_workload(16500, 256, 512, realistic=True))
+    assert k[0] == "igemm_dense_i8<128,128,2,2,4,2,1,0>", k
+
+
 def test_dense_igemm_k128(device, monkeypatch):
     """k-tiles of 128 bytes (whole cache lines per tile row, four MFMA phases, two ring stages): taken by itself for a
     long K with enough tiles, forced here on ragged M / N, K tails that end inside a k-tile (at every 16-byte chunk),

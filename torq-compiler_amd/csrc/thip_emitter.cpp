@@ -429,7 +429,8 @@ class Emitter {
             // those sizes a dense tile is 10-50 % faster.
             if (M >= 4096 && igemmStreamFits(N, K, outDtype) && !getenv("THIP_NO_STREAM")) {
                 const bool expanding = N >= 2 * K;
-                const bool take = K <= 128 ? (M >= 200000 || (expanding && M >= 40000))
+                const char *em = getenv("THIP_STREAM_EXPAND_MIN_M");  // tuning: the pixel count from which an expanding layer streams
+                const bool take = K <= 128 ? (M >= 200000 || (expanding && M >= (em ? atoll(em) : 40000)))
                                            : ((expanding && M >= 25000 && M * N < (1LL << 28)) || (addFollows && M >= 400000));
                 if (take) return kIgemmStream;
             }
@@ -439,6 +440,14 @@ class Emitter {
             // activations are streamed once (these shapes are bandwidth-bound, padded MFMA work is free)
             if (N <= 128 && M >= 16384) {
                 return N <= 32 ? kIgemmDense256x32 : N <= 64 ? kIgemmDense256x64 : kIgemmDense256x128;
+            }
+            // a short K (up to six k-tiles) over at least two tiles per CU: the 128 x 128 tile, which the launcher then runs
+            // two stages deep with four blocks per CU, so that the prologues and epilogues that dominate such tiles
+            // overlap (256 -> 1024 channels at 56 x 56, batch 8: 13.5 us against 16.2 on 128 x 256; 64 -> 256 over 100 352
+            // pixels: 10.4 against 12.0; from 400 000 pixels x 960 channels the wider tile is 3 % ahead again)
+            const bool shortK = K > 0 && ((K <= 256 && M * N < (1LL << 28) && M < 600000) || (K <= 384 && M < 65536));
+            if (shortK && N > 128 && tiles(kIgemmDense128x128) >= 512 && (roundUp(N, 128) - N) * 8 <= N && !getenv("THIP_NO_SHORTK_TILE")) {
+                return kIgemmDense128x128;
             }
             // a long K on the largest tile: k-tiles of 128 bytes, whole cache lines per row (THIP_NO_K128 keeps 64)
             if (K >= 1024 && tiles(kIgemmDense256x256) >= 224 && !getenv("THIP_NO_K128")) return kIgemmDense256x256K128;
