@@ -144,16 +144,16 @@ class Loaded:
 # (KiB per dispatch; the factors are what the same counters read for a plain 256 MiB copy, --copy-calibration).
 # They belong to the kernels as they were when the counters were read: TRAFFIC_KERNELS_SHA256 is the hash of
 # torq-compiler_amd/csrc/thip_kernels.hip at that time, and a run on other kernel sources reports traffic null.
-TRAFFIC_KERNELS_SHA256 = "9cb10d3054d24f3372e6f0504791071531a333473fe8e5f1eedaa8e9aca5e12d"
+TRAFFIC_KERNELS_SHA256 = "14708ffe8581b1b77a10368c380d7e1826282843df2c54729aac89b2a054379e"
 MEASURED_TRAFFIC = {
-    "fc_4096x4096x4096": (49385.0 * 1.9995 + 16604.4 * 1.0000) * 1024,
+    "fc_4096x4096x4096": (49387.5 * 1.9995 + 16576.9 * 1.0000) * 1024,
     "fc_512x4096x4096": (16446.0 * 1.9995 + 2048.0 * 1.0000) * 1024,
     "fc_16x2048x8192": (8408.0 * 1.9995 + 256.0 * 1.0000) * 1024,
-    "conv_112x112x32_o64_3x3": (369.7 * 1.9995 + 784.0 * 1.0000) * 1024,
-    "conv3x3_56x56x256_o256_b32": (17251.6 * 1.9995 + 26008.1 * 1.0000) * 1024,
-    "depthwise_b64": (15446.7 * 1.9995 + 7063.2 * 1.0000) * 1024,
-    "depthwise_s1_b256": (63712.4 * 1.9995 + 113183.0 * 1.0000) * 1024,
-    "maxpool_b64": (25151.2 * 1.9995 + 12544.0 * 1.0000) * 1024,
+    "conv_112x112x32_o64_3x3": (365.7 * 1.9995 + 784.0 * 1.0000) * 1024,
+    "conv3x3_56x56x256_o256_b32": (17257.9 * 1.9995 + 26010.3 * 1.0000) * 1024,
+    "depthwise_b64": (15436.1 * 1.9995 + 7063.3 * 1.0000) * 1024,
+    "depthwise_s1_b256": (63691.2 * 1.9995 + 113179.2 * 1.0000) * 1024,
+    "maxpool_b64": (25121.0 * 1.9995 + 12544.0 * 1.0000) * 1024,
     "avgpool_b64": (2001.0 * 1.9995 + 80.0 * 1.0000) * 1024,
     "add_b64": (4723.0 * 1.9995 + 4704.0 * 1.0000) * 1024,
 }
