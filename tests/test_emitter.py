@@ -107,6 +107,19 @@ def test_dense_k128_records(monkeypatch):
         assert int(d.ops[0]["variant"]) == 14 and int(d.ops[0]["Kp"]) % 128 == 0
 
 
+def test_dense_tile_choice_by_rounds_of_tiles():
+    """K of 513 .. 1024 and more than a tenth of the last round of 256 x 256 tiles idle: two half-size blocks per CU."""
+    def variant(M, K, N):
+        wl = w.fully_connected_workload(M, K, N, realistic=True, zeros=True)
+        return int(desc_interp.Descriptor(wl.program.serialize()).ops[0]["variant"])
+    assert variant(100352, 768, 512) == 6      # 784 tiles: 3.06 rounds
+    assert variant(100352, 1024, 512) == 6
+    assert variant(100352, 1536, 512) == 14    # a long K: 128-byte k-tiles on the largest tile
+    assert variant(4096, 768, 4096) == 4       # 256 tiles: one full round
+    assert variant(6000, 1024, 4096) == 14     # 384 tiles, K = 1024: no gain measured
+    assert variant(6000, 896, 4096) == 6
+
+
 def test_conv2d_window_loader_records():
     """A multiple of 16 channels: the record asks for the ring kernel's window addressing (loader 3, a page of
     zero-point bytes as its table, K rounded up to whole k-tiles); other channel counts or the switch keep the gather

@@ -450,7 +450,14 @@ class Emitter {
                 return kIgemmDense128x128;
             }
             // a long K on the largest tile: k-tiles of 128 bytes, whole cache lines per row (THIP_NO_K128 keeps 64)
-            if (K >= 1024 && tiles(kIgemmDense256x256) >= 224 && !getenv("THIP_NO_K128")) return kIgemmDense256x256K128;
+            // (one block per CU pays for a mostly empty last round of tiles in full, two half-size blocks per CU run
+            // it at nearly twice the speed: with K of 513 .. 1024 and more than a tenth of the last round idle the
+            // largest tile is skipped - 100 352 x 768 x 512, 784 tiles: 56.3 us on 128 x 256 against 74.7; K = 1024: 69.3
+            // against 80.4; with 392 tiles and K = 1024 both take 39 us, and from K = 1536 the 128-byte k-tiles win)
+            const int64_t t256 = tiles(kIgemmDense256x256), rounds256 = (t256 + 255) / 256;
+            const bool idleLastRound = (rounds256 * 256 - t256) * 10 > rounds256 * 256;
+            const bool skipLargest = K > 512 && K <= 1024 && idleLastRound && (K < 1024 || t256 >= 512) && !getenv("THIP_NO_ROUND_RULE");
+            if (K >= 1024 && tiles(kIgemmDense256x256) >= 224 && !skipLargest && !getenv("THIP_NO_K128")) return kIgemmDense256x256K128;
             // otherwise the largest tile that still gives (nearly) every CU a tile and does not pad N by more than an
             // eighth where a narrower tile that fills the chip would not (padded columns are computed too)
             const uint32_t order[] = {kIgemmDense256x256, kIgemmDense128x256, kIgemmDense128x128, kIgemmDense64x128, kIgemmDense128x64};
@@ -460,7 +467,7 @@ class Emitter {
                 const uint32_t v = order[i];
                 // a short K leaves a 256 x 256 tile (one block per CU) mostly prologue and epilogue; two blocks per CU
                 // of half the size overlap them (256 -> 1024 channels at 56 x 56, batch 32: 75 -> 54 us)
-                if (v == kIgemmDense256x256 && K > 0 && K <= 512) continue;
+                if (v == kIgemmDense256x256 && K > 0 && (K <= 512 || skipLargest)) continue;
                 if (v == kIgemmDense64x128 && (wasteful(v) || getenv("THIP_NO_64X128"))) continue;
                 if (!enough(v)) continue;
                 bool better = false;
