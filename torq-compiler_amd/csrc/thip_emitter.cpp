@@ -522,7 +522,11 @@ class Emitter {
         // get one (a long K per tile amortises its prologue and epilogue), unless it pads N by more than an eighth
         // (a short K leaves the largest tile mostly prologue and epilogue, as in the dense choice: 64 -> 256 at 56 x 56,
         // batch 32, K = 576: 24.7 us on 128 x 256 against 27.5)
-        if (K > 640 && tiles(kIgemmDense256x256) >= 128 && !wasteful(kIgemmDense256x256)) {
+        // (and, as there, up to K = 1024 a mostly idle last round of the largest tiles costs more than two half-size
+        // blocks per CU: 112 -> 512 at 56 x 56, batch 32, K = 1008, 3.06 rounds: 68.1 us against 80.1)
+        const int64_t t256 = tiles(kIgemmDense256x256), rounds256 = (t256 + 255) / 256;
+        const bool idleLastRound = (rounds256 * 256 - t256) * 10 > rounds256 * 256 && !getenv("THIP_NO_ROUND_RULE");
+        if (K > 640 && !(K <= 1024 && idleLastRound) && tiles(kIgemmDense256x256) >= 128 && !wasteful(kIgemmDense256x256)) {
             return (C % 128 == 0 && !getenv("THIP_NO_K128")) ? kIgemmDense256x256K128 : kIgemmDense256x256;
         }
         if (tiles(kIgemmDense128x256) >= 128 && !wasteful(kIgemmDense128x256)) return kIgemmDense128x256;
