@@ -115,7 +115,8 @@ def test_dense_tile_choice_by_rounds_of_tiles():
     assert variant(100352, 768, 512) == 6      # 784 tiles: 3.06 rounds
     assert variant(100352, 1024, 512) == 6
     assert variant(100352, 1536, 512) == 14    # a long K: 128-byte k-tiles on the largest tile
-    assert variant(4096, 768, 4096) == 4       # 256 tiles: one full round
+    assert variant(4096, 768, 4096) == 14      # 256 tiles, one full round: the largest tile, 128-byte k-tiles from K = 576
+    assert variant(4096, 528, 4096) == 4       # K would be padded by a quarter: 64-byte k-tiles
     assert variant(6000, 1024, 4096) == 14     # 384 tiles, K = 1024: no gain measured
     assert variant(6000, 896, 4096) == 6
 

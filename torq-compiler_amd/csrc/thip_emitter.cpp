@@ -457,7 +457,9 @@ class Emitter {
             const int64_t t256 = tiles(kIgemmDense256x256), rounds256 = (t256 + 255) / 256;
             const bool idleLastRound = (rounds256 * 256 - t256) * 10 > rounds256 * 256;
             const bool skipLargest = K > 512 && K <= 1024 && idleLastRound && (K < 1024 || t256 >= 512) && !getenv("THIP_NO_ROUND_RULE");
-            if (K >= 1024 && tiles(kIgemmDense256x256) >= 224 && !skipLargest && !getenv("THIP_NO_K128")) return kIgemmDense256x256K128;
+            // (the 128-byte k-tiles are ahead from K = 576 on, padded to whole k-tiles: 8192 x 640 x 4096 32.7 us against
+            // 36.8, 16384 x 768 x 4096 71.3 against 78.7, 4096 x 960 x 4096 23.0 against 23.4)
+            if (K > 512 && (roundUp(K, 128) - K) * 8 <= K && tiles(kIgemmDense256x256) >= 224 && !skipLargest && !getenv("THIP_NO_K128")) return kIgemmDense256x256K128;
             // otherwise the largest tile that still gives (nearly) every CU a tile and does not pad N by more than an
             // eighth where a narrower tile that fills the chip would not (padded columns are computed too)
             const uint32_t order[] = {kIgemmDense256x256, kIgemmDense128x256, kIgemmDense128x128, kIgemmDense64x128, kIgemmDense128x64};
