@@ -155,6 +155,24 @@ def test_dense_igemm_every_tile_variant(device, variant, monkeypatch):
     check(device, w.conv2d_workload(N=2, H=28, W=28, C=192, O=32, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True))
 
 
+def test_dense_igemm_64x128_long_k(device, monkeypatch):
+    """The 64 x 128 tile with a long K in whole 128-byte k-tiles: ragged M and N, every epilogue; other K keep 64 bytes."""
+    k = check(device, w.fully_connected_workload(512, 4096, 4096, realistic=True), via="device")
+    assert k[0] == "igemm_dense_k128_i8<64,128,2,2,3,2,1,0>", k                          # chosen without a switch
+    monkeypatch.setenv("THIP_IGEMM_DENSE_VARIANT", "13")
+    k = check(device, w.fully_connected_workload(500, 4096, 2064, realistic=True), via="device")
+    assert k[0] == "igemm_dense_k128_i8<64,128,2,2,3,2,1,0>", k
+    k = check(device, w.fully_connected_workload(500, 4224, 2064))                       # the literal requant range
+    assert k[0] == "igemm_dense_k128_i8<64,128,2,2,3,2,2,0>", k
+    k = check(device, w.fully_connected_workload(300, 4096, 2056, realistic=True))       # N % 16 != 0: staged epilogue
+    assert k[0] == "igemm_dense_k128_i8<64,128,2,2,3,2,0,0>", k
+    k = check(device, w.fully_connected_workload(500, 4160, 2064, realistic=True))       # K % 128 != 0
+    assert k[0] == "igemm_dense_i8<64,128,2,2,4,2,1,0>", k
+    monkeypatch.setenv("THIP_NO_K128", "1")
+    k = check(device, w.fully_connected_workload(500, 4096, 2064, realistic=True))
+    assert k[0] == "igemm_dense_i8<64,128,2,2,4,2,1,0>", k
+
+
 def test_dense_igemm_short_k(device, monkeypatch):
     """Up to six k-tiles over at least two 128 x 128 tiles per CU: two ring stages, four blocks per CU (K of one to six
     k-tiles, ragged M / N / K, every epilogue); fewer tiles or a longer K keep the deeper ring."""
@@ -297,7 +315,7 @@ def test_conv2d_int32_output(device):
 def test_fully_connected_config1(device, mkn):
     M = mkn[0]
     check(device, w.fully_connected_workload(*mkn, realistic=True), via="device",
-          kernel=("fc_skinny<1,4>" if M == 1 else "fc_skinny_mfma") if M <= 16 else ("igemm_dense_i8" if M >= 512 else None))
+          kernel=("fc_skinny<1,4>" if M == 1 else "fc_skinny_mfma") if M <= 16 else ("igemm_dense_k128_i8" if M >= 512 else None))
 
 
 def test_fully_connected_config1_literal_ranges(device):

@@ -38,6 +38,7 @@ struct Tuning {
     int fcWideU = 0;                // THIP_FC_WIDE_U: k-steps per register buffer of the wide bf16 kernel
     int fcWideWaves = 0;            // THIP_FC_WIDE_WAVES=4 / 8 / 16: waves per block of the wide bf16 kernel (0: by weight format and rows)
     int denseShortK = 384;          // THIP_DENSE_SHORT_K: padded K up to which the 128 x 128 dense tile runs two stages deep, four blocks per CU
+    bool noK128 = false;            // THIP_NO_K128: no 128-byte k-tiles chosen at launch (the emitter reads the same switch for its own choice)
     bool noFcDeep = false;          // THIP_NO_FC_DEEP
     bool noFcWide = false;          // THIP_NO_FC_WIDE
     bool addGeneric = false;        // THIP_ADD_GENERIC: the quantised add always through the 64-bit ACT stage

@@ -1648,7 +1648,12 @@ hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, const LaunchCtx &ct
     case kIgemmDense256x32: return launchIgemmDense<256, 32, 4, 1, 3, 2>(a, ctx);
     case kIgemmStream: return launchIgemmStream(a, ctx);
     case kIgemmDense128x64: return launchIgemmDense<128, 64, 2, 2, 4, 2>(a, ctx);
-    case kIgemmDense64x128: return launchIgemmDense<64, 128, 2, 2, 4, 2>(a, ctx);
+    case kIgemmDense64x128:
+        // a long K in whole 128-byte k-tiles: whole cache lines per tile row here as well, three stages deep
+        // (512 x 4096 x 4096: 12.8 us against 13.9, 256 x 4096 x 8192: 13.1 against 15.0; at K = 2048 the 64-byte
+        // k-tiles with four stages are ahead, 7.7 against 8.1)
+        if (a.Kp >= 4096 && a.Kp % 128 == 0 && !ctx.tuning->noK128) return launchIgemmDense<64, 128, 2, 2, 3, 2, false, 128>(a, ctx);
+        return launchIgemmDense<64, 128, 2, 2, 4, 2>(a, ctx);
     case kIgemmDense256x256K128: return launchIgemmDense<256, 256, 2, 2, 2, 1, false, 128>(a, ctx);
     default: return hipErrorInvalidValue;
     }
@@ -3625,6 +3630,7 @@ Tuning tuningFromEnvironment() {
     if (const char *v = getenv("THIP_FC_WIDE_U")) t.fcWideU = atoi(v);
     if (const char *v = getenv("THIP_FC_WIDE_WAVES")) t.fcWideWaves = atoi(v);
     if (const char *v = getenv("THIP_DENSE_SHORT_K")) t.denseShortK = atoi(v);
+    t.noK128 = flag("THIP_NO_K128");
     t.noFcDeep = flag("THIP_NO_FC_DEEP");
     t.noFcWide = flag("THIP_NO_FC_WIDE");
     t.maxpoolGeneric = flag("THIP_MAXPOOL_GENERIC");
