@@ -144,16 +144,16 @@ class Loaded:
 # (KiB per dispatch; the factors are what the same counters read for a plain 256 MiB copy, --copy-calibration).
 # They belong to the kernels as they were when the counters were read: TRAFFIC_KERNELS_SHA256 is the hash of
 # torq-compiler_amd/csrc/thip_kernels.hip at that time, and a run on other kernel sources reports traffic null.
-TRAFFIC_KERNELS_SHA256 = "14708ffe8581b1b77a10368c380d7e1826282843df2c54729aac89b2a054379e"
+TRAFFIC_KERNELS_SHA256 = "bed2729f1807b217227519131718d56a02bba90f10eabec2670110657f35a6be"
 MEASURED_TRAFFIC = {
-    "fc_4096x4096x4096": (49387.5 * 1.9995 + 16576.9 * 1.0000) * 1024,
-    "fc_512x4096x4096": (16446.0 * 1.9995 + 2048.0 * 1.0000) * 1024,
+    "fc_4096x4096x4096": (49387.5 * 1.9995 + 16579.9 * 1.0000) * 1024,
+    "fc_512x4096x4096": (16453.0 * 1.9995 + 2048.0 * 1.0000) * 1024,
     "fc_16x2048x8192": (8408.0 * 1.9995 + 256.0 * 1.0000) * 1024,
-    "conv_112x112x32_o64_3x3": (365.7 * 1.9995 + 784.0 * 1.0000) * 1024,
-    "conv3x3_56x56x256_o256_b32": (17257.9 * 1.9995 + 26010.3 * 1.0000) * 1024,
-    "depthwise_b64": (15436.1 * 1.9995 + 7063.3 * 1.0000) * 1024,
-    "depthwise_s1_b256": (63691.2 * 1.9995 + 113179.2 * 1.0000) * 1024,
-    "maxpool_b64": (25121.0 * 1.9995 + 12544.0 * 1.0000) * 1024,
+    "conv_112x112x32_o64_3x3": (370.7 * 1.9995 + 784.0 * 1.0000) * 1024,
+    "conv3x3_56x56x256_o256_b32": (17256.9 * 1.9995 + 26039.9 * 1.0000) * 1024,
+    "depthwise_b64": (15411.1 * 1.9995 + 7063.2 * 1.0000) * 1024,
+    "depthwise_s1_b256": (63696.5 * 1.9995 + 113145.4 * 1.0000) * 1024,
+    "maxpool_b64": (25113.5 * 1.9995 + 12544.0 * 1.0000) * 1024,
     "avgpool_b64": (2001.0 * 1.9995 + 80.0 * 1.0000) * 1024,
     "add_b64": (4723.0 * 1.9995 + 4704.0 * 1.0000) * 1024,
 }
