@@ -173,6 +173,26 @@ def test_dense_igemm_64x128_long_k(device, monkeypatch):
     assert k[0] == "igemm_dense_i8<64,128,2,2,4,2,1,0>", k
 
 
+def test_dense_igemm_128_wide_tiles_long_k(device, monkeypatch):
+    """The 128 x 128 and 128 x 256 tiles with a long K in whole 128-byte k-tiles: ragged M and N, every epilogue."""
+    k = check(device, w.fully_connected_workload(1500, 4096, 4096, realistic=True), via="device")
+    assert k[0] == "igemm_dense_k128_i8<128,128,2,2,2,2,1,0>", k                         # chosen without a switch
+    k = check(device, w.fully_connected_workload(1000, 4096, 4096, realistic=True), via="device")
+    assert k[0] == "igemm_dense_i8<128,128,2,2,4,2,1,0>", k                              # one tile per CU: the deeper ring
+    monkeypatch.setenv("THIP_IGEMM_DENSE_VARIANT", "5")
+    k = check(device, w.fully_connected_workload(1100, 4224, 4112))                      # the literal requant range
+    assert k[0] == "igemm_dense_k128_i8<128,128,2,2,2,2,2,0>", k
+    k = check(device, w.fully_connected_workload(1100, 4096, 4104, realistic=True))      # N % 16 != 0: staged epilogue
+    assert k[0] == "igemm_dense_k128_i8<128,128,2,2,2,2,0,0>", k
+    monkeypatch.setenv("THIP_IGEMM_DENSE_VARIANT", "6")
+    for wl, tail in ((w.fully_connected_workload(700, 4096, 2064, realistic=True), "1,0>"), (w.fully_connected_workload(700, 4224, 2064), "2,0>"),
+                     (w.fully_connected_workload(300, 4096, 2056, realistic=True), "0,0>")):
+        k = check(device, wl)
+        assert k[0] == "igemm_dense_k128_i8<128,256,2,2,2,1," + tail, k
+    k = check(device, w.fully_connected_workload(700, 4160, 2064, realistic=True))       # K % 128 != 0
+    assert k[0] == "igemm_dense_i8<128,256,2,2,3,2,1,0>", k
+
+
 def test_dense_igemm_short_k(device, monkeypatch):
     """Up to six k-tiles over at least two 128 x 128 tiles per CU: two ring stages, four blocks per CU (K of one to six
     k-tiles, ragged M / N / K, every epilogue); fewer tiles or a longer K keep the deeper ring."""

@@ -1640,8 +1640,16 @@ hipError_t launchIgemm(const IgemmArgs &a, uint32_t variant, const LaunchCtx &ct
         // prologues and epilogues overlap (256 -> 1024 channels at 56 x 56, batch 8: 13.5 us against 17.4)
         // (with fewer than two tiles per CU there is nothing to overlap, and the deeper ring is 2 us ahead)
         if (a.Kp <= ctx.tuning->denseShortK && (long long)((a.M + 127) / 128) * (a.Np / 128) >= 512) return launchIgemmDense<128, 128, 2, 2, 2, 4>(a, ctx);
+        // a long K in whole 128-byte k-tiles and more tiles than CUs: whole cache lines per tile row, two stages
+        // (1536 x 4096 x 4096: 28.8 us against 35.1; with one tile per CU the four-stage ring is ahead, 20.8 against 22.7)
+        if (a.Kp >= 4096 && a.Kp % 128 == 0 && (long long)((a.M + 127) / 128) * (a.Np / 128) > 256 && !ctx.tuning->noK128) {
+            return launchIgemmDense<128, 128, 2, 2, 2, 2, false, 128>(a, ctx);
+        }
         return launchIgemmDense<128, 128, 2, 2, 4, 2>(a, ctx);
-    case kIgemmDense128x256: return launchIgemmDense<128, 256, 2, 2, 3, 2>(a, ctx);
+    case kIgemmDense128x256:
+        // (the same on this tile, one block per CU: 1024 x 8192 x 8192 64.1 us against 72.3, never behind)
+        if (a.Kp >= 4096 && a.Kp % 128 == 0 && !ctx.tuning->noK128) return launchIgemmDense<128, 256, 2, 2, 2, 1, false, 128>(a, ctx);
+        return launchIgemmDense<128, 256, 2, 2, 3, 2>(a, ctx);
     case kIgemmDense64x64: return launchIgemmDense<64, 64, 2, 2, 4, 4>(a, ctx);
     case kIgemmDense256x128: return launchIgemmDense<256, 128, 2, 2, 3, 2>(a, ctx);
     case kIgemmDense256x64: return launchIgemmDense<256, 64, 4, 1, 3, 2>(a, ctx);
