@@ -119,6 +119,20 @@ def test_conv2d_window_ring_k128(device, monkeypatch):
     assert k[0].startswith("igemm_dense_conv_i8<64,64,2,2,4,4,0,"), k
 
 
+@pytest.mark.parametrize("variant,name", [(5, "igemm_dense_conv_i8<128,128,2,2,2,2,"), (6, "igemm_dense_conv_i8<128,256,2,2,2,1,")])
+def test_conv2d_window_ring_128_wide_tiles_long_k(device, variant, name, monkeypatch):
+    """The 128-wide window tiles with K >= 2304 in whole 128-byte k-tiles: 128 channels of the window per k-tile row."""
+    monkeypatch.setenv("THIP_WINDOW_VARIANT", str(variant))
+    for kw in (dict(N=3, H=29, W=31, C=256, O=144, pad=(1, 1, 1, 1), input_zp=-90), dict(N=5, H=27, W=25, C=128, O=48, KH=5, KW=4, stride=(2, 2), pad=(1, 0, 2, 0), output_zp=-7, output_min=-128),
+               dict(N=2, H=20, W=33, C=384, O=130, KH=3, KW=3, stride=(1, 2), pad=(0, 1, 1, 0)), dict(N=2, H=30, W=30, C=96, O=64, KH=4, KW=7, pad=(3, 3, 1, 2))):
+        k = check(device, w.conv2d_workload(realistic=True, **kw), via="device")
+        assert k[0].startswith(name), (kw, k)
+    k = check(device, w.conv2d_workload(N=2, H=32, W=32, C=256, O=64, realistic=False))   # the literal requant range
+    assert k[0].startswith(name), k
+    k = check(device, w.conv2d_workload(N=2, H=32, W=32, C=208, O=64, realistic=True))    # K = 1872: 64-byte k-tiles
+    assert not k[0].startswith(name), k
+
+
 @pytest.mark.parametrize("variant", [None, 14, 9])
 def test_conv2d_window_ring_few_channels(device, variant, monkeypatch):
     """Fewer channels than a k-tile: the chunks of one k-tile span several taps and window rows."""
