@@ -144,18 +144,18 @@ class Loaded:
 # (KiB per dispatch; the factors are what the same counters read for a plain 256 MiB copy, --copy-calibration).
 # They belong to the kernels as they were when the counters were read: TRAFFIC_KERNELS_SHA256 is the hash of
 # torq-compiler_amd/csrc/thip_kernels.hip at that time, and a run on other kernel sources reports traffic null.
-TRAFFIC_KERNELS_SHA256 = "18f296e5d4e2264b889b30c4eacf2c92f12d3c66b8c4ca33abd47e0d706f5329"
+TRAFFIC_KERNELS_SHA256 = "498b446dba470eb0a1564fc040c7726ae2d71d341dbd32598aad90886f2b63c4"
 MEASURED_TRAFFIC = {
-    "fc_4096x4096x4096": (49387.5 * 1.9996 + 16603.9 * 1.0000) * 1024,
-    "fc_512x4096x4096": (16446.0 * 1.9996 + 2048.0 * 1.0000) * 1024,
-    "fc_16x2048x8192": (8401.0 * 1.9996 + 256.0 * 1.0000) * 1024,
-    "conv_112x112x32_o64_3x3": (370.7 * 1.9996 + 784.0 * 1.0000) * 1024,
-    "conv3x3_56x56x256_o256_b32": (17258.0 * 1.9996 + 25939.5 * 1.0000) * 1024,
-    "depthwise_b64": (15430.5 * 1.9996 + 7063.3 * 1.0000) * 1024,
-    "depthwise_s1_b256": (63688.6 * 1.9996 + 113180.2 * 1.0000) * 1024,
-    "maxpool_b64": (25118.1 * 1.9996 + 12544.0 * 1.0000) * 1024,
-    "avgpool_b64": (2001.0 * 1.9996 + 80.0 * 1.0000) * 1024,
-    "add_b64": (4717.0 * 1.9996 + 4704.0 * 1.0000) * 1024,
+    "fc_4096x4096x4096": (49387.0 * 1.9995 + 16582.3 * 1.0000) * 1024,
+    "fc_512x4096x4096": (16453.0 * 1.9995 + 2048.0 * 1.0000) * 1024,
+    "fc_16x2048x8192": (8408.0 * 1.9995 + 256.0 * 1.0000) * 1024,
+    "conv_112x112x32_o64_3x3": (366.7 * 1.9995 + 784.0 * 1.0000) * 1024,
+    "conv3x3_56x56x256_o256_b32": (17254.1 * 1.9995 + 25992.5 * 1.0000) * 1024,
+    "depthwise_b64": (15443.1 * 1.9995 + 7063.2 * 1.0000) * 1024,
+    "depthwise_s1_b256": (63722.4 * 1.9995 + 113158.0 * 1.0000) * 1024,
+    "maxpool_b64": (25122.4 * 1.9995 + 12544.0 * 1.0000) * 1024,
+    "avgpool_b64": (2001.0 * 1.9995 + 80.0 * 1.0000) * 1024,
+    "add_b64": (4723.0 * 1.9995 + 4704.0 * 1.0000) * 1024,
 }
 
 
