@@ -423,14 +423,15 @@ class Emitter {
             // A small weight matrix over many pixels: keep it in LDS and stream the pixels.  Measured against the dense
             // tiles on pointwise shapes of 16 .. 960 channels over 12 544 .. 802 816 pixels: with at most four k-steps
             // per pixel group (the depth of its prefetch ring) it is ahead from about 200 000 pixels, and from 40 000
-            // where N >= 2 K (the output dominates: the expanding convolutions); with a longer K only where N >= 2 K,
+            // where N >= 2 K and K <= 32 (the output dominates: the first expanding convolutions of a mobile network;
+            // 64 -> 384 over 50 176 pixels is 9.0 us on a dense tile against 10.6); with a longer K only where N >= 2 K,
             // up to 2^28 outputs (beyond that its passes over the activations, one per 256 channels, cost more), or
             // where an add follows a very large image (the fused add saves more than the dense tile gains); below
             // those sizes a dense tile is 10-50 % faster.
             if (M >= 4096 && igemmStreamFits(N, K, outDtype) && !getenv("THIP_NO_STREAM")) {
                 const bool expanding = N >= 2 * K;
                 const char *em = getenv("THIP_STREAM_EXPAND_MIN_M");  // tuning: the pixel count from which an expanding layer streams
-                const bool take = K <= 128 ? (M >= 200000 || (expanding && M >= (em ? atoll(em) : 40000)))
+                const bool take = K <= 128 ? (M >= 200000 || (expanding && K <= 32 && M >= (em ? atoll(em) : 40000)))
                                            : ((expanding && M >= 25000 && M * N < (1LL << 28)) || (addFollows && M >= 400000));
                 if (take) return kIgemmStream;
             }
