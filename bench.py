@@ -142,9 +142,14 @@ class Loaded:
 
 # HBM bytes per launch of each workload's kernel, from rocprofv3 counters: FETCH_SIZE * 1.9995 + WRITE_SIZE * 1.0
 # (KiB per dispatch; the factors are what the same counters read for a plain 256 MiB copy, --copy-calibration).
-# They belong to the kernels as they were when the counters were read: TRAFFIC_KERNELS_SHA256 is the hash of
-# torq-compiler_amd/csrc/thip_kernels.hip at that time, and a run on other kernel sources reports traffic null.
-TRAFFIC_KERNELS_SHA256 = "498b446dba470eb0a1564fc040c7726ae2d71d341dbd32598aad90886f2b63c4"
+# They belong to the kernels as they were when the counters were read: TRAFFIC_SOURCES_SHA256 holds the hashes of
+# the kernel sources (under torq-compiler_amd/csrc) at that time, and a run whose kernel source -- the file the
+# workload's kernel lives in, or the helpers every kernel file includes -- has changed since reports traffic null.
+TRAFFIC_SOURCES_SHA256 = {
+    "thip_kernels_common.h": "89eff9b09a9cb00a464dea200f5c893757370fca1f92043d5425a4065d9b0096",
+    "thip_igemm.hip": "cc9944efbf5c09fdbfc49c93ded4d9c2b7af354a827f1dd1489ea76b28049485",
+    "thip_bandwidth.hip": "aa515d4402c1add8c14c40a2640ee69f316f3db48147c20798fe853213b03281",
+}
 MEASURED_TRAFFIC = {
     "fc_4096x4096x4096": (49387.0 * 1.9995 + 16582.3 * 1.0000) * 1024,
     "fc_512x4096x4096": (16453.0 * 1.9995 + 2048.0 * 1.0000) * 1024,
@@ -159,9 +164,14 @@ MEASURED_TRAFFIC = {
 }
 
 
-def kernels_sha256():
-    with open(os.path.join(ROOT, "torq-compiler_amd", "csrc", "thip_kernels.hip"), "rb") as f:
-        return hashlib.sha256(f.read()).hexdigest()
+def traffic_still_valid(name):
+    """Whether the kernel sources behind workload `name` are the ones its MEASURED_TRAFFIC entry was read on."""
+    family = "thip_igemm.hip" if name.startswith(("fc_", "conv")) else "thip_bandwidth.hip"
+    for source in ("thip_kernels_common.h", family):
+        with open(os.path.join(ROOT, "torq-compiler_amd", "csrc", source), "rb") as f:
+            if hashlib.sha256(f.read()).hexdigest() != TRAFFIC_SOURCES_SHA256[source]:
+                return False
+    return True
 
 
 # The traffic shape of the benchmark's bandwidth rows for the streaming-floor calibration: 16-byte reads per 16-byte
@@ -174,7 +184,7 @@ STREAM_SHAPES = {
 
 
 def roofline(wl, bound, ms, name=None):
-    traffic = MEASURED_TRAFFIC.get(name) if kernels_sha256() == TRAFFIC_KERNELS_SHA256 else None
+    traffic = MEASURED_TRAFFIC.get(name) if name in MEASURED_TRAFFIC and traffic_still_valid(name) else None
     traffic = None if traffic is None else int(round(traffic))
     if bound == "mfma":
         achieved = wl.ops / (ms * 1e-3) / 1e12

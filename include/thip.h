@@ -101,6 +101,14 @@ thip_status_t thip_program_constant(thip_program_t *program, int32_t dtype, int3
 thip_status_t thip_program_tensor(thip_program_t *program, int32_t dtype, int32_t rank,
                                   const int64_t *shape, thip_value_t *out_value);
 
+/* The same bytes under another shape: `shape` elements of `base` (a binding or an intermediate), starting
+ * `element_offset` elements into it.  What tensor.collapse_shape / tensor.expand_shape around an op (the patterns
+ * create them, compiler/torq/Conversions/LinalgToTorqHL/Conv2DMatmulPattern.cpp:105,134,411) and a contiguous
+ * tensor.extract_slice / insert_slice become once bufferized: no op, no copy.  A view may be read and may be the
+ * `init` of fully_connected, matmul, add, transpose and the elementwise ops; the rank-4 image ops take whole values. */
+thip_status_t thip_program_view(thip_program_t *program, thip_value_t base, int64_t element_offset,
+                                int32_t rank, const int64_t *shape, thip_value_t *out_value);
+
 /* The op records.  Field names and meaning are those of the TorqHL op
  * definitions; `init` is the destination-passing-style output operand
  * (compiler/torq/Dialect/TorqHL/TorqHLOps.td:27-46). */

@@ -1,83 +1,8 @@
 """Shared helpers of the test-suite: run a workload through the C-ABI, evaluate it with the oracle."""
 import numpy as np
 
-from oracle import oracle as orc
-
-
-def oracle_eval(wl):
-    """Expected outputs of a single-op workload, computed by the CPU oracle."""
-    a = dict(wl.attrs)
-    kind = wl.name.split("_")[0]
-    x = wl.inputs[0]
-    if kind == "conv2d":
-        layout = orc.NHWC if a.pop("nhwc") else orc.NCHW
-        w, sb = a.pop("weights"), a.pop("scale_bias")
-        return [orc.conv2d(x, w, sb, layout=layout, **a)]
-    if kind == "depthwise":
-        layout = orc.NHWC if a.pop("nhwc") else orc.NCHW
-        w, sb = a.pop("weights"), a.pop("scale_bias")
-        return [orc.depthwise_conv2d(x, w, sb, layout=layout, **a)]
-    if kind == "fully":
-        w, sb = a.pop("weights"), a.pop("scale_bias")
-        return [orc.fully_connected(x, w, sb, **a)]
-    if kind == "fcbf16":
-        return [orc.fully_connected_bf16(x, a["weights"], a["bias"], output_min=a["output_min"], output_max=a["output_max"])]
-    if kind in ("convbf16", "dwbf16"):
-        fn = orc.conv2d_bf16 if kind == "convbf16" else orc.depthwise_conv2d_bf16
-        return [fn(x, a["weights"], a["bias"], pad=a["pad"], stride=a["stride"], output_min=a["output_min"], output_max=a["output_max"],
-                   layout=orc.NHWC if a["nhwc"] else orc.NCHW)]
-    if kind == "pwadd":
-        wp, sbp, pa = a["pw"]
-        aw, asb, aa = a["add"]
-        y = orc.conv2d(x, wp, sbp, layout=orc.NHWC, **pa)
-        return [orc.add(wl.inputs[1], y, aw, asb, **aa) if a["other_first"] else orc.add(y, wl.inputs[1], aw, asb, **aa)]
-    if kind == "branches":
-        ya, yb, yc = [orc.fully_connected(x, wt, sb, **at) for wt, sb, at in a["fcs"]]
-        (w0, sb0, a0), (w1, sb1, a1) = a["adds"]
-        return [orc.add(orc.add(ya, yb, w0, sb0, **a0), yc, w1, sb1, **a1)]
-    if kind == "fma":
-        return [orc.fma(x, a.pop("weights"), a.pop("scale_bias"), **a)]
-    if kind == "mul":
-        return [orc.mul(x, wl.inputs[1], a.pop("scale_bias"), **a)]
-    if kind == "binary":
-        return [orc.elementwise_binary(a["op_type"], x, wl.inputs[1], is_unsigned=a["is_unsigned"])]
-    if kind == "compare":
-        return [orc.elementwise_compare(a["op_type"], x, wl.inputs[1], is_unsigned=a["is_unsigned"])]
-    if kind == "unary":
-        return [orc.elementwise_unary(a["op_type"], x)]
-    if kind == "shift":
-        return [orc.elementwise_shift(a["op_type"], x, wl.inputs[1], round=a["round"])]
-    if kind == "table":
-        return [orc.table(x, a["words"], a["out_dtype"])]
-    if kind == "act":
-        return [orc.act(x, a["name"], min_int=a["min_int"], max_int=a["max_int"], out_dtype=a["out_dtype"])]
-    if kind == "avgpoolbf16":
-        return [orc.avg_pool2d_bf16(x, a["weights"], a["bias"], output_min=a["output_min"], output_max=a["output_max"])]
-    if kind == "expandmm":
-        w16 = orc.expand_weights(a["weights"], a["scale"], a["qbias"], block_size=a["block"], output_min=a["expand_min"],
-                                 output_max=a["expand_max"])
-        res = [orc.matmul_bf16(x, w16, a["bias"], output_min=a["output_min"], output_max=a["output_max"])]
-        return res if a["fold"] else res + [w16[None]]
-    if kind == "addbf16":
-        return [orc.add_bf16(wl.inputs[0], wl.inputs[1], a["weights"], a["bias"], output_min=a["output_min"], output_max=a["output_max"])]
-    if kind == "matmul":
-        res = orc.matmul(x, a["input2"], a["scale_bias"], output_zp=a["output_zp"], output_min=a["output_min"], output_max=a["output_max"],
-                         shift=a["shift"], out_dtype=a["out_dtype"])
-        return [res.reshape(wl.outputs[0][0])]
-    if kind == "matmulbf16":
-        res = orc.matmul_bf16(x, a["input2"], a["bias"])
-        return [res.reshape(wl.outputs[0][0])]
-    if kind == "maxpool":
-        layout = orc.NHWC if a.pop("nhwc") else orc.NCHW
-        return [orc.maxpool2d(x, layout=layout, **a)]
-    if kind == "avgpool":
-        sb = a.pop("scale_bias")
-        a.pop("input_zp")
-        return [orc.avg_pool2d(x, sb, **a)]
-    if kind == "add":
-        w, sb = a.pop("weights"), a.pop("scale_bias")
-        return [orc.add(wl.inputs[0], wl.inputs[1], w, sb, **a)]
-    raise ValueError(wl.name)
+from oracle.programs import (BF16_TALLY, assert_bf16_close, assert_bit_exact, bf16_ordered,  # noqa: F401  (re-exported)
+                             eval_network as oracle_network, eval_workload as oracle_eval)
 
 
 def run_on_gpu(device, wl, via="host"):
@@ -108,70 +33,3 @@ def families(kernels):
     return [k.split("<")[0] for k in kernels]
 
 
-def assert_bit_exact(got, want, what=""):
-    assert got.shape == want.shape and got.dtype == want.dtype, (what, got.shape, want.shape, got.dtype, want.dtype)
-    if not np.array_equal(got, want):
-        bad = np.argwhere(got != want)
-        first = tuple(bad[0])
-        raise AssertionError("%s: %d of %d elements differ; first at %s: got %d want %d"
-                             % (what, len(bad), got.size, first, int(got[first]), int(want[first])))
-
-
-def bf16_ordered(bits):
-    """bf16 bit patterns -> integers whose order and spacing are those of the values (one step = one ULP)."""
-    b = np.asarray(bits, dtype=np.uint16).astype(np.int32)
-    return np.where(b < 0x8000, b, 0x8000 - b)
-
-
-# Tally of the bf16 comparisons of this process: per call, (what, elements compared, elements beyond `ulps` steps that
-# only the cancellation bound admitted).  tests/test_bf16.py reports and bounds it after its GPU cases.
-BF16_TALLY = []
-
-
-def assert_bf16_close(got, want, what="", ulps=1, magnitude=None):
-    """The bf16 rows are tolerance rows: at most `ulps` bf16 steps from the oracle per element.
-
-    `magnitude` (sum of |products| + |bias| per element) admits, for sums that cancel, the error a different
-    order of fp32 additions can make: 2^-17 of it (a bf16 step is 2^-8 of the result, so where nothing cancels the
-    ULP bound is the binding one)."""
-    assert got.shape == want.shape and got.dtype == np.uint16 and want.dtype == np.uint16, (what, got.shape, want.shape)
-    bad = np.abs(bf16_ordered(got) - bf16_ordered(want)) > ulps
-    if magnitude is not None:
-        gf = (got.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
-        wf = (want.astype(np.uint32) << 16).view(np.float32).astype(np.float64)
-        beyond = int(bad.sum())
-        bad &= ~(np.abs(gf - wf) <= np.asarray(magnitude, dtype=np.float64).reshape(got.shape) * 2.0 ** -17)
-        BF16_TALLY.append((what, int(got.size), beyond - int(bad.sum())))
-    else:
-        BF16_TALLY.append((what, int(got.size), 0))
-    if bad.any():
-        first = tuple(np.argwhere(bad)[0])
-        raise AssertionError("%s: %d of %d elements differ by more than %d bf16 ULP; first at %s: got 0x%04x want 0x%04x"
-                             % (what, int(bad.sum()), got.size, ulps, first, int(got[first]), int(want[first])))
-
-
-def oracle_network(wl, return_all=False):
-    """Replays a network workload (wl.attrs['layers']) layer by layer with the CPU oracle, N,H,W,C."""
-    layers = wl.attrs["layers"]
-    x = wl.inputs[0]
-    if not wl.attrs["nhwc"]:
-        x = np.ascontiguousarray(x.transpose(0, 2, 3, 1))
-    tensors = [x]
-    for L in layers:
-        src = [tensors[i] for i in L.inputs]
-        a = dict(L.attrs)
-        if L.op == "conv2d":
-            t = orc.conv2d(src[0], L.weights, L.scale_bias, layout=orc.NHWC, **a)
-        elif L.op == "depthwise_conv2d":
-            t = orc.depthwise_conv2d(src[0], L.weights, L.scale_bias, layout=orc.NHWC, **a)
-        elif L.op == "add":
-            t = orc.add(src[0], src[1], L.weights, L.scale_bias, **a)
-        elif L.op == "avg_pool2d":
-            a.pop("input_zp")
-            t = orc.avg_pool2d(src[0], L.scale_bias, **a)
-        elif L.op == "fully_connected":
-            t = orc.fully_connected(src[0].reshape(src[0].shape[0], -1), L.weights, L.scale_bias, **a)
-        else:
-            raise ValueError(L.op)
-        tensors.append(t)
-    return tensors if return_all else tensors[-1]

@@ -13,7 +13,8 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libthip.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
-SOURCES = ["thip_kernels.hip", "thip_driver.cpp", "thip_emitter.cpp", "thip_validate.cpp", "thip_status.cpp"]
+SOURCES = ["thip_igemm.hip", "thip_bandwidth.hip", "thip_bf16.hip", "thip_device_util.hip", "thip_driver.cpp", "thip_emitter.cpp",
+           "thip_validate.cpp", "thip_status.cpp"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
@@ -25,8 +26,20 @@ COMMON = ["-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
           "-Xclang", "-target-feature", "-Xclang", "-dot6-insts"]
 
 
-def _compile(src, extra):
+HEADERS = ["thip_kernels.h", "thip_kernels_common.h", "thip_descriptor.h", "thip_status.h", "thip_validate.h"]
+
+
+def _up_to_date(src, obj):
+    if not os.path.exists(obj):
+        return False
+    deps = [os.path.join(CSRC, src)] + [os.path.join(CSRC, h) for h in HEADERS] + [os.path.join(os.path.dirname(HERE), "include", "thip.h"), __file__]
+    return all(os.path.getmtime(d) <= os.path.getmtime(obj) for d in deps if os.path.exists(d))
+
+
+def _compile(src, extra, force=True):
     obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ".o")
+    if not force and _up_to_date(src, obj):
+        return obj, ""
     cmd = [HIPCC] + COMMON + extra + ["-c", os.path.join(CSRC, src), "-o", obj]
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l and "dot6-insts" not in l)
@@ -35,10 +48,12 @@ def _compile(src, extra):
     return obj, out
 
 
-def build(verbose=False, extra=()):
+def build(verbose=False, extra=(), force=True):
+    """Compiles every source and links the library.  force=False (the command line's default: a developer's edit
+    loop) recompiles only sources older than their object file."""
     os.makedirs(OBJ_DIR, exist_ok=True)
-    with ThreadPoolExecutor(max_workers=4) as pool:
-        results = list(pool.map(lambda s: _compile(s, list(extra)), SOURCES))
+    with ThreadPoolExecutor(max_workers=8) as pool:
+        results = list(pool.map(lambda s: _compile(s, list(extra), force), SOURCES))
     objs = [r[0] for r in results]
     if verbose:
         for _, out in results:
@@ -52,4 +67,5 @@ def build(verbose=False, extra=()):
 
 
 if __name__ == "__main__":
-    print(build(verbose=True, extra=sys.argv[1:]))
+    args = sys.argv[1:]
+    print(build(verbose=True, extra=[a for a in args if a != "--force"], force="--force" in args))

@@ -28,7 +28,9 @@
 
 namespace thip {
 
-enum ValueKind { kValueBinding = 0, kValueConstant = 1, kValueTensor = 2 };
+// kValueView: `shape` elements of value `base` starting `viewOffset` elements into it (thip_program_view); `base`
+// is a binding or an intermediate, never another view
+enum ValueKind { kValueBinding = 0, kValueConstant = 1, kValueTensor = 2, kValueView = 3 };
 
 struct Value {
     ValueKind kind;
@@ -36,6 +38,8 @@ struct Value {
     int32_t rank;
     int64_t shape[THIP_MAX_RANK];
     uint32_t binding;
+    thip_value_t base = -1;
+    int64_t viewOffset = 0;
     std::vector<uint8_t> data;
     int64_t numel() const {
         int64_t n = 1;
@@ -180,6 +184,10 @@ class Emitter {
         if (thip_status_t s = checkValue(id, what, &v)) return s;
         if (v->kind == kValueBinding) {
             *out = bindingRef(*v, false);
+        } else if (v->kind == kValueView) {
+            if (thip_status_t s = literalInput(v->base, what, out)) return s;
+            if (state_[v->base].nhwcOfNchw) return fail(THIP_UNIMPLEMENTED, "%s: a view of an N,C,H,W intermediate", what);
+            out->offset += (uint64_t)v->viewOffset * elemSize(v->dtype);
         } else if (v->kind == kValueConstant) {
             if (!state_[id].defined) {
                 state_[id].ref = newConst(v->data);
@@ -265,6 +273,7 @@ class Emitter {
         }
         if (v->dtype != dtype) return fail(THIP_INVALID_ARGUMENT, "%s: init element type mismatch", what);
         if (v->kind == kValueConstant) return fail(THIP_INVALID_ARGUMENT, "%s: init cannot be a constant", what);
+        if (v->kind == kValueView) return fail(THIP_UNIMPLEMENTED, "%s: init cannot be a view", what);
         const uint64_t bytes = (uint64_t)(N * H * W * physC(id, C)) * elemSize(dtype);
         const bool sameInMemory = declaredNhwc || C == 1 || H * W == 1;
         if (v->kind == kValueTensor) {
@@ -308,7 +317,22 @@ class Emitter {
                         (long long)v->numel(), (long long)numel);
         }
         if (v->kind == kValueConstant) return fail(THIP_INVALID_ARGUMENT, "%s: init cannot be a constant", what);
-        if (v->kind == kValueTensor) {
+        if (v->kind == kValueView) {
+            // a slice of a binding, or of an intermediate that is allocated whole when its first slice is written
+            const Value &b = prog_.values[(size_t)v->base];
+            if (b.kind == kValueTensor) {
+                if (!state_[v->base].defined) {
+                    state_[v->base].ref = newTemp((uint64_t)b.numel() * elemSize(b.dtype));
+                    state_[v->base].defined = true;
+                    state_[v->base].nhwcOfNchw = false;
+                }
+                if (state_[v->base].nhwcOfNchw) return fail(THIP_UNIMPLEMENTED, "%s: a view of an N,C,H,W intermediate", what);
+                *out = state_[v->base].ref;
+            } else {
+                *out = bindingRef(b, true);
+            }
+            out->offset += (uint64_t)v->viewOffset * elemSize(dtype);
+        } else if (v->kind == kValueTensor) {
             state_[id].ref = newTemp((uint64_t)(physElems ? physElems : numel) * elemSize(dtype));
             state_[id].defined = true;
             state_[id].nhwcOfNchw = false;
@@ -1894,6 +1918,12 @@ void Emitter::planChannelPadding() {
         if (chan[v] == 0) chan[v] = C;
         else if (chan[v] != C) chan[v] = -1;
     };
+    for (size_t v = 0; v < n; v++) {
+        if (prog_.values[v].kind == kValueView) {
+            bar((thip_value_t)v);
+            bar(prog_.values[v].base);
+        }
+    }
     for (const HlOp &op : prog_.ops) {
         switch (op.kind) {
         case kHlConv2d:
@@ -1953,7 +1983,9 @@ void Emitter::planExpandFolding() {
     const size_t n = prog_.values.size();
     std::vector<int> reads(n, 0), asMatmulRhs(n, 0);
     auto read = [&](thip_value_t v) {
-        if (v >= 0 && (size_t)v < n) reads[(size_t)v]++;
+        if (v < 0 || (size_t)v >= n) return;
+        reads[(size_t)v]++;
+        if (prog_.values[(size_t)v].kind == kValueView) reads[(size_t)prog_.values[(size_t)v].base]++;  // a read of a view reads its base
     };
     for (const HlOp &op : prog_.ops) {
         switch (op.kind) {
@@ -2190,6 +2222,28 @@ thip_status_t thip_program_constant(thip_program_t *program, int32_t dtype, int3
 thip_status_t thip_program_tensor(thip_program_t *program, int32_t dtype, int32_t rank, const int64_t *shape,
                                   thip_value_t *out_value) {
     return addValue(program, kValueTensor, 0, dtype, rank, shape, nullptr, 0, out_value);
+}
+
+thip_status_t thip_program_view(thip_program_t *program, thip_value_t base, int64_t element_offset, int32_t rank,
+                                const int64_t *shape, thip_value_t *out_value) {
+    if (!program || !out_value) return fail(THIP_INVALID_ARGUMENT, "null program or result pointer");
+    if (base < 0 || (size_t)base >= program->values.size()) return fail(THIP_INVALID_ARGUMENT, "thip_program_view: value %d does not exist", (int)base);
+    // a view of a view names the underlying value directly
+    const Value b = program->values[(size_t)base];
+    const thip_value_t root = b.kind == kValueView ? b.base : base;
+    const int64_t rootOffset = b.kind == kValueView ? b.viewOffset : 0;
+    if (b.kind == kValueConstant) return fail(THIP_UNIMPLEMENTED, "thip_program_view: a view of a constant (declare the constant in the shape it is used in)");
+    if (thip_status_t s = addValue(program, kValueView, 0, b.dtype, rank, shape, nullptr, 0, out_value)) return s;
+    Value &v = program->values.back();
+    if (element_offset < 0 || element_offset > b.numel() || v.numel() > b.numel() - element_offset) {
+        program->values.pop_back();
+        return fail(THIP_INVALID_ARGUMENT, "thip_program_view: elements %lld .. %lld lie outside the %lld of value %d", (long long)element_offset,
+                    (long long)(element_offset + v.numel()), (long long)b.numel(), (int)base);
+    }
+    v.base = root;
+    v.viewOffset = rootOffset + element_offset;
+    v.binding = program->values[(size_t)root].binding;
+    return THIP_OK;
 }
 
 #define THIP_DEFINE_HL(fn, type, kindEnum, member)                                        \

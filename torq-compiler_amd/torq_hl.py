@@ -84,6 +84,14 @@ class Program:
                                               rt._shape_array(shape), ctypes.byref(v)))
         return Value(self, v.value, shape, dtype, "tensor")
 
+    def view(self, base, shape, offset=0):
+        """The same bytes under another shape (tensor.collapse_shape / expand_shape / a contiguous slice): `shape`
+        elements of `base` starting `offset` elements into it."""
+        v = ctypes.c_int32()
+        rt.check(rt.lib().thip_program_view(self._h, base.index, int(offset), len(shape), rt._shape_array(shape),
+                                            ctypes.byref(v)))
+        return Value(self, v.value, shape, base.dtype, "view")
+
     def _as_value(self, x):
         if isinstance(x, Value):
             return x

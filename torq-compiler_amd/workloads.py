@@ -794,3 +794,134 @@ def mobilenet_v2_workload(batch=1, resolution=224, classes=1000, seed=1006, nhwc
     wl = Workload("mobilenet_v2_b%d_%d" % (batch, resolution), p, [x], [((batch, classes), np.int8)], 2 * macs,
                   wbytes + x.nbytes + batch * classes, dict(layers=layers, shapes=shapes, nhwc=nhwc))
     return wl
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# benchmark configuration 4: one decode step of a Gemma-3-1B-shaped decoder, the part of it that is on this path
+# ---------------------------------------------------------------------------------------------------------------
+
+class DecoderOp:
+    """One TorqHL op of a decoder-step workload, by the names of the tensors it reads and writes, so that a checker
+    can replay it (kind "linear": torq_hl.expand_weights folded into a bf16 torq_hl.matmul; "scores" / "context":
+    the batched bf16 matmuls of the attention against the two caches; "add": bf16 torq_hl.add)."""
+
+    def __init__(self, kind, out, inputs, shape, **params):
+        self.kind = kind
+        self.out = out
+        self.inputs = inputs
+        self.shape = tuple(shape)
+        self.params = params
+
+
+def _block_quantized(rng, K, N, block, gain):
+    """int8 weights K x N, uniform in [-128, 127] (standard deviation 73.9), symmetric (no zero point, as the
+    benchmark configuration says) with one bf16 scale per `block` input rows and output channel, drawn so that the
+    expanded weights have a standard deviation of about gain / sqrt(K)."""
+    wq = rng.integers(-128, 128, size=(K, N), dtype=np.int8)
+    scale = to_bf16(rng.uniform(0.75, 1.25, size=(K // block, N)) * (gain / (73.9 * np.sqrt(K))))
+    return wq, scale, np.zeros((K // block, N), dtype=np.float32)
+
+
+def decoder_step_workload(batch=1, layers=26, hidden=1152, heads=4, head_dim=256, ffn=6912, vocab=262144, cache_len=1024,
+                          block=128, expose=False, seed=1040):
+    """benchmark configuration 4 as ONE program: a decode step (one new token per sequence, `batch` sequences) of a
+    decoder with `layers` layers, `heads` query heads over ONE key / value head, a gated feed-forward block and
+    the vocabulary projection, on key / value caches of `cache_len` positions.
+
+    Per layer, in data-flow order: q, k, v = x W (three bf16 matmuls whose int8 weights pass through
+    torq_hl.expand_weights: bf16 scales per `block` input rows; k and v also leave the program, the caller appends
+    them to its caches); scores = q K^T per sequence (torq_hl.matmul against the key cache, which is kept position-
+    major [batch, cache_len, head_dim] and transposed by a torq_hl.transpose that the serialiser folds into the
+    matmul); context = scores V (torq_hl.matmul against the value cache, kept dimension-major [batch, head_dim,
+    cache_len] and transposed the same way); o = context W_o; h = add(x, o); gate, up = h W; a = add(gate, up);
+    d = a W_down; x' = add(h, d).  Then logits = x W_vocab.  What a real decoder has between these ops -- the
+    normalisations, the rotary embedding, the softmax over the scores, the gated activation and the embedding
+    lookup -- are not ops of this path: scores feed the context matmul directly, the gate is an add, and the
+    token embeddings arrive as the input binding.  Scales are chosen so that every tensor stays of order one.
+
+    Bindings: 0 x [batch, hidden]; 1 key cache [layers * batch, cache_len, head_dim]; 2 value cache
+    [layers * batch, head_dim, cache_len]; 3 logits [batch, vocab]; 4 new keys [layers, batch, head_dim];
+    5 new values likewise; expose=True adds 6: every intermediate of every layer, one after another (wl.attrs
+    ["trace"] maps names to (offset, shape)), so that each op can be checked on the inputs the GPU gave it."""
+    rng = np.random.default_rng(seed)
+    M, B = batch, batch
+    qdim = heads * head_dim
+    p = Program()
+    p.set_name("decoder_step_b%d_l%d" % (batch, layers))
+    x_in = to_bf16(rng.standard_normal((M, hidden)))
+    kcache = to_bf16(rng.standard_normal((layers * B, cache_len, head_dim)))
+    vcache = to_bf16(rng.standard_normal((layers * B, head_dim, cache_len)))
+    bx = p.binding(0, x_in.shape, np.uint16)
+    bk = p.binding(1, kcache.shape, np.uint16)
+    bv = p.binding(2, vcache.shape, np.uint16)
+    blog = p.binding(3, (M, vocab), np.uint16)
+    bkn = p.binding(4, (layers, M, head_dim), np.uint16)
+    bvn = p.binding(5, (layers, M, head_dim), np.uint16)
+    trace, trace_elems = {}, 0
+    per_layer = [("q", (M, qdim)), ("scores", (B, heads, cache_len)), ("context", (B, heads, head_dim)), ("o", (M, hidden)),
+                 ("h", (M, hidden)), ("gate", (M, ffn)), ("up", (M, ffn)), ("a", (M, ffn)), ("d", (M, hidden)), ("x", (M, hidden))]
+    if expose:
+        for l in range(layers):
+            for name, shape in per_layer:
+                trace["%s%d" % (name, l)] = (trace_elems, shape)
+                trace_elems += int(np.prod(shape))
+        btrace = p.binding(6, (trace_elems,), np.uint16)
+    zero = np.zeros(1, dtype=np.float32)
+    noclamp = dict(output_zp=0, output_min=NO_CLAMP[0], output_max=NO_CLAMP[1])
+    half = to_bf16(np.array([0.70703125, 0.70703125], dtype=np.float32))  # keeps a sum of two unit tensors at unit size
+    ops, weight_bytes, macs = [], 0, 0
+
+    def dest(name, shape):
+        if not expose:
+            return p.tensor(shape, np.uint16)
+        off, _ = trace[name]
+        return p.view(btrace, shape, off)
+
+    def linear(out, src_name, src, K, N, gain, init=None):
+        nonlocal weight_bytes, macs
+        wq, scale, qbias = _block_quantized(rng, K, N, block, gain)
+        w16 = p.expand_weights(wq, scale, qbias, block_size=block, output_min=NO_CLAMP[0], output_max=NO_CLAMP[1])
+        y = p.matmul(src, w16, zero, init=init if init is not None else dest(out, (M, N)), shift=0, **noclamp)
+        ops.append(DecoderOp("linear", out, [src_name], (M, N), weights=wq, scale=scale, qbias=qbias, block=block))
+        weight_bytes += wq.nbytes
+        macs += M * K * N
+        return y
+
+    def add(out, a_name, a, b_name, b, shape):
+        y = p.add(a, b, half, zero, init=dest(out, shape), shift_factor=0, **noclamp)
+        ops.append(DecoderOp("add", out, [a_name, b_name], shape, weights=half, bias=zero))
+        return y
+
+    x, xn = bx, "x_in"
+    for l in range(layers):
+        n = lambda s: "%s%d" % (s, l)
+        q = linear(n("q"), xn, x, hidden, qdim, 1.0 / 512)
+        linear(n("k"), xn, x, hidden, head_dim, 1.0, init=p.view(bkn, (M, head_dim), l * M * head_dim))
+        linear(n("v"), xn, x, hidden, head_dim, 1.0, init=p.view(bvn, (M, head_dim), l * M * head_dim))
+        keys = p.transpose(p.view(bk, (B, cache_len, head_dim), l * B * cache_len * head_dim), (0, 2, 1))
+        scores = p.matmul(p.view(q, (B, heads, head_dim)), keys, zero, init=dest(n("scores"), (B, heads, cache_len)), shift=0, **noclamp)
+        ops.append(DecoderOp("scores", n("scores"), [n("q")], (B, heads, cache_len), layer=l))
+        values = p.transpose(p.view(bv, (B, head_dim, cache_len), l * B * head_dim * cache_len), (0, 2, 1))
+        context = p.matmul(scores, values, zero, init=dest(n("context"), (B, heads, head_dim)), shift=0, **noclamp)
+        ops.append(DecoderOp("context", n("context"), [n("scores")], (B, heads, head_dim), layer=l))
+        macs += 2 * B * heads * cache_len * head_dim
+        o = linear(n("o"), n("context"), p.view(context, (M, qdim)), qdim, hidden, 1.0)
+        h = add(n("h"), xn, x, n("o"), o, (M, hidden))
+        gate = linear(n("gate"), n("h"), h, hidden, ffn, 1.0)
+        up = linear(n("up"), n("h"), h, hidden, ffn, 1.0)
+        a = add(n("a"), n("gate"), gate, n("up"), up, (M, ffn))
+        d = linear(n("d"), n("a"), a, ffn, hidden, 1.0)
+        x = add(n("x"), n("h"), h, n("d"), d, (M, hidden))
+        xn = n("x")
+    linear("logits", xn, x, hidden, vocab, 1.0, init=blog)
+    inputs = [x_in, kcache, vcache]
+    outputs = [((M, vocab), np.uint16), ((layers, M, head_dim), np.uint16), ((layers, M, head_dim), np.uint16)]
+    if expose:
+        outputs.append(((trace_elems,), np.uint16))
+    # algorithmic bytes: every int8 weight once (the figure a weight-streaming decode step is priced against), the
+    # block scales, both caches and the activations that enter and leave
+    scale_bytes = weight_bytes // block * 2
+    bytes_ = weight_bytes + scale_bytes + kcache.nbytes + vcache.nbytes + x_in.nbytes + 2 * M * vocab + 4 * layers * M * head_dim
+    attrs = dict(ops=ops, trace=trace, batch=batch, layers=layers, heads=heads, head_dim=head_dim, cache_len=cache_len,
+                 hidden=hidden, ffn=ffn, vocab=vocab, weight_bytes=weight_bytes, expose=expose)
+    return Workload("decoder_step_b%d_l%d" % (batch, layers), p, inputs, outputs, 2 * macs, bytes_, attrs)
