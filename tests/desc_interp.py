@@ -25,7 +25,9 @@ TEMP = np.dtype([("size", "<u8")])
 CONST = np.dtype([("offset", "<u8"), ("size", "<u8")])
 
 K_TRANSPOSE, K_IGEMM, K_FC_SKINNY, K_DW, K_MAXPOOL, K_AVGPOOL, K_ADD, K_FC_BF16, K_ADD_BF16, K_IM2COL_BF16, K_DW_BF16 = 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11
-K_AVGPOOL_BF16, K_EXPAND, K_ELTWISE = 12, 13, 14
+K_AVGPOOL_BF16, K_EXPAND, K_ELTWISE, K_DEC_LINEAR, K_DEC_MATMUL = 12, 13, 14, 15, 16
+DEC_EXT = np.dtype([(n, REF, (3,)) for n in ["weights", "qscale", "qbias", "bias", "out"]] + [("N", "<i4", (3,)), ("reserved0", "<i4"), ("res", REF), ("add_out", REF)] +
+                   [(n, "<i4") for n in ["aw0", "aw1", "abias", "alo", "ahi"]] + [("reserved1", "<i4", (3,))])
 INT_BY_SIZE = {1: np.int8, 2: np.int16, 4: np.int32}
 OUT_NP = {1: np.int8, 2: np.int16, 3: np.int32}
 
@@ -289,6 +291,49 @@ def run(blob, binding_arrays):
             bias = view(op["bias"], N * 4).view(np.float32)
             res = orc.fully_connected_bf16(x, wt, bias, output_min=mn, output_max=mx)
             view(op["out"], M * N * 2).view(np.uint16)[:] = res.reshape(-1)
+        elif kind == K_DEC_LINEAR:
+            # grouped linear on block-quantized weights: every matrix as the expansion followed by the matmul, then the folded add
+            M, K, block, nmat, flags = int(op["M"]), int(op["K"]), int(op["gran"]), int(op["w0"]), int(op["w1"])
+            x = view(op["in0"], M * K * 2).view(np.uint16).reshape(M, K)
+            ext = np.frombuffer(view(op["table"], DEC_EXT.itemsize).tobytes(), dtype=DEC_EXT, count=1)[0]
+            G, kblocks = K // block, (K + 127) // 128
+            ys = []
+            for m in range(nmat):
+                N = int(ext["N"][m])
+                tiles = N // 16
+                frag = view(ext["weights"][m], tiles * kblocks * 2048).view(np.int8).reshape(tiles, kblocks, 2, 4, 16, 2, 8)  # [t][b][p][g][c][j & 1][e]
+                full = frag.transpose(0, 4, 1, 2, 5, 3, 6).reshape(N, kblocks * 128)  # [t, c][b, p, j & 1, g, e]: k = 128 b + 32 (2 p + (j & 1)) + 8 g + e
+                assert not full[:, K:].any()
+                sc = view(ext["qscale"][m], tiles * G * 64).view(np.float32).reshape(tiles, G, 16).transpose(1, 0, 2).reshape(G, N)
+                assert np.array_equal(orc.from_bf16(orc.to_bf16(sc)), sc), "block scales are bf16 values"
+                bi = (view(ext["qbias"][m], tiles * G * 64).view(np.float32).reshape(tiles, G, 16).transpose(1, 0, 2).reshape(G, N)
+                      if int(ext["qbias"][m]["space"]) else np.zeros((G, N), np.float32))
+                w16 = orc.expand_weights(np.ascontiguousarray(full[:, :K].T), orc.to_bf16(sc), np.ascontiguousarray(bi), block_size=block,
+                                         output_min=int(op["bias0"]), output_max=int(op["scale0"]))
+                bias = view(ext["bias"][m], N * 4).view(np.float32)
+                assert np.all(bias == bias[0])
+                y = orc.matmul_bf16(x, w16, bias[:1], output_min=mn, output_max=mx)[0]
+                ys.append(y)
+                if int(ext["out"][m]["space"]):
+                    view(ext["out"][m], M * N * 2).view(np.uint16)[:] = y.reshape(-1)
+            if flags & 6:
+                N = int(ext["N"][0])
+                wts = np.array([ext["aw0"], ext["aw1"]], dtype=np.uint16)
+                ab = np.array([ext["abias"]], dtype=np.int32).view(np.float32)
+                if flags & 2:
+                    res = view(ext["res"], M * N * 2).view(np.uint16).reshape(M, N).copy()
+                    first, second = (res, ys[0]) if flags & 8 else (ys[0], res)
+                else:
+                    first, second = ys[0], ys[1]
+                z = orc.add_bf16(first, second, wts, ab, output_min=int(ext["alo"]), output_max=int(ext["ahi"]))
+                view(ext["add_out"], M * N * 2).view(np.uint16)[:] = z.reshape(-1)
+        elif kind == K_DEC_MATMUL:
+            B, M, K, N = int(op["TB"]), int(op["M"]), int(op["K"]), int(op["Nn"])
+            a = view(op["in0"], (1 if int(op["w0"]) else B) * M * K * 2).view(np.uint16).reshape(-1, M, K)
+            w = view(op["weights"], (1 if int(op["w1"]) else B) * N * K * 2).view(np.uint16).reshape(-1, N, K)
+            res = orc.matmul_bf16(a, np.ascontiguousarray(w.transpose(0, 2, 1)), np.array([op["bias0"]], dtype=np.int32).view(np.float32),
+                                  output_min=mn, output_max=mx)
+            view(op["out"], B * M * N * 2).view(np.uint16)[:] = res.reshape(-1)
         elif kind == K_AVGPOOL_BF16:
             Nimg, H, W, C = (int(op[k]) for k in ["N", "H", "W", "C"])
             x = view(op["in0"], Nimg * H * W * C * 2).view(np.uint16).reshape(Nimg, H, W, C)

@@ -13,7 +13,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libthip.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
-SOURCES = ["thip_igemm.hip", "thip_bandwidth.hip", "thip_bf16.hip", "thip_device_util.hip", "thip_driver.cpp", "thip_emitter.cpp",
+SOURCES = ["thip_igemm.hip", "thip_bandwidth.hip", "thip_bf16.hip", "thip_decode.hip", "thip_device_util.hip", "thip_driver.cpp", "thip_emitter.cpp",
            "thip_validate.cpp", "thip_status.cpp"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")

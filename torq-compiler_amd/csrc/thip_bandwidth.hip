@@ -957,11 +957,7 @@ __global__ __launch_bounds__(256) void add_bf16(AddBf16Args p) {
     }
 #pragma unroll
     for (int e = 0; e < VEC; e++) {
-        const float x0 = __uint_as_float((uint32_t)a.h[e] << 16), x1 = __uint_as_float((uint32_t)b.h[e] << 16);
-        float acc = __fmul_rn(x0, p.w0);
-        acc = __fadd_rn(acc, __fmul_rn(x1, p.w1));
-        const float t0 = __fadd_rn(acc, p.bias);
-        o.h[e] = bf16Bits(t0 < p.lo ? p.lo : (t0 > p.hi ? p.hi : t0));
+        o.h[e] = addBf16One(a.h[e], b.h[e], p.w0, p.w1, p.bias, p.lo, p.hi);
     }
     if (VEC == 8) {
         *(v4i *)(p.out + i0) = o.v;

@@ -19,24 +19,6 @@ namespace thip {
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
-typedef float v2f __attribute__((ext_vector_type(2)));
-
-// Four int8 weights of a dword to bf16 pairs: w * scale + bias in fp32 (the product of an 8-bit weight and a
-// bf16 scale is exact, so the fused multiply-add rounds once, like a multiply followed by an add), optional
-// clamp, round to nearest even.
-template <bool CLAMP>
-__device__ __forceinline__ void expandQ8(int d, float sc, float bi, float lo, float hi, int *o0, int *o1) {
-    float f[4];
-#pragma unroll
-    for (int j = 0; j < 4; j++) {
-        f[j] = __builtin_fmaf((float)(int8_t)(d >> (8 * j)), sc, bi);
-        if (CLAMP) f[j] = f[j] < lo ? lo : (f[j] > hi ? hi : f[j]);
-    }
-    *o0 = __builtin_bit_cast(int, __builtin_convertvector((v2f){f[0], f[1]}, v2bf));
-    *o1 = __builtin_bit_cast(int, __builtin_convertvector((v2f){f[2], f[3]}, v2bf));
-}
-
 // Bias, clamp, round to bf16 and store one 32 x 32 accumulator tile: register 4 q + e of lane (r, h) is
 // out[m0 + r][n0 + 8 q + 4 h + e].  fcBf16StoreQuad stores the four registers of one q.
 __device__ __forceinline__ void fcBf16StoreQuad(const FcBf16Args &p, const float (&a)[4], int m0, int n0, int r, int h, int q) {

@@ -1,0 +1,340 @@
+// gfx950 kernels of decode-shaped bf16 programs (a decoder's step: at most 32 input rows per linear, so every
+// matrix is read once and the weights are the traffic): dec_linear, the grouped linear on block-quantized int8
+// weights (torq_hl.expand_weights folded into torq_hl.matmul, the add behind it folded into the epilogue), and
+// dec_matmul, the batched small matmul against a run-time operand held [N][K] (the attention's two products).
+//
+// Both use v_mfma_f32_16x16x32_bf16 with the weights as the row operand: a lane (c = lane & 15, g = lane >> 4) feeds
+// weight column c and input row c, each with the 8 consecutive k of group g, and receives
+// D[n = 4 g + e][m = c] in register e: four neighbouring output columns of one input row.  fp32 products of bf16
+// values are exact; only the order of the additions differs from a sum in k order.
+#include "thip_kernels_common.h"
+
+namespace thip {
+
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+
+constexpr int kDecWaves = 8;  // waves of a workgroup = ways K is split inside it
+
+__device__ __forceinline__ unsigned ldsOffset(const void *p) {
+    return (unsigned)(uintptr_t)(__attribute__((address_space(3))) const int8_t *)p;
+}
+
+// MR: groups of 16 input rows (1 or 2).  CH: k-blocks of a wave whose input rows are loaded together (their registers
+// are double-buffered when a wave owns more than CH k-blocks: 2 * CH * 16 * MR registers).  QB: the block biases exist.
+// QC: the expansion clamps.
+template <int MR, int CH, bool QB, bool QC>
+__global__ __launch_bounds__(kDecWaves * 64) void dec_linear(DecLinearArgs p, FastDiv qblk) {
+    extern __shared__ __attribute__((aligned(16))) int8_t smem[];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int c = lane & 15, g = lane >> 4;
+    // the tile of this workgroup: (matrix, 16 columns of it); a pair owns the same columns of both matrices
+    int tile = (int)blockIdx.x, seg = 0;
+    if (!p.pair) {
+        if (p.nseg > 1 && tile >= p.N[0] / 16) {
+            tile -= p.N[0] / 16;
+            seg = 1;
+            if (p.nseg > 2 && tile >= p.N[1] / 16) {
+                tile -= p.N[1] / 16;
+                seg = 2;
+            }
+        }
+    }
+    const int nmat = p.pair ? 2 : 1;
+    const int kblocks = (p.K + 127) >> 7;
+    const int nkb = wave < kblocks ? (kblocks - wave + kDecWaves - 1) / kDecWaves : 0;  // k-blocks wave, wave + 8, ...
+    const int maxkb = (kblocks + kDecWaves - 1) / kDecWaves;
+    const int G = p.K / p.qblock;
+    const unsigned regionBytes = (unsigned)(maxkb * nmat) * 2048u;
+    int8_t *region = smem + (size_t)wave * regionBytes;
+    const unsigned regionLds = ldsOffset(smem) + (unsigned)wave * regionBytes;
+    const int8_t *wsrc[2];
+    const float *qs[2], *qbp[2];
+    {
+        const int s0 = p.pair ? 0 : seg, s1 = p.pair ? 1 : seg;
+        wsrc[0] = s0 == 0 ? p.w[0] : s0 == 1 ? p.w[1] : p.w[2];
+        wsrc[1] = s1 == 0 ? p.w[0] : s1 == 1 ? p.w[1] : p.w[2];
+        qs[0] = s0 == 0 ? p.qscale[0] : s0 == 1 ? p.qscale[1] : p.qscale[2];
+        qs[1] = s1 == 0 ? p.qscale[0] : s1 == 1 ? p.qscale[1] : p.qscale[2];
+        qbp[0] = s0 == 0 ? p.qbias[0] : s0 == 1 ? p.qbias[1] : p.qbias[2];
+        qbp[1] = s1 == 0 ? p.qbias[0] : s1 == 1 ? p.qbias[1] : p.qbias[2];
+    }
+    // the wave's whole share of the weights, one burst: 2 KiB per k-block and matrix, straight into its LDS region
+    for (int i = 0; i < nkb; i++) {
+        const int kb = wave + kDecWaves * i;
+        for (int m = 0; m < nmat; m++) {
+            const int8_t *src = wsrc[m] + (((size_t)tile * kblocks + kb) * 2) * 1024 + (size_t)lane * 16;
+            const unsigned dst = regionLds + (unsigned)(i * nmat + m) * 2048u;
+            dmaLoad16(src, dst);
+            dmaLoad16(src + 1024, dst + 1024u);
+        }
+    }
+    struct XBuf {
+        v4i x[CH][4][MR];
+        float sc[CH][2], bi[CH][2];
+    };
+    // Loads only; a k-block the wave does not have, a row beyond M and a k beyond K read nothing and feed zeros.
+    auto loadChunk = [&](int ch, XBuf &b) {
+#pragma unroll
+        for (int u = 0; u < CH; u++) {
+            const int i = ch * CH + u;
+            const bool on = i < nkb;
+            const int kb = wave + kDecWaves * i;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const int k = kb * 128 + 32 * j + 8 * g;
+#pragma unroll
+                for (int mr = 0; mr < MR; mr++) {
+                    const int row = c + 16 * mr;
+                    b.x[u][j][mr] = (on && row < p.M && k < p.K) ? *(const v4i *)(p.x + (size_t)row * p.K + k) : v4i{0, 0, 0, 0};
+                }
+            }
+            // the 128 rows of a k-block lie in one quantisation block (qblock % 128 == 0)
+            const size_t gi = on ? (size_t)fastDiv((uint32_t)(kb * 128), qblk) : 0;
+#pragma unroll
+            for (int m = 0; m < 2; m++) {
+                if (m < nmat) {
+                    const size_t at = ((size_t)tile * G + gi) * 16 + c;
+                    b.sc[u][m] = on ? qs[m][at] : 0.0f;
+                    b.bi[u][m] = (QB && on) ? qbp[m][at] : 0.0f;
+                } else {
+                    b.sc[u][m] = 0.0f;
+                    b.bi[u][m] = 0.0f;
+                }
+            }
+        }
+    };
+    v4f acc[2][MR];
+#pragma unroll
+    for (int m = 0; m < 2; m++) {
+#pragma unroll
+        for (int mr = 0; mr < MR; mr++) acc[m][mr] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    auto computeChunk = [&](int ch, const XBuf &b) {
+#pragma unroll
+        for (int u = 0; u < CH; u++) {
+            const int i = ch * CH + u;
+            if (i >= nkb) break;
+#pragma unroll
+            for (int m = 0; m < 2; m++) {
+                if (m >= nmat) break;
+                const int8_t *wl = region + (size_t)(i * nmat + m) * 2048 + (size_t)lane * 16;
+                const v4i p0 = *(const v4i *)wl, p1 = *(const v4i *)(wl + 1024);
+                const int dw[8] = {p0[0], p0[1], p0[2], p0[3], p1[0], p1[1], p1[2], p1[3]};
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    int o[4];
+                    expandQ8<QC>(dw[2 * j], b.sc[u][m], b.bi[u][m], p.qlo, p.qhi, &o[0], &o[1]);
+                    expandQ8<QC>(dw[2 * j + 1], b.sc[u][m], b.bi[u][m], p.qlo, p.qhi, &o[2], &o[3]);
+                    const v8bf wfrag = __builtin_bit_cast(v8bf, v4i{o[0], o[1], o[2], o[3]});
+#pragma unroll
+                    for (int mr = 0; mr < MR; mr++) {
+                        acc[m][mr] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wfrag, __builtin_bit_cast(v8bf, b.x[u][j][mr]), acc[m][mr], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    };
+    const int nchunks = (nkb + CH - 1) / CH;
+    XBuf b0, b1;
+    loadChunk(0, b0);
+    waitVmcnt<0>();  // the DMA burst (and the first chunk's rows) has landed; the compiler counts only its own loads
+    for (int ch = 0; ch < nchunks; ch += 2) {
+        if (ch + 1 < nchunks) loadChunk(ch + 1, b1);
+        computeChunk(ch, b0);
+        if (ch + 1 < nchunks) {
+            if (ch + 2 < nchunks) loadChunk(ch + 2, b0);
+            computeChunk(ch + 1, b1);
+        }
+    }
+    // the waves' partial sums meet in LDS: each leaves its own in its own region (its weights are used up)
+    asm volatile("s_waitcnt lgkmcnt(0)" : : : "memory");
+#pragma unroll
+    for (int m = 0; m < 2; m++) {
+#pragma unroll
+        for (int mr = 0; mr < MR; mr++) {
+            if (m < nmat) ((v4f *)region)[(m * MR + mr) * 64 + lane] = acc[m][mr];
+        }
+    }
+    __syncthreads();
+    if (wave >= MR) return;
+    const int mr = wave;  // this wave finishes row group `wave`
+    const int row = c + 16 * mr;
+    if (row >= p.M) return;
+    const int s0 = p.pair ? 0 : seg;
+    const int Nseg = s0 == 0 ? p.N[0] : s0 == 1 ? p.N[1] : p.N[2];
+    const int n = tile * 16 + 4 * g;
+    uint16_t y[2][4];
+#pragma unroll
+    for (int m = 0; m < 2; m++) {
+        if (m >= nmat) break;
+        v4f s = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+        for (int w = 0; w < kDecWaves; w++) {
+            const v4f t = ((const v4f *)(smem + (size_t)w * regionBytes))[(m * MR + mr) * 64 + lane];
+            s += t;
+        }
+        const int sm = p.pair ? m : seg;
+        const float *bias = sm == 0 ? p.bias[0] : sm == 1 ? p.bias[1] : p.bias[2];
+        uint16_t *out = sm == 0 ? p.out[0] : sm == 1 ? p.out[1] : p.out[2];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const float t0 = s[e] + bias[n + e];
+            y[m][e] = bf16Bits(t0 < p.lo ? p.lo : (t0 > p.hi ? p.hi : t0));
+        }
+        if (out) {
+            *(v2i *)(out + (size_t)row * Nseg + n) = v2i{(int)((uint32_t)y[m][0] | ((uint32_t)y[m][1] << 16)), (int)((uint32_t)y[m][2] | ((uint32_t)y[m][3] << 16))};
+        }
+    }
+    if (p.add_mode == 0) return;
+    uint16_t z[4];
+    if (p.add_mode == 1) {
+        const v2i rv = *(const v2i *)(p.res + (size_t)row * Nseg + n);
+        const uint16_t r[4] = {(uint16_t)rv[0], (uint16_t)((uint32_t)rv[0] >> 16), (uint16_t)rv[1], (uint16_t)((uint32_t)rv[1] >> 16)};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            z[e] = p.res_first ? addBf16One(r[e], y[0][e], p.aw0, p.aw1, p.abias, p.alo, p.ahi) : addBf16One(y[0][e], r[e], p.aw0, p.aw1, p.abias, p.alo, p.ahi);
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) z[e] = addBf16One(y[0][e], y[1][e], p.aw0, p.aw1, p.abias, p.alo, p.ahi);
+    }
+    *(v2i *)(p.add_out + (size_t)row * Nseg + n) = v2i{(int)((uint32_t)z[0] | ((uint32_t)z[1] << 16)), (int)((uint32_t)z[2] | ((uint32_t)z[3] << 16))};
+}
+
+template <int MR, int CH, bool QB, bool QC>
+static hipError_t launchDecLinearT(const DecLinearArgs &a, int tiles, size_t lds, const LaunchCtx &ctx) {
+    auto kernel = dec_linear<MR, CH, QB, QC>;
+    static std::once_flag once;
+    static hipError_t configured = hipSuccess;
+    std::call_once(once, [&] { configured = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); });
+    if (configured != hipSuccess) return configured;
+    THIP_ENQUEUE(ctx, kernelLabel("dec_linear", {MR, CH, (int)QB, (int)QC, a.pair ? 2 : a.nseg, a.add_mode}), kernel, dim3((unsigned)tiles), dim3(kDecWaves * 64), lds, a,
+                 makeFastDiv((uint32_t)a.qblock));
+    return hipGetLastError();
+}
+
+// LDS a launch needs: every wave's share of the weights (the partial sums reuse it).
+static size_t decLinearLds(int K, int nmat) {
+    const int kblocks = (K + 127) / 128, maxkb = (kblocks + kDecWaves - 1) / kDecWaves;
+    return (size_t)kDecWaves * maxkb * nmat * 2048;
+}
+
+hipError_t launchDecLinear(const DecLinearArgs &a, const LaunchCtx &ctx) {
+    if (!a.x || a.M <= 0 || a.M > kDecMaxRows || a.K <= 0 || a.K % 8 != 0 || a.qblock <= 0 || a.qblock % 128 != 0 || a.K % a.qblock != 0) return hipErrorInvalidValue;
+    if (a.nseg < 1 || a.nseg > kDecMaxSegments || (a.pair && a.nseg != 2) || (((uintptr_t)a.x) & 15)) return hipErrorInvalidValue;
+    if (a.add_mode < 0 || a.add_mode > 2 || (a.add_mode == 1 && (a.nseg != 1 || !a.res)) || (a.add_mode == 2 && !a.pair) || (a.pair && a.add_mode != 2)) return hipErrorInvalidValue;
+    if (a.add_mode != 0 && (!a.add_out || (((uintptr_t)a.add_out) & 7) || (a.res && (((uintptr_t)a.res) & 7)))) return hipErrorInvalidValue;
+    long long tiles = 0;
+    bool anyBias = false;
+    for (int s = 0; s < a.nseg; s++) {
+        if (!a.w[s] || !a.qscale[s] || !a.bias[s] || a.N[s] <= 0 || a.N[s] % 16 != 0) return hipErrorInvalidValue;
+        if ((((uintptr_t)a.w[s]) & 15) || (((uintptr_t)a.qscale[s]) & 3) || (((uintptr_t)a.qbias[s]) & 3) || (((uintptr_t)a.bias[s]) & 3) || (((uintptr_t)a.out[s]) & 7)) return hipErrorInvalidValue;
+        if (!a.out[s] && a.add_mode == 0) return hipErrorInvalidValue;  // a result nobody receives
+        anyBias = anyBias || a.qbias[s] != nullptr;
+        tiles += a.N[s] / 16;
+    }
+    for (int s = 0; s < a.nseg; s++) {
+        if (anyBias && !a.qbias[s]) return hipErrorInvalidValue;  // all matrices of a launch with block biases, or none
+    }
+    if (a.pair) {
+        if (a.N[0] != a.N[1]) return hipErrorInvalidValue;
+        tiles = a.N[0] / 16;
+    }
+    const size_t lds = decLinearLds(a.K, a.pair ? 2 : 1);
+    if (tiles <= 0 || tiles > 65535 || lds > 152 * 1024) return hipErrorInvalidValue;
+    const bool clamp = !(a.qlo == -INFINITY && a.qhi == INFINITY);
+    const int t = (int)tiles;
+    if (a.M <= 16) {
+        if (clamp) return anyBias ? launchDecLinearT<1, 2, true, true>(a, t, lds, ctx) : launchDecLinearT<1, 2, false, true>(a, t, lds, ctx);
+        return anyBias ? launchDecLinearT<1, 2, true, false>(a, t, lds, ctx) : launchDecLinearT<1, 2, false, false>(a, t, lds, ctx);
+    }
+    if (clamp) return anyBias ? launchDecLinearT<2, 1, true, true>(a, t, lds, ctx) : launchDecLinearT<2, 1, false, true>(a, t, lds, ctx);
+    return anyBias ? launchDecLinearT<2, 1, true, false>(a, t, lds, ctx) : launchDecLinearT<2, 1, false, false>(a, t, lds, ctx);
+}
+
+// dec_matmul: a workgroup owns 16 columns (rows of w) of one batch element; its eight waves split K in steps of 32
+// (wave, wave + 8, ...), each lane loading 16 bytes of its weight row and of its input row per step; the partial
+// sums meet in LDS.  A wave's loads of up to ST steps are all issued before the first MFMA.
+template <int MR, int ST>
+__global__ __launch_bounds__(kDecWaves * 64) void dec_matmul(DecMatmulArgs p) {
+    __shared__ v4f red[kDecWaves][MR][64];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int c = lane & 15, g = lane >> 4;
+    const int n0 = (int)blockIdx.x * 16, b = (int)blockIdx.y;
+    const uint16_t *a = p.a + (size_t)b * p.a_stride, *w = p.w + (size_t)b * p.w_stride;
+    const int steps = (p.K + 31) >> 5;
+    const int nrow = n0 + c < p.N ? n0 + c : p.N - 1;  // clamped columns are never stored
+    v4f acc[MR];
+#pragma unroll
+    for (int mr = 0; mr < MR; mr++) acc[mr] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int s0 = wave; s0 < steps; s0 += kDecWaves * ST) {
+        v4i wv[ST], xv[ST][MR];
+#pragma unroll
+        for (int u = 0; u < ST; u++) {
+            const int k = (s0 + kDecWaves * u) * 32 + 8 * g;
+            const bool in = k < p.K;  // K % 8 == 0: a piece lies inside K or outside
+            wv[u] = in ? *(const v4i *)(w + (size_t)nrow * p.K + k) : v4i{0, 0, 0, 0};
+#pragma unroll
+            for (int mr = 0; mr < MR; mr++) {
+                const int row = c + 16 * mr;
+                xv[u][mr] = (in && row < p.M) ? *(const v4i *)(a + (size_t)row * p.K + k) : v4i{0, 0, 0, 0};
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < ST; u++) {
+#pragma unroll
+            for (int mr = 0; mr < MR; mr++) {
+                acc[mr] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8bf, wv[u]), __builtin_bit_cast(v8bf, xv[u][mr]), acc[mr], 0, 0, 0);
+            }
+        }
+    }
+#pragma unroll
+    for (int mr = 0; mr < MR; mr++) red[wave][mr][lane] = acc[mr];
+    __syncthreads();
+    if (wave >= MR) return;
+    const int mr = wave, row = c + 16 * mr;
+    if (row >= p.M) return;
+    v4f s = v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int wv = 0; wv < kDecWaves; wv++) s += red[wv][mr][lane];
+    const int n = n0 + 4 * g;
+    uint16_t *out = p.out + (size_t)b * p.out_stride + (size_t)row * p.N;
+    uint16_t y[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const float t0 = s[e] + p.bias;
+        y[e] = bf16Bits(t0 < p.lo ? p.lo : (t0 > p.hi ? p.hi : t0));
+    }
+    if ((p.N & 3) == 0 && n + 3 < p.N) {
+        *(v2i *)(out + n) = v2i{(int)((uint32_t)y[0] | ((uint32_t)y[1] << 16)), (int)((uint32_t)y[2] | ((uint32_t)y[3] << 16))};
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            if (n + e < p.N) out[n + e] = y[e];
+        }
+    }
+}
+
+hipError_t launchDecMatmul(const DecMatmulArgs &a, const LaunchCtx &ctx) {
+    if (!a.a || !a.w || !a.out || a.B <= 0 || a.B > 65535 || a.M <= 0 || a.M > kDecMaxRows || a.K <= 0 || a.K % 8 != 0 || a.N <= 0) return hipErrorInvalidValue;
+    if (a.a_stride < 0 || a.w_stride < 0 || a.out_stride < 0 || a.a_stride % 8 != 0 || a.w_stride % 8 != 0) return hipErrorInvalidValue;
+    if (((((uintptr_t)a.a) | ((uintptr_t)a.w)) & 15) || (((uintptr_t)a.out) & (a.N % 4 == 0 ? 7 : 1)) || (a.N % 4 == 0 && a.out_stride % 4 != 0)) return hipErrorInvalidValue;
+    const long long tiles = ((long long)a.N + 15) / 16;
+    if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
+    const dim3 grid((unsigned)tiles, (unsigned)a.B);
+    // steps of 32 per wave: up to four are one round of loads
+    const int perWave = ((a.K + 31) / 32 + kDecWaves - 1) / kDecWaves;
+    if (a.M <= 16) {
+        if (perWave <= 1) THIP_ENQUEUE(ctx, "dec_matmul<1,1>", (dec_matmul<1, 1>), grid, dim3(kDecWaves * 64), 0, a);
+        else if (perWave <= 2) THIP_ENQUEUE(ctx, "dec_matmul<1,2>", (dec_matmul<1, 2>), grid, dim3(kDecWaves * 64), 0, a);
+        else THIP_ENQUEUE(ctx, "dec_matmul<1,4>", (dec_matmul<1, 4>), grid, dim3(kDecWaves * 64), 0, a);
+    } else {
+        if (perWave <= 1) THIP_ENQUEUE(ctx, "dec_matmul<2,1>", (dec_matmul<2, 1>), grid, dim3(kDecWaves * 64), 0, a);
+        else if (perWave <= 2) THIP_ENQUEUE(ctx, "dec_matmul<2,2>", (dec_matmul<2, 2>), grid, dim3(kDecWaves * 64), 0, a);
+        else THIP_ENQUEUE(ctx, "dec_matmul<2,4>", (dec_matmul<2, 4>), grid, dim3(kDecWaves * 64), 0, a);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace thip

@@ -91,7 +91,39 @@ enum Kind : uint32_t {
     // element), bias0 / scale0 / shift / output_zp / output_min / output_max = the ACT stage (fma, mul) or
     // output_min / output_max = the clip range (the others)
     kKindEltwise = 14,
+    // Decode-shaped bf16 linear on block-quantized int8 weights (torq_hl.expand_weights folded into torq_hl.matmul),
+    // up to three matrices on the same M <= 32 input rows in one launch, the torq_hl.add behind it folded in:
+    // in0 = x [M][K] bf16, gran = rows per quantisation block (a multiple of 128), w0 = number of matrices, w1 =
+    // DecLinearFlags, output_min / output_max = float bits of the matmuls' clamp, bias0 / scale0 = float bits of the
+    // expansions' clamp, table = a DecLinearExt in the constant segment (the per-matrix operands), out = the first
+    // buffer the launch writes, Nn = its row length.
+    kKindDecLinear = 15,
+    // Batch of small bf16 matmuls against a run-time operand held [N][K]: in0 = a [TB][M][K] (w0 != 0: one [M][K] for
+    // every batch), weights = [TB][Nn][K] (w1 != 0: shared), out [TB][M][Nn]; M <= 32; bias0 = float bits of the one
+    // bias, output_min / output_max = float bits of the clamp.
+    kKindDecMatmul = 16,
 };
+
+enum DecLinearFlags : int32_t {
+    kDecPair = 1,         // two matrices of equal width; a workgroup owns the same columns of both, the add joins them
+    kDecAddResidual = 2,  // add_out = add(res, y) (kDecResFirst) or add(y, res)
+    kDecAddPair = 4,      // add_out = add(y0, y1)
+    kDecResFirst = 8,
+};
+
+// Per-matrix operands of a kKindDecLinear record.  weights: int8 in the dec16 fragment order (thip_kernels.h),
+// qscale / qbias: float [N / 16][K / gran][16] (qbias.space none: every bias is zero), bias: float [N], out: bf16
+// [M][N] (space none: not stored, the folded add is its only reader).
+struct DecLinearExt {
+    DescRef weights[3], qscale[3], qbias[3], bias[3], out[3];
+    int32_t N[3];
+    int32_t reserved0;
+    DescRef res, add_out;
+    int32_t aw0, aw1;           // bf16 bits of the add's two weights
+    int32_t abias, alo, ahi;    // float bits of its bias and clamp
+    int32_t reserved1[3];
+};
+static_assert(sizeof(DecLinearExt) == 15 * 16 + 16 + 2 * 16 + 32, "DecLinearExt layout");
 
 // Variants of kKindIgemm: how the A (activation) tile is gathered.
 enum IgemmLoader : uint32_t {

@@ -108,6 +108,8 @@ static const char *opKernelName(const DescOp &op) {
     case kKindAvgPoolBf16: return "avgpool_bf16";
     case kKindExpandWeights: return "expand_weights_bf16";
     case kKindEltwise: return "eltwise_int";
+    case kKindDecLinear: return "dec_linear";
+    case kKindDecMatmul: return "dec_matmul";
     default: return "unknown";
     }
 }
@@ -282,6 +284,51 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
         err = launchExpandWeights(a, ctx);
         break;
     }
+    case kKindDecLinear: {
+        DecLinearExt x;
+        memcpy(&x, e->blob.data() + e->header.data_offset + e->consts[op.table.index].offset + op.table.offset, sizeof(x));  // the host copy
+        DecLinearArgs a;
+        memset(&a, 0, sizeof(a));
+        a.x = (const uint16_t *)resolve(e, op.in0, bp);
+        a.M = op.M; a.K = op.K; a.qblock = (int32_t)op.gran;
+        a.nseg = op.w0;
+        a.pair = (op.w1 & kDecPair) ? 1 : 0;
+        for (int m = 0; m < op.w0 && m < kDecMaxSegments; m++) {
+            a.w[m] = (const int8_t *)resolve(e, x.weights[m], bp);
+            a.qscale[m] = (const float *)resolve(e, x.qscale[m], bp);
+            a.qbias[m] = (const float *)resolve(e, x.qbias[m], bp);
+            a.bias[m] = (const float *)resolve(e, x.bias[m], bp);
+            a.out[m] = (uint16_t *)resolve(e, x.out[m], bp);
+            a.N[m] = x.N[m];
+        }
+        memcpy(&a.lo, &op.output_min, 4);
+        memcpy(&a.hi, &op.output_max, 4);
+        memcpy(&a.qlo, &op.bias0, 4);
+        memcpy(&a.qhi, &op.scale0, 4);
+        a.add_mode = (op.w1 & kDecAddResidual) ? 1 : (op.w1 & kDecAddPair) ? 2 : 0;
+        a.res_first = (op.w1 & kDecResFirst) ? 1 : 0;
+        if (a.add_mode) {
+            a.res = (const uint16_t *)resolve(e, x.res, bp);
+            a.add_out = (uint16_t *)resolve(e, x.add_out, bp);
+            const uint32_t w0 = (uint32_t)x.aw0 << 16, w1 = (uint32_t)x.aw1 << 16;
+            memcpy(&a.aw0, &w0, 4);
+            memcpy(&a.aw1, &w1, 4);
+            memcpy(&a.abias, &x.abias, 4);
+            memcpy(&a.alo, &x.alo, 4);
+            memcpy(&a.ahi, &x.ahi, 4);
+        }
+        err = launchDecLinear(a, ctx);
+        break;
+    }
+    case kKindDecMatmul: {
+        DecMatmulArgs a{(const uint16_t *)resolve(e, op.in0, bp), (const uint16_t *)resolve(e, op.weights, bp), (uint16_t *)resolve(e, op.out, bp),
+                        op.TB, op.M, op.K, op.Nn, op.w0 ? 0 : (int64_t)op.M * op.K, op.w1 ? 0 : (int64_t)op.Nn * op.K, (int64_t)op.M * op.Nn, 0.0f, 0.0f, 0.0f};
+        memcpy(&a.bias, &op.bias0, 4);
+        memcpy(&a.lo, &op.output_min, 4);
+        memcpy(&a.hi, &op.output_max, 4);
+        err = launchDecMatmul(a, ctx);
+        break;
+    }
     default: return fail(THIP_INTERNAL, "op %u has unknown kind %u", i, op.kind);
     }
     if (err != hipSuccess) {
@@ -392,7 +439,8 @@ static thip_status_t dumpOpOutput(thip_executable_t *e, uint32_t i, uint8_t *con
     case kKindAvgPool: shape = {op.N, op.C}; break;
     case kKindAdd: shape = {op.C}; break;
     case kKindEltwise: shape = {op.C}; outType(); break;
-    case kKindFcBf16: shape = {op.M, op.Nn}; bf16(); break;
+    case kKindFcBf16: case kKindDecLinear: shape = {op.M, op.Nn}; bf16(); break;
+    case kKindDecMatmul: shape = {op.TB, op.M, op.Nn}; bf16(); break;
     case kKindAddBf16: shape = {op.C}; bf16(); break;
     case kKindIm2colBf16: shape = {op.N, op.OH, op.OW, op.Kp}; bf16(); break;
     case kKindDepthwiseBf16: shape = {op.N, op.OH, op.OW, op.C}; bf16(); break;

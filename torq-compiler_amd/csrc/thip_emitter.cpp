@@ -682,6 +682,24 @@ class Emitter {
     // Operands of an integer elementwise op: element types, and the record's common fields.
     thip_status_t eltwiseCommon(const char *what, thip_value_t input, thip_value_t init, DescOp *op);
     thip_status_t emitAvgPoolBf16(const thip_hl_avg_pool2d_t &c);
+    // ---- decode-shaped bf16 programs (at most 32 rows per matmul): fewer, wider launches -----------------------
+    // A torq_hl.transpose that emits no kernel: its result is read once, as input2 of a bf16 matmul with at most 32
+    // rows, which then reads the transpose's input as its [N][K] operand (result value -> index of the transpose).
+    std::map<thip_value_t, size_t> foldedTranspose_;
+    std::vector<char> consumed_;  // per op of the program: already emitted as part of an earlier op's record
+    void planDecodeFolding();
+    // A bf16 matmul that the grouped linear kernel can take: two-dimensional input1 of at most 32 rows, input2 a folded
+    // expand_weights with blocks of a multiple of 128 rows, N a multiple of 16.
+    struct DecCandidate {
+        const thip_hl_matmul_t *mm;
+        const thip_hl_expand_weights_t *ew;
+        int64_t M, K, N, block;
+        float bias;
+    };
+    bool decodeCandidate(size_t at, DecCandidate *out);
+    size_t nextLiveOp(size_t at) const;
+    thip_status_t tryEmitDecodeLinear(size_t at, bool *handled);
+    thip_status_t emitDecodeMatmul(const thip_hl_matmul_t &c, size_t transposeAt);
     // Operands of an expand_weights checked and measured.
     struct ExpandShape {
         const Value *w, *scale, *bias, *init;
@@ -1207,6 +1225,7 @@ thip_status_t Emitter::emitFullyConnectedBf16(const thip_hl_fully_connected_t &c
 thip_status_t Emitter::emitMatmulBf16(const thip_hl_matmul_t &c) {
     const char *what = "torq_hl.matmul (bf16)";
     if (thip_status_t s = checkFloatAct(what, c.shift, 0, 0, c.output_zp)) return s;
+    if (const auto ft = foldedTranspose_.find(c.input2); ft != foldedTranspose_.end()) return emitDecodeMatmul(c, ft->second);
     const Value *a, *b, *init, *bv;
     if (thip_status_t s = checkValue(c.input1, "torq_hl.matmul input1", &a)) return s;
     if (thip_status_t s = checkValue(c.input2, "torq_hl.matmul input2", &b)) return s;
@@ -1877,6 +1896,267 @@ thip_status_t Emitter::emitTransposeOp(const thip_hl_transpose_t &c) {
     return THIP_OK;
 }
 
+// ---- decode-shaped programs ------------------------------------------------------------------------------------
+// A decoder's step is a chain of some hundred small dependent ops on one to 32 rows: what it costs is the number of
+// launches and the memory round trips inside each.  The ops are therefore grouped: linears that read the same rows
+// become one record (query, key and value projections), two linears whose results meet in an add become one record
+// that computes both and adds (gate and up), the add behind a linear moves into its epilogue (residual connections),
+// and a transpose in front of a matmul's input2 is read in place.  THIP_NO_DECODE_FUSION leaves every op its own record.
+
+void Emitter::planDecodeFolding() {
+    foldedTranspose_.clear();
+    consumed_.assign(prog_.ops.size(), 0);
+    if (getenv("THIP_NO_DECODE_FUSION")) return;
+    const size_t n = prog_.values.size();
+    auto valid = [&](thip_value_t v) { return v >= 0 && (size_t)v < n; };
+    for (size_t t = 0; t < prog_.ops.size(); t++) {
+        if (prog_.ops[t].kind != kHlTranspose) continue;
+        const thip_hl_transpose_t &tr = prog_.ops[t].u.tr;
+        if (!valid(tr.init) || !valid(tr.input)) continue;
+        const Value &res = prog_.values[(size_t)tr.init], &src = prog_.values[(size_t)tr.input];
+        if (res.kind != kValueTensor || res.dtype != THIP_DTYPE_BF16 || src.dtype != THIP_DTYPE_BF16 || src.kind == kValueConstant) continue;
+        const bool swap2 = tr.rank == 2 && tr.perm[0] == 1 && tr.perm[1] == 0;
+        const bool swap3 = tr.rank == 3 && tr.perm[0] == 0 && tr.perm[1] == 2 && tr.perm[2] == 1;
+        if ((!swap2 && !swap3) || src.rank != tr.rank || res.rank != tr.rank || valueReads_[(size_t)tr.init] != 1) continue;
+        bool shapeOk = true;
+        for (int i = 0; i < tr.rank; i++) shapeOk = shapeOk && res.shape[i] == src.shape[tr.perm[i]];
+        if (!shapeOk) continue;  // emitTransposeOp reports it
+        for (size_t m = t + 1; m < prog_.ops.size(); m++) {
+            if (prog_.ops[m].kind != kHlMatmul || prog_.ops[m].u.mm.input2 != tr.init) continue;
+            const thip_hl_matmul_t &mm = prog_.ops[m].u.mm;
+            if (!valid(mm.input1) || !valid(mm.init) || mm.input1 == tr.init) break;
+            const Value &a = prog_.values[(size_t)mm.input1];
+            if (a.dtype != THIP_DTYPE_BF16 || a.rank < 2 || a.rank > 3 || a.shape[a.rank - 2] > kDecMaxRows) break;
+            const int64_t batches = std::max<int64_t>(a.rank == 3 ? a.shape[0] : 1, res.rank == 3 ? res.shape[0] : 1);
+            if (batches > 65535 || a.shape[a.rank - 1] % 8 != 0) break;
+            foldedTranspose_[tr.init] = t;
+            break;
+        }
+    }
+}
+
+thip_status_t Emitter::emitDecodeMatmul(const thip_hl_matmul_t &c, size_t transposeAt) {
+    const char *what = "torq_hl.matmul (bf16, transposed input2 read in place)";
+    const thip_hl_transpose_t &tr = prog_.ops[transposeAt].u.tr;
+    const Value *a, *w, *init, *bv;
+    if (thip_status_t s = checkValue(c.input1, "torq_hl.matmul input1", &a)) return s;
+    if (thip_status_t s = checkValue(tr.input, "torq_hl.transpose input", &w)) return s;
+    if (thip_status_t s = checkValue(c.init, "torq_hl.matmul init", &init)) return s;
+    if (init->dtype != THIP_DTYPE_BF16) return fail(THIP_INVALID_ARGUMENT, "%s: init must be bf16", what);
+    if (state_[c.input1].nhwcOfNchw || state_[tr.input].nhwcOfNchw) return fail(THIP_UNIMPLEMENTED, "%s: N,C,H,W intermediates are not accepted", what);
+    const int64_t Ba = a->rank == 3 ? a->shape[0] : 1, Bw = w->rank == 3 ? w->shape[0] : 1;
+    const int64_t M = a->shape[a->rank - 2], K = a->shape[a->rank - 1];
+    const int64_t N = w->shape[w->rank - 2], K2 = w->shape[w->rank - 1];  // the transpose's input: [N][K]
+    if (K != K2) return fail(THIP_INVALID_ARGUMENT, "%s: inner dimensions differ (%lld vs %lld)", what, (long long)K, (long long)K2);
+    const int64_t B = std::max(Ba, Bw);
+    if ((Ba != B && Ba != 1) || (Bw != B && Bw != 1)) return fail(THIP_INVALID_ARGUMENT, "%s: batch dimensions do not broadcast", what);
+    if (thip_status_t s = constantData(c.scale_bias, "torq_hl.matmul scale_bias", THIP_DTYPE_F32, &bv)) return s;
+    if (bv->numel() < 1) return fail(THIP_INVALID_ARGUMENT, "%s: scale_bias is empty", what);
+    if (!fitsInt32(B * M * N) || !fitsInt32(B * M * K) || !fitsInt32(B * K * N)) return fail(THIP_UNIMPLEMENTED, "%s: tensor too large for 32-bit indexing", what);
+    DescOp op;
+    memset(&op, 0, sizeof(op));
+    op.kind = kKindDecMatmul;
+    op.out_dtype = THIP_DTYPE_BF16;
+    op.output_min = c.output_min;
+    op.output_max = c.output_max;
+    memcpy(&op.bias0, bv->data.data(), 4);
+    op.TB = (int32_t)B; op.M = (int32_t)M; op.K = (int32_t)K; op.Kp = (int32_t)K; op.Nn = (int32_t)N; op.Np = (int32_t)N;
+    op.w0 = (Ba == 1 && B > 1) ? 1 : 0;
+    op.w1 = (Bw == 1 && B > 1) ? 1 : 0;
+    if (thip_status_t s = literalInput(c.input1, "torq_hl.matmul input1", &op.in0)) return s;
+    if (thip_status_t s = literalInput(tr.input, "torq_hl.transpose input", &op.weights)) return s;
+    if (thip_status_t s = literalOutput(c.init, "torq_hl.matmul init", THIP_DTYPE_BF16, B * M * N, &op.out)) return s;
+    if ((op.in0.offset & 15) || (op.weights.offset & 15) || (op.out.offset & 7)) return fail(THIP_UNIMPLEMENTED, "%s: a view at an offset that is no multiple of 16 bytes", what);
+    ops_.push_back(op);
+    return THIP_OK;
+}
+
+size_t Emitter::nextLiveOp(size_t at) const {
+    for (size_t i = at + 1; i < prog_.ops.size(); i++) {
+        const HlOp &op = prog_.ops[i];
+        if (consumed_[i]) continue;
+        if (op.kind == kHlExpandWeights && foldedExpand_.count(op.u.ew.init)) continue;
+        if (op.kind == kHlTranspose && foldedTranspose_.count(op.u.tr.init)) continue;
+        return i;
+    }
+    return prog_.ops.size();
+}
+
+bool Emitter::decodeCandidate(size_t at, DecCandidate *out) {
+    if (at >= prog_.ops.size() || prog_.ops[at].kind != kHlMatmul || consumed_[at]) return false;
+    const thip_hl_matmul_t &c = prog_.ops[at].u.mm;
+    const size_t n = prog_.values.size();
+    if (c.input1 < 0 || (size_t)c.input1 >= n || c.input2 < 0 || (size_t)c.input2 >= n || c.init < 0 || (size_t)c.init >= n || c.scale_bias < 0 || (size_t)c.scale_bias >= n) return false;
+    const auto folded = foldedExpand_.find(c.input2);
+    if (folded == foldedExpand_.end() || c.shift != 0 || c.output_zp != 0) return false;
+    const Value &a = prog_.values[(size_t)c.input1], &init = prog_.values[(size_t)c.init], &bv = prog_.values[(size_t)c.scale_bias];
+    if (a.dtype != THIP_DTYPE_BF16 || init.dtype != THIP_DTYPE_BF16 || a.rank != 2 || state_[c.input1].nhwcOfNchw) return false;
+    if (bv.kind != kValueConstant || bv.dtype != THIP_DTYPE_F32 || bv.numel() < 1) return false;
+    const thip_hl_expand_weights_t &ew = *folded->second;
+    if (ew.input < 0 || (size_t)ew.input >= n || ew.scale < 0 || (size_t)ew.scale >= n || ew.scale_bias < 0 || (size_t)ew.scale_bias >= n) return false;
+    const Value &w = prog_.values[(size_t)ew.input], &sc = prog_.values[(size_t)ew.scale], &qb = prog_.values[(size_t)ew.scale_bias];
+    if (w.dtype != THIP_DTYPE_I8 || w.rank != 2 || sc.dtype != THIP_DTYPE_BF16 || qb.dtype != THIP_DTYPE_F32) return false;
+    const int64_t M = a.shape[0], K = a.shape[1], N = w.shape[1], block = ew.block_size;
+    if (w.shape[0] != K || M > kDecMaxRows || K % 8 != 0 || N % 16 != 0 || N / 16 > 1024 || block <= 0 || block % 128 != 0 || K % block != 0) return false;
+    const int64_t G = K / block;
+    if (sc.numel() != G * N || qb.numel() % G != 0 || qb.numel() / G < N || init.numel() != M * N) return false;
+    if (((K + 127) / 128 + 7) / 8 > 9) return false;  // a workgroup's share of the weights (16 columns of the whole K) must fit a CU's LDS
+    out->mm = &c;
+    out->ew = &ew;
+    out->M = M; out->K = K; out->N = N; out->block = block;
+    memcpy(&out->bias, bv.data.data(), 4);
+    return true;
+}
+
+thip_status_t Emitter::tryEmitDecodeLinear(size_t at, bool *handled) {
+    *handled = false;
+    if (getenv("THIP_NO_DECODE_FUSION")) return THIP_OK;
+    DecCandidate c0;
+    if (!decodeCandidate(at, &c0)) return THIP_OK;
+    const size_t end = prog_.ops.size();
+    const size_t j1 = nextLiveOp(at), j2 = j1 < end ? nextLiveOp(j1) : end;
+    auto sameGroup = [&](const DecCandidate &a, const DecCandidate &b) {
+        return a.mm->input1 == b.mm->input1 && a.K == b.K && a.M == b.M && a.block == b.block && a.mm->output_min == b.mm->output_min &&
+               a.mm->output_max == b.mm->output_max && a.ew->output_min == b.ew->output_min && a.ew->output_max == b.ew->output_max &&
+               a.mm->init != b.mm->init;
+    };
+    auto bf16Add = [&](size_t i, const thip_hl_add_t **out) {
+        if (i >= end || prog_.ops[i].kind != kHlAdd) return false;
+        const thip_hl_add_t &ad = prog_.ops[i].u.add;
+        const size_t n = prog_.values.size();
+        if (ad.input1 < 0 || (size_t)ad.input1 >= n || ad.input2 < 0 || (size_t)ad.input2 >= n || ad.init < 0 || (size_t)ad.init >= n ||
+            ad.weights < 0 || (size_t)ad.weights >= n || ad.scale_bias < 0 || (size_t)ad.scale_bias >= n) return false;
+        const Value &x = prog_.values[(size_t)ad.input1], &y = prog_.values[(size_t)ad.input2], &z = prog_.values[(size_t)ad.init];
+        const Value &w = prog_.values[(size_t)ad.weights], &sb = prog_.values[(size_t)ad.scale_bias];
+        if (x.dtype != THIP_DTYPE_BF16 || y.dtype != THIP_DTYPE_BF16 || z.dtype != THIP_DTYPE_BF16 || ad.segment_output || ad.rhs_is_scalar) return false;
+        if (ad.shift_factor != 0 || ad.input_zp != 0 || ad.output_zp != 0) return false;
+        if (w.kind != kValueConstant || w.dtype != THIP_DTYPE_BF16 || w.numel() < 2 || sb.kind != kValueConstant || sb.dtype != THIP_DTYPE_F32 || sb.numel() < 1) return false;
+        if (x.numel() != y.numel() || x.numel() != z.numel()) return false;
+        *out = &ad;
+        return true;
+    };
+    // the matrices of the record, and the add folded into it
+    std::vector<DecCandidate> mats{c0};
+    std::vector<size_t> members{at};
+    const thip_hl_add_t *add = nullptr;
+    int flags = 0;
+    DecCandidate c1, c2;
+    const thip_hl_add_t *ad = nullptr;
+    const bool pairFits = ((c0.K + 127) / 128 + 7) / 8 <= 4;  // twice the share of one matrix
+    if (pairFits && j1 < end && decodeCandidate(j1, &c1) && sameGroup(c0, c1) && c0.N == c1.N && bf16Add(j2, &ad) &&
+        ((ad->input1 == c0.mm->init && ad->input2 == c1.mm->init) || (ad->input1 == c1.mm->init && ad->input2 == c0.mm->init)) &&
+        ad->init != c0.mm->init && ad->init != c1.mm->init) {
+        // gate and up: matrix 0 is the producer of the add's input1
+        if (ad->input1 == c0.mm->init) mats = {c0, c1};
+        else mats = {c1, c0};
+        members = {at, j1, j2};
+        add = ad;
+        flags = kDecPair | kDecAddPair;
+    } else if (j1 < end && decodeCandidate(j1, &c1) && sameGroup(c0, c1)) {
+        mats.push_back(c1);
+        members.push_back(j1);
+        if (j2 < end && decodeCandidate(j2, &c2) && sameGroup(c0, c2) && c1.mm->init != c2.mm->init) {
+            mats.push_back(c2);
+            members.push_back(j2);
+        }
+    } else if (bf16Add(j1, &ad) && ((ad->input1 == c0.mm->init) != (ad->input2 == c0.mm->init)) && ad->init != c0.mm->init) {
+        const thip_value_t other = ad->input1 == c0.mm->init ? ad->input2 : ad->input1;
+        // the other operand must exist already: a binding, or an intermediate some earlier record wrote
+        const Value &ov = prog_.values[(size_t)other];
+        const bool ready = ov.kind == kValueBinding || (ov.kind == kValueView ? (prog_.values[(size_t)ov.base].kind == kValueBinding || state_[ov.base].defined) : state_[other].defined);
+        if (ready && !state_[other].nhwcOfNchw && ov.numel() == c0.M * c0.N) {
+            members = {at, j1};
+            add = ad;
+            flags = kDecAddResidual | (ad->input1 == c0.mm->init ? 0 : kDecResFirst);
+        }
+    }
+    const char *what = "torq_hl.matmul (bf16, grouped)";
+    DescOp op;
+    memset(&op, 0, sizeof(op));
+    op.kind = kKindDecLinear;
+    op.out_dtype = THIP_DTYPE_BF16;
+    op.output_min = c0.mm->output_min;
+    op.output_max = c0.mm->output_max;
+    op.bias0 = c0.ew->output_min;
+    op.scale0 = c0.ew->output_max;
+    op.M = (int32_t)c0.M; op.K = (int32_t)c0.K; op.Kp = (int32_t)c0.K;
+    op.gran = (uint32_t)c0.block;
+    op.w0 = (int32_t)mats.size();
+    op.w1 = flags;
+    if (thip_status_t s = literalInput(c0.mm->input1, "torq_hl.matmul input1", &op.in0)) return s;
+    if (op.in0.offset & 15) return THIP_OK;  // a view at an odd offset: the ungrouped path takes it
+    DecLinearExt x;
+    memset(&x, 0, sizeof(x));
+    const int kblocks = (int)((c0.K + 127) / 128);
+    // block biases: stored only if any of them is non-zero in any matrix of the record
+    bool anyBias = false;
+    for (const DecCandidate &m : mats) {
+        const Value &qb = prog_.values[(size_t)m.ew->scale_bias];
+        const float *bd = (const float *)qb.data.data();
+        const int64_t cols = qb.numel() / (m.K / m.block);
+        for (int64_t g = 0; g < m.K / m.block && !anyBias; g++) {
+            for (int64_t n = 0; n < m.N && !anyBias; n++) anyBias = bd[g * cols + n] != 0.0f;
+        }
+    }
+    for (size_t mi = 0; mi < mats.size(); mi++) {
+        const DecCandidate &m = mats[mi];
+        const Value &w = prog_.values[(size_t)m.ew->input], &sc = prog_.values[(size_t)m.ew->scale], &qb = prog_.values[(size_t)m.ew->scale_bias];
+        const int8_t *wd = (const int8_t *)w.data.data();
+        std::vector<int8_t> packed(decWeightBytes((int)m.N, (int)m.K), 0);
+        for (int64_t k = 0; k < m.K; k++) {
+            const int8_t *row = wd + k * m.N;
+            for (int64_t n = 0; n < m.N; n++) packed[decWeightOffset((int)n, (int)k, kblocks)] = row[n];
+        }
+        const int64_t G = m.K / m.block, tiles = m.N / 16, cols = qb.numel() / G;
+        std::vector<float> scales((size_t)(tiles * G * 16)), biases(anyBias ? (size_t)(tiles * G * 16) : 0);
+        const uint16_t *sd = (const uint16_t *)sc.data.data();
+        const float *bd = (const float *)qb.data.data();
+        for (int64_t t = 0; t < tiles; t++) {
+            for (int64_t g = 0; g < G; g++) {
+                for (int64_t cidx = 0; cidx < 16; cidx++) {
+                    scales[(size_t)((t * G + g) * 16 + cidx)] = floatFromBf16(sd[g * m.N + t * 16 + cidx]);
+                    if (anyBias) biases[(size_t)((t * G + g) * 16 + cidx)] = bd[g * cols + t * 16 + cidx];
+                }
+            }
+        }
+        x.weights[mi] = newConst(packed);
+        x.qscale[mi] = newConst(scales);
+        if (anyBias) x.qbias[mi] = newConst(biases);
+        x.bias[mi] = newConst(std::vector<float>((size_t)m.N, m.bias));
+        x.N[mi] = (int32_t)m.N;
+        // the result is stored unless its only reader is the add folded into this record
+        const Value &iv = prog_.values[(size_t)m.mm->init];
+        const bool onlyTheAdd = add && iv.kind == kValueTensor && valueReads_[(size_t)m.mm->init] == 1;
+        if (!onlyTheAdd) {
+            if (thip_status_t s = literalOutput(m.mm->init, "torq_hl.matmul init", THIP_DTYPE_BF16, m.M * m.N, &x.out[mi])) return s;
+            if (x.out[mi].offset & 7) return fail(THIP_UNIMPLEMENTED, "%s: init is a view at an offset that is no multiple of 8 bytes", what);
+        }
+    }
+    if (add) {
+        const Value &w = prog_.values[(size_t)add->weights], &sb = prog_.values[(size_t)add->scale_bias];
+        x.aw0 = ((const uint16_t *)w.data.data())[0];
+        x.aw1 = ((const uint16_t *)w.data.data())[1];
+        memcpy(&x.abias, sb.data.data(), 4);
+        x.alo = add->output_min;
+        x.ahi = add->output_max;
+        if (flags & kDecAddResidual) {
+            const thip_value_t other = add->input1 == c0.mm->init ? add->input2 : add->input1;
+            if (thip_status_t s = literalInput(other, "torq_hl.add operand", &x.res)) return s;
+        }
+        if (thip_status_t s = literalOutput(add->init, "torq_hl.add init", THIP_DTYPE_BF16, c0.M * c0.N, &x.add_out)) return s;
+        if ((x.res.offset & 7) || (x.add_out.offset & 7)) return fail(THIP_UNIMPLEMENTED, "%s: the add behind it works on a view at an offset that is no multiple of 8 bytes", what);
+    }
+    std::vector<uint8_t> blob(sizeof(x));
+    memcpy(blob.data(), &x, sizeof(x));
+    op.table = newConst(blob);
+    op.out = add ? x.add_out : x.out[0];
+    op.Nn = (int32_t)mats[0].N; op.Np = (int32_t)mats[0].N;
+    ops_.push_back(op);
+    for (size_t mbr : members) consumed_[mbr] = 1;
+    *handled = true;
+    return THIP_OK;
+}
+
 // Decides which intermediates are stored with their channel axis padded to a multiple of 16.
 // A pointwise convolution over such a tensor streams it with 16-byte loads (the dense loader)
 // instead of gathering 8-byte pieces, which is what the 24-channel bottlenecks of mobile
@@ -2067,10 +2347,18 @@ void Emitter::fuseResidualAdd() {
 thip_status_t Emitter::run(void **outBlob, size_t *outSize) {
     planChannelPadding();
     planExpandFolding();
+    planDecodeFolding();
     for (size_t at = 0; at < prog_.ops.size(); at++) {
         const HlOp &op = prog_.ops[at];
         thip_status_t s = THIP_OK;
         addFollows_ = false;
+        if (consumed_[at]) continue;
+        if (op.kind == kHlTranspose && foldedTranspose_.count(op.u.tr.init)) continue;  // read in place by its matmul
+        if (op.kind == kHlMatmul) {
+            bool handled = false;
+            if ((s = tryEmitDecodeLinear(at, &handled))) return s;
+            if (handled) continue;
+        }
         if (op.kind == kHlConv2d && at + 1 < prog_.ops.size() && prog_.ops[at + 1].kind == kHlAdd && !getenv("THIP_NO_ADD_FUSION")) {
             const thip_value_t y = op.u.conv.init;
             const thip_hl_add_t &next = prog_.ops[at + 1].u.add;

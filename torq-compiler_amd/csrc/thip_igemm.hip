@@ -469,21 +469,6 @@ __global__ __launch_bounds__(256) void igemm_i8(IgemmArgs p) {
 // column operand: accumulator register r of lane l then holds
 // C[m = l & 31][n = 8 * (r / 4) + 4 * (l >> 5) + (r & 3)], four consecutive
 // output channels per register group, which requantise into one 32-bit store.
-__device__ __forceinline__ void dmaLoad16(const void *gptr, unsigned ldsAddr) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(ldsAddr), "v"(gptr) : "memory", "m0");
-}
-
-// Same with the address split into a wave-uniform 64-bit base (SGPR pair) and a 32-bit per-lane
-// offset: advancing along K is then scalar work only.
-__device__ __forceinline__ void dmaLoad16(const void *base, uint32_t laneOffset, unsigned ldsAddr) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(ldsAddr), "v"(laneOffset), "s"(base) : "memory", "m0");
-}
-
-template <int N>
-__device__ __forceinline__ void waitVmcnt() {
-    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
-}
-
 // DIRECT selects the epilogue: 0 staged through LDS (any output type, ragged N, the 64-bit requant tail), or in
 // registers (int8 output, N % 16 == 0: the launcher checks) with 1 the plain 32-bit tail or 2 the general 32-bit tail
 // (a pre-shift, a clamp of acc + bias or a zero point that does not fold: e.g. small shifts under large scales,

@@ -194,6 +194,64 @@ inline int fcBf16PreferredSplit(int M, int N, int K) {
     return split < 2 ? 1 : (int)split;
 }
 hipError_t launchFcBf16(const FcBf16Args &a, const LaunchCtx &ctx);
+// ---- decode-shaped bf16 programs: at most 32 input rows, the weights dominate the traffic ---------------------
+//
+// dec_linear: out[m][n] = bf16(clamp(sum_k x[m][k] * W[k][n] + bias[n])) with W = the expansion of block-quantized
+// int8 weights (torq_hl.expand_weights folded into its matmul): W[k][n] = bf16(clamp(w * qscale[k / qblock][n] +
+// qbias[k / qblock][n], qlo, qhi)).  One launch serves up to three matrices that read the same input rows
+// (`nseg` segments: q, k, v of an attention block), or two matrices of equal width whose results are added
+// (`pair`: gate and up), and can apply the torq_hl.add that follows to its result (a residual connection).  A
+// workgroup owns 16 output columns: it brings its whole share of the weights into LDS with one burst of LDS-DMA
+// loads, its eight waves split K, and their partial sums meet in LDS.
+//
+// Weight layout ("dec16"): for column tile t (16 columns), k-block b (128 input rows) and piece p (0, 1): 64 lanes x
+// 16 bytes, lane l = column l & 15 and k-group g = l >> 4; bytes 0..7 of the lane are rows 32 (2 p) + 8 g + 0..7 of
+// the k-block, bytes 8..15 rows 32 (2 p + 1) + 8 g + 0..7 (what one lane feeds to two v_mfma_f32_16x16x32_bf16).
+// Zero padded to whole k-blocks.  Scales (and biases) as float [tile][K / qblock][16].
+constexpr int kDecMaxSegments = 3;
+constexpr int kDecMaxRows = 32;
+struct DecLinearArgs {
+    const uint16_t *x;  // [M][K] bf16
+    int32_t M, K, qblock;
+    int32_t nseg;       // matrices of this launch, 1..3
+    int32_t pair;       // 1: two matrices of equal N; a workgroup owns the same 16 columns of both and adds its two results
+    const int8_t *w[kDecMaxSegments];
+    const float *qscale[kDecMaxSegments];
+    const float *qbias[kDecMaxSegments];  // null: every bias is zero (symmetric quantisation)
+    const float *bias[kDecMaxSegments];   // [N] per matrix
+    uint16_t *out[kDecMaxSegments];       // [M][N] per matrix; null: not stored (the fused add is its only reader)
+    int32_t N[kDecMaxSegments];           // multiples of 16
+    float lo, hi;                         // the matmuls' clamp
+    float qlo, qhi;                       // the expansions' clamp
+    // the torq_hl.add behind the matmul(s): 0 none; 1 add_out = add(res, y) when res_first, else add(y, res), res laid out
+    // like the result (one matrix only); 2 add_out = add(y0, y1) (pair)
+    int32_t add_mode, res_first;
+    const uint16_t *res;
+    uint16_t *add_out;
+    float aw0, aw1, abias, alo, ahi;
+};
+// Byte offset of int8 weight (n, k) in the dec16 order, for K padded to `kblocks` blocks of 128.
+inline size_t decWeightOffset(int n, int k, int kblocks) {
+    const int t = n >> 4, c = n & 15, b = k >> 7, kk = k & 127, j = kk >> 5, g = (kk & 31) >> 3, e = kk & 7;
+    return ((((size_t)t * kblocks + b) * 2 + (size_t)(j >> 1)) * 64 + (size_t)(g * 16 + c)) * 16 + (size_t)((j & 1) * 8 + e);
+}
+inline size_t decWeightBytes(int N, int K) { return (size_t)((N + 15) / 16) * ((K + 127) / 128) * 2048; }
+hipError_t launchDecLinear(const DecLinearArgs &a, const LaunchCtx &ctx);
+
+// dec_matmul: out[b][m][n] = bf16(clamp(sum_k a[b][m][k] * w[b][n][k] + bias)) for a batch of small matmuls whose
+// second operand is a run-time tensor held [N][K] (a key cache; a value cache kept dimension-major): M <= 32 rows
+// (the query heads of one sequence), K % 8 == 0.  a_stride / w_stride / out_stride: elements between batches (0:
+// the operand is shared by every batch).
+struct DecMatmulArgs {
+    const uint16_t *a;
+    const uint16_t *w;
+    uint16_t *out;
+    int32_t B, M, K, N;
+    int64_t a_stride, w_stride, out_stride;
+    float bias, lo, hi;
+};
+hipError_t launchDecMatmul(const DecMatmulArgs &a, const LaunchCtx &ctx);
+
 // Sustained v_mfma_i32_32x32x32_i8 rate (TOP/s, 1 multiply-add = 2 ops) of `blocks` workgroups of four waves that
 // do nothing else, on constant or on random operand bytes.  Allocates and frees its own few KiB.
 hipError_t measureMfmaRate(int randomOperands, int blocks, int iterations, hipStream_t stream, double *outTops);

@@ -290,4 +290,51 @@ __host__ __device__ inline bool residualAddFolded(int32_t w0, int32_t w1, int32_
     return true;
 }
 
+typedef __bf16 v2bf __attribute__((ext_vector_type(2)));
+typedef float v2f __attribute__((ext_vector_type(2)));
+
+// Four int8 weights of a dword to bf16 pairs: w * scale + bias in fp32 (the product of an 8-bit weight and a
+// bf16 scale is exact, so the fused multiply-add rounds once, like a multiply followed by an add), optional
+// clamp, round to nearest even.
+template <bool CLAMP>
+__device__ __forceinline__ void expandQ8(int d, float sc, float bi, float lo, float hi, int *o0, int *o1) {
+    float f[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        f[j] = __builtin_fmaf((float)(int8_t)(d >> (8 * j)), sc, bi);
+        if (CLAMP) f[j] = f[j] < lo ? lo : (f[j] > hi ? hi : f[j]);
+    }
+    *o0 = __builtin_bit_cast(int, __builtin_convertvector((v2f){f[0], f[1]}, v2bf));
+    *o1 = __builtin_bit_cast(int, __builtin_convertvector((v2f){f[2], f[3]}, v2bf));
+}
+
+// torq_hl.add on bf16, one element: no fused multiply-add -- the second product is added to the first (both exact in
+// fp32), then the bias, as the ACT stage does; clamp; round to nearest even.
+__device__ __forceinline__ uint16_t addBf16One(uint16_t a, uint16_t b, float w0, float w1, float bias, float lo, float hi) {
+    const float x0 = __uint_as_float((uint32_t)a << 16), x1 = __uint_as_float((uint32_t)b << 16);
+    float acc = __fmul_rn(x0, w0);
+    acc = __fadd_rn(acc, __fmul_rn(x1, w1));
+    const float t0 = __fadd_rn(acc, bias);
+    return bf16Bits(t0 < lo ? lo : (t0 > hi ? hi : t0));
+}
+
+// global -> LDS without registers (global_load_lds_dwordx4): the 64 lanes of a wave write 64 x 16 bytes = 1 KiB of
+// consecutive LDS starting at ldsAddr (wave-uniform), each from its own global address.  The load counts in vmcnt
+// like any other; the compiler does not see it, so whoever issues it waits for it by hand (waitVmcnt).
+__device__ __forceinline__ void dmaLoad16(const void *gptr, unsigned ldsAddr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(ldsAddr), "v"(gptr) : "memory", "m0");
+}
+
+// Same with the address split into a wave-uniform 64-bit base (SGPR pair) and a 32-bit per-lane
+// offset: advancing along K is then scalar work only.
+__device__ __forceinline__ void dmaLoad16(const void *base, uint32_t laneOffset, unsigned ldsAddr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(ldsAddr), "v"(laneOffset), "s"(base) : "memory", "m0");
+}
+
+template <int N>
+__device__ __forceinline__ void waitVmcnt() {
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+
 }  // namespace thip

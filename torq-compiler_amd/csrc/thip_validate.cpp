@@ -128,6 +128,30 @@ static uint64_t refRoom(const DescriptorView *e, const DescRef &r) {
     }
 }
 
+// An operand reference that does not sit in the record itself (it came out of a constant blob): names an existing
+// buffer, at an offset inside it.
+static thip_status_t checkLooseRef(const DescriptorView *e, uint32_t i, const DescRef &r) {
+    uint64_t limit = 0;
+    switch (r.space) {
+    case kSpaceNone: return THIP_OK;
+    case kSpaceBinding:
+        if (r.index >= e->header.binding_count) return fail(THIP_INVALID_ARGUMENT, "op %u names binding %u of %u", i, r.index, e->header.binding_count);
+        limit = e->bindings[r.index].size;
+        break;
+    case kSpaceTemp:
+        if (r.index >= e->header.temp_count) return fail(THIP_INVALID_ARGUMENT, "op %u names intermediate %u of %u", i, r.index, e->header.temp_count);
+        limit = e->temps[r.index].size;
+        break;
+    case kSpaceConst:
+        if (r.index >= e->header.const_count) return fail(THIP_INVALID_ARGUMENT, "op %u names constant %u of %u", i, r.index, e->header.const_count);
+        limit = e->consts[r.index].size;
+        break;
+    default: return fail(THIP_INVALID_ARGUMENT, "op %u has an operand in unknown space %u", i, r.space);
+    }
+    if (r.offset > limit) return fail(THIP_INVALID_ARGUMENT, "op %u operand offset %llu is past its buffer (%llu)", i, (unsigned long long)r.offset, (unsigned long long)limit);
+    return THIP_OK;
+}
+
 // Checks, once at creation, that every kernel record stays inside the buffers it names.
 thip_status_t checkOpFootprint(const DescriptorView *e, uint32_t i) {
     const DescOp &op = e->ops[i];
@@ -344,6 +368,61 @@ thip_status_t checkOpFootprint(const DescriptorView *e, uint32_t i) {
             if ((s = need(op.in1, fcBf16WorkspaceBytes(op.M, op.Nn, op.w0), "workspace"))) return s;
         }
         return need(op.out, mul(op.M, op.Nn) * 2, "out");
+    }
+    case kKindDecLinear: {
+        if (!positive({op.M, op.K}) || op.M > kDecMaxRows || op.K % 8 != 0 || op.gran == 0 || op.gran % 128 != 0 || (uint32_t)op.K % op.gran != 0 ||
+            op.w0 < 1 || op.w0 > kDecMaxSegments || (op.w1 & ~(kDecPair | kDecAddResidual | kDecAddPair | kDecResFirst))) {
+            return fail(THIP_INVALID_ARGUMENT, "op %u: bad grouped-linear record", i);
+        }
+        const bool pair = op.w1 & kDecPair, addRes = op.w1 & kDecAddResidual, addPair = op.w1 & kDecAddPair;
+        if ((pair && op.w0 != 2) || pair != addPair || (addRes && (addPair || op.w0 != 1))) return fail(THIP_INVALID_ARGUMENT, "op %u: bad grouped-linear flags", i);
+        if ((s = need(op.in0, mul(op.M, op.K) * 2, "in"))) return s;
+        if (op.table.space != kSpaceConst) return fail(THIP_INVALID_ARGUMENT, "op %u: the per-matrix operands must be a constant", i);
+        if ((s = need(op.table, sizeof(DecLinearExt), "per-matrix operands"))) return s;
+        if ((op.table.offset & 7) != 0) return fail(THIP_INVALID_ARGUMENT, "op %u: misaligned per-matrix operands", i);
+        DecLinearExt x;
+        memcpy(&x, e->blob + e->header.data_offset + e->consts[op.table.index].offset + op.table.offset, sizeof(x));
+        const uint64_t G = (uint64_t)op.K / op.gran;
+        bool anyBias = false, allBias = true;
+        for (int m = 0; m < op.w0; m++) {
+            const DescRef *refs[] = {&x.weights[m], &x.qscale[m], &x.qbias[m], &x.bias[m], &x.out[m]};
+            for (const DescRef *r : refs) {
+                if ((s = checkLooseRef(e, i, *r))) return s;
+            }
+            if (x.N[m] <= 0 || x.N[m] % 16 != 0 || x.N[m] > (1 << 24)) return fail(THIP_INVALID_ARGUMENT, "op %u: matrix %d has %d columns", i, m, x.N[m]);
+            const uint64_t tiles = (uint64_t)x.N[m] / 16;
+            if ((s = need(x.weights[m], decWeightBytes(x.N[m], op.K), "weights"))) return s;
+            if ((s = need(x.qscale[m], tiles * G * 64, "block scales"))) return s;
+            if (x.qbias[m].space != kSpaceNone && (s = need(x.qbias[m], tiles * G * 64, "block biases"))) return s;
+            anyBias = anyBias || x.qbias[m].space != kSpaceNone;
+            allBias = allBias && x.qbias[m].space != kSpaceNone;
+            if ((s = need(x.bias[m], (uint64_t)x.N[m] * 4, "bias"))) return s;
+            if (x.out[m].space == kSpaceNone) {
+                if (!addRes && !addPair) return fail(THIP_INVALID_ARGUMENT, "op %u: matrix %d has no destination", i, m);
+            } else if ((s = need(x.out[m], mul(op.M, x.N[m]) * 2, "out"))) {
+                return s;
+            }
+            if ((x.weights[m].offset & 15) || (x.qscale[m].offset & 3) || (x.qbias[m].offset & 3) || (x.bias[m].offset & 3) || (x.out[m].offset & 7)) {
+                return fail(THIP_INVALID_ARGUMENT, "op %u: misaligned operand of matrix %d", i, m);
+            }
+        }
+        if (anyBias != allBias) return fail(THIP_INVALID_ARGUMENT, "op %u: block biases on some matrices only", i);
+        if (pair && x.N[0] != x.N[1]) return fail(THIP_INVALID_ARGUMENT, "op %u: a pair of unequal widths", i);
+        if (addRes || addPair) {
+            if ((s = checkLooseRef(e, i, x.res)) || (s = checkLooseRef(e, i, x.add_out))) return s;
+            if (addRes && (s = need(x.res, mul(op.M, x.N[0]) * 2, "residual"))) return s;
+            if ((s = need(x.add_out, mul(op.M, x.N[0]) * 2, "sum"))) return s;
+            if ((x.res.offset & 7) || (x.add_out.offset & 7)) return fail(THIP_INVALID_ARGUMENT, "op %u: misaligned operand of the folded add", i);
+        }
+        if ((op.in0.offset & 15) != 0) return fail(THIP_INVALID_ARGUMENT, "op %u: misaligned input", i);
+        return THIP_OK;
+    }
+    case kKindDecMatmul: {
+        if (!positive({op.TB, op.M, op.K, op.Nn}) || op.M > kDecMaxRows || op.K % 8 != 0 || op.TB > 65535) return fail(THIP_INVALID_ARGUMENT, "op %u: bad batched-matmul extents", i);
+        if ((s = need(op.in0, mul(op.w0 ? 1 : op.TB, op.M, op.K) * 2, "in1"))) return s;
+        if ((s = need(op.weights, mul(op.w1 ? 1 : op.TB, op.Nn, op.K) * 2, "in2"))) return s;
+        if ((op.in0.offset & 15) || (op.weights.offset & 15) || (op.out.offset & 7)) return fail(THIP_INVALID_ARGUMENT, "op %u: misaligned operand", i);
+        return need(op.out, mul(op.TB, op.M, op.Nn) * 2, "out");
     }
     default: return fail(THIP_INVALID_ARGUMENT, "op %u has unknown kind %u", i, op.kind);
     }
