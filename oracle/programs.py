@@ -172,10 +172,12 @@ def _decoder_op(op, src, caches, batch, rows, columns=None):
         wq, scale, qbias = pr["weights"], pr["scale"], pr["qbias"]
         if columns is not None:
             wq, scale, qbias = wq[:, columns], scale[:, columns], qbias[:, columns]
-        w16 = orc.expand_weights(np.ascontiguousarray(wq), np.ascontiguousarray(scale), np.ascontiguousarray(qbias), block_size=pr["block"])
+        w16 = orc.expand_weights(np.ascontiguousarray(wq), np.ascontiguousarray(scale), np.ascontiguousarray(qbias), block_size=pr["block"],
+                                 output_min=pr.get("expand_min", orc.NO_CLAMP_MIN), output_max=pr.get("expand_max", orc.NO_CLAMP_MAX))
         x = src[0].reshape(R, wq.shape[0])
         # input2 of the matmul is the K x N expansion; summed over k in order like every oracle matmul
-        want = orc.matmul_bf16(x, w16, np.zeros(1, np.float32))[0]
+        want = orc.matmul_bf16(x, w16, np.zeros(1, np.float32), output_min=pr.get("output_min", orc.NO_CLAMP_MIN),
+                               output_max=pr.get("output_max", orc.NO_CLAMP_MAX))[0]
         return want, np.abs(_f64(x)) @ np.abs(_f64(w16))
     if op.kind in ("scores", "context"):
         kc, vc = caches
@@ -246,3 +248,32 @@ def eval_decoder_step(wl, rows=None):
     L = a["layers"]
     return dict(logits=tensors["logits"], columns=cols, k=np.stack([tensors["k%d" % l] for l in range(L)]),
                 v=np.stack([tensors["v%d" % l] for l in range(L)]))
+
+
+def check_grouped_linear(wl, outputs, compare_close, compare_exact):
+    """A grouped_linear_workload's outputs, each op on the inputs the GPU gave it (hidden intermediates of a
+    "pair_hidden" program are the oracle's own: what the add reads is then one rounding further from a binding)."""
+    tensors = {"x_in": wl.inputs[0]}
+    for name, arr in zip(wl.attrs["names"], outputs):
+        tensors[name] = arr
+    M = wl.inputs[0].shape[0]
+    rows = list(range(M))
+    for op in wl.attrs["ops"]:
+        src = [tensors[n] for n in op.inputs]
+        want, mag = _decoder_op(op, src, None, M, rows)
+        if op.out not in tensors:
+            tensors[op.out] = want  # never stored by the program
+            continue
+        got = tensors[op.out]
+        hidden_inputs = any(n not in wl.attrs["names"] and n != "x_in" for n in op.inputs)
+        if op.kind == "add" and not hidden_inputs:
+            compare_exact(got.reshape(want.shape), want, "%s %s" % (wl.name, op.out))
+        elif op.kind == "add":
+            # each hidden operand may be one bf16 step (2^-8 of its size) from the oracle's: the sum moves by at most
+            # the weighted steps of both, plus its own rounding
+            w0, w1 = (abs(float(v)) for v in orc.from_bf16(op.params["weights"])[:2])
+            room = 2.0 ** -8 * (w0 * np.abs(_f64(src[0])) + w1 * np.abs(_f64(src[1]))) + 2.0 ** -8 * np.abs(_f64(want))
+            bad = np.abs(_f64(got.reshape(want.shape)) - _f64(want)) > room.reshape(want.shape)
+            assert not bad.any(), "%s %s: %d elements beyond the propagated bound" % (wl.name, op.out, int(bad.sum()))
+        else:
+            compare_close(got.reshape(want.shape), want, "%s %s" % (wl.name, op.out), magnitude=mag.reshape(want.shape))

@@ -26,7 +26,7 @@ CONST = np.dtype([("offset", "<u8"), ("size", "<u8")])
 
 K_TRANSPOSE, K_IGEMM, K_FC_SKINNY, K_DW, K_MAXPOOL, K_AVGPOOL, K_ADD, K_FC_BF16, K_ADD_BF16, K_IM2COL_BF16, K_DW_BF16 = 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11
 K_AVGPOOL_BF16, K_EXPAND, K_ELTWISE, K_DEC_LINEAR, K_DEC_MATMUL = 12, 13, 14, 15, 16
-DEC_EXT = np.dtype([(n, REF, (3,)) for n in ["weights", "qscale", "qbias", "bias", "out"]] + [("N", "<i4", (3,)), ("reserved0", "<i4"), ("res", REF), ("add_out", REF)] +
+DEC_EXT = np.dtype([(n, REF, (3,)) for n in ["weights", "bias", "out"]] + [("N", "<i4", (3,)), ("has_qbias", "<i4"), ("res", REF), ("add_out", REF)] +
                    [(n, "<i4") for n in ["aw0", "aw1", "abias", "alo", "ahi"]] + [("reserved1", "<i4", (3,))])
 INT_BY_SIZE = {1: np.int8, 2: np.int16, 4: np.int32}
 OUT_NP = {1: np.int8, 2: np.int16, 3: np.int32}
@@ -296,19 +296,24 @@ def run(blob, binding_arrays):
             M, K, block, nmat, flags = int(op["M"]), int(op["K"]), int(op["gran"]), int(op["w0"]), int(op["w1"])
             x = view(op["in0"], M * K * 2).view(np.uint16).reshape(M, K)
             ext = np.frombuffer(view(op["table"], DEC_EXT.itemsize).tobytes(), dtype=DEC_EXT, count=1)[0]
-            G, kblocks = K // block, (K + 127) // 128
+            G, kblocks = K // block, K // 128
+            has_bias = int(ext["has_qbias"])
+            slot = 2048 + 64 + (64 if has_bias else 0)
             ys = []
             for m in range(nmat):
                 N = int(ext["N"][m])
                 tiles = N // 16
-                frag = view(ext["weights"][m], tiles * kblocks * 2048).view(np.int8).reshape(tiles, kblocks, 2, 4, 16, 2, 8)  # [t][b][p][g][c][j & 1][e]
+                slots = view(ext["weights"][m], tiles * kblocks * slot).reshape(tiles, kblocks, slot)
+                frag = np.ascontiguousarray(slots[:, :, :2048]).view(np.int8).reshape(tiles, kblocks, 2, 4, 16, 2, 8)  # [t][b][p][g][c][j & 1][e]
                 full = frag.transpose(0, 4, 1, 2, 5, 3, 6).reshape(N, kblocks * 128)  # [t, c][b, p, j & 1, g, e]: k = 128 b + 32 (2 p + (j & 1)) + 8 g + e
-                assert not full[:, K:].any()
-                sc = view(ext["qscale"][m], tiles * G * 64).view(np.float32).reshape(tiles, G, 16).transpose(1, 0, 2).reshape(G, N)
-                assert np.array_equal(orc.from_bf16(orc.to_bf16(sc)), sc), "block scales are bf16 values"
-                bi = (view(ext["qbias"][m], tiles * G * 64).view(np.float32).reshape(tiles, G, 16).transpose(1, 0, 2).reshape(G, N)
-                      if int(ext["qbias"][m]["space"]) else np.zeros((G, N), np.float32))
-                w16 = orc.expand_weights(np.ascontiguousarray(full[:, :K].T), orc.to_bf16(sc), np.ascontiguousarray(bi), block_size=block,
+                per_kb = np.ascontiguousarray(slots[:, :, 2048:2112]).view(np.float32).reshape(tiles, kblocks, 16).transpose(1, 0, 2).reshape(kblocks, N)
+                assert np.array_equal(orc.from_bf16(orc.to_bf16(per_kb)), per_kb), "block scales are bf16 values"
+                which = (np.arange(G) * block) // 128  # a quantisation block's scale is repeated in each of its k-blocks
+                assert np.array_equal(per_kb, per_kb[which][(np.arange(kblocks) * 128) // block])
+                sc = per_kb[which]
+                bi = (np.ascontiguousarray(slots[:, :, 2112:2176]).view(np.float32).reshape(tiles, kblocks, 16).transpose(1, 0, 2).reshape(kblocks, N)[which]
+                      if has_bias else np.zeros((G, N), np.float32))
+                w16 = orc.expand_weights(np.ascontiguousarray(full.T), orc.to_bf16(sc), np.ascontiguousarray(bi), block_size=block,
                                          output_min=int(op["bias0"]), output_max=int(op["scale0"]))
                 bias = view(ext["bias"][m], N * 4).view(np.float32)
                 assert np.all(bias == bias[0])

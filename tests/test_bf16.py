@@ -324,9 +324,10 @@ def test_gpu_bf16_avg_pool(device):
 @pytest.mark.gpu
 def test_gpu_expand_weights(device):
     """Block-quantized weights: expanded in registers by the matmul (decoder shapes at 1 and 32 tokens, split K, ragged
-    N, an expansion clamp), expanded at serialisation (many rows), and as a kernel of its own, whose result is bit-exact."""
+    N, an expansion clamp), by the grouped decode kernel where its shape rules hold (blocks of a multiple of 128 rows, N a
+    multiple of 16, at most 32 rows), expanded at serialisation (many rows), and as a kernel of its own, whose result is bit-exact."""
     f = lambda bits: np.abs(orc.from_bf16(bits).astype(np.float64))
-    cases = [(w.expand_weights_workload(), "q8"), (w.expand_weights_workload(M=1, K=1152, N=1024, block=128), "q8"),
+    cases = [(w.expand_weights_workload(), "q8"), (w.expand_weights_workload(M=1, K=1152, N=1024, block=128), "grouped"),
              (w.expand_weights_workload(M=32, K=6912, N=1152, block=64), "q8"), (w.expand_weights_workload(M=9, K=6912, N=200, block=128), "q8"), (w.expand_weights_workload(M=5, K=192, N=45, block=96, bias_pad=1), "q8"),
              (w.expand_weights_workload(M=7, K=128, N=70, expand_clamp=(-0.004, 0.006), clamp=(-0.05, 0.05)), "q8"),
              (w.expand_weights_workload(M=70, K=128, N=40, block=64), "folded"), (w.expand_weights_workload(M=2, K=64, N=33, fold=False, bias_pad=1), "own")]
@@ -341,7 +342,7 @@ def test_gpu_expand_weights(device):
             assert_bit_exact(got[1], want[1], wl.name + " expansion")
             assert families(kernels) == ["expand_weights_bf16", "transpose_i8", "fc_bf16"], kernels
         else:
-            assert families(kernels) == ["fc_bf16"], kernels
+            assert families(kernels) == ["dec_linear" if how == "grouped" else "fc_bf16"], kernels
 
 
 @pytest.mark.gpu

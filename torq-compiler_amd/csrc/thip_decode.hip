@@ -14,20 +14,69 @@ namespace thip {
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-constexpr int kDecWaves = 8;  // waves of a workgroup = ways K is split inside it
+constexpr int kDecWaves = 8;  // compute waves of a workgroup = ways K is split inside it; one more wave prefetches
 
 __device__ __forceinline__ unsigned ldsOffset(const void *p) {
     return (unsigned)(uintptr_t)(__attribute__((address_space(3))) const int8_t *)p;
 }
 
-// MR: groups of 16 input rows (1 or 2).  CH: k-blocks of a wave whose input rows are loaded together (their registers
-// are double-buffered when a wave owns more than CH k-blocks: 2 * CH * 16 * MR registers).  QB: the block biases exist.
+// 64 lanes x 4 bytes, global -> LDS (see dmaLoad16).
+__device__ __forceinline__ void dmaLoad4(const void *gptr, unsigned ldsAddr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dword %1, off" : : "s"(ldsAddr), "v"(gptr) : "memory", "m0");
+}
+
+// s_waitcnt vmcnt(n) for a wave-uniform run-time n (the instruction takes an immediate).
+__device__ __forceinline__ void waitVmcntDyn(int n) {
+#define THIP_VMCNT_CASE(k) \
+    case k: waitVmcnt<k>(); break;
+    switch (n) {
+        THIP_VMCNT_CASE(0) THIP_VMCNT_CASE(1) THIP_VMCNT_CASE(2) THIP_VMCNT_CASE(3) THIP_VMCNT_CASE(4) THIP_VMCNT_CASE(5) THIP_VMCNT_CASE(6) THIP_VMCNT_CASE(7)
+        THIP_VMCNT_CASE(8) THIP_VMCNT_CASE(9) THIP_VMCNT_CASE(10) THIP_VMCNT_CASE(11) THIP_VMCNT_CASE(12) THIP_VMCNT_CASE(13) THIP_VMCNT_CASE(14) THIP_VMCNT_CASE(15)
+        THIP_VMCNT_CASE(16) THIP_VMCNT_CASE(17) THIP_VMCNT_CASE(18) THIP_VMCNT_CASE(19) THIP_VMCNT_CASE(20) THIP_VMCNT_CASE(21) THIP_VMCNT_CASE(22) THIP_VMCNT_CASE(23)
+        THIP_VMCNT_CASE(24) THIP_VMCNT_CASE(25) THIP_VMCNT_CASE(26) THIP_VMCNT_CASE(27) THIP_VMCNT_CASE(28) THIP_VMCNT_CASE(29) THIP_VMCNT_CASE(30) THIP_VMCNT_CASE(31)
+        THIP_VMCNT_CASE(32) THIP_VMCNT_CASE(33) THIP_VMCNT_CASE(34) THIP_VMCNT_CASE(35) THIP_VMCNT_CASE(36) THIP_VMCNT_CASE(37) THIP_VMCNT_CASE(38) THIP_VMCNT_CASE(39)
+        THIP_VMCNT_CASE(40) THIP_VMCNT_CASE(41) THIP_VMCNT_CASE(42) THIP_VMCNT_CASE(43) THIP_VMCNT_CASE(44) THIP_VMCNT_CASE(45) THIP_VMCNT_CASE(46) THIP_VMCNT_CASE(47)
+    default: break;  // 48 or more may stay in flight: more than a wave of these kernels ever has
+    }
+#undef THIP_VMCNT_CASE
+}
+
+// The prefetch wave of a workgroup: one 4-byte read of every 128-byte line of this workgroup's share of
+// [base, base + bytes), into 256 bytes of LDS that nobody reads (`sinkLds`).  The lines arrive in the last-level
+// cache, where the next launch finds them.  LDS-DMA loads, because a load into a register returns whenever it
+// likes: the compiler, which takes the result of an asm statement for available at once, gives that register to
+// the next address computation, and the data that arrives later then overwrites an address.  The caller waits for
+// vmcnt(0) before the wave ends (the LDS belongs to the workgroup until then).
+__device__ __forceinline__ void prefetchLines(const void *base, long long bytes, int lane, unsigned sinkLds) {
+    if (!base || bytes <= 0) return;
+    const long long lines = (bytes + 127) >> 7;
+    const long long groups = (long long)gridDim.x * gridDim.y;
+    const long long per = (lines + groups - 1) / groups;
+    const long long first = ((long long)blockIdx.y * gridDim.x + blockIdx.x) * per;
+    const long long last = first + per < lines ? first + per : lines;
+    for (long long l = first + lane; l < last; l += 64) dmaLoad4((const int8_t *)base + l * 128, sinkLds);
+}
+constexpr int kDecSinkBytes = 256;
+
+constexpr int kDecLdsSlot = 2048 + 128;  // a k-block's weights, scales and (room for) biases in LDS
+
+// MR: groups of 16 input rows (1 or 2).  XLDS: the input rows come through LDS as well (at most four rows): then every
+// global load of a wave is an LDS-DMA load issued up front and each k-block is computed as soon as it has landed.
+// Otherwise the rows come through registers, CH k-blocks at a time, double-buffered.  QB: the slots carry block biases.
 // QC: the expansion clamps.
-template <int MR, int CH, bool QB, bool QC>
-__global__ __launch_bounds__(kDecWaves * 64) void dec_linear(DecLinearArgs p, FastDiv qblk) {
+template <int MR, int CH, bool XLDS, bool QB, bool QC>
+__global__ __launch_bounds__((kDecWaves + 1) * 64) void dec_linear(DecLinearArgs p) {
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    if (wave == kDecWaves) {
+        const int kb8 = ((p.K >> 7) + kDecWaves - 1) / kDecWaves;  // the compute waves' regions come first (see below)
+        const unsigned computeLds = (unsigned)kDecWaves * (unsigned)kb8 * (unsigned)((XLDS ? p.M * 256 : 0) + (p.pair ? 2 : 1) * kDecLdsSlot);
+        if (!(p.ablate & 4)) prefetchLines(p.prefetch, p.prefetch_bytes, lane, ldsOffset(smem) + computeLds);
+        __syncthreads();
+        waitVmcnt<0>();
+        return;
+    }
     const int c = lane & 15, g = lane >> 4;
     // the tile of this workgroup: (matrix, 16 columns of it); a pair owns the same columns of both matrices
     int tile = (int)blockIdx.x, seg = 0;
@@ -42,110 +91,115 @@ __global__ __launch_bounds__(kDecWaves * 64) void dec_linear(DecLinearArgs p, Fa
         }
     }
     const int nmat = p.pair ? 2 : 1;
-    const int kblocks = (p.K + 127) >> 7;
+    const int kblocks = p.K >> 7;  // K % 128 == 0
     const int nkb = wave < kblocks ? (kblocks - wave + kDecWaves - 1) / kDecWaves : 0;  // k-blocks wave, wave + 8, ...
     const int maxkb = (kblocks + kDecWaves - 1) / kDecWaves;
-    const int G = p.K / p.qblock;
-    const unsigned regionBytes = (unsigned)(maxkb * nmat) * 2048u;
+    const int slotBytes = kDecSlotBytes + (QB ? 64 : 0);
+    const int xRowBytes = XLDS ? p.M * 256 : 0;  // a k-block of the input rows in LDS
+    const unsigned regionBytes = (unsigned)maxkb * (unsigned)(xRowBytes + nmat * kDecLdsSlot);
     int8_t *region = smem + (size_t)wave * regionBytes;
+    int8_t *slots = region + (size_t)maxkb * xRowBytes;
     const unsigned regionLds = ldsOffset(smem) + (unsigned)wave * regionBytes;
+    const unsigned slotsLds = regionLds + (unsigned)(maxkb * xRowBytes);
     const int8_t *wsrc[2];
-    const float *qs[2], *qbp[2];
     {
         const int s0 = p.pair ? 0 : seg, s1 = p.pair ? 1 : seg;
         wsrc[0] = s0 == 0 ? p.w[0] : s0 == 1 ? p.w[1] : p.w[2];
         wsrc[1] = s1 == 0 ? p.w[0] : s1 == 1 ? p.w[1] : p.w[2];
-        qs[0] = s0 == 0 ? p.qscale[0] : s0 == 1 ? p.qscale[1] : p.qscale[2];
-        qs[1] = s1 == 0 ? p.qscale[0] : s1 == 1 ? p.qscale[1] : p.qscale[2];
-        qbp[0] = s0 == 0 ? p.qbias[0] : s0 == 1 ? p.qbias[1] : p.qbias[2];
-        qbp[1] = s1 == 0 ? p.qbias[0] : s1 == 1 ? p.qbias[1] : p.qbias[2];
     }
-    // the wave's whole share of the weights, one burst: 2 KiB per k-block and matrix, straight into its LDS region
-    for (int i = 0; i < nkb; i++) {
+    if (XLDS) {
+        // lane l brings 16 bytes of row l >> 4: a k-block of one row is 16 lanes x 16 bytes
+        for (int i = 0; i < nkb; i++) {
+            const int kb = wave + kDecWaves * i;
+            if (lane < 16 * p.M) dmaLoad16(p.x + (size_t)(lane >> 4) * p.K + kb * 128 + (lane & 15) * 8, regionLds + (unsigned)(i * xRowBytes));
+        }
+    }
+    // the wave's whole share of the weights, one burst: per k-block and matrix 2 KiB and the scales, straight into LDS
+    for (int i = 0; i < ((p.ablate & 1) ? 0 : nkb); i++) {
         const int kb = wave + kDecWaves * i;
         for (int m = 0; m < nmat; m++) {
-            const int8_t *src = wsrc[m] + (((size_t)tile * kblocks + kb) * 2) * 1024 + (size_t)lane * 16;
-            const unsigned dst = regionLds + (unsigned)(i * nmat + m) * 2048u;
-            dmaLoad16(src, dst);
-            dmaLoad16(src + 1024, dst + 1024u);
+            const int8_t *src = wsrc[m] + ((size_t)tile * kblocks + kb) * slotBytes;
+            const unsigned dst = slotsLds + (unsigned)(i * nmat + m) * kDecLdsSlot;
+            dmaLoad16(src + (size_t)lane * 16, dst);
+            dmaLoad16(src + 1024 + (size_t)lane * 16, dst + 1024u);
+            if (lane < (QB ? 32 : 16)) dmaLoad4(src + 2048 + (size_t)lane * 4, dst + 2048u);
         }
     }
-    struct XBuf {
-        v4i x[CH][4][MR];
-        float sc[CH][2], bi[CH][2];
-    };
-    // Loads only; a k-block the wave does not have, a row beyond M and a k beyond K read nothing and feed zeros.
-    auto loadChunk = [&](int ch, XBuf &b) {
-#pragma unroll
-        for (int u = 0; u < CH; u++) {
-            const int i = ch * CH + u;
-            const bool on = i < nkb;
-            const int kb = wave + kDecWaves * i;
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int k = kb * 128 + 32 * j + 8 * g;
-#pragma unroll
-                for (int mr = 0; mr < MR; mr++) {
-                    const int row = c + 16 * mr;
-                    b.x[u][j][mr] = (on && row < p.M && k < p.K) ? *(const v4i *)(p.x + (size_t)row * p.K + k) : v4i{0, 0, 0, 0};
-                }
-            }
-            // the 128 rows of a k-block lie in one quantisation block (qblock % 128 == 0)
-            const size_t gi = on ? (size_t)fastDiv((uint32_t)(kb * 128), qblk) : 0;
-#pragma unroll
-            for (int m = 0; m < 2; m++) {
-                if (m < nmat) {
-                    const size_t at = ((size_t)tile * G + gi) * 16 + c;
-                    b.sc[u][m] = on ? qs[m][at] : 0.0f;
-                    b.bi[u][m] = (QB && on) ? qbp[m][at] : 0.0f;
-                } else {
-                    b.sc[u][m] = 0.0f;
-                    b.bi[u][m] = 0.0f;
-                }
-            }
-        }
-    };
     v4f acc[2][MR];
 #pragma unroll
     for (int m = 0; m < 2; m++) {
 #pragma unroll
         for (int mr = 0; mr < MR; mr++) acc[m][mr] = v4f{0.0f, 0.0f, 0.0f, 0.0f};
     }
-    auto computeChunk = [&](int ch, const XBuf &b) {
+    // one k-block of one matrix: 32 weights of the lane expanded, four MFMAs per row group
+    auto kblock = [&](int i, int m, const v4i (&xp)[4][MR]) {
+        const int8_t *slot = slots + (size_t)(i * nmat + m) * kDecLdsSlot;
+        const v4i p0 = *(const v4i *)(slot + lane * 16), p1 = *(const v4i *)(slot + 1024 + lane * 16);
+        const float sc = *(const float *)(slot + 2048 + c * 4);
+        const float bi = QB ? *(const float *)(slot + 2048 + 64 + c * 4) : 0.0f;
+        const int dw[8] = {p0[0], p0[1], p0[2], p0[3], p1[0], p1[1], p1[2], p1[3]};
 #pragma unroll
-        for (int u = 0; u < CH; u++) {
-            const int i = ch * CH + u;
-            if (i >= nkb) break;
+        for (int j = 0; j < 4; j++) {
+            int o[4];
+            expandQ8<QC>(dw[2 * j], sc, bi, p.qlo, p.qhi, &o[0], &o[1]);
+            expandQ8<QC>(dw[2 * j + 1], sc, bi, p.qlo, p.qhi, &o[2], &o[3]);
+            const v8bf wfrag = __builtin_bit_cast(v8bf, v4i{o[0], o[1], o[2], o[3]});
 #pragma unroll
-            for (int m = 0; m < 2; m++) {
-                if (m >= nmat) break;
-                const int8_t *wl = region + (size_t)(i * nmat + m) * 2048 + (size_t)lane * 16;
-                const v4i p0 = *(const v4i *)wl, p1 = *(const v4i *)(wl + 1024);
-                const int dw[8] = {p0[0], p0[1], p0[2], p0[3], p1[0], p1[1], p1[2], p1[3]};
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    int o[4];
-                    expandQ8<QC>(dw[2 * j], b.sc[u][m], b.bi[u][m], p.qlo, p.qhi, &o[0], &o[1]);
-                    expandQ8<QC>(dw[2 * j + 1], b.sc[u][m], b.bi[u][m], p.qlo, p.qhi, &o[2], &o[3]);
-                    const v8bf wfrag = __builtin_bit_cast(v8bf, v4i{o[0], o[1], o[2], o[3]});
-#pragma unroll
-                    for (int mr = 0; mr < MR; mr++) {
-                        acc[m][mr] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wfrag, __builtin_bit_cast(v8bf, b.x[u][j][mr]), acc[m][mr], 0, 0, 0);
-                    }
-                }
+            for (int mr = 0; mr < MR; mr++) {
+                acc[m][mr] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wfrag, __builtin_bit_cast(v8bf, xp[j][mr]), acc[m][mr], 0, 0, 0);
             }
         }
     };
-    const int nchunks = (nkb + CH - 1) / CH;
-    XBuf b0, b1;
-    loadChunk(0, b0);
-    waitVmcnt<0>();  // the DMA burst (and the first chunk's rows) has landed; the compiler counts only its own loads
-    for (int ch = 0; ch < nchunks; ch += 2) {
-        if (ch + 1 < nchunks) loadChunk(ch + 1, b1);
-        computeChunk(ch, b0);
-        if (ch + 1 < nchunks) {
-            if (ch + 2 < nchunks) loadChunk(ch + 2, b0);
-            computeChunk(ch + 1, b1);
+    if constexpr (XLDS) {
+        const int xrow = (c < p.M ? c : 0) * 256 + g * 16;  // lanes of rows the input does not have read row 0 (never stored)
+        for (int i = 0; i < ((p.ablate & 2) ? 0 : nkb); i++) {
+            waitVmcntDyn((p.ablate & 1) ? 0 : (nkb - 1 - i) * 3 * nmat);  // everything up to this k-block has landed
+            v4i xp[4][MR];
+#pragma unroll
+            for (int j = 0; j < 4; j++) xp[j][0] = *(const v4i *)(region + (size_t)i * xRowBytes + xrow + j * 64);
+            kblock(i, 0, xp);
+            if (nmat > 1) kblock(i, 1, xp);
+        }
+    } else {
+        struct XBuf {
+            v4i x[CH][4][MR];
+        };
+        // Loads only; a k-block the wave does not have and a row beyond M read nothing and feed zeros.
+        auto loadChunk = [&](int ch, XBuf &b) {
+#pragma unroll
+            for (int u = 0; u < CH; u++) {
+                const int i = ch * CH + u;
+                const int kb = wave + kDecWaves * i;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+#pragma unroll
+                    for (int mr = 0; mr < MR; mr++) {
+                        const int row = c + 16 * mr;
+                        b.x[u][j][mr] = (i < nkb && row < p.M) ? *(const v4i *)(p.x + (size_t)row * p.K + kb * 128 + 32 * j + 8 * g) : v4i{0, 0, 0, 0};
+                    }
+                }
+            }
+        };
+        auto computeChunk = [&](int ch, const XBuf &b) {
+#pragma unroll
+            for (int u = 0; u < CH; u++) {
+                const int i = ch * CH + u;
+                if (i >= nkb) break;
+                kblock(i, 0, b.x[u]);
+                if (nmat > 1) kblock(i, 1, b.x[u]);
+            }
+        };
+        const int nchunks = (nkb + CH - 1) / CH;
+        XBuf b0, b1;
+        loadChunk(0, b0);
+        waitVmcnt<0>();  // the DMA burst (and the first chunk's rows) has landed; the compiler counts only its own loads
+        for (int ch = 0; ch < nchunks; ch += 2) {
+            if (ch + 1 < nchunks) loadChunk(ch + 1, b1);
+            computeChunk(ch, b0);
+            if (ch + 1 < nchunks) {
+                if (ch + 2 < nchunks) loadChunk(ch + 2, b0);
+                computeChunk(ch + 1, b1);
+            }
         }
     }
     // the waves' partial sums meet in LDS: each leaves its own in its own region (its weights are used up)
@@ -165,6 +219,16 @@ __global__ __launch_bounds__(kDecWaves * 64) void dec_linear(DecLinearArgs p, Fa
     const int s0 = p.pair ? 0 : seg;
     const int Nseg = s0 == 0 ? p.N[0] : s0 == 1 ? p.N[1] : p.N[2];
     const int n = tile * 16 + 4 * g;
+    // what the epilogue reads from memory, issued before the sums are collected
+    v4f bias4[2];
+#pragma unroll
+    for (int m = 0; m < 2; m++) {
+        const int sm = p.pair ? m : seg;
+        const float *bias = sm == 0 ? p.bias[0] : sm == 1 ? p.bias[1] : p.bias[2];
+        bias4[m] = m < nmat ? *(const v4f *)(bias + n) : v4f{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    v2i rv = v2i{0, 0};
+    if (p.add_mode == 1) rv = *(const v2i *)(p.res + (size_t)row * Nseg + n);
     uint16_t y[2][4];
 #pragma unroll
     for (int m = 0; m < 2; m++) {
@@ -175,11 +239,10 @@ __global__ __launch_bounds__(kDecWaves * 64) void dec_linear(DecLinearArgs p, Fa
             s += t;
         }
         const int sm = p.pair ? m : seg;
-        const float *bias = sm == 0 ? p.bias[0] : sm == 1 ? p.bias[1] : p.bias[2];
         uint16_t *out = sm == 0 ? p.out[0] : sm == 1 ? p.out[1] : p.out[2];
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            const float t0 = s[e] + bias[n + e];
+            const float t0 = s[e] + bias4[m][e];
             y[m][e] = bf16Bits(t0 < p.lo ? p.lo : (t0 > p.hi ? p.hi : t0));
         }
         if (out) {
@@ -189,7 +252,6 @@ __global__ __launch_bounds__(kDecWaves * 64) void dec_linear(DecLinearArgs p, Fa
     if (p.add_mode == 0) return;
     uint16_t z[4];
     if (p.add_mode == 1) {
-        const v2i rv = *(const v2i *)(p.res + (size_t)row * Nseg + n);
         const uint16_t r[4] = {(uint16_t)rv[0], (uint16_t)((uint32_t)rv[0] >> 16), (uint16_t)rv[1], (uint16_t)((uint32_t)rv[1] >> 16)};
 #pragma unroll
         for (int e = 0; e < 4; e++) {
@@ -202,65 +264,79 @@ __global__ __launch_bounds__(kDecWaves * 64) void dec_linear(DecLinearArgs p, Fa
     *(v2i *)(p.add_out + (size_t)row * Nseg + n) = v2i{(int)((uint32_t)z[0] | ((uint32_t)z[1] << 16)), (int)((uint32_t)z[2] | ((uint32_t)z[3] << 16))};
 }
 
-template <int MR, int CH, bool QB, bool QC>
+template <int MR, int CH, bool XLDS, bool QB, bool QC>
 static hipError_t launchDecLinearT(const DecLinearArgs &a, int tiles, size_t lds, const LaunchCtx &ctx) {
-    auto kernel = dec_linear<MR, CH, QB, QC>;
+    auto kernel = dec_linear<MR, CH, XLDS, QB, QC>;
     static std::once_flag once;
     static hipError_t configured = hipSuccess;
     std::call_once(once, [&] { configured = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); });
     if (configured != hipSuccess) return configured;
-    THIP_ENQUEUE(ctx, kernelLabel("dec_linear", {MR, CH, (int)QB, (int)QC, a.pair ? 2 : a.nseg, a.add_mode}), kernel, dim3((unsigned)tiles), dim3(kDecWaves * 64), lds, a,
-                 makeFastDiv((uint32_t)a.qblock));
+    THIP_ENQUEUE(ctx, kernelLabel("dec_linear", {MR, CH, (int)XLDS, (int)QB, (int)QC, a.pair ? 2 : a.nseg, a.add_mode}), kernel, dim3((unsigned)tiles), dim3((kDecWaves + (a.prefetch ? 1 : 0)) * 64), lds, a);
     return hipGetLastError();
 }
 
-// LDS a launch needs: every wave's share of the weights (the partial sums reuse it).
-static size_t decLinearLds(int K, int nmat) {
-    const int kblocks = (K + 127) / 128, maxkb = (kblocks + kDecWaves - 1) / kDecWaves;
-    return (size_t)kDecWaves * maxkb * nmat * 2048;
+// LDS a launch needs: every wave's share of the weights, and of the input rows when they come through LDS (the
+// partial sums reuse it).
+static size_t decLinearLds(int K, int nmat, int xRows) {
+    const int kblocks = K / 128, maxkb = (kblocks + kDecWaves - 1) / kDecWaves;
+    return (size_t)kDecWaves * maxkb * (size_t)(xRows * 256 + nmat * kDecLdsSlot) + kDecSinkBytes;  // and the prefetch wave's sink
+}
+constexpr size_t kDecMaxLds = 152 * 1024;
+constexpr int kDecLdsRows = 4;  // up to this many input rows may come through LDS
+
+template <bool QB, bool QC>
+static hipError_t launchDecLinearQ(const DecLinearArgs &a, int tiles, const LaunchCtx &ctx) {
+    const int nmat = a.pair ? 2 : 1;
+    if (a.M <= kDecLdsRows && decLinearLds(a.K, nmat, a.M) <= kDecMaxLds) return launchDecLinearT<1, 1, true, QB, QC>(a, tiles, decLinearLds(a.K, nmat, a.M), ctx);
+    const size_t lds = decLinearLds(a.K, nmat, 0);
+    if (a.M <= 16) return launchDecLinearT<1, 2, false, QB, QC>(a, tiles, lds, ctx);
+    return launchDecLinearT<2, 1, false, QB, QC>(a, tiles, lds, ctx);
 }
 
 hipError_t launchDecLinear(const DecLinearArgs &a, const LaunchCtx &ctx) {
-    if (!a.x || a.M <= 0 || a.M > kDecMaxRows || a.K <= 0 || a.K % 8 != 0 || a.qblock <= 0 || a.qblock % 128 != 0 || a.K % a.qblock != 0) return hipErrorInvalidValue;
+    if (!a.x || a.M <= 0 || a.M > kDecMaxRows || a.K <= 0 || a.K % 128 != 0 || a.qblock <= 0 || a.qblock % 128 != 0 || a.K % a.qblock != 0) return hipErrorInvalidValue;
     if (a.nseg < 1 || a.nseg > kDecMaxSegments || (a.pair && a.nseg != 2) || (((uintptr_t)a.x) & 15)) return hipErrorInvalidValue;
     if (a.add_mode < 0 || a.add_mode > 2 || (a.add_mode == 1 && (a.nseg != 1 || !a.res)) || (a.add_mode == 2 && !a.pair) || (a.pair && a.add_mode != 2)) return hipErrorInvalidValue;
     if (a.add_mode != 0 && (!a.add_out || (((uintptr_t)a.add_out) & 7) || (a.res && (((uintptr_t)a.res) & 7)))) return hipErrorInvalidValue;
+    if (a.prefetch_bytes < 0 || (a.prefetch_bytes > 0 && (!a.prefetch || (((uintptr_t)a.prefetch) & 3)))) return hipErrorInvalidValue;
     long long tiles = 0;
-    bool anyBias = false;
     for (int s = 0; s < a.nseg; s++) {
-        if (!a.w[s] || !a.qscale[s] || !a.bias[s] || a.N[s] <= 0 || a.N[s] % 16 != 0) return hipErrorInvalidValue;
-        if ((((uintptr_t)a.w[s]) & 15) || (((uintptr_t)a.qscale[s]) & 3) || (((uintptr_t)a.qbias[s]) & 3) || (((uintptr_t)a.bias[s]) & 3) || (((uintptr_t)a.out[s]) & 7)) return hipErrorInvalidValue;
+        if (!a.w[s] || !a.bias[s] || a.N[s] <= 0 || a.N[s] % 16 != 0) return hipErrorInvalidValue;
+        if ((((uintptr_t)a.w[s]) & 15) || (((uintptr_t)a.bias[s]) & 15) || (((uintptr_t)a.out[s]) & 7)) return hipErrorInvalidValue;
         if (!a.out[s] && a.add_mode == 0) return hipErrorInvalidValue;  // a result nobody receives
-        anyBias = anyBias || a.qbias[s] != nullptr;
         tiles += a.N[s] / 16;
-    }
-    for (int s = 0; s < a.nseg; s++) {
-        if (anyBias && !a.qbias[s]) return hipErrorInvalidValue;  // all matrices of a launch with block biases, or none
     }
     if (a.pair) {
         if (a.N[0] != a.N[1]) return hipErrorInvalidValue;
         tiles = a.N[0] / 16;
     }
-    const size_t lds = decLinearLds(a.K, a.pair ? 2 : 1);
-    if (tiles <= 0 || tiles > 65535 || lds > 152 * 1024) return hipErrorInvalidValue;
+    if (tiles <= 0 || tiles > 65535 || decLinearLds(a.K, a.pair ? 2 : 1, 0) > kDecMaxLds) return hipErrorInvalidValue;
     const bool clamp = !(a.qlo == -INFINITY && a.qhi == INFINITY);
     const int t = (int)tiles;
-    if (a.M <= 16) {
-        if (clamp) return anyBias ? launchDecLinearT<1, 2, true, true>(a, t, lds, ctx) : launchDecLinearT<1, 2, false, true>(a, t, lds, ctx);
-        return anyBias ? launchDecLinearT<1, 2, true, false>(a, t, lds, ctx) : launchDecLinearT<1, 2, false, false>(a, t, lds, ctx);
+    if (ctx.tuning->decAblate) {
+        DecLinearArgs b = a;
+        b.ablate = ctx.tuning->decAblate;
+        return launchDecLinearQ<false, false>(b, t, ctx);
     }
-    if (clamp) return anyBias ? launchDecLinearT<2, 1, true, true>(a, t, lds, ctx) : launchDecLinearT<2, 1, false, true>(a, t, lds, ctx);
-    return anyBias ? launchDecLinearT<2, 1, true, false>(a, t, lds, ctx) : launchDecLinearT<2, 1, false, false>(a, t, lds, ctx);
+    if (clamp) return a.has_qbias ? launchDecLinearQ<true, true>(a, t, ctx) : launchDecLinearQ<false, true>(a, t, ctx);
+    return a.has_qbias ? launchDecLinearQ<true, false>(a, t, ctx) : launchDecLinearQ<false, false>(a, t, ctx);
 }
 
 // dec_matmul: a workgroup owns 16 columns (rows of w) of one batch element; its eight waves split K in steps of 32
 // (wave, wave + 8, ...), each lane loading 16 bytes of its weight row and of its input row per step; the partial
 // sums meet in LDS.  A wave's loads of up to ST steps are all issued before the first MFMA.
 template <int MR, int ST>
-__global__ __launch_bounds__(kDecWaves * 64) void dec_matmul(DecMatmulArgs p) {
+__global__ __launch_bounds__((kDecWaves + 1) * 64) void dec_matmul(DecMatmulArgs p) {
     __shared__ v4f red[kDecWaves][MR][64];
+    __shared__ int sink[kDecSinkBytes / 4];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    if (wave == kDecWaves) {
+        prefetchLines(p.prefetch, p.prefetch_bytes, lane, ldsOffset(sink));
+        __syncthreads();
+        waitVmcnt<0>();
+        return;
+    }
     const int c = lane & 15, g = lane >> 4;
     const int n0 = (int)blockIdx.x * 16, b = (int)blockIdx.y;
     const uint16_t *a = p.a + (size_t)b * p.a_stride, *w = p.w + (size_t)b * p.w_stride;
@@ -320,19 +396,20 @@ hipError_t launchDecMatmul(const DecMatmulArgs &a, const LaunchCtx &ctx) {
     if (!a.a || !a.w || !a.out || a.B <= 0 || a.B > 65535 || a.M <= 0 || a.M > kDecMaxRows || a.K <= 0 || a.K % 8 != 0 || a.N <= 0) return hipErrorInvalidValue;
     if (a.a_stride < 0 || a.w_stride < 0 || a.out_stride < 0 || a.a_stride % 8 != 0 || a.w_stride % 8 != 0) return hipErrorInvalidValue;
     if (((((uintptr_t)a.a) | ((uintptr_t)a.w)) & 15) || (((uintptr_t)a.out) & (a.N % 4 == 0 ? 7 : 1)) || (a.N % 4 == 0 && a.out_stride % 4 != 0)) return hipErrorInvalidValue;
+    if (a.prefetch_bytes < 0 || (a.prefetch_bytes > 0 && (!a.prefetch || (((uintptr_t)a.prefetch) & 3)))) return hipErrorInvalidValue;
     const long long tiles = ((long long)a.N + 15) / 16;
     if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
     const dim3 grid((unsigned)tiles, (unsigned)a.B);
     // steps of 32 per wave: up to four are one round of loads
     const int perWave = ((a.K + 31) / 32 + kDecWaves - 1) / kDecWaves;
     if (a.M <= 16) {
-        if (perWave <= 1) THIP_ENQUEUE(ctx, "dec_matmul<1,1>", (dec_matmul<1, 1>), grid, dim3(kDecWaves * 64), 0, a);
-        else if (perWave <= 2) THIP_ENQUEUE(ctx, "dec_matmul<1,2>", (dec_matmul<1, 2>), grid, dim3(kDecWaves * 64), 0, a);
-        else THIP_ENQUEUE(ctx, "dec_matmul<1,4>", (dec_matmul<1, 4>), grid, dim3(kDecWaves * 64), 0, a);
+        if (perWave <= 1) THIP_ENQUEUE(ctx, "dec_matmul<1,1>", (dec_matmul<1, 1>), grid, dim3((kDecWaves + (a.prefetch ? 1 : 0)) * 64), 0, a);
+        else if (perWave <= 2) THIP_ENQUEUE(ctx, "dec_matmul<1,2>", (dec_matmul<1, 2>), grid, dim3((kDecWaves + (a.prefetch ? 1 : 0)) * 64), 0, a);
+        else THIP_ENQUEUE(ctx, "dec_matmul<1,4>", (dec_matmul<1, 4>), grid, dim3((kDecWaves + (a.prefetch ? 1 : 0)) * 64), 0, a);
     } else {
-        if (perWave <= 1) THIP_ENQUEUE(ctx, "dec_matmul<2,1>", (dec_matmul<2, 1>), grid, dim3(kDecWaves * 64), 0, a);
-        else if (perWave <= 2) THIP_ENQUEUE(ctx, "dec_matmul<2,2>", (dec_matmul<2, 2>), grid, dim3(kDecWaves * 64), 0, a);
-        else THIP_ENQUEUE(ctx, "dec_matmul<2,4>", (dec_matmul<2, 4>), grid, dim3(kDecWaves * 64), 0, a);
+        if (perWave <= 1) THIP_ENQUEUE(ctx, "dec_matmul<2,1>", (dec_matmul<2, 1>), grid, dim3((kDecWaves + (a.prefetch ? 1 : 0)) * 64), 0, a);
+        else if (perWave <= 2) THIP_ENQUEUE(ctx, "dec_matmul<2,2>", (dec_matmul<2, 2>), grid, dim3((kDecWaves + (a.prefetch ? 1 : 0)) * 64), 0, a);
+        else THIP_ENQUEUE(ctx, "dec_matmul<2,4>", (dec_matmul<2, 4>), grid, dim3((kDecWaves + (a.prefetch ? 1 : 0)) * 64), 0, a);
     }
     return hipGetLastError();
 }

@@ -93,14 +93,16 @@ enum Kind : uint32_t {
     kKindEltwise = 14,
     // Decode-shaped bf16 linear on block-quantized int8 weights (torq_hl.expand_weights folded into torq_hl.matmul),
     // up to three matrices on the same M <= 32 input rows in one launch, the torq_hl.add behind it folded in:
-    // in0 = x [M][K] bf16, gran = rows per quantisation block (a multiple of 128), w0 = number of matrices, w1 =
-    // DecLinearFlags, output_min / output_max = float bits of the matmuls' clamp, bias0 / scale0 = float bits of the
-    // expansions' clamp, table = a DecLinearExt in the constant segment (the per-matrix operands), out = the first
-    // buffer the launch writes, Nn = its row length.
+    // in0 = x [M][K] bf16 (K % 128 == 0), gran = rows per quantisation block (a multiple of 128), w0 = number of
+    // matrices, w1 = DecLinearFlags, output_min / output_max = float bits of the matmuls' clamp, bias0 / scale0 =
+    // float bits of the expansions' clamp, table = a DecLinearExt in the constant segment (the per-matrix operands),
+    // out = the first buffer the launch writes, Nn = its row length.  scale / TR: see kKindDecMatmul.
     kKindDecLinear = 15,
     // Batch of small bf16 matmuls against a run-time operand held [N][K]: in0 = a [TB][M][K] (w0 != 0: one [M][K] for
     // every batch), weights = [TB][Nn][K] (w1 != 0: shared), out [TB][M][Nn]; M <= 32; bias0 = float bits of the one
-    // bias, output_min / output_max = float bits of the clamp.
+    // bias, output_min / output_max = float bits of the clamp.  Both decode kinds: scale = constants that the NEXT
+    // record streams (space none: nothing), TS = their size in 128-byte lines: the launch touches them so that they
+    // are in the last-level cache by the time that record runs.
     kKindDecMatmul = 16,
 };
 
@@ -111,19 +113,19 @@ enum DecLinearFlags : int32_t {
     kDecResFirst = 8,
 };
 
-// Per-matrix operands of a kKindDecLinear record.  weights: int8 in the dec16 fragment order (thip_kernels.h),
-// qscale / qbias: float [N / 16][K / gran][16] (qbias.space none: every bias is zero), bias: float [N], out: bf16
-// [M][N] (space none: not stored, the folded add is its only reader).
+// Per-matrix operands of a kKindDecLinear record.  weights: int8 in the dec16 slot order with the block scales (and,
+// has_qbias, block biases) inline (thip_kernels.h), bias: float [N], out: bf16 [M][N] (space none: not stored, the
+// folded add is its only reader).
 struct DecLinearExt {
-    DescRef weights[3], qscale[3], qbias[3], bias[3], out[3];
+    DescRef weights[3], bias[3], out[3];
     int32_t N[3];
-    int32_t reserved0;
+    int32_t has_qbias;
     DescRef res, add_out;
     int32_t aw0, aw1;           // bf16 bits of the add's two weights
     int32_t abias, alo, ahi;    // float bits of its bias and clamp
     int32_t reserved1[3];
 };
-static_assert(sizeof(DecLinearExt) == 15 * 16 + 16 + 2 * 16 + 32, "DecLinearExt layout");
+static_assert(sizeof(DecLinearExt) == 9 * 16 + 16 + 2 * 16 + 32, "DecLinearExt layout");
 
 // Variants of kKindIgemm: how the A (activation) tile is gathered.
 enum IgemmLoader : uint32_t {

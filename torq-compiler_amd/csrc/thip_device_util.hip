@@ -205,6 +205,7 @@ Tuning tuningFromEnvironment() {
     t.noFcWide = flag("THIP_NO_FC_WIDE");
     t.maxpoolGeneric = flag("THIP_MAXPOOL_GENERIC");
     t.addGeneric = flag("THIP_ADD_GENERIC");
+    if (const char *v = getenv("THIP_DEC_ABLATE")) t.decAblate = atoi(v);
     return t;
 }
 

@@ -43,6 +43,7 @@ struct Tuning {
     bool noFcWide = false;          // THIP_NO_FC_WIDE
     bool addGeneric = false;        // THIP_ADD_GENERIC: the quantised add always through the 64-bit ACT stage
     bool maxpoolGeneric = false;    // THIP_MAXPOOL_GENERIC: the any-window max pool kernel also for 2 x 2 stride 2
+    int decAblate = 0;              // THIP_DEC_ABLATE: parts of dec_linear left out, for timing experiments (wrong results)
 };
 Tuning tuningFromEnvironment();
 
@@ -204,20 +205,22 @@ hipError_t launchFcBf16(const FcBf16Args &a, const LaunchCtx &ctx);
 // workgroup owns 16 output columns: it brings its whole share of the weights into LDS with one burst of LDS-DMA
 // loads, its eight waves split K, and their partial sums meet in LDS.
 //
-// Weight layout ("dec16"): for column tile t (16 columns), k-block b (128 input rows) and piece p (0, 1): 64 lanes x
-// 16 bytes, lane l = column l & 15 and k-group g = l >> 4; bytes 0..7 of the lane are rows 32 (2 p) + 8 g + 0..7 of
-// the k-block, bytes 8..15 rows 32 (2 p + 1) + 8 g + 0..7 (what one lane feeds to two v_mfma_f32_16x16x32_bf16).
-// Zero padded to whole k-blocks.  Scales (and biases) as float [tile][K / qblock][16].
+// Weight layout ("dec16"): for column tile t (16 columns) and k-block b (128 input rows) one slot of kDecSlotBytes
+// (+ 64 with block biases): first 2 KiB of weights, piece p (0, 1) = 64 lanes x 16 bytes, lane l = column l & 15 and
+// k-group g = l >> 4; bytes 0..7 of the lane are rows 32 (2 p) + 8 g + 0..7 of the k-block, bytes 8..15 rows
+// 32 (2 p + 1) + 8 g + 0..7 (what one lane feeds to two v_mfma_f32_16x16x32_bf16); zero padded to whole k-blocks.
+// Then the block's 16 scales as floats (the scale of quantisation block b * 128 / qblock: repeated per k-block, so
+// that a workgroup's whole share is one contiguous stretch), then, if the record has block biases, its 16 biases.
 constexpr int kDecMaxSegments = 3;
 constexpr int kDecMaxRows = 32;
+constexpr int kDecSlotBytes = 2048 + 64;
 struct DecLinearArgs {
     const uint16_t *x;  // [M][K] bf16
     int32_t M, K, qblock;
     int32_t nseg;       // matrices of this launch, 1..3
     int32_t pair;       // 1: two matrices of equal N; a workgroup owns the same 16 columns of both and adds its two results
+    int32_t has_qbias;  // the slots carry block biases (all matrices of a launch, or none)
     const int8_t *w[kDecMaxSegments];
-    const float *qscale[kDecMaxSegments];
-    const float *qbias[kDecMaxSegments];  // null: every bias is zero (symmetric quantisation)
     const float *bias[kDecMaxSegments];   // [N] per matrix
     uint16_t *out[kDecMaxSegments];       // [M][N] per matrix; null: not stored (the fused add is its only reader)
     int32_t N[kDecMaxSegments];           // multiples of 16
@@ -229,13 +232,23 @@ struct DecLinearArgs {
     const uint16_t *res;
     uint16_t *add_out;
     float aw0, aw1, abias, alo, ahi;
+    // constants the NEXT record will stream (its weights): this launch reads one 4-byte word of every 128-byte line of
+    // them, which brings them into the last-level cache while its own work runs (null: nothing)
+    const void *prefetch;
+    int64_t prefetch_bytes;
+    int32_t ablate;  // timing experiments only (THIP_DEC_ABLATE; results are wrong): 1 no weight loads, 2 no arithmetic, 4 no prefetch wave work
 };
+inline int decSlotBytes(bool hasBias) { return kDecSlotBytes + (hasBias ? 64 : 0); }
 // Byte offset of int8 weight (n, k) in the dec16 order, for K padded to `kblocks` blocks of 128.
-inline size_t decWeightOffset(int n, int k, int kblocks) {
+inline size_t decWeightOffset(int n, int k, int kblocks, bool hasBias) {
     const int t = n >> 4, c = n & 15, b = k >> 7, kk = k & 127, j = kk >> 5, g = (kk & 31) >> 3, e = kk & 7;
-    return ((((size_t)t * kblocks + b) * 2 + (size_t)(j >> 1)) * 64 + (size_t)(g * 16 + c)) * 16 + (size_t)((j & 1) * 8 + e);
+    return ((size_t)t * kblocks + b) * decSlotBytes(hasBias) + ((size_t)(j >> 1) * 64 + (size_t)(g * 16 + c)) * 16 + (size_t)((j & 1) * 8 + e);
 }
-inline size_t decWeightBytes(int N, int K) { return (size_t)((N + 15) / 16) * ((K + 127) / 128) * 2048; }
+// Byte offset of the scale (which = 0) or bias (which = 1) of column n for k-block b.
+inline size_t decScaleOffset(int n, int b, int kblocks, bool hasBias, int which) {
+    return ((size_t)(n >> 4) * kblocks + b) * decSlotBytes(hasBias) + 2048 + (size_t)which * 64 + (size_t)(n & 15) * 4;
+}
+inline size_t decWeightBytes(int N, int K, bool hasBias) { return (size_t)((N + 15) / 16) * ((K + 127) / 128) * decSlotBytes(hasBias); }
 hipError_t launchDecLinear(const DecLinearArgs &a, const LaunchCtx &ctx);
 
 // dec_matmul: out[b][m][n] = bf16(clamp(sum_k a[b][m][k] * w[b][n][k] + bias)) for a batch of small matmuls whose
@@ -249,6 +262,8 @@ struct DecMatmulArgs {
     int32_t B, M, K, N;
     int64_t a_stride, w_stride, out_stride;
     float bias, lo, hi;
+    const void *prefetch;  // as in DecLinearArgs
+    int64_t prefetch_bytes;
 };
 hipError_t launchDecMatmul(const DecMatmulArgs &a, const LaunchCtx &ctx);
 

@@ -172,6 +172,15 @@ thip_status_t checkOpFootprint(const DescriptorView *e, uint32_t i) {
     };
     const uint64_t outElem = op.out_dtype == THIP_DTYPE_I32 ? 4 : op.out_dtype == THIP_DTYPE_I16 ? 2 : 1;
     thip_status_t s = THIP_OK;
+    // decode kinds: `scale` names constants a launch only touches (the next record's weights), TS lines of 128 bytes
+    // from there on, possibly across several constants: they must lie inside the constant segment
+    auto prefetchRangeOk = [&]() {
+        if (op.scale.space == kSpaceNone) return true;
+        if (op.scale.space != kSpaceConst || op.TS <= 0 || (op.scale.offset & 3)) return false;
+        const uint64_t segment = e->header.total_size - e->header.data_offset;
+        const uint64_t start = e->consts[op.scale.index].offset + op.scale.offset, bytes = ((uint64_t)op.TS - 1) * 128 + 4;
+        return start <= segment && bytes <= segment - start;
+    };
     if (op.shift < 0 || op.shift > 63) return fail(THIP_INVALID_ARGUMENT, "op %u: shift %d is outside 0..63", i, op.shift);
     if (op.pre_shift != 0 && (op.pre_shift < 0 || op.pre_shift > 30 || (int64_t)op.shift + op.pre_shift != 33 || op.shift < 0 || op.shift > 63 ||
                               (op.kind != kKindIgemm && op.kind != kKindDepthwise))) {
@@ -370,7 +379,7 @@ thip_status_t checkOpFootprint(const DescriptorView *e, uint32_t i) {
         return need(op.out, mul(op.M, op.Nn) * 2, "out");
     }
     case kKindDecLinear: {
-        if (!positive({op.M, op.K}) || op.M > kDecMaxRows || op.K % 8 != 0 || op.gran == 0 || op.gran % 128 != 0 || (uint32_t)op.K % op.gran != 0 ||
+        if (!positive({op.M, op.K}) || op.M > kDecMaxRows || op.K % 128 != 0 || op.gran == 0 || op.gran % 128 != 0 || (uint32_t)op.K % op.gran != 0 ||
             op.w0 < 1 || op.w0 > kDecMaxSegments || (op.w1 & ~(kDecPair | kDecAddResidual | kDecAddPair | kDecResFirst))) {
             return fail(THIP_INVALID_ARGUMENT, "op %u: bad grouped-linear record", i);
         }
@@ -382,31 +391,24 @@ thip_status_t checkOpFootprint(const DescriptorView *e, uint32_t i) {
         if ((op.table.offset & 7) != 0) return fail(THIP_INVALID_ARGUMENT, "op %u: misaligned per-matrix operands", i);
         DecLinearExt x;
         memcpy(&x, e->blob + e->header.data_offset + e->consts[op.table.index].offset + op.table.offset, sizeof(x));
-        const uint64_t G = (uint64_t)op.K / op.gran;
-        bool anyBias = false, allBias = true;
+        if (x.has_qbias != 0 && x.has_qbias != 1) return fail(THIP_INVALID_ARGUMENT, "op %u: bad block-bias flag", i);
         for (int m = 0; m < op.w0; m++) {
-            const DescRef *refs[] = {&x.weights[m], &x.qscale[m], &x.qbias[m], &x.bias[m], &x.out[m]};
+            const DescRef *refs[] = {&x.weights[m], &x.bias[m], &x.out[m]};
             for (const DescRef *r : refs) {
                 if ((s = checkLooseRef(e, i, *r))) return s;
             }
             if (x.N[m] <= 0 || x.N[m] % 16 != 0 || x.N[m] > (1 << 24)) return fail(THIP_INVALID_ARGUMENT, "op %u: matrix %d has %d columns", i, m, x.N[m]);
-            const uint64_t tiles = (uint64_t)x.N[m] / 16;
-            if ((s = need(x.weights[m], decWeightBytes(x.N[m], op.K), "weights"))) return s;
-            if ((s = need(x.qscale[m], tiles * G * 64, "block scales"))) return s;
-            if (x.qbias[m].space != kSpaceNone && (s = need(x.qbias[m], tiles * G * 64, "block biases"))) return s;
-            anyBias = anyBias || x.qbias[m].space != kSpaceNone;
-            allBias = allBias && x.qbias[m].space != kSpaceNone;
+            if ((s = need(x.weights[m], decWeightBytes(x.N[m], op.K, x.has_qbias != 0), "weights"))) return s;
             if ((s = need(x.bias[m], (uint64_t)x.N[m] * 4, "bias"))) return s;
             if (x.out[m].space == kSpaceNone) {
                 if (!addRes && !addPair) return fail(THIP_INVALID_ARGUMENT, "op %u: matrix %d has no destination", i, m);
             } else if ((s = need(x.out[m], mul(op.M, x.N[m]) * 2, "out"))) {
                 return s;
             }
-            if ((x.weights[m].offset & 15) || (x.qscale[m].offset & 3) || (x.qbias[m].offset & 3) || (x.bias[m].offset & 3) || (x.out[m].offset & 7)) {
+            if ((x.weights[m].offset & 15) || (x.bias[m].offset & 15) || (x.out[m].offset & 7)) {
                 return fail(THIP_INVALID_ARGUMENT, "op %u: misaligned operand of matrix %d", i, m);
             }
         }
-        if (anyBias != allBias) return fail(THIP_INVALID_ARGUMENT, "op %u: block biases on some matrices only", i);
         if (pair && x.N[0] != x.N[1]) return fail(THIP_INVALID_ARGUMENT, "op %u: a pair of unequal widths", i);
         if (addRes || addPair) {
             if ((s = checkLooseRef(e, i, x.res)) || (s = checkLooseRef(e, i, x.add_out))) return s;
@@ -415,6 +417,7 @@ thip_status_t checkOpFootprint(const DescriptorView *e, uint32_t i) {
             if ((x.res.offset & 7) || (x.add_out.offset & 7)) return fail(THIP_INVALID_ARGUMENT, "op %u: misaligned operand of the folded add", i);
         }
         if ((op.in0.offset & 15) != 0) return fail(THIP_INVALID_ARGUMENT, "op %u: misaligned input", i);
+        if (!prefetchRangeOk()) return fail(THIP_INVALID_ARGUMENT, "op %u: bad prefetch range", i);
         return THIP_OK;
     }
     case kKindDecMatmul: {
@@ -422,6 +425,7 @@ thip_status_t checkOpFootprint(const DescriptorView *e, uint32_t i) {
         if ((s = need(op.in0, mul(op.w0 ? 1 : op.TB, op.M, op.K) * 2, "in1"))) return s;
         if ((s = need(op.weights, mul(op.w1 ? 1 : op.TB, op.Nn, op.K) * 2, "in2"))) return s;
         if ((op.in0.offset & 15) || (op.weights.offset & 15) || (op.out.offset & 7)) return fail(THIP_INVALID_ARGUMENT, "op %u: misaligned operand", i);
+        if (!prefetchRangeOk()) return fail(THIP_INVALID_ARGUMENT, "op %u: bad prefetch range", i);
         return need(op.out, mul(op.TB, op.M, op.Nn) * 2, "out");
     }
     default: return fail(THIP_INVALID_ARGUMENT, "op %u has unknown kind %u", i, op.kind);

@@ -925,3 +925,67 @@ def decoder_step_workload(batch=1, layers=26, hidden=1152, heads=4, head_dim=256
     attrs = dict(ops=ops, trace=trace, batch=batch, layers=layers, heads=heads, head_dim=head_dim, cache_len=cache_len,
                  hidden=hidden, ffn=ffn, vocab=vocab, weight_bytes=weight_bytes, expose=expose)
     return Workload("decoder_step_b%d_l%d" % (batch, layers), p, inputs, outputs, 2 * macs, bytes_, attrs)
+
+
+def grouped_linear_workload(M=3, K=256, N=64, mode="single", block=128, zero_points=False, clamp=None, expand_clamp=None, seed=1050):
+    """Small programs of the shapes a decoder layer is made of, every result an output binding: mode "single" one
+    linear; "concat" three linears (N, N / 2, N / 2 columns) on the same rows; "pair" two linears whose results an
+    add joins (both also stored); "pair_hidden" the same with the two results intermediates that only the add
+    reads; "residual" / "residual_first" a linear and the add of its result with (behind / in front of) the input
+    rows (K == N).  zero_points: asymmetric quantisation (block biases -zp * scale, as the matmul patterns produce
+    them).  attrs: ops (DecoderOp list), names (output names in binding order)."""
+    rng = np.random.default_rng(seed)
+    p = Program()
+    x_in = to_bf16(rng.standard_normal((M, K)))
+    bx = p.binding(0, (M, K), np.uint16)
+    zero = np.zeros(1, dtype=np.float32)
+    lo, hi = NO_CLAMP if clamp is None else (float_bits(clamp[0]), float_bits(clamp[1]))
+    elo, ehi = NO_CLAMP if expand_clamp is None else (float_bits(expand_clamp[0]), float_bits(expand_clamp[1]))
+    ops, names, outputs = [], [], []
+
+    def out_binding(name, shape):
+        names.append(name)
+        outputs.append((shape, np.uint16))
+        return p.binding(len(names), shape, np.uint16)
+
+    def linear(name, n, init):
+        wq = rng.integers(-128, 128, size=(K, n), dtype=np.int8)
+        scale = to_bf16(rng.uniform(0.75, 1.25, size=(K // block, n)) / (73.9 * np.sqrt(K)))
+        qbias = np.zeros((K // block, n), dtype=np.float32)
+        if zero_points:
+            qbias = (-rng.integers(-8, 9, size=(K // block, n))).astype(np.float32) * from_bf16_np(scale)
+        w16 = p.expand_weights(wq, scale, qbias, block_size=block, output_min=elo, output_max=ehi)
+        y = p.matmul(bx, w16, zero, init=init, output_zp=0, output_min=lo, output_max=hi, shift=0)
+        ops.append(DecoderOp("linear", name, ["x_in"], (M, n), weights=wq, scale=scale, qbias=qbias, block=block, output_min=lo, output_max=hi,
+                             expand_min=elo, expand_max=ehi))
+        return y
+
+    def add(name, a_name, a, b_name, b, shape):
+        wts = to_bf16(np.array([0.75, -0.5], dtype=np.float32))
+        bias = np.array([0.125], dtype=np.float32)
+        y = p.add(a, b, wts, bias, init=out_binding(name, shape), output_zp=0, output_min=NO_CLAMP[0], output_max=NO_CLAMP[1], shift_factor=0)
+        ops.append(DecoderOp("add", name, [a_name, b_name], shape, weights=wts, bias=bias))
+        return y
+
+    if mode == "single":
+        linear("y", N, out_binding("y", (M, N)))
+    elif mode == "concat":
+        for i, n in enumerate((N, N // 2, N // 2)):
+            linear("y%d" % i, n, out_binding("y%d" % i, (M, n)))
+    elif mode in ("pair", "pair_hidden"):
+        hidden = mode == "pair_hidden"
+        g = linear("g", N, p.tensor((M, N), np.uint16) if hidden else out_binding("g", (M, N)))
+        u = linear("u", N, p.tensor((M, N), np.uint16) if hidden else out_binding("u", (M, N)))
+        add("a", "g", g, "u", u, (M, N))
+    elif mode in ("residual", "residual_first"):
+        assert K == N
+        y = linear("y", N, out_binding("y", (M, N)))
+        if mode == "residual":
+            add("z", "y", y, "x_in", bx, (M, N))
+        else:
+            add("z", "x_in", bx, "y", y, (M, N))
+    else:
+        raise ValueError(mode)
+    attrs = dict(ops=ops, names=names)
+    name = "grouped_%s_%dx%dx%d_b%d%s" % (mode, M, K, N, block, "_zp" if zero_points else "")
+    return Workload(name, p, [x_in], outputs, 2 * M * K * N, 0, attrs)
