@@ -82,9 +82,57 @@ def workload_table(pkg):
 
 
 def network_table(pkg):
-    """Whole-network workloads (benchmark configuration 3); selectable with --workload, reported as images/s."""
+    """Whole-network workloads (benchmark configurations 3 and 4); selectable with --workload."""
     w = pkg.workloads
-    return {"mbv2_b%d" % b: (lambda b=b: w.mobilenet_v2_workload(batch=b), "mfma") for b in (1, 32, 256)}
+    table = {"mbv2_b%d" % b: (lambda b=b: w.mobilenet_v2_workload(batch=b), "mfma") for b in (1, 32, 256)}
+    table.update({"decoder_b%d" % b: (lambda b=b: w.decoder_step_workload(batch=b), "hbm") for b in DECODER_BATCHES})
+    return table
+
+
+DECODER_BATCHES = (1, 32)
+# What a decode step is priced against: every int8 weight of the 26 layers and of the vocabulary projection once per
+# step, whatever the batch (26 * 26 836 992 + 301 989 888 bytes).
+DECODER_WEIGHT_BYTES = 999751680
+
+
+def decoder_parity(pkg, dev, batch):
+    """The decoder step checked against the oracle: a two-layer twin of the program at the same batch with every
+    intermediate exposed, each op on the inputs the GPU gave it (<= 1 bf16 ULP, the adds bit-exact; every sequence at
+    one token, the first and last otherwise), with the full-width vocabulary projection on sampled columns."""
+    from oracle import programs as prog
+    wl = pkg.workloads.decoder_step_workload(batch=batch, layers=2, expose=True)
+    o = Loaded(pkg, dev, wl)
+    try:
+        o.exe.run_device(o.ptrs, o.lens)
+        got = [o.output(i) for i in range(len(wl.outputs))]
+        prog.check_decoder_step(wl, got, prog.assert_bf16_close, prog.assert_bit_exact, rows=None if batch <= 2 else [0, batch - 1])
+        return True
+    except AssertionError as e:
+        print("decoder step differs from the oracle: %s" % e, file=sys.stderr)
+        return False
+    finally:
+        o.close()
+
+
+def decoder_row(pkg, dev, batch, pre_ms, check):
+    """One decode step (26 layers + vocabulary projection) as ONE graph-replayed program: ms per step, steps and
+    tokens per second, and the int8 weight bytes per second against HBM's 8 TB/s.  1 GB of weights per step: every
+    step finds them cold.  The ops between these (normalisation, rotary embedding, softmax, the gate's activation)
+    are not on this path, so the figure is for the linears and attention matmuls only."""
+    o = Loaded(pkg, dev, pkg.workloads.decoder_step_workload(batch=batch))
+    o.precondition(pre_ms)
+    o.run(5)
+    ms = min(o.run(20) for _ in range(3))
+    names = o.exe.op_kernels()
+    row = {"ms": round(ms, 4), "steps_per_s": round(1e3 / ms, 1), "tokens_per_s": round(batch * 1e3 / ms, 1), "kernels": len(names),
+           "scope": "linears + attention matmuls + residual adds + vocabulary projection only", "weight_bytes": o.wl.attrs["weight_bytes"],
+           "GB/s": round(o.wl.attrs["weight_bytes"] / (ms * 1e-3) / 1e9, 1), "frac": round(o.wl.attrs["weight_bytes"] / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 5),
+           "kernel_families": sorted(set(k.split("<")[0] for k in names))}
+    assert o.wl.attrs["weight_bytes"] == DECODER_WEIGHT_BYTES
+    o.close()
+    if check:
+        row["parity_checked"] = decoder_parity(pkg, dev, batch)
+    return row
 
 
 class Loaded:
@@ -197,10 +245,12 @@ def roofline(wl, bound, ms, name=None):
 
 def verify_sample(loaded):
     """Checks the GPU result of the timed workload against the oracle (sampled rows for the big GEMMs)."""
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
-    from helpers import oracle_eval, oracle_network
     from oracle import oracle as orc
+    from oracle.programs import assert_bf16_close, eval_network as oracle_network, eval_workload as oracle_eval
     wl = loaded.wl
+    if wl.name.startswith("decoder_step"):
+        import torq_compiler_amd as pkg
+        return decoder_parity(pkg, loaded.dev, wl.attrs["batch"])
     got = loaded.output()
     if wl.name.startswith("mobilenet_v2"):
         n = min(4, wl.inputs[0].shape[0])
@@ -215,7 +265,6 @@ def verify_sample(loaded):
         return bool(np.array_equal(got[rows], want))
     if wl.name.startswith("fcbf16") or wl.name.startswith("expandmm"):
         # tolerance row: one bf16 ULP, or the fp32 reordering error where the sum cancels
-        from helpers import assert_bf16_close
         f = lambda bits: np.abs(orc.from_bf16(bits).astype(np.float64))
         if wl.name.startswith("expandmm"):
             a = wl.attrs
@@ -508,8 +557,7 @@ def main():
     mbv2 = {}
     if not args.no_others:
         if not args.no_cpu:
-            sys.path.insert(0, os.path.join(ROOT, "tests"))
-            from helpers import oracle_network
+            from oracle.programs import eval_network as oracle_network
         for batch in (1, 32, 256):
             o = Loaded(pkg, dev, pkg.workloads.mobilenet_v2_workload(batch=batch))
             o.precondition(pre_ms)
@@ -525,6 +573,13 @@ def main():
             ok = ok and same if same is not None else ok
             o.close()
 
+    decoder = {}
+    if not args.no_others:
+        for batch in DECODER_BATCHES:
+            decoder["batch_%d" % batch] = decoder_row(pkg, dev, batch, pre_ms, not args.no_cpu)
+            if not args.no_cpu:
+                ok = ok and decoder["batch_%d" % batch]["parity_checked"]
+
     result = {
         "metric": "int8 GOP/s (fully_connected with fused requant), 1 MAC = 2 ops",
         "value": round(wl.ops / (wall_ms * 1e-3) / 1e9, 1),
@@ -536,7 +591,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16" if args.workload.startswith(("fcbf16", "expandmm")) else "int8",
+        "dtype": "bf16" if args.workload.startswith(("fcbf16", "expandmm", "decoder")) else "int8",
         "data": "synthetic",
         "config": {"workload": args.workload, "kernels": kernels, "parity_checked": ok,
                    "algorithmic_ops": wl.ops, "algorithmic_bytes": wl.bytes, "buffer_sets": main_sets,
@@ -551,6 +606,8 @@ def main():
         result["per_op"] = per_op
     if mbv2:
         result["mobilenet_v2_int8_224"] = mbv2
+    if decoder:
+        result["decoder_step"] = decoder
     dev.close()
     print(json.dumps(result))
     if ok is False:

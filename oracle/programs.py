@@ -203,25 +203,26 @@ def vocabulary_sample(vocab, count=2048, seed=7):
     return np.unique(cols)
 
 
-def check_decoder_step(wl, outputs, compare_close, compare_exact):
+def check_decoder_step(wl, outputs, compare_close, compare_exact, rows=None):
     """Every op of an exposed decoder-step workload (expose=True) checked on the inputs the GPU gave it: the
     oracle evaluates the op on the GPU's own intermediates, so one op's rounding does not reach the next comparison.
     outputs: the program's output arrays (logits, new keys, new values, trace).  compare_close(got, want, what,
-    magnitude) for the matmuls (tolerance rows), compare_exact(got, want, what) for the adds."""
+    magnitude) for the matmuls (tolerance rows), compare_exact(got, want, what) for the adds.  rows: the sequences
+    to check (all when None; a sequence's step depends on its own row and caches only)."""
     a = wl.attrs
     assert a["expose"], "needs the workload built with expose=True"
     logits, knew, vnew, trace = outputs
     x_in, kc, vc = wl.inputs
     M = a["batch"]
-    tensors = {"x_in": x_in}
+    rows = list(range(M)) if rows is None else list(rows)
+    tensors = {"x_in": x_in[rows]}
     for name, (off, shape) in a["trace"].items():
-        tensors[name] = trace[off:off + int(np.prod(shape))].reshape(shape)
+        tensors[name] = trace[off:off + int(np.prod(shape))].reshape(shape)[rows]
     for l in range(a["layers"]):
-        tensors["k%d" % l] = knew[l]
-        tensors["v%d" % l] = vnew[l]
+        tensors["k%d" % l] = knew[l][rows]
+        tensors["v%d" % l] = vnew[l][rows]
     cols = vocabulary_sample(a["vocab"])
-    tensors["logits"] = logits[:, cols]
-    rows = list(range(M))
+    tensors["logits"] = logits[rows][:, cols]
     for op in wl.attrs["ops"]:
         src = [tensors[n] for n in op.inputs]
         want, mag = _decoder_op(op, src, (kc, vc), M, rows, columns=cols if op.out == "logits" else None)
