@@ -14,7 +14,8 @@ namespace thip {
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-constexpr int kDecWaves = 8;  // compute waves of a workgroup = ways K is split inside it; one more wave prefetches
+constexpr int kDecWaves = 8;      // waves of a dec_matmul workgroup = ways K is split inside it
+constexpr int kDecMaxWaves = 16;  // dec_linear: between 8 and 16, one k-block each where K allows (DecLinearArgs::nwaves)
 
 __device__ __forceinline__ unsigned ldsOffset(const void *p) {
     return (unsigned)(uintptr_t)(__attribute__((address_space(3))) const int8_t *)p;
@@ -41,23 +42,6 @@ __device__ __forceinline__ void waitVmcntDyn(int n) {
 #undef THIP_VMCNT_CASE
 }
 
-// The prefetch wave of a workgroup: one 4-byte read of every 128-byte line of this workgroup's share of
-// [base, base + bytes), into 256 bytes of LDS that nobody reads (`sinkLds`).  The lines arrive in the last-level
-// cache, where the next launch finds them.  LDS-DMA loads, because a load into a register returns whenever it
-// likes: the compiler, which takes the result of an asm statement for available at once, gives that register to
-// the next address computation, and the data that arrives later then overwrites an address.  The caller waits for
-// vmcnt(0) before the wave ends (the LDS belongs to the workgroup until then).
-__device__ __forceinline__ void prefetchLines(const void *base, long long bytes, int lane, unsigned sinkLds) {
-    if (!base || bytes <= 0) return;
-    const long long lines = (bytes + 127) >> 7;
-    const long long groups = (long long)gridDim.x * gridDim.y;
-    const long long per = (lines + groups - 1) / groups;
-    const long long first = ((long long)blockIdx.y * gridDim.x + blockIdx.x) * per;
-    const long long last = first + per < lines ? first + per : lines;
-    for (long long l = first + lane; l < last; l += 64) dmaLoad4((const int8_t *)base + l * 128, sinkLds);
-}
-constexpr int kDecSinkBytes = 256;
-
 constexpr int kDecLdsSlot = 2048 + 128;  // a k-block's weights, scales and (room for) biases in LDS
 
 // MR: groups of 16 input rows (1 or 2).  XLDS: the input rows come through LDS as well (at most four rows): then every
@@ -65,18 +49,11 @@ constexpr int kDecLdsSlot = 2048 + 128;  // a k-block's weights, scales and (roo
 // Otherwise the rows come through registers, CH k-blocks at a time, double-buffered.  QB: the slots carry block biases.
 // QC: the expansion clamps.
 template <int MR, int CH, bool XLDS, bool QB, bool QC>
-__global__ __launch_bounds__((kDecWaves + 1) * 64) void dec_linear(DecLinearArgs p) {
+__global__ __launch_bounds__(kDecMaxWaves * 64) void dec_linear(DecLinearArgs p) {
     extern __shared__ __attribute__((aligned(16))) int8_t smem[];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    if (wave == kDecWaves) {
-        const int kb8 = ((p.K >> 7) + kDecWaves - 1) / kDecWaves;  // the compute waves' regions come first (see below)
-        const unsigned computeLds = (unsigned)kDecWaves * (unsigned)kb8 * (unsigned)((XLDS ? p.M * 256 : 0) + (p.pair ? 2 : 1) * kDecLdsSlot);
-        if (!(p.ablate & 4)) prefetchLines(p.prefetch, p.prefetch_bytes, lane, ldsOffset(smem) + computeLds);
-        __syncthreads();
-        waitVmcnt<0>();
-        return;
-    }
+    const int NW = p.nwaves;  // waves of this workgroup: k-blocks wave, wave + NW, ... are this wave's
     const int c = lane & 15, g = lane >> 4;
     // the tile of this workgroup: (matrix, 16 columns of it); a pair owns the same columns of both matrices
     int tile = (int)blockIdx.x, seg = 0;
@@ -92,8 +69,8 @@ __global__ __launch_bounds__((kDecWaves + 1) * 64) void dec_linear(DecLinearArgs
     }
     const int nmat = p.pair ? 2 : 1;
     const int kblocks = p.K >> 7;  // K % 128 == 0
-    const int nkb = wave < kblocks ? (kblocks - wave + kDecWaves - 1) / kDecWaves : 0;  // k-blocks wave, wave + 8, ...
-    const int maxkb = (kblocks + kDecWaves - 1) / kDecWaves;
+    const int nkb = wave < kblocks ? (kblocks - wave + NW - 1) / NW : 0;  
+    const int maxkb = (kblocks + NW - 1) / NW;
     const int slotBytes = kDecSlotBytes + (QB ? 64 : 0);
     const int xRowBytes = XLDS ? p.M * 256 : 0;  // a k-block of the input rows in LDS
     const unsigned regionBytes = (unsigned)maxkb * (unsigned)(xRowBytes + nmat * kDecLdsSlot);
@@ -110,13 +87,13 @@ __global__ __launch_bounds__((kDecWaves + 1) * 64) void dec_linear(DecLinearArgs
     if (XLDS) {
         // lane l brings 16 bytes of row l >> 4: a k-block of one row is 16 lanes x 16 bytes
         for (int i = 0; i < nkb; i++) {
-            const int kb = wave + kDecWaves * i;
+            const int kb = wave + NW * i;
             if (lane < 16 * p.M) dmaLoad16(p.x + (size_t)(lane >> 4) * p.K + kb * 128 + (lane & 15) * 8, regionLds + (unsigned)(i * xRowBytes));
         }
     }
     // the wave's whole share of the weights, one burst: per k-block and matrix 2 KiB and the scales, straight into LDS
     for (int i = 0; i < ((p.ablate & 1) ? 0 : nkb); i++) {
-        const int kb = wave + kDecWaves * i;
+        const int kb = wave + NW * i;
         for (int m = 0; m < nmat; m++) {
             const int8_t *src = wsrc[m] + ((size_t)tile * kblocks + kb) * slotBytes;
             const unsigned dst = slotsLds + (unsigned)(i * nmat + m) * kDecLdsSlot;
@@ -169,7 +146,7 @@ __global__ __launch_bounds__((kDecWaves + 1) * 64) void dec_linear(DecLinearArgs
 #pragma unroll
             for (int u = 0; u < CH; u++) {
                 const int i = ch * CH + u;
-                const int kb = wave + kDecWaves * i;
+                const int kb = wave + NW * i;
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
 #pragma unroll
@@ -234,7 +211,7 @@ __global__ __launch_bounds__((kDecWaves + 1) * 64) void dec_linear(DecLinearArgs
     for (int m = 0; m < 2; m++) {
         if (m >= nmat) break;
         v4f s = v4f{0.0f, 0.0f, 0.0f, 0.0f};
-        for (int w = 0; w < kDecWaves; w++) {
+        for (int w = 0; w < NW; w++) {
             const v4f t = ((const v4f *)(smem + (size_t)w * regionBytes))[(m * MR + mr) * 64 + lane];
             s += t;
         }
@@ -271,34 +248,49 @@ static hipError_t launchDecLinearT(const DecLinearArgs &a, int tiles, size_t lds
     static hipError_t configured = hipSuccess;
     std::call_once(once, [&] { configured = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); });
     if (configured != hipSuccess) return configured;
-    THIP_ENQUEUE(ctx, kernelLabel("dec_linear", {MR, CH, (int)XLDS, (int)QB, (int)QC, a.pair ? 2 : a.nseg, a.add_mode}), kernel, dim3((unsigned)tiles), dim3((kDecWaves + (a.prefetch ? 1 : 0)) * 64), lds, a);
+    THIP_ENQUEUE(ctx, kernelLabel("dec_linear", {MR, CH, (int)XLDS, (int)QB, (int)QC, a.pair ? 2 : a.nseg, a.add_mode}), kernel, dim3((unsigned)tiles), dim3((unsigned)a.nwaves * 64), lds, a);
     return hipGetLastError();
 }
 
 // LDS a launch needs: every wave's share of the weights, and of the input rows when they come through LDS (the
 // partial sums reuse it).
-static size_t decLinearLds(int K, int nmat, int xRows) {
-    const int kblocks = K / 128, maxkb = (kblocks + kDecWaves - 1) / kDecWaves;
-    return (size_t)kDecWaves * maxkb * (size_t)(xRows * 256 + nmat * kDecLdsSlot) + kDecSinkBytes;  // and the prefetch wave's sink
+static size_t decLinearLds(int K, int nmat, int xRows, int nwaves) {
+    const int kblocks = K / 128, maxkb = (kblocks + nwaves - 1) / nwaves;
+    return (size_t)nwaves * maxkb * (size_t)(xRows * 256 + nmat * kDecLdsSlot);
+}
+// Waves per workgroup: one k-block each where K has between 8 and 16 of them, 16 for a longer K (a wave's
+// arithmetic is the launch's critical path: 128 x 16 weights expanded per k-block and matrix).
+int decLinearWaves(int K) {
+    const int kblocks = K / 128;
+    return kblocks < kDecWaves ? kDecWaves : (kblocks > kDecMaxWaves ? kDecMaxWaves : kblocks);
 }
 constexpr size_t kDecMaxLds = 152 * 1024;
 constexpr int kDecLdsRows = 4;  // up to this many input rows may come through LDS
 
 template <bool QB, bool QC>
-static hipError_t launchDecLinearQ(const DecLinearArgs &a, int tiles, const LaunchCtx &ctx) {
+static hipError_t launchDecLinearQ(const DecLinearArgs &in, int tiles, const LaunchCtx &ctx) {
+    DecLinearArgs a = in;
     const int nmat = a.pair ? 2 : 1;
-    if (a.M <= kDecLdsRows && decLinearLds(a.K, nmat, a.M) <= kDecMaxLds) return launchDecLinearT<1, 1, true, QB, QC>(a, tiles, decLinearLds(a.K, nmat, a.M), ctx);
-    const size_t lds = decLinearLds(a.K, nmat, 0);
+    if (a.M <= kDecLdsRows) {
+        // the input rows through LDS as well, with the most waves whose regions still fit
+        for (int nw = a.nwaves; nw >= kDecWaves; nw--) {
+            if (decLinearLds(a.K, nmat, a.M, nw) > kDecMaxLds) continue;
+            a.nwaves = nw;
+            return launchDecLinearT<1, 1, true, QB, QC>(a, tiles, decLinearLds(a.K, nmat, a.M, nw), ctx);
+        }
+    }
+    const size_t lds = decLinearLds(a.K, nmat, 0, a.nwaves);
     if (a.M <= 16) return launchDecLinearT<1, 2, false, QB, QC>(a, tiles, lds, ctx);
     return launchDecLinearT<2, 1, false, QB, QC>(a, tiles, lds, ctx);
 }
 
-hipError_t launchDecLinear(const DecLinearArgs &a, const LaunchCtx &ctx) {
+hipError_t launchDecLinear(const DecLinearArgs &in, const LaunchCtx &ctx) {
+    DecLinearArgs a = in;
+    a.nwaves = a.K > 0 ? decLinearWaves(a.K) : kDecWaves;
     if (!a.x || a.M <= 0 || a.M > kDecMaxRows || a.K <= 0 || a.K % 128 != 0 || a.qblock <= 0 || a.qblock % 128 != 0 || a.K % a.qblock != 0) return hipErrorInvalidValue;
     if (a.nseg < 1 || a.nseg > kDecMaxSegments || (a.pair && a.nseg != 2) || (((uintptr_t)a.x) & 15)) return hipErrorInvalidValue;
     if (a.add_mode < 0 || a.add_mode > 2 || (a.add_mode == 1 && (a.nseg != 1 || !a.res)) || (a.add_mode == 2 && !a.pair) || (a.pair && a.add_mode != 2)) return hipErrorInvalidValue;
     if (a.add_mode != 0 && (!a.add_out || (((uintptr_t)a.add_out) & 7) || (a.res && (((uintptr_t)a.res) & 7)))) return hipErrorInvalidValue;
-    if (a.prefetch_bytes < 0 || (a.prefetch_bytes > 0 && (!a.prefetch || (((uintptr_t)a.prefetch) & 3)))) return hipErrorInvalidValue;
     long long tiles = 0;
     for (int s = 0; s < a.nseg; s++) {
         if (!a.w[s] || !a.bias[s] || a.N[s] <= 0 || a.N[s] % 16 != 0) return hipErrorInvalidValue;
@@ -310,7 +302,7 @@ hipError_t launchDecLinear(const DecLinearArgs &a, const LaunchCtx &ctx) {
         if (a.N[0] != a.N[1]) return hipErrorInvalidValue;
         tiles = a.N[0] / 16;
     }
-    if (tiles <= 0 || tiles > 65535 || decLinearLds(a.K, a.pair ? 2 : 1, 0) > kDecMaxLds) return hipErrorInvalidValue;
+    if (tiles <= 0 || tiles > 65535 || decLinearLds(a.K, a.pair ? 2 : 1, 0, a.nwaves) > kDecMaxLds) return hipErrorInvalidValue;
     const bool clamp = !(a.qlo == -INFINITY && a.qhi == INFINITY);
     const int t = (int)tiles;
     if (ctx.tuning->decAblate) {
@@ -326,17 +318,10 @@ hipError_t launchDecLinear(const DecLinearArgs &a, const LaunchCtx &ctx) {
 // (wave, wave + 8, ...), each lane loading 16 bytes of its weight row and of its input row per step; the partial
 // sums meet in LDS.  A wave's loads of up to ST steps are all issued before the first MFMA.
 template <int MR, int ST>
-__global__ __launch_bounds__((kDecWaves + 1) * 64) void dec_matmul(DecMatmulArgs p) {
+__global__ __launch_bounds__(kDecWaves * 64) void dec_matmul(DecMatmulArgs p) {
     __shared__ v4f red[kDecWaves][MR][64];
-    __shared__ int sink[kDecSinkBytes / 4];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-    if (wave == kDecWaves) {
-        prefetchLines(p.prefetch, p.prefetch_bytes, lane, ldsOffset(sink));
-        __syncthreads();
-        waitVmcnt<0>();
-        return;
-    }
     const int c = lane & 15, g = lane >> 4;
     const int n0 = (int)blockIdx.x * 16, b = (int)blockIdx.y;
     const uint16_t *a = p.a + (size_t)b * p.a_stride, *w = p.w + (size_t)b * p.w_stride;
@@ -396,20 +381,19 @@ hipError_t launchDecMatmul(const DecMatmulArgs &a, const LaunchCtx &ctx) {
     if (!a.a || !a.w || !a.out || a.B <= 0 || a.B > 65535 || a.M <= 0 || a.M > kDecMaxRows || a.K <= 0 || a.K % 8 != 0 || a.N <= 0) return hipErrorInvalidValue;
     if (a.a_stride < 0 || a.w_stride < 0 || a.out_stride < 0 || a.a_stride % 8 != 0 || a.w_stride % 8 != 0) return hipErrorInvalidValue;
     if (((((uintptr_t)a.a) | ((uintptr_t)a.w)) & 15) || (((uintptr_t)a.out) & (a.N % 4 == 0 ? 7 : 1)) || (a.N % 4 == 0 && a.out_stride % 4 != 0)) return hipErrorInvalidValue;
-    if (a.prefetch_bytes < 0 || (a.prefetch_bytes > 0 && (!a.prefetch || (((uintptr_t)a.prefetch) & 3)))) return hipErrorInvalidValue;
     const long long tiles = ((long long)a.N + 15) / 16;
     if (tiles > 0x7fffffffLL) return hipErrorInvalidValue;
     const dim3 grid((unsigned)tiles, (unsigned)a.B);
     // steps of 32 per wave: up to four are one round of loads
     const int perWave = ((a.K + 31) / 32 + kDecWaves - 1) / kDecWaves;
     if (a.M <= 16) {
-        if (perWave <= 1) THIP_ENQUEUE(ctx, "dec_matmul<1,1>", (dec_matmul<1, 1>), grid, dim3((kDecWaves + (a.prefetch ? 1 : 0)) * 64), 0, a);
-        else if (perWave <= 2) THIP_ENQUEUE(ctx, "dec_matmul<1,2>", (dec_matmul<1, 2>), grid, dim3((kDecWaves + (a.prefetch ? 1 : 0)) * 64), 0, a);
-        else THIP_ENQUEUE(ctx, "dec_matmul<1,4>", (dec_matmul<1, 4>), grid, dim3((kDecWaves + (a.prefetch ? 1 : 0)) * 64), 0, a);
+        if (perWave <= 1) THIP_ENQUEUE(ctx, "dec_matmul<1,1>", (dec_matmul<1, 1>), grid, dim3(kDecWaves * 64), 0, a);
+        else if (perWave <= 2) THIP_ENQUEUE(ctx, "dec_matmul<1,2>", (dec_matmul<1, 2>), grid, dim3(kDecWaves * 64), 0, a);
+        else THIP_ENQUEUE(ctx, "dec_matmul<1,4>", (dec_matmul<1, 4>), grid, dim3(kDecWaves * 64), 0, a);
     } else {
-        if (perWave <= 1) THIP_ENQUEUE(ctx, "dec_matmul<2,1>", (dec_matmul<2, 1>), grid, dim3((kDecWaves + (a.prefetch ? 1 : 0)) * 64), 0, a);
-        else if (perWave <= 2) THIP_ENQUEUE(ctx, "dec_matmul<2,2>", (dec_matmul<2, 2>), grid, dim3((kDecWaves + (a.prefetch ? 1 : 0)) * 64), 0, a);
-        else THIP_ENQUEUE(ctx, "dec_matmul<2,4>", (dec_matmul<2, 4>), grid, dim3((kDecWaves + (a.prefetch ? 1 : 0)) * 64), 0, a);
+        if (perWave <= 1) THIP_ENQUEUE(ctx, "dec_matmul<2,1>", (dec_matmul<2, 1>), grid, dim3(kDecWaves * 64), 0, a);
+        else if (perWave <= 2) THIP_ENQUEUE(ctx, "dec_matmul<2,2>", (dec_matmul<2, 2>), grid, dim3(kDecWaves * 64), 0, a);
+        else THIP_ENQUEUE(ctx, "dec_matmul<2,4>", (dec_matmul<2, 4>), grid, dim3(kDecWaves * 64), 0, a);
     }
     return hipGetLastError();
 }

@@ -96,13 +96,11 @@ enum Kind : uint32_t {
     // in0 = x [M][K] bf16 (K % 128 == 0), gran = rows per quantisation block (a multiple of 128), w0 = number of
     // matrices, w1 = DecLinearFlags, output_min / output_max = float bits of the matmuls' clamp, bias0 / scale0 =
     // float bits of the expansions' clamp, table = a DecLinearExt in the constant segment (the per-matrix operands),
-    // out = the first buffer the launch writes, Nn = its row length.  scale / TR: see kKindDecMatmul.
+    // out = the first buffer the launch writes, Nn = its row length.
     kKindDecLinear = 15,
     // Batch of small bf16 matmuls against a run-time operand held [N][K]: in0 = a [TB][M][K] (w0 != 0: one [M][K] for
     // every batch), weights = [TB][Nn][K] (w1 != 0: shared), out [TB][M][Nn]; M <= 32; bias0 = float bits of the one
-    // bias, output_min / output_max = float bits of the clamp.  Both decode kinds: scale = constants that the NEXT
-    // record streams (space none: nothing), TS = their size in 128-byte lines: the launch touches them so that they
-    // are in the last-level cache by the time that record runs.
+    // bias, output_min / output_max = float bits of the clamp.
     kKindDecMatmul = 16,
 };
 

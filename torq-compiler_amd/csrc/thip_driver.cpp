@@ -294,10 +294,6 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
         a.nseg = op.w0;
         a.pair = (op.w1 & kDecPair) ? 1 : 0;
         a.has_qbias = x.has_qbias;
-        if (op.scale.space == kSpaceConst && op.TS > 0) {
-            a.prefetch = resolve(e, op.scale, bp);
-            a.prefetch_bytes = (int64_t)op.TS * 128;
-        }
         for (int m = 0; m < op.w0 && m < kDecMaxSegments; m++) {
             a.w[m] = (const int8_t *)resolve(e, x.weights[m], bp);
             a.bias[m] = (const float *)resolve(e, x.bias[m], bp);
@@ -325,12 +321,7 @@ static thip_status_t launchOp(thip_executable_t *e, uint32_t i, uint8_t *const *
     }
     case kKindDecMatmul: {
         DecMatmulArgs a{(const uint16_t *)resolve(e, op.in0, bp), (const uint16_t *)resolve(e, op.weights, bp), (uint16_t *)resolve(e, op.out, bp),
-                        op.TB, op.M, op.K, op.Nn, op.w0 ? 0 : (int64_t)op.M * op.K, op.w1 ? 0 : (int64_t)op.Nn * op.K, (int64_t)op.M * op.Nn, 0.0f, 0.0f, 0.0f,
-                        nullptr, 0};
-        if (op.scale.space == kSpaceConst && op.TS > 0) {
-            a.prefetch = resolve(e, op.scale, bp);
-            a.prefetch_bytes = (int64_t)op.TS * 128;
-        }
+                        op.TB, op.M, op.K, op.Nn, op.w0 ? 0 : (int64_t)op.M * op.K, op.w1 ? 0 : (int64_t)op.Nn * op.K, (int64_t)op.M * op.Nn, 0.0f, 0.0f, 0.0f};
         memcpy(&a.bias, &op.bias0, 4);
         memcpy(&a.lo, &op.output_min, 4);
         memcpy(&a.hi, &op.output_max, 4);

@@ -700,7 +700,6 @@ class Emitter {
     size_t nextLiveOp(size_t at) const;
     thip_status_t tryEmitDecodeLinear(size_t at, bool *handled);
     thip_status_t emitDecodeMatmul(const thip_hl_matmul_t &c, size_t transposeAt);
-    void planDecodePrefetch(const std::vector<DescConst> &ctable);
     // Operands of an expand_weights checked and measured.
     struct ExpandShape {
         const Value *w, *scale, *bias, *init;
@@ -1983,6 +1982,13 @@ size_t Emitter::nextLiveOp(size_t at) const {
     return prog_.ops.size();
 }
 
+// LDS a workgroup of the grouped linear kernel needs for its share of ONE matrix: 16 columns of the whole K, in whole
+// k-blocks per wave.
+static int64_t decLinearShare(int64_t K) {
+    const int64_t kblocks = K / 128, waves = kblocks < 8 ? 8 : (kblocks > 16 ? 16 : kblocks);
+    return waves * ((kblocks + waves - 1) / waves) * (2048 + 128);
+}
+
 bool Emitter::decodeCandidate(size_t at, DecCandidate *out) {
     if (at >= prog_.ops.size() || prog_.ops[at].kind != kHlMatmul || consumed_[at]) return false;
     const thip_hl_matmul_t &c = prog_.ops[at].u.mm;
@@ -2001,7 +2007,7 @@ bool Emitter::decodeCandidate(size_t at, DecCandidate *out) {
     if (w.shape[0] != K || M > kDecMaxRows || K % 128 != 0 || N % 16 != 0 || N / 16 > 1024 || block <= 0 || block % 128 != 0 || K % block != 0) return false;
     const int64_t G = K / block;
     if (sc.numel() != G * N || qb.numel() % G != 0 || qb.numel() / G < N || init.numel() != M * N) return false;
-    if ((K / 128 + 7) / 8 * 8 * (2048 + 128) > 152 * 1024) return false;  // a workgroup's share of the weights (16 columns of the whole K) must fit a CU's LDS
+    if (decLinearShare(K) > 152 * 1024) return false;  // a workgroup's share of the weights (16 columns of the whole K) must fit a CU's LDS
     out->mm = &c;
     out->ew = &ew;
     out->M = M; out->K = K; out->N = N; out->block = block;
@@ -2043,7 +2049,7 @@ thip_status_t Emitter::tryEmitDecodeLinear(size_t at, bool *handled) {
     int flags = 0;
     DecCandidate c1, c2;
     const thip_hl_add_t *ad = nullptr;
-    const bool pairFits = (c0.K / 128 + 7) / 8 * 8 * 2 * (2048 + 128) <= 152 * 1024;  // twice the share of one matrix
+    const bool pairFits = 2 * decLinearShare(c0.K) <= 152 * 1024;  // twice the share of one matrix
     if (pairFits && j1 < end && decodeCandidate(j1, &c1) && sameGroup(c0, c1) && c0.N == c1.N && bf16Add(j2, &ad) &&
         ((ad->input1 == c0.mm->init && ad->input2 == c1.mm->init) || (ad->input1 == c1.mm->init && ad->input2 == c0.mm->init)) &&
         ad->init != c0.mm->init && ad->init != c1.mm->init) {
@@ -2158,47 +2164,6 @@ thip_status_t Emitter::tryEmitDecodeLinear(size_t at, bool *handled) {
     for (size_t mbr : members) consumed_[mbr] = 1;
     *handled = true;
     return THIP_OK;
-}
-
-// Weights do not depend on activations: a decode record can bring the constants of a record behind it into the
-// last-level cache while its own kernel runs (its prefetch wave touches every line of them), so that the chain does
-// not pay an HBM round trip per launch.  Record i takes the first record within the next three that streams
-// constants and that no earlier record has taken; of a very large matrix only the first kPrefetchCap bytes.
-void Emitter::planDecodePrefetch(const std::vector<DescConst> &ctable) {
-    // Off unless THIP_DECODE_PREFETCH is set: measured on a 26-layer decoder step at one token it costs the
-    // prefetching launches more than it saves the prefetched ones, whose time is launch and latency, not HBM
-    // (step 900 us without, 1173 us with; the matrix-heavy launch 7.6 -> 7.2 us, a 16-workgroup attention
-    // launch that prefetches 8 MB 4.2 -> 12.3 us).
-    if (!getenv("THIP_DECODE_PREFETCH")) return;
-    constexpr uint64_t kPrefetchCap = 24u << 20;
-    const size_t n = ops_.size();
-    std::vector<uint32_t> firstConst(n, 0);
-    std::vector<uint64_t> bytes(n, 0);
-    for (size_t i = 0; i < n; i++) {
-        const DescOp &op = ops_[i];
-        if (op.kind == kKindDecLinear) {
-            DecLinearExt x;
-            memcpy(&x, consts_[op.table.index].data(), sizeof(x));
-            const uint32_t first = x.weights[0].index, last = x.weights[op.w0 - 1].index;
-            firstConst[i] = first;
-            bytes[i] = ctable[last].offset + ctable[last].size - ctable[first].offset;
-        } else if (op.kind == kKindFcBf16 && op.weights.space == kSpaceConst) {
-            firstConst[i] = op.weights.index;
-            bytes[i] = ctable[op.weights.index].size;
-        }
-        if (bytes[i] > kPrefetchCap) bytes[i] = kPrefetchCap;
-    }
-    std::vector<char> taken(n, 0);
-    for (size_t i = 0; i < n; i++) {
-        if (ops_[i].kind != kKindDecLinear && ops_[i].kind != kKindDecMatmul) continue;
-        for (size_t j = i + 1; j < n && j <= i + 3; j++) {
-            if (bytes[j] == 0 || taken[j]) continue;
-            taken[j] = 1;
-            ops_[i].scale = DescRef{kSpaceConst, firstConst[j], 0};
-            ops_[i].TS = (int32_t)((bytes[j] + 127) / 128);
-            break;
-        }
-    }
 }
 
 // Decides which intermediates are stored with their channel axis padded to a multiple of 16.
@@ -2467,7 +2432,6 @@ thip_status_t Emitter::run(void **outBlob, size_t *outSize) {
         dataOff = (uint64_t)roundUp((int64_t)(dataOff + consts_[i].size()), (int64_t)kDataAlign);
     }
     h.total_size = h.data_offset + dataOff;
-    planDecodePrefetch(ctable);
 
     uint8_t *blob = (uint8_t *)calloc(1, (size_t)h.total_size);
     if (!blob) return fail(THIP_RESOURCE_EXHAUSTED, "out of memory serialising %llu bytes", (unsigned long long)h.total_size);

@@ -232,11 +232,8 @@ struct DecLinearArgs {
     const uint16_t *res;
     uint16_t *add_out;
     float aw0, aw1, abias, alo, ahi;
-    // constants the NEXT record will stream (its weights): this launch reads one 4-byte word of every 128-byte line of
-    // them, which brings them into the last-level cache while its own work runs (null: nothing)
-    const void *prefetch;
-    int64_t prefetch_bytes;
-    int32_t ablate;  // timing experiments only (THIP_DEC_ABLATE; results are wrong): 1 no weight loads, 2 no arithmetic, 4 no prefetch wave work
+    int32_t nwaves;  // waves per workgroup; the launcher sets it (decLinearWaves)
+    int32_t ablate;  // timing experiments only (THIP_DEC_ABLATE; results are wrong): 1 no weight loads, 2 no arithmetic
 };
 inline int decSlotBytes(bool hasBias) { return kDecSlotBytes + (hasBias ? 64 : 0); }
 // Byte offset of int8 weight (n, k) in the dec16 order, for K padded to `kblocks` blocks of 128.
@@ -249,6 +246,7 @@ inline size_t decScaleOffset(int n, int b, int kblocks, bool hasBias, int which)
     return ((size_t)(n >> 4) * kblocks + b) * decSlotBytes(hasBias) + 2048 + (size_t)which * 64 + (size_t)(n & 15) * 4;
 }
 inline size_t decWeightBytes(int N, int K, bool hasBias) { return (size_t)((N + 15) / 16) * ((K + 127) / 128) * decSlotBytes(hasBias); }
+int decLinearWaves(int K);
 hipError_t launchDecLinear(const DecLinearArgs &a, const LaunchCtx &ctx);
 
 // dec_matmul: out[b][m][n] = bf16(clamp(sum_k a[b][m][k] * w[b][n][k] + bias)) for a batch of small matmuls whose
@@ -262,8 +260,6 @@ struct DecMatmulArgs {
     int32_t B, M, K, N;
     int64_t a_stride, w_stride, out_stride;
     float bias, lo, hi;
-    const void *prefetch;  // as in DecLinearArgs
-    int64_t prefetch_bytes;
 };
 hipError_t launchDecMatmul(const DecMatmulArgs &a, const LaunchCtx &ctx);
 

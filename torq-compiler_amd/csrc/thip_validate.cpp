@@ -172,23 +172,6 @@ thip_status_t checkOpFootprint(const DescriptorView *e, uint32_t i) {
     };
     const uint64_t outElem = op.out_dtype == THIP_DTYPE_I32 ? 4 : op.out_dtype == THIP_DTYPE_I16 ? 2 : 1;
     thip_status_t s = THIP_OK;
-    // decode kinds: `scale` names constants a launch only touches (the next record's weights), TS lines of 128 bytes
-    // from there on, possibly across several constants: they must lie inside the constant segment
-    auto prefetchRangeOk = [&]() {
-        if (op.scale.space == kSpaceNone) return true;
-        if (op.scale.space != kSpaceConst || op.TS <= 0 || (op.scale.offset & 3)) return false;
-        const uint64_t segment = e->header.total_size - e->header.data_offset;
-        const uint64_t start = e->consts[op.scale.index].offset + op.scale.offset, bytes = ((uint64_t)op.TS - 1) * 128 + 4;
-        return start <= segment && bytes <= segment - start;
-    };
-    if (op.shift < 0 || op.shift > 63) return fail(THIP_INVALID_ARGUMENT, "op %u: shift %d is outside 0..63", i, op.shift);
-    if (op.pre_shift != 0 && (op.pre_shift < 0 || op.pre_shift > 30 || (int64_t)op.shift + op.pre_shift != 33 || op.shift < 0 || op.shift > 63 ||
-                              (op.kind != kKindIgemm && op.kind != kKindDepthwise))) {
-        return fail(THIP_INVALID_ARGUMENT, "op %u: pre_shift %d does not complete shift %d to 33", i, op.pre_shift, op.shift);
-    }
-    if (op.t0_clamp != 0 && (op.t0_clamp < 0 || op.pre_shift <= 0 || op.pre_shift > 30 || op.t0_clamp >= (1 << (31 - op.pre_shift)))) {
-        return fail(THIP_INVALID_ARGUMENT, "op %u: t0_clamp %d does not fit pre_shift %d", i, op.t0_clamp, op.pre_shift);
-    }
     switch (op.kind) {
     case kKindTranspose: {
         if (!positive({op.TB, op.TR, op.TS})) return fail(THIP_INVALID_ARGUMENT, "op %u: bad transpose extents", i);
@@ -417,7 +400,6 @@ thip_status_t checkOpFootprint(const DescriptorView *e, uint32_t i) {
             if ((x.res.offset & 7) || (x.add_out.offset & 7)) return fail(THIP_INVALID_ARGUMENT, "op %u: misaligned operand of the folded add", i);
         }
         if ((op.in0.offset & 15) != 0) return fail(THIP_INVALID_ARGUMENT, "op %u: misaligned input", i);
-        if (!prefetchRangeOk()) return fail(THIP_INVALID_ARGUMENT, "op %u: bad prefetch range", i);
         return THIP_OK;
     }
     case kKindDecMatmul: {
@@ -425,7 +407,6 @@ thip_status_t checkOpFootprint(const DescriptorView *e, uint32_t i) {
         if ((s = need(op.in0, mul(op.w0 ? 1 : op.TB, op.M, op.K) * 2, "in1"))) return s;
         if ((s = need(op.weights, mul(op.w1 ? 1 : op.TB, op.Nn, op.K) * 2, "in2"))) return s;
         if ((op.in0.offset & 15) || (op.weights.offset & 15) || (op.out.offset & 7)) return fail(THIP_INVALID_ARGUMENT, "op %u: misaligned operand", i);
-        if (!prefetchRangeOk()) return fail(THIP_INVALID_ARGUMENT, "op %u: bad prefetch range", i);
         return need(op.out, mul(op.TB, op.M, op.Nn) * 2, "out");
     }
     default: return fail(THIP_INVALID_ARGUMENT, "op %u has unknown kind %u", i, op.kind);
