@@ -223,8 +223,9 @@ def traffic_still_valid(name):
 
 
 # The traffic shape of the benchmark's bandwidth rows for the streaming-floor calibration: 16-byte reads per 16-byte
-# write (1, 2 or 4) and bytes written per launch.  The floor is what a kernel with next to no arithmetic takes for
-# the same bytes on the same buffers-larger-than-cache rotation: no op of that size can be faster on this card.
+# write (1, 2 or 4) and bytes written per launch.  The floor is what the fastest of a family of kernels with next to
+# no arithmetic (1 to 8 items per thread, one pass or persistent, default or non-temporal cache policy) takes for the
+# same bytes on the same buffers-larger-than-cache rotation.
 STREAM_SHAPES = {
     "depthwise_b64": (4, 64 * 28 * 28 * 144), "depthwise_s1_b256": (1, 256 * 56 * 56 * 144), "maxpool_b64": (4, 64 * 56 * 56 * 64),
     "add_b64": (2, 64 * 56 * 56 * 24), "rescale_b64": (1, 64 * 56 * 56 * 24), "mul_b64": (2, 64 * 56 * 56 * 24),
@@ -538,8 +539,9 @@ def main():
                 if name in STREAM_SHAPES:
                     rd, wbytes = STREAM_SHAPES[name]
                     wbytes = wbytes // 16 * 16
-                    floor_us = min(dev.stream_floor(rd, wbytes, cold=True) for _ in range(3))  # the first call meets a card that has idled
+                    floor_us, floor_kernel = min(dev.stream_floor(rd, wbytes, cold=True, variant=True) for _ in range(3))  # the first call meets a card that has idled
                     row["streaming_floor_us"] = round(floor_us, 2)
+                    row["streaming_floor_kernel"] = floor_kernel
                     row["frac_of_streaming_floor"] = round(floor_us / (ms * 1e3), 3)
             else:
                 ms = warm

@@ -441,12 +441,17 @@ thip_status_t thip_device_synchronize(thip_device_t *device);
 thip_status_t thip_device_mfma_rate(thip_device_t *device, int32_t random_operands, int32_t workgroups,
                                     int32_t iterations, double *out_tops);
 
-/* Calibration for the benchmark (no counterpart in the reference): microseconds per launch of a kernel with next to
- * no arithmetic that reads reads_per_write (1, 2 or 4) 16-byte pieces for every 16 bytes it writes, write_bytes
- * written per launch: what this memory system gives a bandwidth-bound op of that size and read/write mix.
- * cold != 0: every launch on other buffers, more of them than the last-level cache holds. */
+/* Calibration for the benchmark (no counterpart in the reference): microseconds per launch of the fastest of a family
+ * of kernels with next to no arithmetic (1 to 8 16-byte items per thread, one pass or a persistent grid-stride grid,
+ * default or non-temporal cache policy) that read reads_per_write (1, 2 or 4) 16-byte pieces for every 16 bytes they
+ * write, write_bytes written per launch: what this memory system gives a bandwidth-bound op of that size and
+ * read/write mix.  cold != 0: every launch on other buffers, more of them than the last-level cache holds.
+ * The _tuned form also names the winner ("stream_floor<reads, items per thread, persistent, non-temporal>"). */
 thip_status_t thip_device_stream_floor(thip_device_t *device, int32_t reads_per_write, size_t write_bytes,
                                        int32_t cold, double *out_microseconds);
+thip_status_t thip_device_stream_floor_tuned(thip_device_t *device, int32_t reads_per_write, size_t write_bytes,
+                                             int32_t cold, double *out_microseconds, char *out_variant,
+                                             size_t variant_capacity);
 
 /* What a descriptor blob holds, in the terms of the reference's executable schema
  * (runtime/schemas/torq_executable_def.fbs): ExecutableDef :168-197, Binding :28-48, Segment :13-24.  These read

@@ -207,7 +207,7 @@ __device__ __forceinline__ void loadDwords(const int8_t *src, int (&dst)[G]) {
         typename DwordVec<G>::type v;
         int w[G];
     } u;
-    u.v = *(const typename DwordVec<G>::type *)src;
+    u.v = *(const typename DwordVec<G>::type *)src;  // neighbouring threads and strips read the same bytes again: default cache policy
 #pragma unroll
     for (int g = 0; g < G; g++) dst[g] = u.w[g];
 }
@@ -514,7 +514,11 @@ __global__ __launch_bounds__(256, OCC) void depthwise3x3_strip_i8(DepthwiseArgs 
                         } u;
 #pragma unroll
                         for (int g = 0; g < G; g++) u.w[g] = o[q][g];
-                        *(typename DwordVec<G>::type *)(orow + (size_t)q * p.C) = u.v;
+                        // written once, read by another kernel: the non-temporal policy at stride 2 (56 x 56 x 144, batch 64:
+                        // 11.4 -> 10.8 us cold); at stride 1 the 4-byte pieces of neighbouring threads complete each other's
+                        // lines in the cache, and the same policy costs 58 -> 64 us at batch 256
+                        if (S == 2) streamStore<typename DwordVec<G>::type>(orow + (size_t)q * p.C, u.v);
+                        else *(typename DwordVec<G>::type *)(orow + (size_t)q * p.C) = u.v;
                     }
                 }
             }
@@ -709,7 +713,7 @@ __global__ __launch_bounds__(256) void maxpool2x2_i8(MaxPoolArgs p, WorkSplit ws
     splitWork(t, ws, cgi, ox, oy, n);
     const int8_t *src = p.in + (((size_t)n * p.H + 2 * oy) * p.W + 2 * ox) * p.C + cgi * 16;
     const size_t row = (size_t)p.W * p.C;
-    const v4i a = *(const v4i *)src, b = *(const v4i *)(src + p.C), c = *(const v4i *)(src + row), d = *(const v4i *)(src + row + p.C);
+    const v4i a = streamLoad<v4i>(src), b = streamLoad<v4i>(src + p.C), c = streamLoad<v4i>(src + row), d = streamLoad<v4i>(src + row + p.C);
     v4i o;
 #pragma unroll
     for (int q = 0; q < 4; q++) {
@@ -717,7 +721,7 @@ __global__ __launch_bounds__(256) void maxpool2x2_i8(MaxPoolArgs p, WorkSplit ws
                                       maxSplit(splitBytes((uint32_t)c[q]), splitBytes((uint32_t)d[q])));
         o[q] = (int)joinBytes(m);
     }
-    *(v4i *)(p.out + (((size_t)n * p.OH + oy) * p.OW + ox) * p.C + cgi * 16) = o;
+    streamStore<v4i>(p.out + (((size_t)n * p.OH + oy) * p.OW + ox) * p.C + cgi * 16, o);
 }
 
 template <int VEC>
@@ -835,8 +839,8 @@ __global__ __launch_bounds__(256) void add_i8(AddArgs p, int32_t folded) {
     const long long rnd = roundTerm(p.rq.shift);
     if (i0 + VEC <= p.count) {
         if constexpr (FAST && VEC == 16) {
-            const v4i a = *(const v4i *)(p.in0 + i0), b = *(const v4i *)(p.in1 + i0);
-            *(v4i *)(p.out + i0) = residualAdd16<true>(a, b, false, p.w0, p.w1, p.bias, p.scale, rnd, p.rq, folded);
+            const v4i a = streamLoad<v4i>(p.in0 + i0), b = streamLoad<v4i>(p.in1 + i0);
+            streamStore<v4i>(p.out + i0, residualAdd16<true>(a, b, false, p.w0, p.w1, p.bias, p.scale, rnd, p.rq, folded));
         } else {
             Pack<VEC> a, b, o;
             a.v = *(const typename ByteVec<VEC>::type *)(p.in0 + i0);

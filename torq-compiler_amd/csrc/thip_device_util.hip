@@ -110,64 +110,133 @@ hipError_t measureMfmaRate(int randomOperands, int blocks, int iterations, hipSt
     return err;
 }
 
-// Calibration: what a kernel with no arithmetic to speak of reaches on this memory system for a transfer of a given
-// size: every thread reads RD 16-byte pieces (from RD separate streams, perfectly coalesced), combines them with one
-// instruction each and writes 16 bytes.  RD = 1 is a plain copy, RD = 2 the traffic shape of an elementwise add,
-// RD = 4 that of a 2 x 2 pooling or a stride-2 3 x 3 depthwise convolution.
-template <int RD>
+// ---------------------------------------------------------------------------
+// Calibration: what a kernel with next to no arithmetic takes to move a given number of bytes, i.e. the floor under
+// every bandwidth-bound op of that traffic shape on this GPU.  RD 16-byte reads per 16-byte write and lane (reads of
+// RD planes of one buffer, one xor per extra read).  A family, because the floor must be the best a copy can do, not
+// one arbitrary copy: U 16-byte items per thread whose loads are all issued before the first store (1, 2, 4, 8);
+// a grid of one item group per thread, or a persistent grid (every CU full, grid-stride loop); default or non-temporal
+// cache policy.  measureStreamRate times all of them and reports the fastest.
+// ---------------------------------------------------------------------------
+template <int RD, int U, bool PERSIST, bool NT>
 __global__ __launch_bounds__(256) void stream_floor(const v4i *__restrict__ in, v4i *__restrict__ out, size_t items) {
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= items) return;
-    v4i v[RD];
+    const size_t stride = PERSIST ? (size_t)gridDim.x * 256 * U : items + (size_t)256 * U;  // one pass unless persistent
+    for (size_t base = (size_t)blockIdx.x * 256 * U; base < items; base += stride) {
+        v4i v[U][RD];
 #pragma unroll
-    for (int r = 0; r < RD; r++) v[r] = in[(size_t)r * items + i];
-    v4i m = v[0];
+        for (int u = 0; u < U; u++) {
+            const size_t i = base + (size_t)u * 256 + threadIdx.x;  // a wave's loads cover 1 KiB in a row
 #pragma unroll
-    for (int r = 1; r < RD; r++) {
-        m[0] ^= v[r][0];
-        m[1] ^= v[r][1];
-        m[2] ^= v[r][2];
-        m[3] ^= v[r][3];
+            for (int r = 0; r < RD; r++) {
+                if (i < items) v[u][r] = NT ? __builtin_nontemporal_load(in + (size_t)r * items + i) : in[(size_t)r * items + i];
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const size_t i = base + (size_t)u * 256 + threadIdx.x;
+            if (i >= items) continue;
+            v4i m = v[u][0];
+#pragma unroll
+            for (int r = 1; r < RD; r++) {
+                m[0] ^= v[u][r][0];
+                m[1] ^= v[u][r][1];
+                m[2] ^= v[u][r][2];
+                m[3] ^= v[u][r][3];
+            }
+            if (NT) __builtin_nontemporal_store(m, out + i);
+            else out[i] = m;
+        }
     }
-    out[i] = m;
 }
 
-hipError_t measureStreamRate(int readsPerWrite, size_t writeBytes, int cold, hipStream_t stream, double *outMicroseconds) {
+struct StreamVariant {
+    int u, persist, nt;
+};
+
+template <int RD, int U, bool PERSIST, bool NT>
+static void launchStreamFloor(const v4i *in, v4i *out, size_t items, int cus, hipStream_t stream) {
+    const size_t groups = (items + (size_t)256 * U - 1) / ((size_t)256 * U);
+    const size_t resident = (size_t)cus * 8;  // eight workgroups of four waves fill a CU's wave slots
+    const unsigned blocks = (unsigned)(PERSIST && groups > resident ? resident : groups);
+    hipLaunchKernelGGL((stream_floor<RD, U, PERSIST, NT>), dim3(blocks), dim3(256), 0, stream, in, out, items);
+}
+
+template <int RD>
+static void launchStreamFloorRd(const StreamVariant &v, const v4i *in, v4i *out, size_t items, int cus, hipStream_t stream) {
+#define THIP_STREAM_CASE(U)                                                                                   \
+    if (v.u == U) {                                                                                           \
+        if (v.persist) {                                                                                      \
+            if (v.nt) launchStreamFloor<RD, U, true, true>(in, out, items, cus, stream);                      \
+            else launchStreamFloor<RD, U, true, false>(in, out, items, cus, stream);                          \
+        } else {                                                                                              \
+            if (v.nt) launchStreamFloor<RD, U, false, true>(in, out, items, cus, stream);                     \
+            else launchStreamFloor<RD, U, false, false>(in, out, items, cus, stream);                         \
+        }                                                                                                     \
+        return;                                                                                               \
+    }
+    THIP_STREAM_CASE(1)
+    THIP_STREAM_CASE(2)
+    THIP_STREAM_CASE(4)
+    THIP_STREAM_CASE(8)
+#undef THIP_STREAM_CASE
+}
+
+hipError_t measureStreamRate(int readsPerWrite, size_t writeBytes, int cold, hipStream_t stream, double *outMicroseconds, char *outVariant, size_t variantCapacity) {
     if ((readsPerWrite != 1 && readsPerWrite != 2 && readsPerWrite != 4) || writeBytes < 4096 || writeBytes % 16 != 0 || writeBytes > (1ull << 31) ||
         !outMicroseconds) {
         return hipErrorInvalidValue;
     }
+    int device = 0, cus = 0;
+    hipError_t err = hipGetDevice(&device);
+    if (err == hipSuccess) err = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device);
+    if (err != hipSuccess) return err;
     const size_t items = writeBytes / 16, perSet = writeBytes * (size_t)(readsPerWrite + 1);
     // cold: dispatch i works on buffer set i mod n, the sets together twice the size of the 256 MiB last-level cache
     int sets = cold ? (int)((512ull << 20) / perSet) + 1 : 1;
     sets = sets < (cold ? 2 : 1) ? 2 : (sets > 160 ? 160 : sets);
     std::vector<v4i *> in((size_t)sets, nullptr), out((size_t)sets, nullptr);
     hipEvent_t e0 = nullptr, e1 = nullptr;
-    hipError_t err = hipSuccess;
     for (int s = 0; s < sets && err == hipSuccess; s++) {
         err = hipMalloc((void **)&in[(size_t)s], writeBytes * (size_t)readsPerWrite);
         if (err == hipSuccess) err = hipMalloc((void **)&out[(size_t)s], writeBytes);
         if (err == hipSuccess) err = hipMemsetAsync(in[(size_t)s], s + 1, writeBytes * (size_t)readsPerWrite, stream);
     }
-    auto launch = [&](int s) {
-        const dim3 grid((unsigned)((items + 255) / 256));
-        if (readsPerWrite == 1) hipLaunchKernelGGL(stream_floor<1>, grid, dim3(256), 0, stream, in[(size_t)s], out[(size_t)s], items);
-        else if (readsPerWrite == 2) hipLaunchKernelGGL(stream_floor<2>, grid, dim3(256), 0, stream, in[(size_t)s], out[(size_t)s], items);
-        else hipLaunchKernelGGL(stream_floor<4>, grid, dim3(256), 0, stream, in[(size_t)s], out[(size_t)s], items);
+    auto launch = [&](const StreamVariant &v, int s) {
+        if (readsPerWrite == 1) launchStreamFloorRd<1>(v, in[(size_t)s], out[(size_t)s], items, cus, stream);
+        else if (readsPerWrite == 2) launchStreamFloorRd<2>(v, in[(size_t)s], out[(size_t)s], items, cus, stream);
+        else launchStreamFloorRd<4>(v, in[(size_t)s], out[(size_t)s], items, cus, stream);
     };
     if (err == hipSuccess) err = hipEventCreate(&e0);
     if (err == hipSuccess) err = hipEventCreate(&e1);
+    double best = 0.0;
+    StreamVariant bestVariant{1, 0, 0};
     if (err == hipSuccess) {
-        for (int s = 0; s < sets; s++) launch(s);  // first touch
-        const int iterations = sets * 3 > 30 ? sets * 3 : 30;
-        err = hipEventRecord(e0, stream);
-        for (int i = 0; i < iterations; i++) launch(i % sets);
-        if (err == hipSuccess) err = hipGetLastError();
-        if (err == hipSuccess) err = hipEventRecord(e1, stream);
-        if (err == hipSuccess) err = hipEventSynchronize(e1);
-        float ms = 0.f;
-        if (err == hipSuccess) err = hipEventElapsedTime(&ms, e0, e1);
-        if (err == hipSuccess) *outMicroseconds = (double)ms * 1e3 / iterations;
+        for (int s = 0; s < sets; s++) launch(bestVariant, s);  // first touch
+        const int iterations = sets * 2 > 24 ? sets * 2 : 24;
+        for (int u = 1; u <= 8 && err == hipSuccess; u *= 2) {
+            if (readsPerWrite * u > 16) continue;  // more than 64 registers of loads in flight per thread gain nothing
+            for (int mode = 0; mode < 4 && err == hipSuccess; mode++) {
+                const StreamVariant v{u, mode & 1, mode >> 1};
+                err = hipEventRecord(e0, stream);
+                for (int i = 0; i < iterations; i++) launch(v, i % sets);
+                if (err == hipSuccess) err = hipGetLastError();
+                if (err == hipSuccess) err = hipEventRecord(e1, stream);
+                if (err == hipSuccess) err = hipEventSynchronize(e1);
+                float ms = 0.f;
+                if (err == hipSuccess) err = hipEventElapsedTime(&ms, e0, e1);
+                const double us = (double)ms * 1e3 / iterations;
+                if (err == hipSuccess && (best == 0.0 || us < best)) {
+                    best = us;
+                    bestVariant = v;
+                }
+            }
+        }
+        if (err == hipSuccess) {
+            *outMicroseconds = best;
+            if (outVariant && variantCapacity) {
+                snprintf(outVariant, variantCapacity, "stream_floor<%d,%d,%d,%d>", readsPerWrite, bestVariant.u, bestVariant.persist, bestVariant.nt);
+            }
+        }
     }
     if (e0) (void)hipEventDestroy(e0);
     if (e1) (void)hipEventDestroy(e1);

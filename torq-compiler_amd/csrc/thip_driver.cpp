@@ -652,9 +652,14 @@ thip_status_t thip_device_mfma_rate(thip_device_t *device, int32_t random_operan
 }
 
 thip_status_t thip_device_stream_floor(thip_device_t *device, int32_t reads_per_write, size_t write_bytes, int32_t cold, double *out_microseconds) {
+    return thip_device_stream_floor_tuned(device, reads_per_write, write_bytes, cold, out_microseconds, nullptr, 0);
+}
+
+thip_status_t thip_device_stream_floor_tuned(thip_device_t *device, int32_t reads_per_write, size_t write_bytes, int32_t cold, double *out_microseconds,
+                                             char *out_variant, size_t variant_capacity) {
     if (!device || !out_microseconds) return fail(THIP_INVALID_ARGUMENT, "null argument");
     THIP_HIP(hipSetDevice(device->ordinal), "hipSetDevice");
-    const hipError_t err = measureStreamRate(reads_per_write, write_bytes, cold, nullptr, out_microseconds);
+    const hipError_t err = measureStreamRate(reads_per_write, write_bytes, cold, nullptr, out_microseconds, out_variant, variant_capacity);
     if (err == hipErrorInvalidValue) return fail(THIP_INVALID_ARGUMENT, "reads_per_write is 1, 2 or 4; write_bytes a multiple of 16 from 4 KiB to 2 GiB");
     THIP_HIP(err, "measuring the streaming floor");
     return THIP_OK;

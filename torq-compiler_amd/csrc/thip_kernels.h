@@ -267,10 +267,13 @@ hipError_t launchDecMatmul(const DecMatmulArgs &a, const LaunchCtx &ctx);
 // do nothing else, on constant or on random operand bytes.  Allocates and frees its own few KiB.
 hipError_t measureMfmaRate(int randomOperands, int blocks, int iterations, hipStream_t stream, double *outTops);
 
-// Microseconds per launch of a streaming kernel with next to no arithmetic that reads readsPerWrite (1, 2 or 4)
-// 16-byte pieces per 16 bytes written, writeBytes written per launch; cold: on rotating buffer sets larger than the
-// last-level cache.  Allocates and frees its buffers.
-hipError_t measureStreamRate(int readsPerWrite, size_t writeBytes, int cold, hipStream_t stream, double *outMicroseconds);
+// Microseconds per launch of the fastest of a family of streaming kernels with next to no arithmetic (1, 2, 4 or 8
+// 16-byte items per thread, one pass or a persistent grid-stride grid, default or non-temporal cache policy) that
+// read readsPerWrite (1, 2 or 4) 16-byte pieces per 16 bytes written, writeBytes written per launch; cold: on
+// rotating buffer sets larger than the last-level cache.  outVariant (may be null) receives the winner's name,
+// "stream_floor<reads, items per thread, persistent, non-temporal>".  Allocates and frees its buffers.
+hipError_t measureStreamRate(int readsPerWrite, size_t writeBytes, int cold, hipStream_t stream, double *outMicroseconds, char *outVariant = nullptr,
+                             size_t variantCapacity = 0);
 
 // The library's static scratch array (device memory that needs no allocation): its size and its address on the
 // current device (ask once per device, with that device current).

@@ -337,4 +337,16 @@ __device__ __forceinline__ void waitVmcnt() {
 }
 
 
+// Loads and stores of data that is used once (a bandwidth-bound op's input and output): the non-temporal cache policy.
+// A plain copy of 64 MB .. 512 MB reaches 5.7 .. 6.5 TB/s with it against 4.9 .. 5.7 TB/s with the default policy
+// (the calibration family of thip_device_stream_floor: the non-temporal member wins every shape).
+template <typename T>
+__device__ __forceinline__ T streamLoad(const void *p) {
+    return __builtin_nontemporal_load((const T *)p);
+}
+template <typename T>
+__device__ __forceinline__ void streamStore(void *p, T v) {
+    __builtin_nontemporal_store(v, (T *)p);
+}
+
 }  // namespace thip

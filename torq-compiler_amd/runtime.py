@@ -45,7 +45,7 @@ EXPORTED_SYMBOLS = [
     "thip_program_serialize", "thip_blob_free",
     "thip_device_create", "thip_device_destroy", "thip_device_name", "thip_device_alloc",
     "thip_device_free", "thip_device_h2d", "thip_device_d2h", "thip_device_synchronize",
-    "thip_device_set_event_log", "thip_device_set_dump_dirs", "thip_device_mfma_rate", "thip_device_stream_floor", "thip_infer_format", "thip_descriptor_validate", "thip_descriptor_info", "thip_descriptor_binding", "thip_descriptor_segment",
+    "thip_device_set_event_log", "thip_device_set_dump_dirs", "thip_device_mfma_rate", "thip_device_stream_floor", "thip_device_stream_floor_tuned", "thip_infer_format", "thip_descriptor_validate", "thip_descriptor_info", "thip_descriptor_binding", "thip_descriptor_segment",
     "thip_executable_create", "thip_executable_destroy", "thip_executable_run",
     "thip_executable_enqueue", "thip_executable_enqueue_noalloc", "thip_executable_wait", "thip_executable_set_wait_timeout", "thip_executable_time", "thip_executable_time_rotating",
     "thip_executable_op_count", "thip_executable_op_kernel", "thip_executable_binding_count",
@@ -283,6 +283,7 @@ def lib():
     L.thip_device_set_dump_dirs.argtypes = [vp, ctypes.c_char_p, ctypes.c_char_p]
     L.thip_device_mfma_rate.argtypes = [vp, i32, i32, i32, P(ctypes.c_double)]
     L.thip_device_stream_floor.argtypes = [vp, i32, sz, i32, P(ctypes.c_double)]
+    L.thip_device_stream_floor_tuned.argtypes = [vp, i32, sz, i32, P(ctypes.c_double), ctypes.c_char_p, sz]
     L.thip_infer_format.argtypes = [vp, sz, sz, ctypes.c_char_p, P(sz)]
     L.thip_descriptor_validate.argtypes = [vp, sz]
     L.thip_descriptor_info.argtypes = [vp, sz, vp]
@@ -364,11 +365,13 @@ class Device:
         check(lib().thip_device_mfma_rate(self._h, int(bool(random_operands)), int(workgroups), int(iterations), ctypes.byref(tops)))
         return tops.value
 
-    def stream_floor(self, reads_per_write, write_bytes, cold=True):
-        """Microseconds per launch of a streaming kernel with next to no arithmetic (benchmark calibration)."""
+    def stream_floor(self, reads_per_write, write_bytes, cold=True, variant=False):
+        """Microseconds per launch of the fastest streaming kernel with next to no arithmetic (benchmark calibration);
+        variant=True: (microseconds, name of the winning kernel)."""
         us = ctypes.c_double()
-        check(lib().thip_device_stream_floor(self._h, int(reads_per_write), int(write_bytes), int(bool(cold)), ctypes.byref(us)))
-        return us.value
+        name = ctypes.create_string_buffer(64)
+        check(lib().thip_device_stream_floor_tuned(self._h, int(reads_per_write), int(write_bytes), int(bool(cold)), ctypes.byref(us), name, 64))
+        return (us.value, name.value.decode()) if variant else us.value
 
     def set_dump_dirs(self, io_data_dir=None, buffers_dir=None):
         """Debug dumps of the bindings of blocking dispatches / of every buffer a kernel record wrote (None: off)."""
