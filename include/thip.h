@@ -562,9 +562,11 @@ thip_status_t thip_executable_wait(thip_executable_t *executable);
  * destroying it leaves its device memory in place.  The process itself stays usable. */
 thip_status_t thip_executable_set_wait_timeout(thip_executable_t *executable, int64_t milliseconds);
 
-/* thip_executable_enqueue for callers that cannot allocate device memory (code under HIP graph capture, tight
- * serving loops, harnesses that forbid it).  It has no counterpart in the reference.  The dispatch is enqueued
- * kernel by kernel (no graph is built), on device bindings only, and makes no hipMalloc / hipFree or allocating
+/* thip_executable_enqueue for callers that cannot allocate device memory at dispatch time (tight serving loops,
+ * harnesses that forbid hipMalloc after start-up, a process one of whose other streams is under HIP graph capture,
+ * during which allocation is not permitted).  It has no counterpart in the reference.  The dispatch is enqueued on
+ * the executable's own stream like every other dispatch (its kernels do not become part of a graph somebody else is
+ * capturing), kernel by kernel (no graph is built), on device bindings only, and makes no hipMalloc / hipFree or allocating
  * library call: the scratch memory of the program's kernels (the partial sums of a bf16
  * fully_connected / matmul whose K is split over blocks) is taken from an array that is part of the library's
  * device image instead of the executable's intermediates.  The results are those of thip_executable_enqueue.

@@ -14,11 +14,8 @@
 #include "iree/hal/api.h"
 
 #include "thip.h"
+#include "thip_driver.h"
 #include "thip_native_executable.h"
-
-// Provided by the driver sources described above.
-iree_status_t iree_hal_thip_driver_create(iree_string_view_t identifier, int32_t device_ordinal, iree_allocator_t host_allocator,
-                                          iree_hal_driver_t** out_driver);
 
 static iree_status_t iree_hal_thip_driver_factory_enumerate(void* self, iree_host_size_t* out_driver_info_count,
                                                             const iree_hal_driver_info_t** out_driver_infos) {

@@ -217,6 +217,36 @@ def test_gpu_eltwise(device):
         assert families(kernels) == ["eltwise_int"]
 
 
+@pytest.mark.gpu
+def test_gpu_eltwise_kernel_does_not_depend_on_where_a_binding_lies(device):
+    """Device bindings need 16-byte alignment and nothing more: the kernel an executable names when it is created is the
+    one that runs for bindings at any such address (the vector width is bounded by those 16 bytes), results included."""
+    from torq_compiler_amd import Executable
+    for wl in (w.act_workload("i2i", (9999,), np.int32, np.int8), w.fma_workload((4099,), np.int16, np.int8, scale=0.0009, output_zp=-7),
+               w.act_workload("abs", (777,), np.int32, np.int32)):
+        exe = Executable(device, wl.program.serialize())
+        named = exe.op_kernels()
+        assert named[0].startswith("eltwise_int<") and not named[0].endswith(",1>"), named
+        want = oracle_eval(wl)[0]
+        for offset in (0, 16, 48):
+            x = wl.inputs[0]
+            src = device.alloc(x.nbytes + 64)
+            dst = device.alloc(want.nbytes + 64)
+            staged = device.upload(x)
+            # upload() gives a fresh allocation; place the input at the offset through a second copy on the host side
+            host = np.zeros(x.nbytes + 64, dtype=np.uint8)
+            host[offset:offset + x.nbytes] = x.reshape(-1).view(np.uint8)
+            device.free(staged)
+            runtime.check(runtime.lib().thip_device_h2d(device.handle, src, host.ctypes.data, host.nbytes))
+            exe.run_device([src + offset, dst + offset], [x.nbytes, want.nbytes])
+            got = device.download(dst, (want.nbytes + 64,), np.uint8)[offset:offset + want.nbytes].view(want.dtype).reshape(want.shape)
+            assert_bit_exact(got, want, "%s at +%d" % (wl.name, offset))
+            assert exe.op_kernels() == named
+            device.free(src)
+            device.free(dst)
+        exe.close()
+
+
 # ---- comparisons, logical ops, bitwise not, shifts ------------------------------------------------------------------
 def test_oracle_compare_logical_and_not():
     """What pins them is the arith op each mode replaces (ArithToTorqHLPattern.cpp:104-131,181-251): numpy's comparison /

@@ -352,8 +352,11 @@ def test_fully_connected_config1(device, mkn):
           kernel=("fc_skinny<1,4>" if M == 1 else "fc_skinny_mfma") if M <= 16 else ("igemm_dense_k128_i8" if M >= 512 else None))
 
 
-def test_fully_connected_config1_literal_ranges(device):
-    check(device, w.fully_connected_workload(16, 2048, 8192))
+@pytest.mark.parametrize("mkn", [(1, 2048, 2048), (16, 2048, 8192), (512, 4096, 4096)])
+def test_fully_connected_config1_literal_ranges(device, mkn):
+    # the benchmark's own requant range (shift 6 .. 12 under multipliers of 2^30 and more): every output saturates, and the
+    # dense tiles requantise it through the pre-shifted 32-bit tail with the accumulator clamped first
+    check(device, w.fully_connected_workload(*mkn), via="device")
 
 
 @pytest.mark.parametrize("mkn", [(1, 1, 1), (1, 61, 1991), (4, 1024, 1024), (1, 2000, 97), (16, 3, 7), (17, 128, 70),

@@ -1118,7 +1118,9 @@ __global__ __launch_bounds__(256) void table_lookup(EltwiseArgs p) {
 
 template <typename TIN, typename TOUT>
 static hipError_t launchTableT(const EltwiseArgs &a, const LaunchCtx &ctx) {
-    constexpr int VEC = sizeof(TIN) == 1 && sizeof(TOUT) == 1 ? 16 : 8;
+    // 16 bytes of the wider side per thread: the widest access is then 16 bytes, the alignment every device binding has
+    // (a wider one would make the kernel depend on where a binding happens to lie, dispatch by dispatch)
+    constexpr int VEC = 16 / (int)(sizeof(TIN) > sizeof(TOUT) ? sizeof(TIN) : sizeof(TOUT));
     const bool aligned = (((uintptr_t)a.in0) & (sizeof(TIN) * VEC - 1)) == 0 && (((uintptr_t)a.out) & (sizeof(TOUT) * VEC - 1)) == 0;
     if (aligned) {
         const long long threads = (a.count + VEC - 1) / VEC;
@@ -1131,7 +1133,9 @@ static hipError_t launchTableT(const EltwiseArgs &a, const LaunchCtx &ctx) {
 
 template <typename TIN, typename TOUT>
 static hipError_t launchEltwiseT(const EltwiseArgs &a, const LaunchCtx &ctx) {
-    constexpr int VEC = sizeof(TIN) == 1 && sizeof(TOUT) == 1 ? 16 : 8;
+    // 16 bytes of the wider side per thread: the widest access is then 16 bytes, the alignment every device binding has
+    // (a wider one would make the kernel depend on where a binding happens to lie, dispatch by dispatch)
+    constexpr int VEC = 16 / (int)(sizeof(TIN) > sizeof(TOUT) ? sizeof(TIN) : sizeof(TOUT));
     const uintptr_t bits = (uintptr_t)a.in0 | (eltwiseTwoInputs(a.op) ? (uintptr_t)a.in1 : 0);
     const bool aligned = (bits & (sizeof(TIN) * VEC - 1)) == 0 && (((uintptr_t)a.out) & (sizeof(TOUT) * VEC - 1)) == 0;
     if (aligned) {

@@ -430,6 +430,36 @@ class Emitter {
         op->t0_clamp = (int32_t)bound;
     }
 
+    // What the tile choice knows about the machine, and every cut-off measured on it, in one place: a different part
+    // (another CU count, another LDS size) is re-tuned here and nowhere else.  Tile counts are in units of the chip.
+    struct TileRule {
+        static constexpr int64_t kCus = 256;                // compute units (8 XCDs of 32)
+        static constexpr int64_t kFillsChip = kCus * 7 / 8; // 224 tiles: a one-block-per-CU tile (nearly) fills the chip
+        static constexpr int64_t kFillsChipSmall = kCus * 3 / 4;  // 192: the same for the 128-wide and narrower tiles
+        static constexpr int64_t kHalfChip = kCus / 2;      // 128: a window tile with a long K pays from half the CUs on
+        static constexpr int64_t kTwoPerCu = 2 * kCus;      // 512 tiles
+        static constexpr int64_t kSmallTilesMax = kCus * 5 / 2;   // 640 small tiles: beyond, a tile column reads the image once
+        static constexpr int64_t kIdleShareDen = 10;        // a last round of tiles more than 1/10 idle counts as idle
+        static constexpr int64_t kPadShareDen = 8;          // padding N (or K) by more than 1/8 counts as wasteful
+        // the streaming kernel (weights resident in LDS)
+        static constexpr int64_t kStreamMinM = 4096;
+        static constexpr int64_t kStreamAlwaysM = 200000;   // K <= 128: ahead from here whatever N
+        static constexpr int64_t kStreamExpandM = 40000;    // N >= 2 K, K <= 32
+        static constexpr int64_t kStreamLongKExpandM = 25000;     // K > 128, N >= 2 K
+        static constexpr int64_t kStreamLongKMaxOutputs = 1LL << 28;
+        static constexpr int64_t kStreamAddM = 400000;      // K > 128 with an add behind it
+        static constexpr int64_t kStreamShortK = 128, kStreamTinyK = 32;
+        // dense tiles
+        static constexpr int64_t kColumnMinM = 16384;       // N <= 128: one tile column from this many rows
+        static constexpr int64_t kShortK = 256, kShortKMaxOutputs = 1LL << 28, kShortKMaxM = 600000;
+        static constexpr int64_t kShortKWide = 384, kShortKWideMaxM = 65536;
+        static constexpr int64_t kLargestTileMinK = 512;    // up to here the 256 x 256 tile is mostly prologue and epilogue
+        static constexpr int64_t kRoundRuleMaxK = 1024;     // the idle-last-round rule applies up to this K
+        static constexpr int64_t kK128From = 4096;          // 128-byte k-tiles on the 128 x 128 tile from this K
+        // window tiles
+        static constexpr int64_t kWindowLargestMinK = 640;
+    };
+
     // Tile choice.  THIP_IGEMM_VARIANT / THIP_IGEMM_DENSE_VARIANT force one (for tuning runs).  addFollows: the
     // record's only reader is a torq_hl.add right behind it, which the streaming kernel and the 64 x 64 tile can fold.
     static uint32_t chooseIgemmVariant(int64_t M, int64_t N, bool dense, int64_t K = 0, int32_t outDtype = 0, bool runs = false, bool addFollows = false) {
@@ -452,26 +482,26 @@ class Emitter {
             // up to 2^28 outputs (beyond that its passes over the activations, one per 256 channels, cost more), or
             // where an add follows a very large image (the fused add saves more than the dense tile gains); below
             // those sizes a dense tile is 10-50 % faster.
-            if (M >= 4096 && igemmStreamFits(N, K, outDtype) && !getenv("THIP_NO_STREAM")) {
+            if (M >= TileRule::kStreamMinM && igemmStreamFits(N, K, outDtype) && !getenv("THIP_NO_STREAM")) {
                 const bool expanding = N >= 2 * K;
                 const char *em = getenv("THIP_STREAM_EXPAND_MIN_M");  // tuning: the pixel count from which an expanding layer streams
-                const bool take = K <= 128 ? (M >= 200000 || (expanding && K <= 32 && M >= (em ? atoll(em) : 40000)))
-                                           : ((expanding && M >= 25000 && M * N < (1LL << 28)) || (addFollows && M >= 400000));
+                const bool take = K <= TileRule::kStreamShortK ? (M >= TileRule::kStreamAlwaysM || (expanding && K <= TileRule::kStreamTinyK && M >= (em ? atoll(em) : TileRule::kStreamExpandM)))
+                                           : ((expanding && M >= TileRule::kStreamLongKExpandM && M * N < TileRule::kStreamLongKMaxOutputs) || (addFollows && M >= TileRule::kStreamAddM));
                 if (take) return kIgemmStream;
             }
             // an add behind it: the small tile folds the add into its epilogue, which beats a larger tile plus an add kernel
             if (addFollows && outDtype == THIP_DTYPE_I8 && N % 16 == 0) return kIgemmDense64x64;
             // N narrower than a tile: one tile column of the narrowest tile that covers N, so the
             // activations are streamed once (these shapes are bandwidth-bound, padded MFMA work is free)
-            if (N <= 128 && M >= 16384) {
+            if (N <= 128 && M >= TileRule::kColumnMinM) {
                 return N <= 32 ? kIgemmDense256x32 : N <= 64 ? kIgemmDense256x64 : kIgemmDense256x128;
             }
             // a short K (up to six k-tiles) over at least two tiles per CU: the 128 x 128 tile, which the launcher then runs
             // two stages deep with four blocks per CU, so that the prologues and epilogues that dominate such tiles
             // overlap (256 -> 1024 channels at 56 x 56, batch 8: 13.5 us against 16.2 on 128 x 256; 64 -> 256 over 100 352
             // pixels: 10.4 against 12.0; from 400 000 pixels x 960 channels the wider tile is 3 % ahead again)
-            const bool shortK = K > 0 && ((K <= 256 && M * N < (1LL << 28) && M < 600000) || (K <= 384 && M < 65536));
-            if (shortK && N > 128 && tiles(kIgemmDense128x128) >= 512 && (roundUp(N, 128) - N) * 8 <= N && !getenv("THIP_NO_SHORTK_TILE")) {
+            const bool shortK = K > 0 && ((K <= TileRule::kShortK && M * N < TileRule::kShortKMaxOutputs && M < TileRule::kShortKMaxM) || (K <= TileRule::kShortKWide && M < TileRule::kShortKWideMaxM));
+            if (shortK && N > 128 && tiles(kIgemmDense128x128) >= TileRule::kTwoPerCu && (roundUp(N, 128) - N) * TileRule::kPadShareDen <= N && !getenv("THIP_NO_SHORTK_TILE")) {
                 return kIgemmDense128x128;
             }
             // a long K on the largest tile: k-tiles of 128 bytes, whole cache lines per row (THIP_NO_K128 keeps 64)
@@ -479,25 +509,25 @@ class Emitter {
             // it at nearly twice the speed: with K of 513 .. 1024 and more than a tenth of the last round idle the
             // largest tile is skipped - 100 352 x 768 x 512, 784 tiles: 56.3 us on 128 x 256 against 74.7; K = 1024: 69.3
             // against 80.4; with 392 tiles and K = 1024 both take 39 us, and from K = 1536 the 128-byte k-tiles win)
-            const int64_t t256 = tiles(kIgemmDense256x256), rounds256 = (t256 + 255) / 256;
-            const bool idleLastRound = (rounds256 * 256 - t256) * 10 > rounds256 * 256;
-            const bool skipLargest = K > 512 && K <= 1024 && idleLastRound && (K < 1024 || t256 >= 512) && !getenv("THIP_NO_ROUND_RULE");
+            const int64_t t256 = tiles(kIgemmDense256x256), rounds256 = (t256 + TileRule::kCus - 1) / TileRule::kCus;
+            const bool idleLastRound = (rounds256 * TileRule::kCus - t256) * TileRule::kIdleShareDen > rounds256 * TileRule::kCus;
+            const bool skipLargest = K > TileRule::kLargestTileMinK && K <= TileRule::kRoundRuleMaxK && idleLastRound && (K < TileRule::kRoundRuleMaxK || t256 >= TileRule::kTwoPerCu) && !getenv("THIP_NO_ROUND_RULE");
             // (the 128-byte k-tiles are ahead from K = 576 on, padded to whole k-tiles: 8192 x 640 x 4096 32.7 us against
             // 36.8, 16384 x 768 x 4096 71.3 against 78.7, 4096 x 960 x 4096 23.0 against 23.4)
-            if (K > 512 && (roundUp(K, 128) - K) * 8 <= K && tiles(kIgemmDense256x256) >= 224 && !skipLargest && !getenv("THIP_NO_K128")) return kIgemmDense256x256K128;
+            if (K > TileRule::kLargestTileMinK && (roundUp(K, 128) - K) * TileRule::kPadShareDen <= K && tiles(kIgemmDense256x256) >= TileRule::kFillsChip && !skipLargest && !getenv("THIP_NO_K128")) return kIgemmDense256x256K128;
             // otherwise the largest tile that still gives (nearly) every CU a tile and does not pad N by more than an
             // eighth where a narrower tile that fills the chip would not (padded columns are computed too)
             // a long K in whole 128-byte k-tiles on more 128 x 128 tiles than CUs: the launcher runs that tile with
             // 128-byte k-tiles, ahead of the wider tile (1536 x 4096 x 4096: 28.8 us against 31.7, 3000 rows: 54.5 against 60.1)
-            if (K >= 4096 && K % 128 == 0 && tiles(kIgemmDense128x128) > 256 && (roundUp(N, 128) - N) * 8 <= N && !getenv("THIP_NO_K128")) return kIgemmDense128x128;
+            if (K >= TileRule::kK128From && K % 128 == 0 && tiles(kIgemmDense128x128) > TileRule::kCus && (roundUp(N, 128) - N) * TileRule::kPadShareDen <= N && !getenv("THIP_NO_K128")) return kIgemmDense128x128;
             const uint32_t order[] = {kIgemmDense256x256, kIgemmDense128x256, kIgemmDense128x128, kIgemmDense64x128, kIgemmDense128x64};
-            auto enough = [&](uint32_t v) { return tiles(v) >= (v == kIgemmDense128x128 || v == kIgemmDense128x64 ? 192 : 224); };
-            auto wasteful = [&](uint32_t v) { return (roundUp(N, igemmTile(v).bn) - N) * 8 > N; };
+            auto enough = [&](uint32_t v) { return tiles(v) >= (v == kIgemmDense128x128 || v == kIgemmDense128x64 ? TileRule::kFillsChipSmall : TileRule::kFillsChip); };
+            auto wasteful = [&](uint32_t v) { return (roundUp(N, igemmTile(v).bn) - N) * TileRule::kPadShareDen > N; };
             for (size_t i = 0; i < sizeof(order) / sizeof(order[0]); i++) {
                 const uint32_t v = order[i];
                 // a short K leaves a 256 x 256 tile (one block per CU) mostly prologue and epilogue; two blocks per CU
                 // of half the size overlap them (256 -> 1024 channels at 56 x 56, batch 32: 75 -> 54 us)
-                if (v == kIgemmDense256x256 && K > 0 && (K <= 512 || skipLargest)) continue;
+                if (v == kIgemmDense256x256 && K > 0 && (K <= TileRule::kLargestTileMinK || skipLargest)) continue;
                 if (v == kIgemmDense64x128 && (wasteful(v) || getenv("THIP_NO_64X128"))) continue;
                 if (!enough(v)) continue;
                 bool better = false;
@@ -512,9 +542,9 @@ class Emitter {
             if (v >= 0 && v < (long)kIgemmDense256x256) return (uint32_t)v;
         }
         // window-row runs of a few-channel image, few output channels: the streaming kernel gathers them too
-        if (runs && M >= 4096 && N <= 128 && igemmStreamFits(N, K, outDtype) && !getenv("THIP_NO_STREAM")) return kIgemmStream;
+        if (runs && M >= TileRule::kStreamMinM && N <= 128 && igemmStreamFits(N, K, outDtype) && !getenv("THIP_NO_STREAM")) return kIgemmStream;
         // Enough 128x128 tiles to give every CU work (and N wide enough to use them); otherwise the small tile.
-        if (N > 64 && tiles(kIgemm128x128x64) >= 256) return kIgemm128x128x64;
+        if (N > 64 && tiles(kIgemm128x128x64) >= TileRule::kCus) return kIgemm128x128x64;
         return kIgemm64x64x64;
     }
 
@@ -534,32 +564,32 @@ class Emitter {
         // (144 channels are 256 either way: 144 -> 144 at 56 x 56, batch 32, 45.1 us on 256 x 256 against 48.3 on 128 x 128)
         auto wasteful = [&](uint32_t v) {
             const int64_t np = roundUp(N, igemmTile(v).bn);
-            return np > roundUp(N, 128) && (np - N) * 8 > N;
+            return np > roundUp(N, 128) && (np - N) * TileRule::kPadShareDen > N;
         };
         // up to two small tiles per CU: the 64 x 64 tile (four blocks per CU) spreads a small convolution over the chip
         // (256 -> 256 at 14 x 14: 10.3 us against 13.7 on 7 tiles of 128 x 128; 512 -> 512 at 14 x 14, batch 16, 392
         // tiles: 17.8 against 24.2; at 784 tiles the 128 x 128 tile is ahead, 14.5 against 19.8)
-        if (tiles(kIgemmDense64x64) <= 512) return kIgemmDense64x64;
+        if (tiles(kIgemmDense64x64) <= TileRule::kTwoPerCu) return kIgemmDense64x64;
         // few output channels: one tile column, the image is read once (64 -> 64 at 112 x 112, batch 32: 27.8 us against
         // 41.1 with 128 x 128 tiles).  At most 64 output channels never take a wider tile (32 -> 64 at 112 x 112, batch
         // 3 / 4: 6.2 / 7.2 us on 588 / 784 small tiles, 6.5 / 6.6 on one column of 256 x 64, 7.0 / 7.1 on 128 x 128); up
         // to 128 take theirs with a tile per CU, below that the 128 x 128 tile wins (128 -> 128 at 28 x 28, batch 8: 8.5 us
         // against 12.4)
         // (and at most 32 take the 32-wide column: 32 -> 16 at 112 x 112, batch 32: 19.2 us against 22.4)
-        if (N <= 64) return tiles(kIgemmDense64x64) <= 640 ? kIgemmDense64x64 : N <= 32 ? kIgemmDense256x32 : kIgemmDense256x64;
-        if (N <= 128 && tiles(kIgemmDense256x128) >= 224) return kIgemmDense256x128;
+        if (N <= 64) return tiles(kIgemmDense64x64) <= TileRule::kSmallTilesMax ? kIgemmDense64x64 : N <= 32 ? kIgemmDense256x32 : kIgemmDense256x64;
+        if (N <= 128 && tiles(kIgemmDense256x128) >= TileRule::kFillsChip) return kIgemmDense256x128;
         // measured on 3x3 convolutions of 64 .. 512 channels at batch 1 .. 64: the largest tile wins as soon as half the CUs
         // get one (a long K per tile amortises its prologue and epilogue), unless it pads N by more than an eighth
         // (a short K leaves the largest tile mostly prologue and epilogue, as in the dense choice: 64 -> 256 at 56 x 56,
         // batch 32, K = 576: 24.7 us on 128 x 256 against 27.5)
         // (and, as there, up to K = 1024 a mostly idle last round of the largest tiles costs more than two half-size
         // blocks per CU: 112 -> 512 at 56 x 56, batch 32, K = 1008, 3.06 rounds: 68.1 us against 80.1)
-        const int64_t t256 = tiles(kIgemmDense256x256), rounds256 = (t256 + 255) / 256;
-        const bool idleLastRound = (rounds256 * 256 - t256) * 10 > rounds256 * 256 && !getenv("THIP_NO_ROUND_RULE");
-        if (K > 640 && !(K <= 1024 && idleLastRound) && tiles(kIgemmDense256x256) >= 128 && !wasteful(kIgemmDense256x256)) {
+        const int64_t t256 = tiles(kIgemmDense256x256), rounds256 = (t256 + TileRule::kCus - 1) / TileRule::kCus;
+        const bool idleLastRound = (rounds256 * TileRule::kCus - t256) * TileRule::kIdleShareDen > rounds256 * TileRule::kCus && !getenv("THIP_NO_ROUND_RULE");
+        if (K > TileRule::kWindowLargestMinK && !(K <= TileRule::kRoundRuleMaxK && idleLastRound) && tiles(kIgemmDense256x256) >= TileRule::kHalfChip && !wasteful(kIgemmDense256x256)) {
             return (C % 128 == 0 && !getenv("THIP_NO_K128")) ? kIgemmDense256x256K128 : kIgemmDense256x256;
         }
-        if (tiles(kIgemmDense128x256) >= 128 && !wasteful(kIgemmDense128x256)) return kIgemmDense128x256;
+        if (tiles(kIgemmDense128x256) >= TileRule::kHalfChip && !wasteful(kIgemmDense128x256)) return kIgemmDense128x256;
         return kIgemmDense128x128;
     }
 
