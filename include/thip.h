@@ -604,6 +604,16 @@ thip_status_t thip_executable_binding_count(thip_executable_t *executable, uint3
 thip_status_t thip_executable_binding_size(thip_executable_t *executable, uint32_t binding,
                                            size_t *out_size);
 
+/* The GEMM tile that thip_program_serialize gives an integer conv2d / fully_connected / matmul of M output pixels
+ * (rows), N output channels and a reduction of K bytes, without building the program: `addressing` 0 = a dense
+ * [M][K] operand (1x1 convolution, fully_connected, matmul), 1 = gathered taps, 2 = whole window rows of a
+ * few-channel image, 3 = a KxK window on an image of C channels; `add_follows`: the result's only reader is a
+ * torq_hl.add right behind it.  *out_variant is the record's tile number, `name` its tile ("igemm_dense_i8_256x256x64", ...).  The
+ * THIP_* tuning switches apply as they do at serialisation.  (The role the kernel selectors of
+ * compiler/torq/Conversions/TorqHLToTorqHW/Conv2DToHw.cpp:150-186 play for the NPU; for tuning tools and tests.) */
+thip_status_t thip_gemm_tile_choice(int32_t addressing, int64_t M, int64_t N, int64_t K, int64_t C, int32_t out_dtype,
+                                    int32_t add_follows, uint32_t *out_variant, char *name, size_t capacity);
+
 /* Per-dispatch event log (role of TorqEventLog, runtime/torq_hw/inc/TorqEventLog.h:19-46, .cpp:48,97-101): when a
  * path is set every dispatch appends rows in the reference's runtime CSV columns (doc/user-manual/profiling.md:53-63)
  * dispatch_name, invocation_id, action_id, timestamp_us, event -- event an EventType name plus _BEGIN / _END:

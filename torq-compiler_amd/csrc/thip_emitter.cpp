@@ -116,6 +116,11 @@ class Emitter {
     explicit Emitter(const thip_program_t &prog) : prog_(prog), state_(prog.values.size()) {}
 
     thip_status_t run(void **outBlob, size_t *outSize);
+    // The tile a GEMM-shaped record of this geometry gets (the rule emitIgemm applies), for thip_gemm_tile_choice.
+    static uint32_t tileChoice(uint32_t loader, int64_t M, int64_t N, int64_t K, int64_t C, int32_t outDtype, bool addFollows) {
+        return loader == kLoaderWindow ? chooseWindowVariant(M, N, C, K)
+                                       : chooseIgemmVariant(M, N, loader == kLoaderDense, K, outDtype, loader == kLoaderRuns, addFollows);
+    }
 
   private:
     const thip_program_t &prog_;
@@ -598,8 +603,7 @@ class Emitter {
     template <typename WeightAt>
     void emitIgemm(DescOp base, int64_t M, int64_t N, int64_t K, uint32_t loader, WeightAt wAt) {
         const bool dense = loader == kLoaderDense;
-        const uint32_t variant = loader == kLoaderWindow ? chooseWindowVariant(M, N, base.C, K)
-                                                         : chooseIgemmVariant(M, N, dense, K, base.out_dtype, loader == kLoaderRuns, addFollows_);
+        const uint32_t variant = tileChoice(loader, M, N, K, base.C, base.out_dtype, addFollows_);
         const IgemmTile &t = igemmTile(variant);
         const int64_t Kp = roundUp(K, t.bk), Np = roundUp(N, t.bn);
         std::vector<int8_t> packed((size_t)(Np * Kp), 0);
@@ -2570,6 +2574,17 @@ thip_status_t thip_program_view(thip_program_t *program, thip_value_t base, int6
     v.base = root;
     v.viewOffset = rootOffset + element_offset;
     v.binding = program->values[(size_t)root].binding;
+    return THIP_OK;
+}
+
+thip_status_t thip_gemm_tile_choice(int32_t addressing, int64_t M, int64_t N, int64_t K, int64_t C, int32_t out_dtype, int32_t add_follows,
+                                    uint32_t *out_variant, char *name, size_t capacity) {
+    if (!out_variant) return fail(THIP_INVALID_ARGUMENT, "thip_gemm_tile_choice: null result pointer");
+    if (addressing < (int32_t)kLoaderDense || addressing > (int32_t)kLoaderWindow) return fail(THIP_INVALID_ARGUMENT, "thip_gemm_tile_choice: addressing %d is none of 0 .. 3", (int)addressing);
+    if (M < 1 || N < 1 || K < 1 || C < 1) return fail(THIP_INVALID_ARGUMENT, "thip_gemm_tile_choice: M, N, K and C must be positive");
+    const uint32_t v = Emitter::tileChoice((uint32_t)addressing, M, N, K, C, (int32_t)out_dtype, add_follows != 0);
+    *out_variant = v;
+    if (name && capacity) snprintf(name, capacity, "%s", igemmTile(v).name);
     return THIP_OK;
 }
 

@@ -39,7 +39,7 @@ BINDING_HOST, BINDING_DEVICE = 0, 1
 EXPORTED_SYMBOLS = [
     "thip_status_message", "thip_version", "thip_descriptor_version",
     "thip_program_create", "thip_program_destroy", "thip_program_set_name", "thip_program_binding", "thip_program_constant",
-    "thip_program_tensor", "thip_program_view", "thip_hl_conv2d", "thip_hl_depthwise_conv2d", "thip_hl_fully_connected",
+    "thip_program_tensor", "thip_program_view", "thip_gemm_tile_choice", "thip_hl_conv2d", "thip_hl_depthwise_conv2d", "thip_hl_fully_connected",
     "thip_hl_matmul", "thip_hl_maxpool2d", "thip_hl_avg_pool2d", "thip_hl_add", "thip_hl_transpose", "thip_hl_expand_weights",
     "thip_hl_fma", "thip_hl_mul", "thip_hl_act", "thip_hl_elementwisebinary", "thip_hl_elementwiseunary", "thip_hl_elementwiseshift", "thip_hl_table",
     "thip_program_serialize", "thip_blob_free",
@@ -260,6 +260,7 @@ def lib():
     L.thip_program_constant.argtypes = [vp, i32, i32, P(ctypes.c_int64), vp, sz, P(i32)]
     L.thip_program_tensor.argtypes = [vp, i32, i32, P(ctypes.c_int64), P(i32)]
     L.thip_program_view.argtypes = [vp, i32, ctypes.c_int64, i32, P(ctypes.c_int64), P(i32)]
+    L.thip_gemm_tile_choice.argtypes = [i32, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, i32, i32, P(ctypes.c_uint32), ctypes.c_char_p, ctypes.c_size_t]
     for name, st in [("thip_hl_conv2d", HlConv2d), ("thip_hl_depthwise_conv2d", HlDepthwiseConv2d),
                      ("thip_hl_fully_connected", HlFullyConnected), ("thip_hl_matmul", HlMatmul),
                      ("thip_hl_maxpool2d", HlMaxPool2d), ("thip_hl_avg_pool2d", HlAvgPool2d),
@@ -389,6 +390,17 @@ def infer_format(blob):
     size = ctypes.c_size_t(0)
     check(lib().thip_infer_format(blob, len(blob), 32, buf, ctypes.byref(size)))
     return buf.value.decode(), size.value
+
+
+ADDRESSING_DENSE, ADDRESSING_GATHER, ADDRESSING_RUNS, ADDRESSING_WINDOW = 0, 1, 2, 3
+
+
+def gemm_tile_choice(addressing, M, N, K, C=1, out_dtype=1, add_follows=False):
+    """(tile number, tile name) the serialiser gives an integer GEMM-shaped op of this geometry (thip_gemm_tile_choice)."""
+    v = ctypes.c_uint32()
+    buf = ctypes.create_string_buffer(64)
+    check(lib().thip_gemm_tile_choice(int(addressing), int(M), int(N), int(K), int(C), int(out_dtype), int(bool(add_follows)), ctypes.byref(v), buf, 64))
+    return v.value, buf.value.decode()
 
 
 def make_state(ptrs, lengths, flags, constants=None):
