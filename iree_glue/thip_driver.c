@@ -1,11 +1,17 @@
-// The HAL driver object of "thip": enumerates the one default device and creates HAL devices on GPU ordinals.
-// Counterpart of runtime/driver/torq_driver.c:35-157 without its executable loaders and shared allocator (the thip
-// device brings its own executable cache and allocator, both thin layers over include/thip.h).
+// The HAL driver object of "thip": enumerates the one default device and creates it.  Counterpart of
+// runtime/driver/torq_driver.c:35-157.  The device it creates is the reference's own synchronous device
+// (iree_hal_torq_device_create, runtime/driver/torq_device.h:36-41) over IREE's heap allocator: its executable cache
+// (runtime/driver/nop_executable_cache.cc, with the two hunks of README.md) prepares "thip-gfx950" executables, its
+// command buffer (runtime/driver/torq_command_buffer.c, one hunk) dispatches them, and its buffers reach the library
+// as host pointers, which the library stages.  No CPU executable loaders: a module compiled for this target holds none.
 #include "thip_driver.h"
 
+#include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
-#include "thip_device.h"
+#include "thip.h"
+#include "torq_device.h"
 
 typedef struct iree_hal_thip_driver_t {
   iree_hal_resource_t resource;
@@ -68,7 +74,19 @@ static iree_status_t iree_hal_thip_driver_create_device_by_id(iree_hal_driver_t*
                                                               iree_allocator_t host_allocator, iree_hal_device_t** out_device) {
   iree_hal_thip_driver_t* driver = iree_hal_thip_driver_cast(base);
   const int32_t ordinal = device_id == IREE_HAL_DEVICE_ID_DEFAULT ? driver->default_ordinal : (int32_t)device_id;
-  return iree_hal_thip_device_create(driver->identifier, ordinal, host_allocator, out_device);
+  // the executables of a process share one GPU (thip_native_executable.cc reads THIP_DEVICE_ORDINAL with the first)
+  char text[16];
+  snprintf(text, sizeof(text), "%d", (int)ordinal);
+  setenv("THIP_DEVICE_ORDINAL", text, /*overwrite=*/1);
+  iree_hal_torq_device_params_t device_params;
+  iree_hal_torq_device_params_initialize(&device_params);
+  device_params.is_dmabuf_mode = false;
+  iree_hal_allocator_t* device_allocator = NULL;
+  IREE_RETURN_IF_ERROR(iree_hal_allocator_create_heap(IREE_SV("local"), host_allocator, host_allocator, &device_allocator));
+  iree_status_t status = iree_hal_torq_device_create(driver->identifier, &device_params, /*loader_count=*/0, /*loaders=*/NULL,
+                                                     device_allocator, host_allocator, out_device);
+  iree_hal_allocator_release(device_allocator);
+  return status;
 }
 
 static iree_status_t iree_hal_thip_driver_create_device_by_path(iree_hal_driver_t* base, iree_string_view_t driver_name,

@@ -1,21 +1,12 @@
 // Registration of the HAL driver "thip" with IREE's driver registry: the counterpart of
 // runtime/driver/registration/driver_module.c:95-168 (factory enumerate / try_create for one driver name).
 //
-// The driver and device objects themselves are the reference's (runtime/driver/torq_driver.c, torq_device.c) with
-// three substitutions, all of them calls into include/thip.h:
-//   - the device owns one thip_device_t (thip_device_create(ordinal) at creation, thip_device_destroy at the end);
-//   - its allocator hands out device-local buffers from thip_device_alloc / thip_device_free and moves data with
-//     thip_device_h2d / thip_device_d2h (the roles of TorqHw::allocateDeviceBuffer / writeXram / readXram,
-//     runtime/torq_hw/inc/TorqHw.h:96-121); host-visible buffers stay plain host memory and are staged by the library;
-//   - its command buffer's dispatch (runtime/driver/torq_command_buffer.c:390-512) builds the dispatch state as
-//     before and calls iree_hal_thip_native_executable_run, passing for every binding whether its buffer came from
-//     thip_device_alloc.
+// The driver object is thip_driver.c; the device it creates is the reference's own (see there).
 #include "iree/base/api.h"
 #include "iree/hal/api.h"
 
 #include "thip.h"
 #include "thip_driver.h"
-#include "thip_native_executable.h"
 
 static iree_status_t iree_hal_thip_driver_factory_enumerate(void* self, iree_host_size_t* out_driver_info_count,
                                                             const iree_hal_driver_info_t** out_driver_infos) {

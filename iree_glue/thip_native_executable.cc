@@ -4,7 +4,10 @@
 // types and statuses.
 #include "thip_native_executable.h"
 
+#include <stdlib.h>
 #include <string.h>
+
+#include "iree/base/internal/synchronization.h"
 
 typedef struct iree_hal_thip_native_executable_t {
   iree_hal_resource_t resource;
@@ -20,22 +23,68 @@ static iree_status_t iree_hal_thip_status(thip_status_t status) {
   return iree_make_status((iree_status_code_t)status, "%s", thip_status_message());
 }
 
+// The one thip_device_t of the process, counted by the executables that use it.
+static iree_slim_mutex_t iree_hal_thip_shared_mutex = IREE_SLIM_MUTEX_INIT;
+static thip_device_t* iree_hal_thip_shared_device = NULL;
+static int iree_hal_thip_shared_users = 0;
+
+static iree_status_t iree_hal_thip_shared_device_acquire(thip_device_t** out_device) {
+  iree_status_t status = iree_ok_status();
+  iree_slim_mutex_lock(&iree_hal_thip_shared_mutex);
+  if (!iree_hal_thip_shared_device) {
+    const char* ordinal = getenv("THIP_DEVICE_ORDINAL");
+    status = iree_hal_thip_status(thip_device_create(ordinal ? atoi(ordinal) : 0, &iree_hal_thip_shared_device));
+  }
+  if (iree_status_is_ok(status)) {
+    ++iree_hal_thip_shared_users;
+    *out_device = iree_hal_thip_shared_device;
+  }
+  iree_slim_mutex_unlock(&iree_hal_thip_shared_mutex);
+  return status;
+}
+
+static void iree_hal_thip_shared_device_release(void) {
+  iree_slim_mutex_lock(&iree_hal_thip_shared_mutex);
+  if (--iree_hal_thip_shared_users == 0) {
+    thip_device_destroy(iree_hal_thip_shared_device);
+    iree_hal_thip_shared_device = NULL;
+  }
+  iree_slim_mutex_unlock(&iree_hal_thip_shared_mutex);
+}
+
+thip_device_t* iree_hal_thip_device_handle(void) {
+  iree_slim_mutex_lock(&iree_hal_thip_shared_mutex);
+  thip_device_t* device = iree_hal_thip_shared_device;
+  iree_slim_mutex_unlock(&iree_hal_thip_shared_mutex);
+  return device;
+}
+
+bool iree_hal_thip_native_executable_isa(iree_hal_executable_t* executable) {
+  return iree_hal_resource_is(executable, &iree_hal_thip_native_executable_vtable);
+}
+
 static iree_hal_thip_native_executable_t* iree_hal_thip_native_executable_cast(iree_hal_executable_t* base_value) {
   IREE_HAL_ASSERT_TYPE(base_value, &iree_hal_thip_native_executable_vtable);
   return (iree_hal_thip_native_executable_t*)base_value;
 }
 
-iree_status_t iree_hal_thip_native_executable_create(thip_device_t* thip_device, iree_allocator_t host_allocator,
+iree_status_t iree_hal_thip_native_executable_create(iree_hal_device_t* device, iree_allocator_t host_allocator,
                                                      const iree_hal_executable_params_t* executable_params,
                                                      iree_hal_executable_t** out_executable) {
-  IREE_ASSERT_ARGUMENT(thip_device);
+  (void)device;  // buffers reach the dispatch as host pointers whatever device allocated them
   IREE_ASSERT_ARGUMENT(executable_params);
   IREE_ASSERT_ARGUMENT(out_executable);
   *out_executable = NULL;
   IREE_TRACE_ZONE_BEGIN(z0);
 
   iree_hal_thip_native_executable_t* executable = NULL;
-  iree_status_t status = iree_allocator_malloc(host_allocator, sizeof(*executable), (void**)&executable);
+  thip_device_t* thip_device = NULL;
+  iree_status_t status = iree_hal_thip_shared_device_acquire(&thip_device);
+  if (!iree_status_is_ok(status)) {
+    IREE_TRACE_ZONE_END(z0);
+    return status;
+  }
+  status = iree_allocator_malloc(host_allocator, sizeof(*executable), (void**)&executable);
   if (iree_status_is_ok(status)) {
     iree_hal_resource_initialize(&iree_hal_thip_native_executable_vtable, &executable->resource);
     executable->host_allocator = host_allocator;
@@ -47,8 +96,9 @@ iree_status_t iree_hal_thip_native_executable_create(thip_device_t* thip_device,
   }
   if (iree_status_is_ok(status)) {
     *out_executable = (iree_hal_executable_t*)executable;
-  } else if (executable) {
-    iree_allocator_free(host_allocator, executable);
+  } else {
+    if (executable) iree_allocator_free(host_allocator, executable);
+    iree_hal_thip_shared_device_release();
   }
   IREE_TRACE_ZONE_END(z0);
   return status;
@@ -60,6 +110,7 @@ static void iree_hal_thip_native_executable_destroy(iree_hal_executable_t* base_
   IREE_TRACE_ZONE_BEGIN(z0);
   thip_executable_destroy(executable->executable);
   iree_allocator_free(host_allocator, executable);
+  iree_hal_thip_shared_device_release();
   IREE_TRACE_ZONE_END(z0);
 }
 
