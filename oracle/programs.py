@@ -278,3 +278,33 @@ def check_grouped_linear(wl, outputs, compare_close, compare_exact):
             assert not bad.any(), "%s %s: %d elements beyond the propagated bound" % (wl.name, op.out, int(bad.sum()))
         else:
             compare_close(got.reshape(want.shape), want, "%s %s" % (wl.name, op.out), magnitude=mag.reshape(want.shape))
+
+
+def check_attention(wl, outputs, compare_close):
+    """An attention_workload's context against the two matmuls it stands for (orc.matmul_bf16 twice, the scores
+    rounded to bf16 in between).  The scores never leave the GPU, so the context is checked on the oracle's scores,
+    with room for the one thing that may differ: a score whose exact value lies within the fp32 summation-order
+    allowance (2^-17 of its sum of |products|) of a bf16 rounding boundary may be either neighbour, and moves the
+    context by its bf16 step times the value it multiplies."""
+    q, keys, vals = wl.inputs
+    if q.ndim == 2:
+        q, keys, vals = q[None], keys[None], vals[None]
+    b1 = np.array([wl.attrs["bias"][0]], np.float32)
+    b2 = np.array([wl.attrs["bias"][1]], np.float32)
+    lo1, hi1 = wl.attrs["clamp1"]
+    lo2, hi2 = wl.attrs["clamp2"]
+    kT = np.ascontiguousarray(keys.transpose(0, 2, 1))
+    vT = np.ascontiguousarray(vals.transpose(0, 2, 1))
+    scores = orc.matmul_bf16(q, kT, b1, output_min=lo1, output_max=hi1)
+    want = orc.matmul_bf16(scores, vT, b2, output_min=lo2, output_max=hi2)
+    exact = np.einsum("bhd,bdt->bht", _f64(q), _f64(kT)) + float(b1[0])
+    mag1 = np.einsum("bhd,bdt->bht", np.abs(_f64(q)), np.abs(_f64(kT))) + abs(float(b1[0]))
+    sf = _f64(scores)
+    step = np.spacing(np.abs(orc.from_bf16(scores)).astype(np.float32)).astype(np.float64) * 65536.0  # a bf16 step at each score
+    boundary = sf + np.where(exact >= sf, 0.5, -0.5) * step
+    either = np.abs(exact - boundary) <= mag1 * 2.0 ** -17
+    room = np.einsum("bht,btd->bhd", either * step, np.abs(_f64(vT)))
+    mag2 = np.einsum("bht,btd->bhd", np.abs(sf), np.abs(_f64(vT))) + abs(float(b2[0]))
+    got = outputs[0].reshape(want.shape)
+    compare_close(got, want, wl.name, magnitude=mag2 + room * 2.0 ** 17)
+    return int(either.sum()), int(either.size)

@@ -127,6 +127,20 @@ def test_transposed_operand_is_read_in_place():
         assert np.array_equal(res, want)
 
 
+ATTENTION = [dict(B=1, H=4, D=256, T=1024, D2=256), dict(B=3, H=1, D=32, T=64, D2=16), dict(B=2, H=16, D=64, T=128, D2=48),
+             dict(B=5, H=7, D=96, T=192, D2=80, bias=(0.5, -0.25), clamp1=(-1.0, 1.5), clamp2=(-0.5, 0.75)),
+             dict(B=1, H=4, D=128, T=256, D2=64, rank2=True)]
+
+
+@pytest.mark.parametrize("case", ATTENTION + [dict(B=2, H=4, D=64, T=96, D2=24)], ids=_case_id)
+def test_attention_records(case):
+    """scores = q K^T, context = scores V with the scores an intermediate: two records reading the caches in place."""
+    wl = w.attention_workload(**case)
+    blob, outs = _interp(wl)
+    assert _kinds(blob) == [K_DEC_MATMUL, K_DEC_MATMUL]
+    prog.check_attention(wl, outs, lambda g, want, what, magnitude=None: prog.assert_bit_exact(g, want, what))
+
+
 # ---- GPU ----------------------------------------------------------------------------------------------------------
 
 def _run_gpu(device, wl, dispatches=1):
@@ -209,6 +223,19 @@ def test_gpu_grouped_linear(device, case):
     results, kernels = _run_gpu(device, wl)
     assert len(kernels) == 1 and kernels[0].startswith("dec_linear<"), kernels
     prog.check_grouped_linear(wl, results[0], prog.assert_bf16_close, prog.assert_bit_exact)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", ATTENTION + [dict(B=32, H=4, D=256, T=1024, D2=256), dict(B=2, H=4, D=256, T=4096, D2=256)], ids=_case_id)
+def test_gpu_attention(device, case):
+    """One decode step of attention with the scores hidden between its two matmuls, against the oracle's two matmuls;
+    eager, captured and replayed dispatches agree bit for bit."""
+    wl = w.attention_workload(**case)
+    results, kernels = _run_gpu(device, wl, dispatches=3)
+    assert [k.split("<")[0] for k in kernels] == ["dec_matmul", "dec_matmul"], kernels
+    for outs in results:
+        prog.check_attention(wl, outs, prog.assert_bf16_close)
+    assert all(np.array_equal(outs[0], results[0][0]) for outs in results[1:])
 
 
 @pytest.mark.gpu

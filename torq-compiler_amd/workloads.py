@@ -927,6 +927,33 @@ def decoder_step_workload(batch=1, layers=26, hidden=1152, heads=4, head_dim=256
     return Workload("decoder_step_b%d_l%d" % (batch, layers), p, inputs, outputs, 2 * macs, bytes_, attrs)
 
 
+def attention_workload(B=2, H=4, D=256, T=1024, D2=256, bias=(0.0, 0.0), clamp1=None, clamp2=None, rank2=False, seed=1045):
+    """One decode step of attention as the decoder workload chains it: scores = q K^T against a key cache held
+    [B, T, D], context = scores V against a value cache held dimension-major [B, D2, T] (both through a
+    torq_hl.transpose that is read in place), the scores an intermediate nobody else reads.  Bindings: 0 q [B, H, D],
+    1 keys, 2 values, 3 context [B, H, D2].  rank2: B == 1 with rank-2 operands."""
+    rng = np.random.default_rng(seed)
+    lead = () if rank2 else (B,)
+    assert not rank2 or B == 1
+    q = to_bf16(rng.standard_normal(lead + (H, D)))
+    keys = to_bf16(rng.standard_normal(lead + (T, D)) / np.sqrt(D))
+    vals = to_bf16(rng.standard_normal(lead + (D2, T)) / np.sqrt(T))
+    perm = (1, 0) if rank2 else (0, 2, 1)
+    p = Program()
+    bq = p.binding(0, q.shape, np.uint16)
+    bk = p.binding(1, keys.shape, np.uint16)
+    bv = p.binding(2, vals.shape, np.uint16)
+    out = p.binding(3, lead + (H, D2), np.uint16)
+    lo1, hi1 = NO_CLAMP if clamp1 is None else (float_bits(clamp1[0]), float_bits(clamp1[1]))
+    lo2, hi2 = NO_CLAMP if clamp2 is None else (float_bits(clamp2[0]), float_bits(clamp2[1]))
+    scores = p.matmul(bq, p.transpose(bk, perm), np.array([bias[0]], np.float32), init=p.tensor(lead + (H, T), np.uint16), output_zp=0,
+                      output_min=lo1, output_max=hi1, shift=0)
+    p.matmul(scores, p.transpose(bv, perm), np.array([bias[1]], np.float32), init=out, output_zp=0, output_min=lo2, output_max=hi2, shift=0)
+    attrs = dict(bias=bias, clamp1=(lo1, hi1), clamp2=(lo2, hi2))
+    return Workload("attention_%dx%dx%dx%dx%d" % (B, H, D, T, D2), p, [q, keys, vals], [(lead + (H, D2), np.uint16)],
+                    2 * B * H * T * (D + D2), 2 * (q.size + keys.size + vals.size + B * H * D2), attrs)
+
+
 def grouped_linear_workload(M=3, K=256, N=64, mode="single", block=128, zero_points=False, clamp=None, expand_clamp=None, seed=1050):
     """Small programs of the shapes a decoder layer is made of, every result an output binding: mode "single" one
     linear; "concat" three linears (N, N / 2, N / 2 columns) on the same rows; "pair" two linears whose results an
