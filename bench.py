@@ -465,11 +465,26 @@ def main():
                          "bandwidth rows of per_op are timed")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (a 1x1 max pool), to scale rocprofv3's FETCH_SIZE / WRITE_SIZE by")
+    ap.add_argument("--stream-floor", action="store_true",
+                    help="only the streaming-floor calibration: the fastest member of the family for the traffic shape of every "
+                         "bandwidth row and for a 256 MiB copy, cold; one JSON line (for a run under rocprofv3)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
 
     pkg = import_package()
+    if args.stream_floor:
+        dev = pkg.Device(0)
+        rows = {}
+        for name, (rd, wbytes) in list(STREAM_SHAPES.items()) + [("copy_256MiB", (1, 256 << 20))]:
+            wbytes = wbytes // 16 * 16
+            us, kernel = min(dev.stream_floor(rd, wbytes, cold=True, variant=True) for _ in range(3))
+            moved = (rd + 1) * wbytes
+            rows[name] = {"reads_per_write": rd, "bytes": moved, "us": round(us, 2), "kernel": kernel, "GB/s": round(moved / us / 1e3, 1),
+                          "frac": round(moved / us / 1e3 / PEAK_HBM_GBS, 3)}
+        dev.close()
+        print(json.dumps({"streaming_floor": rows}))
+        return
     table = workload_table(pkg)
     nets = network_table(pkg)
     if args.workload in nets:

@@ -195,7 +195,8 @@ def test_gpu_decoder_step_batches(device, batch):
         through_lds = [k.startswith("dec_linear<1,1,1,") for k in linears]
         assert all(through_lds) if batch <= 2 else (sum(through_lds) == len(linears) - 2 and all(k.startswith(("dec_linear<1,1,1,", "dec_linear<1,2,0,")) for k in linears)), kernels
     else:
-        assert all(k.startswith("dec_linear<1,2,0," if batch <= 16 else "dec_linear<2,1,0,") for k in linears), kernels
+        # (few column tiles share their rows out over several workgroups, each with at most 16 of them)
+        assert all(k.startswith(("dec_linear<1,2,0,", "dec_linear<2,1,0,") if batch > 16 else "dec_linear<1,2,0,") for k in linears), kernels
 
 
 @pytest.mark.gpu

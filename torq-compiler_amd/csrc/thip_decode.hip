@@ -55,6 +55,10 @@ __global__ __launch_bounds__(kDecMaxWaves * 64) void dec_linear(DecLinearArgs p)
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int NW = p.nwaves;  // waves of this workgroup: k-blocks wave, wave + NW, ... are this wave's
     const int c = lane & 15, g = lane >> 4;
+    // the input rows of this workgroup: grid.y workgroups share a column tile, rows_per_group rows each
+    const int row0 = (int)blockIdx.y * p.rows_per_group;
+    const int M = p.M - row0 < p.rows_per_group ? p.M - row0 : p.rows_per_group;
+    const uint16_t *x = p.x + (size_t)row0 * p.K;
     // the tile of this workgroup: (matrix, 16 columns of it); a pair owns the same columns of both matrices
     int tile = (int)blockIdx.x, seg = 0;
     if (!p.pair) {
@@ -72,7 +76,7 @@ __global__ __launch_bounds__(kDecMaxWaves * 64) void dec_linear(DecLinearArgs p)
     const int nkb = wave < kblocks ? (kblocks - wave + NW - 1) / NW : 0;  
     const int maxkb = (kblocks + NW - 1) / NW;
     const int slotBytes = kDecSlotBytes + (QB ? 64 : 0);
-    const int xRowBytes = XLDS ? p.M * 256 : 0;  // a k-block of the input rows in LDS
+    const int xRowBytes = XLDS ? M * 256 : 0;  // a k-block of the input rows in LDS
     const unsigned regionBytes = (unsigned)maxkb * (unsigned)(xRowBytes + nmat * kDecLdsSlot);
     int8_t *region = smem + (size_t)wave * regionBytes;
     int8_t *slots = region + (size_t)maxkb * xRowBytes;
@@ -88,7 +92,7 @@ __global__ __launch_bounds__(kDecMaxWaves * 64) void dec_linear(DecLinearArgs p)
         // lane l brings 16 bytes of row l >> 4: a k-block of one row is 16 lanes x 16 bytes
         for (int i = 0; i < nkb; i++) {
             const int kb = wave + NW * i;
-            if (lane < 16 * p.M) dmaLoad16(p.x + (size_t)(lane >> 4) * p.K + kb * 128 + (lane & 15) * 8, regionLds + (unsigned)(i * xRowBytes));
+            if (lane < 16 * M) dmaLoad16(x + (size_t)(lane >> 4) * p.K + kb * 128 + (lane & 15) * 8, regionLds + (unsigned)(i * xRowBytes));
         }
     }
     // the wave's whole share of the weights, one burst: per k-block and matrix 2 KiB and the scales, straight into LDS
@@ -128,7 +132,7 @@ __global__ __launch_bounds__(kDecMaxWaves * 64) void dec_linear(DecLinearArgs p)
         }
     };
     if constexpr (XLDS) {
-        const int xrow = (c < p.M ? c : 0) * 256 + g * 16;  // lanes of rows the input does not have read row 0 (never stored)
+        const int xrow = (c < M ? c : 0) * 256 + g * 16;  // lanes of rows the input does not have read row 0 (never stored)
         for (int i = 0; i < ((p.ablate & 2) ? 0 : nkb); i++) {
             waitVmcntDyn((p.ablate & 1) ? 0 : (nkb - 1 - i) * 3 * nmat);  // everything up to this k-block has landed
             v4i xp[4][MR];
@@ -152,7 +156,7 @@ __global__ __launch_bounds__(kDecMaxWaves * 64) void dec_linear(DecLinearArgs p)
 #pragma unroll
                     for (int mr = 0; mr < MR; mr++) {
                         const int row = c + 16 * mr;
-                        b.x[u][j][mr] = (i < nkb && row < p.M) ? *(const v4i *)(p.x + (size_t)row * p.K + kb * 128 + 32 * j + 8 * g) : v4i{0, 0, 0, 0};
+                        b.x[u][j][mr] = (i < nkb && row < M) ? *(const v4i *)(x + (size_t)row * p.K + kb * 128 + 32 * j + 8 * g) : v4i{0, 0, 0, 0};
                     }
                 }
             }
@@ -191,8 +195,8 @@ __global__ __launch_bounds__(kDecMaxWaves * 64) void dec_linear(DecLinearArgs p)
     __syncthreads();
     if (wave >= MR) return;
     const int mr = wave;  // this wave finishes row group `wave`
-    const int row = c + 16 * mr;
-    if (row >= p.M) return;
+    if (c + 16 * mr >= M) return;
+    const int row = row0 + c + 16 * mr;  // as the whole launch counts them
     const int s0 = p.pair ? 0 : seg;
     const int Nseg = s0 == 0 ? p.N[0] : s0 == 1 ? p.N[1] : p.N[2];
     const int n = tile * 16 + 4 * g;
@@ -248,7 +252,9 @@ static hipError_t launchDecLinearT(const DecLinearArgs &a, int tiles, size_t lds
     static hipError_t configured = hipSuccess;
     std::call_once(once, [&] { configured = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); });
     if (configured != hipSuccess) return configured;
-    THIP_ENQUEUE(ctx, kernelLabel("dec_linear", {MR, CH, (int)XLDS, (int)QB, (int)QC, a.pair ? 2 : a.nseg, a.add_mode}), kernel, dim3((unsigned)tiles), dim3((unsigned)a.nwaves * 64), lds, a);
+    const int groups = (a.M + a.rows_per_group - 1) / a.rows_per_group;
+    THIP_ENQUEUE(ctx, kernelLabel("dec_linear", {MR, CH, (int)XLDS, (int)QB, (int)QC, a.pair ? 2 : a.nseg, a.add_mode}), kernel, dim3((unsigned)tiles, (unsigned)groups),
+                 dim3((unsigned)a.nwaves * 64), lds, a);
     return hipGetLastError();
 }
 
@@ -267,10 +273,23 @@ int decLinearWaves(int K) {
 constexpr size_t kDecMaxLds = 152 * 1024;
 constexpr int kDecLdsRows = 4;  // up to this many input rows may come through LDS
 
+// Workgroups per column tile.  A workgroup streams its rows of the input next to its 16 columns of the weights: with few
+// column tiles and many rows (32 rows of K = 6912 are 442 KB per workgroup against 110 KB of weights, on 72 of 256 CUs)
+// the rows are the traffic, and sharing them out over several workgroups, each re-reading the weights, spreads it over
+// the chip.  As many groups as keep the launch within one workgroup per CU, at least eight rows each.
+static int decLinearRowGroups(int M, int tiles, const Tuning *tuning) {
+    if (M <= kDecLdsRows) return 1;
+    int groups = (tuning && tuning->decTargetGroups > 0 ? tuning->decTargetGroups : 256) / tiles;
+    const int most = (M + 7) / 8;
+    groups = groups < 1 ? 1 : (groups > most ? most : groups);
+    return groups;
+}
+
 template <bool QB, bool QC>
 static hipError_t launchDecLinearQ(const DecLinearArgs &in, int tiles, const LaunchCtx &ctx) {
     DecLinearArgs a = in;
     const int nmat = a.pair ? 2 : 1;
+    a.rows_per_group = a.M;
     if (a.M <= kDecLdsRows) {
         // the input rows through LDS as well, with the most waves whose regions still fit
         for (int nw = a.nwaves; nw >= kDecWaves; nw--) {
@@ -279,8 +298,10 @@ static hipError_t launchDecLinearQ(const DecLinearArgs &in, int tiles, const Lau
             return launchDecLinearT<1, 1, true, QB, QC>(a, tiles, decLinearLds(a.K, nmat, a.M, nw), ctx);
         }
     }
+    const int groups = decLinearRowGroups(a.M, tiles, ctx.tuning);
+    a.rows_per_group = (a.M + groups - 1) / groups;
     const size_t lds = decLinearLds(a.K, nmat, 0, a.nwaves);
-    if (a.M <= 16) return launchDecLinearT<1, 2, false, QB, QC>(a, tiles, lds, ctx);
+    if (a.rows_per_group <= 16) return launchDecLinearT<1, 2, false, QB, QC>(a, tiles, lds, ctx);
     return launchDecLinearT<2, 1, false, QB, QC>(a, tiles, lds, ctx);
 }
 

@@ -275,6 +275,7 @@ Tuning tuningFromEnvironment() {
     t.maxpoolGeneric = flag("THIP_MAXPOOL_GENERIC");
     t.addGeneric = flag("THIP_ADD_GENERIC");
     if (const char *v = getenv("THIP_DEC_ABLATE")) t.decAblate = atoi(v);
+    if (const char *v = getenv("THIP_DEC_TARGET_WORKGROUPS")) t.decTargetGroups = atoi(v);
     return t;
 }
 

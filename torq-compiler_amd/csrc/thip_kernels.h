@@ -44,6 +44,7 @@ struct Tuning {
     bool addGeneric = false;        // THIP_ADD_GENERIC: the quantised add always through the 64-bit ACT stage
     bool maxpoolGeneric = false;    // THIP_MAXPOOL_GENERIC: the any-window max pool kernel also for 2 x 2 stride 2
     int decAblate = 0;              // THIP_DEC_ABLATE: parts of dec_linear left out, for timing experiments (wrong results)
+    int decTargetGroups = 0;        // THIP_DEC_TARGET_WORKGROUPS: workgroups a dec_linear launch with few column tiles shares its rows out to (0: 256)
 };
 Tuning tuningFromEnvironment();
 
@@ -233,6 +234,7 @@ struct DecLinearArgs {
     uint16_t *add_out;
     float aw0, aw1, abias, alo, ahi;
     int32_t nwaves;  // waves per workgroup; the launcher sets it (decLinearWaves)
+    int32_t rows_per_group;  // input rows of a workgroup; the launcher sets it (grid.y workgroups share a column tile)
     int32_t ablate;  // timing experiments only (THIP_DEC_ABLATE; results are wrong): 1 no weight loads, 2 no arithmetic
 };
 inline int decSlotBytes(bool hasBias) { return kDecSlotBytes + (hasBias ? 64 : 0); }
