@@ -56,7 +56,8 @@ def workload_table(pkg):
         "conv3x3_28x28x512_o512_b32": (lambda: w.conv2d_workload(N=32, H=28, W=28, C=512, O=512, realistic=True), "mfma"),
         # a channel count that is no multiple of the 64-byte k-tile: k-tiles straddle the window's taps
         "conv3x3_56x56x96_o96_b32": (lambda: w.conv2d_workload(N=32, H=56, W=56, C=96, O=96, realistic=True), "mfma"),
-        "conv1x1_56x56x256_o1024_b32": (lambda: w.conv2d_workload(N=32, H=56, W=56, C=256, O=1024, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True), "mfma"),
+        # (26 MB in, 103 MB out, 53 GOP: 16 us of HBM traffic at 8 TB/s against 10.5 us of MFMA work at 5 POP/s -- the memory side bounds it)
+        "conv1x1_56x56x256_o1024_b32": (lambda: w.conv2d_workload(N=32, H=56, W=56, C=256, O=1024, KH=1, KW=1, pad=(0, 0, 0, 0), realistic=True), "hbm"),
         "depthwise_b64": (lambda: w.depthwise_workload(N=64), "hbm"),
         "depthwise_b1": (lambda: w.depthwise_workload(N=1), "hbm"),
         "depthwise_s1_b256": (lambda: w.depthwise_workload(N=256, stride=(1, 1), pad=(1, 1, 1, 1)), "hbm"),
@@ -194,19 +195,20 @@ class Loaded:
 # the kernel sources (under torq-compiler_amd/csrc) at that time, and a run whose kernel source -- the file the
 # workload's kernel lives in, or the helpers every kernel file includes -- has changed since reports traffic null.
 TRAFFIC_SOURCES_SHA256 = {
-    "thip_kernels_common.h": "89eff9b09a9cb00a464dea200f5c893757370fca1f92043d5425a4065d9b0096",
-    "thip_igemm.hip": "cc9944efbf5c09fdbfc49c93ded4d9c2b7af354a827f1dd1489ea76b28049485",
-    "thip_bandwidth.hip": "aa515d4402c1add8c14c40a2640ee69f316f3db48147c20798fe853213b03281",
+    "thip_kernels_common.h": "9e7783387939bacca5e8a40e8a9859135213407975bcc967c50e4c8025feb72a",
+    "thip_igemm.hip": "f2244679f589b21aad8bad523ae60b45d6b6f0838057052313d119ff49bbd712",
+    "thip_bandwidth.hip": "f152f95926c1fabe7debb7b708689096163480bbd0983aff0dff443ebb6f1667",
 }
 MEASURED_TRAFFIC = {
-    "fc_4096x4096x4096": (49387.0 * 1.9995 + 16582.3 * 1.0000) * 1024,
+    "fc_4096x4096x4096": (49385.0 * 1.9995 + 16581.2 * 1.0000) * 1024,
     "fc_512x4096x4096": (16453.0 * 1.9995 + 2048.0 * 1.0000) * 1024,
     "fc_16x2048x8192": (8408.0 * 1.9995 + 256.0 * 1.0000) * 1024,
-    "conv_112x112x32_o64_3x3": (366.7 * 1.9995 + 784.0 * 1.0000) * 1024,
-    "conv3x3_56x56x256_o256_b32": (17254.1 * 1.9995 + 25992.5 * 1.0000) * 1024,
-    "depthwise_b64": (15443.1 * 1.9995 + 7063.2 * 1.0000) * 1024,
-    "depthwise_s1_b256": (63722.4 * 1.9995 + 113158.0 * 1.0000) * 1024,
-    "maxpool_b64": (25122.4 * 1.9995 + 12544.0 * 1.0000) * 1024,
+    "conv_112x112x32_o64_3x3": (370.7 * 1.9995 + 784.0 * 1.0000) * 1024,
+    "conv3x3_56x56x256_o256_b32": (17259.9 * 1.9995 + 25990.4 * 1.0000) * 1024,
+    "conv1x1_56x56x256_o1024_b32": (14417.5 * 1.9995 + 100352.0 * 1.0000) * 1024,
+    "depthwise_b64": (14212.7 * 1.9995 + 7810.1 * 1.0000) * 1024,
+    "depthwise_s1_b256": (63709.1 * 1.9995 + 113146.6 * 1.0000) * 1024,
+    "maxpool_b64": (25477.1 * 1.9995 + 12544.0 * 1.0000) * 1024,
     "avgpool_b64": (2001.0 * 1.9995 + 80.0 * 1.0000) * 1024,
     "add_b64": (4723.0 * 1.9995 + 4704.0 * 1.0000) * 1024,
 }
