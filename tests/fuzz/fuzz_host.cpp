@@ -1,8 +1,9 @@
 // Host-side fuzz of the emitter and the descriptor validation, meant to be built with
 // -fsanitize=address,undefined (tests/test_fuzz.py does that and runs it).  Nothing here touches a GPU.
 //
-//   1. random programs through the C-ABI emitter (thip_program_* / thip_hl_*): sane and insane attribute values;
-//      every call must come back with a status;
+//   1. random programs through the C-ABI emitter (thip_program_* / thip_hl_*): single int8 ops and decode-shaped bf16
+//      programs (grouped linears on block-quantized weights, views, folded transposes), sane and insane attribute
+//      values; every call must come back with a status;
 //   2. every blob the emitter produces must validate; mutated copies (bit flips in the header, the kernel records,
 //      the tables; truncations) must come back with a status, never a crash or a sanitizer report;
 //   3. the CPU oracle on small random shapes (its indexing under the address sanitizer).
@@ -60,10 +61,153 @@ static thip_value_t binding(thip_program_t *p, uint32_t index, std::vector<int64
     return id;
 }
 
+static thip_value_t constantRaw(thip_program_t *p, int32_t dtype, std::vector<int64_t> shape, size_t elemBytes, int fill) {
+    size_t n = 1;
+    for (int64_t d : shape) n *= (size_t)d;
+    std::vector<uint8_t> v(n * elemBytes);
+    for (auto &x : v) x = fill < 0 ? (uint8_t)rng() : (uint8_t)fill;
+    if (dtype == THIP_DTYPE_BF16 && fill < 0) {
+        for (size_t i = 0; i < n; i++) v[2 * i + 1] = (uint8_t)(0x3b + (rng() & 3));  // finite, small
+    }
+    thip_value_t id = -1;
+    thip_program_constant(p, dtype, (int32_t)shape.size(), shape.data(), v.data(), v.size(), &id);
+    return id;
+}
+
+// A decode-shaped bf16 program: one to three linears on block-quantized int8 weights over the same rows (sometimes a
+// pair joined by an add, sometimes a residual add behind one), results into bindings, intermediates or views of a
+// binding, and sometimes a small matmul against a transposed run-time operand -- the shapes the grouping and the
+// slot packing of the serialiser are written for, and the ones just outside them.
+static thip_status_t buildDecodeProgram(thip_program_t *p, bool insane) {
+    const int64_t M = insane ? pick(1, 40) : pick(1, 32);
+    const int64_t block = (rng() % 4 == 0) ? 64 * pick(1, 5) : 128 * pick(1, 2);
+    const int64_t K = (rng() % 5 == 0) ? 16 * pick(1, 30) : block * pick(1, 4);
+    const int32_t noLo = (int32_t)0xff800000, noHi = 0x7f800000;
+    uint32_t nextBinding = 0;
+    const thip_value_t x = binding(p, nextBinding++, {M, K}, THIP_DTYPE_BF16);
+    const thip_value_t zero = constantRaw(p, THIP_DTYPE_F32, {1}, 4, 0);
+    const int mode = (int)(rng() % 5);  // 0 single, 1 several on the same rows, 2 pair + add, 3 residual add, 4 attention-shaped matmul
+    auto linear = [&](int64_t N, thip_value_t init, thip_value_t *result) -> thip_status_t {
+        if (K % block != 0) return THIP_INVALID_ARGUMENT;  // no such expansion exists
+        const int64_t G = K / block;
+        thip_hl_expand_weights_t e;
+        memset(&e, 0, sizeof(e));
+        e.input = constantRaw(p, THIP_DTYPE_I8, {K, N}, 1, -1);
+        e.scale = constantRaw(p, THIP_DTYPE_BF16, {G, N}, 2, -1);
+        e.scale_bias = constantRaw(p, THIP_DTYPE_F32, {G, N + (N & 1)}, 4, (rng() & 1) ? 0 : 0x3c);
+        e.block_size = insane && rng() % 4 == 0 ? wild() : (int32_t)block;
+        e.output_min = noLo;
+        e.output_max = noHi;
+        int64_t wshape[2] = {K, N};
+        if (thip_status_t s = thip_program_tensor(p, THIP_DTYPE_BF16, 2, wshape, &e.init)) return s;
+        if (thip_status_t s = thip_hl_expand_weights(p, &e)) return s;
+        thip_hl_matmul_t m;
+        memset(&m, 0, sizeof(m));
+        m.init = init;
+        m.output_min = noLo;
+        m.output_max = noHi;
+        m.shift = insane && rng() % 6 == 0 ? wild() : 0;
+        m.scale_bias = zero;
+        m.input1 = x;
+        m.input2 = e.init;
+        *result = init;
+        return thip_hl_matmul(p, &m);
+    };
+    auto result = [&](int64_t N, int how) -> thip_value_t {  // how: 0 binding, 1 intermediate, 2 a view into a larger binding
+        thip_value_t v = -1;
+        int64_t shape[2] = {M, N};
+        if (how == 1) {
+            thip_program_tensor(p, THIP_DTYPE_BF16, 2, shape, &v);
+        } else if (how == 2) {
+            const thip_value_t base = binding(p, nextBinding++, {3, M, N}, THIP_DTYPE_BF16);
+            thip_program_view(p, base, (insane && rng() % 3 == 0 ? (int64_t)wild() : M * N * pick(0, 2)), 2, shape, &v);
+        } else {
+            v = binding(p, nextBinding++, {M, N}, THIP_DTYPE_BF16);
+        }
+        return v;
+    };
+    auto add = [&](thip_value_t a, thip_value_t b, int64_t N) -> thip_status_t {
+        thip_hl_add_t c;
+        memset(&c, 0, sizeof(c));
+        c.init = binding(p, nextBinding++, {M, N}, THIP_DTYPE_BF16);
+        c.output_min = noLo;
+        c.output_max = noHi;
+        c.weights = constantRaw(p, THIP_DTYPE_BF16, {2}, 2, -1);
+        c.scale_bias = constantRaw(p, THIP_DTYPE_F32, {1}, 4, 0);
+        c.input1 = a;
+        c.input2 = b;
+        return thip_hl_add(p, &c);
+    };
+    const int64_t N = (rng() % 5 == 0) ? pick(1, 70) : 16 * pick(1, 6);
+    thip_value_t y0 = -1, y1 = -1, y2 = -1;
+    switch (mode) {
+    case 0: return linear(N, result(N, (int)(rng() % 3)), &y0);
+    case 1: {
+        if (thip_status_t s = linear(N, result(N, (int)(rng() % 3)), &y0)) return s;
+        const int64_t N2 = 16 * pick(1, 3);
+        if (thip_status_t s = linear(N2, result(N2, (int)(rng() % 3)), &y1)) return s;
+        if (rng() & 1) return linear(N2, result(N2, 0), &y2);
+        return THIP_OK;
+    }
+    case 2: {
+        const int how = (int)(rng() % 2);
+        if (thip_status_t s = linear(N, result(N, how), &y0)) return s;
+        if (thip_status_t s = linear(N, result(N, how), &y1)) return s;
+        return add(y0, y1, N);
+    }
+    case 3: {
+        if (thip_status_t s = linear(K, result(K, (int)(rng() % 2)), &y0)) return s;  // a residual needs N == K
+        return (rng() & 1) ? add(y0, x, K) : add(x, y0, K);
+    }
+    default: {
+        const int64_t B = pick(1, 3), H = pick(1, insane ? 40 : 8), D = 8 * pick(1, 8), T = pick(1, 40);
+        const thip_value_t q = binding(p, nextBinding++, {B, H, D}, THIP_DTYPE_BF16);
+        const thip_value_t keys = binding(p, nextBinding++, {B, T, D}, THIP_DTYPE_BF16);
+        thip_hl_transpose_t t;
+        memset(&t, 0, sizeof(t));
+        t.rank = 3;
+        t.perm[0] = 0; t.perm[1] = 2; t.perm[2] = insane && rng() % 4 == 0 ? wild() : 1;
+        t.input = keys;
+        int64_t tshape[3] = {B, D, T};
+        if (thip_status_t s = thip_program_tensor(p, THIP_DTYPE_BF16, 3, tshape, &t.init)) return s;
+        if (thip_status_t s = thip_hl_transpose(p, &t)) return s;
+        thip_hl_matmul_t m;
+        memset(&m, 0, sizeof(m));
+        m.init = binding(p, nextBinding++, {B, H, T}, THIP_DTYPE_BF16);
+        m.output_min = noLo;
+        m.output_max = noHi;
+        m.scale_bias = zero;
+        m.input1 = q;
+        m.input2 = t.init;
+        return thip_hl_matmul(p, &m);
+    }
+    }
+}
+
 // One random program; `insane` also randomises attributes beyond what any pattern would produce.
 static bool buildProgram(bool insane, Blob *out, long *statuses) {
     thip_program_t *p = nullptr;
     if (thip_program_create(&p) != THIP_OK) return false;
+    if (rng() % 4 == 0) {
+        const thip_status_t st = buildDecodeProgram(p, insane);
+        statuses[st == THIP_OK ? 0 : 1]++;
+        bool have = false;
+        if (st == THIP_OK) {
+            void *blob = nullptr;
+            size_t size = 0;
+            const thip_status_t ss = thip_program_serialize(p, &blob, &size);
+            statuses[ss == THIP_OK ? 2 : 3]++;
+            if (ss == THIP_OK) {
+                out->words.assign((size + 7) / 8, 0);
+                out->size = size;
+                memcpy(out->data(), blob, size);
+                thip_blob_free(blob);
+                have = true;
+            }
+        }
+        thip_program_destroy(p);
+        return have;
+    }
     const int64_t N = pick(1, 2), H = pick(1, 9), W = pick(1, 9), C = pick(1, 40), O = pick(1, 40);
     const int64_t KH = pick(1, 3), KW = pick(1, 3);
     const bool nhwc = rng() & 1;
@@ -212,7 +356,7 @@ static void oracleSmoke() {
 
 int main(int argc, char **argv) {
     const int programs = argc > 1 ? atoi(argv[1]) : 300, mutations = argc > 2 ? atoi(argv[2]) : 60;
-    long statuses[4] = {0, 0, 0, 0}, valid = 0, refused = 0, accepted = 0;
+    long statuses[4] = {0, 0, 0, 0}, valid = 0, refused = 0, accepted = 0, grouped = 0;
     for (int it = 0; it < programs; it++) {
         Blob blob;
         const bool insane = it % 3 == 2;
@@ -224,6 +368,10 @@ int main(int argc, char **argv) {
         }
         valid++;
         const thip::DescHeader *h = (const thip::DescHeader *)blob.data();
+        {
+            const thip::DescOp *ops = (const thip::DescOp *)(blob.data() + h->ops_offset);
+            for (uint32_t i = 0; i < h->op_count; i++) grouped += ops[i].kind == thip::kKindDecLinear || ops[i].kind == thip::kKindDecMatmul;
+        }
         const size_t structured = (size_t)h->data_offset;  // header + records + tables: where a flip matters
         for (int m = 0; m < mutations; m++) {
             Blob bad = blob;
@@ -251,9 +399,9 @@ int main(int argc, char **argv) {
         }
     }
     oracleSmoke();
-    printf("programs built %ld (refused by the emitter %ld), serialised %ld (refused %ld), valid blobs %ld, mutants refused %ld / accepted %ld\n",
-           statuses[0], statuses[1], statuses[2], statuses[3], valid, refused, accepted);
-    if (valid < programs / 4 || refused == 0) {
+    printf("programs built %ld (refused by the emitter %ld), serialised %ld (refused %ld), valid blobs %ld (grouped-linear / in-place-matmul records %ld), mutants refused %ld / accepted %ld\n",
+           statuses[0], statuses[1], statuses[2], statuses[3], valid, grouped, refused, accepted);
+    if (valid < programs / 4 || refused == 0 || (programs >= 200 && grouped == 0)) {
         printf("FAIL: the fuzz did not reach both outcomes\n");
         return 1;
     }

@@ -13,6 +13,7 @@ import subprocess
 import numpy as np
 import pytest
 
+import desc_interp
 from torq_compiler_amd import runtime, workloads as w
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -36,17 +37,24 @@ def _validate(blob_bytes, size=None):
     lambda: w.matmul_workload(2, 9, 61, 37), lambda: w.fully_connected_bf16_workload(1, 6912, 256),
     lambda: w.expand_weights_workload(M=4, K=256, N=96, block=32), lambda: w.pointwise_add_workload(N=1, H=16, W=16, C=32, O=32),
     lambda: w.mobilenet_v2_workload(batch=1, resolution=32, classes=10, width=0.25),
-], ids=["conv_runs", "conv_gather", "depthwise", "fc", "matmul", "fc_bf16_splitk", "expand_mm", "conv_add", "network"])
+    lambda: w.grouped_linear_workload(mode="pair", zero_points=True), lambda: w.grouped_linear_workload(mode="concat", M=32),
+    lambda: w.grouped_linear_workload(mode="residual", K=256, N=256), lambda: w.attention_workload(B=2, H=4, D=64, T=128, D2=64),
+    lambda: w.decoder_step_workload(batch=3, layers=1, hidden=256, heads=2, head_dim=64, ffn=384, vocab=512, cache_len=64),
+], ids=["conv_runs", "conv_gather", "depthwise", "fc", "matmul", "fc_bf16_splitk", "expand_mm", "conv_add", "network", "linear_pair", "linear_concat",
+        "linear_residual", "attention", "decoder_step"])
 def test_mutated_descriptors_return_a_status(make):
     blob = bytearray(make().program.serialize())
     assert _validate(blob) == runtime.OK
     header = np.frombuffer(bytes(blob[:88]), dtype="<u8")
     structured = int(header[8])  # data_offset: header, records and tables lie below it
+    # the grouped linear records keep their per-matrix operand references in a constant (their `table`): mutate those too
+    d = desc_interp.Descriptor(bytes(blob))
+    ext = [(structured + int(d.consts[int(o["table"]["index"])]["offset"]) + int(o["table"]["offset"]), 224) for o in d.ops if int(o["kind"]) == 15]
     rng = np.random.default_rng(len(blob))
     outcomes = set()
     for _ in range(400):
         bad = bytearray(blob)
-        how = int(rng.integers(0, 4))
+        how = int(rng.integers(0, 5 if ext else 4))
         size = None
         if how == 0:
             size = int(rng.integers(0, len(bad)))
@@ -56,9 +64,13 @@ def test_mutated_descriptors_return_a_status(make):
         elif how == 2:
             for _ in range(int(rng.integers(1, 4))):
                 bad[int(rng.integers(0, structured))] ^= 1 << int(rng.integers(0, 8))
-        else:
+        elif how == 3:
             at = int(rng.integers(0, structured // 4)) * 4
             bad[at:at + 4] = int(rng.choice([0, 0xffffffff, 0x7fffffff, 0x80000000, int(rng.integers(0, 1 << 32))])).to_bytes(4, "little")
+        else:
+            start, size_ext = ext[int(rng.integers(0, len(ext)))]
+            at = start + int(rng.integers(0, size_ext // 4)) * 4
+            bad[at:at + 4] = int(rng.choice([0, 0xffffffff, 0x7fffffff, 0x80000000, 3, int(rng.integers(0, 1 << 32))])).to_bytes(4, "little")
         outcomes.add(_validate(bad, size))
     assert runtime.INVALID_ARGUMENT in outcomes  # and whatever else came back was a status: the process is still here
 
