@@ -90,10 +90,30 @@ def test_iree_glue_covers_every_op_entry_point():
     listed = set(re.findall(r"^\| `(iree_hal_torq_\w+)` \|", readme, re.M))
     used = {n for n in re.findall(r"\b(iree_hal_torq_\w+)\(", text) if not n.endswith("_t")}
     assert used == listed, sorted(used ^ listed)
-    # the hunks the README asks for in the reference's files call only what the glue defines
-    hunks = set(re.findall(r"^\+.*?\b(iree_hal_thip_\w+)\s*\(", readme, re.M))
+    # the hunks for the reference's own files call only what the glue defines
+    patch = open(os.path.join(gdir, "reference_hunks.patch")).read()
+    hunks = set(re.findall(r"^\+.*?\b(iree_hal_thip_\w+)\s*\(", patch, re.M))
     assert hunks and hunks <= defined, sorted(hunks - defined)
+    assert "IREE_HAL_THIP_EXECUTABLE_FORMAT" in sources["thip_native_executable.h"] and "IREE_HAL_THIP_EXECUTABLE_FORMAT" in patch
+
     abi = set(re.findall(r"\b(thip_[a-z_0-9]+)\s*\(", text))
     abi = {n for n in abi if not n.endswith("_t")}
     exported = set(runtime.EXPORTED_SYMBOLS)
     assert abi <= exported, sorted(abi - exported)
+
+
+def test_reference_hunks_apply(tmp_path):
+    """iree_glue/reference_hunks.patch against the reference checkout, where there is one (a dry run on copies)."""
+    import shutil
+    import subprocess
+    ref = "/root/reference/runtime/driver"
+    if not os.path.isdir(ref) or not shutil.which("patch"):
+        pytest.skip("no reference checkout (or no patch tool) on this machine")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    dst = tmp_path / "runtime" / "driver"
+    dst.mkdir(parents=True)
+    for name in ("nop_executable_cache.cc", "torq_command_buffer.c"):
+        shutil.copy(os.path.join(ref, name), dst / name)
+    run = subprocess.run(["patch", "-p1", "--dry-run", "-i", os.path.join(root, "iree_glue", "reference_hunks.patch")], cwd=tmp_path,
+                         stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    assert run.returncode == 0 and "FAILED" not in run.stdout and "fuzz" not in run.stdout, run.stdout
