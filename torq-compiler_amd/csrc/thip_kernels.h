@@ -204,7 +204,8 @@ hipError_t launchFcBf16(const FcBf16Args &a, const LaunchCtx &ctx);
 // (`nseg` segments: q, k, v of an attention block), or two matrices of equal width whose results are added
 // (`pair`: gate and up), and can apply the torq_hl.add that follows to its result (a residual connection).  A
 // workgroup owns 16 output columns: it brings its whole share of the weights into LDS with one burst of LDS-DMA
-// loads, its eight waves split K, and their partial sums meet in LDS.
+// loads, its eight to sixteen waves split K, and their partial sums meet in LDS; where few column tiles meet many
+// input rows, several workgroups share a tile and take a group of the rows each.
 //
 // Weight layout ("dec16"): for column tile t (16 columns) and k-block b (128 input rows) one slot of kDecSlotBytes
 // (+ 64 with block biases): first 2 KiB of weights, piece p (0, 1) = 64 lanes x 16 bytes, lane l = column l & 15 and
